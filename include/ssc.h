@@ -1,0 +1,233 @@
+/*
+ * ssc.h -- C ABI of the MI355X (gfx950) sparse steerable convolution hot path.
+ *
+ * Every entry point takes plain device pointers, sizes and a HIP stream
+ * (passed as void*; NULL = the null stream) and returns 0 on success or a
+ * negative SSC_E* code; ssc_last_error() then holds a readable message for the
+ * calling thread.  No entry point allocates device memory: the caller supplies
+ * outputs and, where stated, a workspace whose size the matching
+ * *_workspace_bytes() function reports.  Kernels are enqueued on `stream` and
+ * the call returns without synchronising unless its comment says otherwise.
+ * Results are reproducible run to run: no floating-point atomics are used and
+ * every accumulation order is fixed.
+ *
+ * All index tensors are int32, all feature tensors fp32, row-major and
+ * contiguous unless strides are passed explicitly.
+ *
+ * Each declaration cites the interface of the reference implementation
+ * (paths relative to SS_Conv_lib/) that it stands in for.
+ */
+#ifndef SSC_H_
+#define SSC_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SSC_OK 0
+#define SSC_EINVAL (-1)    /* bad argument (reference: std::invalid_argument / TV_ASSERT_INVALID_ARG) */
+#define SSC_ERUNTIME (-2)  /* runtime check failed (reference: std::runtime_error / TV_ASSERT_RT_ERR) */
+#define SSC_EWORKSPACE (-3)/* workspace too small */
+#define SSC_EHIP (-4)      /* a HIP call failed */
+
+#define SSC_MAX_KERNEL_VOLUME 256 /* src/conv/indice_conv.h:44 */
+
+typedef void *ssc_stream_t; /* hipStream_t */
+
+/* Library version (major*10000 + minor*100 + patch). */
+int ssc_version(void);
+
+/* Message of the last failing call on this thread ("" if none). */
+const char *ssc_last_error(void);
+
+/* Geometry of one sparse convolution / pooling window.
+ * Mirrors the argument list of get_indice_pairs_3d
+ * (src/ss_conv_ops.cu:31, src/conv/indice_conv.h:21-27). */
+typedef struct ssc_geometry {
+  int32_t batch_size;
+  int32_t out_shape[3];
+  int32_t ksize[3];
+  int32_t stride[3];
+  int32_t padding[3];
+  int32_t dilation[3];
+  int32_t subm;      /* 1: submanifold (stride forced to 1, padding to ksize/2; indice_conv.h:70-74) */
+  int32_t transpose; /* must be 0: transposed rulebooks are not built */
+} ssc_geometry;
+
+/* ------------------------------------------------------------------------
+ * Rulebook ("indice pairs").  Replaces getIndicePair<3>
+ * (src/conv/indice_conv.h:21-131; GPU kernels src/conv/indice_cuda_functor.cu:23-66,
+ * 113-149; CPU algorithm src/conv/geometry.h:18-80,140-189,241-288).
+ *
+ * Two calls because the number of active outputs is data dependent:
+ *   ssc_rulebook_count: marks every reachable output voxel, ranks them and
+ *     writes the count to *n_out_host.  SYNCHRONISES `stream` (the reference
+ *     learns the same number from torch::_unique, indice_conv.h:120).
+ *   ssc_rulebook_emit: writes out_indices[n_out,4] (b,x,y,z) in ascending
+ *     order of the flat key ((b*X+x)*Y+y)*Z+z (the order of the reference's GPU
+ *     path), pairs[K,2,n_in] (plane 0 input rows, plane 1 output rows, -1
+ *     padded) and pair_num[K].  Within one offset the pairs are in ascending
+ *     input-row order (the order of the reference's CPU path); the GPU path of
+ *     the reference leaves that order to an atomic race.
+ * With subm=1 out_indices is not written (outputs are the inputs) and n_out=n_in.
+ * The same workspace must be passed, untouched, to both calls.
+ * Limits: K = prod(ksize) <= 256; batch_size*prod(out_shape) < 2^31.
+ * ---------------------------------------------------------------------- */
+size_t ssc_rulebook_workspace_bytes(const ssc_geometry *g, int64_t n_in);
+
+int ssc_rulebook_count(const int32_t *indices /* [n_in,4] device */, int64_t n_in,
+                       const ssc_geometry *g, void *workspace, size_t workspace_bytes,
+                       int32_t *n_out_host /* host */, ssc_stream_t stream);
+
+int ssc_rulebook_emit(const int32_t *indices, int64_t n_in, const ssc_geometry *g,
+                      void *workspace, size_t workspace_bytes,
+                      int32_t *out_indices /* [n_out,4] device; may be NULL when subm */,
+                      int32_t *pairs /* [K,2,n_in] device */,
+                      int32_t *pair_num /* [K] device */, ssc_stream_t stream);
+
+/* ------------------------------------------------------------------------
+ * Sparse convolution forward.  Replaces indiceConv<float>
+ * (src/conv/indice_conv.h:247-343; bound as indice_conv_fp32,
+ * src/ss_conv_ops_api.cpp:21) together with the gather / scatter-add kernels
+ * it launches (src/conv/reordering_cuda_functor.cu:23-272):
+ *   out[o,:] = sum_k sum_{(i,o) in pairs[k]} features[i,:] * filters[k]
+ * as one output-stationary implicit GEMM on fp32 MFMA, offsets accumulated in
+ * ascending k.  `filters` is addressed as filters[k*fs_k + ci*fs_ci + co*fs_co]
+ * (element strides), so both a contiguous [K,Cin,Cout] kernel and the
+ * reference's permuted view of [Cout,Cin,K] (ss_conv/convolution.py:56) work.
+ * `inverse` swaps the roles of the two pair planes (indice_conv.h:307,330).
+ * `subm` is accepted for signature parity; the centre offset is treated like
+ * any other offset.  pair_num stays on the device: no host synchronisation.
+ * Every row of out[n_out,Cout] is written (zeros where no pair lands).
+ * ---------------------------------------------------------------------- */
+size_t ssc_conv_workspace_bytes(int64_t n_out, int32_t kernel_volume, int32_t c_in,
+                                int32_t c_out, int64_t pair_stride);
+
+int ssc_conv_fwd_f32(const float *features /* [n_in,c_in] */, int64_t n_in, int32_t c_in,
+                     const float *filters, int64_t fs_k, int64_t fs_ci, int64_t fs_co,
+                     int32_t c_out, const int32_t *pairs /* [K,2,pair_stride] */,
+                     int64_t pair_stride, const int32_t *pair_num /* [K] device */,
+                     int32_t kernel_volume, int32_t inverse, int32_t subm,
+                     float *out /* [n_out,c_out] */, int64_t n_out, void *workspace,
+                     size_t workspace_bytes, ssc_stream_t stream);
+
+/* ------------------------------------------------------------------------
+ * Steerable kernel synthesis.  Replaces SE3Kernel.combination
+ * (ss_conv/utils/kernel.py:267-299: one einsum "uvb,bijxyz->uivjxyz" per pair
+ * of irreps, two torch.cat) fused with the permute of
+ * ss_conv/convolution.py:56: writes the dense kernel directly as contiguous
+ * out[K,c_in,c_out].
+ *   chan_out[c_out,3] : (irrep index i, multiplicity index u, component a)
+ *   chan_in [c_in ,3] : (irrep index j, multiplicity index v, component b)
+ *   blocks[n_i*n_j,6] : (weight offset, basis offset, n_beta, m_in, d_out, d_in),
+ *                       n_beta = 0 for an absent block (zeros, kernel.py:287-291)
+ *   basis             : all kernel_i_j buffers [n_beta,d_out,d_in,K] concatenated
+ * ---------------------------------------------------------------------- */
+int ssc_kernel_combine_f32(const float *weight, const float *basis,
+                           const int32_t *chan_out, const int32_t *chan_in,
+                           const int32_t *blocks, int32_t n_irreps_in,
+                           int32_t kernel_volume, int32_t c_in, int32_t c_out,
+                           float *out /* [K,c_in,c_out] */, ssc_stream_t stream);
+
+/* ------------------------------------------------------------------------
+ * Rulebook pooling.  Replace indiceMaxPool<float> (src/pool/indice_maxpool.h:15-50,
+ * kernels src/pool/indice_maxpool_cuda_functor.cu:22-156), indiceAvgPool<float>
+ * (src/pool/indice_avgpool.h:17-52, kernels src/pool/indice_avgpool_cuda_functor.cu:21-171)
+ * and indiceSummaryRF (src/ss_conv_ops.cu:116-145, src/pool/indiceSummaryRF.cu:21-36).
+ *   max: out[o,c] = max(0, max_{(i,o)} features[i,c])      (output starts at 0, indice_maxpool.h:24)
+ *   avg: out[o,c] = sum_{k ascending} features[i_k,c] / (float)summaryrf[o]
+ *   rf : rf[o]    = number of pairs that target o
+ * One output-stationary launch over all offsets instead of one launch per offset.
+ * ---------------------------------------------------------------------- */
+size_t ssc_pool_workspace_bytes(int64_t n_out, int32_t kernel_volume);
+
+int ssc_pool_max_f32(const float *features, int32_t channels, const int32_t *pairs,
+                     int64_t pair_stride, const int32_t *pair_num, int32_t kernel_volume,
+                     float *out, int64_t n_out, void *workspace, size_t workspace_bytes,
+                     ssc_stream_t stream);
+
+int ssc_pool_avg_f32(const float *features, int32_t channels, const int32_t *pairs,
+                     int64_t pair_stride, const int32_t *pair_num, int32_t kernel_volume,
+                     const int32_t *summaryrf /* [n_out] */, float *out, int64_t n_out,
+                     void *workspace, size_t workspace_bytes, ssc_stream_t stream);
+
+int ssc_summary_rf(const int32_t *pairs, int64_t pair_stride, const int32_t *pair_num,
+                   int32_t kernel_volume, int32_t *rf /* [n_out] */, int64_t n_out,
+                   void *workspace, size_t workspace_bytes, ssc_stream_t stream);
+
+/* ------------------------------------------------------------------------
+ * Segment ("global") pooling over row ranges offsets[s]..offsets[s+1].
+ * Replace global_avgpool_fp / global_maxpool_fp (src/pool/global_avgpool.cpp:13-20,
+ * src/pool/global_avgpool_cuda_kernel.cu:16-42, src/pool/global_maxpool_cuda_kernel.cu:16-43).
+ *   avg: sum of the segment's rows divided by its length (empty segment: 0/0 = NaN)
+ *   max: maximum and the row index of its first occurrence (empty: -inf, -1)
+ * ---------------------------------------------------------------------- */
+int ssc_segment_avg_f32(const float *feats /* [sum_n,c] */, const int32_t *offsets /* [b+1] */,
+                        float *out /* [b,c] */, int32_t n_segments, int32_t channels,
+                        ssc_stream_t stream);
+
+int ssc_segment_max_f32(const float *feats, const int32_t *offsets, float *out,
+                        int32_t *out_idx /* [b,c] */, int32_t n_segments, int32_t channels,
+                        ssc_stream_t stream);
+
+/* ------------------------------------------------------------------------
+ * Point <-> voxel.
+ * ssc_voxel_coords: voxel index of each point, (int)((p + half) / unit) in fp32
+ *   with IEEE division and truncation (ss_conv/sp_ops/voxelize.py:85-86).
+ * ssc_unique_*: sorted unique rows of an int32 [n,4] (b,x,y,z) table with the
+ *   inverse map and counts; stands in for torch.unique(dim=0, return_inverse,
+ *   return_counts) at voxelize.py:88.  count SYNCHRONISES `stream`.
+ *   Coordinates must satisfy 0 <= b < dims[0], 0 <= x < dims[1], ... and
+ *   prod(dims) < 2^31.
+ * ssc_voxel_map: replaces voxel2point_map (src/voxelize/voxel2point.cpp:12-18,
+ *   src/voxelize/voxel2point_cuda_kernel.cu:16-42).  out_maps must be
+ *   pre-initialised as the reference's caller does (functional.py:344-349).
+ *   Modes 3/4 list the points of a voxel in ascending point order (the
+ *   reference leaves the order to an atomic race).
+ * ssc_voxel_reduce_f32: replaces voxelize_fp (src/voxelize/voxelize_cuda_kernel.h:18-40):
+ *   out[v,c] = sum_i mult * feats[map[v,i],c], mult = 1/count in mode 4 else 1.
+ *   Every row of out is written.
+ * ssc_three_nn / ssc_three_interp_f32: replace three_nn / three_interpolate_fp
+ *   (src/voxelize/interpolation.cpp, src/voxelize/interpolate_cuda_kernel.cu:8-121).
+ *   Rows are (b,x,y,z) floats; a known row counts only for queries with the
+ *   same b; ties keep the lower index; dist2 holds squared distances.
+ * ---------------------------------------------------------------------- */
+int ssc_voxel_coords(const float *points /* [n,3] */, const int64_t *batch_ids /* [n] */,
+                     int64_t n, const float half_extent[3], const float unit[3],
+                     int32_t *coords /* [n,4] */, ssc_stream_t stream);
+
+size_t ssc_unique_workspace_bytes(const int32_t dims[4], int64_t n);
+
+int ssc_unique_count(const int32_t *coords /* [n,4] */, int64_t n, const int32_t dims[4],
+                     void *workspace, size_t workspace_bytes, int32_t *n_unique_host,
+                     ssc_stream_t stream);
+
+int ssc_unique_emit(const int32_t *coords, int64_t n, const int32_t dims[4], void *workspace,
+                    size_t workspace_bytes, int64_t n_unique, int32_t *unique /* [m,4] */,
+                    int32_t *inverse /* [n] */, int32_t *counts /* [m]; may be NULL */,
+                    ssc_stream_t stream);
+
+int ssc_voxel_map(const int32_t *inverse /* [n] */, const int32_t *ids /* [n] */,
+                  int32_t *out_maps /* [m,max_active+1] */, int32_t n_point, int32_t n_voxel,
+                  int32_t max_active, int32_t mode, ssc_stream_t stream);
+
+int ssc_voxel_reduce_f32(const float *feats /* [n,c] */, float *out /* [m,c] */,
+                         const int32_t *maps /* [m,max_active+1] */, int32_t mode,
+                         int32_t n_voxel, int32_t max_active, int32_t channels,
+                         ssc_stream_t stream);
+
+int ssc_three_nn(int32_t n, int32_t m, const float *unknown /* [n,4] */,
+                 const float *known /* [m,4] */, float *dist2 /* [n,3] */,
+                 int32_t *idx /* [n,3] */, ssc_stream_t stream);
+
+int ssc_three_interp_f32(int32_t c, int32_t m, int32_t n, const float *feats /* [m,c] */,
+                         const int32_t *idx /* [n,3] */, const float *weight /* [n,3] */,
+                         float *out /* [n,c] */, ssc_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SSC_H_ */

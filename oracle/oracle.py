@@ -1,0 +1,462 @@
+"""CPU oracle for the sparse steerable convolution hot path.
+
+TEST INFRASTRUCTURE, NOT PRODUCT CODE.  Only tests/, __graft_entry__.smoke()
+and bench.py's cpu_baseline leg may import this module; the product package
+never does.
+
+Every function restates the reference algorithm in NumPy on top of the scalar
+C routines of ssc_oracle.c and cites the reference file:line it follows
+(paths relative to the reference's SS_Conv_lib/).  When oracle/_ref/libssc_ref.so
+is present (the reference's own CPU sources, compiled by oracle/Makefile) the
+``ref_*`` functions call it; tests use them to pin the restatement.
+
+Pinning status (what each function is checked against, see tests/test_oracle_*.py):
+  rulebook_conv / rulebook_subm   reference CPU build (_ref), committed golden
+                                  vectors, brute-force definition, invariants
+  conv_fwd                        torch.nn.functional.conv3d closed form; _ref gather/scatter
+  maxpool_fwd                     F.max_pool3d(relu(dense)); _ref functor
+  avgpool_fwd                     F.avg_pool3d(count_include_pad=True)
+  segment_avg / segment_max       numpy reductions
+  point2voxel                     np.unique(axis=0) semantics, per-voxel means, invariants
+  three_nn / three_interp         brute force with argsort on tiny inputs
+  combine                         torch.einsum on the same buffers (library routine)
+"""
+import ctypes
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_ORACLE_SO = os.path.join(_HERE, "_build", "libssc_oracle.so")
+_REF_SO = os.path.join(_HERE, "_ref", "libssc_ref.so")
+
+_ip = ctypes.POINTER(ctypes.c_int)
+_fp = ctypes.POINTER(ctypes.c_float)
+
+
+def build(force=False):
+    """Compile the checker libraries with oracle/Makefile (gcc only)."""
+    import subprocess
+    args = ["make", "-C", _HERE, "-j3"]
+    if force:
+        args.insert(1, "-B")
+    subprocess.run(args, check=True, stdout=subprocess.PIPE, stderr=subprocess.STDOUT)
+
+
+def _load(path):
+    return ctypes.CDLL(path) if os.path.exists(path) else None
+
+
+_lib = None
+_ref = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_ORACLE_SO):
+            build()
+        _lib = ctypes.CDLL(_ORACLE_SO)
+    return _lib
+
+
+def ref_lib():
+    """The compiled reference CPU code, or None when it was never built."""
+    global _ref
+    if _ref is None and os.path.exists(_REF_SO):
+        try:
+            import torch  # noqa: F401  (libc10 must be resolvable)
+        except Exception:
+            pass
+        _ref = ctypes.CDLL(_REF_SO)
+    return _ref
+
+
+def _i(a):
+    return a.ctypes.data_as(_ip)
+
+
+def _f(a):
+    return a.ctypes.data_as(_fp)
+
+
+def _i32(a):
+    return np.ascontiguousarray(a, dtype=np.int32)
+
+
+def _f32(a):
+    return np.ascontiguousarray(a, dtype=np.float32)
+
+
+def _triple(v):
+    if isinstance(v, (list, tuple, np.ndarray)):
+        assert len(v) == 3
+        return [int(x) for x in v]
+    return [int(v)] * 3
+
+
+# ---------------------------------------------------------------------------
+# geometry
+# ---------------------------------------------------------------------------
+def conv_output_size(in_shape, ksize, stride, padding, dilation):
+    """ss_conv/sp_ops/ops.py:13-23."""
+    out = []
+    for i in range(len(in_shape)):
+        size = (in_shape[i] + 2 * padding[i] - dilation[i] * (ksize[i] - 1) - 1) // stride[i] + 1
+        out.append(1 if ksize[i] == -1 else size)
+    return out
+
+
+def flat_key(idx, shape):
+    """((b*X+x)*Y+y)*Z+z, utils/tensorview.h:457-468 plus the batch term of
+    src/conv/indice_cuda_functor.cu:60-61."""
+    idx = np.asarray(idx, dtype=np.int64)
+    return ((idx[:, 0] * shape[0] + idx[:, 1]) * shape[1] + idx[:, 2]) * shape[2] + idx[:, 3]
+
+
+# ---------------------------------------------------------------------------
+# rulebook
+# ---------------------------------------------------------------------------
+def _rulebook(fn_conv, fn_subm, indices, batch_size, in_shape, ksize, stride, padding, dilation,
+              subm, need_grid):
+    indices = _i32(indices)
+    n = indices.shape[0]
+    ks, st, pd, dl = _triple(ksize), _triple(stride), _triple(padding), _triple(dilation)
+    if subm:  # src/conv/indice_conv.h:70-74
+        st, pd = [1, 1, 1], [k // 2 for k in ks]
+        out_shape = list(in_shape)
+    else:
+        out_shape = conv_output_size(list(in_shape), ks, st, pd, dl)
+    K = ks[0] * ks[1] * ks[2]
+    pairs = np.full((K, 2, n), -1, dtype=np.int32)
+    num = np.zeros(K, dtype=np.int32)
+    a = [_i32(x) for x in (ks, st, pd, dl, out_shape)]
+    grid = None
+    if need_grid:
+        grid = np.full(batch_size * int(np.prod(out_shape)), -1, dtype=np.int32)
+    if subm:
+        args = [_i(indices), n, batch_size] + [_i(x) for x in a]
+        if need_grid:
+            args.append(_i(grid))
+        n_out = fn_subm(*args, _i(pairs), _i(num))
+        out_idx = indices.copy()
+    else:
+        out_idx = np.zeros((max(n * K, 1), 4), dtype=np.int32)
+        args = [_i(indices), n, batch_size] + [_i(x) for x in a] + [_i(out_idx)]
+        if need_grid:
+            args.append(_i(grid))
+        n_out = fn_conv(*args, _i(pairs), _i(num))
+        out_idx = out_idx[:n_out].copy()
+    assert n_out >= 0
+    return out_idx, pairs, num, out_shape
+
+
+def rulebook(indices, batch_size, in_shape, ksize, stride=1, padding=0, dilation=1, subm=False):
+    """CPU rulebook of the reference (first-touch output numbering):
+    src/conv/geometry.h:140-189 (regular), 241-288 (submanifold), driven as in
+    src/conv/indice_conv.h:21-131.  Returns (out_indices, pairs[K,2,N], num[K], out_shape)."""
+    L = lib()
+    return _rulebook(L.orc_rulebook_conv, L.orc_rulebook_subm, indices, batch_size, in_shape,
+                     ksize, stride, padding, dilation, subm, need_grid=False)
+
+
+def ref_rulebook(indices, batch_size, in_shape, ksize, stride=1, padding=0, dilation=1,
+                 subm=False):
+    """Same call into the compiled reference sources (oracle/_ref)."""
+    R = ref_lib()
+    assert R is not None, "oracle/_ref/libssc_ref.so not built"
+    return _rulebook(R.ref_rulebook_conv, R.ref_rulebook_subm, indices, batch_size, in_shape,
+                     ksize, stride, padding, dilation, subm, need_grid=True)
+
+
+def canonicalize(out_idx, pairs, num, out_shape):
+    """Canonical rulebook order: outputs ascending by flat key (the reference's
+    GPU order, src/conv/indice_conv.h:120), pairs of an offset ascending by
+    input row (the reference's CPU order, src/conv/geometry.h:166-186)."""
+    key = flat_key(out_idx, out_shape)
+    order = np.argsort(key, kind="stable")
+    rank = np.empty_like(order)
+    rank[order] = np.arange(order.size)
+    new_pairs = np.full_like(pairs, -1)
+    for k in range(pairs.shape[0]):
+        n = int(num[k])
+        if n == 0:
+            continue
+        i = pairs[k, 0, :n]
+        o = rank[pairs[k, 1, :n]]
+        s = np.argsort(i, kind="stable")
+        new_pairs[k, 0, :n] = i[s]
+        new_pairs[k, 1, :n] = o[s]
+    return out_idx[order].copy(), new_pairs, num.copy()
+
+
+# ---------------------------------------------------------------------------
+# conv / pool over a rulebook
+# ---------------------------------------------------------------------------
+def conv_fwd(features, filters, pairs, num, n_out, inverse=False, matmul=None):
+    """src/conv/indice_conv.h:247-343, CPU branch: for every non-empty offset
+    gather rows (reordering_cpp_functor.cpp:15-24), GEMM (torch::mm_out, :320)
+    and scatter-add (reordering_cpp_functor.cpp:26-44), offsets ascending.
+    filters is [K, Cin, Cout].  matmul=None uses the scalar C GEMM; pass
+    np.matmul for a BLAS GEMM (what torch::mm is on a CPU)."""
+    L = lib()
+    features = _f32(features)
+    filters = _f32(filters)
+    K, cin, cout = filters.shape
+    out = np.zeros((n_out, cout), dtype=np.float32)
+    for k in range(K):
+        n = int(num[k])
+        if n <= 0:
+            continue
+        rows_g = _i32(pairs[k, 1 if inverse else 0, :n])
+        rows_s = _i32(pairs[k, 0 if inverse else 1, :n])
+        buf = np.empty((n, cin), dtype=np.float32)
+        L.orc_gather_rows(_f(buf), _f(features), _i(rows_g), n, cin)
+        if matmul is None:
+            obuf = np.empty((n, cout), dtype=np.float32)
+            L.orc_mm_f32(_f(obuf), _f(buf), _f(filters[k]), n, cin, cout)
+        else:
+            obuf = _f32(matmul(buf, filters[k]))
+        L.orc_scatter_add_rows(_f(out), _f(obuf), _i(rows_s), n, cout)
+    return out
+
+
+def ref_gather_scatter_conv(features, filters, pairs, num, n_out):
+    """conv_fwd with the reference's own compiled gather / scatter functors and
+    a NumPy GEMM in place of torch::mm."""
+    R = ref_lib()
+    features = _f32(features)
+    filters = _f32(filters)
+    K, cin, cout = filters.shape
+    out = np.zeros((n_out, cout), dtype=np.float32)
+    for k in range(K):
+        n = int(num[k])
+        if n <= 0:
+            continue
+        buf = np.empty((n, cin), dtype=np.float32)
+        R.ref_gather_rows(_f(buf), n, _f(features), features.shape[0], cin,
+                          _i(_i32(pairs[k, 0, :n])), n)
+        obuf = _f32(buf @ filters[k])
+        R.ref_scatter_add_rows(_f(out), n_out, _f(obuf), n, cout, _i(_i32(pairs[k, 1, :n])), n)
+    return out
+
+
+def maxpool_fwd(features, pairs, num, n_out):
+    """src/pool/indice_maxpool.h:15-50 with the CPU functor
+    src/pool/indice_maxpool_cpp_functor.cpp:16-35 (output zero-initialised)."""
+    L = lib()
+    features = _f32(features)
+    c = features.shape[1]
+    out = np.zeros((n_out, c), dtype=np.float32)
+    for k in range(pairs.shape[0]):
+        n = int(num[k])
+        if n > 0:
+            L.orc_maxpool_offset(_f(out), _f(features), _i(_i32(pairs[k, 0, :n])),
+                                 _i(_i32(pairs[k, 1, :n])), n, c)
+    return out
+
+
+def ref_maxpool_fwd(features, pairs, num, n_out):
+    R = ref_lib()
+    features = _f32(features)
+    pairs = _i32(pairs)
+    c = features.shape[1]
+    out = np.zeros((n_out, c), dtype=np.float32)
+    stride = pairs.shape[2]
+    for k in range(pairs.shape[0]):
+        n = int(num[k])
+        if n > 0:
+            R.ref_maxpool_offset(_f(out), n_out, _f(features), features.shape[0], c,
+                                 _i(pairs[k]), stride, n)
+    return out
+
+
+def summary_rf(pairs, num, n_out):
+    """src/ss_conv_ops.cu:116-145 + src/pool/indiceSummaryRF.cu:21-36."""
+    L = lib()
+    rf = np.zeros(n_out, dtype=np.int32)
+    for k in range(pairs.shape[0]):
+        n = int(num[k])
+        if n > 0:
+            L.orc_summary_rf_offset(_i(rf), _i(_i32(pairs[k, 1, :n])), n)
+    return rf
+
+
+def avgpool_fwd(features, pairs, num, n_out, rf=None):
+    """ss_conv/sp_ops/functional.py:162-185 (rf = kernel volume when use_gs)
+    + src/pool/indice_avgpool.h:17-52 with the arithmetic of the CUDA kernel
+    src/pool/indice_avgpool_cuda_functor.cu:159-161."""
+    L = lib()
+    features = _f32(features)
+    c = features.shape[1]
+    if rf is None:
+        rf = np.full(n_out, pairs.shape[0], dtype=np.int32)
+    rf = _i32(rf)
+    out = np.zeros((n_out, c), dtype=np.float32)
+    for k in range(pairs.shape[0]):
+        n = int(num[k])
+        if n > 0:
+            L.orc_avgpool_offset(_f(out), _f(features), _i(_i32(pairs[k, 0, :n])),
+                                 _i(_i32(pairs[k, 1, :n])), n, c, _i(rf))
+    return out
+
+
+def segment_avg(feats, offsets):
+    """src/pool/global_avgpool_cuda_kernel.cu:16-34."""
+    feats, offsets = _f32(feats), _i32(offsets)
+    out = np.zeros((offsets.size - 1, feats.shape[1]), dtype=np.float32)
+    with np.errstate(all="ignore"):
+        lib().orc_segment_avg(_f(feats), _i(offsets), _f(out), offsets.size - 1, feats.shape[1])
+    return out
+
+
+def segment_max(feats, offsets):
+    """src/pool/global_maxpool_cuda_kernel.cu:16-35.  Returns (max, argmax)."""
+    feats, offsets = _f32(feats), _i32(offsets)
+    out = np.zeros((offsets.size - 1, feats.shape[1]), dtype=np.float32)
+    idx = np.zeros(out.shape, dtype=np.int32)
+    lib().orc_segment_max(_f(feats), _i(offsets), _f(out), _i(idx), offsets.size - 1,
+                          feats.shape[1])
+    return out, idx
+
+
+# ---------------------------------------------------------------------------
+# point <-> voxel
+# ---------------------------------------------------------------------------
+def voxel_map(inverse, n_voxel, max_active, mode=4):
+    """ss_conv/sp_ops/functional.py:329-355 + src/voxelize/voxel2point_cuda_kernel.cu:16-37."""
+    inverse = _i32(inverse).reshape(-1)
+    n = inverse.size
+    ids = np.arange(n, dtype=np.int32)
+    if mode in (3, 4):
+        maps = np.zeros((n_voxel, max_active + 1), dtype=np.int32)
+    elif mode == 2:
+        maps = np.full((n_voxel, max_active + 1), -1, dtype=np.int32)
+    elif mode == 1:
+        maps = np.full((n_voxel, max_active + 1), n, dtype=np.int32)
+    else:
+        raise AssertionError
+    lib().orc_voxel_map(_i(inverse), _i(ids), _i(maps), n, max_active, mode)
+    return maps
+
+
+def voxel_reduce(feats, maps, mode=4):
+    """ss_conv/sp_ops/functional.py:297-316 + src/voxelize/voxelize_cuda_kernel.h:18-32."""
+    feats, maps = _f32(feats), _i32(maps)
+    out = np.zeros((maps.shape[0], feats.shape[1]), dtype=np.float32)
+    lib().orc_voxel_reduce(_f(feats), _f(out), _i(maps), mode, maps.shape[0], maps.shape[1] - 1,
+                           feats.shape[1])
+    return out
+
+
+def point2voxel(points, feats, batch_ids, voxel_num_limit, unit_voxel_extent, mode=4):
+    """ss_conv/sp_ops/voxelize.py:29-99.  Returns a dict with valid_points,
+    valid_feats, valid_ids, flag, indices[M,4], inverse, counts, maps, features[M,C].
+    The batch sort is stable (the reference's torch.sort leaves ties unspecified)."""
+    points = _f32(points)
+    feats = _f32(feats)
+    ids = np.asarray(batch_ids, dtype=np.int64)
+    C = feats.shape[1]
+    unit = np.asarray(unit_voxel_extent, dtype=np.float64).astype(np.float32).reshape(1, 3)
+    limit = np.asarray(voxel_num_limit).astype(np.float32).reshape(1, 3)
+    total = limit * unit
+    half = np.float32(0.5) * total
+    uniq_ids = np.unique(ids)
+    B1 = uniq_ids.size
+    ok = (np.abs(points) > half).sum(1) == 0
+    if ok.sum() == 0:
+        flag = np.zeros(B1, dtype=np.float32)
+        vp = np.zeros((B1, 3), dtype=np.float32)
+        vf = np.zeros((B1, C), dtype=np.float32)
+        vi = uniq_ids
+    else:
+        vp, vf, vi = points[ok], feats[ok], ids[ok]
+        uv = np.unique(vi)
+        if uv.size == B1:
+            flag = np.ones(B1, dtype=np.float32)
+        else:
+            flag = np.isin(uniq_ids, uv).astype(np.float32)
+            missing = uniq_ids[flag == 0]
+            vp = np.concatenate([vp, np.zeros((missing.size, 3), np.float32)])
+            vf = np.concatenate([vf, np.zeros((missing.size, C), np.float32)])
+            vi = np.concatenate([vi, missing])
+        order = np.argsort(vi, kind="stable")
+        vp, vf, vi = vp[order], vf[order], vi[order]
+    vox = ((vp + half) / unit).astype(np.int32)  # fp32 add, fp32 divide, truncate
+    table = np.concatenate([vi.astype(np.int32)[:, None], vox], axis=1)
+    uniq, inverse, counts = np.unique(table, axis=0, return_inverse=True, return_counts=True)
+    inverse = inverse.reshape(-1)
+    max_active = 1 if mode in (1, 2) else int(counts.max())
+    maps = voxel_map(inverse, uniq.shape[0], max_active, mode)
+    out = voxel_reduce(vf, maps, mode)
+    return dict(valid_points=vp, valid_feats=vf, valid_ids=vi, flag=flag,
+                indices=uniq.astype(np.int32), inverse=inverse.astype(np.int32),
+                counts=counts.astype(np.int32), maps=maps, features=out, batch_size=B1)
+
+
+def three_nn(unknown, known):
+    """ss_conv/sp_ops/functional.py:361-384 + src/voxelize/interpolate_cuda_kernel.cu:8-55.
+    Returns (sqrt(dist2), idx)."""
+    unknown, known = _f32(unknown), _f32(known)
+    n, m = unknown.shape[0], known.shape[0]
+    d2 = np.zeros((n, 3), dtype=np.float32)
+    idx = np.zeros((n, 3), dtype=np.int32)
+    lib().orc_three_nn(n, m, _f(unknown), _f(known), _f(d2), _i(idx))
+    with np.errstate(all="ignore"):
+        return np.sqrt(d2), idx
+
+
+def three_interp(feats, idx, weight):
+    """src/voxelize/interpolate_cuda_kernel.cu:79-101."""
+    feats, idx, weight = _f32(feats), _i32(idx), _f32(weight)
+    out = np.zeros((idx.shape[0], feats.shape[1]), dtype=np.float32)
+    lib().orc_three_interp(feats.shape[1], feats.shape[0], idx.shape[0], _f(feats), _i(idx),
+                           _f(weight), _f(out))
+    return out
+
+
+def voxel2point(indices, features, spatial_shape, points, batch_ids, voxel_extent=None,
+                unit_voxel_extent=None):
+    """ss_conv/sp_ops/voxelize.py:110-162: voxel centres, 3-NN, inverse-distance
+    weights, interpolation."""
+    shape = np.asarray(spatial_shape, dtype=np.float64)
+    if voxel_extent is not None:
+        unit = (np.asarray(voxel_extent, np.float64) / shape).astype(np.float32)
+        ext = np.asarray(voxel_extent, np.float64).astype(np.float32)
+    else:
+        unit = np.asarray(unit_voxel_extent, np.float64).astype(np.float32)
+        ext = (np.asarray(unit_voxel_extent, np.float64) * shape).astype(np.float32)
+    centres = np.asarray(indices).astype(np.float32)
+    centres[:, 1:] = centres[:, 1:] * unit - np.float32(0.5) * ext + np.float32(0.5) * unit
+    target = np.concatenate([np.asarray(batch_ids).astype(np.float32)[:, None], _f32(points)], 1)
+    dist, idx = three_nn(target, centres)
+    recip = np.float32(1.0) / (dist + np.float32(1e-8))
+    weight = recip / recip.sum(1, keepdims=True)
+    return three_interp(features, idx, weight), idx, weight
+
+
+# ---------------------------------------------------------------------------
+# steerable kernel synthesis
+# ---------------------------------------------------------------------------
+def combine(weight, bases, mults_out, dims_out, mults_in, dims_in, size):
+    """ss_conv/utils/kernel.py:267-299.  bases[i][j] is the [n_beta,d_o,d_i,k,k,k]
+    buffer kernel_i_j or None.  Returns the dense kernel [Cout,Cin,k,k,k]."""
+    weight = np.asarray(weight, dtype=np.float32)
+    off = 0
+    rows = []
+    for i, mi in enumerate(mults_out):
+        cols = []
+        for j, mj in enumerate(mults_in):
+            kij = bases[i][j]
+            if kij is not None:
+                nb = kij.shape[0]
+                w = weight[off:off + mi * mj * nb].reshape(mi, mj, nb)
+                off += mi * mj * nb
+                ker = np.einsum("uvb,bijxyz->uivjxyz", w, np.asarray(kij, np.float32))
+                ker = ker.reshape(mi * dims_out[i], mj * dims_in[j], size, size, size)
+            else:
+                ker = np.zeros((mi * dims_out[i], mj * dims_in[j], size, size, size), np.float32)
+            cols.append(ker)
+        rows.append(np.concatenate(cols, axis=1))
+    assert off == weight.size
+    return np.concatenate(rows, axis=0).astype(np.float32)

@@ -1,0 +1,157 @@
+// Error reporting, fill kernels and the popcount scan shared by the rulebook,
+// voxel-unique and pair re-ordering paths.
+#include "ssc_common.h"
+
+#include <string.h>
+
+namespace ssc {
+
+static thread_local char g_error[512] = "";
+
+int fail(int code, const char *fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_error, sizeof(g_error), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+__global__ void fill_i32_kernel(int32_t *__restrict__ p, int64_t n, int32_t v) {
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  int64_t step = (int64_t)gridDim.x * blockDim.x;
+  for (; i < n; i += step) p[i] = v;
+}
+
+int fill_i32(int32_t *p, int64_t n, int32_t v, hipStream_t s) {
+  if (n <= 0) return SSC_OK;
+  int blocks = (int)(ceil_div(n, 256) < 8192 ? ceil_div(n, 256) : 8192);
+  hipLaunchKernelGGL(fill_i32_kernel, dim3(blocks), dim3(256), 0, s, p, n, v);
+  SSC_LAUNCH_CHECK("fill_i32");
+  return SSC_OK;
+}
+
+int fill_f32(float *p, int64_t n, float v, hipStream_t s) {
+  int32_t bits;
+  memcpy(&bits, &v, sizeof(bits));
+  return fill_i32(reinterpret_cast<int32_t *>(p), n, bits, s);
+}
+
+size_t bit_table_bytes(int64_t n_bits) {
+  int64_t w = bit_words(n_bits);
+  int64_t nb = ceil_div(w, kScanBlockWords);
+  return align_up(w * 4) * 2 + align_up((nb + 1) * 4) + align_up(4);
+}
+
+BitTable bit_table_carve(Carver &c, int64_t n_bits) {
+  BitTable t;
+  t.n_words = bit_words(n_bits);
+  t.n_scan_blocks = ceil_div(t.n_words, kScanBlockWords);
+  t.bits = c.take<uint32_t>(t.n_words);
+  t.prefix = c.take<int32_t>(t.n_words);
+  t.blocksum = c.take<int32_t>(t.n_scan_blocks + 1);
+  t.total = c.take<int32_t>(1);
+  return t;
+}
+
+int bit_table_clear(const BitTable &t, hipStream_t s) {
+  return fill_i32(reinterpret_cast<int32_t *>(t.bits), t.n_words, 0, s);
+}
+
+// Block-wide exclusive scan of one int per thread (kScanThreads threads).
+__device__ __forceinline__ int block_exclusive_scan(int v, int *lds /* [kScanThreads/64 + 1] */,
+                                                    int *block_total) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  int incl = v;
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    int o = __shfl_up(incl, d, 64);
+    if (lane >= d) incl += o;
+  }
+  if (lane == 63) lds[wave] = incl;
+  __syncthreads();
+  int wave_off = 0, tot = 0;
+#pragma unroll
+  for (int w = 0; w < kScanThreads / 64; ++w) {
+    int x = lds[w];
+    if (w < wave) wave_off += x;
+    tot += x;
+  }
+  __syncthreads();
+  *block_total = tot;
+  return wave_off + incl - v;
+}
+
+// Pass 1: popcount sum of each block of kScanBlockWords words.
+__global__ void __launch_bounds__(kScanThreads)
+    popc_blocksum_kernel(const uint32_t *__restrict__ bits, int64_t n_words,
+                         int32_t *__restrict__ blocksum) {
+  __shared__ int lds[kScanThreads / 64 + 1];
+  int64_t base = (int64_t)blockIdx.x * kScanBlockWords + (int64_t)threadIdx.x * kScanItems;
+  int v = 0;
+#pragma unroll
+  for (int i = 0; i < kScanItems; ++i)
+    if (base + i < n_words) v += __popc(bits[base + i]);
+  int tot;
+  block_exclusive_scan(v, lds, &tot);
+  if (threadIdx.x == 0) blocksum[blockIdx.x] = tot;
+}
+
+// Pass 2: one block turns blocksum[] into its exclusive prefix and writes the total.
+__global__ void __launch_bounds__(kScanThreads)
+    popc_blockscan_kernel(int32_t *__restrict__ blocksum, int64_t n_blocks,
+                          int32_t *__restrict__ total) {
+  __shared__ int lds[kScanThreads / 64 + 1];
+  int carry = 0;
+  for (int64_t base = 0; base < n_blocks; base += kScanThreads) {
+    int64_t i = base + threadIdx.x;
+    int v = i < n_blocks ? blocksum[i] : 0;
+    int tot;
+    int ex = block_exclusive_scan(v, lds, &tot);
+    if (i < n_blocks) blocksum[i] = carry + ex;
+    carry += tot;
+  }
+  if (threadIdx.x == 0) total[0] = carry;
+}
+
+// Pass 3: exclusive prefix per word.
+__global__ void __launch_bounds__(kScanThreads)
+    popc_prefix_kernel(const uint32_t *__restrict__ bits, int64_t n_words,
+                       const int32_t *__restrict__ blocksum, int32_t *__restrict__ prefix) {
+  __shared__ int lds[kScanThreads / 64 + 1];
+  int64_t base = (int64_t)blockIdx.x * kScanBlockWords + (int64_t)threadIdx.x * kScanItems;
+  int c[kScanItems];
+  int v = 0;
+#pragma unroll
+  for (int i = 0; i < kScanItems; ++i) {
+    c[i] = base + i < n_words ? __popc(bits[base + i]) : 0;
+    v += c[i];
+  }
+  int tot;
+  int ex = block_exclusive_scan(v, lds, &tot) + blocksum[blockIdx.x];
+#pragma unroll
+  for (int i = 0; i < kScanItems; ++i) {
+    if (base + i < n_words) prefix[base + i] = ex;
+    ex += c[i];
+  }
+}
+
+int bit_table_scan(const BitTable &t, hipStream_t s) {
+  if (t.n_words <= 0) return fill_i32(t.total, 1, 0, s);
+  hipLaunchKernelGGL(popc_blocksum_kernel, dim3((unsigned)t.n_scan_blocks), dim3(kScanThreads), 0,
+                     s, t.bits, t.n_words, t.blocksum);
+  SSC_LAUNCH_CHECK("popc_blocksum");
+  hipLaunchKernelGGL(popc_blockscan_kernel, dim3(1), dim3(kScanThreads), 0, s, t.blocksum,
+                     t.n_scan_blocks, t.total);
+  SSC_LAUNCH_CHECK("popc_blockscan");
+  hipLaunchKernelGGL(popc_prefix_kernel, dim3((unsigned)t.n_scan_blocks), dim3(kScanThreads), 0, s,
+                     t.bits, t.n_words, t.blocksum, t.prefix);
+  SSC_LAUNCH_CHECK("popc_prefix");
+  return SSC_OK;
+}
+
+}  // namespace ssc
+
+extern "C" {
+int ssc_version(void) { return 100; }
+const char *ssc_last_error(void) { return ssc::g_error; }
+}

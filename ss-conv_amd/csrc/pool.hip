@@ -1,0 +1,261 @@
+// Rulebook max / average pooling and segment (global) pooling.
+//
+// Rulebook pooling is output stationary: the pair lists are first transposed
+// into an [n_out, K] table of input rows (-1 = no pair), then every output row
+// is produced once, visiting its inputs in ascending offset order -- the order
+// in which the reference's per-offset launches touch it.  Input rows are read
+// once, output rows written once, no atomics on features.
+#include "ssc_common.h"
+
+// Products and sums below are rounded separately, as the scalar statements of the
+// reference are: no fused multiply-add contraction in this file.
+#pragma clang fp contract(off)
+
+#include <math.h>
+
+namespace ssc {
+
+typedef float float4v __attribute__((ext_vector_type(4)));
+
+__global__ void __launch_bounds__(256)
+    pair_table_kernel(const int32_t *__restrict__ pairs, int64_t pair_stride,
+                      const int32_t *__restrict__ pair_num, int K, int32_t *__restrict__ table) {
+  int k = blockIdx.y;
+  int64_t j = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (j >= pair_num[k]) return;
+  const int32_t *p = pairs + (int64_t)k * 2 * pair_stride;
+  int64_t o = p[pair_stride + j];
+  table[o * K + k] = p[j];
+}
+
+__global__ void __launch_bounds__(256)
+    pair_count_kernel(const int32_t *__restrict__ pairs, int64_t pair_stride,
+                      const int32_t *__restrict__ pair_num, int32_t *__restrict__ rf) {
+  int k = blockIdx.y;
+  int64_t j = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (j >= pair_num[k]) return;
+  atomicAdd(&rf[pairs[((int64_t)k * 2 + 1) * pair_stride + j]], 1);  // integer: exact
+}
+
+// MODE 0: max with zero start (out = max(0, inputs));  MODE 1: sum of in / (float)rf.
+// VEC = 4 when C % 4 == 0 (16-byte accesses), else 1.
+template <int MODE, int VEC>
+__global__ void __launch_bounds__(256)
+    pool_kernel(const float *__restrict__ in, int C, const int32_t *__restrict__ table, int K,
+                const int32_t *__restrict__ rf, float *__restrict__ out, int64_t n_out) {
+  const int cv = C / VEC;
+  int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= n_out * cv) return;
+  int64_t o = idx / cv;
+  int c = (int)(idx - o * cv) * VEC;
+  float acc[VEC];
+#pragma unroll
+  for (int v = 0; v < VEC; ++v) acc[v] = 0.f;
+  float div = 1.f;
+  if (MODE == 1) div = (float)rf[o];
+  const int32_t *t = table + o * K;
+  for (int k = 0; k < K; ++k) {
+    int64_t i = t[k];
+    if (i < 0) continue;
+    float x[VEC];
+    if (VEC == 4) {
+      float4v q = *reinterpret_cast<const float4v *>(in + i * C + c);
+      x[0] = q.x; x[1 % VEC] = q.y; x[2 % VEC] = q.z; x[3 % VEC] = q.w;
+    } else {
+      x[0] = in[i * C + c];
+    }
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) {
+      if (MODE == 0) {
+        if (acc[v] < x[v]) acc[v] = x[v];
+      } else {
+        acc[v] = acc[v] + x[v] / div;
+      }
+    }
+  }
+  if (VEC == 4) {
+    float4v q = {acc[0], acc[1 % VEC], acc[2 % VEC], acc[3 % VEC]};
+    *reinterpret_cast<float4v *>(out + o * C + c) = q;
+  } else {
+    out[o * C + c] = acc[0];
+  }
+}
+
+// Segment pooling: grid (segment, channel block of 64); 16 row lanes x 64
+// channels per block; partial results combined in a fixed order.
+constexpr int kSegRows = 16;
+
+template <bool IS_MAX>
+__global__ void __launch_bounds__(kSegRows * 64)
+    segment_pool_kernel(const float *__restrict__ feats, const int32_t *__restrict__ offsets,
+                        float *__restrict__ out, int32_t *__restrict__ out_idx, int C) {
+  __shared__ float sval[kSegRows][64];
+  __shared__ int sidx[kSegRows][64];
+  const int seg = blockIdx.x;
+  const int cl = threadIdx.x & 63;
+  const int rl = threadIdx.x >> 6;
+  const int c = blockIdx.y * 64 + cl;
+  const int a = offsets[seg], b = offsets[seg + 1];
+  float v = IS_MAX ? -INFINITY : 0.f;
+  int arg = -1;
+  if (c < C) {
+    for (int i = a + rl; i < b; i += kSegRows) {
+      float x = feats[(int64_t)i * C + c];
+      if (IS_MAX) {
+        if (x > v) { v = x; arg = i; }
+      } else {
+        v += x;
+      }
+    }
+  }
+  sval[rl][cl] = v;
+  sidx[rl][cl] = arg;
+  __syncthreads();
+  if (rl == 0 && c < C) {
+#pragma unroll
+    for (int r = 1; r < kSegRows; ++r) {
+      float x = sval[r][cl];
+      if (IS_MAX) {
+        int xi = sidx[r][cl];
+        // first occurrence wins: larger value, or equal value at a lower row
+        if (x > v || (x == v && xi >= 0 && (arg < 0 || xi < arg))) { v = x; arg = xi; }
+      } else {
+        v += x;
+      }
+    }
+    if (IS_MAX) {
+      out[(int64_t)seg * C + c] = v;
+      out_idx[(int64_t)seg * C + c] = arg;
+    } else {
+      out[(int64_t)seg * C + c] = v / (float)(b - a);
+    }
+  }
+}
+
+static int pool_common(const float *features, int channels, const int32_t *pairs,
+                       int64_t pair_stride, const int32_t *pair_num, int K, float *out,
+                       int64_t n_out, void *ws, size_t ws_bytes, hipStream_t s,
+                       int32_t **table_out) {
+  SSC_CHECK(K >= 1 && K <= SSC_MAX_KERNEL_VOLUME, SSC_ERUNTIME, "kernel volume %d out of range", K);
+  SSC_CHECK(channels >= 1 && n_out >= 0 && pair_stride >= 0, SSC_EINVAL, "bad sizes");
+  if (n_out == 0) return SSC_OK;
+  SSC_CHECK(features && pairs && pair_num && out && ws, SSC_EINVAL, "NULL pointer argument");
+  SSC_CHECK(ws_bytes >= align_up((size_t)n_out * K * 4), SSC_EWORKSPACE,
+            "pool workspace too small");
+  int32_t *table = static_cast<int32_t *>(ws);
+  int rc = fill_i32(table, n_out * K, -1, s);
+  if (rc != SSC_OK) return rc;
+  if (pair_stride > 0) {
+    hipLaunchKernelGGL(pair_table_kernel, dim3((unsigned)ceil_div(pair_stride, 256), (unsigned)K),
+                       dim3(256), 0, s, pairs, pair_stride, pair_num, K, table);
+    SSC_LAUNCH_CHECK("pair_table");
+  }
+  *table_out = table;
+  return SSC_OK;
+}
+
+}  // namespace ssc
+
+using namespace ssc;
+
+extern "C" {
+
+size_t ssc_pool_workspace_bytes(int64_t n_out, int32_t kernel_volume) {
+  if (n_out < 0 || kernel_volume < 1) return 0;
+  return align_up((size_t)(n_out > 0 ? n_out : 1) * kernel_volume * 4);
+}
+
+int ssc_pool_max_f32(const float *features, int32_t channels, const int32_t *pairs,
+                     int64_t pair_stride, const int32_t *pair_num, int32_t kernel_volume,
+                     float *out, int64_t n_out, void *workspace, size_t workspace_bytes,
+                     ssc_stream_t stream) {
+  hipStream_t s = (hipStream_t)stream;
+  int32_t *table = nullptr;
+  int rc = pool_common(features, channels, pairs, pair_stride, pair_num, kernel_volume, out, n_out,
+                       workspace, workspace_bytes, s, &table);
+  if (rc != SSC_OK || n_out == 0) return rc;
+  if ((channels & 3) == 0) {
+    int64_t n = n_out * (channels / 4);
+    hipLaunchKernelGGL((pool_kernel<0, 4>), dim3((unsigned)ceil_div(n, 256)), dim3(256), 0, s,
+                       features, channels, table, kernel_volume, (const int32_t *)nullptr, out,
+                       n_out);
+  } else {
+    int64_t n = n_out * channels;
+    hipLaunchKernelGGL((pool_kernel<0, 1>), dim3((unsigned)ceil_div(n, 256)), dim3(256), 0, s,
+                       features, channels, table, kernel_volume, (const int32_t *)nullptr, out,
+                       n_out);
+  }
+  SSC_LAUNCH_CHECK("pool_max");
+  return SSC_OK;
+}
+
+int ssc_pool_avg_f32(const float *features, int32_t channels, const int32_t *pairs,
+                     int64_t pair_stride, const int32_t *pair_num, int32_t kernel_volume,
+                     const int32_t *summaryrf, float *out, int64_t n_out, void *workspace,
+                     size_t workspace_bytes, ssc_stream_t stream) {
+  hipStream_t s = (hipStream_t)stream;
+  SSC_CHECK(n_out == 0 || summaryrf != nullptr, SSC_EINVAL, "summaryrf is NULL");
+  int32_t *table = nullptr;
+  int rc = pool_common(features, channels, pairs, pair_stride, pair_num, kernel_volume, out, n_out,
+                       workspace, workspace_bytes, s, &table);
+  if (rc != SSC_OK || n_out == 0) return rc;
+  if ((channels & 3) == 0) {
+    int64_t n = n_out * (channels / 4);
+    hipLaunchKernelGGL((pool_kernel<1, 4>), dim3((unsigned)ceil_div(n, 256)), dim3(256), 0, s,
+                       features, channels, table, kernel_volume, summaryrf, out, n_out);
+  } else {
+    int64_t n = n_out * channels;
+    hipLaunchKernelGGL((pool_kernel<1, 1>), dim3((unsigned)ceil_div(n, 256)), dim3(256), 0, s,
+                       features, channels, table, kernel_volume, summaryrf, out, n_out);
+  }
+  SSC_LAUNCH_CHECK("pool_avg");
+  return SSC_OK;
+}
+
+int ssc_summary_rf(const int32_t *pairs, int64_t pair_stride, const int32_t *pair_num,
+                   int32_t kernel_volume, int32_t *rf, int64_t n_out, void *workspace,
+                   size_t workspace_bytes, ssc_stream_t stream) {
+  (void)workspace;
+  (void)workspace_bytes;
+  hipStream_t s = (hipStream_t)stream;
+  SSC_CHECK(kernel_volume >= 1 && kernel_volume <= SSC_MAX_KERNEL_VOLUME, SSC_ERUNTIME,
+            "kernel volume out of range");
+  if (n_out == 0) return SSC_OK;
+  SSC_CHECK(pairs && pair_num && rf, SSC_EINVAL, "NULL pointer argument");
+  int rc = fill_i32(rf, n_out, 0, s);
+  if (rc != SSC_OK) return rc;
+  if (pair_stride > 0) {
+    hipLaunchKernelGGL(pair_count_kernel,
+                       dim3((unsigned)ceil_div(pair_stride, 256), (unsigned)kernel_volume),
+                       dim3(256), 0, s, pairs, pair_stride, pair_num, rf);
+    SSC_LAUNCH_CHECK("pair_count");
+  }
+  return SSC_OK;
+}
+
+int ssc_segment_avg_f32(const float *feats, const int32_t *offsets, float *out,
+                        int32_t n_segments, int32_t channels, ssc_stream_t stream) {
+  SSC_CHECK(n_segments >= 0 && channels >= 1, SSC_EINVAL, "bad sizes");
+  if (n_segments == 0) return SSC_OK;
+  SSC_CHECK(feats && offsets && out, SSC_EINVAL, "NULL pointer argument");
+  hipLaunchKernelGGL(segment_pool_kernel<false>,
+                     dim3((unsigned)n_segments, (unsigned)ceil_div(channels, 64)),
+                     dim3(kSegRows * 64), 0, (hipStream_t)stream, feats, offsets, out,
+                     (int32_t *)nullptr, channels);
+  SSC_LAUNCH_CHECK("segment_avg");
+  return SSC_OK;
+}
+
+int ssc_segment_max_f32(const float *feats, const int32_t *offsets, float *out, int32_t *out_idx,
+                        int32_t n_segments, int32_t channels, ssc_stream_t stream) {
+  SSC_CHECK(n_segments >= 0 && channels >= 1, SSC_EINVAL, "bad sizes");
+  if (n_segments == 0) return SSC_OK;
+  SSC_CHECK(feats && offsets && out && out_idx, SSC_EINVAL, "NULL pointer argument");
+  hipLaunchKernelGGL(segment_pool_kernel<true>,
+                     dim3((unsigned)n_segments, (unsigned)ceil_div(channels, 64)),
+                     dim3(kSegRows * 64), 0, (hipStream_t)stream, feats, offsets, out, out_idx,
+                     channels);
+  SSC_LAUNCH_CHECK("segment_max");
+  return SSC_OK;
+}
+}

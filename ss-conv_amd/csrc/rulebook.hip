@@ -1,0 +1,431 @@
+// Rulebook (indice pair) generation and sorted-unique of voxel coordinates.
+//
+// Both are "number a set of grid cells in ascending flat-key order" problems.
+// The set is held as a bit table over the dense key space (1 bit per cell:
+// 32x smaller than the reference's int32 grid, L2/MALL resident at the sizes
+// this path sees) and a popcount prefix turns membership into the rank of the
+// key, i.e. the output row.  No sort, no probing, no result-bearing atomics:
+// atomicOr on the bit table is order independent.
+#include "ssc_common.h"
+
+namespace ssc {
+
+struct Geom {
+  int batch;
+  int os[3], ks[3], st[3], pd[3], dl[3];
+  int K;
+  int subm;
+};
+
+static int make_geom(const ssc_geometry *g, Geom *o) {
+  SSC_CHECK(g != nullptr, SSC_EINVAL, "geometry is NULL");
+  SSC_CHECK(g->transpose == 0, SSC_EINVAL, "transposed rulebooks are not supported");
+  o->batch = g->batch_size;
+  o->subm = g->subm != 0;
+  o->K = 1;
+  for (int a = 0; a < 3; ++a) {
+    o->os[a] = g->out_shape[a];
+    o->ks[a] = g->ksize[a];
+    o->dl[a] = g->dilation[a];
+    if (o->subm) {  // src/conv/indice_conv.h:70-74
+      o->st[a] = 1;
+      o->pd[a] = g->ksize[a] / 2;
+    } else {
+      o->st[a] = g->stride[a];
+      o->pd[a] = g->padding[a];
+    }
+    SSC_CHECK(o->ks[a] >= 1 && o->st[a] >= 1 && o->dl[a] >= 1 && o->pd[a] >= 0 && o->os[a] >= 1,
+              SSC_EINVAL, "bad geometry in dimension %d", a);
+    SSC_CHECK(o->st[a] == 1 || o->dl[a] == 1, SSC_EINVAL,
+              "stride > 1 together with dilation > 1 is not supported");
+    o->K *= o->ks[a];
+  }
+  SSC_CHECK(o->K <= SSC_MAX_KERNEL_VOLUME, SSC_ERUNTIME, "kernel volume %d exceeds %d", o->K,
+            SSC_MAX_KERNEL_VOLUME);
+  SSC_CHECK(o->batch >= 1, SSC_EINVAL, "batch_size must be positive");
+  int64_t cells = (int64_t)o->batch * o->os[0] * o->os[1] * o->os[2];
+  SSC_CHECK(cells < ((int64_t)1 << 31), SSC_ERUNTIME,
+            "batch_size * prod(out_shape) = %lld does not fit 31 bits", (long long)cells);
+  return SSC_OK;
+}
+
+static inline int64_t geom_cells(const Geom &g) {
+  return (int64_t)g.batch * g.os[0] * g.os[1] * g.os[2];
+}
+
+// Output position reached from input coordinate `in` through kernel tap `k` in
+// one dimension: (in + p - k*d) / s when that is a non-negative multiple of s
+// and inside the output extent.  Equivalent to the candidate enumeration of
+// src/conv/geometry.h:18-80 (stride>1 with dilation>1 is rejected on the host).
+__device__ __forceinline__ bool tap_to_out(int in, int k, int s, int p, int d, int extent,
+                                           int *out) {
+  int t = in + p - k * d;
+  if (t < 0) return false;
+  int q = t / s;
+  if (q * s != t || q >= extent) return false;
+  *out = q;
+  return true;
+}
+
+__device__ __forceinline__ bool pair_key(const Geom &g, const int32_t *__restrict__ row, int k,
+                                         uint32_t *key) {
+  int kz = k % g.ks[2];
+  int ky = (k / g.ks[2]) % g.ks[1];
+  int kx = k / (g.ks[2] * g.ks[1]);
+  int ox, oy, oz;
+  if (!tap_to_out(row[1], kx, g.st[0], g.pd[0], g.dl[0], g.os[0], &ox)) return false;
+  if (!tap_to_out(row[2], ky, g.st[1], g.pd[1], g.dl[1], g.os[1], &oy)) return false;
+  if (!tap_to_out(row[3], kz, g.st[2], g.pd[2], g.dl[2], g.os[2], &oz)) return false;
+  *key = (uint32_t)(((row[0] * g.os[0] + ox) * g.os[1] + oy) * g.os[2] + oz);
+  return true;
+}
+
+// Regular conv: mark every output cell reachable from an active input.
+// One thread per (input row, tap).
+__global__ void __launch_bounds__(256)
+    mark_outputs_kernel(const int32_t *__restrict__ indices, int64_t n_in, Geom g,
+                        uint32_t *__restrict__ bits) {
+  int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= n_in * g.K) return;
+  int64_t i = t / g.K;
+  int k = (int)(t - i * g.K);
+  int32_t row[4];
+  *reinterpret_cast<int4 *>(row) = reinterpret_cast<const int4 *>(indices)[i];
+  uint32_t key;
+  if (pair_key(g, row, k, &key)) atomicOr(&bits[key >> 5], 1u << (key & 31u));
+}
+
+// Submanifold / unique: mark the cells of the rows themselves.
+__global__ void __launch_bounds__(256)
+    mark_rows_kernel(const int32_t *__restrict__ coords, int64_t n, int d1, int d2, int d3,
+                     uint32_t *__restrict__ bits) {
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  int4 r = reinterpret_cast<const int4 *>(coords)[i];
+  uint32_t key = (uint32_t)(((r.x * d1 + r.y) * d2 + r.z) * d3 + r.w);
+  atomicOr(&bits[key >> 5], 1u << (key & 31u));
+}
+
+// Decode every set bit into its (b,x,y,z) row, written at the bit's rank.
+__global__ void __launch_bounds__(256)
+    emit_rows_kernel(const uint32_t *__restrict__ bits, const int32_t *__restrict__ prefix,
+                     int64_t n_words, int d1, int d2, int d3, int32_t *__restrict__ out) {
+  int64_t w = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (w >= n_words) return;
+  uint32_t b = bits[w];
+  if (b == 0) return;
+  int r = prefix[w];
+  while (b) {
+    int bit = __ffs(b) - 1;
+    b &= b - 1;
+    uint32_t key = (uint32_t)(w * 32 + bit);
+    int z = key % d3;
+    key /= d3;
+    int y = key % d2;
+    key /= d2;
+    int x = key % d1;
+    int bb = key / d1;
+    reinterpret_cast<int4 *>(out)[r++] = make_int4(bb, x, y, z);
+  }
+}
+
+// rank -> input row, for the submanifold rulebook (outputs keep the input numbering).
+__global__ void __launch_bounds__(256)
+    rank_to_row_kernel(const int32_t *__restrict__ indices, int64_t n_in, Geom g,
+                       const uint32_t *__restrict__ bits, const int32_t *__restrict__ prefix,
+                       int32_t *__restrict__ rank2row) {
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n_in) return;
+  int4 r = reinterpret_cast<const int4 *>(indices)[i];
+  uint32_t key = (uint32_t)(((r.x * g.os[0] + r.y) * g.os[1] + r.z) * g.os[2] + r.w);
+  rank2row[bit_rank(bits, prefix, key)] = (int32_t)i;
+}
+
+__device__ __forceinline__ bool bit_test(const uint32_t *__restrict__ bits, uint32_t key) {
+  return (bits[key >> 5] >> (key & 31u)) & 1u;
+}
+
+// Pair counting: one wave per chunk of 64 input rows, per tap the number of
+// rows of the chunk that own a pair.  chunk_count is [K, n_chunks].
+__global__ void __launch_bounds__(256)
+    count_pairs_kernel(const int32_t *__restrict__ indices, int64_t n_in, Geom g,
+                       const uint32_t *__restrict__ bits, int32_t *__restrict__ chunk_count,
+                       int64_t n_chunks) {
+  int64_t chunk = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (chunk >= n_chunks) return;
+  int lane = threadIdx.x & 63;
+  int64_t i = chunk * 64 + lane;
+  bool live = i < n_in;
+  int32_t row[4] = {0, 0, 0, 0};
+  if (live) *reinterpret_cast<int4 *>(row) = reinterpret_cast<const int4 *>(indices)[i];
+  for (int k = 0; k < g.K; ++k) {
+    uint32_t key;
+    bool ok = live && pair_key(g, row, k, &key);
+    if (ok && g.subm) ok = bit_test(bits, key);
+    unsigned long long m = __ballot(ok);
+    if (lane == 0) chunk_count[(int64_t)k * n_chunks + chunk] = __popcll(m);
+  }
+}
+
+// Per tap: exclusive scan of the chunk counts in place; the total is pair_num[k].
+__global__ void __launch_bounds__(kScanThreads)
+    scan_chunks_kernel(int32_t *__restrict__ chunk_count, int64_t n_chunks,
+                       int32_t *__restrict__ pair_num) {
+  __shared__ int lds[kScanThreads / 64 + 1];
+  int32_t *c = chunk_count + (int64_t)blockIdx.x * n_chunks;
+  int carry = 0;
+  for (int64_t base = 0; base < n_chunks; base += kScanThreads) {
+    int64_t i = base + threadIdx.x;
+    int v = i < n_chunks ? c[i] : 0;
+    // inline block scan (same shape as common.hip's)
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    int incl = v;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      int o = __shfl_up(incl, d, 64);
+      if (lane >= d) incl += o;
+    }
+    if (lane == 63) lds[wave] = incl;
+    __syncthreads();
+    int wave_off = 0, tot = 0;
+#pragma unroll
+    for (int w = 0; w < kScanThreads / 64; ++w) {
+      int x = lds[w];
+      if (w < wave) wave_off += x;
+      tot += x;
+    }
+    __syncthreads();
+    if (i < n_chunks) c[i] = carry + wave_off + incl - v;
+    carry += tot;
+  }
+  if (threadIdx.x == 0) pair_num[blockIdx.x] = carry;
+}
+
+// Pair emission: same traversal as count_pairs_kernel; a row's slot inside tap k
+// is (pairs of earlier chunks) + (earlier lanes of this chunk), which makes the
+// pair list ascending in input row.  The wave also pads slots [num, n_in) of
+// its own 64-slot window with -1.
+__global__ void __launch_bounds__(256)
+    write_pairs_kernel(const int32_t *__restrict__ indices, int64_t n_in, Geom g,
+                       const uint32_t *__restrict__ bits, const int32_t *__restrict__ prefix,
+                       const int32_t *__restrict__ rank2row,
+                       const int32_t *__restrict__ chunk_prefix, int64_t n_chunks,
+                       const int32_t *__restrict__ pair_num, int32_t *__restrict__ pairs) {
+  int64_t chunk = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (chunk >= n_chunks) return;
+  int lane = threadIdx.x & 63;
+  int64_t i = chunk * 64 + lane;
+  bool live = i < n_in;
+  int32_t row[4] = {0, 0, 0, 0};
+  if (live) *reinterpret_cast<int4 *>(row) = reinterpret_cast<const int4 *>(indices)[i];
+  for (int k = 0; k < g.K; ++k) {
+    uint32_t key = 0;
+    bool ok = live && pair_key(g, row, k, &key);
+    if (ok && g.subm) ok = bit_test(bits, key);
+    unsigned long long m = __ballot(ok);
+    int32_t *pin = pairs + ((int64_t)k * 2 + 0) * n_in;
+    int32_t *pout = pairs + ((int64_t)k * 2 + 1) * n_in;
+    if (ok) {
+      int slot = chunk_prefix[(int64_t)k * n_chunks + chunk] +
+                 __popcll(m & ((1ull << lane) - 1ull));
+      int r = bit_rank(bits, prefix, key);
+      if (g.subm) r = rank2row[r];
+      pin[slot] = (int32_t)i;
+      pout[slot] = r;
+    }
+    if (live && i >= pair_num[k]) {
+      pin[i] = -1;
+      pout[i] = -1;
+    }
+  }
+}
+
+// inverse[i] = rank of row i's cell; counts[rank] += 1 (integer atomics: exact).
+__global__ void __launch_bounds__(256)
+    inverse_counts_kernel(const int32_t *__restrict__ coords, int64_t n, int d1, int d2, int d3,
+                          const uint32_t *__restrict__ bits, const int32_t *__restrict__ prefix,
+                          int32_t *__restrict__ inverse, int32_t *__restrict__ counts) {
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  int4 r = reinterpret_cast<const int4 *>(coords)[i];
+  uint32_t key = (uint32_t)(((r.x * d1 + r.y) * d2 + r.z) * d3 + r.w);
+  int rk = bit_rank(bits, prefix, key);
+  inverse[i] = rk;
+  if (counts) atomicAdd(&counts[rk], 1);
+}
+
+struct RulebookWs {
+  BitTable table;
+  int32_t *chunk_count;  // [K, n_chunks]
+  int32_t *rank2row;     // [n_in] (subm)
+  int64_t n_chunks;
+};
+
+static size_t rulebook_ws_bytes(const Geom &g, int64_t n_in) {
+  int64_t n_chunks = ceil_div(n_in > 0 ? n_in : 1, 64);
+  return bit_table_bytes(geom_cells(g)) + align_up((size_t)g.K * n_chunks * 4) +
+         align_up((size_t)(n_in > 0 ? n_in : 1) * 4);
+}
+
+static RulebookWs rulebook_ws_carve(void *ws, const Geom &g, int64_t n_in) {
+  Carver c(ws);
+  RulebookWs w;
+  w.table = bit_table_carve(c, geom_cells(g));
+  w.n_chunks = ceil_div(n_in > 0 ? n_in : 1, 64);
+  w.chunk_count = c.take<int32_t>((size_t)g.K * w.n_chunks);
+  w.rank2row = c.take<int32_t>(n_in > 0 ? n_in : 1);
+  return w;
+}
+
+}  // namespace ssc
+
+using namespace ssc;
+
+extern "C" {
+
+size_t ssc_rulebook_workspace_bytes(const ssc_geometry *g, int64_t n_in) {
+  Geom gg;
+  if (make_geom(g, &gg) != SSC_OK) return 0;
+  return rulebook_ws_bytes(gg, n_in);
+}
+
+int ssc_rulebook_count(const int32_t *indices, int64_t n_in, const ssc_geometry *g,
+                       void *workspace, size_t workspace_bytes, int32_t *n_out_host,
+                       ssc_stream_t stream) {
+  Geom gg;
+  int rc = make_geom(g, &gg);
+  if (rc != SSC_OK) return rc;
+  SSC_CHECK(n_out_host != nullptr, SSC_EINVAL, "n_out_host is NULL");
+  SSC_CHECK(n_in >= 0, SSC_EINVAL, "n_in is negative");
+  SSC_CHECK(n_in * gg.K < ((int64_t)1 << 40), SSC_EINVAL, "n_in * kernel volume too large");
+  if (n_in == 0) {  // src/conv/indice_cuda_functor.cu:262-263
+    *n_out_host = 0;
+    return SSC_OK;
+  }
+  SSC_CHECK(indices != nullptr && workspace != nullptr, SSC_EINVAL, "NULL pointer argument");
+  SSC_CHECK(workspace_bytes >= rulebook_ws_bytes(gg, n_in), SSC_EWORKSPACE,
+            "rulebook workspace too small: %zu < %zu", workspace_bytes,
+            rulebook_ws_bytes(gg, n_in));
+  hipStream_t s = (hipStream_t)stream;
+  RulebookWs w = rulebook_ws_carve(workspace, gg, n_in);
+  if ((rc = bit_table_clear(w.table, s)) != SSC_OK) return rc;
+  if (gg.subm) {
+    hipLaunchKernelGGL(mark_rows_kernel, dim3((unsigned)ceil_div(n_in, 256)), dim3(256), 0, s,
+                       indices, n_in, gg.os[0], gg.os[1], gg.os[2], w.table.bits);
+    SSC_LAUNCH_CHECK("mark_rows");
+  } else {
+    hipLaunchKernelGGL(mark_outputs_kernel, dim3((unsigned)ceil_div(n_in * gg.K, 256)), dim3(256),
+                       0, s, indices, n_in, gg, w.table.bits);
+    SSC_LAUNCH_CHECK("mark_outputs");
+  }
+  if ((rc = bit_table_scan(w.table, s)) != SSC_OK) return rc;
+  int32_t total = 0;
+  SSC_HIP(hipMemcpyAsync(&total, w.table.total, sizeof(int32_t), hipMemcpyDeviceToHost, s));
+  SSC_HIP(hipStreamSynchronize(s));
+  *n_out_host = gg.subm ? (int32_t)n_in : total;
+  return SSC_OK;
+}
+
+int ssc_rulebook_emit(const int32_t *indices, int64_t n_in, const ssc_geometry *g,
+                      void *workspace, size_t workspace_bytes, int32_t *out_indices,
+                      int32_t *pairs, int32_t *pair_num, ssc_stream_t stream) {
+  Geom gg;
+  int rc = make_geom(g, &gg);
+  if (rc != SSC_OK) return rc;
+  hipStream_t s = (hipStream_t)stream;
+  SSC_CHECK(pair_num != nullptr, SSC_EINVAL, "pair_num is NULL");
+  if (n_in == 0) return fill_i32(pair_num, gg.K, 0, s);
+  SSC_CHECK(indices != nullptr && workspace != nullptr && pairs != nullptr, SSC_EINVAL,
+            "NULL pointer argument");
+  SSC_CHECK(gg.subm || out_indices != nullptr, SSC_EINVAL, "out_indices is NULL");
+  SSC_CHECK(workspace_bytes >= rulebook_ws_bytes(gg, n_in), SSC_EWORKSPACE,
+            "rulebook workspace too small");
+  RulebookWs w = rulebook_ws_carve(workspace, gg, n_in);
+  unsigned chunk_blocks = (unsigned)ceil_div(w.n_chunks, 4);
+  if (gg.subm) {
+    hipLaunchKernelGGL(rank_to_row_kernel, dim3((unsigned)ceil_div(n_in, 256)), dim3(256), 0, s,
+                       indices, n_in, gg, w.table.bits, w.table.prefix, w.rank2row);
+    SSC_LAUNCH_CHECK("rank_to_row");
+  } else {
+    hipLaunchKernelGGL(emit_rows_kernel, dim3((unsigned)ceil_div(w.table.n_words, 256)),
+                       dim3(256), 0, s, w.table.bits, w.table.prefix, w.table.n_words, gg.os[0],
+                       gg.os[1], gg.os[2], out_indices);
+    SSC_LAUNCH_CHECK("emit_rows");
+  }
+  hipLaunchKernelGGL(count_pairs_kernel, dim3(chunk_blocks), dim3(256), 0, s, indices, n_in, gg,
+                     w.table.bits, w.chunk_count, w.n_chunks);
+  SSC_LAUNCH_CHECK("count_pairs");
+  hipLaunchKernelGGL(scan_chunks_kernel, dim3(gg.K), dim3(kScanThreads), 0, s, w.chunk_count,
+                     w.n_chunks, pair_num);
+  SSC_LAUNCH_CHECK("scan_chunks");
+  hipLaunchKernelGGL(write_pairs_kernel, dim3(chunk_blocks), dim3(256), 0, s, indices, n_in, gg,
+                     w.table.bits, w.table.prefix, w.rank2row, w.chunk_count, w.n_chunks, pair_num,
+                     pairs);
+  SSC_LAUNCH_CHECK("write_pairs");
+  return SSC_OK;
+}
+
+size_t ssc_unique_workspace_bytes(const int32_t dims[4], int64_t n) {
+  (void)n;
+  int64_t cells = (int64_t)dims[0] * dims[1] * dims[2] * dims[3];
+  if (cells <= 0 || cells >= ((int64_t)1 << 31)) return 0;
+  return bit_table_bytes(cells);
+}
+
+static int unique_check(const int32_t dims[4], int64_t n, const void *ws, size_t ws_bytes,
+                        int64_t *cells) {
+  SSC_CHECK(dims != nullptr, SSC_EINVAL, "dims is NULL");
+  for (int a = 0; a < 4; ++a) SSC_CHECK(dims[a] >= 1, SSC_EINVAL, "dims[%d] must be positive", a);
+  *cells = (int64_t)dims[0] * dims[1] * dims[2] * dims[3];
+  SSC_CHECK(*cells < ((int64_t)1 << 31), SSC_ERUNTIME, "prod(dims) does not fit 31 bits");
+  SSC_CHECK(n >= 0, SSC_EINVAL, "n is negative");
+  SSC_CHECK(n == 0 || ws != nullptr, SSC_EINVAL, "workspace is NULL");
+  SSC_CHECK(n == 0 || ws_bytes >= bit_table_bytes(*cells), SSC_EWORKSPACE,
+            "unique workspace too small");
+  return SSC_OK;
+}
+
+int ssc_unique_count(const int32_t *coords, int64_t n, const int32_t dims[4], void *workspace,
+                     size_t workspace_bytes, int32_t *n_unique_host, ssc_stream_t stream) {
+  int64_t cells;
+  int rc = unique_check(dims, n, workspace, workspace_bytes, &cells);
+  if (rc != SSC_OK) return rc;
+  SSC_CHECK(n_unique_host != nullptr, SSC_EINVAL, "n_unique_host is NULL");
+  if (n == 0) {
+    *n_unique_host = 0;
+    return SSC_OK;
+  }
+  hipStream_t s = (hipStream_t)stream;
+  Carver c(workspace);
+  BitTable t = bit_table_carve(c, cells);
+  if ((rc = bit_table_clear(t, s)) != SSC_OK) return rc;
+  hipLaunchKernelGGL(mark_rows_kernel, dim3((unsigned)ceil_div(n, 256)), dim3(256), 0, s, coords,
+                     n, dims[1], dims[2], dims[3], t.bits);
+  SSC_LAUNCH_CHECK("mark_rows");
+  if ((rc = bit_table_scan(t, s)) != SSC_OK) return rc;
+  SSC_HIP(hipMemcpyAsync(n_unique_host, t.total, sizeof(int32_t), hipMemcpyDeviceToHost, s));
+  SSC_HIP(hipStreamSynchronize(s));
+  return SSC_OK;
+}
+
+int ssc_unique_emit(const int32_t *coords, int64_t n, const int32_t dims[4], void *workspace,
+                    size_t workspace_bytes, int64_t n_unique, int32_t *unique, int32_t *inverse,
+                    int32_t *counts, ssc_stream_t stream) {
+  int64_t cells;
+  int rc = unique_check(dims, n, workspace, workspace_bytes, &cells);
+  if (rc != SSC_OK) return rc;
+  if (n == 0) return SSC_OK;
+  SSC_CHECK(unique != nullptr && inverse != nullptr, SSC_EINVAL, "NULL output pointer");
+  hipStream_t s = (hipStream_t)stream;
+  Carver c(workspace);
+  BitTable t = bit_table_carve(c, cells);
+  if (counts && (rc = fill_i32(counts, n_unique, 0, s)) != SSC_OK) return rc;
+  hipLaunchKernelGGL(emit_rows_kernel, dim3((unsigned)ceil_div(t.n_words, 256)), dim3(256), 0, s,
+                     t.bits, t.prefix, t.n_words, dims[1], dims[2], dims[3], unique);
+  SSC_LAUNCH_CHECK("emit_rows");
+  hipLaunchKernelGGL(inverse_counts_kernel, dim3((unsigned)ceil_div(n, 256)), dim3(256), 0, s,
+                     coords, n, dims[1], dims[2], dims[3], t.bits, t.prefix, inverse, counts);
+  SSC_LAUNCH_CHECK("inverse_counts");
+  return SSC_OK;
+}
+}

@@ -1,0 +1,90 @@
+// Shared host/device helpers for the gfx950 kernels behind include/ssc.h.
+#ifndef SSC_COMMON_H_
+#define SSC_COMMON_H_
+
+#include <hip/hip_runtime.h>
+#include <stdarg.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include "ssc.h"
+
+namespace ssc {
+
+// Thread-local message returned by ssc_last_error().
+int fail(int code, const char *fmt, ...);
+
+#define SSC_CHECK(cond, code, ...)                        \
+  do {                                                    \
+    if (!(cond)) return ::ssc::fail((code), __VA_ARGS__); \
+  } while (0)
+
+#define SSC_HIP(expr)                                                                   \
+  do {                                                                                  \
+    hipError_t e__ = (expr);                                                            \
+    if (e__ != hipSuccess)                                                              \
+      return ::ssc::fail(SSC_EHIP, "%s failed: %s", #expr, hipGetErrorString(e__));     \
+  } while (0)
+
+#define SSC_LAUNCH_CHECK(name)                                                          \
+  do {                                                                                  \
+    hipError_t e__ = hipGetLastError();                                                 \
+    if (e__ != hipSuccess)                                                              \
+      return ::ssc::fail(SSC_EHIP, "launch of %s failed: %s", name, hipGetErrorString(e__)); \
+  } while (0)
+
+static inline size_t align_up(size_t x, size_t a = 256) { return (x + a - 1) / a * a; }
+static inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+// Carves 256-byte aligned regions out of a caller-provided workspace.
+struct Carver {
+  char *base;
+  size_t used;
+  explicit Carver(void *p) : base(static_cast<char *>(p)), used(0) {}
+  template <typename T> T *take(size_t count) {
+    T *p = reinterpret_cast<T *>(base + used);
+    used += align_up(count * sizeof(T));
+    return p;
+  }
+};
+
+// ---- rank/select over a bit table -------------------------------------------------------
+// A set of integer keys in [0, n_bits) is held as a bit table.  After
+// popcount_scan(), rank(key) = prefix[key >> 5] + popc(bits[key >> 5] below key)
+// numbers the keys in ascending order: a minimal perfect hash whose order is
+// the sorted order, so no sort and no probing are needed.
+constexpr int kScanThreads = 256;
+constexpr int kScanItems = 8;  // words per thread
+constexpr int kScanBlockWords = kScanThreads * kScanItems;
+
+struct BitTable {
+  uint32_t *bits;     // [n_words]
+  int32_t *prefix;    // [n_words] exclusive popcount prefix
+  int32_t *blocksum;  // [n_scan_blocks]
+  int32_t *total;     // [1]
+  int64_t n_words;
+  int64_t n_scan_blocks;
+};
+
+static inline int64_t bit_words(int64_t n_bits) { return ceil_div(n_bits, 32); }
+size_t bit_table_bytes(int64_t n_bits);
+BitTable bit_table_carve(Carver &c, int64_t n_bits);
+// Enqueue: zero the table.
+int bit_table_clear(const BitTable &t, hipStream_t s);
+// Enqueue: prefix[], total[0] from bits[].
+int bit_table_scan(const BitTable &t, hipStream_t s);
+
+__device__ __forceinline__ int bit_rank(const uint32_t *__restrict__ bits,
+                                        const int32_t *__restrict__ prefix, uint32_t key) {
+  uint32_t w = key >> 5;
+  uint32_t below = bits[w] & ((1u << (key & 31u)) - 1u);
+  return prefix[w] + __popc(below);
+}
+
+// Enqueue: fill an int32 array (a kernel, so the call may be graph-captured).
+int fill_i32(int32_t *p, int64_t n, int32_t v, hipStream_t s);
+int fill_f32(float *p, int64_t n, float v, hipStream_t s);
+
+}  // namespace ssc
+
+#endif

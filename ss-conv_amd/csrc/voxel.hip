@@ -1,0 +1,222 @@
+// Point <-> voxel kernels: voxel coordinates of points, per-voxel point lists,
+// per-voxel feature reduction, 3-nearest-neighbour search and interpolation.
+#include "ssc_common.h"
+
+// Products and sums below are rounded separately, as the scalar statements of the
+// reference are: no fused multiply-add contraction in this file.  (Plain operators
+// only: the __fmul_rn / __fadd_rn wrappers are compiled before this pragma and
+// would still be fused.)
+#pragma clang fp contract(off)
+
+#include <math.h>
+
+namespace ssc {
+
+typedef float float4v __attribute__((ext_vector_type(4)));
+
+// (int)((p + half) / unit) per axis: fp32 add, IEEE fp32 divide, truncation.
+__global__ void __launch_bounds__(256)
+    voxel_coords_kernel(const float *__restrict__ pts, const int64_t *__restrict__ ids, int64_t n,
+                        float hx, float hy, float hz, float ux, float uy, float uz,
+                        int32_t *__restrict__ coords) {
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  float x = pts[i * 3], y = pts[i * 3 + 1], z = pts[i * 3 + 2];
+  int vx = (int)((x + hx) / ux);
+  int vy = (int)((y + hy) / uy);
+  int vz = (int)((z + hz) / uz);
+  reinterpret_cast<int4 *>(coords)[i] = make_int4((int)ids[i], vx, vy, vz);
+}
+
+// Point lists.  Modes 3/4: slot by atomic counter (any order), then each list is
+// sorted by id so the result does not depend on the race.
+__global__ void __launch_bounds__(256)
+    voxel_map_kernel(const int32_t *__restrict__ inverse, const int32_t *__restrict__ ids,
+                     int32_t *__restrict__ maps, int n_point, int max_active, int mode) {
+  int r = blockIdx.x * blockDim.x + threadIdx.x;
+  if (r >= n_point) return;
+  int32_t *out = maps + (int64_t)inverse[r] * (max_active + 1);
+  int id = ids[r];
+  if (mode == 1) {
+    atomicMin(&out[1], id);
+    out[0] = 1;
+  } else if (mode == 2) {
+    atomicMax(&out[1], id);
+    out[0] = 1;
+  } else {
+    int slot = atomicAdd(&out[0], 1);
+    if (slot < max_active) out[slot + 1] = id;
+  }
+}
+
+__global__ void __launch_bounds__(256)
+    voxel_map_sort_kernel(int32_t *__restrict__ maps, int n_voxel, int max_active) {
+  int v = blockIdx.x * blockDim.x + threadIdx.x;
+  if (v >= n_voxel) return;
+  int32_t *row = maps + (int64_t)v * (max_active + 1);
+  int n = row[0];
+  if (n > max_active) n = max_active;
+  for (int i = 2; i <= n; ++i) {  // insertion sort of row[1..n]
+    int key = row[i];
+    int j = i - 1;
+    while (j >= 1 && row[j] > key) {
+      row[j + 1] = row[j];
+      --j;
+    }
+    row[j + 1] = key;
+  }
+}
+
+// out[v,c] = sum over the voxel's list of mult * feats[p,c]; the product is
+// rounded before the add, as an atomicAdd of a product is.
+__global__ void __launch_bounds__(256)
+    voxel_reduce_kernel(const float *__restrict__ feats, float *__restrict__ out,
+                        const int32_t *__restrict__ maps, int mode, int64_t n_voxel,
+                        int max_active, int C) {
+  int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= n_voxel * C) return;
+  int64_t v = idx / C;
+  int c = (int)(idx - v * C);
+  const int32_t *r = maps + v * (max_active + 1);
+  int na = r[0];
+  float mult = (mode == 4 && na > 0) ? 1.f / (float)na : 1.f;
+  float acc = 0.f;
+  for (int i = 1; i <= na; ++i) {
+    float t = mult * feats[(int64_t)r[i] * C + c];
+    acc = acc + t;
+  }
+  out[idx] = acc;
+}
+
+// Brute-force 3-NN: one thread per query, known rows streamed through LDS.
+constexpr int kNnTile = 256;
+
+__global__ void __launch_bounds__(kNnTile)
+    three_nn_kernel(int n, int m, const float *__restrict__ unknown,
+                    const float *__restrict__ known, float *__restrict__ dist2,
+                    int32_t *__restrict__ idx) {
+  __shared__ float4v tile[kNnTile];
+  int q = blockIdx.x * blockDim.x + threadIdx.x;
+  float4v u = {0.f, 0.f, 0.f, 0.f};
+  if (q < n) u = reinterpret_cast<const float4v *>(unknown)[q];
+  float b1 = INFINITY, b2 = INFINITY, b3 = INFINITY;
+  int i1 = 0, i2 = 0, i3 = 0;
+  for (int base = 0; base < m; base += kNnTile) {
+    int kk = base + threadIdx.x;
+    __syncthreads();
+    if (kk < m) tile[threadIdx.x] = reinterpret_cast<const float4v *>(known)[kk];
+    __syncthreads();
+    int cnt = min(kNnTile, m - base);
+    for (int t = 0; t < cnt; ++t) {
+      float4v p = tile[t];
+      if (p.x != u.x) continue;
+      float dx = u.y - p.y, dy = u.z - p.z, dz = u.w - p.w;
+      float xx = dx * dx, yy = dy * dy, zz = dz * dz;
+      float d = (xx + yy) + zz;
+      int k = base + t;
+      if (d < b1) {
+        b3 = b2; i3 = i2; b2 = b1; i2 = i1; b1 = d; i1 = k;
+      } else if (d < b2) {
+        b3 = b2; i3 = i2; b2 = d; i2 = k;
+      } else if (d < b3) {
+        b3 = d; i3 = k;
+      }
+    }
+  }
+  if (q < n) {
+    dist2[q * 3] = b1; dist2[q * 3 + 1] = b2; dist2[q * 3 + 2] = b3;
+    idx[q * 3] = i1; idx[q * 3 + 1] = i2; idx[q * 3 + 2] = i3;
+  }
+}
+
+// out[q,c] = (w0*f0 + w1*f1) + w2*f2, threads along c for coalesced rows.
+__global__ void __launch_bounds__(256)
+    three_interp_kernel(int C, int n, const float *__restrict__ feats,
+                        const int32_t *__restrict__ idx, const float *__restrict__ weight,
+                        float *__restrict__ out) {
+  int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (e >= (int64_t)n * C) return;
+  int64_t q = e / C;
+  int c = (int)(e - q * C);
+  float a = weight[q * 3] * feats[(int64_t)idx[q * 3] * C + c];
+  float b = weight[q * 3 + 1] * feats[(int64_t)idx[q * 3 + 1] * C + c];
+  float d = weight[q * 3 + 2] * feats[(int64_t)idx[q * 3 + 2] * C + c];
+  out[e] = (a + b) + d;
+}
+
+}  // namespace ssc
+
+using namespace ssc;
+
+extern "C" {
+
+int ssc_voxel_coords(const float *points, const int64_t *batch_ids, int64_t n,
+                     const float half_extent[3], const float unit[3], int32_t *coords,
+                     ssc_stream_t stream) {
+  SSC_CHECK(n >= 0, SSC_EINVAL, "n is negative");
+  if (n == 0) return SSC_OK;
+  SSC_CHECK(points && batch_ids && half_extent && unit && coords, SSC_EINVAL,
+            "NULL pointer argument");
+  hipLaunchKernelGGL(voxel_coords_kernel, dim3((unsigned)ceil_div(n, 256)), dim3(256), 0,
+                     (hipStream_t)stream, points, batch_ids, n, half_extent[0], half_extent[1],
+                     half_extent[2], unit[0], unit[1], unit[2], coords);
+  SSC_LAUNCH_CHECK("voxel_coords");
+  return SSC_OK;
+}
+
+int ssc_voxel_map(const int32_t *inverse, const int32_t *ids, int32_t *out_maps, int32_t n_point,
+                  int32_t n_voxel, int32_t max_active, int32_t mode, ssc_stream_t stream) {
+  SSC_CHECK(mode >= 1 && mode <= 4, SSC_EINVAL, "mode must be 1..4");
+  SSC_CHECK(n_point >= 0 && n_voxel >= 0 && max_active >= 1, SSC_EINVAL, "bad sizes");
+  if (n_point == 0) return SSC_OK;
+  SSC_CHECK(inverse && ids && out_maps, SSC_EINVAL, "NULL pointer argument");
+  hipStream_t s = (hipStream_t)stream;
+  hipLaunchKernelGGL(voxel_map_kernel, dim3((unsigned)ceil_div(n_point, 256)), dim3(256), 0, s,
+                     inverse, ids, out_maps, n_point, max_active, mode);
+  SSC_LAUNCH_CHECK("voxel_map");
+  if (mode >= 3 && n_voxel > 0) {
+    hipLaunchKernelGGL(voxel_map_sort_kernel, dim3((unsigned)ceil_div(n_voxel, 256)), dim3(256), 0,
+                       s, out_maps, n_voxel, max_active);
+    SSC_LAUNCH_CHECK("voxel_map_sort");
+  }
+  return SSC_OK;
+}
+
+int ssc_voxel_reduce_f32(const float *feats, float *out, const int32_t *maps, int32_t mode,
+                         int32_t n_voxel, int32_t max_active, int32_t channels,
+                         ssc_stream_t stream) {
+  SSC_CHECK(n_voxel >= 0 && max_active >= 1 && channels >= 1, SSC_EINVAL, "bad sizes");
+  if (n_voxel == 0) return SSC_OK;
+  SSC_CHECK(feats && out && maps, SSC_EINVAL, "NULL pointer argument");
+  int64_t n = (int64_t)n_voxel * channels;
+  hipLaunchKernelGGL(voxel_reduce_kernel, dim3((unsigned)ceil_div(n, 256)), dim3(256), 0,
+                     (hipStream_t)stream, feats, out, maps, mode, (int64_t)n_voxel, max_active,
+                     channels);
+  SSC_LAUNCH_CHECK("voxel_reduce");
+  return SSC_OK;
+}
+
+int ssc_three_nn(int32_t n, int32_t m, const float *unknown, const float *known, float *dist2,
+                 int32_t *idx, ssc_stream_t stream) {
+  SSC_CHECK(n >= 0 && m >= 0, SSC_EINVAL, "bad sizes");
+  if (n == 0) return SSC_OK;
+  SSC_CHECK(unknown && dist2 && idx && (m == 0 || known), SSC_EINVAL, "NULL pointer argument");
+  hipLaunchKernelGGL(three_nn_kernel, dim3((unsigned)ceil_div(n, kNnTile)), dim3(kNnTile), 0,
+                     (hipStream_t)stream, n, m, unknown, known, dist2, idx);
+  SSC_LAUNCH_CHECK("three_nn");
+  return SSC_OK;
+}
+
+int ssc_three_interp_f32(int32_t c, int32_t m, int32_t n, const float *feats, const int32_t *idx,
+                         const float *weight, float *out, ssc_stream_t stream) {
+  (void)m;
+  SSC_CHECK(c >= 1 && n >= 0, SSC_EINVAL, "bad sizes");
+  if (n == 0) return SSC_OK;
+  SSC_CHECK(feats && idx && weight && out, SSC_EINVAL, "NULL pointer argument");
+  int64_t e = (int64_t)n * c;
+  hipLaunchKernelGGL(three_interp_kernel, dim3((unsigned)ceil_div(e, 256)), dim3(256), 0,
+                     (hipStream_t)stream, c, n, feats, idx, weight, out);
+  SSC_LAUNCH_CHECK("three_interp");
+  return SSC_OK;
+}
+}

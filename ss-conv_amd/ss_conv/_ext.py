@@ -1,0 +1,371 @@
+"""Binding of libssc.so (include/ssc.h) under the names of the reference's
+pybind module ``ss_conv._ext`` (src/ss_conv_ops_api.cpp:15-55).
+
+torch supplies device memory and the current stream; all work happens in the
+HIP kernels of the library.  There is no CPU fallback: without the built
+library the import fails, and without a GPU every call raises.
+"""
+import ctypes
+import os
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(os.path.dirname(_HERE), "lib", "libssc.so")
+
+if not os.path.exists(LIB_PATH):
+    raise ImportError(
+        "libssc.so is not built (%s missing): run `python ss-conv_amd/build.py`" % LIB_PATH)
+
+_lib = ctypes.CDLL(LIB_PATH)
+
+_vp = ctypes.c_void_p
+_i32 = ctypes.c_int32
+_i64 = ctypes.c_int64
+_sz = ctypes.c_size_t
+
+
+class Geometry(ctypes.Structure):
+    """struct ssc_geometry."""
+    _fields_ = [("batch_size", _i32), ("out_shape", _i32 * 3), ("ksize", _i32 * 3),
+                ("stride", _i32 * 3), ("padding", _i32 * 3), ("dilation", _i32 * 3),
+                ("subm", _i32), ("transpose", _i32)]
+
+
+_gp = ctypes.POINTER(Geometry)
+
+_SIGNATURES = {
+    "ssc_version": (ctypes.c_int, []),
+    "ssc_last_error": (ctypes.c_char_p, []),
+    "ssc_rulebook_workspace_bytes": (_sz, [_gp, _i64]),
+    "ssc_rulebook_count": (ctypes.c_int, [_vp, _i64, _gp, _vp, _sz, ctypes.POINTER(_i32), _vp]),
+    "ssc_rulebook_emit": (ctypes.c_int, [_vp, _i64, _gp, _vp, _sz, _vp, _vp, _vp, _vp]),
+    "ssc_conv_workspace_bytes": (_sz, [_i64, _i32, _i32, _i32, _i64]),
+    "ssc_conv_fwd_f32": (ctypes.c_int, [_vp, _i64, _i32, _vp, _i64, _i64, _i64, _i32, _vp, _i64,
+                                        _vp, _i32, _i32, _i32, _vp, _i64, _vp, _sz, _vp]),
+    "ssc_kernel_combine_f32": (ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32,
+                                              _vp, _vp]),
+    "ssc_pool_workspace_bytes": (_sz, [_i64, _i32]),
+    "ssc_pool_max_f32": (ctypes.c_int, [_vp, _i32, _vp, _i64, _vp, _i32, _vp, _i64, _vp, _sz,
+                                        _vp]),
+    "ssc_pool_avg_f32": (ctypes.c_int, [_vp, _i32, _vp, _i64, _vp, _i32, _vp, _vp, _i64, _vp,
+                                        _sz, _vp]),
+    "ssc_summary_rf": (ctypes.c_int, [_vp, _i64, _vp, _i32, _vp, _i64, _vp, _sz, _vp]),
+    "ssc_segment_avg_f32": (ctypes.c_int, [_vp, _vp, _vp, _i32, _i32, _vp]),
+    "ssc_segment_max_f32": (ctypes.c_int, [_vp, _vp, _vp, _vp, _i32, _i32, _vp]),
+    "ssc_voxel_coords": (ctypes.c_int, [_vp, _vp, _i64, ctypes.POINTER(ctypes.c_float),
+                                        ctypes.POINTER(ctypes.c_float), _vp, _vp]),
+    "ssc_unique_workspace_bytes": (_sz, [ctypes.POINTER(_i32), _i64]),
+    "ssc_unique_count": (ctypes.c_int, [_vp, _i64, ctypes.POINTER(_i32), _vp, _sz,
+                                        ctypes.POINTER(_i32), _vp]),
+    "ssc_unique_emit": (ctypes.c_int, [_vp, _i64, ctypes.POINTER(_i32), _vp, _sz, _i64, _vp, _vp,
+                                       _vp, _vp]),
+    "ssc_voxel_map": (ctypes.c_int, [_vp, _vp, _vp, _i32, _i32, _i32, _i32, _vp]),
+    "ssc_voxel_reduce_f32": (ctypes.c_int, [_vp, _vp, _vp, _i32, _i32, _i32, _i32, _vp]),
+    "ssc_three_nn": (ctypes.c_int, [_i32, _i32, _vp, _vp, _vp, _vp, _vp]),
+    "ssc_three_interp_f32": (ctypes.c_int, [_i32, _i32, _i32, _vp, _vp, _vp, _vp, _vp]),
+}
+
+for _name, (_res, _args) in _SIGNATURES.items():
+    _fn = getattr(_lib, _name)
+    _fn.restype = _res
+    _fn.argtypes = _args
+
+EXPORTED_SYMBOLS = tuple(_SIGNATURES)
+
+SSC_EINVAL, SSC_ERUNTIME, SSC_EWORKSPACE, SSC_EHIP = -1, -2, -3, -4
+
+
+def _check(rc):
+    """Map a status code to the exception class the reference raises
+    (utils/tensorview.h:70-90: runtime_error -> RuntimeError, invalid_argument -> ValueError)."""
+    if rc == 0:
+        return
+    msg = _lib.ssc_last_error().decode(errors="replace")
+    if rc == SSC_EINVAL:
+        raise ValueError(msg)
+    raise RuntimeError(msg)
+
+
+def _stream(t):
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _need_gpu(*tensors):
+    for t in tensors:
+        if not t.is_cuda:
+            raise RuntimeError(
+                "ss_conv runs on the GPU only: got a tensor on %s (there is no CPU path)" % t.device)
+
+
+def _ptr(t):
+    return t.data_ptr() if t is not None and t.numel() > 0 else None
+
+
+def _workspace(nbytes, device):
+    return torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=device)
+
+
+def _geometry(batch_size, out_shape, ksize, stride, padding, dilation, subm, transpose):
+    g = Geometry()
+    g.batch_size = int(batch_size)
+    for name, val in (("out_shape", out_shape), ("ksize", ksize), ("stride", stride),
+                      ("padding", padding), ("dilation", dilation)):
+        setattr(g, name, (_i32 * 3)(*[int(v) for v in val]))
+    g.subm = int(bool(subm))
+    g.transpose = int(bool(transpose))
+    return g
+
+
+def get_indice_pairs_3d(indices, batch_size, out_spatial_shape, spatial_shape, kernel_size, stride,
+                        padding, dilation, out_padding, subm, transpose):
+    """src/ss_conv_ops.cu:31 / src/conv/indice_conv.h:21-131.
+    Returns [outids[N_out,4], indicePairs[K,2,N], indiceNum[K]] (all int32)."""
+    if indices.dim() != 2 or indices.size(1) != 4:
+        raise RuntimeError("indices must be [N, 4] (batch, x, y, z)")
+    for lst in (kernel_size, out_spatial_shape, stride, padding, out_padding, dilation):
+        if len(lst) != 3:
+            raise RuntimeError("geometry lists must have 3 entries")
+    _need_gpu(indices)
+    if indices.dtype != torch.int32:
+        indices = indices.int()
+    indices = indices.contiguous()
+    n = indices.size(0)
+    dev = indices.device
+    g = _geometry(batch_size, out_spatial_shape, kernel_size, stride, padding, dilation, subm,
+                  transpose)
+    K = int(kernel_size[0]) * int(kernel_size[1]) * int(kernel_size[2])
+    nbytes = _lib.ssc_rulebook_workspace_bytes(ctypes.byref(g), n)
+    if nbytes == 0:  # geometry rejected: let the count call produce the message
+        nbytes = 256
+    ws = _workspace(nbytes, dev)
+    n_out = _i32(0)
+    s = _stream(indices)
+    _check(_lib.ssc_rulebook_count(_ptr(indices), n, ctypes.byref(g), ws.data_ptr(), ws.numel(),
+                                   ctypes.byref(n_out), s))
+    pairs = torch.empty((K, 2, n), dtype=torch.int32, device=dev)
+    num = torch.empty((K,), dtype=torch.int32, device=dev)
+    outids = indices if subm else torch.empty((n_out.value, 4), dtype=torch.int32, device=dev)
+    _check(_lib.ssc_rulebook_emit(_ptr(indices), n, ctypes.byref(g), ws.data_ptr(), ws.numel(),
+                                  None if subm else _ptr(outids), _ptr(pairs), num.data_ptr(), s))
+    return [outids, pairs, num]
+
+
+def _filter_strides(filters, c_in, c_out):
+    """Element strides (k, ci, co) of a [*kernel, Cin, Cout] tensor seen as [K, Cin, Cout]."""
+    if filters.dim() < 3 or filters.size(-2) != c_in:
+        raise RuntimeError("filters must be [*kernel_size, Cin, Cout] with Cin = features.size(1)")
+    kdims = filters.shape[:-2]
+    kstr = filters.stride()[:-2]
+    ok = True
+    for a in range(len(kdims) - 1):
+        if kdims[a] != 1 and kstr[a] != kstr[a + 1] * kdims[a + 1]:
+            ok = False
+    if not ok:
+        filters = filters.contiguous()
+        kstr = filters.stride()[:-2]
+    return filters, kstr[-1], filters.stride(-2), filters.stride(-1)
+
+
+def indice_conv_fp32(features, filters, indice_pairs, indice_num, num_act_out, inverse, subm):
+    """src/conv/indice_conv.h:247-343 (bound at src/ss_conv_ops_api.cpp:21)."""
+    _need_gpu(features, filters, indice_pairs)
+    if features.dtype != torch.float32 or filters.dtype != torch.float32:
+        raise RuntimeError("indice_conv_fp32 needs float32 features and filters")
+    features = features.contiguous()
+    c_in = features.size(1)
+    c_out = filters.size(-1)
+    filters, fs_k, fs_ci, fs_co = _filter_strides(filters, c_in, c_out)
+    pairs = indice_pairs.int().contiguous() if indice_pairs.dtype != torch.int32 \
+        else indice_pairs.contiguous()
+    num = indice_num.to(device=features.device, dtype=torch.int32).contiguous()
+    K = pairs.size(0)
+    kvol = 1
+    for d in filters.shape[:-2]:
+        kvol *= d
+    if kvol != K:
+        raise RuntimeError("filters have %d offsets but the rulebook has %d" % (kvol, K))
+    n_out = int(num_act_out)
+    out = torch.empty((n_out, c_out), dtype=torch.float32, device=features.device)
+    nbytes = _lib.ssc_conv_workspace_bytes(n_out, K, c_in, c_out, pairs.size(2))
+    ws = _workspace(nbytes, features.device)
+    _check(_lib.ssc_conv_fwd_f32(_ptr(features), features.size(0), c_in, _ptr(filters), fs_k,
+                                 fs_ci, fs_co, c_out, _ptr(pairs), pairs.size(2), num.data_ptr(),
+                                 K, int(inverse), int(subm), _ptr(out), n_out, ws.data_ptr(),
+                                 ws.numel(), _stream(features)))
+    return out
+
+
+def _pool_args(features, indice_pairs, indice_num):
+    _need_gpu(features, indice_pairs)
+    if features.dtype != torch.float32:
+        raise RuntimeError("rulebook pooling needs float32 features")
+    features = features.contiguous()
+    pairs = indice_pairs.int().contiguous() if indice_pairs.dtype != torch.int32 \
+        else indice_pairs.contiguous()
+    num = indice_num.to(device=features.device, dtype=torch.int32).contiguous()
+    return features, pairs, num
+
+
+def indice_maxpool_fp32(features, indice_pairs, indice_num, num_act):
+    """src/pool/indice_maxpool.h:15-50."""
+    features, pairs, num = _pool_args(features, indice_pairs, indice_num)
+    n_out, c, K = int(num_act), features.size(1), pairs.size(0)
+    out = torch.empty((n_out, c), dtype=torch.float32, device=features.device)
+    ws = _workspace(_lib.ssc_pool_workspace_bytes(n_out, K), features.device)
+    _check(_lib.ssc_pool_max_f32(_ptr(features), c, _ptr(pairs), pairs.size(2), num.data_ptr(), K,
+                                 _ptr(out), n_out, ws.data_ptr(), ws.numel(), _stream(features)))
+    return out
+
+
+def indice_avgpool_fp32(features, indice_pairs, indice_num, num_act, summaryrf):
+    """src/pool/indice_avgpool.h:17-52."""
+    features, pairs, num = _pool_args(features, indice_pairs, indice_num)
+    n_out, c, K = int(num_act), features.size(1), pairs.size(0)
+    rf = summaryrf.to(device=features.device, dtype=torch.int32).contiguous()
+    if rf.numel() != n_out:
+        raise RuntimeError("summaryrf must have one entry per output row")
+    out = torch.empty((n_out, c), dtype=torch.float32, device=features.device)
+    ws = _workspace(_lib.ssc_pool_workspace_bytes(n_out, K), features.device)
+    _check(_lib.ssc_pool_avg_f32(_ptr(features), c, _ptr(pairs), pairs.size(2), num.data_ptr(), K,
+                                 _ptr(rf), _ptr(out), n_out, ws.data_ptr(), ws.numel(),
+                                 _stream(features)))
+    return out
+
+
+def indiceSummaryRF(indice_pairs, indice_num, num_act):
+    """src/ss_conv_ops.cu:116-145."""
+    _need_gpu(indice_pairs)
+    pairs = indice_pairs.int().contiguous() if indice_pairs.dtype != torch.int32 \
+        else indice_pairs.contiguous()
+    num = indice_num.to(device=pairs.device, dtype=torch.int32).contiguous()
+    n_out = int(num_act)
+    rf = torch.empty((n_out,), dtype=torch.int32, device=pairs.device)
+    _check(_lib.ssc_summary_rf(_ptr(pairs), pairs.size(2), num.data_ptr(), pairs.size(0),
+                               _ptr(rf), n_out, None, 0, _stream(pairs)))
+    return rf
+
+
+def _seg_args(feats, offsets, out, n_seg, c):
+    _need_gpu(feats, offsets, out)
+    if feats.dtype != torch.float32 or offsets.dtype != torch.int32:
+        raise RuntimeError("segment pooling needs float32 features and int32 offsets")
+    if not (feats.is_contiguous() and offsets.is_contiguous() and out.is_contiguous()):
+        raise RuntimeError("segment pooling needs contiguous tensors")
+    if offsets.numel() != n_seg + 1 or feats.size(1) != c or out.numel() != n_seg * c:
+        raise RuntimeError("segment pooling: inconsistent sizes")
+
+
+def global_avgpool_fp(feats, offsets, out, out_maxidx, n_proposal, c):
+    """src/pool/global_avgpool.cpp:13-20; writes `out` in place."""
+    _seg_args(feats, offsets, out, n_proposal, c)
+    _check(_lib.ssc_segment_avg_f32(_ptr(feats), offsets.data_ptr(), _ptr(out), n_proposal, c,
+                                    _stream(feats)))
+
+
+def global_maxpool_fp(feats, offsets, out, out_maxidx, n_proposal, c):
+    """src/pool/global_maxpool.cpp; writes `out` and `out_maxidx` in place."""
+    _seg_args(feats, offsets, out, n_proposal, c)
+    if out_maxidx.dtype != torch.int32 or not out_maxidx.is_contiguous():
+        raise RuntimeError("out_maxidx must be a contiguous int32 tensor")
+    _check(_lib.ssc_segment_max_f32(_ptr(feats), offsets.data_ptr(), _ptr(out), _ptr(out_maxidx),
+                                    n_proposal, c, _stream(feats)))
+
+
+def voxel2point_map(inverse, ids, out_maps, n_point, max_active, mode):
+    """src/voxelize/voxel2point.cpp:12-18; fills the pre-initialised `out_maps` in place."""
+    _need_gpu(inverse, ids, out_maps)
+    for t in (inverse, ids, out_maps):
+        if t.dtype != torch.int32 or not t.is_contiguous():
+            raise RuntimeError("voxel2point_map needs contiguous int32 tensors")
+    _check(_lib.ssc_voxel_map(_ptr(inverse), _ptr(ids), _ptr(out_maps), int(n_point),
+                              out_maps.size(0), int(max_active), int(mode), _stream(inverse)))
+
+
+def voxelize_fp(feats, out, maps, mode, n_voxel, max_active, c):
+    """src/voxelize/voxelize_cuda_kernel.h:18-40; writes `out` in place."""
+    _need_gpu(feats, out, maps)
+    if feats.dtype != torch.float32 or maps.dtype != torch.int32:
+        raise RuntimeError("voxelize_fp needs float32 features and an int32 map")
+    if not (feats.is_contiguous() and out.is_contiguous() and maps.is_contiguous()):
+        raise RuntimeError("voxelize_fp needs contiguous tensors")
+    _check(_lib.ssc_voxel_reduce_f32(_ptr(feats), _ptr(out), _ptr(maps), int(mode), int(n_voxel),
+                                     int(max_active), int(c), _stream(feats)))
+
+
+def three_nn(n, m, unknown, known, dist2, idx):
+    """src/voxelize/interpolation.cpp three_nn wrapper; fills dist2 and idx in place."""
+    _need_gpu(unknown, known, dist2, idx)
+    if unknown.dtype != torch.float32 or known.dtype != torch.float32 or \
+            dist2.dtype != torch.float32 or idx.dtype != torch.int32:
+        raise RuntimeError("three_nn: wrong dtypes")
+    if unknown.size(-1) != 4 or (known.numel() and known.size(-1) != 4):
+        raise RuntimeError("three_nn rows are (b, x, y, z)")
+    for t in (unknown, known, dist2, idx):
+        if not t.is_contiguous():
+            raise RuntimeError("three_nn needs contiguous tensors")
+    _check(_lib.ssc_three_nn(int(n), int(m), _ptr(unknown), _ptr(known), _ptr(dist2), _ptr(idx),
+                             _stream(unknown)))
+
+
+def three_interpolate_fp(c, m, n, feats, idx, weight, out):
+    """src/voxelize/interpolation.cpp three_interpolate wrapper; fills out in place."""
+    _need_gpu(feats, idx, weight, out)
+    if feats.dtype != torch.float32 or weight.dtype != torch.float32 or idx.dtype != torch.int32:
+        raise RuntimeError("three_interpolate_fp: wrong dtypes")
+    for t in (feats, idx, weight, out):
+        if not t.is_contiguous():
+            raise RuntimeError("three_interpolate_fp needs contiguous tensors")
+    _check(_lib.ssc_three_interp_f32(int(c), int(m), int(n), _ptr(feats), _ptr(idx), _ptr(weight),
+                                     _ptr(out), _stream(feats)))
+
+
+# ---- entry points without a counterpart in the reference's binding ---------------------
+def kernel_combine(weight, basis, chan_out, chan_in, blocks, n_irreps_in, kernel_volume, c_in,
+                   c_out):
+    """Dense kernel [K, Cin, Cout] from the flat weight vector and the stacked
+    basis (ss_conv/utils/kernel.py:267-299 fused with convolution.py:56)."""
+    _need_gpu(weight, basis, chan_out, chan_in, blocks)
+    out = torch.empty((kernel_volume, c_in, c_out), dtype=torch.float32, device=weight.device)
+    _check(_lib.ssc_kernel_combine_f32(_ptr(weight), _ptr(basis), _ptr(chan_out), _ptr(chan_in),
+                                       _ptr(blocks), int(n_irreps_in), int(kernel_volume),
+                                       int(c_in), int(c_out), _ptr(out), _stream(weight)))
+    return out
+
+
+def voxel_coords(points, batch_ids, half_extent, unit):
+    """int32 [N,4] (b, vx, vy, vz) with v = (int)((p + half) / unit) in fp32
+    (ss_conv/sp_ops/voxelize.py:85-86)."""
+    _need_gpu(points, batch_ids)
+    points = points.float().contiguous()
+    ids = batch_ids.long().contiguous()
+    n = points.size(0)
+    coords = torch.empty((n, 4), dtype=torch.int32, device=points.device)
+    h = (ctypes.c_float * 3)(*[float(v) for v in half_extent])
+    u = (ctypes.c_float * 3)(*[float(v) for v in unit])
+    _check(_lib.ssc_voxel_coords(_ptr(points), _ptr(ids), n, h, u, _ptr(coords), _stream(points)))
+    return coords
+
+
+def unique_rows(coords, dims, return_counts=True):
+    """Sorted unique rows of an int32 [N,4] table with inverse and counts: the
+    torch.unique(dim=0, return_inverse=True, return_counts=True) of
+    ss_conv/sp_ops/voxelize.py:88 for rows inside `dims`."""
+    _need_gpu(coords)
+    coords = coords.contiguous()
+    n = coords.size(0)
+    dev = coords.device
+    d = (_i32 * 4)(*[int(v) for v in dims])
+    nbytes = _lib.ssc_unique_workspace_bytes(d, n)
+    if nbytes == 0:
+        raise RuntimeError("unique_rows: prod(dims) must be positive and below 2^31")
+    ws = _workspace(nbytes, dev)
+    m = _i32(0)
+    s = _stream(coords)
+    _check(_lib.ssc_unique_count(_ptr(coords), n, d, ws.data_ptr(), ws.numel(), ctypes.byref(m), s))
+    uniq = torch.empty((m.value, 4), dtype=torch.int32, device=dev)
+    inverse = torch.empty((n,), dtype=torch.int32, device=dev)
+    counts = torch.empty((m.value,), dtype=torch.int32, device=dev) if return_counts else None
+    _check(_lib.ssc_unique_emit(_ptr(coords), n, d, ws.data_ptr(), ws.numel(), m.value, _ptr(uniq),
+                                _ptr(inverse), _ptr(counts), s))
+    return uniq, inverse, counts

@@ -1,0 +1,231 @@
+"""autograd entry points over the native kernels
+(reference: ss_conv/sp_ops/functional.py:22-453; same exported names).
+
+Forward passes run the HIP kernels.  Backward passes are not built yet: a
+Function whose backward is reached raises NotImplementedError instead of
+returning wrong gradients."""
+import torch
+from torch.autograd import Function
+
+from ss_conv import _ext
+from . import ops
+
+
+def _no_backward(name):
+    raise NotImplementedError("backward of %s is not built yet (forward-only build)" % name)
+
+
+class _ConvBase(Function):
+    inverse = False
+    subm = False
+
+    @classmethod
+    def _run(cls, ctx, features, filters, indice_pairs, indice_pair_num, num_activate_out):
+        ctx.save_for_backward(indice_pairs, indice_pair_num, features, filters)
+        return ops.indice_conv_forward(features, filters, indice_pairs, indice_pair_num,
+                                       num_activate_out, cls.inverse, cls.subm)
+
+
+class SparseConvFunction(_ConvBase):
+    @staticmethod
+    def forward(ctx, features, filters, indice_pairs, indice_pair_num, num_activate_out):
+        return SparseConvFunction._run(ctx, features, filters, indice_pairs, indice_pair_num,
+                                       num_activate_out)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        _no_backward("indice_conv")
+
+
+class SparseInverseConvFunction(_ConvBase):
+    inverse = True
+
+    @staticmethod
+    def forward(ctx, features, filters, indice_pairs, indice_pair_num, num_activate_out):
+        return SparseInverseConvFunction._run(ctx, features, filters, indice_pairs,
+                                              indice_pair_num, num_activate_out)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        _no_backward("indice_inverse_conv")
+
+
+class SubMConvFunction(_ConvBase):
+    subm = True
+
+    @staticmethod
+    def forward(ctx, features, filters, indice_pairs, indice_pair_num, num_activate_out):
+        return SubMConvFunction._run(ctx, features, filters, indice_pairs, indice_pair_num,
+                                     num_activate_out)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        _no_backward("indice_subm_conv")
+
+
+class SparseMaxPoolFunction(Function):
+    @staticmethod
+    def forward(ctx, features, indice_pairs, indice_pair_num, num_activate_out):
+        out = ops.indice_maxpool_forward(features, indice_pairs, indice_pair_num, num_activate_out)
+        ctx.save_for_backward(indice_pairs, indice_pair_num, features, out)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        _no_backward("indice_maxpool")
+
+
+class SparseAvgPoolFunction(Function):
+    """use_gs=True (the only value any caller passes) divides by the kernel
+    volume; use_gs=False by the number of contributing inputs
+    (reference: functional.py:162-185)."""
+
+    @staticmethod
+    def forward(ctx, features, indice_pairs, indice_pair_num, num_activate_out, use_gs=True):
+        if use_gs:
+            summaryrf = torch.full((int(num_activate_out),), int(indice_pairs.shape[0]),
+                                   dtype=torch.int32, device=indice_pairs.device)
+        else:
+            summaryrf = _ext.indiceSummaryRF(indice_pairs, indice_pair_num, num_activate_out)
+        out = ops.indice_avgpool_forward(features, indice_pairs, indice_pair_num,
+                                         num_activate_out, summaryrf)
+        ctx.save_for_backward(indice_pairs, indice_pair_num, features, out, summaryrf)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        _no_backward("indice_avgpool")
+
+
+class _SegmentPool(Function):
+    @staticmethod
+    def _alloc(feats, proposals_offset):
+        n_seg = proposals_offset.size(0) - 1
+        c = feats.size(1)
+        assert feats.is_contiguous()
+        assert proposals_offset.is_contiguous()
+        out = torch.zeros((n_seg, c), dtype=torch.float32, device=feats.device)
+        idx = torch.zeros((n_seg, c), dtype=torch.int32, device=feats.device)
+        return n_seg, c, out, idx
+
+
+class GlobalMaxPool(Function):
+    @staticmethod
+    def forward(ctx, feats, proposals_offset):
+        """feats [sum_n, C] float32, proposals_offset [B+1] int32 -> [B, C]."""
+        n_seg, c, out, idx = _SegmentPool._alloc(feats, proposals_offset)
+        _ext.global_maxpool_fp(feats, proposals_offset, out, idx, n_seg, c)
+        ctx.for_backwards = (idx, proposals_offset, feats.size(0))
+        return out
+
+    @staticmethod
+    def backward(ctx, d_output_feats):
+        _no_backward("global_maxpool")
+
+
+class GlobalAvgPool(Function):
+    @staticmethod
+    def forward(ctx, feats, proposals_offset):
+        """feats [sum_n, C] float32, proposals_offset [B+1] int32 -> [B, C]."""
+        n_seg, c, out, idx = _SegmentPool._alloc(feats, proposals_offset)
+        _ext.global_avgpool_fp(feats, proposals_offset, out, idx, n_seg, c)
+        ctx.for_backwards = (idx, proposals_offset, feats.size(0))
+        return out
+
+    @staticmethod
+    def backward(ctx, d_output_feats):
+        _no_backward("global_avgpool")
+
+
+class Voxelization(Function):
+    @staticmethod
+    def forward(ctx, feats, map_rule, mode=4):
+        """feats [N, C], map_rule [M, maxActive+1] int32 -> [M, C]."""
+        assert map_rule.is_contiguous()
+        assert feats.is_contiguous()
+        n, c = feats.size()
+        m = map_rule.size(0)
+        max_active = map_rule.size(1) - 1
+        out = torch.zeros((m, c), dtype=torch.float32, device=feats.device)
+        ctx.for_backwards = (map_rule, mode, max_active, n)
+        _ext.voxelize_fp(feats, out, map_rule, mode, m, max_active, c)
+        return out
+
+    @staticmethod
+    def backward(ctx, d_output_feats):
+        _no_backward("voxelization")
+
+
+class Voxel2Point_Map(Function):
+    @staticmethod
+    def forward(ctx, inverse, nActive, maxActive, mode=4):
+        """inverse [N] (voxel of each point) -> int32 [nActive, maxActive+1]:
+        column 0 the point count, then the point ids (ascending)."""
+        inverse = inverse.view(-1).contiguous().int()
+        n = inverse.size(0)
+        dev = inverse.device
+        ids = torch.arange(n, dtype=torch.int32, device=dev)
+        if mode == 3 or mode == 4:
+            maps = torch.zeros((nActive, maxActive + 1), dtype=torch.int32, device=dev)
+        elif mode == 2:
+            maps = torch.full((nActive, maxActive + 1), -1, dtype=torch.int32, device=dev)
+        elif mode == 1:
+            maps = torch.full((nActive, maxActive + 1), n, dtype=torch.int32, device=dev)
+        else:
+            assert False
+        _ext.voxel2point_map(inverse, ids, maps, n, maxActive, mode)
+        return maps
+
+    @staticmethod
+    def backward(ctx, grad=None):
+        return None, None, None, None
+
+
+class ThreeNN(Function):
+    @staticmethod
+    def forward(ctx, unknown, known):
+        """unknown [n, 4], known [m, 4] rows of (b, x, y, z) -> (dist [n, 3], idx [n, 3] int32)."""
+        assert unknown.is_contiguous()
+        assert known.is_contiguous()
+        n = unknown.size(0)
+        m = known.size(0)
+        dist2 = torch.empty((n, 3), dtype=torch.float32, device=unknown.device)
+        idx = torch.empty((n, 3), dtype=torch.int32, device=unknown.device)
+        _ext.three_nn(n, m, unknown, known, dist2, idx)
+        return torch.sqrt(dist2), idx
+
+    @staticmethod
+    def backward(ctx, a=None, b=None):
+        return None, None
+
+
+class ThreeInterpolate(Function):
+    @staticmethod
+    def forward(ctx, features, idx, weight):
+        """features [m, C], idx [n, 3] int32, weight [n, 3] -> [n, C]."""
+        assert features.is_contiguous()
+        assert idx.is_contiguous()
+        assert weight.is_contiguous()
+        m, c = features.size()
+        n = idx.size(0)
+        ctx.three_interpolate_for_backward = (idx, weight, m)
+        out = torch.empty((n, c), dtype=torch.float32, device=features.device)
+        _ext.three_interpolate_fp(c, m, n, features, idx, weight, out)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        _no_backward("three_interpolate")
+
+
+indice_conv = SparseConvFunction.apply
+indice_inverse_conv = SparseInverseConvFunction.apply
+indice_subm_conv = SubMConvFunction.apply
+indice_maxpool = SparseMaxPoolFunction.apply
+indice_avgpool = SparseAvgPoolFunction.apply
+global_maxpool = GlobalMaxPool.apply
+global_avgpool = GlobalAvgPool.apply
+voxelization = Voxelization.apply
+voxel2point_mapping = Voxel2Point_Map.apply
+three_nn = ThreeNN.apply
+three_interpolate = ThreeInterpolate.apply

@@ -1,0 +1,139 @@
+"""Point cloud <-> sparse voxel tensor (reference: ss_conv/sp_ops/voxelize.py:18-162)."""
+import numpy as np
+import torch
+import torch.nn as nn
+
+from ss_conv import _ext
+from .tensor import SparseTensor
+from .functional import voxelization, voxel2point_mapping, three_nn, three_interpolate
+
+
+class Point2Voxel(nn.Module):
+    """Voxelise a batch of point clouds centred on the origin.
+
+    forward(point_cloud [N,3], feature [N,C], batch_ids [N]) returns
+    (valid_points, SparseTensor, valid_ids, valid_instance_flag) as the
+    reference does (voxelize.py:29-99): points outside the grid are dropped,
+    batch elements left without points get one zero point, points are ordered
+    by batch id (stable), voxel index = (int)((p + half_extent) / unit) in fp32,
+    voxels come out in ascending (b, x, y, z) order and carry the mean (mode 4),
+    sum (3), first (1) or last (2) of their points' features.
+
+    The sorted-unique of voxel rows, the per-voxel point lists and the feature
+    reduction are native kernels; row filtering and the batch sort are torch ops.
+    """
+
+    def __init__(self, voxel_num_limit=[64, 64, 64], unit_voxel_extent=[0.05, 0.05, 0.05],
+                 voxelization_mode=4):
+        super().__init__()
+        self.unit_voxel_extent = torch.tensor(np.asarray(unit_voxel_extent, dtype=np.float64),
+                                              dtype=torch.float32)
+        self.voxel_num_limit = np.array(voxel_num_limit)
+        self.voxelization_mode = voxelization_mode
+
+    def forward(self, point_cloud, feature, batch_ids):
+        assert len(point_cloud.size()) == 2
+        C = feature.size(1)
+        device = point_cloud.device
+
+        unique_origin_ids = torch.unique(batch_ids)
+        B1 = unique_origin_ids.size(0)
+
+        unit = self.unit_voxel_extent.numpy().astype(np.float32)
+        limit = self.voxel_num_limit.astype(np.float32)
+        half = np.float32(0.5) * (limit * unit)  # fp32 throughout, as on the device
+        half_t = torch.from_numpy(half).reshape(1, 3).to(device)
+
+        inside = (torch.abs(point_cloud) > half_t).sum(1) == 0
+        if inside.sum() == 0:
+            valid_instance_flag = torch.zeros(B1, dtype=torch.float32, device=device)
+            valid_point_cloud = torch.zeros(B1, 3, dtype=torch.float32, device=device)
+            valid_feature = torch.zeros(B1, C, dtype=torch.float32, device=device)
+            valid_ids = unique_origin_ids
+        else:
+            valid_point_cloud = point_cloud[inside].contiguous()
+            valid_feature = feature[inside].contiguous()
+            valid_ids = batch_ids[inside].contiguous()
+            unique_valid_ids = torch.unique(valid_ids)
+            B2 = unique_valid_ids.size(0)
+            if B1 == B2:
+                valid_instance_flag = torch.ones(B1, dtype=torch.float32, device=device)
+            else:
+                valid_instance_flag = torch.isin(unique_origin_ids, unique_valid_ids).float()
+                invalid_ids = unique_origin_ids[valid_instance_flag == 0].contiguous()
+                assert len(invalid_ids) == B1 - B2
+                pad = B1 - B2
+                valid_point_cloud = torch.cat(
+                    [valid_point_cloud, torch.zeros(pad, 3, dtype=torch.float32, device=device)], 0)
+                valid_feature = torch.cat(
+                    [valid_feature, torch.zeros(pad, C, dtype=torch.float32, device=device)], 0)
+                valid_ids = torch.cat([valid_ids, invalid_ids], 0)
+            order = torch.sort(valid_ids, stable=True)[1]
+            valid_point_cloud = valid_point_cloud[order].contiguous()
+            valid_feature = valid_feature[order].contiguous()
+            valid_ids = valid_ids[order].contiguous()
+
+        lo = int(valid_ids.min().item())
+        hi = int(valid_ids.max().item())
+        if lo < 0:
+            raise ValueError("batch ids must be non-negative")
+        voxel_index = _ext.voxel_coords(valid_point_cloud, valid_ids, half, unit)
+        # a point exactly on the upper face lands on index == limit, hence the +1
+        dims = [hi + 1] + [int(v) + 1 for v in self.voxel_num_limit]
+        occupied_index, inverse, count = _ext.unique_rows(voxel_index, dims, return_counts=True)
+        nActive = occupied_index.size(0)
+        if self.voxelization_mode == 1 or self.voxelization_mode == 2:
+            maxActive = 1
+        else:
+            maxActive = int(torch.max(count).item())
+        v2p_maps = voxel2point_mapping(inverse, nActive, maxActive, self.voxelization_mode)
+        sparse_feat = voxelization(valid_feature.float().contiguous(), v2p_maps.detach(),
+                                   self.voxelization_mode)
+        sparse_feat = SparseTensor(sparse_feat, occupied_index.detach(),
+                                   self.voxel_num_limit.astype(np.int64), B1)
+        return valid_point_cloud, sparse_feat, valid_ids, valid_instance_flag
+
+
+class Voxel2Point(nn.Module):
+    """Read voxel features back at points by inverse-distance interpolation over
+    the three nearest voxel centres of the same batch element
+    (reference: voxelize.py:102-162).  Without points, returns the voxel
+    centres, their features and their batch ids."""
+
+    def __init__(self, voxel_extent=None, unit_voxel_extent=None):
+        super().__init__()
+        assert voxel_extent is not None or unit_voxel_extent is not None
+        self.voxel_extent = None if voxel_extent is None else \
+            np.asarray(voxel_extent, dtype=np.float64)
+        self.unit_voxel_extent = None if unit_voxel_extent is None else \
+            np.asarray(unit_voxel_extent, dtype=np.float64)
+
+    def forward(self, sparse_feat, point_cloud=None, batch_ids=None):
+        vx_points, vx_feats = self._get_vertice_feats(sparse_feat)
+        if point_cloud is not None:
+            assert batch_ids is not None
+            points = torch.cat([batch_ids.float().unsqueeze(1), point_cloud], dim=1)
+            return self._get_point_feats(points.contiguous(), vx_points, vx_feats)
+        return vx_points[:, 1:].contiguous(), vx_feats, vx_points[:, 0].contiguous()
+
+    def _get_vertice_feats(self, sparse_tensor):
+        feat = sparse_tensor.features
+        device = feat.device
+        shape = np.asarray(sparse_tensor.spatial_shape, dtype=np.float64)
+        if self.voxel_extent is not None:
+            unit = torch.tensor(self.voxel_extent / shape, dtype=torch.float32, device=device)
+            extent = torch.tensor(self.voxel_extent, dtype=torch.float32, device=device)
+        else:
+            unit = torch.tensor(self.unit_voxel_extent, dtype=torch.float32, device=device)
+            extent = torch.tensor(self.unit_voxel_extent * shape, dtype=torch.float32,
+                                  device=device)
+        centres = sparse_tensor.indices.float()
+        centres[:, 1:] = centres[:, 1:] * unit - 0.5 * extent + 0.5 * unit
+        return centres.contiguous().detach(), feat
+
+    def _get_point_feats(self, target_points, query_points, query_feats):
+        dist, idx = three_nn(target_points, query_points)
+        dist_recip = 1.0 / (dist + 1e-8)
+        norm = torch.sum(dist_recip, dim=1, keepdim=True)
+        weight = dist_recip / norm
+        return three_interpolate(query_feats.contiguous(), idx, weight.contiguous())

@@ -1,0 +1,389 @@
+"""GPU parity: every native entry point against the CPU oracle on seeded inputs.
+
+Bars: rulebooks, voxel indices and every other integer result bit-exact;
+fp32 results within rel-L2 1e-5 (conv, which re-associates sums on MFMA) or
+bit-exact where the kernel keeps the oracle's operation order (pools, voxel
+means, interpolation)."""
+import numpy as np
+import pytest
+import torch
+
+import synth
+
+pytestmark = pytest.mark.gpu
+
+REL_L2 = 1e-5
+
+
+def rel_l2(a, b):
+    a = np.asarray(a, dtype=np.float64)
+    b = np.asarray(b, dtype=np.float64)
+    den = np.linalg.norm(b)
+    return np.linalg.norm(a - b) / (den if den > 0 else 1.0)
+
+
+def random_voxels(rng, batch, grid, n):
+    cells = rng.choice(batch * grid ** 3, size=n, replace=False)
+    cells.sort()
+    b, r = cells // grid ** 3, cells % grid ** 3
+    return np.stack([b, r // grid ** 2, (r // grid) % grid, r % grid], 1).astype(np.int32)
+
+
+def gpu_rulebook(idx, batch, grid, k, s, p, d=1, subm=False, device="cuda"):
+    from ss_conv.sp_ops.ops import get_indice_pairs
+    t = torch.from_numpy(idx).to(device)
+    out, pairs, num = get_indice_pairs(t, batch, [grid] * 3, k, s, p, d, 0, subm)
+    torch.cuda.synchronize()
+    return out.cpu().numpy(), pairs.cpu().numpy(), num.cpu().numpy()
+
+
+RULEBOOK_CASES = [
+    # batch, grid, n, k, stride, pad, dil, subm
+    (2, 8, 60, 3, 1, 1, 1, False),
+    (2, 9, 80, 3, 2, 1, 1, False),
+    (3, 8, 70, 2, 2, 0, 1, False),
+    (1, 10, 90, 5, 1, 2, 1, False),
+    (2, 8, 100, 3, 1, 1, 1, True),
+    (2, 7, 50, 3, 2, 0, 1, False),
+    (2, 8, 50, 3, 3, 1, 1, False),
+    (2, 12, 200, 3, 1, 2, 2, False),
+    (4, 16, 1500, 3, 1, 1, 1, False),
+    (2, 8, 1, 3, 1, 1, 1, False),
+    (1, 4, 64, 3, 1, 1, 1, False),   # full grid
+    (2, 16, 300, 5, 1, 2, 1, True),
+]
+
+
+@pytest.mark.parametrize("case", RULEBOOK_CASES)
+def test_rulebook_matches_oracle(case, oracle, device):
+    batch, grid, n, k, s, p, d, subm = case
+    rng = np.random.default_rng(hash(case) % 2 ** 31)
+    idx = random_voxels(rng, batch, grid, n)
+    print("case", case, flush=True)
+    o_idx, o_pairs, o_num, o_shape = oracle.rulebook(idx, batch, [grid] * 3, k, s, p, d, subm)
+    if not subm:
+        o_idx, o_pairs, o_num = oracle.canonicalize(o_idx, o_pairs, o_num, o_shape)
+    g_idx, g_pairs, g_num = gpu_rulebook(idx, batch, grid, k, s, p, d, subm)
+    assert np.array_equal(g_num, o_num)
+    assert np.array_equal(g_idx, o_idx)
+    assert np.array_equal(g_pairs, o_pairs)
+
+
+def test_rulebook_unsorted_input_rows(oracle, device):
+    """Input rows in arbitrary order: outputs still ascending by key, pairs ascending in input row."""
+    rng = np.random.default_rng(5)
+    idx = random_voxels(rng, 2, 10, 150)
+    idx = idx[rng.permutation(idx.shape[0])]
+    o = oracle.canonicalize(*oracle.rulebook(idx, 2, [10] * 3, 3, 1, 1))
+    g = gpu_rulebook(idx, 2, 10, 3, 1, 1)
+    for a, b in zip(g, o):
+        assert np.array_equal(a, b)
+
+
+def test_rulebook_empty_and_errors(device):
+    from ss_conv import _ext
+    empty = torch.zeros((0, 4), dtype=torch.int32, device=device)
+    out, pairs, num = _ext.get_indice_pairs_3d(empty, 1, [8] * 3, [8] * 3, [3] * 3, [1] * 3, [1] * 3,
+                                               [1] * 3, [0] * 3, 0, 0)
+    assert out.shape == (0, 4) and pairs.shape == (27, 2, 0) and int(num.sum()) == 0
+    one = torch.zeros((1, 4), dtype=torch.int32, device=device)
+    with pytest.raises(RuntimeError):  # kernel volume 343 > 256 (reference: indice_conv.h:44)
+        _ext.get_indice_pairs_3d(one, 1, [8] * 3, [8] * 3, [7] * 3, [1] * 3, [3] * 3, [1] * 3,
+                                 [0] * 3, 0, 0)
+    with pytest.raises(RuntimeError):  # wrong list length (reference: indice_conv.h:33-39)
+        _ext.get_indice_pairs_3d(one, 1, [8] * 3, [8] * 3, [3] * 2, [1] * 3, [1] * 3, [1] * 3,
+                                 [0] * 3, 0, 0)
+
+
+def test_rulebook_config1_sizes(oracle, device):
+    c = synth.CONFIGS["cfg1"]
+    pts, _, ids = synth.config_clouds("cfg1")
+    idx = synth.voxel_indices(pts, ids, c["grid"])
+    o = oracle.canonicalize(*oracle.rulebook(idx, c["batch"], [c["grid"]] * 3, 3, 1, 1))
+    g = gpu_rulebook(idx, c["batch"], c["grid"], 3, 1, 1)
+    for a, b in zip(g, o):
+        assert np.array_equal(a, b)
+
+
+CONV_CASES = [
+    # n_vox, grid, k, s, p, cin, cout
+    (300, 10, 3, 1, 1, 32, 32),
+    (300, 10, 3, 1, 1, 64, 128),
+    (200, 10, 3, 2, 1, 128, 256),
+    (200, 8, 3, 1, 1, 3, 152),
+    (150, 8, 5, 1, 2, 200, 200),
+    (100, 8, 3, 1, 1, 5, 7),
+    (100, 8, 2, 2, 0, 16, 20),
+    (900, 12, 3, 1, 1, 64, 64),
+]
+
+
+def _conv_case(oracle, device, n, grid, k, s, p, cin, cout, seed, permuted=False, shuffle=False):
+    from ss_conv import _ext
+    rng = np.random.default_rng(seed)
+    idx = random_voxels(rng, 2, grid, n)
+    if shuffle:
+        idx = idx[rng.permutation(n)]
+    feats = rng.normal(size=(n, cin)).astype(np.float32)
+    K = k ** 3
+    w = (rng.normal(size=(K, cin, cout)) / np.sqrt(K * cin)).astype(np.float32)
+    o_idx, o_pairs, o_num = oracle.canonicalize(*oracle.rulebook(idx, 2, [grid] * 3, k, s, p))
+    # fp64 accumulation of the same sums as the reference's gather-GEMM-scatter
+    ref = np.zeros((o_idx.shape[0], cout), dtype=np.float64)
+    for kk in range(K):
+        m = int(o_num[kk])
+        if m:
+            np.add.at(ref, o_pairs[kk, 1, :m],
+                      feats[o_pairs[kk, 0, :m]].astype(np.float64) @ w[kk].astype(np.float64))
+    # and the fp32 restatement must agree with it
+    ref32 = oracle.conv_fwd(feats, w, o_pairs, o_num, o_idx.shape[0], matmul=np.matmul)
+    assert rel_l2(ref32, ref) < REL_L2
+
+    g_idx, g_pairs, g_num = [torch.from_numpy(x).to(device) for x in
+                             gpu_rulebook(idx, 2, grid, k, s, p)]
+    wt = torch.from_numpy(w).to(device)
+    if permuted:  # the reference's layout: [Cout, Cin, k, k, k] permuted to [k, k, k, Cin, Cout]
+        wt = wt.permute(2, 1, 0).contiguous().reshape(cout, cin, k, k, k).permute(2, 3, 4, 1, 0)
+        assert not wt.is_contiguous()
+    else:
+        wt = wt.reshape(k, k, k, cin, cout)
+    out = _ext.indice_conv_fp32(torch.from_numpy(feats).to(device), wt, g_pairs, g_num,
+                                g_idx.shape[0], 0, 0)
+    torch.cuda.synchronize()
+    err = rel_l2(out.cpu().numpy(), ref)
+    assert err < REL_L2, err
+    return out, ref
+
+
+@pytest.mark.parametrize("case", CONV_CASES)
+def test_conv_matches_oracle(case, oracle, device):
+    print("case", case, flush=True)
+    n, grid, k, s, p, cin, cout = case
+    _conv_case(oracle, device, n, grid, k, s, p, cin, cout, seed=11)
+
+
+def test_conv_reference_filter_layout(oracle, device):
+    _conv_case(oracle, device, 300, 10, 3, 1, 1, 32, 48, seed=12, permuted=True)
+
+
+def test_conv_unsorted_pairs(oracle, device):
+    """Input rows in arbitrary order make the per-offset output rows unsorted: the re-ordering path."""
+    _conv_case(oracle, device, 300, 10, 3, 1, 1, 32, 32, seed=13, shuffle=True)
+
+
+def test_conv_is_reproducible(oracle, device):
+    a, _ = _conv_case(oracle, device, 900, 12, 3, 1, 1, 64, 64, seed=14)
+    b, _ = _conv_case(oracle, device, 900, 12, 3, 1, 1, 64, 64, seed=14)
+    assert torch.equal(a, b)
+
+
+def test_conv_inverse(oracle, device):
+    """inverse=1 swaps the pair planes: features live on the outputs of the forward rulebook."""
+    from ss_conv import _ext
+    rng = np.random.default_rng(21)
+    idx = random_voxels(rng, 2, 10, 200)
+    o_idx, o_pairs, o_num = oracle.canonicalize(*oracle.rulebook(idx, 2, [10] * 3, 3, 2, 1))
+    n_out = o_idx.shape[0]
+    feats = rng.normal(size=(n_out, 16)).astype(np.float32)
+    w = rng.normal(size=(27, 16, 24)).astype(np.float32)
+    ref = oracle.conv_fwd(feats, w, o_pairs, o_num, idx.shape[0], inverse=True, matmul=np.matmul)
+    out = _ext.indice_conv_fp32(torch.from_numpy(feats).to(device),
+                                torch.from_numpy(w).to(device).reshape(3, 3, 3, 16, 24),
+                                torch.from_numpy(o_pairs).to(device),
+                                torch.from_numpy(o_num).to(device), idx.shape[0], 1, 0)
+    assert rel_l2(out.cpu().numpy(), ref) < REL_L2
+
+
+@pytest.mark.parametrize("k,s,p,c", [(2, 2, 0, 64), (3, 2, 1, 32), (3, 1, 1, 5), (2, 2, 0, 256)])
+def test_pools_match_oracle(k, s, p, c, oracle, device):
+    from ss_conv import _ext
+    rng = np.random.default_rng(31)
+    idx = random_voxels(rng, 2, 12, 400)
+    feats = rng.normal(size=(400, c)).astype(np.float32)
+    o_idx, o_pairs, o_num = oracle.canonicalize(*oracle.rulebook(idx, 2, [12] * 3, k, s, p))
+    n_out = o_idx.shape[0]
+    ft = torch.from_numpy(feats).to(device)
+    pt = torch.from_numpy(o_pairs).to(device)
+    nt = torch.from_numpy(o_num).to(device)
+    mx = _ext.indice_maxpool_fp32(ft, pt, nt, n_out).cpu().numpy()
+    assert np.array_equal(mx, oracle.maxpool_fwd(feats, o_pairs, o_num, n_out))
+    rf = _ext.indiceSummaryRF(pt, nt, n_out)
+    assert np.array_equal(rf.cpu().numpy(), oracle.summary_rf(o_pairs, o_num, n_out))
+    full = torch.full((n_out,), k ** 3, dtype=torch.int32, device=device)
+    av = _ext.indice_avgpool_fp32(ft, pt, nt, n_out, full).cpu().numpy()
+    assert np.array_equal(av, oracle.avgpool_fwd(feats, o_pairs, o_num, n_out))
+    av2 = _ext.indice_avgpool_fp32(ft, pt, nt, n_out, rf).cpu().numpy()
+    assert np.array_equal(av2, oracle.avgpool_fwd(feats, o_pairs, o_num, n_out,
+                                                  rf.cpu().numpy()))
+
+
+@pytest.mark.parametrize("c", [1, 32, 200, 512])
+def test_segment_pools(c, oracle, device):
+    from ss_conv.pool import GlobalAvgPool, GlobalMaxPool
+    rng = np.random.default_rng(41)
+    lens = [5, 1, 300, 17, 64]
+    offsets = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    feats = rng.normal(size=(offsets[-1], c)).astype(np.float32)
+    feats[10:40, 0] = 2.5  # ties: the first row of the maximum wins
+    ft, ot = torch.from_numpy(feats).to(device), torch.from_numpy(offsets).to(device)
+    avg = GlobalAvgPool()(ft, ot).cpu().numpy()
+    assert rel_l2(avg, oracle.segment_avg(feats, offsets)) < 1e-6
+    mx = GlobalMaxPool()(ft, ot).cpu().numpy()
+    o_max, o_idx = oracle.segment_max(feats, offsets)
+    assert np.array_equal(mx, o_max)
+    from ss_conv import _ext
+    out = torch.zeros((len(lens), c), device=device)
+    arg = torch.zeros((len(lens), c), dtype=torch.int32, device=device)
+    _ext.global_maxpool_fp(ft, ot, out, arg, len(lens), c)
+    assert np.array_equal(arg.cpu().numpy(), o_idx)
+
+
+def test_segment_pool_empty_segment(oracle, device):
+    from ss_conv import _ext
+    feats = np.arange(12, dtype=np.float32).reshape(4, 3)
+    offsets = np.array([0, 2, 2, 4], dtype=np.int32)
+    ft, ot = torch.from_numpy(feats).to(device), torch.from_numpy(offsets).to(device)
+    out = torch.zeros((3, 3), device=device)
+    arg = torch.zeros((3, 3), dtype=torch.int32, device=device)
+    _ext.global_avgpool_fp(ft, ot, out, arg, 3, 3)
+    o = oracle.segment_avg(feats, offsets)
+    assert np.array_equal(np.isnan(out.cpu().numpy()), np.isnan(o))
+    _ext.global_maxpool_fp(ft, ot, out, arg, 3, 3)
+    om, oi = oracle.segment_max(feats, offsets)
+    assert np.array_equal(out.cpu().numpy(), om) and np.array_equal(arg.cpu().numpy(), oi)
+
+
+@pytest.mark.parametrize("mode", [1, 2, 3, 4])
+def test_point2voxel_matches_oracle(mode, oracle, device):
+    from ss_conv.sp_ops.voxelize import Point2Voxel
+    pts, feats, ids = synth.make_clouds(3, 700, seed=3, channels=6)
+    pts = pts * 1.2  # some points fall outside and are filtered
+    grid = 16
+    ref = oracle.point2voxel(pts, feats, ids, [grid] * 3, [2.0 / grid] * 3, mode)
+    p2v = Point2Voxel([grid] * 3, [2.0 / grid] * 3, mode)
+    vp, st, vi, flag = p2v(torch.from_numpy(pts).to(device), torch.from_numpy(feats).to(device),
+                           torch.from_numpy(ids).to(device))
+    assert np.array_equal(vp.cpu().numpy(), ref["valid_points"])
+    assert np.array_equal(vi.cpu().numpy(), ref["valid_ids"])
+    assert np.array_equal(flag.cpu().numpy(), ref["flag"])
+    assert np.array_equal(st.indices.cpu().numpy(), ref["indices"])
+    assert st.batch_size == ref["batch_size"]
+    assert np.array_equal(st.features.cpu().numpy(), ref["features"])
+
+
+def test_point2voxel_empty_batch_element(oracle, device):
+    """A batch element whose points all fall outside gets one zero point (voxelize.py:68-78)."""
+    from ss_conv.sp_ops.voxelize import Point2Voxel
+    pts, feats, ids = synth.make_clouds(3, 100, seed=4, channels=2)
+    pts[ids == 1] = 50.0
+    ref = oracle.point2voxel(pts, feats, ids, [8] * 3, [0.25] * 3, 4)
+    vp, st, vi, flag = Point2Voxel([8] * 3, [0.25] * 3)(
+        torch.from_numpy(pts).to(device), torch.from_numpy(feats).to(device),
+        torch.from_numpy(ids).to(device))
+    assert flag.cpu().tolist() == [1.0, 0.0, 1.0] == ref["flag"].tolist()
+    assert np.array_equal(st.indices.cpu().numpy(), ref["indices"])
+    assert np.array_equal(st.features.cpu().numpy(), ref["features"])
+    # everything outside (voxelize.py:52-56)
+    pts[:] = 50.0
+    ref = oracle.point2voxel(pts, feats, ids, [8] * 3, [0.25] * 3, 4)
+    vp, st, vi, flag = Point2Voxel([8] * 3, [0.25] * 3)(
+        torch.from_numpy(pts).to(device), torch.from_numpy(feats).to(device),
+        torch.from_numpy(ids).to(device))
+    assert flag.cpu().tolist() == [0.0, 0.0, 0.0]
+    assert np.array_equal(st.indices.cpu().numpy(), ref["indices"])
+
+
+def test_voxel2point_matches_oracle(oracle, device):
+    from ss_conv.sp_ops.voxelize import Point2Voxel, Voxel2Point
+    pts, feats, ids = synth.make_clouds(3, 500, seed=6, channels=10)
+    grid = 16
+    dp, df, di = [torch.from_numpy(x).to(device) for x in (pts, feats, ids)]
+    vp, st, vi, _ = Point2Voxel([grid] * 3, [2.0 / grid] * 3)(dp, df, di)
+    out = Voxel2Point(unit_voxel_extent=[2.0 / grid] * 3)(st, vp, vi)
+    ref, ridx, rw = oracle.voxel2point(st.indices.cpu().numpy(), st.features.cpu().numpy(),
+                                       [grid] * 3, vp.cpu().numpy(), vi.cpu().numpy(),
+                                       unit_voxel_extent=[2.0 / grid] * 3)
+    assert rel_l2(out.cpu().numpy(), ref) < 1e-6
+    # index parity of the search itself, including ties
+    from ss_conv.sp_ops.functional import three_nn
+    centres = Voxel2Point(unit_voxel_extent=[2.0 / grid] * 3)._get_vertice_feats(st)[0]
+    target = torch.cat([vi.float().unsqueeze(1), vp], 1).contiguous()
+    dist, idx = three_nn(target, centres)
+    odist, oidx = oracle.three_nn(target.cpu().numpy(), centres.cpu().numpy())
+    assert np.array_equal(idx.cpu().numpy(), oidx)
+    assert np.array_equal(dist.cpu().numpy(), odist)
+    c2, f2, b2 = Voxel2Point(voxel_extent=[2.0] * 3)(st)
+    assert c2.shape == (st.indices.shape[0], 3) and f2 is st.features
+
+
+def test_kernel_combine_matches_einsum(oracle, device):
+    from ss_conv.utils.kernel import SE3Kernel
+    torch.manual_seed(0)
+    for rs_in, rs_out, size in [([(2, 0), (2, 1), (2, 2), (2, 3)], [(2, 0), (2, 1), (2, 2), (2, 3)], 3),
+                                ([(3, 0)], [(2, 0), (1, 1), (1, 2)], 3),
+                                ([(1, 0), (2, 2)], [(2, 1), (1, 4)], 5)]:
+        ker = SE3Kernel(rs_in, rs_out, size).to(device)
+        got = ker().cpu().numpy()
+        bases = [[getattr(ker, "kernel_%d_%d" % (i, j)) for j in range(len(ker.Rs_in))]
+                 for i in range(len(ker.Rs_out))]
+        bases = [[None if b is None else b.cpu().numpy() for b in row] for row in bases]
+        ref = oracle.combine(ker.weight.detach().cpu().numpy(), bases, ker.multiplicities_out,
+                             ker.dims_out, ker.multiplicities_in, ker.dims_in, size)
+        assert got.shape == ref.shape
+        assert rel_l2(got, ref) < 1e-6
+
+
+def test_convolution_layer_end_to_end(oracle, device):
+    """Point2Voxel -> Convolution against the oracle pipeline and against dense conv3d."""
+    import torch.nn.functional as F
+    from ss_conv.convolution import Convolution
+    from ss_conv.sp_ops.voxelize import Point2Voxel
+    torch.manual_seed(1)
+    rs = [(2, 0), (2, 1), (2, 2), (2, 3)]
+    pts, feats, ids = synth.make_clouds(2, 300, seed=8, channels=32)
+    grid = 12
+    conv = Convolution(rs, rs, 3, stride=1, padding=1).to(device).eval()
+    _, st, _, _ = Point2Voxel([grid] * 3, [2.0 / grid] * 3)(
+        *[torch.from_numpy(x).to(device) for x in (pts, feats, ids)])
+    with torch.no_grad():
+        out = conv(st)
+    dense_kernel = conv.kernel().detach()  # [Cout, Cin, k, k, k]
+    want = F.conv3d(st.dense().cpu().double(), dense_kernel.cpu().double(), stride=1, padding=1)
+    got = out.dense().cpu().double()
+    assert rel_l2(got.numpy(), want.numpy()) < REL_L2
+    w = dense_kernel.permute(2, 3, 4, 1, 0).reshape(27, 32, 32).cpu().numpy()
+    o_idx, o_pairs, o_num = oracle.canonicalize(*oracle.rulebook(
+        st.indices.cpu().numpy(), 2, [grid] * 3, 3, 1, 1))
+    assert np.array_equal(out.indices.cpu().numpy(), o_idx)
+    ref = oracle.conv_fwd(st.features.cpu().numpy(), w, o_pairs, o_num, o_idx.shape[0],
+                          matmul=np.matmul)
+    assert rel_l2(out.features.cpu().numpy(), ref) < REL_L2
+
+
+def test_downsampling_block(oracle, device):
+    """Strided convolution followed by MaxPool and AvgPool (k=2, s=2)."""
+    import torch.nn.functional as F
+    from ss_conv.convolution import Convolution
+    from ss_conv.pool import MaxPool, AvgPool
+    from ss_conv.sp_ops.voxelize import Point2Voxel
+    torch.manual_seed(2)
+    pts, feats, ids = synth.make_clouds(2, 400, seed=9, channels=4)
+    grid = 16
+    conv = Convolution([(4, 0)], [(2, 0), (2, 1)], 3, stride=2, padding=1).to(device).eval()
+    _, st, _, _ = Point2Voxel([grid] * 3, [2.0 / grid] * 3)(
+        *[torch.from_numpy(x).to(device) for x in (pts, feats, ids)])
+    with torch.no_grad():
+        y = conv(st)
+        mx = MaxPool(2, 2)(y)
+        av = AvgPool(2, 2)(y)
+    assert list(y.spatial_shape) == [8, 8, 8] and list(mx.spatial_shape) == [4, 4, 4]
+    dy = y.dense().cpu()
+    assert rel_l2(mx.dense().cpu().numpy(), F.max_pool3d(F.relu(dy), 2, 2).numpy()) < 1e-6
+    assert rel_l2(av.dense().cpu().numpy(), F.avg_pool3d(dy, 2, 2).numpy()) < 1e-6
+
+
+def test_cpu_tensor_is_rejected(device):
+    from ss_conv import _ext
+    with pytest.raises(RuntimeError):
+        _ext.get_indice_pairs_3d(torch.zeros((1, 4), dtype=torch.int32), 1, [8] * 3, [8] * 3,
+                                 [3] * 3, [1] * 3, [1] * 3, [1] * 3, [0] * 3, 0, 0)
