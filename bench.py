@@ -1,0 +1,205 @@
+"""Benchmark of the sparse steerable convolution layer on one MI355X.
+
+One step = one forward of ss_conv.convolution.Convolution on the voxelised
+batch, with everything the reference runs per training forward: rulebook build
+(count + emit), steerable kernel synthesis, and the MFMA sparse convolution.
+Inputs (voxel indices and features) are resident in HBM before the timed
+region.  Workload: BASELINE config 2 by default (32 clouds x 2048 surface
+points, 64^3 grid, irreps (4,4,4,4) -> (8,8,8,8), i.e. 64 -> 128 channels,
+kernel 3, stride 1, padding 1, fp32).
+
+Prints one JSON line; see --help for the other workloads.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for _p in (os.path.join(ROOT, "ss-conv_amd"), os.path.join(ROOT, "oracle")):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+FP32_MFMA_PEAK_TFLOPS = 157.3  # MI355X dense fp32 matrix peak
+
+# HBM bytes per launch of the convolution kernel, from rocprofv3 --pmc
+# FETCH_SIZE / WRITE_SIZE runs scaled by a copy kernel of known size
+# (summaries under profiles/); None until measured for a workload.
+MEASURED_TRAFFIC_BYTES = {}
+
+
+def parse_args():
+    ap = argparse.ArgumentParser(description=__doc__)
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="cfg2", choices=["cfg1", "cfg2", "cfg3", "cfg5"])
+    ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--breakdown", action="store_true",
+                    help="also print per-phase timings to stderr")
+    return ap.parse_args()
+
+
+def cpu_baseline(idx, feats, dense_w, cfg, n_out_expected):
+    """The CPU restatement of the reference layer (serial rulebook, per-offset
+    gather -> BLAS GEMM -> scatter-add) on the full workload, median of 3."""
+    import numpy as np
+    import oracle as O
+    grid = cfg["grid"]
+    times = []
+    n_out = None
+    for _ in range(3):
+        t0 = time.perf_counter()
+        o_idx, pairs, num, _ = O.rulebook(idx, cfg["batch"], [grid] * 3, cfg["kernel"],
+                                          cfg["stride"], cfg["padding"])
+        out = O.conv_fwd(feats, dense_w, pairs, num, o_idx.shape[0], matmul=np.matmul)
+        times.append(time.perf_counter() - t0)
+        n_out = o_idx.shape[0]
+        if sum(times) > 40:
+            break
+    assert n_out == n_out_expected
+    t = sorted(times)[len(times) // 2]
+    try:
+        from threadpoolctl import threadpool_info
+        cores = max([p.get("num_threads", 1) for p in threadpool_info()] + [1])
+    except Exception:
+        cores = os.cpu_count() or 1
+    return {"value": n_out / t, "unit": "active output voxels/s", "cores": int(cores),
+            "kind": "port",
+            "sample": "full %s layer (rulebook + gather/GEMM/scatter conv), median of %d runs, "
+                      "%.2f s each; rulebook and gather/scatter single-thread C, GEMM numpy BLAS"
+                      % (cfg["name"], len(times), t)}, out
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this path uses no second GPU "
+              "(run with --gpus 1)", file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+    import synth
+    from ss_conv import _ext
+    from ss_conv.convolution import Convolution
+    from ss_conv.sp_ops.tensor import SparseTensor
+    from ss_conv.sp_ops.voxelize import Point2Voxel
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(2)
+    dev = torch.device("cuda:0")
+    cfg = dict(synth.CONFIGS[args.workload], name=args.workload)
+    grid = cfg["grid"]
+    rs_in = synth.irreps(cfg["mult_in"], cfg["lmax"])
+    rs_out = synth.irreps(cfg["mult_out"], cfg["lmax"])
+
+    torch.manual_seed(args.seed)
+    pts, feats, ids = synth.config_clouds(args.workload, args.seed)
+    conv = Convolution(rs_in, rs_out, cfg["kernel"], stride=cfg["stride"],
+                       padding=cfg["padding"]).to(dev)
+    conv.train()  # the kernel is synthesised on every forward, as in a training step
+    p2v = Point2Voxel([grid] * 3, [2.0 / grid] * 3)
+    with torch.no_grad():
+        _, st, _, _ = p2v(torch.from_numpy(pts).to(dev), torch.from_numpy(feats).to(dev),
+                          torch.from_numpy(ids).to(dev))
+    indices = st.indices.contiguous()
+    features = st.features.contiguous()
+    n_in, c_in = features.shape
+    c_out = conv.out_channels
+    K = cfg["kernel"] ** 3
+
+    def step():
+        x = SparseTensor(features, indices, st.spatial_shape, st.batch_size)
+        with torch.no_grad():
+            return conv(x)
+
+    for _ in range(args.warmup):
+        out = step()
+    torch.cuda.synchronize()
+
+    _ext.profile_conv(True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        out = step()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    conv_ms = _ext.profile_conv_read()
+    _ext.profile_conv(False)
+
+    n_out = out.features.shape[0]
+    pair_num = out.indice_dict[None][3] if None in out.indice_dict else None
+    x = SparseTensor(features, indices, st.spatial_shape, st.batch_size)
+    with torch.no_grad():
+        from ss_conv.sp_ops.ops import get_indice_pairs
+        _, _, num = get_indice_pairs(indices, st.batch_size, st.spatial_shape, cfg["kernel"],
+                                     cfg["stride"], cfg["padding"])
+    P = int(num.sum().item())
+    ms_per_step = (t1 - t0) * 1e3 / args.steps
+    conv_kernel_ms = sum(conv_ms) / max(len(conv_ms), 1)
+    flops = 2.0 * P * c_in * c_out
+    achieved = flops / (conv_kernel_ms * 1e-3) / 1e12 if conv_kernel_ms > 0 else 0.0
+
+    result = {
+        "metric": "SS-Conv layer active output voxels/s (rulebook + kernel synthesis + conv)",
+        "value": n_out / (ms_per_step * 1e-3),
+        "unit": "active output voxels/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "%s: %d clouds x %d pts, %d^3 grid, %d->%d ch, k=%d s=%d p=%d"
+                               % (args.workload, cfg["batch"], cfg["points"], grid, c_in, c_out,
+                                  cfg["kernel"], cfg["stride"], cfg["padding"]),
+                   "n_in": int(n_in), "n_out": int(n_out), "pairs": P,
+                   "input_voxels_per_s": n_in / (ms_per_step * 1e-3)},
+        "roofline": {"bound": "mfma", "achieved": achieved, "peak": FP32_MFMA_PEAK_TFLOPS,
+                     "unit": "TFLOP/s", "frac": achieved / FP32_MFMA_PEAK_TFLOPS,
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+                     "kernel": "conv_fwd_kernel", "kernel_ms": conv_kernel_ms,
+                     "flops_per_launch": flops},
+    }
+
+    if args.breakdown:
+        def timed(fn, n=10):
+            torch.cuda.synchronize()
+            a = time.perf_counter()
+            for _ in range(n):
+                r = fn()
+            torch.cuda.synchronize()
+            return (time.perf_counter() - a) * 1e3 / n, r
+        with torch.no_grad():
+            t_rb, rb = timed(lambda: get_indice_pairs(indices, st.batch_size, st.spatial_shape,
+                                                      cfg["kernel"], cfg["stride"], cfg["padding"]))
+            t_ks, w = timed(lambda: conv.kernel())
+            wv = w.permute(2, 3, 4, 1, 0)
+            t_cv, _ = timed(lambda: _ext.indice_conv_fp32(features, wv, rb[1], rb[2], n_out, 0, 0))
+        rb_bytes = 16 * n_in + 16 * n_out + 8 * P + 4 * K
+        print("breakdown ms: rulebook %.3f (%.1f GB/s algorithmic) | kernel synthesis %.3f | "
+              "conv call %.3f (MFMA kernel %.3f)" %
+              (t_rb, rb_bytes / t_rb / 1e6, t_ks, t_cv, conv_kernel_ms), file=sys.stderr)
+
+    if not args.no_cpu_baseline:
+        w = conv.kernel().permute(2, 3, 4, 1, 0).reshape(K, c_in, c_out).cpu().numpy()
+        base, ref_out = cpu_baseline(indices.cpu().numpy(), features.cpu().numpy(), w, cfg, n_out)
+        result["cpu_baseline"] = base
+        # the timed GPU result against the CPU port (first-touch vs key order: compare by key)
+        import oracle as O
+        o_idx, _, _, o_shape = O.rulebook(indices.cpu().numpy(), cfg["batch"], [grid] * 3,
+                                          cfg["kernel"], cfg["stride"], cfg["padding"])
+        order = np.argsort(O.flat_key(o_idx, o_shape), kind="stable")
+        got = out.features.cpu().numpy()
+        err = float(np.linalg.norm(got - ref_out[order]) / np.linalg.norm(ref_out))
+        result["parity_rel_l2"] = err
+    else:
+        result["cpu_baseline"] = None
+
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -114,6 +114,15 @@ int ssc_conv_fwd_f32(const float *features /* [n_in,c_in] */, int64_t n_in, int3
                      float *out /* [n_out,c_out] */, int64_t n_out, void *workspace,
                      size_t workspace_bytes, ssc_stream_t stream);
 
+/* Timing of the convolution kernel alone (no counterpart in the reference, whose
+ * timers are commented out, src/conv/indice_conv.h:295,319-341).  While enabled,
+ * every ssc_conv_fwd_f32 call records a pair of HIP events on its stream right
+ * around the launch of the MFMA kernel (ring of 512 calls).
+ * ssc_profile_conv_read waits for the recorded calls and returns their
+ * durations in milliseconds, oldest first; enabling again clears the ring. */
+int ssc_profile_conv(int32_t enable);
+int ssc_profile_conv_read(float *ms /* host */, int32_t capacity, int32_t *count /* host */);
+
 /* ------------------------------------------------------------------------
  * Steerable kernel synthesis.  Replaces SE3Kernel.combination
  * (ss_conv/utils/kernel.py:267-299: one einsum "uvb,bijxyz->uivjxyz" per pair

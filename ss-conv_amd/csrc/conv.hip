@@ -332,11 +332,44 @@ static ConvWs conv_ws_carve(void *ws, const ConvPlan &p, int64_t n_out, int K,
   return w;
 }
 
+// Optional timing of the convolution kernel alone: a ring of event pairs recorded
+// on the caller's stream right around the launch of conv_fwd_kernel.
+constexpr int kProfileRing = 512;
+static bool g_profile_on = false;
+static int g_profile_count = 0;
+static hipEvent_t g_profile_ev[kProfileRing][2];
+static bool g_profile_init = false;
+
 }  // namespace ssc
 
 using namespace ssc;
 
 extern "C" {
+
+int ssc_profile_conv(int32_t enable) {
+  if (enable && !g_profile_init) {
+    for (int i = 0; i < kProfileRing; ++i) {
+      SSC_HIP(hipEventCreate(&g_profile_ev[i][0]));
+      SSC_HIP(hipEventCreate(&g_profile_ev[i][1]));
+    }
+    g_profile_init = true;
+  }
+  g_profile_on = enable != 0;
+  g_profile_count = 0;
+  return SSC_OK;
+}
+
+int ssc_profile_conv_read(float *ms, int32_t capacity, int32_t *count) {
+  SSC_CHECK(ms != nullptr && count != nullptr, SSC_EINVAL, "NULL pointer argument");
+  int n = g_profile_count < kProfileRing ? g_profile_count : kProfileRing;
+  if (n > capacity) n = capacity;
+  for (int i = 0; i < n; ++i) {
+    SSC_HIP(hipEventSynchronize(g_profile_ev[i][1]));
+    SSC_HIP(hipEventElapsedTime(&ms[i], g_profile_ev[i][0], g_profile_ev[i][1]));
+  }
+  *count = n;
+  return SSC_OK;
+}
 
 size_t ssc_conv_workspace_bytes(int64_t n_out, int32_t kernel_volume, int32_t c_in, int32_t c_out,
                                 int64_t pair_stride) {
@@ -408,10 +441,17 @@ int ssc_conv_fwd_f32(const float *features, int64_t n_in, int32_t c_in, const fl
     attr_set = true;
   }
   dim3 grid((unsigned)p.n_tiles, (unsigned)ceil_div(p.ncb, 4));
+  const bool prof = g_profile_on;
+  const int slot = g_profile_count % kProfileRing;
+  if (prof) SSC_HIP(hipEventRecord(g_profile_ev[slot][0], s));
   hipLaunchKernelGGL(conv_fwd_kernel<4>, grid, dim3(256), p.lds_bytes, s, features, c_in, w.packed,
                      w.flag, pairs, w.sorted, pair_stride, plane_g, w.segs, K, p.nch, p.ncb, out,
                      n_out, c_out, p.T);
   SSC_LAUNCH_CHECK("conv_fwd");
+  if (prof) {
+    SSC_HIP(hipEventRecord(g_profile_ev[slot][1], s));
+    ++g_profile_count;
+  }
   return SSC_OK;
 }
 }

@@ -43,6 +43,9 @@ _SIGNATURES = {
     "ssc_conv_workspace_bytes": (_sz, [_i64, _i32, _i32, _i32, _i64]),
     "ssc_conv_fwd_f32": (ctypes.c_int, [_vp, _i64, _i32, _vp, _i64, _i64, _i64, _i32, _vp, _i64,
                                         _vp, _i32, _i32, _i32, _vp, _i64, _vp, _sz, _vp]),
+    "ssc_profile_conv": (ctypes.c_int, [_i32]),
+    "ssc_profile_conv_read": (ctypes.c_int, [ctypes.POINTER(ctypes.c_float), _i32,
+                                             ctypes.POINTER(_i32)]),
     "ssc_kernel_combine_f32": (ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32,
                                               _vp, _vp]),
     "ssc_pool_workspace_bytes": (_sz, [_i64, _i32]),
@@ -369,3 +372,17 @@ def unique_rows(coords, dims, return_counts=True):
     _check(_lib.ssc_unique_emit(_ptr(coords), n, d, ws.data_ptr(), ws.numel(), m.value, _ptr(uniq),
                                 _ptr(inverse), _ptr(counts), s))
     return uniq, inverse, counts
+
+
+def profile_conv(enable):
+    """Start (clearing earlier samples) or stop timing of the convolution kernel."""
+    _check(_lib.ssc_profile_conv(int(bool(enable))))
+
+
+def profile_conv_read():
+    """Durations in ms of the convolution kernel launches recorded since
+    profile_conv(True), oldest first (waits for them to finish)."""
+    buf = (ctypes.c_float * 512)()
+    n = _i32(0)
+    _check(_lib.ssc_profile_conv_read(buf, 512, ctypes.byref(n)))
+    return [float(buf[i]) for i in range(n.value)]
