@@ -46,7 +46,7 @@ def build(force=False, verbose=True):
     procs = []
     for src in SOURCES:
         obj = os.path.join(LIB_DIR, src.replace(".hip", ".o"))
-        cmd = [_hipcc()] + FLAGS + ["-I", os.path.join(ROOT, "include"), "-I", CSRC, "-c",
+        cmd = [_hipcc()] + FLAGS + os.environ.get("SSC_HIPCC_FLAGS", "").split() + ["-I", os.path.join(ROOT, "include"), "-I", CSRC, "-c",
                                     os.path.join(CSRC, src), "-o", obj]
         procs.append((src, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT)))
         objs.append(obj)

@@ -155,149 +155,440 @@ __global__ void __launch_bounds__(256)
   segs[idx] = lo;
 }
 
+// ---- row-block schedule -----------------------------------------------------------------
+// The pairs that land in a tile are cut, offset by offset, into row blocks of 16
+// (the M side of one MFMA); the last block of an offset is padded.  The schedule
+// lists, tile after tile and offset-major inside a tile, for every row block its
+// offset k, its 16 gather rows (-1 = padding) and its 16 tile-local output rows
+// (T = a dummy accumulator row for padding).  The convolution kernel then
+// streams through it without any per-offset bookkeeping.
+__global__ void __launch_bounds__(256)
+    sched_count_kernel(const int32_t *__restrict__ segs, int K, int64_t n_tiles,
+                       int32_t *__restrict__ tile_cnt, int32_t *__restrict__ kofs) {
+  int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= n_tiles) return;
+  int run = 0;
+  for (int k = 0; k < K; ++k) {
+    int n = segs[(t + 1) * K + k] - segs[t * K + k];
+    kofs[t * K + k] = run;
+    run += (n + 15) >> 4;
+  }
+  tile_cnt[t] = run;
+}
+
+// tile_mb[0..n_tiles]: exclusive prefix of tile_cnt (one block).
+__global__ void __launch_bounds__(kScanThreads)
+    sched_scan_kernel(const int32_t *__restrict__ tile_cnt, int64_t n_tiles,
+                      int32_t *__restrict__ tile_mb) {
+  __shared__ int lds[kScanThreads / 64 + 1];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  int carry = 0;
+  for (int64_t base = 0; base < n_tiles; base += kScanThreads) {
+    int64_t i = base + threadIdx.x;
+    int v = i < n_tiles ? tile_cnt[i] : 0;
+    int incl = v;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      int o = __shfl_up(incl, d, 64);
+      if (lane >= d) incl += o;
+    }
+    if (lane == 63) lds[wave] = incl;
+    __syncthreads();
+    int wave_off = 0, tot = 0;
+#pragma unroll
+    for (int w = 0; w < kScanThreads / 64; ++w) {
+      int x = lds[w];
+      if (w < wave) wave_off += x;
+      tot += x;
+    }
+    __syncthreads();
+    if (i < n_tiles) tile_mb[i] = carry + wave_off + incl - v;
+    carry += tot;
+  }
+  if (threadIdx.x == 0) tile_mb[n_tiles] = carry;
+}
+
+// 16 threads per (tile, offset): lane i fills slot i of each of its row blocks.
+__global__ void __launch_bounds__(256)
+    sched_fill_kernel(const int32_t *__restrict__ flag, const int32_t *__restrict__ pairs,
+                      const int32_t *__restrict__ sorted, int64_t pair_stride, int plane_g,
+                      const int32_t *__restrict__ segs, const int32_t *__restrict__ kofs,
+                      const int32_t *__restrict__ tile_mb, int K, int64_t n_tiles, int T,
+                      int32_t *__restrict__ sched_in, int32_t *__restrict__ sched_out,
+                      int32_t *__restrict__ sched_k) {
+  int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  int64_t tk = gid >> 4;
+  int lane = (int)(gid & 15);
+  if (tk >= n_tiles * K) return;
+  int64_t t = tk / K;
+  int k = (int)(tk - t * K);
+  const int32_t *src = flag[0] ? sorted : pairs;
+  int s0 = segs[t * K + k];
+  int n = segs[(t + 1) * K + k] - s0;
+  if (n <= 0) return;
+  const int32_t *pg = src + ((int64_t)k * 2 + plane_g) * pair_stride + s0;
+  const int32_t *ps = src + ((int64_t)k * 2 + (1 - plane_g)) * pair_stride + s0;
+  int64_t mb = (int64_t)tile_mb[t] + kofs[t * K + k];
+  int64_t row0 = t * (int64_t)T;
+  for (int p = lane; p < ((n + 15) & ~15); p += 16, ++mb) {
+    sched_in[mb * 16 + lane] = p < n ? pg[p] : -1;
+    sched_out[mb * 16 + lane] = p < n ? (int)(ps[p] - row0) : T;
+    if (lane == 0) sched_k[mb] = k;
+  }
+}
+
 // ---- the convolution --------------------------------------------------------------------
-// grid = (n_tiles, ceil(ncb / NWAVES)); block = NWAVES waves; wave w owns column
-// block  blockIdx.y*NWAVES + w  (16 columns).
-// Dynamic LDS: acc[T][CN] | abuf[kStage][kAStride] | orow[kStage]
-template <int NWAVES>
-__global__ void __launch_bounds__(NWAVES * 64)
+// One workgroup = one tile of T output rows x 64 output columns, 8 waves:
+//   waves 0-3  consumers: wave w owns output columns [16w, 16w+16) of the
+//              workgroup's column range and does nothing but LDS reads, MFMAs and
+//              the accumulator update;
+//   waves 4-7  producers: gather the input rows of the NEXT stage from global
+//              memory into LDS (rows are prefetched several stages ahead into
+//              registers), so that address arithmetic and memory latency run on
+//              the same SIMDs underneath the MFMA stream.
+// A stage = 4 consecutive row blocks of the schedule (64 pair slots, any mix of
+// offsets) x one 64-channel chunk of Cin; one barrier per stage hands a filled
+// LDS buffer to the consumers and an emptied one back.
+//
+// MFMA orientation: D[16 channels x 16 pairs] = W^T[16 x 4] * F^T[4 x 16], so a
+// lane ends up with 4 consecutive output channels of one pair and adds them to
+// the LDS accumulator row of that pair with one 16-byte read-modify-write.  A
+// column group belongs to exactly one wave, which walks the schedule in order,
+// so every output element sees its offsets added in ascending k: reproducible,
+// no atomics.
+//
+// Dynamic LDS: acc[T+1][68] | abuf[2][64][68] | orow[4][64] | ids[4][8]
+// (output rows and fragment ids of a stage are published two stages ahead, in a
+// ring of four, so the consumers know their next stage before its barrier.)
+constexpr int kRowsAhead = 3;  // stages whose gathered rows are in flight in registers
+constexpr int kIdxAhead = 2;   // further stages whose row indices are in flight
+
+__device__ __forceinline__ void mfma_block(const float4v (&b)[4], const float4v (&a)[4],
+                                           float4v &d) {
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    d = __builtin_amdgcn_mfma_f32_16x16x4f32(b[q].x, a[q].x, d, 0, 0, 0);
+    d = __builtin_amdgcn_mfma_f32_16x16x4f32(b[q].y, a[q].y, d, 0, 0, 0);
+    d = __builtin_amdgcn_mfma_f32_16x16x4f32(b[q].z, a[q].z, d, 0, 0, 0);
+    d = __builtin_amdgcn_mfma_f32_16x16x4f32(b[q].w, a[q].w, d, 0, 0, 0);
+  }
+}
+
+__global__ void __launch_bounds__(512)
     conv_fwd_kernel(const float *__restrict__ features, int cin, const float *__restrict__ packed,
-                    const int32_t *__restrict__ flag, const int32_t *__restrict__ pairs,
-                    const int32_t *__restrict__ sorted, int64_t pair_stride, int plane_g,
-                    const int32_t *__restrict__ segs, int K, int nch, int ncb,
-                    float *__restrict__ out, int64_t n_out, int cout, int T) {
-  constexpr int CN = NWAVES * 16;
-  constexpr int NT = NWAVES * 64;
+                    const int32_t *__restrict__ sched_in, const int32_t *__restrict__ sched_out,
+                    const int32_t *__restrict__ sched_k, const int32_t *__restrict__ tile_mb,
+                    int nch, int ncb, float *__restrict__ out, int64_t n_out, int cout, int T,
+                    int64_t n_tiles) {
+  constexpr int CN = 64;
+  constexpr int AS = CN + 4;
+  constexpr int NP = 256;  // producer threads
+  constexpr int NE = kStage * 16 / NP;
   extern __shared__ __align__(16) float lds[];
   float *acc = lds;
-  float *abuf = acc + (size_t)T * CN;
-  int *orow = reinterpret_cast<int *>(abuf + kStage * kAStride);
+  float *abuf = acc + (size_t)(T + 1) * AS;
+  int *orow = reinterpret_cast<int *>(abuf + 2 * kStage * kAStride);
+  int *ids = orow + 4 * kStage;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
-  const int g = lane >> 4;   // MFMA k-group
-  const int l16 = lane & 15;
-  const int64_t tile = blockIdx.x;
+  const bool producer = wave >= 4;
+  // Consecutive workgroup ids land on different XCDs (8 of them, one L2 each):
+  // give every XCD a contiguous range of tiles so neighbouring tiles, which
+  // gather the same input rows, share an L2.
+  int64_t tile = blockIdx.x;
+  {
+    const int64_t per = n_tiles / 8;
+    if (tile < per * 8) tile = (tile % 8) * per + tile / 8;
+  }
   const int64_t row0 = tile * (int64_t)T;
-  const int cb = blockIdx.y * NWAVES + wave;  // column block of this wave
-  const bool wave_live = cb < ncb;
-  const int32_t *src = flag[0] ? sorted : pairs;
-  const bool vec4 = (cin & 3) == 0;
+  const int mb0 = tile_mb[tile];
+  const int nmb = tile_mb[tile + 1] - mb0;
+  const int nstages = ((nmb + 3) >> 2) * nch;
 
-  for (int i = tid; i < T * CN; i += NT) acc[i] = 0.f;
+  {
+    float4v z = {0.f, 0.f, 0.f, 0.f};
+    float4v *a4 = reinterpret_cast<float4v *>(acc);
+    for (int i = tid; i < (T + 1) * AS / 4; i += 512) a4[i] = z;
+  }
 
-  for (int k = 0; k < K; ++k) {
-    const int s0 = segs[tile * K + k];
-    const int s1 = segs[(tile + 1) * K + k];
-    const int n = s1 - s0;
-    if (n <= 0) continue;
-    const int32_t *pg = src + ((int64_t)k * 2 + plane_g) * pair_stride + s0;
-    const int32_t *ps = src + ((int64_t)k * 2 + (1 - plane_g)) * pair_stride + s0;
-    for (int cc = 0; cc < nch; ++cc) {
-      // weight fragments of (k, chunk cc, column block cb): 16 MFMA steps
-      float4v b[4];
-      if (wave_live) {
-        const float4v *bp = reinterpret_cast<const float4v *>(
-            packed + (((int64_t)k * ncb + cb) * nch + cc) * 1024 + lane * 16);
+  if (producer) {
+    // ------------------------------------------------------------------ producer
+    const int pt = tid - 256;
+    const bool vec4 = (cin & 3) == 0;
+    constexpr int RD = kRowsAhead, NS = kRowsAhead + kIdxAhead + 1;
+    int idx[NS][NE];
+    float4v rows[RD + 1][NE];
+    auto load_idx = [&](int s, int (&ix)[NE]) {
+      const int grp = s / nch;
 #pragma unroll
-        for (int q = 0; q < 4; ++q) b[q] = bp[q];
+      for (int j = 0; j < NE; ++j) {
+        int slot = grp * 64 + ((pt + j * NP) >> 4);
+        ix[j] = (s < nstages && slot < nmb * 16) ? sched_in[(int64_t)mb0 * 16 + slot] : -1;
       }
-      for (int m0 = 0; m0 < n; m0 += kStage) {
-        __syncthreads();  // previous stage fully consumed (and acc zeroed on first pass)
-        // stage: gather up to 64 input rows x 64 channels
-        for (int e = tid; e < kStage * 16; e += NT) {
-          int p = e >> 4, f4 = e & 15;
-          int ch = cc * kKC + f4 * 4;
-          float4v v = {0.f, 0.f, 0.f, 0.f};
-          if (m0 + p < n) {
-            int64_t row = pg[m0 + p];
-            const float *fp = features + row * cin + ch;
-            if (vec4) {
-              if (ch < cin) v = *reinterpret_cast<const float4v *>(fp);
-            } else {
-              if (ch + 0 < cin) v.x = fp[0];
-              if (ch + 1 < cin) v.y = fp[1];
-              if (ch + 2 < cin) v.z = fp[2];
-              if (ch + 3 < cin) v.w = fp[3];
-            }
+    };
+    auto load_rows = [&](int s, const int (&ix)[NE], float4v (&r)[NE]) {
+      const int cc = s % nch;
+#pragma unroll
+      for (int j = 0; j < NE; ++j) {
+        int ch = cc * kKC + ((pt + j * NP) & 15) * 4;
+        float4v v = {0.f, 0.f, 0.f, 0.f};
+#ifdef SSC_DBG_NO_GATHER
+        if (false) {
+#else
+        if (ix[j] >= 0) {
+#endif
+          const float *fp = features + (int64_t)ix[j] * cin + ch;
+          if (vec4) {
+            if (ch < cin) v = *reinterpret_cast<const float4v *>(fp);
+          } else {
+            if (ch + 0 < cin) v.x = fp[0];
+            if (ch + 1 < cin) v.y = fp[1];
+            if (ch + 2 < cin) v.z = fp[2];
+            if (ch + 3 < cin) v.w = fp[3];
           }
-          *reinterpret_cast<float4v *>(abuf + p * kAStride + f4 * 4) = v;
         }
-        if (tid < kStage) orow[tid] = (m0 + tid < n) ? (int)(ps[m0 + tid] - row0) : -1;
-        __syncthreads();
-        if (wave_live) {
-          const int nblk = min(4, (n - m0 + 15) >> 4);
-          for (int m = 0; m < nblk; ++m) {
-            const float4v *ap =
-                reinterpret_cast<const float4v *>(abuf + (m * 16 + l16) * kAStride + g * 16);
+        r[j] = v;
+      }
+    };
+    auto store_rows = [&](int s, const float4v (&r)[NE]) {
+      float *ab = abuf + (s & 1) * kStage * kAStride;
+#pragma unroll
+      for (int j = 0; j < NE; ++j) {
+        int e = pt + j * NP;
+        *reinterpret_cast<float4v *>(ab + (e >> 4) * kAStride + (e & 15) * 4) = r[j];
+      }
+    };
+    // Per-stage metadata handled by threads 0..68: the output row of each of the
+    // 64 slots, the weight-fragment id (k * nch + cc) of the 4 row blocks and of
+    // the first block of the following stage.
+    auto load_meta = [&](int s) -> int {
+      const int grp = s / nch;
+      if (pt < kStage) {
+        int slot = grp * 64 + pt;
+        return (s < nstages && slot < nmb * 16) ? sched_out[(int64_t)mb0 * 16 + slot] : T;
+      }
+      if (pt < kStage + 5) {
+        int j = pt - kStage;
+        int s2 = j < 4 ? s : s + 1;
+        int blk = (s2 / nch) * 4 + (j & 3);
+        if (s2 < nstages && blk < nmb) return sched_k[mb0 + blk] * nch + (s2 % nch);
+      }
+      return -1;
+    };
+    auto store_meta = [&](int s, int v) {
+      if (pt < kStage) orow[(s & 3) * kStage + pt] = v;
+      else if (pt < kStage + 5) ids[(s & 3) * 8 + (pt - kStage)] = v;
+    };
+#pragma unroll
+    for (int i = 0; i < NS; ++i) load_idx(i, idx[i]);
+#pragma unroll
+    for (int i = 0; i <= RD; ++i) load_rows(i, idx[i], rows[i]);
+    store_meta(0, load_meta(0));
+    store_meta(1, load_meta(1));
+    // metadata is fetched two iterations before it is stored, so that waiting for
+    // it never waits for the row loads issued after it (loads return in order)
+    int meta0 = load_meta(2), meta1 = load_meta(3);
+    store_rows(0, rows[0]);
+    __syncthreads();
+    for (int s = 0; s < nstages; ++s) {
+      store_rows(s + 1, rows[1]);
+      store_meta(s + 2, meta0);
+      meta0 = meta1;
+#pragma unroll
+      for (int i = 0; i + 1 < NS; ++i)
+#pragma unroll
+        for (int j = 0; j < NE; ++j) idx[i][j] = idx[i + 1][j];
+#pragma unroll
+      for (int i = 1; i < RD; ++i)
+#pragma unroll
+        for (int j = 0; j < NE; ++j) rows[i][j] = rows[i + 1][j];
+      meta1 = load_meta(s + 4);
+      load_idx(s + NS, idx[NS - 1]);
+      load_rows(s + 1 + RD, idx[RD], rows[RD]);
+      __syncthreads();
+    }
+  } else {
+    // ------------------------------------------------------------------ consumer
+    const int cg = wave;
+    const int g = lane >> 4;
+    const int l16 = lane & 15;
+    const int cb = blockIdx.y * 4 + cg;
+    const bool live = cb < ncb;
+    float *acc_lane = acc + cg * 16 + g * 4;
+    auto load_b = [&](int id, float4v (&b)[4]) {
+      // id = k * nch + cc
+      const int k = id / nch, cc = id - k * nch;
+      const float4v *bp = reinterpret_cast<const float4v *>(
+          packed + (((int64_t)k * ncb + cb) * nch + cc) * 1024 + lane * 16);
+#pragma unroll
+      for (int q = 0; q < 4; ++q) b[q] = bp[q];
+    };
+    auto load_a = [&](const float *ab, int m, float4v (&a)[4]) {
+      const float4v *ap =
+          reinterpret_cast<const float4v *>(ab + (m * 16 + l16) * kAStride + g * 16);
+#ifdef SSC_DBG_NO_A
+      if (n_tiles < 0)
+#endif
+#pragma unroll
+      for (int q = 0; q < 4; ++q) a[q] = ap[q];
+    };
+    auto accumulate = [&](int ol, const float4v &d) {
+      // d = out[pair l16][channels 4g .. 4g+3] of this column group
+      float4v *ptr = reinterpret_cast<float4v *>(acc_lane + ol * AS);
+#ifdef SSC_DBG_NO_RMW
+      if (d.x == 12345.f) *ptr = d;
+#else
+      *ptr = *ptr + d;
+#endif
+    };
+    __syncthreads();
+    // Weight fragments are fetched one whole stage ahead: stage s multiplies with
+    // set (s & 1) while the fragments of stage s+1 stream into the other set.
+    // idc = fragment ids of the current stage, idn = of the next one (the ring
+    // publishes them two stages ahead).
+    int idc[5], idn[5];
+#pragma unroll
+    for (int j = 0; j < 5; ++j) {
+      idc[j] = __builtin_amdgcn_readfirstlane(ids[j]);
+      idn[j] = __builtin_amdgcn_readfirstlane(ids[8 + j]);
+    }
+    float4v bx[4][4], by[4][4];
+    // Only the first block of a run of equal ids is fetched; the rest of the run is
+    // filled in by register copies once the data has arrived (fill_b_stage).
+    auto load_b_stage = [&](const int (&id)[5], float4v (&b)[4][4]) {
+#pragma unroll
+      for (int m = 0; m < 4; ++m)
+        if (id[m] >= 0 && (m == 0 || id[m] != id[m - 1])) load_b(id[m], b[m]);
+    };
+    auto fill_b_stage = [&](const int (&id)[5], float4v (&b)[4][4]) {
+#pragma unroll
+      for (int m = 1; m < 4; ++m)
+        if (id[m] >= 0 && id[m] == id[m - 1]) {
+#pragma unroll
+          for (int q = 0; q < 4; ++q) b[m][q] = b[m - 1][q];
+        }
+    };
+    // one stage out of LDS buffer (s & 1) with fragment set b; prefetches bn for s+1
+    auto run_stage = [&](int s, float4v (&b)[4][4], float4v (&bn)[4][4]) {
+      const float *ab = abuf + (s & 1) * kStage * kAStride;
+      const int *orw = orow + (s & 3) * kStage;
+      load_b_stage(idn, bn);
+      if (idc[3] >= 0) {
+        // full stage: straight-line code so LDS reads, MFMAs and accumulator updates
+        // of neighbouring row blocks can be interleaved by the scheduler
+        float4v a[4][4];
+        int ol[4];
+        float4v d[4];
+#pragma unroll
+        for (int m = 0; m < 4; ++m) {
+          load_a(ab, m, a[m]);
+          ol[m] = orw[m * 16 + l16];
+        }
+#pragma unroll
+        for (int m = 0; m < 4; ++m) {
+          d[m] = float4v{0.f, 0.f, 0.f, 0.f};
+          mfma_block(b[m], a[m], d[m]);
+          accumulate(ol[m], d[m]);
+        }
+      } else {
+        // last, partial stage of the tile
+#pragma unroll
+        for (int m = 0; m < 3; ++m) {
+          if (idc[m] >= 0) {
             float4v a[4];
-#pragma unroll
-            for (int q = 0; q < 4; ++q) a[q] = ap[q];
+            load_a(ab, m, a);
+            const int ol = orw[m * 16 + l16];
             float4v d = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-              d = __builtin_amdgcn_mfma_f32_16x16x4f32(a[q].x, b[q].x, d, 0, 0, 0);
-              d = __builtin_amdgcn_mfma_f32_16x16x4f32(a[q].y, b[q].y, d, 0, 0, 0);
-              d = __builtin_amdgcn_mfma_f32_16x16x4f32(a[q].z, b[q].z, d, 0, 0, 0);
-              d = __builtin_amdgcn_mfma_f32_16x16x4f32(a[q].w, b[q].w, d, 0, 0, 0);
-            }
-            // d[r] = D[row 4g + r][col l16]
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-              int ol = orow[m * 16 + 4 * g + r];
-              if (ol >= 0) acc[ol * CN + wave * 16 + l16] += d[r];
-            }
+            mfma_block(b[m], a, d);
+            accumulate(ol, d);
           }
         }
+      }
+      fill_b_stage(idn, bn);
+      const int *nx = ids + ((s + 2) & 3) * 8;
+#pragma unroll
+      for (int j = 0; j < 5; ++j) {
+        idc[j] = idn[j];
+        idn[j] = __builtin_amdgcn_readfirstlane(nx[j]);
+      }
+    };
+    if (live) {
+      load_b_stage(idc, bx);
+      fill_b_stage(idc, bx);
+    }
+    for (int s = 0; s < nstages; s += 2) {
+#ifdef SSC_DBG_NO_MFMA
+      if (false) {
+#else
+      if (live) {
+#endif
+        run_stage(s, bx, by);
+      }
+      __syncthreads();
+      if (s + 1 < nstages) {
+#ifdef SSC_DBG_NO_MFMA
+        if (false) {
+#else
+        if (live) {
+#endif
+          run_stage(s + 1, by, bx);
+        }
+        __syncthreads();
       }
     }
   }
-  __syncthreads();
   // write the tile
   const int col0 = blockIdx.y * CN;
   if ((cout & 3) == 0) {
-    for (int e = tid; e < T * (CN / 4); e += NT) {
+    for (int e = tid; e < T * (CN / 4); e += 512) {
       int r = e / (CN / 4), c4 = e % (CN / 4);
       int64_t grow = row0 + r;
       int col = col0 + c4 * 4;
       if (grow < n_out && col < cout)
         *reinterpret_cast<float4v *>(out + grow * cout + col) =
-            *reinterpret_cast<const float4v *>(acc + r * CN + c4 * 4);
+            *reinterpret_cast<const float4v *>(acc + r * AS + c4 * 4);
     }
   } else {
-    for (int e = tid; e < T * CN; e += NT) {
+    for (int e = tid; e < T * CN; e += 512) {
       int r = e / CN, c = e % CN;
       int64_t grow = row0 + r;
-      if (grow < n_out && col0 + c < cout) out[grow * cout + col0 + c] = acc[e];
+      if (grow < n_out && col0 + c < cout) out[grow * cout + col0 + c] = acc[r * AS + c];
     }
   }
 }
 
 struct ConvPlan {
   int ncb, nch, T;
-  int64_t n_tiles, words_per_k;
+  int64_t n_tiles, words_per_k, mb_cap;
   size_t lds_bytes;
 };
 
-static int pick_tile(int cn) {
-  // Two workgroups per CU (160 KB LDS): accumulators + staging must stay under 80 KB.
-  size_t budget = 80 * 1024 - (size_t)kStage * kAStride * 4 - kStage * 4 - 512;
-  int t = (int)(budget / ((size_t)cn * 4));
+static size_t conv_lds_bytes(int T) {
+  return ((size_t)(T + 1) * 68 + 2 * (size_t)kStage * kAStride) * 4 + 4 * kStage * 4 + 32 * 4;
+}
+
+static int pick_tile() {
+  // One workgroup per CU: (almost) all of the 160 KB of LDS goes to the accumulators.
+  size_t budget = 160 * 1024 - conv_lds_bytes(0) - 1024;
+  int t = (int)(budget / (68 * 4));
   t = t / 16 * 16;
-  if (t > 1024) t = 1024;
   if (t < kMinTile) t = kMinTile;
   return t;
 }
 
-static ConvPlan make_plan(int64_t n_out, int c_in, int c_out) {
+static ConvPlan make_plan(int64_t n_out, int K, int c_in, int c_out, int64_t pair_stride) {
   ConvPlan p;
   p.ncb = (int)ceil_div(c_out, 16);
   p.nch = (int)ceil_div(c_in, kKC);
-  p.T = pick_tile(64);
+  p.T = pick_tile();
   p.n_tiles = ceil_div(n_out > 0 ? n_out : 1, p.T);
   p.words_per_k = ceil_div(n_out > 0 ? n_out : 1, 32);
-  p.lds_bytes = ((size_t)p.T * 64 + (size_t)kStage * kAStride) * 4 + kStage * 4;
+  // row blocks: at most one partial block per (tile, offset) on top of pairs / 16
+  int64_t max_pairs_k = pair_stride < n_out ? pair_stride : n_out;
+  p.mb_cap = (int64_t)K * (max_pairs_k / 16 + 1) + p.n_tiles * K;
+  p.lds_bytes = conv_lds_bytes(p.T);
   return p;
 }
 
@@ -308,28 +599,31 @@ struct ConvWs {
   int32_t *sorted;
   uint32_t *bits;
   int32_t *prefix;
+  int32_t *tile_cnt, *kofs, *tile_mb, *sched_in, *sched_out, *sched_k;
 };
 
-static size_t conv_ws_bytes(int64_t n_out, int K, int c_in, int c_out, int64_t pair_stride) {
-  ConvPlan p = make_plan(n_out, c_in, c_out);
-  int64_t tiles_max = ceil_div(n_out > 0 ? n_out : 1, kMinTile);
-  return align_up((size_t)K * p.ncb * p.nch * 1024 * 4) + align_up(4) +
-         align_up((size_t)(tiles_max + 1) * K * 4) + align_up((size_t)K * 2 * pair_stride * 4) +
-         2 * align_up((size_t)K * p.words_per_k * 4);
+static size_t conv_ws_walk(void *base, const ConvPlan &p, int K, int64_t pair_stride, ConvWs *w) {
+  Carver c(base);
+  ConvWs t;
+  t.packed = c.take<float>((size_t)K * p.ncb * p.nch * 1024);
+  t.flag = c.take<int32_t>(1);
+  t.segs = c.take<int32_t>((size_t)(p.n_tiles + 1) * K);
+  t.sorted = c.take<int32_t>((size_t)K * 2 * pair_stride);
+  t.bits = c.take<uint32_t>((size_t)K * p.words_per_k);
+  t.prefix = c.take<int32_t>((size_t)K * p.words_per_k);
+  t.tile_cnt = c.take<int32_t>((size_t)p.n_tiles);
+  t.kofs = c.take<int32_t>((size_t)p.n_tiles * K);
+  t.tile_mb = c.take<int32_t>((size_t)p.n_tiles + 1);
+  t.sched_in = c.take<int32_t>((size_t)p.mb_cap * 16);
+  t.sched_out = c.take<int32_t>((size_t)p.mb_cap * 16);
+  t.sched_k = c.take<int32_t>((size_t)p.mb_cap);
+  if (w) *w = t;
+  return c.used;
 }
 
-static ConvWs conv_ws_carve(void *ws, const ConvPlan &p, int64_t n_out, int K,
-                            int64_t pair_stride) {
-  Carver c(ws);
-  ConvWs w;
-  int64_t tiles_max = ceil_div(n_out > 0 ? n_out : 1, kMinTile);
-  w.packed = c.take<float>((size_t)K * p.ncb * p.nch * 1024);
-  w.flag = c.take<int32_t>(1);
-  w.segs = c.take<int32_t>((size_t)(tiles_max + 1) * K);
-  w.sorted = c.take<int32_t>((size_t)K * 2 * pair_stride);
-  w.bits = c.take<uint32_t>((size_t)K * p.words_per_k);
-  w.prefix = c.take<int32_t>((size_t)K * p.words_per_k);
-  return w;
+static size_t conv_ws_bytes(int64_t n_out, int K, int c_in, int c_out, int64_t pair_stride) {
+  ConvPlan p = make_plan(n_out, K, c_in, c_out, pair_stride);
+  return conv_ws_walk(nullptr, p, K, pair_stride, nullptr);
 }
 
 // Optional timing of the convolution kernel alone: a ring of event pairs recorded
@@ -400,8 +694,9 @@ int ssc_conv_fwd_f32(const float *features, int64_t n_in, int32_t c_in, const fl
   SSC_CHECK(workspace_bytes >= need, SSC_EWORKSPACE, "conv workspace too small: %zu < %zu",
             workspace_bytes, need);
 
-  ConvPlan p = make_plan(n_out, c_in, c_out);
-  ConvWs w = conv_ws_carve(workspace, p, n_out, K, pair_stride);
+  ConvPlan p = make_plan(n_out, K, c_in, c_out, pair_stride);
+  ConvWs w;
+  conv_ws_walk(workspace, p, K, pair_stride, &w);
   const int plane_g = inverse ? 1 : 0;
   const int plane_s = 1 - plane_g;
   int rc;
@@ -417,7 +712,8 @@ int ssc_conv_fwd_f32(const float *features, int64_t n_in, int32_t c_in, const fl
                      pair_num, w.flag);
   SSC_LAUNCH_CHECK("check_sorted");
   int64_t nbits_words = (int64_t)K * p.words_per_k;
-  unsigned clear_blocks = (unsigned)(ceil_div(nbits_words, 256) < 4096 ? ceil_div(nbits_words, 256) : 4096);
+  unsigned clear_blocks =
+      (unsigned)(ceil_div(nbits_words, 256) < 4096 ? ceil_div(nbits_words, 256) : 4096);
   hipLaunchKernelGGL(resort_clear_kernel, dim3(clear_blocks), dim3(256), 0, s, w.flag, w.bits,
                      nbits_words);
   hipLaunchKernelGGL(resort_mark_kernel, pair_grid, dim3(256), 0, s, w.flag, pairs, pair_stride,
@@ -433,10 +729,18 @@ int ssc_conv_fwd_f32(const float *features, int64_t n_in, int32_t c_in, const fl
                      w.flag, pairs, w.sorted, pair_stride, plane_s, pair_num, K, p.n_tiles, p.T,
                      w.segs);
   SSC_LAUNCH_CHECK("tile_segments");
+  hipLaunchKernelGGL(sched_count_kernel, dim3((unsigned)ceil_div(p.n_tiles, 256)), dim3(256), 0, s,
+                     w.segs, K, p.n_tiles, w.tile_cnt, w.kofs);
+  hipLaunchKernelGGL(sched_scan_kernel, dim3(1), dim3(kScanThreads), 0, s, w.tile_cnt, p.n_tiles,
+                     w.tile_mb);
+  hipLaunchKernelGGL(sched_fill_kernel, dim3((unsigned)ceil_div(p.n_tiles * K * 16, 256)),
+                     dim3(256), 0, s, w.flag, pairs, w.sorted, pair_stride, plane_g, w.segs,
+                     w.kofs, w.tile_mb, K, p.n_tiles, p.T, w.sched_in, w.sched_out, w.sched_k);
+  SSC_LAUNCH_CHECK("schedule");
 
   static bool attr_set = false;
   if (!attr_set) {
-    SSC_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(conv_fwd_kernel<4>),
+    SSC_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(conv_fwd_kernel),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
     attr_set = true;
   }
@@ -444,9 +748,9 @@ int ssc_conv_fwd_f32(const float *features, int64_t n_in, int32_t c_in, const fl
   const bool prof = g_profile_on;
   const int slot = g_profile_count % kProfileRing;
   if (prof) SSC_HIP(hipEventRecord(g_profile_ev[slot][0], s));
-  hipLaunchKernelGGL(conv_fwd_kernel<4>, grid, dim3(256), p.lds_bytes, s, features, c_in, w.packed,
-                     w.flag, pairs, w.sorted, pair_stride, plane_g, w.segs, K, p.nch, p.ncb, out,
-                     n_out, c_out, p.T);
+  hipLaunchKernelGGL(conv_fwd_kernel, grid, dim3(512), p.lds_bytes, s, features, c_in, w.packed,
+                     w.sched_in, w.sched_out, w.sched_k, w.tile_mb, p.nch, p.ncb, out, n_out,
+                     c_out, p.T, p.n_tiles);
   SSC_LAUNCH_CHECK("conv_fwd");
   if (prof) {
     SSC_HIP(hipEventRecord(g_profile_ev[slot][1], s));
