@@ -157,14 +157,21 @@ __global__ void __launch_bounds__(256)
 
 // ---- row-block schedule -----------------------------------------------------------------
 // The pairs that land in a tile are cut, offset by offset, into row blocks of 16
-// (the M side of one MFMA); the last block of an offset is padded.  The schedule
-// lists, tile after tile and offset-major inside a tile, for every row block its
-// offset k, its 16 gather rows (-1 = padding) and its 16 tile-local output rows
-// (T = a dummy accumulator row for padding).  The convolution kernel then
-// streams through it without any per-offset bookkeeping.
+// (the M side of one MFMA); the last block of an offset is padded.  Four
+// consecutive row blocks form a group (one pipeline stage per 64-channel chunk
+// of Cin); a tile's last group is padded with empty blocks, and a tile without
+// pairs still gets one empty group so that its rows are written.  The schedule
+// lists, tile after tile and offset-major inside a tile:
+//   sched_in [group*64 + slot]  gather row of the slot            (-1 = padding)
+//   sched_out[group*64 + slot]  tile-local output row of the slot (T  = padding, a dummy row)
+//   sched_id [group*4 + block]  offset k of the block             (-1 = empty block)
+//   grp_tile [group]            tile of the group
+//   grp_last [group]            1 when the group is the last one of its tile
+// The convolution kernel streams through it without per-offset bookkeeping.
 __global__ void __launch_bounds__(256)
     sched_count_kernel(const int32_t *__restrict__ segs, int K, int64_t n_tiles,
-                       int32_t *__restrict__ tile_cnt, int32_t *__restrict__ kofs) {
+                       int32_t *__restrict__ tile_cnt, int32_t *__restrict__ tile_nmb,
+                       int32_t *__restrict__ kofs) {
   int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (t >= n_tiles) return;
   int run = 0;
@@ -173,13 +180,15 @@ __global__ void __launch_bounds__(256)
     kofs[t * K + k] = run;
     run += (n + 15) >> 4;
   }
-  tile_cnt[t] = run;
+  tile_nmb[t] = run;
+  int groups = (run + 3) >> 2;
+  tile_cnt[t] = groups > 0 ? groups : 1;
 }
 
-// tile_mb[0..n_tiles]: exclusive prefix of tile_cnt (one block).
+// tile_grp[0..n_tiles]: exclusive prefix of tile_cnt (one block).
 __global__ void __launch_bounds__(kScanThreads)
     sched_scan_kernel(const int32_t *__restrict__ tile_cnt, int64_t n_tiles,
-                      int32_t *__restrict__ tile_mb) {
+                      int32_t *__restrict__ tile_grp) {
   __shared__ int lds[kScanThreads / 64 + 1];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   int carry = 0;
@@ -202,53 +211,91 @@ __global__ void __launch_bounds__(kScanThreads)
       tot += x;
     }
     __syncthreads();
-    if (i < n_tiles) tile_mb[i] = carry + wave_off + incl - v;
+    if (i < n_tiles) tile_grp[i] = carry + wave_off + incl - v;
     carry += tot;
   }
-  if (threadIdx.x == 0) tile_mb[n_tiles] = carry;
+  if (threadIdx.x == 0) tile_grp[n_tiles] = carry;
 }
 
-// 16 threads per (tile, offset): lane i fills slot i of each of its row blocks.
+// 16 threads per (tile, offset): lane i fills slot i of each of its row blocks; the
+// threads of offset 0 also write the tile's padding blocks and its group -> tile map.
 __global__ void __launch_bounds__(256)
     sched_fill_kernel(const int32_t *__restrict__ flag, const int32_t *__restrict__ pairs,
                       const int32_t *__restrict__ sorted, int64_t pair_stride, int plane_g,
                       const int32_t *__restrict__ segs, const int32_t *__restrict__ kofs,
-                      const int32_t *__restrict__ tile_mb, int K, int64_t n_tiles, int T,
-                      int32_t *__restrict__ sched_in, int32_t *__restrict__ sched_out,
-                      int32_t *__restrict__ sched_k) {
+                      const int32_t *__restrict__ tile_nmb, const int32_t *__restrict__ tile_grp,
+                      int K, int64_t n_tiles, int T, int32_t *__restrict__ sched_in,
+                      int32_t *__restrict__ sched_out, int32_t *__restrict__ sched_id,
+                      int32_t *__restrict__ grp_tile, int32_t *__restrict__ grp_last) {
   int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   int64_t tk = gid >> 4;
   int lane = (int)(gid & 15);
   if (tk >= n_tiles * K) return;
   int64_t t = tk / K;
   int k = (int)(tk - t * K);
+  const int64_t g0 = tile_grp[t], g1 = tile_grp[t + 1];
+  if (k == 0) {
+    for (int64_t g = g0 + lane; g < g1; g += 16) {
+      grp_tile[g] = (int32_t)t;
+      grp_last[g] = g + 1 == g1 ? 1 : 0;
+    }
+    for (int64_t mb = g0 * 4 + tile_nmb[t]; mb < g1 * 4; ++mb) {
+      sched_in[mb * 16 + lane] = -1;
+      sched_out[mb * 16 + lane] = T;
+      if (lane == 0) sched_id[mb] = -1;
+    }
+  }
   const int32_t *src = flag[0] ? sorted : pairs;
   int s0 = segs[t * K + k];
   int n = segs[(t + 1) * K + k] - s0;
   if (n <= 0) return;
   const int32_t *pg = src + ((int64_t)k * 2 + plane_g) * pair_stride + s0;
   const int32_t *ps = src + ((int64_t)k * 2 + (1 - plane_g)) * pair_stride + s0;
-  int64_t mb = (int64_t)tile_mb[t] + kofs[t * K + k];
+  int64_t mb = g0 * 4 + kofs[t * K + k];
   int64_t row0 = t * (int64_t)T;
   for (int p = lane; p < ((n + 15) & ~15); p += 16, ++mb) {
     sched_in[mb * 16 + lane] = p < n ? pg[p] : -1;
     sched_out[mb * 16 + lane] = p < n ? (int)(ps[p] - row0) : T;
-    if (lane == 0) sched_k[mb] = k;
+    if (lane == 0) sched_id[mb] = k;
   }
 }
 
+// Tile range of every persistent workgroup: boundary w is the first tile whose
+// group prefix reaches w/n_wg of all groups, so workgroups get equal work, not
+// equal tile counts.
+__global__ void __launch_bounds__(256)
+    sched_split_kernel(const int32_t *__restrict__ tile_grp, int64_t n_tiles, int n_wg,
+                       int32_t *__restrict__ wg_tile) {
+  int w = blockIdx.x * blockDim.x + threadIdx.x;
+  if (w > n_wg) return;
+  int64_t total = tile_grp[n_tiles];
+  int64_t target = (total * w + n_wg - 1) / n_wg;
+  int64_t lo = 0, hi = n_tiles;
+  while (lo < hi) {
+    int64_t mid = (lo + hi) >> 1;
+    if (tile_grp[mid] < target) lo = mid + 1;
+    else hi = mid;
+  }
+  wg_tile[w] = w == n_wg ? (int32_t)n_tiles : (int32_t)lo;
+}
+
 // ---- the convolution --------------------------------------------------------------------
-// One workgroup = one tile of T output rows x 64 output columns, 8 waves:
-//   waves 0-3  consumers: wave w owns output columns [16w, 16w+16) of the
-//              workgroup's column range and does nothing but LDS reads, MFMAs and
-//              the accumulator update;
-//   waves 4-7  producers: gather the input rows of the NEXT stage from global
-//              memory into LDS (rows are prefetched several stages ahead into
-//              registers), so that address arithmetic and memory latency run on
-//              the same SIMDs underneath the MFMA stream.
-// A stage = 4 consecutive row blocks of the schedule (64 pair slots, any mix of
-// offsets) x one 64-channel chunk of Cin; one barrier per stage hands a filled
-// LDS buffer to the consumers and an emptied one back.
+// Persistent kernel: one workgroup (8 waves) per CU walks a contiguous,
+// work-balanced range of tiles.  A workgroup owns T output rows x CN = 64*CGW
+// output columns at a time; the fp32 accumulators of that tile live in LDS.
+//   waves 0-3  consumers: wave w owns the CGW column groups (16 columns each)
+//              w*CGW .. w*CGW+CGW-1 of the workgroup's column range; it reads
+//              the staged input rows from LDS one row block ahead of the MFMAs
+//              and updates the accumulators;
+//   waves 4-7  producers: gather the input rows of the coming stages from global
+//              memory (several stages ahead, in registers) and stage them in
+//              LDS, so that address arithmetic and memory latency run underneath
+//              the MFMA stream -- across tile boundaries too.
+// A stage = one group of the schedule (4 row blocks = 64 pair slots, any mix of
+// offsets) x one 64-channel chunk of Cin.  One barrier per stage hands the buffer
+// filled with stage s+1 to the consumers and the buffer of stage s back to the
+// producers.  After a tile's last stage all waves write the tile out and clear
+// the accumulators.
 //
 // MFMA orientation: D[16 channels x 16 pairs] = W^T[16 x 4] * F^T[4 x 16], so a
 // lane ends up with 4 consecutive output channels of one pair and adds them to
@@ -257,9 +304,9 @@ __global__ void __launch_bounds__(256)
 // so every output element sees its offsets added in ascending k: reproducible,
 // no atomics.
 //
-// Dynamic LDS: acc[T+1][68] | abuf[2][64][68] | orow[4][64] | ids[4][8]
+// Dynamic LDS: acc[T+1][CN+4] | abuf[2][64][68] | orow[4][64] | ids[4][8]
 // (output rows and fragment ids of a stage are published two stages ahead, in a
-// ring of four, so the consumers know their next stage before its barrier.)
+// ring of four.)
 constexpr int kRowsAhead = 3;  // stages whose gathered rows are in flight in registers
 constexpr int kIdxAhead = 2;   // further stages whose row indices are in flight
 
@@ -274,14 +321,19 @@ __device__ __forceinline__ void mfma_block(const float4v (&b)[4], const float4v 
   }
 }
 
-__global__ void __launch_bounds__(512)
+// Exactly two waves per SIMD (one consumer, one producer): the compiler may use
+// up to 256 VGPRs instead of shrinking the register set for a third wave.
+template <int CGW, bool FULLC>
+__global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))
     conv_fwd_kernel(const float *__restrict__ features, int cin, const float *__restrict__ packed,
                     const int32_t *__restrict__ sched_in, const int32_t *__restrict__ sched_out,
-                    const int32_t *__restrict__ sched_k, const int32_t *__restrict__ tile_mb,
-                    int nch, int ncb, float *__restrict__ out, int64_t n_out, int cout, int T,
-                    int64_t n_tiles) {
-  constexpr int CN = 64;
+                    const int32_t *__restrict__ sched_id, const int32_t *__restrict__ grp_tile,
+                    const int32_t *__restrict__ grp_last, const int32_t *__restrict__ tile_grp,
+                    const int32_t *__restrict__ wg_tile,
+                    int nch, int ncb, float *__restrict__ out, int64_t n_out, int cout, int T) {
+  constexpr int CN = 64 * CGW;
   constexpr int AS = CN + 4;
+  constexpr int NT = 512;
   constexpr int NP = 256;  // producer threads
   constexpr int NE = kStage * 16 / NP;
   extern __shared__ __align__(16) float lds[];
@@ -294,52 +346,87 @@ __global__ void __launch_bounds__(512)
   const int lane = tid & 63;
   const int wave = tid >> 6;
   const bool producer = wave >= 4;
-  // Consecutive workgroup ids land on different XCDs (8 of them, one L2 each):
-  // give every XCD a contiguous range of tiles so neighbouring tiles, which
-  // gather the same input rows, share an L2.
-  int64_t tile = blockIdx.x;
+  // Consecutive workgroup ids land on different XCDs (8 of them, one L2 each): give
+  // every XCD a contiguous run of tile ranges so neighbouring tiles, which gather
+  // the same input rows, share an L2.
+  int chunk = blockIdx.x;
   {
-    const int64_t per = n_tiles / 8;
-    if (tile < per * 8) tile = (tile % 8) * per + tile / 8;
+    const int nwg = gridDim.x;
+    if ((nwg & 7) == 0) chunk = (chunk & 7) * (nwg >> 3) + (chunk >> 3);
   }
-  const int64_t row0 = tile * (int64_t)T;
-  const int mb0 = tile_mb[tile];
-  const int nmb = tile_mb[tile + 1] - mb0;
-  const int nstages = ((nmb + 3) >> 2) * nch;
+  const int t_begin = wg_tile[chunk], t_end = wg_tile[chunk + 1];
+  const int64_t g_begin = tile_grp[t_begin], g_end = tile_grp[t_end];
+  const int nstages = (int)(g_end - g_begin) * nch;  // stages of this workgroup
+  const int col0 = blockIdx.y * CN;
 
   {
     float4v z = {0.f, 0.f, 0.f, 0.f};
     float4v *a4 = reinterpret_cast<float4v *>(acc);
-    for (int i = tid; i < (T + 1) * AS / 4; i += 512) a4[i] = z;
+    for (int i = tid; i < (T + 1) * AS / 4; i += NT) a4[i] = z;
   }
+
+  // Tile `tl` is complete: write its rows, clear the accumulators.
+  auto flush_tile = [&](int tl) {
+    const int64_t row0 = (int64_t)tl * T;
+    if ((cout & 3) == 0) {
+      const float4v z = {0.f, 0.f, 0.f, 0.f};
+      for (int e = tid; e < T * (CN / 4); e += NT) {
+        int r = e / (CN / 4), c4 = e % (CN / 4);
+        int64_t grow = row0 + r;
+        int col = col0 + c4 * 4;
+        float4v *ap = reinterpret_cast<float4v *>(acc + r * AS + c4 * 4);
+        // streaming store: the output is not read again by this kernel and must not
+        // push the weights and the gathered rows out of L2
+        if (grow < n_out && col < cout)
+          __builtin_nontemporal_store(*ap, reinterpret_cast<float4v *>(out + grow * cout + col));
+        *ap = z;
+      }
+    } else {
+      for (int e = tid; e < T * CN; e += NT) {
+        int r = e / CN, c = e % CN;
+        int64_t grow = row0 + r;
+        if (grow < n_out && col0 + c < cout)
+          __builtin_nontemporal_store(acc[r * AS + c], out + grow * cout + col0 + c);
+        acc[r * AS + c] = 0.f;
+      }
+    }
+  };
 
   if (producer) {
     // ------------------------------------------------------------------ producer
+    // At the top of iteration i: rows[j] = stage i+1+j (j < RD), idx[j] = indices of
+    // stage i+1+RD+j (j < ID).  Iteration i stores stage i+1 and the metadata of i+2.
     const int pt = tid - 256;
     const bool vec4 = (cin & 3) == 0;
-    constexpr int RD = kRowsAhead, NS = kRowsAhead + kIdxAhead + 1;
-    int idx[NS][NE];
-    float4v rows[RD + 1][NE];
+    constexpr int RD = kRowsAhead, ID = kIdxAhead;
+    int idx[ID][NE];
+    float4v rows[RD][NE];
+    // Every load below is unconditional (addresses are clamped into range, results
+    // are masked afterwards): a load inside a branch would make every later wait
+    // cover all outstanding loads, which return in order, and so expose the latency
+    // of the prefetches issued last.
+    const int g_last = (int)(g_end - g_begin) - 1;  // >= 0 whenever nstages > 0
     auto load_idx = [&](int s, int (&ix)[NE]) {
-      const int grp = s / nch;
+      const int grp = min(s / nch, g_last < 0 ? 0 : g_last);
+      const int64_t base = (g_begin + grp) * 64;
 #pragma unroll
       for (int j = 0; j < NE; ++j) {
-        int slot = grp * 64 + ((pt + j * NP) >> 4);
-        ix[j] = (s < nstages && slot < nmb * 16) ? sched_in[(int64_t)mb0 * 16 + slot] : -1;
+        int v = sched_in[base + ((pt + j * NP) >> 4)];
+        ix[j] = s < nstages ? v : -1;
       }
     };
     auto load_rows = [&](int s, const int (&ix)[NE], float4v (&r)[NE]) {
       const int cc = s % nch;
 #pragma unroll
       for (int j = 0; j < NE; ++j) {
-        int ch = cc * kKC + ((pt + j * NP) & 15) * 4;
-        float4v v = {0.f, 0.f, 0.f, 0.f};
-#ifdef SSC_DBG_NO_GATHER
-        if (false) {
-#else
-        if (ix[j] >= 0) {
-#endif
-          const float *fp = features + (int64_t)ix[j] * cin + ch;
+        const int ch = cc * kKC + ((pt + j * NP) & 15) * 4;
+        const int row = ix[j] < 0 ? 0 : ix[j];  // padding slots read row 0 and drop it
+        const float *fp = features + (int64_t)row * cin + ch;
+        float4v v;
+        if (FULLC) {
+          v = *reinterpret_cast<const float4v *>(fp);
+        } else {
+          v = float4v{0.f, 0.f, 0.f, 0.f};
           if (vec4) {
             if (ch < cin) v = *reinterpret_cast<const float4v *>(fp);
           } else {
@@ -349,6 +436,7 @@ __global__ void __launch_bounds__(512)
             if (ch + 3 < cin) v.w = fp[3];
           }
         }
+        if (ix[j] < 0) v = float4v{0.f, 0.f, 0.f, 0.f};
         r[j] = v;
       }
     };
@@ -360,235 +448,233 @@ __global__ void __launch_bounds__(512)
         *reinterpret_cast<float4v *>(ab + (e >> 4) * kAStride + (e & 15) * 4) = r[j];
       }
     };
-    // Per-stage metadata handled by threads 0..68: the output row of each of the
-    // 64 slots, the weight-fragment id (k * nch + cc) of the 4 row blocks and of
-    // the first block of the following stage.
+    // Per-stage metadata, one value per thread 0..70: the output row of each of the
+    // 64 slots; the weight-fragment base offset of the 4 row blocks and of the first
+    // block of the following stage; the tile; whether the tile ends here.
     auto load_meta = [&](int s) -> int {
-      const int grp = s / nch;
-      if (pt < kStage) {
-        int slot = grp * 64 + pt;
-        return (s < nstages && slot < nmb * 16) ? sched_out[(int64_t)mb0 * 16 + slot] : T;
-      }
-      if (pt < kStage + 5) {
-        int j = pt - kStage;
-        int s2 = j < 4 ? s : s + 1;
-        int blk = (s2 / nch) * 4 + (j & 3);
-        if (s2 < nstages && blk < nmb) return sched_k[mb0 + blk] * nch + (s2 % nch);
-      }
-      return -1;
+      const int sc = min(s, nstages - 1 < 0 ? 0 : nstages - 1);
+      const int64_t g = g_begin + sc / nch;
+      const int cc = sc % nch;
+      const int sn = min(sc + 1, nstages - 1 < 0 ? 0 : nstages - 1);
+      const int64_t gn = g_begin + sn / nch;
+      // one load per thread, from the array its slot of the metadata comes from
+      const int32_t *src = grp_tile + g;                        // thread 69 (and idle ones)
+      if (pt < kStage) src = sched_out + g * 64 + pt;            // threads 0..63
+      else if (pt < kStage + 4) src = sched_id + g * 4 + (pt - kStage);
+      else if (pt == kStage + 4) src = sched_id + gn * 4;
+      else if (pt == kStage + 6) src = grp_last + g;
+      int v = *src;
+      // fragment base = element offset of (k, column block 0, chunk cc) in `packed`
+      if (pt >= kStage && pt < kStage + 4) v = v >= 0 ? (v * ncb * nch + cc) * 1024 : -1;
+      if (pt == kStage + 4)
+        v = (sc + 1 < nstages && v >= 0) ? (v * ncb * nch + sn % nch) * 1024 : -1;
+      if (pt == kStage + 6) v = (v != 0 && cc == nch - 1) ? 1 : 0;
+      if (s >= nstages) v = pt < kStage ? T : -1;
+      return v;
     };
     auto store_meta = [&](int s, int v) {
       if (pt < kStage) orow[(s & 3) * kStage + pt] = v;
-      else if (pt < kStage + 5) ids[(s & 3) * 8 + (pt - kStage)] = v;
+      else if (pt < kStage + 7) ids[(s & 3) * 8 + (pt - kStage)] = v;
     };
+    {
+      int ix0[NE];
+      float4v r0[NE];
+      load_idx(0, ix0);
 #pragma unroll
-    for (int i = 0; i < NS; ++i) load_idx(i, idx[i]);
+      for (int j = 0; j < RD; ++j) {
+        int ix[NE];
+        load_idx(1 + j, ix);
+        load_rows(1 + j, ix, rows[j]);
+      }
 #pragma unroll
-    for (int i = 0; i <= RD; ++i) load_rows(i, idx[i], rows[i]);
-    store_meta(0, load_meta(0));
-    store_meta(1, load_meta(1));
+      for (int j = 0; j < ID; ++j) load_idx(1 + RD + j, idx[j]);
+      load_rows(0, ix0, r0);
+      store_meta(0, load_meta(0));
+      store_meta(1, load_meta(1));
+      store_rows(0, r0);
+    }
     // metadata is fetched two iterations before it is stored, so that waiting for
     // it never waits for the row loads issued after it (loads return in order)
     int meta0 = load_meta(2), meta1 = load_meta(3);
-    store_rows(0, rows[0]);
     __syncthreads();
     for (int s = 0; s < nstages; ++s) {
-      store_rows(s + 1, rows[1]);
+      store_rows(s + 1, rows[0]);
       store_meta(s + 2, meta0);
       meta0 = meta1;
 #pragma unroll
-      for (int i = 0; i + 1 < NS; ++i)
-#pragma unroll
-        for (int j = 0; j < NE; ++j) idx[i][j] = idx[i + 1][j];
-#pragma unroll
-      for (int i = 1; i < RD; ++i)
+      for (int i = 0; i + 1 < RD; ++i)
 #pragma unroll
         for (int j = 0; j < NE; ++j) rows[i][j] = rows[i + 1][j];
       meta1 = load_meta(s + 4);
-      load_idx(s + NS, idx[NS - 1]);
-      load_rows(s + 1 + RD, idx[RD], rows[RD]);
+      load_rows(s + 1 + RD, idx[0], rows[RD - 1]);
+#pragma unroll
+      for (int i = 0; i + 1 < ID; ++i)
+#pragma unroll
+        for (int j = 0; j < NE; ++j) idx[i][j] = idx[i + 1][j];
+      load_idx(s + 1 + RD + ID, idx[ID - 1]);
       __syncthreads();
+      if (ids[(s & 3) * 8 + 6]) {  // the tile ended with stage s
+        flush_tile(ids[(s & 3) * 8 + 5]);
+        __syncthreads();
+      }
     }
   } else {
     // ------------------------------------------------------------------ consumer
-    const int cg = wave;
     const int g = lane >> 4;
     const int l16 = lane & 15;
-    const int cb = blockIdx.y * 4 + cg;
-    const bool live = cb < ncb;
-    float *acc_lane = acc + cg * 16 + g * 4;
-    auto load_b = [&](int id, float4v (&b)[4]) {
-      // id = k * nch + cc
-      const int k = id / nch, cc = id - k * nch;
-      const float4v *bp = reinterpret_cast<const float4v *>(
-          packed + (((int64_t)k * ncb + cb) * nch + cc) * 1024 + lane * 16);
+    const int cb0 = (blockIdx.y * 4 + wave) * CGW;  // first column block of this wave
+    float *acc_lane = acc + wave * CGW * 16 + g * 4;
+    // A column group beyond Cout multiplies with the last real one's fragments; its
+    // accumulator columns are never written out.  This keeps the code branch-free.
+    const float *bbase[CGW];
 #pragma unroll
-      for (int q = 0; q < 4; ++q) b[q] = bp[q];
+    for (int c = 0; c < CGW; ++c)
+      bbase[c] = packed + (int64_t)min(cb0 + c, ncb - 1) * nch * 1024 + lane * 16;
+    auto load_b = [&](int base, float4v (&b)[CGW][4]) {
+#pragma unroll
+      for (int c = 0; c < CGW; ++c) {
+        const float4v *bp = reinterpret_cast<const float4v *>(bbase[c] + base);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) b[c][q] = bp[q];
+      }
     };
     auto load_a = [&](const float *ab, int m, float4v (&a)[4]) {
       const float4v *ap =
           reinterpret_cast<const float4v *>(ab + (m * 16 + l16) * kAStride + g * 16);
-#ifdef SSC_DBG_NO_A
-      if (n_tiles < 0)
-#endif
 #pragma unroll
       for (int q = 0; q < 4; ++q) a[q] = ap[q];
     };
-    auto accumulate = [&](int ol, const float4v &d) {
-      // d = out[pair l16][channels 4g .. 4g+3] of this column group
-      float4v *ptr = reinterpret_cast<float4v *>(acc_lane + ol * AS);
-#ifdef SSC_DBG_NO_RMW
-      if (d.x == 12345.f) *ptr = d;
-#else
-      *ptr = *ptr + d;
-#endif
+    const bool live = cb0 < ncb;
+    // Two sets of weight fragments, each holding the 4 blocks of one stage.  Stage s
+    // multiplies with one set while ALL fragments of stage s+1 are fetched, in one
+    // unconditional batch at the top of the stage, into the other set: a whole
+    // stage of MFMAs (longer than an L2 round trip under load) lies between the
+    // issue of a load and its first use, and the loads are never inside a branch,
+    // so the compiler's wait counts stay exact.
+    //
+    // Every stage runs the same straight-line code.  An empty row block (only at
+    // the end of a tile) has zeros staged for its slots and the dummy row T as
+    // output row, so its MFMAs add zeros to a row that is never written out.
+    float4v bx[4][CGW][4], by[4][CGW][4];
+    auto stage_ids = [&](int s, int (&id)[4]) {
+      const int *meta = ids + (s & 3) * 8;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        int v = __builtin_amdgcn_readfirstlane(meta[j]);
+        id[j] = (s < nstages && v >= 0) ? v : 0;  // any valid fragment for an empty block
+      }
     };
-    __syncthreads();
-    // Weight fragments are fetched one whole stage ahead: stage s multiplies with
-    // set (s & 1) while the fragments of stage s+1 stream into the other set.
-    // idc = fragment ids of the current stage, idn = of the next one (the ring
-    // publishes them two stages ahead).
-    int idc[5], idn[5];
+    auto load_b_stage = [&](int s, float4v (&b)[4][CGW][4]) {
+      int id[4];
+      stage_ids(s, id);
 #pragma unroll
-    for (int j = 0; j < 5; ++j) {
-      idc[j] = __builtin_amdgcn_readfirstlane(ids[j]);
-      idn[j] = __builtin_amdgcn_readfirstlane(ids[8 + j]);
-    }
-    float4v bx[4][4], by[4][4];
-    // Only the first block of a run of equal ids is fetched; the rest of the run is
-    // filled in by register copies once the data has arrived (fill_b_stage).
-    auto load_b_stage = [&](const int (&id)[5], float4v (&b)[4][4]) {
-#pragma unroll
-      for (int m = 0; m < 4; ++m)
-        if (id[m] >= 0 && (m == 0 || id[m] != id[m - 1])) load_b(id[m], b[m]);
+      for (int m = 0; m < 4; ++m) load_b(id[m], b[m]);
     };
-    auto fill_b_stage = [&](const int (&id)[5], float4v (&b)[4][4]) {
-#pragma unroll
-      for (int m = 1; m < 4; ++m)
-        if (id[m] >= 0 && id[m] == id[m - 1]) {
-#pragma unroll
-          for (int q = 0; q < 4; ++q) b[m][q] = b[m - 1][q];
-        }
-    };
-    // one stage out of LDS buffer (s & 1) with fragment set b; prefetches bn for s+1
-    auto run_stage = [&](int s, float4v (&b)[4][4], float4v (&bn)[4][4]) {
+    auto run_stage = [&](int s, float4v (&bc)[4][CGW][4], float4v (&bn)[4][CGW][4]) {
+      load_b_stage(s + 1, bn);  // the ring publishes a stage's ids two stages ahead
+      // keep the batch here: the scheduler would otherwise sink these loads to the
+      // end of the stage to shorten register live ranges, which exposes their latency
+      __builtin_amdgcn_sched_barrier(0);
       const float *ab = abuf + (s & 1) * kStage * kAStride;
       const int *orw = orow + (s & 3) * kStage;
-      load_b_stage(idn, bn);
-      if (idc[3] >= 0) {
-        // full stage: straight-line code so LDS reads, MFMAs and accumulator updates
-        // of neighbouring row blocks can be interleaved by the scheduler
-        float4v a[4][4];
-        int ol[4];
-        float4v d[4];
+      float4v a[2][4];
+      load_a(ab, 0, a[0]);
+      int ol[4];
 #pragma unroll
-        for (int m = 0; m < 4; ++m) {
-          load_a(ab, m, a[m]);
-          ol[m] = orw[m * 16 + l16];
+      for (int m = 0; m < 4; ++m) ol[m] = orw[m * 16 + l16];
+#pragma unroll
+      for (int m = 0; m < 4; ++m) {
+        if (m < 3) load_a(ab, m + 1, a[(m + 1) & 1]);
+        // accumulator rows of this block: read before the MFMAs, added after
+        float4v accr[CGW], d[CGW];
+#pragma unroll
+        for (int c = 0; c < CGW; ++c) {
+          accr[c] = *reinterpret_cast<const float4v *>(acc_lane + ol[m] * AS + c * 16);
+          d[c] = float4v{0.f, 0.f, 0.f, 0.f};
         }
 #pragma unroll
-        for (int m = 0; m < 4; ++m) {
-          d[m] = float4v{0.f, 0.f, 0.f, 0.f};
-          mfma_block(b[m], a[m], d[m]);
-          accumulate(ol[m], d[m]);
-        }
-      } else {
-        // last, partial stage of the tile
+        for (int c = 0; c < CGW; ++c) mfma_block(bc[m][c], a[m & 1], d[c]);
+        // d[c] = out[pair l16][channels 4g .. 4g+3] of column group c of this wave
 #pragma unroll
-        for (int m = 0; m < 3; ++m) {
-          if (idc[m] >= 0) {
-            float4v a[4];
-            load_a(ab, m, a);
-            const int ol = orw[m * 16 + l16];
-            float4v d = {0.f, 0.f, 0.f, 0.f};
-            mfma_block(b[m], a, d);
-            accumulate(ol, d);
-          }
-        }
-      }
-      fill_b_stage(idn, bn);
-      const int *nx = ids + ((s + 2) & 3) * 8;
-#pragma unroll
-      for (int j = 0; j < 5; ++j) {
-        idc[j] = idn[j];
-        idn[j] = __builtin_amdgcn_readfirstlane(nx[j]);
+        for (int c = 0; c < CGW; ++c)
+          *reinterpret_cast<float4v *>(acc_lane + ol[m] * AS + c * 16) = accr[c] + d[c];
       }
     };
-    if (live) {
-      load_b_stage(idc, bx);
-      fill_b_stage(idc, bx);
-    }
+    __syncthreads();
+    if (live && nstages > 0) load_b_stage(0, bx);
     for (int s = 0; s < nstages; s += 2) {
-#ifdef SSC_DBG_NO_MFMA
-      if (false) {
-#else
-      if (live) {
-#endif
-        run_stage(s, bx, by);
-      }
+      if (live) run_stage(s, bx, by);
+      int tl = ids[(s & 3) * 8 + 5], last = ids[(s & 3) * 8 + 6];
       __syncthreads();
-      if (s + 1 < nstages) {
-#ifdef SSC_DBG_NO_MFMA
-        if (false) {
-#else
-        if (live) {
-#endif
-          run_stage(s + 1, by, bx);
-        }
+      if (last) {
+        flush_tile(tl);
         __syncthreads();
       }
-    }
-  }
-  // write the tile
-  const int col0 = blockIdx.y * CN;
-  if ((cout & 3) == 0) {
-    for (int e = tid; e < T * (CN / 4); e += 512) {
-      int r = e / (CN / 4), c4 = e % (CN / 4);
-      int64_t grow = row0 + r;
-      int col = col0 + c4 * 4;
-      if (grow < n_out && col < cout)
-        *reinterpret_cast<float4v *>(out + grow * cout + col) =
-            *reinterpret_cast<const float4v *>(acc + r * AS + c4 * 4);
-    }
-  } else {
-    for (int e = tid; e < T * CN; e += 512) {
-      int r = e / CN, c = e % CN;
-      int64_t grow = row0 + r;
-      if (grow < n_out && col0 + c < cout) out[grow * cout + col0 + c] = acc[r * AS + c];
+      if (s + 1 < nstages) {
+        if (live) run_stage(s + 1, by, bx);
+        tl = ids[((s + 1) & 3) * 8 + 5];
+        last = ids[((s + 1) & 3) * 8 + 6];
+        __syncthreads();
+        if (last) {
+          flush_tile(tl);
+          __syncthreads();
+        }
+      }
     }
   }
 }
 
 struct ConvPlan {
-  int ncb, nch, T;
-  int64_t n_tiles, words_per_k, mb_cap;
+  int ncb, nch, T, cgw, n_wg, n_colblk;
+  int64_t n_tiles, words_per_k, grp_cap;
   size_t lds_bytes;
 };
 
-static size_t conv_lds_bytes(int T) {
-  return ((size_t)(T + 1) * 68 + 2 * (size_t)kStage * kAStride) * 4 + 4 * kStage * 4 + 32 * 4;
+static size_t conv_lds_bytes(int T, int cgw) {
+  return ((size_t)(T + 1) * (cgw * 64 + 4) + 2 * (size_t)kStage * kAStride) * 4 +
+         4 * kStage * 4 + 32 * 4;
 }
 
-static int pick_tile() {
+static int pick_tile(int cgw) {
   // One workgroup per CU: (almost) all of the 160 KB of LDS goes to the accumulators.
-  size_t budget = 160 * 1024 - conv_lds_bytes(0) - 1024;
-  int t = (int)(budget / (68 * 4));
-  t = t / 16 * 16;
+  size_t budget = 160 * 1024 - conv_lds_bytes(0, cgw) - 512;
+  int t = (int)(budget / ((size_t)(cgw * 64 + 4) * 4));
+  t = t / 8 * 8;
   if (t < kMinTile) t = kMinTile;
   return t;
+}
+
+static int device_cu_count() {
+  static int cus = 0;
+  if (cus == 0) {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
+      cus = prop.multiProcessorCount;
+    if (cus <= 0) cus = 256;
+  }
+  return cus;
 }
 
 static ConvPlan make_plan(int64_t n_out, int K, int c_in, int c_out, int64_t pair_stride) {
   ConvPlan p;
   p.ncb = (int)ceil_div(c_out, 16);
   p.nch = (int)ceil_div(c_in, kKC);
-  p.T = pick_tile();
+  p.cgw = 1;  // 64-column tiles: two full-stage sets of weight fragments fit the registers
+  p.T = pick_tile(p.cgw);
   p.n_tiles = ceil_div(n_out > 0 ? n_out : 1, p.T);
   p.words_per_k = ceil_div(n_out > 0 ? n_out : 1, 32);
-  // row blocks: at most one partial block per (tile, offset) on top of pairs / 16
+  // groups: pairs/64 plus, per (tile, offset), up to one partial block, plus one
+  // partial (or empty) group per tile
   int64_t max_pairs_k = pair_stride < n_out ? pair_stride : n_out;
-  p.mb_cap = (int64_t)K * (max_pairs_k / 16 + 1) + p.n_tiles * K;
-  p.lds_bytes = conv_lds_bytes(p.T);
+  p.grp_cap = ((int64_t)K * (max_pairs_k / 16 + 1) + p.n_tiles * K) / 4 + 2 * p.n_tiles + 4;
+  p.n_colblk = (int)ceil_div(p.ncb, 4 * p.cgw);
+  int n_wg = device_cu_count() / p.n_colblk;
+  if (n_wg < 1) n_wg = 1;
+  if (n_wg > p.n_tiles) n_wg = (int)p.n_tiles;
+  if (n_wg >= 8) n_wg = n_wg / 8 * 8;
+  p.n_wg = n_wg;
+  p.lds_bytes = conv_lds_bytes(p.T, p.cgw);
   return p;
 }
 
@@ -599,7 +685,8 @@ struct ConvWs {
   int32_t *sorted;
   uint32_t *bits;
   int32_t *prefix;
-  int32_t *tile_cnt, *kofs, *tile_mb, *sched_in, *sched_out, *sched_k;
+  int32_t *tile_cnt, *tile_nmb, *kofs, *tile_grp, *wg_tile;
+  int32_t *sched_in, *sched_out, *sched_id, *grp_tile, *grp_last;
 };
 
 static size_t conv_ws_walk(void *base, const ConvPlan &p, int K, int64_t pair_stride, ConvWs *w) {
@@ -612,11 +699,15 @@ static size_t conv_ws_walk(void *base, const ConvPlan &p, int K, int64_t pair_st
   t.bits = c.take<uint32_t>((size_t)K * p.words_per_k);
   t.prefix = c.take<int32_t>((size_t)K * p.words_per_k);
   t.tile_cnt = c.take<int32_t>((size_t)p.n_tiles);
+  t.tile_nmb = c.take<int32_t>((size_t)p.n_tiles);
   t.kofs = c.take<int32_t>((size_t)p.n_tiles * K);
-  t.tile_mb = c.take<int32_t>((size_t)p.n_tiles + 1);
-  t.sched_in = c.take<int32_t>((size_t)p.mb_cap * 16);
-  t.sched_out = c.take<int32_t>((size_t)p.mb_cap * 16);
-  t.sched_k = c.take<int32_t>((size_t)p.mb_cap);
+  t.tile_grp = c.take<int32_t>((size_t)p.n_tiles + 1);
+  t.wg_tile = c.take<int32_t>((size_t)p.n_wg + 1);
+  t.sched_in = c.take<int32_t>((size_t)p.grp_cap * 64);
+  t.sched_out = c.take<int32_t>((size_t)p.grp_cap * 64);
+  t.sched_id = c.take<int32_t>((size_t)p.grp_cap * 4);
+  t.grp_tile = c.take<int32_t>((size_t)p.grp_cap);
+  t.grp_last = c.take<int32_t>((size_t)p.grp_cap);
   if (w) *w = t;
   return c.used;
 }
@@ -624,6 +715,23 @@ static size_t conv_ws_walk(void *base, const ConvPlan &p, int K, int64_t pair_st
 static size_t conv_ws_bytes(int64_t n_out, int K, int c_in, int c_out, int64_t pair_stride) {
   ConvPlan p = make_plan(n_out, K, c_in, c_out, pair_stride);
   return conv_ws_walk(nullptr, p, K, pair_stride, nullptr);
+}
+
+template <int CGW, bool FULLC>
+static int launch_conv(const ConvPlan &p, const ConvWs &w, const float *features, int c_in,
+                       float *out, int64_t n_out, int c_out, hipStream_t s) {
+  static bool attr_set = false;
+  if (!attr_set) {
+    SSC_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(conv_fwd_kernel<CGW, FULLC>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+    attr_set = true;
+  }
+  dim3 grid((unsigned)p.n_wg, (unsigned)p.n_colblk);
+  hipLaunchKernelGGL((conv_fwd_kernel<CGW, FULLC>), grid, dim3(512), p.lds_bytes, s, features,
+                     c_in, w.packed, w.sched_in, w.sched_out, w.sched_id, w.grp_tile, w.grp_last,
+                     w.tile_grp, w.wg_tile, p.nch, p.ncb, out, n_out, c_out, p.T);
+  SSC_LAUNCH_CHECK("conv_fwd");
+  return SSC_OK;
 }
 
 // Optional timing of the convolution kernel alone: a ring of event pairs recorded
@@ -730,28 +838,29 @@ int ssc_conv_fwd_f32(const float *features, int64_t n_in, int32_t c_in, const fl
                      w.segs);
   SSC_LAUNCH_CHECK("tile_segments");
   hipLaunchKernelGGL(sched_count_kernel, dim3((unsigned)ceil_div(p.n_tiles, 256)), dim3(256), 0, s,
-                     w.segs, K, p.n_tiles, w.tile_cnt, w.kofs);
+                     w.segs, K, p.n_tiles, w.tile_cnt, w.tile_nmb, w.kofs);
   hipLaunchKernelGGL(sched_scan_kernel, dim3(1), dim3(kScanThreads), 0, s, w.tile_cnt, p.n_tiles,
-                     w.tile_mb);
+                     w.tile_grp);
   hipLaunchKernelGGL(sched_fill_kernel, dim3((unsigned)ceil_div(p.n_tiles * K * 16, 256)),
                      dim3(256), 0, s, w.flag, pairs, w.sorted, pair_stride, plane_g, w.segs,
-                     w.kofs, w.tile_mb, K, p.n_tiles, p.T, w.sched_in, w.sched_out, w.sched_k);
+                     w.kofs, w.tile_nmb, w.tile_grp, K, p.n_tiles, p.T, w.sched_in, w.sched_out,
+                     w.sched_id, w.grp_tile, w.grp_last);
+  hipLaunchKernelGGL(sched_split_kernel, dim3((unsigned)ceil_div(p.n_wg + 1, 256)), dim3(256), 0,
+                     s, w.tile_grp, p.n_tiles, p.n_wg, w.wg_tile);
   SSC_LAUNCH_CHECK("schedule");
 
-  static bool attr_set = false;
-  if (!attr_set) {
-    SSC_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(conv_fwd_kernel),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
-    attr_set = true;
-  }
-  dim3 grid((unsigned)p.n_tiles, (unsigned)ceil_div(p.ncb, 4));
   const bool prof = g_profile_on;
   const int slot = g_profile_count % kProfileRing;
   if (prof) SSC_HIP(hipEventRecord(g_profile_ev[slot][0], s));
-  hipLaunchKernelGGL(conv_fwd_kernel, grid, dim3(512), p.lds_bytes, s, features, c_in, w.packed,
-                     w.sched_in, w.sched_out, w.sched_k, w.tile_mb, p.nch, p.ncb, out, n_out,
-                     c_out, p.T, p.n_tiles);
-  SSC_LAUNCH_CHECK("conv_fwd");
+  // FULLC: Cin is a multiple of 64, so every channel chunk is complete
+  const bool fullc = (c_in % kKC) == 0;
+  if (p.cgw == 2)
+    rc = fullc ? launch_conv<2, true>(p, w, features, c_in, out, n_out, c_out, s)
+               : launch_conv<2, false>(p, w, features, c_in, out, n_out, c_out, s);
+  else
+    rc = fullc ? launch_conv<1, true>(p, w, features, c_in, out, n_out, c_out, s)
+               : launch_conv<1, false>(p, w, features, c_in, out, n_out, c_out, s);
+  if (rc != SSC_OK) return rc;
   if (prof) {
     SSC_HIP(hipEventRecord(g_profile_ev[slot][1], s));
     ++g_profile_count;
