@@ -26,7 +26,7 @@ FP32_MFMA_PEAK_TFLOPS = 157.3  # MI355X dense fp32 matrix peak
 # HBM bytes per launch of the convolution kernel, from rocprofv3 --pmc
 # FETCH_SIZE / WRITE_SIZE runs scaled by a copy kernel of known size
 # (summaries under profiles/); None until measured for a workload.
-MEASURED_TRAFFIC_BYTES = {}
+MEASURED_TRAFFIC_BYTES = {"cfg2": int((19324.3 * 2.0 + 300076.5) * 1024)}
 
 
 def parse_args():
@@ -37,6 +37,10 @@ def parse_args():
     ap.add_argument("--workload", default="cfg2", choices=["cfg1", "cfg2", "cfg3", "cfg5"])
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibration-copy", type=int, default=0, metavar="MIB",
+                    help="also run one plain device copy of MIB mebibytes before the timed "
+                         "region (the known-size kernel that scales rocprofv3's FETCH_SIZE / "
+                         "WRITE_SIZE counters)")
     ap.add_argument("--breakdown", action="store_true",
                     help="also print per-phase timings to stderr")
     return ap.parse_args()
@@ -120,6 +124,13 @@ def main():
     for _ in range(args.warmup):
         out = step()
     torch.cuda.synchronize()
+    if args.calibration_copy > 0:
+        src = torch.ones(args.calibration_copy << 18, dtype=torch.float32, device=dev)
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     _ext.profile_conv(True)
     torch.cuda.synchronize()
