@@ -13,9 +13,12 @@
 // bit-reproducible without atomics.
 #include "ssc_common.h"
 
+#include <type_traits>
+
 namespace ssc {
 
 typedef float float4v __attribute__((ext_vector_type(4)));
+typedef int int4v __attribute__((ext_vector_type(4)));
 
 constexpr int kKC = 64;       // input channels per chunk = 16 MFMA steps of 4
 constexpr int kStage = 64;    // pairs staged per barrier = 4 row blocks of 16
@@ -162,11 +165,12 @@ __global__ void __launch_bounds__(256)
 // of Cin); a tile's last group is padded with empty blocks, and a tile without
 // pairs still gets one empty group so that its rows are written.  The schedule
 // lists, tile after tile and offset-major inside a tile:
-//   sched_in [group*64 + slot]  gather row of the slot            (-1 = padding)
-//   sched_out[group*64 + slot]  tile-local output row of the slot (T  = padding, a dummy row)
-//   sched_id [group*4 + block]  offset k of the block             (-1 = empty block)
-//   grp_tile [group]            tile of the group
-//   grp_last [group]            1 when the group is the last one of its tile
+//   sched_in [group*64 + slot]  gather row of the slot times in_scale (in_pad = padding):
+//                               the row number, or the byte offset of the row
+//   sched_out[group*64 + slot]  byte offset of the slot's accumulator row in the tile
+//                               (tile-local row * out_scale; row T, a dummy, = padding)
+//   grp_meta [group*8 + ...]    0..3 offset k of the 4 blocks (-1 = empty block),
+//                               4 tile of the group, 5 1 when it is the tile's last group
 // The convolution kernel streams through it without per-offset bookkeeping.
 __global__ void __launch_bounds__(256)
     sched_count_kernel(const int32_t *__restrict__ segs, int K, int64_t n_tiles,
@@ -224,9 +228,9 @@ __global__ void __launch_bounds__(256)
                       const int32_t *__restrict__ sorted, int64_t pair_stride, int plane_g,
                       const int32_t *__restrict__ segs, const int32_t *__restrict__ kofs,
                       const int32_t *__restrict__ tile_nmb, const int32_t *__restrict__ tile_grp,
-                      int K, int64_t n_tiles, int T, int32_t *__restrict__ sched_in,
-                      int32_t *__restrict__ sched_out, int32_t *__restrict__ sched_id,
-                      int32_t *__restrict__ grp_tile, int32_t *__restrict__ grp_last) {
+                      int K, int64_t n_tiles, int T, uint32_t in_scale, uint32_t in_pad,
+                      int out_scale, int32_t *__restrict__ sched_in,
+                      int32_t *__restrict__ sched_out, int32_t *__restrict__ grp_meta) {
   int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   int64_t tk = gid >> 4;
   int lane = (int)(gid & 15);
@@ -236,13 +240,15 @@ __global__ void __launch_bounds__(256)
   const int64_t g0 = tile_grp[t], g1 = tile_grp[t + 1];
   if (k == 0) {
     for (int64_t g = g0 + lane; g < g1; g += 16) {
-      grp_tile[g] = (int32_t)t;
-      grp_last[g] = g + 1 == g1 ? 1 : 0;
+      grp_meta[g * 8 + 4] = (int32_t)t;
+      grp_meta[g * 8 + 5] = g + 1 == g1 ? 1 : 0;
+      grp_meta[g * 8 + 6] = 0;
+      grp_meta[g * 8 + 7] = 0;
     }
     for (int64_t mb = g0 * 4 + tile_nmb[t]; mb < g1 * 4; ++mb) {
-      sched_in[mb * 16 + lane] = -1;
-      sched_out[mb * 16 + lane] = T;
-      if (lane == 0) sched_id[mb] = -1;
+      sched_in[mb * 16 + lane] = (int32_t)in_pad;
+      sched_out[mb * 16 + lane] = T * out_scale;
+      if (lane == 0) grp_meta[(mb >> 2) * 8 + (mb & 3)] = -1;
     }
   }
   const int32_t *src = flag[0] ? sorted : pairs;
@@ -254,9 +260,9 @@ __global__ void __launch_bounds__(256)
   int64_t mb = g0 * 4 + kofs[t * K + k];
   int64_t row0 = t * (int64_t)T;
   for (int p = lane; p < ((n + 15) & ~15); p += 16, ++mb) {
-    sched_in[mb * 16 + lane] = p < n ? pg[p] : -1;
-    sched_out[mb * 16 + lane] = p < n ? (int)(ps[p] - row0) : T;
-    if (lane == 0) sched_id[mb] = k;
+    sched_in[mb * 16 + lane] = p < n ? (int32_t)((uint32_t)pg[p] * in_scale) : (int32_t)in_pad;
+    sched_out[mb * 16 + lane] = (p < n ? (int)(ps[p] - row0) : T) * out_scale;
+    if (lane == 0) grp_meta[(mb >> 2) * 8 + (mb & 3)] = k;
   }
 }
 
@@ -281,21 +287,30 @@ __global__ void __launch_bounds__(256)
 
 // ---- the convolution --------------------------------------------------------------------
 // Persistent kernel: one workgroup (8 waves) per CU walks a contiguous,
-// work-balanced range of tiles.  A workgroup owns T output rows x CN = 64*CGW
-// output columns at a time; the fp32 accumulators of that tile live in LDS.
-//   waves 0-3  consumers: wave w owns the CGW column groups (16 columns each)
-//              w*CGW .. w*CGW+CGW-1 of the workgroup's column range; it reads
-//              the staged input rows from LDS one row block ahead of the MFMAs
-//              and updates the accumulators;
+// work-balanced range of tiles.  A workgroup owns T output rows x 64 output
+// columns at a time; the fp32 accumulators of that tile live in LDS.
+//   waves 0-3  consumers: wave w owns 16 columns of the workgroup's column range.
+//              It multiplies the staged input rows of a stage with the weight
+//              fragments of its columns and adds the products to the accumulators.
 //   waves 4-7  producers: gather the input rows of the coming stages from global
-//              memory (several stages ahead, in registers) and stage them in
-//              LDS, so that address arithmetic and memory latency run underneath
-//              the MFMA stream -- across tile boundaries too.
+//              memory (several stages ahead, in registers) and stage them in LDS.
 // A stage = one group of the schedule (4 row blocks = 64 pair slots, any mix of
 // offsets) x one 64-channel chunk of Cin.  One barrier per stage hands the buffer
 // filled with stage s+1 to the consumers and the buffer of stage s back to the
 // producers.  After a tile's last stage all waves write the tile out and clear
 // the accumulators.
+//
+// fp32 MFMAs and ordinary vector-ALU instructions do not overlap on a SIMD, no
+// matter which wave issues them (measured: every VALU instruction next to a
+// stream of v_mfma_f32_16x16x4_f32 costs about five cycles of matrix time), while
+// scalar, LDS and memory instructions of another wave are free.  So the loops
+// below keep vector arithmetic out of the steady state: the schedule already
+// holds byte offsets, addresses are (scalar offset + constant lane offset) of
+// buffer loads, per-stage bookkeeping is scalar loads and scalar arithmetic, and
+// the producers do not touch the VALU except for one add per gathered row chunk.
+// Buffer loads are range-checked by the hardware and return zero outside their
+// buffer: padding slots carry an offset beyond the features and gather zeros,
+// and the prefetches that run past the end of a workgroup's schedule are harmless.
 //
 // MFMA orientation: D[16 channels x 16 pairs] = W^T[16 x 4] * F^T[4 x 16], so a
 // lane ends up with 4 consecutive output channels of one pair and adds them to
@@ -304,47 +319,67 @@ __global__ void __launch_bounds__(256)
 // so every output element sees its offsets added in ascending k: reproducible,
 // no atomics.
 //
-// Dynamic LDS: acc[T+1][CN+4] | abuf[2][64][68] | orow[4][64] | ids[4][8]
-// (output rows and fragment ids of a stage are published two stages ahead, in a
-// ring of four.)
-constexpr int kRowsAhead = 3;  // stages whose gathered rows are in flight in registers
-constexpr int kIdxAhead = 2;   // further stages whose row indices are in flight
+// Dynamic LDS: acc[T+1][68] | abuf[2][64][68]
+constexpr int kCN = 64;        // output columns per workgroup
+constexpr int kAS = kCN + 4;   // accumulator row stride in floats
+constexpr int kRowsAhead = 4;  // stages whose gathered rows are in flight in registers
+constexpr int kIdxAhead = 2;   // further stages whose gather offsets are in flight
+constexpr unsigned kGatherPad = 0xFFFFF000u;  // gather offset of a padding slot (FAST)
+constexpr int kRsrcFlags = 0x00020000;        // raw buffer of 32-bit data
 
-__device__ __forceinline__ void mfma_block(const float4v (&b)[4], const float4v (&a)[4],
-                                           float4v &d) {
-#pragma unroll
-  for (int q = 0; q < 4; ++q) {
-    d = __builtin_amdgcn_mfma_f32_16x16x4f32(b[q].x, a[q].x, d, 0, 0, 0);
-    d = __builtin_amdgcn_mfma_f32_16x16x4f32(b[q].y, a[q].y, d, 0, 0, 0);
-    d = __builtin_amdgcn_mfma_f32_16x16x4f32(b[q].z, a[q].z, d, 0, 0, 0);
-    d = __builtin_amdgcn_mfma_f32_16x16x4f32(b[q].w, a[q].w, d, 0, 0, 0);
-  }
+__device__ __forceinline__ void mfma_quad(const float4v &b, const float4v &a, float4v &d) {
+  d = __builtin_amdgcn_mfma_f32_16x16x4f32(b.x, a.x, d, 0, 0, 0);
+  d = __builtin_amdgcn_mfma_f32_16x16x4f32(b.y, a.y, d, 0, 0, 0);
+  d = __builtin_amdgcn_mfma_f32_16x16x4f32(b.z, a.z, d, 0, 0, 0);
+  d = __builtin_amdgcn_mfma_f32_16x16x4f32(b.w, a.w, d, 0, 0, 0);
 }
 
+__device__ __forceinline__ float4v buf_load4(__amdgpu_buffer_rsrc_t r, int voff, int soff) {
+  return __builtin_bit_cast(float4v, __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, 0));
+}
+__device__ __forceinline__ int buf_load1(__amdgpu_buffer_rsrc_t r, int voff, int soff) {
+  return (int)__builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, 0);
+}
+
+// Position of a stage in the schedule: group index and channel chunk.  Advanced
+// with scalar arithmetic only.
+struct StagePos {
+  int g, cc;
+  __device__ __forceinline__ void advance(int nch) {
+    ++cc;
+    if (cc == nch) {
+      cc = 0;
+      ++g;
+    }
+  }
+};
+
+// FAST: Cin is a multiple of 64 and the features are smaller than 4 GiB; the
+// schedule then holds byte offsets of the gather rows and the gather is a
+// range-checked buffer load.  Otherwise the schedule holds row numbers and the
+// gather uses 64-bit addresses with per-channel masks.
+//
 // Exactly two waves per SIMD (one consumer, one producer): the compiler may use
 // up to 256 VGPRs instead of shrinking the register set for a third wave.
-template <int CGW, bool FULLC>
+template <bool FAST>
 __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))
-    conv_fwd_kernel(const float *__restrict__ features, int cin, const float *__restrict__ packed,
+    conv_fwd_kernel(const float *__restrict__ features, int cin, unsigned feat_bytes,
+                    const float *__restrict__ packed, unsigned packed_bytes,
                     const int32_t *__restrict__ sched_in, const int32_t *__restrict__ sched_out,
-                    const int32_t *__restrict__ sched_id, const int32_t *__restrict__ grp_tile,
-                    const int32_t *__restrict__ grp_last, const int32_t *__restrict__ tile_grp,
-                    const int32_t *__restrict__ wg_tile,
-                    int nch, int ncb, float *__restrict__ out, int64_t n_out, int cout, int T) {
-  constexpr int CN = 64 * CGW;
-  constexpr int AS = CN + 4;
+                    const int32_t *__restrict__ grp_meta, unsigned sched_bytes, unsigned meta_bytes,
+                    const int32_t *__restrict__ tile_grp, const int32_t *__restrict__ wg_tile,
+                    int nch, int ncb, int kvol, float *__restrict__ out, int64_t n_out, int cout,
+                    int T) {
   constexpr int NT = 512;
   constexpr int NP = 256;  // producer threads
   constexpr int NE = kStage * 16 / NP;
   extern __shared__ __align__(16) float lds[];
   float *acc = lds;
-  float *abuf = acc + (size_t)(T + 1) * AS;
-  int *orow = reinterpret_cast<int *>(abuf + 2 * kStage * kAStride);
-  int *ids = orow + 4 * kStage;
+  float *abuf = acc + (size_t)(T + 1) * kAS;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const bool producer = wave >= 4;
   // Consecutive workgroup ids land on different XCDs (8 of them, one L2 each): give
   // every XCD a contiguous run of tile ranges so neighbouring tiles, which gather
@@ -355,14 +390,14 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
     if ((nwg & 7) == 0) chunk = (chunk & 7) * (nwg >> 3) + (chunk >> 3);
   }
   const int t_begin = wg_tile[chunk], t_end = wg_tile[chunk + 1];
-  const int64_t g_begin = tile_grp[t_begin], g_end = tile_grp[t_end];
-  const int nstages = (int)(g_end - g_begin) * nch;  // stages of this workgroup
-  const int col0 = blockIdx.y * CN;
+  const int g_begin = tile_grp[t_begin], g_end = tile_grp[t_end];
+  const int nstages = (g_end - g_begin) * nch;  // stages of this workgroup
+  const int col0 = blockIdx.y * kCN;
 
   {
     float4v z = {0.f, 0.f, 0.f, 0.f};
     float4v *a4 = reinterpret_cast<float4v *>(acc);
-    for (int i = tid; i < (T + 1) * AS / 4; i += NT) a4[i] = z;
+    for (int i = tid; i < (T + 1) * kAS / 4; i += NT) a4[i] = z;
   }
 
   // Tile `tl` is complete: write its rows, clear the accumulators.
@@ -370,11 +405,11 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
     const int64_t row0 = (int64_t)tl * T;
     if ((cout & 3) == 0) {
       const float4v z = {0.f, 0.f, 0.f, 0.f};
-      for (int e = tid; e < T * (CN / 4); e += NT) {
-        int r = e / (CN / 4), c4 = e % (CN / 4);
+      for (int e = tid; e < T * (kCN / 4); e += NT) {
+        int r = e / (kCN / 4), c4 = e % (kCN / 4);
         int64_t grow = row0 + r;
         int col = col0 + c4 * 4;
-        float4v *ap = reinterpret_cast<float4v *>(acc + r * AS + c4 * 4);
+        float4v *ap = reinterpret_cast<float4v *>(acc + r * kAS + c4 * 4);
         // streaming store: the output is not read again by this kernel and must not
         // push the weights and the gathered rows out of L2
         if (grow < n_out && col < cout)
@@ -382,52 +417,60 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
         *ap = z;
       }
     } else {
-      for (int e = tid; e < T * CN; e += NT) {
-        int r = e / CN, c = e % CN;
+      for (int e = tid; e < T * kCN; e += NT) {
+        int r = e / kCN, c = e % kCN;
         int64_t grow = row0 + r;
         if (grow < n_out && col0 + c < cout)
-          __builtin_nontemporal_store(acc[r * AS + c], out + grow * cout + col0 + c);
-        acc[r * AS + c] = 0.f;
+          __builtin_nontemporal_store(acc[r * kAS + c], out + grow * cout + col0 + c);
+        acc[r * kAS + c] = 0.f;
       }
     }
+  };
+  // The tile of stage `pos` ends with it when the group is the tile's last one and
+  // the chunk is the last chunk.  Scalar loads: the address is uniform.
+  auto tile_end = [&](const StagePos &pos, int &tile) -> bool {
+    const int32_t *m = grp_meta + (int64_t)pos.g * 8;
+    tile = m[4];
+    return m[5] != 0 && pos.cc == nch - 1;
   };
 
   if (producer) {
     // ------------------------------------------------------------------ producer
-    // At the top of iteration i: rows[j] = stage i+1+j (j < RD), idx[j] = indices of
-    // stage i+1+RD+j (j < ID).  Iteration i stores stage i+1 and the metadata of i+2.
     const int pt = tid - 256;
-    const bool vec4 = (cin & 3) == 0;
     constexpr int RD = kRowsAhead, ID = kIdxAhead;
+    static_assert(RD == 4 && ID == 2, "the rings below are sized for these distances");
+    const __amdgpu_buffer_rsrc_t rs_in =
+        __builtin_amdgcn_make_buffer_rsrc((void *)sched_in, 0, (int)sched_bytes, kRsrcFlags);
+    const __amdgpu_buffer_rsrc_t rs_feat =
+        __builtin_amdgcn_make_buffer_rsrc((void *)features, 0, (int)feat_bytes, kRsrcFlags);
+    const int idx_voff = (pt >> 4) * 4;    // this thread's slot (plus 16 slots per element)
+    const int chunk_off = (pt & 15) * 16;  // this thread's 16 bytes of a 256-byte row chunk
     int idx[ID][NE];
     float4v rows[RD][NE];
-    // Every load below is unconditional (addresses are clamped into range, results
-    // are masked afterwards): a load inside a branch would make every later wait
-    // cover all outstanding loads, which return in order, and so expose the latency
-    // of the prefetches issued last.
-    const int g_last = (int)(g_end - g_begin) - 1;  // >= 0 whenever nstages > 0
-    auto load_idx = [&](int s, int (&ix)[NE]) {
-      const int grp = min(s / nch, g_last < 0 ? 0 : g_last);
-      const int64_t base = (g_begin + grp) * 64;
+    // Rings indexed by stage number: rows of stage st in rows[st & 3], gather offsets
+    // in idx[st & 1].  The loop is unrolled four times so that every ring index is a
+    // compile-time constant: rotating a ring through register moves would read
+    // registers that loads are still writing, and so wait for those loads one
+    // iteration after their issue.
+    auto load_idx = [&](const StagePos &pos, int s, int (&ix)[NE]) {
 #pragma unroll
       for (int j = 0; j < NE; ++j) {
-        int v = sched_in[base + ((pt + j * NP) >> 4)];
-        ix[j] = s < nstages ? v : -1;
+        int v = buf_load1(rs_in, idx_voff + j * 64, pos.g * 256);
+        if (!FAST) v = s < nstages ? v : -1;  // the pointer gather is not range-checked
+        ix[j] = v;
       }
     };
-    auto load_rows = [&](int s, const int (&ix)[NE], float4v (&r)[NE]) {
-      const int cc = s % nch;
+    auto load_rows = [&](const StagePos &pos, const int (&ix)[NE], float4v (&r)[NE]) {
 #pragma unroll
       for (int j = 0; j < NE; ++j) {
-        const int ch = cc * kKC + ((pt + j * NP) & 15) * 4;
-        const int row = ix[j] < 0 ? 0 : ix[j];  // padding slots read row 0 and drop it
-        const float *fp = features + (int64_t)row * cin + ch;
-        float4v v;
-        if (FULLC) {
-          v = *reinterpret_cast<const float4v *>(fp);
+        if (FAST) {
+          r[j] = buf_load4(rs_feat, ix[j] + chunk_off, pos.cc * 256);
         } else {
-          v = float4v{0.f, 0.f, 0.f, 0.f};
-          if (vec4) {
+          const int ch = pos.cc * kKC + (pt & 15) * 4;
+          const int row = ix[j] < 0 ? 0 : ix[j];  // padding slots read row 0 and drop it
+          const float *fp = features + (int64_t)row * cin + ch;
+          float4v v = float4v{0.f, 0.f, 0.f, 0.f};
+          if ((cin & 3) == 0) {
             if (ch < cin) v = *reinterpret_cast<const float4v *>(fp);
           } else {
             if (ch + 0 < cin) v.x = fp[0];
@@ -435,210 +478,267 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
             if (ch + 2 < cin) v.z = fp[2];
             if (ch + 3 < cin) v.w = fp[3];
           }
+          if (ix[j] < 0) v = float4v{0.f, 0.f, 0.f, 0.f};
+          r[j] = v;
         }
-        if (ix[j] < 0) v = float4v{0.f, 0.f, 0.f, 0.f};
-        r[j] = v;
       }
     };
-    auto store_rows = [&](int s, const float4v (&r)[NE]) {
-      float *ab = abuf + (s & 1) * kStage * kAStride;
+    float *const st_base = abuf + (pt >> 4) * kAStride + (pt & 15) * 4;
+    auto store_rows = [&](int parity, const float4v (&r)[NE]) {
 #pragma unroll
-      for (int j = 0; j < NE; ++j) {
-        int e = pt + j * NP;
-        *reinterpret_cast<float4v *>(ab + (e >> 4) * kAStride + (e & 15) * 4) = r[j];
-      }
+      for (int j = 0; j < NE; ++j)
+        *reinterpret_cast<float4v *>(st_base + (parity * kStage + j * 16) * kAStride) = r[j];
     };
-    // Per-stage metadata, one value per thread 0..70: the output row of each of the
-    // 64 slots; the weight-fragment base offset of the 4 row blocks and of the first
-    // block of the following stage; the tile; whether the tile ends here.
-    auto load_meta = [&](int s) -> int {
-      const int sc = min(s, nstages - 1 < 0 ? 0 : nstages - 1);
-      const int64_t g = g_begin + sc / nch;
-      const int cc = sc % nch;
-      const int sn = min(sc + 1, nstages - 1 < 0 ? 0 : nstages - 1);
-      const int64_t gn = g_begin + sn / nch;
-      // one load per thread, from the array its slot of the metadata comes from
-      const int32_t *src = grp_tile + g;                        // thread 69 (and idle ones)
-      if (pt < kStage) src = sched_out + g * 64 + pt;            // threads 0..63
-      else if (pt < kStage + 4) src = sched_id + g * 4 + (pt - kStage);
-      else if (pt == kStage + 4) src = sched_id + gn * 4;
-      else if (pt == kStage + 6) src = grp_last + g;
-      int v = *src;
-      // fragment base = element offset of (k, column block 0, chunk cc) in `packed`
-      if (pt >= kStage && pt < kStage + 4) v = v >= 0 ? (v * ncb * nch + cc) * 1024 : -1;
-      if (pt == kStage + 4)
-        v = (sc + 1 < nstages && v >= 0) ? (v * ncb * nch + sn % nch) * 1024 : -1;
-      if (pt == kStage + 6) v = (v != 0 && cc == nch - 1) ? 1 : 0;
-      if (s >= nstages) v = pt < kStage ? T : -1;
-      return v;
-    };
-    auto store_meta = [&](int s, int v) {
-      if (pt < kStage) orow[(s & 3) * kStage + pt] = v;
-      else if (pt < kStage + 7) ids[(s & 3) * 8 + (pt - kStage)] = v;
-    };
+    // Prologue.  Loads are issued in the order the loop will wait for them (offsets,
+    // then rows, oldest stage first): the wait counts of the loop are static, so
+    // they must also be right on its first trip.
+    StagePos p_rows = {g_begin, 0};  // stage whose rows are loaded next
+    StagePos p_idx = {g_begin, 0};   // stage whose gather offsets are loaded next
+    StagePos p_cur = {g_begin, 0};   // stage the consumers are working on
     {
-      int ix0[NE];
-      float4v r0[NE];
-      load_idx(0, ix0);
+      int ix[RD + 1][NE];
 #pragma unroll
-      for (int j = 0; j < RD; ++j) {
-        int ix[NE];
-        load_idx(1 + j, ix);
-        load_rows(1 + j, ix, rows[j]);
+      for (int j = 0; j <= RD; ++j) {
+        load_idx(p_idx, j, ix[j]);
+        p_idx.advance(nch);
       }
 #pragma unroll
-      for (int j = 0; j < ID; ++j) load_idx(1 + RD + j, idx[j]);
-      load_rows(0, ix0, r0);
-      store_meta(0, load_meta(0));
-      store_meta(1, load_meta(1));
+      for (int j = 1; j <= ID; ++j) {
+        load_idx(p_idx, RD + j, idx[(RD + j) & 1]);
+        p_idx.advance(nch);
+      }
+      float4v r0[NE];
+      load_rows(p_rows, ix[0], r0);
+      p_rows.advance(nch);
+#pragma unroll
+      for (int j = 1; j <= RD; ++j) {
+        load_rows(p_rows, ix[j], rows[j & 3]);
+        p_rows.advance(nch);
+      }
       store_rows(0, r0);
     }
-    // metadata is fetched two iterations before it is stored, so that waiting for
-    // it never waits for the row loads issued after it (loads return in order)
-    int meta0 = load_meta(2), meta1 = load_meta(3);
     __syncthreads();
-    for (int s = 0; s < nstages; ++s) {
-      store_rows(s + 1, rows[0]);
-      store_meta(s + 2, meta0);
-      meta0 = meta1;
-#pragma unroll
-      for (int i = 0; i + 1 < RD; ++i)
-#pragma unroll
-        for (int j = 0; j < NE; ++j) rows[i][j] = rows[i + 1][j];
-      meta1 = load_meta(s + 4);
-      load_rows(s + 1 + RD, idx[0], rows[RD - 1]);
-#pragma unroll
-      for (int i = 0; i + 1 < ID; ++i)
-#pragma unroll
-        for (int j = 0; j < NE; ++j) idx[i][j] = idx[i + 1][j];
-      load_idx(s + 1 + RD + ID, idx[ID - 1]);
+    // Iteration s stages the rows of stage s+1 and issues the loads of stages s+5
+    // (rows) and s+7 (gather offsets).
+    auto iteration = [&](int s, auto phase) {
+      constexpr int ph = decltype(phase)::value;  // == s & 3
+      int tile;
+      const bool last = tile_end(p_cur, tile);
+      p_cur.advance(nch);
+      store_rows((ph + 1) & 1, rows[(ph + 1) & 3]);
+      load_rows(p_rows, idx[(ph + 1 + RD) & 1], rows[(ph + 1 + RD) & 3]);
+      p_rows.advance(nch);
+      load_idx(p_idx, s + 1 + RD + ID, idx[(ph + 1 + RD + ID) & 1]);
+      p_idx.advance(nch);
       __syncthreads();
-      if (ids[(s & 3) * 8 + 6]) {  // the tile ended with stage s
-        flush_tile(ids[(s & 3) * 8 + 5]);
+      if (last) {
+        flush_tile(tile);
         __syncthreads();
       }
+    };
+    for (int s = 0; s < nstages; s += 4) {
+      iteration(s, std::integral_constant<int, 0>());
+      if (s + 1 >= nstages) break;
+      iteration(s + 1, std::integral_constant<int, 1>());
+      if (s + 2 >= nstages) break;
+      iteration(s + 2, std::integral_constant<int, 2>());
+      if (s + 3 >= nstages) break;
+      iteration(s + 3, std::integral_constant<int, 3>());
     }
   } else {
     // ------------------------------------------------------------------ consumer
     const int g = lane >> 4;
     const int l16 = lane & 15;
-    const int cb0 = (blockIdx.y * 4 + wave) * CGW;  // first column block of this wave
-    float *acc_lane = acc + wave * CGW * 16 + g * 4;
     // A column group beyond Cout multiplies with the last real one's fragments; its
-    // accumulator columns are never written out.  This keeps the code branch-free.
-    const float *bbase[CGW];
+    // accumulator columns are never written out.
+    const int cb = min(blockIdx.y * 4 + wave, ncb - 1);
+    const __amdgpu_buffer_rsrc_t rs_w =
+        __builtin_amdgcn_make_buffer_rsrc((void *)packed, 0, (int)packed_bytes, kRsrcFlags);
+    const __amdgpu_buffer_rsrc_t rs_out =
+        __builtin_amdgcn_make_buffer_rsrc((void *)sched_out, 0, (int)sched_bytes, kRsrcFlags);
+    const int w_voff = lane * 64;           // this lane's 16 floats of a fragment
+    const int w_soff0 = cb * nch * 4096;    // fragments of this wave's column block
+    const int frag_k = ncb * nch * 4096;    // bytes between the fragments of two offsets
+    const int acc_lane = (wave * 16 + g * 4) * 4;  // byte offset of this lane's 4 columns
+    const float *const a_base = abuf + l16 * kAStride + g * 16;
+    char *const acc_bytes = reinterpret_cast<char *>(acc);
+
+    const __amdgpu_buffer_rsrc_t rs_meta =
+        __builtin_amdgcn_make_buffer_rsrc((void *)grp_meta, 0, (int)meta_bytes, kRsrcFlags);
+    // What a stage needs besides the staged rows, fetched one stage ahead:
+    //   w[m][q]  weight fragments of row block m (four 16-byte loads per block)
+    //   orow[m]  LDS byte offset of the accumulator row of this lane's pair
+    //   rec      the schedule record (offsets of the 4 blocks, tile, last-of-tile) of
+    //            the stage AFTER this one, the same in every lane.  It travels through
+    //            vector loads and v_readfirstlane rather than scalar loads: scalar
+    //            loads return out of order, and one in flight would turn every
+    //            partial wait for LDS data below into a wait for everything.
+    struct StageRegs {
+      float4v w[4][4];
+      int orow[4];
+      int4v rec[2];
+    };
+    auto load_rec = [&](const StagePos &pos, int4v (&rec)[2]) {
+      rec[0] = __builtin_bit_cast(int4v, buf_load4(rs_meta, 0, pos.g * 32));
+      rec[1] = __builtin_bit_cast(int4v, buf_load4(rs_meta, 16, pos.g * 32));
+    };
+    // Scalar part of fetching the stage at `pos`, whose record is `rec`: byte offsets
+    // of its four blocks' fragments, its tile and whether the tile ends with it.
+    struct StageScalars {
+      int soff[4];
+      int tile;
+      bool last;
+    };
+    auto stage_scalars = [&](const StagePos &pos, const int4v (&rec)[2]) -> StageScalars {
+      StageScalars sc;
+      const int k[4] = {
+          __builtin_amdgcn_readfirstlane(rec[0].x), __builtin_amdgcn_readfirstlane(rec[0].y),
+          __builtin_amdgcn_readfirstlane(rec[0].z), __builtin_amdgcn_readfirstlane(rec[0].w)};
+      sc.tile = __builtin_amdgcn_readfirstlane(rec[1].x);
+      sc.last = __builtin_amdgcn_readfirstlane(rec[1].y) != 0 && pos.cc == nch - 1;
 #pragma unroll
-    for (int c = 0; c < CGW; ++c)
-      bbase[c] = packed + (int64_t)min(cb0 + c, ncb - 1) * nch * 1024 + lane * 16;
-    auto load_b = [&](int base, float4v (&b)[CGW][4]) {
-#pragma unroll
-      for (int c = 0; c < CGW; ++c) {
-        const float4v *bp = reinterpret_cast<const float4v *>(bbase[c] + base);
-#pragma unroll
-        for (int q = 0; q < 4; ++q) b[c][q] = bp[q];
+      for (int b = 0; b < 4; ++b) {
+        // empty blocks (-1) and records beyond the schedule use the fragments of offset 0
+        const int kk = (k[b] < 0 || k[b] >= kvol) ? 0 : k[b];
+        sc.soff[b] = w_soff0 + kk * frag_k + pos.cc * 4096;
       }
+      return sc;
     };
-    auto load_a = [&](const float *ab, int m, float4v (&a)[4]) {
-      const float4v *ap =
-          reinterpret_cast<const float4v *>(ab + (m * 16 + l16) * kAStride + g * 16);
-#pragma unroll
-      for (int q = 0; q < 4; ++q) a[q] = ap[q];
+    auto fetch_w = [&](const StageScalars &sc, int b, int q, StageRegs &r) {
+      r.w[b][q] = buf_load4(rs_w, w_voff + q * 16, sc.soff[b]);
     };
-    const bool live = cb0 < ncb;
-    // Two sets of weight fragments, each holding the 4 blocks of one stage.  Stage s
-    // multiplies with one set while ALL fragments of stage s+1 are fetched, in one
-    // unconditional batch at the top of the stage, into the other set: a whole
-    // stage of MFMAs (longer than an L2 round trip under load) lies between the
-    // issue of a load and its first use, and the loads are never inside a branch,
-    // so the compiler's wait counts stay exact.
-    //
-    // Every stage runs the same straight-line code.  An empty row block (only at
-    // the end of a tile) has zeros staged for its slots and the dummy row T as
-    // output row, so its MFMAs add zeros to a row that is never written out.
-    float4v bx[4][CGW][4], by[4][CGW][4];
-    auto stage_ids = [&](int s, int (&id)[4]) {
-      const int *meta = ids + (s & 3) * 8;
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        int v = __builtin_amdgcn_readfirstlane(meta[j]);
-        id[j] = (s < nstages && v >= 0) ? v : 0;  // any valid fragment for an empty block
-      }
+    auto fetch_orow = [&](const StagePos &pos, int b, StageRegs &r) {
+      r.orow[b] = buf_load1(rs_out, l16 * 4 + b * 64, pos.g * 256);
     };
-    auto load_b_stage = [&](int s, float4v (&b)[4][CGW][4]) {
-      int id[4];
-      stage_ids(s, id);
-#pragma unroll
-      for (int m = 0; m < 4; ++m) load_b(id[m], b[m]);
-    };
-    auto run_stage = [&](int s, float4v (&bc)[4][CGW][4], float4v (&bn)[4][CGW][4]) {
-      load_b_stage(s + 1, bn);  // the ring publishes a stage's ids two stages ahead
-      // keep the batch here: the scheduler would otherwise sink these loads to the
-      // end of the stage to shorten register live ranges, which exposes their latency
-      __builtin_amdgcn_sched_barrier(0);
-      const float *ab = abuf + (s & 1) * kStage * kAStride;
-      const int *orw = orow + (s & 3) * kStage;
+    // One stage = 4 row blocks, software-pipelined by hand.  A wave issues in order
+    // and the 16 MFMAs of a block form one dependent chain, so whatever follows a
+    // chain in program order waits ~500 cycles for it, and whatever a chain waits
+    // for stalls the matrix pipe.  Therefore, in program order:
+    //   staged rows of block m+1 are read BEFORE the chain of block m starts;
+    //   the accumulator update of block m-1 (add, write) and the accumulator read of
+    //   block m sit AFTER the first four MFMAs of block m, in the shadow of the chain;
+    //   the 22 loads that fetch the next stage's registers are spread over the 16
+    //   groups of four MFMAs: a 16-byte-per-lane load keeps the wave in the issue
+    //   stage for tens of cycles, which a burst of loads would add to the stage and
+    //   which is free behind an MFMA whose successor must wait for it anyway.
+    // Scheduling barriers pin that order (the compiler otherwise moves the LDS reads
+    // next to their first use to shorten live ranges).  LDS operations of a wave
+    // execute in order, so the read of block m's rows after the write of block m-1
+    // sees that write when both blocks touch the same output row.
+    auto run_stage = [&](int parity, const StagePos &next, const StagePos &after,
+                         const StageRegs &cur, StageRegs &nxt, int &tile_next, bool &last_next) {
+      const StageScalars sc = stage_scalars(next, cur.rec);
+      tile_next = sc.tile;
+      last_next = sc.last;
+      const float *ab = a_base + parity * kStage * kAStride;
       float4v a[2][4];
-      load_a(ab, 0, a[0]);
-      int ol[4];
+      auto load_a = [&](int m, float4v (&av)[4]) {
+        const float4v *ap = reinterpret_cast<const float4v *>(ab + m * 16 * kAStride);
 #pragma unroll
-      for (int m = 0; m < 4; ++m) ol[m] = orw[m * 16 + l16];
+        for (int q = 0; q < 4; ++q) av[q] = ap[q];
+      };
+      load_a(0, a[0]);
+      float4v accr, dprev;
+      accr = *reinterpret_cast<const float4v *>(acc_bytes + cur.orow[0] + acc_lane);
 #pragma unroll
       for (int m = 0; m < 4; ++m) {
-        if (m < 3) load_a(ab, m + 1, a[(m + 1) & 1]);
-        // accumulator rows of this block: read before the MFMAs, added after
-        float4v accr[CGW], d[CGW];
-#pragma unroll
-        for (int c = 0; c < CGW; ++c) {
-          accr[c] = *reinterpret_cast<const float4v *>(acc_lane + ol[m] * AS + c * 16);
-          d[c] = float4v{0.f, 0.f, 0.f, 0.f};
+        if (m < 3) load_a(m + 1, a[(m + 1) & 1]);
+        __builtin_amdgcn_sched_barrier(0);
+        float4v d = float4v{0.f, 0.f, 0.f, 0.f};
+        mfma_quad(cur.w[m][0], a[m & 1][0], d);
+        __builtin_amdgcn_sched_barrier(0);
+        fetch_w(sc, m, 0, nxt);
+        if (m > 0) {
+          // dprev = out[pair l16][channels 4g .. 4g+3] of block m-1
+          *reinterpret_cast<float4v *>(acc_bytes + cur.orow[m - 1] + acc_lane) = accr + dprev;
+          accr = *reinterpret_cast<const float4v *>(acc_bytes + cur.orow[m] + acc_lane);
         }
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int c = 0; c < CGW; ++c) mfma_block(bc[m][c], a[m & 1], d[c]);
-        // d[c] = out[pair l16][channels 4g .. 4g+3] of column group c of this wave
-#pragma unroll
-        for (int c = 0; c < CGW; ++c)
-          *reinterpret_cast<float4v *>(acc_lane + ol[m] * AS + c * 16) = accr[c] + d[c];
+        for (int q = 1; q < 4; ++q) {
+          mfma_quad(cur.w[m][q], a[m & 1][q], d);
+          __builtin_amdgcn_sched_barrier(0);
+          fetch_w(sc, m, q, nxt);
+          if (q == 1) fetch_orow(next, m, nxt);
+          if (q == 2 && m >= 2) nxt.rec[m - 2] = __builtin_bit_cast(
+              int4v, buf_load4(rs_meta, (m - 2) * 16, after.g * 32));
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        dprev = d;
       }
+      __builtin_amdgcn_sched_barrier(0);
+      *reinterpret_cast<float4v *>(acc_bytes + cur.orow[3] + acc_lane) = accr + dprev;
     };
+    // Everything the first stage needs, in one batch.
+    auto fetch_all = [&](const StagePos &pos, const StagePos &after, const int4v (&rec)[2],
+                         StageRegs &r, int &tile, bool &last) {
+      const StageScalars sc = stage_scalars(pos, rec);
+      tile = sc.tile;
+      last = sc.last;
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) fetch_w(sc, b, q, r);
+        fetch_orow(pos, b, r);
+      }
+      load_rec(after, r.rec);
+    };
+    StageRegs rx, ry;
+    StagePos p_next = {g_begin, 0};   // stage whose registers are fetched next
+    StagePos p_after = {g_begin, 0};  // the stage after that one
+    p_after.advance(nch);
+    int tile, tile_next;
+    bool last, last_next;
+    {
+      int4v rec0[2];
+      load_rec(p_next, rec0);
+      fetch_all(p_next, p_after, rec0, rx, tile, last);
+      p_next.advance(nch);
+      p_after.advance(nch);
+    }
     __syncthreads();
-    if (live && nstages > 0) load_b_stage(0, bx);
     for (int s = 0; s < nstages; s += 2) {
-      if (live) run_stage(s, bx, by);
-      int tl = ids[(s & 3) * 8 + 5], last = ids[(s & 3) * 8 + 6];
+      run_stage(0, p_next, p_after, rx, ry, tile_next, last_next);
+      p_next.advance(nch);
+      p_after.advance(nch);
       __syncthreads();
       if (last) {
-        flush_tile(tl);
+        flush_tile(tile);
         __syncthreads();
       }
+      tile = tile_next;
+      last = last_next;
       if (s + 1 < nstages) {
-        if (live) run_stage(s + 1, by, bx);
-        tl = ids[((s + 1) & 3) * 8 + 5];
-        last = ids[((s + 1) & 3) * 8 + 6];
+        run_stage(1, p_next, p_after, ry, rx, tile_next, last_next);
+        p_next.advance(nch);
+        p_after.advance(nch);
         __syncthreads();
         if (last) {
-          flush_tile(tl);
+          flush_tile(tile);
           __syncthreads();
         }
+        tile = tile_next;
+        last = last_next;
       }
     }
   }
 }
 
 struct ConvPlan {
-  int ncb, nch, T, cgw, n_wg, n_colblk;
+  int ncb, nch, T, n_wg, n_colblk;
+  bool fast;
   int64_t n_tiles, words_per_k, grp_cap;
   size_t lds_bytes;
 };
 
-static size_t conv_lds_bytes(int T, int cgw) {
-  return ((size_t)(T + 1) * (cgw * 64 + 4) + 2 * (size_t)kStage * kAStride) * 4 +
-         4 * kStage * 4 + 32 * 4;
+static size_t conv_lds_bytes(int T) {
+  return ((size_t)(T + 1) * kAS + 2 * (size_t)kStage * kAStride) * 4;
 }
 
-static int pick_tile(int cgw) {
+static int pick_tile() {
   // One workgroup per CU: (almost) all of the 160 KB of LDS goes to the accumulators.
-  size_t budget = 160 * 1024 - conv_lds_bytes(0, cgw) - 512;
-  int t = (int)(budget / ((size_t)(cgw * 64 + 4) * 4));
+  size_t budget = 160 * 1024 - conv_lds_bytes(0) - 512;
+  int t = (int)(budget / ((size_t)kAS * 4));
   t = t / 8 * 8;
   if (t < kMinTile) t = kMinTile;
   return t;
@@ -656,25 +756,29 @@ static int device_cu_count() {
   return cus;
 }
 
-static ConvPlan make_plan(int64_t n_out, int K, int c_in, int c_out, int64_t pair_stride) {
+static ConvPlan make_plan(int64_t n_in, int64_t n_out, int K, int c_in, int c_out,
+                          int64_t pair_stride) {
   ConvPlan p;
   p.ncb = (int)ceil_div(c_out, 16);
   p.nch = (int)ceil_div(c_in, kKC);
-  p.cgw = 1;  // 64-column tiles: two full-stage sets of weight fragments fit the registers
-  p.T = pick_tile(p.cgw);
+  p.T = pick_tile();
+  // the gather can be a range-checked buffer load when every 64-channel chunk is
+  // complete and byte offsets into the features (plus the padding marker) fit 32 bits
+  p.fast = (c_in % kKC) == 0 && (uint64_t)n_in * c_in * 4 <= (uint64_t)kGatherPad;
   p.n_tiles = ceil_div(n_out > 0 ? n_out : 1, p.T);
   p.words_per_k = ceil_div(n_out > 0 ? n_out : 1, 32);
   // groups: pairs/64 plus, per (tile, offset), up to one partial block, plus one
-  // partial (or empty) group per tile
+  // partial (or empty) group per tile, plus the groups the kernel's prefetches may
+  // touch beyond the end of the schedule
   int64_t max_pairs_k = pair_stride < n_out ? pair_stride : n_out;
-  p.grp_cap = ((int64_t)K * (max_pairs_k / 16 + 1) + p.n_tiles * K) / 4 + 2 * p.n_tiles + 4;
-  p.n_colblk = (int)ceil_div(p.ncb, 4 * p.cgw);
+  p.grp_cap = ((int64_t)K * (max_pairs_k / 16 + 1) + p.n_tiles * K) / 4 + 2 * p.n_tiles + 4 + 16;
+  p.n_colblk = (int)ceil_div(p.ncb, 4);
   int n_wg = device_cu_count() / p.n_colblk;
   if (n_wg < 1) n_wg = 1;
   if (n_wg > p.n_tiles) n_wg = (int)p.n_tiles;
   if (n_wg >= 8) n_wg = n_wg / 8 * 8;
   p.n_wg = n_wg;
-  p.lds_bytes = conv_lds_bytes(p.T, p.cgw);
+  p.lds_bytes = conv_lds_bytes(p.T);
   return p;
 }
 
@@ -686,7 +790,7 @@ struct ConvWs {
   uint32_t *bits;
   int32_t *prefix;
   int32_t *tile_cnt, *tile_nmb, *kofs, *tile_grp, *wg_tile;
-  int32_t *sched_in, *sched_out, *sched_id, *grp_tile, *grp_last;
+  int32_t *sched_in, *sched_out, *grp_meta;
 };
 
 static size_t conv_ws_walk(void *base, const ConvPlan &p, int K, int64_t pair_stride, ConvWs *w) {
@@ -705,31 +809,37 @@ static size_t conv_ws_walk(void *base, const ConvPlan &p, int K, int64_t pair_st
   t.wg_tile = c.take<int32_t>((size_t)p.n_wg + 1);
   t.sched_in = c.take<int32_t>((size_t)p.grp_cap * 64);
   t.sched_out = c.take<int32_t>((size_t)p.grp_cap * 64);
-  t.sched_id = c.take<int32_t>((size_t)p.grp_cap * 4);
-  t.grp_tile = c.take<int32_t>((size_t)p.grp_cap);
-  t.grp_last = c.take<int32_t>((size_t)p.grp_cap);
+  t.grp_meta = c.take<int32_t>((size_t)p.grp_cap * 8);
   if (w) *w = t;
   return c.used;
 }
 
 static size_t conv_ws_bytes(int64_t n_out, int K, int c_in, int c_out, int64_t pair_stride) {
-  ConvPlan p = make_plan(n_out, K, c_in, c_out, pair_stride);
+  // the workspace does not depend on the number of input rows
+  ConvPlan p = make_plan(0, n_out, K, c_in, c_out, pair_stride);
   return conv_ws_walk(nullptr, p, K, pair_stride, nullptr);
 }
 
-template <int CGW, bool FULLC>
-static int launch_conv(const ConvPlan &p, const ConvWs &w, const float *features, int c_in,
-                       float *out, int64_t n_out, int c_out, hipStream_t s) {
+template <bool FAST>
+static int launch_conv(const ConvPlan &p, const ConvWs &w, const float *features, int64_t n_in,
+                       int c_in, int K, float *out, int64_t n_out, int c_out, hipStream_t s) {
   static bool attr_set = false;
   if (!attr_set) {
-    SSC_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(conv_fwd_kernel<CGW, FULLC>),
+    SSC_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(conv_fwd_kernel<FAST>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
     attr_set = true;
   }
+  const uint64_t packed_bytes = (uint64_t)K * p.ncb * p.nch * 4096;
+  const uint64_t sched_bytes = (uint64_t)p.grp_cap * 256;
+  SSC_CHECK(packed_bytes < ((uint64_t)1 << 32) && sched_bytes < ((uint64_t)1 << 32), SSC_ERUNTIME,
+            "convolution too large for 32-bit buffer offsets (filters %llu B, schedule %llu B)",
+            (unsigned long long)packed_bytes, (unsigned long long)sched_bytes);
+  const unsigned feat_bytes = FAST ? (unsigned)((uint64_t)n_in * c_in * 4) : 0u;
   dim3 grid((unsigned)p.n_wg, (unsigned)p.n_colblk);
-  hipLaunchKernelGGL((conv_fwd_kernel<CGW, FULLC>), grid, dim3(512), p.lds_bytes, s, features,
-                     c_in, w.packed, w.sched_in, w.sched_out, w.sched_id, w.grp_tile, w.grp_last,
-                     w.tile_grp, w.wg_tile, p.nch, p.ncb, out, n_out, c_out, p.T);
+  hipLaunchKernelGGL((conv_fwd_kernel<FAST>), grid, dim3(512), p.lds_bytes, s, features, c_in,
+                     feat_bytes, w.packed, (unsigned)packed_bytes, w.sched_in, w.sched_out,
+                     w.grp_meta, (unsigned)sched_bytes, (unsigned)(p.grp_cap * 32), w.tile_grp,
+                     w.wg_tile, p.nch, p.ncb, K, out, n_out, c_out, p.T);
   SSC_LAUNCH_CHECK("conv_fwd");
   return SSC_OK;
 }
@@ -802,7 +912,7 @@ int ssc_conv_fwd_f32(const float *features, int64_t n_in, int32_t c_in, const fl
   SSC_CHECK(workspace_bytes >= need, SSC_EWORKSPACE, "conv workspace too small: %zu < %zu",
             workspace_bytes, need);
 
-  ConvPlan p = make_plan(n_out, K, c_in, c_out, pair_stride);
+  ConvPlan p = make_plan(n_in, n_out, K, c_in, c_out, pair_stride);
   ConvWs w;
   conv_ws_walk(workspace, p, K, pair_stride, &w);
   const int plane_g = inverse ? 1 : 0;
@@ -843,8 +953,9 @@ int ssc_conv_fwd_f32(const float *features, int64_t n_in, int32_t c_in, const fl
                      w.tile_grp);
   hipLaunchKernelGGL(sched_fill_kernel, dim3((unsigned)ceil_div(p.n_tiles * K * 16, 256)),
                      dim3(256), 0, s, w.flag, pairs, w.sorted, pair_stride, plane_g, w.segs,
-                     w.kofs, w.tile_nmb, w.tile_grp, K, p.n_tiles, p.T, w.sched_in, w.sched_out,
-                     w.sched_id, w.grp_tile, w.grp_last);
+                     w.kofs, w.tile_nmb, w.tile_grp, K, p.n_tiles, p.T,
+                     p.fast ? (uint32_t)c_in * 4u : 1u, p.fast ? kGatherPad : 0xFFFFFFFFu, kAS * 4,
+                     w.sched_in, w.sched_out, w.grp_meta);
   hipLaunchKernelGGL(sched_split_kernel, dim3((unsigned)ceil_div(p.n_wg + 1, 256)), dim3(256), 0,
                      s, w.tile_grp, p.n_tiles, p.n_wg, w.wg_tile);
   SSC_LAUNCH_CHECK("schedule");
@@ -852,14 +963,8 @@ int ssc_conv_fwd_f32(const float *features, int64_t n_in, int32_t c_in, const fl
   const bool prof = g_profile_on;
   const int slot = g_profile_count % kProfileRing;
   if (prof) SSC_HIP(hipEventRecord(g_profile_ev[slot][0], s));
-  // FULLC: Cin is a multiple of 64, so every channel chunk is complete
-  const bool fullc = (c_in % kKC) == 0;
-  if (p.cgw == 2)
-    rc = fullc ? launch_conv<2, true>(p, w, features, c_in, out, n_out, c_out, s)
-               : launch_conv<2, false>(p, w, features, c_in, out, n_out, c_out, s);
-  else
-    rc = fullc ? launch_conv<1, true>(p, w, features, c_in, out, n_out, c_out, s)
-               : launch_conv<1, false>(p, w, features, c_in, out, n_out, c_out, s);
+  rc = p.fast ? launch_conv<true>(p, w, features, n_in, c_in, K, out, n_out, c_out, s)
+              : launch_conv<false>(p, w, features, n_in, c_in, K, out, n_out, c_out, s);
   if (rc != SSC_OK) return rc;
   if (prof) {
     SSC_HIP(hipEventRecord(g_profile_ev[slot][1], s));
