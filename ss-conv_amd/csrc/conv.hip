@@ -1,6 +1,6 @@
 // Sparse convolution forward as an output-stationary implicit GEMM on fp32 MFMA.
 //
-// Outputs are cut into tiles of T consecutive rows.  A workgroup owns one tile
+// Outputs are cut into tiles of at most T consecutive rows.  A workgroup owns one tile
 // and CN output columns; its accumulators [T, CN] live in LDS for the whole
 // kernel.  For every kernel offset k the pairs that land in the tile form one
 // contiguous segment of the rulebook (pairs of an offset are ascending in
@@ -136,19 +136,26 @@ __global__ void __launch_bounds__(256)
   sorted[((int64_t)k * 2 + (1 - plane_s)) * pair_stride + pos] = pg[j];
 }
 
-// segs[t*K + k] = first pair of offset k whose scatter row is >= t*T  (t = 0..n_tiles).
+// segs[t*K + k] = first pair of offset k whose scatter row is >= the first row of
+// tile t (t = 0..n_tiles).  Tile rows come from tile_row0[] and the tile count from
+// n_tiles_dev[0]; with tile_row0 == nullptr the tiles are `granule` rows each and
+// there are n_cap of them (the fine grid the work split is computed on).
 __global__ void __launch_bounds__(256)
     tile_segments_kernel(const int32_t *__restrict__ flag, const int32_t *__restrict__ pairs,
                          const int32_t *__restrict__ sorted, int64_t pair_stride, int plane_s,
-                         const int32_t *__restrict__ pair_num, int K, int64_t n_tiles, int T,
+                         const int32_t *__restrict__ pair_num, int K, int64_t n_cap,
+                         const int32_t *__restrict__ n_tiles_dev,
+                         const int32_t *__restrict__ tile_row0, int granule, int64_t n_out,
                          int32_t *__restrict__ segs) {
   int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t n_tiles = tile_row0 ? n_tiles_dev[0] : n_cap;
   if (idx >= (n_tiles + 1) * K) return;
   int64_t t = idx / K;
   int k = (int)(idx - t * K);
   const int32_t *src = flag[0] ? sorted : pairs;
   const int32_t *s = src + ((int64_t)k * 2 + plane_s) * pair_stride;
-  int64_t target = t * (int64_t)T;
+  int64_t target = tile_row0 ? (int64_t)tile_row0[t] : t * (int64_t)granule;
+  if (target > n_out) target = n_out;
   int lo = 0, hi = pair_num[k];
   while (lo < hi) {
     int mid = (lo + hi) >> 1;
@@ -156,6 +163,80 @@ __global__ void __launch_bounds__(256)
     else hi = mid;
   }
   segs[idx] = lo;
+}
+
+// ---- work split ------------------------------------------------------------------------
+// Output rows are dealt to the persistent workgroups in contiguous ranges of equal
+// WORK, not equal length: work(r) = pairs that land in rows < r, plus a per-row
+// share of what every tile costs on top of its pairs (padding of the last row block
+// of each offset, writing the tile out).  Pairs per row come from a fine grid of
+// kSplitGranule rows; range boundaries lie on that grid.  Each range is then cut
+// into tiles of equal height <= T.
+constexpr int kSplitGranule = 64;
+
+// fine_work[b] = sum over offsets of fine_segs[b*K + k]  (pairs in rows < b*granule)
+__global__ void __launch_bounds__(256)
+    split_sum_kernel(const int32_t *__restrict__ fine_segs, int K, int64_t nb,
+                     int32_t *__restrict__ fine_work) {
+  int64_t b = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (b > nb) return;
+  int sum = 0;
+  for (int k = 0; k < K; ++k) sum += fine_segs[b * K + k];
+  fine_work[b] = sum;
+}
+
+// One block.  wg_tile[0..n_wg]: first tile of every workgroup; tile_row0[0..n_tiles]:
+// first row of every tile; n_tiles_dev[0]: number of tiles.
+__global__ void __launch_bounds__(256)
+    split_rows_kernel(const int32_t *__restrict__ fine_work, int64_t nb, int64_t n_out, int T,
+                      int K, int n_wg, int32_t *__restrict__ wg_tile,
+                      int32_t *__restrict__ tile_row0, int32_t *__restrict__ n_tiles_dev) {
+  __shared__ int row_s[257];
+  __shared__ int tile_s[257];
+  // cost of a tile beyond its pairs, in pair slots: half a row block of padding per
+  // offset, and about two stages' worth of time for writing it out
+  const int64_t tile_cost = (int64_t)K * 8 + 128;
+  auto work = [&](int64_t b) -> int64_t {
+    int64_t r = b * kSplitGranule;
+    if (r > n_out) r = n_out;
+    return (int64_t)fine_work[b] * T + r * tile_cost;  // scaled by T to stay in integers
+  };
+  for (int w = threadIdx.x; w <= n_wg; w += blockDim.x) {  // n_wg <= 256
+    const int64_t total = work(nb);
+    const int64_t target = (total * w + n_wg - 1) / n_wg;
+    int64_t lo = 0, hi = nb;
+    while (lo < hi) {
+      int64_t mid = (lo + hi) >> 1;
+      if (work(mid) < target) lo = mid + 1;
+      else hi = mid;
+    }
+    int64_t r = lo * kSplitGranule;
+    if (r > n_out || w == n_wg) r = n_out;
+    if (w == 0) r = 0;
+    row_s[w] = (int)r;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int run = 0;
+    for (int i = 0; i < n_wg; ++i) {
+      tile_s[i] = run;
+      run += (row_s[i + 1] - row_s[i] + T - 1) / T;
+    }
+    tile_s[n_wg] = run;
+    n_tiles_dev[0] = run;
+    tile_row0[run] = (int32_t)n_out;
+  }
+  __syncthreads();
+  for (int w = threadIdx.x; w <= n_wg; w += blockDim.x) {
+    wg_tile[w] = tile_s[w];
+    if (w == n_wg) break;
+    const int rows = row_s[w + 1] - row_s[w];
+    const int nt = tile_s[w + 1] - tile_s[w];
+    if (nt > 0) {
+      const int h = (rows + nt - 1) / nt;
+      for (int j = 0; j < nt; ++j) tile_row0[tile_s[w] + j] = row_s[w] + j * h;
+    }
+  }
 }
 
 // ---- row-block schedule -----------------------------------------------------------------
@@ -173,11 +254,11 @@ __global__ void __launch_bounds__(256)
 //                               4 tile of the group, 5 1 when it is the tile's last group
 // The convolution kernel streams through it without per-offset bookkeeping.
 __global__ void __launch_bounds__(256)
-    sched_count_kernel(const int32_t *__restrict__ segs, int K, int64_t n_tiles,
-                       int32_t *__restrict__ tile_cnt, int32_t *__restrict__ tile_nmb,
-                       int32_t *__restrict__ kofs) {
+    sched_count_kernel(const int32_t *__restrict__ segs, int K,
+                       const int32_t *__restrict__ n_tiles_dev, int32_t *__restrict__ tile_cnt,
+                       int32_t *__restrict__ tile_nmb, int32_t *__restrict__ kofs) {
   int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (t >= n_tiles) return;
+  if (t >= n_tiles_dev[0]) return;
   int run = 0;
   for (int k = 0; k < K; ++k) {
     int n = segs[(t + 1) * K + k] - segs[t * K + k];
@@ -191,9 +272,10 @@ __global__ void __launch_bounds__(256)
 
 // tile_grp[0..n_tiles]: exclusive prefix of tile_cnt (one block).
 __global__ void __launch_bounds__(kScanThreads)
-    sched_scan_kernel(const int32_t *__restrict__ tile_cnt, int64_t n_tiles,
-                      int32_t *__restrict__ tile_grp) {
+    sched_scan_kernel(const int32_t *__restrict__ tile_cnt,
+                      const int32_t *__restrict__ n_tiles_dev, int32_t *__restrict__ tile_grp) {
   __shared__ int lds[kScanThreads / 64 + 1];
+  const int64_t n_tiles = n_tiles_dev[0];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   int carry = 0;
   for (int64_t base = 0; base < n_tiles; base += kScanThreads) {
@@ -228,13 +310,14 @@ __global__ void __launch_bounds__(256)
                       const int32_t *__restrict__ sorted, int64_t pair_stride, int plane_g,
                       const int32_t *__restrict__ segs, const int32_t *__restrict__ kofs,
                       const int32_t *__restrict__ tile_nmb, const int32_t *__restrict__ tile_grp,
-                      int K, int64_t n_tiles, int T, uint32_t in_scale, uint32_t in_pad,
-                      int out_scale, int32_t *__restrict__ sched_in,
+                      int K, const int32_t *__restrict__ n_tiles_dev,
+                      const int32_t *__restrict__ tile_row0, int T, uint32_t in_scale,
+                      uint32_t in_pad, int out_scale, int32_t *__restrict__ sched_in,
                       int32_t *__restrict__ sched_out, int32_t *__restrict__ grp_meta) {
   int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   int64_t tk = gid >> 4;
   int lane = (int)(gid & 15);
-  if (tk >= n_tiles * K) return;
+  if (tk >= (int64_t)n_tiles_dev[0] * K) return;
   int64_t t = tk / K;
   int k = (int)(tk - t * K);
   const int64_t g0 = tile_grp[t], g1 = tile_grp[t + 1];
@@ -258,7 +341,7 @@ __global__ void __launch_bounds__(256)
   const int32_t *pg = src + ((int64_t)k * 2 + plane_g) * pair_stride + s0;
   const int32_t *ps = src + ((int64_t)k * 2 + (1 - plane_g)) * pair_stride + s0;
   int64_t mb = g0 * 4 + kofs[t * K + k];
-  int64_t row0 = t * (int64_t)T;
+  int64_t row0 = tile_row0[t];
   for (int p = lane; p < ((n + 15) & ~15); p += 16, ++mb) {
     sched_in[mb * 16 + lane] = p < n ? (int32_t)((uint32_t)pg[p] * in_scale) : (int32_t)in_pad;
     sched_out[mb * 16 + lane] = (p < n ? (int)(ps[p] - row0) : T) * out_scale;
@@ -266,34 +349,21 @@ __global__ void __launch_bounds__(256)
   }
 }
 
-// Tile range of every persistent workgroup: boundary w is the first tile whose
-// group prefix reaches w/n_wg of all groups, so workgroups get equal work, not
-// equal tile counts.
-__global__ void __launch_bounds__(256)
-    sched_split_kernel(const int32_t *__restrict__ tile_grp, int64_t n_tiles, int n_wg,
-                       int32_t *__restrict__ wg_tile) {
-  int w = blockIdx.x * blockDim.x + threadIdx.x;
-  if (w > n_wg) return;
-  int64_t total = tile_grp[n_tiles];
-  int64_t target = (total * w + n_wg - 1) / n_wg;
-  int64_t lo = 0, hi = n_tiles;
-  while (lo < hi) {
-    int64_t mid = (lo + hi) >> 1;
-    if (tile_grp[mid] < target) lo = mid + 1;
-    else hi = mid;
-  }
-  wg_tile[w] = w == n_wg ? (int32_t)n_tiles : (int32_t)lo;
-}
-
 // ---- the convolution --------------------------------------------------------------------
-// Persistent kernel: one workgroup (8 waves) per CU walks a contiguous,
-// work-balanced range of tiles.  A workgroup owns T output rows x 64 output
-// columns at a time; the fp32 accumulators of that tile live in LDS.
-//   waves 0-3  consumers: wave w owns 16 columns of the workgroup's column range.
-//              It multiplies the staged input rows of a stage with the weight
-//              fragments of its columns and adds the products to the accumulators.
-//   waves 4-7  producers: gather the input rows of the coming stages from global
-//              memory (several stages ahead, in registers) and stage them in LDS.
+// Persistent kernel: one workgroup per CU walks a contiguous, work-balanced range
+// of tiles.  A workgroup owns T output rows x 16*NCW output columns at a time; the
+// fp32 accumulators of that tile live in LDS.
+//   waves 0..NCW-1    consumers: wave w owns 16 columns of the workgroup's column
+//                     range.  It multiplies the staged input rows of a stage with the
+//                     weight fragments of its columns and adds the products to the
+//                     accumulators.
+//   waves NCW..NCW+3  producers: gather the input rows of the coming stages from
+//                     global memory (several stages ahead, in registers) and stage
+//                     them in LDS.
+// NCW = 4 (64 columns) is what the host code launches.  NCW = 8 (128 columns, two
+// consumers per SIMD, tiles half as tall) computes the same result; on the 64 -> 128
+// channel benchmark layer it is 6 % slower, because the shorter tiles pack the row
+// blocks less densely and the weight-fragment traffic per tile row doubles.
 // A stage = one group of the schedule (4 row blocks = 64 pair slots, any mix of
 // offsets) x one 64-channel chunk of Cin.  One barrier per stage hands the buffer
 // filled with stage s+1 to the consumers and the buffer of stage s back to the
@@ -319,9 +389,7 @@ __global__ void __launch_bounds__(256)
 // so every output element sees its offsets added in ascending k: reproducible,
 // no atomics.
 //
-// Dynamic LDS: acc[T+1][68] | abuf[2][64][68]
-constexpr int kCN = 64;        // output columns per workgroup
-constexpr int kAS = kCN + 4;   // accumulator row stride in floats
+// Dynamic LDS: acc[T+1][16*NCW+4] | abuf[2][64][68]
 constexpr int kRowsAhead = 4;  // stages whose gathered rows are in flight in registers
 constexpr int kIdxAhead = 2;   // further stages whose gather offsets are in flight
 constexpr unsigned kGatherPad = 0xFFFFF000u;  // gather offset of a padding slot (FAST)
@@ -359,18 +427,21 @@ struct StagePos {
 // range-checked buffer load.  Otherwise the schedule holds row numbers and the
 // gather uses 64-bit addresses with per-channel masks.
 //
-// Exactly two waves per SIMD (one consumer, one producer): the compiler may use
-// up to 256 VGPRs instead of shrinking the register set for a third wave.
-template <bool FAST>
-__global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))
+// The waves-per-SIMD attribute states the occupancy the workgroup size gives anyway
+// (one workgroup per CU), so that the compiler uses the whole register budget.
+template <bool FAST, int NCW>
+__global__ void __launch_bounds__((NCW + 4) * 64)
+    __attribute__((amdgpu_waves_per_eu((NCW + 4) / 4, (NCW + 4) / 4)))
     conv_fwd_kernel(const float *__restrict__ features, int cin, unsigned feat_bytes,
                     const float *__restrict__ packed, unsigned packed_bytes,
                     const int32_t *__restrict__ sched_in, const int32_t *__restrict__ sched_out,
                     const int32_t *__restrict__ grp_meta, unsigned sched_bytes, unsigned meta_bytes,
                     const int32_t *__restrict__ tile_grp, const int32_t *__restrict__ wg_tile,
-                    int nch, int ncb, int kvol, float *__restrict__ out, int64_t n_out, int cout,
+                    const int32_t *__restrict__ tile_row0, int nch, int ncb, int kvol, float *__restrict__ out, int64_t n_out, int cout,
                     int T) {
-  constexpr int NT = 512;
+  constexpr int kCN = 16 * NCW;   // output columns per workgroup
+  constexpr int kAS = kCN + 4;    // accumulator row stride in floats
+  constexpr int NT = (NCW + 4) * 64;
   constexpr int NP = 256;  // producer threads
   constexpr int NE = kStage * 16 / NP;
   extern __shared__ __align__(16) float lds[];
@@ -380,7 +451,7 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const bool producer = wave >= 4;
+  const bool producer = wave >= NCW;
   // Consecutive workgroup ids land on different XCDs (8 of them, one L2 each): give
   // every XCD a contiguous run of tile ranges so neighbouring tiles, which gather
   // the same input rows, share an L2.
@@ -402,26 +473,26 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
 
   // Tile `tl` is complete: write its rows, clear the accumulators.
   auto flush_tile = [&](int tl) {
-    const int64_t row0 = (int64_t)tl * T;
+    const int row0 = tile_row0[tl];
+    const int rows = tile_row0[tl + 1] - row0;
     if ((cout & 3) == 0) {
       const float4v z = {0.f, 0.f, 0.f, 0.f};
-      for (int e = tid; e < T * (kCN / 4); e += NT) {
+      for (int e = tid; e < rows * (kCN / 4); e += NT) {
         int r = e / (kCN / 4), c4 = e % (kCN / 4);
-        int64_t grow = row0 + r;
         int col = col0 + c4 * 4;
         float4v *ap = reinterpret_cast<float4v *>(acc + r * kAS + c4 * 4);
         // streaming store: the output is not read again by this kernel and must not
         // push the weights and the gathered rows out of L2
-        if (grow < n_out && col < cout)
-          __builtin_nontemporal_store(*ap, reinterpret_cast<float4v *>(out + grow * cout + col));
+        if (col < cout)
+          __builtin_nontemporal_store(
+              *ap, reinterpret_cast<float4v *>(out + (int64_t)(row0 + r) * cout + col));
         *ap = z;
       }
     } else {
-      for (int e = tid; e < T * kCN; e += NT) {
+      for (int e = tid; e < rows * kCN; e += NT) {
         int r = e / kCN, c = e % kCN;
-        int64_t grow = row0 + r;
-        if (grow < n_out && col0 + c < cout)
-          __builtin_nontemporal_store(acc[r * kAS + c], out + grow * cout + col0 + c);
+        if (col0 + c < cout)
+          __builtin_nontemporal_store(acc[r * kAS + c], out + (int64_t)(row0 + r) * cout + col0 + c);
         acc[r * kAS + c] = 0.f;
       }
     }
@@ -436,7 +507,7 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
 
   if (producer) {
     // ------------------------------------------------------------------ producer
-    const int pt = tid - 256;
+    const int pt = tid - NCW * 64;
     constexpr int RD = kRowsAhead, ID = kIdxAhead;
     static_assert(RD == 4 && ID == 2, "the rings below are sized for these distances");
     const __amdgpu_buffer_rsrc_t rs_in =
@@ -551,7 +622,7 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
     const int l16 = lane & 15;
     // A column group beyond Cout multiplies with the last real one's fragments; its
     // accumulator columns are never written out.
-    const int cb = min(blockIdx.y * 4 + wave, ncb - 1);
+    const int cb = min((int)blockIdx.y * NCW + wave, ncb - 1);
     const __amdgpu_buffer_rsrc_t rs_w =
         __builtin_amdgcn_make_buffer_rsrc((void *)packed, 0, (int)packed_bytes, kRsrcFlags);
     const __amdgpu_buffer_rsrc_t rs_out =
@@ -565,72 +636,74 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
 
     const __amdgpu_buffer_rsrc_t rs_meta =
         __builtin_amdgcn_make_buffer_rsrc((void *)grp_meta, 0, (int)meta_bytes, kRsrcFlags);
-    // What a stage needs besides the staged rows, fetched one stage ahead:
-    //   w[m][q]  weight fragments of row block m (four 16-byte loads per block)
-    //   orow[m]  LDS byte offset of the accumulator row of this lane's pair
-    //   rec      the schedule record (offsets of the 4 blocks, tile, last-of-tile) of
-    //            the stage AFTER this one, the same in every lane.  It travels through
-    //            vector loads and v_readfirstlane rather than scalar loads: scalar
-    //            loads return out of order, and one in flight would turn every
-    //            partial wait for LDS data below into a wait for everything.
-    struct StageRegs {
-      float4v w[4][4];
-      int orow[4];
-      int4v rec[2];
+    // Per-lane state of the consumer pipeline.  Row blocks are numbered through the
+    // stages (block 4s+m is block m of stage s); rings are indexed with the block or
+    // stage number, and the loop is unrolled over two stages so that every ring index
+    // is a compile-time constant.
+    //   w[b & 3][q]   weight fragments of block b (four 16-byte loads), fetched three
+    //                 blocks ahead: while block b multiplies, the slot of block b-1 is
+    //                 refilled for block b+3
+    //   orow[b & 3]   LDS byte offset of the accumulator row of this lane's pair in block b
+    //   rec[s & 1]    the schedule record (offsets of the 4 blocks, tile, last-of-tile)
+    //                 of stage s, the same in every lane.  It travels through vector
+    //                 loads and v_readfirstlane rather than scalar loads: scalar loads
+    //                 return out of order, and one in flight would turn every partial
+    //                 wait for LDS data below into a wait for everything.
+    float4v w[4][4];
+    int orow[4];
+    int4v rec[2][2];
+    auto load_rec = [&](const StagePos &pos, int4v (&r)[2]) {
+      r[0] = __builtin_bit_cast(int4v, buf_load4(rs_meta, 0, pos.g * 32));
+      r[1] = __builtin_bit_cast(int4v, buf_load4(rs_meta, 16, pos.g * 32));
     };
-    auto load_rec = [&](const StagePos &pos, int4v (&rec)[2]) {
-      rec[0] = __builtin_bit_cast(int4v, buf_load4(rs_meta, 0, pos.g * 32));
-      rec[1] = __builtin_bit_cast(int4v, buf_load4(rs_meta, 16, pos.g * 32));
+    // Byte offset of the weight fragments of a block at offset k (from a schedule
+    // record, possibly garbage beyond the schedule) and channel chunk cc.
+    auto frag_soff = [&](int k_lane, int cc) -> int {
+      const int k = __builtin_amdgcn_readfirstlane(k_lane);
+      // empty blocks (-1) and records beyond the schedule use the fragments of offset 0
+      const int kk = (k < 0 || k >= kvol) ? 0 : k;
+      return w_soff0 + kk * frag_k + cc * 4096;
     };
-    // Scalar part of fetching the stage at `pos`, whose record is `rec`: byte offsets
-    // of its four blocks' fragments, its tile and whether the tile ends with it.
-    struct StageScalars {
-      int soff[4];
-      int tile;
-      bool last;
+    auto rec_k = [](const int4v &v, int b) -> int {
+      return b == 0 ? v.x : b == 1 ? v.y : b == 2 ? v.z : v.w;
     };
-    auto stage_scalars = [&](const StagePos &pos, const int4v (&rec)[2]) -> StageScalars {
-      StageScalars sc;
-      const int k[4] = {
-          __builtin_amdgcn_readfirstlane(rec[0].x), __builtin_amdgcn_readfirstlane(rec[0].y),
-          __builtin_amdgcn_readfirstlane(rec[0].z), __builtin_amdgcn_readfirstlane(rec[0].w)};
-      sc.tile = __builtin_amdgcn_readfirstlane(rec[1].x);
-      sc.last = __builtin_amdgcn_readfirstlane(rec[1].y) != 0 && pos.cc == nch - 1;
-#pragma unroll
-      for (int b = 0; b < 4; ++b) {
-        // empty blocks (-1) and records beyond the schedule use the fragments of offset 0
-        const int kk = (k[b] < 0 || k[b] >= kvol) ? 0 : k[b];
-        sc.soff[b] = w_soff0 + kk * frag_k + pos.cc * 4096;
-      }
-      return sc;
+    auto fetch_w = [&](int soff, int slot, int q) {
+      w[slot][q] = buf_load4(rs_w, w_voff + q * 16, soff);
     };
-    auto fetch_w = [&](const StageScalars &sc, int b, int q, StageRegs &r) {
-      r.w[b][q] = buf_load4(rs_w, w_voff + q * 16, sc.soff[b]);
+    auto fetch_orow = [&](const StagePos &pos, int m, int slot) {
+      orow[slot] = buf_load1(rs_out, l16 * 4 + m * 64, pos.g * 256);
     };
-    auto fetch_orow = [&](const StagePos &pos, int b, StageRegs &r) {
-      r.orow[b] = buf_load1(rs_out, l16 * 4 + b * 64, pos.g * 256);
+    // An accumulator update whose write is still to come: row address, the row as it
+    // was read, and the product to add.
+    struct Pending {
+      int addr;
+      float4v accr, d;
     };
-    // One stage = 4 row blocks, software-pipelined by hand.  A wave issues in order
-    // and the 16 MFMAs of a block form one dependent chain, so whatever follows a
-    // chain in program order waits ~500 cycles for it, and whatever a chain waits
-    // for stalls the matrix pipe.  Therefore, in program order:
-    //   staged rows of block m+1 are read BEFORE the chain of block m starts;
-    //   the accumulator update of block m-1 (add, write) and the accumulator read of
-    //   block m sit AFTER the first four MFMAs of block m, in the shadow of the chain;
-    //   the 22 loads that fetch the next stage's registers are spread over the 16
-    //   groups of four MFMAs: a 16-byte-per-lane load keeps the wave in the issue
-    //   stage for tens of cycles, which a burst of loads would add to the stage and
+    const int dummy_addr = T * kAS * 4 + acc_lane;
+    Pending pend;  // nothing pending yet: the first write adds zero to the dummy row
+    pend.addr = dummy_addr;
+    pend.accr = float4v{0.f, 0.f, 0.f, 0.f};
+    pend.d = float4v{0.f, 0.f, 0.f, 0.f};
+    // One stage = 4 row blocks, software-pipelined by hand.  In program order:
+    //   the staged rows of block m+1 are read BEFORE the chain of block m starts;
+    //   the accumulator update of the previous block (add, write) and the accumulator
+    //   read of block m sit AFTER the first four MFMAs of block m, in the shadow of
+    //   the chain -- the update of a stage's last block waits, across the barrier,
+    //   for the first block of the next stage, unless the tile ends here;
+    //   the loads for block b+3 (and, once per stage, the record of the stage after
+    //   the next) are spread over the four groups of four MFMAs of block b: a
+    //   16-byte-per-lane load keeps the wave in the issue stage for tens of cycles,
     //   which is free behind an MFMA whose successor must wait for it anyway.
     // Scheduling barriers pin that order (the compiler otherwise moves the LDS reads
     // next to their first use to shorten live ranges).  LDS operations of a wave
     // execute in order, so the read of block m's rows after the write of block m-1
     // sees that write when both blocks touch the same output row.
-    auto run_stage = [&](int parity, const StagePos &next, const StagePos &after,
-                         const StageRegs &cur, StageRegs &nxt, int &tile_next, bool &last_next) {
-      const StageScalars sc = stage_scalars(next, cur.rec);
-      tile_next = sc.tile;
-      last_next = sc.last;
-      const float *ab = a_base + parity * kStage * kAStride;
+    //   cur / next / after: positions of this stage and the two that follow;
+    //   returns tile and last-of-tile of the NEXT stage.
+    auto run_stage = [&](auto parity, bool last_cur, const StagePos &cur, const StagePos &next,
+                         const StagePos &after, int &tile_next, bool &last_next) {
+      constexpr int par = decltype(parity)::value;
+      const float *ab = a_base + par * kStage * kAStride;
       float4v a[2][4];
       auto load_a = [&](int m, float4v (&av)[4]) {
         const float4v *ap = reinterpret_cast<const float4v *>(ab + m * 16 * kAStride);
@@ -638,67 +711,78 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
         for (int q = 0; q < 4; ++q) av[q] = ap[q];
       };
       load_a(0, a[0]);
-      float4v accr, dprev;
-      accr = *reinterpret_cast<const float4v *>(acc_bytes + cur.orow[0] + acc_lane);
 #pragma unroll
       for (int m = 0; m < 4; ++m) {
+        const int slot = m;                 // == (4 * s + m) & 3
+        const int tslot = (m + 3) & 3;      // slot of block b+3 == slot of block b-1
+        const int tm = (m + 3) & 3;         // index of block b+3 inside its stage
+        const bool tnext = m > 0;           // block b+3 belongs to the next stage
         if (m < 3) load_a(m + 1, a[(m + 1) & 1]);
         __builtin_amdgcn_sched_barrier(0);
         float4v d = float4v{0.f, 0.f, 0.f, 0.f};
-        mfma_quad(cur.w[m][0], a[m & 1][0], d);
+        mfma_quad(w[slot][0], a[m & 1][0], d);
         __builtin_amdgcn_sched_barrier(0);
-        fetch_w(sc, m, 0, nxt);
-        if (m > 0) {
-          // dprev = out[pair l16][channels 4g .. 4g+3] of block m-1
-          *reinterpret_cast<float4v *>(acc_bytes + cur.orow[m - 1] + acc_lane) = accr + dprev;
-          accr = *reinterpret_cast<const float4v *>(acc_bytes + cur.orow[m] + acc_lane);
-        }
+        const int soff = tnext ? frag_soff(rec_k(rec[par ^ 1][0], tm), next.cc)
+                               : frag_soff(rec_k(rec[par][0], tm), cur.cc);
+        fetch_w(soff, tslot, 0);
+        // pend.d = out[pair l16][channels 4g .. 4g+3] of the previous block
+        *reinterpret_cast<float4v *>(acc_bytes + pend.addr) = pend.accr + pend.d;
+        pend.addr = orow[slot] + acc_lane;
+        pend.accr = *reinterpret_cast<const float4v *>(acc_bytes + pend.addr);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int q = 1; q < 4; ++q) {
-          mfma_quad(cur.w[m][q], a[m & 1][q], d);
+          mfma_quad(w[slot][q], a[m & 1][q], d);
           __builtin_amdgcn_sched_barrier(0);
-          fetch_w(sc, m, q, nxt);
-          if (q == 1) fetch_orow(next, m, nxt);
-          if (q == 2 && m >= 2) nxt.rec[m - 2] = __builtin_bit_cast(
-              int4v, buf_load4(rs_meta, (m - 2) * 16, after.g * 32));
+          fetch_w(soff, tslot, q);
+          if (q == 1) fetch_orow(tnext ? next : cur, tm, tslot);
+          // this stage's record was last used by block 0: refill it for the stage
+          // after the next
+          if (m == 1 && q >= 2) rec[par][q - 2] = __builtin_bit_cast(
+              int4v, buf_load4(rs_meta, (q - 2) * 16, after.g * 32));
+          if (m == 3 && q == 3) {
+            tile_next = __builtin_amdgcn_readfirstlane(rec[par ^ 1][1].x);
+            last_next =
+                __builtin_amdgcn_readfirstlane(rec[par ^ 1][1].y) != 0 && next.cc == nch - 1;
+          }
           __builtin_amdgcn_sched_barrier(0);
         }
-        dprev = d;
+        pend.d = d;
       }
       __builtin_amdgcn_sched_barrier(0);
-      *reinterpret_cast<float4v *>(acc_bytes + cur.orow[3] + acc_lane) = accr + dprev;
-    };
-    // Everything the first stage needs, in one batch.
-    auto fetch_all = [&](const StagePos &pos, const StagePos &after, const int4v (&rec)[2],
-                         StageRegs &r, int &tile, bool &last) {
-      const StageScalars sc = stage_scalars(pos, rec);
-      tile = sc.tile;
-      last = sc.last;
-#pragma unroll
-      for (int b = 0; b < 4; ++b) {
-#pragma unroll
-        for (int q = 0; q < 4; ++q) fetch_w(sc, b, q, r);
-        fetch_orow(pos, b, r);
+      if (last_cur) {  // the tile is written out after this stage: finish its last update
+        *reinterpret_cast<float4v *>(acc_bytes + pend.addr) = pend.accr + pend.d;
+        pend.addr = dummy_addr;
       }
-      load_rec(after, r.rec);
     };
-    StageRegs rx, ry;
-    StagePos p_next = {g_begin, 0};   // stage whose registers are fetched next
-    StagePos p_after = {g_begin, 0};  // the stage after that one
+    StagePos p_cur = {g_begin, 0};    // stage being multiplied
+    StagePos p_next = {g_begin, 0};   // the stage after it
+    StagePos p_after = {g_begin, 0};  // and the one after that
+    p_next.advance(nch);
+    p_after.advance(nch);
     p_after.advance(nch);
     int tile, tile_next;
     bool last, last_next;
     {
-      int4v rec0[2];
-      load_rec(p_next, rec0);
-      fetch_all(p_next, p_after, rec0, rx, tile, last);
-      p_next.advance(nch);
-      p_after.advance(nch);
+      // what the first stage needs before it starts: its record and the next one,
+      // fragments and rows of its blocks 0..2
+      load_rec(p_cur, rec[0]);
+      load_rec(p_next, rec[1]);
+      tile = __builtin_amdgcn_readfirstlane(rec[0][1].x);
+      last = __builtin_amdgcn_readfirstlane(rec[0][1].y) != 0 && p_cur.cc == nch - 1;
+#pragma unroll
+      for (int b = 0; b < 3; ++b) {
+        const int soff = frag_soff(rec_k(rec[0][0], b), p_cur.cc);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) fetch_w(soff, b, q);
+        fetch_orow(p_cur, b, b);
+      }
     }
     __syncthreads();
     for (int s = 0; s < nstages; s += 2) {
-      run_stage(0, p_next, p_after, rx, ry, tile_next, last_next);
+      run_stage(std::integral_constant<int, 0>(), last, p_cur, p_next, p_after, tile_next,
+                last_next);
+      p_cur.advance(nch);
       p_next.advance(nch);
       p_after.advance(nch);
       __syncthreads();
@@ -709,7 +793,9 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
       tile = tile_next;
       last = last_next;
       if (s + 1 < nstages) {
-        run_stage(1, p_next, p_after, ry, rx, tile_next, last_next);
+        run_stage(std::integral_constant<int, 1>(), last, p_cur, p_next, p_after, tile_next,
+                  last_next);
+        p_cur.advance(nch);
         p_next.advance(nch);
         p_after.advance(nch);
         __syncthreads();
@@ -725,20 +811,20 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
 }
 
 struct ConvPlan {
-  int ncb, nch, T, n_wg, n_colblk;
+  int ncb, nch, T, ncw, n_wg, n_colblk;
   bool fast;
-  int64_t n_tiles, words_per_k, grp_cap;
+  int64_t n_tiles, n_fine, words_per_k, grp_cap;  // n_tiles: upper bound
   size_t lds_bytes;
 };
 
-static size_t conv_lds_bytes(int T) {
-  return ((size_t)(T + 1) * kAS + 2 * (size_t)kStage * kAStride) * 4;
+static size_t conv_lds_bytes(int T, int ncw) {
+  return ((size_t)(T + 1) * (16 * ncw + 4) + 2 * (size_t)kStage * kAStride) * 4;
 }
 
-static int pick_tile() {
+static int pick_tile(int ncw) {
   // One workgroup per CU: (almost) all of the 160 KB of LDS goes to the accumulators.
-  size_t budget = 160 * 1024 - conv_lds_bytes(0) - 512;
-  int t = (int)(budget / ((size_t)kAS * 4));
+  size_t budget = 160 * 1024 - conv_lds_bytes(0, ncw) - 512;
+  int t = (int)(budget / ((size_t)(16 * ncw + 4) * 4));
   t = t / 8 * 8;
   if (t < kMinTile) t = kMinTile;
   return t;
@@ -761,24 +847,27 @@ static ConvPlan make_plan(int64_t n_in, int64_t n_out, int K, int c_in, int c_ou
   ConvPlan p;
   p.ncb = (int)ceil_div(c_out, 16);
   p.nch = (int)ceil_div(c_in, kKC);
-  p.T = pick_tile();
+  p.ncw = 4;
+  p.T = pick_tile(p.ncw);
   // the gather can be a range-checked buffer load when every 64-channel chunk is
   // complete and byte offsets into the features (plus the padding marker) fit 32 bits
   p.fast = (c_in % kKC) == 0 && (uint64_t)n_in * c_in * 4 <= (uint64_t)kGatherPad;
-  p.n_tiles = ceil_div(n_out > 0 ? n_out : 1, p.T);
+  p.n_colblk = (int)ceil_div(p.ncb, p.ncw);
+  int n_wg = device_cu_count() / p.n_colblk;
+  if (n_wg < 1) n_wg = 1;
+  if (n_wg > 256) n_wg = 256;  // the split kernel is one block of 256 threads
+  if (n_wg >= 8) n_wg = n_wg / 8 * 8;
+  p.n_wg = n_wg;
+  // upper bound of the tile count: every workgroup's range ends with a partial tile
+  p.n_tiles = ceil_div(n_out > 0 ? n_out : 1, p.T) + n_wg;
+  p.n_fine = ceil_div(n_out > 0 ? n_out : 1, kSplitGranule);
   p.words_per_k = ceil_div(n_out > 0 ? n_out : 1, 32);
   // groups: pairs/64 plus, per (tile, offset), up to one partial block, plus one
   // partial (or empty) group per tile, plus the groups the kernel's prefetches may
   // touch beyond the end of the schedule
   int64_t max_pairs_k = pair_stride < n_out ? pair_stride : n_out;
   p.grp_cap = ((int64_t)K * (max_pairs_k / 16 + 1) + p.n_tiles * K) / 4 + 2 * p.n_tiles + 4 + 16;
-  p.n_colblk = (int)ceil_div(p.ncb, 4);
-  int n_wg = device_cu_count() / p.n_colblk;
-  if (n_wg < 1) n_wg = 1;
-  if (n_wg > p.n_tiles) n_wg = (int)p.n_tiles;
-  if (n_wg >= 8) n_wg = n_wg / 8 * 8;
-  p.n_wg = n_wg;
-  p.lds_bytes = conv_lds_bytes(p.T);
+  p.lds_bytes = conv_lds_bytes(p.T, p.ncw);
   return p;
 }
 
@@ -790,6 +879,7 @@ struct ConvWs {
   uint32_t *bits;
   int32_t *prefix;
   int32_t *tile_cnt, *tile_nmb, *kofs, *tile_grp, *wg_tile;
+  int32_t *fine_segs, *fine_work, *tile_row0, *n_tiles_dev;
   int32_t *sched_in, *sched_out, *grp_meta;
 };
 
@@ -807,6 +897,10 @@ static size_t conv_ws_walk(void *base, const ConvPlan &p, int K, int64_t pair_st
   t.kofs = c.take<int32_t>((size_t)p.n_tiles * K);
   t.tile_grp = c.take<int32_t>((size_t)p.n_tiles + 1);
   t.wg_tile = c.take<int32_t>((size_t)p.n_wg + 1);
+  t.fine_segs = c.take<int32_t>((size_t)(p.n_fine + 1) * K);
+  t.fine_work = c.take<int32_t>((size_t)p.n_fine + 1);
+  t.tile_row0 = c.take<int32_t>((size_t)p.n_tiles + 1);
+  t.n_tiles_dev = c.take<int32_t>(1);
   t.sched_in = c.take<int32_t>((size_t)p.grp_cap * 64);
   t.sched_out = c.take<int32_t>((size_t)p.grp_cap * 64);
   t.grp_meta = c.take<int32_t>((size_t)p.grp_cap * 8);
@@ -820,12 +914,12 @@ static size_t conv_ws_bytes(int64_t n_out, int K, int c_in, int c_out, int64_t p
   return conv_ws_walk(nullptr, p, K, pair_stride, nullptr);
 }
 
-template <bool FAST>
+template <bool FAST, int NCW>
 static int launch_conv(const ConvPlan &p, const ConvWs &w, const float *features, int64_t n_in,
                        int c_in, int K, float *out, int64_t n_out, int c_out, hipStream_t s) {
   static bool attr_set = false;
   if (!attr_set) {
-    SSC_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(conv_fwd_kernel<FAST>),
+    SSC_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(conv_fwd_kernel<FAST, NCW>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
     attr_set = true;
   }
@@ -836,10 +930,10 @@ static int launch_conv(const ConvPlan &p, const ConvWs &w, const float *features
             (unsigned long long)packed_bytes, (unsigned long long)sched_bytes);
   const unsigned feat_bytes = FAST ? (unsigned)((uint64_t)n_in * c_in * 4) : 0u;
   dim3 grid((unsigned)p.n_wg, (unsigned)p.n_colblk);
-  hipLaunchKernelGGL((conv_fwd_kernel<FAST>), grid, dim3(512), p.lds_bytes, s, features, c_in,
+  hipLaunchKernelGGL((conv_fwd_kernel<FAST, NCW>), grid, dim3((NCW + 4) * 64), p.lds_bytes, s, features, c_in,
                      feat_bytes, w.packed, (unsigned)packed_bytes, w.sched_in, w.sched_out,
                      w.grp_meta, (unsigned)sched_bytes, (unsigned)(p.grp_cap * 32), w.tile_grp,
-                     w.wg_tile, p.nch, p.ncb, K, out, n_out, c_out, p.T);
+                     w.wg_tile, w.tile_row0, p.nch, p.ncb, K, out, n_out, c_out, p.T);
   SSC_LAUNCH_CHECK("conv_fwd");
   return SSC_OK;
 }
@@ -942,29 +1036,38 @@ int ssc_conv_fwd_f32(const float *features, int64_t n_in, int32_t c_in, const fl
                      pair_stride, plane_s, pair_num, w.bits, w.prefix, p.words_per_k, w.sorted);
   SSC_LAUNCH_CHECK("resort");
 
+  // work split on the fine grid, then the tiles and their segments
+  int64_t nfine = (p.n_fine + 1) * K;
+  hipLaunchKernelGGL(tile_segments_kernel, dim3((unsigned)ceil_div(nfine, 256)), dim3(256), 0, s,
+                     w.flag, pairs, w.sorted, pair_stride, plane_s, pair_num, K, p.n_fine,
+                     (const int32_t *)nullptr, (const int32_t *)nullptr, kSplitGranule, n_out,
+                     w.fine_segs);
+  hipLaunchKernelGGL(split_sum_kernel, dim3((unsigned)ceil_div(p.n_fine + 1, 256)), dim3(256), 0, s,
+                     w.fine_segs, K, p.n_fine, w.fine_work);
+  hipLaunchKernelGGL(split_rows_kernel, dim3(1), dim3(256), 0, s, w.fine_work, p.n_fine, n_out,
+                     p.T, K, p.n_wg, w.wg_tile, w.tile_row0, w.n_tiles_dev);
+  SSC_LAUNCH_CHECK("split");
   int64_t nseg = (p.n_tiles + 1) * K;
   hipLaunchKernelGGL(tile_segments_kernel, dim3((unsigned)ceil_div(nseg, 256)), dim3(256), 0, s,
-                     w.flag, pairs, w.sorted, pair_stride, plane_s, pair_num, K, p.n_tiles, p.T,
-                     w.segs);
+                     w.flag, pairs, w.sorted, pair_stride, plane_s, pair_num, K, p.n_tiles,
+                     w.n_tiles_dev, w.tile_row0, 0, n_out, w.segs);
   SSC_LAUNCH_CHECK("tile_segments");
   hipLaunchKernelGGL(sched_count_kernel, dim3((unsigned)ceil_div(p.n_tiles, 256)), dim3(256), 0, s,
-                     w.segs, K, p.n_tiles, w.tile_cnt, w.tile_nmb, w.kofs);
-  hipLaunchKernelGGL(sched_scan_kernel, dim3(1), dim3(kScanThreads), 0, s, w.tile_cnt, p.n_tiles,
-                     w.tile_grp);
+                     w.segs, K, w.n_tiles_dev, w.tile_cnt, w.tile_nmb, w.kofs);
+  hipLaunchKernelGGL(sched_scan_kernel, dim3(1), dim3(kScanThreads), 0, s, w.tile_cnt,
+                     w.n_tiles_dev, w.tile_grp);
   hipLaunchKernelGGL(sched_fill_kernel, dim3((unsigned)ceil_div(p.n_tiles * K * 16, 256)),
                      dim3(256), 0, s, w.flag, pairs, w.sorted, pair_stride, plane_g, w.segs,
-                     w.kofs, w.tile_nmb, w.tile_grp, K, p.n_tiles, p.T,
-                     p.fast ? (uint32_t)c_in * 4u : 1u, p.fast ? kGatherPad : 0xFFFFFFFFu, kAS * 4,
-                     w.sched_in, w.sched_out, w.grp_meta);
-  hipLaunchKernelGGL(sched_split_kernel, dim3((unsigned)ceil_div(p.n_wg + 1, 256)), dim3(256), 0,
-                     s, w.tile_grp, p.n_tiles, p.n_wg, w.wg_tile);
+                     w.kofs, w.tile_nmb, w.tile_grp, K, w.n_tiles_dev, w.tile_row0, p.T,
+                     p.fast ? (uint32_t)c_in * 4u : 1u, p.fast ? kGatherPad : 0xFFFFFFFFu,
+                     (16 * p.ncw + 4) * 4, w.sched_in, w.sched_out, w.grp_meta);
   SSC_LAUNCH_CHECK("schedule");
 
   const bool prof = g_profile_on;
   const int slot = g_profile_count % kProfileRing;
   if (prof) SSC_HIP(hipEventRecord(g_profile_ev[slot][0], s));
-  rc = p.fast ? launch_conv<true>(p, w, features, n_in, c_in, K, out, n_out, c_out, s)
-              : launch_conv<false>(p, w, features, n_in, c_in, K, out, n_out, c_out, s);
+  rc = p.fast ? launch_conv<true, 4>(p, w, features, n_in, c_in, K, out, n_out, c_out, s)
+              : launch_conv<false, 4>(p, w, features, n_in, c_in, K, out, n_out, c_out, s);
   if (rc != SSC_OK) return rc;
   if (prof) {
     SSC_HIP(hipEventRecord(g_profile_ev[slot][1], s));
