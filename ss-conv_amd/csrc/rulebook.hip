@@ -80,19 +80,52 @@ __device__ __forceinline__ bool pair_key(const Geom &g, const int32_t *__restric
   return true;
 }
 
-// Regular conv: mark every output cell reachable from an active input.
-// One thread per (input row, tap).
+// Regular conv: mark every output cell reachable from an active input, and count
+// the pairs of every 64-row chunk (chunk_count is [K, n_chunks]; for a regular
+// convolution a pair exists wherever the geometry allows it, so the counts do not
+// depend on the table).  One wave per chunk of 64 input rows, one lane per row.
+// The taps of one (kx, ky) differ in z only, so their output cells are neighbours
+// in the key space: their bits are gathered into one mask per 32-bit word, the word
+// is read first, and the atomic is issued only when it would change the word
+// (most cells are reached from several inputs).
 __global__ void __launch_bounds__(256)
-    mark_outputs_kernel(const int32_t *__restrict__ indices, int64_t n_in, Geom g,
-                        uint32_t *__restrict__ bits) {
-  int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (t >= n_in * g.K) return;
-  int64_t i = t / g.K;
-  int k = (int)(t - i * g.K);
-  int32_t row[4];
-  *reinterpret_cast<int4 *>(row) = reinterpret_cast<const int4 *>(indices)[i];
-  uint32_t key;
-  if (pair_key(g, row, k, &key)) atomicOr(&bits[key >> 5], 1u << (key & 31u));
+    mark_count_kernel(const int32_t *__restrict__ indices, int64_t n_in, Geom g,
+                      uint32_t *__restrict__ bits, int32_t *__restrict__ chunk_count,
+                      int64_t n_chunks) {
+  int64_t chunk = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (chunk >= n_chunks) return;
+  const int lane = threadIdx.x & 63;
+  int64_t i = chunk * 64 + lane;
+  const bool live = i < n_in;
+  int32_t row[4] = {0, 0, 0, 0};
+  if (live) *reinterpret_cast<int4 *>(row) = reinterpret_cast<const int4 *>(indices)[i];
+  int k = 0;
+  for (int kx = 0; kx < g.ks[0]; ++kx) {
+    int ox = 0;
+    const bool okx = live && tap_to_out(row[1], kx, g.st[0], g.pd[0], g.dl[0], g.os[0], &ox);
+    for (int ky = 0; ky < g.ks[1]; ++ky) {
+      int oy = 0;
+      const bool okxy = okx && tap_to_out(row[2], ky, g.st[1], g.pd[1], g.dl[1], g.os[1], &oy);
+      const uint32_t base = (uint32_t)(((row[0] * g.os[0] + ox) * g.os[1] + oy) * g.os[2]);
+      uint32_t word = 0xFFFFFFFFu, mask = 0u;
+      for (int kz = 0; kz < g.ks[2]; ++kz, ++k) {
+        int oz = 0;
+        const bool ok = okxy && tap_to_out(row[3], kz, g.st[2], g.pd[2], g.dl[2], g.os[2], &oz);
+        unsigned long long m = __ballot(ok);
+        if (lane == 0) chunk_count[(int64_t)k * n_chunks + chunk] = __popcll(m);
+        if (ok) {
+          const uint32_t key = base + (uint32_t)oz;
+          if ((key >> 5) != word) {
+            if (mask != 0u && (bits[word] & mask) != mask) atomicOr(&bits[word], mask);
+            word = key >> 5;
+            mask = 0u;
+          }
+          mask |= 1u << (key & 31u);
+        }
+      }
+      if (mask != 0u && (bits[word] & mask) != mask) atomicOr(&bits[word], mask);
+    }
+  }
 }
 
 // Submanifold / unique: mark the cells of the rows themselves.
@@ -115,17 +148,31 @@ __global__ void __launch_bounds__(256)
   uint32_t b = bits[w];
   if (b == 0) return;
   int r = prefix[w];
+  // the word's first cell is decoded once; its other cells differ in z only, unless
+  // the word runs over the end of a z row (extents that are not multiples of 32)
+  uint32_t key0 = (uint32_t)(w * 32);
+  const int z0 = key0 % d3;
+  key0 /= d3;
+  const int y0 = key0 % d2;
+  key0 /= d2;
+  const int x0 = key0 % d1;
+  const int b0 = key0 / d1;
   while (b) {
     int bit = __ffs(b) - 1;
     b &= b - 1;
-    uint32_t key = (uint32_t)(w * 32 + bit);
-    int z = key % d3;
-    key /= d3;
-    int y = key % d2;
-    key /= d2;
-    int x = key % d1;
-    int bb = key / d1;
-    reinterpret_cast<int4 *>(out)[r++] = make_int4(bb, x, y, z);
+    int z = z0 + bit;
+    if (z < d3) {
+      reinterpret_cast<int4 *>(out)[r++] = make_int4(b0, x0, y0, z);
+    } else {
+      uint32_t key = (uint32_t)(w * 32 + bit);
+      z = key % d3;
+      key /= d3;
+      int y = key % d2;
+      key /= d2;
+      int x = key % d1;
+      int bb = key / d1;
+      reinterpret_cast<int4 *>(out)[r++] = make_int4(bb, x, y, z);
+    }
   }
 }
 
@@ -145,8 +192,9 @@ __device__ __forceinline__ bool bit_test(const uint32_t *__restrict__ bits, uint
   return (bits[key >> 5] >> (key & 31u)) & 1u;
 }
 
-// Pair counting: one wave per chunk of 64 input rows, per tap the number of
-// rows of the chunk that own a pair.  chunk_count is [K, n_chunks].
+// Pair counting for the submanifold rulebook (a pair needs its output cell to be
+// active): one wave per chunk of 64 input rows, per tap the number of rows of the
+// chunk that own a pair.  chunk_count is [K, n_chunks].
 __global__ void __launch_bounds__(256)
     count_pairs_kernel(const int32_t *__restrict__ indices, int64_t n_in, Geom g,
                        const uint32_t *__restrict__ bits, int32_t *__restrict__ chunk_count,
@@ -218,24 +266,44 @@ __global__ void __launch_bounds__(256)
   bool live = i < n_in;
   int32_t row[4] = {0, 0, 0, 0};
   if (live) *reinterpret_cast<int4 *>(row) = reinterpret_cast<const int4 *>(indices)[i];
-  for (int k = 0; k < g.K; ++k) {
-    uint32_t key = 0;
-    bool ok = live && pair_key(g, row, k, &key);
-    if (ok && g.subm) ok = bit_test(bits, key);
-    unsigned long long m = __ballot(ok);
-    int32_t *pin = pairs + ((int64_t)k * 2 + 0) * n_in;
-    int32_t *pout = pairs + ((int64_t)k * 2 + 1) * n_in;
-    if (ok) {
-      int slot = chunk_prefix[(int64_t)k * n_chunks + chunk] +
-                 __popcll(m & ((1ull << lane) - 1ull));
-      int r = bit_rank(bits, prefix, key);
-      if (g.subm) r = rank2row[r];
-      pin[slot] = (int32_t)i;
-      pout[slot] = r;
-    }
-    if (live && i >= pair_num[k]) {
-      pin[i] = -1;
-      pout[i] = -1;
+  // The taps of one (kx, ky) differ in z only: their cells are neighbours in the key
+  // space, so the table word and its prefix are loaded once per word, not per tap.
+  uint32_t word = 0xFFFFFFFFu, wbits = 0u;
+  int wprefix = 0;
+  int k = 0;
+  for (int kx = 0; kx < g.ks[0]; ++kx) {
+    int ox = 0;
+    const bool okx = live && tap_to_out(row[1], kx, g.st[0], g.pd[0], g.dl[0], g.os[0], &ox);
+    for (int ky = 0; ky < g.ks[1]; ++ky) {
+      int oy = 0;
+      const bool okxy = okx && tap_to_out(row[2], ky, g.st[1], g.pd[1], g.dl[1], g.os[1], &oy);
+      const uint32_t base = (uint32_t)(((row[0] * g.os[0] + ox) * g.os[1] + oy) * g.os[2]);
+      for (int kz = 0; kz < g.ks[2]; ++kz, ++k) {
+        int oz = 0;
+        bool ok = okxy && tap_to_out(row[3], kz, g.st[2], g.pd[2], g.dl[2], g.os[2], &oz);
+        const uint32_t key = base + (uint32_t)oz;
+        if (ok && (key >> 5) != word) {
+          word = key >> 5;
+          wbits = bits[word];
+          wprefix = prefix[word];
+        }
+        if (ok && g.subm) ok = (wbits >> (key & 31u)) & 1u;
+        unsigned long long m = __ballot(ok);
+        int32_t *pin = pairs + ((int64_t)k * 2 + 0) * n_in;
+        int32_t *pout = pairs + ((int64_t)k * 2 + 1) * n_in;
+        if (ok) {
+          int slot = chunk_prefix[(int64_t)k * n_chunks + chunk] +
+                     __popcll(m & ((1ull << lane) - 1ull));
+          int r = wprefix + __popc(wbits & ((1u << (key & 31u)) - 1u));
+          if (g.subm) r = rank2row[r];
+          pin[slot] = (int32_t)i;
+          pout[slot] = r;
+        }
+        if (live && i >= pair_num[k]) {
+          pin[i] = -1;
+          pout[i] = -1;
+        }
+      }
     }
   }
 }
@@ -314,9 +382,9 @@ int ssc_rulebook_count(const int32_t *indices, int64_t n_in, const ssc_geometry 
                        indices, n_in, gg.os[0], gg.os[1], gg.os[2], w.table.bits);
     SSC_LAUNCH_CHECK("mark_rows");
   } else {
-    hipLaunchKernelGGL(mark_outputs_kernel, dim3((unsigned)ceil_div(n_in * gg.K, 256)), dim3(256),
-                       0, s, indices, n_in, gg, w.table.bits);
-    SSC_LAUNCH_CHECK("mark_outputs");
+    hipLaunchKernelGGL(mark_count_kernel, dim3((unsigned)ceil_div(w.n_chunks, 4)), dim3(256), 0, s,
+                       indices, n_in, gg, w.table.bits, w.chunk_count, w.n_chunks);
+    SSC_LAUNCH_CHECK("mark_count");
   }
   if ((rc = bit_table_scan(w.table, s)) != SSC_OK) return rc;
   int32_t total = 0;
@@ -352,9 +420,11 @@ int ssc_rulebook_emit(const int32_t *indices, int64_t n_in, const ssc_geometry *
                        gg.os[1], gg.os[2], out_indices);
     SSC_LAUNCH_CHECK("emit_rows");
   }
-  hipLaunchKernelGGL(count_pairs_kernel, dim3(chunk_blocks), dim3(256), 0, s, indices, n_in, gg,
-                     w.table.bits, w.chunk_count, w.n_chunks);
-  SSC_LAUNCH_CHECK("count_pairs");
+  if (gg.subm) {  // a regular convolution's counts were taken while marking the table
+    hipLaunchKernelGGL(count_pairs_kernel, dim3(chunk_blocks), dim3(256), 0, s, indices, n_in, gg,
+                       w.table.bits, w.chunk_count, w.n_chunks);
+    SSC_LAUNCH_CHECK("count_pairs");
+  }
   hipLaunchKernelGGL(scan_chunks_kernel, dim3(gg.K), dim3(kScanThreads), 0, s, w.chunk_count,
                      w.n_chunks, pair_num);
   SSC_LAUNCH_CHECK("scan_chunks");
