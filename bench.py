@@ -41,6 +41,10 @@ def parse_args():
                     help="also run one plain device copy of MIB mebibytes before the timed "
                          "region (the known-size kernel that scales rocprofv3's FETCH_SIZE / "
                          "WRITE_SIZE counters)")
+    ap.add_argument("--ops", action="store_true",
+                    help="also time the other operators of the path (pools, global pools, "
+                         "Point2Voxel, Voxel2Point) against their algorithmic HBM bytes; "
+                         "table on stderr")
     ap.add_argument("--breakdown", action="store_true",
                     help="also print per-phase timings to stderr")
     return ap.parse_args()
@@ -75,6 +79,90 @@ def cpu_baseline(idx, feats, dense_w, cfg, n_out_expected):
             "sample": "full %s layer (rulebook + gather/GEMM/scatter conv), median of %d runs, "
                       "%.2f s each; rulebook and gather/scatter single-thread C, GEMM numpy BLAS"
                       % (cfg["name"], len(times), t)}, out
+
+
+def ops_table(torch, _ext, synth, dev, seed):
+    """Times the bandwidth-bound operators of the path on synthetic inputs of the
+    benchmark shapes and prints time, algorithmic bytes and GB/s (of 8000 GB/s HBM
+    peak) for each.  Rulebooks are built outside the timed region, except for the
+    "module" rows, which time the user-facing layer as the reference runs it."""
+    import numpy as np
+    from ss_conv.pool import MaxPool, AvgPool, GlobalAvgPool, GlobalMaxPool
+    from ss_conv.sp_ops.ops import get_indice_pairs, get_conv_output_size
+    from ss_conv.sp_ops.tensor import SparseTensor
+    from ss_conv.sp_ops.voxelize import Point2Voxel, Voxel2Point
+
+    def timed(fn, n=20, warm=3):
+        for _ in range(warm):
+            fn()
+        torch.cuda.synchronize()
+        a = time.perf_counter()
+        for _ in range(n):
+            r = fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - a) * 1e3 / n, r
+
+    rows = []
+
+    def report(name, ms, nbytes, note=""):
+        gbs = nbytes / ms / 1e6
+        rows.append("%-44s %8.3f ms %9.2f MB %8.1f GB/s %5.1f%% of HBM  %s"
+                    % (name, ms, nbytes / 1e6, gbs, gbs / 80.0, note))
+
+    # pools on the output of the stride-2 layer: 32 clouds at 32^3, 256 channels
+    cfg = synth.CONFIGS["cfg3"]
+    pts, feats, ids = synth.config_clouds("cfg3", seed)
+    idx = torch.from_numpy(synth.voxel_indices(pts, ids, cfg["grid"])).to(dev)
+    shape = [cfg["grid"]] * 3
+    o_idx, _, _ = get_indice_pairs(idx, cfg["batch"], shape, 3, 2, 1)
+    shape2 = get_conv_output_size(shape, [3] * 3, [2] * 3, [1] * 3, [1] * 3)
+    C = 256
+    x = torch.randn(o_idx.shape[0], C, device=dev)
+    st = SparseTensor(x, o_idx, shape2, cfg["batch"])
+    p_idx, p_pairs, p_num = get_indice_pairs(o_idx, cfg["batch"], shape2, 2, 2, 0)
+    P = int(p_num.sum().item())
+    n_in, n_out = x.shape[0], p_idx.shape[0]
+    nbytes = 4 * C * (n_in + n_out) + 8 * P
+    ms, _ = timed(lambda: _ext.indice_maxpool_fp32(x, p_pairs, p_num, n_out))
+    report("max pool k2 s2 (kernel, %d->%d rows, C=%d)" % (n_in, n_out, C), ms, nbytes)
+    rf = _ext.indiceSummaryRF(p_pairs, p_num, n_out)
+    ms, _ = timed(lambda: _ext.indice_avgpool_fp32(x, p_pairs, p_num, n_out, rf))
+    report("avg pool k2 s2 (kernel)", ms, nbytes)
+    mp = MaxPool(2, 2)
+    ms, _ = timed(lambda: mp(st))
+    report("MaxPool module (rulebook + kernel)", ms, nbytes + 16 * (n_in + n_out), "incl. rulebook")
+
+    # global pools: 32 segments over the pooled rows, 512 channels
+    C = 512
+    f = torch.randn(n_in, C, device=dev)
+    offs = st.get_offsets().int().contiguous()
+    B = offs.numel() - 1
+    nbytes = 4 * C * (n_in + B) + 4 * (B + 1)
+    ga, gm = GlobalAvgPool(), GlobalMaxPool()
+    ms, _ = timed(lambda: ga(f, offs))
+    report("GlobalAvgPool (%d rows, %d segments, C=%d)" % (n_in, B, C), ms, nbytes)
+    ms, _ = timed(lambda: gm(f, offs))
+    report("GlobalMaxPool", ms, nbytes + 4 * C * B)
+
+    # Point2Voxel on the cfg2 clouds (65536 points, 64 channels) and Voxel2Point back
+    cfg = synth.CONFIGS["cfg2"]
+    pts, feats, ids = synth.config_clouds("cfg2", seed)
+    C = 64
+    tp = torch.from_numpy(pts).to(dev)
+    tf = torch.randn(tp.shape[0], C, device=dev)
+    ti = torch.from_numpy(ids).to(dev)
+    p2v = Point2Voxel([cfg["grid"]] * 3, [2.0 / cfg["grid"]] * 3)
+    ms, r = timed(lambda: p2v(tp, tf, ti), n=10)
+    N, M = tp.shape[0], r[1].features.shape[0]
+    report("Point2Voxel module (%d pts -> %d voxels, C=%d)" % (N, M, C), ms,
+           N * (12 + 8 + 4 * C) + M * (16 + 4 * C) + 4 * N, "torch filtering + sort included")
+    v2p = Voxel2Point(unit_voxel_extent=[2.0 / cfg["grid"]] * 3)
+    vp, vs, vi = r[0], r[1], r[2]
+    ms, _ = timed(lambda: v2p(vs, vp, vi), n=5, warm=1)
+    n = vp.shape[0]
+    report("Voxel2Point module (%d pts, %d voxels, C=%d)" % (n, M, C), ms,
+           4 * C * 4 * n + 16 * (n + M) + 24 * n, "3-NN search: n*M/B distance tests")
+    print("\n".join(rows), file=sys.stderr)
 
 
 def main():
@@ -193,6 +281,9 @@ def main():
         print("breakdown ms: rulebook %.3f (%.1f GB/s algorithmic) | kernel synthesis %.3f | "
               "conv call %.3f (MFMA kernel %.3f)" %
               (t_rb, rb_bytes / t_rb / 1e6, t_ks, t_cv, conv_kernel_ms), file=sys.stderr)
+
+    if args.ops:
+        ops_table(torch, _ext, synth, dev, args.seed)
 
     if not args.no_cpu_baseline:
         w = conv.kernel().permute(2, 3, 4, 1, 0).reshape(K, c_in, c_out).cpu().numpy()

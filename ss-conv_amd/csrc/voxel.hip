@@ -88,7 +88,11 @@ __global__ void __launch_bounds__(256)
   out[idx] = acc;
 }
 
-// Brute-force 3-NN: one thread per query, known rows streamed through LDS.
+// Brute-force 3-NN: one thread per query, known rows streamed through LDS in tiles.
+// A known row only counts for queries of the same batch element, so a tile none of
+// whose rows falls into the batch range of the block's queries is skipped after its
+// load; with rows grouped by batch element (the usual case) a block then scans its
+// own element's rows only.  The scan order, and with it the tie rule, is unchanged.
 constexpr int kNnTile = 256;
 
 __global__ void __launch_bounds__(kNnTile)
@@ -96,16 +100,39 @@ __global__ void __launch_bounds__(kNnTile)
                     const float *__restrict__ known, float *__restrict__ dist2,
                     int32_t *__restrict__ idx) {
   __shared__ float4v tile[kNnTile];
+  __shared__ float red[2][kNnTile / 64];
   int q = blockIdx.x * blockDim.x + threadIdx.x;
   float4v u = {0.f, 0.f, 0.f, 0.f};
   if (q < n) u = reinterpret_cast<const float4v *>(unknown)[q];
+  // batch range of the block's queries
+  float lo = q < n ? u.x : INFINITY, hi = q < n ? u.x : -INFINITY;
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) {
+    lo = fminf(lo, __shfl_xor(lo, d, 64));
+    hi = fmaxf(hi, __shfl_xor(hi, d, 64));
+  }
+  if ((threadIdx.x & 63) == 0) {
+    red[0][threadIdx.x >> 6] = lo;
+    red[1][threadIdx.x >> 6] = hi;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int w = 0; w < kNnTile / 64; ++w) {
+    lo = fminf(lo, red[0][w]);
+    hi = fmaxf(hi, red[1][w]);
+  }
   float b1 = INFINITY, b2 = INFINITY, b3 = INFINITY;
   int i1 = 0, i2 = 0, i3 = 0;
   for (int base = 0; base < m; base += kNnTile) {
     int kk = base + threadIdx.x;
     __syncthreads();
-    if (kk < m) tile[threadIdx.x] = reinterpret_cast<const float4v *>(known)[kk];
-    __syncthreads();
+    bool hit = false;
+    if (kk < m) {
+      float4v p = reinterpret_cast<const float4v *>(known)[kk];
+      tile[threadIdx.x] = p;
+      hit = p.x >= lo && p.x <= hi;
+    }
+    if (!__syncthreads_or(hit)) continue;
     int cnt = min(kNnTile, m - base);
     for (int t = 0; t < cnt; ++t) {
       float4v p = tile[t];
