@@ -193,22 +193,13 @@ __global__ void __launch_bounds__(256)
                       int32_t *__restrict__ tile_row0, int32_t *__restrict__ n_tiles_dev) {
   __shared__ int row_s[257];
   __shared__ int tile_s[257];
-  // the searches below are chains of dependent reads: do them in LDS when the fine
-  // grid fits (it does up to ~790 k output rows), else in global memory
-  constexpr int kFineLds = 12288;
-  __shared__ int fine_s[kFineLds];
-  const bool in_lds = nb + 1 <= kFineLds;
-  if (in_lds)
-    for (int64_t b = threadIdx.x; b <= nb; b += blockDim.x) fine_s[b] = fine_work[b];
-  __syncthreads();
   // cost of a tile beyond its pairs, in pair slots: half a row block of padding per
   // offset, and about two stages' worth of time for writing it out
   const int64_t tile_cost = (int64_t)K * 8 + 128;
   auto work = [&](int64_t b) -> int64_t {
     int64_t r = b * kSplitGranule;
     if (r > n_out) r = n_out;
-    const int pairs_below = in_lds ? fine_s[b] : fine_work[b];
-    return (int64_t)pairs_below * T + r * tile_cost;  // scaled by T to stay in integers
+    return (int64_t)fine_work[b] * T + r * tile_cost;  // scaled by T to stay in integers
   };
   for (int w = threadIdx.x; w <= n_wg; w += blockDim.x) {  // n_wg <= 256
     const int64_t total = work(nb);

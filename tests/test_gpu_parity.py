@@ -115,6 +115,10 @@ CONV_CASES = [
     (100, 8, 3, 1, 1, 5, 7),
     (100, 8, 2, 2, 0, 16, 20),
     (900, 12, 3, 1, 1, 64, 64),
+    # many tiles per workgroup range, several tiles per range boundary, 2 column blocks
+    (6000, 24, 3, 1, 1, 64, 80),
+    # two channel chunks on the buffer-load gather path, 3 column blocks
+    (1500, 16, 3, 1, 1, 128, 136),
 ]
 
 
@@ -314,6 +318,24 @@ def test_voxel2point_matches_oracle(oracle, device):
     assert np.array_equal(dist.cpu().numpy(), odist)
     c2, f2, b2 = Voxel2Point(voxel_extent=[2.0] * 3)(st)
     assert c2.shape == (st.indices.shape[0], 3) and f2 is st.features
+
+
+def test_three_nn_unsorted_and_many_tiles(oracle, device):
+    """Known rows in arbitrary order (batch elements interleaved) and more than one
+    tile of 256 rows per batch element: the tile skipping must not change a result."""
+    from ss_conv.sp_ops.functional import three_nn
+    rng = np.random.default_rng(21)
+    m, n, nb = 3000, 700, 5
+    known = np.concatenate([rng.integers(0, nb, size=(m, 1)).astype(np.float32),
+                            rng.integers(0, 12, size=(m, 3)).astype(np.float32) * 0.25], 1)
+    unknown = np.concatenate([rng.integers(0, nb + 1, size=(n, 1)).astype(np.float32),
+                              rng.uniform(0, 3, size=(n, 3)).astype(np.float32)], 1)
+    for kn in (known, known[np.argsort(known[:, 0], kind="stable")]):
+        dist, idx = three_nn(torch.from_numpy(unknown).to(device).contiguous(),
+                             torch.from_numpy(np.ascontiguousarray(kn)).to(device))
+        odist, oidx = oracle.three_nn(unknown, np.ascontiguousarray(kn))
+        assert np.array_equal(idx.cpu().numpy(), oidx)
+        assert np.array_equal(dist.cpu().numpy(), odist)
 
 
 def test_kernel_combine_matches_einsum(oracle, device):
