@@ -1,16 +1,20 @@
 // Sparse convolution forward as an output-stationary implicit GEMM on fp32 MFMA.
 //
-// Outputs are cut into tiles of at most T consecutive rows.  A workgroup owns one tile
-// and CN output columns; its accumulators [T, CN] live in LDS for the whole
-// kernel.  For every kernel offset k the pairs that land in the tile form one
-// contiguous segment of the rulebook (pairs of an offset are ascending in
+// Outputs are cut into tiles of at most T consecutive rows.  A workgroup owns one
+// tile and 64 output columns at a time; the tile's accumulators live in LDS until
+// the tile is complete.  For every kernel offset k the pairs that land in the tile
+// form one contiguous segment of the rulebook (pairs of an offset are ascending in
 // output row), so they are packed 16 at a time into the M side of
-// v_mfma_f32_16x16x4_f32: the gathered input rows are staged in LDS, the
-// matching 16x16 weight fragments stay in registers, and the product is added
-// to the LDS accumulators at the pairs' output rows.  Only occupied
-// (row, offset) slots cost MFMA work, and because each wave owns a fixed set
-// of columns and walks the offsets in ascending order the result is
-// bit-reproducible without atomics.
+// v_mfma_f32_16x16x4_f32: the gathered input rows are staged in LDS, the matching
+// 16x16 weight fragments are held in registers, and the product is added to the
+// LDS accumulators at the pairs' output rows.  Only occupied (row, offset) slots
+// cost MFMA work, and because each wave owns a fixed set of columns and walks the
+// offsets in ascending order the result is bit-reproducible without atomics.
+//
+// Host side of a call: pack the filters into MFMA fragment order; check that the
+// pairs are sorted (re-order them if not); split the output rows over the
+// workgroups by work and cut the ranges into tiles; build the row-block schedule;
+// launch the persistent kernel.
 #include "ssc_common.h"
 
 #include <type_traits>
@@ -392,7 +396,7 @@ __global__ void __launch_bounds__(256)
 // Dynamic LDS: acc[T+1][16*NCW+4] | abuf[2][64][68]
 constexpr int kRowsAhead = 4;  // stages whose gathered rows are in flight in registers
 constexpr int kIdxAhead = 2;   // further stages whose gather offsets are in flight
-constexpr unsigned kGatherPad = 0xFFFFF000u;  // gather offset of a padding slot (FAST)
+constexpr unsigned kGatherPad = 0xFFFFF000u;  // byte offset that gathers zeros (beyond any feature buffer)
 constexpr int kRsrcFlags = 0x00020000;        // raw buffer of 32-bit data
 
 __device__ __forceinline__ void mfma_quad(const float4v &b, const float4v &a, float4v &d) {
@@ -422,14 +426,18 @@ struct StagePos {
   }
 };
 
-// FAST: Cin is a multiple of 64 and the features are smaller than 4 GiB; the
-// schedule then holds byte offsets of the gather rows and the gather is a
-// range-checked buffer load.  Otherwise the schedule holds row numbers and the
-// gather uses 64-bit addresses with per-channel masks.
+// GATHER selects how the producers read the input rows:
+//   1  Cin is a multiple of 64 and the features are smaller than 4 GiB: the schedule
+//      holds byte offsets of the gather rows and the gather is a range-checked
+//      buffer load;
+//   2  the same with Cin a multiple of 4 only: in the last channel chunk the lanes
+//      beyond Cin gather from the padding offset, i.e. zeros;
+//   0  anything else: the schedule holds row numbers and the gather uses 64-bit
+//      addresses with per-channel masks.
 //
 // The waves-per-SIMD attribute states the occupancy the workgroup size gives anyway
 // (one workgroup per CU), so that the compiler uses the whole register budget.
-template <bool FAST, int NCW>
+template <int GATHER, int NCW>
 __global__ void __launch_bounds__((NCW + 4) * 64)
     __attribute__((amdgpu_waves_per_eu((NCW + 4) / 4, (NCW + 4) / 4)))
     conv_fwd_kernel(const float *__restrict__ features, int cin, unsigned feat_bytes,
@@ -437,8 +445,8 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
                     const int32_t *__restrict__ sched_in, const int32_t *__restrict__ sched_out,
                     const int32_t *__restrict__ grp_meta, unsigned sched_bytes, unsigned meta_bytes,
                     const int32_t *__restrict__ tile_grp, const int32_t *__restrict__ wg_tile,
-                    const int32_t *__restrict__ tile_row0, int nch, int ncb, int kvol, float *__restrict__ out, int64_t n_out, int cout,
-                    int T) {
+                    const int32_t *__restrict__ tile_row0, int nch, int ncb, int kvol,
+                    float *__restrict__ out, int cout, int T) {
   constexpr int kCN = 16 * NCW;   // output columns per workgroup
   constexpr int kAS = kCN + 4;    // accumulator row stride in floats
   constexpr int NT = (NCW + 4) * 64;
@@ -516,6 +524,8 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
         __builtin_amdgcn_make_buffer_rsrc((void *)features, 0, (int)feat_bytes, kRsrcFlags);
     const int idx_voff = (pt >> 4) * 4;    // this thread's slot (plus 16 slots per element)
     const int chunk_off = (pt & 15) * 16;  // this thread's 16 bytes of a 256-byte row chunk
+    // this thread's 4 channels of the last chunk lie beyond Cin
+    const bool beyond_cin = (nch - 1) * kKC + (pt & 15) * 4 >= cin;
     int idx[ID][NE];
     float4v rows[RD][NE];
     // Rings indexed by stage number: rows of stage st in rows[st & 3], gather offsets
@@ -527,15 +537,18 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
 #pragma unroll
       for (int j = 0; j < NE; ++j) {
         int v = buf_load1(rs_in, idx_voff + j * 64, pos.g * 256);
-        if (!FAST) v = s < nstages ? v : -1;  // the pointer gather is not range-checked
+        if (GATHER == 0) v = s < nstages ? v : -1;  // the pointer gather is not range-checked
         ix[j] = v;
       }
     };
     auto load_rows = [&](const StagePos &pos, const int (&ix)[NE], float4v (&r)[NE]) {
 #pragma unroll
       for (int j = 0; j < NE; ++j) {
-        if (FAST) {
+        if (GATHER == 1) {
           r[j] = buf_load4(rs_feat, ix[j] + chunk_off, pos.cc * 256);
+        } else if (GATHER == 2) {
+          const int off = (pos.cc == nch - 1 && beyond_cin) ? (int)kGatherPad : ix[j];
+          r[j] = buf_load4(rs_feat, off + chunk_off, pos.cc * 256);
         } else {
           const int ch = pos.cc * kKC + (pt & 15) * 4;
           const int row = ix[j] < 0 ? 0 : ix[j];  // padding slots read row 0 and drop it
@@ -812,7 +825,7 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
 
 struct ConvPlan {
   int ncb, nch, T, ncw, n_wg, n_colblk;
-  bool fast;
+  int gather;  // conv_fwd_kernel's GATHER
   int64_t n_tiles, n_fine, words_per_k, grp_cap;  // n_tiles: upper bound
   size_t lds_bytes;
 };
@@ -849,9 +862,11 @@ static ConvPlan make_plan(int64_t n_in, int64_t n_out, int K, int c_in, int c_ou
   p.nch = (int)ceil_div(c_in, kKC);
   p.ncw = 4;
   p.T = pick_tile(p.ncw);
-  // the gather can be a range-checked buffer load when every 64-channel chunk is
-  // complete and byte offsets into the features (plus the padding marker) fit 32 bits
-  p.fast = (c_in % kKC) == 0 && (uint64_t)n_in * c_in * 4 <= (uint64_t)kGatherPad;
+  // the gather can be a range-checked buffer load when rows are multiples of 16 bytes
+  // and byte offsets into the features (plus the padding marker) fit 32 bits
+  p.gather = 0;
+  if ((c_in & 3) == 0 && (uint64_t)n_in * c_in * 4 <= (uint64_t)kGatherPad)
+    p.gather = (c_in % kKC) == 0 ? 1 : 2;
   p.n_colblk = (int)ceil_div(p.ncb, p.ncw);
   int n_wg = device_cu_count() / p.n_colblk;
   if (n_wg < 1) n_wg = 1;
@@ -914,12 +929,12 @@ static size_t conv_ws_bytes(int64_t n_out, int K, int c_in, int c_out, int64_t p
   return conv_ws_walk(nullptr, p, K, pair_stride, nullptr);
 }
 
-template <bool FAST, int NCW>
+template <int GATHER, int NCW>
 static int launch_conv(const ConvPlan &p, const ConvWs &w, const float *features, int64_t n_in,
-                       int c_in, int K, float *out, int64_t n_out, int c_out, hipStream_t s) {
+                       int c_in, int K, float *out, int c_out, hipStream_t s) {
   static bool attr_set = false;
   if (!attr_set) {
-    SSC_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(conv_fwd_kernel<FAST, NCW>),
+    SSC_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(conv_fwd_kernel<GATHER, NCW>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
     attr_set = true;
   }
@@ -928,12 +943,12 @@ static int launch_conv(const ConvPlan &p, const ConvWs &w, const float *features
   SSC_CHECK(packed_bytes < ((uint64_t)1 << 32) && sched_bytes < ((uint64_t)1 << 32), SSC_ERUNTIME,
             "convolution too large for 32-bit buffer offsets (filters %llu B, schedule %llu B)",
             (unsigned long long)packed_bytes, (unsigned long long)sched_bytes);
-  const unsigned feat_bytes = FAST ? (unsigned)((uint64_t)n_in * c_in * 4) : 0u;
+  const unsigned feat_bytes = GATHER != 0 ? (unsigned)((uint64_t)n_in * c_in * 4) : 0u;
   dim3 grid((unsigned)p.n_wg, (unsigned)p.n_colblk);
-  hipLaunchKernelGGL((conv_fwd_kernel<FAST, NCW>), grid, dim3((NCW + 4) * 64), p.lds_bytes, s, features, c_in,
+  hipLaunchKernelGGL((conv_fwd_kernel<GATHER, NCW>), grid, dim3((NCW + 4) * 64), p.lds_bytes, s, features, c_in,
                      feat_bytes, w.packed, (unsigned)packed_bytes, w.sched_in, w.sched_out,
                      w.grp_meta, (unsigned)sched_bytes, (unsigned)(p.grp_cap * 32), w.tile_grp,
-                     w.wg_tile, w.tile_row0, p.nch, p.ncb, K, out, n_out, c_out, p.T);
+                     w.wg_tile, w.tile_row0, p.nch, p.ncb, K, out, c_out, p.T);
   SSC_LAUNCH_CHECK("conv_fwd");
   return SSC_OK;
 }
@@ -1059,15 +1074,19 @@ int ssc_conv_fwd_f32(const float *features, int64_t n_in, int32_t c_in, const fl
   hipLaunchKernelGGL(sched_fill_kernel, dim3((unsigned)ceil_div(p.n_tiles * K * 16, 256)),
                      dim3(256), 0, s, w.flag, pairs, w.sorted, pair_stride, plane_g, w.segs,
                      w.kofs, w.tile_nmb, w.tile_grp, K, w.n_tiles_dev, w.tile_row0, p.T,
-                     p.fast ? (uint32_t)c_in * 4u : 1u, p.fast ? kGatherPad : 0xFFFFFFFFu,
+                     p.gather ? (uint32_t)c_in * 4u : 1u, p.gather ? kGatherPad : 0xFFFFFFFFu,
                      (16 * p.ncw + 4) * 4, w.sched_in, w.sched_out, w.grp_meta);
   SSC_LAUNCH_CHECK("schedule");
 
   const bool prof = g_profile_on;
   const int slot = g_profile_count % kProfileRing;
   if (prof) SSC_HIP(hipEventRecord(g_profile_ev[slot][0], s));
-  rc = p.fast ? launch_conv<true, 4>(p, w, features, n_in, c_in, K, out, n_out, c_out, s)
-              : launch_conv<false, 4>(p, w, features, n_in, c_in, K, out, n_out, c_out, s);
+  if (p.gather == 1)
+    rc = launch_conv<1, 4>(p, w, features, n_in, c_in, K, out, c_out, s);
+  else if (p.gather == 2)
+    rc = launch_conv<2, 4>(p, w, features, n_in, c_in, K, out, c_out, s);
+  else
+    rc = launch_conv<0, 4>(p, w, features, n_in, c_in, K, out, c_out, s);
   if (rc != SSC_OK) return rc;
   if (prof) {
     SSC_HIP(hipEventRecord(g_profile_ev[slot][1], s));
