@@ -99,14 +99,25 @@ __global__ void __launch_bounds__(kSegRows * 64)
   float v = IS_MAX ? -INFINITY : 0.f;
   int arg = -1;
   if (c < C) {
-    for (int i = a + rl; i < b; i += kSegRows) {
-      float x = feats[(int64_t)i * C + c];
+    auto take = [&](float x, int i) {
       if (IS_MAX) {
         if (x > v) { v = x; arg = i; }
       } else {
         v += x;
       }
+    };
+    // eight rows per trip: the loads are independent and in flight together, the
+    // rows are then folded in ascending order, as a one-row-per-trip loop would
+    constexpr int U = 8;
+    int i = a + rl;
+    for (; i + (U - 1) * kSegRows < b; i += U * kSegRows) {
+      float x[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) x[u] = feats[(int64_t)(i + u * kSegRows) * C + c];
+#pragma unroll
+      for (int u = 0; u < U; ++u) take(x[u], i + u * kSegRows);
     }
+    for (; i < b; i += kSegRows) take(feats[(int64_t)i * C + c], i);
   }
   sval[rl][cl] = v;
   sidx[rl][cl] = arg;
