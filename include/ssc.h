@@ -219,6 +219,33 @@ int ssc_unique_emit(const int32_t *coords, int64_t n, const int32_t dims[4], voi
                     int32_t *inverse /* [n] */, int32_t *counts /* [m]; may be NULL */,
                     ssc_stream_t stream);
 
+/* Point filter and batch partition of Point2Voxel.forward
+ * (ss_conv/sp_ops/voxelize.py:40-83: drop the points outside the grid, give every batch
+ * element left without points one zero point, order by batch id), for batch ids that
+ * are non-decreasing and lie in [0, SSC_P2V_MAX_IDS): a stream compaction instead of
+ * torch.unique / boolean indexing / torch.sort.
+ * ssc_p2v_scan marks the surviving points and counts them per id; it SYNCHRONISES
+ *   `stream` and fills three host arrays: hist_all[id] = points with that id,
+ *   hist_valid[id] = survivors with that id, flags = {an id is out of range, ids
+ *   decrease somewhere}.  With a flag set the caller must take another path.
+ * ssc_p2v_compact (same workspace, untouched in between) writes the m = sum(hist_valid)
+ *   + #{id: hist_all > 0, hist_valid == 0} rows of the result: points [m,3], features
+ *   [m,channels], ids [m], and the voxel coordinates (b, vx, vy, vz) of every row as
+ *   ssc_voxel_coords computes them. */
+#define SSC_P2V_MAX_IDS 4096
+size_t ssc_p2v_workspace_bytes(int64_t n);
+int ssc_p2v_scan(const float *points /* [n,3] */, const int64_t *batch_ids /* [n] */, int64_t n,
+                 const float half_extent[3], void *workspace, size_t workspace_bytes,
+                 int32_t *hist_all_host /* [SSC_P2V_MAX_IDS] */,
+                 int32_t *hist_valid_host /* [SSC_P2V_MAX_IDS] */, int32_t *flags_host /* [2] */,
+                 ssc_stream_t stream);
+int ssc_p2v_compact(const float *points, const float *feats /* [n,channels] */,
+                    const int64_t *batch_ids, int64_t n, int32_t channels,
+                    const float half_extent[3], const float unit[3], void *workspace,
+                    size_t workspace_bytes, float *out_points /* [m,3] */,
+                    float *out_feats /* [m,channels] */, int64_t *out_ids /* [m] */,
+                    int32_t *out_coords /* [m,4] */, ssc_stream_t stream);
+
 int ssc_voxel_map(const int32_t *inverse /* [n] */, const int32_t *ids /* [n] */,
                   int32_t *out_maps /* [m,max_active+1] */, int32_t n_point, int32_t n_voxel,
                   int32_t max_active, int32_t mode, ssc_stream_t stream);

@@ -247,3 +247,231 @@ int ssc_three_interp_f32(int32_t c, int32_t m, int32_t n, const float *feats, co
   return SSC_OK;
 }
 }
+
+// ---- point filter and batch partition of Point2Voxel -------------------------------------
+// The reference's forward (ss_conv/sp_ops/voxelize.py:40-83) drops the points outside
+// the grid, gives every batch element left without points one zero point, and orders
+// the survivors by batch id (stable).  For batch ids that are already non-decreasing
+// and small non-negative integers -- clouds concatenated one after the other -- that is a
+// stream compaction plus a shift per batch element: no sort, no unique.
+namespace ssc {
+
+// Pass 1: one wave per 64 points.  inside bit per point (a ballot: no atomics),
+// histograms of all ids and of the surviving ids (one atomic per distinct id and
+// wave), flags[0] |= 1 for an id outside [0, SSC_P2V_MAX_IDS), flags[1] |= 1 when ids decrease.
+__global__ void __launch_bounds__(256)
+    p2v_scan_kernel(const float *__restrict__ pts, const int64_t *__restrict__ ids, int64_t n,
+                    float hx, float hy, float hz, uint32_t *__restrict__ bits,
+                    int32_t *__restrict__ hist_all, int32_t *__restrict__ hist_valid,
+                    int32_t *__restrict__ flags) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int lane = threadIdx.x & 63;
+  const bool live = i < n;
+  bool inside = false;
+  int64_t id = -1;
+  if (live) {
+    const float x = pts[i * 3], y = pts[i * 3 + 1], z = pts[i * 3 + 2];
+    inside = !(fabsf(x) > hx) && !(fabsf(y) > hy) && !(fabsf(z) > hz);
+    id = ids[i];
+    if (id < 0 || id >= SSC_P2V_MAX_IDS) atomicOr(&flags[0], 1);
+    if (i > 0 && ids[i - 1] > id) atomicOr(&flags[1], 1);
+  }
+  const unsigned long long in_mask = __ballot(inside);
+  if (live && (lane & 31) == 0) bits[i >> 5] = (uint32_t)(in_mask >> (lane & 32));
+  const bool ok_id = live && id >= 0 && id < SSC_P2V_MAX_IDS;
+  unsigned long long todo = __ballot(ok_id);
+  while (todo) {  // one trip per distinct id of the wave
+    const int first = __ffsll((long long)todo) - 1;
+    const int v = __shfl((int)id, first, 64);
+    const unsigned long long same = __ballot(ok_id && (int)id == v);
+    if (lane == first) {
+      atomicAdd(&hist_all[v], __popcll(same));
+      const int nv = __popcll(same & in_mask);
+      if (nv) atomicAdd(&hist_valid[v], nv);
+    }
+    todo &= ~same;
+  }
+}
+
+// One block: start[e] = survivors with an id below e; shift[e] = ids below e that are
+// present but have no survivor (each of them receives one zero point).
+__global__ void __launch_bounds__(256)
+    p2v_prefix_kernel(const int32_t *__restrict__ hist_all, const int32_t *__restrict__ hist_valid,
+                      int32_t *__restrict__ start, int32_t *__restrict__ shift) {
+  constexpr int PER = SSC_P2V_MAX_IDS / 256;
+  __shared__ int s_valid[256], s_empty[256];
+  const int t = threadIdx.x;
+  int sv = 0, se = 0;
+  for (int j = 0; j < PER; ++j) {
+    const int e = t * PER + j;
+    sv += hist_valid[e];
+    se += (hist_all[e] > 0 && hist_valid[e] == 0) ? 1 : 0;
+  }
+  s_valid[t] = sv;
+  s_empty[t] = se;
+  __syncthreads();
+  int bv = 0, be = 0;
+  for (int u = 0; u < t; ++u) {
+    bv += s_valid[u];
+    be += s_empty[u];
+  }
+  for (int j = 0; j < PER; ++j) {
+    const int e = t * PER + j;
+    start[e] = bv;
+    shift[e] = be;
+    bv += hist_valid[e];
+    be += (hist_all[e] > 0 && hist_valid[e] == 0) ? 1 : 0;
+  }
+}
+
+// Pass 2a: surviving point i goes to row rank(i) + shift[id]; threads n..n+MAX_IDS-1
+// write the zero point of an id without survivors.  Also writes the voxel coordinates
+// ((int)((p + half) / unit) in fp32, as voxel_coords_kernel does).
+__global__ void __launch_bounds__(256)
+    p2v_compact_kernel(const float *__restrict__ pts, const int64_t *__restrict__ ids, int64_t n,
+                       const uint32_t *__restrict__ bits, const int32_t *__restrict__ prefix,
+                       const int32_t *__restrict__ hist_all,
+                       const int32_t *__restrict__ hist_valid, const int32_t *__restrict__ start,
+                       const int32_t *__restrict__ shift, float hx, float hy, float hz, float ux,
+                       float uy, float uz, float *__restrict__ out_pts,
+                       int64_t *__restrict__ out_ids, int32_t *__restrict__ coords,
+                       int32_t *__restrict__ dest) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  float x = 0.f, y = 0.f, z = 0.f;
+  int64_t id;
+  int pos;
+  if (i < n) {
+    const bool inside = (bits[i >> 5] >> (i & 31)) & 1u;
+    id = ids[i];
+    pos = inside ? bit_rank(bits, prefix, (uint32_t)i) + shift[id] : -1;
+    dest[i] = pos;
+    if (!inside) return;
+    x = pts[i * 3];
+    y = pts[i * 3 + 1];
+    z = pts[i * 3 + 2];
+  } else {
+    id = i - n;
+    if (id >= SSC_P2V_MAX_IDS || hist_all[id] == 0 || hist_valid[id] != 0) return;
+    pos = start[id] + shift[id];
+  }
+  out_pts[(int64_t)pos * 3] = x;
+  out_pts[(int64_t)pos * 3 + 1] = y;
+  out_pts[(int64_t)pos * 3 + 2] = z;
+  out_ids[pos] = id;
+  const int vx = (int)((x + hx) / ux);
+  const int vy = (int)((y + hy) / uy);
+  const int vz = (int)((z + hz) / uz);
+  reinterpret_cast<int4 *>(coords)[pos] = make_int4((int)id, vx, vy, vz);
+}
+
+// Pass 2b: feature rows follow their points (dest[i] from pass 2a, -1 = dropped);
+// rows n..n+MAX_IDS-1 stand for the zero points.
+__global__ void __launch_bounds__(256)
+    p2v_feats_kernel(const float *__restrict__ feats, int64_t n, int C,
+                     const int32_t *__restrict__ dest, const int32_t *__restrict__ hist_all,
+                     const int32_t *__restrict__ hist_valid, const int32_t *__restrict__ start,
+                     const int32_t *__restrict__ shift, float *__restrict__ out) {
+  const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t i = e / C;
+  const int c = (int)(e - i * C);
+  if (i < n) {
+    const int pos = dest[i];
+    if (pos >= 0) out[(int64_t)pos * C + c] = feats[e];
+  } else {
+    const int64_t id = i - n;
+    if (id >= SSC_P2V_MAX_IDS || hist_all[id] == 0 || hist_valid[id] != 0) return;
+    out[(int64_t)(start[id] + shift[id]) * C + c] = 0.f;
+  }
+}
+
+struct P2vWs {
+  BitTable table;
+  int32_t *hist_all, *hist_valid, *flags, *start, *shift, *dest;
+};
+
+static size_t p2v_ws_walk(void *base, int64_t n, P2vWs *w) {
+  Carver c(base);
+  P2vWs t;
+  t.table = bit_table_carve(c, n > 0 ? n : 1);
+  t.hist_all = c.take<int32_t>(SSC_P2V_MAX_IDS);
+  t.hist_valid = c.take<int32_t>(SSC_P2V_MAX_IDS);  // directly behind hist_all
+  t.flags = c.take<int32_t>(2);
+  t.start = c.take<int32_t>(SSC_P2V_MAX_IDS);
+  t.shift = c.take<int32_t>(SSC_P2V_MAX_IDS);
+  t.dest = c.take<int32_t>(n > 0 ? n : 1);
+  if (w) *w = t;
+  return c.used;
+}
+
+}  // namespace ssc
+
+extern "C" {
+
+size_t ssc_p2v_workspace_bytes(int64_t n) {
+  if (n < 0) return 0;
+  // the carve sizes do not depend on the base address
+  return ssc::p2v_ws_walk(nullptr, n, nullptr);
+}
+
+int ssc_p2v_scan(const float *points, const int64_t *batch_ids, int64_t n,
+                 const float half_extent[3], void *workspace, size_t workspace_bytes,
+                 int32_t *hist_all_host, int32_t *hist_valid_host, int32_t *flags_host,
+                 ssc_stream_t stream) {
+  SSC_CHECK(n > 0, SSC_EINVAL, "n must be positive");
+  SSC_CHECK(n < ((int64_t)1 << 31), SSC_EINVAL, "n must fit 31 bits");
+  SSC_CHECK(points && batch_ids && half_extent && workspace && hist_all_host && hist_valid_host &&
+                flags_host,
+            SSC_EINVAL, "NULL pointer argument");
+  SSC_CHECK(workspace_bytes >= ssc_p2v_workspace_bytes(n), SSC_EWORKSPACE,
+            "p2v workspace too small");
+  hipStream_t s = (hipStream_t)stream;
+  P2vWs w;
+  p2v_ws_walk(workspace, n, &w);
+  int rc;
+  // hist_all, hist_valid and flags are cleared with one fill (they are adjacent up to
+  // alignment padding, which the fill covers as well)
+  const int64_t clear_n = (w.flags + 2) - w.hist_all;
+  if ((rc = fill_i32(w.hist_all, clear_n, 0, s)) != SSC_OK) return rc;
+  hipLaunchKernelGGL(p2v_scan_kernel, dim3((unsigned)ceil_div(n, 256)), dim3(256), 0, s, points,
+                     batch_ids, n, half_extent[0], half_extent[1], half_extent[2], w.table.bits,
+                     w.hist_all, w.hist_valid, w.flags);
+  SSC_LAUNCH_CHECK("p2v_scan");
+  if ((rc = bit_table_scan(w.table, s)) != SSC_OK) return rc;
+  hipLaunchKernelGGL(p2v_prefix_kernel, dim3(1), dim3(256), 0, s, w.hist_all, w.hist_valid,
+                     w.start, w.shift);
+  SSC_LAUNCH_CHECK("p2v_prefix");
+  SSC_HIP(hipMemcpyAsync(hist_all_host, w.hist_all, SSC_P2V_MAX_IDS * sizeof(int32_t),
+                         hipMemcpyDeviceToHost, s));
+  SSC_HIP(hipMemcpyAsync(hist_valid_host, w.hist_valid, SSC_P2V_MAX_IDS * sizeof(int32_t),
+                         hipMemcpyDeviceToHost, s));
+  SSC_HIP(hipMemcpyAsync(flags_host, w.flags, 2 * sizeof(int32_t), hipMemcpyDeviceToHost, s));
+  SSC_HIP(hipStreamSynchronize(s));
+  return SSC_OK;
+}
+
+int ssc_p2v_compact(const float *points, const float *feats, const int64_t *batch_ids, int64_t n,
+                    int32_t channels, const float half_extent[3], const float unit[3],
+                    void *workspace, size_t workspace_bytes, float *out_points, float *out_feats,
+                    int64_t *out_ids, int32_t *out_coords, ssc_stream_t stream) {
+  SSC_CHECK(n > 0 && channels >= 1, SSC_EINVAL, "bad sizes");
+  SSC_CHECK(points && feats && batch_ids && half_extent && unit && workspace && out_points &&
+                out_feats && out_ids && out_coords,
+            SSC_EINVAL, "NULL pointer argument");
+  SSC_CHECK(workspace_bytes >= ssc_p2v_workspace_bytes(n), SSC_EWORKSPACE,
+            "p2v workspace too small");
+  hipStream_t s = (hipStream_t)stream;
+  P2vWs w;
+  p2v_ws_walk(workspace, n, &w);
+  const int64_t rows = n + SSC_P2V_MAX_IDS;
+  hipLaunchKernelGGL(p2v_compact_kernel, dim3((unsigned)ceil_div(rows, 256)), dim3(256), 0, s,
+                     points, batch_ids, n, w.table.bits, w.table.prefix, w.hist_all, w.hist_valid,
+                     w.start, w.shift, half_extent[0], half_extent[1], half_extent[2], unit[0],
+                     unit[1], unit[2], out_points, out_ids, out_coords, w.dest);
+  SSC_LAUNCH_CHECK("p2v_compact");
+  hipLaunchKernelGGL(p2v_feats_kernel, dim3((unsigned)ceil_div(rows * channels, 256)), dim3(256), 0,
+                     s, feats, n, (int)channels, w.dest, w.hist_all, w.hist_valid, w.start,
+                     w.shift, out_feats);
+  SSC_LAUNCH_CHECK("p2v_feats");
+  return SSC_OK;
+}
+}

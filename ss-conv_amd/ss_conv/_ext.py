@@ -58,6 +58,12 @@ _SIGNATURES = {
     "ssc_segment_max_f32": (ctypes.c_int, [_vp, _vp, _vp, _vp, _i32, _i32, _vp]),
     "ssc_voxel_coords": (ctypes.c_int, [_vp, _vp, _i64, ctypes.POINTER(ctypes.c_float),
                                         ctypes.POINTER(ctypes.c_float), _vp, _vp]),
+    "ssc_p2v_workspace_bytes": (_sz, [_i64]),
+    "ssc_p2v_scan": (ctypes.c_int, [_vp, _vp, _i64, ctypes.POINTER(ctypes.c_float), _vp, _sz,
+                                    _vp, _vp, _vp, _vp]),
+    "ssc_p2v_compact": (ctypes.c_int, [_vp, _vp, _vp, _i64, _i32, ctypes.POINTER(ctypes.c_float),
+                                       ctypes.POINTER(ctypes.c_float), _vp, _sz, _vp, _vp, _vp,
+                                       _vp, _vp]),
     "ssc_unique_workspace_bytes": (_sz, [ctypes.POINTER(_i32), _i64]),
     "ssc_unique_count": (ctypes.c_int, [_vp, _i64, ctypes.POINTER(_i32), _vp, _sz,
                                         ctypes.POINTER(_i32), _vp]),
@@ -348,6 +354,55 @@ def voxel_coords(points, batch_ids, half_extent, unit):
     u = (ctypes.c_float * 3)(*[float(v) for v in unit])
     _check(_lib.ssc_voxel_coords(_ptr(points), _ptr(ids), n, h, u, _ptr(coords), _stream(points)))
     return coords
+
+
+P2V_MAX_IDS = 4096
+
+
+def p2v_filter(points, feats, batch_ids, half_extent, unit):
+    """Filter + batch partition of Point2Voxel.forward (ss_conv/sp_ops/voxelize.py:40-83)
+    for float32 points/features and int64 batch ids that are non-decreasing and below
+    P2V_MAX_IDS.  Returns None when the inputs do not qualify (or no point survives);
+    otherwise (valid_points, valid_feats, valid_ids, voxel_coords, origin_ids, instance_flag)
+    with origin_ids / instance_flag as host lists."""
+    import numpy as np
+    if not (points.is_cuda and feats.is_cuda and batch_ids.is_cuda):
+        return None
+    if points.dtype != torch.float32 or feats.dtype != torch.float32 or \
+            batch_ids.dtype != torch.int64 or points.dim() != 2 or points.size(1) != 3:
+        return None
+    n = points.size(0)
+    if n == 0 or feats.size(0) != n or batch_ids.numel() != n:
+        return None
+    points, feats, batch_ids = points.contiguous(), feats.contiguous(), batch_ids.contiguous()
+    dev = points.device
+    ws = _workspace(_lib.ssc_p2v_workspace_bytes(n), dev)
+    h = (ctypes.c_float * 3)(*[float(v) for v in half_extent])
+    u = (ctypes.c_float * 3)(*[float(v) for v in unit])
+    hist_all = np.empty(P2V_MAX_IDS, dtype=np.int32)
+    hist_valid = np.empty(P2V_MAX_IDS, dtype=np.int32)
+    flags = np.empty(2, dtype=np.int32)
+    s = _stream(points)
+    _check(_lib.ssc_p2v_scan(_ptr(points), _ptr(batch_ids), n, h, ws.data_ptr(), ws.numel(),
+                             hist_all.ctypes.data, hist_valid.ctypes.data, flags.ctypes.data, s))
+    if flags[0] or flags[1]:
+        return None
+    present = hist_all > 0
+    alive = hist_valid > 0
+    n_valid = int(hist_valid.sum())
+    if n_valid == 0:
+        return None
+    origin_ids = np.nonzero(present)[0]
+    m = n_valid + int((present & ~alive).sum())
+    c = feats.size(1)
+    out_p = torch.empty((m, 3), dtype=torch.float32, device=dev)
+    out_f = torch.empty((m, c), dtype=torch.float32, device=dev)
+    out_i = torch.empty((m,), dtype=torch.int64, device=dev)
+    coords = torch.empty((m, 4), dtype=torch.int32, device=dev)
+    _check(_lib.ssc_p2v_compact(_ptr(points), _ptr(feats), _ptr(batch_ids), n, c, h, u,
+                                ws.data_ptr(), ws.numel(), _ptr(out_p), _ptr(out_f), _ptr(out_i),
+                                _ptr(coords), s))
+    return out_p, out_f, out_i, coords, origin_ids, alive[origin_ids].astype(np.float32)
 
 
 def unique_rows(coords, dims, return_counts=True):

@@ -36,14 +36,25 @@ class Point2Voxel(nn.Module):
         C = feature.size(1)
         device = point_cloud.device
 
-        unique_origin_ids = torch.unique(batch_ids)
-        B1 = unique_origin_ids.size(0)
-
         unit = self.unit_voxel_extent.numpy().astype(np.float32)
         limit = self.voxel_num_limit.astype(np.float32)
         half = np.float32(0.5) * (limit * unit)  # fp32 throughout, as on the device
-        half_t = torch.from_numpy(half).reshape(1, 3).to(device)
 
+        # Clouds concatenated in batch order with small non-negative ids: filter and
+        # partition in native kernels (one host read); anything else takes the
+        # reference's sequence of torch operations below.
+        fast = _ext.p2v_filter(point_cloud, feature, batch_ids, half, unit) \
+            if point_cloud.is_cuda else None
+        if fast is not None:
+            valid_point_cloud, valid_feature, valid_ids, voxel_index, origin_ids, alive = fast
+            B1 = len(origin_ids)
+            valid_instance_flag = torch.from_numpy(alive).to(device)
+            return self._voxelize(valid_point_cloud, valid_feature, valid_ids, voxel_index,
+                                  int(origin_ids[-1]), valid_instance_flag, B1)
+
+        half_t = torch.from_numpy(half).reshape(1, 3).to(device)
+        unique_origin_ids = torch.unique(batch_ids)
+        B1 = unique_origin_ids.size(0)
         inside = (torch.abs(point_cloud) > half_t).sum(1) == 0
         if inside.sum() == 0:
             valid_instance_flag = torch.zeros(B1, dtype=torch.float32, device=device)
@@ -78,8 +89,14 @@ class Point2Voxel(nn.Module):
         if lo < 0:
             raise ValueError("batch ids must be non-negative")
         voxel_index = _ext.voxel_coords(valid_point_cloud, valid_ids, half, unit)
+        return self._voxelize(valid_point_cloud, valid_feature, valid_ids, voxel_index, hi,
+                              valid_instance_flag, B1)
+
+    def _voxelize(self, valid_point_cloud, valid_feature, valid_ids, voxel_index, max_id,
+                  valid_instance_flag, B1):
+        """Unique voxels, per-voxel point lists and feature reduction (voxelize.py:85-99)."""
         # a point exactly on the upper face lands on index == limit, hence the +1
-        dims = [hi + 1] + [int(v) + 1 for v in self.voxel_num_limit]
+        dims = [max_id + 1] + [int(v) + 1 for v in self.voxel_num_limit]
         occupied_index, inverse, count = _ext.unique_rows(voxel_index, dims, return_counts=True)
         nActive = occupied_index.size(0)
         if self.voxelization_mode == 1 or self.voxelization_mode == 2:

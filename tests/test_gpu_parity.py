@@ -297,6 +297,27 @@ def test_point2voxel_empty_batch_element(oracle, device):
     assert np.array_equal(st.indices.cpu().numpy(), ref["indices"])
 
 
+def test_point2voxel_unsorted_ids_and_outliers(oracle, device):
+    """Points in arbitrary order (batch ids not sorted: the torch path) and in batch
+    order (the native filter) give the oracle's result; some points lie outside the grid."""
+    from ss_conv.sp_ops.voxelize import Point2Voxel
+    pts, feats, ids = synth.make_clouds(4, 300, seed=9, channels=6)
+    pts = pts * 1.2  # pushes part of every cloud outside [-1, 1]^3
+    grid = 8
+    rng = np.random.default_rng(3)
+    for perm in (np.arange(len(ids)), rng.permutation(len(ids))):
+        p, f, i = pts[perm], feats[perm], ids[perm]
+        ref = oracle.point2voxel(p, f, i, [grid] * 3, [2.0 / grid] * 3, 4)
+        vp, st, vi, flag = Point2Voxel([grid] * 3, [2.0 / grid] * 3)(
+            torch.from_numpy(p).to(device), torch.from_numpy(f).to(device),
+            torch.from_numpy(i).to(device))
+        assert np.array_equal(st.indices.cpu().numpy(), ref["indices"])
+        assert np.array_equal(vp.cpu().numpy(), ref["valid_points"])
+        assert np.array_equal(vi.cpu().numpy(), ref["valid_ids"])
+        assert np.array_equal(st.features.cpu().numpy(), ref["features"])
+        assert flag.cpu().tolist() == ref["flag"].tolist()
+
+
 def test_voxel2point_matches_oracle(oracle, device):
     from ss_conv.sp_ops.voxelize import Point2Voxel, Voxel2Point
     pts, feats, ids = synth.make_clouds(3, 500, seed=6, channels=10)
