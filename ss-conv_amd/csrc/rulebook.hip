@@ -83,7 +83,7 @@ __device__ __forceinline__ bool pair_key(const Geom &g, const int32_t *__restric
 // Regular conv: mark every output cell reachable from an active input, and count
 // the pairs of every 64-row chunk (chunk_count is [K, n_chunks]; for a regular
 // convolution a pair exists wherever the geometry allows it, so the counts do not
-// depend on the table).  One wave per chunk of 64 input rows, one lane per row.
+// depend on the table).  One wave per chunk of 64 input rows and x offset, one lane per row.
 // The taps of one (kx, ky) differ in z only, so their output cells are neighbours
 // in the key space: their bits are gathered into one mask per 32-bit word, the word
 // is read first, and the atomic is issued only when it would change the word
@@ -99,8 +99,10 @@ __global__ void __launch_bounds__(256)
   const bool live = i < n_in;
   int32_t row[4] = {0, 0, 0, 0};
   if (live) *reinterpret_cast<int4 *>(row) = reinterpret_cast<const int4 *>(indices)[i];
-  int k = 0;
-  for (int kx = 0; kx < g.ks[0]; ++kx) {
+  // blockIdx.y = kx: the taps of one x offset per wave, for more waves in flight
+  const int kx = blockIdx.y;
+  int k = kx * g.ks[1] * g.ks[2];
+  {
     int ox = 0;
     const bool okx = live && tap_to_out(row[1], kx, g.st[0], g.pd[0], g.dl[0], g.os[0], &ox);
     for (int ky = 0; ky < g.ks[1]; ++ky) {
@@ -270,8 +272,10 @@ __global__ void __launch_bounds__(256)
   // space, so the table word and its prefix are loaded once per word, not per tap.
   uint32_t word = 0xFFFFFFFFu, wbits = 0u;
   int wprefix = 0;
-  int k = 0;
-  for (int kx = 0; kx < g.ks[0]; ++kx) {
+  // blockIdx.y = kx: the taps of one x offset per wave, for more waves in flight
+  const int kx = blockIdx.y;
+  int k = kx * g.ks[1] * g.ks[2];
+  {
     int ox = 0;
     const bool okx = live && tap_to_out(row[1], kx, g.st[0], g.pd[0], g.dl[0], g.os[0], &ox);
     for (int ky = 0; ky < g.ks[1]; ++ky) {
@@ -382,7 +386,8 @@ int ssc_rulebook_count(const int32_t *indices, int64_t n_in, const ssc_geometry 
                        indices, n_in, gg.os[0], gg.os[1], gg.os[2], w.table.bits);
     SSC_LAUNCH_CHECK("mark_rows");
   } else {
-    hipLaunchKernelGGL(mark_count_kernel, dim3((unsigned)ceil_div(w.n_chunks, 4)), dim3(256), 0, s,
+    hipLaunchKernelGGL(mark_count_kernel,
+                       dim3((unsigned)ceil_div(w.n_chunks, 4), (unsigned)gg.ks[0]), dim3(256), 0, s,
                        indices, n_in, gg, w.table.bits, w.chunk_count, w.n_chunks);
     SSC_LAUNCH_CHECK("mark_count");
   }
@@ -428,7 +433,8 @@ int ssc_rulebook_emit(const int32_t *indices, int64_t n_in, const ssc_geometry *
   hipLaunchKernelGGL(scan_chunks_kernel, dim3(gg.K), dim3(kScanThreads), 0, s, w.chunk_count,
                      w.n_chunks, pair_num);
   SSC_LAUNCH_CHECK("scan_chunks");
-  hipLaunchKernelGGL(write_pairs_kernel, dim3(chunk_blocks), dim3(256), 0, s, indices, n_in, gg,
+  hipLaunchKernelGGL(write_pairs_kernel, dim3(chunk_blocks, (unsigned)gg.ks[0]), dim3(256), 0, s,
+                     indices, n_in, gg,
                      w.table.bits, w.table.prefix, w.rank2row, w.chunk_count, w.n_chunks, pair_num,
                      pairs);
   SSC_LAUNCH_CHECK("write_pairs");
