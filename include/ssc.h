@@ -114,6 +114,31 @@ int ssc_conv_fwd_f32(const float *features /* [n_in,c_in] */, int64_t n_in, int3
                      float *out /* [n_out,c_out] */, int64_t n_out, void *workspace,
                      size_t workspace_bytes, ssc_stream_t stream);
 
+/* ----------------------------------------------------------------------
+ * Gradients of the sparse convolution -- replaces indice_conv_backward_fp32
+ * (src/ss_conv_ops_api.cpp:22, src/conv/indice_conv.h:344-426).
+ *
+ * Input gradient: no entry point of its own.  It is ssc_conv_fwd_f32 applied to
+ * out_grad with `inverse` flipped, c_in and c_out exchanged and the filter strides
+ * fs_ci and fs_co exchanged (input_grad[i] = sum_k out_grad[o] * W[k]^T over the same
+ * pairs).
+ *
+ * ssc_conv_bwd_filter_f32: filters_grad[k][ci][co] = sum over the pairs (i, o) of
+ *   offset k of features[i][ci] * out_grad[o][co], written with the element strides
+ *   gs_k, gs_ci, gs_co (every element is written; no atomics; the summation order is
+ *   fixed, so two runs give identical bits).  `inverse` is the flag of the forward
+ *   call.
+ * ---------------------------------------------------------------------- */
+size_t ssc_conv_bwd_filter_workspace_bytes(int32_t kernel_volume, int32_t c_in, int32_t c_out,
+                                           int64_t pair_stride);
+int ssc_conv_bwd_filter_f32(const float *features /* [n_in,c_in] */, int64_t n_in, int32_t c_in,
+                            const float *out_grad /* [n_out,c_out] */, int64_t n_out,
+                            int32_t c_out, const int32_t *pairs /* [K,2,pair_stride] */,
+                            int64_t pair_stride, const int32_t *pair_num /* [K] */,
+                            int32_t kernel_volume, int32_t inverse, float *filters_grad,
+                            int64_t gs_k, int64_t gs_ci, int64_t gs_co, void *workspace,
+                            size_t workspace_bytes, ssc_stream_t stream);
+
 /* Timing of the convolution kernel alone (no counterpart in the reference, whose
  * timers are commented out, src/conv/indice_conv.h:295,319-341).  While enabled,
  * every ssc_conv_fwd_f32 call records a pair of HIP events on its stream right

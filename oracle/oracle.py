@@ -221,6 +221,30 @@ def conv_fwd(features, filters, pairs, num, n_out, inverse=False, matmul=None):
     return out
 
 
+def conv_bwd(features, filters, out_grad, pairs, num, inverse=False):
+    """src/conv/indice_conv.h:344-426, CPU branch: for every non-empty offset gather the
+    input rows and the output-gradient rows (:383-390), filters_grad[k] = in^T * out_grad
+    (torch::mm_out, :407), in_buffer = out_grad * W[k]^T (:408), scatter-add into the
+    input gradient (:409-413).  filters is [K, Cin, Cout]; products in float64, rounded
+    once (the order of a BLAS reduction is not part of the reference's contract).
+    Returns (input_grad [N_in, Cin], filters_grad [K, Cin, Cout])."""
+    features, filters, out_grad = _f32(features), _f32(filters), _f32(out_grad)
+    K, cin, cout = filters.shape
+    d_in = np.zeros(features.shape, dtype=np.float64)
+    d_w = np.zeros(filters.shape, dtype=np.float64)
+    for k in range(K):
+        n = int(num[k])
+        if n <= 0:
+            continue
+        rows_i = pairs[k, 1 if inverse else 0, :n]
+        rows_o = pairs[k, 0 if inverse else 1, :n]
+        fin = features[rows_i].astype(np.float64)
+        gout = out_grad[rows_o].astype(np.float64)
+        d_w[k] = fin.T @ gout
+        np.add.at(d_in, rows_i, gout @ filters[k].astype(np.float64).T)
+    return d_in.astype(np.float32), d_w.astype(np.float32)
+
+
 def ref_gather_scatter_conv(features, filters, pairs, num, n_out):
     """conv_fwd with the reference's own compiled gather / scatter functors and
     a NumPy GEMM in place of torch::mm."""

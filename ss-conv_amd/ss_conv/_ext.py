@@ -43,6 +43,9 @@ _SIGNATURES = {
     "ssc_conv_workspace_bytes": (_sz, [_i64, _i32, _i32, _i32, _i64]),
     "ssc_conv_fwd_f32": (ctypes.c_int, [_vp, _i64, _i32, _vp, _i64, _i64, _i64, _i32, _vp, _i64,
                                         _vp, _i32, _i32, _i32, _vp, _i64, _vp, _sz, _vp]),
+    "ssc_conv_bwd_filter_workspace_bytes": (_sz, [_i32, _i32, _i32, _i64]),
+    "ssc_conv_bwd_filter_f32": (ctypes.c_int, [_vp, _i64, _i32, _vp, _i64, _i32, _vp, _i64, _vp,
+                                               _i32, _i32, _vp, _i64, _i64, _i64, _vp, _sz, _vp]),
     "ssc_profile_conv": (ctypes.c_int, [_i32]),
     "ssc_profile_conv_read": (ctypes.c_int, [ctypes.POINTER(ctypes.c_float), _i32,
                                              ctypes.POINTER(_i32)]),
@@ -203,6 +206,41 @@ def indice_conv_fp32(features, filters, indice_pairs, indice_num, num_act_out, i
                                  K, int(inverse), int(subm), _ptr(out), n_out, ws.data_ptr(),
                                  ws.numel(), _stream(features)))
     return out
+
+
+def indice_conv_backward_fp32(features, filters, out_bp, indice_pairs, indice_num, inverse, subm):
+    """src/conv/indice_conv.h:344-426 (bound at src/ss_conv_ops_api.cpp:22): returns
+    [input_bp like features, filters_bp shaped like filters]."""
+    _need_gpu(features, filters, out_bp, indice_pairs)
+    if features.dtype != torch.float32 or filters.dtype != torch.float32 or \
+            out_bp.dtype != torch.float32:
+        raise RuntimeError("indice_conv_backward_fp32 needs float32 tensors")
+    features = features.contiguous()
+    out_bp = out_bp.contiguous()
+    n_in, c_in = features.shape
+    n_out, c_out = out_bp.shape
+    filters, fs_k, fs_ci, fs_co = _filter_strides(filters, c_in, c_out)
+    pairs = indice_pairs.int().contiguous() if indice_pairs.dtype != torch.int32 \
+        else indice_pairs.contiguous()
+    num = indice_num.to(device=features.device, dtype=torch.int32).contiguous()
+    K = pairs.size(0)
+    dev = features.device
+    s = _stream(features)
+    # input gradient: the forward kernel on out_bp, pairs swapped, filters transposed
+    input_bp = torch.empty((n_in, c_in), dtype=torch.float32, device=dev)
+    ws = _workspace(_lib.ssc_conv_workspace_bytes(n_in, K, c_out, c_in, pairs.size(2)), dev)
+    _check(_lib.ssc_conv_fwd_f32(_ptr(out_bp), n_out, c_out, _ptr(filters), fs_k, fs_co, fs_ci,
+                                 c_in, _ptr(pairs), pairs.size(2), num.data_ptr(), K,
+                                 0 if inverse else 1, int(subm), _ptr(input_bp), n_in,
+                                 ws.data_ptr(), ws.numel(), s))
+    # filter gradient
+    filters_bp = torch.empty(tuple(filters.shape), dtype=torch.float32, device=dev)
+    ws2 = _workspace(_lib.ssc_conv_bwd_filter_workspace_bytes(K, c_in, c_out, pairs.size(2)), dev)
+    _check(_lib.ssc_conv_bwd_filter_f32(_ptr(features), n_in, c_in, _ptr(out_bp), n_out, c_out,
+                                        _ptr(pairs), pairs.size(2), num.data_ptr(), K,
+                                        int(inverse), _ptr(filters_bp), c_in * c_out, c_out, 1,
+                                        ws2.data_ptr(), ws2.numel(), s))
+    return [input_bp, filters_bp]
 
 
 def _pool_args(features, indice_pairs, indice_num):

@@ -1,9 +1,10 @@
 """autograd entry points over the native kernels
 (reference: ss_conv/sp_ops/functional.py:22-453; same exported names).
 
-Forward passes run the HIP kernels.  Backward passes are not built yet: a
-Function whose backward is reached raises NotImplementedError instead of
-returning wrong gradients."""
+Forward passes run the HIP kernels, and so do the backward passes of the three
+convolution Functions.  The other backward passes are not built yet: a Function
+whose backward is reached raises NotImplementedError instead of returning wrong
+gradients."""
 import torch
 from torch.autograd import Function
 
@@ -25,6 +26,15 @@ class _ConvBase(Function):
         return ops.indice_conv_forward(features, filters, indice_pairs, indice_pair_num,
                                        num_activate_out, cls.inverse, cls.subm)
 
+    @classmethod
+    def _grad(cls, ctx, grad_output):
+        """(reference: functional.py:38-43, 60-65, 82-87)"""
+        indice_pairs, indice_pair_num, features, filters = ctx.saved_tensors
+        input_bp, filters_bp = ops.indice_conv_backward(
+            features, filters, grad_output.contiguous(), indice_pairs, indice_pair_num,
+            cls.inverse, cls.subm)
+        return input_bp, filters_bp, None, None, None
+
 
 class SparseConvFunction(_ConvBase):
     @staticmethod
@@ -34,7 +44,7 @@ class SparseConvFunction(_ConvBase):
 
     @staticmethod
     def backward(ctx, grad_output):
-        _no_backward("indice_conv")
+        return SparseConvFunction._grad(ctx, grad_output)
 
 
 class SparseInverseConvFunction(_ConvBase):
@@ -47,7 +57,7 @@ class SparseInverseConvFunction(_ConvBase):
 
     @staticmethod
     def backward(ctx, grad_output):
-        _no_backward("indice_inverse_conv")
+        return SparseInverseConvFunction._grad(ctx, grad_output)
 
 
 class SubMConvFunction(_ConvBase):
@@ -60,7 +70,7 @@ class SubMConvFunction(_ConvBase):
 
     @staticmethod
     def backward(ctx, grad_output):
-        _no_backward("indice_subm_conv")
+        return SubMConvFunction._grad(ctx, grad_output)
 
 
 class SparseMaxPoolFunction(Function):

@@ -72,7 +72,11 @@ def indice_conv_forward(features, filters, indice_pairs, indice_pair_num, num_ac
 
 def indice_conv_backward(features, filters, out_bp, indice_pairs, indice_pair_num, inverse=False,
                          subm=False):
-    raise NotImplementedError("the backward pass of the sparse convolution is not built yet")
+    """[input_bp, filters_bp] (reference: sp_ops/ops.py:116-150)."""
+    if filters.dtype == torch.float32:
+        return _ext.indice_conv_backward_fp32(features, filters, out_bp, indice_pairs,
+                                              indice_pair_num, int(inverse), int(subm))
+    raise NotImplementedError("only float32 convolution is built")
 
 
 def indice_maxpool_forward(features, indice_pairs, indice_pair_num, num_activate_out):

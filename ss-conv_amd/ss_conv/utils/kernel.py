@@ -122,6 +122,40 @@ def orthogonal_(tensor, gain=1):
 
 
 # ---- kernel module ----------------------------------------------------------------------
+class _Combine(torch.autograd.Function):
+    """dense[k, (j,v,b), (i,u,a)] = sum_n weight_ij[u,v,n] * basis_ij[n,a,b,k] in one native
+    launch; the gradient with respect to the weights is the same contraction against the
+    fixed basis, block by block (the blocks are small: torch einsum)."""
+
+    @staticmethod
+    def forward(ctx, weight, module):
+        basis, chan_out, chan_in, blocks, _ = module._tables
+        ctx.module = module
+        return _ext.kernel_combine(weight.detach().float().contiguous(), basis, chan_out, chan_in,
+                                   blocks, len(module.multiplicities_in), module.size ** 3,
+                                   module.n_in, module.n_out)
+
+    @staticmethod
+    def backward(ctx, grad):  # grad: [K, Cin, Cout]
+        m = ctx.module
+        K = m.size ** 3
+        grads = []
+        o_off = 0
+        for i, (mi, di) in enumerate(zip(m.multiplicities_out, m.dims_out)):
+            i_off = 0
+            for j, (mj, dj) in enumerate(zip(m.multiplicities_in, m.dims_in)):
+                kij = getattr(m, "kernel_{}_{}".format(i, j))
+                if kij is not None:
+                    nb = kij.size(0)
+                    g = grad[:, i_off:i_off + mj * dj, o_off:o_off + mi * di]
+                    g = g.reshape(K, mj, dj, mi, di)
+                    basis = kij.to(grad.dtype).reshape(nb, di, dj, K)
+                    grads.append(torch.einsum("kvbua,nabk->uvn", g, basis).reshape(-1))
+                i_off += mj * dj
+            o_off += mi * di
+        return torch.cat(grads), None
+
+
 class SE3Kernel(torch.nn.Module):
     """Dense steerable kernel [Cout, Cin, k, k, k] = sum_beta weight * basis.
 
@@ -209,17 +243,12 @@ class SE3Kernel(torch.nn.Module):
 
     def combination(self, weight):
         """[Cout, Cin, k, k, k] view of the natively contracted [K, Cin, Cout] kernel
-        (reference: kernel.py:267-299)."""
+        (reference: kernel.py:267-299).  Differentiable with respect to `weight`."""
         if not weight.is_cuda:
             raise RuntimeError("SE3Kernel runs on the GPU only: move the module to a cuda device")
-        if weight.requires_grad and torch.is_grad_enabled():
-            weight = weight.detach()  # forward-only build: no gradient flows to kernel.weight
         if self._tables is None or self._tables[4] != weight.device:
             self._build_tables(weight.device)
-        basis, chan_out, chan_in, blocks, _ = self._tables
-        dense = _ext.kernel_combine(weight.float().contiguous(), basis, chan_out, chan_in, blocks,
-                                    len(self.multiplicities_in), self.size ** 3, self.n_in,
-                                    self.n_out)
+        dense = _Combine.apply(weight, self)
         k = self.size
         return dense.permute(2, 1, 0).reshape(self.n_out, self.n_in, k, k, k)
 

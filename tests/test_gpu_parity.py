@@ -403,6 +403,108 @@ def test_convolution_layer_end_to_end(oracle, device):
     assert rel_l2(out.features.cpu().numpy(), ref) < REL_L2
 
 
+BWD_CASES = [
+    # n_vox, grid, k, s, p, cin, cout
+    (300, 10, 3, 1, 1, 32, 32),
+    (900, 12, 3, 1, 1, 64, 128),
+    (200, 10, 3, 2, 1, 128, 72),
+    (200, 8, 3, 1, 1, 3, 152),
+    (150, 8, 5, 1, 2, 40, 24),
+    (100, 8, 2, 2, 0, 5, 7),
+]
+
+
+@pytest.mark.parametrize("case", BWD_CASES)
+def test_conv_backward_matches_oracle(case, oracle, device):
+    """Input and filter gradients through the C ABI against the restated backward."""
+    from ss_conv import _ext
+    print("case", case, flush=True)
+    n, grid, k, s, p, cin, cout = case
+    rng = np.random.default_rng(41)
+    idx = random_voxels(rng, 2, grid, n)
+    feats = rng.normal(size=(n, cin)).astype(np.float32)
+    K = k ** 3
+    w = (rng.normal(size=(K, cin, cout)) / np.sqrt(K * cin)).astype(np.float32)
+    o_idx, o_pairs, o_num = oracle.canonicalize(*oracle.rulebook(idx, 2, [grid] * 3, k, s, p))
+    g_out = rng.normal(size=(o_idx.shape[0], cout)).astype(np.float32)
+    ref_in, ref_w = oracle.conv_bwd(feats, w, g_out, o_pairs, o_num)
+    g_idx, g_pairs, g_num = [torch.from_numpy(x).to(device) for x in
+                             gpu_rulebook(idx, 2, grid, k, s, p)]
+    wt = torch.from_numpy(w).to(device).reshape(k, k, k, cin, cout)
+    d_in, d_w = _ext.indice_conv_backward_fp32(
+        torch.from_numpy(feats).to(device), wt, torch.from_numpy(g_out).to(device), g_pairs,
+        g_num, 0, 0)
+    assert d_w.shape == wt.shape
+    assert rel_l2(d_in.cpu().numpy(), ref_in) < REL_L2
+    assert rel_l2(d_w.cpu().numpy().reshape(K, cin, cout), ref_w) < REL_L2
+    # twice the same bits
+    d_in2, d_w2 = _ext.indice_conv_backward_fp32(
+        torch.from_numpy(feats).to(device), wt, torch.from_numpy(g_out).to(device), g_pairs,
+        g_num, 0, 0)
+    assert torch.equal(d_w, d_w2) and torch.equal(d_in, d_in2)
+    # the inverse convolution's backward: roles of the two row planes exchanged
+    wi = torch.from_numpy(np.ascontiguousarray(np.transpose(w, (0, 2, 1)))).to(device) \
+        .reshape(k, k, k, cout, cin)
+    e_in, e_w = _ext.indice_conv_backward_fp32(
+        torch.from_numpy(g_out).to(device), wi, torch.from_numpy(feats).to(device), g_pairs,
+        g_num, 1, 0)
+    oref_in, oref_w = oracle.conv_bwd(g_out, np.transpose(w, (0, 2, 1)).copy(), feats, o_pairs,
+                                      o_num, inverse=True)
+    assert rel_l2(e_in.cpu().numpy(), oref_in) < REL_L2
+    assert rel_l2(e_w.cpu().numpy().reshape(K, cout, cin), oref_w) < REL_L2
+
+
+def test_layer_gradients(oracle, device):
+    """loss.backward() through Convolution: gradient of the input features against the
+    restated backward, gradient of kernel.weight against torch autograd through an
+    einsum statement of the kernel synthesis (ss_conv/utils/kernel.py:267-299)."""
+    from ss_conv.convolution import Convolution
+    from ss_conv.sp_ops.tensor import SparseTensor
+    torch.manual_seed(2)
+    rs_in, rs_out = [(2, 0), (1, 1), (1, 2)], [(3, 0), (2, 1)]
+    rng = np.random.default_rng(5)
+    grid, n = 9, 250
+    idx = random_voxels(rng, 2, grid, n)
+    conv = Convolution(rs_in, rs_out, 3, stride=1, padding=1).to(device).train()
+    cin, cout = conv.in_channels, conv.out_channels
+    feats = torch.from_numpy(rng.normal(size=(n, cin)).astype(np.float32)).to(device)
+    feats.requires_grad_(True)
+    x = SparseTensor(feats, torch.from_numpy(idx).to(device), [grid] * 3, 2)
+    out = conv(x)
+    g_out = torch.from_numpy(rng.normal(size=tuple(out.features.shape)).astype(np.float32))
+    (out.features * g_out.to(device)).sum().backward()
+
+    ker = conv.kernel
+    w_dense = ker().detach().permute(2, 3, 4, 1, 0).reshape(27, cin, cout).cpu().numpy()
+    o_idx, o_pairs, o_num = oracle.canonicalize(*oracle.rulebook(idx, 2, [grid] * 3, 3, 1, 1))
+    assert np.array_equal(out.indices.cpu().numpy(), o_idx)
+    ref_in, ref_w = oracle.conv_bwd(feats.detach().cpu().numpy(), w_dense, g_out.numpy(), o_pairs,
+                                    o_num)
+    assert rel_l2(feats.grad.cpu().numpy(), ref_in) < REL_L2
+    # kernel.weight: chain ref_w [K, Cin, Cout] through the synthesis, in float64 on the CPU
+    wt = ker.weight.detach().cpu().double().requires_grad_(True)
+    rows, off = [], 0
+    for i, (mi, di) in enumerate(zip(ker.multiplicities_out, ker.dims_out)):
+        cols = []
+        for j, (mj, dj) in enumerate(zip(ker.multiplicities_in, ker.dims_in)):
+            kij = getattr(ker, "kernel_%d_%d" % (i, j))
+            if kij is None:
+                cols.append(torch.zeros(mi * di, mj * dj, 3, 3, 3, dtype=torch.float64))
+                continue
+            nb = kij.size(0)
+            wb = wt[off:off + mi * mj * nb].view(mi, mj, nb)
+            off += mi * mj * nb
+            blk = torch.einsum("uvn,nabxyz->uavbxyz", wb, kij.detach().cpu().double())
+            cols.append(blk.reshape(mi * di, mj * dj, 3, 3, 3))
+        rows.append(torch.cat(cols, 1))
+    dense = torch.cat(rows, 0)  # [Cout, Cin, 3, 3, 3]
+    assert rel_l2(dense.detach().permute(2, 3, 4, 1, 0).reshape(27, cin, cout).numpy(),
+                  w_dense) < 1e-6
+    (dense.permute(2, 3, 4, 1, 0).reshape(27, cin, cout) *
+     torch.from_numpy(ref_w).double()).sum().backward()
+    assert rel_l2(ker.weight.grad.cpu().numpy(), wt.grad.numpy()) < REL_L2
+
+
 def test_downsampling_block(oracle, device):
     """Strided convolution followed by MaxPool and AvgPool (k=2, s=2)."""
     import torch.nn.functional as F

@@ -47,6 +47,41 @@ def test_conv_equals_dense_conv3d(k, s, p, d, oracle):
         assert float(want.abs().sum(1)[mask].max()) == 0.0
 
 
+@pytest.mark.parametrize("k,s,p", [(3, 1, 1), (3, 2, 1), (2, 2, 0)])
+def test_conv_backward_equals_dense_autograd(k, s, p, oracle):
+    """The restated backward equals torch's autograd through F.conv3d on the densified
+    input: gradient with respect to the active inputs and to the kernel, for an output
+    gradient that is zero at inactive outputs."""
+    rng = np.random.default_rng(31)
+    batch, grid, n, cin, cout = 2, 7, 60, 3, 4
+    idx = random_voxels(rng, batch, grid, n)
+    feats = rng.normal(size=(n, cin)).astype(np.float32)
+    K = k ** 3
+    w = rng.normal(size=(K, cin, cout)).astype(np.float32)
+    o_idx, pairs, num, o_shape = oracle.rulebook(idx, batch, [grid] * 3, k, s, p)
+    g_out = rng.normal(size=(o_idx.shape[0], cout)).astype(np.float32)
+    d_in, d_w = oracle.conv_bwd(feats, w, g_out, pairs, num)
+
+    x = dense(idx, feats, batch, grid).requires_grad_(True)
+    kernel = torch.from_numpy(w).double().reshape(k, k, k, cin, cout).permute(4, 3, 0, 1, 2) \
+        .contiguous().requires_grad_(True)
+    out = F.conv3d(x, kernel, stride=s, padding=p)
+    assert list(out.shape[2:]) == [int(v) for v in o_shape]
+    go = torch.zeros_like(out)
+    t = torch.from_numpy(o_idx).long()
+    go[t[:, 0], :, t[:, 1], t[:, 2], t[:, 3]] = torch.from_numpy(g_out).double()
+    out.backward(go)
+    ref_in = at_rows(x.grad, idx)
+    ref_w = kernel.grad.permute(2, 3, 4, 1, 0).reshape(K, cin, cout).numpy()
+    assert np.allclose(d_in, ref_in, atol=1e-4)
+    assert np.allclose(d_w, ref_w, atol=1e-4)
+    # the input gradient of an inverse convolution flows the other way through the pairs
+    d_in_inv, d_w_inv = oracle.conv_bwd(g_out, np.transpose(w, (0, 2, 1)).copy(), feats, pairs,
+                                        num, inverse=True)
+    assert d_in_inv.shape == g_out.shape and d_w_inv.shape == (K, cout, cin)
+    assert np.allclose(d_w_inv, np.transpose(d_w, (0, 2, 1)), atol=1e-4)
+
+
 def test_conv_inverse_is_transpose(oracle):
     """<conv(x), y> == <x, conv_inverse(y)> with the transposed per-offset matrices."""
     rng = np.random.default_rng(2)
