@@ -109,6 +109,21 @@ def ops_table(torch, _ext, synth, dev, seed):
         rows.append("%-44s %8.3f ms %9.2f MB %8.1f GB/s %5.1f%% of HBM  %s"
                     % (name, ms, nbytes / 1e6, gbs, gbs / 80.0, note))
 
+    # convolution backward on the benchmark layer (cfg2: 64 -> 128 channels)
+    cfg = synth.CONFIGS["cfg2"]
+    pts, feats, ids = synth.config_clouds("cfg2", seed)
+    idx = torch.from_numpy(synth.voxel_indices(pts, ids, cfg["grid"])).to(dev)
+    o_idx, pairs, num = get_indice_pairs(idx, cfg["batch"], [cfg["grid"]] * 3, 3, 1, 1)
+    cin, cout, K = 64, 128, 27
+    f = torch.randn(idx.shape[0], cin, device=dev)
+    w = torch.randn(3, 3, 3, cin, cout, device=dev) / (K * cin) ** 0.5
+    go = torch.randn(o_idx.shape[0], cout, device=dev)
+    P = int(num.sum().item())
+    ms, _ = timed(lambda: _ext.indice_conv_backward_fp32(f, w, go, pairs, num, 0, 0), n=10)
+    rows.append("%-44s %8.3f ms %9.2f GFLOP %7.1f TFLOP/s %5.1f%% of fp32 MFMA peak"
+                % ("conv backward, cfg2 (input + filter gradient)", ms, 4.0 * P * cin * cout / 1e9,
+                   4.0 * P * cin * cout / ms / 1e9, 4.0 * P * cin * cout / ms / 1e9 / 1.573))
+
     # pools on the output of the stride-2 layer: 32 clouds at 32^3, 256 channels
     cfg = synth.CONFIGS["cfg3"]
     pts, feats, ids = synth.config_clouds("cfg3", seed)
@@ -286,7 +301,7 @@ def main():
         ops_table(torch, _ext, synth, dev, args.seed)
 
     if not args.no_cpu_baseline:
-        w = conv.kernel().permute(2, 3, 4, 1, 0).reshape(K, c_in, c_out).cpu().numpy()
+        w = conv.kernel().detach().permute(2, 3, 4, 1, 0).reshape(K, c_in, c_out).cpu().numpy()
         base, ref_out = cpu_baseline(indices.cpu().numpy(), features.cpu().numpy(), w, cfg, n_out)
         result["cpu_baseline"] = base
         # the timed GPU result against the CPU port (first-touch vs key order: compare by key)

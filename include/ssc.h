@@ -192,6 +192,23 @@ int ssc_summary_rf(const int32_t *pairs, int64_t pair_stride, const int32_t *pai
                    int32_t kernel_volume, int32_t *rf /* [n_out] */, int64_t n_out,
                    void *workspace, size_t workspace_bytes, ssc_stream_t stream);
 
+/* Backward of rulebook pooling -- replaces indice_maxpool_backward_fp32 /
+ * indice_avgpool_backward_fp32 (src/ss_conv_ops_api.cpp, src/pool/indice_maxpool.h:52-86,
+ * src/pool/indice_avgpool.h:54-90).  in_grad [n_in, channels] is written completely:
+ *   max: in_grad[i] = sum over the pairs (i, o), offsets ascending, of out_grad[o] where
+ *        features[i] == out_features[o] (element-wise);
+ *   avg: in_grad[i] = sum over the pairs of out_grad[o] / (float)summaryrf[o].
+ * Workspace: ssc_pool_workspace_bytes(n_in, kernel_volume). */
+int ssc_pool_max_bwd_f32(const float *features, const float *out_features, const float *out_grad,
+                         int32_t channels, const int32_t *pairs, int64_t pair_stride,
+                         const int32_t *pair_num, int32_t kernel_volume, float *in_grad,
+                         int64_t n_in, void *workspace, size_t workspace_bytes,
+                         ssc_stream_t stream);
+int ssc_pool_avg_bwd_f32(const float *out_grad, int32_t channels, const int32_t *pairs,
+                         int64_t pair_stride, const int32_t *pair_num, int32_t kernel_volume,
+                         const int32_t *summaryrf, float *in_grad, int64_t n_in, void *workspace,
+                         size_t workspace_bytes, ssc_stream_t stream);
+
 /* ------------------------------------------------------------------------
  * Segment ("global") pooling over row ranges offsets[s]..offsets[s+1].
  * Replace global_avgpool_fp / global_maxpool_fp (src/pool/global_avgpool.cpp:13-20,
@@ -206,6 +223,16 @@ int ssc_segment_avg_f32(const float *feats /* [sum_n,c] */, const int32_t *offse
 int ssc_segment_max_f32(const float *feats, const int32_t *offsets, float *out,
                         int32_t *out_idx /* [b,c] */, int32_t n_segments, int32_t channels,
                         ssc_stream_t stream);
+
+/* Backward of the segment pools -- replaces global_avgpool_bp / global_maxpool_bp
+ * (src/pool/global_avgpool_cuda_kernel.cu:44-62, global_maxpool_cuda_kernel.cu:45-60).
+ * in_grad [n_rows, channels] is written completely (rows outside every segment get 0). */
+int ssc_segment_avg_bwd_f32(const float *out_grad /* [n_segments,channels] */,
+                            const int32_t *offsets, float *in_grad, int64_t n_rows,
+                            int32_t n_segments, int32_t channels, ssc_stream_t stream);
+int ssc_segment_max_bwd_f32(const float *out_grad, const int32_t *out_idx /* arg-max rows */,
+                            float *in_grad, int64_t n_rows, int32_t n_segments, int32_t channels,
+                            ssc_stream_t stream);
 
 /* ------------------------------------------------------------------------
  * Point <-> voxel.
@@ -287,6 +314,19 @@ int ssc_three_nn(int32_t n, int32_t m, const float *unknown /* [n,4] */,
 int ssc_three_interp_f32(int32_t c, int32_t m, int32_t n, const float *feats /* [m,c] */,
                          const int32_t *idx /* [n,3] */, const float *weight /* [n,3] */,
                          float *out /* [n,c] */, ssc_stream_t stream);
+
+/* Backward of the two operators above -- replace voxelize_bp
+ * (src/voxelize/voxelize_cuda_kernel.h:44-58) and three_interpolate_bp
+ * (src/voxelize/interpolate_cuda_kernel.cu:104-121).  Both write their gradient
+ * completely.  The interpolation gradient accumulates with float atomics (several
+ * queries share a row), as the reference does: its last bits depend on the order. */
+int ssc_voxel_reduce_bwd_f32(const float *out_grad /* [m,c] */, float *feats_grad /* [n,c] */,
+                             const int32_t *maps, int32_t mode, int32_t n_voxel,
+                             int32_t max_active, int32_t channels, int64_t n_point,
+                             ssc_stream_t stream);
+int ssc_three_interp_bwd_f32(int32_t c, int32_t n, int32_t m, const float *out_grad /* [n,c] */,
+                             const int32_t *idx, const float *weight,
+                             float *points_grad /* [m,c] */, ssc_stream_t stream);
 
 #ifdef __cplusplus
 }

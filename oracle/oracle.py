@@ -295,6 +295,80 @@ def ref_maxpool_fwd(features, pairs, num, n_out):
     return out
 
 
+def maxpool_bwd(features, out_features, out_grad, pairs, num):
+    """src/pool/indice_maxpool_cuda_functor.cu:426-455, offsets ascending: the gradient of an
+    output row goes to every input of its window that equals the pooled value."""
+    features, out_features, out_grad = _f32(features), _f32(out_features), _f32(out_grad)
+    din = np.zeros_like(features)
+    for k in range(pairs.shape[0]):
+        n = int(num[k])
+        if n <= 0:
+            continue
+        ri, ro = pairs[k, 0, :n], pairs[k, 1, :n]
+        hit = features[ri] == out_features[ro]
+        din[ri] = (din[ri] + np.where(hit, out_grad[ro], np.float32(0))).astype(np.float32)
+    return din
+
+
+def avgpool_bwd(out_grad, pairs, num, n_in, rf):
+    """src/pool/indice_avgpool_cuda_functor.cu (backward kernels), offsets ascending:
+    din[i] += dout[o] / (float)rf[o]."""
+    out_grad = _f32(out_grad)
+    din = np.zeros((n_in, out_grad.shape[1]), dtype=np.float32)
+    rf = np.asarray(rf).astype(np.float32)
+    for k in range(pairs.shape[0]):
+        n = int(num[k])
+        if n <= 0:
+            continue
+        ri, ro = pairs[k, 0, :n], pairs[k, 1, :n]
+        din[ri] = (din[ri] + out_grad[ro] / rf[ro][:, None]).astype(np.float32)
+    return din
+
+
+def segment_avg_bwd(out_grad, offsets, n_rows):
+    """src/pool/global_avgpool_cuda_kernel.cu:44-55."""
+    out_grad = _f32(out_grad)
+    din = np.zeros((n_rows, out_grad.shape[1]), dtype=np.float32)
+    for s in range(len(offsets) - 1):
+        a, b = int(offsets[s]), int(offsets[s + 1])
+        if b > a:
+            din[a:b] = out_grad[s] / np.float32(b - a)
+    return din
+
+
+def segment_max_bwd(out_grad, arg, n_rows):
+    """src/pool/global_maxpool_cuda_kernel.cu:45-53."""
+    out_grad = _f32(out_grad)
+    din = np.zeros((n_rows, out_grad.shape[1]), dtype=np.float32)
+    for s in range(out_grad.shape[0]):
+        for c in range(out_grad.shape[1]):
+            if arg[s, c] >= 0:
+                din[arg[s, c], c] += out_grad[s, c]
+    return din
+
+
+def voxel_reduce_bwd(out_grad, maps, mode, n_point):
+    """src/voxelize/voxelize_cuda_kernel.h:44-58."""
+    out_grad = _f32(out_grad)
+    din = np.zeros((n_point, out_grad.shape[1]), dtype=np.float32)
+    for v in range(maps.shape[0]):
+        na = int(maps[v, 0])
+        mult = np.float32(1.0) / np.float32(na) if (mode == 4 and na > 0) else np.float32(1.0)
+        for i in range(1, na + 1):
+            din[maps[v, i]] += mult * out_grad[v]
+    return din
+
+
+def three_interp_bwd(out_grad, idx, weight, m):
+    """src/voxelize/interpolate_cuda_kernel.cu:104-121 (accumulated in float64: the
+    reference's atomic order is not fixed)."""
+    out_grad, weight = _f32(out_grad), _f32(weight)
+    g = np.zeros((m, out_grad.shape[1]), dtype=np.float64)
+    for j in range(3):
+        np.add.at(g, idx[:, j], out_grad.astype(np.float64) * weight[:, j:j + 1].astype(np.float64))
+    return g.astype(np.float32)
+
+
 def summary_rf(pairs, num, n_out):
     """src/ss_conv_ops.cu:116-145 + src/pool/indiceSummaryRF.cu:21-36."""
     L = lib()

@@ -17,15 +17,18 @@ namespace ssc {
 
 typedef float float4v __attribute__((ext_vector_type(4)));
 
+// table[key row * K + k] = the other row of the pair; key_plane 1 keys by output rows
+// (forward), 0 by input rows (backward).
 __global__ void __launch_bounds__(256)
     pair_table_kernel(const int32_t *__restrict__ pairs, int64_t pair_stride,
-                      const int32_t *__restrict__ pair_num, int K, int32_t *__restrict__ table) {
+                      const int32_t *__restrict__ pair_num, int K, int key_plane,
+                      int32_t *__restrict__ table) {
   int k = blockIdx.y;
   int64_t j = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (j >= pair_num[k]) return;
   const int32_t *p = pairs + (int64_t)k * 2 * pair_stride;
-  int64_t o = p[pair_stride + j];
-  table[o * K + k] = p[j];
+  int64_t key = p[key_plane * pair_stride + j];
+  table[key * K + k] = p[(1 - key_plane) * pair_stride + j];
 }
 
 __global__ void __launch_bounds__(256)
@@ -143,6 +146,67 @@ __global__ void __launch_bounds__(kSegRows * 64)
   }
 }
 
+// Backward of rulebook pooling, input stationary: every input row visits its pairs in
+// ascending offset order, the order of the reference's per-offset launches
+// (src/pool/indice_maxpool_cuda_functor.cu:426-455: din[i] += dout[o] where in[i] == out[o];
+// src/pool/indice_avgpool_cuda_functor.cu: din[i] += dout[o] / (float)rf[o]).
+// table is [n_in, K] of output rows.  MODE 0 max, 1 average.
+template <int MODE>
+__global__ void __launch_bounds__(256)
+    pool_bwd_kernel(const float *__restrict__ in, const float *__restrict__ out,
+                    const float *__restrict__ dout, int C, const int32_t *__restrict__ table,
+                    int K, const int32_t *__restrict__ rf, float *__restrict__ din, int64_t n_in) {
+  int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= n_in * C) return;
+  int64_t i = idx / C;
+  int c = (int)(idx - i * C);
+  const int32_t *t = table + i * K;
+  float acc = 0.f;
+  float x = MODE == 0 ? in[idx] : 0.f;
+  for (int k = 0; k < K; ++k) {
+    int64_t o = t[k];
+    if (o < 0) continue;
+    float g = dout[o * C + c];
+    if (MODE == 0) {
+      if (x == out[o * C + c]) acc = acc + g;
+    } else {
+      acc = acc + g / (float)rf[o];
+    }
+  }
+  din[idx] = acc;
+}
+
+// Backward of the segment pools (src/pool/global_avgpool_cuda_kernel.cu:44-62,
+// global_maxpool_cuda_kernel.cu:45-60): average spreads dout / len over the segment's
+// rows; max routes dout to the arg-max row.  din must be zero for the max variant.
+__global__ void __launch_bounds__(256)
+    segment_avg_bwd_kernel(const float *__restrict__ dout, const int32_t *__restrict__ offsets,
+                           int n_seg, int C, float *__restrict__ din, int64_t n_rows) {
+  int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= n_rows * C) return;
+  int64_t r = idx / C;
+  int c = (int)(idx - r * C);
+  int lo = 0, hi = n_seg;  // the segment s with offsets[s] <= r < offsets[s+1]
+  while (hi - lo > 1) {
+    int mid = (lo + hi) >> 1;
+    if (offsets[mid] <= r) lo = mid;
+    else hi = mid;
+  }
+  float v = 0.f;
+  if (r >= offsets[0] && r < offsets[n_seg])
+    v = dout[(int64_t)lo * C + c] / (float)(offsets[lo + 1] - offsets[lo]);
+  din[idx] = v;
+}
+
+__global__ void __launch_bounds__(256)
+    segment_max_bwd_kernel(const float *__restrict__ dout, const int32_t *__restrict__ arg,
+                           int64_t n, int C, float *__restrict__ din) {
+  int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= n) return;
+  int a = arg[idx];
+  if (a >= 0) din[(int64_t)a * C + (idx % C)] = dout[idx];
+}
+
 static int pool_common(const float *features, int channels, const int32_t *pairs,
                        int64_t pair_stride, const int32_t *pair_num, int K, float *out,
                        int64_t n_out, void *ws, size_t ws_bytes, hipStream_t s,
@@ -158,7 +222,7 @@ static int pool_common(const float *features, int channels, const int32_t *pairs
   if (rc != SSC_OK) return rc;
   if (pair_stride > 0) {
     hipLaunchKernelGGL(pair_table_kernel, dim3((unsigned)ceil_div(pair_stride, 256), (unsigned)K),
-                       dim3(256), 0, s, pairs, pair_stride, pair_num, K, table);
+                       dim3(256), 0, s, pairs, pair_stride, pair_num, K, 1, table);
     SSC_LAUNCH_CHECK("pair_table");
   }
   *table_out = table;
@@ -267,6 +331,92 @@ int ssc_segment_max_f32(const float *feats, const int32_t *offsets, float *out, 
                      dim3(kSegRows * 64), 0, (hipStream_t)stream, feats, offsets, out, out_idx,
                      channels);
   SSC_LAUNCH_CHECK("segment_max");
+  return SSC_OK;
+}
+
+static int pool_bwd(int mode, const float *features, const float *out_features,
+                    const float *out_grad, int channels, const int32_t *pairs, int64_t pair_stride,
+                    const int32_t *pair_num, int K, const int32_t *summaryrf, float *in_grad,
+                    int64_t n_in, void *ws, size_t ws_bytes, hipStream_t s) {
+  SSC_CHECK(K >= 1 && K <= SSC_MAX_KERNEL_VOLUME, SSC_ERUNTIME, "kernel volume %d out of range", K);
+  SSC_CHECK(channels >= 1 && n_in >= 0 && pair_stride >= 0, SSC_EINVAL, "bad sizes");
+  if (n_in == 0) return SSC_OK;
+  SSC_CHECK(in_grad && ws, SSC_EINVAL, "NULL pointer argument");
+  SSC_CHECK(pair_stride == 0 || (out_grad && pairs && pair_num), SSC_EINVAL,
+            "NULL pointer argument");
+  SSC_CHECK(mode == 1 || pair_stride == 0 || (features && out_features), SSC_EINVAL,
+            "NULL pointer argument");
+  SSC_CHECK(mode == 0 || pair_stride == 0 || summaryrf, SSC_EINVAL, "summaryrf is NULL");
+  SSC_CHECK(ws_bytes >= align_up((size_t)n_in * K * 4), SSC_EWORKSPACE,
+            "pool backward workspace too small");
+  int32_t *table = static_cast<int32_t *>(ws);
+  int rc = fill_i32(table, n_in * K, -1, s);
+  if (rc != SSC_OK) return rc;
+  if (pair_stride > 0) {
+    hipLaunchKernelGGL(pair_table_kernel, dim3((unsigned)ceil_div(pair_stride, 256), (unsigned)K),
+                       dim3(256), 0, s, pairs, pair_stride, pair_num, K, 0, table);
+    SSC_LAUNCH_CHECK("pair_table");
+  }
+  const int64_t n = n_in * channels;
+  if (mode == 0)
+    hipLaunchKernelGGL((pool_bwd_kernel<0>), dim3((unsigned)ceil_div(n, 256)), dim3(256), 0, s,
+                       features, out_features, out_grad, channels, table, K, summaryrf, in_grad,
+                       n_in);
+  else
+    hipLaunchKernelGGL((pool_bwd_kernel<1>), dim3((unsigned)ceil_div(n, 256)), dim3(256), 0, s,
+                       features, out_features, out_grad, channels, table, K, summaryrf, in_grad,
+                       n_in);
+  SSC_LAUNCH_CHECK("pool_bwd");
+  return SSC_OK;
+}
+
+int ssc_pool_max_bwd_f32(const float *features, const float *out_features, const float *out_grad,
+                         int32_t channels, const int32_t *pairs, int64_t pair_stride,
+                         const int32_t *pair_num, int32_t kernel_volume, float *in_grad,
+                         int64_t n_in, void *workspace, size_t workspace_bytes,
+                         ssc_stream_t stream) {
+  return pool_bwd(0, features, out_features, out_grad, channels, pairs, pair_stride, pair_num,
+                  kernel_volume, nullptr, in_grad, n_in, workspace, workspace_bytes,
+                  (hipStream_t)stream);
+}
+
+int ssc_pool_avg_bwd_f32(const float *out_grad, int32_t channels, const int32_t *pairs,
+                         int64_t pair_stride, const int32_t *pair_num, int32_t kernel_volume,
+                         const int32_t *summaryrf, float *in_grad, int64_t n_in, void *workspace,
+                         size_t workspace_bytes, ssc_stream_t stream) {
+  return pool_bwd(1, nullptr, nullptr, out_grad, channels, pairs, pair_stride, pair_num,
+                  kernel_volume, summaryrf, in_grad, n_in, workspace, workspace_bytes,
+                  (hipStream_t)stream);
+}
+
+int ssc_segment_avg_bwd_f32(const float *out_grad, const int32_t *offsets, float *in_grad,
+                            int64_t n_rows, int32_t n_segments, int32_t channels,
+                            ssc_stream_t stream) {
+  SSC_CHECK(n_segments >= 0 && channels >= 1 && n_rows >= 0, SSC_EINVAL, "bad sizes");
+  if (n_rows == 0) return SSC_OK;
+  SSC_CHECK(in_grad != nullptr, SSC_EINVAL, "in_grad is NULL");
+  if (n_segments == 0) return fill_f32(in_grad, n_rows * channels, 0.f, (hipStream_t)stream);
+  SSC_CHECK(out_grad && offsets, SSC_EINVAL, "NULL pointer argument");
+  hipLaunchKernelGGL(segment_avg_bwd_kernel, dim3((unsigned)ceil_div(n_rows * channels, 256)),
+                     dim3(256), 0, (hipStream_t)stream, out_grad, offsets, (int)n_segments,
+                     (int)channels, in_grad, n_rows);
+  SSC_LAUNCH_CHECK("segment_avg_bwd");
+  return SSC_OK;
+}
+
+int ssc_segment_max_bwd_f32(const float *out_grad, const int32_t *out_idx, float *in_grad,
+                            int64_t n_rows, int32_t n_segments, int32_t channels,
+                            ssc_stream_t stream) {
+  SSC_CHECK(n_segments >= 0 && channels >= 1 && n_rows >= 0, SSC_EINVAL, "bad sizes");
+  if (n_rows == 0) return SSC_OK;
+  SSC_CHECK(in_grad != nullptr, SSC_EINVAL, "in_grad is NULL");
+  int rc = fill_f32(in_grad, n_rows * channels, 0.f, (hipStream_t)stream);
+  if (rc != SSC_OK || n_segments == 0) return rc;
+  SSC_CHECK(out_grad && out_idx, SSC_EINVAL, "NULL pointer argument");
+  const int64_t n = (int64_t)n_segments * channels;
+  hipLaunchKernelGGL(segment_max_bwd_kernel, dim3((unsigned)ceil_div(n, 256)), dim3(256), 0,
+                     (hipStream_t)stream, out_grad, out_idx, n, (int)channels, in_grad);
+  SSC_LAUNCH_CHECK("segment_max_bwd");
   return SSC_OK;
 }
 }

@@ -475,3 +475,82 @@ int ssc_p2v_compact(const float *points, const float *feats, const int64_t *batc
   return SSC_OK;
 }
 }
+
+// ---- backward of the feature reduction and of the interpolation ---------------------------
+namespace ssc {
+
+// d_feats[p,c] = mult * d_out[v,c] for every point p in voxel v's list (a point is in at
+// most one list, so these are plain stores); src/voxelize/voxelize_cuda_kernel.h:44-58.
+__global__ void __launch_bounds__(256)
+    voxel_reduce_bwd_kernel(const float *__restrict__ d_out, float *__restrict__ d_feats,
+                            const int32_t *__restrict__ maps, int mode, int64_t n_voxel,
+                            int max_active, int C) {
+  int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= n_voxel * C) return;
+  int64_t v = idx / C;
+  int c = (int)(idx - v * C);
+  const int32_t *r = maps + v * (max_active + 1);
+  int na = r[0];
+  float mult = (mode == 4 && na > 0) ? 1.f / (float)na : 1.f;
+  float g = mult * d_out[idx];
+  for (int i = 1; i <= na; ++i) d_feats[(int64_t)r[i] * C + c] = g;
+}
+
+// grad_points[idx[q,j], c] += grad_out[q,c] * weight[q,j]: several queries share a row, so
+// this accumulates with float atomics, as src/voxelize/interpolate_cuda_kernel.cu:104-121
+// does (the order of the additions, hence the last bits, is not fixed there either).
+__global__ void __launch_bounds__(256)
+    three_interp_bwd_kernel(int C, int n, const float *__restrict__ grad_out,
+                            const int32_t *__restrict__ idx, const float *__restrict__ weight,
+                            float *__restrict__ grad_points) {
+  int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (e >= (int64_t)n * C) return;
+  int64_t q = e / C;
+  int c = (int)(e - q * C);
+  float g = grad_out[e];
+#pragma unroll
+  for (int j = 0; j < 3; ++j) {
+    float t = g * weight[q * 3 + j];
+    atomicAdd(&grad_points[(int64_t)idx[q * 3 + j] * C + c], t);
+  }
+}
+
+}  // namespace ssc
+
+extern "C" {
+
+int ssc_voxel_reduce_bwd_f32(const float *out_grad, float *feats_grad, const int32_t *maps,
+                             int32_t mode, int32_t n_voxel, int32_t max_active, int32_t channels,
+                             int64_t n_point, ssc_stream_t stream) {
+  SSC_CHECK(n_voxel >= 0 && max_active >= 1 && channels >= 1 && n_point >= 0, SSC_EINVAL,
+            "bad sizes");
+  if (n_point == 0) return SSC_OK;
+  SSC_CHECK(feats_grad != nullptr, SSC_EINVAL, "feats_grad is NULL");
+  hipStream_t s = (hipStream_t)stream;
+  int rc = ssc::fill_f32(feats_grad, n_point * channels, 0.f, s);
+  if (rc != SSC_OK || n_voxel == 0) return rc;
+  SSC_CHECK(out_grad && maps, SSC_EINVAL, "NULL pointer argument");
+  int64_t n = (int64_t)n_voxel * channels;
+  hipLaunchKernelGGL(ssc::voxel_reduce_bwd_kernel, dim3((unsigned)ssc::ceil_div(n, 256)), dim3(256),
+                     0, s, out_grad, feats_grad, maps, mode, (int64_t)n_voxel, max_active, channels);
+  SSC_LAUNCH_CHECK("voxel_reduce_bwd");
+  return SSC_OK;
+}
+
+int ssc_three_interp_bwd_f32(int32_t c, int32_t n, int32_t m, const float *out_grad,
+                             const int32_t *idx, const float *weight, float *points_grad,
+                             ssc_stream_t stream) {
+  SSC_CHECK(c >= 1 && n >= 0 && m >= 0, SSC_EINVAL, "bad sizes");
+  if (m == 0) return SSC_OK;
+  SSC_CHECK(points_grad != nullptr, SSC_EINVAL, "points_grad is NULL");
+  hipStream_t s = (hipStream_t)stream;
+  int rc = ssc::fill_f32(points_grad, (int64_t)m * c, 0.f, s);
+  if (rc != SSC_OK || n == 0) return rc;
+  SSC_CHECK(out_grad && idx && weight, SSC_EINVAL, "NULL pointer argument");
+  int64_t e = (int64_t)n * c;
+  hipLaunchKernelGGL(ssc::three_interp_bwd_kernel, dim3((unsigned)ssc::ceil_div(e, 256)), dim3(256),
+                     0, s, c, n, out_grad, idx, weight, points_grad);
+  SSC_LAUNCH_CHECK("three_interp_bwd");
+  return SSC_OK;
+}
+}

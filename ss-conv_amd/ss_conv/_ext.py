@@ -46,6 +46,14 @@ _SIGNATURES = {
     "ssc_conv_bwd_filter_workspace_bytes": (_sz, [_i32, _i32, _i32, _i64]),
     "ssc_conv_bwd_filter_f32": (ctypes.c_int, [_vp, _i64, _i32, _vp, _i64, _i32, _vp, _i64, _vp,
                                                _i32, _i32, _vp, _i64, _i64, _i64, _vp, _sz, _vp]),
+    "ssc_pool_max_bwd_f32": (ctypes.c_int, [_vp, _vp, _vp, _i32, _vp, _i64, _vp, _i32, _vp, _i64,
+                                            _vp, _sz, _vp]),
+    "ssc_pool_avg_bwd_f32": (ctypes.c_int, [_vp, _i32, _vp, _i64, _vp, _i32, _vp, _vp, _i64, _vp,
+                                            _sz, _vp]),
+    "ssc_segment_avg_bwd_f32": (ctypes.c_int, [_vp, _vp, _vp, _i64, _i32, _i32, _vp]),
+    "ssc_segment_max_bwd_f32": (ctypes.c_int, [_vp, _vp, _vp, _i64, _i32, _i32, _vp]),
+    "ssc_voxel_reduce_bwd_f32": (ctypes.c_int, [_vp, _vp, _vp, _i32, _i32, _i32, _i32, _i64, _vp]),
+    "ssc_three_interp_bwd_f32": (ctypes.c_int, [_i32, _i32, _i32, _vp, _vp, _vp, _vp, _vp]),
     "ssc_profile_conv": (ctypes.c_int, [_i32]),
     "ssc_profile_conv_read": (ctypes.c_int, [ctypes.POINTER(ctypes.c_float), _i32,
                                              ctypes.POINTER(_i32)]),
@@ -278,6 +286,82 @@ def indice_avgpool_fp32(features, indice_pairs, indice_num, num_act, summaryrf):
                                  _ptr(rf), _ptr(out), n_out, ws.data_ptr(), ws.numel(),
                                  _stream(features)))
     return out
+
+
+def indice_maxpool_backward_fp32(features, out_features, out_bp, indice_pairs, indice_num):
+    """src/pool/indice_maxpool.h:52-86: gradient of the pooled rows routed to the inputs
+    that equal the maximum."""
+    features, pairs, num = _pool_args(features, indice_pairs, indice_num)
+    out_features = out_features.contiguous()
+    out_bp = out_bp.contiguous()
+    _need_gpu(out_features, out_bp)
+    n_in, c = features.shape
+    K = pairs.size(0)
+    din = torch.empty((n_in, c), dtype=torch.float32, device=features.device)
+    ws = _workspace(_lib.ssc_pool_workspace_bytes(n_in, K), features.device)
+    _check(_lib.ssc_pool_max_bwd_f32(_ptr(features), _ptr(out_features), _ptr(out_bp), c,
+                                     _ptr(pairs), pairs.size(2), num.data_ptr(), K, _ptr(din),
+                                     n_in, ws.data_ptr(), ws.numel(), _stream(features)))
+    return din
+
+
+def indice_avgpool_backward_fp32(features, out_features, out_bp, indice_pairs, indice_num,
+                                 summaryrf):
+    """src/pool/indice_avgpool.h:54-90."""
+    features, pairs, num = _pool_args(features, indice_pairs, indice_num)
+    out_bp = out_bp.contiguous()
+    _need_gpu(out_bp, summaryrf)
+    rf = summaryrf.int().contiguous()
+    n_in, c = features.shape
+    K = pairs.size(0)
+    din = torch.empty((n_in, c), dtype=torch.float32, device=features.device)
+    ws = _workspace(_lib.ssc_pool_workspace_bytes(n_in, K), features.device)
+    _check(_lib.ssc_pool_avg_bwd_f32(_ptr(out_bp), c, _ptr(pairs), pairs.size(2), num.data_ptr(),
+                                     K, _ptr(rf), _ptr(din), n_in, ws.data_ptr(), ws.numel(),
+                                     _stream(features)))
+    return din
+
+
+def global_avgpool_bp(d_feats, offsets, out_maxidx, d_out, n_proposal, c):
+    """src/pool/global_avgpool.cpp global_avgpool_bp wrapper; fills d_feats in place."""
+    _seg_args(d_feats, offsets, d_out, n_proposal, c)
+    _check(_lib.ssc_segment_avg_bwd_f32(_ptr(d_out), _ptr(offsets), _ptr(d_feats), d_feats.size(0),
+                                        int(n_proposal), int(c), _stream(d_feats)))
+
+
+def global_maxpool_bp(d_feats, offsets, out_maxidx, d_out, n_proposal, c):
+    """src/pool/global_maxpool.cpp global_maxpool_bp wrapper; fills d_feats in place."""
+    _seg_args(d_feats, offsets, d_out, n_proposal, c)
+    _need_gpu(out_maxidx)
+    _check(_lib.ssc_segment_max_bwd_f32(_ptr(d_out), _ptr(out_maxidx.int().contiguous()),
+                                        _ptr(d_feats), d_feats.size(0), int(n_proposal), int(c),
+                                        _stream(d_feats)))
+
+
+def voxelize_bp(d_out, d_feats, maps, mode, n_voxel, max_active, c):
+    """src/voxelize/voxelize.cpp voxelize_bp wrapper; fills d_feats in place."""
+    _need_gpu(d_out, d_feats, maps)
+    if d_out.dtype != torch.float32 or d_feats.dtype != torch.float32 or maps.dtype != torch.int32:
+        raise RuntimeError("voxelize_bp: wrong dtypes")
+    for t in (d_out, d_feats, maps):
+        if not t.is_contiguous():
+            raise RuntimeError("voxelize_bp needs contiguous tensors")
+    _check(_lib.ssc_voxel_reduce_bwd_f32(_ptr(d_out), _ptr(d_feats), _ptr(maps), int(mode),
+                                         int(n_voxel), int(max_active), int(c), d_feats.size(0),
+                                         _stream(d_out)))
+
+
+def three_interpolate_bp(c, n, m, grad_out, idx, weight, grad_points):
+    """src/voxelize/interpolation.cpp three_interpolate_bp wrapper; fills grad_points in place."""
+    _need_gpu(grad_out, idx, weight, grad_points)
+    if grad_out.dtype != torch.float32 or weight.dtype != torch.float32 or \
+            idx.dtype != torch.int32 or grad_points.dtype != torch.float32:
+        raise RuntimeError("three_interpolate_bp: wrong dtypes")
+    for t in (grad_out, idx, weight, grad_points):
+        if not t.is_contiguous():
+            raise RuntimeError("three_interpolate_bp needs contiguous tensors")
+    _check(_lib.ssc_three_interp_bwd_f32(int(c), int(n), int(m), _ptr(grad_out), _ptr(idx),
+                                         _ptr(weight), _ptr(grad_points), _stream(grad_out)))
 
 
 def indiceSummaryRF(indice_pairs, indice_num, num_act):

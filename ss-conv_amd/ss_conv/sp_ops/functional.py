@@ -1,19 +1,12 @@
 """autograd entry points over the native kernels
 (reference: ss_conv/sp_ops/functional.py:22-453; same exported names).
 
-Forward passes run the HIP kernels, and so do the backward passes of the three
-convolution Functions.  The other backward passes are not built yet: a Function
-whose backward is reached raises NotImplementedError instead of returning wrong
-gradients."""
+Forward and backward passes run the HIP kernels (float32 only)."""
 import torch
 from torch.autograd import Function
 
 from ss_conv import _ext
 from . import ops
-
-
-def _no_backward(name):
-    raise NotImplementedError("backward of %s is not built yet (forward-only build)" % name)
 
 
 class _ConvBase(Function):
@@ -82,7 +75,10 @@ class SparseMaxPoolFunction(Function):
 
     @staticmethod
     def backward(ctx, grad_output):
-        _no_backward("indice_maxpool")
+        indice_pairs, indice_pair_num, features, out = ctx.saved_tensors
+        input_bp = ops.indice_maxpool_backward(features, out, grad_output.contiguous(),
+                                               indice_pairs, indice_pair_num)
+        return input_bp, None, None, None
 
 
 class SparseAvgPoolFunction(Function):
@@ -104,7 +100,10 @@ class SparseAvgPoolFunction(Function):
 
     @staticmethod
     def backward(ctx, grad_output):
-        _no_backward("indice_avgpool")
+        indice_pairs, indice_pair_num, features, out, summaryrf = ctx.saved_tensors
+        input_bp = ops.indice_avgpool_backward(features, out, grad_output.contiguous(),
+                                               indice_pairs, indice_pair_num, summaryrf)
+        return input_bp, None, None, None, None
 
 
 class _SegmentPool(Function):
@@ -130,7 +129,11 @@ class GlobalMaxPool(Function):
 
     @staticmethod
     def backward(ctx, d_output_feats):
-        _no_backward("global_maxpool")
+        idx, proposals_offset, n_rows = ctx.for_backwards
+        n_seg, c = d_output_feats.size()
+        d_feats = torch.zeros((n_rows, c), dtype=torch.float32, device=d_output_feats.device)
+        _ext.global_maxpool_bp(d_feats, proposals_offset, idx, d_output_feats.contiguous(), n_seg, c)
+        return d_feats, None
 
 
 class GlobalAvgPool(Function):
@@ -144,7 +147,11 @@ class GlobalAvgPool(Function):
 
     @staticmethod
     def backward(ctx, d_output_feats):
-        _no_backward("global_avgpool")
+        idx, proposals_offset, n_rows = ctx.for_backwards
+        n_seg, c = d_output_feats.size()
+        d_feats = torch.zeros((n_rows, c), dtype=torch.float32, device=d_output_feats.device)
+        _ext.global_avgpool_bp(d_feats, proposals_offset, idx, d_output_feats.contiguous(), n_seg, c)
+        return d_feats, None
 
 
 class Voxelization(Function):
@@ -163,7 +170,11 @@ class Voxelization(Function):
 
     @staticmethod
     def backward(ctx, d_output_feats):
-        _no_backward("voxelization")
+        map_rule, mode, max_active, n = ctx.for_backwards
+        m, c = d_output_feats.size()
+        d_feats = torch.zeros((n, c), dtype=torch.float32, device=d_output_feats.device)
+        _ext.voxelize_bp(d_output_feats.contiguous(), d_feats, map_rule, mode, m, max_active, c)
+        return d_feats, None, None
 
 
 class Voxel2Point_Map(Function):
@@ -225,7 +236,11 @@ class ThreeInterpolate(Function):
 
     @staticmethod
     def backward(ctx, grad_out):
-        _no_backward("three_interpolate")
+        idx, weight, m = ctx.three_interpolate_for_backward
+        n, c = grad_out.size()
+        grad_features = torch.zeros((m, c), dtype=torch.float32, device=grad_out.device)
+        _ext.three_interpolate_bp(c, n, m, grad_out.contiguous(), idx, weight, grad_features)
+        return grad_features, None, None
 
 
 indice_conv = SparseConvFunction.apply

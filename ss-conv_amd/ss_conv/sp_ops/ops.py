@@ -86,7 +86,10 @@ def indice_maxpool_forward(features, indice_pairs, indice_pair_num, num_activate
 
 
 def indice_maxpool_backward(features, out_features, out_bp, indice_pairs, indice_pair_num):
-    raise NotImplementedError("the backward pass of max pooling is not built yet")
+    if features.dtype == torch.float32:
+        return _ext.indice_maxpool_backward_fp32(features, out_features, out_bp, indice_pairs,
+                                                 indice_pair_num)
+    raise NotImplementedError("only float32 pooling is built")
 
 
 def indice_avgpool_forward(features, indice_pairs, indice_pair_num, num_activate_out, summaryrf):
@@ -98,4 +101,7 @@ def indice_avgpool_forward(features, indice_pairs, indice_pair_num, num_activate
 
 def indice_avgpool_backward(features, out_features, out_bp, indice_pairs, indice_pair_num,
                             summaryrf):
-    raise NotImplementedError("the backward pass of average pooling is not built yet")
+    if features.dtype == torch.float32:
+        return _ext.indice_avgpool_backward_fp32(features, out_features, out_bp, indice_pairs,
+                                                 indice_pair_num, summaryrf)
+    raise NotImplementedError("only float32 pooling is built")

@@ -366,7 +366,7 @@ def test_kernel_combine_matches_einsum(oracle, device):
                                 ([(3, 0)], [(2, 0), (1, 1), (1, 2)], 3),
                                 ([(1, 0), (2, 2)], [(2, 1), (1, 4)], 5)]:
         ker = SE3Kernel(rs_in, rs_out, size).to(device)
-        got = ker().cpu().numpy()
+        got = ker().detach().cpu().numpy()
         bases = [[getattr(ker, "kernel_%d_%d" % (i, j)) for j in range(len(ker.Rs_in))]
                  for i in range(len(ker.Rs_out))]
         bases = [[None if b is None else b.cpu().numpy() for b in row] for row in bases]
@@ -505,6 +505,72 @@ def test_layer_gradients(oracle, device):
     assert rel_l2(ker.weight.grad.cpu().numpy(), wt.grad.numpy()) < REL_L2
 
 
+@pytest.mark.parametrize("k,s,p,c", [(2, 2, 0, 64), (3, 2, 1, 32), (3, 1, 1, 5)])
+def test_pool_backward_matches_oracle(k, s, p, c, oracle, device):
+    """Max / avg pooling gradients through autograd (bit-exact: same order of additions)."""
+    from ss_conv.sp_ops.functional import indice_avgpool, indice_maxpool
+    rng = np.random.default_rng(23)
+    n, grid = 400, 10
+    idx = random_voxels(rng, 2, grid, n)
+    feats = rng.normal(size=(n, c)).astype(np.float32)
+    o_idx, o_pairs, o_num = oracle.canonicalize(*oracle.rulebook(idx, 2, [grid] * 3, k, s, p))
+    g_idx, g_pairs, g_num = [torch.from_numpy(x).to(device) for x in
+                             gpu_rulebook(idx, 2, grid, k, s, p)]
+    g_out = rng.normal(size=(o_idx.shape[0], c)).astype(np.float32)
+    for op, name in ((indice_maxpool, "max"), (indice_avgpool, "avg")):
+        x = torch.from_numpy(feats).to(device).requires_grad_(True)
+        y = op(x, g_pairs, g_num, g_idx.shape[0])
+        (y * torch.from_numpy(g_out).to(device)).sum().backward()
+        if name == "max":
+            pooled = oracle.maxpool_fwd(feats, o_pairs, o_num, o_idx.shape[0])
+            ref = oracle.maxpool_bwd(feats, pooled, g_out, o_pairs, o_num)
+        else:
+            ref = oracle.avgpool_bwd(g_out, o_pairs, o_num, n,
+                                     np.full(o_idx.shape[0], k ** 3, dtype=np.int32))
+        assert np.array_equal(x.grad.cpu().numpy(), ref), name
+
+
+def test_segment_voxel_interp_backward(oracle, device):
+    from ss_conv.sp_ops.functional import (global_avgpool, global_maxpool, voxelization,
+                                           three_interpolate)
+    rng = np.random.default_rng(29)
+    n, c = 500, 70
+    feats = rng.normal(size=(n, c)).astype(np.float32)
+    offsets = np.array([0, 120, 120, 333, 500], dtype=np.int32)
+    g = rng.normal(size=(4, c)).astype(np.float32)
+    offs = torch.from_numpy(offsets).to(device)
+    x = torch.from_numpy(feats).to(device).requires_grad_(True)
+    (global_avgpool(x, offs) * torch.from_numpy(g).to(device))[[0, 2, 3]].sum().backward()
+    ref = oracle.segment_avg_bwd(g, offsets, n)
+    assert np.array_equal(x.grad.cpu().numpy(), ref)
+    x = torch.from_numpy(feats).to(device).requires_grad_(True)
+    (global_maxpool(x, offs) * torch.from_numpy(g).to(device))[[0, 2, 3]].sum().backward()
+    _, arg = oracle.segment_max(feats, offsets)
+    g_used = g.copy()
+    g_used[1] = 0  # the empty segment's output (-inf) is left out of the loss
+    assert np.array_equal(x.grad.cpu().numpy(), oracle.segment_max_bwd(g_used, arg, n))
+    # voxel mean
+    inverse = rng.integers(0, 60, size=n).astype(np.int32)
+    inverse[:60] = np.arange(60)
+    counts = np.bincount(inverse, minlength=60)
+    maps = oracle.voxel_map(inverse, 60, int(counts.max()), 4)
+    gv = rng.normal(size=(60, c)).astype(np.float32)
+    x = torch.from_numpy(feats).to(device).requires_grad_(True)
+    y = voxelization(x, torch.from_numpy(maps).to(device), 4)
+    (y * torch.from_numpy(gv).to(device)).sum().backward()
+    assert np.array_equal(x.grad.cpu().numpy(), oracle.voxel_reduce_bwd(gv, maps, 4, n))
+    # interpolation (atomic accumulation: tolerance, not bit equality)
+    m, q = 90, 400
+    vf = rng.normal(size=(m, c)).astype(np.float32)
+    idx3 = rng.integers(0, m, size=(q, 3)).astype(np.int32)
+    w3 = rng.uniform(size=(q, 3)).astype(np.float32)
+    gq = rng.normal(size=(q, c)).astype(np.float32)
+    x = torch.from_numpy(vf).to(device).requires_grad_(True)
+    y = three_interpolate(x, torch.from_numpy(idx3).to(device), torch.from_numpy(w3).to(device))
+    (y * torch.from_numpy(gq).to(device)).sum().backward()
+    assert rel_l2(x.grad.cpu().numpy(), oracle.three_interp_bwd(gq, idx3, w3, m)) < REL_L2
+
+
 def test_downsampling_block(oracle, device):
     """Strided convolution followed by MaxPool and AvgPool (k=2, s=2)."""
     import torch.nn.functional as F
@@ -525,6 +591,48 @@ def test_downsampling_block(oracle, device):
     dy = y.dense().cpu()
     assert rel_l2(mx.dense().cpu().numpy(), F.max_pool3d(F.relu(dy), 2, 2).numpy()) < 1e-6
     assert rel_l2(av.dense().cpu().numpy(), F.avg_pool3d(dy, 2, 2).numpy()) < 1e-6
+
+
+def test_training_step_end_to_end(device):
+    """Point2Voxel -> Convolution -> BatchNorm -> ReLU -> strided Convolution -> MaxPool ->
+    GlobalAvgPool + Voxel2Point, loss.backward(), one SGD step: every parameter receives
+    a finite gradient and the loss of the same batch goes down."""
+    from ss_conv.batchnorm import BatchNorm
+    from ss_conv.convolution import Convolution
+    from ss_conv.pool import MaxPool, GlobalAvgPool
+    from ss_conv.sp_ops.voxelize import Point2Voxel, Voxel2Point
+    torch.manual_seed(3)
+    rs_in = [(4, 0)]
+    rs_conv = [(12, 0)]  # scalar fields only, so that a plain ReLU is equivariant
+    pts, feats, ids = synth.make_clouds(2, 400, seed=12, channels=4)
+    grid = 12
+    conv = Convolution(rs_in, rs_conv, 3, stride=1, padding=1).to(device)
+    bn = BatchNorm(rs_conv).to(device)
+    conv2 = Convolution(rs_conv, [(8, 0)], 3, stride=2, padding=1).to(device)
+    params = list(conv.parameters()) + list(bn.parameters()) + list(conv2.parameters())
+    opt = torch.optim.SGD(params, lr=1e-2)
+    dp, df, di = [torch.from_numpy(x).to(device) for x in (pts, feats, ids)]
+    target = torch.randn(2, 8, device=device)
+
+    def loss_fn():
+        vp, st, vi, _ = Point2Voxel([grid] * 3, [2.0 / grid] * 3)(dp, df.clone().requires_grad_(True), di)
+        y = bn(conv(st))
+        y.features = torch.relu(y.features)
+        y = MaxPool(2, 2)(conv2(y))
+        pooled = GlobalAvgPool()(y)
+        back = Voxel2Point(unit_voxel_extent=[2.0 / 3] * 3)(y, vp, vi)
+        return ((pooled - target) ** 2).mean() + 1e-3 * (back ** 2).mean()
+
+    conv.train(); conv2.train(); bn.train()
+    l0 = loss_fn()
+    opt.zero_grad()
+    l0.backward()
+    for p in params:
+        assert p.grad is not None and torch.isfinite(p.grad).all()
+    assert float(conv.kernel.weight.grad.abs().sum()) > 0
+    opt.step()
+    l1 = loss_fn()
+    assert l1.item() < l0.item()
 
 
 def test_cpu_tensor_is_rejected(device):

@@ -131,6 +131,77 @@ def test_pools_equal_dense_pools(k, s, p, oracle):
         assert np.array_equal(mx, oracle.ref_maxpool_fwd(feats, pairs, num, o_idx.shape[0]))
 
 
+@pytest.mark.parametrize("k,s,p", [(2, 2, 0), (3, 2, 1), (3, 1, 1)])
+def test_pool_backward_equals_dense_autograd(k, s, p, oracle):
+    """Backward of avg pooling equals autograd through F.avg_pool3d; backward of max pooling
+    equals autograd through F.max_pool3d(relu(.)) on data without ties (every positive
+    window maximum unique)."""
+    rng = np.random.default_rng(13)
+    batch, grid, n, c = 2, 8, 150, 3
+    idx = random_voxels(rng, batch, grid, n)
+    feats = rng.normal(size=(n, c)).astype(np.float32)
+    o_idx, pairs, num, shape = oracle.rulebook(idx, batch, [grid] * 3, k, s, p)
+    g_out = rng.normal(size=(o_idx.shape[0], c)).astype(np.float32)
+    t = torch.from_numpy(o_idx).long()
+
+    x = dense(idx, feats, batch, grid).requires_grad_(True)
+    y = F.avg_pool3d(x, k, s, p, count_include_pad=True)
+    go = torch.zeros_like(y)
+    go[t[:, 0], :, t[:, 1], t[:, 2], t[:, 3]] = torch.from_numpy(g_out).double()
+    y.backward(go)
+    rf = np.full(o_idx.shape[0], k ** 3, dtype=np.int32)
+    got = oracle.avgpool_bwd(g_out, pairs, num, n, rf)
+    assert np.allclose(got, at_rows(x.grad, idx), atol=1e-6)
+
+    x = dense(idx, feats, batch, grid).requires_grad_(True)
+    y = F.max_pool3d(torch.relu(x), k, s, p)
+    y.backward(go)
+    pooled = oracle.maxpool_fwd(feats, pairs, num, o_idx.shape[0])
+    got = oracle.maxpool_bwd(feats, pooled, g_out, pairs, num)
+    # inputs <= 0 never equal a positive maximum; where the window maximum is 0 (all
+    # inputs negative) neither side passes a gradient to a real input
+    assert np.allclose(got, at_rows(x.grad, idx), atol=1e-6)
+
+
+def test_segment_and_voxel_backward(oracle):
+    """Segment pools, voxel mean and interpolation backward against torch autograd."""
+    rng = np.random.default_rng(17)
+    n, c = 40, 3
+    feats = rng.normal(size=(n, c)).astype(np.float32)
+    offsets = np.array([0, 7, 7, 25, 40], dtype=np.int32)
+    g = rng.normal(size=(4, c)).astype(np.float32)
+    x = torch.from_numpy(feats).double().requires_grad_(True)
+    segs = [x[a:b] for a, b in zip(offsets[:-1], offsets[1:])]
+    mean = torch.stack([s.mean(0) if len(s) else torch.zeros(c, dtype=torch.float64) for s in segs])
+    (mean * torch.from_numpy(g).double()).sum().backward()
+    assert np.allclose(oracle.segment_avg_bwd(g, offsets, n), x.grad.numpy(), atol=1e-6)
+    x.grad = None
+    mx = torch.stack([s.max(0)[0] if len(s) else torch.zeros(c, dtype=torch.float64) for s in segs])
+    (mx * torch.from_numpy(g).double()).sum().backward()
+    _, arg = oracle.segment_max(feats, offsets)
+    assert np.allclose(oracle.segment_max_bwd(g, arg, n), x.grad.numpy(), atol=1e-6)
+    # voxel mean: 3 voxels over 7 points
+    inverse = np.array([0, 2, 0, 1, 2, 2, 0], dtype=np.int32)
+    maps = oracle.voxel_map(inverse, 3, 3, 4)
+    pf = rng.normal(size=(7, c)).astype(np.float32)
+    gv = rng.normal(size=(3, c)).astype(np.float32)
+    x = torch.from_numpy(pf).double().requires_grad_(True)
+    vm = torch.stack([x[torch.from_numpy(np.nonzero(inverse == v)[0])].mean(0) for v in range(3)])
+    (vm * torch.from_numpy(gv).double()).sum().backward()
+    assert np.allclose(oracle.voxel_reduce_bwd(gv, maps, 4, 7), x.grad.numpy(), atol=1e-6)
+    # interpolation
+    m, q = 9, 20
+    vf = rng.normal(size=(m, c)).astype(np.float32)
+    idx3 = rng.integers(0, m, size=(q, 3)).astype(np.int32)
+    w3 = rng.uniform(size=(q, 3)).astype(np.float32)
+    gq = rng.normal(size=(q, c)).astype(np.float32)
+    x = torch.from_numpy(vf).double().requires_grad_(True)
+    out = sum(x[torch.from_numpy(idx3[:, j]).long()] * torch.from_numpy(w3[:, j:j + 1]).double()
+              for j in range(3))
+    (out * torch.from_numpy(gq).double()).sum().backward()
+    assert np.allclose(oracle.three_interp_bwd(gq, idx3, w3, m), x.grad.numpy(), atol=1e-5)
+
+
 def test_segment_pools(oracle):
     rng = np.random.default_rng(5)
     lens = [4, 1, 33, 7]
