@@ -593,6 +593,48 @@ def test_downsampling_block(oracle, device):
     assert rel_l2(av.dense().cpu().numpy(), F.avg_pool3d(dy, 2, 2).numpy()) < 1e-6
 
 
+def test_submanifold_reuse_and_inverse(oracle, device):
+    """subm=True keeps the active set (dense conv3d sampled at the input sites), layers
+    sharing an indice_key reuse one rulebook, and an inverse convolution maps a strided
+    layer's output back onto the sites of its input (sp_ops/conv.py:124-136)."""
+    import torch.nn.functional as F
+    from ss_conv.convolution import Convolution
+    from ss_conv.sp_ops.tensor import SparseTensor
+    torch.manual_seed(4)
+    rng = np.random.default_rng(8)
+    grid, n = 10, 300
+    idx = random_voxels(rng, 2, grid, n)
+    rs = [(4, 0), (2, 1)]
+    feats = torch.from_numpy(rng.normal(size=(n, 10)).astype(np.float32)).to(device)
+    x = SparseTensor(feats, torch.from_numpy(idx).to(device), [grid] * 3, 2)
+    a = Convolution(rs, rs, 3, padding=1, subm=True, indice_key="s1").to(device).eval()
+    b = Convolution(rs, rs, 3, padding=1, subm=True, indice_key="s1").to(device).eval()
+    with torch.no_grad():
+        y = a(x)
+        assert list(x.indice_dict.keys()) == ["s1"]
+        pairs_first = x.indice_dict["s1"][2]
+        z = b(y)
+        assert z.indice_dict["s1"][2] is pairs_first  # the rulebook was not rebuilt
+    assert torch.equal(y.indices, x.indices) and torch.equal(z.indices, x.indices)
+    want = F.conv3d(x.dense().cpu().double(), a.kernel().detach().cpu().double(), padding=1)
+    t = torch.from_numpy(idx).long()
+    assert rel_l2(y.features.cpu().numpy(), want[t[:, 0], :, t[:, 1], t[:, 2], t[:, 3]].numpy()) \
+        < REL_L2
+    # strided layer and its inverse
+    down = Convolution(rs, rs, 3, stride=2, padding=1, indice_key="d1").to(device).eval()
+    up = Convolution(rs, rs, 3, indice_key="d1", inverse=True).to(device).eval()
+    with torch.no_grad():
+        d = down(z)
+        u = up(d)
+    assert torch.equal(u.indices, x.indices) and list(u.spatial_shape) == [grid] * 3
+    # the inverse convolution is the transpose of the strided one over the same pairs
+    o_idx, o_pairs, o_num = oracle.canonicalize(*oracle.rulebook(idx, 2, [grid] * 3, 3, 2, 1))
+    w_up = up.kernel().detach().permute(2, 3, 4, 1, 0).reshape(27, 10, 10).cpu().numpy()
+    ref = oracle.conv_fwd(d.features.cpu().numpy(), w_up, o_pairs, o_num, n, inverse=True,
+                          matmul=np.matmul)
+    assert rel_l2(u.features.cpu().numpy(), ref) < REL_L2
+
+
 def test_training_step_end_to_end(device):
     """Point2Voxel -> Convolution -> BatchNorm -> ReLU -> strided Convolution -> MaxPool ->
     GlobalAvgPool + Voxel2Point, loss.backward(), one SGD step: every parameter receives
