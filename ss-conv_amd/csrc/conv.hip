@@ -254,8 +254,11 @@ __global__ void __launch_bounds__(256)
 //                               the row number, or the byte offset of the row
 //   sched_out[group*64 + slot]  byte offset of the slot's accumulator row in the tile
 //                               (tile-local row * out_scale; row T, a dummy, = padding)
-//   grp_meta [group*8 + ...]    0..3 offset k of the 4 blocks (-1 = empty block),
-//                               4 tile of the group, 5 1 when it is the tile's last group
+//   grp_meta [group*8 + ...]    0..3 offset k of the 4 blocks times k_scale (the byte
+//                               distance between the weight fragments of two offsets;
+//                               an empty block has 0), 4 first output row of the
+//                               group's tile, 5 rows of the tile, negated when the
+//                               group is not the tile's last one
 // The convolution kernel streams through it without per-offset bookkeeping.
 __global__ void __launch_bounds__(256)
     sched_count_kernel(const int32_t *__restrict__ segs, int K,
@@ -316,8 +319,9 @@ __global__ void __launch_bounds__(256)
                       const int32_t *__restrict__ tile_nmb, const int32_t *__restrict__ tile_grp,
                       int K, const int32_t *__restrict__ n_tiles_dev,
                       const int32_t *__restrict__ tile_row0, int T, uint32_t in_scale,
-                      uint32_t in_pad, int out_scale, int32_t *__restrict__ sched_in,
-                      int32_t *__restrict__ sched_out, int32_t *__restrict__ grp_meta) {
+                      uint32_t in_pad, int out_scale, int k_scale,
+                      int32_t *__restrict__ sched_in, int32_t *__restrict__ sched_out,
+                      int32_t *__restrict__ grp_meta) {
   int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   int64_t tk = gid >> 4;
   int lane = (int)(gid & 15);
@@ -327,15 +331,16 @@ __global__ void __launch_bounds__(256)
   const int64_t g0 = tile_grp[t], g1 = tile_grp[t + 1];
   if (k == 0) {
     for (int64_t g = g0 + lane; g < g1; g += 16) {
-      grp_meta[g * 8 + 4] = (int32_t)t;
-      grp_meta[g * 8 + 5] = g + 1 == g1 ? 1 : 0;
+      const int rows = tile_row0[t + 1] - tile_row0[t];
+      grp_meta[g * 8 + 4] = tile_row0[t];
+      grp_meta[g * 8 + 5] = g + 1 == g1 ? rows : -rows;
       grp_meta[g * 8 + 6] = 0;
       grp_meta[g * 8 + 7] = 0;
     }
     for (int64_t mb = g0 * 4 + tile_nmb[t]; mb < g1 * 4; ++mb) {
       sched_in[mb * 16 + lane] = (int32_t)in_pad;
       sched_out[mb * 16 + lane] = T * out_scale;
-      if (lane == 0) grp_meta[(mb >> 2) * 8 + (mb & 3)] = -1;
+      if (lane == 0) grp_meta[(mb >> 2) * 8 + (mb & 3)] = 0;
     }
   }
   const int32_t *src = flag[0] ? sorted : pairs;
@@ -349,7 +354,7 @@ __global__ void __launch_bounds__(256)
   for (int p = lane; p < ((n + 15) & ~15); p += 16, ++mb) {
     sched_in[mb * 16 + lane] = p < n ? (int32_t)((uint32_t)pg[p] * in_scale) : (int32_t)in_pad;
     sched_out[mb * 16 + lane] = (p < n ? (int)(ps[p] - row0) : T) * out_scale;
-    if (lane == 0) grp_meta[(mb >> 2) * 8 + (mb & 3)] = k;
+    if (lane == 0) grp_meta[(mb >> 2) * 8 + (mb & 3)] = k * k_scale;
   }
 }
 
@@ -399,15 +404,12 @@ constexpr int kIdxAhead = 2;   // further stages whose gather offsets are in fli
 constexpr unsigned kGatherPad = 0xFFFFF000u;  // byte offset that gathers zeros (beyond any feature buffer)
 constexpr int kRsrcFlags = 0x00020000;        // raw buffer of 32-bit data
 
-__device__ __forceinline__ void mfma_quad(const float4v &b, const float4v &a, float4v &d) {
-  d = __builtin_amdgcn_mfma_f32_16x16x4f32(b.x, a.x, d, 0, 0, 0);
-  d = __builtin_amdgcn_mfma_f32_16x16x4f32(b.y, a.y, d, 0, 0, 0);
-  d = __builtin_amdgcn_mfma_f32_16x16x4f32(b.z, a.z, d, 0, 0, 0);
-  d = __builtin_amdgcn_mfma_f32_16x16x4f32(b.w, a.w, d, 0, 0, 0);
-}
-
 __device__ __forceinline__ float4v buf_load4(__amdgpu_buffer_rsrc_t r, int voff, int soff) {
   return __builtin_bit_cast(float4v, __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, 0));
+}
+typedef int int2v __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ int2v buf_load2(__amdgpu_buffer_rsrc_t r, int voff, int soff) {
+  return __builtin_bit_cast(int2v, __builtin_amdgcn_raw_buffer_load_b64(r, voff, soff, 0));
 }
 __device__ __forceinline__ int buf_load1(__amdgpu_buffer_rsrc_t r, int voff, int soff) {
   return (int)__builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, 0);
@@ -445,8 +447,7 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
                     const int32_t *__restrict__ sched_in, const int32_t *__restrict__ sched_out,
                     const int32_t *__restrict__ grp_meta, unsigned sched_bytes, unsigned meta_bytes,
                     const int32_t *__restrict__ tile_grp, const int32_t *__restrict__ wg_tile,
-                    const int32_t *__restrict__ tile_row0, int nch, int ncb, int kvol,
-                    float *__restrict__ out, int cout, int T) {
+                    int nch, int ncb, float *__restrict__ out, int cout, int T) {
   constexpr int kCN = 16 * NCW;   // output columns per workgroup
   constexpr int kAS = kCN + 4;    // accumulator row stride in floats
   constexpr int NT = (NCW + 4) * 64;
@@ -480,21 +481,38 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
   }
 
   // Tile `tl` is complete: write its rows, clear the accumulators.
-  auto flush_tile = [&](int tl) {
-    const int row0 = tile_row0[tl];
-    const int rows = tile_row0[tl + 1] - row0;
+  auto flush_tile = [&](int row0, int rows) {
     if ((cout & 3) == 0) {
+      // A thread keeps its 4 columns and walks down the rows, NT / (kCN / 4) rows per
+      // step: addresses advance by constants, so a step is little more than its LDS
+      // read, LDS clear and store, and four reads are in flight before the first store
+      // (one at a time, every step would pay the full LDS latency while the matrix
+      // cores idle).
       const float4v z = {0.f, 0.f, 0.f, 0.f};
-      for (int e = tid; e < rows * (kCN / 4); e += NT) {
-        int r = e / (kCN / 4), c4 = e % (kCN / 4);
-        int col = col0 + c4 * 4;
-        float4v *ap = reinterpret_cast<float4v *>(acc + r * kAS + c4 * 4);
-        // streaming store: the output is not read again by this kernel and must not
-        // push the weights and the gathered rows out of L2
-        if (col < cout)
-          __builtin_nontemporal_store(
-              *ap, reinterpret_cast<float4v *>(out + (int64_t)(row0 + r) * cout + col));
-        *ap = z;
+      constexpr int U = 4;
+      constexpr int RS = NT / (kCN / 4);  // rows per step
+      const int r_t = tid / (kCN / 4), c_t = (tid % (kCN / 4)) * 4;
+      const bool col_ok = col0 + c_t < cout;
+      float *lp = acc + r_t * kAS + c_t;
+      float *gp = out + (int64_t)(row0 + r_t) * cout + col0 + c_t;
+      const int64_t gstep = (int64_t)RS * cout;
+      for (int r = r_t; r < rows; r += U * RS) {
+        float4v v[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+          if (r + u * RS < rows) {
+            float4v *ap = reinterpret_cast<float4v *>(lp + u * RS * kAS);
+            v[u] = *ap;
+            *ap = z;
+          }
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+          // streaming store: the output is not read again by this kernel and must not
+          // push the weights and the gathered rows out of L2
+          if (r + u * RS < rows && col_ok)
+            __builtin_nontemporal_store(v[u], reinterpret_cast<float4v *>(gp + u * gstep));
+        lp += U * RS * kAS;
+        gp += U * gstep;
       }
     } else {
       for (int e = tid; e < rows * kCN; e += NT) {
@@ -505,12 +523,15 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
       }
     }
   };
-  // The tile of stage `pos` ends with it when the group is the tile's last one and
-  // the chunk is the last chunk.  Scalar loads: the address is uniform.
-  auto tile_end = [&](const StagePos &pos, int &tile) -> bool {
+  // The tile of stage `pos` (first row, rows) ends with it when the group is the
+  // tile's last one and the chunk is the last chunk.  Scalar loads: the address is
+  // uniform.
+  auto tile_end = [&](const StagePos &pos, int &row0, int &rows) -> bool {
     const int32_t *m = grp_meta + (int64_t)pos.g * 8;
-    tile = m[4];
-    return m[5] != 0 && pos.cc == nch - 1;
+    row0 = m[4];
+    const int r = m[5];
+    rows = r < 0 ? -r : r;
+    return r > 0 && pos.cc == nch - 1;
   };
 
   if (producer) {
@@ -606,8 +627,8 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
     // (rows) and s+7 (gather offsets).
     auto iteration = [&](int s, auto phase) {
       constexpr int ph = decltype(phase)::value;  // == s & 3
-      int tile;
-      const bool last = tile_end(p_cur, tile);
+      int t_row0, t_rows;
+      const bool last = tile_end(p_cur, t_row0, t_rows);
       p_cur.advance(nch);
       store_rows((ph + 1) & 1, rows[(ph + 1) & 3]);
       load_rows(p_rows, idx[(ph + 1 + RD) & 1], rows[(ph + 1 + RD) & 3]);
@@ -616,19 +637,24 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
       p_idx.advance(nch);
       __syncthreads();
       if (last) {
-        flush_tile(tile);
+        flush_tile(t_row0, t_rows);
         __syncthreads();
       }
     };
-    for (int s = 0; s < nstages; s += 4) {
+    // Whole groups of four stages first, the remainder after the loop: an early exit
+    // from the middle of the unrolled body would share the loop's back edge, and the
+    // static wait counts at the top of the body would then have to allow for a trip
+    // that follows a shorter one.
+    int s = 0;
+    for (; s + 4 <= nstages; s += 4) {
       iteration(s, std::integral_constant<int, 0>());
-      if (s + 1 >= nstages) break;
       iteration(s + 1, std::integral_constant<int, 1>());
-      if (s + 2 >= nstages) break;
       iteration(s + 2, std::integral_constant<int, 2>());
-      if (s + 3 >= nstages) break;
       iteration(s + 3, std::integral_constant<int, 3>());
     }
+    if (s < nstages) iteration(s, std::integral_constant<int, 0>());
+    if (s + 1 < nstages) iteration(s + 1, std::integral_constant<int, 1>());
+    if (s + 2 < nstages) iteration(s + 2, std::integral_constant<int, 2>());
   } else {
     // ------------------------------------------------------------------ consumer
     const int g = lane >> 4;
@@ -642,7 +668,6 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
         __builtin_amdgcn_make_buffer_rsrc((void *)sched_out, 0, (int)sched_bytes, kRsrcFlags);
     const int w_voff = lane * 64;           // this lane's 16 floats of a fragment
     const int w_soff0 = cb * nch * 4096;    // fragments of this wave's column block
-    const int frag_k = ncb * nch * 4096;    // bytes between the fragments of two offsets
     const int acc_lane = (wave * 16 + g * 4) * 4;  // byte offset of this lane's 4 columns
     const float *const a_base = abuf + l16 * kAStride + g * 16;
     char *const acc_bytes = reinterpret_cast<char *>(acc);
@@ -657,7 +682,7 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
     //                 blocks ahead: while block b multiplies, the slot of block b-1 is
     //                 refilled for block b+3
     //   orow[b & 3]   LDS byte offset of the accumulator row of this lane's pair in block b
-    //   rec[s & 1]    the schedule record (offsets of the 4 blocks, tile, last-of-tile)
+    //   rec[s & 1]    the schedule record (offsets of the 4 blocks, rows of the tile)
     //                 of stage s, the same in every lane.  It travels through vector
     //                 loads and v_readfirstlane rather than scalar loads: scalar loads
     //                 return out of order, and one in flight would turn every partial
@@ -665,17 +690,36 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
     float4v w[4][4];
     int orow[4];
     int4v rec[2][2];
+    // Second half of a record: only its first two words are used.  An 8-byte load:
+    // a wider one would still write the two unused registers when it lands, and
+    // whatever the compiler keeps there in the meantime would have to wait for it.
+    auto load_rec_tail = [&](const StagePos &pos) -> int4v {
+      const int2v t = buf_load2(rs_meta, 16, pos.g * 32);
+      return int4v{t.x, t.y, 0, 0};
+    };
+    // First row and rows of the tile of a stage, and whether the tile ends with the
+    // stage, from the second half of its record.
+    struct TileEnd {
+      int row0, rows;
+      bool last;
+    };
+    auto tile_end_of = [&](const int4v &tail, const StagePos &pos) -> TileEnd {
+      TileEnd e;
+      e.row0 = __builtin_amdgcn_readfirstlane(tail.x);
+      const int r = __builtin_amdgcn_readfirstlane(tail.y);
+      e.rows = r < 0 ? -r : r;
+      e.last = r > 0 && pos.cc == nch - 1;
+      return e;
+    };
     auto load_rec = [&](const StagePos &pos, int4v (&r)[2]) {
       r[0] = __builtin_bit_cast(int4v, buf_load4(rs_meta, 0, pos.g * 32));
-      r[1] = __builtin_bit_cast(int4v, buf_load4(rs_meta, 16, pos.g * 32));
+      r[1] = load_rec_tail(pos);
     };
-    // Byte offset of the weight fragments of a block at offset k (from a schedule
-    // record, possibly garbage beyond the schedule) and channel chunk cc.
-    auto frag_soff = [&](int k_lane, int cc) -> int {
-      const int k = __builtin_amdgcn_readfirstlane(k_lane);
-      // empty blocks (-1) and records beyond the schedule use the fragments of offset 0
-      const int kk = (k < 0 || k >= kvol) ? 0 : k;
-      return w_soff0 + kk * frag_k + cc * 4096;
+    // Byte offset of the weight fragments of a block: the offset's part comes from the
+    // schedule record (0 for empty blocks and, the loads being range-checked, for
+    // records beyond the schedule), `base` is the part of this wave and channel chunk.
+    auto frag_soff = [&](int rec_lane, int base) -> int {
+      return __builtin_amdgcn_readfirstlane(rec_lane) + base;
     };
     auto rec_k = [](const int4v &v, int b) -> int {
       return b == 0 ? v.x : b == 1 ? v.y : b == 2 ? v.z : v.w;
@@ -697,69 +741,82 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
     pend.addr = dummy_addr;
     pend.accr = float4v{0.f, 0.f, 0.f, 0.f};
     pend.d = float4v{0.f, 0.f, 0.f, 0.f};
-    // One stage = 4 row blocks, software-pipelined by hand.  In program order:
-    //   the staged rows of block m+1 are read BEFORE the chain of block m starts;
-    //   the accumulator update of the previous block (add, write) and the accumulator
-    //   read of block m sit AFTER the first four MFMAs of block m, in the shadow of
-    //   the chain -- the update of a stage's last block waits, across the barrier,
-    //   for the first block of the next stage, unless the tile ends here;
-    //   the loads for block b+3 (and, once per stage, the record of the stage after
-    //   the next) are spread over the four groups of four MFMAs of block b: a
-    //   16-byte-per-lane load keeps the wave in the issue stage for tens of cycles,
-    //   which is free behind an MFMA whose successor must wait for it anyway.
-    // Scheduling barriers pin that order (the compiler otherwise moves the LDS reads
-    // next to their first use to shorten live ranges).  LDS operations of a wave
-    // execute in order, so the read of block m's rows after the write of block m-1
-    // sees that write when both blocks touch the same output row.
+    // One stage = 4 row blocks of 16 MFMAs each, software-pipelined by hand.  A wave
+    // issues at most one instruction every few cycles, and a dependent MFMA can only
+    // issue when its predecessor is through the pipeline, so between two MFMAs of a
+    // chain a handful of other instructions issue for free -- and no more than that:
+    // everything else a block needs is therefore spread, one small piece per gap,
+    // over the 16 gaps of the block, and scheduling barriers pin it there:
+    //   gap 0      fragment offset of block b+3 (from the schedule record)
+    //   gaps 1,4,8,12  the four fragment loads of block b+3 (the slot of block b-1)
+    //   gap 2      accumulator update of the previous block: add, write
+    //   gap 3      accumulator read of this block (LDS operations of a wave execute
+    //              in order, so it sees the write of gap 2 when both blocks touch
+    //              the same output row)
+    //   gap 5      output rows of block b+3
+    //   gaps 6,7,9,10  the staged rows of block m+1
+    //   gaps 11,13 once per stage: the record of the stage after the next; tile and
+    //              last-of-tile of the next stage
+    // The update of a stage's last block waits, across the barrier, for the first
+    // block of the next stage, unless the tile ends here.
     //   cur / next / after: positions of this stage and the two that follow;
-    //   returns tile and last-of-tile of the NEXT stage.
+    //   returns the tile rows and last-of-tile of the NEXT stage.
     auto run_stage = [&](auto parity, bool last_cur, const StagePos &cur, const StagePos &next,
-                         const StagePos &after, int &tile_next, bool &last_next) {
+                         const StagePos &after, TileEnd &end_next) {
       constexpr int par = decltype(parity)::value;
       const float *ab = a_base + par * kStage * kAStride;
+      const int base_cur = w_soff0 + cur.cc * 4096;
+      const int base_next = w_soff0 + next.cc * 4096;
       float4v a[2][4];
-      auto load_a = [&](int m, float4v (&av)[4]) {
-        const float4v *ap = reinterpret_cast<const float4v *>(ab + m * 16 * kAStride);
-#pragma unroll
-        for (int q = 0; q < 4; ++q) av[q] = ap[q];
+      auto load_a = [&](int m, int q, float4v (&av)[4]) {
+        av[q] = reinterpret_cast<const float4v *>(ab + m * 16 * kAStride)[q];
       };
-      load_a(0, a[0]);
+#pragma unroll
+      for (int q = 0; q < 4; ++q) load_a(0, q, a[0]);
 #pragma unroll
       for (int m = 0; m < 4; ++m) {
         const int slot = m;                 // == (4 * s + m) & 3
         const int tslot = (m + 3) & 3;      // slot of block b+3 == slot of block b-1
         const int tm = (m + 3) & 3;         // index of block b+3 inside its stage
         const bool tnext = m > 0;           // block b+3 belongs to the next stage
-        if (m < 3) load_a(m + 1, a[(m + 1) & 1]);
-        __builtin_amdgcn_sched_barrier(0);
         float4v d = float4v{0.f, 0.f, 0.f, 0.f};
-        mfma_quad(w[slot][0], a[m & 1][0], d);
-        __builtin_amdgcn_sched_barrier(0);
-        const int soff = tnext ? frag_soff(rec_k(rec[par ^ 1][0], tm), next.cc)
-                               : frag_soff(rec_k(rec[par][0], tm), cur.cc);
-        fetch_w(soff, tslot, 0);
-        // pend.d = out[pair l16][channels 4g .. 4g+3] of the previous block
-        *reinterpret_cast<float4v *>(acc_bytes + pend.addr) = pend.accr + pend.d;
-        pend.addr = orow[slot] + acc_lane;
-        pend.accr = *reinterpret_cast<const float4v *>(acc_bytes + pend.addr);
-        __builtin_amdgcn_sched_barrier(0);
+        int soff = 0;
 #pragma unroll
-        for (int q = 1; q < 4; ++q) {
-          mfma_quad(w[slot][q], a[m & 1][q], d);
+        for (int i = 0; i < 16; ++i) {
+          const int q = i >> 2, j = i & 3;
           __builtin_amdgcn_sched_barrier(0);
-          fetch_w(soff, tslot, q);
-          if (q == 1) fetch_orow(tnext ? next : cur, tm, tslot);
+          d = __builtin_amdgcn_mfma_f32_16x16x4f32(w[slot][q][j], a[m & 1][q][j], d, 0, 0, 0);
+          __builtin_amdgcn_sched_barrier(0);
+          if (i == 0)
+            soff = tnext ? frag_soff(rec_k(rec[par ^ 1][0], tm), base_next)
+                         : frag_soff(rec_k(rec[par][0], tm), base_cur);
+          if (i == 1) fetch_w(soff, tslot, 0);
+          if (i == 2)  // pend.d = out[pair l16][channels 4g .. 4g+3] of the previous block
+            *reinterpret_cast<float4v *>(acc_bytes + pend.addr) = pend.accr + pend.d;
+          if (i == 3) {
+            pend.addr = orow[slot] + acc_lane;
+            pend.accr = *reinterpret_cast<const float4v *>(acc_bytes + pend.addr);
+          }
+          if (i == 4) fetch_w(soff, tslot, 1);
+          if (i == 5) fetch_orow(tnext ? next : cur, tm, tslot);
+          if (m < 3) {
+            if (i == 6) load_a(m + 1, 0, a[(m + 1) & 1]);
+            if (i == 7) load_a(m + 1, 1, a[(m + 1) & 1]);
+            if (i == 9) load_a(m + 1, 2, a[(m + 1) & 1]);
+            if (i == 10) load_a(m + 1, 3, a[(m + 1) & 1]);
+          }
+          if (i == 8) fetch_w(soff, tslot, 2);
+          if (i == 12) fetch_w(soff, tslot, 3);
           // this stage's record was last used by block 0: refill it for the stage
           // after the next
-          if (m == 1 && q >= 2) rec[par][q - 2] = __builtin_bit_cast(
-              int4v, buf_load4(rs_meta, (q - 2) * 16, after.g * 32));
-          if (m == 3 && q == 3) {
-            tile_next = __builtin_amdgcn_readfirstlane(rec[par ^ 1][1].x);
-            last_next =
-                __builtin_amdgcn_readfirstlane(rec[par ^ 1][1].y) != 0 && next.cc == nch - 1;
+          if (m == 1 && i == 11)
+            rec[par][0] = __builtin_bit_cast(int4v, buf_load4(rs_meta, 0, after.g * 32));
+          if (m == 1 && i == 13) rec[par][1] = load_rec_tail(after);
+          if (m == 3 && i == 13) {
+            end_next = tile_end_of(rec[par ^ 1][1], next);
           }
-          __builtin_amdgcn_sched_barrier(0);
         }
+        __builtin_amdgcn_sched_barrier(0);
         pend.d = d;
       }
       __builtin_amdgcn_sched_barrier(0);
@@ -774,52 +831,53 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
     p_next.advance(nch);
     p_after.advance(nch);
     p_after.advance(nch);
-    int tile, tile_next;
-    bool last, last_next;
+    TileEnd end, end_next;
     {
       // what the first stage needs before it starts: its record and the next one,
       // fragments and rows of its blocks 0..2
       load_rec(p_cur, rec[0]);
       load_rec(p_next, rec[1]);
-      tile = __builtin_amdgcn_readfirstlane(rec[0][1].x);
-      last = __builtin_amdgcn_readfirstlane(rec[0][1].y) != 0 && p_cur.cc == nch - 1;
+      end = tile_end_of(rec[0][1], p_cur);
+      // Loads are issued in the order of the loop (fragments 0 and 1, the output rows,
+      // fragments 2 and 3, block after block) and pinned there: the wait counts of the
+      // loop are static and must hold on its first trip as well, so a load that the
+      // prologue issued late would make every trip wait for nearly all loads in flight.
 #pragma unroll
       for (int b = 0; b < 3; ++b) {
-        const int soff = frag_soff(rec_k(rec[0][0], b), p_cur.cc);
-#pragma unroll
-        for (int q = 0; q < 4; ++q) fetch_w(soff, b, q);
+        const int soff = frag_soff(rec_k(rec[0][0], b), w_soff0 + p_cur.cc * 4096);
+        __builtin_amdgcn_sched_barrier(0);
+        fetch_w(soff, b, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        fetch_w(soff, b, 1);
+        __builtin_amdgcn_sched_barrier(0);
         fetch_orow(p_cur, b, b);
+        __builtin_amdgcn_sched_barrier(0);
+        fetch_w(soff, b, 2);
+        __builtin_amdgcn_sched_barrier(0);
+        fetch_w(soff, b, 3);
+        __builtin_amdgcn_sched_barrier(0);
       }
     }
     __syncthreads();
-    for (int s = 0; s < nstages; s += 2) {
-      run_stage(std::integral_constant<int, 0>(), last, p_cur, p_next, p_after, tile_next,
-                last_next);
+    auto step = [&](auto parity) {
+      run_stage(parity, end.last, p_cur, p_next, p_after, end_next);
       p_cur.advance(nch);
       p_next.advance(nch);
       p_after.advance(nch);
       __syncthreads();
-      if (last) {
-        flush_tile(tile);
+      if (end.last) {
+        flush_tile(end.row0, end.rows);
         __syncthreads();
       }
-      tile = tile_next;
-      last = last_next;
-      if (s + 1 < nstages) {
-        run_stage(std::integral_constant<int, 1>(), last, p_cur, p_next, p_after, tile_next,
-                  last_next);
-        p_cur.advance(nch);
-        p_next.advance(nch);
-        p_after.advance(nch);
-        __syncthreads();
-        if (last) {
-          flush_tile(tile);
-          __syncthreads();
-        }
-        tile = tile_next;
-        last = last_next;
-      }
+      end = end_next;
+    };
+    // pairs of stages first, an odd last stage after the loop (see the producer's loop)
+    int s = 0;
+    for (; s + 2 <= nstages; s += 2) {
+      step(std::integral_constant<int, 0>());
+      step(std::integral_constant<int, 1>());
     }
+    if (s < nstages) step(std::integral_constant<int, 0>());
   }
 }
 
@@ -948,7 +1006,7 @@ static int launch_conv(const ConvPlan &p, const ConvWs &w, const float *features
   hipLaunchKernelGGL((conv_fwd_kernel<GATHER, NCW>), grid, dim3((NCW + 4) * 64), p.lds_bytes, s, features, c_in,
                      feat_bytes, w.packed, (unsigned)packed_bytes, w.sched_in, w.sched_out,
                      w.grp_meta, (unsigned)sched_bytes, (unsigned)(p.grp_cap * 32), w.tile_grp,
-                     w.wg_tile, w.tile_row0, p.nch, p.ncb, K, out, c_out, p.T);
+                     w.wg_tile, p.nch, p.ncb, out, c_out, p.T);
   SSC_LAUNCH_CHECK("conv_fwd");
   return SSC_OK;
 }
@@ -1075,7 +1133,8 @@ int ssc_conv_fwd_f32(const float *features, int64_t n_in, int32_t c_in, const fl
                      dim3(256), 0, s, w.flag, pairs, w.sorted, pair_stride, plane_g, w.segs,
                      w.kofs, w.tile_nmb, w.tile_grp, K, w.n_tiles_dev, w.tile_row0, p.T,
                      p.gather ? (uint32_t)c_in * 4u : 1u, p.gather ? kGatherPad : 0xFFFFFFFFu,
-                     (16 * p.ncw + 4) * 4, w.sched_in, w.sched_out, w.grp_meta);
+                     (16 * p.ncw + 4) * 4, p.ncb * p.nch * 4096, w.sched_in, w.sched_out,
+                     w.grp_meta);
   SSC_LAUNCH_CHECK("schedule");
 
   const bool prof = g_profile_on;
