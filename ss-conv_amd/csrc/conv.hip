@@ -144,13 +144,17 @@ __global__ void __launch_bounds__(256)
 // tile t (t = 0..n_tiles).  Tile rows come from tile_row0[] and the tile count from
 // n_tiles_dev[0]; with tile_row0 == nullptr the tiles are `granule` rows each and
 // there are n_cap of them (the fine grid the work split is computed on).
+// With spill_end != nullptr also spill[t*K + k] = how far the last row block of tile
+// t-1 may reach into tile t: the first pair at or after segs[t*K + k], at most 15
+// further, whose row is >= spill_end[t].
 __global__ void __launch_bounds__(256)
     tile_segments_kernel(const int32_t *__restrict__ flag, const int32_t *__restrict__ pairs,
                          const int32_t *__restrict__ sorted, int64_t pair_stride, int plane_s,
                          const int32_t *__restrict__ pair_num, int K, int64_t n_cap,
                          const int32_t *__restrict__ n_tiles_dev,
                          const int32_t *__restrict__ tile_row0, int granule, int64_t n_out,
-                         int32_t *__restrict__ segs) {
+                         int32_t *__restrict__ segs, const int32_t *__restrict__ spill_end,
+                         int32_t *__restrict__ spill) {
   int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   const int64_t n_tiles = tile_row0 ? n_tiles_dev[0] : n_cap;
   if (idx >= (n_tiles + 1) * K) return;
@@ -167,6 +171,14 @@ __global__ void __launch_bounds__(256)
     else hi = mid;
   }
   segs[idx] = lo;
+  if (spill_end) {
+    const int bound = spill_end[t];
+    const int n = pair_num[k];
+    int cnt = 0;
+#pragma unroll
+    for (int j = 0; j < 15; ++j) cnt += (lo + j < n && s[lo + j] < bound) ? 1 : 0;  // rows ascend
+    spill[idx] = lo + cnt;
+  }
 }
 
 // ---- work split ------------------------------------------------------------------------
@@ -177,6 +189,13 @@ __global__ void __launch_bounds__(256)
 // kSplitGranule rows; range boundaries lie on that grid.  Each range is then cut
 // into tiles of equal height <= T.
 constexpr int kSplitGranule = 64;
+// The accumulator window of a workgroup holds kSpillRows more rows than a tile is
+// high: the last row block that an offset contributes to a tile may then be filled
+// up with the offset's next pairs, whose rows lie in the following tile (at most
+// kSpillRows into it), instead of being padded.  Rows map to accumulator slots
+// modulo the window height, so what such a block adds to the next tile's rows is
+// still there when that tile's turn comes.
+constexpr int kSpillRows = 128;
 
 // fine_work[b] = sum over offsets of fine_segs[b*K + k]  (pairs in rows < b*granule)
 __global__ void __launch_bounds__(256)
@@ -190,16 +209,21 @@ __global__ void __launch_bounds__(256)
 }
 
 // One block.  wg_tile[0..n_wg]: first tile of every workgroup; tile_row0[0..n_tiles]:
-// first row of every tile; n_tiles_dev[0]: number of tiles.
+// first row of every tile; n_tiles_dev[0]: number of tiles; spill_end[0..n_tiles]:
+// rows below spill_end[t] may be touched by the last row blocks of tile t-1 (the
+// first row of tile t itself when t starts a workgroup's range: no spill across
+// ranges); tile_slot0[t]: accumulator slot of the first row of tile t.  T is the
+// largest tile height, window the height of the accumulator window.
 __global__ void __launch_bounds__(256)
     split_rows_kernel(const int32_t *__restrict__ fine_work, int64_t nb, int64_t n_out, int T,
-                      int K, int n_wg, int32_t *__restrict__ wg_tile,
-                      int32_t *__restrict__ tile_row0, int32_t *__restrict__ n_tiles_dev) {
+                      int window, int K, int n_wg, int32_t *__restrict__ wg_tile,
+                      int32_t *__restrict__ tile_row0, int32_t *__restrict__ n_tiles_dev,
+                      int32_t *__restrict__ spill_end, int32_t *__restrict__ tile_slot0) {
   __shared__ int row_s[257];
   __shared__ int tile_s[257];
-  // cost of a tile beyond its pairs, in pair slots: half a row block of padding per
-  // offset, and about two stages' worth of time for writing it out
-  const int64_t tile_cost = (int64_t)K * 8 + 128;
+  // cost of a tile beyond its pairs, in pair slots: some padding per offset, and
+  // about two stages' worth of time for writing it out
+  const int64_t tile_cost = (int64_t)K * 2 + 128;
   auto work = [&](int64_t b) -> int64_t {
     int64_t r = b * kSplitGranule;
     if (r > n_out) r = n_out;
@@ -229,6 +253,7 @@ __global__ void __launch_bounds__(256)
     tile_s[n_wg] = run;
     n_tiles_dev[0] = run;
     tile_row0[run] = (int32_t)n_out;
+    spill_end[run] = (int32_t)n_out;
   }
   __syncthreads();
   for (int w = threadIdx.x; w <= n_wg; w += blockDim.x) {
@@ -238,37 +263,73 @@ __global__ void __launch_bounds__(256)
     const int nt = tile_s[w + 1] - tile_s[w];
     if (nt > 0) {
       const int h = (rows + nt - 1) / nt;
-      for (int j = 0; j < nt; ++j) tile_row0[tile_s[w] + j] = row_s[w] + j * h;
+      for (int j = 0; j < nt; ++j) {
+        const int r = row_s[w] + j * h;
+        tile_row0[tile_s[w] + j] = r;
+        spill_end[tile_s[w] + j] = j == 0 ? r : min(r + window - T, row_s[w + 1]);
+        tile_slot0[tile_s[w] + j] = (j * h) % window;
+      }
     }
   }
 }
 
 // ---- row-block schedule -----------------------------------------------------------------
-// The pairs that land in a tile are cut, offset by offset, into row blocks of 16
-// (the M side of one MFMA); the last block of an offset is padded.  Four
+// The pairs a tile works on (its share of every offset) are cut, offset by offset,
+// into row blocks of 16 (the M side of one MFMA); where the share could not be
+// filled up to a whole block, the last block is padded.  Four
 // consecutive row blocks form a group (one pipeline stage per 64-channel chunk
 // of Cin); a tile's last group is padded with empty blocks, and a tile without
 // pairs still gets one empty group so that its rows are written.  The schedule
 // lists, tile after tile and offset-major inside a tile:
 //   sched_in [group*64 + slot]  gather row of the slot times in_scale (in_pad = padding):
 //                               the row number, or the byte offset of the row
-//   sched_out[group*64 + slot]  byte offset of the slot's accumulator row in the tile
-//                               (tile-local row * out_scale; row T, a dummy, = padding)
+//   sched_out[group*64 + slot]  byte offset of the slot's accumulator row (accumulator
+//                               slot * out_scale; slot T, a dummy, = padding)
 //   grp_meta [group*8 + ...]    0..3 offset k of the 4 blocks times k_scale (the byte
 //                               distance between the weight fragments of two offsets;
 //                               an empty block has 0), 4 first output row of the
 //                               group's tile, 5 rows of the tile, negated when the
-//                               group is not the tile's last one
+//                               group is not the tile's last one, 6 accumulator slot
+//                               of the tile's first row
 // The convolution kernel streams through it without per-offset bookkeeping.
+// share_first/share_cnt[t*K + k]: the pairs of offset k that tile t works on.  They
+// begin where the previous tile of the same workgroup stopped and end with the last
+// pair of a row of tile t, rounded up to a whole row block with pairs of the next
+// tile's rows as far as spill[] allows.  One thread per (workgroup, offset) walks
+// the workgroup's tiles in order.
 __global__ void __launch_bounds__(256)
-    sched_count_kernel(const int32_t *__restrict__ segs, int K,
+    share_kernel(const int32_t *__restrict__ segs, const int32_t *__restrict__ spill, int K,
+                 int n_wg, const int32_t *__restrict__ wg_tile,
+                 int32_t *__restrict__ share_first, int32_t *__restrict__ share_cnt) {
+  const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= n_wg * K) return;
+  const int w = idx / K, k = idx - w * K;
+  const int t0 = wg_tile[w], t1 = wg_tile[w + 1];
+  if (t0 >= t1) return;
+  int s = segs[(int64_t)t0 * K + k];
+  for (int t = t0; t < t1; ++t) {
+    const int q = segs[(int64_t)(t + 1) * K + k];   // first pair of a later tile's row
+    const int lim = spill[(int64_t)(t + 1) * K + k];  // >= q
+    int e = s;
+    if (q > s) {
+      e = s + ((q - s + 15) & ~15);
+      if (e > lim) e = lim;
+    }
+    share_first[(int64_t)t * K + k] = s;
+    share_cnt[(int64_t)t * K + k] = e - s;
+    s = e;
+  }
+}
+
+__global__ void __launch_bounds__(256)
+    sched_count_kernel(const int32_t *__restrict__ share_cnt, int K,
                        const int32_t *__restrict__ n_tiles_dev, int32_t *__restrict__ tile_cnt,
                        int32_t *__restrict__ tile_nmb, int32_t *__restrict__ kofs) {
   int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (t >= n_tiles_dev[0]) return;
   int run = 0;
   for (int k = 0; k < K; ++k) {
-    int n = segs[(t + 1) * K + k] - segs[t * K + k];
+    int n = share_cnt[t * K + k];
     kofs[t * K + k] = run;
     run += (n + 15) >> 4;
   }
@@ -315,10 +376,12 @@ __global__ void __launch_bounds__(kScanThreads)
 __global__ void __launch_bounds__(256)
     sched_fill_kernel(const int32_t *__restrict__ flag, const int32_t *__restrict__ pairs,
                       const int32_t *__restrict__ sorted, int64_t pair_stride, int plane_g,
-                      const int32_t *__restrict__ segs, const int32_t *__restrict__ kofs,
+                      const int32_t *__restrict__ share_first,
+                      const int32_t *__restrict__ share_cnt, const int32_t *__restrict__ kofs,
                       const int32_t *__restrict__ tile_nmb, const int32_t *__restrict__ tile_grp,
                       int K, const int32_t *__restrict__ n_tiles_dev,
-                      const int32_t *__restrict__ tile_row0, int T, uint32_t in_scale,
+                      const int32_t *__restrict__ tile_row0,
+                      const int32_t *__restrict__ tile_slot0, int T, uint32_t in_scale,
                       uint32_t in_pad, int out_scale, int k_scale,
                       int32_t *__restrict__ sched_in, int32_t *__restrict__ sched_out,
                       int32_t *__restrict__ grp_meta) {
@@ -334,7 +397,7 @@ __global__ void __launch_bounds__(256)
       const int rows = tile_row0[t + 1] - tile_row0[t];
       grp_meta[g * 8 + 4] = tile_row0[t];
       grp_meta[g * 8 + 5] = g + 1 == g1 ? rows : -rows;
-      grp_meta[g * 8 + 6] = 0;
+      grp_meta[g * 8 + 6] = tile_slot0[t];
       grp_meta[g * 8 + 7] = 0;
     }
     for (int64_t mb = g0 * 4 + tile_nmb[t]; mb < g1 * 4; ++mb) {
@@ -344,16 +407,23 @@ __global__ void __launch_bounds__(256)
     }
   }
   const int32_t *src = flag[0] ? sorted : pairs;
-  int s0 = segs[t * K + k];
-  int n = segs[(t + 1) * K + k] - s0;
+  int s0 = share_first[t * K + k];
+  int n = share_cnt[t * K + k];
   if (n <= 0) return;
   const int32_t *pg = src + ((int64_t)k * 2 + plane_g) * pair_stride + s0;
   const int32_t *ps = src + ((int64_t)k * 2 + (1 - plane_g)) * pair_stride + s0;
   int64_t mb = g0 * 4 + kofs[t * K + k];
-  int64_t row0 = tile_row0[t];
+  // accumulator slot of a row: rows map to slots modulo the window height T; the
+  // rows a tile touches span less than T, so one conditional subtraction does it
+  const int slot_off = tile_slot0[t] - tile_row0[t];
   for (int p = lane; p < ((n + 15) & ~15); p += 16, ++mb) {
     sched_in[mb * 16 + lane] = p < n ? (int32_t)((uint32_t)pg[p] * in_scale) : (int32_t)in_pad;
-    sched_out[mb * 16 + lane] = (p < n ? (int)(ps[p] - row0) : T) * out_scale;
+    int slot = T;
+    if (p < n) {
+      slot = ps[p] + slot_off;
+      if (slot >= T) slot -= T;
+    }
+    sched_out[mb * 16 + lane] = slot * out_scale;
     if (lane == 0) grp_meta[(mb >> 2) * 8 + (mb & 3)] = k * k_scale;
   }
 }
@@ -407,9 +477,9 @@ constexpr int kRsrcFlags = 0x00020000;        // raw buffer of 32-bit data
 __device__ __forceinline__ float4v buf_load4(__amdgpu_buffer_rsrc_t r, int voff, int soff) {
   return __builtin_bit_cast(float4v, __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, 0));
 }
-typedef int int2v __attribute__((ext_vector_type(2)));
-__device__ __forceinline__ int2v buf_load2(__amdgpu_buffer_rsrc_t r, int voff, int soff) {
-  return __builtin_bit_cast(int2v, __builtin_amdgcn_raw_buffer_load_b64(r, voff, soff, 0));
+typedef int int3v __attribute__((ext_vector_type(3)));
+__device__ __forceinline__ int3v buf_load3(__amdgpu_buffer_rsrc_t r, int voff, int soff) {
+  return __builtin_bit_cast(int3v, __builtin_amdgcn_raw_buffer_load_b96(r, voff, soff, 0));
 }
 __device__ __forceinline__ int buf_load1(__amdgpu_buffer_rsrc_t r, int voff, int soff) {
   return (int)__builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, 0);
@@ -481,7 +551,8 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
   }
 
   // Tile `tl` is complete: write its rows, clear the accumulators.
-  auto flush_tile = [&](int row0, int rows) {
+  // (slot0 = accumulator slot of the tile's first row; slots wrap around at T)
+  auto flush_tile = [&](int row0, int rows, int slot0) {
     if ((cout & 3) == 0) {
       // A thread keeps its 4 columns and walks down the rows, NT / (kCN / 4) rows per
       // step: addresses advance by constants, so a step is little more than its LDS
@@ -493,7 +564,6 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
       constexpr int RS = NT / (kCN / 4);  // rows per step
       const int r_t = tid / (kCN / 4), c_t = (tid % (kCN / 4)) * 4;
       const bool col_ok = col0 + c_t < cout;
-      float *lp = acc + r_t * kAS + c_t;
       float *gp = out + (int64_t)(row0 + r_t) * cout + col0 + c_t;
       const int64_t gstep = (int64_t)RS * cout;
       for (int r = r_t; r < rows; r += U * RS) {
@@ -501,7 +571,9 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
 #pragma unroll
         for (int u = 0; u < U; ++u)
           if (r + u * RS < rows) {
-            float4v *ap = reinterpret_cast<float4v *>(lp + u * RS * kAS);
+            int sl = slot0 + r + u * RS;
+            if (sl >= T) sl -= T;
+            float4v *ap = reinterpret_cast<float4v *>(acc + sl * kAS + c_t);
             v[u] = *ap;
             *ap = z;
           }
@@ -511,24 +583,26 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
           // push the weights and the gathered rows out of L2
           if (r + u * RS < rows && col_ok)
             __builtin_nontemporal_store(v[u], reinterpret_cast<float4v *>(gp + u * gstep));
-        lp += U * RS * kAS;
         gp += U * gstep;
       }
     } else {
       for (int e = tid; e < rows * kCN; e += NT) {
         int r = e / kCN, c = e % kCN;
+        int sl = slot0 + r;
+        if (sl >= T) sl -= T;
         if (col0 + c < cout)
-          __builtin_nontemporal_store(acc[r * kAS + c], out + (int64_t)(row0 + r) * cout + col0 + c);
-        acc[r * kAS + c] = 0.f;
+          __builtin_nontemporal_store(acc[sl * kAS + c], out + (int64_t)(row0 + r) * cout + col0 + c);
+        acc[sl * kAS + c] = 0.f;
       }
     }
   };
   // The tile of stage `pos` (first row, rows) ends with it when the group is the
   // tile's last one and the chunk is the last chunk.  Scalar loads: the address is
   // uniform.
-  auto tile_end = [&](const StagePos &pos, int &row0, int &rows) -> bool {
+  auto tile_end = [&](const StagePos &pos, int &row0, int &rows, int &slot0) -> bool {
     const int32_t *m = grp_meta + (int64_t)pos.g * 8;
     row0 = m[4];
+    slot0 = m[6];
     const int r = m[5];
     rows = r < 0 ? -r : r;
     return r > 0 && pos.cc == nch - 1;
@@ -627,8 +701,8 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
     // (rows) and s+7 (gather offsets).
     auto iteration = [&](int s, auto phase) {
       constexpr int ph = decltype(phase)::value;  // == s & 3
-      int t_row0, t_rows;
-      const bool last = tile_end(p_cur, t_row0, t_rows);
+      int t_row0, t_rows, t_slot0;
+      const bool last = tile_end(p_cur, t_row0, t_rows, t_slot0);
       p_cur.advance(nch);
       store_rows((ph + 1) & 1, rows[(ph + 1) & 3]);
       load_rows(p_rows, idx[(ph + 1 + RD) & 1], rows[(ph + 1 + RD) & 3]);
@@ -637,7 +711,7 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
       p_idx.advance(nch);
       __syncthreads();
       if (last) {
-        flush_tile(t_row0, t_rows);
+        flush_tile(t_row0, t_rows, t_slot0);
         __syncthreads();
       }
     };
@@ -690,17 +764,17 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
     float4v w[4][4];
     int orow[4];
     int4v rec[2][2];
-    // Second half of a record: only its first two words are used.  An 8-byte load:
-    // a wider one would still write the two unused registers when it lands, and
-    // whatever the compiler keeps there in the meantime would have to wait for it.
+    // Second half of a record: only its first three words are used.  A 12-byte load:
+    // a wider one would still write the unused register when it lands, and whatever
+    // the compiler keeps there in the meantime would have to wait for it.
     auto load_rec_tail = [&](const StagePos &pos) -> int4v {
-      const int2v t = buf_load2(rs_meta, 16, pos.g * 32);
-      return int4v{t.x, t.y, 0, 0};
+      const int3v t = buf_load3(rs_meta, 16, pos.g * 32);
+      return int4v{t.x, t.y, t.z, 0};
     };
     // First row and rows of the tile of a stage, and whether the tile ends with the
     // stage, from the second half of its record.
     struct TileEnd {
-      int row0, rows;
+      int row0, rows, slot0;
       bool last;
     };
     auto tile_end_of = [&](const int4v &tail, const StagePos &pos) -> TileEnd {
@@ -708,6 +782,7 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
       e.row0 = __builtin_amdgcn_readfirstlane(tail.x);
       const int r = __builtin_amdgcn_readfirstlane(tail.y);
       e.rows = r < 0 ? -r : r;
+      e.slot0 = __builtin_amdgcn_readfirstlane(tail.z);
       e.last = r > 0 && pos.cc == nch - 1;
       return e;
     };
@@ -866,7 +941,7 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
       p_after.advance(nch);
       __syncthreads();
       if (end.last) {
-        flush_tile(end.row0, end.rows);
+        flush_tile(end.row0, end.rows, end.slot0);
         __syncthreads();
       }
       end = end_next;
@@ -882,7 +957,8 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
 }
 
 struct ConvPlan {
-  int ncb, nch, T, ncw, n_wg, n_colblk;
+  int ncb, nch, T, ncw, n_wg, n_colblk;  // T: rows of the accumulator window
+  int tile_rows;                         // largest tile height
   int gather;  // conv_fwd_kernel's GATHER
   int64_t n_tiles, n_fine, words_per_k, grp_cap;  // n_tiles: upper bound
   size_t lds_bytes;
@@ -920,6 +996,7 @@ static ConvPlan make_plan(int64_t n_in, int64_t n_out, int K, int c_in, int c_ou
   p.nch = (int)ceil_div(c_in, kKC);
   p.ncw = 4;
   p.T = pick_tile(p.ncw);
+  p.tile_rows = p.T - kSpillRows;
   // the gather can be a range-checked buffer load when rows are multiples of 16 bytes
   // and byte offsets into the features (plus the padding marker) fit 32 bits
   p.gather = 0;
@@ -932,7 +1009,7 @@ static ConvPlan make_plan(int64_t n_in, int64_t n_out, int K, int c_in, int c_ou
   if (n_wg >= 8) n_wg = n_wg / 8 * 8;
   p.n_wg = n_wg;
   // upper bound of the tile count: every workgroup's range ends with a partial tile
-  p.n_tiles = ceil_div(n_out > 0 ? n_out : 1, p.T) + n_wg;
+  p.n_tiles = ceil_div(n_out > 0 ? n_out : 1, p.tile_rows) + n_wg;
   p.n_fine = ceil_div(n_out > 0 ? n_out : 1, kSplitGranule);
   p.words_per_k = ceil_div(n_out > 0 ? n_out : 1, 32);
   // groups: pairs/64 plus, per (tile, offset), up to one partial block, plus one
@@ -953,6 +1030,7 @@ struct ConvWs {
   int32_t *prefix;
   int32_t *tile_cnt, *tile_nmb, *kofs, *tile_grp, *wg_tile;
   int32_t *fine_segs, *fine_work, *tile_row0, *n_tiles_dev;
+  int32_t *spill_end, *tile_slot0, *spill, *share_first, *share_cnt;
   int32_t *sched_in, *sched_out, *grp_meta;
 };
 
@@ -973,6 +1051,11 @@ static size_t conv_ws_walk(void *base, const ConvPlan &p, int K, int64_t pair_st
   t.fine_segs = c.take<int32_t>((size_t)(p.n_fine + 1) * K);
   t.fine_work = c.take<int32_t>((size_t)p.n_fine + 1);
   t.tile_row0 = c.take<int32_t>((size_t)p.n_tiles + 1);
+  t.spill_end = c.take<int32_t>((size_t)p.n_tiles + 1);
+  t.tile_slot0 = c.take<int32_t>((size_t)p.n_tiles + 1);
+  t.spill = c.take<int32_t>((size_t)(p.n_tiles + 1) * K);
+  t.share_first = c.take<int32_t>((size_t)p.n_tiles * K);
+  t.share_cnt = c.take<int32_t>((size_t)p.n_tiles * K);
   t.n_tiles_dev = c.take<int32_t>(1);
   t.sched_in = c.take<int32_t>((size_t)p.grp_cap * 64);
   t.sched_out = c.take<int32_t>((size_t)p.grp_cap * 64);
@@ -1114,24 +1197,28 @@ int ssc_conv_fwd_f32(const float *features, int64_t n_in, int32_t c_in, const fl
   hipLaunchKernelGGL(tile_segments_kernel, dim3((unsigned)ceil_div(nfine, 256)), dim3(256), 0, s,
                      w.flag, pairs, w.sorted, pair_stride, plane_s, pair_num, K, p.n_fine,
                      (const int32_t *)nullptr, (const int32_t *)nullptr, kSplitGranule, n_out,
-                     w.fine_segs);
+                     w.fine_segs, (const int32_t *)nullptr, (int32_t *)nullptr);
   hipLaunchKernelGGL(split_sum_kernel, dim3((unsigned)ceil_div(p.n_fine + 1, 256)), dim3(256), 0, s,
                      w.fine_segs, K, p.n_fine, w.fine_work);
   hipLaunchKernelGGL(split_rows_kernel, dim3(1), dim3(256), 0, s, w.fine_work, p.n_fine, n_out,
-                     p.T, K, p.n_wg, w.wg_tile, w.tile_row0, w.n_tiles_dev);
+                     p.tile_rows, p.T, K, p.n_wg, w.wg_tile, w.tile_row0, w.n_tiles_dev,
+                     w.spill_end, w.tile_slot0);
   SSC_LAUNCH_CHECK("split");
   int64_t nseg = (p.n_tiles + 1) * K;
   hipLaunchKernelGGL(tile_segments_kernel, dim3((unsigned)ceil_div(nseg, 256)), dim3(256), 0, s,
                      w.flag, pairs, w.sorted, pair_stride, plane_s, pair_num, K, p.n_tiles,
-                     w.n_tiles_dev, w.tile_row0, 0, n_out, w.segs);
+                     w.n_tiles_dev, w.tile_row0, 0, n_out, w.segs, w.spill_end, w.spill);
   SSC_LAUNCH_CHECK("tile_segments");
+  hipLaunchKernelGGL(share_kernel, dim3((unsigned)ceil_div((int64_t)p.n_wg * K, 256)), dim3(256),
+                     0, s, w.segs, w.spill, K, p.n_wg, w.wg_tile, w.share_first, w.share_cnt);
   hipLaunchKernelGGL(sched_count_kernel, dim3((unsigned)ceil_div(p.n_tiles, 256)), dim3(256), 0, s,
-                     w.segs, K, w.n_tiles_dev, w.tile_cnt, w.tile_nmb, w.kofs);
+                     w.share_cnt, K, w.n_tiles_dev, w.tile_cnt, w.tile_nmb, w.kofs);
   hipLaunchKernelGGL(sched_scan_kernel, dim3(1), dim3(kScanThreads), 0, s, w.tile_cnt,
                      w.n_tiles_dev, w.tile_grp);
   hipLaunchKernelGGL(sched_fill_kernel, dim3((unsigned)ceil_div(p.n_tiles * K * 16, 256)),
-                     dim3(256), 0, s, w.flag, pairs, w.sorted, pair_stride, plane_g, w.segs,
-                     w.kofs, w.tile_nmb, w.tile_grp, K, w.n_tiles_dev, w.tile_row0, p.T,
+                     dim3(256), 0, s, w.flag, pairs, w.sorted, pair_stride, plane_g,
+                     w.share_first, w.share_cnt, w.kofs, w.tile_nmb, w.tile_grp, K,
+                     w.n_tiles_dev, w.tile_row0, w.tile_slot0, p.T,
                      p.gather ? (uint32_t)c_in * 4u : 1u, p.gather ? kGatherPad : 0xFFFFFFFFu,
                      (16 * p.ncw + 4) * 4, p.ncb * p.nch * 4096, w.sched_in, w.sched_out,
                      w.grp_meta);
