@@ -195,7 +195,7 @@ constexpr int kSplitGranule = 64;
 // kSpillRows into it), instead of being padded.  Rows map to accumulator slots
 // modulo the window height, so what such a block adds to the next tile's rows is
 // still there when that tile's turn comes.
-constexpr int kSpillRows = 128;
+constexpr int kSpillRows = 160;
 
 // fine_work[b] = sum over offsets of fine_segs[b*K + k]  (pairs in rows < b*granule)
 __global__ void __launch_bounds__(256)
