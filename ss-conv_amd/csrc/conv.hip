@@ -742,9 +742,13 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
         __builtin_amdgcn_make_buffer_rsrc((void *)sched_out, 0, (int)sched_bytes, kRsrcFlags);
     const int w_voff = lane * 64;           // this lane's 16 floats of a fragment
     const int w_soff0 = cb * nch * 4096;    // fragments of this wave's column block
-    const int acc_lane = (wave * 16 + g * 4) * 4;  // byte offset of this lane's 4 columns
     const float *const a_base = abuf + l16 * kAStride + g * 16;
-    char *const acc_bytes = reinterpret_cast<char *>(acc);
+    // The accumulators are addressed with 32-bit LDS byte addresses (acc_lane includes
+    // the base of acc): no pointer arithmetic left for the vector ALU.
+    typedef __attribute__((address_space(3))) float4v lds_float4v;
+    const int acc_base = (int)(size_t)(__attribute__((address_space(3))) char *)acc;
+    auto lds_load4 = [](int addr) -> float4v { return *(lds_float4v *)(size_t)addr; };
+    auto lds_store4 = [](int addr, const float4v &v) { *(lds_float4v *)(size_t)addr = v; };
 
     const __amdgpu_buffer_rsrc_t rs_meta =
         __builtin_amdgcn_make_buffer_rsrc((void *)grp_meta, 0, (int)meta_bytes, kRsrcFlags);
@@ -811,6 +815,8 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
       int addr;
       float4v accr, d;
     };
+    // LDS address of this lane's 4 columns in accumulator row 0
+    const int acc_lane = acc_base + (wave * 16 + g * 4) * 4;
     const int dummy_addr = T * kAS * 4 + acc_lane;
     Pending pend;  // nothing pending yet: the first write adds zero to the dummy row
     pend.addr = dummy_addr;
@@ -822,16 +828,16 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
     // chain a handful of other instructions issue for free -- and no more than that:
     // everything else a block needs is therefore spread, one small piece per gap,
     // over the 16 gaps of the block, and scheduling barriers pin it there:
-    //   gap 0      fragment offset of block b+3 (from the schedule record)
-    //   gaps 1,4,8,12  the four fragment loads of block b+3 (the slot of block b-1)
-    //   gap 2      accumulator update of the previous block: add, write
+    //   gap 2      fragment offset of block b+3 (from the schedule record); accumulator
+    //              update of the previous block: add, write; once per stage, tile and
+    //              last-of-tile of the next stage
     //   gap 3      accumulator read of this block (LDS operations of a wave execute
     //              in order, so it sees the write of gap 2 when both blocks touch
     //              the same output row)
+    //   gaps 4,7,9,12  the four fragment loads of block b+3 (the slot of block b-1)
     //   gap 5      output rows of block b+3
-    //   gaps 6,7,9,10  the staged rows of block m+1
-    //   gaps 11,13 once per stage: the record of the stage after the next; tile and
-    //              last-of-tile of the next stage
+    //   gaps 6,8,10,11  the staged rows of block m+1
+    //   gaps 13,14 once per stage: the record of the stage after the next
     // The update of a stage's last block waits, across the barrier, for the first
     // block of the next stage, unless the tile ends here.
     //   cur / next / after: positions of this stage and the two that follow;
@@ -862,41 +868,41 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
           __builtin_amdgcn_sched_barrier(0);
           d = __builtin_amdgcn_mfma_f32_16x16x4f32(w[slot][q][j], a[m & 1][q][j], d, 0, 0, 0);
           __builtin_amdgcn_sched_barrier(0);
-          if (i == 0)
+          // all vector-ALU work of the block in one gap: a vector-ALU instruction
+          // next to the matrix chain costs about ten cycles for leaving and re-entering
+          // the chain, whatever follows it in the same gap is cheap
+          if (i == 2) {
             soff = tnext ? frag_soff(rec_k(rec[par ^ 1][0], tm), base_next)
                          : frag_soff(rec_k(rec[par][0], tm), base_cur);
-          if (i == 1) fetch_w(soff, tslot, 0);
-          if (i == 2)  // pend.d = out[pair l16][channels 4g .. 4g+3] of the previous block
-            *reinterpret_cast<float4v *>(acc_bytes + pend.addr) = pend.accr + pend.d;
-          if (i == 3) {
+            if (m == 3) end_next = tile_end_of(rec[par ^ 1][1], next);
+            // pend.d = out[pair l16][channels 4g .. 4g+3] of the previous block
+            lds_store4(pend.addr, pend.accr + pend.d);
             pend.addr = orow[slot] + acc_lane;
-            pend.accr = *reinterpret_cast<const float4v *>(acc_bytes + pend.addr);
           }
-          if (i == 4) fetch_w(soff, tslot, 1);
+          if (i == 3) pend.accr = lds_load4(pend.addr);
+          if (i == 4) fetch_w(soff, tslot, 0);
           if (i == 5) fetch_orow(tnext ? next : cur, tm, tslot);
           if (m < 3) {
             if (i == 6) load_a(m + 1, 0, a[(m + 1) & 1]);
-            if (i == 7) load_a(m + 1, 1, a[(m + 1) & 1]);
-            if (i == 9) load_a(m + 1, 2, a[(m + 1) & 1]);
-            if (i == 10) load_a(m + 1, 3, a[(m + 1) & 1]);
+            if (i == 8) load_a(m + 1, 1, a[(m + 1) & 1]);
+            if (i == 10) load_a(m + 1, 2, a[(m + 1) & 1]);
+            if (i == 11) load_a(m + 1, 3, a[(m + 1) & 1]);
           }
-          if (i == 8) fetch_w(soff, tslot, 2);
+          if (i == 7) fetch_w(soff, tslot, 1);
+          if (i == 9) fetch_w(soff, tslot, 2);
           if (i == 12) fetch_w(soff, tslot, 3);
           // this stage's record was last used by block 0: refill it for the stage
           // after the next
-          if (m == 1 && i == 11)
+          if (m == 1 && i == 13)
             rec[par][0] = __builtin_bit_cast(int4v, buf_load4(rs_meta, 0, after.g * 32));
-          if (m == 1 && i == 13) rec[par][1] = load_rec_tail(after);
-          if (m == 3 && i == 13) {
-            end_next = tile_end_of(rec[par ^ 1][1], next);
-          }
+          if (m == 1 && i == 14) rec[par][1] = load_rec_tail(after);
         }
         __builtin_amdgcn_sched_barrier(0);
         pend.d = d;
       }
       __builtin_amdgcn_sched_barrier(0);
       if (last_cur) {  // the tile is written out after this stage: finish its last update
-        *reinterpret_cast<float4v *>(acc_bytes + pend.addr) = pend.accr + pend.d;
+        lds_store4(pend.addr, pend.accr + pend.d);
         pend.addr = dummy_addr;
       }
     };
