@@ -36,8 +36,10 @@ constexpr int kMinTile = 64;
 // out so that one wave reads it as four coalesced 16-byte loads per lane.
 __global__ void __launch_bounds__(256)
     pack_filters_kernel(const float *__restrict__ w, int64_t fs_k, int64_t fs_ci, int64_t fs_co,
-                        int K, int cin, int cout, int ncb, int nch, float *__restrict__ packed) {
+                        int K, int cin, int cout, int ncb, int nch, float *__restrict__ packed,
+                        int32_t *__restrict__ flag) {
   int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx == 0) flag[0] = 0;  // the pair-order flag of the kernels that follow
   int64_t total = (int64_t)K * ncb * nch * 1024;
   if (idx >= total) return;
   int c = idx & 15;
@@ -144,6 +146,8 @@ __global__ void __launch_bounds__(256)
 // tile t (t = 0..n_tiles).  Tile rows come from tile_row0[] and the tile count from
 // n_tiles_dev[0]; with tile_row0 == nullptr the tiles are `granule` rows each and
 // there are n_cap of them (the fine grid the work split is computed on).
+// With fine_segs != nullptr (segments of a grid of `granule` rows, computed before) the
+// search starts from the grid cell of the tile's first row instead of the whole list.
 // With spill_end != nullptr also spill[t*K + k] = how far the last row block of tile
 // t-1 may reach into tile t: the first pair at or after segs[t*K + k], at most 15
 // further, whose row is >= spill_end[t].
@@ -153,8 +157,8 @@ __global__ void __launch_bounds__(256)
                          const int32_t *__restrict__ pair_num, int K, int64_t n_cap,
                          const int32_t *__restrict__ n_tiles_dev,
                          const int32_t *__restrict__ tile_row0, int granule, int64_t n_out,
-                         int32_t *__restrict__ segs, const int32_t *__restrict__ spill_end,
-                         int32_t *__restrict__ spill) {
+                         int32_t *__restrict__ segs, const int32_t *__restrict__ fine_segs,
+                         const int32_t *__restrict__ spill_end, int32_t *__restrict__ spill) {
   int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   const int64_t n_tiles = tile_row0 ? n_tiles_dev[0] : n_cap;
   if (idx >= (n_tiles + 1) * K) return;
@@ -165,6 +169,11 @@ __global__ void __launch_bounds__(256)
   int64_t target = tile_row0 ? (int64_t)tile_row0[t] : t * (int64_t)granule;
   if (target > n_out) target = n_out;
   int lo = 0, hi = pair_num[k];
+  if (fine_segs) {
+    const int64_t cell = target / granule;  // target <= n_out: a cell of the grid or its end
+    lo = fine_segs[cell * K + k];
+    if ((cell + 1) * granule <= n_out) hi = fine_segs[(cell + 1) * K + k];
+  }
   while (lo < hi) {
     int mid = (lo + hi) >> 1;
     if (s[mid] < target) lo = mid + 1;
@@ -179,6 +188,33 @@ __global__ void __launch_bounds__(256)
     for (int j = 0; j < 15; ++j) cnt += (lo + j < n && s[lo + j] < bound) ? 1 : 0;  // rows ascend
     spill[idx] = lo + cnt;
   }
+}
+
+// The same segments for a regular grid of `granule` rows (cells c = 0..n_cells, cell
+// n_cells being the end), computed from the pairs' side: one thread per pair; the pair
+// that is the first of its offset at or beyond a cell boundary writes that boundary.
+__global__ void __launch_bounds__(256)
+    grid_segments_kernel(const int32_t *__restrict__ flag, const int32_t *__restrict__ pairs,
+                         const int32_t *__restrict__ sorted, int64_t pair_stride, int plane_s,
+                         const int32_t *__restrict__ pair_num, int K, int64_t n_cells,
+                         int granule, int32_t *__restrict__ segs) {
+  const int k = blockIdx.y;
+  const int64_t j = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int n = pair_num[k];
+  if (j >= n && !(j == 0 && n == 0)) return;
+  const int32_t *src = flag[0] ? sorted : pairs;
+  const int32_t *s = src + ((int64_t)k * 2 + plane_s) * pair_stride;
+  // boundary c (first row c*granule) is served by the first pair whose row is at or
+  // beyond it: pair j serves the boundaries in (row[j-1], row[j]]
+  int64_t c_next = 0;  // first boundary beyond this pair
+  if (n > 0) {
+    const int64_t c1 = s[j] / granule;
+    const int64_t c0 = j > 0 ? (int64_t)s[j - 1] / granule + 1 : 0;
+    for (int64_t c = c0; c <= c1 && c <= n_cells; ++c) segs[c * K + k] = (int32_t)j;
+    c_next = c1 + 1;
+  }
+  if (n == 0 || j == n - 1)  // boundaries beyond the last pair
+    for (int64_t c = c_next; c <= n_cells; ++c) segs[c * K + k] = n;
 }
 
 // ---- work split ------------------------------------------------------------------------
@@ -197,15 +233,45 @@ constexpr int kSplitGranule = 64;
 // still there when that tile's turn comes.
 constexpr int kSpillRows = 160;
 
-// fine_work[b] = sum over offsets of fine_segs[b*K + k]  (pairs in rows < b*granule)
+// cost of a tile beyond its pairs, in pair slots: some padding per offset, and about
+// two stages' worth of time for writing it out
+__device__ __forceinline__ int64_t split_tile_cost(int K) { return (int64_t)K * 2 + 128; }
+
+// Work in rows below cell b of the fine grid (scaled by T to stay in integers).
+__device__ __forceinline__ int64_t split_work(int64_t pairs_below, int64_t b, int64_t n_out,
+                                              int T, int K) {
+  int64_t r = b * kSplitGranule;
+  if (r > n_out) r = n_out;
+  return pairs_below * T + r * split_tile_cost(K);
+}
+
+// One thread per cell boundary b = 0..nb of the fine grid: the ranges whose first row
+// is boundary b are those whose target (w/n_wg of the total work) lies in
+// (work(b-1), work(b)].  range_row0[w], w = 0..n_wg.
 __global__ void __launch_bounds__(256)
-    split_sum_kernel(const int32_t *__restrict__ fine_segs, int K, int64_t nb,
-                     int32_t *__restrict__ fine_work) {
+    split_bounds_kernel(const int32_t *__restrict__ fine_segs, int K, int64_t nb, int64_t n_out,
+                        int T, int n_wg, int32_t *__restrict__ range_row0) {
   int64_t b = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (b > nb) return;
-  int sum = 0;
-  for (int k = 0; k < K; ++k) sum += fine_segs[b * K + k];
-  fine_work[b] = sum;
+  int64_t below = 0, below_prev = 0, all = 0;
+  for (int k = 0; k < K; ++k) {
+    below += fine_segs[b * K + k];
+    if (b > 0) below_prev += fine_segs[(b - 1) * K + k];
+    all += fine_segs[nb * K + k];
+  }
+  const int64_t total = split_work(all, nb, n_out, T, K);
+  // ranges w with ceil(total * w / n_wg) <= work, i.e. w <= work * n_wg / total
+  auto reached = [&](int64_t work) -> int64_t {
+    if (total <= 0) return n_wg + 1;
+    int64_t c = work * n_wg / total + 1;
+    return c > n_wg + 1 ? n_wg + 1 : c;
+  };
+  const int64_t w0 = b > 0 ? reached(split_work(below_prev, b - 1, n_out, T, K)) : 0;
+  const int64_t w1 = reached(split_work(below, b, n_out, T, K));
+  int64_t r = b * kSplitGranule;
+  if (r > n_out) r = n_out;
+  for (int64_t w = w0; w < w1; ++w)
+    range_row0[w] = (w == 0) ? 0 : (w == n_wg ? (int32_t)n_out : (int32_t)r);
 }
 
 // One block.  wg_tile[0..n_wg]: first tile of every workgroup; tile_row0[0..n_tiles]:
@@ -215,45 +281,42 @@ __global__ void __launch_bounds__(256)
 // ranges); tile_slot0[t]: accumulator slot of the first row of tile t.  T is the
 // largest tile height, window the height of the accumulator window.
 __global__ void __launch_bounds__(256)
-    split_rows_kernel(const int32_t *__restrict__ fine_work, int64_t nb, int64_t n_out, int T,
-                      int window, int K, int n_wg, int32_t *__restrict__ wg_tile,
-                      int32_t *__restrict__ tile_row0, int32_t *__restrict__ n_tiles_dev,
-                      int32_t *__restrict__ spill_end, int32_t *__restrict__ tile_slot0) {
+    split_rows_kernel(const int32_t *__restrict__ range_row0, int64_t n_out, int T, int window,
+                      int n_wg, int32_t *__restrict__ wg_tile, int32_t *__restrict__ tile_row0,
+                      int32_t *__restrict__ n_tiles_dev, int32_t *__restrict__ spill_end,
+                      int32_t *__restrict__ tile_slot0) {
   __shared__ int row_s[257];
   __shared__ int tile_s[257];
-  // cost of a tile beyond its pairs, in pair slots: some padding per offset, and
-  // about two stages' worth of time for writing it out
-  const int64_t tile_cost = (int64_t)K * 2 + 128;
-  auto work = [&](int64_t b) -> int64_t {
-    int64_t r = b * kSplitGranule;
-    if (r > n_out) r = n_out;
-    return (int64_t)fine_work[b] * T + r * tile_cost;  // scaled by T to stay in integers
-  };
   for (int w = threadIdx.x; w <= n_wg; w += blockDim.x) {  // n_wg <= 256
-    const int64_t total = work(nb);
-    const int64_t target = (total * w + n_wg - 1) / n_wg;
-    int64_t lo = 0, hi = nb;
-    while (lo < hi) {
-      int64_t mid = (lo + hi) >> 1;
-      if (work(mid) < target) lo = mid + 1;
-      else hi = mid;
-    }
-    int64_t r = lo * kSplitGranule;
-    if (r > n_out || w == n_wg) r = n_out;
+    int r = range_row0[w];
     if (w == 0) r = 0;
-    row_s[w] = (int)r;
+    if (w == n_wg) r = (int)n_out;
+    row_s[w] = r;
   }
   __syncthreads();
-  if (threadIdx.x == 0) {
-    int run = 0;
-    for (int i = 0; i < n_wg; ++i) {
-      tile_s[i] = run;
-      run += (row_s[i + 1] - row_s[i] + T - 1) / T;
+  {
+    // exclusive scan of the tile counts of the (at most 256) ranges, one per thread
+    __shared__ int wave_sum[4];
+    const int w = threadIdx.x, lane = w & 63;
+    const int nt = w < n_wg ? (row_s[w + 1] - row_s[w] + T - 1) / T : 0;
+    int incl = nt;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      int o = __shfl_up(incl, d, 64);
+      if (lane >= d) incl += o;
     }
-    tile_s[n_wg] = run;
-    n_tiles_dev[0] = run;
-    tile_row0[run] = (int32_t)n_out;
-    spill_end[run] = (int32_t)n_out;
+    if (lane == 63) wave_sum[w >> 6] = incl;
+    __syncthreads();
+    int before = 0;
+    for (int i = 0; i < (w >> 6); ++i) before += wave_sum[i];
+    if (w < n_wg) tile_s[w] = before + incl - nt;
+    if (w == 255) {
+      const int run = before + incl;
+      tile_s[n_wg] = run;
+      n_tiles_dev[0] = run;
+      tile_row0[run] = (int32_t)n_out;
+      spill_end[run] = (int32_t)n_out;
+    }
   }
   __syncthreads();
   for (int w = threadIdx.x; w <= n_wg; w += blockDim.x) {
@@ -307,35 +370,61 @@ __global__ void __launch_bounds__(256)
   const int t0 = wg_tile[w], t1 = wg_tile[w + 1];
   if (t0 >= t1) return;
   int s = segs[(int64_t)t0 * K + k];
-  for (int t = t0; t < t1; ++t) {
-    const int q = segs[(int64_t)(t + 1) * K + k];   // first pair of a later tile's row
-    const int lim = spill[(int64_t)(t + 1) * K + k];  // >= q
-    int e = s;
-    if (q > s) {
-      e = s + ((q - s + 15) & ~15);
-      if (e > lim) e = lim;
+  // eight tiles at a time: their loads are issued together, the chain through s is
+  // arithmetic only
+  constexpr int U = 8;
+  for (int tb = t0; tb < t1; tb += U) {
+    int q[U], lim[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int t = tb + u < t1 ? tb + u : t1 - 1;
+      q[u] = segs[(int64_t)(t + 1) * K + k];    // first pair of a later tile's row
+      lim[u] = spill[(int64_t)(t + 1) * K + k];  // >= q
     }
-    share_first[(int64_t)t * K + k] = s;
-    share_cnt[(int64_t)t * K + k] = e - s;
-    s = e;
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int t = tb + u;
+      if (t < t1) {
+        int e = s;
+        if (q[u] > s) {
+          e = s + ((q[u] - s + 15) & ~15);
+          if (e > lim[u]) e = lim[u];
+        }
+        share_first[(int64_t)t * K + k] = s;
+        share_cnt[(int64_t)t * K + k] = e - s;
+        s = e;
+      }
+    }
   }
 }
 
+// One wave per tile, lanes over the offsets: kofs[t*K + k] = row blocks of tile t
+// before offset k, tile_nmb[t] = its row blocks, tile_cnt[t] = its groups (at least one).
 __global__ void __launch_bounds__(256)
     sched_count_kernel(const int32_t *__restrict__ share_cnt, int K,
                        const int32_t *__restrict__ n_tiles_dev, int32_t *__restrict__ tile_cnt,
                        int32_t *__restrict__ tile_nmb, int32_t *__restrict__ kofs) {
-  int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (t >= n_tiles_dev[0]) return;
+  const int lane = threadIdx.x & 63;
+  const int64_t t = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  if (t >= n_tiles_dev[0]) return;  // the same for the whole wave
   int run = 0;
-  for (int k = 0; k < K; ++k) {
-    int n = share_cnt[t * K + k];
-    kofs[t * K + k] = run;
-    run += (n + 15) >> 4;
+  for (int k0 = 0; k0 < K; k0 += 64) {
+    const int k = k0 + lane;
+    const int nb = k < K ? (share_cnt[t * K + k] + 15) >> 4 : 0;
+    int incl = nb;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      int o = __shfl_up(incl, d, 64);
+      if (lane >= d) incl += o;
+    }
+    if (k < K) kofs[t * K + k] = run + incl - nb;
+    run += __shfl(incl, 63, 64);
   }
-  tile_nmb[t] = run;
-  int groups = (run + 3) >> 2;
-  tile_cnt[t] = groups > 0 ? groups : 1;
+  if (lane == 0) {
+    tile_nmb[t] = run;
+    int groups = (run + 3) >> 2;
+    tile_cnt[t] = groups > 0 ? groups : 1;
+  }
 }
 
 // tile_grp[0..n_tiles]: exclusive prefix of tile_cnt (one block).
@@ -1035,7 +1124,7 @@ struct ConvWs {
   uint32_t *bits;
   int32_t *prefix;
   int32_t *tile_cnt, *tile_nmb, *kofs, *tile_grp, *wg_tile;
-  int32_t *fine_segs, *fine_work, *tile_row0, *n_tiles_dev;
+  int32_t *fine_segs, *range_row0, *tile_row0, *n_tiles_dev;
   int32_t *spill_end, *tile_slot0, *spill, *share_first, *share_cnt;
   int32_t *sched_in, *sched_out, *grp_meta;
 };
@@ -1055,7 +1144,7 @@ static size_t conv_ws_walk(void *base, const ConvPlan &p, int K, int64_t pair_st
   t.tile_grp = c.take<int32_t>((size_t)p.n_tiles + 1);
   t.wg_tile = c.take<int32_t>((size_t)p.n_wg + 1);
   t.fine_segs = c.take<int32_t>((size_t)(p.n_fine + 1) * K);
-  t.fine_work = c.take<int32_t>((size_t)p.n_fine + 1);
+  t.range_row0 = c.take<int32_t>((size_t)p.n_wg + 1);
   t.tile_row0 = c.take<int32_t>((size_t)p.n_tiles + 1);
   t.spill_end = c.take<int32_t>((size_t)p.n_tiles + 1);
   t.tile_slot0 = c.take<int32_t>((size_t)p.n_tiles + 1);
@@ -1177,10 +1266,9 @@ int ssc_conv_fwd_f32(const float *features, int64_t n_in, int32_t c_in, const fl
 
   int64_t packed_n = (int64_t)K * p.ncb * p.nch * 1024;
   hipLaunchKernelGGL(pack_filters_kernel, dim3((unsigned)ceil_div(packed_n, 256)), dim3(256), 0, s,
-                     filters, fs_k, fs_ci, fs_co, K, c_in, c_out, p.ncb, p.nch, w.packed);
+                     filters, fs_k, fs_ci, fs_co, K, c_in, c_out, p.ncb, p.nch, w.packed, w.flag);
   SSC_LAUNCH_CHECK("pack_filters");
 
-  if ((rc = fill_i32(w.flag, 1, 0, s)) != SSC_OK) return rc;
   dim3 pair_grid((unsigned)ceil_div(pair_stride, 256), (unsigned)K);
   hipLaunchKernelGGL(check_sorted_kernel, pair_grid, dim3(256), 0, s, pairs, pair_stride, plane_s,
                      pair_num, w.flag);
@@ -1199,25 +1287,23 @@ int ssc_conv_fwd_f32(const float *features, int64_t n_in, int32_t c_in, const fl
   SSC_LAUNCH_CHECK("resort");
 
   // work split on the fine grid, then the tiles and their segments
-  int64_t nfine = (p.n_fine + 1) * K;
-  hipLaunchKernelGGL(tile_segments_kernel, dim3((unsigned)ceil_div(nfine, 256)), dim3(256), 0, s,
-                     w.flag, pairs, w.sorted, pair_stride, plane_s, pair_num, K, p.n_fine,
-                     (const int32_t *)nullptr, (const int32_t *)nullptr, kSplitGranule, n_out,
-                     w.fine_segs, (const int32_t *)nullptr, (int32_t *)nullptr);
-  hipLaunchKernelGGL(split_sum_kernel, dim3((unsigned)ceil_div(p.n_fine + 1, 256)), dim3(256), 0, s,
-                     w.fine_segs, K, p.n_fine, w.fine_work);
-  hipLaunchKernelGGL(split_rows_kernel, dim3(1), dim3(256), 0, s, w.fine_work, p.n_fine, n_out,
-                     p.tile_rows, p.T, K, p.n_wg, w.wg_tile, w.tile_row0, w.n_tiles_dev,
-                     w.spill_end, w.tile_slot0);
+  hipLaunchKernelGGL(grid_segments_kernel, pair_grid, dim3(256), 0, s, w.flag, pairs, w.sorted,
+                     pair_stride, plane_s, pair_num, K, p.n_fine, kSplitGranule, w.fine_segs);
+  hipLaunchKernelGGL(split_bounds_kernel, dim3((unsigned)ceil_div(p.n_fine + 1, 256)), dim3(256), 0,
+                     s, w.fine_segs, K, p.n_fine, n_out, p.tile_rows, p.n_wg, w.range_row0);
+  hipLaunchKernelGGL(split_rows_kernel, dim3(1), dim3(256), 0, s, w.range_row0, n_out, p.tile_rows,
+                     p.T, p.n_wg, w.wg_tile, w.tile_row0, w.n_tiles_dev, w.spill_end,
+                     w.tile_slot0);
   SSC_LAUNCH_CHECK("split");
   int64_t nseg = (p.n_tiles + 1) * K;
   hipLaunchKernelGGL(tile_segments_kernel, dim3((unsigned)ceil_div(nseg, 256)), dim3(256), 0, s,
                      w.flag, pairs, w.sorted, pair_stride, plane_s, pair_num, K, p.n_tiles,
-                     w.n_tiles_dev, w.tile_row0, 0, n_out, w.segs, w.spill_end, w.spill);
+                     w.n_tiles_dev, w.tile_row0, kSplitGranule, n_out, w.segs, w.fine_segs,
+                     w.spill_end, w.spill);
   SSC_LAUNCH_CHECK("tile_segments");
   hipLaunchKernelGGL(share_kernel, dim3((unsigned)ceil_div((int64_t)p.n_wg * K, 256)), dim3(256),
                      0, s, w.segs, w.spill, K, p.n_wg, w.wg_tile, w.share_first, w.share_cnt);
-  hipLaunchKernelGGL(sched_count_kernel, dim3((unsigned)ceil_div(p.n_tiles, 256)), dim3(256), 0, s,
+  hipLaunchKernelGGL(sched_count_kernel, dim3((unsigned)ceil_div(p.n_tiles, 4)), dim3(256), 0, s,
                      w.share_cnt, K, w.n_tiles_dev, w.tile_cnt, w.tile_nmb, w.kofs);
   hipLaunchKernelGGL(sched_scan_kernel, dim3(1), dim3(kScanThreads), 0, s, w.tile_cnt,
                      w.n_tiles_dev, w.tile_grp);
