@@ -177,6 +177,57 @@ def ops_table(torch, _ext, synth, dev, seed):
     n = vp.shape[0]
     report("Voxel2Point module (%d pts, %d voxels, C=%d)" % (n, M, C), ms,
            4 * C * 4 * n + 16 * (n + M) + 24 * n, "3-NN search: n*M/B distance tests")
+
+    # BatchNorm + gated Activation after the cfg2 layer: irrep(8,8,8,8) fields = 128 columns
+    # plus 24 gate scalars, on the layer's 600k output rows
+    from ss_conv import bnact
+    from ss_conv.activation import Activation
+    from ss_conv.batchnorm import BatchNorm
+    from ss_conv.fused import BatchNormActivation
+    Rs = synth.irreps(8, 3)
+    n_gates = sum(m for m, l in Rs[1:])
+    bn = BatchNorm(Rs + [(n_gates, 0)]).to(dev)
+    act = Activation(Rs, (torch.relu, torch.sigmoid)).to(dev)
+    fused = BatchNormActivation(bn, act).train()
+    n_rows = 600000
+    c_in = bn.num_channels
+    c_out = c_in - n_gates
+    x = torch.randn(n_rows, c_in, device=dev)
+    zi = torch.zeros(n_rows, 4, dtype=torch.int32, device=dev)
+    with torch.no_grad():
+        ms, _ = timed(lambda: fused(SparseTensor(x, zi, [64] * 3, 32)), n=10)
+        report("BatchNorm+Activation fused, training (%d rows, %d->%d ch)" % (n_rows, c_in, c_out),
+               ms, 4 * n_rows * (3 * c_in + c_out), "statistics read the rows twice")
+        fused.eval()
+        ms, _ = timed(lambda: fused(SparseTensor(x, zi, [64] * 3, 32)), n=10)
+        report("BatchNorm+Activation fused, evaluation", ms, 4 * n_rows * (c_in + c_out))
+        fused.train()
+        keep = bnact.usable
+        bnact.usable = lambda t: False   # the layers' torch code, for comparison
+        try:
+            ms, _ = timed(lambda: fused(SparseTensor(x, zi, [64] * 3, 32)), n=10)
+        finally:
+            bnact.usable = keep
+        report("same layers as torch ops, training", ms, 4 * n_rows * (3 * c_in + c_out),
+               "same algorithmic bytes")
+    xg = x.clone().requires_grad_(True)
+    dy = torch.randn(n_rows, c_out, device=dev)
+
+    def step():
+        y = fused(SparseTensor(xg, zi, [64] * 3, 32)).features
+        y.backward(dy)
+        xg.grad = None
+    ms, _ = timed(step, n=10)
+    nbytes = 4 * n_rows * (3 * c_in + c_out + 2 * (c_in + c_out) + c_in)
+    report("BatchNorm+Activation fused, forward + backward", ms, nbytes,
+           "backward reads rows and gradients twice")
+    keep = bnact.usable
+    bnact.usable = lambda t: False
+    try:
+        ms, _ = timed(step, n=5)
+    finally:
+        bnact.usable = keep
+    report("same layers as torch ops, forward + backward", ms, nbytes, "same algorithmic bytes")
     print("\n".join(rows), file=sys.stderr)
 
 

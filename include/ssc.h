@@ -328,6 +328,80 @@ int ssc_three_interp_bwd_f32(int32_t c, int32_t n, int32_t m, const float *out_g
                              const int32_t *idx, const float *weight,
                              float *points_grad /* [m,c] */, ssc_stream_t stream);
 
+/* ------------------------------------------------------------------------
+ * SE(3) batch normalisation and gated non-linearity over feature rows [n, c_in].
+ * Replace the torch code of BatchNorm.forward (ss_conv/batchnorm.py:49-136) and
+ * Activation._gate (ss_conv/activation.py:55-100) and their autograd.
+ *
+ * Channel layout, described once per layer by int32 tables on the device:
+ *   field_of[c]     field (block of 2l+1 columns) of input column c
+ *   scalar_idx[c]   ordinal of column c among the scalar (l = 0) columns, -1 otherwise
+ *   field_first[f], field_dim[f]   first column and number of columns of field f
+ *   out_mode[j]     for output column j < c_out: 0 copy, 1 scalar activation,
+ *                   2 multiplied by the activation of its gate (NULL: all 0)
+ *   gate_col[j]     input column of the gate of output column j (read when mode 2)
+ *   gated_first[c], gated_dim[c]   for a gate column c >= c_out: the output columns
+ *                   it gates (dim 0 or NULL: none)
+ *
+ * ssc_bn_prepare_f32 turns statistics into per-column constants:
+ *   training != 0: shift = column mean for scalar columns (0 elsewhere); norm of a
+ *     field = mean over rows of the sum of its (x - shift)^2; running_mean /
+ *     running_var move by `momentum` towards them (batchnorm.py:73-100)
+ *   training == 0: shift and norm are the running statistics
+ *   scale[c] = weight[field] / sqrt(norm[field] + eps)   (weight NULL: 1)
+ *   add[c]   = bias[scalar_idx[c]] for scalar columns    (bias NULL: 0)
+ *   field_rstd[f] = 1 / sqrt(norm[f] + eps)
+ * ssc_bnact_fwd_f32: z = (x - shift) * scale + add (a NULL vector is the identity);
+ *   y[:, j] = z_j | act_scalar(z_j + pre_bias[j]) | z_j * act_gate(z_g + pre_bias[g]).
+ * ssc_bnact_bwd_sums_f32: with dz = dL/dz of every input column (the activation's
+ *   chain rule applied to dy), sums[c] = sum over rows of dz, sums[c_in + c] = sum
+ *   over rows of dz * (x - shift): what the parameter gradients and the gradient
+ *   through the batch statistics need.
+ * ssc_bnact_bwd_f32: dx = scale * (dz - dz_mean) - coef * (x - shift)
+ *   (dz_mean / coef NULL: 0; the caller derives them from the sums).
+ * Sums are accumulated per block of rows and added in block order: reproducible.
+ * ---------------------------------------------------------------------- */
+#define SSC_ACT_NONE 0
+#define SSC_ACT_RELU 1
+#define SSC_ACT_SIGMOID 2
+#define SSC_ACT_TANH 3
+
+size_t ssc_bn_workspace_bytes(int64_t n, int32_t c);
+
+int ssc_bn_prepare_f32(const float *x /* [n,c] */, int64_t n, int32_t c, const int32_t *field_of,
+                       const int32_t *scalar_idx, const int32_t *field_first,
+                       const int32_t *field_dim, int32_t n_fields, int32_t training, float eps,
+                       float momentum, const float *weight /* [n_fields] or NULL */,
+                       const float *bias /* [n_scalar] or NULL */,
+                       float *running_mean /* [n_scalar], in/out */,
+                       float *running_var /* [n_fields], in/out */, float *shift /* [c] */,
+                       float *scale /* [c] */, float *add /* [c] */,
+                       float *field_rstd /* [n_fields] */, void *workspace,
+                       size_t workspace_bytes, ssc_stream_t stream);
+
+int ssc_bnact_fwd_f32(const float *x /* [n,c_in] */, int64_t n, int32_t c_in, const float *shift,
+                      const float *scale, const float *add, const float *pre_bias /* [c_in] */,
+                      const int32_t *out_mode /* [c_out] */, const int32_t *gate_col /* [c_out] */,
+                      int32_t act_scalar, int32_t act_gate, float *y /* [n,c_out] */,
+                      int32_t c_out, ssc_stream_t stream);
+
+int ssc_bnact_bwd_sums_f32(const float *x, const float *dy /* [n,c_out] */, int64_t n,
+                           int32_t c_in, int32_t c_out, const float *shift, const float *scale,
+                           const float *add, const float *pre_bias, const int32_t *out_mode,
+                           const int32_t *gate_col, const int32_t *gated_first /* [c_in] */,
+                           const int32_t *gated_dim /* [c_in] */, int32_t act_scalar,
+                           int32_t act_gate, float *sums /* [2*c_in] */, void *workspace,
+                           size_t workspace_bytes /* ssc_bn_workspace_bytes(n, c_in) */,
+                           ssc_stream_t stream);
+
+int ssc_bnact_bwd_f32(const float *x, const float *dy, int64_t n, int32_t c_in, int32_t c_out,
+                      const float *shift, const float *scale, const float *add,
+                      const float *pre_bias, const int32_t *out_mode, const int32_t *gate_col,
+                      const int32_t *gated_first, const int32_t *gated_dim, int32_t act_scalar,
+                      int32_t act_gate, const float *dz_mean /* [c_in] or NULL */,
+                      const float *coef /* [c_in] or NULL */, float *dx /* [n,c_in] */,
+                      ssc_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

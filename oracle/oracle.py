@@ -558,3 +558,199 @@ def combine(weight, bases, mults_out, dims_out, mults_in, dims_in, size):
         rows.append(np.concatenate(cols, axis=1))
     assert off == weight.size
     return np.concatenate(rows, axis=0).astype(np.float32)
+
+
+# ---- SE(3) batch norm and gated non-linearity ---------------------------------------------
+_ACTS = {
+    None: (lambda u: u, lambda u: np.ones_like(u)),
+    "relu": (lambda u: np.maximum(u, 0.0), lambda u: (u > 0).astype(u.dtype)),
+    "sigmoid": (lambda u: 1.0 / (1.0 + np.exp(-u)),
+                lambda u: (1.0 / (1.0 + np.exp(-u))) * (1.0 - 1.0 / (1.0 + np.exp(-u)))),
+    "tanh": (lambda u: np.tanh(u), lambda u: 1.0 - np.tanh(u) ** 2),
+}
+
+
+def batchnorm_fwd(x, Rs, weight=None, bias=None, running_mean=None, running_var=None, eps=1e-5,
+                  momentum=0.1, training=True, dtype=np.float64):
+    """The reference's field loop (ss_conv/batchnorm.py:49-136), field by field:
+    scalars are centred by their (batch or running) mean, every field is divided by the root
+    of its (batch or running) mean squared norm plus eps, then weight per field and bias per
+    scalar.  Returns (y, running_mean', running_var'), the running statistics moved by
+    `momentum` when training (batchnorm.py:45-46)."""
+    x = np.asarray(x, dtype=dtype)
+    n = x.shape[0]
+    n_scalar = sum(m for m, l in Rs if l == 0)
+    n_field = sum(m for m, l in Rs)
+    rm = np.zeros(n_scalar, dtype) if running_mean is None else np.asarray(running_mean, dtype).copy()
+    rv = np.ones(n_field, dtype) if running_var is None else np.asarray(running_var, dtype).copy()
+    new_rm, new_rv = rm.copy(), rv.copy()
+    out = []
+    ix = irm = irv = iw = ib = 0
+    for m, l in Rs:
+        d = 2 * l + 1
+        field = x[:, ix:ix + m * d].reshape(n, m, d)
+        ix += m * d
+        if d == 1:
+            if training:
+                mean = field.mean(0).reshape(-1)
+                new_rm[irm:irm + m] = (1 - momentum) * rm[irm:irm + m] + momentum * mean
+            else:
+                mean = rm[irm:irm + m]
+            irm += m
+            field = field - mean.reshape(1, m, 1)
+        if training:
+            norm = (field ** 2).sum(2).mean(0)
+            new_rv[irv:irv + m] = (1 - momentum) * rv[irv:irv + m] + momentum * norm
+        else:
+            norm = rv[irv:irv + m]
+        irv += m
+        scale = (norm + eps) ** -0.5
+        if weight is not None:
+            scale = scale * np.asarray(weight, dtype)[iw:iw + m]
+            iw += m
+        field = field * scale.reshape(1, m, 1)
+        if bias is not None and d == 1:
+            field = field + np.asarray(bias, dtype)[ib:ib + m].reshape(1, m, 1)
+            ib += m
+        out.append(field.reshape(n, m * d))
+    assert ix == x.shape[1]
+    return np.concatenate(out, axis=1), new_rm, new_rv
+
+
+def gate_fwd(y, Rs, scalar_bias=None, gate_bias=None, act_scalar=None, act_gate=None,
+             dtype=np.float64):
+    """Activation._gate (ss_conv/activation.py:55-100): the first entry of Rs, if scalar, goes
+    through act_scalar(y + scalar_bias); every non-scalar field is multiplied by
+    act_gate(g + gate_bias) of its gate scalar, the gates being the columns after the
+    fields.  An activation given as None leaves its columns unchanged (and, for the gates,
+    drops the gate columns unused)."""
+    y = np.asarray(y, dtype=dtype)
+    n = y.shape[0]
+    out_dim = sum(m * (2 * l + 1) for m, l in Rs)
+    gates = None
+    if act_gate is not None:
+        g = y[:, out_dim:]
+        if gate_bias is not None:
+            g = g + np.asarray(gate_bias, dtype).reshape(1, -1)
+        gates = _ACTS[act_gate][0](g)
+    z = np.empty((n, out_dim), dtype)
+    begin_y = begin_g = 0
+    for i, (m, l) in enumerate(Rs):
+        if m == 0:
+            continue
+        d = 2 * l + 1
+        field = y[:, begin_y:begin_y + m * d]
+        if l == 0:
+            if act_scalar is not None and i == 0:
+                if scalar_bias is not None:
+                    field = field + np.asarray(scalar_bias, dtype).reshape(1, -1)
+                field = _ACTS[act_scalar][0](field)
+        elif gates is not None:
+            fg = gates[:, begin_g:begin_g + m].reshape(n, m, 1)
+            field = (field.reshape(n, m, d) * fg).reshape(n, m * d)
+            begin_g += m
+        z[:, begin_y:begin_y + m * d] = field
+        begin_y += m * d
+    return z
+
+
+def bn_gate_fwd(x, Rs_bn, Rs_act, params, eps=1e-5, training=True, act_scalar="relu",
+                act_gate="sigmoid", running=None):
+    """gate_fwd(batchnorm_fwd(x)) with params = dict(weight, bias, scalar_bias, gate_bias);
+    Rs_act None: batch norm alone; Rs_bn None: the gate alone."""
+    y = np.asarray(x, dtype=np.float64)
+    if Rs_bn is not None:
+        rm, rv = running if running is not None else (None, None)
+        y, _, _ = batchnorm_fwd(y, Rs_bn, params.get("weight"), params.get("bias"), rm, rv, eps,
+                                0.1, training)
+    if Rs_act is not None:
+        y = gate_fwd(y, Rs_act, params.get("scalar_bias"), params.get("gate_bias"), act_scalar,
+                     act_gate)
+    return y
+
+
+def bn_gate_bwd(x, dy, Rs_bn, Rs_act, params, eps=1e-5, training=True, act_scalar="relu",
+                act_gate="sigmoid", running=None):
+    """Gradients of sum(dy * bn_gate_fwd(x)) with respect to x and to every entry of params,
+    by the chain rule through the two layers (what torch autograd computes for the
+    reference's modules; pinned against central differences of bn_gate_fwd).
+    Returns dict(x=..., weight=..., bias=..., scalar_bias=..., gate_bias=...)."""
+    x = np.asarray(x, dtype=np.float64)
+    dy = np.asarray(dy, dtype=np.float64)
+    n, c_in = x.shape
+    grads = {}
+    # ---- forward pieces
+    if Rs_bn is not None:
+        cols = []
+        for m, l in Rs_bn:
+            for _ in range(m):
+                cols.append(2 * l + 1)
+        field_of = np.repeat(np.arange(len(cols)), cols)
+        is_scalar = np.repeat(np.array(cols) == 1, cols)
+        rm, rv = running if running is not None else (np.zeros(is_scalar.sum()), np.ones(len(cols)))
+        shift = np.zeros(c_in)
+        shift[is_scalar] = x[:, is_scalar].mean(0) if training else np.asarray(rm, np.float64)
+        xc = x - shift
+        if training:
+            norm = np.zeros(len(cols))
+            np.add.at(norm, field_of, (xc ** 2).mean(0))
+        else:
+            norm = np.asarray(rv, np.float64)
+        rstd = (norm + eps) ** -0.5
+        w = np.ones(len(cols)) if params.get("weight") is None else np.asarray(params["weight"], np.float64)
+        scale = (rstd * w)[field_of]
+        add = np.zeros(c_in)
+        if params.get("bias") is not None:
+            add[is_scalar] = np.asarray(params["bias"], np.float64)
+        z = xc * scale + add
+    else:
+        z = x
+    # ---- through the gate: dz
+    if Rs_act is not None:
+        out_dim = sum(m * (2 * l + 1) for m, l in Rs_act)
+        dz = np.zeros_like(z)
+        sb, gb = params.get("scalar_bias"), params.get("gate_bias")
+        col = g = 0
+        for i, (m, l) in enumerate(Rs_act):
+            d = 2 * l + 1
+            for _ in range(m):
+                sl = slice(col, col + d)
+                if l == 0:
+                    if act_scalar is not None and i == 0:
+                        u = z[:, sl] + (0.0 if sb is None else np.asarray(sb, np.float64)[col:col + d])
+                        dz[:, sl] = dy[:, sl] * _ACTS[act_scalar][1](u)
+                    else:
+                        dz[:, sl] = dy[:, sl]
+                elif act_gate is not None:
+                    gc = out_dim + g
+                    u = z[:, gc] + (0.0 if gb is None else np.asarray(gb, np.float64)[g])
+                    dz[:, sl] = dy[:, sl] * _ACTS[act_gate][0](u)[:, None]
+                    dz[:, gc] = (dy[:, sl] * z[:, sl]).sum(1) * _ACTS[act_gate][1](u)
+                    g += 1
+                else:
+                    dz[:, sl] = dy[:, sl]
+                col += d
+        m0 = Rs_act[0][0] if (Rs_act[0][1] == 0 and act_scalar is not None) else 0
+        if sb is not None:
+            grads["scalar_bias"] = dz[:, :m0].sum(0)
+        if gb is not None:
+            grads["gate_bias"] = dz[:, out_dim:out_dim + g].sum(0)
+    else:
+        dz = dy
+    # ---- through the batch norm
+    if Rs_bn is not None:
+        col_b = dz.sum(0)
+        field_a = np.zeros(len(cols))
+        np.add.at(field_a, field_of, (dz * xc).sum(0))
+        if params.get("bias") is not None:
+            grads["bias"] = col_b[is_scalar]
+        if params.get("weight") is not None:
+            grads["weight"] = rstd * field_a
+        dx = dz * scale
+        if training:
+            dx = dx - np.where(is_scalar, col_b / n, 0.0) * scale
+            dx = dx - (scale * (rstd ** 2 * field_a)[field_of] / n) * xc
+        grads["x"] = dx
+    else:
+        grads["x"] = dz
+    return grads

@@ -1,0 +1,647 @@
+// SE(3) batch normalisation and gated non-linearity over feature rows [N, C], as
+// bandwidth-bound kernels: the statistics take two reads of the features, the
+// fused normalise + gate pass one read and one write.
+//
+// Channel layout (the layout of the reference layers, ss_conv/batchnorm.py:49-136 and
+// ss_conv/activation.py:55-100): C_in columns = the fields of Rs (2l+1 columns each)
+// followed by one gate scalar per non-scalar field; the output keeps the first C_out
+// columns.  Tables describe it once per layer:
+//   field_of[c]     field of input column c            scalar_idx[c]  ordinal of c among
+//   field_first[f]  first column of field f                           the scalar columns,
+//   field_dim[f]    columns of field f                                -1 for the others
+//   out_mode[j]     0 copy, 1 scalar activation, 2 multiplied by its gate
+//   gate_col[j]     input column of the gate of output column j (mode 2)
+//   gated_first[c], gated_dim[c]   for a gate column c: the output columns it gates
+//
+// Threads run along the columns (coalesced rows), so what belongs to a column sits in
+// registers; a block covers a slab of rows and writes one partial sum per column, and
+// the partials are added in block order: the same result on every run.
+#include "ssc_common.h"
+
+namespace ssc {
+
+constexpr int kBnThreads = 256;
+constexpr int kBnMaxBlocks = 1024;
+constexpr int kBnMaxBwdChannels = 1536;  // column tables of the backward kernels: 48 KB of LDS
+
+struct BnShape {
+  int tx, ty;             // threads along columns / rows (tx * ty == kBnThreads)
+  int rows_per_block;
+  int blocks;
+};
+
+// `c` counts the units a thread handles: columns, or groups of four columns.
+static BnShape bn_shape(int64_t n, int c) {
+  BnShape s;
+  s.tx = 16;
+  while (s.tx < c && s.tx < kBnThreads) s.tx <<= 1;
+  s.ty = kBnThreads / s.tx;
+  int64_t rpb = ceil_div(n > 0 ? n : 1, kBnMaxBlocks);
+  rpb = ceil_div(rpb, s.ty) * s.ty;  // whole trips of the row lanes
+  if (rpb < 4 * s.ty) rpb = 4 * s.ty;
+  s.rows_per_block = (int)rpb;
+  s.blocks = (int)ceil_div(n > 0 ? n : 1, rpb);
+  return s;
+}
+
+__device__ __forceinline__ float act_fn(int kind, float u) {
+  switch (kind) {
+    case SSC_ACT_RELU: return u > 0.f ? u : 0.f;
+    case SSC_ACT_SIGMOID: return 1.f / (1.f + __expf(-u));
+    case SSC_ACT_TANH: return tanhf(u);
+    default: return u;
+  }
+}
+// derivative of act_fn at u
+__device__ __forceinline__ float act_grad(int kind, float u) {
+  switch (kind) {
+    case SSC_ACT_RELU: return u > 0.f ? 1.f : 0.f;
+    case SSC_ACT_SIGMOID: {
+      float s = 1.f / (1.f + __expf(-u));
+      return s * (1.f - s);
+    }
+    case SSC_ACT_TANH: {
+      float t = tanhf(u);
+      return 1.f - t * t;
+    }
+    default: return 1.f;
+  }
+}
+
+// Sum over the row lanes of a block, in lane order; valid in row lane 0.
+__device__ __forceinline__ float reduce_rows(float v, float *red, int tx, int ty, int TX, int TY) {
+  red[ty * TX + tx] = v;
+  __syncthreads();
+  float s = 0.f;
+  if (ty == 0)
+    for (int i = 0; i < TY; ++i) s += red[i * TX + tx];
+  __syncthreads();
+  return s;
+}
+
+// Kernels that stream the rows come in two widths: V = 4 (a thread owns four
+// consecutive columns and moves 16 bytes per access; needs column counts divisible by
+// four) and V = 1.
+template <int V> struct Vec;
+template <> struct Vec<1> {
+  float v[1];
+  __device__ __forceinline__ void load(const float *p) { v[0] = p[0]; }
+  __device__ __forceinline__ void store(float *p) const { p[0] = v[0]; }
+};
+template <> struct Vec<4> {
+  float v[4];
+  __device__ __forceinline__ void load(const float *p) {
+    float4 t = *reinterpret_cast<const float4 *>(p);
+    v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+  }
+  __device__ __forceinline__ void store(float *p) const {
+    *reinterpret_cast<float4 *>(p) = make_float4(v[0], v[1], v[2], v[3]);
+  }
+};
+
+// partial[b*C + c] = sum over the rows of block b of x[r,c] (SQUARE == 0) or of
+// (x[r,c] - shift[c])^2 (SQUARE == 1).
+template <int SQUARE, int V>
+__global__ void __launch_bounds__(kBnThreads)
+    bn_partial_kernel(const float *__restrict__ x, int64_t n, int C, int TX, int rows_per_block,
+                      const float *__restrict__ shift, float *__restrict__ partial) {
+  __shared__ float red[kBnThreads];
+  const int TY = kBnThreads / TX;
+  const int tx = threadIdx.x % TX, ty = threadIdx.x / TX;
+  const int64_t r0 = (int64_t)blockIdx.x * rows_per_block;
+  const int64_t r1 = r0 + rows_per_block < n ? r0 + rows_per_block : n;
+  for (int c0 = 0; c0 < C; c0 += TX * V) {
+    const int c = c0 + tx * V;
+    float acc[2][V];
+    float sh[V];
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+      acc[0][i] = acc[1][i] = 0.f;
+      sh[i] = (SQUARE && c + i < C) ? shift[c + i] : 0.f;
+    }
+    if (c < C) {
+      int64_t r = r0 + ty;
+      for (; r + TY < r1; r += 2 * TY) {  // two rows in flight
+        Vec<V> a, b;
+        a.load(x + r * C + c);
+        b.load(x + (r + TY) * C + c);
+#pragma unroll
+        for (int i = 0; i < V; ++i) {
+          float va = a.v[i] - sh[i], vb = b.v[i] - sh[i];
+          acc[0][i] += SQUARE ? va * va : va;
+          acc[1][i] += SQUARE ? vb * vb : vb;
+        }
+      }
+      if (r < r1) {
+        Vec<V> a;
+        a.load(x + r * C + c);
+#pragma unroll
+        for (int i = 0; i < V; ++i) {
+          float va = a.v[i] - sh[i];
+          acc[0][i] += SQUARE ? va * va : va;
+        }
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+      float s = reduce_rows(acc[0][i] + acc[1][i], red, tx, ty, TX, TY);
+      if (ty == 0 && c + i < C) partial[(int64_t)blockIdx.x * C + c + i] = s;
+    }
+  }
+}
+
+// out[c] = inv_n * sum over blocks of partial[b*C + c]; with scalar_idx, 0 for the
+// columns that are not scalars.  16 columns x 16 slices of the blocks per workgroup; a
+// column's slices are added in slice order.
+__global__ void __launch_bounds__(256)
+    bn_colsum_kernel(const float *__restrict__ partial, int nb, int C, double inv_n,
+                     const int32_t *__restrict__ scalar_idx, float *__restrict__ out) {
+  __shared__ double red[16][16];
+  const int cx = threadIdx.x & 15, part = threadIdx.x >> 4;
+  const int c = blockIdx.x * 16 + cx;
+  double s = 0.0;
+  if (c < C && (scalar_idx == nullptr || scalar_idx[c] >= 0))
+    for (int b = part; b < nb; b += 16) s += partial[(int64_t)b * C + c];
+  red[part][cx] = s;
+  __syncthreads();
+  if (part == 0 && c < C) {
+    double t = 0.0;
+    for (int i = 0; i < 16; ++i) t += red[i][cx];
+    out[c] = (float)(t * inv_n);
+  }
+}
+
+// One block.  From the column mean squares (training) or the running statistics
+// (evaluation): per-column shift / scale / add, per-field 1/sqrt(norm + eps), and the
+// running statistics' update (reference: batchnorm.py:73-112).
+__global__ void __launch_bounds__(256)
+    bn_finalize_kernel(int C, int training, float eps, float momentum,
+                       const int32_t *__restrict__ field_of,
+                       const int32_t *__restrict__ scalar_idx,
+                       const int32_t *__restrict__ field_first,
+                       const int32_t *__restrict__ field_dim, int n_fields,
+                       const float *__restrict__ weight, const float *__restrict__ bias,
+                       float *__restrict__ running_mean, float *__restrict__ running_var,
+                       float *__restrict__ shift, float *__restrict__ scale,
+                       float *__restrict__ add, float *__restrict__ field_rstd,
+                       const float *__restrict__ col_msq /* [C], training only */) {
+  if (training) {
+    for (int c = threadIdx.x; c < C; c += blockDim.x) {
+      const int si = scalar_idx[c];
+      if (si >= 0) running_mean[si] = (1.f - momentum) * running_mean[si] + momentum * shift[c];
+    }
+  } else {
+    for (int c = threadIdx.x; c < C; c += blockDim.x) {
+      const int si = scalar_idx[c];
+      shift[c] = si >= 0 ? running_mean[si] : 0.f;
+    }
+  }
+  __syncthreads();
+  for (int f = threadIdx.x; f < n_fields; f += blockDim.x) {
+    float norm;
+    if (training) {
+      norm = 0.f;
+      for (int j = 0; j < field_dim[f]; ++j) norm += col_msq[field_first[f] + j];
+      running_var[f] = (1.f - momentum) * running_var[f] + momentum * norm;
+    } else {
+      norm = running_var[f];
+    }
+    field_rstd[f] = 1.f / sqrtf(norm + eps);
+  }
+  __syncthreads();
+  for (int c = threadIdx.x; c < C; c += blockDim.x) {
+    const int f = field_of[c];
+    scale[c] = field_rstd[f] * (weight ? weight[f] : 1.f);
+    const int si = scalar_idx[c];
+    add[c] = (bias && si >= 0) ? bias[si] : 0.f;
+  }
+}
+
+// Per-column constants of the normalisation (identity when the pointers are null).
+struct ColAffine {
+  const float *shift, *scale, *add, *pre_bias;
+  __device__ __forceinline__ float z(float x, int c) const {
+    float v = x;
+    if (shift) v -= shift[c];
+    if (scale) v *= scale[c];
+    if (add) v += add[c];
+    return v;
+  }
+  __device__ __forceinline__ float pb(int c) const { return pre_bias ? pre_bias[c] : 0.f; }
+};
+
+// y[r, j] = activation of the normalised x[r, j] (see out_mode above)
+template <int V>
+__global__ void __launch_bounds__(kBnThreads)
+    bnact_fwd_kernel(const float *__restrict__ x, int64_t n, int c_in, int c_out, int TX,
+                     int rows_per_block, ColAffine aff, const int32_t *__restrict__ out_mode,
+                     const int32_t *__restrict__ gate_col, int act_s, int act_g,
+                     float *__restrict__ y) {
+  const int TY = kBnThreads / TX;
+  const int tx = threadIdx.x % TX, ty = threadIdx.x / TX;
+  const int64_t r0 = (int64_t)blockIdx.x * rows_per_block;
+  const int64_t r1 = r0 + rows_per_block < n ? r0 + rows_per_block : n;
+  for (int j = tx * V; j < c_out; j += TX * V) {
+    int mode[V], g[V];
+    float sh[V], sc[V], ad[V], pbj[V], gsh[V], gsc[V], gad[V];
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+      const int c = j + i < c_out ? j + i : j;  // V == 4 only with c_out % 4 == 0
+      mode[i] = out_mode ? out_mode[c] : 0;
+      g[i] = mode[i] == 2 ? gate_col[c] : c;
+      sh[i] = aff.shift ? aff.shift[c] : 0.f;
+      sc[i] = aff.scale ? aff.scale[c] : 1.f;
+      ad[i] = aff.add ? aff.add[c] : 0.f;
+      pbj[i] = aff.pb(c);
+      gsh[i] = aff.shift ? aff.shift[g[i]] : 0.f;
+      gsc[i] = aff.scale ? aff.scale[g[i]] : 1.f;
+      gad[i] = (aff.add ? aff.add[g[i]] : 0.f) + aff.pb(g[i]);
+    }
+    for (int64_t r = r0 + ty; r < r1; r += TY) {
+      const float *xr = x + r * c_in;
+      Vec<V> a;
+      a.load(xr + j);
+#pragma unroll
+      for (int i = 0; i < V; ++i) {
+        float v = (a.v[i] - sh[i]) * sc[i] + ad[i];
+        if (mode[i] == 1) {
+          v = act_fn(act_s, v + pbj[i]);
+        } else if (mode[i] == 2) {
+          // the columns of a field share their gate: neighbouring lanes read the same word
+          float gv = (xr[g[i]] - gsh[i]) * gsc[i] + gad[i];
+          v *= act_fn(act_g, gv);
+        }
+        a.v[i] = v;
+      }
+      a.store(y + r * c_out + j);
+    }
+  }
+}
+
+// Per-column constants and tables of the backward kernels, staged in LDS once per block:
+// the row loops then read nothing but rows from memory.
+struct ColTables {
+  float *shift, *scale, *add, *pre;      // [c_in]
+  int *mode, *gate, *gfirst, *gdim;      // [c_in] (mode/gate: output columns only)
+  __device__ __forceinline__ float z(float x, int c) const {
+    return (x - shift[c]) * scale[c] + add[c];
+  }
+};
+
+__device__ __forceinline__ ColTables stage_tables(float *lds, int c_in, int c_out,
+                                                  const ColAffine &aff,
+                                                  const int32_t *__restrict__ out_mode,
+                                                  const int32_t *__restrict__ gate_col,
+                                                  const int32_t *__restrict__ gated_first,
+                                                  const int32_t *__restrict__ gated_dim) {
+  ColTables t;
+  t.shift = lds;
+  t.scale = lds + c_in;
+  t.add = lds + 2 * c_in;
+  t.pre = lds + 3 * c_in;
+  t.mode = reinterpret_cast<int *>(lds + 4 * c_in);
+  t.gate = t.mode + c_in;
+  t.gfirst = t.mode + 2 * c_in;
+  t.gdim = t.mode + 3 * c_in;
+  for (int c = threadIdx.x; c < c_in; c += blockDim.x) {
+    t.shift[c] = aff.shift ? aff.shift[c] : 0.f;
+    t.scale[c] = aff.scale ? aff.scale[c] : 1.f;
+    t.add[c] = aff.add ? aff.add[c] : 0.f;
+    t.pre[c] = aff.pre_bias ? aff.pre_bias[c] : 0.f;
+    t.mode[c] = (out_mode && c < c_out) ? out_mode[c] : 0;
+    t.gate[c] = (out_mode && c < c_out && out_mode[c] == 2) ? gate_col[c] : c;
+    t.gfirst[c] = gated_dim ? gated_first[c] : 0;
+    t.gdim[c] = (gated_dim && c >= c_out) ? gated_dim[c] : 0;
+  }
+  __syncthreads();
+  return t;
+}
+
+// Gradient reaching the normalised value of input column c at row r (xr, dr: the row
+// of x and of dy; xc = xr[c]).
+__device__ __forceinline__ float bnact_dz(const float *__restrict__ xr,
+                                          const float *__restrict__ dr, float xc, int c, int c_out,
+                                          const ColTables &t, int act_s, int act_g) {
+  if (c < c_out) {
+    const int mode = t.mode[c];
+    float d = dr[c];
+    if (mode == 1) {
+      d *= act_grad(act_s, t.z(xc, c) + t.pre[c]);
+    } else if (mode == 2) {
+      const int g = t.gate[c];
+      d *= act_fn(act_g, t.z(xr[g], g) + t.pre[g]);
+    }
+    return d;
+  }
+  const int dim = t.gdim[c];
+  if (dim <= 0) return 0.f;
+  const int first = t.gfirst[c];
+  float acc = 0.f;
+  for (int j = first; j < first + dim; ++j) acc += dr[j] * t.z(xr[j], j);
+  return acc * act_grad(act_g, t.z(xc, c) + t.pre[c]);
+}
+
+// Work items of the backward kernels: the output columns in groups of V, then the gate
+// columns one by one (a gate's gradient sums over its whole field, about as much work
+// as a group of plain columns).
+struct BwdItem {
+  int c;       // first column
+  int width;   // V for a group, 1 for a gate column, 0 beyond the last item
+};
+template <int V>
+__device__ __forceinline__ BwdItem bwd_item(int it, int c_in, int c_out) {
+  const int nvec = c_out / V;
+  BwdItem w;
+  if (it < nvec) {
+    w.c = it * V;
+    w.width = V;
+  } else {
+    w.c = c_out + (it - nvec);
+    w.width = w.c < c_in ? 1 : 0;
+  }
+  return w;
+}
+static int bwd_items(int c_in, int c_out, int V) { return c_out / V + (c_in - c_out); }
+
+// partial[b*2C + c] = sum of dz over the rows of block b, partial[b*2C + C + c] = sum of
+// dz * (x - shift)
+template <int V>
+__global__ void __launch_bounds__(kBnThreads)
+    bnact_bwd_partial_kernel(const float *__restrict__ x, const float *__restrict__ dy, int64_t n,
+                             int c_in, int c_out, int TX, int rows_per_block, ColAffine aff,
+                             const int32_t *__restrict__ out_mode,
+                             const int32_t *__restrict__ gate_col,
+                             const int32_t *__restrict__ gated_first,
+                             const int32_t *__restrict__ gated_dim, int act_s, int act_g,
+                             float *__restrict__ partial) {
+  __shared__ float red[kBnThreads];
+  extern __shared__ float lds[];
+  const ColTables t =
+      stage_tables(lds, c_in, c_out, aff, out_mode, gate_col, gated_first, gated_dim);
+  const int TY = kBnThreads / TX;
+  const int tx = threadIdx.x % TX, ty = threadIdx.x / TX;
+  const int64_t r0 = (int64_t)blockIdx.x * rows_per_block;
+  const int64_t r1 = r0 + rows_per_block < n ? r0 + rows_per_block : n;
+  const int n_items = c_out / V + (c_in - c_out);
+  for (int it0 = 0; it0 < n_items; it0 += TX) {
+    const BwdItem w = bwd_item<V>(it0 + tx, c_in, c_out);
+    float sb[V], sa[V], sh[V];
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+      sb[i] = sa[i] = 0.f;
+      sh[i] = i < w.width ? t.shift[w.c + i] : 0.f;
+    }
+    if (w.width == V) {
+      for (int64_t r = r0 + ty; r < r1; r += TY) {
+        const float *xr = x + r * c_in;
+        const float *dr = dy + r * c_out;
+        Vec<V> a;
+        a.load(xr + w.c);
+#pragma unroll
+        for (int i = 0; i < V; ++i) {
+          float d = bnact_dz(xr, dr, a.v[i], w.c + i, c_out, t, act_s, act_g);
+          sb[i] += d;
+          sa[i] += d * (a.v[i] - sh[i]);
+        }
+      }
+    } else if (w.width == 1) {
+      for (int64_t r = r0 + ty; r < r1; r += TY) {
+        const float *xr = x + r * c_in;
+        const float xc = xr[w.c];
+        float d = bnact_dz(xr, dy + r * c_out, xc, w.c, c_out, t, act_s, act_g);
+        sb[0] += d;
+        sa[0] += d * (xc - sh[0]);
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+      float tb = reduce_rows(sb[i], red, tx, ty, TX, TY);
+      float ta = reduce_rows(sa[i], red, tx, ty, TX, TY);
+      if (ty == 0 && i < w.width) {
+        partial[(int64_t)blockIdx.x * 2 * c_in + w.c + i] = tb;
+        partial[(int64_t)blockIdx.x * 2 * c_in + c_in + w.c + i] = ta;
+      }
+    }
+  }
+}
+
+// dx[r,c] = scale[c] * (dz - dz_mean[c]) - coef[c] * (x[r,c] - shift[c])
+template <int V>
+__global__ void __launch_bounds__(kBnThreads)
+    bnact_bwd_kernel(const float *__restrict__ x, const float *__restrict__ dy, int64_t n, int c_in,
+                     int c_out, int TX, int rows_per_block, ColAffine aff,
+                     const int32_t *__restrict__ out_mode, const int32_t *__restrict__ gate_col,
+                     const int32_t *__restrict__ gated_first,
+                     const int32_t *__restrict__ gated_dim, int act_s, int act_g,
+                     const float *__restrict__ dz_mean, const float *__restrict__ coef,
+                     float *__restrict__ dx) {
+  extern __shared__ float lds[];
+  const ColTables t =
+      stage_tables(lds, c_in, c_out, aff, out_mode, gate_col, gated_first, gated_dim);
+  const int TY = kBnThreads / TX;
+  const int tx = threadIdx.x % TX, ty = threadIdx.x / TX;
+  const int64_t r0 = (int64_t)blockIdx.x * rows_per_block;
+  const int64_t r1 = r0 + rows_per_block < n ? r0 + rows_per_block : n;
+  const int n_items = c_out / V + (c_in - c_out);
+  for (int it = tx; it < n_items; it += TX) {
+    const BwdItem w = bwd_item<V>(it, c_in, c_out);
+    float sh[V], sc[V], dm[V], cf[V];
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+      const int k = i < w.width ? w.c + i : w.c;
+      sh[i] = t.shift[k];
+      sc[i] = t.scale[k];
+      dm[i] = dz_mean ? dz_mean[k] : 0.f;
+      cf[i] = coef ? coef[k] : 0.f;
+    }
+    if (w.width == V) {
+      for (int64_t r = r0 + ty; r < r1; r += TY) {
+        const float *xr = x + r * c_in;
+        const float *dr = dy + r * c_out;
+        Vec<V> a;
+        a.load(xr + w.c);
+#pragma unroll
+        for (int i = 0; i < V; ++i) {
+          float d = bnact_dz(xr, dr, a.v[i], w.c + i, c_out, t, act_s, act_g);
+          a.v[i] = sc[i] * (d - dm[i]) - cf[i] * (a.v[i] - sh[i]);
+        }
+        a.store(dx + r * c_in + w.c);
+      }
+    } else if (w.width == 1) {
+      for (int64_t r = r0 + ty; r < r1; r += TY) {
+        const float *xr = x + r * c_in;
+        const float xc = xr[w.c];
+        float d = bnact_dz(xr, dy + r * c_out, xc, w.c, c_out, t, act_s, act_g);
+        dx[r * c_in + w.c] = sc[0] * (d - dm[0]) - cf[0] * (xc - sh[0]);
+      }
+    }
+  }
+}
+
+// bytes of LDS for the staged column tables
+static size_t bn_tables_lds(int c_in) { return (size_t)c_in * 8 * sizeof(float); }
+
+// Partial sums of at most kBnMaxBlocks row slabs (whatever the thread layout), two per
+// column, plus one vector of column values.
+static size_t bn_ws_bytes(int64_t n, int c) {
+  int64_t blocks = n < kBnMaxBlocks ? (n > 0 ? n : 1) : kBnMaxBlocks;
+  return align_up((size_t)blocks * 2 * c * sizeof(float)) + align_up((size_t)c * sizeof(float));
+}
+
+static bool act_ok(int a) { return a >= SSC_ACT_NONE && a <= SSC_ACT_TANH; }
+
+}  // namespace ssc
+
+using namespace ssc;
+
+extern "C" {
+
+size_t ssc_bn_workspace_bytes(int64_t n, int32_t c) {
+  if (n < 0 || c < 1) return 0;
+  return bn_ws_bytes(n, c);
+}
+
+int ssc_bn_prepare_f32(const float *x, int64_t n, int32_t c, const int32_t *field_of,
+                       const int32_t *scalar_idx, const int32_t *field_first,
+                       const int32_t *field_dim, int32_t n_fields, int32_t training, float eps,
+                       float momentum, const float *weight, const float *bias,
+                       float *running_mean, float *running_var, float *shift, float *scale,
+                       float *add, float *field_rstd, void *workspace, size_t workspace_bytes,
+                       ssc_stream_t stream) {
+  SSC_CHECK(n >= 0 && c >= 1 && n_fields >= 1, SSC_EINVAL, "negative or empty size");
+  SSC_CHECK(field_of && scalar_idx && field_first && field_dim && running_var && shift && scale &&
+                add && field_rstd && workspace,
+            SSC_EINVAL, "NULL pointer argument");
+  SSC_CHECK(!training || n > 0, SSC_EINVAL, "batch statistics of an empty batch");
+  SSC_CHECK(!training || x != nullptr, SSC_EINVAL, "x is NULL");
+  size_t need = bn_ws_bytes(n, c);
+  SSC_CHECK(workspace_bytes >= need, SSC_EWORKSPACE, "batch-norm workspace too small: %zu < %zu",
+            workspace_bytes, need);
+  hipStream_t s = (hipStream_t)stream;
+  const int V = (c & 3) == 0 ? 4 : 1;
+  BnShape sh = bn_shape(n, c / V);
+  Carver cv(workspace);
+  float *partial = cv.take<float>((size_t)sh.blocks * 2 * c);
+  float *col_msq = cv.take<float>((size_t)c);
+  const double inv_n = n > 0 ? 1.0 / (double)n : 0.0;
+  if (training) {
+    if (V == 4)
+      hipLaunchKernelGGL((bn_partial_kernel<0, 4>), dim3(sh.blocks), dim3(kBnThreads), 0, s, x, n,
+                         c, sh.tx, sh.rows_per_block, (const float *)nullptr, partial);
+    else
+      hipLaunchKernelGGL((bn_partial_kernel<0, 1>), dim3(sh.blocks), dim3(kBnThreads), 0, s, x, n,
+                         c, sh.tx, sh.rows_per_block, (const float *)nullptr, partial);
+    hipLaunchKernelGGL(bn_colsum_kernel, dim3((unsigned)ceil_div(c, 16)), dim3(256), 0, s, partial,
+                       sh.blocks, c, inv_n, scalar_idx, shift);
+    if (V == 4)
+      hipLaunchKernelGGL((bn_partial_kernel<1, 4>), dim3(sh.blocks), dim3(kBnThreads), 0, s, x, n,
+                         c, sh.tx, sh.rows_per_block, shift, partial);
+    else
+      hipLaunchKernelGGL((bn_partial_kernel<1, 1>), dim3(sh.blocks), dim3(kBnThreads), 0, s, x, n,
+                         c, sh.tx, sh.rows_per_block, shift, partial);
+  }
+  if (training)
+    hipLaunchKernelGGL(bn_colsum_kernel, dim3((unsigned)ceil_div(c, 16)), dim3(256), 0, s, partial,
+                       sh.blocks, c, inv_n, (const int32_t *)nullptr, col_msq);
+  hipLaunchKernelGGL(bn_finalize_kernel, dim3(1), dim3(256), 0, s, c, training, eps, momentum,
+                     field_of, scalar_idx, field_first, field_dim,
+                     n_fields, weight, bias, running_mean, running_var, shift, scale, add,
+                     field_rstd, col_msq);
+  SSC_LAUNCH_CHECK("bn_prepare");
+  return SSC_OK;
+}
+
+int ssc_bnact_fwd_f32(const float *x, int64_t n, int32_t c_in, const float *shift,
+                      const float *scale, const float *add, const float *pre_bias,
+                      const int32_t *out_mode, const int32_t *gate_col, int32_t act_scalar,
+                      int32_t act_gate, float *y, int32_t c_out, ssc_stream_t stream) {
+  SSC_CHECK(n >= 0 && c_in >= 1 && c_out >= 1 && c_out <= c_in, SSC_EINVAL,
+            "bad shape: n %lld, c_in %d, c_out %d", (long long)n, c_in, c_out);
+  SSC_CHECK(act_ok(act_scalar) && act_ok(act_gate), SSC_EINVAL, "unknown activation code");
+  if (n == 0) return SSC_OK;
+  SSC_CHECK(x && y, SSC_EINVAL, "NULL pointer argument");
+  SSC_CHECK(out_mode == nullptr || gate_col != nullptr, SSC_EINVAL, "gate_col is NULL");
+  const int V = ((c_in | c_out) & 3) == 0 ? 4 : 1;
+  BnShape sh = bn_shape(n, c_out / V);
+  ColAffine aff = {shift, scale, add, pre_bias};
+  if (V == 4)
+    hipLaunchKernelGGL(bnact_fwd_kernel<4>, dim3(sh.blocks), dim3(kBnThreads), 0,
+                       (hipStream_t)stream, x, n, c_in, c_out, sh.tx, sh.rows_per_block, aff,
+                       out_mode, gate_col, act_scalar, act_gate, y);
+  else
+    hipLaunchKernelGGL(bnact_fwd_kernel<1>, dim3(sh.blocks), dim3(kBnThreads), 0,
+                       (hipStream_t)stream, x, n, c_in, c_out, sh.tx, sh.rows_per_block, aff,
+                       out_mode, gate_col, act_scalar, act_gate, y);
+  SSC_LAUNCH_CHECK("bnact_fwd");
+  return SSC_OK;
+}
+
+int ssc_bnact_bwd_sums_f32(const float *x, const float *dy, int64_t n, int32_t c_in, int32_t c_out,
+                           const float *shift, const float *scale, const float *add,
+                           const float *pre_bias, const int32_t *out_mode,
+                           const int32_t *gate_col, const int32_t *gated_first,
+                           const int32_t *gated_dim, int32_t act_scalar, int32_t act_gate,
+                           float *sums, void *workspace, size_t workspace_bytes,
+                           ssc_stream_t stream) {
+  SSC_CHECK(n >= 0 && c_in >= 1 && c_out >= 1 && c_out <= c_in, SSC_EINVAL,
+            "bad shape: n %lld, c_in %d, c_out %d", (long long)n, c_in, c_out);
+  SSC_CHECK(act_ok(act_scalar) && act_ok(act_gate), SSC_EINVAL, "unknown activation code");
+  SSC_CHECK(c_in <= kBnMaxBwdChannels, SSC_EINVAL, "at most %d channels in the backward pass",
+            kBnMaxBwdChannels);
+  SSC_CHECK(sums && workspace, SSC_EINVAL, "NULL pointer argument");
+  SSC_CHECK(n == 0 || (x && dy), SSC_EINVAL, "NULL pointer argument");
+  size_t need = bn_ws_bytes(n, c_in);
+  SSC_CHECK(workspace_bytes >= need, SSC_EWORKSPACE, "batch-norm workspace too small: %zu < %zu",
+            workspace_bytes, need);
+  hipStream_t s = (hipStream_t)stream;
+  if (n == 0) return fill_f32(sums, 2 * (int64_t)c_in, 0.f, s);
+  const int V = ((c_in | c_out) & 3) == 0 ? 4 : 1;
+  BnShape sh = bn_shape(n, bwd_items(c_in, c_out, V));
+  float *partial = static_cast<float *>(workspace);
+  ColAffine aff = {shift, scale, add, pre_bias};
+  if (V == 4)
+    hipLaunchKernelGGL(bnact_bwd_partial_kernel<4>, dim3(sh.blocks), dim3(kBnThreads),
+                       bn_tables_lds(c_in), s, x, dy,
+                       n, c_in, c_out, sh.tx, sh.rows_per_block, aff, out_mode, gate_col,
+                       gated_first, gated_dim, act_scalar, act_gate, partial);
+  else
+    hipLaunchKernelGGL(bnact_bwd_partial_kernel<1>, dim3(sh.blocks), dim3(kBnThreads),
+                       bn_tables_lds(c_in), s, x, dy,
+                       n, c_in, c_out, sh.tx, sh.rows_per_block, aff, out_mode, gate_col,
+                       gated_first, gated_dim, act_scalar, act_gate, partial);
+  hipLaunchKernelGGL(bn_colsum_kernel, dim3((unsigned)ceil_div(2 * c_in, 16)), dim3(256), 0, s,
+                     partial, sh.blocks, 2 * c_in, 1.0, (const int32_t *)nullptr, sums);
+  SSC_LAUNCH_CHECK("bnact_bwd_sums");
+  return SSC_OK;
+}
+
+int ssc_bnact_bwd_f32(const float *x, const float *dy, int64_t n, int32_t c_in, int32_t c_out,
+                      const float *shift, const float *scale, const float *add,
+                      const float *pre_bias, const int32_t *out_mode, const int32_t *gate_col,
+                      const int32_t *gated_first, const int32_t *gated_dim, int32_t act_scalar,
+                      int32_t act_gate, const float *dz_mean, const float *coef, float *dx,
+                      ssc_stream_t stream) {
+  SSC_CHECK(n >= 0 && c_in >= 1 && c_out >= 1 && c_out <= c_in, SSC_EINVAL,
+            "bad shape: n %lld, c_in %d, c_out %d", (long long)n, c_in, c_out);
+  SSC_CHECK(act_ok(act_scalar) && act_ok(act_gate), SSC_EINVAL, "unknown activation code");
+  SSC_CHECK(c_in <= kBnMaxBwdChannels, SSC_EINVAL, "at most %d channels in the backward pass",
+            kBnMaxBwdChannels);
+  if (n == 0) return SSC_OK;
+  SSC_CHECK(x && dy && dx, SSC_EINVAL, "NULL pointer argument");
+  const int V = ((c_in | c_out) & 3) == 0 ? 4 : 1;
+  BnShape sh = bn_shape(n, bwd_items(c_in, c_out, V));
+  ColAffine aff = {shift, scale, add, pre_bias};
+  if (V == 4)
+    hipLaunchKernelGGL(bnact_bwd_kernel<4>, dim3(sh.blocks), dim3(kBnThreads),
+                       bn_tables_lds(c_in), (hipStream_t)stream, x, dy, n, c_in, c_out, sh.tx, sh.rows_per_block, aff,
+                       out_mode, gate_col, gated_first, gated_dim, act_scalar, act_gate, dz_mean,
+                       coef, dx);
+  else
+    hipLaunchKernelGGL(bnact_bwd_kernel<1>, dim3(sh.blocks), dim3(kBnThreads),
+                       bn_tables_lds(c_in), (hipStream_t)stream, x, dy, n, c_in, c_out, sh.tx, sh.rows_per_block, aff,
+                       out_mode, gate_col, gated_first, gated_dim, act_scalar, act_gate, dz_mean,
+                       coef, dx);
+  SSC_LAUNCH_CHECK("bnact_bwd");
+  return SSC_OK;
+}
+}

@@ -143,55 +143,50 @@ __global__ void __launch_bounds__(256)
 }
 
 // segs[t*K + k] = first pair of offset k whose scatter row is >= the first row of
-// tile t (t = 0..n_tiles).  Tile rows come from tile_row0[] and the tile count from
-// n_tiles_dev[0]; with tile_row0 == nullptr the tiles are `granule` rows each and
-// there are n_cap of them (the fine grid the work split is computed on).
-// With fine_segs != nullptr (segments of a grid of `granule` rows, computed before) the
-// search starts from the grid cell of the tile's first row instead of the whole list.
-// With spill_end != nullptr also spill[t*K + k] = how far the last row block of tile
-// t-1 may reach into tile t: the first pair at or after segs[t*K + k], at most 15
-// further, whose row is >= spill_end[t].
+// tile t (t = 0..n_tiles; tile rows from tile_row0[], tile count from n_tiles_dev[0]).
+// The search starts from the cell of the tile's first row in grid_segs[], the same
+// segments for a regular grid of `granule` rows (grid_segments_kernel).
+// Also spill[t*K + k] = how far the last row block of tile t-1 may reach into tile t:
+// the first pair at or after segs[t*K + k], at most 15 further, whose row is >=
+// spill_end[t].
 __global__ void __launch_bounds__(256)
     tile_segments_kernel(const int32_t *__restrict__ flag, const int32_t *__restrict__ pairs,
                          const int32_t *__restrict__ sorted, int64_t pair_stride, int plane_s,
-                         const int32_t *__restrict__ pair_num, int K, int64_t n_cap,
+                         const int32_t *__restrict__ pair_num, int K,
                          const int32_t *__restrict__ n_tiles_dev,
-                         const int32_t *__restrict__ tile_row0, int granule, int64_t n_out,
-                         int32_t *__restrict__ segs, const int32_t *__restrict__ fine_segs,
-                         const int32_t *__restrict__ spill_end, int32_t *__restrict__ spill) {
+                         const int32_t *__restrict__ tile_row0, int64_t n_out,
+                         const int32_t *__restrict__ grid_segs, int granule,
+                         const int32_t *__restrict__ spill_end, int32_t *__restrict__ segs,
+                         int32_t *__restrict__ spill) {
   int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  const int64_t n_tiles = tile_row0 ? n_tiles_dev[0] : n_cap;
+  const int64_t n_tiles = n_tiles_dev[0];
   if (idx >= (n_tiles + 1) * K) return;
   int64_t t = idx / K;
   int k = (int)(idx - t * K);
   const int32_t *src = flag[0] ? sorted : pairs;
   const int32_t *s = src + ((int64_t)k * 2 + plane_s) * pair_stride;
-  int64_t target = tile_row0 ? (int64_t)tile_row0[t] : t * (int64_t)granule;
+  int64_t target = tile_row0[t];
   if (target > n_out) target = n_out;
-  int lo = 0, hi = pair_num[k];
-  if (fine_segs) {
-    const int64_t cell = target / granule;  // target <= n_out: a cell of the grid or its end
-    lo = fine_segs[cell * K + k];
-    if ((cell + 1) * granule <= n_out) hi = fine_segs[(cell + 1) * K + k];
-  }
+  const int n = pair_num[k];
+  const int64_t cell = target / granule;  // a cell of the grid, or its end
+  int lo = grid_segs[cell * K + k];
+  int hi = (cell + 1) * granule <= n_out ? grid_segs[(cell + 1) * K + k] : n;
   while (lo < hi) {
     int mid = (lo + hi) >> 1;
     if (s[mid] < target) lo = mid + 1;
     else hi = mid;
   }
   segs[idx] = lo;
-  if (spill_end) {
-    const int bound = spill_end[t];
-    const int n = pair_num[k];
-    int cnt = 0;
+  const int bound = spill_end[t];
+  int cnt = 0;
 #pragma unroll
-    for (int j = 0; j < 15; ++j) cnt += (lo + j < n && s[lo + j] < bound) ? 1 : 0;  // rows ascend
-    spill[idx] = lo + cnt;
-  }
+  for (int j = 0; j < 15; ++j) cnt += (lo + j < n && s[lo + j] < bound) ? 1 : 0;  // rows ascend
+  spill[idx] = lo + cnt;
 }
 
-// The same segments for a regular grid of `granule` rows (cells c = 0..n_cells, cell
-// n_cells being the end), computed from the pairs' side: one thread per pair; the pair
+// segs[c*K + k] = first pair of offset k whose scatter row is >= c*granule, for the
+// cells c = 0..n_cells of a regular grid (cell n_cells being the end), computed from
+// the pairs' side: one thread per pair; the pair
 // that is the first of its offset at or beyond a cell boundary writes that boundary.
 __global__ void __launch_bounds__(256)
     grid_segments_kernel(const int32_t *__restrict__ flag, const int32_t *__restrict__ pairs,
@@ -1297,9 +1292,8 @@ int ssc_conv_fwd_f32(const float *features, int64_t n_in, int32_t c_in, const fl
   SSC_LAUNCH_CHECK("split");
   int64_t nseg = (p.n_tiles + 1) * K;
   hipLaunchKernelGGL(tile_segments_kernel, dim3((unsigned)ceil_div(nseg, 256)), dim3(256), 0, s,
-                     w.flag, pairs, w.sorted, pair_stride, plane_s, pair_num, K, p.n_tiles,
-                     w.n_tiles_dev, w.tile_row0, kSplitGranule, n_out, w.segs, w.fine_segs,
-                     w.spill_end, w.spill);
+                     w.flag, pairs, w.sorted, pair_stride, plane_s, pair_num, K, w.n_tiles_dev,
+                     w.tile_row0, n_out, w.fine_segs, kSplitGranule, w.spill_end, w.segs, w.spill);
   SSC_LAUNCH_CHECK("tile_segments");
   hipLaunchKernelGGL(share_kernel, dim3((unsigned)ceil_div((int64_t)p.n_wg * K, 256)), dim3(256),
                      0, s, w.segs, w.spill, K, p.n_wg, w.wg_tile, w.share_first, w.share_cnt);

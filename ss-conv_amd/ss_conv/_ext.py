@@ -84,6 +84,16 @@ _SIGNATURES = {
     "ssc_voxel_reduce_f32": (ctypes.c_int, [_vp, _vp, _vp, _i32, _i32, _i32, _i32, _vp]),
     "ssc_three_nn": (ctypes.c_int, [_i32, _i32, _vp, _vp, _vp, _vp, _vp]),
     "ssc_three_interp_f32": (ctypes.c_int, [_i32, _i32, _i32, _vp, _vp, _vp, _vp, _vp]),
+    "ssc_bn_workspace_bytes": (_sz, [_i64, _i32]),
+    "ssc_bn_prepare_f32": (ctypes.c_int, [_vp, _i64, _i32, _vp, _vp, _vp, _vp, _i32, _i32,
+                                          ctypes.c_float, ctypes.c_float, _vp, _vp, _vp, _vp, _vp,
+                                          _vp, _vp, _vp, _vp, _sz, _vp]),
+    "ssc_bnact_fwd_f32": (ctypes.c_int, [_vp, _i64, _i32, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32,
+                                         _vp, _i32, _vp]),
+    "ssc_bnact_bwd_sums_f32": (ctypes.c_int, [_vp, _vp, _i64, _i32, _i32, _vp, _vp, _vp, _vp, _vp,
+                                              _vp, _vp, _vp, _i32, _i32, _vp, _vp, _sz, _vp]),
+    "ssc_bnact_bwd_f32": (ctypes.c_int, [_vp, _vp, _i64, _i32, _i32, _vp, _vp, _vp, _vp, _vp, _vp,
+                                         _vp, _vp, _i32, _i32, _vp, _vp, _vp, _vp]),
 }
 
 for _name, (_res, _args) in _SIGNATURES.items():
@@ -549,6 +559,68 @@ def unique_rows(coords, dims, return_counts=True):
     _check(_lib.ssc_unique_emit(_ptr(coords), n, d, ws.data_ptr(), ws.numel(), m.value, _ptr(uniq),
                                 _ptr(inverse), _ptr(counts), s))
     return uniq, inverse, counts
+
+
+ACT_NONE, ACT_RELU, ACT_SIGMOID, ACT_TANH = 0, 1, 2, 3
+
+
+def bn_prepare(x, layout, training, eps, momentum, weight, bias, running_mean, running_var):
+    """Per-column constants of the SE(3) batch norm (reference: batchnorm.py:73-112).
+    `layout` holds the int32 tables field_of, scalar_idx, field_first, field_dim.
+    Updates the running statistics in place when training.
+    Returns (shift[c], scale[c], add[c], field_rstd[n_fields])."""
+    _need_gpu(x)
+    n, c = x.size(0), x.size(1)
+    dev = x.device
+    n_fields = layout["field_first"].numel()
+    shift = torch.empty(c, dtype=torch.float32, device=dev)
+    scale = torch.empty(c, dtype=torch.float32, device=dev)
+    add = torch.empty(c, dtype=torch.float32, device=dev)
+    rstd = torch.empty(n_fields, dtype=torch.float32, device=dev)
+    ws = _workspace(_lib.ssc_bn_workspace_bytes(n, c), dev)
+    _check(_lib.ssc_bn_prepare_f32(
+        _ptr(x), n, c, layout["field_of"].data_ptr(), layout["scalar_idx"].data_ptr(),
+        layout["field_first"].data_ptr(), layout["field_dim"].data_ptr(), n_fields,
+        int(bool(training)), float(eps), float(momentum), _ptr(weight), _ptr(bias),
+        _ptr(running_mean), running_var.data_ptr(), shift.data_ptr(), scale.data_ptr(),
+        add.data_ptr(), rstd.data_ptr(), ws.data_ptr(), ws.numel(), _stream(x)))
+    return shift, scale, add, rstd
+
+
+def bnact_forward(x, shift, scale, add, pre_bias, out_mode, gate_col, act_scalar, act_gate, c_out):
+    """y[n, c_out] = gated activation of the normalised rows (activation.py:55-100)."""
+    _need_gpu(x)
+    y = torch.empty((x.size(0), c_out), dtype=torch.float32, device=x.device)
+    _check(_lib.ssc_bnact_fwd_f32(_ptr(x), x.size(0), x.size(1), _ptr(shift), _ptr(scale),
+                                  _ptr(add), _ptr(pre_bias), _ptr(out_mode), _ptr(gate_col),
+                                  int(act_scalar), int(act_gate), _ptr(y), c_out, _stream(x)))
+    return y
+
+
+def bnact_backward_sums(x, dy, shift, scale, add, pre_bias, out_mode, gate_col, gated_first,
+                        gated_dim, act_scalar, act_gate):
+    """sums[2, c_in]: per input column the sum over rows of dz and of dz * (x - shift)."""
+    _need_gpu(x, dy)
+    n, c_in = x.size(0), x.size(1)
+    sums = torch.empty((2, c_in), dtype=torch.float32, device=x.device)
+    ws = _workspace(_lib.ssc_bn_workspace_bytes(n, c_in), x.device)
+    _check(_lib.ssc_bnact_bwd_sums_f32(
+        _ptr(x), _ptr(dy), n, c_in, dy.size(1), _ptr(shift), _ptr(scale), _ptr(add),
+        _ptr(pre_bias), _ptr(out_mode), _ptr(gate_col), _ptr(gated_first), _ptr(gated_dim),
+        int(act_scalar), int(act_gate), sums.data_ptr(), ws.data_ptr(), ws.numel(), _stream(x)))
+    return sums
+
+
+def bnact_backward(x, dy, shift, scale, add, pre_bias, out_mode, gate_col, gated_first, gated_dim,
+                   act_scalar, act_gate, dz_mean, coef):
+    """dx = scale * (dz - dz_mean) - coef * (x - shift)."""
+    _need_gpu(x, dy)
+    dx = torch.empty_like(x)
+    _check(_lib.ssc_bnact_bwd_f32(
+        _ptr(x), _ptr(dy), x.size(0), x.size(1), dy.size(1), _ptr(shift), _ptr(scale), _ptr(add),
+        _ptr(pre_bias), _ptr(out_mode), _ptr(gate_col), _ptr(gated_first), _ptr(gated_dim),
+        int(act_scalar), int(act_gate), _ptr(dz_mean), _ptr(coef), _ptr(dx), _stream(x)))
+    return dx
 
 
 def profile_conv(enable):

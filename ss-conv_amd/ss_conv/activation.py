@@ -8,6 +8,7 @@ import torch
 import torch.nn as nn
 import torch.utils.checkpoint
 
+from ss_conv import bnact
 from ss_conv.utils.utils import Rs2dim
 
 
@@ -84,9 +85,43 @@ class Activation(nn.Module):
         self.register_buffer('_gate_of', torch.tensor(gate_of, dtype=torch.long),
                              persistent=False)
 
+        # the library's kernel covers identity / relu / sigmoid / tanh on the usual layout
+        # (scalars first); other layers keep the torch code below
+        self._codes = (bnact.activation_code(scalar_activation if self.scalar_act is not None
+                                             else None),
+                       bnact.activation_code(gate_activation if self.gate_act is not None
+                                             else None))
+        self._kernel_ok = None not in self._codes and bnact.canonical(self.Rs)
+        if self._kernel_ok:
+            self._tables_cpu, self._c_out, self._n_gates = bnact.gate_layout(
+                self.Rs, self.scalar_act is not None, self.gate_act is not None)
+        self._tables_dev = {}
+
+    def fill_plan(self, plan, device):
+        """Add the activation half to a bnact.BnActPlan."""
+        key = str(device)
+        if key not in self._tables_dev:
+            self._tables_dev[key] = bnact.to_device(self._tables_cpu, device)
+        plan.act = self._tables_dev[key]
+        plan.act_scalar, plan.act_gate = self._codes
+        plan.c_out = self._c_out
+        plan.n_scalar_act = self.multiplicities[0] if self.scalar_act is not None else 0
+        plan.n_gates = self._n_gates
+        return plan
+
+    def biases(self):
+        return (self.scalar_act.bias if self.scalar_act is not None else None,
+                self.gate_act.bias if self.gate_act is not None else None)
+
     def forward(self, input):
         if self.scalar_act is not None or self.gate_act is not None:
             features = input.features
+            if (self._kernel_ok and bnact.usable(features) and features.size(0) > 0
+                    and features.size(1) == self._c_out + self._n_gates):
+                sb, gb = self.biases()
+                input.features = bnact.bn_act(features, None, None, sb, gb,
+                                              self.fill_plan(bnact.BnActPlan(), features.device))
+                return input
             if self.checkpoint and torch.is_grad_enabled() and features.requires_grad:
                 features = torch.utils.checkpoint.checkpoint(self._gate, features,
                                                              use_reentrant=False)

@@ -5,10 +5,14 @@ Scalar fields are centred by their mean; every field (a block of 2l+1 channels)
 is divided by the root of its mean squared norm.  Buffers and parameters keep
 the reference's names and shapes: running_mean [scalars], running_var [fields],
 weight [fields], bias [scalars].  The per-field loop of the reference is
-replaced by index tables, so the layer is a handful of torch ops whatever Rs is.
+replaced by index tables.  Float32 features on the GPU run on the library's kernels
+(two reads of the rows for the statistics, one read and one write to normalise, and a
+hand-written backward pass); anything else takes the torch ops below.
 """
 import torch
 import torch.nn as nn
+
+from ss_conv import bnact
 
 
 class BatchNorm(nn.Module):
@@ -46,6 +50,27 @@ class BatchNorm(nn.Module):
                              persistent=False)
         self.register_buffer('_scalar_cols', torch.tensor(scalar_cols, dtype=torch.long),
                              persistent=False)
+        self._layout_cpu = bnact.field_layout(Rs)
+        self._layout_dev = {}
+
+    def layout(self, device):
+        """Channel tables of the kernels on `device`."""
+        key = str(device)
+        if key not in self._layout_dev:
+            self._layout_dev[key] = bnact.to_device(self._layout_cpu, device)
+        return self._layout_dev[key]
+
+    def plan(self, device):
+        """The batch-norm half of a bnact.BnActPlan."""
+        p = bnact.BnActPlan()
+        p.bn = self.layout(device)
+        p.training = self.training
+        p.eps = self.eps
+        p.momentum = self.momentum
+        p.running_mean = self.running_mean
+        p.running_var = self.running_var
+        p.c_out = self.num_channels
+        return p
 
     def __repr__(self):
         return "{} (Rs={}, eps={}, momentum={})".format(self.__class__.__name__, self.Rs, self.eps,
@@ -61,6 +86,10 @@ class BatchNorm(nn.Module):
                 x.size(1), self.num_channels))
         if self.reduce != 'mean':
             raise ValueError("Invalid reduce option {}".format(self.reduce))
+        if bnact.usable(x) and x.size(0) > 0:
+            input.features = bnact.bn_act(x, self.weight, self.bias, None, None,
+                                          self.plan(x.device))
+            return input
         n_fields = self.running_var.numel()
         shift = x.new_zeros(self.num_channels)
         if self._scalar_cols.numel() > 0:

@@ -682,3 +682,121 @@ def test_cpu_tensor_is_rejected(device):
     with pytest.raises(RuntimeError):
         _ext.get_indice_pairs_3d(torch.zeros((1, 4), dtype=torch.int32), 1, [8] * 3, [8] * 3,
                                  [3] * 3, [1] * 3, [1] * 3, [1] * 3, [0] * 3, 0, 0)
+
+
+# ---- SE(3) batch norm + gated non-linearity ---------------------------------------------------
+BNACT_CASES = [
+    # Rs of the activation, rows, layers ("bn", "act", "fused"), training
+    ([(4, 0), (4, 1), (4, 2)], 1000, "fused", True),
+    ([(4, 0), (4, 1), (4, 2)], 1000, "fused", False),
+    ([(4, 0), (4, 1), (4, 2)], 777, "bn", True),
+    ([(4, 0), (4, 1), (4, 2)], 777, "bn", False),
+    ([(4, 0), (4, 1), (4, 2)], 777, "act", True),
+    ([(3, 0), (2, 1), (2, 2)], 333, "fused", True),            # 23 columns: the scalar-width kernels
+    ([(3, 0), (2, 1), (2, 2)], 333, "act", True),
+    ([(8, 0), (8, 1), (8, 2), (8, 3), (8, 4)], 5000, "fused", True),   # 232 columns
+    ([(32, 0), (32, 1), (32, 2), (32, 3)], 3000, "fused", True),       # 608 columns: several passes
+    ([(2, 0), (1, 1)], 3, "fused", True),
+    ([(16, 0)], 100, "fused", True),                                   # scalars only, no gates
+]
+
+
+def _bnact_modules(Rs, acts, device, rng):
+    from ss_conv.activation import Activation
+    from ss_conv.batchnorm import BatchNorm
+    n_gates = sum(m for m, _ in Rs[1:])
+    Rs_bn = list(Rs) + ([(n_gates, 0)] if n_gates else [])
+    bn = BatchNorm(Rs_bn).to(device)
+    act = Activation(Rs, acts).to(device)
+    with torch.no_grad():
+        for p in list(bn.parameters()) + list(act.parameters()):
+            p.copy_(torch.from_numpy(rng.normal(size=tuple(p.shape)).astype(np.float32)))
+        bn.weight.add_(1.0)
+        bn.running_mean.copy_(torch.from_numpy(rng.normal(size=tuple(bn.running_mean.shape)).astype(np.float32)))
+        bn.running_var.copy_(torch.from_numpy(rng.uniform(0.5, 2, size=tuple(bn.running_var.shape)).astype(np.float32)))
+    return bn, act, Rs_bn
+
+
+@pytest.mark.parametrize("case", BNACT_CASES)
+def test_batchnorm_activation_match_oracle(case, oracle, device):
+    from ss_conv.fused import BatchNormActivation
+    from ss_conv.sp_ops.tensor import SparseTensor
+    Rs, n, which, training = case
+    print("case", case, flush=True)
+    rng = np.random.default_rng(len(Rs) * 1000 + n)
+    bn, act, Rs_bn = _bnact_modules(Rs, (torch.relu, torch.sigmoid), device, rng)
+    c_in = sum(m * (2 * l + 1) for m, l in Rs_bn)
+    x_np = (rng.normal(size=(n, c_in)) * 2 + 0.3).astype(np.float32)
+    x = torch.from_numpy(x_np).to(device).requires_grad_(True)
+    module = {"bn": bn, "act": act, "fused": BatchNormActivation(bn, act)}[which]
+    module.train(training)
+    running = (bn.running_mean.cpu().numpy().copy(), bn.running_var.cpu().numpy().copy())
+    st = SparseTensor(x, torch.zeros(n, 4, dtype=torch.int32, device=device), [4, 4, 4], 1)
+    y = module(st).features
+    dy_np = rng.normal(size=tuple(y.shape)).astype(np.float32)
+    y.backward(torch.from_numpy(dy_np).to(device))
+    torch.cuda.synchronize()
+
+    sb = act.scalar_act.bias if act.scalar_act is not None else None
+    gb = act.gate_act.bias if act.gate_act is not None else None
+    as_np = lambda t: None if t is None else t.detach().cpu().numpy()  # noqa: E731
+    params = dict(weight=as_np(bn.weight), bias=as_np(bn.bias), scalar_bias=as_np(sb),
+                  gate_bias=as_np(gb))
+    use_bn, use_act = which in ("bn", "fused"), which in ("act", "fused")
+    kw = dict(training=training, act_scalar="relu", act_gate="sigmoid" if gb is not None else None,
+              running=running)
+    args = (Rs_bn if use_bn else None, Rs if use_act else None, params)
+    want = oracle.bn_gate_fwd(x_np, *args, **kw)
+    assert rel_l2(y.detach().cpu().numpy(), want) < REL_L2
+    grads = oracle.bn_gate_bwd(x_np, dy_np, *args, **kw)
+    assert rel_l2(x.grad.cpu().numpy(), grads["x"]) < REL_L2
+    got = dict(weight=bn.weight.grad, bias=bn.bias.grad, scalar_bias=None if sb is None else sb.grad,
+               gate_bias=None if gb is None else gb.grad)
+    for k, g in grads.items():
+        if k == "x":
+            continue
+        assert got[k] is not None, k
+        assert rel_l2(got[k].cpu().numpy(), g) < 1e-4, k   # sums over all rows in fp32
+    if use_bn and training:
+        _, rm, rv = oracle.batchnorm_fwd(x_np, Rs_bn, params["weight"], params["bias"], *running)
+        assert rel_l2(bn.running_mean.cpu().numpy(), rm) < REL_L2
+        assert rel_l2(bn.running_var.cpu().numpy(), rv) < REL_L2
+
+
+def test_batchnorm_activation_other_cases(oracle, device):
+    """tanh activations, layers without bias or affine parameters, an activation the kernels
+    do not cover (torch code on the GPU), and reproducibility."""
+    from ss_conv.activation import Activation
+    from ss_conv.batchnorm import BatchNorm
+    from ss_conv.fused import BatchNormActivation
+    from ss_conv.sp_ops.tensor import SparseTensor
+    rng = np.random.default_rng(77)
+    Rs = [(4, 0), (3, 1), (2, 2)]
+    Rs_bn = Rs + [(5, 0)]
+    n, c_in = 600, 4 + 9 + 10 + 5
+    x_np = rng.normal(size=(n, c_in)).astype(np.float32)
+    idx = torch.zeros(n, 4, dtype=torch.int32, device=device)
+
+    def run(bn, act):
+        m = BatchNormActivation(bn, act).to(device).train()
+        st = SparseTensor(torch.from_numpy(x_np).to(device), idx, [4, 4, 4], 1)
+        return m(st).features.detach().cpu().numpy()
+
+    y = run(BatchNorm(Rs_bn, affine=False), Activation(Rs, (torch.tanh, torch.tanh), bias=False))
+    want = oracle.bn_gate_fwd(x_np, Rs_bn, Rs, {}, act_scalar="tanh", act_gate="tanh")
+    assert rel_l2(y, want) < REL_L2
+    y = run(BatchNorm(Rs_bn), Activation(Rs, (None, torch.sigmoid)))
+    want = oracle.bn_gate_fwd(x_np, Rs_bn, Rs, {}, act_scalar=None, act_gate="sigmoid")
+    assert rel_l2(y, want) < REL_L2
+    y1 = run(BatchNorm(Rs_bn), Activation(Rs, (torch.relu, torch.sigmoid)))
+    y2 = run(BatchNorm(Rs_bn), Activation(Rs, (torch.relu, torch.sigmoid)))
+    assert np.array_equal(y1, y2)
+    # softplus is not one of the kernels' activations: the layers fall back to torch ops
+    soft = torch.nn.functional.softplus
+    act = Activation(Rs, (soft, torch.sigmoid))
+    assert not act._kernel_ok
+    y = run(BatchNorm(Rs_bn), act)
+    z, _, _ = oracle.batchnorm_fwd(x_np, Rs_bn)
+    z[:, :4] = np.log1p(np.exp(z[:, :4]))
+    want = oracle.gate_fwd(z, Rs, act_scalar=None, act_gate="sigmoid")
+    assert rel_l2(y, want) < REL_L2
