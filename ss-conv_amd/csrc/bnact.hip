@@ -341,18 +341,48 @@ __device__ __forceinline__ float bnact_dz(const float *__restrict__ xr,
   return acc * act_grad(act_g, t.z(xc, c) + t.pre[c]);
 }
 
+// What a thread keeps in registers for its group of V output columns.
+template <int V> struct GroupConst {
+  int mode[V], g[V];
+  float sh[V], sc[V], ad[V], pre[V], gsh[V], gsc[V], gadp[V];
+  __device__ __forceinline__ void init(const ColTables &t, int c0) {
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+      const int c = c0 + i;
+      mode[i] = t.mode[c];
+      g[i] = t.gate[c];
+      sh[i] = t.shift[c];
+      sc[i] = t.scale[c];
+      ad[i] = t.add[c];
+      pre[i] = t.pre[c];
+      gsh[i] = t.shift[g[i]];
+      gsc[i] = t.scale[g[i]];
+      gadp[i] = t.add[g[i]] + t.pre[g[i]];
+    }
+  }
+  // dz of column i of the group: x and dy of the column, xr the row of x
+  __device__ __forceinline__ float dz(int i, float x, float dy, const float *__restrict__ xr,
+                                      int act_s, int act_g) const {
+    if (mode[i] == 1) return dy * act_grad(act_s, (x - sh[i]) * sc[i] + ad[i] + pre[i]);
+    if (mode[i] == 2) return dy * act_fn(act_g, (xr[g[i]] - gsh[i]) * gsc[i] + gadp[i]);
+    return dy;
+  }
+};
+
 // Work items of the backward kernels: the output columns in groups of V, then the gate
 // columns one by one (a gate's gradient sums over its whole field, about as much work
 // as a group of plain columns).
 struct BwdItem {
   int c;       // first column
   int width;   // V for a group, 1 for a gate column, 0 beyond the last item
+  bool group;  // a group of output columns (not a gate column)
 };
 template <int V>
 __device__ __forceinline__ BwdItem bwd_item(int it, int c_in, int c_out) {
   const int nvec = c_out / V;
   BwdItem w;
-  if (it < nvec) {
+  w.group = it < nvec;
+  if (w.group) {
     w.c = it * V;
     w.width = V;
   } else {
@@ -391,15 +421,17 @@ __global__ void __launch_bounds__(kBnThreads)
       sb[i] = sa[i] = 0.f;
       sh[i] = i < w.width ? t.shift[w.c + i] : 0.f;
     }
-    if (w.width == V) {
+    if (w.group) {
+      GroupConst<V> gc;
+      gc.init(t, w.c);
       for (int64_t r = r0 + ty; r < r1; r += TY) {
         const float *xr = x + r * c_in;
-        const float *dr = dy + r * c_out;
-        Vec<V> a;
+        Vec<V> a, dv;
         a.load(xr + w.c);
+        dv.load(dy + r * c_out + w.c);
 #pragma unroll
         for (int i = 0; i < V; ++i) {
-          float d = bnact_dz(xr, dr, a.v[i], w.c + i, c_out, t, act_s, act_g);
+          float d = gc.dz(i, a.v[i], dv.v[i], xr, act_s, act_g);
           sb[i] += d;
           sa[i] += d * (a.v[i] - sh[i]);
         }
@@ -454,15 +486,17 @@ __global__ void __launch_bounds__(kBnThreads)
       dm[i] = dz_mean ? dz_mean[k] : 0.f;
       cf[i] = coef ? coef[k] : 0.f;
     }
-    if (w.width == V) {
+    if (w.group) {
+      GroupConst<V> gc;
+      gc.init(t, w.c);
       for (int64_t r = r0 + ty; r < r1; r += TY) {
         const float *xr = x + r * c_in;
-        const float *dr = dy + r * c_out;
-        Vec<V> a;
+        Vec<V> a, dv;
         a.load(xr + w.c);
+        dv.load(dy + r * c_out + w.c);
 #pragma unroll
         for (int i = 0; i < V; ++i) {
-          float d = bnact_dz(xr, dr, a.v[i], w.c + i, c_out, t, act_s, act_g);
+          float d = gc.dz(i, a.v[i], dv.v[i], xr, act_s, act_g);
           a.v[i] = sc[i] * (d - dm[i]) - cf[i] * (a.v[i] - sh[i]);
         }
         a.store(dx + r * c_in + w.c);
