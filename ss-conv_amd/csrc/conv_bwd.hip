@@ -6,11 +6,15 @@
 //
 // Per offset this is a tall-skinny product [Cin x P_k] * [P_k x Cout] on fp32 MFMA.
 // A workgroup owns one offset, one 64 x 64 tile of (ci, co) and one contiguous range
-// of the offset's pairs; it gathers 64 pairs at a time into LDS -- transposed, channel
-// major, so that a lane reads the four pairs of four MFMAs with one 16-byte read --
-// and keeps its 64 x 64 tile in registers (wave w owns rows 16w .. 16w+15).  Ranges
-// are reduced by a second kernel in ascending order, so the result does not depend on
-// timing: no atomics.
+// of the offset's pairs; it gathers 64 pairs at a time into LDS, rows as they lie in
+// memory.  Which pair sits in which k slot of an MFMA does not matter for the sum, and
+// neither does which channel a lane stands for, as long as the result is stored
+// accordingly: lane l of channel block j stands for channel 4l + j, so one 16-byte LDS
+// read of a gathered row hands a lane its operands for all four channel blocks, and
+// two such reads (features, output gradient) feed 16 MFMAs.  Every wave keeps the
+// whole 64 x 64 tile (16 independent accumulators) over a quarter of the pairs; the
+// four waves' tiles are added in wave order at the end, and the ranges of pairs by a
+// second kernel in ascending order: the result does not depend on timing, no atomics.
 #include "ssc_common.h"
 
 namespace ssc {
@@ -38,15 +42,21 @@ __device__ __forceinline__ float4v load_quad(const float *__restrict__ m, int64_
   return v;
 }
 
-// grid: x = range of pairs, y = offset k, z = tile (ci tile major).  256 threads.
-__global__ void __launch_bounds__(256)
-    conv_bwd_filter_kernel(const float *__restrict__ feats, int cin,
-                           const float *__restrict__ dout, int cout,
+// grid: x = range of pairs, y = offset k, z = tile (ci tile major).  256 threads, four
+// workgroups per CU (one wave of each per SIMD: 128 registers a wave).
+// BUF: rows are multiples of 16 bytes and both matrices are below 4 GiB, so the gathers
+// are range-checked buffer loads at 32-bit byte offsets (a row beyond the range's pairs
+// gets an offset outside the buffer and reads zeros): no 64-bit address arithmetic and
+// no branches around the loads.
+template <bool BUF>
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4)))
+    conv_bwd_filter_kernel(const float *__restrict__ feats, int cin, unsigned feat_bytes,
+                           const float *__restrict__ dout, int cout, unsigned dout_bytes,
                            const int32_t *__restrict__ pairs, int64_t pair_stride,
                            const int32_t *__restrict__ pair_num, int plane_in, int n_split,
                            int n_co_tiles, float *__restrict__ partial) {
-  __shared__ __align__(16) float ft[kBwTile * kBwStride];  // features, [ci][pair]
-  __shared__ __align__(16) float dt[kBwTile * kBwStride];  // output gradient, [co][pair]
+  __shared__ __align__(16) float ft[kBwChunk * kBwStride];  // features, [pair][ci]
+  __shared__ __align__(16) float dt[kBwChunk * kBwStride];  // output gradient, [pair][co]
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l16 = lane & 15, g = lane >> 4;
   const int s = blockIdx.x, k = blockIdx.y, K = gridDim.y;
@@ -60,39 +70,53 @@ __global__ void __launch_bounds__(256)
   const int32_t *rows_in = pairs + ((int64_t)k * 2 + plane_in) * pair_stride;
   const int32_t *rows_out = pairs + ((int64_t)k * 2 + (1 - plane_in)) * pair_stride;
 
-  // staging: thread -> pair tid & 63, channel quads (tid >> 6) + 4j
-  const int sp = tid & 63, sq = tid >> 6;
+  // staging: 16 threads per gathered row (256 contiguous bytes), pairs (tid >> 4) + 16j
+  const int sp = tid >> 4, sq = (tid & 15) * 4;
   float4v rf[4], rd[4];
+  const __amdgpu_buffer_rsrc_t rs_f =
+      __builtin_amdgcn_make_buffer_rsrc((void *)feats, 0, (int)feat_bytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rs_d =
+      __builtin_amdgcn_make_buffer_rsrc((void *)dout, 0, (int)dout_bytes, 0x00020000);
+  // a quad of channels beyond the matrix width reads zeros as well
+  const unsigned col_f = ci0 + sq < cin ? (unsigned)(ci0 + sq) * 4u : 0xFFFFF000u;
+  const unsigned col_d = co0 + sq < cout ? (unsigned)(co0 + sq) * 4u : 0xFFFFF000u;
   auto fetch = [&](int p0) {
-    const int p = p0 + sp;
-    const int64_t ri = p < p_end ? rows_in[p] : -1;
-    const int64_t ro = p < p_end ? rows_out[p] : -1;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      rf[j] = load_quad(feats, ri, ci0 + (sq + 4 * j) * 4, cin);
-      rd[j] = load_quad(dout, ro, co0 + (sq + 4 * j) * 4, cout);
+      const int p = p0 + sp + 16 * j;
+      if (BUF) {
+        const unsigned ri = p < p_end ? (unsigned)rows_in[p] * (unsigned)(cin * 4) : 0xFFFFF000u;
+        const unsigned ro = p < p_end ? (unsigned)rows_out[p] * (unsigned)(cout * 4) : 0xFFFFF000u;
+        // saturating: an offset that is already outside stays outside
+        const unsigned of = ri > 0xFFFFF000u - col_f ? 0xFFFFF000u : ri + col_f;
+        const unsigned od = ro > 0xFFFFF000u - col_d ? 0xFFFFF000u : ro + col_d;
+        rf[j] = __builtin_bit_cast(float4v, __builtin_amdgcn_raw_buffer_load_b128(rs_f, (int)of, 0, 0));
+        rd[j] = __builtin_bit_cast(float4v, __builtin_amdgcn_raw_buffer_load_b128(rs_d, (int)od, 0, 0));
+      } else {
+        const int64_t ri = p < p_end ? rows_in[p] : -1;
+        const int64_t ro = p < p_end ? rows_out[p] : -1;
+        rf[j] = load_quad(feats, ri, ci0 + sq, cin);
+        rd[j] = load_quad(dout, ro, co0 + sq, cout);
+      }
     }
   };
   auto stage = [&]() {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const int ch = (sq + 4 * j) * 4;
-      ft[(ch + 0) * kBwStride + sp] = rf[j].x;
-      ft[(ch + 1) * kBwStride + sp] = rf[j].y;
-      ft[(ch + 2) * kBwStride + sp] = rf[j].z;
-      ft[(ch + 3) * kBwStride + sp] = rf[j].w;
-      dt[(ch + 0) * kBwStride + sp] = rd[j].x;
-      dt[(ch + 1) * kBwStride + sp] = rd[j].y;
-      dt[(ch + 2) * kBwStride + sp] = rd[j].z;
-      dt[(ch + 3) * kBwStride + sp] = rd[j].w;
+      *reinterpret_cast<float4v *>(ft + (sp + 16 * j) * kBwStride + sq) = rf[j];
+      *reinterpret_cast<float4v *>(dt + (sp + 16 * j) * kBwStride + sq) = rd[j];
     }
   };
 
-  float4v acc[4];
+  // acc[jm][jn]: D[ci0 + 4*(4g + r) + jm][co0 + 4*l16 + jn] in component r
+  float4v acc[4][4];
 #pragma unroll
-  for (int j = 0; j < 4; ++j) acc[j] = float4v{0.f, 0.f, 0.f, 0.f};
-  const float *a_row = ft + (wave * 16 + l16) * kBwStride + g * 4;
-  const float *b_row = dt + l16 * kBwStride + g * 4;
+  for (int jm = 0; jm < 4; ++jm)
+#pragma unroll
+    for (int jn = 0; jn < 4; ++jn) acc[jm][jn] = float4v{0.f, 0.f, 0.f, 0.f};
+  // k slot g of this wave's MFMA step tt is pair 4 * (wave + 4 * tt) + g of the chunk
+  const float *a_row = ft + (4 * wave + g) * kBwStride + 4 * l16;
+  const float *b_row = dt + (4 * wave + g) * kBwStride + 4 * l16;
 
   if (p_begin < p_end) fetch(p_begin);
   for (int p0 = p_begin; p0 < p_end; p0 += kBwChunk) {
@@ -100,32 +124,39 @@ __global__ void __launch_bounds__(256)
     __syncthreads();
     if (p0 + kBwChunk < p_end) fetch(p0 + kBwChunk);  // in flight during the MFMAs
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      // lane (l16, g) holds the pairs 16q + 4g .. +3 of its channel row: MFMA t of this
-      // group multiplies pair 16q + 4g + t on both operands
-      const float4v a = *reinterpret_cast<const float4v *>(a_row + q * 16);
+    for (int tt = 0; tt < 4; ++tt) {
+      const float4v a = *reinterpret_cast<const float4v *>(a_row + tt * 16 * kBwStride);
+      const float4v b = *reinterpret_cast<const float4v *>(b_row + tt * 16 * kBwStride);
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const float4v b = *reinterpret_cast<const float4v *>(b_row + j * 16 * kBwStride + q * 16);
-        acc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.x, b.x, acc[j], 0, 0, 0);
-        acc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.y, b.y, acc[j], 0, 0, 0);
-        acc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.z, b.z, acc[j], 0, 0, 0);
-        acc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.w, b.w, acc[j], 0, 0, 0);
-      }
+      for (int jm = 0; jm < 4; ++jm)
+#pragma unroll
+        for (int jn = 0; jn < 4; ++jn)
+          acc[jm][jn] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[jm], b[jn], acc[jm][jn], 0, 0, 0);
     }
     __syncthreads();
   }
-  // acc[j] = D[ci = 16*wave + 4g + r][co = 16j + l16], r = component
-  float *dst = partial + ((int64_t)s * K + k) * cin * cout;
+  // Add the four waves' tiles in wave order through LDS (tile[ci][co], 64 x 64 floats in
+  // the staging memory), then write the tile out.
+  float *tile = ft;
+  static_assert(2 * kBwChunk * kBwStride >= kBwTile * kBwTile, "the tile fits the staging memory");
+  for (int w = 0; w < 4; ++w) {
+    if (wave == w) {
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const int co = co0 + j * 16 + l16;
-    if (co >= cout) continue;
-    const int ci = ci0 + wave * 16 + g * 4;
-    if (ci + 0 < cin) dst[(int64_t)(ci + 0) * cout + co] = acc[j].x;
-    if (ci + 1 < cin) dst[(int64_t)(ci + 1) * cout + co] = acc[j].y;
-    if (ci + 2 < cin) dst[(int64_t)(ci + 2) * cout + co] = acc[j].z;
-    if (ci + 3 < cin) dst[(int64_t)(ci + 3) * cout + co] = acc[j].w;
+      for (int jm = 0; jm < 4; ++jm)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          // the four column blocks of a lane are four neighbouring columns
+          float4v *t = reinterpret_cast<float4v *>(tile + (4 * (4 * g + r) + jm) * kBwTile + 4 * l16);
+          const float4v v = {acc[jm][0][r], acc[jm][1][r], acc[jm][2][r], acc[jm][3][r]};
+          *t = w == 0 ? v : *t + v;
+        }
+    }
+    __syncthreads();
+  }
+  float *dst = partial + ((int64_t)s * K + k) * cin * cout;
+  for (int e = tid; e < kBwTile * kBwTile; e += 256) {
+    const int ci = ci0 + e / kBwTile, co = co0 + e % kBwTile;
+    if (ci < cin && co < cout) dst[(int64_t)ci * cout + co] = tile[e];
   }
 }
 
@@ -146,9 +177,10 @@ __global__ void __launch_bounds__(256)
 }
 
 static int bwd_split(int K, int c_in, int c_out, int64_t pair_stride) {
-  // enough workgroups to fill the chip a few times over, but ranges of at least 8 chunks
+  // as many workgroups as the chip holds at once (4 per CU on 256 CUs) when the tiles
+  // alone are fewer, but ranges of at least 8 chunks
   const int64_t tiles = ceil_div(c_in, kBwTile) * ceil_div(c_out, kBwTile) * K;
-  int64_t s = ceil_div(1024, tiles);
+  int64_t s = 1024 / tiles;
   const int64_t max_s = ceil_div(pair_stride > 0 ? pair_stride : 1, 8 * kBwChunk);
   if (s > max_s) s = max_s;
   if (s < 1) s = 1;
@@ -204,10 +236,19 @@ int ssc_conv_bwd_filter_f32(const float *features, int64_t n_in, int32_t c_in,
   float *partial = static_cast<float *>(workspace);
   // features are gathered through the plane the forward pass gathered them through
   const int plane_in = inverse ? 1 : 0;
-  hipLaunchKernelGGL(conv_bwd_filter_kernel,
-                     dim3((unsigned)n_split, (unsigned)K, (unsigned)(n_ci_tiles * n_co_tiles)),
-                     dim3(256), 0, s, features, c_in, out_grad, c_out, pairs, pair_stride, pair_num,
-                     plane_in, n_split, n_co_tiles, partial);
+  const dim3 grid((unsigned)n_split, (unsigned)K, (unsigned)(n_ci_tiles * n_co_tiles));
+  const uint64_t feat_bytes = (uint64_t)n_in * c_in * 4, dout_bytes = (uint64_t)n_out * c_out * 4;
+  // the largest byte offset must stay below the marker that stands for "outside"
+  const bool buf = (c_in & 3) == 0 && (c_out & 3) == 0 && feat_bytes <= 0xFFFFF000u &&
+                   dout_bytes <= 0xFFFFF000u;
+  if (buf)
+    hipLaunchKernelGGL(conv_bwd_filter_kernel<true>, grid, dim3(256), 0, s, features, c_in,
+                       (unsigned)feat_bytes, out_grad, c_out, (unsigned)dout_bytes, pairs,
+                       pair_stride, pair_num, plane_in, n_split, n_co_tiles, partial);
+  else
+    hipLaunchKernelGGL(conv_bwd_filter_kernel<false>, grid, dim3(256), 0, s, features, c_in, 0u,
+                       out_grad, c_out, 0u, pairs, pair_stride, pair_num, plane_in, n_split,
+                       n_co_tiles, partial);
   SSC_LAUNCH_CHECK("conv_bwd_filter");
   hipLaunchKernelGGL(conv_bwd_reduce_kernel, dim3((unsigned)ceil_div(per, 256)), dim3(256), 0, s,
                      partial, n_split, K, c_in, c_out, filters_grad, gs_k, gs_ci, gs_co);
