@@ -80,25 +80,36 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))
   // a quad of channels beyond the matrix width reads zeros as well
   const unsigned col_f = ci0 + sq < cin ? (unsigned)(ci0 + sq) * 4u : 0xFFFFF000u;
   const unsigned col_d = co0 + sq < cout ? (unsigned)(co0 + sq) * 4u : 0xFFFFF000u;
+  // row numbers of the chunk after the one being fetched: the gathers never wait for
+  // their own index loads
+  int idx_i[4], idx_o[4];
+  auto fetch_idx = [&](int p0) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int p = p0 + sp + 16 * j;
+      idx_i[j] = p < p_end ? rows_in[p] : -1;
+      idx_o[j] = p < p_end ? rows_out[p] : -1;
+    }
+  };
   auto fetch = [&](int p0) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int p = p0 + sp + 16 * j;
       if (BUF) {
-        const unsigned ri = p < p_end ? (unsigned)rows_in[p] * (unsigned)(cin * 4) : 0xFFFFF000u;
-        const unsigned ro = p < p_end ? (unsigned)rows_out[p] * (unsigned)(cout * 4) : 0xFFFFF000u;
+        const unsigned ri = idx_i[j] >= 0 ? (unsigned)idx_i[j] * (unsigned)(cin * 4) : 0xFFFFF000u;
+        const unsigned ro = idx_o[j] >= 0 ? (unsigned)idx_o[j] * (unsigned)(cout * 4) : 0xFFFFF000u;
         // saturating: an offset that is already outside stays outside
         const unsigned of = ri > 0xFFFFF000u - col_f ? 0xFFFFF000u : ri + col_f;
         const unsigned od = ro > 0xFFFFF000u - col_d ? 0xFFFFF000u : ro + col_d;
         rf[j] = __builtin_bit_cast(float4v, __builtin_amdgcn_raw_buffer_load_b128(rs_f, (int)of, 0, 0));
         rd[j] = __builtin_bit_cast(float4v, __builtin_amdgcn_raw_buffer_load_b128(rs_d, (int)od, 0, 0));
       } else {
-        const int64_t ri = p < p_end ? rows_in[p] : -1;
-        const int64_t ro = p < p_end ? rows_out[p] : -1;
-        rf[j] = load_quad(feats, ri, ci0 + sq, cin);
-        rd[j] = load_quad(dout, ro, co0 + sq, cout);
+        (void)p;
+        rf[j] = load_quad(feats, idx_i[j], ci0 + sq, cin);
+        rd[j] = load_quad(dout, idx_o[j], co0 + sq, cout);
       }
     }
+    fetch_idx(p0 + kBwChunk);
   };
   auto stage = [&]() {
 #pragma unroll
@@ -118,7 +129,10 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))
   const float *a_row = ft + (4 * wave + g) * kBwStride + 4 * l16;
   const float *b_row = dt + (4 * wave + g) * kBwStride + 4 * l16;
 
-  if (p_begin < p_end) fetch(p_begin);
+  if (p_begin < p_end) {
+    fetch_idx(p_begin);
+    fetch(p_begin);
+  }
   for (int p0 = p_begin; p0 < p_end; p0 += kBwChunk) {
     stage();
     __syncthreads();
