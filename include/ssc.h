@@ -82,6 +82,17 @@ int ssc_rulebook_count(const int32_t *indices /* [n_in,4] device */, int64_t n_i
                        const ssc_geometry *g, void *workspace, size_t workspace_bytes,
                        int32_t *n_out_host /* host */, ssc_stream_t stream);
 
+/* The same, and *in_order_host = 1 when the input rows come in strictly ascending
+ * (b, x, y, z) order (0 otherwise; repeated rows count as disorder).  For such inputs the
+ * pairs ssc_rulebook_emit writes ascend, offset by offset, in the output rows as well as
+ * in the input rows, which ssc_conv_fwd_f32 can be told (SSC_CONV_PAIRS_CANONICAL); for
+ * other inputs only the input rows of an offset ascend.  No counterpart in the reference:
+ * it saves the convolution's own order check. */
+int ssc_rulebook_count_ordered(const int32_t *indices, int64_t n_in, const ssc_geometry *g,
+                               void *workspace, size_t workspace_bytes,
+                               int32_t *n_out_host /* host */, int32_t *in_order_host /* host */,
+                               ssc_stream_t stream);
+
 int ssc_rulebook_emit(const int32_t *indices, int64_t n_in, const ssc_geometry *g,
                       void *workspace, size_t workspace_bytes,
                       int32_t *out_indices /* [n_out,4] device; may be NULL when subm */,
@@ -99,10 +110,18 @@ int ssc_rulebook_emit(const int32_t *indices, int64_t n_in, const ssc_geometry *
  * (element strides), so both a contiguous [K,Cin,Cout] kernel and the
  * reference's permuted view of [Cout,Cin,K] (ss_conv/convolution.py:56) work.
  * `inverse` swaps the roles of the two pair planes (indice_conv.h:307,330).
- * `subm` is accepted for signature parity; the centre offset is treated like
- * any other offset.  pair_num stays on the device: no host synchronisation.
+ * `subm`: bit 0 is the reference's flag, accepted for signature parity (the centre
+ * offset is treated like any other offset).  Bit 1 (SSC_CONV_PAIRS_CANONICAL) is the
+ * caller's promise that, for every offset, the rows that are accumulated into (the
+ * output rows; the input rows when `inverse`) ascend strictly -- true of the input rows of
+ * every rulebook ssc_rulebook_emit writes, and of the output rows when
+ * ssc_rulebook_count_ordered reported ordered input: the order check and the kernels that
+ * would re-order the pairs are then not launched.  Without the bit any order is accepted.
+ * pair_num stays on the device: no host synchronisation.
  * Every row of out[n_out,Cout] is written (zeros where no pair lands).
  * ---------------------------------------------------------------------- */
+#define SSC_CONV_PAIRS_CANONICAL 2
+
 size_t ssc_conv_workspace_bytes(int64_t n_out, int32_t kernel_volume, int32_t c_in,
                                 int32_t c_out, int64_t pair_stride);
 

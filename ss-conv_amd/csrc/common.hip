@@ -39,7 +39,7 @@ int fill_f32(float *p, int64_t n, float v, hipStream_t s) {
 size_t bit_table_bytes(int64_t n_bits) {
   int64_t w = bit_words(n_bits);
   int64_t nb = ceil_div(w, kScanBlockWords);
-  return align_up(w * 4) * 2 + align_up((nb + 1) * 4) + align_up(4);
+  return align_up(w * 4) * 2 + align_up((nb + 1) * 4) + align_up(8);
 }
 
 BitTable bit_table_carve(Carver &c, int64_t n_bits) {
@@ -49,7 +49,7 @@ BitTable bit_table_carve(Carver &c, int64_t n_bits) {
   t.bits = c.take<uint32_t>(t.n_words);
   t.prefix = c.take<int32_t>(t.n_words);
   t.blocksum = c.take<int32_t>(t.n_scan_blocks + 1);
-  t.total = c.take<int32_t>(1);
+  t.total = c.take<int32_t>(2);  // [1]: a flag word for the table's user
   return t;
 }
 

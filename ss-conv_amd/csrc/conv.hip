@@ -1235,7 +1235,6 @@ int ssc_conv_fwd_f32(const float *features, int64_t n_in, int32_t c_in, const fl
                      int32_t kernel_volume, int32_t inverse, int32_t subm, float *out,
                      int64_t n_out, void *workspace, size_t workspace_bytes,
                      ssc_stream_t stream) {
-  (void)subm;
   const int K = kernel_volume;
   SSC_CHECK(K >= 1 && K <= SSC_MAX_KERNEL_VOLUME, SSC_ERUNTIME, "kernel volume %d out of range", K);
   SSC_CHECK(c_in >= 1 && c_out >= 1, SSC_EINVAL, "channel counts must be positive");
@@ -1265,21 +1264,23 @@ int ssc_conv_fwd_f32(const float *features, int64_t n_in, int32_t c_in, const fl
   SSC_LAUNCH_CHECK("pack_filters");
 
   dim3 pair_grid((unsigned)ceil_div(pair_stride, 256), (unsigned)K);
-  hipLaunchKernelGGL(check_sorted_kernel, pair_grid, dim3(256), 0, s, pairs, pair_stride, plane_s,
-                     pair_num, w.flag);
-  SSC_LAUNCH_CHECK("check_sorted");
-  int64_t nbits_words = (int64_t)K * p.words_per_k;
-  unsigned clear_blocks =
-      (unsigned)(ceil_div(nbits_words, 256) < 4096 ? ceil_div(nbits_words, 256) : 4096);
-  hipLaunchKernelGGL(resort_clear_kernel, dim3(clear_blocks), dim3(256), 0, s, w.flag, w.bits,
-                     nbits_words);
-  hipLaunchKernelGGL(resort_mark_kernel, pair_grid, dim3(256), 0, s, w.flag, pairs, pair_stride,
-                     plane_s, pair_num, w.bits, p.words_per_k);
-  hipLaunchKernelGGL(resort_scan_kernel, dim3(K), dim3(kScanThreads), 0, s, w.flag, w.bits,
-                     w.prefix, p.words_per_k);
-  hipLaunchKernelGGL(resort_scatter_kernel, pair_grid, dim3(256), 0, s, w.flag, pairs,
-                     pair_stride, plane_s, pair_num, w.bits, w.prefix, p.words_per_k, w.sorted);
-  SSC_LAUNCH_CHECK("resort");
+  if ((subm & SSC_CONV_PAIRS_CANONICAL) == 0) {  // otherwise flag[0] stays 0: pairs in order
+    hipLaunchKernelGGL(check_sorted_kernel, pair_grid, dim3(256), 0, s, pairs, pair_stride, plane_s,
+                       pair_num, w.flag);
+    SSC_LAUNCH_CHECK("check_sorted");
+    int64_t nbits_words = (int64_t)K * p.words_per_k;
+    unsigned clear_blocks =
+        (unsigned)(ceil_div(nbits_words, 256) < 4096 ? ceil_div(nbits_words, 256) : 4096);
+    hipLaunchKernelGGL(resort_clear_kernel, dim3(clear_blocks), dim3(256), 0, s, w.flag, w.bits,
+                       nbits_words);
+    hipLaunchKernelGGL(resort_mark_kernel, pair_grid, dim3(256), 0, s, w.flag, pairs, pair_stride,
+                       plane_s, pair_num, w.bits, p.words_per_k);
+    hipLaunchKernelGGL(resort_scan_kernel, dim3(K), dim3(kScanThreads), 0, s, w.flag, w.bits,
+                       w.prefix, p.words_per_k);
+    hipLaunchKernelGGL(resort_scatter_kernel, pair_grid, dim3(256), 0, s, w.flag, pairs,
+                       pair_stride, plane_s, pair_num, w.bits, w.prefix, p.words_per_k, w.sorted);
+    SSC_LAUNCH_CHECK("resort");
+  }
 
   // work split on the fine grid, then the tiles and their segments
   hipLaunchKernelGGL(grid_segments_kernel, pair_grid, dim3(256), 0, s, w.flag, pairs, w.sorted,

@@ -80,10 +80,19 @@ __device__ __forceinline__ bool pair_key(const Geom &g, const int32_t *__restric
   return true;
 }
 
+// (b, x, y, z) of row a strictly before row b in key order
+__device__ __forceinline__ bool row_before(const int4 &a, const int4 &b) {
+  if (a.x != b.x) return a.x < b.x;
+  if (a.y != b.y) return a.y < b.y;
+  if (a.z != b.z) return a.z < b.z;
+  return a.w < b.w;
+}
+
 // Regular conv: mark every output cell reachable from an active input, and count
 // the pairs of every 64-row chunk (chunk_count is [K, n_chunks]; for a regular
 // convolution a pair exists wherever the geometry allows it, so the counts do not
 // depend on the table).  One wave per chunk of 64 input rows and x offset, one lane per row.
+// disorder[0] |= 1 when some input row does not come strictly before its successor.
 // The taps of one (kx, ky) differ in z only, so their output cells are neighbours
 // in the key space: their bits are gathered into one mask per 32-bit word, the word
 // is read first, and the atomic is issued only when it would change the word
@@ -91,7 +100,7 @@ __device__ __forceinline__ bool pair_key(const Geom &g, const int32_t *__restric
 __global__ void __launch_bounds__(256)
     mark_count_kernel(const int32_t *__restrict__ indices, int64_t n_in, Geom g,
                       uint32_t *__restrict__ bits, int32_t *__restrict__ chunk_count,
-                      int64_t n_chunks) {
+                      int64_t n_chunks, int32_t *__restrict__ disorder) {
   int64_t chunk = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (chunk >= n_chunks) return;
   const int lane = threadIdx.x & 63;
@@ -99,6 +108,9 @@ __global__ void __launch_bounds__(256)
   const bool live = i < n_in;
   int32_t row[4] = {0, 0, 0, 0};
   if (live) *reinterpret_cast<int4 *>(row) = reinterpret_cast<const int4 *>(indices)[i];
+  if (blockIdx.y == 0 && i + 1 < n_in &&
+      !row_before(*reinterpret_cast<int4 *>(row), reinterpret_cast<const int4 *>(indices)[i + 1]))
+    atomicOr(disorder, 1);
   // blockIdx.y = kx: the taps of one x offset per wave, for more waves in flight
   const int kx = blockIdx.y;
   int k = kx * g.ks[1] * g.ks[2];
@@ -133,10 +145,12 @@ __global__ void __launch_bounds__(256)
 // Submanifold / unique: mark the cells of the rows themselves.
 __global__ void __launch_bounds__(256)
     mark_rows_kernel(const int32_t *__restrict__ coords, int64_t n, int d1, int d2, int d3,
-                     uint32_t *__restrict__ bits) {
+                     uint32_t *__restrict__ bits, int32_t *__restrict__ disorder) {
   int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= n) return;
   int4 r = reinterpret_cast<const int4 *>(coords)[i];
+  if (disorder && i + 1 < n && !row_before(r, reinterpret_cast<const int4 *>(coords)[i + 1]))
+    atomicOr(disorder, 1);
   uint32_t key = (uint32_t)(((r.x * d1 + r.y) * d2 + r.z) * d3 + r.w);
   atomicOr(&bits[key >> 5], 1u << (key & 31u));
 }
@@ -364,14 +378,24 @@ size_t ssc_rulebook_workspace_bytes(const ssc_geometry *g, int64_t n_in) {
 int ssc_rulebook_count(const int32_t *indices, int64_t n_in, const ssc_geometry *g,
                        void *workspace, size_t workspace_bytes, int32_t *n_out_host,
                        ssc_stream_t stream) {
+  int32_t in_order = 0;
+  return ssc_rulebook_count_ordered(indices, n_in, g, workspace, workspace_bytes, n_out_host,
+                                    &in_order, stream);
+}
+
+int ssc_rulebook_count_ordered(const int32_t *indices, int64_t n_in, const ssc_geometry *g,
+                               void *workspace, size_t workspace_bytes, int32_t *n_out_host,
+                               int32_t *in_order_host, ssc_stream_t stream) {
   Geom gg;
   int rc = make_geom(g, &gg);
   if (rc != SSC_OK) return rc;
-  SSC_CHECK(n_out_host != nullptr, SSC_EINVAL, "n_out_host is NULL");
+  SSC_CHECK(n_out_host != nullptr && in_order_host != nullptr, SSC_EINVAL,
+            "n_out_host or in_order_host is NULL");
   SSC_CHECK(n_in >= 0, SSC_EINVAL, "n_in is negative");
   SSC_CHECK(n_in * gg.K < ((int64_t)1 << 40), SSC_EINVAL, "n_in * kernel volume too large");
   if (n_in == 0) {  // src/conv/indice_cuda_functor.cu:262-263
     *n_out_host = 0;
+    *in_order_host = 1;
     return SSC_OK;
   }
   SSC_CHECK(indices != nullptr && workspace != nullptr, SSC_EINVAL, "NULL pointer argument");
@@ -381,21 +405,28 @@ int ssc_rulebook_count(const int32_t *indices, int64_t n_in, const ssc_geometry 
   hipStream_t s = (hipStream_t)stream;
   RulebookWs w = rulebook_ws_carve(workspace, gg, n_in);
   if ((rc = bit_table_clear(w.table, s)) != SSC_OK) return rc;
+  // total[0]: the table's popcount (written by the scan); total[1]: the disorder flag,
+  // cleared here and set by the marking kernel.  This call ends with a host read, so it
+  // cannot be part of a captured graph anyway: a memset is fine.
+  SSC_HIP(hipMemsetAsync(w.table.total, 0, 2 * sizeof(int32_t), s));
   if (gg.subm) {
     hipLaunchKernelGGL(mark_rows_kernel, dim3((unsigned)ceil_div(n_in, 256)), dim3(256), 0, s,
-                       indices, n_in, gg.os[0], gg.os[1], gg.os[2], w.table.bits);
+                       indices, n_in, gg.os[0], gg.os[1], gg.os[2], w.table.bits,
+                       w.table.total + 1);
     SSC_LAUNCH_CHECK("mark_rows");
   } else {
     hipLaunchKernelGGL(mark_count_kernel,
                        dim3((unsigned)ceil_div(w.n_chunks, 4), (unsigned)gg.ks[0]), dim3(256), 0, s,
-                       indices, n_in, gg, w.table.bits, w.chunk_count, w.n_chunks);
+                       indices, n_in, gg, w.table.bits, w.chunk_count, w.n_chunks,
+                       w.table.total + 1);
     SSC_LAUNCH_CHECK("mark_count");
   }
   if ((rc = bit_table_scan(w.table, s)) != SSC_OK) return rc;
-  int32_t total = 0;
-  SSC_HIP(hipMemcpyAsync(&total, w.table.total, sizeof(int32_t), hipMemcpyDeviceToHost, s));
+  int32_t host[2] = {0, 0};
+  SSC_HIP(hipMemcpyAsync(host, w.table.total, sizeof(host), hipMemcpyDeviceToHost, s));
   SSC_HIP(hipStreamSynchronize(s));
-  *n_out_host = gg.subm ? (int32_t)n_in : total;
+  *n_out_host = gg.subm ? (int32_t)n_in : host[0];
+  *in_order_host = host[1] == 0 ? 1 : 0;
   return SSC_OK;
 }
 
@@ -476,7 +507,8 @@ int ssc_unique_count(const int32_t *coords, int64_t n, const int32_t dims[4], vo
   BitTable t = bit_table_carve(c, cells);
   if ((rc = bit_table_clear(t, s)) != SSC_OK) return rc;
   hipLaunchKernelGGL(mark_rows_kernel, dim3((unsigned)ceil_div(n, 256)), dim3(256), 0, s, coords,
-                     n, dims[1], dims[2], dims[3], t.bits);
+                     n, dims[1], dims[2], dims[3], t.bits,
+                     (int32_t *)nullptr);
   SSC_LAUNCH_CHECK("mark_rows");
   if ((rc = bit_table_scan(t, s)) != SSC_OK) return rc;
   SSC_HIP(hipMemcpyAsync(n_unique_host, t.total, sizeof(int32_t), hipMemcpyDeviceToHost, s));

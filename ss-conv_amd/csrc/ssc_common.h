@@ -61,7 +61,7 @@ struct BitTable {
   uint32_t *bits;     // [n_words]
   int32_t *prefix;    // [n_words] exclusive popcount prefix
   int32_t *blocksum;  // [n_scan_blocks]
-  int32_t *total;     // [1]
+  int32_t *total;     // [2]: popcount of the table; a flag word for the table's user
   int64_t n_words;
   int64_t n_scan_blocks;
 };

@@ -39,6 +39,8 @@ _SIGNATURES = {
     "ssc_last_error": (ctypes.c_char_p, []),
     "ssc_rulebook_workspace_bytes": (_sz, [_gp, _i64]),
     "ssc_rulebook_count": (ctypes.c_int, [_vp, _i64, _gp, _vp, _sz, ctypes.POINTER(_i32), _vp]),
+    "ssc_rulebook_count_ordered": (ctypes.c_int, [_vp, _i64, _gp, _vp, _sz, ctypes.POINTER(_i32),
+                                                  ctypes.POINTER(_i32), _vp]),
     "ssc_rulebook_emit": (ctypes.c_int, [_vp, _i64, _gp, _vp, _sz, _vp, _vp, _vp, _vp]),
     "ssc_conv_workspace_bytes": (_sz, [_i64, _i32, _i32, _i32, _i64]),
     "ssc_conv_fwd_f32": (ctypes.c_int, [_vp, _i64, _i32, _vp, _i64, _i64, _i64, _i32, _vp, _i64,
@@ -170,14 +172,21 @@ def get_indice_pairs_3d(indices, batch_size, out_spatial_shape, spatial_shape, k
         nbytes = 256
     ws = _workspace(nbytes, dev)
     n_out = _i32(0)
+    in_order = _i32(0)
     s = _stream(indices)
-    _check(_lib.ssc_rulebook_count(_ptr(indices), n, ctypes.byref(g), ws.data_ptr(), ws.numel(),
-                                   ctypes.byref(n_out), s))
+    _check(_lib.ssc_rulebook_count_ordered(_ptr(indices), n, ctypes.byref(g), ws.data_ptr(),
+                                           ws.numel(), ctypes.byref(n_out),
+                                           ctypes.byref(in_order), s))
     pairs = torch.empty((K, 2, n), dtype=torch.int32, device=dev)
     num = torch.empty((K,), dtype=torch.int32, device=dev)
     outids = indices if subm else torch.empty((n_out.value, 4), dtype=torch.int32, device=dev)
     _check(_lib.ssc_rulebook_emit(_ptr(indices), n, ctypes.byref(g), ws.data_ptr(), ws.numel(),
                                   None if subm else _ptr(outids), _ptr(pairs), num.data_ptr(), s))
+    # Pairs of an offset always ascend in the input rows, and in the output rows too when
+    # the input rows came in key order: the convolution may then skip its order check
+    # (the first flag serves a call that accumulates into output rows, the second one
+    # with `inverse`, which accumulates into input rows).
+    pairs._ssc_canonical = (bool(in_order.value), True)
     return [outids, pairs, num]
 
 
@@ -195,6 +204,14 @@ def _filter_strides(filters, c_in, c_out):
         filters = filters.contiguous()
         kstr = filters.stride()[:-2]
     return filters, kstr[-1], filters.stride(-2), filters.stride(-1)
+
+
+def _conv_flags(indice_pairs, subm, inverse):
+    """The `subm` argument of ssc_conv_fwd_f32: the reference's flag plus the promise of
+    canonical pair order for rulebooks that get_indice_pairs_3d built."""
+    canonical = getattr(indice_pairs, "_ssc_canonical", (False, False))[1 if inverse else 0] and \
+        indice_pairs.dtype == torch.int32 and indice_pairs.is_contiguous()
+    return int(bool(subm)) | (2 if canonical else 0)
 
 
 def indice_conv_fp32(features, filters, indice_pairs, indice_num, num_act_out, inverse, subm):
@@ -221,8 +238,8 @@ def indice_conv_fp32(features, filters, indice_pairs, indice_num, num_act_out, i
     ws = _workspace(nbytes, features.device)
     _check(_lib.ssc_conv_fwd_f32(_ptr(features), features.size(0), c_in, _ptr(filters), fs_k,
                                  fs_ci, fs_co, c_out, _ptr(pairs), pairs.size(2), num.data_ptr(),
-                                 K, int(inverse), int(subm), _ptr(out), n_out, ws.data_ptr(),
-                                 ws.numel(), _stream(features)))
+                                 K, int(inverse), _conv_flags(indice_pairs, subm, inverse), _ptr(out), n_out,
+                                 ws.data_ptr(), ws.numel(), _stream(features)))
     return out
 
 
@@ -249,7 +266,8 @@ def indice_conv_backward_fp32(features, filters, out_bp, indice_pairs, indice_nu
     ws = _workspace(_lib.ssc_conv_workspace_bytes(n_in, K, c_out, c_in, pairs.size(2)), dev)
     _check(_lib.ssc_conv_fwd_f32(_ptr(out_bp), n_out, c_out, _ptr(filters), fs_k, fs_co, fs_ci,
                                  c_in, _ptr(pairs), pairs.size(2), num.data_ptr(), K,
-                                 0 if inverse else 1, int(subm), _ptr(input_bp), n_in,
+                                 0 if inverse else 1, _conv_flags(indice_pairs, subm, not inverse),
+                                 _ptr(input_bp), n_in,
                                  ws.data_ptr(), ws.numel(), s))
     # filter gradient
     filters_bp = torch.empty(tuple(filters.shape), dtype=torch.float32, device=dev)

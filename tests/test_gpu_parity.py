@@ -800,3 +800,36 @@ def test_batchnorm_activation_other_cases(oracle, device):
     z[:, :4] = np.log1p(np.exp(z[:, :4]))
     want = oracle.gate_fwd(z, Rs, act_scalar=None, act_gate="sigmoid")
     assert rel_l2(y, want) < REL_L2
+
+
+def test_conv_order_promise_follows_the_input_order(oracle, device):
+    """The rulebook reports whether its input rows came in key order; only then may the
+    convolution skip its own order check.  Both ways must give the oracle's result."""
+    from ss_conv import _ext
+    from ss_conv.sp_ops.ops import get_indice_pairs
+    rng = np.random.default_rng(21)
+    n, grid, cin, cout, k = 400, 10, 32, 48, 3
+    idx_sorted = random_voxels(rng, 2, grid, n)
+    feats = rng.normal(size=(n, cin)).astype(np.float32)
+    w = (rng.normal(size=(k ** 3, cin, cout)) / np.sqrt(27 * cin)).astype(np.float32)
+    perm = rng.permutation(n)
+    for idx, f, want_flag in ((idx_sorted, feats, True), (idx_sorted[perm], feats[perm], False)):
+        t = torch.from_numpy(idx).to(device)
+        o_idx, pairs, num = get_indice_pairs(t, 2, [grid] * 3, k, 1, 1, 1, 0, False)
+        assert pairs._ssc_canonical == (want_flag, True)
+        out = _ext.indice_conv_fp32(torch.from_numpy(f).to(device),
+                                    torch.from_numpy(w).to(device).reshape(k, k, k, cin, cout),
+                                    pairs, num, o_idx.shape[0], 0, 0)
+        r_idx, r_pairs, r_num = oracle.canonicalize(*oracle.rulebook(idx, 2, [grid] * 3, k, 1, 1))
+        # the oracle numbers pairs by input row as given, outputs by key: same convention
+        ref = oracle.conv_fwd(f, w, r_pairs, r_num, r_idx.shape[0], matmul=np.matmul)
+        assert np.array_equal(o_idx.cpu().numpy(), r_idx)
+        assert rel_l2(out.cpu().numpy(), ref) < REL_L2
+        # the input gradient accumulates into input rows: always in order
+        go = rng.normal(size=(r_idx.shape[0], cout)).astype(np.float32)
+        gi, _ = _ext.indice_conv_backward_fp32(
+            torch.from_numpy(f).to(device),
+            torch.from_numpy(w).to(device).reshape(k, k, k, cin, cout),
+            torch.from_numpy(go).to(device), pairs, num, 0, 0)
+        want, _ = oracle.conv_bwd(f, w, go, r_pairs, r_num)
+        assert rel_l2(gi.cpu().numpy(), want) < REL_L2
