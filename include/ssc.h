@@ -330,6 +330,14 @@ int ssc_three_nn(int32_t n, int32_t m, const float *unknown /* [n,4] */,
                  const float *known /* [m,4] */, float *dist2 /* [n,3] */,
                  int32_t *idx /* [n,3] */, ssc_stream_t stream);
 
+/* The same search with a small workspace for the batch range of every 256 known rows:
+ * blocks of queries then skip the known rows of other batch elements without loading
+ * them (known rows grouped by batch element, as Voxel2Point passes them, are scanned
+ * once per batch element instead of once per block).  Results are identical. */
+size_t ssc_three_nn_workspace_bytes(int32_t m);
+int ssc_three_nn_ws(int32_t n, int32_t m, const float *unknown, const float *known, float *dist2,
+                    int32_t *idx, void *workspace, size_t workspace_bytes, ssc_stream_t stream);
+
 int ssc_three_interp_f32(int32_t c, int32_t m, int32_t n, const float *feats /* [m,c] */,
                          const int32_t *idx /* [n,3] */, const float *weight /* [n,3] */,
                          float *out /* [n,c] */, ssc_stream_t stream);

@@ -88,20 +88,71 @@ __global__ void __launch_bounds__(256)
   out[idx] = acc;
 }
 
-// Brute-force 3-NN: one thread per query, known rows streamed through LDS in tiles.
+// Brute-force 3-NN: known rows streamed through LDS in tiles.
 // A known row only counts for queries of the same batch element, so a tile none of
 // whose rows falls into the batch range of the block's queries is skipped after its
 // load; with rows grouped by batch element (the usual case) a block then scans its
 // own element's rows only.  The scan order, and with it the tie rule, is unchanged.
+// With tile_range (the batch range of every tile, from nn_tile_range_kernel) a tile
+// outside the block's range is not even loaded.
 constexpr int kNnTile = 256;
+
+// tile_range[2t], tile_range[2t+1] = smallest and largest batch value of known rows
+// t*256 .. t*256+255.  One block per tile.
+__global__ void __launch_bounds__(kNnTile)
+    nn_tile_range_kernel(int m, const float *__restrict__ known, float *__restrict__ tile_range) {
+  __shared__ float red[2][kNnTile / 64];
+  const int kk = blockIdx.x * kNnTile + threadIdx.x;
+  float lo = INFINITY, hi = -INFINITY;
+  if (kk < m) lo = hi = known[(int64_t)kk * 4];
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) {
+    lo = fminf(lo, __shfl_xor(lo, d, 64));
+    hi = fmaxf(hi, __shfl_xor(hi, d, 64));
+  }
+  if ((threadIdx.x & 63) == 0) {
+    red[0][threadIdx.x >> 6] = lo;
+    red[1][threadIdx.x >> 6] = hi;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < kNnTile / 64; ++w) {
+      lo = fminf(lo, red[0][w]);
+      hi = fmaxf(hi, red[1][w]);
+    }
+    tile_range[2 * blockIdx.x] = lo;
+    tile_range[2 * blockIdx.x + 1] = hi;
+  }
+}
+
+// Eight lanes per query, each scanning every eighth row of a tile; their three best are
+// merged at the end.  Scanning in row order and replacing on strictly smaller distance
+// keeps the three smallest (distance, row) pairs in lexicographic order, so the merge
+// compares (distance, row) and the result is the sequential scan's, ties included.
+constexpr int kNnLanes = 8;
+
+struct Best3 {
+  float b1, b2, b3;
+  int i1, i2, i3;
+  __device__ __forceinline__ void insert(float d, int k) {  // (d, k) after every kept pair it ties
+    if (d < b1 || (d == b1 && k < i1)) {
+      b3 = b2; i3 = i2; b2 = b1; i2 = i1; b1 = d; i1 = k;
+    } else if (d < b2 || (d == b2 && k < i2)) {
+      b3 = b2; i3 = i2; b2 = d; i2 = k;
+    } else if (d < b3 || (d == b3 && k < i3)) {
+      b3 = d; i3 = k;
+    }
+  }
+};
 
 __global__ void __launch_bounds__(kNnTile)
     three_nn_kernel(int n, int m, const float *__restrict__ unknown,
-                    const float *__restrict__ known, float *__restrict__ dist2,
-                    int32_t *__restrict__ idx) {
+                    const float *__restrict__ known, const float *__restrict__ tile_range,
+                    float *__restrict__ dist2, int32_t *__restrict__ idx) {
   __shared__ float4v tile[kNnTile];
   __shared__ float red[2][kNnTile / 64];
-  int q = blockIdx.x * blockDim.x + threadIdx.x;
+  const int q = blockIdx.x * (kNnTile / kNnLanes) + threadIdx.x / kNnLanes;
+  const int sub = threadIdx.x % kNnLanes;
   float4v u = {0.f, 0.f, 0.f, 0.f};
   if (q < n) u = reinterpret_cast<const float4v *>(unknown)[q];
   // batch range of the block's queries
@@ -121,9 +172,12 @@ __global__ void __launch_bounds__(kNnTile)
     lo = fminf(lo, red[0][w]);
     hi = fmaxf(hi, red[1][w]);
   }
-  float b1 = INFINITY, b2 = INFINITY, b3 = INFINITY;
-  int i1 = 0, i2 = 0, i3 = 0;
+  Best3 best = {INFINITY, INFINITY, INFINITY, 0, 0, 0};
   for (int base = 0; base < m; base += kNnTile) {
+    if (tile_range) {  // the same for the whole block
+      const int t = base / kNnTile;
+      if (tile_range[2 * t] > hi || tile_range[2 * t + 1] < lo) continue;
+    }
     int kk = base + threadIdx.x;
     __syncthreads();
     bool hit = false;
@@ -134,25 +188,38 @@ __global__ void __launch_bounds__(kNnTile)
     }
     if (!__syncthreads_or(hit)) continue;
     int cnt = min(kNnTile, m - base);
-    for (int t = 0; t < cnt; ++t) {
+    for (int t = sub; t < cnt; t += kNnLanes) {
       float4v p = tile[t];
       if (p.x != u.x) continue;
       float dx = u.y - p.y, dy = u.z - p.z, dz = u.w - p.w;
       float xx = dx * dx, yy = dy * dy, zz = dz * dz;
       float d = (xx + yy) + zz;
       int k = base + t;
-      if (d < b1) {
-        b3 = b2; i3 = i2; b2 = b1; i2 = i1; b1 = d; i1 = k;
-      } else if (d < b2) {
-        b3 = b2; i3 = i2; b2 = d; i2 = k;
-      } else if (d < b3) {
-        b3 = d; i3 = k;
+      // rows come in ascending order within a lane: strictly smaller replaces
+      if (d < best.b1) {
+        best.b3 = best.b2; best.i3 = best.i2; best.b2 = best.b1; best.i2 = best.i1;
+        best.b1 = d; best.i1 = k;
+      } else if (d < best.b2) {
+        best.b3 = best.b2; best.i3 = best.i2; best.b2 = d; best.i2 = k;
+      } else if (d < best.b3) {
+        best.b3 = d; best.i3 = k;
       }
     }
   }
-  if (q < n) {
-    dist2[q * 3] = b1; dist2[q * 3 + 1] = b2; dist2[q * 3 + 2] = b3;
-    idx[q * 3] = i1; idx[q * 3 + 1] = i2; idx[q * 3 + 2] = i3;
+  // merge the lanes of a query (a slot that was never filled is (inf, 0) in every lane)
+#pragma unroll
+  for (int d = 1; d < kNnLanes; d <<= 1) {
+    const float o1 = __shfl_xor(best.b1, d, 64), o2 = __shfl_xor(best.b2, d, 64),
+                o3 = __shfl_xor(best.b3, d, 64);
+    const int j1 = __shfl_xor(best.i1, d, 64), j2 = __shfl_xor(best.i2, d, 64),
+              j3 = __shfl_xor(best.i3, d, 64);
+    if (o1 < INFINITY) best.insert(o1, j1);
+    if (o2 < INFINITY) best.insert(o2, j2);
+    if (o3 < INFINITY) best.insert(o3, j3);
+  }
+  if (q < n && sub == 0) {
+    dist2[q * 3] = best.b1; dist2[q * 3 + 1] = best.b2; dist2[q * 3 + 2] = best.b3;
+    idx[q * 3] = best.i1; idx[q * 3 + 1] = best.i2; idx[q * 3 + 2] = best.i3;
   }
 }
 
@@ -228,8 +295,32 @@ int ssc_three_nn(int32_t n, int32_t m, const float *unknown, const float *known,
   SSC_CHECK(n >= 0 && m >= 0, SSC_EINVAL, "bad sizes");
   if (n == 0) return SSC_OK;
   SSC_CHECK(unknown && dist2 && idx && (m == 0 || known), SSC_EINVAL, "NULL pointer argument");
-  hipLaunchKernelGGL(three_nn_kernel, dim3((unsigned)ceil_div(n, kNnTile)), dim3(kNnTile), 0,
-                     (hipStream_t)stream, n, m, unknown, known, dist2, idx);
+  hipLaunchKernelGGL(three_nn_kernel, dim3((unsigned)ceil_div(n, kNnTile / kNnLanes)), dim3(kNnTile), 0,
+                     (hipStream_t)stream, n, m, unknown, known, (const float *)nullptr, dist2, idx);
+  SSC_LAUNCH_CHECK("three_nn");
+  return SSC_OK;
+}
+
+size_t ssc_three_nn_workspace_bytes(int32_t m) {
+  if (m < 0) return 0;
+  return align_up((size_t)ceil_div(m > 0 ? m : 1, kNnTile) * 2 * sizeof(float));
+}
+
+int ssc_three_nn_ws(int32_t n, int32_t m, const float *unknown, const float *known, float *dist2,
+                    int32_t *idx, void *workspace, size_t workspace_bytes, ssc_stream_t stream) {
+  SSC_CHECK(n >= 0 && m >= 0, SSC_EINVAL, "bad sizes");
+  if (n == 0) return SSC_OK;
+  SSC_CHECK(unknown && dist2 && idx && (m == 0 || known), SSC_EINVAL, "NULL pointer argument");
+  SSC_CHECK(workspace != nullptr && workspace_bytes >= ssc_three_nn_workspace_bytes(m),
+            SSC_EWORKSPACE, "three_nn workspace too small");
+  float *tile_range = static_cast<float *>(workspace);
+  if (m > 0) {
+    hipLaunchKernelGGL(nn_tile_range_kernel, dim3((unsigned)ceil_div(m, kNnTile)), dim3(kNnTile), 0,
+                       (hipStream_t)stream, m, known, tile_range);
+    SSC_LAUNCH_CHECK("nn_tile_range");
+  }
+  hipLaunchKernelGGL(three_nn_kernel, dim3((unsigned)ceil_div(n, kNnTile / kNnLanes)), dim3(kNnTile), 0,
+                     (hipStream_t)stream, n, m, unknown, known, tile_range, dist2, idx);
   SSC_LAUNCH_CHECK("three_nn");
   return SSC_OK;
 }

@@ -85,6 +85,8 @@ _SIGNATURES = {
     "ssc_voxel_map": (ctypes.c_int, [_vp, _vp, _vp, _i32, _i32, _i32, _i32, _vp]),
     "ssc_voxel_reduce_f32": (ctypes.c_int, [_vp, _vp, _vp, _i32, _i32, _i32, _i32, _vp]),
     "ssc_three_nn": (ctypes.c_int, [_i32, _i32, _vp, _vp, _vp, _vp, _vp]),
+    "ssc_three_nn_workspace_bytes": (_sz, [_i32]),
+    "ssc_three_nn_ws": (ctypes.c_int, [_i32, _i32, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
     "ssc_three_interp_f32": (ctypes.c_int, [_i32, _i32, _i32, _vp, _vp, _vp, _vp, _vp]),
     "ssc_bn_workspace_bytes": (_sz, [_i64, _i32]),
     "ssc_bn_prepare_f32": (ctypes.c_int, [_vp, _i64, _i32, _vp, _vp, _vp, _vp, _i32, _i32,
@@ -463,8 +465,9 @@ def three_nn(n, m, unknown, known, dist2, idx):
     for t in (unknown, known, dist2, idx):
         if not t.is_contiguous():
             raise RuntimeError("three_nn needs contiguous tensors")
-    _check(_lib.ssc_three_nn(int(n), int(m), _ptr(unknown), _ptr(known), _ptr(dist2), _ptr(idx),
-                             _stream(unknown)))
+    ws = _workspace(_lib.ssc_three_nn_workspace_bytes(int(m)), unknown.device)
+    _check(_lib.ssc_three_nn_ws(int(n), int(m), _ptr(unknown), _ptr(known), _ptr(dist2), _ptr(idx),
+                                ws.data_ptr(), ws.numel(), _stream(unknown)))
 
 
 def three_interpolate_fp(c, m, n, feats, idx, weight, out):
