@@ -257,23 +257,36 @@ __global__ void __launch_bounds__(kBnThreads)
       gsc[i] = aff.scale ? aff.scale[g[i]] : 1.f;
       gad[i] = (aff.add ? aff.add[g[i]] : 0.f) + aff.pb(g[i]);
     }
-    for (int64_t r = r0 + ty; r < r1; r += TY) {
+    // the next row's loads are in flight while the current row is worked on
+    Vec<V> a, an;
+    float xg[V], xgn[V];
+    auto load_row = [&](int64_t r, Vec<V> &dst, float (&dg)[V]) {
       const float *xr = x + r * c_in;
-      Vec<V> a;
-      a.load(xr + j);
+      dst.load(xr + j);
+#pragma unroll
+      // the columns of a field share their gate: neighbouring lanes read the same word
+      for (int i = 0; i < V; ++i) dg[i] = xr[g[i]];
+    };
+    int64_t r = r0 + ty;
+    if (r < r1) load_row(r, a, xg);
+    for (; r < r1; r += TY) {
+      load_row(r + TY < r1 ? r + TY : r, an, xgn);  // the last trip reloads its own row
+      Vec<V> o;
 #pragma unroll
       for (int i = 0; i < V; ++i) {
         float v = (a.v[i] - sh[i]) * sc[i] + ad[i];
         if (mode[i] == 1) {
           v = act_fn(act_s, v + pbj[i]);
         } else if (mode[i] == 2) {
-          // the columns of a field share their gate: neighbouring lanes read the same word
-          float gv = (xr[g[i]] - gsh[i]) * gsc[i] + gad[i];
+          float gv = (xg[i] - gsh[i]) * gsc[i] + gad[i];
           v *= act_fn(act_g, gv);
         }
-        a.v[i] = v;
+        o.v[i] = v;
       }
-      a.store(y + r * c_out + j);
+      o.store(y + r * c_out + j);
+      a = an;
+#pragma unroll
+      for (int i = 0; i < V; ++i) xg[i] = xgn[i];
     }
   }
 }
@@ -360,12 +373,53 @@ template <int V> struct GroupConst {
       gadp[i] = t.add[g[i]] + t.pre[g[i]];
     }
   }
-  // dz of column i of the group: x and dy of the column, xr the row of x
-  __device__ __forceinline__ float dz(int i, float x, float dy, const float *__restrict__ xr,
-                                      int act_s, int act_g) const {
+  // dz of column i of the group: x and dy of the column, xg the row's value in the
+  // column of the gate
+  __device__ __forceinline__ float dz(int i, float x, float dy, float xg, int act_s,
+                                      int act_g) const {
     if (mode[i] == 1) return dy * act_grad(act_s, (x - sh[i]) * sc[i] + ad[i] + pre[i]);
-    if (mode[i] == 2) return dy * act_fn(act_g, (xr[g[i]] - gsh[i]) * gsc[i] + gadp[i]);
+    if (mode[i] == 2) return dy * act_fn(act_g, (xg - gsh[i]) * gsc[i] + gadp[i]);
     return dy;
+  }
+};
+
+// One row's worth of a group's inputs: the group's columns of x and dy and the values in
+// its gates' columns.  Loaded one row ahead of its use, so that a wave always has the next
+// row's loads in flight while it works on the current one.
+template <int V> struct GroupRow {
+  Vec<V> x, dy;
+  float xg[V];
+  __device__ __forceinline__ void load(const float *__restrict__ xr, const float *__restrict__ dr,
+                                       int c0, const GroupConst<V> &gc) {
+    x.load(xr + c0);
+    dy.load(dr + c0);
+#pragma unroll
+    for (int i = 0; i < V; ++i) xg[i] = xr[gc.g[i]];
+  }
+};
+
+// A gate column's inputs for one row: its own value and, for a field of up to kMaxDim
+// columns, the field's x and dy.  Loaded one row ahead like GroupRow.
+constexpr int kGateMaxDim = 9;  // fields up to l = 4; wider fields take the plain loop
+struct GateRow {
+  float xc, xs[kGateMaxDim], ds[kGateMaxDim];
+  __device__ __forceinline__ void load(const float *__restrict__ xr, const float *__restrict__ dr,
+                                       int c, int first, int dim) {
+    xc = xr[c];
+#pragma unroll
+    for (int j = 0; j < kGateMaxDim; ++j) {
+      xs[j] = j < dim ? xr[first + j] : 0.f;
+      ds[j] = j < dim ? dr[first + j] : 0.f;
+    }
+  }
+  // dz of the gate column (see bnact_dz)
+  __device__ __forceinline__ float dz(const ColTables &t, int c, int first, int dim,
+                                      int act_g) const {
+    float acc = 0.f;
+#pragma unroll
+    for (int j = 0; j < kGateMaxDim; ++j)
+      if (j < dim) acc += ds[j] * t.z(xs[j], first + j);
+    return acc * act_grad(act_g, t.z(xc, c) + t.pre[c]);
   }
 };
 
@@ -424,25 +478,42 @@ __global__ void __launch_bounds__(kBnThreads)
     if (w.group) {
       GroupConst<V> gc;
       gc.init(t, w.c);
-      for (int64_t r = r0 + ty; r < r1; r += TY) {
-        const float *xr = x + r * c_in;
-        Vec<V> a, dv;
-        a.load(xr + w.c);
-        dv.load(dy + r * c_out + w.c);
+      GroupRow<V> cur, nxt;
+      int64_t r = r0 + ty;
+      if (r < r1) cur.load(x + r * c_in, dy + r * c_out, w.c, gc);
+      for (; r < r1; r += TY) {
+        const int64_t rn = r + TY < r1 ? r + TY : r;  // the last trip reloads its own row
+        nxt.load(x + rn * c_in, dy + rn * c_out, w.c, gc);
 #pragma unroll
         for (int i = 0; i < V; ++i) {
-          float d = gc.dz(i, a.v[i], dv.v[i], xr, act_s, act_g);
+          float d = gc.dz(i, cur.x.v[i], cur.dy.v[i], cur.xg[i], act_s, act_g);
           sb[i] += d;
-          sa[i] += d * (a.v[i] - sh[i]);
+          sa[i] += d * (cur.x.v[i] - sh[i]);
         }
+        cur = nxt;
       }
     } else if (w.width == 1) {
-      for (int64_t r = r0 + ty; r < r1; r += TY) {
-        const float *xr = x + r * c_in;
-        const float xc = xr[w.c];
-        float d = bnact_dz(xr, dy + r * c_out, xc, w.c, c_out, t, act_s, act_g);
-        sb[0] += d;
-        sa[0] += d * (xc - sh[0]);
+      const int dim = t.gdim[w.c], first = t.gfirst[w.c];
+      if (dim > 0 && dim <= kGateMaxDim) {
+        GateRow cur, nxt;
+        int64_t r = r0 + ty;
+        if (r < r1) cur.load(x + r * c_in, dy + r * c_out, w.c, first, dim);
+        for (; r < r1; r += TY) {
+          const int64_t rn = r + TY < r1 ? r + TY : r;
+          nxt.load(x + rn * c_in, dy + rn * c_out, w.c, first, dim);
+          float d = cur.dz(t, w.c, first, dim, act_g);
+          sb[0] += d;
+          sa[0] += d * (cur.xc - sh[0]);
+          cur = nxt;
+        }
+      } else {
+        for (int64_t r = r0 + ty; r < r1; r += TY) {
+          const float *xr = x + r * c_in;
+          const float xc = xr[w.c];
+          float d = bnact_dz(xr, dy + r * c_out, xc, w.c, c_out, t, act_s, act_g);
+          sb[0] += d;
+          sa[0] += d * (xc - sh[0]);
+        }
       }
     }
 #pragma unroll
@@ -489,24 +560,41 @@ __global__ void __launch_bounds__(kBnThreads)
     if (w.group) {
       GroupConst<V> gc;
       gc.init(t, w.c);
-      for (int64_t r = r0 + ty; r < r1; r += TY) {
-        const float *xr = x + r * c_in;
-        Vec<V> a, dv;
-        a.load(xr + w.c);
-        dv.load(dy + r * c_out + w.c);
+      GroupRow<V> cur, nxt;
+      int64_t r = r0 + ty;
+      if (r < r1) cur.load(x + r * c_in, dy + r * c_out, w.c, gc);
+      for (; r < r1; r += TY) {
+        const int64_t rn = r + TY < r1 ? r + TY : r;  // the last trip reloads its own row
+        nxt.load(x + rn * c_in, dy + rn * c_out, w.c, gc);
+        Vec<V> o;
 #pragma unroll
         for (int i = 0; i < V; ++i) {
-          float d = gc.dz(i, a.v[i], dv.v[i], xr, act_s, act_g);
-          a.v[i] = sc[i] * (d - dm[i]) - cf[i] * (a.v[i] - sh[i]);
+          float d = gc.dz(i, cur.x.v[i], cur.dy.v[i], cur.xg[i], act_s, act_g);
+          o.v[i] = sc[i] * (d - dm[i]) - cf[i] * (cur.x.v[i] - sh[i]);
         }
-        a.store(dx + r * c_in + w.c);
+        o.store(dx + r * c_in + w.c);
+        cur = nxt;
       }
     } else if (w.width == 1) {
-      for (int64_t r = r0 + ty; r < r1; r += TY) {
-        const float *xr = x + r * c_in;
-        const float xc = xr[w.c];
-        float d = bnact_dz(xr, dy + r * c_out, xc, w.c, c_out, t, act_s, act_g);
-        dx[r * c_in + w.c] = sc[0] * (d - dm[0]) - cf[0] * (xc - sh[0]);
+      const int dim = t.gdim[w.c], first = t.gfirst[w.c];
+      if (dim > 0 && dim <= kGateMaxDim) {
+        GateRow cur, nxt;
+        int64_t r = r0 + ty;
+        if (r < r1) cur.load(x + r * c_in, dy + r * c_out, w.c, first, dim);
+        for (; r < r1; r += TY) {
+          const int64_t rn = r + TY < r1 ? r + TY : r;
+          nxt.load(x + rn * c_in, dy + rn * c_out, w.c, first, dim);
+          float d = cur.dz(t, w.c, first, dim, act_g);
+          dx[r * c_in + w.c] = sc[0] * (d - dm[0]) - cf[0] * (cur.xc - sh[0]);
+          cur = nxt;
+        }
+      } else {
+        for (int64_t r = r0 + ty; r < r1; r += TY) {
+          const float *xr = x + r * c_in;
+          const float xc = xr[w.c];
+          float d = bnact_dz(xr, dy + r * c_out, xc, w.c, c_out, t, act_s, act_g);
+          dx[r * c_in + w.c] = sc[0] * (d - dm[0]) - cf[0] * (xc - sh[0]);
+        }
       }
     }
   }
