@@ -31,9 +31,11 @@ constexpr int kMinTile = 64;
 
 // ---- weight packing ---------------------------------------------------------------------
 // packed[((k*NCB + ncb)*NCH + cc)*1024 + lane*16 + c] =
-//     W[k][cc*64 + (lane/16)*16 + c][ncb*16 + lane%16]           (0 outside Cin/Cout)
-// i.e. the B fragment of MFMA step c of chunk cc for column block ncb, laid
-// out so that one wave reads it as four coalesced 16-byte loads per lane.
+//     W[k][cc*64 + (c/4)*16 + (lane/16)*4 + c%4][ncb*16 + lane%16]   (0 outside Cin/Cout)
+// i.e. the weight fragment of MFMA step c of chunk cc for column block ncb, laid out so
+// that one wave reads it as four coalesced 16-byte loads per lane.  The four steps of
+// load q cover the 16 channels 16q .. 16q+15 of the chunk (lane group g has channels
+// 16q + 4g .. +3), so a layer with few input channels needs only its first loads.
 __global__ void __launch_bounds__(256)
     pack_filters_kernel(const float *__restrict__ w, int64_t fs_k, int64_t fs_ci, int64_t fs_co,
                         int K, int cin, int cout, int ncb, int nch, float *__restrict__ packed,
@@ -49,7 +51,7 @@ __global__ void __launch_bounds__(256)
   r /= nch;
   int cb = r % ncb;
   int k = (int)(r / ncb);
-  int ci = cc * kKC + (lane >> 4) * 16 + c;
+  int ci = cc * kKC + (c >> 2) * 16 + (lane >> 4) * 4 + (c & 3);
   int co = cb * 16 + (lane & 15);
   float v = 0.f;
   if (ci < cin && co < cout) v = w[k * fs_k + ci * fs_ci + co * fs_co];
@@ -593,7 +595,10 @@ struct StagePos {
 //
 // The waves-per-SIMD attribute states the occupancy the workgroup size gives anyway
 // (one workgroup per CU), so that the compiler uses the whole register budget.
-template <int GATHER, int NCW>
+// NQ: 16-channel quarters of a chunk that hold input channels (4 unless the layer has
+// a single chunk with at most 48 channels): MFMA steps, fragment loads and staged-row
+// reads of the other quarters are left out.
+template <int GATHER, int NCW, int NQ>
 __global__ void __launch_bounds__((NCW + 4) * 64)
     __attribute__((amdgpu_waves_per_eu((NCW + 4) / 4, (NCW + 4) / 4)))
     conv_fwd_kernel(const float *__restrict__ features, int cin, unsigned feat_bytes,
@@ -826,7 +831,7 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
         __builtin_amdgcn_make_buffer_rsrc((void *)sched_out, 0, (int)sched_bytes, kRsrcFlags);
     const int w_voff = lane * 64;           // this lane's 16 floats of a fragment
     const int w_soff0 = cb * nch * 4096;    // fragments of this wave's column block
-    const float *const a_base = abuf + l16 * kAStride + g * 16;
+    const float *const a_base = abuf + l16 * kAStride + g * 4;
     // The accumulators are addressed with 32-bit LDS byte addresses (acc_lane includes
     // the base of acc): no pointer arithmetic left for the vector ALU.
     typedef __attribute__((address_space(3))) float4v lds_float4v;
@@ -912,6 +917,7 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
     // chain a handful of other instructions issue for free -- and no more than that:
     // everything else a block needs is therefore spread, one small piece per gap,
     // over the 16 gaps of the block, and scheduling barriers pin it there:
+    // (gap numbers for NQ = 4, i.e. 16 MFMAs a block)
     //   gap 2      fragment offset of block b+3 (from the schedule record); accumulator
     //              update of the previous block: add, write; once per stage, tile and
     //              last-of-tile of the next stage
@@ -934,10 +940,19 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
       const int base_next = w_soff0 + next.cc * 4096;
       float4v a[2][4];
       auto load_a = [&](int m, int q, float4v (&av)[4]) {
-        av[q] = reinterpret_cast<const float4v *>(ab + m * 16 * kAStride)[q];
+        av[q] = *reinterpret_cast<const float4v *>(ab + m * 16 * kAStride + q * 16);
       };
 #pragma unroll
-      for (int q = 0; q < 4; ++q) load_a(0, q, a[0]);
+      for (int q = 0; q < NQ; ++q) load_a(0, q, a[0]);
+      // gaps of the pieces of a block (see above); with fewer than 16 MFMAs they move
+      // closer together, in the same order
+      constexpr int kSteps = 4 * NQ;
+      constexpr int kGapAlu = NQ == 4 ? 2 : 1, kGapAcc = kGapAlu + 1;
+      constexpr int kGapW[4] = {NQ == 4 ? 4 : 2, NQ == 4 ? 7 : 3, NQ == 4 ? 9 : 4, 12};
+      constexpr int kGapRow = NQ == 4 ? 5 : 2;  // after fragment load 0 in the same gap
+      constexpr int kGapA[4] = {NQ == 4 ? 6 : kSteps / 2, NQ == 4 ? 8 : kSteps / 2 + 1,
+                                NQ == 4 ? 10 : kSteps / 2 + 2, 11};
+      constexpr int kGapRec0 = NQ == 4 ? 13 : kSteps - 2, kGapRec1 = NQ == 4 ? 14 : kSteps - 1;
 #pragma unroll
       for (int m = 0; m < 4; ++m) {
         const int slot = m;                 // == (4 * s + m) & 3
@@ -947,7 +962,7 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
         float4v d = float4v{0.f, 0.f, 0.f, 0.f};
         int soff = 0;
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
+        for (int i = 0; i < kSteps; ++i) {
           const int q = i >> 2, j = i & 3;
           __builtin_amdgcn_sched_barrier(0);
           d = __builtin_amdgcn_mfma_f32_16x16x4f32(w[slot][q][j], a[m & 1][q][j], d, 0, 0, 0);
@@ -955,7 +970,7 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
           // all vector-ALU work of the block in one gap: a vector-ALU instruction
           // next to the matrix chain costs about ten cycles for leaving and re-entering
           // the chain, whatever follows it in the same gap is cheap
-          if (i == 2) {
+          if (i == kGapAlu) {
             soff = tnext ? frag_soff(rec_k(rec[par ^ 1][0], tm), base_next)
                          : frag_soff(rec_k(rec[par][0], tm), base_cur);
             if (m == 3) end_next = tile_end_of(rec[par ^ 1][1], next);
@@ -963,23 +978,22 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
             lds_store4(pend.addr, pend.accr + pend.d);
             pend.addr = orow[slot] + acc_lane;
           }
-          if (i == 3) pend.accr = lds_load4(pend.addr);
-          if (i == 4) fetch_w(soff, tslot, 0);
-          if (i == 5) fetch_orow(tnext ? next : cur, tm, tslot);
+          if (i == kGapAcc) pend.accr = lds_load4(pend.addr);
+          if (i == kGapW[0]) fetch_w(soff, tslot, 0);
+          if (i == kGapRow) fetch_orow(tnext ? next : cur, tm, tslot);
+#pragma unroll
+          for (int qq = 1; qq < NQ; ++qq)
+            if (i == kGapW[qq]) fetch_w(soff, tslot, qq);
           if (m < 3) {
-            if (i == 6) load_a(m + 1, 0, a[(m + 1) & 1]);
-            if (i == 8) load_a(m + 1, 1, a[(m + 1) & 1]);
-            if (i == 10) load_a(m + 1, 2, a[(m + 1) & 1]);
-            if (i == 11) load_a(m + 1, 3, a[(m + 1) & 1]);
+#pragma unroll
+            for (int qq = 0; qq < NQ; ++qq)
+              if (i == kGapA[qq]) load_a(m + 1, qq, a[(m + 1) & 1]);
           }
-          if (i == 7) fetch_w(soff, tslot, 1);
-          if (i == 9) fetch_w(soff, tslot, 2);
-          if (i == 12) fetch_w(soff, tslot, 3);
           // this stage's record was last used by block 0: refill it for the stage
           // after the next
-          if (m == 1 && i == 13)
+          if (m == 1 && i == kGapRec0)
             rec[par][0] = __builtin_bit_cast(int4v, buf_load4(rs_meta, 0, after.g * 32));
-          if (m == 1 && i == 14) rec[par][1] = load_rec_tail(after);
+          if (m == 1 && i == kGapRec1) rec[par][1] = load_rec_tail(after);
         }
         __builtin_amdgcn_sched_barrier(0);
         pend.d = d;
@@ -1003,8 +1017,8 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
       load_rec(p_cur, rec[0]);
       load_rec(p_next, rec[1]);
       end = tile_end_of(rec[0][1], p_cur);
-      // Loads are issued in the order of the loop (fragments 0 and 1, the output rows,
-      // fragments 2 and 3, block after block) and pinned there: the wait counts of the
+      // Loads are issued in the order of the loop (fragment 0, the output rows, the other
+      // fragments, block after block) and pinned there: the wait counts of the
       // loop are static and must hold on its first trip as well, so a load that the
       // prologue issued late would make every trip wait for nearly all loads in flight.
 #pragma unroll
@@ -1013,14 +1027,13 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
         __builtin_amdgcn_sched_barrier(0);
         fetch_w(soff, b, 0);
         __builtin_amdgcn_sched_barrier(0);
-        fetch_w(soff, b, 1);
-        __builtin_amdgcn_sched_barrier(0);
         fetch_orow(p_cur, b, b);
         __builtin_amdgcn_sched_barrier(0);
-        fetch_w(soff, b, 2);
-        __builtin_amdgcn_sched_barrier(0);
-        fetch_w(soff, b, 3);
-        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int q = 1; q < NQ; ++q) {
+          fetch_w(soff, b, q);
+          __builtin_amdgcn_sched_barrier(0);
+        }
       }
     }
     __syncthreads();
@@ -1160,12 +1173,12 @@ static size_t conv_ws_bytes(int64_t n_out, int K, int c_in, int c_out, int64_t p
   return conv_ws_walk(nullptr, p, K, pair_stride, nullptr);
 }
 
-template <int GATHER, int NCW>
+template <int GATHER, int NCW, int NQ>
 static int launch_conv(const ConvPlan &p, const ConvWs &w, const float *features, int64_t n_in,
                        int c_in, int K, float *out, int c_out, hipStream_t s) {
   static bool attr_set = false;
   if (!attr_set) {
-    SSC_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(conv_fwd_kernel<GATHER, NCW>),
+    SSC_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(conv_fwd_kernel<GATHER, NCW, NQ>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
     attr_set = true;
   }
@@ -1176,7 +1189,7 @@ static int launch_conv(const ConvPlan &p, const ConvWs &w, const float *features
             (unsigned long long)packed_bytes, (unsigned long long)sched_bytes);
   const unsigned feat_bytes = GATHER != 0 ? (unsigned)((uint64_t)n_in * c_in * 4) : 0u;
   dim3 grid((unsigned)p.n_wg, (unsigned)p.n_colblk);
-  hipLaunchKernelGGL((conv_fwd_kernel<GATHER, NCW>), grid, dim3((NCW + 4) * 64), p.lds_bytes, s, features, c_in,
+  hipLaunchKernelGGL((conv_fwd_kernel<GATHER, NCW, NQ>), grid, dim3((NCW + 4) * 64), p.lds_bytes, s, features, c_in,
                      feat_bytes, w.packed, (unsigned)packed_bytes, w.sched_in, w.sched_out,
                      w.grp_meta, (unsigned)sched_bytes, (unsigned)(p.grp_cap * 32), w.tile_grp,
                      w.wg_tile, p.nch, p.ncb, out, c_out, p.T);
@@ -1314,12 +1327,20 @@ int ssc_conv_fwd_f32(const float *features, int64_t n_in, int32_t c_in, const fl
   const bool prof = g_profile_on;
   const int slot = g_profile_count % kProfileRing;
   if (prof) SSC_HIP(hipEventRecord(g_profile_ev[slot][0], s));
-  if (p.gather == 1)
-    rc = launch_conv<1, 4>(p, w, features, n_in, c_in, K, out, c_out, s);
-  else if (p.gather == 2)
-    rc = launch_conv<2, 4>(p, w, features, n_in, c_in, K, out, c_out, s);
-  else
-    rc = launch_conv<0, 4>(p, w, features, n_in, c_in, K, out, c_out, s);
+  // quarters of the (only) chunk that hold input channels; layers with several chunks
+  // run all four everywhere
+  const int nq = p.nch == 1 ? (int)ceil_div(c_in, 16) : 4;
+#define SSC_CONV_LAUNCH(G, Q) launch_conv<G, 4, Q>(p, w, features, n_in, c_in, K, out, c_out, s)
+  if (p.gather == 1) {
+    rc = SSC_CONV_LAUNCH(1, 4);
+  } else if (p.gather == 2) {
+    rc = nq == 1 ? SSC_CONV_LAUNCH(2, 1) : nq == 2 ? SSC_CONV_LAUNCH(2, 2)
+       : nq == 3 ? SSC_CONV_LAUNCH(2, 3) : SSC_CONV_LAUNCH(2, 4);
+  } else {
+    rc = nq == 1 ? SSC_CONV_LAUNCH(0, 1) : nq == 2 ? SSC_CONV_LAUNCH(0, 2)
+       : nq == 3 ? SSC_CONV_LAUNCH(0, 3) : SSC_CONV_LAUNCH(0, 4);
+  }
+#undef SSC_CONV_LAUNCH
   if (rc != SSC_OK) return rc;
   if (prof) {
     SSC_HIP(hipEventRecord(g_profile_ev[slot][1], s));

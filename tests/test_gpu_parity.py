@@ -119,6 +119,9 @@ CONV_CASES = [
     (6000, 24, 3, 1, 1, 64, 80),
     # two channel chunks on the buffer-load gather path, 3 column blocks
     (1500, 16, 3, 1, 1, 128, 136),
+    # a single chunk with three 16-channel quarters in use, both gather paths
+    (700, 12, 3, 1, 1, 40, 64),
+    (700, 12, 3, 1, 1, 37, 24),
 ]
 
 
