@@ -836,3 +836,67 @@ def test_conv_order_promise_follows_the_input_order(oracle, device):
             torch.from_numpy(go).to(device), pairs, num, 0, 0)
         want, _ = oracle.conv_bwd(f, w, go, r_pairs, r_num)
         assert rel_l2(gi.cpu().numpy(), want) < REL_L2
+
+
+def test_backbone_forward_matches_oracle(oracle, device):
+    """The fourth benchmark configuration at reduced size: Point2Voxel -> four stages of
+    [Convolution k3 -> BatchNorm -> gated Activation] with irreps (8,8,8,8) -> (16,...) ->
+    (32,...) -> (32,...), stride 2 at stages 2 and 3 -> GlobalAvgPool and Voxel2Point, in
+    training mode (batch statistics), against the oracle's composition of the same steps."""
+    from ss_conv.activation import Activation
+    from ss_conv.batchnorm import BatchNorm
+    from ss_conv.convolution import Convolution
+    from ss_conv.fused import BatchNormActivation
+    from ss_conv.pool import GlobalAvgPool
+    from ss_conv.sp_ops.voxelize import Point2Voxel, Voxel2Point
+    torch.manual_seed(3)
+    batch, grid = 3, 24
+    pts, feats, ids = synth.make_clouds(batch, 700, seed=10, channels=3)
+    rs_in = [(3, 0)]
+    stages = [(synth.irreps(8, 3), 1), (synth.irreps(16, 3), 2), (synth.irreps(32, 3), 2),
+              (synth.irreps(32, 3), 1)]
+    p2v = Point2Voxel([grid] * 3, [2.0 / grid] * 3)
+    vp, st, vi, _ = p2v(*[torch.from_numpy(x).to(device) for x in (pts, feats, ids)])
+    # oracle side starts from the same voxels
+    o_idx = st.indices.cpu().numpy()
+    o_feat = st.features.cpu().numpy().astype(np.float64)
+    shape = [grid] * 3
+    x = st
+    for si, (rs, stride) in enumerate(stages):
+        n_gates = sum(m for m, _ in rs[1:])
+        rs_gated = rs + [(n_gates, 0)]
+        conv = Convolution(rs_in, rs_gated, 3, stride=stride, padding=1).to(device).train()
+        block = BatchNormActivation(BatchNorm(rs_gated), Activation(rs, (torch.relu, torch.sigmoid)))
+        block = block.to(device).train()
+        with torch.no_grad():
+            for p in block.parameters():
+                p.add_(torch.randn_like(p) * 0.3)
+            x = block(conv(x))
+        # oracle: rulebook, convolution with the layer's synthesised kernel, batch norm, gate
+        cin = sum(m * (2 * l + 1) for m, l in rs_in)
+        cout = sum(m * (2 * l + 1) for m, l in rs_gated)
+        w = conv.kernel().detach().permute(2, 3, 4, 1, 0).reshape(27, cin, cout).cpu().numpy()
+        r_idx, r_pairs, r_num, r_shape = oracle.rulebook(o_idx, batch, shape, 3, stride, 1)
+        r_idx, r_pairs, r_num = oracle.canonicalize(r_idx, r_pairs, r_num, r_shape)
+        y = oracle.conv_fwd(o_feat.astype(np.float32), w, r_pairs, r_num, r_idx.shape[0],
+                            matmul=np.matmul)
+        as_np = lambda t: t.detach().cpu().numpy()  # noqa: E731
+        params = dict(weight=as_np(block.bn.weight), bias=as_np(block.bn.bias),
+                      scalar_bias=as_np(block.act.scalar_act.bias),
+                      gate_bias=as_np(block.act.gate_act.bias))
+        o_feat = oracle.bn_gate_fwd(y, rs_gated, rs, params, training=True)
+        o_idx, shape, rs_in = r_idx, list(r_shape), rs
+        assert np.array_equal(x.indices.cpu().numpy(), o_idx), si
+        err = rel_l2(x.features.cpu().numpy(), o_feat)
+        print("stage", si, "rows", o_idx.shape[0], "rel-l2", err, flush=True)
+        assert err < REL_L2, (si, err)
+    # heads: per-cloud mean of the voxel features, and the features read back at the points
+    offs = x.get_offsets().int().contiguous()
+    pooled = GlobalAvgPool()(x.features.contiguous(), offs).cpu().numpy()
+    want = oracle.segment_avg(o_feat.astype(np.float32), offs.cpu().numpy())
+    assert rel_l2(pooled, want) < REL_L2
+    v2p = Voxel2Point(unit_voxel_extent=[2.0 / s for s in shape])
+    at_points = v2p(x, vp, vi).cpu().numpy()
+    want = oracle.voxel2point(o_idx, o_feat.astype(np.float32), shape, vp.cpu().numpy(),
+                              vi.cpu().numpy(), unit_voxel_extent=[2.0 / s for s in shape])[0]
+    assert rel_l2(at_points, want) < REL_L2
