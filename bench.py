@@ -228,6 +228,36 @@ def ops_table(torch, _ext, synth, dev, seed):
     finally:
         bnact.usable = keep
     report("same layers as torch ops, forward + backward", ms, nbytes, "same algorithmic bytes")
+
+    # the whole backbone of the fourth configuration: Point2Voxel (64^3) -> four stages of
+    # [Convolution k3 -> BatchNorm -> gated Activation], irreps (8,8,8,8) -> (16,...) ->
+    # (32,...) -> (32,...), stride 2 at stages 2 and 3 -> GlobalAvgPool + Voxel2Point
+    from ss_conv.convolution import Convolution
+    pts, feats, ids = synth.make_clouds(32, 1024, seed=seed, channels=3)
+    tp, tf, ti = [torch.from_numpy(a).to(dev) for a in (pts, feats, ids)]
+    p2v = Point2Voxel([64] * 3, [2.0 / 64] * 3)
+    layers, rs_in = [], [(3, 0)]
+    for mult, stride in ((8, 1), (16, 2), (32, 2), (32, 1)):
+        rs = synth.irreps(mult, 3)
+        gated = rs + [(sum(m for m, l in rs[1:]), 0)]
+        conv = Convolution(rs_in, gated, 3, stride=stride, padding=1).to(dev).eval()
+        block = BatchNormActivation(BatchNorm(gated), Activation(rs, (torch.relu, torch.sigmoid)))
+        layers.append((conv, block.to(dev).eval()))
+        rs_in = rs
+    gap = GlobalAvgPool()
+
+    def backbone():
+        vp, x, vi, _ = p2v(tp, tf, ti)
+        for conv, block in layers:
+            x = block(conv(x))
+        pooled = gap(x.features.contiguous(), x.get_offsets().int().contiguous())
+        v2p = Voxel2Point(unit_voxel_extent=[2.0 / s for s in x.spatial_shape])
+        return pooled, v2p(x, vp, vi), x
+    with torch.no_grad():
+        ms, r = timed(backbone, n=5, warm=2)
+    rows.append("%-44s %8.3f ms   (%d clouds x 1024 points; %d voxels after stage 4, %d channels)"
+                % ("backbone forward, 4th configuration (eval)", ms, 32, r[2].features.shape[0],
+                   r[2].features.shape[1]))
     print("\n".join(rows), file=sys.stderr)
 
 
