@@ -133,6 +133,21 @@ int ssc_conv_fwd_f32(const float *features /* [n_in,c_in] */, int64_t n_in, int3
                      float *out /* [n_out,c_out] */, int64_t n_out, void *workspace,
                      size_t workspace_bytes, ssc_stream_t stream);
 
+/* Half-precision storage: features, filters and out hold IEEE binary16 elements.  Replaces
+ * indiceConv<at::Half> (bound as indice_conv_half, src/ss_conv_ops.cu:74-78,
+ * src/ss_conv_ops_api.cpp:23).  Same arguments and workspace as ssc_conv_fwd_f32 (strides
+ * in elements).  The arithmetic is that of the fp32 call -- the rows are widened on their
+ * way into LDS, products and sums run on fp32 MFMA -- and each output element is rounded
+ * to half once (nearest even), where the reference rounds after every offset's GEMM and
+ * again in every scatter-add (src/conv/reordering_cuda_functor.cu:158-210). */
+int ssc_conv_fwd_f16(const void *features /* [n_in,c_in] half */, int64_t n_in, int32_t c_in,
+                     const void *filters /* half */, int64_t fs_k, int64_t fs_ci, int64_t fs_co,
+                     int32_t c_out, const int32_t *pairs /* [K,2,pair_stride] */,
+                     int64_t pair_stride, const int32_t *pair_num /* [K] device */,
+                     int32_t kernel_volume, int32_t inverse, int32_t subm,
+                     void *out /* [n_out,c_out] half */, int64_t n_out, void *workspace,
+                     size_t workspace_bytes, ssc_stream_t stream);
+
 /* ----------------------------------------------------------------------
  * Gradients of the sparse convolution -- replaces indice_conv_backward_fp32
  * (src/ss_conv_ops_api.cpp:22, src/conv/indice_conv.h:344-426).
@@ -156,6 +171,19 @@ int ssc_conv_bwd_filter_f32(const float *features /* [n_in,c_in] */, int64_t n_i
                             int64_t pair_stride, const int32_t *pair_num /* [K] */,
                             int32_t kernel_volume, int32_t inverse, float *filters_grad,
                             int64_t gs_k, int64_t gs_ci, int64_t gs_co, void *workspace,
+                            size_t workspace_bytes, ssc_stream_t stream);
+
+/* Half-precision storage (features, out_grad and filters_grad hold IEEE binary16):
+ * replaces the filter half of indiceConvBackward<at::Half> (bound as
+ * indice_conv_backward_half, src/ss_conv_ops.cu:79-83, src/ss_conv_ops_api.cpp:24).
+ * Products and sums in fp32, one rounding per element of filters_grad; same workspace. */
+int ssc_conv_bwd_filter_f16(const void *features /* [n_in,c_in] half */, int64_t n_in,
+                            int32_t c_in, const void *out_grad /* [n_out,c_out] half */,
+                            int64_t n_out, int32_t c_out,
+                            const int32_t *pairs /* [K,2,pair_stride] */, int64_t pair_stride,
+                            const int32_t *pair_num /* [K] */, int32_t kernel_volume,
+                            int32_t inverse, void *filters_grad /* half */, int64_t gs_k,
+                            int64_t gs_ci, int64_t gs_co, void *workspace,
                             size_t workspace_bytes, ssc_stream_t stream);
 
 /* Timing of the convolution kernel alone (no counterpart in the reference, whose

@@ -36,8 +36,9 @@ constexpr int kMinTile = 64;
 // that one wave reads it as four coalesced 16-byte loads per lane.  The four steps of
 // load q cover the 16 channels 16q .. 16q+15 of the chunk (lane group g has channels
 // 16q + 4g .. +3), so a layer with few input channels needs only its first loads.
+template <typename IO>
 __global__ void __launch_bounds__(256)
-    pack_filters_kernel(const float *__restrict__ w, int64_t fs_k, int64_t fs_ci, int64_t fs_co,
+    pack_filters_kernel(const IO *__restrict__ w, int64_t fs_k, int64_t fs_ci, int64_t fs_co,
                         int K, int cin, int cout, int ncb, int nch, float *__restrict__ packed,
                         int32_t *__restrict__ flag) {
   int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -54,7 +55,7 @@ __global__ void __launch_bounds__(256)
   int ci = cc * kKC + (c >> 2) * 16 + (lane >> 4) * 4 + (c & 3);
   int co = cb * 16 + (lane & 15);
   float v = 0.f;
-  if (ci < cin && co < cout) v = w[k * fs_k + ci * fs_ci + co * fs_co];
+  if (ci < cin && co < cout) v = (float)w[k * fs_k + ci * fs_ci + co * fs_co];
   packed[idx] = v;
 }
 
@@ -571,6 +572,44 @@ __device__ __forceinline__ int buf_load1(__amdgpu_buffer_rsrc_t r, int voff, int
   return (int)__builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, 0);
 }
 
+// Element type of the features, the filters and the output.  The arithmetic is fp32
+// either way: half-precision rows are widened when the producers stage them and the
+// accumulators are rounded once, when a finished tile is written.
+typedef int int2v __attribute__((ext_vector_type(2)));
+typedef _Float16 half4v __attribute__((ext_vector_type(4)));
+template <typename IO> struct Io;
+template <> struct Io<float> {
+  static constexpr int kBytes = 4;
+  typedef float4v Raw;  // four channels as they are loaded
+  static __device__ __forceinline__ Raw gather(__amdgpu_buffer_rsrc_t r, int voff, int soff) {
+    return buf_load4(r, voff, soff);
+  }
+  static __device__ __forceinline__ Raw load(const float *p) {
+    return *reinterpret_cast<const float4v *>(p);
+  }
+  static __device__ __forceinline__ void store_stream(float *p, const float4v &v) {
+    __builtin_nontemporal_store(v, reinterpret_cast<float4v *>(p));
+  }
+};
+template <> struct Io<_Float16> {
+  static constexpr int kBytes = 2;
+  typedef int2v Raw;
+  static __device__ __forceinline__ Raw gather(__amdgpu_buffer_rsrc_t r, int voff, int soff) {
+    return __builtin_bit_cast(int2v, __builtin_amdgcn_raw_buffer_load_b64(r, voff, soff, 0));
+  }
+  static __device__ __forceinline__ Raw load(const _Float16 *p) {
+    return *reinterpret_cast<const int2v *>(p);
+  }
+  static __device__ __forceinline__ void store_stream(_Float16 *p, const float4v &v) {
+    const half4v h = __builtin_convertvector(v, half4v);  // round to nearest even
+    __builtin_nontemporal_store(__builtin_bit_cast(int2v, h), reinterpret_cast<int2v *>(p));
+  }
+};
+__device__ __forceinline__ float4v widen(const float4v &v) { return v; }
+__device__ __forceinline__ float4v widen(const int2v &v) {
+  return __builtin_convertvector(__builtin_bit_cast(half4v, v), float4v);
+}
+
 // Position of a stage in the schedule: group index and channel chunk.  Advanced
 // with scalar arithmetic only.
 struct StagePos {
@@ -598,16 +637,18 @@ struct StagePos {
 // NQ: 16-channel quarters of a chunk that hold input channels (4 unless the layer has
 // a single chunk with at most 48 channels): MFMA steps, fragment loads and staged-row
 // reads of the other quarters are left out.
-template <int GATHER, int NCW, int NQ>
+template <typename IO, int GATHER, int NCW, int NQ>
 __global__ void __launch_bounds__((NCW + 4) * 64)
     __attribute__((amdgpu_waves_per_eu((NCW + 4) / 4, (NCW + 4) / 4)))
-    conv_fwd_kernel(const float *__restrict__ features, int cin, unsigned feat_bytes,
+    conv_fwd_kernel(const IO *__restrict__ features, int cin, unsigned feat_bytes,
                     const float *__restrict__ packed, unsigned packed_bytes,
                     const int32_t *__restrict__ sched_in, const int32_t *__restrict__ sched_out,
                     const int32_t *__restrict__ grp_meta, unsigned sched_bytes, unsigned meta_bytes,
                     const int32_t *__restrict__ tile_grp, const int32_t *__restrict__ wg_tile,
-                    int nch, int ncb, float *__restrict__ out, int cout, int T) {
+                    int nch, int ncb, IO *__restrict__ out, int cout, int T) {
   constexpr int kCN = 16 * NCW;   // output columns per workgroup
+  constexpr int kEB = Io<IO>::kBytes;
+  typedef typename Io<IO>::Raw Raw;
   constexpr int kAS = kCN + 4;    // accumulator row stride in floats
   constexpr int NT = (NCW + 4) * 64;
   constexpr int NP = 256;  // producer threads
@@ -653,7 +694,7 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
       constexpr int RS = NT / (kCN / 4);  // rows per step
       const int r_t = tid / (kCN / 4), c_t = (tid % (kCN / 4)) * 4;
       const bool col_ok = col0 + c_t < cout;
-      float *gp = out + (int64_t)(row0 + r_t) * cout + col0 + c_t;
+      IO *gp = out + (int64_t)(row0 + r_t) * cout + col0 + c_t;
       const int64_t gstep = (int64_t)RS * cout;
       for (int r = r_t; r < rows; r += U * RS) {
         float4v v[U];
@@ -671,7 +712,7 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
           // streaming store: the output is not read again by this kernel and must not
           // push the weights and the gathered rows out of L2
           if (r + u * RS < rows && col_ok)
-            __builtin_nontemporal_store(v[u], reinterpret_cast<float4v *>(gp + u * gstep));
+            Io<IO>::store_stream(gp + u * gstep, v[u]);
         gp += U * gstep;
       }
     } else {
@@ -680,7 +721,7 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
         int sl = slot0 + r;
         if (sl >= T) sl -= T;
         if (col0 + c < cout)
-          __builtin_nontemporal_store(acc[sl * kAS + c], out + (int64_t)(row0 + r) * cout + col0 + c);
+          __builtin_nontemporal_store((IO)acc[sl * kAS + c], out + (int64_t)(row0 + r) * cout + col0 + c);
         acc[sl * kAS + c] = 0.f;
       }
     }
@@ -707,11 +748,13 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
     const __amdgpu_buffer_rsrc_t rs_feat =
         __builtin_amdgcn_make_buffer_rsrc((void *)features, 0, (int)feat_bytes, kRsrcFlags);
     const int idx_voff = (pt >> 4) * 4;    // this thread's slot (plus 16 slots per element)
-    const int chunk_off = (pt & 15) * 16;  // this thread's 16 bytes of a 256-byte row chunk
+    const int chunk_off = (pt & 15) * 4 * kEB;  // this thread's 4 channels of a 64-channel row chunk
     // this thread's 4 channels of the last chunk lie beyond Cin
     const bool beyond_cin = (nch - 1) * kKC + (pt & 15) * 4 >= cin;
+    // rows in flight stay as loaded (half precision: half the registers)
+    typedef std::conditional_t<GATHER == 0, float4v, Raw> Held;
     int idx[ID][NE];
-    float4v rows[RD][NE];
+    Held rows[RD][NE];
     // Rings indexed by stage number: rows of stage st in rows[st & 3], gather offsets
     // in idx[st & 1].  The loop is unrolled four times so that every ring index is a
     // compile-time constant: rotating a ring through register moves would read
@@ -725,26 +768,26 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
         ix[j] = v;
       }
     };
-    auto load_rows = [&](const StagePos &pos, const int (&ix)[NE], float4v (&r)[NE]) {
+    auto load_rows = [&](const StagePos &pos, const int (&ix)[NE], Held (&r)[NE]) {
 #pragma unroll
       for (int j = 0; j < NE; ++j) {
-        if (GATHER == 1) {
-          r[j] = buf_load4(rs_feat, ix[j] + chunk_off, pos.cc * 256);
-        } else if (GATHER == 2) {
+        if constexpr (GATHER == 1) {
+          r[j] = Io<IO>::gather(rs_feat, ix[j] + chunk_off, pos.cc * (kKC * kEB));
+        } else if constexpr (GATHER == 2) {
           const int off = (pos.cc == nch - 1 && beyond_cin) ? (int)kGatherPad : ix[j];
-          r[j] = buf_load4(rs_feat, off + chunk_off, pos.cc * 256);
+          r[j] = Io<IO>::gather(rs_feat, off + chunk_off, pos.cc * (kKC * kEB));
         } else {
           const int ch = pos.cc * kKC + (pt & 15) * 4;
           const int row = ix[j] < 0 ? 0 : ix[j];  // padding slots read row 0 and drop it
-          const float *fp = features + (int64_t)row * cin + ch;
+          const IO *fp = features + (int64_t)row * cin + ch;
           float4v v = float4v{0.f, 0.f, 0.f, 0.f};
           if ((cin & 3) == 0) {
-            if (ch < cin) v = *reinterpret_cast<const float4v *>(fp);
+            if (ch < cin) v = widen(Io<IO>::load(fp));
           } else {
-            if (ch + 0 < cin) v.x = fp[0];
-            if (ch + 1 < cin) v.y = fp[1];
-            if (ch + 2 < cin) v.z = fp[2];
-            if (ch + 3 < cin) v.w = fp[3];
+            if (ch + 0 < cin) v.x = (float)fp[0];
+            if (ch + 1 < cin) v.y = (float)fp[1];
+            if (ch + 2 < cin) v.z = (float)fp[2];
+            if (ch + 3 < cin) v.w = (float)fp[3];
           }
           if (ix[j] < 0) v = float4v{0.f, 0.f, 0.f, 0.f};
           r[j] = v;
@@ -752,10 +795,10 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
       }
     };
     float *const st_base = abuf + (pt >> 4) * kAStride + (pt & 15) * 4;
-    auto store_rows = [&](int parity, const float4v (&r)[NE]) {
+    auto store_rows = [&](int parity, const Held (&r)[NE]) {
 #pragma unroll
       for (int j = 0; j < NE; ++j)
-        *reinterpret_cast<float4v *>(st_base + (parity * kStage + j * 16) * kAStride) = r[j];
+        *reinterpret_cast<float4v *>(st_base + (parity * kStage + j * 16) * kAStride) = widen(r[j]);
     };
     // Prologue.  Loads are issued in the order the loop will wait for them (offsets,
     // then rows, oldest stage first): the wait counts of the loop are static, so
@@ -775,7 +818,7 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
         load_idx(p_idx, RD + j, idx[(RD + j) & 1]);
         p_idx.advance(nch);
       }
-      float4v r0[NE];
+      Held r0[NE];
       load_rows(p_rows, ix[0], r0);
       p_rows.advance(nch);
 #pragma unroll
@@ -1093,17 +1136,17 @@ static int device_cu_count() {
 }
 
 static ConvPlan make_plan(int64_t n_in, int64_t n_out, int K, int c_in, int c_out,
-                          int64_t pair_stride) {
+                          int64_t pair_stride, int elem_bytes = 4) {
   ConvPlan p;
   p.ncb = (int)ceil_div(c_out, 16);
   p.nch = (int)ceil_div(c_in, kKC);
   p.ncw = 4;
   p.T = pick_tile(p.ncw);
   p.tile_rows = p.T - kSpillRows;
-  // the gather can be a range-checked buffer load when rows are multiples of 16 bytes
-  // and byte offsets into the features (plus the padding marker) fit 32 bits
+  // the gather can be a range-checked buffer load when rows are multiples of four
+  // channels and byte offsets into the features (plus the padding marker) fit 32 bits
   p.gather = 0;
-  if ((c_in & 3) == 0 && (uint64_t)n_in * c_in * 4 <= (uint64_t)kGatherPad)
+  if ((c_in & 3) == 0 && (uint64_t)n_in * c_in * elem_bytes <= (uint64_t)kGatherPad)
     p.gather = (c_in % kKC) == 0 ? 1 : 2;
   p.n_colblk = (int)ceil_div(p.ncb, p.ncw);
   int n_wg = device_cu_count() / p.n_colblk;
@@ -1173,12 +1216,12 @@ static size_t conv_ws_bytes(int64_t n_out, int K, int c_in, int c_out, int64_t p
   return conv_ws_walk(nullptr, p, K, pair_stride, nullptr);
 }
 
-template <int GATHER, int NCW, int NQ>
-static int launch_conv(const ConvPlan &p, const ConvWs &w, const float *features, int64_t n_in,
-                       int c_in, int K, float *out, int c_out, hipStream_t s) {
+template <typename IO, int GATHER, int NCW, int NQ>
+static int launch_conv(const ConvPlan &p, const ConvWs &w, const IO *features, int64_t n_in,
+                       int c_in, int K, IO *out, int c_out, hipStream_t s) {
   static bool attr_set = false;
   if (!attr_set) {
-    SSC_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(conv_fwd_kernel<GATHER, NCW, NQ>),
+    SSC_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(conv_fwd_kernel<IO, GATHER, NCW, NQ>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
     attr_set = true;
   }
@@ -1187,9 +1230,9 @@ static int launch_conv(const ConvPlan &p, const ConvWs &w, const float *features
   SSC_CHECK(packed_bytes < ((uint64_t)1 << 32) && sched_bytes < ((uint64_t)1 << 32), SSC_ERUNTIME,
             "convolution too large for 32-bit buffer offsets (filters %llu B, schedule %llu B)",
             (unsigned long long)packed_bytes, (unsigned long long)sched_bytes);
-  const unsigned feat_bytes = GATHER != 0 ? (unsigned)((uint64_t)n_in * c_in * 4) : 0u;
+  const unsigned feat_bytes = GATHER != 0 ? (unsigned)((uint64_t)n_in * c_in * sizeof(IO)) : 0u;
   dim3 grid((unsigned)p.n_wg, (unsigned)p.n_colblk);
-  hipLaunchKernelGGL((conv_fwd_kernel<GATHER, NCW, NQ>), grid, dim3((NCW + 4) * 64), p.lds_bytes, s, features, c_in,
+  hipLaunchKernelGGL((conv_fwd_kernel<IO, GATHER, NCW, NQ>), grid, dim3((NCW + 4) * 64), p.lds_bytes, s, features, c_in,
                      feat_bytes, w.packed, (unsigned)packed_bytes, w.sched_in, w.sched_out,
                      w.grp_meta, (unsigned)sched_bytes, (unsigned)(p.grp_cap * 32), w.tile_grp,
                      w.wg_tile, p.nch, p.ncb, out, c_out, p.T);
@@ -1241,13 +1284,29 @@ size_t ssc_conv_workspace_bytes(int64_t n_out, int32_t kernel_volume, int32_t c_
   if (n_out < 0 || kernel_volume < 1 || c_in < 1 || c_out < 1 || pair_stride < 0) return 0;
   return conv_ws_bytes(n_out, kernel_volume, c_in, c_out, pair_stride);
 }
+}  // extern "C"
 
-int ssc_conv_fwd_f32(const float *features, int64_t n_in, int32_t c_in, const float *filters,
-                     int64_t fs_k, int64_t fs_ci, int64_t fs_co, int32_t c_out,
-                     const int32_t *pairs, int64_t pair_stride, const int32_t *pair_num,
-                     int32_t kernel_volume, int32_t inverse, int32_t subm, float *out,
-                     int64_t n_out, void *workspace, size_t workspace_bytes,
-                     ssc_stream_t stream) {
+template <typename IO>
+__global__ void __launch_bounds__(256) zero_rows_kernel(IO *__restrict__ p, int64_t n) {
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t step = (int64_t)gridDim.x * blockDim.x;
+  for (; i < n; i += step) p[i] = (IO)0.f;
+}
+template <typename IO> static int fill_zero(IO *p, int64_t n, hipStream_t s) {
+  if (n <= 0) return SSC_OK;
+  const int64_t blocks = ceil_div(n, 256) < 8192 ? ceil_div(n, 256) : 8192;
+  hipLaunchKernelGGL(zero_rows_kernel<IO>, dim3((unsigned)blocks), dim3(256), 0, s, p, n);
+  SSC_LAUNCH_CHECK("zero_rows");
+  return SSC_OK;
+}
+
+// The forward convolution for features, filters and output of element type IO.
+template <typename IO>
+static int conv_fwd(const IO *features, int64_t n_in, int32_t c_in, const IO *filters,
+                    int64_t fs_k, int64_t fs_ci, int64_t fs_co, int32_t c_out,
+                    const int32_t *pairs, int64_t pair_stride, const int32_t *pair_num,
+                    int32_t kernel_volume, int32_t inverse, int32_t subm, IO *out, int64_t n_out,
+                    void *workspace, size_t workspace_bytes, ssc_stream_t stream) {
   const int K = kernel_volume;
   SSC_CHECK(K >= 1 && K <= SSC_MAX_KERNEL_VOLUME, SSC_ERUNTIME, "kernel volume %d out of range", K);
   SSC_CHECK(c_in >= 1 && c_out >= 1, SSC_EINVAL, "channel counts must be positive");
@@ -1257,14 +1316,14 @@ int ssc_conv_fwd_f32(const float *features, int64_t n_in, int32_t c_in, const fl
   if (n_out == 0) return SSC_OK;
   SSC_CHECK(out != nullptr, SSC_EINVAL, "out is NULL");
   hipStream_t s = (hipStream_t)stream;
-  if (pair_stride == 0 || n_in == 0) return fill_f32(out, n_out * c_out, 0.f, s);
+  if (pair_stride == 0 || n_in == 0) return fill_zero(out, n_out * c_out, s);
   SSC_CHECK(features && filters && pairs && pair_num && workspace, SSC_EINVAL,
             "NULL pointer argument");
   size_t need = conv_ws_bytes(n_out, K, c_in, c_out, pair_stride);
   SSC_CHECK(workspace_bytes >= need, SSC_EWORKSPACE, "conv workspace too small: %zu < %zu",
             workspace_bytes, need);
 
-  ConvPlan p = make_plan(n_in, n_out, K, c_in, c_out, pair_stride);
+  ConvPlan p = make_plan(n_in, n_out, K, c_in, c_out, pair_stride, (int)sizeof(IO));
   ConvWs w;
   conv_ws_walk(workspace, p, K, pair_stride, &w);
   const int plane_g = inverse ? 1 : 0;
@@ -1272,7 +1331,7 @@ int ssc_conv_fwd_f32(const float *features, int64_t n_in, int32_t c_in, const fl
   int rc;
 
   int64_t packed_n = (int64_t)K * p.ncb * p.nch * 1024;
-  hipLaunchKernelGGL(pack_filters_kernel, dim3((unsigned)ceil_div(packed_n, 256)), dim3(256), 0, s,
+  hipLaunchKernelGGL(pack_filters_kernel<IO>, dim3((unsigned)ceil_div(packed_n, 256)), dim3(256), 0, s,
                      filters, fs_k, fs_ci, fs_co, K, c_in, c_out, p.ncb, p.nch, w.packed, w.flag);
   SSC_LAUNCH_CHECK("pack_filters");
 
@@ -1319,7 +1378,8 @@ int ssc_conv_fwd_f32(const float *features, int64_t n_in, int32_t c_in, const fl
                      dim3(256), 0, s, w.flag, pairs, w.sorted, pair_stride, plane_g,
                      w.share_first, w.share_cnt, w.kofs, w.tile_nmb, w.tile_grp, K,
                      w.n_tiles_dev, w.tile_row0, w.tile_slot0, p.T,
-                     p.gather ? (uint32_t)c_in * 4u : 1u, p.gather ? kGatherPad : 0xFFFFFFFFu,
+                     p.gather ? (uint32_t)c_in * (uint32_t)sizeof(IO) : 1u,
+                     p.gather ? kGatherPad : 0xFFFFFFFFu,
                      (16 * p.ncw + 4) * 4, p.ncb * p.nch * 4096, w.sched_in, w.sched_out,
                      w.grp_meta);
   SSC_LAUNCH_CHECK("schedule");
@@ -1330,8 +1390,12 @@ int ssc_conv_fwd_f32(const float *features, int64_t n_in, int32_t c_in, const fl
   // quarters of the (only) chunk that hold input channels; layers with several chunks
   // run all four everywhere
   const int nq = p.nch == 1 ? (int)ceil_div(c_in, 16) : 4;
-#define SSC_CONV_LAUNCH(G, Q) launch_conv<G, 4, Q>(p, w, features, n_in, c_in, K, out, c_out, s)
-  if (p.gather == 1) {
+#define SSC_CONV_LAUNCH(G, Q) launch_conv<IO, G, 4, Q>(p, w, features, n_in, c_in, K, out, c_out, s)
+  if constexpr (sizeof(IO) == 2) {
+    // half precision: one instance per gather mode (all four quarters)
+    rc = p.gather == 1 ? SSC_CONV_LAUNCH(1, 4)
+       : p.gather == 2 ? SSC_CONV_LAUNCH(2, 4) : SSC_CONV_LAUNCH(0, 4);
+  } else if (p.gather == 1) {
     rc = SSC_CONV_LAUNCH(1, 4);
   } else if (p.gather == 2) {
     rc = nq == 1 ? SSC_CONV_LAUNCH(2, 1) : nq == 2 ? SSC_CONV_LAUNCH(2, 2)
@@ -1340,6 +1404,7 @@ int ssc_conv_fwd_f32(const float *features, int64_t n_in, int32_t c_in, const fl
     rc = nq == 1 ? SSC_CONV_LAUNCH(0, 1) : nq == 2 ? SSC_CONV_LAUNCH(0, 2)
        : nq == 3 ? SSC_CONV_LAUNCH(0, 3) : SSC_CONV_LAUNCH(0, 4);
   }
+  (void)nq;
 #undef SSC_CONV_LAUNCH
   if (rc != SSC_OK) return rc;
   if (prof) {
@@ -1347,5 +1412,30 @@ int ssc_conv_fwd_f32(const float *features, int64_t n_in, int32_t c_in, const fl
     ++g_profile_count;
   }
   return SSC_OK;
+}
+
+extern "C" {
+
+int ssc_conv_fwd_f32(const float *features, int64_t n_in, int32_t c_in, const float *filters,
+                     int64_t fs_k, int64_t fs_ci, int64_t fs_co, int32_t c_out,
+                     const int32_t *pairs, int64_t pair_stride, const int32_t *pair_num,
+                     int32_t kernel_volume, int32_t inverse, int32_t subm, float *out,
+                     int64_t n_out, void *workspace, size_t workspace_bytes,
+                     ssc_stream_t stream) {
+  return conv_fwd<float>(features, n_in, c_in, filters, fs_k, fs_ci, fs_co, c_out, pairs,
+                         pair_stride, pair_num, kernel_volume, inverse, subm, out, n_out, workspace,
+                         workspace_bytes, stream);
+}
+
+int ssc_conv_fwd_f16(const void *features, int64_t n_in, int32_t c_in, const void *filters,
+                     int64_t fs_k, int64_t fs_ci, int64_t fs_co, int32_t c_out,
+                     const int32_t *pairs, int64_t pair_stride, const int32_t *pair_num,
+                     int32_t kernel_volume, int32_t inverse, int32_t subm, void *out,
+                     int64_t n_out, void *workspace, size_t workspace_bytes,
+                     ssc_stream_t stream) {
+  return conv_fwd<_Float16>(static_cast<const _Float16 *>(features), n_in, c_in,
+                            static_cast<const _Float16 *>(filters), fs_k, fs_ci, fs_co, c_out,
+                            pairs, pair_stride, pair_num, kernel_volume, inverse, subm,
+                            static_cast<_Float16 *>(out), n_out, workspace, workspace_bytes, stream);
 }
 }

@@ -17,6 +17,8 @@
 // second kernel in ascending order: the result does not depend on timing, no atomics.
 #include "ssc_common.h"
 
+#include <type_traits>
+
 namespace ssc {
 
 typedef float float4v __attribute__((ext_vector_type(4)));
@@ -25,33 +27,57 @@ constexpr int kBwChunk = 64;    // pairs per LDS stage
 constexpr int kBwStride = 68;   // floats per channel row in LDS (64 pairs + 4)
 constexpr int kBwTile = 64;     // channels per tile side
 
-// One 16-byte piece (4 channels) of row `row`, zero outside the matrix.
-__device__ __forceinline__ float4v load_quad(const float *__restrict__ m, int64_t row, int ch,
+// Rows of float or half-precision elements; the products and sums are fp32 either way
+// (half rows are widened when they are staged in LDS).
+typedef int int2v __attribute__((ext_vector_type(2)));
+typedef _Float16 half4v __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ float4v widen4(const float4v &v) { return v; }
+__device__ __forceinline__ float4v widen4(const int2v &v) {
+  return __builtin_convertvector(__builtin_bit_cast(half4v, v), float4v);
+}
+__device__ __forceinline__ float4v load4(const float *p) {
+  return *reinterpret_cast<const float4v *>(p);
+}
+__device__ __forceinline__ float4v load4(const _Float16 *p) {
+  return widen4(*reinterpret_cast<const int2v *>(p));
+}
+// four channels at byte offset `off` of a buffer, as loaded
+__device__ __forceinline__ float4v buf_quad(__amdgpu_buffer_rsrc_t r, unsigned off, const float *) {
+  return __builtin_bit_cast(float4v, __builtin_amdgcn_raw_buffer_load_b128(r, (int)off, 0, 0));
+}
+__device__ __forceinline__ int2v buf_quad(__amdgpu_buffer_rsrc_t r, unsigned off,
+                                          const _Float16 *) {
+  return __builtin_bit_cast(int2v, __builtin_amdgcn_raw_buffer_load_b64(r, (int)off, 0, 0));
+}
+
+// Four channels of row `row`, zero outside the matrix.
+template <typename IO>
+__device__ __forceinline__ float4v load_quad(const IO *__restrict__ m, int64_t row, int ch,
                                              int width) {
   float4v v = {0.f, 0.f, 0.f, 0.f};
   if (row < 0) return v;
-  const float *p = m + row * width + ch;
+  const IO *p = m + row * width + ch;
   if ((width & 3) == 0) {
-    if (ch < width) v = *reinterpret_cast<const float4v *>(p);
+    if (ch < width) v = load4(p);
   } else {
-    if (ch + 0 < width) v.x = p[0];
-    if (ch + 1 < width) v.y = p[1];
-    if (ch + 2 < width) v.z = p[2];
-    if (ch + 3 < width) v.w = p[3];
+    if (ch + 0 < width) v.x = (float)p[0];
+    if (ch + 1 < width) v.y = (float)p[1];
+    if (ch + 2 < width) v.z = (float)p[2];
+    if (ch + 3 < width) v.w = (float)p[3];
   }
   return v;
 }
 
 // grid: x = range of pairs, y = offset k, z = tile (ci tile major).  256 threads, four
 // workgroups per CU (one wave of each per SIMD: 128 registers a wave).
-// BUF: rows are multiples of 16 bytes and both matrices are below 4 GiB, so the gathers
+// BUF: rows are multiples of four channels and both matrices are below 4 GiB, so the gathers
 // are range-checked buffer loads at 32-bit byte offsets (a row beyond the range's pairs
 // gets an offset outside the buffer and reads zeros): no 64-bit address arithmetic and
 // no branches around the loads.
-template <bool BUF>
+template <typename IO, bool BUF>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4)))
-    conv_bwd_filter_kernel(const float *__restrict__ feats, int cin, unsigned feat_bytes,
-                           const float *__restrict__ dout, int cout, unsigned dout_bytes,
+    conv_bwd_filter_kernel(const IO *__restrict__ feats, int cin, unsigned feat_bytes,
+                           const IO *__restrict__ dout, int cout, unsigned dout_bytes,
                            const int32_t *__restrict__ pairs, int64_t pair_stride,
                            const int32_t *__restrict__ pair_num, int plane_in, int n_split,
                            int n_co_tiles, float *__restrict__ partial) {
@@ -72,14 +98,18 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))
 
   // staging: 16 threads per gathered row (256 contiguous bytes), pairs (tid >> 4) + 16j
   const int sp = tid >> 4, sq = (tid & 15) * 4;
-  float4v rf[4], rd[4];
+  constexpr unsigned kEB = sizeof(IO);
+  // rows in flight: as loaded from a buffer, or widened already by the pointer path
+  typedef std::conditional_t<BUF, decltype(buf_quad(__amdgpu_buffer_rsrc_t(), 0u, (const IO *)nullptr)),
+                             float4v> Held;
+  Held rf[4], rd[4];
   const __amdgpu_buffer_rsrc_t rs_f =
       __builtin_amdgcn_make_buffer_rsrc((void *)feats, 0, (int)feat_bytes, 0x00020000);
   const __amdgpu_buffer_rsrc_t rs_d =
       __builtin_amdgcn_make_buffer_rsrc((void *)dout, 0, (int)dout_bytes, 0x00020000);
   // a quad of channels beyond the matrix width reads zeros as well
-  const unsigned col_f = ci0 + sq < cin ? (unsigned)(ci0 + sq) * 4u : 0xFFFFF000u;
-  const unsigned col_d = co0 + sq < cout ? (unsigned)(co0 + sq) * 4u : 0xFFFFF000u;
+  const unsigned col_f = ci0 + sq < cin ? (unsigned)(ci0 + sq) * kEB : 0xFFFFF000u;
+  const unsigned col_d = co0 + sq < cout ? (unsigned)(co0 + sq) * kEB : 0xFFFFF000u;
   // row numbers of the chunk after the one being fetched: the gathers never wait for
   // their own index loads
   int idx_i[4], idx_o[4];
@@ -95,14 +125,14 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int p = p0 + sp + 16 * j;
-      if (BUF) {
-        const unsigned ri = idx_i[j] >= 0 ? (unsigned)idx_i[j] * (unsigned)(cin * 4) : 0xFFFFF000u;
-        const unsigned ro = idx_o[j] >= 0 ? (unsigned)idx_o[j] * (unsigned)(cout * 4) : 0xFFFFF000u;
+      if constexpr (BUF) {
+        const unsigned ri = idx_i[j] >= 0 ? (unsigned)idx_i[j] * ((unsigned)cin * kEB) : 0xFFFFF000u;
+        const unsigned ro = idx_o[j] >= 0 ? (unsigned)idx_o[j] * ((unsigned)cout * kEB) : 0xFFFFF000u;
         // saturating: an offset that is already outside stays outside
         const unsigned of = ri > 0xFFFFF000u - col_f ? 0xFFFFF000u : ri + col_f;
         const unsigned od = ro > 0xFFFFF000u - col_d ? 0xFFFFF000u : ro + col_d;
-        rf[j] = __builtin_bit_cast(float4v, __builtin_amdgcn_raw_buffer_load_b128(rs_f, (int)of, 0, 0));
-        rd[j] = __builtin_bit_cast(float4v, __builtin_amdgcn_raw_buffer_load_b128(rs_d, (int)od, 0, 0));
+        rf[j] = buf_quad(rs_f, of, feats);
+        rd[j] = buf_quad(rs_d, od, dout);
       } else {
         (void)p;
         rf[j] = load_quad(feats, idx_i[j], ci0 + sq, cin);
@@ -114,8 +144,8 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))
   auto stage = [&]() {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      *reinterpret_cast<float4v *>(ft + (sp + 16 * j) * kBwStride + sq) = rf[j];
-      *reinterpret_cast<float4v *>(dt + (sp + 16 * j) * kBwStride + sq) = rd[j];
+      *reinterpret_cast<float4v *>(ft + (sp + 16 * j) * kBwStride + sq) = widen4(rf[j]);
+      *reinterpret_cast<float4v *>(dt + (sp + 16 * j) * kBwStride + sq) = widen4(rd[j]);
     }
   };
 
@@ -175,9 +205,10 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))
 }
 
 // out[e] = partial[0][e] + partial[1][e] + ... in that order; out may have any strides.
+template <typename IO>
 __global__ void __launch_bounds__(256)
     conv_bwd_reduce_kernel(const float *__restrict__ partial, int n_split, int K, int cin, int cout,
-                           float *__restrict__ out, int64_t os_k, int64_t os_ci, int64_t os_co) {
+                           IO *__restrict__ out, int64_t os_k, int64_t os_ci, int64_t os_co) {
   const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   const int64_t per = (int64_t)K * cin * cout;
   if (e >= per) return;
@@ -187,7 +218,7 @@ __global__ void __launch_bounds__(256)
   const int64_t r = e / cout;
   const int ci = (int)(r % cin);
   const int k = (int)(r / cin);
-  out[k * os_k + ci * os_ci + co * os_co] = v;
+  out[k * os_k + ci * os_ci + co * os_co] = (IO)v;
 }
 
 static int bwd_split(int K, int c_in, int c_out, int64_t pair_stride) {
@@ -214,12 +245,15 @@ size_t ssc_conv_bwd_filter_workspace_bytes(int32_t kernel_volume, int32_t c_in, 
   return align_up((size_t)s * kernel_volume * c_in * c_out * sizeof(float));
 }
 
-int ssc_conv_bwd_filter_f32(const float *features, int64_t n_in, int32_t c_in,
-                            const float *out_grad, int64_t n_out, int32_t c_out,
-                            const int32_t *pairs, int64_t pair_stride, const int32_t *pair_num,
-                            int32_t kernel_volume, int32_t inverse, float *filters_grad,
-                            int64_t gs_k, int64_t gs_ci, int64_t gs_co, void *workspace,
-                            size_t workspace_bytes, ssc_stream_t stream) {
+}  // extern "C"
+
+template <typename IO>
+static int conv_bwd_filter(const IO *features, int64_t n_in, int32_t c_in, const IO *out_grad,
+                           int64_t n_out, int32_t c_out, const int32_t *pairs,
+                           int64_t pair_stride, const int32_t *pair_num, int32_t kernel_volume,
+                           int32_t inverse, IO *filters_grad, int64_t gs_k, int64_t gs_ci,
+                           int64_t gs_co, void *workspace, size_t workspace_bytes,
+                           ssc_stream_t stream) {
   const int K = kernel_volume;
   SSC_CHECK(K >= 1 && K <= SSC_MAX_KERNEL_VOLUME, SSC_ERUNTIME, "kernel volume %d out of range", K);
   SSC_CHECK(c_in >= 1 && c_out >= 1, SSC_EINVAL, "channel counts must be positive");
@@ -233,7 +267,7 @@ int ssc_conv_bwd_filter_f32(const float *features, int64_t n_in, int32_t c_in,
               SSC_EWORKSPACE, "conv backward workspace too small");
     int rc = fill_f32(static_cast<float *>(workspace), per, 0.f, s);
     if (rc != SSC_OK) return rc;
-    hipLaunchKernelGGL(conv_bwd_reduce_kernel, dim3((unsigned)ceil_div(per, 256)), dim3(256), 0, s,
+    hipLaunchKernelGGL(conv_bwd_reduce_kernel<IO>, dim3((unsigned)ceil_div(per, 256)), dim3(256), 0, s,
                        static_cast<const float *>(workspace), 1, K, c_in, c_out, filters_grad, gs_k,
                        gs_ci, gs_co);
     SSC_LAUNCH_CHECK("conv_bwd_reduce");
@@ -251,22 +285,48 @@ int ssc_conv_bwd_filter_f32(const float *features, int64_t n_in, int32_t c_in,
   // features are gathered through the plane the forward pass gathered them through
   const int plane_in = inverse ? 1 : 0;
   const dim3 grid((unsigned)n_split, (unsigned)K, (unsigned)(n_ci_tiles * n_co_tiles));
-  const uint64_t feat_bytes = (uint64_t)n_in * c_in * 4, dout_bytes = (uint64_t)n_out * c_out * 4;
+  const uint64_t feat_bytes = (uint64_t)n_in * c_in * sizeof(IO);
+  const uint64_t dout_bytes = (uint64_t)n_out * c_out * sizeof(IO);
   // the largest byte offset must stay below the marker that stands for "outside"
   const bool buf = (c_in & 3) == 0 && (c_out & 3) == 0 && feat_bytes <= 0xFFFFF000u &&
                    dout_bytes <= 0xFFFFF000u;
   if (buf)
-    hipLaunchKernelGGL(conv_bwd_filter_kernel<true>, grid, dim3(256), 0, s, features, c_in,
+    hipLaunchKernelGGL((conv_bwd_filter_kernel<IO, true>), grid, dim3(256), 0, s, features, c_in,
                        (unsigned)feat_bytes, out_grad, c_out, (unsigned)dout_bytes, pairs,
                        pair_stride, pair_num, plane_in, n_split, n_co_tiles, partial);
   else
-    hipLaunchKernelGGL(conv_bwd_filter_kernel<false>, grid, dim3(256), 0, s, features, c_in, 0u,
+    hipLaunchKernelGGL((conv_bwd_filter_kernel<IO, false>), grid, dim3(256), 0, s, features, c_in, 0u,
                        out_grad, c_out, 0u, pairs, pair_stride, pair_num, plane_in, n_split,
                        n_co_tiles, partial);
   SSC_LAUNCH_CHECK("conv_bwd_filter");
-  hipLaunchKernelGGL(conv_bwd_reduce_kernel, dim3((unsigned)ceil_div(per, 256)), dim3(256), 0, s,
+  hipLaunchKernelGGL(conv_bwd_reduce_kernel<IO>, dim3((unsigned)ceil_div(per, 256)), dim3(256), 0, s,
                      partial, n_split, K, c_in, c_out, filters_grad, gs_k, gs_ci, gs_co);
   SSC_LAUNCH_CHECK("conv_bwd_reduce");
   return SSC_OK;
+}
+
+extern "C" {
+
+int ssc_conv_bwd_filter_f32(const float *features, int64_t n_in, int32_t c_in,
+                            const float *out_grad, int64_t n_out, int32_t c_out,
+                            const int32_t *pairs, int64_t pair_stride, const int32_t *pair_num,
+                            int32_t kernel_volume, int32_t inverse, float *filters_grad,
+                            int64_t gs_k, int64_t gs_ci, int64_t gs_co, void *workspace,
+                            size_t workspace_bytes, ssc_stream_t stream) {
+  return conv_bwd_filter<float>(features, n_in, c_in, out_grad, n_out, c_out, pairs, pair_stride,
+                                pair_num, kernel_volume, inverse, filters_grad, gs_k, gs_ci, gs_co,
+                                workspace, workspace_bytes, stream);
+}
+
+int ssc_conv_bwd_filter_f16(const void *features, int64_t n_in, int32_t c_in,
+                            const void *out_grad, int64_t n_out, int32_t c_out,
+                            const int32_t *pairs, int64_t pair_stride, const int32_t *pair_num,
+                            int32_t kernel_volume, int32_t inverse, void *filters_grad,
+                            int64_t gs_k, int64_t gs_ci, int64_t gs_co, void *workspace,
+                            size_t workspace_bytes, ssc_stream_t stream) {
+  return conv_bwd_filter<_Float16>(
+      static_cast<const _Float16 *>(features), n_in, c_in, static_cast<const _Float16 *>(out_grad),
+      n_out, c_out, pairs, pair_stride, pair_num, kernel_volume, inverse,
+      static_cast<_Float16 *>(filters_grad), gs_k, gs_ci, gs_co, workspace, workspace_bytes, stream);
 }
 }

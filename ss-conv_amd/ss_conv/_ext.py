@@ -45,7 +45,11 @@ _SIGNATURES = {
     "ssc_conv_workspace_bytes": (_sz, [_i64, _i32, _i32, _i32, _i64]),
     "ssc_conv_fwd_f32": (ctypes.c_int, [_vp, _i64, _i32, _vp, _i64, _i64, _i64, _i32, _vp, _i64,
                                         _vp, _i32, _i32, _i32, _vp, _i64, _vp, _sz, _vp]),
+    "ssc_conv_fwd_f16": (ctypes.c_int, [_vp, _i64, _i32, _vp, _i64, _i64, _i64, _i32, _vp, _i64,
+                                        _vp, _i32, _i32, _i32, _vp, _i64, _vp, _sz, _vp]),
     "ssc_conv_bwd_filter_workspace_bytes": (_sz, [_i32, _i32, _i32, _i64]),
+    "ssc_conv_bwd_filter_f16": (ctypes.c_int, [_vp, _i64, _i32, _vp, _i64, _i32, _vp, _i64, _vp,
+                                               _i32, _i32, _vp, _i64, _i64, _i64, _vp, _sz, _vp]),
     "ssc_conv_bwd_filter_f32": (ctypes.c_int, [_vp, _i64, _i32, _vp, _i64, _i32, _vp, _i64, _vp,
                                                _i32, _i32, _vp, _i64, _i64, _i64, _vp, _sz, _vp]),
     "ssc_pool_max_bwd_f32": (ctypes.c_int, [_vp, _vp, _vp, _i32, _vp, _i64, _vp, _i32, _vp, _i64,
@@ -216,11 +220,11 @@ def _conv_flags(indice_pairs, subm, inverse):
     return int(bool(subm)) | (2 if canonical else 0)
 
 
-def indice_conv_fp32(features, filters, indice_pairs, indice_num, num_act_out, inverse, subm):
-    """src/conv/indice_conv.h:247-343 (bound at src/ss_conv_ops_api.cpp:21)."""
+def _indice_conv(dtype, entry, name, features, filters, indice_pairs, indice_num, num_act_out,
+                 inverse, subm):
     _need_gpu(features, filters, indice_pairs)
-    if features.dtype != torch.float32 or filters.dtype != torch.float32:
-        raise RuntimeError("indice_conv_fp32 needs float32 features and filters")
+    if features.dtype != dtype or filters.dtype != dtype:
+        raise RuntimeError("%s needs %s features and filters" % (name, dtype))
     features = features.contiguous()
     c_in = features.size(1)
     c_out = filters.size(-1)
@@ -235,23 +239,34 @@ def indice_conv_fp32(features, filters, indice_pairs, indice_num, num_act_out, i
     if kvol != K:
         raise RuntimeError("filters have %d offsets but the rulebook has %d" % (kvol, K))
     n_out = int(num_act_out)
-    out = torch.empty((n_out, c_out), dtype=torch.float32, device=features.device)
+    out = torch.empty((n_out, c_out), dtype=dtype, device=features.device)
     nbytes = _lib.ssc_conv_workspace_bytes(n_out, K, c_in, c_out, pairs.size(2))
     ws = _workspace(nbytes, features.device)
-    _check(_lib.ssc_conv_fwd_f32(_ptr(features), features.size(0), c_in, _ptr(filters), fs_k,
-                                 fs_ci, fs_co, c_out, _ptr(pairs), pairs.size(2), num.data_ptr(),
-                                 K, int(inverse), _conv_flags(indice_pairs, subm, inverse), _ptr(out), n_out,
-                                 ws.data_ptr(), ws.numel(), _stream(features)))
+    _check(entry(_ptr(features), features.size(0), c_in, _ptr(filters), fs_k, fs_ci, fs_co, c_out,
+                 _ptr(pairs), pairs.size(2), num.data_ptr(), K, int(inverse),
+                 _conv_flags(indice_pairs, subm, inverse), _ptr(out), n_out, ws.data_ptr(),
+                 ws.numel(), _stream(features)))
     return out
 
 
-def indice_conv_backward_fp32(features, filters, out_bp, indice_pairs, indice_num, inverse, subm):
-    """src/conv/indice_conv.h:344-426 (bound at src/ss_conv_ops_api.cpp:22): returns
-    [input_bp like features, filters_bp shaped like filters]."""
+def indice_conv_fp32(features, filters, indice_pairs, indice_num, num_act_out, inverse, subm):
+    """src/conv/indice_conv.h:247-343 (bound at src/ss_conv_ops_api.cpp:21)."""
+    return _indice_conv(torch.float32, _lib.ssc_conv_fwd_f32, "indice_conv_fp32", features,
+                        filters, indice_pairs, indice_num, num_act_out, inverse, subm)
+
+
+def indice_conv_half(features, filters, indice_pairs, indice_num, num_act_out, inverse, subm):
+    """indiceConv<at::Half> (src/ss_conv_ops.cu:74-78, bound at src/ss_conv_ops_api.cpp:23):
+    half-precision tensors, fp32 arithmetic, one rounding per output element."""
+    return _indice_conv(torch.float16, _lib.ssc_conv_fwd_f16, "indice_conv_half", features,
+                        filters, indice_pairs, indice_num, num_act_out, inverse, subm)
+
+
+def _indice_conv_backward(dtype, fwd_entry, filter_entry, name, features, filters, out_bp,
+                          indice_pairs, indice_num, inverse, subm):
     _need_gpu(features, filters, out_bp, indice_pairs)
-    if features.dtype != torch.float32 or filters.dtype != torch.float32 or \
-            out_bp.dtype != torch.float32:
-        raise RuntimeError("indice_conv_backward_fp32 needs float32 tensors")
+    if features.dtype != dtype or filters.dtype != dtype or out_bp.dtype != dtype:
+        raise RuntimeError("%s needs %s tensors" % (name, dtype))
     features = features.contiguous()
     out_bp = out_bp.contiguous()
     n_in, c_in = features.shape
@@ -264,21 +279,35 @@ def indice_conv_backward_fp32(features, filters, out_bp, indice_pairs, indice_nu
     dev = features.device
     s = _stream(features)
     # input gradient: the forward kernel on out_bp, pairs swapped, filters transposed
-    input_bp = torch.empty((n_in, c_in), dtype=torch.float32, device=dev)
+    input_bp = torch.empty((n_in, c_in), dtype=dtype, device=dev)
     ws = _workspace(_lib.ssc_conv_workspace_bytes(n_in, K, c_out, c_in, pairs.size(2)), dev)
-    _check(_lib.ssc_conv_fwd_f32(_ptr(out_bp), n_out, c_out, _ptr(filters), fs_k, fs_co, fs_ci,
-                                 c_in, _ptr(pairs), pairs.size(2), num.data_ptr(), K,
-                                 0 if inverse else 1, _conv_flags(indice_pairs, subm, not inverse),
-                                 _ptr(input_bp), n_in,
-                                 ws.data_ptr(), ws.numel(), s))
+    _check(fwd_entry(_ptr(out_bp), n_out, c_out, _ptr(filters), fs_k, fs_co, fs_ci, c_in,
+                     _ptr(pairs), pairs.size(2), num.data_ptr(), K, 0 if inverse else 1,
+                     _conv_flags(indice_pairs, subm, not inverse), _ptr(input_bp), n_in,
+                     ws.data_ptr(), ws.numel(), s))
     # filter gradient
-    filters_bp = torch.empty(tuple(filters.shape), dtype=torch.float32, device=dev)
+    filters_bp = torch.empty(tuple(filters.shape), dtype=dtype, device=dev)
     ws2 = _workspace(_lib.ssc_conv_bwd_filter_workspace_bytes(K, c_in, c_out, pairs.size(2)), dev)
-    _check(_lib.ssc_conv_bwd_filter_f32(_ptr(features), n_in, c_in, _ptr(out_bp), n_out, c_out,
-                                        _ptr(pairs), pairs.size(2), num.data_ptr(), K,
-                                        int(inverse), _ptr(filters_bp), c_in * c_out, c_out, 1,
-                                        ws2.data_ptr(), ws2.numel(), s))
+    _check(filter_entry(_ptr(features), n_in, c_in, _ptr(out_bp), n_out, c_out, _ptr(pairs),
+                        pairs.size(2), num.data_ptr(), K, int(inverse), _ptr(filters_bp),
+                        c_in * c_out, c_out, 1, ws2.data_ptr(), ws2.numel(), s))
     return [input_bp, filters_bp]
+
+
+def indice_conv_backward_fp32(features, filters, out_bp, indice_pairs, indice_num, inverse, subm):
+    """src/conv/indice_conv.h:344-426 (bound at src/ss_conv_ops_api.cpp:22): returns
+    [input_bp like features, filters_bp shaped like filters]."""
+    return _indice_conv_backward(torch.float32, _lib.ssc_conv_fwd_f32,
+                                 _lib.ssc_conv_bwd_filter_f32, "indice_conv_backward_fp32",
+                                 features, filters, out_bp, indice_pairs, indice_num, inverse, subm)
+
+
+def indice_conv_backward_half(features, filters, out_bp, indice_pairs, indice_num, inverse, subm):
+    """indiceConvBackward<at::Half> (src/ss_conv_ops.cu:79-83, bound at
+    src/ss_conv_ops_api.cpp:24): half-precision tensors, fp32 arithmetic."""
+    return _indice_conv_backward(torch.float16, _lib.ssc_conv_fwd_f16,
+                                 _lib.ssc_conv_bwd_filter_f16, "indice_conv_backward_half",
+                                 features, filters, out_bp, indice_pairs, indice_num, inverse, subm)
 
 
 def _pool_args(features, indice_pairs, indice_num):

@@ -67,7 +67,10 @@ def indice_conv_forward(features, filters, indice_pairs, indice_pair_num, num_ac
     if filters.dtype == torch.float32:
         return _ext.indice_conv_fp32(features, filters, indice_pairs, indice_pair_num,
                                      num_activate_out, int(inverse), int(subm))
-    raise NotImplementedError("only float32 convolution is built")
+    if filters.dtype == torch.half:
+        return _ext.indice_conv_half(features, filters, indice_pairs, indice_pair_num,
+                                     num_activate_out, int(inverse), int(subm))
+    raise NotImplementedError("convolution is built for float32 and half filters")
 
 
 def indice_conv_backward(features, filters, out_bp, indice_pairs, indice_pair_num, inverse=False,
@@ -76,7 +79,10 @@ def indice_conv_backward(features, filters, out_bp, indice_pairs, indice_pair_nu
     if filters.dtype == torch.float32:
         return _ext.indice_conv_backward_fp32(features, filters, out_bp, indice_pairs,
                                               indice_pair_num, int(inverse), int(subm))
-    raise NotImplementedError("only float32 convolution is built")
+    if filters.dtype == torch.half:
+        return _ext.indice_conv_backward_half(features, filters, out_bp, indice_pairs,
+                                              indice_pair_num, int(inverse), int(subm))
+    raise NotImplementedError("convolution is built for float32 and half filters")
 
 
 def indice_maxpool_forward(features, indice_pairs, indice_pair_num, num_activate_out):
