@@ -11,6 +11,7 @@ kernel 3, stride 1, padding 1, fp32).
 Prints one JSON line; see --help for the other workloads.
 """
 import argparse
+import gc
 import json
 import os
 import sys
@@ -32,8 +33,8 @@ MEASURED_TRAFFIC_BYTES = {"cfg2": int((18694.4 * 2.0 + 300076.5) * 1024)}
 def parse_args():
     ap = argparse.ArgumentParser(description=__doc__)
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="cfg2", choices=["cfg1", "cfg2", "cfg3", "cfg5"])
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -123,6 +124,17 @@ def ops_table(torch, _ext, synth, dev, seed):
     rows.append("%-44s %8.3f ms %9.2f GFLOP %7.1f TFLOP/s %5.1f%% of fp32 MFMA peak"
                 % ("conv backward, cfg2 (input + filter gradient)", ms, 4.0 * P * cin * cout / 1e9,
                    4.0 * P * cin * cout / ms / 1e9, 4.0 * P * cin * cout / ms / 1e9 / 1.573))
+    # the same layer on half-precision tensors (fp32 arithmetic, half the row bytes)
+    fh, wh, goh = f.half(), w.half(), go.half()
+    n_out_rows = o_idx.shape[0]
+    ms32, _ = timed(lambda: _ext.indice_conv_fp32(f, w, pairs, num, n_out_rows, 0, 0), n=10)
+    ms16, _ = timed(lambda: _ext.indice_conv_half(fh, wh, pairs, num, n_out_rows, 0, 0), n=10)
+    msb16, _ = timed(lambda: _ext.indice_conv_backward_half(fh, wh, goh, pairs, num, 0, 0), n=10)
+    for name, t, fl in (("conv forward call, cfg2, float32", ms32, 2.0), ("conv forward call, cfg2, half", ms16, 2.0),
+                        ("conv backward, cfg2, half", msb16, 4.0)):
+        rows.append("%-44s %8.3f ms %9.2f GFLOP %7.1f TFLOP/s %5.1f%% of fp32 MFMA peak"
+                    % (name, t, fl * P * cin * cout / 1e9, fl * P * cin * cout / t / 1e9,
+                       fl * P * cin * cout / t / 1e9 / 1.573))
 
     # pools on the output of the stride-2 layer: 32 clouds at 32^3, 256 channels
     cfg = synth.CONFIGS["cfg3"]
@@ -317,12 +329,18 @@ def main():
         del src, dst
 
     _ext.profile_conv(True)
+    # The interpreter's cyclic garbage collector stays out of the timed region, as in
+    # timeit: a full collection of a process that has imported torch takes 30-40 ms, many
+    # times the region itself, and when it falls due depends on allocation counts only.
+    gc.collect()
+    gc.disable()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(args.steps):
         out = step()
     torch.cuda.synchronize()
     t1 = time.perf_counter()
+    gc.enable()
     conv_ms = _ext.profile_conv_read()
     _ext.profile_conv(False)
 
