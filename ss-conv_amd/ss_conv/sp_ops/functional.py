@@ -1,7 +1,7 @@
 """autograd entry points over the native kernels
 (reference: ss_conv/sp_ops/functional.py:22-453; same exported names).
 
-Forward and backward passes run the HIP kernels (float32 only)."""
+Forward and backward passes run the HIP kernels (float32; the convolution also on half)."""
 import torch
 from torch.autograd import Function
 
