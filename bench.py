@@ -27,7 +27,7 @@ FP32_MFMA_PEAK_TFLOPS = 157.3  # MI355X dense fp32 matrix peak
 # HBM bytes per launch of the convolution kernel, from rocprofv3 --pmc
 # FETCH_SIZE / WRITE_SIZE runs scaled by a copy kernel of known size
 # (summaries under profiles/); None until measured for a workload.
-MEASURED_TRAFFIC_BYTES = {"cfg2": int((18694.4 * 2.0 + 300076.5) * 1024)}
+MEASURED_TRAFFIC_BYTES = {"cfg2": int((18669.6 * 2.0 + 300076.5) * 1024)}
 
 
 def parse_args():
