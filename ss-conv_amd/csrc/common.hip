@@ -53,8 +53,21 @@ BitTable bit_table_carve(Carver &c, int64_t n_bits) {
   return t;
 }
 
+// bits[] = 0 and total[0..1] = 0 in one launch.
+__global__ void __launch_bounds__(256)
+    bit_clear_kernel(uint32_t *__restrict__ bits, int64_t n_words, int32_t *__restrict__ total) {
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < 2) total[i] = 0;
+  const int64_t step = (int64_t)gridDim.x * blockDim.x;
+  for (; i < n_words; i += step) bits[i] = 0u;
+}
+
 int bit_table_clear(const BitTable &t, hipStream_t s) {
-  return fill_i32(reinterpret_cast<int32_t *>(t.bits), t.n_words, 0, s);
+  const int64_t want = ceil_div(t.n_words > 0 ? t.n_words : 1, 256);
+  const int blocks = (int)(want < 8192 ? want : 8192);
+  hipLaunchKernelGGL(bit_clear_kernel, dim3(blocks), dim3(256), 0, s, t.bits, t.n_words, t.total);
+  SSC_LAUNCH_CHECK("bit_clear");
+  return SSC_OK;
 }
 
 // Block-wide exclusive scan of one int per thread (kScanThreads threads).
@@ -96,28 +109,18 @@ __global__ void __launch_bounds__(kScanThreads)
   if (threadIdx.x == 0) blocksum[blockIdx.x] = tot;
 }
 
-// Pass 2: one block turns blocksum[] into its exclusive prefix and writes the total.
-__global__ void __launch_bounds__(kScanThreads)
-    popc_blockscan_kernel(int32_t *__restrict__ blocksum, int64_t n_blocks,
-                          int32_t *__restrict__ total) {
-  __shared__ int lds[kScanThreads / 64 + 1];
-  int carry = 0;
-  for (int64_t base = 0; base < n_blocks; base += kScanThreads) {
-    int64_t i = base + threadIdx.x;
-    int v = i < n_blocks ? blocksum[i] : 0;
-    int tot;
-    int ex = block_exclusive_scan(v, lds, &tot);
-    if (i < n_blocks) blocksum[i] = carry + ex;
-    carry += tot;
-  }
-  if (threadIdx.x == 0) total[0] = carry;
-}
-
-// Pass 3: exclusive prefix per word.
+// Pass 2: exclusive prefix per word.  Every block first adds up the sums of the blocks
+// before it (at most 2^31 / 32 / kScanBlockWords = 32768 values), which saves the launch
+// of a scan over blocksum[]; the last block also writes the total.
 __global__ void __launch_bounds__(kScanThreads)
     popc_prefix_kernel(const uint32_t *__restrict__ bits, int64_t n_words,
-                       const int32_t *__restrict__ blocksum, int32_t *__restrict__ prefix) {
+                       const int32_t *__restrict__ blocksum, int32_t *__restrict__ prefix,
+                       int32_t *__restrict__ total) {
   __shared__ int lds[kScanThreads / 64 + 1];
+  int before = 0;
+  for (int64_t b = threadIdx.x; b < (int64_t)blockIdx.x; b += kScanThreads) before += blocksum[b];
+  int block_off;
+  block_exclusive_scan(before, lds, &block_off);
   int64_t base = (int64_t)blockIdx.x * kScanBlockWords + (int64_t)threadIdx.x * kScanItems;
   int c[kScanItems];
   int v = 0;
@@ -127,12 +130,13 @@ __global__ void __launch_bounds__(kScanThreads)
     v += c[i];
   }
   int tot;
-  int ex = block_exclusive_scan(v, lds, &tot) + blocksum[blockIdx.x];
+  int ex = block_exclusive_scan(v, lds, &tot) + block_off;
 #pragma unroll
   for (int i = 0; i < kScanItems; ++i) {
     if (base + i < n_words) prefix[base + i] = ex;
     ex += c[i];
   }
+  if (blockIdx.x == gridDim.x - 1 && threadIdx.x == 0) total[0] = block_off + tot;
 }
 
 int bit_table_scan(const BitTable &t, hipStream_t s) {
@@ -140,11 +144,8 @@ int bit_table_scan(const BitTable &t, hipStream_t s) {
   hipLaunchKernelGGL(popc_blocksum_kernel, dim3((unsigned)t.n_scan_blocks), dim3(kScanThreads), 0,
                      s, t.bits, t.n_words, t.blocksum);
   SSC_LAUNCH_CHECK("popc_blocksum");
-  hipLaunchKernelGGL(popc_blockscan_kernel, dim3(1), dim3(kScanThreads), 0, s, t.blocksum,
-                     t.n_scan_blocks, t.total);
-  SSC_LAUNCH_CHECK("popc_blockscan");
   hipLaunchKernelGGL(popc_prefix_kernel, dim3((unsigned)t.n_scan_blocks), dim3(kScanThreads), 0, s,
-                     t.bits, t.n_words, t.blocksum, t.prefix);
+                     t.bits, t.n_words, t.blocksum, t.prefix, t.total);
   SSC_LAUNCH_CHECK("popc_prefix");
   return SSC_OK;
 }

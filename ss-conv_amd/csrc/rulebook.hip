@@ -404,11 +404,9 @@ int ssc_rulebook_count_ordered(const int32_t *indices, int64_t n_in, const ssc_g
             rulebook_ws_bytes(gg, n_in));
   hipStream_t s = (hipStream_t)stream;
   RulebookWs w = rulebook_ws_carve(workspace, gg, n_in);
-  if ((rc = bit_table_clear(w.table, s)) != SSC_OK) return rc;
   // total[0]: the table's popcount (written by the scan); total[1]: the disorder flag,
-  // cleared here and set by the marking kernel.  This call ends with a host read, so it
-  // cannot be part of a captured graph anyway: a memset is fine.
-  SSC_HIP(hipMemsetAsync(w.table.total, 0, 2 * sizeof(int32_t), s));
+  // cleared with the table and set by the marking kernel.
+  if ((rc = bit_table_clear(w.table, s)) != SSC_OK) return rc;
   if (gg.subm) {
     hipLaunchKernelGGL(mark_rows_kernel, dim3((unsigned)ceil_div(n_in, 256)), dim3(256), 0, s,
                        indices, n_in, gg.os[0], gg.os[1], gg.os[2], w.table.bits,
