@@ -36,27 +36,42 @@ constexpr int kMinTile = 64;
 // that one wave reads it as four coalesced 16-byte loads per lane.  The four steps of
 // load q cover the 16 channels 16q .. 16q+15 of the chunk (lane group g has channels
 // 16q + 4g .. +3), so a layer with few input channels needs only its first loads.
+//
+// Half-precision filters are packed for v_mfma_f32_16x16x32_f16 instead, two steps of 32
+// channels per chunk (halves, 2 KiB per fragment):
+// packed[((k*NCB + ncb)*NCH + cc)*1024 + q*512 + lane*8 + j] =
+//     W[k][cc*64 + 32q + (lane/16)*8 + j][ncb*16 + lane%16]
+// i.e. one 16-byte load per lane and step.  Which of a step's 32 channels sits in which of
+// a lane's 8 slots does not matter for the sum as long as the staged rows use the same
+// assignment; they do (lane group g reads channels 32q + 8g .. +7 of its row).
 template <typename IO>
 __global__ void __launch_bounds__(256)
     pack_filters_kernel(const IO *__restrict__ w, int64_t fs_k, int64_t fs_ci, int64_t fs_co,
-                        int K, int cin, int cout, int ncb, int nch, float *__restrict__ packed,
+                        int K, int cin, int cout, int ncb, int nch, void *__restrict__ packed_out,
                         int32_t *__restrict__ flag) {
   int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (idx == 0) flag[0] = 0;  // the pair-order flag of the kernels that follow
   int64_t total = (int64_t)K * ncb * nch * 1024;
   if (idx >= total) return;
-  int c = idx & 15;
-  int lane = (idx >> 4) & 63;
   int64_t r = idx >> 10;
   int cc = r % nch;
   r /= nch;
   int cb = r % ncb;
   int k = (int)(r / ncb);
-  int ci = cc * kKC + (c >> 2) * 16 + (lane >> 4) * 4 + (c & 3);
+  int lane, ci;
+  if constexpr (sizeof(IO) == 2) {
+    const int j = idx & 7, q = (idx >> 9) & 1;
+    lane = (idx >> 3) & 63;
+    ci = cc * kKC + 32 * q + (lane >> 4) * 8 + j;
+  } else {
+    const int c = idx & 15;
+    lane = (idx >> 4) & 63;
+    ci = cc * kKC + (c >> 2) * 16 + (lane >> 4) * 4 + (c & 3);
+  }
   int co = cb * 16 + (lane & 15);
-  float v = 0.f;
-  if (ci < cin && co < cout) v = (float)w[k * fs_k + ci * fs_ci + co * fs_co];
-  packed[idx] = v;
+  IO v = (IO)0.f;
+  if (ci < cin && co < cout) v = w[k * fs_k + ci * fs_ci + co * fs_co];
+  static_cast<IO *>(packed_out)[idx] = v;
 }
 
 // ---- pair order -------------------------------------------------------------------------
@@ -572,20 +587,33 @@ __device__ __forceinline__ int buf_load1(__amdgpu_buffer_rsrc_t r, int voff, int
   return (int)__builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, 0);
 }
 
-// Element type of the features, the filters and the output.  The arithmetic is fp32
-// either way: half-precision rows are widened when the producers stage them and the
-// accumulators are rounded once, when a finished tile is written.
+// Element type of the features, the filters and the output.  float: fp32 rows in LDS,
+// v_mfma_f32_16x16x4_f32.  _Float16: half rows in LDS, v_mfma_f32_16x16x32_f16; the
+// accumulators are fp32 either way and are rounded once, when a finished tile is written.
 typedef int int2v __attribute__((ext_vector_type(2)));
 typedef _Float16 half4v __attribute__((ext_vector_type(4)));
+typedef _Float16 half8v __attribute__((ext_vector_type(8)));
 template <typename IO> struct Io;
 template <> struct Io<float> {
   static constexpr int kBytes = 4;
+  static constexpr int kRowBytes = kAStride * 4;  // a staged row of 64 channels in LDS
+  static constexpr int kFragBytes = 4096;         // packed filters of (offset, column block, chunk)
   typedef float4v Raw;  // four channels as they are loaded
+  static __device__ __forceinline__ Raw zero() { return Raw{0.f, 0.f, 0.f, 0.f}; }
   static __device__ __forceinline__ Raw gather(__amdgpu_buffer_rsrc_t r, int voff, int soff) {
     return buf_load4(r, voff, soff);
   }
   static __device__ __forceinline__ Raw load(const float *p) {
     return *reinterpret_cast<const float4v *>(p);
+  }
+  // the first n (possibly <= 0 or > 4) of four channels, zeros for the rest
+  static __device__ __forceinline__ Raw load_first(const float *p, int n) {
+    Raw v = zero();
+    if (n > 0) v.x = p[0];
+    if (n > 1) v.y = p[1];
+    if (n > 2) v.z = p[2];
+    if (n > 3) v.w = p[3];
+    return v;
   }
   static __device__ __forceinline__ void store_stream(float *p, const float4v &v) {
     __builtin_nontemporal_store(v, reinterpret_cast<float4v *>(p));
@@ -593,22 +621,29 @@ template <> struct Io<float> {
 };
 template <> struct Io<_Float16> {
   static constexpr int kBytes = 2;
+  static constexpr int kRowBytes = 144;  // 128 + 16: 16-byte aligned, bank spread as for float
+  static constexpr int kFragBytes = 2048;
   typedef int2v Raw;
+  static __device__ __forceinline__ Raw zero() { return Raw{0, 0}; }
   static __device__ __forceinline__ Raw gather(__amdgpu_buffer_rsrc_t r, int voff, int soff) {
     return __builtin_bit_cast(int2v, __builtin_amdgcn_raw_buffer_load_b64(r, voff, soff, 0));
   }
   static __device__ __forceinline__ Raw load(const _Float16 *p) {
     return *reinterpret_cast<const int2v *>(p);
   }
+  static __device__ __forceinline__ Raw load_first(const _Float16 *p, int n) {
+    half4v v = {(_Float16)0.f, (_Float16)0.f, (_Float16)0.f, (_Float16)0.f};
+    if (n > 0) v.x = p[0];
+    if (n > 1) v.y = p[1];
+    if (n > 2) v.z = p[2];
+    if (n > 3) v.w = p[3];
+    return __builtin_bit_cast(int2v, v);
+  }
   static __device__ __forceinline__ void store_stream(_Float16 *p, const float4v &v) {
     const half4v h = __builtin_convertvector(v, half4v);  // round to nearest even
     __builtin_nontemporal_store(__builtin_bit_cast(int2v, h), reinterpret_cast<int2v *>(p));
   }
 };
-__device__ __forceinline__ float4v widen(const float4v &v) { return v; }
-__device__ __forceinline__ float4v widen(const int2v &v) {
-  return __builtin_convertvector(__builtin_bit_cast(half4v, v), float4v);
-}
 
 // Position of a stage in the schedule: group index and channel chunk.  Advanced
 // with scalar arithmetic only.
@@ -641,13 +676,16 @@ template <typename IO, int GATHER, int NCW, int NQ>
 __global__ void __launch_bounds__((NCW + 4) * 64)
     __attribute__((amdgpu_waves_per_eu((NCW + 4) / 4, (NCW + 4) / 4)))
     conv_fwd_kernel(const IO *__restrict__ features, int cin, unsigned feat_bytes,
-                    const float *__restrict__ packed, unsigned packed_bytes,
+                    const void *__restrict__ packed, unsigned packed_bytes,
                     const int32_t *__restrict__ sched_in, const int32_t *__restrict__ sched_out,
                     const int32_t *__restrict__ grp_meta, unsigned sched_bytes, unsigned meta_bytes,
                     const int32_t *__restrict__ tile_grp, const int32_t *__restrict__ wg_tile,
                     int nch, int ncb, IO *__restrict__ out, int cout, int T) {
   constexpr int kCN = 16 * NCW;   // output columns per workgroup
   constexpr int kEB = Io<IO>::kBytes;
+  constexpr bool kHalf = kEB == 2;
+  constexpr int kRowB = Io<IO>::kRowBytes;    // bytes of a staged row
+  constexpr int kFragB = Io<IO>::kFragBytes;  // bytes of a packed filter fragment
   typedef typename Io<IO>::Raw Raw;
   constexpr int kAS = kCN + 4;    // accumulator row stride in floats
   constexpr int NT = (NCW + 4) * 64;
@@ -751,8 +789,7 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
     const int chunk_off = (pt & 15) * 4 * kEB;  // this thread's 4 channels of a 64-channel row chunk
     // this thread's 4 channels of the last chunk lie beyond Cin
     const bool beyond_cin = (nch - 1) * kKC + (pt & 15) * 4 >= cin;
-    // rows in flight stay as loaded (half precision: half the registers)
-    typedef std::conditional_t<GATHER == 0, float4v, Raw> Held;
+    typedef Raw Held;
     int idx[ID][NE];
     Held rows[RD][NE];
     // Rings indexed by stage number: rows of stage st in rows[st & 3], gather offsets
@@ -780,25 +817,22 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
           const int ch = pos.cc * kKC + (pt & 15) * 4;
           const int row = ix[j] < 0 ? 0 : ix[j];  // padding slots read row 0 and drop it
           const IO *fp = features + (int64_t)row * cin + ch;
-          float4v v = float4v{0.f, 0.f, 0.f, 0.f};
+          Held v = Io<IO>::zero();
           if ((cin & 3) == 0) {
-            if (ch < cin) v = widen(Io<IO>::load(fp));
-          } else {
-            if (ch + 0 < cin) v.x = (float)fp[0];
-            if (ch + 1 < cin) v.y = (float)fp[1];
-            if (ch + 2 < cin) v.z = (float)fp[2];
-            if (ch + 3 < cin) v.w = (float)fp[3];
+            if (ch < cin) v = Io<IO>::load(fp);
+          } else {  // rows are not aligned: one element at a time
+            v = Io<IO>::load_first(fp, cin - ch);
           }
-          if (ix[j] < 0) v = float4v{0.f, 0.f, 0.f, 0.f};
+          if (ix[j] < 0) v = Io<IO>::zero();
           r[j] = v;
         }
       }
     };
-    float *const st_base = abuf + (pt >> 4) * kAStride + (pt & 15) * 4;
+    char *const st_base = reinterpret_cast<char *>(abuf) + (pt >> 4) * kRowB + (pt & 15) * 4 * kEB;
     auto store_rows = [&](int parity, const Held (&r)[NE]) {
 #pragma unroll
       for (int j = 0; j < NE; ++j)
-        *reinterpret_cast<float4v *>(st_base + (parity * kStage + j * 16) * kAStride) = widen(r[j]);
+        *reinterpret_cast<Held *>(st_base + (parity * kStage + j * 16) * kRowB) = r[j];
     };
     // Prologue.  Loads are issued in the order the loop will wait for them (offsets,
     // then rows, oldest stage first): the wait counts of the loop are static, so
@@ -872,9 +906,15 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
         __builtin_amdgcn_make_buffer_rsrc((void *)packed, 0, (int)packed_bytes, kRsrcFlags);
     const __amdgpu_buffer_rsrc_t rs_out =
         __builtin_amdgcn_make_buffer_rsrc((void *)sched_out, 0, (int)sched_bytes, kRsrcFlags);
-    const int w_voff = lane * 64;           // this lane's 16 floats of a fragment
-    const int w_soff0 = cb * nch * 4096;    // fragments of this wave's column block
-    const float *const a_base = abuf + l16 * kAStride + g * 4;
+    // 16-byte pieces of operands a lane handles per row block: weight fragment loads, and
+    // as many reads of its staged row (float: 4 MFMA steps of 4 channels each, a quarter
+    // of the chunk; half: one MFMA step of 32 channels, lane group g has 8 of them)
+    constexpr int NF = kHalf ? 2 : NQ;
+    typedef std::conditional_t<kHalf, int4v, float4v> Frag;
+    const int w_voff = kHalf ? lane * 16 : lane * 64;  // this lane's part of a fragment
+    constexpr int kWStep = kHalf ? 1024 : 16;          // from one 16-byte piece to the next
+    const int w_soff0 = cb * nch * kFragB;  // fragments of this wave's column block
+    const char *const a_base = reinterpret_cast<const char *>(abuf) + l16 * kRowB + g * 16;
     // The accumulators are addressed with 32-bit LDS byte addresses (acc_lane includes
     // the base of acc): no pointer arithmetic left for the vector ALU.
     typedef __attribute__((address_space(3))) float4v lds_float4v;
@@ -897,7 +937,7 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
     //                 loads and v_readfirstlane rather than scalar loads: scalar loads
     //                 return out of order, and one in flight would turn every partial
     //                 wait for LDS data below into a wait for everything.
-    float4v w[4][4];
+    Frag w[4][NF];
     int orow[4];
     int4v rec[2][2];
     // Second half of a record: only its first three words are used.  A 12-byte load:
@@ -936,7 +976,7 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
       return b == 0 ? v.x : b == 1 ? v.y : b == 2 ? v.z : v.w;
     };
     auto fetch_w = [&](int soff, int slot, int q) {
-      w[slot][q] = buf_load4(rs_w, w_voff + q * 16, soff);
+      w[slot][q] = __builtin_bit_cast(Frag, buf_load4(rs_w, w_voff + q * kWStep, soff));
     };
     auto fetch_orow = [&](const StagePos &pos, int m, int slot) {
       orow[slot] = buf_load1(rs_out, l16 * 4 + m * 64, pos.g * 256);
@@ -978,24 +1018,29 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
     auto run_stage = [&](auto parity, bool last_cur, const StagePos &cur, const StagePos &next,
                          const StagePos &after, TileEnd &end_next) {
       constexpr int par = decltype(parity)::value;
-      const float *ab = a_base + par * kStage * kAStride;
-      const int base_cur = w_soff0 + cur.cc * 4096;
-      const int base_next = w_soff0 + next.cc * 4096;
-      float4v a[2][4];
-      auto load_a = [&](int m, int q, float4v (&av)[4]) {
-        av[q] = *reinterpret_cast<const float4v *>(ab + m * 16 * kAStride + q * 16);
+      const char *ab = a_base + par * kStage * kRowB;
+      const int base_cur = w_soff0 + cur.cc * kFragB;
+      const int base_next = w_soff0 + next.cc * kFragB;
+      Frag a[2][NF];
+      auto load_a = [&](int m, int q, Frag (&av)[NF]) {
+        av[q] = *reinterpret_cast<const Frag *>(ab + m * 16 * kRowB + q * 64);
       };
 #pragma unroll
-      for (int q = 0; q < NQ; ++q) load_a(0, q, a[0]);
+      for (int q = 0; q < NF; ++q) load_a(0, q, a[0]);
       // gaps of the pieces of a block (see above); with fewer than 16 MFMAs they move
       // closer together, in the same order
-      constexpr int kSteps = 4 * NQ;
-      constexpr int kGapAlu = NQ == 4 ? 2 : 1, kGapAcc = kGapAlu + 1;
-      constexpr int kGapW[4] = {NQ == 4 ? 4 : 2, NQ == 4 ? 7 : 3, NQ == 4 ? 9 : 4, 12};
-      constexpr int kGapRow = NQ == 4 ? 5 : 2;  // after fragment load 0 in the same gap
-      constexpr int kGapA[4] = {NQ == 4 ? 6 : kSteps / 2, NQ == 4 ? 8 : kSteps / 2 + 1,
-                                NQ == 4 ? 10 : kSteps / 2 + 2, 11};
-      constexpr int kGapRec0 = NQ == 4 ? 13 : kSteps - 2, kGapRec1 = NQ == 4 ? 14 : kSteps - 1;
+      // half: two MFMAs a block, so the pieces sit behind the first or the second
+      constexpr int kSteps = kHalf ? 2 : 4 * NQ;
+      constexpr bool kFull = !kHalf && NQ == 4;
+      constexpr int kGapAlu = kHalf ? 0 : kFull ? 2 : 1, kGapAcc = kHalf ? 0 : kGapAlu + 1;
+      constexpr int kGapW[4] = {kHalf ? 0 : kFull ? 4 : 2, kHalf ? 1 : kFull ? 7 : 3, kFull ? 9 : 4,
+                                12};
+      constexpr int kGapRow = kHalf ? 0 : kFull ? 5 : 2;  // after fragment load 0 in the same gap
+      constexpr int kGapA[4] = {kHalf ? 1 : kFull ? 6 : kSteps / 2,
+                                kHalf ? 1 : kFull ? 8 : kSteps / 2 + 1,
+                                kFull ? 10 : kSteps / 2 + 2, 11};
+      constexpr int kGapRec0 = kHalf ? 1 : kFull ? 13 : kSteps - 2;
+      constexpr int kGapRec1 = kHalf ? 1 : kFull ? 14 : kSteps - 1;
 #pragma unroll
       for (int m = 0; m < 4; ++m) {
         const int slot = m;                 // == (4 * s + m) & 3
@@ -1006,9 +1051,15 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
         int soff = 0;
 #pragma unroll
         for (int i = 0; i < kSteps; ++i) {
-          const int q = i >> 2, j = i & 3;
           __builtin_amdgcn_sched_barrier(0);
-          d = __builtin_amdgcn_mfma_f32_16x16x4f32(w[slot][q][j], a[m & 1][q][j], d, 0, 0, 0);
+          if constexpr (kHalf) {
+            d = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8v, w[slot][i]),
+                                                       __builtin_bit_cast(half8v, a[m & 1][i]), d,
+                                                       0, 0, 0);
+          } else {
+            const int q = i >> 2, j = i & 3;
+            d = __builtin_amdgcn_mfma_f32_16x16x4f32(w[slot][q][j], a[m & 1][q][j], d, 0, 0, 0);
+          }
           __builtin_amdgcn_sched_barrier(0);
           // all vector-ALU work of the block in one gap: a vector-ALU instruction
           // next to the matrix chain costs about ten cycles for leaving and re-entering
@@ -1025,11 +1076,11 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
           if (i == kGapW[0]) fetch_w(soff, tslot, 0);
           if (i == kGapRow) fetch_orow(tnext ? next : cur, tm, tslot);
 #pragma unroll
-          for (int qq = 1; qq < NQ; ++qq)
+          for (int qq = 1; qq < NF; ++qq)
             if (i == kGapW[qq]) fetch_w(soff, tslot, qq);
           if (m < 3) {
 #pragma unroll
-            for (int qq = 0; qq < NQ; ++qq)
+            for (int qq = 0; qq < NF; ++qq)
               if (i == kGapA[qq]) load_a(m + 1, qq, a[(m + 1) & 1]);
           }
           // this stage's record was last used by block 0: refill it for the stage
@@ -1066,14 +1117,14 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
       // prologue issued late would make every trip wait for nearly all loads in flight.
 #pragma unroll
       for (int b = 0; b < 3; ++b) {
-        const int soff = frag_soff(rec_k(rec[0][0], b), w_soff0 + p_cur.cc * 4096);
+        const int soff = frag_soff(rec_k(rec[0][0], b), w_soff0 + p_cur.cc * kFragB);
         __builtin_amdgcn_sched_barrier(0);
         fetch_w(soff, b, 0);
         __builtin_amdgcn_sched_barrier(0);
         fetch_orow(p_cur, b, b);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int q = 1; q < NQ; ++q) {
+        for (int q = 1; q < NF; ++q) {
           fetch_w(soff, b, q);
           __builtin_amdgcn_sched_barrier(0);
         }
@@ -1225,7 +1276,7 @@ static int launch_conv(const ConvPlan &p, const ConvWs &w, const IO *features, i
                                 hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
     attr_set = true;
   }
-  const uint64_t packed_bytes = (uint64_t)K * p.ncb * p.nch * 4096;
+  const uint64_t packed_bytes = (uint64_t)K * p.ncb * p.nch * Io<IO>::kFragBytes;
   const uint64_t sched_bytes = (uint64_t)p.grp_cap * 256;
   SSC_CHECK(packed_bytes < ((uint64_t)1 << 32) && sched_bytes < ((uint64_t)1 << 32), SSC_ERUNTIME,
             "convolution too large for 32-bit buffer offsets (filters %llu B, schedule %llu B)",
@@ -1380,7 +1431,8 @@ static int conv_fwd(const IO *features, int64_t n_in, int32_t c_in, const IO *fi
                      w.n_tiles_dev, w.tile_row0, w.tile_slot0, p.T,
                      p.gather ? (uint32_t)c_in * (uint32_t)sizeof(IO) : 1u,
                      p.gather ? kGatherPad : 0xFFFFFFFFu,
-                     (16 * p.ncw + 4) * 4, p.ncb * p.nch * 4096, w.sched_in, w.sched_out,
+                     (16 * p.ncw + 4) * 4, p.ncb * p.nch * Io<IO>::kFragBytes, w.sched_in,
+                     w.sched_out,
                      w.grp_meta);
   SSC_LAUNCH_CHECK("schedule");
 

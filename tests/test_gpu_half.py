@@ -2,14 +2,17 @@
 ssc_conv_bwd_filter_f16; reference: indice_conv_half / indice_conv_backward_half,
 src/ss_conv_ops.cu:74-83).
 
-The library computes in fp32 and rounds every result element to half once.  Two bars:
+The library multiplies half values exactly, accumulates in fp32 (forward and input
+gradient on v_mfma_f32_16x16x32_f16, filter gradient on fp32 MFMA over widened rows) and
+rounds every result element to half once.  Two bars:
   * against the oracle: the sums of the half-valued inputs taken in float64 are exact to
     well below half precision, so every result element must lie within half a unit in the
     last place of half of them (plus the fp32 accumulation error, which the fp32 tests
     bound at rel-L2 1e-5);
-  * against the fp32 entry points on the widened inputs: the same kernels do the same
-    operations in the same order, so rounding the fp32 result must give the same bits, at
-    any size.
+  * against the fp32 entry points on the widened inputs, at any size: the filter gradient
+    runs the same operations in the same order, so rounding the fp32 result must give the
+    same bits; forward and input gradient add the same exact products in another order, so
+    they may differ from the rounded fp32 result by one unit in the last place at most.
 """
 import numpy as np
 import pytest
@@ -32,6 +35,15 @@ def within_half_rounding(got, exact):
     bound = HALF_EPS * np.abs(exact) + HALF_TINY + ACC_SLACK * rms
     bad = np.abs(got - exact) > bound
     return not bad.any(), int(bad.sum())
+
+
+def within_one_ulp(got_half, want_fp32):
+    """got_half (torch half) against the fp32 result it should be a rounding of."""
+    got = got_half.detach().double()
+    want = want_fp32.detach().double()
+    rms = float(want.pow(2).mean().sqrt()) if want.numel() else 0.0
+    bound = 2.0 ** -10 * want.abs() + 2.0 ** -24 + ACC_SLACK * rms
+    return bool(((got - want).abs() <= bound).all())
 
 
 def conv_sums(feats, w, pairs, num, n_out):
@@ -91,7 +103,7 @@ def test_conv_half_matches_oracle(case, oracle, device):
     ok, n_bad = within_half_rounding(out.cpu().numpy(), ref)
     assert ok, n_bad
     out32 = _ext.indice_conv_fp32(f_h.float(), w_h.float(), g_pairs, g_num, g_idx.shape[0], 0, 0)
-    assert torch.equal(out, out32.half())
+    assert within_one_ulp(out, out32)
 
 
 def test_conv_half_inverse_unsorted_and_strided_filters(oracle, device):
@@ -171,12 +183,13 @@ def test_conv_backward_half_matches_oracle(case, oracle, device):
     assert ok, ("filter gradient", n_bad)
     e_in, e_w = _ext.indice_conv_backward_fp32(f_h.float(), w_h.float(), go_h.float(), g_pairs,
                                                g_num, 0, 0)
-    assert torch.equal(d_in, e_in.half()) and torch.equal(d_w, e_w.half())
+    assert within_one_ulp(d_in, e_in) and torch.equal(d_w, e_w.half())
 
 
 def test_conv_half_benchmark_size_equals_rounded_fp32(device):
     """The second benchmark configuration (32 clouds, 64^3, 64 -> 128 channels): the half
-    entry points give the rounded results of the fp32 entry points, bit for bit."""
+    entry points give the rounded results of the fp32 entry points (the filter gradient bit
+    for bit, the others to one unit in the last place)."""
     from ss_conv import _ext
     from ss_conv.sp_ops.ops import get_indice_pairs
     cfg = synth.CONFIGS["cfg2"]
@@ -195,12 +208,12 @@ def test_conv_half_benchmark_size_equals_rounded_fp32(device):
     n_out = out_idx.shape[0]
     out = _ext.indice_conv_half(f_h, w_h, pairs, num, n_out, 0, 0)
     out32 = _ext.indice_conv_fp32(f_h.float(), w_h.float(), pairs, num, n_out, 0, 0)
-    assert torch.equal(out, out32.half())
+    assert within_one_ulp(out, out32)
     go_h = torch.randn((n_out, cout), device=device, generator=gen).half()
     d_in, d_w = _ext.indice_conv_backward_half(f_h, w_h, go_h, pairs, num, 0, 0)
     e_in, e_w = _ext.indice_conv_backward_fp32(f_h.float(), w_h.float(), go_h.float(), pairs, num,
                                                0, 0)
-    assert torch.equal(d_in, e_in.half()) and torch.equal(d_w, e_w.half())
+    assert within_one_ulp(d_in, e_in) and torch.equal(d_w, e_w.half())
 
 
 def test_conv_half_empty_and_dtype_errors(device):
@@ -220,7 +233,7 @@ def test_conv_half_empty_and_dtype_errors(device):
 def test_convolution_layer_on_half_features(device):
     """Convolution on a half-precision SparseTensor: the kernel is synthesised in fp32 and
     rounded to the features' type; forward and gradients equal the fp32 layer's on the
-    widened values, rounded."""
+    widened values to one unit in the last place of half."""
     from ss_conv.convolution import Convolution
     from ss_conv.sp_ops.tensor import SparseTensor
     torch.manual_seed(4)
@@ -239,9 +252,9 @@ def test_convolution_layer_on_half_features(device):
     from ss_conv.sp_ops.ops import get_indice_pairs
     out_idx, pairs, num = get_indice_pairs(idx, 2, [grid] * 3, 3, 1, 1, 1, 0, False)
     y32 = Fsp.indice_conv(x32, w_h.float(), pairs, num, out_idx.shape[0])
-    assert torch.equal(y, y32.half())
+    assert within_one_ulp(y, y32)
     g = torch.randn_like(y32).half()
     y.backward(g)
     y32.backward(g.float())
-    assert torch.equal(x_h.grad, x32.grad.half())
+    assert within_one_ulp(x_h.grad, x32.grad)
     assert conv.kernel.weight.grad is not None and torch.isfinite(conv.kernel.weight.grad).all()
