@@ -30,12 +30,14 @@ constexpr int kAStride = 68;  // floats per staged row (64 + 4: 16-byte aligned,
 constexpr int kMinTile = 64;
 
 // ---- weight packing ---------------------------------------------------------------------
-// packed[((k*NCB + ncb)*NCH + cc)*1024 + lane*16 + c] =
-//     W[k][cc*64 + (c/4)*16 + (lane/16)*4 + c%4][ncb*16 + lane%16]   (0 outside Cin/Cout)
-// i.e. the weight fragment of MFMA step c of chunk cc for column block ncb, laid out so
-// that one wave reads it as four coalesced 16-byte loads per lane.  The four steps of
-// load q cover the 16 channels 16q .. 16q+15 of the chunk (lane group g has channels
-// 16q + 4g .. +3), so a layer with few input channels needs only its first loads.
+// packed[((k*NCB + ncb)*NCH + cc)*1024 + q*256 + lane*4 + j] =
+//     W[k][cc*64 + 16q + (lane/16)*4 + j][ncb*16 + lane%16]   (0 outside Cin/Cout)
+// i.e. the weight fragments of MFMA steps 4q + j of chunk cc for column block ncb, laid
+// out so that a wave reads them as four 16-byte loads per lane, each load one contiguous
+// KiB (lane l at byte 16 l): 8 cache lines an instruction, where a lane-major layout
+// (64 bytes per lane) touches 32.  The four steps of load q cover the 16 channels
+// 16q .. 16q+15 of the chunk (lane group g has channels 16q + 4g .. +3), so a layer with
+// few input channels needs only its first loads.
 //
 // Half-precision filters are packed for v_mfma_f32_16x16x32_f16 instead, two steps of 32
 // channels per chunk (halves, 2 KiB per fragment):
@@ -64,9 +66,9 @@ __global__ void __launch_bounds__(256)
     lane = (idx >> 3) & 63;
     ci = cc * kKC + 32 * q + (lane >> 4) * 8 + j;
   } else {
-    const int c = idx & 15;
-    lane = (idx >> 4) & 63;
-    ci = cc * kKC + (c >> 2) * 16 + (lane >> 4) * 4 + (c & 3);
+    const int j = idx & 3, q = (idx >> 8) & 3;
+    lane = (idx >> 2) & 63;
+    ci = cc * kKC + q * 16 + (lane >> 4) * 4 + j;
   }
   int co = cb * 16 + (lane & 15);
   IO v = (IO)0.f;
@@ -911,8 +913,8 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
     // of the chunk; half: one MFMA step of 32 channels, lane group g has 8 of them)
     constexpr int NF = kHalf ? 2 : NQ;
     typedef std::conditional_t<kHalf, int4v, float4v> Frag;
-    const int w_voff = kHalf ? lane * 16 : lane * 64;  // this lane's part of a fragment
-    constexpr int kWStep = kHalf ? 1024 : 16;          // from one 16-byte piece to the next
+    const int w_voff = lane * 16;  // this lane's 16 bytes of a KiB of fragments
+    constexpr int kWStep = 1024;   // from one 16-byte piece to the next
     const int w_soff0 = cb * nch * kFragB;  // fragments of this wave's column block
     const char *const a_base = reinterpret_cast<const char *>(abuf) + l16 * kRowB + g * 16;
     // The accumulators are addressed with 32-bit LDS byte addresses (acc_lane includes
