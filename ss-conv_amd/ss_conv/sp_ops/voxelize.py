@@ -48,7 +48,10 @@ class Point2Voxel(nn.Module):
         if fast is not None:
             valid_point_cloud, valid_feature, valid_ids, voxel_index, origin_ids, alive = fast
             B1 = len(origin_ids)
-            valid_instance_flag = torch.from_numpy(alive).to(device)
+            # all clouds kept points (the usual case): a fill on the device instead of a
+            # synchronous upload
+            valid_instance_flag = torch.ones(B1, dtype=torch.float32, device=device) \
+                if bool(alive.all()) else torch.from_numpy(alive).to(device)
             return self._voxelize(valid_point_cloud, valid_feature, valid_ids, voxel_index,
                                   int(origin_ids[-1]), valid_instance_flag, B1)
 
@@ -124,6 +127,7 @@ class Voxel2Point(nn.Module):
             np.asarray(voxel_extent, dtype=np.float64)
         self.unit_voxel_extent = None if unit_voxel_extent is None else \
             np.asarray(unit_voxel_extent, dtype=np.float64)
+        self._consts = {}  # (device, grid shape) -> (unit, extent) on the device
 
     def forward(self, sparse_feat, point_cloud=None, batch_ids=None):
         vx_points, vx_feats = self._get_vertice_feats(sparse_feat)
@@ -136,14 +140,20 @@ class Voxel2Point(nn.Module):
     def _get_vertice_feats(self, sparse_tensor):
         feat = sparse_tensor.features
         device = feat.device
-        shape = np.asarray(sparse_tensor.spatial_shape, dtype=np.float64)
-        if self.voxel_extent is not None:
-            unit = torch.tensor(self.voxel_extent / shape, dtype=torch.float32, device=device)
-            extent = torch.tensor(self.voxel_extent, dtype=torch.float32, device=device)
-        else:
-            unit = torch.tensor(self.unit_voxel_extent, dtype=torch.float32, device=device)
-            extent = torch.tensor(self.unit_voxel_extent * shape, dtype=torch.float32,
-                                  device=device)
+        # the two 3-vectors depend on the grid shape only: uploaded once (an upload from
+        # pageable memory is a synchronous copy of ~50 us)
+        key = (str(device), tuple(int(v) for v in sparse_tensor.spatial_shape))
+        if key not in self._consts:
+            shape = np.asarray(sparse_tensor.spatial_shape, dtype=np.float64)
+            if self.voxel_extent is not None:
+                unit = torch.tensor(self.voxel_extent / shape, dtype=torch.float32, device=device)
+                extent = torch.tensor(self.voxel_extent, dtype=torch.float32, device=device)
+            else:
+                unit = torch.tensor(self.unit_voxel_extent, dtype=torch.float32, device=device)
+                extent = torch.tensor(self.unit_voxel_extent * shape, dtype=torch.float32,
+                                      device=device)
+            self._consts[key] = (unit, extent)
+        unit, extent = self._consts[key]
         centres = sparse_tensor.indices.float()
         centres[:, 1:] = centres[:, 1:] * unit - 0.5 * extent + 0.5 * unit
         return centres.contiguous().detach(), feat
