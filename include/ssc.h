@@ -457,6 +457,18 @@ int ssc_bnact_bwd_f32(const float *x, const float *dy, int64_t n, int32_t c_in, 
                       const float *coef /* [c_in] or NULL */, float *dx /* [n,c_in] */,
                       ssc_stream_t stream);
 
+/* ------------------------------------------------------------------------
+ * One factor per row and field: y[r][c] = x[r][c] * scale[r][field_of[c]].  Replaces the
+ * expand / cat / multiply of the per-field dropout (ss_conv/dropout.py:29-46: a field's
+ * 2l+1 components share one Bernoulli draw); the draws themselves stay with the caller,
+ * so the random stream is the reference's.  The backward pass is the same call on the
+ * output gradient.  x and y may be the same buffer.
+ * ---------------------------------------------------------------------- */
+int ssc_field_scale_f32(const float *x /* [n,c] */, int64_t n, int32_t c,
+                        const float *scale /* [n,n_fields] */, int32_t n_fields,
+                        const int32_t *field_of /* [c] */, float *y /* [n,c] */,
+                        ssc_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -612,6 +612,33 @@ static size_t bn_ws_bytes(int64_t n, int c) {
 
 static bool act_ok(int a) { return a >= SSC_ACT_NONE && a <= SSC_ACT_TANH; }
 
+
+// y[r][c] = x[r][c] * scale[r][field_of[c]]: one factor per row and field, shared by the
+// field's 2l+1 components (the per-field dropout masks, ss_conv/dropout.py:25-46).
+// One thread per 4 columns (V = 4) or per column.
+typedef float float4v __attribute__((ext_vector_type(4)));
+template <int V>
+__global__ void __launch_bounds__(256)
+    field_scale_kernel(const float *__restrict__ x, int64_t n, int c, const float *__restrict__ scale,
+                       int n_fields, const int32_t *__restrict__ field_of, float *__restrict__ y) {
+  const int cv = c / V;
+  const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (e >= n * cv) return;
+  const int64_t r = e / cv;
+  const int col = (int)(e - r * cv) * V;
+  const float *s = scale + r * n_fields;
+  if (V == 4) {
+    float4v v = *reinterpret_cast<const float4v *>(x + r * c + col);
+    v.x *= s[field_of[col]];
+    v.y *= s[field_of[col + 1]];
+    v.z *= s[field_of[col + 2]];
+    v.w *= s[field_of[col + 3]];
+    *reinterpret_cast<float4v *>(y + r * c + col) = v;
+  } else {
+    y[r * c + col] = x[r * c + col] * s[field_of[col]];
+  }
+}
+
 }  // namespace ssc
 
 using namespace ssc;
@@ -764,6 +791,26 @@ int ssc_bnact_bwd_f32(const float *x, const float *dy, int64_t n, int32_t c_in, 
                        out_mode, gate_col, gated_first, gated_dim, act_scalar, act_gate, dz_mean,
                        coef, dx);
   SSC_LAUNCH_CHECK("bnact_bwd");
+  return SSC_OK;
+}
+
+int ssc_field_scale_f32(const float *x, int64_t n, int32_t c, const float *scale, int32_t n_fields,
+                        const int32_t *field_of, float *y, ssc_stream_t stream) {
+  SSC_CHECK(n >= 0 && c >= 1 && n_fields >= 1, SSC_EINVAL, "bad shape: n %lld, c %d, fields %d",
+            (long long)n, c, n_fields);
+  if (n == 0) return SSC_OK;
+  SSC_CHECK(x && scale && field_of && y, SSC_EINVAL, "NULL pointer argument");
+  const int V = (c & 3) == 0 ? 4 : 1;
+  const int64_t items = n * (c / V);
+  SSC_CHECK(ceil_div(items, 256) < ((int64_t)1 << 31), SSC_EINVAL, "tensor too large");
+  const dim3 grid((unsigned)ceil_div(items, 256));
+  if (V == 4)
+    hipLaunchKernelGGL(field_scale_kernel<4>, grid, dim3(256), 0, (hipStream_t)stream, x, n, c,
+                       scale, n_fields, field_of, y);
+  else
+    hipLaunchKernelGGL(field_scale_kernel<1>, grid, dim3(256), 0, (hipStream_t)stream, x, n, c,
+                       scale, n_fields, field_of, y);
+  SSC_LAUNCH_CHECK("field_scale");
   return SSC_OK;
 }
 }

@@ -100,6 +100,7 @@ _SIGNATURES = {
                                          _vp, _i32, _vp]),
     "ssc_bnact_bwd_sums_f32": (ctypes.c_int, [_vp, _vp, _i64, _i32, _i32, _vp, _vp, _vp, _vp, _vp,
                                               _vp, _vp, _vp, _i32, _i32, _vp, _vp, _sz, _vp]),
+    "ssc_field_scale_f32": (ctypes.c_int, [_vp, _i64, _i32, _vp, _i32, _vp, _vp, _vp]),
     "ssc_bnact_bwd_f32": (ctypes.c_int, [_vp, _vp, _i64, _i32, _i32, _vp, _vp, _vp, _vp, _vp, _vp,
                                          _vp, _vp, _i32, _i32, _vp, _vp, _vp, _vp]),
 }
@@ -671,6 +672,23 @@ def bnact_backward(x, dy, shift, scale, add, pre_bias, out_mode, gate_col, gated
         _ptr(pre_bias), _ptr(out_mode), _ptr(gate_col), _ptr(gated_first), _ptr(gated_dim),
         int(act_scalar), int(act_gate), _ptr(dz_mean), _ptr(coef), _ptr(dx), _stream(x)))
     return dx
+
+
+def field_scale(x, scale, field_of):
+    """y[r, c] = x[r, c] * scale[r, field_of[c]] for float32 x [n, C], scale [n, F] and an
+    int32 table field_of [C] (the multiply of ss_conv/dropout.py:44-45)."""
+    _need_gpu(x, scale, field_of)
+    if x.dtype != torch.float32 or scale.dtype != torch.float32 or field_of.dtype != torch.int32:
+        raise RuntimeError("field_scale: wrong dtypes")
+    x = x.contiguous()
+    scale = scale.contiguous()
+    n, c = x.shape
+    if scale.size(0) != n or field_of.numel() != c:
+        raise RuntimeError("field_scale: shapes do not match")
+    y = torch.empty_like(x)
+    _check(_lib.ssc_field_scale_f32(_ptr(x), n, c, _ptr(scale), scale.size(1), _ptr(field_of),
+                                    _ptr(y), _stream(x)))
+    return y
 
 
 def profile_conv(enable):

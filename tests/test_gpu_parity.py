@@ -838,6 +838,35 @@ def test_conv_order_promise_follows_the_input_order(oracle, device):
         assert rel_l2(gi.cpu().numpy(), want) < REL_L2
 
 
+@pytest.mark.parametrize("rs", [[(8, 0), (8, 1), (8, 2), (8, 3)], [(3, 0), (2, 2)], [(5, 1)]])
+def test_dropout_kernel_matches_expanded_masks(rs, device):
+    """Dropout on the GPU: masks drawn as the reference draws them (ss_conv/dropout.py:32-45),
+    multiplied in by ssc_field_scale_f32 -- same bits as the expanded product, forward and
+    backward."""
+    from ss_conv.dropout import Dropout
+    from ss_conv.sp_ops.tensor import SparseTensor
+    n = 3000
+    c = sum(m * (2 * l + 1) for m, l in rs)
+    drop = Dropout(rs, p=0.4).to(device).train()
+    x = torch.randn(n, c, device=device, requires_grad=True)
+    idx = torch.zeros((n, 4), dtype=torch.int32, device=device)
+    state = torch.cuda.get_rng_state(device)
+    y = drop(SparseTensor(x, idx, [4, 4, 4], 1)).features
+    torch.cuda.set_rng_state(state, device)
+    noises = []
+    for m, l in rs:
+        noise = x.new_empty(n, m).bernoulli_(0.6).div_(0.6)
+        noises.append(noise.unsqueeze(2).expand(-1, -1, 2 * l + 1).contiguous().view(n, -1))
+    noise = torch.cat(noises, dim=1)
+    assert torch.equal(y, x.detach() * noise)
+    g = torch.randn_like(y)
+    y.backward(g)
+    assert torch.equal(x.grad, g * noise)
+    drop.eval()
+    t = SparseTensor(x.detach(), idx, [4, 4, 4], 1)
+    assert drop(t).features is t.features
+
+
 def test_backbone_forward_matches_oracle(oracle, device):
     """The fourth benchmark configuration at reduced size: Point2Voxel -> four stages of
     [Convolution k3 -> BatchNorm -> gated Activation] with irreps (8,8,8,8) -> (16,...) ->

@@ -333,6 +333,27 @@ def test_dropout():
     assert 0.3 < (y == 0).float().mean() < 0.7
 
 
+def test_dropout_draws_the_masks_like_the_reference():
+    """Same seed, same masks: one new_empty(n, m).bernoulli_(1 - p).div_(1 - p) per entry of
+    Rs, in order, expanded over the 2l+1 components (ss_conv/dropout.py:32-45)."""
+    from ss_conv.dropout import Dropout
+    Rs = [(3, 0), (0, 1), (2, 1), (1, 2)]
+    x = torch.randn(50, 3 + 6 + 5)
+    drop = Dropout(Rs, p=0.3).train()
+    torch.manual_seed(7)
+    y = drop(_Holder(x.clone())).features
+    torch.manual_seed(7)
+    noises = []
+    for m, l in Rs:
+        if m == 0:
+            continue
+        noise = x.new_empty(50, m).bernoulli_(0.7).div_(0.7)
+        noises.append(noise.unsqueeze(2).expand(-1, -1, 2 * l + 1).contiguous().view(50, -1))
+    assert torch.equal(y, x * torch.cat(noises, dim=1))
+    for p, value in ((0.0, x), (1.0, torch.zeros_like(x))):
+        assert torch.equal(Dropout(Rs, p=p).train()(_Holder(x.clone())).features, value)
+
+
 def test_synthetic_generator_is_seeded():
     import synth
     a = synth.make_clouds(2, 100, seed=5, rotate=True, channels=3)
