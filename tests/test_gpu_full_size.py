@@ -1,0 +1,128 @@
+"""GPU parity at the full sizes of the benchmark configurations (32 clouds x 2048 points at
+64^3 with stride 1 and 2; 8 clouds x 16384 points at 128^3 with a 5^3 kernel).
+
+Rulebooks: bit-exact against the oracle, which runs these sizes in seconds.
+Convolution, forward and both gradients: against the oracle's gather-GEMM-scatter where
+that finishes in seconds, and at every size against a float64 statement of the same sums
+(src/conv/indice_conv.h:296-338, 385-421) evaluated with torch on the GPU -- a different
+formulation (one GEMM and one index_add per offset) of the same numbers -- plus two
+properties that do not depend on the size: linearity in the features, and the column sums
+of the output, which must equal sum_k (sum of the gathered rows of offset k) . W[k]."""
+import numpy as np
+import pytest
+import torch
+
+import synth
+from test_gpu_parity import REL_L2, rel_l2
+
+pytestmark = pytest.mark.gpu
+
+FULL = ["cfg2", "cfg3", "cfg5"]
+
+
+def _channels(cfg, key):
+    return sum(cfg[key] * (2 * l + 1) for l in range(cfg["lmax"] + 1))
+
+
+def _voxels(name):
+    cfg = synth.CONFIGS[name]
+    pts, _, ids = synth.config_clouds(name, seed=1)
+    return cfg, synth.voxel_indices(pts, ids, cfg["grid"])
+
+
+def _gpu_rulebook(cfg, idx, device):
+    from ss_conv.sp_ops.ops import get_indice_pairs
+    t = torch.from_numpy(idx).to(device)
+    return get_indice_pairs(t, cfg["batch"], [cfg["grid"]] * 3, cfg["kernel"], cfg["stride"],
+                            cfg["padding"], 1, 0, False)
+
+
+def _rel(a, b):
+    return float((a.double() - b).norm() / b.norm().clamp_min(1e-300))
+
+
+@pytest.mark.parametrize("name", FULL)
+def test_rulebook_full_size_matches_oracle(name, oracle, device):
+    print("config", name, flush=True)
+    cfg, idx = _voxels(name)
+    want = oracle.canonicalize(*oracle.rulebook(idx, cfg["batch"], [cfg["grid"]] * 3,
+                                                cfg["kernel"], cfg["stride"], cfg["padding"]))
+    got = _gpu_rulebook(cfg, idx, device)
+    for g, w in zip(got, want):
+        assert np.array_equal(g.cpu().numpy(), w)
+
+
+@pytest.mark.parametrize("name", FULL)
+def test_conv_full_size(name, oracle, device):
+    from ss_conv import _ext
+    print("config", name, flush=True)
+    cfg, idx = _voxels(name)
+    k = cfg["kernel"]
+    K = k ** 3
+    cin, cout = _channels(cfg, "mult_in"), _channels(cfg, "mult_out")
+    out_idx, pairs, num = _gpu_rulebook(cfg, idx, device)
+    n_in, n_out = idx.shape[0], out_idx.shape[0]
+    nums = num.cpu().numpy()
+    gen = torch.Generator(device).manual_seed(9)
+    f = torch.randn((n_in, cin), device=device, generator=gen)
+    w = torch.randn((K, cin, cout), device=device, generator=gen) / (K * cin) ** 0.5
+    w5 = w.reshape(k, k, k, cin, cout)
+    go = torch.randn((n_out, cout), device=device, generator=gen)
+
+    out = _ext.indice_conv_fp32(f, w5, pairs, num, n_out, 0, 0)
+    d_in, d_w = _ext.indice_conv_backward_fp32(f, w5, go, pairs, num, 0, 0)
+
+    # float64 statement of the three results, offset by offset
+    ref = torch.zeros((n_out, cout), dtype=torch.float64, device=device)
+    ref_in = torch.zeros((n_in, cin), dtype=torch.float64, device=device)
+    ref_w = torch.zeros((K, cin, cout), dtype=torch.float64, device=device)
+    col_sums = torch.zeros(cout, dtype=torch.float64, device=device)
+    for kk in range(K):
+        m = int(nums[kk])
+        if m == 0:
+            continue
+        i_rows, o_rows = pairs[kk, 0, :m].long(), pairs[kk, 1, :m].long()
+        fi, gk, wk = f[i_rows].double(), go[o_rows].double(), w[kk].double()
+        ref.index_add_(0, o_rows, fi @ wk)
+        ref_in.index_add_(0, i_rows, gk @ wk.t())
+        ref_w[kk] = fi.t() @ gk
+        col_sums += fi.sum(0) @ wk
+    assert _rel(out, ref) < REL_L2
+    assert _rel(d_in, ref_in) < REL_L2
+    assert _rel(d_w.reshape(K, cin, cout), ref_w) < REL_L2
+    # column sums: every pair counted once, none dropped
+    assert _rel(out.double().sum(0), col_sums) < REL_L2
+    # linearity in the features
+    f2 = torch.randn((n_in, cin), device=device, generator=gen)
+    out2 = _ext.indice_conv_fp32(f2, w5, pairs, num, n_out, 0, 0)
+    mix = _ext.indice_conv_fp32(2.0 * f + f2, w5, pairs, num, n_out, 0, 0)
+    assert _rel(mix, 2.0 * out.double() + out2.double()) < REL_L2
+    # rows no pair lands on are zero (every active output has at least one pair here, so
+    # this holds trivially unless the rulebook and the convolution disagree on n_out)
+    assert out.shape == (n_out, cout) and bool(torch.isfinite(out).all())
+    if name != "cfg5":  # the CPU restatement of this size takes seconds; cfg5's takes minutes
+        o_ref = oracle.conv_fwd(f.cpu().numpy(), w.cpu().numpy(), pairs.cpu().numpy(), nums,
+                                n_out, matmul=np.matmul)
+        assert rel_l2(out.cpu().numpy(), o_ref) < REL_L2
+
+
+def test_layer_chain_full_size(device):
+    """cfg3's stride-2 layer followed by average pooling and the global pools at full size:
+    sizes and invariants (pooling a non-negative tensor's maximum dominates its average;
+    the segment mean of a constant column is the constant)."""
+    from ss_conv.pool import AvgPool, MaxPool, GlobalAvgPool
+    from ss_conv.sp_ops.tensor import SparseTensor
+    cfg, idx = _voxels("cfg3")
+    t = torch.from_numpy(idx).to(device)
+    x = torch.rand((idx.shape[0], 64), device=device)
+    x[:, 0] = 3.0
+    st = SparseTensor(x, t, [cfg["grid"]] * 3, cfg["batch"])
+    mx = MaxPool(3, 2, 1)(SparseTensor(x, t, [cfg["grid"]] * 3, cfg["batch"]))
+    av = AvgPool(3, 2, 1)(st)
+    assert torch.equal(mx.indices, av.indices)
+    assert bool((mx.features >= av.features - 1e-6).all())
+    assert bool((mx.features[:, 0] == 3.0).all())
+    offs = av.get_offsets().int().contiguous()
+    pooled = GlobalAvgPool()(mx.features.contiguous(), offs)
+    assert pooled.shape == (cfg["batch"], 64)
+    assert torch.allclose(pooled[:, 0], torch.full((cfg["batch"],), 3.0, device=device))
