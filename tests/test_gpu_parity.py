@@ -838,6 +838,39 @@ def test_conv_order_promise_follows_the_input_order(oracle, device):
         assert rel_l2(gi.cpu().numpy(), want) < REL_L2
 
 
+def test_conv_call_replays_in_a_hip_graph(device):
+    """The convolution call enqueues kernels only (no host read, no memset), so a captured
+    graph of it can be replayed: every replay, with eager work and synchronisations in
+    between, gives the bits of the eager call on the same buffers."""
+    from ss_conv import _ext
+    rng = np.random.default_rng(31)
+    grid, n, cin, cout = 16, 2500, 64, 96
+    idx = random_voxels(rng, 2, grid, n)
+    g_idx, g_pairs, g_num = [torch.from_numpy(x).to(device) for x in
+                             gpu_rulebook(idx, 2, grid, 3, 1, 1)]
+    n_out = g_idx.shape[0]
+    f = torch.randn((n, cin), device=device)
+    w = torch.randn((3, 3, 3, cin, cout), device=device) / (27 * cin) ** 0.5
+    eager = _ext.indice_conv_fp32(f, w, g_pairs, g_num, n_out, 0, 0)  # also the warm-up
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            captured = _ext.indice_conv_fp32(f, w, g_pairs, g_num, n_out, 0, 0)
+    torch.cuda.current_stream().wait_stream(side)
+    for trial in range(4):
+        if trial:  # new values in the captured input buffers, eager result for them
+            f.copy_(torch.randn((n, cin), device=device))
+            w.copy_(torch.randn((3, 3, 3, cin, cout), device=device) / (27 * cin) ** 0.5)
+            eager = _ext.indice_conv_fp32(f, w, g_pairs, g_num, n_out, 0, 0)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(captured, eager), trial
+
+
 @pytest.mark.parametrize("rs", [[(8, 0), (8, 1), (8, 2), (8, 3)], [(3, 0), (2, 2)], [(5, 1)]])
 def test_dropout_kernel_matches_expanded_masks(rs, device):
     """Dropout on the GPU: masks drawn as the reference draws them (ss_conv/dropout.py:32-45),
