@@ -735,10 +735,28 @@ def test_batchnorm_activation_match_oracle(case, oracle, device):
     module.train(training)
     running = (bn.running_mean.cpu().numpy().copy(), bn.running_var.cpu().numpy().copy())
     st = SparseTensor(x, torch.zeros(n, 4, dtype=torch.int32, device=device), [4, 4, 4], 1)
-    y = module(st).features
-    dy_np = rng.normal(size=tuple(y.shape)).astype(np.float32)
-    y.backward(torch.from_numpy(dy_np).to(device))
-    torch.cuda.synchronize()
+    # the layers must run on the library's kernels here, not on their torch code
+    from ss_conv import _ext
+    calls = {"fwd": 0, "bwd": 0}
+    real_fwd, real_bwd = _ext.bnact_forward, _ext.bnact_backward
+
+    def counted_fwd(*a, **k):
+        calls["fwd"] += 1
+        return real_fwd(*a, **k)
+
+    def counted_bwd(*a, **k):
+        calls["bwd"] += 1
+        return real_bwd(*a, **k)
+
+    _ext.bnact_forward, _ext.bnact_backward = counted_fwd, counted_bwd
+    try:
+        y = module(st).features
+        dy_np = rng.normal(size=tuple(y.shape)).astype(np.float32)
+        y.backward(torch.from_numpy(dy_np).to(device))
+        torch.cuda.synchronize()
+    finally:
+        _ext.bnact_forward, _ext.bnact_backward = real_fwd, real_bwd
+    assert calls == {"fwd": 1, "bwd": 1}, calls
 
     sb = act.scalar_act.bias if act.scalar_act is not None else None
     gb = act.gate_act.bias if act.gate_act is not None else None
