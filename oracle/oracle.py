@@ -122,6 +122,10 @@ def _rulebook(fn_conv, fn_subm, indices, batch_size, in_shape, ksize, stride, pa
     indices = _i32(indices)
     n = indices.shape[0]
     ks, st, pd, dl = _triple(ksize), _triple(stride), _triple(padding), _triple(dilation)
+    # the reference refuses a stride and a dilation above 1 on the same axis
+    # (ss_conv/sp_ops/conv.py:50-51); its candidate enumeration is only valid without
+    if not subm and any(s > 1 and d > 1 for s, d in zip(st, dl)):
+        raise ValueError("stride > 1 together with dilation > 1 is not supported")
     if subm:  # src/conv/indice_conv.h:70-74
         st, pd = [1, 1, 1], [k // 2 for k in ks]
         out_shape = list(in_shape)

@@ -186,9 +186,14 @@ def get_indice_pairs_3d(indices, batch_size, out_spatial_shape, spatial_shape, k
                                            ctypes.byref(in_order), s))
     pairs = torch.empty((K, 2, n), dtype=torch.int32, device=dev)
     num = torch.empty((K,), dtype=torch.int32, device=dev)
-    outids = indices if subm else torch.empty((n_out.value, 4), dtype=torch.int32, device=dev)
+    # a geometry may leave no output at all (every candidate clipped): the library still
+    # wants a valid pointer, so at least one row is allocated and the result is a slice of it
+    out_buf = None if subm else torch.empty((max(n_out.value, 1), 4), dtype=torch.int32,
+                                            device=dev)
+    outids = indices if subm else out_buf[:n_out.value]
     _check(_lib.ssc_rulebook_emit(_ptr(indices), n, ctypes.byref(g), ws.data_ptr(), ws.numel(),
-                                  None if subm else _ptr(outids), _ptr(pairs), num.data_ptr(), s))
+                                  None if subm else out_buf.data_ptr(), _ptr(pairs),
+                                  num.data_ptr(), s))
     # Pairs of an offset always ascend in the input rows, and in the output rows too when
     # the input rows came in key order: the convolution may then skip its order check
     # (the first flag serves a call that accumulates into output rows, the second one

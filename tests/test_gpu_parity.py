@@ -95,6 +95,102 @@ def test_rulebook_empty_and_errors(device):
                                  [0] * 3, 0, 0)
 
 
+def test_rulebook_without_any_output(oracle, device):
+    """A stride can step over every candidate of a voxel: no active output at all.  The
+    rulebook is empty, and convolution, pooling and their gradients on it return empty or
+    zero tensors (the reference allocates zero-row tensors, indice_conv.h:49-56,278)."""
+    from ss_conv import _ext
+    idx = np.array([[0, 1, 0, 0], [1, 4, 2, 1]], dtype=np.int32)
+    geo = dict(batch=2, shape=[13, 4, 4], ks=[2, 2, 2], st=[3, 3, 2], pd=[1, 2, 1])
+    o_idx, o_pairs, o_num, _ = oracle.rulebook(idx, geo["batch"], geo["shape"], geo["ks"],
+                                               geo["st"], geo["pd"])
+    assert o_idx.shape[0] == 0 and int(o_num.sum()) == 0
+    t = torch.from_numpy(idx).to(device)
+    from ss_conv.sp_ops.ops import get_indice_pairs
+    out, pairs, num = get_indice_pairs(t, geo["batch"], geo["shape"], geo["ks"], geo["st"],
+                                       geo["pd"], 1, 0, False)
+    assert out.shape == (0, 4) and int(num.sum()) == 0 and bool((pairs == -1).all())
+    f = torch.randn((2, 8), device=device)
+    w = torch.randn((2, 2, 2, 8, 12), device=device)
+    y = _ext.indice_conv_fp32(f, w, pairs, num, 0, 0, 0)
+    assert y.shape == (0, 12)
+    d_in, d_w = _ext.indice_conv_backward_fp32(f, w, y, pairs, num, 0, 0)
+    assert d_in.shape == f.shape and not d_in.any() and d_w.shape == w.shape and not d_w.any()
+    assert _ext.indice_maxpool_fp32(f, pairs, num, 0).shape == (0, 8)
+    rf = _ext.indiceSummaryRF(pairs, num, 0)
+    assert rf.shape == (0,)
+    assert _ext.indice_avgpool_fp32(f, pairs, num, 0, rf).shape == (0, 8)
+
+
+@pytest.mark.parametrize("seed", [1, 2, 3])
+def test_anisotropic_geometries_match_oracle(seed, oracle, device):
+    """Kernel size, stride, padding and dilation differing per axis, non-cubic grids, inputs
+    in key order or shuffled, regular and submanifold: rulebook bit-exact, convolution
+    (forward, both gradients) and both pools against the oracle, 40 seeded cases a seed."""
+    from ss_conv import _ext
+    from ss_conv.sp_ops.ops import get_indice_pairs
+    rng = np.random.default_rng(seed)
+    done = 0
+    while done < 40:
+        batch = int(rng.integers(1, 4))
+        shape = [int(rng.integers(3, 14)) for _ in range(3)]
+        ks = [int(rng.integers(1, 4)) for _ in range(3)]
+        st = [int(rng.integers(1, 4)) for _ in range(3)]
+        dl = [int(rng.integers(1, 3)) if t == 1 else 1 for t in st]
+        pd = [int(rng.integers(0, 3)) for _ in range(3)]
+        subm = bool(rng.integers(0, 4) == 0)
+        if subm:
+            ks, st = [k | 1 for k in ks], [1, 1, 1]
+        out_shape = [(n + 2 * p - d * (k - 1) - 1) // t + 1
+                     for n, p, d, k, t in zip(shape, pd, dl, ks, st)]
+        if min(out_shape) < 1:
+            continue
+        done += 1
+        cells = batch * shape[0] * shape[1] * shape[2]
+        n = int(rng.integers(1, min(cells, 400) + 1))
+        flat = np.sort(rng.choice(cells, size=n, replace=False))
+        vol = shape[0] * shape[1] * shape[2]
+        b, r = flat // vol, flat % vol
+        idx = np.stack([b, r // (shape[1] * shape[2]), (r // shape[2]) % shape[1],
+                        r % shape[2]], 1).astype(np.int32)
+        if rng.integers(0, 3) == 0:
+            idx = idx[rng.permutation(n)]
+        case = (batch, shape, ks, st, pd, dl, subm, n)
+        print("case", case, flush=True)
+        raw = oracle.rulebook(idx, batch, shape, ks, st, pd, dl, subm)
+        # submanifold outputs keep the input numbering; regular ones are numbered by key
+        o_idx, o_pairs, o_num = raw[:3] if subm else oracle.canonicalize(*raw)
+        g = get_indice_pairs(torch.from_numpy(idx).to(device), batch, shape, ks, st, pd, dl, 0, subm)
+        for got, want in zip(g, (o_idx, o_pairs, o_num)):
+            assert np.array_equal(got.cpu().numpy(), want), case
+        K = ks[0] * ks[1] * ks[2]
+        n_out = o_idx.shape[0]
+        cin, cout = int(rng.choice([3, 8, 16, 37, 64, 72])), int(rng.choice([5, 16, 24, 64, 80]))
+        f = rng.normal(size=(n, cin)).astype(np.float32)
+        w = (rng.normal(size=(K, cin, cout)) / np.sqrt(K * cin)).astype(np.float32)
+        go = rng.normal(size=(n_out, cout)).astype(np.float32)
+        ft, wt, got_ = [torch.from_numpy(a).to(device) for a in (f, w, go)]
+        wt = wt.reshape(*ks, cin, cout)
+        y = _ext.indice_conv_fp32(ft, wt, g[1], g[2], n_out, 0, int(subm))
+        d_in, d_w = _ext.indice_conv_backward_fp32(ft, wt, got_, g[1], g[2], 0, int(subm))
+        assert rel_l2(y.cpu().numpy(), oracle.conv_fwd(f, w, o_pairs, o_num, n_out,
+                                                       matmul=np.matmul)) < REL_L2, case
+        r_in, r_w = oracle.conv_bwd(f, w, go, o_pairs, o_num)
+        assert rel_l2(d_in.cpu().numpy(), r_in) < REL_L2, case
+        assert rel_l2(d_w.cpu().numpy().reshape(K, cin, cout), r_w) < REL_L2, case
+        c = int(rng.choice([4, 7, 32]))
+        pf = rng.normal(size=(n, c)).astype(np.float32)
+        pt = torch.from_numpy(pf).to(device)
+        mx = _ext.indice_maxpool_fp32(pt, g[1], g[2], n_out)
+        assert np.array_equal(mx.cpu().numpy(), oracle.maxpool_fwd(pf, o_pairs, o_num, n_out)), case
+        rf = _ext.indiceSummaryRF(g[1], g[2], n_out)
+        o_rf = oracle.summary_rf(o_pairs, o_num, n_out)
+        assert np.array_equal(rf.cpu().numpy(), o_rf), case
+        av = _ext.indice_avgpool_fp32(pt, g[1], g[2], n_out, rf)
+        assert np.array_equal(av.cpu().numpy(),
+                              oracle.avgpool_fwd(pf, o_pairs, o_num, n_out, o_rf)), case
+
+
 def test_rulebook_config1_sizes(oracle, device):
     c = synth.CONFIGS["cfg1"]
     pts, _, ids = synth.config_clouds("cfg1")

@@ -146,3 +146,57 @@ def test_invariants_subm(oracle):
 def test_empty_input(oracle):
     o_idx, pairs, num, _ = oracle.rulebook(np.zeros((0, 4), np.int32), 1, [8] * 3, 3, 1, 1)
     assert o_idx.shape == (0, 4) and pairs.shape == (27, 2, 0) and num.sum() == 0
+
+
+def test_stride_with_dilation_is_refused(oracle):
+    """The reference asserts stride == 1 or dilation == 1 per axis (ss_conv/sp_ops/conv.py:50-51):
+    its candidate enumeration (geometry.h:18-80) yields offsets outside the kernel otherwise."""
+    idx = np.array([[0, 2, 2, 2]], dtype=np.int32)
+    with pytest.raises(ValueError):
+        oracle.rulebook(idx, 1, [8] * 3, [1, 1, 3], [3, 1, 1], [2, 0, 1], [2, 1, 1])
+    # on different axes both are fine
+    o_idx, _, num, _ = oracle.rulebook(idx, 1, [8] * 3, [1, 1, 3], [1, 2, 1], [0, 0, 1], [1, 1, 2])
+    assert o_idx.shape[0] == int(num.sum()) == 2  # z + 1 - 2 kz in {3, 1, -1}: two inside
+
+
+def test_anisotropic_geometries_against_brute_force(oracle):
+    """Kernel size, stride, padding and dilation differing per axis on a non-cubic grid: the
+    pairs must be exactly those (input, offset) whose output position is integral and inside
+    the output grid: out * s = in + p - k * d."""
+    rng = np.random.default_rng(12)
+    for _ in range(40):
+        shape = [int(rng.integers(3, 10)) for _ in range(3)]
+        ks = [int(rng.integers(1, 4)) for _ in range(3)]
+        st = [int(rng.integers(1, 4)) for _ in range(3)]
+        dl = [int(rng.integers(1, 3)) if s == 1 else 1 for s in st]
+        pd = [int(rng.integers(0, 3)) for _ in range(3)]
+        out_shape = [(n + 2 * p - d * (k - 1) - 1) // s + 1
+                     for n, p, d, k, s in zip(shape, pd, dl, ks, st)]
+        if min(out_shape) < 1:
+            continue
+        cells = 2 * shape[0] * shape[1] * shape[2]
+        n = int(rng.integers(1, min(cells, 60) + 1))
+        flat = np.sort(rng.choice(cells, size=n, replace=False))
+        vol = shape[0] * shape[1] * shape[2]
+        b, r = flat // vol, flat % vol
+        idx = np.stack([b, r // (shape[1] * shape[2]), (r // shape[2]) % shape[1],
+                        r % shape[2]], 1).astype(np.int32)
+        o_idx, pairs, num, o_shape = oracle.rulebook(idx, 2, shape, ks, st, pd, dl)
+        assert list(o_shape) == out_shape
+        want = set()
+        for i, (bb, x, y, z) in enumerate(idx):
+            for kx in range(ks[0]):
+                for ky in range(ks[1]):
+                    for kz in range(ks[2]):
+                        num_ = [x + pd[0] - kx * dl[0], y + pd[1] - ky * dl[1], z + pd[2] - kz * dl[2]]
+                        if any(v % s for v, s in zip(num_, st)):
+                            continue
+                        o = [v // s for v, s in zip(num_, st)]
+                        if all(0 <= v < m for v, m in zip(o, out_shape)):
+                            want.add((i, (kx * ks[1] + ky) * ks[2] + kz, bb, *o))
+        got = set()
+        for k in range(len(num)):
+            for j in range(int(num[k])):
+                i, o = int(pairs[k, 0, j]), int(pairs[k, 1, j])
+                got.add((i, k, *[int(v) for v in o_idx[o]]))
+        assert got == want, (shape, ks, st, pd, dl)
