@@ -417,6 +417,66 @@ def test_point2voxel_unsorted_ids_and_outliers(oracle, device):
         assert flag.cpu().tolist() == ref["flag"].tolist()
 
 
+@pytest.mark.parametrize("seed", [1, 2])
+def test_point_voxel_random_configurations(seed, oracle, device):
+    """Point2Voxel and Voxel2Point on 40 seeded configurations a seed: 1-5 clouds (some empty,
+    some entirely outside, ids with gaps, points in batch order or shuffled), non-cubic voxel
+    limits, anisotropic voxel extents, all four reduction modes, points exactly on cell faces
+    and duplicated points.  Voxel lists, features, 3-NN indices and distances bit-exact."""
+    from ss_conv.sp_ops.functional import three_nn
+    from ss_conv.sp_ops.voxelize import Point2Voxel, Voxel2Point
+    rng = np.random.default_rng(seed)
+    for case in range(40):
+        B = int(rng.integers(1, 6))
+        limit = [int(rng.integers(2, 20)) for _ in range(3)]
+        unit = [float(rng.choice([0.05, 0.1, 0.125, 0.3, 0.07])) for _ in range(3)]
+        mode = int(rng.integers(1, 5))
+        C = int(rng.choice([1, 3, 6, 16, 33]))
+        counts = [int(rng.integers(0, 300)) for _ in range(B)]
+        if sum(counts) == 0:
+            counts[0] = 5
+        ids = np.concatenate([np.full(c, b, dtype=np.int64) for b, c in enumerate(counts)])
+        if rng.integers(0, 3) == 0:
+            ids = ids * 2 + 1
+        n = len(ids)
+        half = 0.5 * np.array(limit) * np.array(unit)
+        scale = float(rng.choice([0.5, 1.0, 1.3]))
+        pts = (rng.uniform(-1, 1, size=(n, 3)) * half * scale).astype(np.float32)
+        on_face = rng.integers(0, 10, size=n) == 0
+        u32 = np.array(unit, np.float32)
+        pts[on_face] = (np.round(pts[on_face] / u32) * u32).astype(np.float32)
+        if n > 4:
+            pts[rng.integers(0, n, size=n // 8)] = pts[rng.integers(0, n, size=n // 8)]
+        if rng.integers(0, 4) == 0 and B > 1:
+            pts[ids == ids[0]] = 1e3
+        feats = rng.normal(size=(n, C)).astype(np.float32)
+        if rng.integers(0, 4) == 0:
+            perm = rng.permutation(n)
+            pts, feats, ids = pts[perm], feats[perm], ids[perm]
+        print("case", case, B, limit, unit, mode, C, n, flush=True)
+        ref = oracle.point2voxel(pts, feats, ids, limit, unit, mode)
+        vp, st, vi, flag = Point2Voxel(limit, unit, mode)(
+            torch.from_numpy(pts).to(device), torch.from_numpy(feats).to(device),
+            torch.from_numpy(ids).to(device))
+        assert np.array_equal(vp.cpu().numpy(), ref["valid_points"]), case
+        assert np.array_equal(vi.cpu().numpy(), ref["valid_ids"]), case
+        assert np.array_equal(flag.cpu().numpy(), ref["flag"]), case
+        assert np.array_equal(st.indices.cpu().numpy(), ref["indices"]), case
+        assert st.batch_size == ref["batch_size"], case
+        assert np.array_equal(st.features.cpu().numpy(), ref["features"]), case
+        v2p = Voxel2Point(unit_voxel_extent=unit)
+        out = v2p(st, vp, vi)
+        want, _, _ = oracle.voxel2point(st.indices.cpu().numpy(), st.features.cpu().numpy(), limit,
+                                        vp.cpu().numpy(), vi.cpu().numpy(), unit_voxel_extent=unit)
+        assert rel_l2(out.cpu().numpy(), want) < REL_L2, case
+        centres = v2p._get_vertice_feats(st)[0]
+        target = torch.cat([vi.float().unsqueeze(1), vp], 1).contiguous()
+        dist, idx = three_nn(target, centres)
+        odist, oidx = oracle.three_nn(target.cpu().numpy(), centres.cpu().numpy())
+        assert np.array_equal(idx.cpu().numpy(), oidx), case
+        assert np.array_equal(dist.cpu().numpy(), odist), case
+
+
 def test_voxel2point_matches_oracle(oracle, device):
     from ss_conv.sp_ops.voxelize import Point2Voxel, Voxel2Point
     pts, feats, ids = synth.make_clouds(3, 500, seed=6, channels=10)
