@@ -21,7 +21,8 @@
 namespace ssc {
 
 constexpr int kBnThreads = 256;
-constexpr int kBnMaxBlocks = 1024;
+constexpr int kBnMaxBlocks = 1024;      // row slabs of the kernels that leave partial sums
+constexpr int kBnMaxApplyBlocks = 4096; // row slabs of the backward apply kernel (no partial sums)
 constexpr int kBnMaxBwdChannels = 1536;  // column tables of the backward kernels: 48 KB of LDS
 
 struct BnShape {
@@ -31,12 +32,13 @@ struct BnShape {
 };
 
 // `c` counts the units a thread handles: columns, or groups of four columns.
-static BnShape bn_shape(int64_t n, int c) {
+static BnShape bn_shape(int64_t n, int c, int max_tx = kBnThreads,
+                        int max_blocks = kBnMaxBlocks) {
   BnShape s;
   s.tx = 16;
-  while (s.tx < c && s.tx < kBnThreads) s.tx <<= 1;
+  while (s.tx < c && s.tx < max_tx) s.tx <<= 1;
   s.ty = kBnThreads / s.tx;
-  int64_t rpb = ceil_div(n > 0 ? n : 1, kBnMaxBlocks);
+  int64_t rpb = ceil_div(n > 0 ? n : 1, max_blocks);
   rpb = ceil_div(rpb, s.ty) * s.ty;  // whole trips of the row lanes
   if (rpb < 4 * s.ty) rpb = 4 * s.ty;
   s.rows_per_block = (int)rpb;
@@ -426,26 +428,35 @@ struct GateRow {
 // Work items of the backward kernels: the output columns in groups of V, then the gate
 // columns one by one (a gate's gradient sums over its whole field, about as much work
 // as a group of plain columns).
+// The groups are padded to a multiple of TX items (TX <= 64 threads take one item each per
+// pass), so that a pass is all groups or all gate columns: the two kinds run different
+// code, and lanes of one wave that disagreed would execute both.
 struct BwdItem {
   int c;       // first column
-  int width;   // V for a group, 1 for a gate column, 0 beyond the last item
+  int width;   // V for a group, 1 for a gate column, 0 for padding and beyond the last item
   bool group;  // a group of output columns (not a gate column)
 };
+__host__ __device__ __forceinline__ int bwd_groups_padded(int c_out, int V, int TX) {
+  return (c_out / V + TX - 1) / TX * TX;
+}
 template <int V>
-__device__ __forceinline__ BwdItem bwd_item(int it, int c_in, int c_out) {
-  const int nvec = c_out / V;
+__device__ __forceinline__ BwdItem bwd_item(int it, int c_in, int c_out, int TX) {
+  const int nvec = c_out / V, nvp = bwd_groups_padded(c_out, V, TX);
   BwdItem w;
   w.group = it < nvec;
-  if (w.group) {
+  if (it < nvp) {
     w.c = it * V;
-    w.width = V;
+    w.width = w.group ? V : 0;
   } else {
-    w.c = c_out + (it - nvec);
+    w.c = c_out + (it - nvp);
     w.width = w.c < c_in ? 1 : 0;
   }
   return w;
 }
-static int bwd_items(int c_in, int c_out, int V) { return c_out / V + (c_in - c_out); }
+// thread shape of the backward kernels: at most one wave of items per row of threads
+static BnShape bwd_shape(int64_t n, int c_out, int V, int max_blocks = kBnMaxBlocks) {
+  return bn_shape(n, c_out / V, 64, max_blocks);
+}
 
 // partial[b*2C + c] = sum of dz over the rows of block b, partial[b*2C + C + c] = sum of
 // dz * (x - shift)
@@ -466,9 +477,9 @@ __global__ void __launch_bounds__(kBnThreads)
   const int tx = threadIdx.x % TX, ty = threadIdx.x / TX;
   const int64_t r0 = (int64_t)blockIdx.x * rows_per_block;
   const int64_t r1 = r0 + rows_per_block < n ? r0 + rows_per_block : n;
-  const int n_items = c_out / V + (c_in - c_out);
+  const int n_items = bwd_groups_padded(c_out, V, TX) + (c_in - c_out);
   for (int it0 = 0; it0 < n_items; it0 += TX) {
-    const BwdItem w = bwd_item<V>(it0 + tx, c_in, c_out);
+    const BwdItem w = bwd_item<V>(it0 + tx, c_in, c_out, TX);
     float sb[V], sa[V], sh[V];
 #pragma unroll
     for (int i = 0; i < V; ++i) {
@@ -545,9 +556,9 @@ __global__ void __launch_bounds__(kBnThreads)
   const int tx = threadIdx.x % TX, ty = threadIdx.x / TX;
   const int64_t r0 = (int64_t)blockIdx.x * rows_per_block;
   const int64_t r1 = r0 + rows_per_block < n ? r0 + rows_per_block : n;
-  const int n_items = c_out / V + (c_in - c_out);
+  const int n_items = bwd_groups_padded(c_out, V, TX) + (c_in - c_out);
   for (int it = tx; it < n_items; it += TX) {
-    const BwdItem w = bwd_item<V>(it, c_in, c_out);
+    const BwdItem w = bwd_item<V>(it, c_in, c_out, TX);
     float sh[V], sc[V], dm[V], cf[V];
 #pragma unroll
     for (int i = 0; i < V; ++i) {
@@ -598,6 +609,136 @@ __global__ void __launch_bounds__(kBnThreads)
       }
     }
   }
+}
+
+// Both backward kernels in the form used when a row fits one pass: TX threads per row,
+// thread tx owns the group of V output columns tx*V .. (c_out/V groups) AND the gate
+// column c_out + tx (c_in - c_out gates), TX >= both counts.  A gate column's gradient is
+// act'(gate) * sum_j dy[j] * z[j] over its field's columns; the threads that own those
+// columns have x[j] and dy[j] in registers anyway, so they leave the products in LDS and
+// the gate's thread adds them up in ascending column order -- the sum, and its rounding,
+// of the plain loop (bnact_dz), without reading the field's columns again.
+//   APPLY = false: partial[b*2C + c] = sum of dz over the block's rows,
+//                  partial[b*2C + C + c] = sum of dz * (x - shift)
+//   APPLY = true:  dx[r,c] = scale[c] * (dz - dz_mean[c]) - coef[c] * (x[r,c] - shift[c])
+template <int V, bool APPLY>
+__global__ void __launch_bounds__(kBnThreads)
+    bnact_bwd_row_kernel(const float *__restrict__ x, const float *__restrict__ dy, int64_t n,
+                         int c_in, int c_out, int TX, int rows_per_block, ColAffine aff,
+                         const int32_t *__restrict__ out_mode,
+                         const int32_t *__restrict__ gate_col,
+                         const int32_t *__restrict__ gated_first,
+                         const int32_t *__restrict__ gated_dim, int act_s, int act_g,
+                         const float *__restrict__ dz_mean, const float *__restrict__ coef,
+                         float *__restrict__ dx, float *__restrict__ partial) {
+  __shared__ float red[kBnThreads];
+  extern __shared__ float lds[];
+  const ColTables t =
+      stage_tables(lds, c_in, c_out, aff, out_mode, gate_col, gated_first, gated_dim);
+  const int TY = kBnThreads / TX;
+  float *prod = lds + 8 * c_in;  // [2][TY][c_out]: dy * z of the row's output columns
+  const int tx = threadIdx.x % TX, ty = threadIdx.x / TX;
+  const int64_t r0 = (int64_t)blockIdx.x * rows_per_block;
+  const int64_t r1 = r0 + rows_per_block < n ? r0 + rows_per_block : n;
+  const bool has_group = tx < c_out / V;
+  const int c0 = has_group ? tx * V : 0;
+  const int cg = c_out + tx;  // this thread's gate column
+  const bool own_gate_col = cg < c_in;
+  const int cgs = own_gate_col ? cg : 0;
+  // a gate without a field (dim 0) has dz = 0, as in bnact_dz
+  const int gfirst = own_gate_col ? t.gfirst[cgs] : 0, gdim = own_gate_col ? t.gdim[cgs] : 0;
+  const float g_sh = t.shift[cgs], g_sc = t.scale[cgs], g_adp = t.add[cgs] + t.pre[cgs];
+  GroupConst<V> gc;
+  gc.init(t, c0);
+  float sh[V], sc[V], dm[V], cf[V], sb[V], sa[V];
+#pragma unroll
+  for (int i = 0; i < V; ++i) {
+    sh[i] = t.shift[c0 + i];
+    sc[i] = t.scale[c0 + i];
+    dm[i] = (APPLY && dz_mean) ? dz_mean[c0 + i] : 0.f;
+    cf[i] = (APPLY && coef) ? coef[c0 + i] : 0.f;
+    sb[i] = sa[i] = 0.f;
+  }
+  const float g_dm = (APPLY && dz_mean) ? dz_mean[cgs] : 0.f;
+  const float g_cf = (APPLY && coef) ? coef[cgs] : 0.f;
+  float sbg = 0.f, sag = 0.f;
+  // rows are taken TY at a time by the whole block (the trip count is the same for every
+  // thread: there is a barrier in the loop); a thread's row may lie beyond the slab
+  GroupRow<V> cur, nxt;
+  float xg_cur = 0.f, xg_nxt = 0.f;
+  auto load_row = [&](int64_t r, GroupRow<V> &row, float &xgate) {
+    if (has_group) row.load(x + r * c_in, dy + r * c_out, c0, gc);
+    if (own_gate_col) xgate = x[r * c_in + cg];
+  };
+  if (r0 + ty < r1) load_row(r0 + ty, cur, xg_cur);
+  int par = 0;
+  for (int64_t rb = r0; rb < r1; rb += TY) {
+    const int64_t r = rb + ty;
+    const bool live = r < r1;
+    const int64_t rn = r + TY < r1 ? r + TY : (live ? r : r1 - 1);  // a row that exists
+    load_row(rn, nxt, xg_nxt);
+    float *prow = prod + ((size_t)par * TY + ty) * c_out;
+    if (has_group && live) {
+      Vec<V> o;
+#pragma unroll
+      for (int i = 0; i < V; ++i) {
+        const float xv = cur.x.v[i], dv = cur.dy.v[i];
+        prow[c0 + i] = dv * ((xv - sh[i]) * sc[i] + gc.ad[i]);
+        const float d = gc.dz(i, xv, dv, cur.xg[i], act_s, act_g);
+        if (APPLY) {
+          o.v[i] = sc[i] * (d - dm[i]) - cf[i] * (xv - sh[i]);
+        } else {
+          sb[i] += d;
+          sa[i] += d * (xv - sh[i]);
+        }
+      }
+      if (APPLY) o.store(dx + r * c_in + c0);
+    }
+    __syncthreads();
+    if (own_gate_col && live) {
+      float acc = 0.f;
+      for (int j = 0; j < gdim; ++j) acc += prow[gfirst + j];
+      const float d = gdim > 0 ? acc * act_grad(act_g, (xg_cur - g_sh) * g_sc + g_adp) : 0.f;
+      if (APPLY) {
+        dx[r * c_in + cg] = g_sc * (d - g_dm) - g_cf * (xg_cur - g_sh);
+      } else {
+        sbg += d;
+        sag += d * (xg_cur - g_sh);
+      }
+    }
+    cur = nxt;
+    xg_cur = xg_nxt;
+    par ^= 1;
+  }
+  if (!APPLY) {
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+      const float tb = reduce_rows(sb[i], red, tx, ty, TX, TY);
+      const float ta = reduce_rows(sa[i], red, tx, ty, TX, TY);
+      if (ty == 0 && has_group) {
+        partial[(int64_t)blockIdx.x * 2 * c_in + c0 + i] = tb;
+        partial[(int64_t)blockIdx.x * 2 * c_in + c_in + c0 + i] = ta;
+      }
+    }
+    const float tb = reduce_rows(sbg, red, tx, ty, TX, TY);
+    const float ta = reduce_rows(sag, red, tx, ty, TX, TY);
+    if (ty == 0 && own_gate_col) {
+      partial[(int64_t)blockIdx.x * 2 * c_in + cg] = tb;
+      partial[(int64_t)blockIdx.x * 2 * c_in + c_in + cg] = ta;
+    }
+  }
+}
+
+// Thread shape of bnact_bwd_row_kernel, or tx = 0 when a row does not fit one pass.
+static BnShape bwd_row_shape(int64_t n, int c_in, int c_out, int V, int max_blocks) {
+  const int items = c_out / V > c_in - c_out ? c_out / V : c_in - c_out;
+  BnShape s;
+  s.tx = 0;
+  if (items > kBnThreads) return s;
+  return bn_shape(n, items, kBnThreads, max_blocks);
+}
+static size_t bwd_row_lds(int c_in, int c_out, int tx) {
+  return ((size_t)c_in * 8 + 2 * (size_t)(kBnThreads / tx) * c_out) * sizeof(float);
 }
 
 // bytes of LDS for the staged column tables
@@ -745,10 +886,25 @@ int ssc_bnact_bwd_sums_f32(const float *x, const float *dy, int64_t n, int32_t c
   hipStream_t s = (hipStream_t)stream;
   if (n == 0) return fill_f32(sums, 2 * (int64_t)c_in, 0.f, s);
   const int V = ((c_in | c_out) & 3) == 0 ? 4 : 1;
-  BnShape sh = bn_shape(n, bwd_items(c_in, c_out, V));
+  BnShape sh = bwd_shape(n, c_out, V);
   float *partial = static_cast<float *>(workspace);
   ColAffine aff = {shift, scale, add, pre_bias};
-  if (V == 4)
+  const BnShape rs = bwd_row_shape(n, c_in, c_out, V, kBnMaxBlocks);
+  if (rs.tx > 0 && bwd_row_lds(c_in, c_out, rs.tx) <= 64 * 1024) {
+    // a row fits one pass: gate gradients from the products the group threads leave in LDS
+    const size_t lds_bytes = bwd_row_lds(c_in, c_out, rs.tx);
+    if (V == 4)
+      hipLaunchKernelGGL((bnact_bwd_row_kernel<4, false>), dim3(rs.blocks), dim3(kBnThreads),
+                         lds_bytes, s, x, dy, n, c_in, c_out, rs.tx, rs.rows_per_block, aff,
+                         out_mode, gate_col, gated_first, gated_dim, act_scalar, act_gate,
+                         (const float *)nullptr, (const float *)nullptr, (float *)nullptr, partial);
+    else
+      hipLaunchKernelGGL((bnact_bwd_row_kernel<1, false>), dim3(rs.blocks), dim3(kBnThreads),
+                         lds_bytes, s, x, dy, n, c_in, c_out, rs.tx, rs.rows_per_block, aff,
+                         out_mode, gate_col, gated_first, gated_dim, act_scalar, act_gate,
+                         (const float *)nullptr, (const float *)nullptr, (float *)nullptr, partial);
+    sh = rs;
+  } else if (V == 4)
     hipLaunchKernelGGL(bnact_bwd_partial_kernel<4>, dim3(sh.blocks), dim3(kBnThreads),
                        bn_tables_lds(c_in), s, x, dy,
                        n, c_in, c_out, sh.tx, sh.rows_per_block, aff, out_mode, gate_col,
@@ -778,9 +934,22 @@ int ssc_bnact_bwd_f32(const float *x, const float *dy, int64_t n, int32_t c_in, 
   if (n == 0) return SSC_OK;
   SSC_CHECK(x && dy && dx, SSC_EINVAL, "NULL pointer argument");
   const int V = ((c_in | c_out) & 3) == 0 ? 4 : 1;
-  BnShape sh = bn_shape(n, bwd_items(c_in, c_out, V));
+  BnShape sh = bwd_shape(n, c_out, V, kBnMaxApplyBlocks);
   ColAffine aff = {shift, scale, add, pre_bias};
-  if (V == 4)
+  const BnShape rs = bwd_row_shape(n, c_in, c_out, V, kBnMaxApplyBlocks);
+  if (rs.tx > 0 && bwd_row_lds(c_in, c_out, rs.tx) <= 64 * 1024) {
+    const size_t lds_bytes = bwd_row_lds(c_in, c_out, rs.tx);
+    if (V == 4)
+      hipLaunchKernelGGL((bnact_bwd_row_kernel<4, true>), dim3(rs.blocks), dim3(kBnThreads),
+                         lds_bytes, (hipStream_t)stream, x, dy, n, c_in, c_out, rs.tx,
+                         rs.rows_per_block, aff, out_mode, gate_col, gated_first, gated_dim,
+                         act_scalar, act_gate, dz_mean, coef, dx, (float *)nullptr);
+    else
+      hipLaunchKernelGGL((bnact_bwd_row_kernel<1, true>), dim3(rs.blocks), dim3(kBnThreads),
+                         lds_bytes, (hipStream_t)stream, x, dy, n, c_in, c_out, rs.tx,
+                         rs.rows_per_block, aff, out_mode, gate_col, gated_first, gated_dim,
+                         act_scalar, act_gate, dz_mean, coef, dx, (float *)nullptr);
+  } else if (V == 4)
     hipLaunchKernelGGL(bnact_bwd_kernel<4>, dim3(sh.blocks), dim3(kBnThreads),
                        bn_tables_lds(c_in), (hipStream_t)stream, x, dy, n, c_in, c_out, sh.tx, sh.rows_per_block, aff,
                        out_mode, gate_col, gated_first, gated_dim, act_scalar, act_gate, dz_mean,
