@@ -151,29 +151,64 @@ __global__ void __launch_bounds__(kSegRows * 64)
 // (src/pool/indice_maxpool_cuda_functor.cu:426-455: din[i] += dout[o] where in[i] == out[o];
 // src/pool/indice_avgpool_cuda_functor.cu: din[i] += dout[o] / (float)rf[o]).
 // table is [n_in, K] of output rows.  MODE 0 max, 1 average.
-template <int MODE>
+template <int MODE, int VEC>
 __global__ void __launch_bounds__(256)
     pool_bwd_kernel(const float *__restrict__ in, const float *__restrict__ out,
                     const float *__restrict__ dout, int C, const int32_t *__restrict__ table,
                     int K, const int32_t *__restrict__ rf, float *__restrict__ din, int64_t n_in) {
+  // VEC = 4 when C % 4 == 0 (16-byte accesses), else 1; per column the arithmetic and its
+  // order are those of the one-column form
+  const int cv = C / VEC;
   int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (idx >= n_in * C) return;
-  int64_t i = idx / C;
-  int c = (int)(idx - i * C);
+  if (idx >= n_in * cv) return;
+  int64_t i = idx / cv;
+  int c = (int)(idx - i * cv) * VEC;
   const int32_t *t = table + i * K;
-  float acc = 0.f;
-  float x = MODE == 0 ? in[idx] : 0.f;
+  float acc[VEC], x[VEC];
+#pragma unroll
+  for (int v = 0; v < VEC; ++v) {
+    acc[v] = 0.f;
+    x[v] = 0.f;
+  }
+  if (MODE == 0) {
+    if (VEC == 4) {
+      float4v q = *reinterpret_cast<const float4v *>(in + i * C + c);
+      x[0] = q.x; x[1 % VEC] = q.y; x[2 % VEC] = q.z; x[3 % VEC] = q.w;
+    } else {
+      x[0] = in[i * C + c];
+    }
+  }
   for (int k = 0; k < K; ++k) {
     int64_t o = t[k];
     if (o < 0) continue;
-    float g = dout[o * C + c];
-    if (MODE == 0) {
-      if (x == out[o * C + c]) acc = acc + g;
+    float g[VEC], y[VEC];
+    if (VEC == 4) {
+      float4v q = *reinterpret_cast<const float4v *>(dout + o * C + c);
+      g[0] = q.x; g[1 % VEC] = q.y; g[2 % VEC] = q.z; g[3 % VEC] = q.w;
+      if (MODE == 0) {
+        float4v p = *reinterpret_cast<const float4v *>(out + o * C + c);
+        y[0] = p.x; y[1 % VEC] = p.y; y[2 % VEC] = p.z; y[3 % VEC] = p.w;
+      }
     } else {
-      acc = acc + g / (float)rf[o];
+      g[0] = dout[o * C + c];
+      if (MODE == 0) y[0] = out[o * C + c];
+    }
+    const float div = MODE == 1 ? (float)rf[o] : 1.f;
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) {
+      if (MODE == 0) {
+        if (x[v] == y[v]) acc[v] = acc[v] + g[v];
+      } else {
+        acc[v] = acc[v] + g[v] / div;
+      }
     }
   }
-  din[idx] = acc;
+  if (VEC == 4) {
+    float4v q = {acc[0], acc[1 % VEC], acc[2 % VEC], acc[3 % VEC]};
+    *reinterpret_cast<float4v *>(din + i * C + c) = q;
+  } else {
+    din[i * C + c] = acc[0];
+  }
 }
 
 // Backward of the segment pools (src/pool/global_avgpool_cuda_kernel.cu:44-62,
@@ -357,15 +392,18 @@ static int pool_bwd(int mode, const float *features, const float *out_features,
                        dim3(256), 0, s, pairs, pair_stride, pair_num, K, 0, table);
     SSC_LAUNCH_CHECK("pair_table");
   }
-  const int64_t n = n_in * channels;
-  if (mode == 0)
-    hipLaunchKernelGGL((pool_bwd_kernel<0>), dim3((unsigned)ceil_div(n, 256)), dim3(256), 0, s,
-                       features, out_features, out_grad, channels, table, K, summaryrf, in_grad,
-                       n_in);
-  else
-    hipLaunchKernelGGL((pool_bwd_kernel<1>), dim3((unsigned)ceil_div(n, 256)), dim3(256), 0, s,
-                       features, out_features, out_grad, channels, table, K, summaryrf, in_grad,
-                       n_in);
+  const int vec = (channels & 3) == 0 ? 4 : 1;
+  const int64_t n = n_in * (channels / vec);
+  const dim3 grid((unsigned)ceil_div(n, 256));
+#define SSC_POOL_BWD(M, V)                                                                  \
+  hipLaunchKernelGGL((pool_bwd_kernel<M, V>), grid, dim3(256), 0, s, features, out_features, \
+                     out_grad, channels, table, K, summaryrf, in_grad, n_in)
+  if (mode == 0) {
+    if (vec == 4) SSC_POOL_BWD(0, 4); else SSC_POOL_BWD(0, 1);
+  } else {
+    if (vec == 4) SSC_POOL_BWD(1, 4); else SSC_POOL_BWD(1, 1);
+  }
+#undef SSC_POOL_BWD
   SSC_LAUNCH_CHECK("pool_bwd");
   return SSC_OK;
 }
