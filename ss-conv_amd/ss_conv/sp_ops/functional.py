@@ -149,7 +149,8 @@ class GlobalAvgPool(Function):
     def backward(ctx, d_output_feats):
         idx, proposals_offset, n_rows = ctx.for_backwards
         n_seg, c = d_output_feats.size()
-        d_feats = torch.zeros((n_rows, c), dtype=torch.float32, device=d_output_feats.device)
+        # every row is written by the kernel (zero outside the segments): no zero fill first
+        d_feats = torch.empty((n_rows, c), dtype=torch.float32, device=d_output_feats.device)
         _ext.global_avgpool_bp(d_feats, proposals_offset, idx, d_output_feats.contiguous(), n_seg, c)
         return d_feats, None
 

@@ -730,6 +730,36 @@ def test_segment_voxel_interp_backward(oracle, device):
     assert rel_l2(x.grad.cpu().numpy(), oracle.three_interp_bwd(gq, idx3, w3, m)) < REL_L2
 
 
+def test_point2voxel_passes_gradients_to_the_point_features(device):
+    """Voxel means are differentiable in the point features (the reference keeps them in the
+    autograd graph through its boolean-mask indexing, voxelize.py:60-83, and voxelize_bp):
+    a point inside the grid receives gv[its voxel] / (points in the voxel), a dropped one 0."""
+    from ss_conv.sp_ops.voxelize import Point2Voxel
+    pts, feats, ids = synth.make_clouds(3, 400, seed=8, channels=5)
+    pts = pts * 1.2  # part of every cloud falls outside
+    grid = 8
+    unit = np.float32(2.0 / grid)
+    x = torch.from_numpy(feats).to(device).requires_grad_(True)
+    vp, st, vi, _ = Point2Voxel([grid] * 3, [2.0 / grid] * 3)(
+        torch.from_numpy(pts).to(device), x, torch.from_numpy(ids).to(device))
+    gv = torch.randn_like(st.features)
+    st.features.backward(gv)
+    half = np.float32(0.5) * (np.float32(grid) * unit)
+    inside = (np.abs(pts) > half).sum(1) == 0
+    assert inside.sum() == vp.shape[0] and 0 < inside.sum() < len(ids)
+    cells = ((pts[inside] + half) / unit).astype(np.int32)
+    keys = ((ids[inside] * (grid + 1) + cells[:, 0]) * (grid + 1) + cells[:, 1]) * (grid + 1) + cells[:, 2]
+    vox = st.indices.cpu().numpy().astype(np.int64)
+    vkeys = ((vox[:, 0] * (grid + 1) + vox[:, 1]) * (grid + 1) + vox[:, 2]) * (grid + 1) + vox[:, 3]
+    inv = np.searchsorted(vkeys, keys)
+    assert np.array_equal(vkeys[inv], keys)
+    counts = np.bincount(inv, minlength=len(vkeys)).astype(np.float32)
+    want = np.zeros_like(feats)
+    want[inside] = gv.cpu().numpy()[inv] / counts[inv][:, None]
+    assert x.grad is not None
+    assert rel_l2(x.grad.cpu().numpy(), want) < 1e-6
+
+
 def test_downsampling_block(oracle, device):
     """Strided convolution followed by MaxPool and AvgPool (k=2, s=2)."""
     import torch.nn.functional as F
