@@ -366,6 +366,23 @@ size_t ssc_three_nn_workspace_bytes(int32_t m);
 int ssc_three_nn_ws(int32_t n, int32_t m, const float *unknown, const float *known, float *dist2,
                     int32_t *idx, void *workspace, size_t workspace_bytes, ssc_stream_t stream);
 
+/* The same search when the known rows are voxel centres: known[j] is the centre of voxel
+ * voxel_indices[j] = (b, x, y, z) of a grid of dims[3] cells per batch element, i.e.
+ * known[j] = (b, origin + (xyz + 0.5) * unit) up to rounding (what Voxel2Point computes,
+ * ss_conv/sp_ops/voxelize.py:131-140).  The neighbours are looked up around the query's own
+ * cell through an occupancy bit table instead of among all m rows; distances, indices and
+ * ties are those of ssc_three_nn.  The voxel rows must be distinct.  A query far from every
+ * voxel is scanned against all rows; many such queries, a query with a batch value outside
+ * 0 .. batch_size-1 or a voxel row outside the grid make the call fall back to the plain
+ * scan by itself. */
+size_t ssc_three_nn_grid_workspace_bytes(int32_t n, int32_t m, int32_t batch_size,
+                                         const int32_t dims[3]);
+int ssc_three_nn_grid(int32_t n, int32_t m, const float *unknown /* [n,4] */,
+                      const float *known /* [m,4] */, const int32_t *voxel_indices /* [m,4] */,
+                      int32_t batch_size, const int32_t dims[3], const float origin[3],
+                      const float unit[3], float *dist2 /* [n,3] */, int32_t *idx /* [n,3] */,
+                      void *workspace, size_t workspace_bytes, ssc_stream_t stream);
+
 int ssc_three_interp_f32(int32_t c, int32_t m, int32_t n, const float *feats /* [m,c] */,
                          const int32_t *idx /* [n,3] */, const float *weight /* [n,3] */,
                          float *out /* [n,c] */, ssc_stream_t stream);

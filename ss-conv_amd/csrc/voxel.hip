@@ -148,7 +148,10 @@ struct Best3 {
 __global__ void __launch_bounds__(kNnTile)
     three_nn_kernel(int n, int m, const float *__restrict__ unknown,
                     const float *__restrict__ known, const float *__restrict__ tile_range,
-                    float *__restrict__ dist2, int32_t *__restrict__ idx) {
+                    float *__restrict__ dist2, int32_t *__restrict__ idx,
+                    const int32_t *__restrict__ only_if, int only_above) {
+  // (a condition on a device-side counter, the same for every thread of the grid)
+  if (only_if && only_if[0] <= only_above) return;
   __shared__ float4v tile[kNnTile];
   __shared__ float red[2][kNnTile / 64];
   const int q = blockIdx.x * (kNnTile / kNnLanes) + threadIdx.x / kNnLanes;
@@ -296,7 +299,8 @@ int ssc_three_nn(int32_t n, int32_t m, const float *unknown, const float *known,
   if (n == 0) return SSC_OK;
   SSC_CHECK(unknown && dist2 && idx && (m == 0 || known), SSC_EINVAL, "NULL pointer argument");
   hipLaunchKernelGGL(three_nn_kernel, dim3((unsigned)ceil_div(n, kNnTile / kNnLanes)), dim3(kNnTile), 0,
-                     (hipStream_t)stream, n, m, unknown, known, (const float *)nullptr, dist2, idx);
+                     (hipStream_t)stream, n, m, unknown, known, (const float *)nullptr, dist2, idx,
+                     (const int32_t *)nullptr, 0);
   SSC_LAUNCH_CHECK("three_nn");
   return SSC_OK;
 }
@@ -320,7 +324,314 @@ int ssc_three_nn_ws(int32_t n, int32_t m, const float *unknown, const float *kno
     SSC_LAUNCH_CHECK("nn_tile_range");
   }
   hipLaunchKernelGGL(three_nn_kernel, dim3((unsigned)ceil_div(n, kNnTile / kNnLanes)), dim3(kNnTile), 0,
-                     (hipStream_t)stream, n, m, unknown, known, tile_range, dist2, idx);
+                     (hipStream_t)stream, n, m, unknown, known, tile_range, dist2, idx,
+                     (const int32_t *)nullptr, 0);
+  SSC_LAUNCH_CHECK("three_nn");
+  return SSC_OK;
+}
+
+}  // extern "C"
+
+// ---- 3-NN among voxel centres by grid search ----------------------------------------------
+// When the known rows are the centres of voxels whose integer coordinates are at hand, a
+// query's neighbours are found around its own cell instead of among all rows: a bit table
+// over the cells says which are occupied, the rank of a set bit gives the voxel's row
+// (through rank2row, so the rows need not be in key order), and cells are visited in shells
+// of growing Chebyshev distance r.  After shell r every cell not yet visited differs from
+// the query's cell by more than r in some axis, so its centre is at least `bound` away
+// (the distance to the nearest unvisited layer of centres); once the third best distance
+// is below that bound the result is final.  Distances are computed from the same operands
+// by the same expression as the plain scan and candidates are ranked by (distance, row):
+// the result is the plain scan's, ties included.  A query that does not settle within
+// kGridNnMaxShell shells (a far-away point, a nearly empty cloud) is put on a list and
+// scanned against all rows by a wave of a second kernel; when more than an eighth of the
+// queries end up there the plain scan, launched behind with the list's length as its
+// condition, redoes the call instead.  The voxel rows must be distinct; a voxel row outside
+// the grid, or a query whose batch value is not one of 0 .. batch-1, sends the call to the
+// plain scan as well.
+namespace ssc {
+
+constexpr int kGridNnMaxShell = 3;
+
+struct GridNn {
+  int batch, dim[3];
+  float origin[3], unit[3];
+};
+
+__device__ __forceinline__ bool nng_inside(const int4 &r, const GridNn &g) {
+  return r.x >= 0 && r.x < g.batch && r.y >= 0 && r.y < g.dim[0] && r.z >= 0 && r.z < g.dim[1] &&
+         r.w >= 0 && r.w < g.dim[2];
+}
+
+__global__ void __launch_bounds__(256)
+    nng_mark_kernel(const int32_t *__restrict__ coords, int m, GridNn g,
+                    uint32_t *__restrict__ bits, int32_t *__restrict__ unsettled) {
+  const int j = blockIdx.x * blockDim.x + threadIdx.x;
+  if (j >= m) return;
+  const int4 r = reinterpret_cast<const int4 *>(coords)[j];
+  if (!nng_inside(r, g)) {  // a voxel the table cannot hold: only the plain scan sees it
+    atomicOr(unsettled, 1 << 30);
+    return;
+  }
+  const uint32_t key = (uint32_t)(((r.x * g.dim[0] + r.y) * g.dim[1] + r.z) * g.dim[2] + r.w);
+  atomicOr(&bits[key >> 5], 1u << (key & 31u));
+}
+
+__global__ void __launch_bounds__(256)
+    nng_rank2row_kernel(const int32_t *__restrict__ coords, int m, GridNn g,
+                        const uint32_t *__restrict__ bits, const int32_t *__restrict__ prefix,
+                        int32_t *__restrict__ rank2row) {
+  const int j = blockIdx.x * blockDim.x + threadIdx.x;
+  if (j >= m) return;
+  const int4 r = reinterpret_cast<const int4 *>(coords)[j];
+  if (!nng_inside(r, g)) return;
+  const uint32_t key = (uint32_t)(((r.x * g.dim[0] + r.y) * g.dim[1] + r.z) * g.dim[2] + r.w);
+  rank2row[bit_rank(bits, prefix, key)] = j;
+}
+
+// Eight lanes per query share the columns (x, y) of a shell; their candidates are merged
+// after every shell (an all-to-all exchange, so each lane knows the query's three best and
+// takes the same decision).  A query that has not settled after the last shell is appended
+// to `list`; `counter` counts them (and is forced far above n by nng_mark_kernel or by a
+// query with an impossible batch value, which sends the whole call to the plain scan).
+constexpr int kGridNnLanes = 8;
+constexpr int kGridNnAll = 1 << 30;  // counter value that means "redo every query"
+
+__device__ __forceinline__ void nng_merge_lanes(Best3 &b) {
+#pragma unroll
+  for (int d = 1; d < kGridNnLanes; d <<= 1) {
+    const float o1 = __shfl_xor(b.b1, d, 64), o2 = __shfl_xor(b.b2, d, 64),
+                o3 = __shfl_xor(b.b3, d, 64);
+    const int j1 = __shfl_xor(b.i1, d, 64), j2 = __shfl_xor(b.i2, d, 64),
+              j3 = __shfl_xor(b.i3, d, 64);
+    if (o1 < INFINITY) b.insert(o1, j1);
+    if (o2 < INFINITY) b.insert(o2, j2);
+    if (o3 < INFINITY) b.insert(o3, j3);
+  }
+}
+
+__global__ void __launch_bounds__(256)
+    three_nn_grid_kernel(int n, int m, const float *__restrict__ unknown,
+                         const float *__restrict__ known, GridNn g,
+                         const uint32_t *__restrict__ bits, const int32_t *__restrict__ prefix,
+                         const int32_t *__restrict__ rank2row, float *__restrict__ dist2,
+                         int32_t *__restrict__ idx, int32_t *__restrict__ counter,
+                         int32_t *__restrict__ list) {
+  const int q = blockIdx.x * (256 / kGridNnLanes) + threadIdx.x / kGridNnLanes;
+  const int sub = threadIdx.x % kGridNnLanes;
+  const bool live = q < n;  // dead groups run along (the shuffles want every lane)
+  float4v u = {-1.f, 0.f, 0.f, 0.f};
+  if (live) u = reinterpret_cast<const float4v *>(unknown)[q];
+  const Best3 none = {INFINITY, INFINITY, INFINITY, 0, 0, 0};
+  Best3 acc = none;  // the query's three best so far, the same in its eight lanes
+  const float pos[3] = {u.y, u.z, u.w};
+  const int b = (int)u.x;
+  const bool batch_ok = (float)b == u.x && b >= 0 && b < g.batch;
+  bool settled = !live;
+  if (live && !batch_ok) {
+    if (sub == 0) atomicOr(counter, kGridNnAll);
+    settled = true;
+  }
+  int c[3] = {0, 0, 0};
+#pragma unroll
+  for (int a = 0; a < 3; ++a) {
+    const int v = (int)floorf((pos[a] - g.origin[a]) / g.unit[a]);
+    c[a] = v < 0 ? 0 : (v >= g.dim[a] ? g.dim[a] - 1 : v);
+  }
+  for (int r = 0; r <= kGridNnMaxShell; ++r) {
+    Best3 cur = none;
+    if (!settled) {
+      const int x0 = max(c[0] - r, 0), x1 = min(c[0] + r, g.dim[0] - 1);
+      const int y0 = max(c[1] - r, 0), y1 = min(c[1] + r, g.dim[1] - 1);
+      const int z0 = max(c[2] - r, 0), z1 = min(c[2] + r, g.dim[2] - 1);
+      const int ny = y1 - y0 + 1, ncol = (x1 - x0 + 1) * ny;
+      for (int col = sub; col < ncol; col += kGridNnLanes) {
+        const int x = x0 + col / ny, y = y0 + col % ny;
+        // cells of the shell only: in the interior of the box just the two end cells in z
+        const bool face = abs(x - c[0]) == r || abs(y - c[1]) == r;
+        const uint32_t base = (uint32_t)(((b * g.dim[0] + x) * g.dim[1] + y) * g.dim[2]);
+        uint32_t wi = 0xFFFFFFFFu, w = 0u;
+        int wp = 0;
+        for (int z = z0; z <= z1; ++z) {
+          if (!face && abs(z - c[2]) != r) continue;
+          const uint32_t key = base + (uint32_t)z;
+          if ((key >> 5) != wi) {
+            wi = key >> 5;
+            w = bits[wi];
+            wp = w ? prefix[wi] : 0;
+          }
+          if ((w >> (key & 31u)) & 1u) {
+            const int row = rank2row[wp + __popc(w & ((1u << (key & 31u)) - 1u))];
+            const float4v p = reinterpret_cast<const float4v *>(known)[row];
+            if (p.x == u.x) {
+              const float dx = u.y - p.y, dy = u.z - p.z, dz = u.w - p.w;
+              const float xx = dx * dx, yy = dy * dy, zz = dz * dz;
+              cur.insert((xx + yy) + zz, row);
+            }
+          }
+        }
+      }
+    }
+    nng_merge_lanes(cur);
+    if (!settled) {
+      if (cur.b1 < INFINITY) acc.insert(cur.b1, cur.i1);
+      if (cur.b2 < INFINITY) acc.insert(cur.b2, cur.i2);
+      if (cur.b3 < INFINITY) acc.insert(cur.b3, cur.i3);
+      // distance to the nearest layer of centres that has not been visited
+      float bound = INFINITY;
+#pragma unroll
+      for (int a = 0; a < 3; ++a) {
+        if (c[a] - r - 1 >= 0)
+          bound = fminf(bound, pos[a] - (g.origin[a] + ((float)(c[a] - r) - 0.5f) * g.unit[a]));
+        if (c[a] + r + 1 <= g.dim[a] - 1)
+          bound = fminf(bound, (g.origin[a] + ((float)(c[a] + r) + 1.5f) * g.unit[a]) - pos[a]);
+      }
+      if (bound == INFINITY) {
+        settled = true;  // the whole grid of this batch element has been visited
+      } else if (bound > 0.f && acc.b3 < bound * bound * 0.9999f) {
+        settled = true;
+      } else if (r == kGridNnMaxShell && sub == 0) {
+        const int at = atomicAdd(counter, 1);
+        if (at >= 0 && at < n) list[at] = q;
+      }
+    }
+  }
+  if (live && sub == 0) {
+    dist2[q * 3] = acc.b1; dist2[q * 3 + 1] = acc.b2; dist2[q * 3 + 2] = acc.b3;
+    idx[q * 3] = acc.i1; idx[q * 3 + 1] = acc.i2; idx[q * 3 + 2] = acc.i3;
+  }
+}
+
+// The queries the grid search left open, one workgroup each: all rows, 256 at a time with
+// four loads in flight per thread, then the threads' candidates merged through LDS.
+// (Nothing to do when the counter says that the plain scan redoes the call.)
+__global__ void __launch_bounds__(256)
+    three_nn_list_kernel(int n, int m, const float *__restrict__ unknown,
+                         const float *__restrict__ known, const int32_t *__restrict__ counter,
+                         const int32_t *__restrict__ list, int redo_above,
+                         float *__restrict__ dist2, int32_t *__restrict__ idx) {
+  __shared__ float sd[4][3];
+  __shared__ int si[4][3];
+  const int count = counter[0];
+  if (count <= 0 || count > redo_above) return;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  for (int e = blockIdx.x; e < count; e += gridDim.x) {
+    const int q = list[e];
+    const float4v u = reinterpret_cast<const float4v *>(unknown)[q];
+    Best3 best = {INFINITY, INFINITY, INFINITY, 0, 0, 0};
+    auto consider = [&](const float4v &p, int row) {
+      if (p.x != u.x) return;
+      const float dx = u.y - p.y, dy = u.z - p.z, dz = u.w - p.w;
+      const float xx = dx * dx, yy = dy * dy, zz = dz * dz;
+      best.insert((xx + yy) + zz, row);
+    };
+    int row = threadIdx.x;
+    for (; row + 3 * 256 < m; row += 4 * 256) {
+      float4v p[4];
+#pragma unroll
+      for (int k = 0; k < 4; ++k) p[k] = reinterpret_cast<const float4v *>(known)[row + k * 256];
+#pragma unroll
+      for (int k = 0; k < 4; ++k) consider(p[k], row + k * 256);
+    }
+    for (; row < m; row += 256) consider(reinterpret_cast<const float4v *>(known)[row], row);
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const float o1 = __shfl_xor(best.b1, d, 64), o2 = __shfl_xor(best.b2, d, 64),
+                  o3 = __shfl_xor(best.b3, d, 64);
+      const int j1 = __shfl_xor(best.i1, d, 64), j2 = __shfl_xor(best.i2, d, 64),
+                j3 = __shfl_xor(best.i3, d, 64);
+      if (o1 < INFINITY) best.insert(o1, j1);
+      if (o2 < INFINITY) best.insert(o2, j2);
+      if (o3 < INFINITY) best.insert(o3, j3);
+    }
+    if (lane == 0) {
+      sd[wave][0] = best.b1; sd[wave][1] = best.b2; sd[wave][2] = best.b3;
+      si[wave][0] = best.i1; si[wave][1] = best.i2; si[wave][2] = best.i3;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      for (int w = 1; w < 4; ++w)
+        for (int k = 0; k < 3; ++k)
+          if (sd[w][k] < INFINITY) best.insert(sd[w][k], si[w][k]);
+      dist2[q * 3] = best.b1; dist2[q * 3 + 1] = best.b2; dist2[q * 3 + 2] = best.b3;
+      idx[q * 3] = best.i1; idx[q * 3 + 1] = best.i2; idx[q * 3 + 2] = best.i3;
+    }
+    __syncthreads();
+  }
+}
+
+static int64_t nng_cells(int32_t batch, const int32_t *dims) {
+  if (batch < 1 || !dims || dims[0] < 1 || dims[1] < 1 || dims[2] < 1) return -1;
+  const int64_t cells = (int64_t)batch * dims[0] * dims[1] * dims[2];
+  return cells < ((int64_t)1 << 31) ? cells : -1;
+}
+
+}  // namespace ssc
+
+extern "C" {
+
+size_t ssc_three_nn_grid_workspace_bytes(int32_t n, int32_t m, int32_t batch_size,
+                                         const int32_t dims[3]) {
+  const int64_t cells = nng_cells(batch_size, dims);
+  if (cells < 0 || m < 0 || n < 0) return 0;
+  return bit_table_bytes(cells) + align_up((size_t)(m > 0 ? m : 1) * sizeof(int32_t)) +
+         align_up((size_t)(n > 0 ? n : 1) * sizeof(int32_t));
+}
+
+int ssc_three_nn_grid(int32_t n, int32_t m, const float *unknown, const float *known,
+                      const int32_t *voxel_indices, int32_t batch_size, const int32_t dims[3],
+                      const float origin[3], const float unit[3], float *dist2, int32_t *idx,
+                      void *workspace, size_t workspace_bytes, ssc_stream_t stream) {
+  SSC_CHECK(n >= 0 && m >= 0, SSC_EINVAL, "bad sizes");
+  const int64_t cells = nng_cells(batch_size, dims);
+  SSC_CHECK(cells > 0, SSC_EINVAL, "batch_size * prod(dims) must be positive and below 2^31");
+  SSC_CHECK(origin && unit && unit[0] > 0.f && unit[1] > 0.f && unit[2] > 0.f, SSC_EINVAL,
+            "voxel extents must be positive");
+  if (n == 0) return SSC_OK;
+  SSC_CHECK(unknown && dist2 && idx && (m == 0 || (known && voxel_indices)), SSC_EINVAL,
+            "NULL pointer argument");
+  SSC_CHECK(workspace != nullptr &&
+                workspace_bytes >= ssc_three_nn_grid_workspace_bytes(n, m, batch_size, dims),
+            SSC_EWORKSPACE, "three_nn_grid workspace too small");
+  hipStream_t s = (hipStream_t)stream;
+  GridNn g;
+  g.batch = batch_size;
+  for (int a = 0; a < 3; ++a) {
+    g.dim[a] = dims[a];
+    g.origin[a] = origin[a];
+    g.unit[a] = unit[a];
+  }
+  Carver c(workspace);
+  BitTable t = bit_table_carve(c, cells);
+  int32_t *rank2row = c.take<int32_t>((size_t)(m > 0 ? m : 1));
+  int32_t *list = c.take<int32_t>((size_t)n);
+  // t.total[1] is cleared with the table and not used by the scan: the counter of the
+  // queries left open
+  int32_t *counter = t.total + 1;
+  int rc;
+  if ((rc = bit_table_clear(t, s)) != SSC_OK) return rc;
+  if (m > 0) {
+    hipLaunchKernelGGL(nng_mark_kernel, dim3((unsigned)ceil_div(m, 256)), dim3(256), 0, s,
+                       voxel_indices, m, g, t.bits, counter);
+    SSC_LAUNCH_CHECK("nng_mark");
+  }
+  if ((rc = bit_table_scan(t, s)) != SSC_OK) return rc;
+  if (m > 0) {
+    hipLaunchKernelGGL(nng_rank2row_kernel, dim3((unsigned)ceil_div(m, 256)), dim3(256), 0, s,
+                       voxel_indices, m, g, t.bits, t.prefix, rank2row);
+    SSC_LAUNCH_CHECK("nng_rank2row");
+  }
+  hipLaunchKernelGGL(three_nn_grid_kernel, dim3((unsigned)ceil_div(n, 256 / kGridNnLanes)),
+                     dim3(256), 0, s, n, m, unknown, known, g, t.bits, t.prefix, rank2row, dist2,
+                     idx, counter, list);
+  SSC_LAUNCH_CHECK("three_nn_grid");
+  const int redo_above = n / 8;
+  hipLaunchKernelGGL(three_nn_list_kernel, dim3(512), dim3(256), 0, s, n, m, unknown, known,
+                     counter, list, redo_above, dist2, idx);
+  SSC_LAUNCH_CHECK("three_nn_list");
+  hipLaunchKernelGGL(three_nn_kernel, dim3((unsigned)ceil_div(n, kNnTile / kNnLanes)), dim3(kNnTile),
+                     0, s, n, m, unknown, known, (const float *)nullptr, dist2, idx,
+                     (const int32_t *)counter, redo_above);
   SSC_LAUNCH_CHECK("three_nn");
   return SSC_OK;
 }

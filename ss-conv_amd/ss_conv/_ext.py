@@ -91,6 +91,10 @@ _SIGNATURES = {
     "ssc_three_nn": (ctypes.c_int, [_i32, _i32, _vp, _vp, _vp, _vp, _vp]),
     "ssc_three_nn_workspace_bytes": (_sz, [_i32]),
     "ssc_three_nn_ws": (ctypes.c_int, [_i32, _i32, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
+    "ssc_three_nn_grid_workspace_bytes": (_sz, [_i32, _i32, _i32, ctypes.POINTER(_i32)]),
+    "ssc_three_nn_grid": (ctypes.c_int, [_i32, _i32, _vp, _vp, _vp, _i32, ctypes.POINTER(_i32),
+                                         ctypes.POINTER(ctypes.c_float),
+                                         ctypes.POINTER(ctypes.c_float), _vp, _vp, _vp, _sz, _vp]),
     "ssc_three_interp_f32": (ctypes.c_int, [_i32, _i32, _i32, _vp, _vp, _vp, _vp, _vp]),
     "ssc_bn_workspace_bytes": (_sz, [_i64, _i32]),
     "ssc_bn_prepare_f32": (ctypes.c_int, [_vp, _i64, _i32, _vp, _vp, _vp, _vp, _i32, _i32,
@@ -503,6 +507,35 @@ def three_nn(n, m, unknown, known, dist2, idx):
     ws = _workspace(_lib.ssc_three_nn_workspace_bytes(int(m)), unknown.device)
     _check(_lib.ssc_three_nn_ws(int(n), int(m), _ptr(unknown), _ptr(known), _ptr(dist2), _ptr(idx),
                                 ws.data_ptr(), ws.numel(), _stream(unknown)))
+
+
+def three_nn_grid(unknown, known, voxel_indices, batch_size, dims, origin, unit):
+    """three_nn for known rows that are the centres of the voxels `voxel_indices` (int32
+    [m, 4], distinct, inside a grid of `dims` cells per batch element with cell size `unit`
+    and lower corner `origin`): same result, found around each query's own cell.
+    Returns (dist2 [n, 3] float32, idx [n, 3] int32)."""
+    _need_gpu(unknown, known, voxel_indices)
+    if unknown.dtype != torch.float32 or known.dtype != torch.float32 or \
+            voxel_indices.dtype != torch.int32:
+        raise RuntimeError("three_nn_grid: wrong dtypes")
+    if not (unknown.is_contiguous() and known.is_contiguous() and voxel_indices.is_contiguous()):
+        raise RuntimeError("three_nn_grid: tensors must be contiguous")
+    n, m = unknown.size(0), known.size(0)
+    if voxel_indices.size(0) != m:
+        raise RuntimeError("three_nn_grid: one voxel row per known row")
+    d = (_i32 * 3)(*[int(v) for v in dims])
+    o = (ctypes.c_float * 3)(*[float(v) for v in origin])
+    u = (ctypes.c_float * 3)(*[float(v) for v in unit])
+    nbytes = _lib.ssc_three_nn_grid_workspace_bytes(n, m, int(batch_size), d)
+    if nbytes == 0:
+        raise RuntimeError("three_nn_grid: batch_size * prod(dims) must be positive and below 2^31")
+    ws = _workspace(nbytes, unknown.device)
+    dist2 = torch.empty((n, 3), dtype=torch.float32, device=unknown.device)
+    idx = torch.empty((n, 3), dtype=torch.int32, device=unknown.device)
+    _check(_lib.ssc_three_nn_grid(n, m, _ptr(unknown), _ptr(known), _ptr(voxel_indices),
+                                  int(batch_size), d, o, u, _ptr(dist2), _ptr(idx), ws.data_ptr(),
+                                  ws.numel(), _stream(unknown)))
+    return dist2, idx
 
 
 def three_interpolate_fp(c, m, n, feats, idx, weight, out):

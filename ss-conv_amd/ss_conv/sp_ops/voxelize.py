@@ -137,7 +137,7 @@ class Voxel2Point(nn.Module):
         if point_cloud is not None:
             assert batch_ids is not None
             points = torch.cat([batch_ids.float().unsqueeze(1), point_cloud], dim=1)
-            return self._get_point_feats(points.contiguous(), vx_points, vx_feats)
+            return self._get_point_feats(points.contiguous(), vx_points, vx_feats, sparse_feat)
         return vx_points[:, 1:].contiguous(), vx_feats, vx_points[:, 0].contiguous()
 
     def _get_vertice_feats(self, sparse_tensor):
@@ -161,8 +161,33 @@ class Voxel2Point(nn.Module):
         centres[:, 1:] = centres[:, 1:] * unit - 0.5 * extent + 0.5 * unit
         return centres.contiguous().detach(), feat
 
-    def _get_point_feats(self, target_points, query_points, query_feats):
-        dist, idx = three_nn(target_points, query_points)
+    def _grid(self, sparse_tensor):
+        """(unit, origin) of the voxel grid as float32 host arrays: the numbers the centres
+        were computed from in _get_vertice_feats."""
+        shape = np.asarray(sparse_tensor.spatial_shape, dtype=np.float64)
+        if self.voxel_extent is not None:
+            unit, extent = self.voxel_extent / shape, self.voxel_extent
+        else:
+            unit, extent = self.unit_voxel_extent, self.unit_voxel_extent * shape
+        unit = unit.astype(np.float32)
+        extent = np.asarray(extent, dtype=np.float64).astype(np.float32)
+        return unit, np.float32(-0.5) * extent
+
+    def _get_point_feats(self, target_points, query_points, query_feats, sparse_tensor=None):
+        indices = None if sparse_tensor is None else sparse_tensor.indices
+        if indices is not None and target_points.is_cuda and indices.dtype == torch.int32 \
+                and target_points.dtype == torch.float32:
+            # the known points are voxel centres: search around each point's own cell
+            unit, origin = self._grid(sparse_tensor)
+            dist2, idx = _ext.three_nn_grid(target_points, query_points, indices.contiguous(),
+                                            sparse_tensor.batch_size,
+                                            # (a point on the upper face of the grid has
+                                            # voxel index == shape, voxelize.py:85-86)
+                                            [int(v) + 1 for v in sparse_tensor.spatial_shape],
+                                            origin, unit)
+            dist = torch.sqrt(dist2)
+        else:
+            dist, idx = three_nn(target_points, query_points)
         dist_recip = 1.0 / (dist + 1e-8)
         norm = torch.sum(dist_recip, dim=1, keepdim=True)
         weight = dist_recip / norm

@@ -477,6 +477,52 @@ def test_point_voxel_random_configurations(seed, oracle, device):
         assert np.array_equal(dist.cpu().numpy(), odist), case
 
 
+@pytest.mark.parametrize("seed", [1, 2, 3])
+def test_three_nn_grid_equals_plain_scan(seed, device):
+    """The grid search among voxel centres returns the plain scan's distances and indices,
+    ties included: dense and nearly empty grids, anisotropic cells, voxel rows in arbitrary
+    order, queries inside, on cell faces, outside the grid and in batch elements without
+    voxels (the last kinds make the call fall back to the plain scan)."""
+    from ss_conv import _ext
+    rng = np.random.default_rng(seed)
+    for case in range(25):
+        batch = int(rng.integers(1, 5))
+        dims = [int(rng.integers(1, 20)) for _ in range(3)]
+        unit = np.array([float(rng.choice([0.05, 0.1, 0.3, 1.0])) for _ in range(3)], np.float32)
+        origin = (np.float32(-0.5) * (unit * np.array(dims, np.float32))).astype(np.float32)
+        cells = batch * dims[0] * dims[1] * dims[2]
+        fill = float(rng.choice([0.002, 0.05, 0.5, 1.0]))
+        m = max(1, min(cells, int(cells * fill)))
+        flat = rng.choice(cells, size=m, replace=False)
+        if rng.integers(0, 2):
+            flat.sort()
+        vol = dims[0] * dims[1] * dims[2]
+        b, r = flat // vol, flat % vol
+        vox = np.stack([b, r // (dims[1] * dims[2]), (r // dims[2]) % dims[1], r % dims[2]],
+                       1).astype(np.int32)
+        centres = np.concatenate([vox[:, :1].astype(np.float32),
+                                  vox[:, 1:].astype(np.float32) * unit + origin
+                                  + np.float32(0.5) * unit], 1).astype(np.float32)
+        n = int(rng.integers(1, 600))
+        extent = unit * np.array(dims, np.float32)
+        pts = (rng.uniform(-0.5, 0.5, size=(n, 3)) * extent * float(rng.choice([1.0, 1.0, 2.5])))
+        pts = pts.astype(np.float32)
+        on_face = rng.integers(0, 6, size=n) == 0
+        pts[on_face] = (np.round(pts[on_face] / unit) * unit).astype(np.float32)
+        exact = rng.integers(0, 6, size=n) == 0   # exactly on a centre: ties between neighbours
+        pts[exact] = centres[rng.integers(0, m, size=int(exact.sum())), 1:]
+        qb = rng.integers(0, batch + 1, size=n).astype(np.float32)  # batch + 1: no such element
+        unknown = np.concatenate([qb[:, None], pts], 1).astype(np.float32)
+        print("case", case, batch, dims, unit.tolist(), m, n, flush=True)
+        u_t, k_t, v_t = [torch.from_numpy(a).to(device) for a in (unknown, centres, vox)]
+        d_grid, i_grid = _ext.three_nn_grid(u_t, k_t, v_t, batch, dims, origin, unit)
+        d_ref = torch.empty((n, 3), dtype=torch.float32, device=device)
+        i_ref = torch.empty((n, 3), dtype=torch.int32, device=device)
+        _ext.three_nn(n, m, u_t, k_t, d_ref, i_ref)
+        assert torch.equal(d_grid, d_ref), case
+        assert torch.equal(i_grid, i_ref), case
+
+
 def test_voxel2point_matches_oracle(oracle, device):
     from ss_conv.sp_ops.voxelize import Point2Voxel, Voxel2Point
     pts, feats, ids = synth.make_clouds(3, 500, seed=6, channels=10)
