@@ -330,7 +330,9 @@ int ssc_unique_emit(const int32_t *coords, int64_t n, const int32_t dims[4], voi
  * ssc_p2v_compact (same workspace, untouched in between) writes the m = sum(hist_valid)
  *   + #{id: hist_all > 0, hist_valid == 0} rows of the result: points [m,3], features
  *   [m,channels], ids [m], and the voxel coordinates (b, vx, vy, vz) of every row as
- *   ssc_voxel_coords computes them. */
+ *   ssc_voxel_coords computes them; out_dest [n] (may be NULL) receives the output row of
+ *   every input row, -1 for a dropped one (what a caller needs to send gradients of the
+ *   output features back to the input features). */
 #define SSC_P2V_MAX_IDS 4096
 size_t ssc_p2v_workspace_bytes(int64_t n);
 int ssc_p2v_scan(const float *points /* [n,3] */, const int64_t *batch_ids /* [n] */, int64_t n,
@@ -343,7 +345,8 @@ int ssc_p2v_compact(const float *points, const float *feats /* [n,channels] */,
                     const float half_extent[3], const float unit[3], void *workspace,
                     size_t workspace_bytes, float *out_points /* [m,3] */,
                     float *out_feats /* [m,channels] */, int64_t *out_ids /* [m] */,
-                    int32_t *out_coords /* [m,4] */, ssc_stream_t stream);
+                    int32_t *out_coords /* [m,4] */, int32_t *out_dest /* [n] or NULL */,
+                    ssc_stream_t stream);
 
 int ssc_voxel_map(const int32_t *inverse /* [n] */, const int32_t *ids /* [n] */,
                   int32_t *out_maps /* [m,max_active+1] */, int32_t n_point, int32_t n_voxel,

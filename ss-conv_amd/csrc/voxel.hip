@@ -854,7 +854,8 @@ int ssc_p2v_scan(const float *points, const int64_t *batch_ids, int64_t n,
 int ssc_p2v_compact(const float *points, const float *feats, const int64_t *batch_ids, int64_t n,
                     int32_t channels, const float half_extent[3], const float unit[3],
                     void *workspace, size_t workspace_bytes, float *out_points, float *out_feats,
-                    int64_t *out_ids, int32_t *out_coords, ssc_stream_t stream) {
+                    int64_t *out_ids, int32_t *out_coords, int32_t *out_dest,
+                    ssc_stream_t stream) {
   SSC_CHECK(n > 0 && channels >= 1, SSC_EINVAL, "bad sizes");
   SSC_CHECK(points && feats && batch_ids && half_extent && unit && workspace && out_points &&
                 out_feats && out_ids && out_coords,
@@ -864,14 +865,16 @@ int ssc_p2v_compact(const float *points, const float *feats, const int64_t *batc
   hipStream_t s = (hipStream_t)stream;
   P2vWs w;
   p2v_ws_walk(workspace, n, &w);
+  // where every input row went (-1: dropped), for the caller if it asks
+  int32_t *dest = out_dest ? out_dest : w.dest;
   const int64_t rows = n + SSC_P2V_MAX_IDS;
   hipLaunchKernelGGL(p2v_compact_kernel, dim3((unsigned)ceil_div(rows, 256)), dim3(256), 0, s,
                      points, batch_ids, n, w.table.bits, w.table.prefix, w.hist_all, w.hist_valid,
                      w.start, w.shift, half_extent[0], half_extent[1], half_extent[2], unit[0],
-                     unit[1], unit[2], out_points, out_ids, out_coords, w.dest);
+                     unit[1], unit[2], out_points, out_ids, out_coords, dest);
   SSC_LAUNCH_CHECK("p2v_compact");
   hipLaunchKernelGGL(p2v_feats_kernel, dim3((unsigned)ceil_div(rows * channels, 256)), dim3(256), 0,
-                     s, feats, n, (int)channels, w.dest, w.hist_all, w.hist_valid, w.start,
+                     s, feats, n, (int)channels, dest, w.hist_all, w.hist_valid, w.start,
                      w.shift, out_feats);
   SSC_LAUNCH_CHECK("p2v_feats");
   return SSC_OK;

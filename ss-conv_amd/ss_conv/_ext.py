@@ -80,7 +80,7 @@ _SIGNATURES = {
                                     _vp, _vp, _vp, _vp]),
     "ssc_p2v_compact": (ctypes.c_int, [_vp, _vp, _vp, _i64, _i32, ctypes.POINTER(ctypes.c_float),
                                        ctypes.POINTER(ctypes.c_float), _vp, _sz, _vp, _vp, _vp,
-                                       _vp, _vp]),
+                                       _vp, _vp, _vp]),
     "ssc_unique_workspace_bytes": (_sz, [ctypes.POINTER(_i32), _i64]),
     "ssc_unique_count": (ctypes.c_int, [_vp, _i64, ctypes.POINTER(_i32), _vp, _sz,
                                         ctypes.POINTER(_i32), _vp]),
@@ -580,6 +580,26 @@ def voxel_coords(points, batch_ids, half_extent, unit):
 P2V_MAX_IDS = 4096
 
 
+class _P2vFeatures(torch.autograd.Function):
+    """The compacted feature rows as a function of the input rows: row dest[i] of the output
+    is row i of the input (rows that stand for empty clouds are zeros), so the gradient of
+    input row i is row dest[i] of the output's, or zero for a dropped row."""
+
+    @staticmethod
+    def forward(ctx, feats, out_f, dest):
+        ctx.save_for_backward(dest)
+        ctx.n = feats.size(0)
+        return out_f.clone()  # (an output must not be one of the inputs)
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        (dest,) = ctx.saved_tensors
+        kept = dest >= 0
+        grad_in = grad_out.new_zeros((ctx.n, grad_out.size(1)))
+        grad_in[kept] = grad_out[dest[kept].long()]
+        return grad_in, None, None
+
+
 def p2v_filter(points, feats, batch_ids, half_extent, unit):
     """Filter + batch partition of Point2Voxel.forward (ss_conv/sp_ops/voxelize.py:40-83)
     for float32 points/features and int64 batch ids that are non-decreasing and below
@@ -620,9 +640,13 @@ def p2v_filter(points, feats, batch_ids, half_extent, unit):
     out_f = torch.empty((m, c), dtype=torch.float32, device=dev)
     out_i = torch.empty((m,), dtype=torch.int64, device=dev)
     coords = torch.empty((m, 4), dtype=torch.int32, device=dev)
-    _check(_lib.ssc_p2v_compact(_ptr(points), _ptr(feats), _ptr(batch_ids), n, c, h, u,
+    needs_grad = torch.is_grad_enabled() and feats.requires_grad
+    dest = torch.empty((n,), dtype=torch.int32, device=dev) if needs_grad else None
+    _check(_lib.ssc_p2v_compact(_ptr(points), _ptr(feats.detach()), _ptr(batch_ids), n, c, h, u,
                                 ws.data_ptr(), ws.numel(), _ptr(out_p), _ptr(out_f), _ptr(out_i),
-                                _ptr(coords), s))
+                                _ptr(coords), _ptr(dest), s))
+    if needs_grad:  # keep the point features in the autograd graph
+        out_f = _P2vFeatures.apply(feats, out_f, dest)
     return out_p, out_f, out_i, coords, origin_ids, alive[origin_ids].astype(np.float32)
 
 

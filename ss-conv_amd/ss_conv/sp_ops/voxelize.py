@@ -43,11 +43,10 @@ class Point2Voxel(nn.Module):
         # Clouds concatenated in batch order with small non-negative ids: filter and
         # partition in native kernels (one host read); anything else takes the
         # reference's sequence of torch operations below.
-        # (the native filter returns plain tensors: when the features carry a gradient the
-        # torch operations below keep them in the autograd graph, as the reference does)
-        needs_grad = torch.is_grad_enabled() and feature.requires_grad
+        # (the native filter keeps the features in the autograd graph when they carry a
+        # gradient, as the reference's boolean-mask indexing does)
         fast = _ext.p2v_filter(point_cloud, feature, batch_ids, half, unit) \
-            if point_cloud.is_cuda and not needs_grad else None
+            if point_cloud.is_cuda else None
         if fast is not None:
             valid_point_cloud, valid_feature, valid_ids, voxel_index, origin_ids, alive = fast
             B1 = len(origin_ids)
