@@ -150,6 +150,25 @@ int bit_table_scan(const BitTable &t, hipStream_t s) {
   return SSC_OK;
 }
 
+int read_back_view(const void **view, const void *src_dev, size_t bytes, hipStream_t s) {
+  static thread_local char *pinned = nullptr;
+  SSC_CHECK(bytes <= kReadBackBytes, SSC_EINVAL, "read-back of %zu bytes exceeds the pinned block",
+            bytes);
+  if (pinned == nullptr)
+    SSC_HIP(hipHostMalloc((void **)&pinned, kReadBackBytes, hipHostMallocPortable));
+  if (bytes > 0) SSC_HIP(hipMemcpyAsync(pinned, src_dev, bytes, hipMemcpyDeviceToHost, s));
+  SSC_HIP(hipStreamSynchronize(s));
+  *view = pinned;
+  return SSC_OK;
+}
+
+int read_back(void *dst_host, const void *src_dev, size_t bytes, hipStream_t s) {
+  const void *view;
+  int rc = read_back_view(&view, src_dev, bytes, s);
+  if (rc == SSC_OK) memcpy(dst_host, view, bytes);
+  return rc;
+}
+
 }  // namespace ssc
 
 extern "C" {

@@ -420,9 +420,8 @@ int ssc_rulebook_count_ordered(const int32_t *indices, int64_t n_in, const ssc_g
     SSC_LAUNCH_CHECK("mark_count");
   }
   if ((rc = bit_table_scan(w.table, s)) != SSC_OK) return rc;
-  int32_t host[2] = {0, 0};
-  SSC_HIP(hipMemcpyAsync(host, w.table.total, sizeof(host), hipMemcpyDeviceToHost, s));
-  SSC_HIP(hipStreamSynchronize(s));
+  int32_t host[2];
+  if ((rc = read_back(host, w.table.total, sizeof(host), s)) != SSC_OK) return rc;
   *n_out_host = gg.subm ? (int32_t)n_in : host[0];
   *in_order_host = host[1] == 0 ? 1 : 0;
   return SSC_OK;
@@ -509,9 +508,7 @@ int ssc_unique_count(const int32_t *coords, int64_t n, const int32_t dims[4], vo
                      (int32_t *)nullptr);
   SSC_LAUNCH_CHECK("mark_rows");
   if ((rc = bit_table_scan(t, s)) != SSC_OK) return rc;
-  SSC_HIP(hipMemcpyAsync(n_unique_host, t.total, sizeof(int32_t), hipMemcpyDeviceToHost, s));
-  SSC_HIP(hipStreamSynchronize(s));
-  return SSC_OK;
+  return read_back(n_unique_host, t.total, sizeof(int32_t), s);
 }
 
 int ssc_unique_emit(const int32_t *coords, int64_t n, const int32_t dims[4], void *workspace,

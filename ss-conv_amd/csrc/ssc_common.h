@@ -85,6 +85,15 @@ __device__ __forceinline__ int bit_rank(const uint32_t *__restrict__ bits,
 int fill_i32(int32_t *p, int64_t n, int32_t v, hipStream_t s);
 int fill_f32(float *p, int64_t n, float v, hipStream_t s);
 
+// Bring `bytes` (at most kReadBackBytes) of device memory to the host behind the work queued
+// on `s` and wait for it.  The copy lands in a block of pinned host memory that each host
+// thread keeps for the life of the process, so nothing is staged through a pageable buffer;
+// `*view` points into that block and holds until the thread's next read-back.
+constexpr size_t kReadBackBytes = 64 << 10;
+int read_back_view(const void **view, const void *src_dev, size_t bytes, hipStream_t s);
+// The same, moved on to `dst_host`.
+int read_back(void *dst_host, const void *src_dev, size_t bytes, hipStream_t s);
+
 }  // namespace ssc
 
 #endif

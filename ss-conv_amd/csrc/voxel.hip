@@ -9,6 +9,7 @@
 #pragma clang fp contract(off)
 
 #include <math.h>
+#include <string.h>
 
 namespace ssc {
 
@@ -842,12 +843,14 @@ int ssc_p2v_scan(const float *points, const int64_t *batch_ids, int64_t n,
   hipLaunchKernelGGL(p2v_prefix_kernel, dim3(1), dim3(256), 0, s, w.hist_all, w.hist_valid,
                      w.start, w.shift);
   SSC_LAUNCH_CHECK("p2v_prefix");
-  SSC_HIP(hipMemcpyAsync(hist_all_host, w.hist_all, SSC_P2V_MAX_IDS * sizeof(int32_t),
-                         hipMemcpyDeviceToHost, s));
-  SSC_HIP(hipMemcpyAsync(hist_valid_host, w.hist_valid, SSC_P2V_MAX_IDS * sizeof(int32_t),
-                         hipMemcpyDeviceToHost, s));
-  SSC_HIP(hipMemcpyAsync(flags_host, w.flags, 2 * sizeof(int32_t), hipMemcpyDeviceToHost, s));
-  SSC_HIP(hipStreamSynchronize(s));
+  // the two histograms and the flags sit side by side: one copy brings all three
+  static_assert((2 * SSC_P2V_MAX_IDS + 256) * sizeof(int32_t) <= kReadBackBytes, "pinned block");
+  const void *view;
+  if ((rc = read_back_view(&view, w.hist_all, clear_n * sizeof(int32_t), s)) != SSC_OK) return rc;
+  const int32_t *land = (const int32_t *)view;
+  memcpy(hist_all_host, land, SSC_P2V_MAX_IDS * sizeof(int32_t));
+  memcpy(hist_valid_host, land + (w.hist_valid - w.hist_all), SSC_P2V_MAX_IDS * sizeof(int32_t));
+  memcpy(flags_host, land + (w.flags - w.hist_all), 2 * sizeof(int32_t));
   return SSC_OK;
 }
 
