@@ -69,6 +69,46 @@ def test_rulebook_matches_oracle(case, oracle, device):
     assert np.array_equal(g_pairs, o_pairs)
 
 
+@pytest.mark.parametrize("case", [RULEBOOK_CASES[1], RULEBOOK_CASES[4], RULEBOOK_CASES[8]])
+@pytest.mark.parametrize("shuffle", [False, True])
+def test_rulebook_count_then_emit_entry_points(case, shuffle, device):
+    """The library offers the rulebook in two ways: ssc_rulebook_count(_ordered) followed
+    by ssc_rulebook_emit, and ssc_rulebook_build followed by ssc_rulebook_rows (the one the
+    Python side calls).  Both give the same tensors and the same order flag."""
+    import ctypes
+    from ss_conv import _ext
+    batch, grid, n, k, s, p, d, subm = case
+    rng = np.random.default_rng(11)
+    idx = random_voxels(rng, batch, grid, n)
+    if shuffle:
+        idx = idx[rng.permutation(idx.shape[0])]
+    print("case", case, shuffle, flush=True)
+    t = torch.from_numpy(idx).to(device)
+    out_shape = [grid] * 3 if subm else [(grid + 2 * p - d * (k - 1) - 1) // s + 1] * 3
+    want = _ext.get_indice_pairs_3d(t, batch, out_shape, [grid] * 3, [k] * 3, [s] * 3, [p] * 3,
+                                    [d] * 3, [0] * 3, int(subm), 0)
+    g = _ext._geometry(batch, out_shape, [k] * 3, [s] * 3, [p] * 3, [d] * 3, subm, 0)
+    lib = _ext._lib
+    nbytes = lib.ssc_rulebook_workspace_bytes(ctypes.byref(g), n)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=device)
+    n_out, in_order = ctypes.c_int32(0), ctypes.c_int32(-1)
+    assert lib.ssc_rulebook_count_ordered(t.data_ptr(), n, ctypes.byref(g), ws.data_ptr(), nbytes,
+                                          ctypes.byref(n_out), ctypes.byref(in_order), None) == 0
+    assert n_out.value == want[0].shape[0]
+    assert bool(in_order.value) == want[1]._ssc_canonical[0] == (not shuffle)
+    K = k ** 3
+    out = torch.full((max(n_out.value, 1), 4), -7, dtype=torch.int32, device=device)
+    pairs = torch.full((K, 2, n), -7, dtype=torch.int32, device=device)
+    num = torch.full((K,), -7, dtype=torch.int32, device=device)
+    assert lib.ssc_rulebook_emit(t.data_ptr(), n, ctypes.byref(g), ws.data_ptr(), nbytes,
+                                 None if subm else out.data_ptr(), pairs.data_ptr(),
+                                 num.data_ptr(), None) == 0
+    torch.cuda.synchronize()
+    if not subm:
+        assert torch.equal(out[:n_out.value], want[0])
+    assert torch.equal(pairs, want[1]) and torch.equal(num, want[2])
+
+
 def test_rulebook_unsorted_input_rows(oracle, device):
     """Input rows in arbitrary order: outputs still ascending by key, pairs ascending in input row."""
     rng = np.random.default_rng(5)
