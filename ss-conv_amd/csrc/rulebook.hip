@@ -155,12 +155,11 @@ __global__ void __launch_bounds__(256)
   atomicOr(&bits[key >> 5], 1u << (key & 31u));
 }
 
-// Decode every set bit into its (b,x,y,z) row, written at the bit's rank.
-__global__ void __launch_bounds__(256)
-    emit_rows_kernel(const uint32_t *__restrict__ bits, const int32_t *__restrict__ prefix,
-                     int64_t n_words, int d1, int d2, int d3, int32_t *__restrict__ out) {
-  int64_t w = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (w >= n_words) return;
+// Decode every set bit of word w into its (b,x,y,z) row, written at the bit's rank.
+__device__ __forceinline__ void emit_rows_of_word(const uint32_t *__restrict__ bits,
+                                                  const int32_t *__restrict__ prefix, int64_t w,
+                                                  int d1, int d2, int d3,
+                                                  int32_t *__restrict__ out) {
   uint32_t b = bits[w];
   if (b == 0) return;
   int r = prefix[w];
@@ -190,6 +189,13 @@ __global__ void __launch_bounds__(256)
       reinterpret_cast<int4 *>(out)[r++] = make_int4(bb, x, y, z);
     }
   }
+}
+
+__global__ void __launch_bounds__(256)
+    emit_rows_kernel(const uint32_t *__restrict__ bits, const int32_t *__restrict__ prefix,
+                     int64_t n_words, int d1, int d2, int d3, int32_t *__restrict__ out) {
+  int64_t w = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (w < n_words) emit_rows_of_word(bits, prefix, w, d1, d2, d3, out);
 }
 
 // rank -> input row, for the submanifold rulebook (outputs keep the input numbering).
@@ -269,12 +275,26 @@ __global__ void __launch_bounds__(kScanThreads)
 // is (pairs of earlier chunks) + (earlier lanes of this chunk), which makes the
 // pair list ascending in input row.  The wave also pads slots [num, n_in) of
 // its own 64-slot window with -1.
+//
+// The grid's rows y >= ks[0] (a regular convolution has them, a submanifold one does not)
+// do an unrelated job that needs nothing but the scanned table either: they decode the
+// table into out_indices[], strided over its words.  One launch, and the two jobs, each
+// short and bound by latency, run side by side.
 __global__ void __launch_bounds__(256)
     write_pairs_kernel(const int32_t *__restrict__ indices, int64_t n_in, Geom g,
                        const uint32_t *__restrict__ bits, const int32_t *__restrict__ prefix,
                        const int32_t *__restrict__ rank2row,
                        const int32_t *__restrict__ chunk_prefix, int64_t n_chunks,
-                       const int32_t *__restrict__ pair_num, int32_t *__restrict__ pairs) {
+                       const int32_t *__restrict__ pair_num, int32_t *__restrict__ pairs,
+                       int64_t n_words, int32_t *__restrict__ out_indices) {
+  if ((int)blockIdx.y >= g.ks[0]) {
+    const int64_t step = (int64_t)(gridDim.y - g.ks[0]) * gridDim.x * blockDim.x;
+    int64_t w = ((int64_t)(blockIdx.y - g.ks[0]) * gridDim.x + blockIdx.x) * blockDim.x +
+                threadIdx.x;
+    for (; w < n_words; w += step)
+      emit_rows_of_word(bits, prefix, w, g.os[0], g.os[1], g.os[2], out_indices);
+    return;
+  }
   int64_t chunk = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (chunk >= n_chunks) return;
   int lane = threadIdx.x & 63;
@@ -447,11 +467,6 @@ int ssc_rulebook_emit(const int32_t *indices, int64_t n_in, const ssc_geometry *
     hipLaunchKernelGGL(rank_to_row_kernel, dim3((unsigned)ceil_div(n_in, 256)), dim3(256), 0, s,
                        indices, n_in, gg, w.table.bits, w.table.prefix, w.rank2row);
     SSC_LAUNCH_CHECK("rank_to_row");
-  } else {
-    hipLaunchKernelGGL(emit_rows_kernel, dim3((unsigned)ceil_div(w.table.n_words, 256)),
-                       dim3(256), 0, s, w.table.bits, w.table.prefix, w.table.n_words, gg.os[0],
-                       gg.os[1], gg.os[2], out_indices);
-    SSC_LAUNCH_CHECK("emit_rows");
   }
   if (gg.subm) {  // a regular convolution's counts were taken while marking the table
     hipLaunchKernelGGL(count_pairs_kernel, dim3(chunk_blocks), dim3(256), 0, s, indices, n_in, gg,
@@ -461,10 +476,12 @@ int ssc_rulebook_emit(const int32_t *indices, int64_t n_in, const ssc_geometry *
   hipLaunchKernelGGL(scan_chunks_kernel, dim3(gg.K), dim3(kScanThreads), 0, s, w.chunk_count,
                      w.n_chunks, pair_num);
   SSC_LAUNCH_CHECK("scan_chunks");
-  hipLaunchKernelGGL(write_pairs_kernel, dim3(chunk_blocks, (unsigned)gg.ks[0]), dim3(256), 0, s,
-                     indices, n_in, gg,
-                     w.table.bits, w.table.prefix, w.rank2row, w.chunk_count, w.n_chunks, pair_num,
-                     pairs);
+  // rows of the grid beyond the kernel's x extent write out_indices[] (see the kernel)
+  int64_t row_blocks = gg.subm ? 0 : ceil_div(ceil_div(w.table.n_words, 256), chunk_blocks);
+  if (row_blocks > 4096) row_blocks = 4096;
+  hipLaunchKernelGGL(write_pairs_kernel, dim3(chunk_blocks, (unsigned)(gg.ks[0] + row_blocks)),
+                     dim3(256), 0, s, indices, n_in, gg, w.table.bits, w.table.prefix, w.rank2row,
+                     w.chunk_count, w.n_chunks, pair_num, pairs, w.table.n_words, out_indices);
   SSC_LAUNCH_CHECK("write_pairs");
   return SSC_OK;
 }
