@@ -46,15 +46,20 @@ constexpr int kMinTile = 64;
 // i.e. one 16-byte load per lane and step.  Which of a step's 32 channels sits in which of
 // a lane's 8 slots does not matter for the sum as long as the staged rows use the same
 // assignment; they do (lane group g reads channels 32q + 8g .. +7 of its row).
+struct PackArgs {
+  const void *w;  // filters, addressed as w[k*fs_k + ci*fs_ci + co*fs_co]
+  int64_t fs_k, fs_ci, fs_co;
+  int K, cin, cout, ncb, nch;
+  void *packed_out;
+};
+
+// Element idx of the packed filters.
 template <typename IO>
-__global__ void __launch_bounds__(256)
-    pack_filters_kernel(const IO *__restrict__ w, int64_t fs_k, int64_t fs_ci, int64_t fs_co,
-                        int K, int cin, int cout, int ncb, int nch, void *__restrict__ packed_out,
-                        int32_t *__restrict__ flag) {
-  int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (idx == 0) flag[0] = 0;  // the pair-order flag of the kernels that follow
-  int64_t total = (int64_t)K * ncb * nch * 1024;
-  if (idx >= total) return;
+__device__ __forceinline__ void pack_filter_element(const PackArgs &a, int64_t idx) {
+  const IO *__restrict__ w = static_cast<const IO *>(a.w);
+  const int64_t fs_k = a.fs_k, fs_ci = a.fs_ci, fs_co = a.fs_co;
+  const int cin = a.cin, cout = a.cout, ncb = a.ncb, nch = a.nch;
+  void *packed_out = a.packed_out;
   int64_t r = idx >> 10;
   int cc = r % nch;
   r /= nch;
@@ -74,6 +79,13 @@ __global__ void __launch_bounds__(256)
   IO v = (IO)0.f;
   if (ci < cin && co < cout) v = w[k * fs_k + ci * fs_ci + co * fs_co];
   static_cast<IO *>(packed_out)[idx] = v;
+}
+
+template <typename IO>
+__global__ void __launch_bounds__(256) pack_filters_kernel(PackArgs a, int32_t *__restrict__ flag) {
+  int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx == 0) flag[0] = 0;  // the pair-order flag of the kernels that follow
+  if (idx < (int64_t)a.K * a.ncb * a.nch * 1024) pack_filter_element<IO>(a, idx);
 }
 
 // ---- pair order -------------------------------------------------------------------------
@@ -208,16 +220,31 @@ __global__ void __launch_bounds__(256)
 // cells c = 0..n_cells of a regular grid (cell n_cells being the end), computed from
 // the pairs' side: one thread per pair; the pair
 // that is the first of its offset at or beyond a cell boundary writes that boundary.
+//
+// Rows y >= K of the grid, when the launch has them, do an unrelated job that depends on
+// nothing before it: they pack the filters (strided over the packed elements) and clear
+// flag[0] for the kernels that follow.  Such a launch is told that the pairs are in order
+// (`pairs_in_order`) and does not read the flag itself.
+template <typename IO>
 __global__ void __launch_bounds__(256)
-    grid_segments_kernel(const int32_t *__restrict__ flag, const int32_t *__restrict__ pairs,
-                         const int32_t *__restrict__ sorted, int64_t pair_stride, int plane_s,
-                         const int32_t *__restrict__ pair_num, int K, int64_t n_cells,
-                         int granule, int32_t *__restrict__ segs) {
+    grid_segments_kernel(int32_t *__restrict__ flag, int pairs_in_order,
+                         const int32_t *__restrict__ pairs, const int32_t *__restrict__ sorted,
+                         int64_t pair_stride, int plane_s, const int32_t *__restrict__ pair_num,
+                         int K, int64_t n_cells, int granule, int32_t *__restrict__ segs,
+                         PackArgs pack) {
+  if ((int)blockIdx.y >= K) {
+    const int64_t total = (int64_t)pack.K * pack.ncb * pack.nch * 1024;
+    const int64_t step = (int64_t)(gridDim.y - K) * gridDim.x * blockDim.x;
+    int64_t idx = ((int64_t)(blockIdx.y - K) * gridDim.x + blockIdx.x) * blockDim.x + threadIdx.x;
+    if (idx == 0) flag[0] = 0;
+    for (; idx < total; idx += step) pack_filter_element<IO>(pack, idx);
+    return;
+  }
   const int k = blockIdx.y;
   const int64_t j = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   const int n = pair_num[k];
   if (j >= n && !(j == 0 && n == 0)) return;
-  const int32_t *src = flag[0] ? sorted : pairs;
+  const int32_t *src = (!pairs_in_order && flag[0]) ? sorted : pairs;
   const int32_t *s = src + ((int64_t)k * 2 + plane_s) * pair_stride;
   // boundary c (first row c*granule) is served by the first pair whose row is at or
   // beyond it: pair j serves the boundaries in (row[j-1], row[j]]
@@ -1383,13 +1410,17 @@ static int conv_fwd(const IO *features, int64_t n_in, int32_t c_in, const IO *fi
   const int plane_s = 1 - plane_g;
   int rc;
 
-  int64_t packed_n = (int64_t)K * p.ncb * p.nch * 1024;
-  hipLaunchKernelGGL(pack_filters_kernel<IO>, dim3((unsigned)ceil_div(packed_n, 256)), dim3(256), 0, s,
-                     filters, fs_k, fs_ci, fs_co, K, c_in, c_out, p.ncb, p.nch, w.packed, w.flag);
-  SSC_LAUNCH_CHECK("pack_filters");
+  const int64_t packed_n = (int64_t)K * p.ncb * p.nch * 1024;
+  const PackArgs pack = {filters, fs_k, fs_ci, fs_co, K, c_in, c_out, p.ncb, p.nch, w.packed};
+  const bool in_order = (subm & SSC_CONV_PAIRS_CANONICAL) != 0;
+  if (!in_order) {  // otherwise the filters are packed beside the first kernel of the split
+    hipLaunchKernelGGL(pack_filters_kernel<IO>, dim3((unsigned)ceil_div(packed_n, 256)), dim3(256),
+                       0, s, pack, w.flag);
+    SSC_LAUNCH_CHECK("pack_filters");
+  }
 
   dim3 pair_grid((unsigned)ceil_div(pair_stride, 256), (unsigned)K);
-  if ((subm & SSC_CONV_PAIRS_CANONICAL) == 0) {  // otherwise flag[0] stays 0: pairs in order
+  if (!in_order) {  // otherwise flag[0] is 0: pairs in order
     hipLaunchKernelGGL(check_sorted_kernel, pair_grid, dim3(256), 0, s, pairs, pair_stride, plane_s,
                        pair_num, w.flag);
     SSC_LAUNCH_CHECK("check_sorted");
@@ -1408,8 +1439,14 @@ static int conv_fwd(const IO *features, int64_t n_in, int32_t c_in, const IO *fi
   }
 
   // work split on the fine grid, then the tiles and their segments
-  hipLaunchKernelGGL(grid_segments_kernel, pair_grid, dim3(256), 0, s, w.flag, pairs, w.sorted,
-                     pair_stride, plane_s, pair_num, K, p.n_fine, kSplitGranule, w.fine_segs);
+  dim3 seg_grid = pair_grid;
+  if (in_order) {
+    int64_t rows = ceil_div(ceil_div(packed_n, 256), pair_grid.x);
+    seg_grid.y += (unsigned)(rows < 4096 ? rows : 4096);
+  }
+  hipLaunchKernelGGL(grid_segments_kernel<IO>, seg_grid, dim3(256), 0, s, w.flag, in_order ? 1 : 0,
+                     pairs, w.sorted, pair_stride, plane_s, pair_num, K, p.n_fine, kSplitGranule,
+                     w.fine_segs, pack);
   hipLaunchKernelGGL(split_bounds_kernel, dim3((unsigned)ceil_div(p.n_fine + 1, 256)), dim3(256), 0,
                      s, w.fine_segs, K, p.n_fine, n_out, p.tile_rows, p.n_wg, w.range_row0);
   hipLaunchKernelGGL(split_rows_kernel, dim3(1), dim3(256), 0, s, w.range_row0, n_out, p.tile_rows,
