@@ -109,6 +109,20 @@ def test_rulebook_count_then_emit_entry_points(case, shuffle, device):
     assert torch.equal(pairs, want[1]) and torch.equal(num, want[2])
 
 
+def test_rulebook_few_voxels_in_a_large_grid(oracle, device):
+    """300 voxels in 40 x 128^3 cells: the table has 2.6 M words, the input five chunks.
+    (The blocks that decode the table into output rows ride on the grid of the kernel that
+    writes the pairs, which is sized by the input: here they must stride over the table.)"""
+    rng = np.random.default_rng(3)
+    cells = np.unique(rng.integers(0, 40 * 128 ** 3, size=300))
+    b, r = cells // 128 ** 3, cells % 128 ** 3
+    idx = np.stack([b, r // 128 ** 2, (r // 128) % 128, r % 128], 1).astype(np.int32)
+    o = oracle.canonicalize(*oracle.rulebook(idx, 40, [128] * 3, 3, 1, 1))
+    g = gpu_rulebook(idx, 40, 128, 3, 1, 1)
+    for a, b in zip(g, o):
+        assert np.array_equal(a, b)
+
+
 def test_rulebook_unsorted_input_rows(oracle, device):
     """Input rows in arbitrary order: outputs still ascending by key, pairs ascending in input row."""
     rng = np.random.default_rng(5)
