@@ -208,8 +208,12 @@ def ops_table(torch, _ext, synth, dev, seed):
     zi = torch.zeros(n_rows, 4, dtype=torch.int32, device=dev)
     with torch.no_grad():
         ms, _ = timed(lambda: fused(SparseTensor(x, zi, [64] * 3, 32)), n=10)
+        # statistics: the rows once (sums, sums of squares), the scalar columns a second
+        # time (centred squares); then the rows once more for the output
+        n_scalar = Rs[0][0] + n_gates
+        fwd_cols = 2 * c_in + n_scalar + c_out
         report("BatchNorm+Activation fused, training (%d rows, %d->%d ch)" % (n_rows, c_in, c_out),
-               ms, 4 * n_rows * (3 * c_in + c_out), "statistics read the rows twice")
+               ms, 4 * n_rows * fwd_cols, "statistics read the scalar columns twice")
         fused.eval()
         ms, _ = timed(lambda: fused(SparseTensor(x, zi, [64] * 3, 32)), n=10)
         report("BatchNorm+Activation fused, evaluation", ms, 4 * n_rows * (c_in + c_out))
@@ -220,7 +224,7 @@ def ops_table(torch, _ext, synth, dev, seed):
             ms, _ = timed(lambda: fused(SparseTensor(x, zi, [64] * 3, 32)), n=10)
         finally:
             bnact.usable = keep
-        report("same layers as torch ops, training", ms, 4 * n_rows * (3 * c_in + c_out),
+        report("same layers as torch ops, training", ms, 4 * n_rows * fwd_cols,
                "same algorithmic bytes")
     xg = x.clone().requires_grad_(True)
     dy = torch.randn(n_rows, c_out, device=dev)
@@ -230,7 +234,7 @@ def ops_table(torch, _ext, synth, dev, seed):
         y.backward(dy)
         xg.grad = None
     ms, _ = timed(step, n=10)
-    nbytes = 4 * n_rows * (3 * c_in + c_out + 2 * (c_in + c_out) + c_in)
+    nbytes = 4 * n_rows * (fwd_cols + 2 * (c_in + c_out) + c_in)
     report("BatchNorm+Activation fused, forward + backward", ms, nbytes,
            "backward reads rows and gradients twice")
     keep = bnact.usable

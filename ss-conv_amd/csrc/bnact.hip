@@ -101,12 +101,17 @@ template <> struct Vec<4> {
   }
 };
 
-// partial[b*C + c] = sum over the rows of block b of x[r,c] (SQUARE == 0) or of
-// (x[r,c] - shift[c])^2 (SQUARE == 1).
+// Statistics of the rows of block b, column by column.
+// SQUARE == 0: partial[b*C + c] = sum of x[r,c] and partial_sq[b*C + c] = sum of x[r,c]^2.
+// SQUARE == 1: partial_sq[b*C + c] = sum of (x[r,c] - shift[c])^2, for the groups of V
+// columns that hold a scalar column (scalar_idx[c] >= 0) only: the other columns are not
+// centred (their shift is 0), so the first pass already has their sum of squares, and
+// this pass neither reads nor writes them.
 template <int SQUARE, int V>
 __global__ void __launch_bounds__(kBnThreads)
     bn_partial_kernel(const float *__restrict__ x, int64_t n, int C, int TX, int rows_per_block,
-                      const float *__restrict__ shift, float *__restrict__ partial) {
+                      const float *__restrict__ shift, const int32_t *__restrict__ scalar_idx,
+                      float *__restrict__ partial, float *__restrict__ partial_sq) {
   __shared__ float red[kBnThreads];
   const int TY = kBnThreads / TX;
   const int tx = threadIdx.x % TX, ty = threadIdx.x / TX;
@@ -114,14 +119,21 @@ __global__ void __launch_bounds__(kBnThreads)
   const int64_t r1 = r0 + rows_per_block < n ? r0 + rows_per_block : n;
   for (int c0 = 0; c0 < C; c0 += TX * V) {
     const int c = c0 + tx * V;
-    float acc[2][V];
+    float acc[2][V], accq[2][V];
     float sh[V];
+    bool wanted = c < C;
+    if (SQUARE) {
+      bool any = false;
+#pragma unroll
+      for (int i = 0; i < V; ++i) any = any || (c + i < C && scalar_idx[c + i] >= 0);
+      wanted = any;
+    }
 #pragma unroll
     for (int i = 0; i < V; ++i) {
-      acc[0][i] = acc[1][i] = 0.f;
+      acc[0][i] = acc[1][i] = accq[0][i] = accq[1][i] = 0.f;
       sh[i] = (SQUARE && c + i < C) ? shift[c + i] : 0.f;
     }
-    if (c < C) {
+    if (wanted) {
       int64_t r = r0 + ty;
       for (; r + TY < r1; r += 2 * TY) {  // two rows in flight
         Vec<V> a, b;
@@ -130,8 +142,12 @@ __global__ void __launch_bounds__(kBnThreads)
 #pragma unroll
         for (int i = 0; i < V; ++i) {
           float va = a.v[i] - sh[i], vb = b.v[i] - sh[i];
-          acc[0][i] += SQUARE ? va * va : va;
-          acc[1][i] += SQUARE ? vb * vb : vb;
+          if (!SQUARE) {
+            acc[0][i] += va;
+            acc[1][i] += vb;
+          }
+          accq[0][i] += va * va;
+          accq[1][i] += vb * vb;
         }
       }
       if (r < r1) {
@@ -140,14 +156,19 @@ __global__ void __launch_bounds__(kBnThreads)
 #pragma unroll
         for (int i = 0; i < V; ++i) {
           float va = a.v[i] - sh[i];
-          acc[0][i] += SQUARE ? va * va : va;
+          if (!SQUARE) acc[0][i] += va;
+          accq[0][i] += va * va;
         }
       }
     }
 #pragma unroll
     for (int i = 0; i < V; ++i) {
-      float s = reduce_rows(acc[0][i] + acc[1][i], red, tx, ty, TX, TY);
-      if (ty == 0 && c + i < C) partial[(int64_t)blockIdx.x * C + c + i] = s;
+      if (!SQUARE) {
+        float s = reduce_rows(acc[0][i] + acc[1][i], red, tx, ty, TX, TY);
+        if (ty == 0 && c + i < C) partial[(int64_t)blockIdx.x * C + c + i] = s;
+      }
+      float q = reduce_rows(accq[0][i] + accq[1][i], red, tx, ty, TX, TY);
+      if (ty == 0 && wanted && c + i < C) partial_sq[(int64_t)blockIdx.x * C + c + i] = q;
     }
   }
 }
@@ -812,27 +833,32 @@ int ssc_bn_prepare_f32(const float *x, int64_t n, int32_t c, const int32_t *fiel
   BnShape sh = bn_shape(n, c / V);
   Carver cv(workspace);
   float *partial = cv.take<float>((size_t)sh.blocks * 2 * c);
+  float *partial_sq = partial + (size_t)sh.blocks * c;
   float *col_msq = cv.take<float>((size_t)c);
   const double inv_n = n > 0 ? 1.0 / (double)n : 0.0;
   if (training) {
+    // sums and sums of squares in one pass over the rows; the column means (of the scalar
+    // columns; 0 elsewhere) go to shift[]; a second pass over the scalar columns replaces
+    // their sums of squares by centred ones
     if (V == 4)
       hipLaunchKernelGGL((bn_partial_kernel<0, 4>), dim3(sh.blocks), dim3(kBnThreads), 0, s, x, n,
-                         c, sh.tx, sh.rows_per_block, (const float *)nullptr, partial);
+                         c, sh.tx, sh.rows_per_block, (const float *)nullptr, scalar_idx, partial,
+                         partial_sq);
     else
       hipLaunchKernelGGL((bn_partial_kernel<0, 1>), dim3(sh.blocks), dim3(kBnThreads), 0, s, x, n,
-                         c, sh.tx, sh.rows_per_block, (const float *)nullptr, partial);
+                         c, sh.tx, sh.rows_per_block, (const float *)nullptr, scalar_idx, partial,
+                         partial_sq);
     hipLaunchKernelGGL(bn_colsum_kernel, dim3((unsigned)ceil_div(c, 16)), dim3(256), 0, s, partial,
                        sh.blocks, c, inv_n, scalar_idx, shift);
     if (V == 4)
       hipLaunchKernelGGL((bn_partial_kernel<1, 4>), dim3(sh.blocks), dim3(kBnThreads), 0, s, x, n,
-                         c, sh.tx, sh.rows_per_block, shift, partial);
+                         c, sh.tx, sh.rows_per_block, shift, scalar_idx, partial, partial_sq);
     else
       hipLaunchKernelGGL((bn_partial_kernel<1, 1>), dim3(sh.blocks), dim3(kBnThreads), 0, s, x, n,
-                         c, sh.tx, sh.rows_per_block, shift, partial);
+                         c, sh.tx, sh.rows_per_block, shift, scalar_idx, partial, partial_sq);
+    hipLaunchKernelGGL(bn_colsum_kernel, dim3((unsigned)ceil_div(c, 16)), dim3(256), 0, s,
+                       partial_sq, sh.blocks, c, inv_n, (const int32_t *)nullptr, col_msq);
   }
-  if (training)
-    hipLaunchKernelGGL(bn_colsum_kernel, dim3((unsigned)ceil_div(c, 16)), dim3(256), 0, s, partial,
-                       sh.blocks, c, inv_n, (const int32_t *)nullptr, col_msq);
   hipLaunchKernelGGL(bn_finalize_kernel, dim3(1), dim3(256), 0, s, c, training, eps, momentum,
                      field_of, scalar_idx, field_first, field_dim,
                      n_fields, weight, bias, running_mean, running_var, shift, scale, add,
