@@ -174,22 +174,25 @@ __global__ void __launch_bounds__(kBnThreads)
 }
 
 // out[c] = inv_n * sum over blocks of partial[b*C + c]; with scalar_idx, 0 for the
-// columns that are not scalars.  16 columns x 16 slices of the blocks per workgroup; a
-// column's slices are added in slice order.
+// columns that are not scalars.  kColsumCols columns x 64 slices of the blocks per
+// workgroup (few columns each, for enough workgroups: the sums are a chain of dependent
+// loads); a column's slices are added in slice order.
+constexpr int kColsumCols = 4;
 __global__ void __launch_bounds__(256)
     bn_colsum_kernel(const float *__restrict__ partial, int nb, int C, double inv_n,
                      const int32_t *__restrict__ scalar_idx, float *__restrict__ out) {
-  __shared__ double red[16][16];
-  const int cx = threadIdx.x & 15, part = threadIdx.x >> 4;
-  const int c = blockIdx.x * 16 + cx;
+  constexpr int kSlices = 256 / kColsumCols;
+  __shared__ double red[kSlices][kColsumCols];
+  const int cx = threadIdx.x % kColsumCols, part = threadIdx.x / kColsumCols;
+  const int c = blockIdx.x * kColsumCols + cx;
   double s = 0.0;
   if (c < C && (scalar_idx == nullptr || scalar_idx[c] >= 0))
-    for (int b = part; b < nb; b += 16) s += partial[(int64_t)b * C + c];
+    for (int b = part; b < nb; b += kSlices) s += partial[(int64_t)b * C + c];
   red[part][cx] = s;
   __syncthreads();
   if (part == 0 && c < C) {
     double t = 0.0;
-    for (int i = 0; i < 16; ++i) t += red[i][cx];
+    for (int i = 0; i < kSlices; ++i) t += red[i][cx];
     out[c] = (float)(t * inv_n);
   }
 }
@@ -848,7 +851,7 @@ int ssc_bn_prepare_f32(const float *x, int64_t n, int32_t c, const int32_t *fiel
       hipLaunchKernelGGL((bn_partial_kernel<0, 1>), dim3(sh.blocks), dim3(kBnThreads), 0, s, x, n,
                          c, sh.tx, sh.rows_per_block, (const float *)nullptr, scalar_idx, partial,
                          partial_sq);
-    hipLaunchKernelGGL(bn_colsum_kernel, dim3((unsigned)ceil_div(c, 16)), dim3(256), 0, s, partial,
+    hipLaunchKernelGGL(bn_colsum_kernel, dim3((unsigned)ceil_div(c, kColsumCols)), dim3(256), 0, s, partial,
                        sh.blocks, c, inv_n, scalar_idx, shift);
     if (V == 4)
       hipLaunchKernelGGL((bn_partial_kernel<1, 4>), dim3(sh.blocks), dim3(kBnThreads), 0, s, x, n,
@@ -856,7 +859,7 @@ int ssc_bn_prepare_f32(const float *x, int64_t n, int32_t c, const int32_t *fiel
     else
       hipLaunchKernelGGL((bn_partial_kernel<1, 1>), dim3(sh.blocks), dim3(kBnThreads), 0, s, x, n,
                          c, sh.tx, sh.rows_per_block, shift, scalar_idx, partial, partial_sq);
-    hipLaunchKernelGGL(bn_colsum_kernel, dim3((unsigned)ceil_div(c, 16)), dim3(256), 0, s,
+    hipLaunchKernelGGL(bn_colsum_kernel, dim3((unsigned)ceil_div(c, kColsumCols)), dim3(256), 0, s,
                        partial_sq, sh.blocks, c, inv_n, (const int32_t *)nullptr, col_msq);
   }
   hipLaunchKernelGGL(bn_finalize_kernel, dim3(1), dim3(256), 0, s, c, training, eps, momentum,
@@ -940,7 +943,7 @@ int ssc_bnact_bwd_sums_f32(const float *x, const float *dy, int64_t n, int32_t c
                        bn_tables_lds(c_in), s, x, dy,
                        n, c_in, c_out, sh.tx, sh.rows_per_block, aff, out_mode, gate_col,
                        gated_first, gated_dim, act_scalar, act_gate, partial);
-  hipLaunchKernelGGL(bn_colsum_kernel, dim3((unsigned)ceil_div(2 * c_in, 16)), dim3(256), 0, s,
+  hipLaunchKernelGGL(bn_colsum_kernel, dim3((unsigned)ceil_div(2 * c_in, kColsumCols)), dim3(256), 0, s,
                      partial, sh.blocks, 2 * c_in, 1.0, (const int32_t *)nullptr, sums);
   SSC_LAUNCH_CHECK("bnact_bwd_sums");
   return SSC_OK;
