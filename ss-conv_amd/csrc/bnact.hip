@@ -119,7 +119,8 @@ __global__ void __launch_bounds__(kBnThreads)
   const int64_t r1 = r0 + rows_per_block < n ? r0 + rows_per_block : n;
   for (int c0 = 0; c0 < C; c0 += TX * V) {
     const int c = c0 + tx * V;
-    float acc[2][V], accq[2][V];
+    constexpr int U = 4;  // rows in flight per thread
+    float acc[U][V], accq[U][V];
     float sh[V];
     bool wanted = c < C;
     if (SQUARE) {
@@ -130,44 +131,43 @@ __global__ void __launch_bounds__(kBnThreads)
     }
 #pragma unroll
     for (int i = 0; i < V; ++i) {
-      acc[0][i] = acc[1][i] = accq[0][i] = accq[1][i] = 0.f;
+#pragma unroll
+      for (int u = 0; u < U; ++u) acc[u][i] = accq[u][i] = 0.f;
       sh[i] = (SQUARE && c + i < C) ? shift[c + i] : 0.f;
     }
     if (wanted) {
       int64_t r = r0 + ty;
-      for (; r + TY < r1; r += 2 * TY) {  // two rows in flight
-        Vec<V> a, b;
-        a.load(x + r * C + c);
-        b.load(x + (r + TY) * C + c);
+      for (; r + (U - 1) * TY < r1; r += U * TY) {
+        Vec<V> a[U];
 #pragma unroll
-        for (int i = 0; i < V; ++i) {
-          float va = a.v[i] - sh[i], vb = b.v[i] - sh[i];
-          if (!SQUARE) {
-            acc[0][i] += va;
-            acc[1][i] += vb;
+        for (int u = 0; u < U; ++u) a[u].load(x + (r + u * TY) * C + c);
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+          for (int i = 0; i < V; ++i) {
+            const float v = a[u].v[i] - sh[i];
+            if (!SQUARE) acc[u][i] += v;
+            accq[u][i] += v * v;
           }
-          accq[0][i] += va * va;
-          accq[1][i] += vb * vb;
-        }
       }
-      if (r < r1) {
+      for (; r < r1; r += TY) {  // at most U - 1 rows are left
         Vec<V> a;
         a.load(x + r * C + c);
 #pragma unroll
         for (int i = 0; i < V; ++i) {
-          float va = a.v[i] - sh[i];
-          if (!SQUARE) acc[0][i] += va;
-          accq[0][i] += va * va;
+          const float v = a.v[i] - sh[i];
+          if (!SQUARE) acc[0][i] += v;
+          accq[0][i] += v * v;
         }
       }
     }
 #pragma unroll
     for (int i = 0; i < V; ++i) {
       if (!SQUARE) {
-        float s = reduce_rows(acc[0][i] + acc[1][i], red, tx, ty, TX, TY);
+        float s = reduce_rows((acc[0][i] + acc[1][i]) + (acc[2][i] + acc[3][i]), red, tx, ty, TX, TY);
         if (ty == 0 && c + i < C) partial[(int64_t)blockIdx.x * C + c + i] = s;
       }
-      float q = reduce_rows(accq[0][i] + accq[1][i], red, tx, ty, TX, TY);
+      float q = reduce_rows((accq[0][i] + accq[1][i]) + (accq[2][i] + accq[3][i]), red, tx, ty, TX, TY);
       if (ty == 0 && wanted && c + i < C) partial_sq[(int64_t)blockIdx.x * C + c + i] = q;
     }
   }
