@@ -182,7 +182,7 @@ def ops_table(torch, _ext, synth, dev, seed):
     ms, r = timed(lambda: p2v(tp, tf, ti), n=20)
     N, M = tp.shape[0], r[1].features.shape[0]
     report("Point2Voxel module (%d pts -> %d voxels, C=%d)" % (N, M, C), ms,
-           N * (12 + 8 + 4 * C) + M * (16 + 4 * C) + 4 * N, "3 host reads of data-dependent sizes")
+           N * (12 + 8 + 4 * C) + M * (16 + 4 * C) + 4 * N, "2 host reads of data-dependent sizes")
     v2p = Voxel2Point(unit_voxel_extent=[2.0 / cfg["grid"]] * 3)
     vp, vs, vi = r[0], r[1], r[2]
     ms, _ = timed(lambda: v2p(vs, vp, vi), n=20, warm=3)

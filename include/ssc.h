@@ -318,6 +318,21 @@ int ssc_unique_emit(const int32_t *coords, int64_t n, const int32_t dims[4], voi
                     int32_t *inverse /* [n] */, int32_t *counts /* [m]; may be NULL */,
                     ssc_stream_t stream);
 
+/* The same result with one wait of the host instead of two or three
+ * (ss_conv/sp_ops/voxelize.py:88-93: torch.unique(dim=0, return_inverse, return_counts)
+ * followed by the largest count): inverse[n] and counts have sizes known beforehand when
+ * counts is given room for n entries (entries beyond the number of distinct rows stay 0),
+ * so ssc_unique_build fills both, then SYNCHRONISES `stream` for
+ * totals_host[0] = number of distinct rows and totals_host[1] = largest count;
+ * ssc_unique_rows then writes unique[m,4] from the same, untouched workspace. */
+int ssc_unique_build(const int32_t *coords /* [n,4] */, int64_t n, const int32_t dims[4],
+                     void *workspace, size_t workspace_bytes, int32_t *inverse /* [n] */,
+                     int32_t *counts /* [n] */, int32_t *totals_host /* [2] host */,
+                     ssc_stream_t stream);
+
+int ssc_unique_rows(const int32_t dims[4], int64_t n, void *workspace, size_t workspace_bytes,
+                    int32_t *unique /* [m,4] */, ssc_stream_t stream);
+
 /* Point filter and batch partition of Point2Voxel.forward
  * (ss_conv/sp_ops/voxelize.py:40-83: drop the points outside the grid, give every batch
  * element left without points one zero point, order by batch id), for batch ids that

@@ -346,18 +346,32 @@ __global__ void __launch_bounds__(256)
   }
 }
 
-// inverse[i] = rank of row i's cell; counts[rank] += 1 (integer atomics: exact).
+// inverse[i] = rank of row i's cell; counts[rank] += 1 (integer atomics: exact).  With
+// max_count, max_count[0] = the largest count: the row that raises a cell's count to its
+// final value sees that value, so the maximum over all rows of (count seen + 1) is it
+// (one atomic per wave).
 __global__ void __launch_bounds__(256)
     inverse_counts_kernel(const int32_t *__restrict__ coords, int64_t n, int d1, int d2, int d3,
                           const uint32_t *__restrict__ bits, const int32_t *__restrict__ prefix,
-                          int32_t *__restrict__ inverse, int32_t *__restrict__ counts) {
+                          int32_t *__restrict__ inverse, int32_t *__restrict__ counts,
+                          int32_t *__restrict__ max_count) {
   int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= n) return;
-  int4 r = reinterpret_cast<const int4 *>(coords)[i];
-  uint32_t key = (uint32_t)(((r.x * d1 + r.y) * d2 + r.z) * d3 + r.w);
-  int rk = bit_rank(bits, prefix, key);
-  inverse[i] = rk;
-  if (counts) atomicAdd(&counts[rk], 1);
+  int seen = 0;
+  if (i < n) {
+    int4 r = reinterpret_cast<const int4 *>(coords)[i];
+    uint32_t key = (uint32_t)(((r.x * d1 + r.y) * d2 + r.z) * d3 + r.w);
+    int rk = bit_rank(bits, prefix, key);
+    inverse[i] = rk;
+    if (counts) seen = atomicAdd(&counts[rk], 1) + 1;
+  }
+  if (max_count) {
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) {
+      const int o = __shfl_xor(seen, d, 64);
+      seen = o > seen ? o : seen;
+    }
+    if ((threadIdx.x & 63) == 0 && seen > 0) atomicMax(max_count, seen);
+  }
 }
 
 struct RulebookWs {
@@ -544,8 +558,55 @@ int ssc_unique_emit(const int32_t *coords, int64_t n, const int32_t dims[4], voi
                      t.bits, t.prefix, t.n_words, dims[1], dims[2], dims[3], unique);
   SSC_LAUNCH_CHECK("emit_rows");
   hipLaunchKernelGGL(inverse_counts_kernel, dim3((unsigned)ceil_div(n, 256)), dim3(256), 0, s,
-                     coords, n, dims[1], dims[2], dims[3], t.bits, t.prefix, inverse, counts);
+                     coords, n, dims[1], dims[2], dims[3], t.bits, t.prefix, inverse, counts,
+                     (int32_t *)nullptr);
   SSC_LAUNCH_CHECK("inverse_counts");
+  return SSC_OK;
+}
+
+int ssc_unique_build(const int32_t *coords, int64_t n, const int32_t dims[4], void *workspace,
+                     size_t workspace_bytes, int32_t *inverse, int32_t *counts,
+                     int32_t *totals_host, ssc_stream_t stream) {
+  int64_t cells;
+  int rc = unique_check(dims, n, workspace, workspace_bytes, &cells);
+  if (rc != SSC_OK) return rc;
+  SSC_CHECK(totals_host != nullptr, SSC_EINVAL, "totals_host is NULL");
+  if (n == 0) {
+    totals_host[0] = totals_host[1] = 0;
+    return SSC_OK;
+  }
+  SSC_CHECK(inverse != nullptr && counts != nullptr, SSC_EINVAL, "NULL output pointer");
+  hipStream_t s = (hipStream_t)stream;
+  Carver c(workspace);
+  BitTable t = bit_table_carve(c, cells);
+  // total[0]: the number of distinct rows (written by the scan); total[1]: the largest
+  // count, cleared with the table
+  if ((rc = bit_table_clear(t, s)) != SSC_OK) return rc;
+  hipLaunchKernelGGL(mark_rows_kernel, dim3((unsigned)ceil_div(n, 256)), dim3(256), 0, s, coords,
+                     n, dims[1], dims[2], dims[3], t.bits, (int32_t *)nullptr);
+  SSC_LAUNCH_CHECK("mark_rows");
+  if ((rc = bit_table_scan(t, s)) != SSC_OK) return rc;
+  if ((rc = fill_i32(counts, n, 0, s)) != SSC_OK) return rc;
+  hipLaunchKernelGGL(inverse_counts_kernel, dim3((unsigned)ceil_div(n, 256)), dim3(256), 0, s,
+                     coords, n, dims[1], dims[2], dims[3], t.bits, t.prefix, inverse, counts,
+                     t.total + 1);
+  SSC_LAUNCH_CHECK("inverse_counts");
+  return read_back(totals_host, t.total, 2 * sizeof(int32_t), s);
+}
+
+int ssc_unique_rows(const int32_t dims[4], int64_t n, void *workspace, size_t workspace_bytes,
+                    int32_t *unique, ssc_stream_t stream) {
+  int64_t cells;
+  int rc = unique_check(dims, n, workspace, workspace_bytes, &cells);
+  if (rc != SSC_OK) return rc;
+  if (n == 0) return SSC_OK;
+  SSC_CHECK(unique != nullptr, SSC_EINVAL, "unique is NULL");
+  Carver c(workspace);
+  BitTable t = bit_table_carve(c, cells);
+  hipLaunchKernelGGL(emit_rows_kernel, dim3((unsigned)ceil_div(t.n_words, 256)), dim3(256), 0,
+                     (hipStream_t)stream, t.bits, t.prefix, t.n_words, dims[1], dims[2], dims[3],
+                     unique);
+  SSC_LAUNCH_CHECK("emit_rows");
   return SSC_OK;
 }
 }

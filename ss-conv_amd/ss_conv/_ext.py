@@ -82,6 +82,9 @@ _SIGNATURES = {
                                        ctypes.POINTER(ctypes.c_float), _vp, _sz, _vp, _vp, _vp,
                                        _vp, _vp, _vp]),
     "ssc_unique_workspace_bytes": (_sz, [ctypes.POINTER(_i32), _i64]),
+    "ssc_unique_build": (ctypes.c_int, [_vp, _i64, ctypes.POINTER(_i32), _vp, _sz, _vp, _vp,
+                                        ctypes.POINTER(_i32), _vp]),
+    "ssc_unique_rows": (ctypes.c_int, [ctypes.POINTER(_i32), _i64, _vp, _sz, _vp, _vp]),
     "ssc_unique_count": (ctypes.c_int, [_vp, _i64, ctypes.POINTER(_i32), _vp, _sz,
                                         ctypes.POINTER(_i32), _vp]),
     "ssc_unique_emit": (ctypes.c_int, [_vp, _i64, ctypes.POINTER(_i32), _vp, _sz, _i64, _vp, _vp,
@@ -672,6 +675,30 @@ def unique_rows(coords, dims, return_counts=True):
     _check(_lib.ssc_unique_emit(_ptr(coords), n, d, ws.data_ptr(), ws.numel(), m.value, _ptr(uniq),
                                 _ptr(inverse), _ptr(counts), s))
     return uniq, inverse, counts
+
+
+def unique_rows_max(coords, dims):
+    """unique_rows with counts, and the largest count as a Python int, with one wait of the
+    host for both sizes (ss_conv/sp_ops/voxelize.py:88-93)."""
+    _need_gpu(coords)
+    coords = coords.contiguous()
+    n = coords.size(0)
+    dev = coords.device
+    d = (_i32 * 4)(*[int(v) for v in dims])
+    nbytes = _lib.ssc_unique_workspace_bytes(d, n)
+    if nbytes == 0:
+        raise RuntimeError("unique_rows: prod(dims) must be positive and below 2^31")
+    ws = _workspace(nbytes, dev)
+    inverse = torch.empty((n,), dtype=torch.int32, device=dev)
+    counts = torch.empty((max(n, 1),), dtype=torch.int32, device=dev)
+    totals = (_i32 * 2)(0, 0)
+    s = _stream(coords)
+    _check(_lib.ssc_unique_build(_ptr(coords), n, d, ws.data_ptr(), ws.numel(), _ptr(inverse),
+                                 counts.data_ptr(), totals, s))
+    m = int(totals[0])
+    uniq = torch.empty((m, 4), dtype=torch.int32, device=dev)
+    _check(_lib.ssc_unique_rows(d, n, ws.data_ptr(), ws.numel(), _ptr(uniq), s))
+    return uniq, inverse, counts[:m], int(totals[1])
 
 
 ACT_NONE, ACT_RELU, ACT_SIGMOID, ACT_TANH = 0, 1, 2, 3

@@ -102,12 +102,12 @@ class Point2Voxel(nn.Module):
         """Unique voxels, per-voxel point lists and feature reduction (voxelize.py:85-99)."""
         # a point exactly on the upper face lands on index == limit, hence the +1
         dims = [max_id + 1] + [int(v) + 1 for v in self.voxel_num_limit]
-        occupied_index, inverse, count = _ext.unique_rows(voxel_index, dims, return_counts=True)
+        occupied_index, inverse, count, largest = _ext.unique_rows_max(voxel_index, dims)
         nActive = occupied_index.size(0)
         if self.voxelization_mode == 1 or self.voxelization_mode == 2:
             maxActive = 1
         else:
-            maxActive = int(torch.max(count).item())
+            maxActive = largest
         v2p_maps = voxel2point_mapping(inverse, nActive, maxActive, self.voxelization_mode)
         sparse_feat = voxelization(valid_feature.float().contiguous(), v2p_maps.detach(),
                                    self.voxelization_mode)

@@ -428,6 +428,28 @@ def test_point2voxel_matches_oracle(mode, oracle, device):
     assert np.array_equal(st.features.cpu().numpy(), ref["features"])
 
 
+@pytest.mark.parametrize("n,dims", [(1, [1, 3, 3, 3]), (500, [2, 4, 5, 6]), (20000, [3, 17, 9, 33]),
+                                    (4000, [2, 64, 64, 64])])
+def test_unique_rows_both_entry_point_pairs(n, dims, device):
+    """Sorted distinct voxel rows, inverse, counts and the largest count
+    (torch.unique(dim=0, return_inverse=True, return_counts=True) in
+    ss_conv/sp_ops/voxelize.py:88), through ssc_unique_count + ssc_unique_emit and through
+    ssc_unique_build + ssc_unique_rows."""
+    from ss_conv import _ext
+    gen = torch.Generator().manual_seed(n)
+    rows = torch.stack([torch.randint(0, d, (n,), generator=gen) for d in dims], 1).int().to(device)
+    print("n", n, "dims", dims, flush=True)
+    want_u, want_inv, want_cnt = torch.unique(rows.long(), dim=0, return_inverse=True,
+                                              return_counts=True)
+    u1, inv1, cnt1 = _ext.unique_rows(rows, dims, return_counts=True)
+    u2, inv2, cnt2, largest = _ext.unique_rows_max(rows, dims)
+    for u, inv, cnt in ((u1, inv1, cnt1), (u2, inv2, cnt2)):
+        assert torch.equal(u.long(), want_u)
+        assert torch.equal(inv.long(), want_inv)
+        assert torch.equal(cnt.long(), want_cnt)
+    assert largest == int(want_cnt.max())
+
+
 def test_point2voxel_empty_batch_element(oracle, device):
     """A batch element whose points all fall outside gets one zero point (voxelize.py:68-78)."""
     from ss_conv.sp_ops.voxelize import Point2Voxel
