@@ -46,6 +46,12 @@ def parse_args():
                     help="also time the other operators of the path (pools, global pools, "
                          "Point2Voxel, Voxel2Point) against their algorithmic HBM bytes; "
                          "table on stderr")
+    ap.add_argument("--backbone", action="store_true",
+                    help="also run the backbone of the fourth configuration (Point2Voxel -> four "
+                         "[Convolution -> BatchNorm -> gated Activation] stages -> GlobalAvgPool + "
+                         "Voxel2Point, evaluation mode) and print, stage by stage, pairs, flops "
+                         "and the convolution kernel's time and fraction of the fp32 MFMA peak; "
+                         "table on stderr")
     ap.add_argument("--breakdown", action="store_true",
                     help="also print per-phase timings to stderr")
     return ap.parse_args()
@@ -245,10 +251,26 @@ def ops_table(torch, _ext, synth, dev, seed):
         bnact.usable = keep
     report("same layers as torch ops, forward + backward", ms, nbytes, "same algorithmic bytes")
 
-    # the whole backbone of the fourth configuration: Point2Voxel (64^3) -> four stages of
-    # [Convolution k3 -> BatchNorm -> gated Activation], irreps (8,8,8,8) -> (16,...) ->
-    # (32,...) -> (32,...), stride 2 at stages 2 and 3 -> GlobalAvgPool + Voxel2Point
+    # the whole backbone of the fourth configuration
+    backbone = build_backbone(torch, synth, dev, seed)
+    with torch.no_grad():
+        ms, r = timed(backbone, n=5, warm=2)
+    rows.append("%-44s %8.3f ms   (%d clouds x 1024 points; %d voxels after stage 4, %d channels)"
+                % ("backbone forward, 4th configuration (eval)", ms, 32, r[2].features.shape[0],
+                   r[2].features.shape[1]))
+    print("\n".join(rows), file=sys.stderr)
+
+
+def build_backbone(torch, synth, dev, seed):
+    """The backbone of the fourth configuration in evaluation mode: inputs, layers and a
+    function that runs it and returns (pooled, point features, last SparseTensor, stages),
+    stages being the SparseTensor after every convolution."""
+    from ss_conv.activation import Activation
+    from ss_conv.batchnorm import BatchNorm
     from ss_conv.convolution import Convolution
+    from ss_conv.fused import BatchNormActivation
+    from ss_conv.pool import GlobalAvgPool
+    from ss_conv.sp_ops.voxelize import Point2Voxel, Voxel2Point
     pts, feats, ids = synth.make_clouds(32, 1024, seed=seed, channels=3)
     tp, tf, ti = [torch.from_numpy(a).to(dev) for a in (pts, feats, ids)]
     p2v = Point2Voxel([64] * 3, [2.0 / 64] * 3)
@@ -264,16 +286,48 @@ def ops_table(torch, _ext, synth, dev, seed):
 
     def backbone():
         vp, x, vi, _ = p2v(tp, tf, ti)
+        stages = []
         for conv, block in layers:
-            x = block(conv(x))
+            n_in = x.features.shape[0]
+            y = conv(x)
+            stages.append((n_in, y.features.shape[0], y.indice_dict[None][3], conv.in_channels,
+                           conv.out_channels))
+            x = block(y)
         pooled = gap(x.features.contiguous(), x.get_offsets().int().contiguous())
         v2p = Voxel2Point(unit_voxel_extent=[2.0 / s for s in x.spatial_shape])
-        return pooled, v2p(x, vp, vi), x
+        return pooled, v2p(x, vp, vi), x, stages
+    return backbone
+
+
+def backbone_table(torch, _ext, synth, dev, seed, n=5, warm=2):
+    """Runs the backbone of the fourth configuration and prints one row per convolution
+    stage: rows, pairs, flops, the MFMA kernel's time (HIP events around its launch) and
+    its fraction of the fp32 MFMA peak; then the whole forward."""
+    backbone = build_backbone(torch, synth, dev, seed)
     with torch.no_grad():
-        ms, r = timed(backbone, n=5, warm=2)
-    rows.append("%-44s %8.3f ms   (%d clouds x 1024 points; %d voxels after stage 4, %d channels)"
-                % ("backbone forward, 4th configuration (eval)", ms, 32, r[2].features.shape[0],
-                   r[2].features.shape[1]))
+        for _ in range(warm):
+            r = backbone()
+        torch.cuda.synchronize()
+        _ext.profile_conv(True)
+        a = time.perf_counter()
+        for _ in range(n):
+            r = backbone()
+        torch.cuda.synchronize()
+        ms = (time.perf_counter() - a) * 1e3 / n
+        conv_ms = _ext.profile_conv_read()
+        _ext.profile_conv(False)
+    stages = r[3]
+    rows = ["backbone of the fourth configuration (32 clouds x 1024 points, 64^3, evaluation mode):"]
+    for i, (n_in, n_out, num, cin, cout) in enumerate(stages):
+        P = int(num.sum().item())
+        t = sum(conv_ms[i::len(stages)]) / max(len(conv_ms[i::len(stages)]), 1)
+        fl = 2.0 * P * cin * cout
+        rows.append("  stage %d: %7d -> %7d rows, %4d -> %4d ch, %9d pairs, %8.3f GFLOP, conv kernel "
+                    "%8.3f ms = %6.1f TFLOP/s = %5.1f%% of fp32 MFMA peak"
+                    % (i + 1, n_in, n_out, cin, cout, P, fl / 1e9, t, fl / t / 1e9,
+                       fl / t / 1e9 / (FP32_MFMA_PEAK_TFLOPS / 100.0)))
+    rows.append("  whole forward %.3f ms (%d voxels after stage 4, %d channels)"
+                % (ms, r[2].features.shape[0], r[2].features.shape[1]))
     print("\n".join(rows), file=sys.stderr)
 
 
@@ -402,6 +456,8 @@ def main():
 
     if args.ops:
         ops_table(torch, _ext, synth, dev, args.seed)
+    if args.backbone:
+        backbone_table(torch, _ext, synth, dev, args.seed)
 
     if not args.no_cpu_baseline:
         w = conv.kernel().detach().permute(2, 3, 4, 1, 0).reshape(K, c_in, c_out).cpu().numpy()
