@@ -24,6 +24,8 @@ import math
 import numpy as np
 import torch
 
+from .cache_file import cached_npy
+
 
 # ---- rotations (ZYZ Euler angles) -----------------------------------------------------
 def _as_float(x):
@@ -202,7 +204,7 @@ def get_matrices_kernel(As, eps=1e-10):
                              eps)
 
 
-@functools.lru_cache(maxsize=None)
+@cached_npy("trans_Q")
 def _Q_J_np(J, order_in, order_out):
     do, di, dj = 2 * order_out + 1, 2 * order_in + 1, 2 * J + 1
     n = do * di * dj

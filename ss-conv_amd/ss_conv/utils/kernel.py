@@ -7,7 +7,6 @@ cached per process.  The contraction with the weights -- the part that runs in
 every training forward -- is one HIP kernel that writes the dense kernel in the
 [K, Cin, Cout] layout the sparse convolution consumes.
 """
-import functools
 import math
 
 import numpy as np
@@ -15,9 +14,10 @@ import torch
 
 from ss_conv import _ext
 from .SO3 import irr_repr, real_sh_np, basis_transformation_Q_J
+from .cache_file import cached_npy
 
 
-@functools.lru_cache(maxsize=None)
+@cached_npy("sh_cube")
 def _sample_sh_cube_np(size, J):
     """Y_J on the integer grid centred on the kernel, float64 [2J+1, x, y, z]
     (reference: kernel.py:12-28; the centre voxel follows utils/SO3.py:125-127)."""
