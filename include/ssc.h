@@ -99,6 +99,30 @@ int ssc_rulebook_emit(const int32_t *indices, int64_t n_in, const ssc_geometry *
                       int32_t *pairs /* [K,2,n_in] device */,
                       int32_t *pair_num /* [K] device */, ssc_stream_t stream);
 
+/* The same rulebook with the host's wait moved behind the work that does not depend on the
+ * number of outputs (the reference blocks in torch::_unique with the GPU idle,
+ * src/conv/indice_conv.h:120):
+ *   ssc_rulebook_begin enqueues marking and ranking, starts the copy of the totals to the
+ *     host, and then enqueues pairs[K,2,n_in] and pair_num[K], whose sizes are known
+ *     beforehand.  It returns without waiting.
+ *   ssc_rulebook_finish, called on the same host thread, waits for the totals only (work
+ *     enqueued after ssc_rulebook_begin keeps running) and reports n_out and the input order
+ *     as ssc_rulebook_count_ordered does.
+ *   ssc_rulebook_rows then writes out_indices[n_out,4] (nothing for subm).
+ * A row of `indices` whose batch index lies outside [0, batch_size) -- for subm: whose cell
+ * lies outside the grid -- is left out of the rulebook and ssc_rulebook_finish (like
+ * ssc_rulebook_count) returns SSC_EINVAL; the reference reads and writes outside its grid
+ * buffer for such a row (src/conv/indice_cuda_functor.cu:60-61). */
+int ssc_rulebook_begin(const int32_t *indices, int64_t n_in, const ssc_geometry *g,
+                       void *workspace, size_t workspace_bytes,
+                       int32_t *pairs /* [K,2,n_in] device */, int32_t *pair_num /* [K] device */,
+                       ssc_stream_t stream);
+int ssc_rulebook_finish(const ssc_geometry *g, int64_t n_in, int32_t *n_out_host /* host */,
+                        int32_t *in_order_host /* host */);
+int ssc_rulebook_rows(const ssc_geometry *g, int64_t n_in, void *workspace,
+                      size_t workspace_bytes, int32_t *out_indices /* [n_out,4] device */,
+                      ssc_stream_t stream);
+
 /* ------------------------------------------------------------------------
  * Sparse convolution forward.  Replaces indiceConv<float>
  * (src/conv/indice_conv.h:247-343; bound as indice_conv_fp32,
@@ -147,6 +171,45 @@ int ssc_conv_fwd_f16(const void *features /* [n_in,c_in] half */, int64_t n_in, 
                      int32_t kernel_volume, int32_t inverse, int32_t subm,
                      void *out /* [n_out,c_out] half */, int64_t n_out, void *workspace,
                      size_t workspace_bytes, ssc_stream_t stream);
+
+/* The same convolution in three steps whose results have different lifetimes, for callers
+ * that run several convolutions over one rulebook (the reference caches the rulebook under
+ * an indice_key, ss_conv/sp_ops/conv.py:124-136, and rebuilds everything else per call;
+ * its backward pass walks the same pairs again, src/conv/indice_conv.h:344-426):
+ *   ssc_conv_plan_build: the row-block schedule of the kernel (what ssc_conv_fwd_* derives
+ *     from the pairs on every call).  The plan stays valid while pairs, pair_num, n_out,
+ *     kernel_volume, c_in, c_out, elem_bytes (4: float, 2: half), `inverse` and the number
+ *     of feature rows n_in stay the same; `scratch` is needed during the call only.
+ *     flags: SSC_CONV_PAIRS_CANONICAL as for ssc_conv_fwd_f32.
+ *   ssc_conv_pack_filters_*: the filters in the kernel's fragment order; valid while the
+ *     filter values stay the same.
+ *   ssc_conv_run_*: the MFMA kernel alone.  Results are bit-identical to ssc_conv_fwd_*.
+ * Pairs with one scatter row twice inside an offset are not supported by either form (a
+ * rulebook never has them). */
+size_t ssc_conv_plan_bytes(int64_t n_out, int32_t kernel_volume, int32_t c_in, int32_t c_out,
+                           int64_t pair_stride);
+size_t ssc_conv_plan_scratch_bytes(int64_t n_out, int32_t kernel_volume, int32_t c_in,
+                                   int32_t c_out, int64_t pair_stride);
+size_t ssc_conv_packed_bytes(int32_t kernel_volume, int32_t c_in, int32_t c_out);
+int ssc_conv_plan_build(const int32_t *pairs /* [K,2,pair_stride] */, int64_t pair_stride,
+                        const int32_t *pair_num /* [K] device */, int32_t kernel_volume,
+                        int32_t inverse, int32_t flags, int64_t n_in, int64_t n_out, int32_t c_in,
+                        int32_t c_out, int32_t elem_bytes, void *plan, size_t plan_bytes,
+                        void *scratch, size_t scratch_bytes, ssc_stream_t stream);
+int ssc_conv_pack_filters_f32(const float *filters, int64_t fs_k, int64_t fs_ci, int64_t fs_co,
+                              int32_t kernel_volume, int32_t c_in, int32_t c_out, void *packed,
+                              size_t packed_bytes, ssc_stream_t stream);
+int ssc_conv_pack_filters_f16(const void *filters, int64_t fs_k, int64_t fs_ci, int64_t fs_co,
+                              int32_t kernel_volume, int32_t c_in, int32_t c_out, void *packed,
+                              size_t packed_bytes, ssc_stream_t stream);
+int ssc_conv_run_f32(const float *features /* [n_in,c_in] */, int64_t n_in, int32_t c_in,
+                     const void *packed, size_t packed_bytes, const void *plan, size_t plan_bytes,
+                     int64_t pair_stride, int32_t kernel_volume, int32_t c_out,
+                     float *out /* [n_out,c_out] */, int64_t n_out, ssc_stream_t stream);
+int ssc_conv_run_f16(const void *features /* [n_in,c_in] half */, int64_t n_in, int32_t c_in,
+                     const void *packed, size_t packed_bytes, const void *plan, size_t plan_bytes,
+                     int64_t pair_stride, int32_t kernel_volume, int32_t c_out,
+                     void *out /* [n_out,c_out] half */, int64_t n_out, ssc_stream_t stream);
 
 /* ----------------------------------------------------------------------
  * Gradients of the sparse convolution -- replaces indice_conv_backward_fp32
@@ -288,8 +351,8 @@ int ssc_segment_max_bwd_f32(const float *out_grad, const int32_t *out_idx /* arg
  * ssc_unique_*: sorted unique rows of an int32 [n,4] (b,x,y,z) table with the
  *   inverse map and counts; stands in for torch.unique(dim=0, return_inverse,
  *   return_counts) at voxelize.py:88.  count SYNCHRONISES `stream`.
- *   Coordinates must satisfy 0 <= b < dims[0], 0 <= x < dims[1], ... and
- *   prod(dims) < 2^31.
+ *   Coordinates must satisfy 0 <= b < dims[0], 0 <= x < dims[1], ... (a row that does
+ *   not is left out and the counting call returns SSC_EINVAL) and prod(dims) < 2^31.
  * ssc_voxel_map: replaces voxel2point_map (src/voxelize/voxel2point.cpp:12-18,
  *   src/voxelize/voxel2point_cuda_kernel.cu:16-42).  out_maps must be
  *   pre-initialised as the reference's caller does (functional.py:344-349).

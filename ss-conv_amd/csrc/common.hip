@@ -39,7 +39,7 @@ int fill_f32(float *p, int64_t n, float v, hipStream_t s) {
 size_t bit_table_bytes(int64_t n_bits) {
   int64_t w = bit_words(n_bits);
   int64_t nb = ceil_div(w, kScanBlockWords);
-  return align_up(w * 4) * 2 + align_up((nb + 1) * 4) + align_up(8);
+  return align_up(w * 4) * 2 + align_up((nb + 1) * 4) + align_up(4 * sizeof(int32_t));
 }
 
 BitTable bit_table_carve(Carver &c, int64_t n_bits) {
@@ -49,15 +49,15 @@ BitTable bit_table_carve(Carver &c, int64_t n_bits) {
   t.bits = c.take<uint32_t>(t.n_words);
   t.prefix = c.take<int32_t>(t.n_words);
   t.blocksum = c.take<int32_t>(t.n_scan_blocks + 1);
-  t.total = c.take<int32_t>(2);  // [1]: a flag word for the table's user
+  t.total = c.take<int32_t>(4);  // [1]: flag word, [2], [3]: for the table's user
   return t;
 }
 
-// bits[] = 0 and total[0..1] = 0 in one launch.
+// bits[] = 0 and total[0..3] = 0 in one launch.
 __global__ void __launch_bounds__(256)
     bit_clear_kernel(uint32_t *__restrict__ bits, int64_t n_words, int32_t *__restrict__ total) {
   int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i < 2) total[i] = 0;
+  if (i < 4) total[i] = 0;
   const int64_t step = (int64_t)gridDim.x * blockDim.x;
   for (; i < n_words; i += step) bits[i] = 0u;
 }
@@ -150,16 +150,40 @@ int bit_table_scan(const BitTable &t, hipStream_t s) {
   return SSC_OK;
 }
 
-int read_back_view(const void **view, const void *src_dev, size_t bytes, hipStream_t s) {
-  static thread_local char *pinned = nullptr;
+// The pinned block and the event of the calling host thread.
+struct ReadBack {
+  char *pinned = nullptr;
+  hipEvent_t done = nullptr;
+  bool pending = false;
+};
+static thread_local ReadBack g_read_back;
+
+int read_back_begin(const void *src_dev, size_t bytes, hipStream_t s) {
+  ReadBack &r = g_read_back;
   SSC_CHECK(bytes <= kReadBackBytes, SSC_EINVAL, "read-back of %zu bytes exceeds the pinned block",
             bytes);
-  if (pinned == nullptr)
-    SSC_HIP(hipHostMalloc((void **)&pinned, kReadBackBytes, hipHostMallocPortable));
-  if (bytes > 0) SSC_HIP(hipMemcpyAsync(pinned, src_dev, bytes, hipMemcpyDeviceToHost, s));
-  SSC_HIP(hipStreamSynchronize(s));
-  *view = pinned;
+  if (r.pinned == nullptr)
+    SSC_HIP(hipHostMalloc((void **)&r.pinned, kReadBackBytes, hipHostMallocPortable));
+  if (r.done == nullptr) SSC_HIP(hipEventCreateWithFlags(&r.done, hipEventDisableTiming));
+  if (bytes > 0) SSC_HIP(hipMemcpyAsync(r.pinned, src_dev, bytes, hipMemcpyDeviceToHost, s));
+  SSC_HIP(hipEventRecord(r.done, s));
+  r.pending = true;
   return SSC_OK;
+}
+
+int read_back_end(const void **view) {
+  ReadBack &r = g_read_back;
+  SSC_CHECK(r.pending, SSC_ERUNTIME, "no read-back was started on this thread");
+  r.pending = false;
+  SSC_HIP(hipEventSynchronize(r.done));
+  *view = r.pinned;
+  return SSC_OK;
+}
+
+int read_back_view(const void **view, const void *src_dev, size_t bytes, hipStream_t s) {
+  int rc = read_back_begin(src_dev, bytes, s);
+  if (rc != SSC_OK) return rc;
+  return read_back_end(view);
 }
 
 int read_back(void *dst_host, const void *src_dev, size_t bytes, hipStream_t s) {

@@ -84,7 +84,7 @@ __device__ __forceinline__ void pack_filter_element(const PackArgs &a, int64_t i
 template <typename IO>
 __global__ void __launch_bounds__(256) pack_filters_kernel(PackArgs a, int32_t *__restrict__ flag) {
   int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (idx == 0) flag[0] = 0;  // the pair-order flag of the kernels that follow
+  if (idx == 0 && flag != nullptr) flag[0] = 0;  // the pair-order flag of the kernels that follow
   if (idx < (int64_t)a.K * a.ncb * a.nch * 1024) pack_filter_element<IO>(a, idx);
 }
 
@@ -1247,23 +1247,54 @@ static ConvPlan make_plan(int64_t n_in, int64_t n_out, int K, int c_in, int c_ou
   return p;
 }
 
+// Device buffers of a convolution call, in three groups with different lifetimes:
+//   packed   the filters in MFMA fragment order: as long as the filters keep their values;
+//   plan     what the convolution kernel reads besides features and filters (the row-block
+//            schedule and the tile ranges of the workgroups): as long as the rulebook, the
+//            channel counts, the element type and the direction (`inverse`) stay the same;
+//   scratch  intermediate tables of the kernels that build the plan: until it is built.
 struct ConvWs {
-  float *packed;
+  void *packed;
+  // plan
+  int32_t *tile_grp, *wg_tile;
+  int32_t *sched_in, *sched_out, *grp_meta;
+  // scratch
   int32_t *flag;
   int32_t *segs;
   int32_t *sorted;
   uint32_t *bits;
   int32_t *prefix;
-  int32_t *tile_cnt, *tile_nmb, *kofs, *tile_grp, *wg_tile;
+  int32_t *tile_cnt, *tile_nmb, *kofs;
   int32_t *fine_segs, *range_row0, *tile_row0, *n_tiles_dev;
   int32_t *spill_end, *tile_slot0, *spill, *share_first, *share_cnt;
-  int32_t *sched_in, *sched_out, *grp_meta;
 };
 
-static size_t conv_ws_walk(void *base, const ConvPlan &p, int K, int64_t pair_stride, ConvWs *w) {
+// 4 KiB per fragment for either element type (half fragments use the first half).
+static size_t conv_packed_bytes(const ConvPlan &p, int K) {
+  return align_up((size_t)K * p.ncb * p.nch * 4096);
+}
+
+static size_t conv_plan_walk(void *base, const ConvPlan &p, ConvWs *w) {
+  Carver c(base);
+  int32_t *tile_grp = c.take<int32_t>((size_t)p.n_tiles + 1);
+  int32_t *wg_tile = c.take<int32_t>((size_t)p.n_wg + 1);
+  int32_t *sched_in = c.take<int32_t>((size_t)p.grp_cap * 64);
+  int32_t *sched_out = c.take<int32_t>((size_t)p.grp_cap * 64);
+  int32_t *grp_meta = c.take<int32_t>((size_t)p.grp_cap * 8);
+  if (w) {
+    w->tile_grp = tile_grp;
+    w->wg_tile = wg_tile;
+    w->sched_in = sched_in;
+    w->sched_out = sched_out;
+    w->grp_meta = grp_meta;
+  }
+  return c.used;
+}
+
+static size_t conv_scratch_walk(void *base, const ConvPlan &p, int K, int64_t pair_stride,
+                                ConvWs *w) {
   Carver c(base);
   ConvWs t;
-  t.packed = c.take<float>((size_t)K * p.ncb * p.nch * 1024);
   t.flag = c.take<int32_t>(1);
   t.segs = c.take<int32_t>((size_t)(p.n_tiles + 1) * K);
   t.sorted = c.take<int32_t>((size_t)K * 2 * pair_stride);
@@ -1272,8 +1303,6 @@ static size_t conv_ws_walk(void *base, const ConvPlan &p, int K, int64_t pair_st
   t.tile_cnt = c.take<int32_t>((size_t)p.n_tiles);
   t.tile_nmb = c.take<int32_t>((size_t)p.n_tiles);
   t.kofs = c.take<int32_t>((size_t)p.n_tiles * K);
-  t.tile_grp = c.take<int32_t>((size_t)p.n_tiles + 1);
-  t.wg_tile = c.take<int32_t>((size_t)p.n_wg + 1);
   t.fine_segs = c.take<int32_t>((size_t)(p.n_fine + 1) * K);
   t.range_row0 = c.take<int32_t>((size_t)p.n_wg + 1);
   t.tile_row0 = c.take<int32_t>((size_t)p.n_tiles + 1);
@@ -1283,11 +1312,37 @@ static size_t conv_ws_walk(void *base, const ConvPlan &p, int K, int64_t pair_st
   t.share_first = c.take<int32_t>((size_t)p.n_tiles * K);
   t.share_cnt = c.take<int32_t>((size_t)p.n_tiles * K);
   t.n_tiles_dev = c.take<int32_t>(1);
-  t.sched_in = c.take<int32_t>((size_t)p.grp_cap * 64);
-  t.sched_out = c.take<int32_t>((size_t)p.grp_cap * 64);
-  t.grp_meta = c.take<int32_t>((size_t)p.grp_cap * 8);
-  if (w) *w = t;
+  if (w) {
+    w->flag = t.flag;
+    w->segs = t.segs;
+    w->sorted = t.sorted;
+    w->bits = t.bits;
+    w->prefix = t.prefix;
+    w->tile_cnt = t.tile_cnt;
+    w->tile_nmb = t.tile_nmb;
+    w->kofs = t.kofs;
+    w->fine_segs = t.fine_segs;
+    w->range_row0 = t.range_row0;
+    w->tile_row0 = t.tile_row0;
+    w->spill_end = t.spill_end;
+    w->tile_slot0 = t.tile_slot0;
+    w->spill = t.spill;
+    w->share_first = t.share_first;
+    w->share_cnt = t.share_cnt;
+    w->n_tiles_dev = t.n_tiles_dev;
+  }
   return c.used;
+}
+
+// The one-workspace form of ssc_conv_fwd_*: packed | plan | scratch.
+static size_t conv_ws_walk(void *base, const ConvPlan &p, int K, int64_t pair_stride, ConvWs *w) {
+  char *b = static_cast<char *>(base);
+  size_t used = 0;
+  if (w) w->packed = b;
+  used += conv_packed_bytes(p, K);
+  used += conv_plan_walk(b ? b + used : nullptr, p, w);
+  used += conv_scratch_walk(b ? b + used : nullptr, p, K, pair_stride, w);
+  return used;
 }
 
 static size_t conv_ws_bytes(int64_t n_out, int K, int c_in, int c_out, int64_t pair_stride) {
@@ -1380,43 +1435,29 @@ template <typename IO> static int fill_zero(IO *p, int64_t n, hipStream_t s) {
   return SSC_OK;
 }
 
-// The forward convolution for features, filters and output of element type IO.
-template <typename IO>
-static int conv_fwd(const IO *features, int64_t n_in, int32_t c_in, const IO *filters,
-                    int64_t fs_k, int64_t fs_ci, int64_t fs_co, int32_t c_out,
-                    const int32_t *pairs, int64_t pair_stride, const int32_t *pair_num,
-                    int32_t kernel_volume, int32_t inverse, int32_t subm, IO *out, int64_t n_out,
-                    void *workspace, size_t workspace_bytes, ssc_stream_t stream) {
-  const int K = kernel_volume;
-  SSC_CHECK(K >= 1 && K <= SSC_MAX_KERNEL_VOLUME, SSC_ERUNTIME, "kernel volume %d out of range", K);
-  SSC_CHECK(c_in >= 1 && c_out >= 1, SSC_EINVAL, "channel counts must be positive");
-  SSC_CHECK(n_in >= 0 && n_out >= 0 && pair_stride >= 0, SSC_EINVAL, "negative size");
-  SSC_CHECK(n_out < ((int64_t)1 << 31) && n_in < ((int64_t)1 << 31), SSC_EINVAL,
-            "row counts must fit 31 bits");
-  if (n_out == 0) return SSC_OK;
-  SSC_CHECK(out != nullptr, SSC_EINVAL, "out is NULL");
-  hipStream_t s = (hipStream_t)stream;
-  if (pair_stride == 0 || n_in == 0) return fill_zero(out, n_out * c_out, s);
-  SSC_CHECK(features && filters && pairs && pair_num && workspace, SSC_EINVAL,
-            "NULL pointer argument");
-  size_t need = conv_ws_bytes(n_out, K, c_in, c_out, pair_stride);
-  SSC_CHECK(workspace_bytes >= need, SSC_EWORKSPACE, "conv workspace too small: %zu < %zu",
-            workspace_bytes, need);
-
-  ConvPlan p = make_plan(n_in, n_out, K, c_in, c_out, pair_stride, (int)sizeof(IO));
-  ConvWs w;
-  conv_ws_walk(workspace, p, K, pair_stride, &w);
+// Enqueue the kernels that build the plan of a convolution over `pairs` into w (plan and
+// scratch parts).  `pack`, when given, is packed on the way: beside the first kernel of the
+// work split for canonical pairs, by a launch of its own otherwise.  PACK_IO: element type
+// of the filters to pack (float when there is nothing to pack).
+template <typename PACK_IO>
+static int conv_plan_build(const ConvPlan &p, const ConvWs &w, const int32_t *pairs,
+                           int64_t pair_stride, const int32_t *pair_num, int K, int inverse,
+                           bool in_order, int c_in, int64_t n_out, int elem_bytes,
+                           const PackArgs *pack, hipStream_t s) {
   const int plane_g = inverse ? 1 : 0;
   const int plane_s = 1 - plane_g;
-  int rc;
-
-  const int64_t packed_n = (int64_t)K * p.ncb * p.nch * 1024;
-  const PackArgs pack = {filters, fs_k, fs_ci, fs_co, K, c_in, c_out, p.ncb, p.nch, w.packed};
-  const bool in_order = (subm & SSC_CONV_PAIRS_CANONICAL) != 0;
+  const int64_t packed_n = pack ? (int64_t)K * p.ncb * p.nch * 1024 : 0;
+  PackArgs pk = {nullptr, 0, 0, 0, 0, 0, 0, 0, 0, nullptr};
+  if (pack) pk = *pack;
   if (!in_order) {  // otherwise the filters are packed beside the first kernel of the split
-    hipLaunchKernelGGL(pack_filters_kernel<IO>, dim3((unsigned)ceil_div(packed_n, 256)), dim3(256),
-                       0, s, pack, w.flag);
-    SSC_LAUNCH_CHECK("pack_filters");
+    if (pack) {
+      hipLaunchKernelGGL(pack_filters_kernel<PACK_IO>, dim3((unsigned)ceil_div(packed_n, 256)),
+                         dim3(256), 0, s, pk, w.flag);
+      SSC_LAUNCH_CHECK("pack_filters");
+    } else {
+      int rc = fill_i32(w.flag, 1, 0, s);
+      if (rc != SSC_OK) return rc;
+    }
   }
 
   dim3 pair_grid((unsigned)ceil_div(pair_stride, 256), (unsigned)K);
@@ -1440,13 +1481,13 @@ static int conv_fwd(const IO *features, int64_t n_in, int32_t c_in, const IO *fi
 
   // work split on the fine grid, then the tiles and their segments
   dim3 seg_grid = pair_grid;
-  if (in_order) {
-    int64_t rows = ceil_div(ceil_div(packed_n, 256), pair_grid.x);
+  if (in_order) {  // extra rows: pack the filters (if any) and clear flag[0]
+    int64_t rows = ceil_div(ceil_div(packed_n > 0 ? packed_n : 1, 256), pair_grid.x);
     seg_grid.y += (unsigned)(rows < 4096 ? rows : 4096);
   }
-  hipLaunchKernelGGL(grid_segments_kernel<IO>, seg_grid, dim3(256), 0, s, w.flag, in_order ? 1 : 0,
-                     pairs, w.sorted, pair_stride, plane_s, pair_num, K, p.n_fine, kSplitGranule,
-                     w.fine_segs, pack);
+  hipLaunchKernelGGL(grid_segments_kernel<PACK_IO>, seg_grid, dim3(256), 0, s, w.flag,
+                     in_order ? 1 : 0, pairs, w.sorted, pair_stride, plane_s, pair_num, K, p.n_fine,
+                     kSplitGranule, w.fine_segs, pk);
   hipLaunchKernelGGL(split_bounds_kernel, dim3((unsigned)ceil_div(p.n_fine + 1, 256)), dim3(256), 0,
                      s, w.fine_segs, K, p.n_fine, n_out, p.tile_rows, p.n_wg, w.range_row0);
   hipLaunchKernelGGL(split_rows_kernel, dim3(1), dim3(256), 0, s, w.range_row0, n_out, p.tile_rows,
@@ -1464,17 +1505,23 @@ static int conv_fwd(const IO *features, int64_t n_in, int32_t c_in, const IO *fi
                      w.share_cnt, K, w.n_tiles_dev, w.tile_cnt, w.tile_nmb, w.kofs);
   hipLaunchKernelGGL(sched_scan_kernel, dim3(1), dim3(kScanThreads), 0, s, w.tile_cnt,
                      w.n_tiles_dev, w.tile_grp);
+  const int frag_bytes = elem_bytes == 2 ? Io<_Float16>::kFragBytes : Io<float>::kFragBytes;
   hipLaunchKernelGGL(sched_fill_kernel, dim3((unsigned)ceil_div(p.n_tiles * K * 16, 256)),
                      dim3(256), 0, s, w.flag, pairs, w.sorted, pair_stride, plane_g,
                      w.share_first, w.share_cnt, w.kofs, w.tile_nmb, w.tile_grp, K,
                      w.n_tiles_dev, w.tile_row0, w.tile_slot0, p.T,
-                     p.gather ? (uint32_t)c_in * (uint32_t)sizeof(IO) : 1u,
-                     p.gather ? kGatherPad : 0xFFFFFFFFu,
-                     (16 * p.ncw + 4) * 4, p.ncb * p.nch * Io<IO>::kFragBytes, w.sched_in,
-                     w.sched_out,
-                     w.grp_meta);
+                     p.gather ? (uint32_t)c_in * (uint32_t)elem_bytes : 1u,
+                     p.gather ? kGatherPad : 0xFFFFFFFFu, (16 * p.ncw + 4) * 4,
+                     p.ncb * p.nch * frag_bytes, w.sched_in, w.sched_out, w.grp_meta);
   SSC_LAUNCH_CHECK("schedule");
+  return SSC_OK;
+}
 
+// Enqueue the convolution kernel over a built plan and packed filters.
+template <typename IO>
+static int conv_run(const ConvPlan &p, const ConvWs &w, const IO *features, int64_t n_in, int c_in,
+                    int K, IO *out, int c_out, hipStream_t s) {
+  int rc;
   const bool prof = g_profile_on;
   const int slot = g_profile_count % kProfileRing;
   if (prof) SSC_HIP(hipEventRecord(g_profile_ev[slot][0], s));
@@ -1505,6 +1552,86 @@ static int conv_fwd(const IO *features, int64_t n_in, int32_t c_in, const IO *fi
   return SSC_OK;
 }
 
+static int conv_check_sizes(int K, int c_in, int c_out, int64_t n_in, int64_t n_out,
+                            int64_t pair_stride) {
+  SSC_CHECK(K >= 1 && K <= SSC_MAX_KERNEL_VOLUME, SSC_ERUNTIME, "kernel volume %d out of range", K);
+  SSC_CHECK(c_in >= 1 && c_out >= 1, SSC_EINVAL, "channel counts must be positive");
+  SSC_CHECK(n_in >= 0 && n_out >= 0 && pair_stride >= 0, SSC_EINVAL, "negative size");
+  SSC_CHECK(n_out < ((int64_t)1 << 31) && n_in < ((int64_t)1 << 31), SSC_EINVAL,
+            "row counts must fit 31 bits");
+  return SSC_OK;
+}
+
+// The forward convolution for features, filters and output of element type IO.
+template <typename IO>
+static int conv_fwd(const IO *features, int64_t n_in, int32_t c_in, const IO *filters,
+                    int64_t fs_k, int64_t fs_ci, int64_t fs_co, int32_t c_out,
+                    const int32_t *pairs, int64_t pair_stride, const int32_t *pair_num,
+                    int32_t kernel_volume, int32_t inverse, int32_t subm, IO *out, int64_t n_out,
+                    void *workspace, size_t workspace_bytes, ssc_stream_t stream) {
+  const int K = kernel_volume;
+  int rc = conv_check_sizes(K, c_in, c_out, n_in, n_out, pair_stride);
+  if (rc != SSC_OK) return rc;
+  if (n_out == 0) return SSC_OK;
+  SSC_CHECK(out != nullptr, SSC_EINVAL, "out is NULL");
+  hipStream_t s = (hipStream_t)stream;
+  if (pair_stride == 0 || n_in == 0) return fill_zero(out, n_out * c_out, s);
+  SSC_CHECK(features && filters && pairs && pair_num && workspace, SSC_EINVAL,
+            "NULL pointer argument");
+  size_t need = conv_ws_bytes(n_out, K, c_in, c_out, pair_stride);
+  SSC_CHECK(workspace_bytes >= need, SSC_EWORKSPACE, "conv workspace too small: %zu < %zu",
+            workspace_bytes, need);
+
+  ConvPlan p = make_plan(n_in, n_out, K, c_in, c_out, pair_stride, (int)sizeof(IO));
+  ConvWs w;
+  conv_ws_walk(workspace, p, K, pair_stride, &w);
+  const PackArgs pack = {filters, fs_k, fs_ci, fs_co, K, c_in, c_out, p.ncb, p.nch, w.packed};
+  const bool in_order = (subm & SSC_CONV_PAIRS_CANONICAL) != 0;
+  rc = conv_plan_build<IO>(p, w, pairs, pair_stride, pair_num, K, inverse, in_order, c_in, n_out,
+                           (int)sizeof(IO), &pack, s);
+  if (rc != SSC_OK) return rc;
+  return conv_run<IO>(p, w, features, n_in, c_in, K, out, c_out, s);
+}
+
+template <typename IO>
+static int conv_pack(const IO *filters, int64_t fs_k, int64_t fs_ci, int64_t fs_co, int K, int c_in,
+                     int c_out, void *packed, size_t packed_bytes, hipStream_t s) {
+  int rc = conv_check_sizes(K, c_in, c_out, 0, 0, 0);
+  if (rc != SSC_OK) return rc;
+  SSC_CHECK(filters != nullptr && packed != nullptr, SSC_EINVAL, "NULL pointer argument");
+  ConvPlan p = make_plan(0, 1, K, c_in, c_out, 0, (int)sizeof(IO));
+  SSC_CHECK(packed_bytes >= conv_packed_bytes(p, K), SSC_EWORKSPACE,
+            "buffer of the packed filters too small: %zu < %zu", packed_bytes,
+            conv_packed_bytes(p, K));
+  const PackArgs pack = {filters, fs_k, fs_ci, fs_co, K, c_in, c_out, p.ncb, p.nch, packed};
+  const int64_t packed_n = (int64_t)K * p.ncb * p.nch * 1024;
+  hipLaunchKernelGGL(pack_filters_kernel<IO>, dim3((unsigned)ceil_div(packed_n, 256)), dim3(256), 0,
+                     s, pack, (int32_t *)nullptr);
+  SSC_LAUNCH_CHECK("pack_filters");
+  return SSC_OK;
+}
+
+template <typename IO>
+static int conv_planned(const IO *features, int64_t n_in, int32_t c_in, const void *packed,
+                        size_t packed_bytes, const void *plan, size_t plan_bytes, int64_t pair_stride,
+                        int32_t K, int32_t c_out, IO *out, int64_t n_out, hipStream_t s) {
+  int rc = conv_check_sizes(K, c_in, c_out, n_in, n_out, pair_stride);
+  if (rc != SSC_OK) return rc;
+  if (n_out == 0) return SSC_OK;
+  SSC_CHECK(out != nullptr, SSC_EINVAL, "out is NULL");
+  if (pair_stride == 0 || n_in == 0) return fill_zero(out, n_out * c_out, s);
+  SSC_CHECK(features && packed && plan, SSC_EINVAL, "NULL pointer argument");
+  ConvPlan p = make_plan(n_in, n_out, K, c_in, c_out, pair_stride, (int)sizeof(IO));
+  SSC_CHECK(packed_bytes >= conv_packed_bytes(p, K), SSC_EWORKSPACE,
+            "buffer of the packed filters too small");
+  SSC_CHECK(plan_bytes >= conv_plan_walk(nullptr, p, nullptr), SSC_EWORKSPACE,
+            "plan buffer too small");
+  ConvWs w = {};
+  w.packed = const_cast<void *>(packed);
+  conv_plan_walk(const_cast<void *>(plan), p, &w);
+  return conv_run<IO>(p, w, features, n_in, c_in, K, out, c_out, s);
+}
+
 extern "C" {
 
 int ssc_conv_fwd_f32(const float *features, int64_t n_in, int32_t c_in, const float *filters,
@@ -1528,5 +1655,80 @@ int ssc_conv_fwd_f16(const void *features, int64_t n_in, int32_t c_in, const voi
                             static_cast<const _Float16 *>(filters), fs_k, fs_ci, fs_co, c_out,
                             pairs, pair_stride, pair_num, kernel_volume, inverse, subm,
                             static_cast<_Float16 *>(out), n_out, workspace, workspace_bytes, stream);
+}
+
+size_t ssc_conv_packed_bytes(int32_t kernel_volume, int32_t c_in, int32_t c_out) {
+  if (kernel_volume < 1 || c_in < 1 || c_out < 1) return 0;
+  return conv_packed_bytes(make_plan(0, 1, kernel_volume, c_in, c_out, 0), kernel_volume);
+}
+
+size_t ssc_conv_plan_bytes(int64_t n_out, int32_t kernel_volume, int32_t c_in, int32_t c_out,
+                           int64_t pair_stride) {
+  if (n_out < 0 || kernel_volume < 1 || c_in < 1 || c_out < 1 || pair_stride < 0) return 0;
+  return conv_plan_walk(nullptr, make_plan(0, n_out, kernel_volume, c_in, c_out, pair_stride),
+                        nullptr);
+}
+
+size_t ssc_conv_plan_scratch_bytes(int64_t n_out, int32_t kernel_volume, int32_t c_in,
+                                   int32_t c_out, int64_t pair_stride) {
+  if (n_out < 0 || kernel_volume < 1 || c_in < 1 || c_out < 1 || pair_stride < 0) return 0;
+  return conv_scratch_walk(nullptr, make_plan(0, n_out, kernel_volume, c_in, c_out, pair_stride),
+                           kernel_volume, pair_stride, nullptr);
+}
+
+int ssc_conv_plan_build(const int32_t *pairs, int64_t pair_stride, const int32_t *pair_num,
+                        int32_t kernel_volume, int32_t inverse, int32_t flags, int64_t n_in,
+                        int64_t n_out, int32_t c_in, int32_t c_out, int32_t elem_bytes, void *plan,
+                        size_t plan_bytes, void *scratch, size_t scratch_bytes,
+                        ssc_stream_t stream) {
+  const int K = kernel_volume;
+  int rc = conv_check_sizes(K, c_in, c_out, n_in, n_out, pair_stride);
+  if (rc != SSC_OK) return rc;
+  SSC_CHECK(elem_bytes == 4 || elem_bytes == 2, SSC_EINVAL, "elem_bytes must be 4 or 2");
+  if (n_out == 0 || pair_stride == 0 || n_in == 0) return SSC_OK;  // nothing to schedule
+  SSC_CHECK(pairs && pair_num && plan && scratch, SSC_EINVAL, "NULL pointer argument");
+  ConvPlan p = make_plan(n_in, n_out, K, c_in, c_out, pair_stride, elem_bytes);
+  SSC_CHECK(plan_bytes >= conv_plan_walk(nullptr, p, nullptr), SSC_EWORKSPACE,
+            "plan buffer too small");
+  SSC_CHECK(scratch_bytes >= conv_scratch_walk(nullptr, p, K, pair_stride, nullptr),
+            SSC_EWORKSPACE, "plan scratch too small");
+  ConvWs w = {};
+  conv_plan_walk(plan, p, &w);
+  conv_scratch_walk(scratch, p, K, pair_stride, &w);
+  return conv_plan_build<float>(p, w, pairs, pair_stride, pair_num, K, inverse,
+                                (flags & SSC_CONV_PAIRS_CANONICAL) != 0, c_in, n_out, elem_bytes,
+                                nullptr, (hipStream_t)stream);
+}
+
+int ssc_conv_pack_filters_f32(const float *filters, int64_t fs_k, int64_t fs_ci, int64_t fs_co,
+                              int32_t kernel_volume, int32_t c_in, int32_t c_out, void *packed,
+                              size_t packed_bytes, ssc_stream_t stream) {
+  return conv_pack<float>(filters, fs_k, fs_ci, fs_co, kernel_volume, c_in, c_out, packed,
+                          packed_bytes, (hipStream_t)stream);
+}
+
+int ssc_conv_pack_filters_f16(const void *filters, int64_t fs_k, int64_t fs_ci, int64_t fs_co,
+                              int32_t kernel_volume, int32_t c_in, int32_t c_out, void *packed,
+                              size_t packed_bytes, ssc_stream_t stream) {
+  return conv_pack<_Float16>(static_cast<const _Float16 *>(filters), fs_k, fs_ci, fs_co,
+                             kernel_volume, c_in, c_out, packed, packed_bytes,
+                             (hipStream_t)stream);
+}
+
+int ssc_conv_run_f32(const float *features, int64_t n_in, int32_t c_in, const void *packed,
+                     size_t packed_bytes, const void *plan, size_t plan_bytes, int64_t pair_stride,
+                     int32_t kernel_volume, int32_t c_out, float *out, int64_t n_out,
+                     ssc_stream_t stream) {
+  return conv_planned<float>(features, n_in, c_in, packed, packed_bytes, plan, plan_bytes,
+                             pair_stride, kernel_volume, c_out, out, n_out, (hipStream_t)stream);
+}
+
+int ssc_conv_run_f16(const void *features, int64_t n_in, int32_t c_in, const void *packed,
+                     size_t packed_bytes, const void *plan, size_t plan_bytes, int64_t pair_stride,
+                     int32_t kernel_volume, int32_t c_out, void *out, int64_t n_out,
+                     ssc_stream_t stream) {
+  return conv_planned<_Float16>(static_cast<const _Float16 *>(features), n_in, c_in, packed,
+                                packed_bytes, plan, plan_bytes, pair_stride, kernel_volume, c_out,
+                                static_cast<_Float16 *>(out), n_out, (hipStream_t)stream);
 }
 }

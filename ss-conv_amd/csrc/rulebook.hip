@@ -88,6 +88,27 @@ __device__ __forceinline__ bool row_before(const int4 &a, const int4 &b) {
   return a.w < b.w;
 }
 
+// Flag word of a table (total[1]): bit 0 = the rows do not come in strictly ascending key
+// order; bit 1 = some row lies outside the grid.  Such a row is skipped by every kernel (its
+// key would address memory outside the table), and the host turns the bit into an error.
+constexpr int kFlagDisorder = 1;
+constexpr int kFlagBadRow = 2;
+
+// A regular convolution reaches only output cells inside the grid whatever the spatial
+// coordinates of a row are, so only its batch index must be checked; a submanifold
+// rulebook and the unique-rows table use the row's own cell.
+__device__ __forceinline__ bool batch_in_range(const int32_t *row, const Geom &g) {
+  return (unsigned)row[0] < (unsigned)g.batch;
+}
+__device__ __forceinline__ bool cell_in_range(const int4 &r, int d0, int d1, int d2, int d3) {
+  return (unsigned)r.x < (unsigned)d0 && (unsigned)r.y < (unsigned)d1 &&
+         (unsigned)r.z < (unsigned)d2 && (unsigned)r.w < (unsigned)d3;
+}
+__device__ __forceinline__ bool row_usable(const int32_t *row, const Geom &g) {
+  if (!g.subm) return batch_in_range(row, g);
+  return cell_in_range(*reinterpret_cast<const int4 *>(row), g.batch, g.os[0], g.os[1], g.os[2]);
+}
+
 // Regular conv: mark every output cell reachable from an active input, and count
 // the pairs of every 64-row chunk (chunk_count is [K, n_chunks]; for a regular
 // convolution a pair exists wherever the geometry allows it, so the counts do not
@@ -105,12 +126,16 @@ __global__ void __launch_bounds__(256)
   if (chunk >= n_chunks) return;
   const int lane = threadIdx.x & 63;
   int64_t i = chunk * 64 + lane;
-  const bool live = i < n_in;
+  bool live = i < n_in;
   int32_t row[4] = {0, 0, 0, 0};
   if (live) *reinterpret_cast<int4 *>(row) = reinterpret_cast<const int4 *>(indices)[i];
   if (blockIdx.y == 0 && i + 1 < n_in &&
       !row_before(*reinterpret_cast<int4 *>(row), reinterpret_cast<const int4 *>(indices)[i + 1]))
-    atomicOr(disorder, 1);
+    atomicOr(disorder, kFlagDisorder);
+  if (live && !batch_in_range(row, g)) {
+    if (blockIdx.y == 0) atomicOr(disorder, kFlagBadRow);
+    live = false;
+  }
   // blockIdx.y = kx: the taps of one x offset per wave, for more waves in flight
   const int kx = blockIdx.y;
   int k = kx * g.ks[1] * g.ks[2];
@@ -144,13 +169,17 @@ __global__ void __launch_bounds__(256)
 
 // Submanifold / unique: mark the cells of the rows themselves.
 __global__ void __launch_bounds__(256)
-    mark_rows_kernel(const int32_t *__restrict__ coords, int64_t n, int d1, int d2, int d3,
-                     uint32_t *__restrict__ bits, int32_t *__restrict__ disorder) {
+    mark_rows_kernel(const int32_t *__restrict__ coords, int64_t n, int d0, int d1, int d2, int d3,
+                     uint32_t *__restrict__ bits, int32_t *__restrict__ flags, int want_order) {
   int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= n) return;
   int4 r = reinterpret_cast<const int4 *>(coords)[i];
-  if (disorder && i + 1 < n && !row_before(r, reinterpret_cast<const int4 *>(coords)[i + 1]))
-    atomicOr(disorder, 1);
+  if (want_order && i + 1 < n && !row_before(r, reinterpret_cast<const int4 *>(coords)[i + 1]))
+    atomicOr(flags, kFlagDisorder);
+  if (!cell_in_range(r, d0, d1, d2, d3)) {
+    atomicOr(flags, kFlagBadRow);
+    return;
+  }
   uint32_t key = (uint32_t)(((r.x * d1 + r.y) * d2 + r.z) * d3 + r.w);
   atomicOr(&bits[key >> 5], 1u << (key & 31u));
 }
@@ -206,6 +235,7 @@ __global__ void __launch_bounds__(256)
   int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= n_in) return;
   int4 r = reinterpret_cast<const int4 *>(indices)[i];
+  if (!cell_in_range(r, g.batch, g.os[0], g.os[1], g.os[2])) return;
   uint32_t key = (uint32_t)(((r.x * g.os[0] + r.y) * g.os[1] + r.z) * g.os[2] + r.w);
   rank2row[bit_rank(bits, prefix, key)] = (int32_t)i;
 }
@@ -228,6 +258,7 @@ __global__ void __launch_bounds__(256)
   bool live = i < n_in;
   int32_t row[4] = {0, 0, 0, 0};
   if (live) *reinterpret_cast<int4 *>(row) = reinterpret_cast<const int4 *>(indices)[i];
+  live = live && row_usable(row, g);
   for (int k = 0; k < g.K; ++k) {
     uint32_t key;
     bool ok = live && pair_key(g, row, k, &key);
@@ -302,6 +333,7 @@ __global__ void __launch_bounds__(256)
   bool live = i < n_in;
   int32_t row[4] = {0, 0, 0, 0};
   if (live) *reinterpret_cast<int4 *>(row) = reinterpret_cast<const int4 *>(indices)[i];
+  const bool usable = live && row_usable(row, g);  // (a row outside the grid owns no pair)
   // The taps of one (kx, ky) differ in z only: their cells are neighbours in the key
   // space, so the table word and its prefix are loaded once per word, not per tap.
   uint32_t word = 0xFFFFFFFFu, wbits = 0u;
@@ -311,7 +343,7 @@ __global__ void __launch_bounds__(256)
   int k = kx * g.ks[1] * g.ks[2];
   {
     int ox = 0;
-    const bool okx = live && tap_to_out(row[1], kx, g.st[0], g.pd[0], g.dl[0], g.os[0], &ox);
+    const bool okx = usable && tap_to_out(row[1], kx, g.st[0], g.pd[0], g.dl[0], g.os[0], &ox);
     for (int ky = 0; ky < g.ks[1]; ++ky) {
       int oy = 0;
       const bool okxy = okx && tap_to_out(row[2], ky, g.st[1], g.pd[1], g.dl[1], g.os[1], &oy);
@@ -351,7 +383,8 @@ __global__ void __launch_bounds__(256)
 // final value sees that value, so the maximum over all rows of (count seen + 1) is it
 // (one atomic per wave).
 __global__ void __launch_bounds__(256)
-    inverse_counts_kernel(const int32_t *__restrict__ coords, int64_t n, int d1, int d2, int d3,
+    inverse_counts_kernel(const int32_t *__restrict__ coords, int64_t n, int d0, int d1, int d2,
+                          int d3,
                           const uint32_t *__restrict__ bits, const int32_t *__restrict__ prefix,
                           int32_t *__restrict__ inverse, int32_t *__restrict__ counts,
                           int32_t *__restrict__ max_count) {
@@ -359,10 +392,14 @@ __global__ void __launch_bounds__(256)
   int seen = 0;
   if (i < n) {
     int4 r = reinterpret_cast<const int4 *>(coords)[i];
-    uint32_t key = (uint32_t)(((r.x * d1 + r.y) * d2 + r.z) * d3 + r.w);
-    int rk = bit_rank(bits, prefix, key);
-    inverse[i] = rk;
-    if (counts) seen = atomicAdd(&counts[rk], 1) + 1;
+    if (cell_in_range(r, d0, d1, d2, d3)) {
+      uint32_t key = (uint32_t)(((r.x * d1 + r.y) * d2 + r.z) * d3 + r.w);
+      int rk = bit_rank(bits, prefix, key);
+      inverse[i] = rk;
+      if (counts) seen = atomicAdd(&counts[rk], 1) + 1;
+    } else {
+      inverse[i] = -1;  // a row outside the grid: the call reports it
+    }
   }
   if (max_count) {
 #pragma unroll
@@ -401,6 +438,82 @@ static RulebookWs rulebook_ws_carve(void *ws, const Geom &g, int64_t n_in) {
 
 using namespace ssc;
 
+// ---- host side of the rulebook ------------------------------------------------------------
+static int rulebook_check(const ssc_geometry *g, Geom *gg, const int32_t *indices, int64_t n_in,
+                          const void *workspace, size_t workspace_bytes) {
+  int rc = make_geom(g, gg);
+  if (rc != SSC_OK) return rc;
+  SSC_CHECK(n_in >= 0, SSC_EINVAL, "n_in is negative");
+  SSC_CHECK(n_in * gg->K < ((int64_t)1 << 40), SSC_EINVAL, "n_in * kernel volume too large");
+  if (n_in == 0) return SSC_OK;
+  SSC_CHECK(indices != nullptr && workspace != nullptr, SSC_EINVAL, "NULL pointer argument");
+  SSC_CHECK(workspace_bytes >= rulebook_ws_bytes(*gg, n_in), SSC_EWORKSPACE,
+            "rulebook workspace too small: %zu < %zu", workspace_bytes,
+            rulebook_ws_bytes(*gg, n_in));
+  return SSC_OK;
+}
+
+// Enqueue: clear the table, mark the output cells (counting the pairs of every chunk on the
+// way for a regular convolution), scan.  Afterwards total[0] = number of marked cells,
+// total[1] = flags.
+static int rulebook_mark_and_scan(const int32_t *indices, int64_t n_in, const Geom &gg,
+                                  const RulebookWs &w, hipStream_t s) {
+  int rc;
+  if ((rc = bit_table_clear(w.table, s)) != SSC_OK) return rc;
+  if (gg.subm) {
+    hipLaunchKernelGGL(mark_rows_kernel, dim3((unsigned)ceil_div(n_in, 256)), dim3(256), 0, s,
+                       indices, n_in, gg.batch, gg.os[0], gg.os[1], gg.os[2], w.table.bits,
+                       w.table.total + 1, 1);
+    SSC_LAUNCH_CHECK("mark_rows");
+  } else {
+    hipLaunchKernelGGL(mark_count_kernel,
+                       dim3((unsigned)ceil_div(w.n_chunks, 4), (unsigned)gg.ks[0]), dim3(256), 0, s,
+                       indices, n_in, gg, w.table.bits, w.chunk_count, w.n_chunks,
+                       w.table.total + 1);
+    SSC_LAUNCH_CHECK("mark_count");
+  }
+  return bit_table_scan(w.table, s);
+}
+
+// Enqueue: the pair lists and, with out_indices, the output rows (one launch for both).
+static int rulebook_pairs(const int32_t *indices, int64_t n_in, const Geom &gg,
+                          const RulebookWs &w, int32_t *out_indices, int32_t *pairs,
+                          int32_t *pair_num, hipStream_t s) {
+  unsigned chunk_blocks = (unsigned)ceil_div(w.n_chunks, 4);
+  if (gg.subm) {  // a regular convolution's counts were taken while marking the table
+    hipLaunchKernelGGL(rank_to_row_kernel, dim3((unsigned)ceil_div(n_in, 256)), dim3(256), 0, s,
+                       indices, n_in, gg, w.table.bits, w.table.prefix, w.rank2row);
+    SSC_LAUNCH_CHECK("rank_to_row");
+    hipLaunchKernelGGL(count_pairs_kernel, dim3(chunk_blocks), dim3(256), 0, s, indices, n_in, gg,
+                       w.table.bits, w.chunk_count, w.n_chunks);
+    SSC_LAUNCH_CHECK("count_pairs");
+  }
+  hipLaunchKernelGGL(scan_chunks_kernel, dim3(gg.K), dim3(kScanThreads), 0, s, w.chunk_count,
+                     w.n_chunks, pair_num);
+  SSC_LAUNCH_CHECK("scan_chunks");
+  // rows of the grid beyond the kernel's x extent write out_indices[] (see the kernel)
+  int64_t row_blocks = (gg.subm || out_indices == nullptr)
+                           ? 0
+                           : ceil_div(ceil_div(w.table.n_words, 256), chunk_blocks);
+  if (row_blocks > 4096) row_blocks = 4096;
+  hipLaunchKernelGGL(write_pairs_kernel, dim3(chunk_blocks, (unsigned)(gg.ks[0] + row_blocks)),
+                     dim3(256), 0, s, indices, n_in, gg, w.table.bits, w.table.prefix, w.rank2row,
+                     w.chunk_count, w.n_chunks, pair_num, pairs, w.table.n_words, out_indices);
+  SSC_LAUNCH_CHECK("write_pairs");
+  return SSC_OK;
+}
+
+// The two totals as the host sees them.
+static int rulebook_totals(const int32_t *host, const Geom &gg, int64_t n_in, int32_t *n_out_host,
+                           int32_t *in_order_host) {
+  SSC_CHECK((host[1] & kFlagBadRow) == 0, SSC_EINVAL,
+            "an input row lies outside the grid (batch index not in [0, %d)%s)", gg.batch,
+            gg.subm ? ", or a coordinate outside the spatial shape" : "");
+  *n_out_host = gg.subm ? (int32_t)n_in : host[0];
+  *in_order_host = (host[1] & kFlagDisorder) == 0 ? 1 : 0;
+  return SSC_OK;
+}
+
 extern "C" {
 
 size_t ssc_rulebook_workspace_bytes(const ssc_geometry *g, int64_t n_in) {
@@ -421,82 +534,87 @@ int ssc_rulebook_count_ordered(const int32_t *indices, int64_t n_in, const ssc_g
                                void *workspace, size_t workspace_bytes, int32_t *n_out_host,
                                int32_t *in_order_host, ssc_stream_t stream) {
   Geom gg;
-  int rc = make_geom(g, &gg);
+  int rc = rulebook_check(g, &gg, indices, n_in, workspace, workspace_bytes);
   if (rc != SSC_OK) return rc;
   SSC_CHECK(n_out_host != nullptr && in_order_host != nullptr, SSC_EINVAL,
             "n_out_host or in_order_host is NULL");
-  SSC_CHECK(n_in >= 0, SSC_EINVAL, "n_in is negative");
-  SSC_CHECK(n_in * gg.K < ((int64_t)1 << 40), SSC_EINVAL, "n_in * kernel volume too large");
   if (n_in == 0) {  // src/conv/indice_cuda_functor.cu:262-263
     *n_out_host = 0;
     *in_order_host = 1;
     return SSC_OK;
   }
-  SSC_CHECK(indices != nullptr && workspace != nullptr, SSC_EINVAL, "NULL pointer argument");
-  SSC_CHECK(workspace_bytes >= rulebook_ws_bytes(gg, n_in), SSC_EWORKSPACE,
-            "rulebook workspace too small: %zu < %zu", workspace_bytes,
-            rulebook_ws_bytes(gg, n_in));
   hipStream_t s = (hipStream_t)stream;
   RulebookWs w = rulebook_ws_carve(workspace, gg, n_in);
-  // total[0]: the table's popcount (written by the scan); total[1]: the disorder flag,
-  // cleared with the table and set by the marking kernel.
-  if ((rc = bit_table_clear(w.table, s)) != SSC_OK) return rc;
-  if (gg.subm) {
-    hipLaunchKernelGGL(mark_rows_kernel, dim3((unsigned)ceil_div(n_in, 256)), dim3(256), 0, s,
-                       indices, n_in, gg.os[0], gg.os[1], gg.os[2], w.table.bits,
-                       w.table.total + 1);
-    SSC_LAUNCH_CHECK("mark_rows");
-  } else {
-    hipLaunchKernelGGL(mark_count_kernel,
-                       dim3((unsigned)ceil_div(w.n_chunks, 4), (unsigned)gg.ks[0]), dim3(256), 0, s,
-                       indices, n_in, gg, w.table.bits, w.chunk_count, w.n_chunks,
-                       w.table.total + 1);
-    SSC_LAUNCH_CHECK("mark_count");
-  }
-  if ((rc = bit_table_scan(w.table, s)) != SSC_OK) return rc;
+  if ((rc = rulebook_mark_and_scan(indices, n_in, gg, w, s)) != SSC_OK) return rc;
   int32_t host[2];
   if ((rc = read_back(host, w.table.total, sizeof(host), s)) != SSC_OK) return rc;
-  *n_out_host = gg.subm ? (int32_t)n_in : host[0];
-  *in_order_host = host[1] == 0 ? 1 : 0;
-  return SSC_OK;
+  return rulebook_totals(host, gg, n_in, n_out_host, in_order_host);
 }
 
 int ssc_rulebook_emit(const int32_t *indices, int64_t n_in, const ssc_geometry *g,
                       void *workspace, size_t workspace_bytes, int32_t *out_indices,
                       int32_t *pairs, int32_t *pair_num, ssc_stream_t stream) {
   Geom gg;
-  int rc = make_geom(g, &gg);
+  int rc = rulebook_check(g, &gg, indices, n_in, workspace, workspace_bytes);
   if (rc != SSC_OK) return rc;
   hipStream_t s = (hipStream_t)stream;
   SSC_CHECK(pair_num != nullptr, SSC_EINVAL, "pair_num is NULL");
   if (n_in == 0) return fill_i32(pair_num, gg.K, 0, s);
-  SSC_CHECK(indices != nullptr && workspace != nullptr && pairs != nullptr, SSC_EINVAL,
-            "NULL pointer argument");
+  SSC_CHECK(pairs != nullptr, SSC_EINVAL, "pairs is NULL");
   SSC_CHECK(gg.subm || out_indices != nullptr, SSC_EINVAL, "out_indices is NULL");
+  RulebookWs w = rulebook_ws_carve(workspace, gg, n_in);
+  return rulebook_pairs(indices, n_in, gg, w, out_indices, pairs, pair_num, s);
+}
+
+int ssc_rulebook_begin(const int32_t *indices, int64_t n_in, const ssc_geometry *g,
+                       void *workspace, size_t workspace_bytes, int32_t *pairs, int32_t *pair_num,
+                       ssc_stream_t stream) {
+  Geom gg;
+  int rc = rulebook_check(g, &gg, indices, n_in, workspace, workspace_bytes);
+  if (rc != SSC_OK) return rc;
+  hipStream_t s = (hipStream_t)stream;
+  SSC_CHECK(pair_num != nullptr, SSC_EINVAL, "pair_num is NULL");
+  if (n_in == 0) return fill_i32(pair_num, gg.K, 0, s);
+  SSC_CHECK(pairs != nullptr, SSC_EINVAL, "pairs is NULL");
+  RulebookWs w = rulebook_ws_carve(workspace, gg, n_in);
+  if ((rc = rulebook_mark_and_scan(indices, n_in, gg, w, s)) != SSC_OK) return rc;
+  // the totals start their way to the host now; the pair lists, whose size does not depend
+  // on them, are computed while they travel and the host wakes up
+  if ((rc = read_back_begin(w.table.total, 2 * sizeof(int32_t), s)) != SSC_OK) return rc;
+  return rulebook_pairs(indices, n_in, gg, w, nullptr, pairs, pair_num, s);
+}
+
+int ssc_rulebook_finish(const ssc_geometry *g, int64_t n_in, int32_t *n_out_host,
+                        int32_t *in_order_host) {
+  Geom gg;
+  int rc = make_geom(g, &gg);
+  if (rc != SSC_OK) return rc;
+  SSC_CHECK(n_out_host != nullptr && in_order_host != nullptr, SSC_EINVAL,
+            "n_out_host or in_order_host is NULL");
+  if (n_in == 0) {
+    *n_out_host = 0;
+    *in_order_host = 1;
+    return SSC_OK;
+  }
+  const void *view;
+  if ((rc = read_back_end(&view)) != SSC_OK) return rc;
+  return rulebook_totals(static_cast<const int32_t *>(view), gg, n_in, n_out_host, in_order_host);
+}
+
+int ssc_rulebook_rows(const ssc_geometry *g, int64_t n_in, void *workspace, size_t workspace_bytes,
+                      int32_t *out_indices, ssc_stream_t stream) {
+  Geom gg;
+  int rc = make_geom(g, &gg);
+  if (rc != SSC_OK) return rc;
+  if (n_in == 0 || gg.subm) return SSC_OK;
+  SSC_CHECK(workspace != nullptr && out_indices != nullptr, SSC_EINVAL, "NULL pointer argument");
   SSC_CHECK(workspace_bytes >= rulebook_ws_bytes(gg, n_in), SSC_EWORKSPACE,
             "rulebook workspace too small");
   RulebookWs w = rulebook_ws_carve(workspace, gg, n_in);
-  unsigned chunk_blocks = (unsigned)ceil_div(w.n_chunks, 4);
-  if (gg.subm) {
-    hipLaunchKernelGGL(rank_to_row_kernel, dim3((unsigned)ceil_div(n_in, 256)), dim3(256), 0, s,
-                       indices, n_in, gg, w.table.bits, w.table.prefix, w.rank2row);
-    SSC_LAUNCH_CHECK("rank_to_row");
-  }
-  if (gg.subm) {  // a regular convolution's counts were taken while marking the table
-    hipLaunchKernelGGL(count_pairs_kernel, dim3(chunk_blocks), dim3(256), 0, s, indices, n_in, gg,
-                       w.table.bits, w.chunk_count, w.n_chunks);
-    SSC_LAUNCH_CHECK("count_pairs");
-  }
-  hipLaunchKernelGGL(scan_chunks_kernel, dim3(gg.K), dim3(kScanThreads), 0, s, w.chunk_count,
-                     w.n_chunks, pair_num);
-  SSC_LAUNCH_CHECK("scan_chunks");
-  // rows of the grid beyond the kernel's x extent write out_indices[] (see the kernel)
-  int64_t row_blocks = gg.subm ? 0 : ceil_div(ceil_div(w.table.n_words, 256), chunk_blocks);
-  if (row_blocks > 4096) row_blocks = 4096;
-  hipLaunchKernelGGL(write_pairs_kernel, dim3(chunk_blocks, (unsigned)(gg.ks[0] + row_blocks)),
-                     dim3(256), 0, s, indices, n_in, gg, w.table.bits, w.table.prefix, w.rank2row,
-                     w.chunk_count, w.n_chunks, pair_num, pairs, w.table.n_words, out_indices);
-  SSC_LAUNCH_CHECK("write_pairs");
+  hipLaunchKernelGGL(emit_rows_kernel, dim3((unsigned)ceil_div(w.table.n_words, 256)), dim3(256), 0,
+                     (hipStream_t)stream, w.table.bits, w.table.prefix, w.table.n_words, gg.os[0],
+                     gg.os[1], gg.os[2], out_indices);
+  SSC_LAUNCH_CHECK("emit_rows");
   return SSC_OK;
 }
 
@@ -520,6 +638,11 @@ static int unique_check(const int32_t dims[4], int64_t n, const void *ws, size_t
   return SSC_OK;
 }
 
+static int unique_bad_row(const int32_t dims[4]) {
+  return fail(SSC_EINVAL, "a row lies outside the grid of (%d, %d, %d, %d) cells", dims[0], dims[1],
+              dims[2], dims[3]);
+}
+
 int ssc_unique_count(const int32_t *coords, int64_t n, const int32_t dims[4], void *workspace,
                      size_t workspace_bytes, int32_t *n_unique_host, ssc_stream_t stream) {
   int64_t cells;
@@ -535,11 +658,14 @@ int ssc_unique_count(const int32_t *coords, int64_t n, const int32_t dims[4], vo
   BitTable t = bit_table_carve(c, cells);
   if ((rc = bit_table_clear(t, s)) != SSC_OK) return rc;
   hipLaunchKernelGGL(mark_rows_kernel, dim3((unsigned)ceil_div(n, 256)), dim3(256), 0, s, coords,
-                     n, dims[1], dims[2], dims[3], t.bits,
-                     (int32_t *)nullptr);
+                     n, dims[0], dims[1], dims[2], dims[3], t.bits, t.total + 1, 0);
   SSC_LAUNCH_CHECK("mark_rows");
   if ((rc = bit_table_scan(t, s)) != SSC_OK) return rc;
-  return read_back(n_unique_host, t.total, sizeof(int32_t), s);
+  int32_t host[2];
+  if ((rc = read_back(host, t.total, sizeof(host), s)) != SSC_OK) return rc;
+  if (host[1] & kFlagBadRow) return unique_bad_row(dims);
+  *n_unique_host = host[0];
+  return SSC_OK;
 }
 
 int ssc_unique_emit(const int32_t *coords, int64_t n, const int32_t dims[4], void *workspace,
@@ -558,8 +684,8 @@ int ssc_unique_emit(const int32_t *coords, int64_t n, const int32_t dims[4], voi
                      t.bits, t.prefix, t.n_words, dims[1], dims[2], dims[3], unique);
   SSC_LAUNCH_CHECK("emit_rows");
   hipLaunchKernelGGL(inverse_counts_kernel, dim3((unsigned)ceil_div(n, 256)), dim3(256), 0, s,
-                     coords, n, dims[1], dims[2], dims[3], t.bits, t.prefix, inverse, counts,
-                     (int32_t *)nullptr);
+                     coords, n, dims[0], dims[1], dims[2], dims[3], t.bits, t.prefix, inverse,
+                     counts, (int32_t *)nullptr);
   SSC_LAUNCH_CHECK("inverse_counts");
   return SSC_OK;
 }
@@ -579,19 +705,24 @@ int ssc_unique_build(const int32_t *coords, int64_t n, const int32_t dims[4], vo
   hipStream_t s = (hipStream_t)stream;
   Carver c(workspace);
   BitTable t = bit_table_carve(c, cells);
-  // total[0]: the number of distinct rows (written by the scan); total[1]: the largest
-  // count, cleared with the table
+  // total[0]: the number of distinct rows (written by the scan); total[1]: flags;
+  // total[2]: the largest count; all cleared with the table
   if ((rc = bit_table_clear(t, s)) != SSC_OK) return rc;
   hipLaunchKernelGGL(mark_rows_kernel, dim3((unsigned)ceil_div(n, 256)), dim3(256), 0, s, coords,
-                     n, dims[1], dims[2], dims[3], t.bits, (int32_t *)nullptr);
+                     n, dims[0], dims[1], dims[2], dims[3], t.bits, t.total + 1, 0);
   SSC_LAUNCH_CHECK("mark_rows");
   if ((rc = bit_table_scan(t, s)) != SSC_OK) return rc;
   if ((rc = fill_i32(counts, n, 0, s)) != SSC_OK) return rc;
   hipLaunchKernelGGL(inverse_counts_kernel, dim3((unsigned)ceil_div(n, 256)), dim3(256), 0, s,
-                     coords, n, dims[1], dims[2], dims[3], t.bits, t.prefix, inverse, counts,
-                     t.total + 1);
+                     coords, n, dims[0], dims[1], dims[2], dims[3], t.bits, t.prefix, inverse,
+                     counts, t.total + 2);
   SSC_LAUNCH_CHECK("inverse_counts");
-  return read_back(totals_host, t.total, 2 * sizeof(int32_t), s);
+  int32_t host[3];
+  if ((rc = read_back(host, t.total, sizeof(host), s)) != SSC_OK) return rc;
+  if (host[1] & kFlagBadRow) return unique_bad_row(dims);
+  totals_host[0] = host[0];
+  totals_host[1] = host[2];
+  return SSC_OK;
 }
 
 int ssc_unique_rows(const int32_t dims[4], int64_t n, void *workspace, size_t workspace_bytes,

@@ -61,7 +61,7 @@ struct BitTable {
   uint32_t *bits;     // [n_words]
   int32_t *prefix;    // [n_words] exclusive popcount prefix
   int32_t *blocksum;  // [n_scan_blocks]
-  int32_t *total;     // [2]: popcount of the table; a flag word for the table's user
+  int32_t *total;     // [4]: popcount of the table; a flag word; two words for the table's user
   int64_t n_words;
   int64_t n_scan_blocks;
 };
@@ -91,6 +91,11 @@ int fill_f32(float *p, int64_t n, float v, hipStream_t s);
 // `*view` points into that block and holds until the thread's next read-back.
 constexpr size_t kReadBackBytes = 64 << 10;
 int read_back_view(const void **view, const void *src_dev, size_t bytes, hipStream_t s);
+// The same in two steps: read_back_begin queues the copy and an event behind the work on
+// `s` and returns; read_back_end, on the same host thread, waits for that event only, so
+// work queued on `s` after read_back_begin keeps the GPU busy while the host wakes up.
+int read_back_begin(const void *src_dev, size_t bytes, hipStream_t s);
+int read_back_end(const void **view);
 // The same, moved on to `dst_host`.
 int read_back(void *dst_host, const void *src_dev, size_t bytes, hipStream_t s);
 

@@ -42,7 +42,23 @@ _SIGNATURES = {
     "ssc_rulebook_count_ordered": (ctypes.c_int, [_vp, _i64, _gp, _vp, _sz, ctypes.POINTER(_i32),
                                                   ctypes.POINTER(_i32), _vp]),
     "ssc_rulebook_emit": (ctypes.c_int, [_vp, _i64, _gp, _vp, _sz, _vp, _vp, _vp, _vp]),
+    "ssc_rulebook_begin": (ctypes.c_int, [_vp, _i64, _gp, _vp, _sz, _vp, _vp, _vp]),
+    "ssc_rulebook_finish": (ctypes.c_int, [_gp, _i64, ctypes.POINTER(_i32), ctypes.POINTER(_i32)]),
+    "ssc_rulebook_rows": (ctypes.c_int, [_gp, _i64, _vp, _sz, _vp, _vp]),
     "ssc_conv_workspace_bytes": (_sz, [_i64, _i32, _i32, _i32, _i64]),
+    "ssc_conv_plan_bytes": (_sz, [_i64, _i32, _i32, _i32, _i64]),
+    "ssc_conv_plan_scratch_bytes": (_sz, [_i64, _i32, _i32, _i32, _i64]),
+    "ssc_conv_packed_bytes": (_sz, [_i32, _i32, _i32]),
+    "ssc_conv_plan_build": (ctypes.c_int, [_vp, _i64, _vp, _i32, _i32, _i32, _i64, _i64, _i32, _i32,
+                                           _i32, _vp, _sz, _vp, _sz, _vp]),
+    "ssc_conv_pack_filters_f32": (ctypes.c_int, [_vp, _i64, _i64, _i64, _i32, _i32, _i32, _vp, _sz,
+                                                 _vp]),
+    "ssc_conv_pack_filters_f16": (ctypes.c_int, [_vp, _i64, _i64, _i64, _i32, _i32, _i32, _vp, _sz,
+                                                 _vp]),
+    "ssc_conv_run_f32": (ctypes.c_int, [_vp, _i64, _i32, _vp, _sz, _vp, _sz, _i64, _i32, _i32, _vp,
+                                        _i64, _vp]),
+    "ssc_conv_run_f16": (ctypes.c_int, [_vp, _i64, _i32, _vp, _sz, _vp, _sz, _i64, _i32, _i32, _vp,
+                                        _i64, _vp]),
     "ssc_conv_fwd_f32": (ctypes.c_int, [_vp, _i64, _i32, _vp, _i64, _i64, _i64, _i32, _vp, _i64,
                                         _vp, _i32, _i32, _i32, _vp, _i64, _vp, _sz, _vp]),
     "ssc_conv_fwd_f16": (ctypes.c_int, [_vp, _i64, _i32, _vp, _i64, _i64, _i64, _i32, _vp, _i64,
@@ -163,6 +179,31 @@ def _geometry(batch_size, out_shape, ksize, stride, padding, dilation, subm, tra
     return g
 
 
+class RulebookMeta(object):
+    """What the library knows about a pairs tensor that it wrote itself: for which direction
+    the pairs of every offset ascend in the rows that are accumulated into (`canonical`:
+    (forward, inverse)), and the convolution plans built over it so far.  It hangs on the
+    tensor object as ``_ssc_meta`` and counts only while the tensor's version counter stands
+    where it stood when the rulebook was written: an in-place edit of the pairs makes the
+    convolution treat them as pairs of unknown origin."""
+    __slots__ = ("version", "canonical", "plans")
+    MAX_PLANS = 8
+
+    def __init__(self, version, canonical):
+        self.version = version
+        self.canonical = canonical
+        self.plans = {}
+
+
+def rulebook_meta(indice_pairs):
+    """The RulebookMeta of a pairs tensor, or None when it has none that still holds."""
+    meta = getattr(indice_pairs, "_ssc_meta", None)
+    if meta is None or meta.version != indice_pairs._version or \
+            indice_pairs.dtype != torch.int32 or not indice_pairs.is_contiguous():
+        return None
+    return meta
+
+
 def get_indice_pairs_3d(indices, batch_size, out_spatial_shape, spatial_shape, kernel_size, stride,
                         padding, dilation, out_padding, subm, transpose):
     """src/ss_conv_ops.cu:31 / src/conv/indice_conv.h:21-131.
@@ -180,32 +221,35 @@ def get_indice_pairs_3d(indices, batch_size, out_spatial_shape, spatial_shape, k
     dev = indices.device
     g = _geometry(batch_size, out_spatial_shape, kernel_size, stride, padding, dilation, subm,
                   transpose)
+    gref = ctypes.byref(g)
     K = int(kernel_size[0]) * int(kernel_size[1]) * int(kernel_size[2])
-    nbytes = _lib.ssc_rulebook_workspace_bytes(ctypes.byref(g), n)
-    if nbytes == 0:  # geometry rejected: let the count call produce the message
+    nbytes = _lib.ssc_rulebook_workspace_bytes(gref, n)
+    if nbytes == 0:  # geometry rejected: let the first call produce the message
         nbytes = 256
     ws = _workspace(nbytes, dev)
-    n_out = _i32(0)
-    in_order = _i32(0)
-    s = _stream(indices)
-    _check(_lib.ssc_rulebook_count_ordered(_ptr(indices), n, ctypes.byref(g), ws.data_ptr(),
-                                           ws.numel(), ctypes.byref(n_out),
-                                           ctypes.byref(in_order), s))
     pairs = torch.empty((K, 2, n), dtype=torch.int32, device=dev)
     num = torch.empty((K,), dtype=torch.int32, device=dev)
-    # a geometry may leave no output at all (every candidate clipped): the library still
-    # wants a valid pointer, so at least one row is allocated and the result is a slice of it
-    out_buf = None if subm else torch.empty((max(n_out.value, 1), 4), dtype=torch.int32,
-                                            device=dev)
-    outids = indices if subm else out_buf[:n_out.value]
-    _check(_lib.ssc_rulebook_emit(_ptr(indices), n, ctypes.byref(g), ws.data_ptr(), ws.numel(),
-                                  None if subm else out_buf.data_ptr(), _ptr(pairs),
-                                  num.data_ptr(), s))
+    s = _stream(indices)
+    # marking, ranking and the pair lists are queued; the host then waits for the number of
+    # outputs only, while the pair lists are still being written
+    _check(_lib.ssc_rulebook_begin(_ptr(indices), n, gref, ws.data_ptr(), ws.numel(), _ptr(pairs),
+                                   num.data_ptr(), s))
+    n_out = _i32(0)
+    in_order = _i32(0)
+    _check(_lib.ssc_rulebook_finish(gref, n, ctypes.byref(n_out), ctypes.byref(in_order)))
+    if subm:
+        outids = indices
+    else:
+        # a geometry may leave no output at all (every candidate clipped): the library still
+        # wants a valid pointer, so at least one row is allocated and the result is a slice
+        out_buf = torch.empty((max(n_out.value, 1), 4), dtype=torch.int32, device=dev)
+        outids = out_buf[:n_out.value]
+        _check(_lib.ssc_rulebook_rows(gref, n, ws.data_ptr(), ws.numel(), out_buf.data_ptr(), s))
     # Pairs of an offset always ascend in the input rows, and in the output rows too when
     # the input rows came in key order: the convolution may then skip its order check
     # (the first flag serves a call that accumulates into output rows, the second one
     # with `inverse`, which accumulates into input rows).
-    pairs._ssc_canonical = (bool(in_order.value), True)
+    pairs._ssc_meta = RulebookMeta(pairs._version, (bool(in_order.value), True))
     return [outids, pairs, num]
 
 
@@ -225,22 +269,91 @@ def _filter_strides(filters, c_in, c_out):
     return filters, kstr[-1], filters.stride(-2), filters.stride(-1)
 
 
-def _conv_flags(indice_pairs, subm, inverse):
-    """The `subm` argument of ssc_conv_fwd_f32: the reference's flag plus the promise of
-    canonical pair order for rulebooks that get_indice_pairs_3d built."""
-    canonical = getattr(indice_pairs, "_ssc_canonical", (False, False))[1 if inverse else 0] and \
-        indice_pairs.dtype == torch.int32 and indice_pairs.is_contiguous()
-    return int(bool(subm)) | (2 if canonical else 0)
+_ENTRIES = {
+    torch.float32: (_lib.ssc_conv_fwd_f32, _lib.ssc_conv_pack_filters_f32, _lib.ssc_conv_run_f32,
+                    _lib.ssc_conv_bwd_filter_f32),
+    torch.float16: (_lib.ssc_conv_fwd_f16, _lib.ssc_conv_pack_filters_f16, _lib.ssc_conv_run_f16,
+                    _lib.ssc_conv_bwd_filter_f16),
+}
 
 
-def _indice_conv(dtype, entry, name, features, filters, indice_pairs, indice_num, num_act_out,
-                 inverse, subm):
+def _packed_filters(owner, filters, fs, K, c_in, c_out, stream):
+    """The filters in the kernel's fragment order.  The buffers are kept on the tensor the
+    caller passed (`owner`), one per way of reading it (forward, or transposed for the input
+    gradient), and reused while that tensor's version counter stands still: evaluation-mode
+    layers, whose kernel is synthesised once, pack once."""
+    key = (filters.data_ptr(), tuple(fs), K, c_in, c_out)
+    held = getattr(owner, "_ssc_packed", None)
+    if held is None or held[0] != owner._version:
+        held = (owner._version, {})
+        owner._ssc_packed = held
+    packed = held[1].get(key)
+    if packed is None:
+        packed = _workspace(_lib.ssc_conv_packed_bytes(K, c_in, c_out), filters.device)
+        _check(_ENTRIES[filters.dtype][1](_ptr(filters), fs[0], fs[1], fs[2], K, c_in, c_out,
+                                         packed.data_ptr(), packed.numel(), stream))
+        held[1][key] = packed
+    return packed
+
+
+def _planned_conv(meta, features, owner, filters, fs, pairs, num, K, c_in, c_out, n_out, inverse):
+    """out[n_out, c_out] through a cached plan: the schedule is built on the first call of a
+    (direction, channel counts, element type, row counts) combination over this rulebook
+    and reused afterwards; later calls launch the filter packing (unless cached as well)
+    and the MFMA kernel only."""
+    dev = features.device
+    s = _stream(features)
+    n_in = features.size(0)
+    stride = pairs.size(2)
+    eb = features.element_size()
+    key = (bool(inverse), c_in, c_out, eb, n_in, n_out)
+    plan = meta.plans.get(key)
+    if plan is None:
+        plan = _workspace(_lib.ssc_conv_plan_bytes(n_out, K, c_in, c_out, stride), dev)
+        scratch = _workspace(_lib.ssc_conv_plan_scratch_bytes(n_out, K, c_in, c_out, stride), dev)
+        flags = 2 if meta.canonical[1 if inverse else 0] else 0
+        _check(_lib.ssc_conv_plan_build(_ptr(pairs), stride, num.data_ptr(), K, int(bool(inverse)),
+                                        flags, n_in, n_out, c_in, c_out, eb, plan.data_ptr(),
+                                        plan.numel(), scratch.data_ptr(), scratch.numel(), s))
+        if len(meta.plans) >= RulebookMeta.MAX_PLANS:
+            meta.plans.clear()
+        meta.plans[key] = plan
+    packed = _packed_filters(owner, filters, fs, K, c_in, c_out, s)
+    out = torch.empty((n_out, c_out), dtype=features.dtype, device=dev)
+    _check(_ENTRIES[features.dtype][2](_ptr(features), n_in, c_in, packed.data_ptr(),
+                                       packed.numel(), plan.data_ptr(), plan.numel(), stride, K,
+                                       c_out, _ptr(out), n_out, s))
+    return out
+
+
+def _conv_any(features, owner, filters, fs, indice_pairs, pairs, num, K, c_in, c_out, n_out,
+              inverse, subm):
+    """One convolution call: through the rulebook's cached plan when the pairs tensor is one
+    this library wrote, through the one-call entry point (order check, schedule and kernel
+    every time) for pairs of any other origin."""
+    meta = rulebook_meta(indice_pairs)
+    if meta is not None and pairs is indice_pairs:
+        return _planned_conv(meta, features, owner, filters, fs, pairs, num, K, c_in, c_out, n_out,
+                             inverse)
+    out = torch.empty((n_out, c_out), dtype=features.dtype, device=features.device)
+    ws = _workspace(_lib.ssc_conv_workspace_bytes(n_out, K, c_in, c_out, pairs.size(2)),
+                    features.device)
+    _check(_ENTRIES[features.dtype][0](
+        _ptr(features), features.size(0), c_in, _ptr(filters), fs[0], fs[1], fs[2], c_out,
+        _ptr(pairs), pairs.size(2), num.data_ptr(), K, int(bool(inverse)), int(bool(subm)),
+        _ptr(out), n_out, ws.data_ptr(), ws.numel(), _stream(features)))
+    return out
+
+
+def _indice_conv(dtype, name, features, filters, indice_pairs, indice_num, num_act_out, inverse,
+                 subm):
     _need_gpu(features, filters, indice_pairs)
     if features.dtype != dtype or filters.dtype != dtype:
         raise RuntimeError("%s needs %s features and filters" % (name, dtype))
     features = features.contiguous()
     c_in = features.size(1)
     c_out = filters.size(-1)
+    owner = filters
     filters, fs_k, fs_ci, fs_co = _filter_strides(filters, c_in, c_out)
     pairs = indice_pairs.int().contiguous() if indice_pairs.dtype != torch.int32 \
         else indice_pairs.contiguous()
@@ -251,32 +364,25 @@ def _indice_conv(dtype, entry, name, features, filters, indice_pairs, indice_num
         kvol *= d
     if kvol != K:
         raise RuntimeError("filters have %d offsets but the rulebook has %d" % (kvol, K))
-    n_out = int(num_act_out)
-    out = torch.empty((n_out, c_out), dtype=dtype, device=features.device)
-    nbytes = _lib.ssc_conv_workspace_bytes(n_out, K, c_in, c_out, pairs.size(2))
-    ws = _workspace(nbytes, features.device)
-    _check(entry(_ptr(features), features.size(0), c_in, _ptr(filters), fs_k, fs_ci, fs_co, c_out,
-                 _ptr(pairs), pairs.size(2), num.data_ptr(), K, int(inverse),
-                 _conv_flags(indice_pairs, subm, inverse), _ptr(out), n_out, ws.data_ptr(),
-                 ws.numel(), _stream(features)))
-    return out
+    return _conv_any(features, owner, filters, (fs_k, fs_ci, fs_co), indice_pairs, pairs, num, K,
+                     c_in, c_out, int(num_act_out), inverse, subm)
 
 
 def indice_conv_fp32(features, filters, indice_pairs, indice_num, num_act_out, inverse, subm):
     """src/conv/indice_conv.h:247-343 (bound at src/ss_conv_ops_api.cpp:21)."""
-    return _indice_conv(torch.float32, _lib.ssc_conv_fwd_f32, "indice_conv_fp32", features,
-                        filters, indice_pairs, indice_num, num_act_out, inverse, subm)
+    return _indice_conv(torch.float32, "indice_conv_fp32", features, filters, indice_pairs,
+                        indice_num, num_act_out, inverse, subm)
 
 
 def indice_conv_half(features, filters, indice_pairs, indice_num, num_act_out, inverse, subm):
     """indiceConv<at::Half> (src/ss_conv_ops.cu:74-78, bound at src/ss_conv_ops_api.cpp:23):
     half-precision tensors, fp32 arithmetic, one rounding per output element."""
-    return _indice_conv(torch.float16, _lib.ssc_conv_fwd_f16, "indice_conv_half", features,
-                        filters, indice_pairs, indice_num, num_act_out, inverse, subm)
+    return _indice_conv(torch.float16, "indice_conv_half", features, filters, indice_pairs,
+                        indice_num, num_act_out, inverse, subm)
 
 
-def _indice_conv_backward(dtype, fwd_entry, filter_entry, name, features, filters, out_bp,
-                          indice_pairs, indice_num, inverse, subm):
+def _indice_conv_backward(dtype, name, features, filters, out_bp, indice_pairs, indice_num,
+                          inverse, subm):
     _need_gpu(features, filters, out_bp, indice_pairs)
     if features.dtype != dtype or filters.dtype != dtype or out_bp.dtype != dtype:
         raise RuntimeError("%s needs %s tensors" % (name, dtype))
@@ -284,6 +390,7 @@ def _indice_conv_backward(dtype, fwd_entry, filter_entry, name, features, filter
     out_bp = out_bp.contiguous()
     n_in, c_in = features.shape
     n_out, c_out = out_bp.shape
+    owner = filters
     filters, fs_k, fs_ci, fs_co = _filter_strides(filters, c_in, c_out)
     pairs = indice_pairs.int().contiguous() if indice_pairs.dtype != torch.int32 \
         else indice_pairs.contiguous()
@@ -292,35 +399,29 @@ def _indice_conv_backward(dtype, fwd_entry, filter_entry, name, features, filter
     dev = features.device
     s = _stream(features)
     # input gradient: the forward kernel on out_bp, pairs swapped, filters transposed
-    input_bp = torch.empty((n_in, c_in), dtype=dtype, device=dev)
-    ws = _workspace(_lib.ssc_conv_workspace_bytes(n_in, K, c_out, c_in, pairs.size(2)), dev)
-    _check(fwd_entry(_ptr(out_bp), n_out, c_out, _ptr(filters), fs_k, fs_co, fs_ci, c_in,
-                     _ptr(pairs), pairs.size(2), num.data_ptr(), K, 0 if inverse else 1,
-                     _conv_flags(indice_pairs, subm, not inverse), _ptr(input_bp), n_in,
-                     ws.data_ptr(), ws.numel(), s))
+    input_bp = _conv_any(out_bp, owner, filters, (fs_k, fs_co, fs_ci), indice_pairs, pairs, num, K,
+                         c_out, c_in, n_in, not inverse, subm)
     # filter gradient
     filters_bp = torch.empty(tuple(filters.shape), dtype=dtype, device=dev)
     ws2 = _workspace(_lib.ssc_conv_bwd_filter_workspace_bytes(K, c_in, c_out, pairs.size(2)), dev)
-    _check(filter_entry(_ptr(features), n_in, c_in, _ptr(out_bp), n_out, c_out, _ptr(pairs),
-                        pairs.size(2), num.data_ptr(), K, int(inverse), _ptr(filters_bp),
-                        c_in * c_out, c_out, 1, ws2.data_ptr(), ws2.numel(), s))
+    _check(_ENTRIES[dtype][3](_ptr(features), n_in, c_in, _ptr(out_bp), n_out, c_out, _ptr(pairs),
+                              pairs.size(2), num.data_ptr(), K, int(inverse), _ptr(filters_bp),
+                              c_in * c_out, c_out, 1, ws2.data_ptr(), ws2.numel(), s))
     return [input_bp, filters_bp]
 
 
 def indice_conv_backward_fp32(features, filters, out_bp, indice_pairs, indice_num, inverse, subm):
     """src/conv/indice_conv.h:344-426 (bound at src/ss_conv_ops_api.cpp:22): returns
     [input_bp like features, filters_bp shaped like filters]."""
-    return _indice_conv_backward(torch.float32, _lib.ssc_conv_fwd_f32,
-                                 _lib.ssc_conv_bwd_filter_f32, "indice_conv_backward_fp32",
-                                 features, filters, out_bp, indice_pairs, indice_num, inverse, subm)
+    return _indice_conv_backward(torch.float32, "indice_conv_backward_fp32", features, filters,
+                                 out_bp, indice_pairs, indice_num, inverse, subm)
 
 
 def indice_conv_backward_half(features, filters, out_bp, indice_pairs, indice_num, inverse, subm):
     """indiceConvBackward<at::Half> (src/ss_conv_ops.cu:79-83, bound at
     src/ss_conv_ops_api.cpp:24): half-precision tensors, fp32 arithmetic."""
-    return _indice_conv_backward(torch.float16, _lib.ssc_conv_fwd_f16,
-                                 _lib.ssc_conv_bwd_filter_f16, "indice_conv_backward_half",
-                                 features, filters, out_bp, indice_pairs, indice_num, inverse, subm)
+    return _indice_conv_backward(torch.float16, "indice_conv_backward_half", features, filters,
+                                 out_bp, indice_pairs, indice_num, inverse, subm)
 
 
 def _pool_args(features, indice_pairs, indice_num):

@@ -16,6 +16,9 @@ class _ConvBase(Function):
     @classmethod
     def _run(cls, ctx, features, filters, indice_pairs, indice_pair_num, num_activate_out):
         ctx.save_for_backward(indice_pairs, indice_pair_num, features, filters)
+        # what the library noted on the pairs tensor it wrote (order promises, cached plans)
+        # travels with the context, should the saved tensor come back as another object
+        ctx.ssc_meta = getattr(indice_pairs, "_ssc_meta", None)
         return ops.indice_conv_forward(features, filters, indice_pairs, indice_pair_num,
                                        num_activate_out, cls.inverse, cls.subm)
 
@@ -23,6 +26,8 @@ class _ConvBase(Function):
     def _grad(cls, ctx, grad_output):
         """(reference: functional.py:38-43, 60-65, 82-87)"""
         indice_pairs, indice_pair_num, features, filters = ctx.saved_tensors
+        if ctx.ssc_meta is not None and getattr(indice_pairs, "_ssc_meta", None) is None:
+            indice_pairs._ssc_meta = ctx.ssc_meta
         input_bp, filters_bp = ops.indice_conv_backward(
             features, filters, grad_output.contiguous(), indice_pairs, indice_pair_num,
             cls.inverse, cls.subm)

@@ -73,8 +73,10 @@ def test_rulebook_matches_oracle(case, oracle, device):
 @pytest.mark.parametrize("shuffle", [False, True])
 def test_rulebook_count_then_emit_entry_points(case, shuffle, device):
     """The library offers the rulebook in two ways: ssc_rulebook_count(_ordered) followed
-    by ssc_rulebook_emit, and ssc_rulebook_build followed by ssc_rulebook_rows (the one the
-    Python side calls).  Both give the same tensors and the same order flag."""
+    by ssc_rulebook_emit (the host waits for the number of outputs before anything else is
+    queued), and ssc_rulebook_begin / ssc_rulebook_finish / ssc_rulebook_rows (the pair
+    lists are queued before the wait; the one the Python side calls).  Both give the same
+    tensors and the same order flag."""
     import ctypes
     from ss_conv import _ext
     batch, grid, n, k, s, p, d, subm = case
@@ -95,7 +97,7 @@ def test_rulebook_count_then_emit_entry_points(case, shuffle, device):
     assert lib.ssc_rulebook_count_ordered(t.data_ptr(), n, ctypes.byref(g), ws.data_ptr(), nbytes,
                                           ctypes.byref(n_out), ctypes.byref(in_order), None) == 0
     assert n_out.value == want[0].shape[0]
-    assert bool(in_order.value) == want[1]._ssc_canonical[0] == (not shuffle)
+    assert bool(in_order.value) == _ext.rulebook_meta(want[1]).canonical[0] == (not shuffle)
     K = k ** 3
     out = torch.full((max(n_out.value, 1), 4), -7, dtype=torch.int32, device=device)
     pairs = torch.full((K, 2, n), -7, dtype=torch.int32, device=device)
@@ -1145,7 +1147,7 @@ def test_conv_order_promise_follows_the_input_order(oracle, device):
     for idx, f, want_flag in ((idx_sorted, feats, True), (idx_sorted[perm], feats[perm], False)):
         t = torch.from_numpy(idx).to(device)
         o_idx, pairs, num = get_indice_pairs(t, 2, [grid] * 3, k, 1, 1, 1, 0, False)
-        assert pairs._ssc_canonical == (want_flag, True)
+        assert _ext.rulebook_meta(pairs).canonical == (want_flag, True)
         out = _ext.indice_conv_fp32(torch.from_numpy(f).to(device),
                                     torch.from_numpy(w).to(device).reshape(k, k, k, cin, cout),
                                     pairs, num, o_idx.shape[0], 0, 0)
@@ -1288,3 +1290,139 @@ def test_backbone_forward_matches_oracle(oracle, device):
     want = oracle.voxel2point(o_idx, o_feat.astype(np.float32), shape, vp.cpu().numpy(),
                               vi.cpu().numpy(), unit_voxel_extent=[2.0 / s for s in shape])[0]
     assert rel_l2(at_points, want) < REL_L2
+
+
+def test_rows_outside_the_grid_are_reported(device):
+    """A batch index beyond batch_size (regular rulebook), a coordinate equal to the shape
+    (submanifold rulebook) and a row outside dims (unique rows) would address memory outside
+    the bit table: the rows are skipped on the device and the call raises ValueError."""
+    from ss_conv import _ext
+    from ss_conv.sp_ops.ops import get_indice_pairs
+    rng = np.random.default_rng(5)
+    idx = random_voxels(rng, 2, 8, 100)
+    bad_batch = idx.copy()
+    bad_batch[17, 0] = 2
+    with pytest.raises(ValueError, match="outside the grid"):
+        get_indice_pairs(torch.from_numpy(bad_batch).to(device), 2, [8] * 3, 3, 1, 1, 1, 0, False)
+    negative = idx.copy()
+    negative[3, 0] = -1
+    with pytest.raises(ValueError, match="outside the grid"):
+        get_indice_pairs(torch.from_numpy(negative).to(device), 2, [8] * 3, 3, 2, 1, 1, 0, False)
+    on_the_face = idx.copy()
+    on_the_face[40, 2] = 8
+    with pytest.raises(ValueError, match="outside the grid"):
+        get_indice_pairs(torch.from_numpy(on_the_face).to(device), 2, [8] * 3, 3, 1, 1, 1, 0, True)
+    # the same row is fine for a regular convolution: its taps are clipped to the grid
+    t = torch.from_numpy(on_the_face).to(device)
+    o_idx, pairs, num = get_indice_pairs(t, 2, [8] * 3, 3, 1, 1, 1, 0, False)
+    assert int(o_idx[:, 1:].max()) <= 7 and int(o_idx[:, 1:].min()) >= 0
+    with pytest.raises(ValueError, match="outside the grid"):
+        _ext.unique_rows(t, [2, 8, 8, 8])
+    with pytest.raises(ValueError, match="outside the grid"):
+        _ext.unique_rows_max(t, [2, 8, 8, 8])
+    u, inv, cnt, largest = _ext.unique_rows_max(t, [2, 9, 9, 9])
+    assert u.shape[0] == 100 and largest == 1
+    # the good rulebook still works after the failed calls
+    o2, p2, n2 = get_indice_pairs(torch.from_numpy(idx).to(device), 2, [8] * 3, 3, 1, 1, 1, 0, False)
+    assert int(n2.sum()) > 0
+    torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("subm", [False, True])
+def test_cached_plan_gives_identical_results(subm, oracle, device):
+    """Convolutions over one rulebook share the row-block schedule: the second call of a
+    (direction, channel counts) combination reuses the plan built by the first and must
+    return the same bits, as must the one-call entry point; forward, input gradient and a
+    layer with other channel counts each keep their own plan; an in-place edit of the pairs
+    drops the promise."""
+    from ss_conv import _ext
+    from ss_conv.sp_ops.ops import get_indice_pairs
+    rng = np.random.default_rng(31)
+    n, grid, cin, cout, k = 3000, 20, 64, 96, 3
+    idx = random_voxels(rng, 2, grid, n)
+    t = torch.from_numpy(idx).to(device)
+    o_idx, pairs, num = get_indice_pairs(t, 2, [grid] * 3, k, 1, 1, 1, 0, subm)
+    n_out = o_idx.shape[0]
+    meta = _ext.rulebook_meta(pairs)
+    assert meta is not None and meta.canonical == (True, True) and len(meta.plans) == 0
+    f = torch.randn((n, cin), device=device)
+    w = torch.randn((k, k, k, cin, cout), device=device) / (27 * cin) ** 0.5
+    go = torch.randn((n_out, cout), device=device)
+    out1 = _ext.indice_conv_fp32(f, w, pairs, num, n_out, 0, int(subm))
+    assert len(meta.plans) == 1
+    out2 = _ext.indice_conv_fp32(f, w, pairs, num, n_out, 0, int(subm))
+    assert len(meta.plans) == 1 and torch.equal(out1, out2)
+    # a clone carries no promise: order check, schedule and kernel in one call
+    out3 = _ext.indice_conv_fp32(f, w, pairs.clone(), num, n_out, 0, int(subm))
+    assert torch.equal(out1, out3)
+    r_idx, r_pairs, r_num, r_shape = oracle.rulebook(idx, 2, [grid] * 3, k, 1, 1, 1, subm)
+    if not subm:
+        r_idx, r_pairs, r_num = oracle.canonicalize(r_idx, r_pairs, r_num, r_shape)
+    ref = oracle.conv_fwd(f.cpu().numpy(), w.reshape(27, cin, cout).cpu().numpy(), r_pairs, r_num,
+                          n_out, matmul=np.matmul)
+    assert rel_l2(out1.cpu().numpy(), ref) < REL_L2
+    # new filter values, same plan (the filters are packed again)
+    w2 = w * 0.5
+    assert rel_l2(_ext.indice_conv_fp32(f, w2, pairs, num, n_out, 0, int(subm)).cpu().numpy(),
+                  0.5 * ref) < REL_L2
+    # filters changed in place: the packed copy kept on the tensor must not be reused
+    w2.mul_(4.0)
+    assert rel_l2(_ext.indice_conv_fp32(f, w2, pairs, num, n_out, 0, int(subm)).cpu().numpy(),
+                  2.0 * ref) < REL_L2
+    gi1, gw1 = _ext.indice_conv_backward_fp32(f, w, go, pairs, num, 0, int(subm))
+    assert len(meta.plans) == 2
+    gi2, gw2 = _ext.indice_conv_backward_fp32(f, w, go, pairs, num, 0, int(subm))
+    assert len(meta.plans) == 2 and torch.equal(gi1, gi2) and torch.equal(gw1, gw2)
+    gi3, gw3 = _ext.indice_conv_backward_fp32(f, w, go, pairs.clone(), num, 0, int(subm))
+    assert torch.equal(gi1, gi3) and torch.equal(gw1, gw3)
+    ri, rw = oracle.conv_bwd(f.cpu().numpy(), w.reshape(27, cin, cout).cpu().numpy(),
+                             go.cpu().numpy(), r_pairs, r_num)
+    assert rel_l2(gi1.cpu().numpy(), ri) < REL_L2
+    # other channel counts over the same rulebook: a plan of their own
+    fh = torch.randn((n, 24), device=device)
+    wh = torch.randn((k, k, k, 24, 40), device=device)
+    oh = _ext.indice_conv_fp32(fh, wh, pairs, num, n_out, 0, int(subm))
+    assert len(meta.plans) == 3
+    assert torch.equal(oh, _ext.indice_conv_fp32(fh, wh, pairs.clone(), num, n_out, 0, int(subm)))
+    # half precision over the same rulebook
+    o16 = _ext.indice_conv_half(f.half(), w.half(), pairs, num, n_out, 0, int(subm))
+    assert len(meta.plans) == 4
+    assert torch.equal(o16, _ext.indice_conv_half(f.half(), w.half(), pairs.clone(), num, n_out, 0,
+                                                  int(subm)))
+    # an in-place edit of the pairs: the promise and the plans no longer count
+    pairs[:, :, 0] += 0
+    assert _ext.rulebook_meta(pairs) is None
+    assert torch.equal(out1, _ext.indice_conv_fp32(f, w, pairs, num, n_out, 0, int(subm)))
+
+
+def test_layer_reuses_plan_under_an_indice_key(device):
+    """Two submanifold layers under one indice_key, and a second forward of the same layer in
+    evaluation mode: the rulebook, the plan and the packed filters are built once."""
+    from ss_conv import _ext
+    from ss_conv.sp_ops.conv import SparseConvolution
+    from ss_conv.sp_ops.tensor import SparseTensor
+    rng = np.random.default_rng(8)
+    idx = random_voxels(rng, 2, 16, 1500)
+    t = torch.from_numpy(idx).to(device)
+    torch.manual_seed(0)
+    a = SparseConvolution(3, 32, 32, 3, subm=True, bias=False, indice_key="s").to(device).eval()
+    b = SparseConvolution(3, 32, 32, 3, subm=True, bias=False, indice_key="s").to(device).eval()
+    x = torch.randn((idx.shape[0], 32), device=device)
+    with torch.no_grad():
+        st = SparseTensor(x, t, [16] * 3, 2)
+        y = b(a(st))
+        pairs = st.indice_dict["s"][2]
+        meta = _ext.rulebook_meta(pairs)
+        assert meta is not None and len(meta.plans) == 1
+        packed_a = a.weight._ssc_packed[1]
+        st2 = SparseTensor(x, t, [16] * 3, 2)
+        st2.indice_dict = st.indice_dict
+        y2 = b(a(st2))
+        assert len(meta.plans) == 1 and a.weight._ssc_packed[1] is packed_a
+        assert torch.equal(y.features, y2.features)
+        # the layers one by one through the one-call entry point
+        z = _ext.indice_conv_fp32(x, a.weight, pairs.clone(), st.indice_dict["s"][3],
+                                  idx.shape[0], 0, 1)
+        z = _ext.indice_conv_fp32(z, b.weight, pairs.clone(), st.indice_dict["s"][3],
+                                  idx.shape[0], 0, 1)
+        assert torch.equal(z, y.features)
