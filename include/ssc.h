@@ -102,21 +102,27 @@ int ssc_rulebook_emit(const int32_t *indices, int64_t n_in, const ssc_geometry *
 /* The same rulebook with the host's wait moved behind the work that does not depend on the
  * number of outputs (the reference blocks in torch::_unique with the GPU idle,
  * src/conv/indice_conv.h:120):
- *   ssc_rulebook_begin enqueues marking and ranking, starts the copy of the totals to the
- *     host, and then enqueues pairs[K,2,n_in] and pair_num[K], whose sizes are known
- *     beforehand.  It returns without waiting.
+ *   ssc_rulebook_begin enqueues marking and ranking (the totals land in pinned host memory),
+ *     and then pairs[K,2,n_in] and pair_num[K], whose sizes are known beforehand.  With
+ *     out_indices it also writes the output rows; the buffer must then hold
+ *     ssc_rulebook_out_bound() rows (min(n_in * K, batch_size * prod(out_shape)): room for
+ *     any outcome), of which the first n_out are written.  It returns without waiting.
  *   ssc_rulebook_finish, called on the same host thread, waits for the totals only (work
  *     enqueued after ssc_rulebook_begin keeps running) and reports n_out and the input order
  *     as ssc_rulebook_count_ordered does.
- *   ssc_rulebook_rows then writes out_indices[n_out,4] (nothing for subm).
+ *   ssc_rulebook_rows then writes out_indices[n_out,4] for a caller that did not pass
+ *     out_indices to ssc_rulebook_begin (nothing for subm).
+ * One rulebook may be between begin and finish per host thread.
  * A row of `indices` whose batch index lies outside [0, batch_size) -- for subm: whose cell
  * lies outside the grid -- is left out of the rulebook and ssc_rulebook_finish (like
  * ssc_rulebook_count) returns SSC_EINVAL; the reference reads and writes outside its grid
  * buffer for such a row (src/conv/indice_cuda_functor.cu:60-61). */
+size_t ssc_rulebook_out_bound(const ssc_geometry *g, int64_t n_in);
 int ssc_rulebook_begin(const int32_t *indices, int64_t n_in, const ssc_geometry *g,
                        void *workspace, size_t workspace_bytes,
                        int32_t *pairs /* [K,2,n_in] device */, int32_t *pair_num /* [K] device */,
-                       ssc_stream_t stream);
+                       int32_t *out_indices /* [out_capacity,4] device, or NULL */,
+                       int64_t out_capacity, ssc_stream_t stream);
 int ssc_rulebook_finish(const ssc_geometry *g, int64_t n_in, int32_t *n_out_host /* host */,
                         int32_t *in_order_host /* host */);
 int ssc_rulebook_rows(const ssc_geometry *g, int64_t n_in, void *workspace,

@@ -70,43 +70,12 @@ int bit_table_clear(const BitTable &t, hipStream_t s) {
   return SSC_OK;
 }
 
-// Block-wide exclusive scan of one int per thread (kScanThreads threads).
-__device__ __forceinline__ int block_exclusive_scan(int v, int *lds /* [kScanThreads/64 + 1] */,
-                                                    int *block_total) {
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  int incl = v;
-#pragma unroll
-  for (int d = 1; d < 64; d <<= 1) {
-    int o = __shfl_up(incl, d, 64);
-    if (lane >= d) incl += o;
-  }
-  if (lane == 63) lds[wave] = incl;
-  __syncthreads();
-  int wave_off = 0, tot = 0;
-#pragma unroll
-  for (int w = 0; w < kScanThreads / 64; ++w) {
-    int x = lds[w];
-    if (w < wave) wave_off += x;
-    tot += x;
-  }
-  __syncthreads();
-  *block_total = tot;
-  return wave_off + incl - v;
-}
-
 // Pass 1: popcount sum of each block of kScanBlockWords words.
 __global__ void __launch_bounds__(kScanThreads)
     popc_blocksum_kernel(const uint32_t *__restrict__ bits, int64_t n_words,
                          int32_t *__restrict__ blocksum) {
   __shared__ int lds[kScanThreads / 64 + 1];
-  int64_t base = (int64_t)blockIdx.x * kScanBlockWords + (int64_t)threadIdx.x * kScanItems;
-  int v = 0;
-#pragma unroll
-  for (int i = 0; i < kScanItems; ++i)
-    if (base + i < n_words) v += __popc(bits[base + i]);
-  int tot;
-  block_exclusive_scan(v, lds, &tot);
-  if (threadIdx.x == 0) blocksum[blockIdx.x] = tot;
+  popc_blocksum_block(bits, n_words, blockIdx.x, blocksum, lds);
 }
 
 // Pass 2: exclusive prefix per word.  Every block first adds up the sums of the blocks
@@ -115,7 +84,7 @@ __global__ void __launch_bounds__(kScanThreads)
 __global__ void __launch_bounds__(kScanThreads)
     popc_prefix_kernel(const uint32_t *__restrict__ bits, int64_t n_words,
                        const int32_t *__restrict__ blocksum, int32_t *__restrict__ prefix,
-                       int32_t *__restrict__ total) {
+                       int32_t *__restrict__ total, int32_t *__restrict__ mirror) {
   __shared__ int lds[kScanThreads / 64 + 1];
   int before = 0;
   for (int64_t b = threadIdx.x; b < (int64_t)blockIdx.x; b += kScanThreads) before += blocksum[b];
@@ -136,18 +105,30 @@ __global__ void __launch_bounds__(kScanThreads)
     if (base + i < n_words) prefix[base + i] = ex;
     ex += c[i];
   }
-  if (blockIdx.x == gridDim.x - 1 && threadIdx.x == 0) total[0] = block_off + tot;
+  if (blockIdx.x == gridDim.x - 1 && threadIdx.x == 0) {
+    total[0] = block_off + tot;
+    if (mirror != nullptr) {  // total[1..3] were written by kernels before this one
+      mirror[0] = block_off + tot;
+      mirror[1] = total[1];
+      mirror[2] = total[2];
+      mirror[3] = total[3];
+    }
+  }
 }
 
-int bit_table_scan(const BitTable &t, hipStream_t s) {
+int bit_table_scan_prefix(const BitTable &t, hipStream_t s, int32_t *mirror) {
+  hipLaunchKernelGGL(popc_prefix_kernel, dim3((unsigned)t.n_scan_blocks), dim3(kScanThreads), 0, s,
+                     t.bits, t.n_words, t.blocksum, t.prefix, t.total, mirror);
+  SSC_LAUNCH_CHECK("popc_prefix");
+  return SSC_OK;
+}
+
+int bit_table_scan(const BitTable &t, hipStream_t s, int32_t *mirror) {
   if (t.n_words <= 0) return fill_i32(t.total, 1, 0, s);
   hipLaunchKernelGGL(popc_blocksum_kernel, dim3((unsigned)t.n_scan_blocks), dim3(kScanThreads), 0,
                      s, t.bits, t.n_words, t.blocksum);
   SSC_LAUNCH_CHECK("popc_blocksum");
-  hipLaunchKernelGGL(popc_prefix_kernel, dim3((unsigned)t.n_scan_blocks), dim3(kScanThreads), 0, s,
-                     t.bits, t.n_words, t.blocksum, t.prefix, t.total);
-  SSC_LAUNCH_CHECK("popc_prefix");
-  return SSC_OK;
+  return bit_table_scan_prefix(t, s, mirror);
 }
 
 // The pinned block and the event of the calling host thread.
@@ -158,13 +139,40 @@ struct ReadBack {
 };
 static thread_local ReadBack g_read_back;
 
+static int read_back_init(ReadBack &r) {
+  // (pinned memory from hipHostMalloc is mapped into the device's address space at the same
+  // address and coherent with the host at event boundaries)
+  if (r.pinned == nullptr)
+    SSC_HIP(hipHostMalloc((void **)&r.pinned, kReadBackBytes,
+                          hipHostMallocPortable | hipHostMallocMapped));
+  if (r.done == nullptr) SSC_HIP(hipEventCreateWithFlags(&r.done, hipEventDisableTiming));
+  return SSC_OK;
+}
+
+int read_back_mirror(int32_t **mirror) {
+  ReadBack &r = g_read_back;
+  int rc = read_back_init(r);
+  if (rc != SSC_OK) return rc;
+  void *dev = nullptr;
+  SSC_HIP(hipHostGetDevicePointer(&dev, r.pinned, 0));
+  *mirror = static_cast<int32_t *>(dev);
+  return SSC_OK;
+}
+
+int read_back_mirror_queued(hipStream_t s) {
+  ReadBack &r = g_read_back;
+  SSC_CHECK(r.done != nullptr, SSC_ERUNTIME, "read_back_mirror was not called on this thread");
+  SSC_HIP(hipEventRecord(r.done, s));
+  r.pending = true;
+  return SSC_OK;
+}
+
 int read_back_begin(const void *src_dev, size_t bytes, hipStream_t s) {
   ReadBack &r = g_read_back;
   SSC_CHECK(bytes <= kReadBackBytes, SSC_EINVAL, "read-back of %zu bytes exceeds the pinned block",
             bytes);
-  if (r.pinned == nullptr)
-    SSC_HIP(hipHostMalloc((void **)&r.pinned, kReadBackBytes, hipHostMallocPortable));
-  if (r.done == nullptr) SSC_HIP(hipEventCreateWithFlags(&r.done, hipEventDisableTiming));
+  int rc = read_back_init(r);
+  if (rc != SSC_OK) return rc;
   if (bytes > 0) SSC_HIP(hipMemcpyAsync(r.pinned, src_dev, bytes, hipMemcpyDeviceToHost, s));
   SSC_HIP(hipEventRecord(r.done, s));
   r.pending = true;

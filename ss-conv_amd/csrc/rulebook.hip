@@ -269,37 +269,43 @@ __global__ void __launch_bounds__(256)
 }
 
 // Per tap: exclusive scan of the chunk counts in place; the total is pair_num[k].
-__global__ void __launch_bounds__(kScanThreads)
-    scan_chunks_kernel(int32_t *__restrict__ chunk_count, int64_t n_chunks,
-                       int32_t *__restrict__ pair_num) {
-  __shared__ int lds[kScanThreads / 64 + 1];
-  int32_t *c = chunk_count + (int64_t)blockIdx.x * n_chunks;
+__device__ __forceinline__ void scan_chunks_of_tap(int32_t *__restrict__ chunk_count,
+                                                   int64_t n_chunks, int k,
+                                                   int32_t *__restrict__ pair_num, int *lds) {
+  int32_t *c = chunk_count + (int64_t)k * n_chunks;
   int carry = 0;
   for (int64_t base = 0; base < n_chunks; base += kScanThreads) {
     int64_t i = base + threadIdx.x;
     int v = i < n_chunks ? c[i] : 0;
-    // inline block scan (same shape as common.hip's)
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    int incl = v;
-#pragma unroll
-    for (int d = 1; d < 64; d <<= 1) {
-      int o = __shfl_up(incl, d, 64);
-      if (lane >= d) incl += o;
-    }
-    if (lane == 63) lds[wave] = incl;
-    __syncthreads();
-    int wave_off = 0, tot = 0;
-#pragma unroll
-    for (int w = 0; w < kScanThreads / 64; ++w) {
-      int x = lds[w];
-      if (w < wave) wave_off += x;
-      tot += x;
-    }
-    __syncthreads();
-    if (i < n_chunks) c[i] = carry + wave_off + incl - v;
+    int tot;
+    int ex = block_exclusive_scan(v, lds, &tot);
+    if (i < n_chunks) c[i] = carry + ex;
     carry += tot;
   }
-  if (threadIdx.x == 0) pair_num[blockIdx.x] = carry;
+  if (threadIdx.x == 0) pair_num[k] = carry;
+}
+
+__global__ void __launch_bounds__(kScanThreads)
+    scan_chunks_kernel(int32_t *__restrict__ chunk_count, int64_t n_chunks,
+                       int32_t *__restrict__ pair_num) {
+  __shared__ int lds[kScanThreads / 64 + 1];
+  scan_chunks_of_tap(chunk_count, n_chunks, blockIdx.x, pair_num, lds);
+}
+
+// Two jobs that both need nothing but the marking kernel's results, in one launch: blocks
+// below n_scan_blocks run the first pass of the table's popcount scan, the K blocks after
+// them scan the chunk counts of one tap each (regular convolutions only: a submanifold
+// rulebook counts its pairs after the table is ranked).
+__global__ void __launch_bounds__(kScanThreads)
+    blocksum_scan_chunks_kernel(const uint32_t *__restrict__ bits, int64_t n_words,
+                                int32_t *__restrict__ blocksum, int64_t n_scan_blocks,
+                                int32_t *__restrict__ chunk_count, int64_t n_chunks,
+                                int32_t *__restrict__ pair_num) {
+  __shared__ int lds[kScanThreads / 64 + 1];
+  if ((int64_t)blockIdx.x < n_scan_blocks)
+    popc_blocksum_block(bits, n_words, blockIdx.x, blocksum, lds);
+  else
+    scan_chunks_of_tap(chunk_count, n_chunks, (int)(blockIdx.x - n_scan_blocks), pair_num, lds);
 }
 
 // Pair emission: same traversal as count_pairs_kernel; a row's slot inside tap k
@@ -455,9 +461,12 @@ static int rulebook_check(const ssc_geometry *g, Geom *gg, const int32_t *indice
 
 // Enqueue: clear the table, mark the output cells (counting the pairs of every chunk on the
 // way for a regular convolution), scan.  Afterwards total[0] = number of marked cells,
-// total[1] = flags.
+// total[1] = flags, both also in `mirror` when given.  With pair_num, a regular
+// convolution's chunk counts are scanned beside the first pass of the table scan (and
+// rulebook_pairs must be told so).
 static int rulebook_mark_and_scan(const int32_t *indices, int64_t n_in, const Geom &gg,
-                                  const RulebookWs &w, hipStream_t s) {
+                                  const RulebookWs &w, int32_t *pair_num, int32_t *mirror,
+                                  hipStream_t s) {
   int rc;
   if ((rc = bit_table_clear(w.table, s)) != SSC_OK) return rc;
   if (gg.subm) {
@@ -465,20 +474,25 @@ static int rulebook_mark_and_scan(const int32_t *indices, int64_t n_in, const Ge
                        indices, n_in, gg.batch, gg.os[0], gg.os[1], gg.os[2], w.table.bits,
                        w.table.total + 1, 1);
     SSC_LAUNCH_CHECK("mark_rows");
-  } else {
-    hipLaunchKernelGGL(mark_count_kernel,
-                       dim3((unsigned)ceil_div(w.n_chunks, 4), (unsigned)gg.ks[0]), dim3(256), 0, s,
-                       indices, n_in, gg, w.table.bits, w.chunk_count, w.n_chunks,
-                       w.table.total + 1);
-    SSC_LAUNCH_CHECK("mark_count");
+    return bit_table_scan(w.table, s, mirror);
   }
-  return bit_table_scan(w.table, s);
+  hipLaunchKernelGGL(mark_count_kernel, dim3((unsigned)ceil_div(w.n_chunks, 4), (unsigned)gg.ks[0]),
+                     dim3(256), 0, s, indices, n_in, gg, w.table.bits, w.chunk_count, w.n_chunks,
+                     w.table.total + 1);
+  SSC_LAUNCH_CHECK("mark_count");
+  if (pair_num == nullptr) return bit_table_scan(w.table, s, mirror);
+  hipLaunchKernelGGL(blocksum_scan_chunks_kernel, dim3((unsigned)(w.table.n_scan_blocks + gg.K)),
+                     dim3(kScanThreads), 0, s, w.table.bits, w.table.n_words, w.table.blocksum,
+                     w.table.n_scan_blocks, w.chunk_count, w.n_chunks, pair_num);
+  SSC_LAUNCH_CHECK("blocksum_scan_chunks");
+  return bit_table_scan_prefix(w.table, s, mirror);
 }
 
 // Enqueue: the pair lists and, with out_indices, the output rows (one launch for both).
+// chunks_scanned: rulebook_mark_and_scan has scanned the chunk counts already.
 static int rulebook_pairs(const int32_t *indices, int64_t n_in, const Geom &gg,
                           const RulebookWs &w, int32_t *out_indices, int32_t *pairs,
-                          int32_t *pair_num, hipStream_t s) {
+                          int32_t *pair_num, bool chunks_scanned, hipStream_t s) {
   unsigned chunk_blocks = (unsigned)ceil_div(w.n_chunks, 4);
   if (gg.subm) {  // a regular convolution's counts were taken while marking the table
     hipLaunchKernelGGL(rank_to_row_kernel, dim3((unsigned)ceil_div(n_in, 256)), dim3(256), 0, s,
@@ -488,9 +502,11 @@ static int rulebook_pairs(const int32_t *indices, int64_t n_in, const Geom &gg,
                        w.table.bits, w.chunk_count, w.n_chunks);
     SSC_LAUNCH_CHECK("count_pairs");
   }
-  hipLaunchKernelGGL(scan_chunks_kernel, dim3(gg.K), dim3(kScanThreads), 0, s, w.chunk_count,
-                     w.n_chunks, pair_num);
-  SSC_LAUNCH_CHECK("scan_chunks");
+  if (gg.subm || !chunks_scanned) {
+    hipLaunchKernelGGL(scan_chunks_kernel, dim3(gg.K), dim3(kScanThreads), 0, s, w.chunk_count,
+                       w.n_chunks, pair_num);
+    SSC_LAUNCH_CHECK("scan_chunks");
+  }
   // rows of the grid beyond the kernel's x extent write out_indices[] (see the kernel)
   int64_t row_blocks = (gg.subm || out_indices == nullptr)
                            ? 0
@@ -501,6 +517,13 @@ static int rulebook_pairs(const int32_t *indices, int64_t n_in, const Geom &gg,
                      w.chunk_count, w.n_chunks, pair_num, pairs, w.table.n_words, out_indices);
   SSC_LAUNCH_CHECK("write_pairs");
   return SSC_OK;
+}
+
+// An upper bound of the number of outputs that needs no look at the data.
+static int64_t rulebook_out_bound(const Geom &gg, int64_t n_in) {
+  if (gg.subm) return n_in;
+  const int64_t by_pairs = n_in * gg.K, cells = geom_cells(gg);
+  return by_pairs < cells ? by_pairs : cells;
 }
 
 // The two totals as the host sees them.
@@ -545,7 +568,7 @@ int ssc_rulebook_count_ordered(const int32_t *indices, int64_t n_in, const ssc_g
   }
   hipStream_t s = (hipStream_t)stream;
   RulebookWs w = rulebook_ws_carve(workspace, gg, n_in);
-  if ((rc = rulebook_mark_and_scan(indices, n_in, gg, w, s)) != SSC_OK) return rc;
+  if ((rc = rulebook_mark_and_scan(indices, n_in, gg, w, nullptr, nullptr, s)) != SSC_OK) return rc;
   int32_t host[2];
   if ((rc = read_back(host, w.table.total, sizeof(host), s)) != SSC_OK) return rc;
   return rulebook_totals(host, gg, n_in, n_out_host, in_order_host);
@@ -563,12 +586,18 @@ int ssc_rulebook_emit(const int32_t *indices, int64_t n_in, const ssc_geometry *
   SSC_CHECK(pairs != nullptr, SSC_EINVAL, "pairs is NULL");
   SSC_CHECK(gg.subm || out_indices != nullptr, SSC_EINVAL, "out_indices is NULL");
   RulebookWs w = rulebook_ws_carve(workspace, gg, n_in);
-  return rulebook_pairs(indices, n_in, gg, w, out_indices, pairs, pair_num, s);
+  return rulebook_pairs(indices, n_in, gg, w, out_indices, pairs, pair_num, false, s);
+}
+
+size_t ssc_rulebook_out_bound(const ssc_geometry *g, int64_t n_in) {
+  Geom gg;
+  if (n_in < 0 || make_geom(g, &gg) != SSC_OK) return 0;
+  return (size_t)rulebook_out_bound(gg, n_in);
 }
 
 int ssc_rulebook_begin(const int32_t *indices, int64_t n_in, const ssc_geometry *g,
                        void *workspace, size_t workspace_bytes, int32_t *pairs, int32_t *pair_num,
-                       ssc_stream_t stream) {
+                       int32_t *out_indices, int64_t out_capacity, ssc_stream_t stream) {
   Geom gg;
   int rc = rulebook_check(g, &gg, indices, n_in, workspace, workspace_bytes);
   if (rc != SSC_OK) return rc;
@@ -576,12 +605,18 @@ int ssc_rulebook_begin(const int32_t *indices, int64_t n_in, const ssc_geometry 
   SSC_CHECK(pair_num != nullptr, SSC_EINVAL, "pair_num is NULL");
   if (n_in == 0) return fill_i32(pair_num, gg.K, 0, s);
   SSC_CHECK(pairs != nullptr, SSC_EINVAL, "pairs is NULL");
+  SSC_CHECK(out_indices == nullptr || out_capacity >= rulebook_out_bound(gg, n_in), SSC_EINVAL,
+            "out_indices holds %lld rows, fewer than the bound of %lld", (long long)out_capacity,
+            (long long)rulebook_out_bound(gg, n_in));
   RulebookWs w = rulebook_ws_carve(workspace, gg, n_in);
-  if ((rc = rulebook_mark_and_scan(indices, n_in, gg, w, s)) != SSC_OK) return rc;
-  // the totals start their way to the host now; the pair lists, whose size does not depend
-  // on them, are computed while they travel and the host wakes up
-  if ((rc = read_back_begin(w.table.total, 2 * sizeof(int32_t), s)) != SSC_OK) return rc;
-  return rulebook_pairs(indices, n_in, gg, w, nullptr, pairs, pair_num, s);
+  // the kernel that finishes the scan leaves the totals in pinned host memory; the pair
+  // lists (and the output rows, when the caller brought room for any number of them), whose
+  // sizes do not depend on the totals, are computed while the host wakes up
+  int32_t *mirror = nullptr;
+  if ((rc = read_back_mirror(&mirror)) != SSC_OK) return rc;
+  if ((rc = rulebook_mark_and_scan(indices, n_in, gg, w, pair_num, mirror, s)) != SSC_OK) return rc;
+  if ((rc = read_back_mirror_queued(s)) != SSC_OK) return rc;
+  return rulebook_pairs(indices, n_in, gg, w, out_indices, pairs, pair_num, true, s);
 }
 
 int ssc_rulebook_finish(const ssc_geometry *g, int64_t n_in, int32_t *n_out_host,

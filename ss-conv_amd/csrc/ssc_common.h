@@ -71,8 +71,52 @@ size_t bit_table_bytes(int64_t n_bits);
 BitTable bit_table_carve(Carver &c, int64_t n_bits);
 // Enqueue: zero the table.
 int bit_table_clear(const BitTable &t, hipStream_t s);
-// Enqueue: prefix[], total[0] from bits[].
-int bit_table_scan(const BitTable &t, hipStream_t s);
+// Enqueue: prefix[], total[0] from bits[].  With `mirror` (memory the device can write and
+// the host can read, see read_back_mirror), the kernel that writes total[0] also copies
+// total[0..3] there, which saves the copy a host that waits for them would otherwise queue.
+int bit_table_scan(const BitTable &t, hipStream_t s, int32_t *mirror = nullptr);
+// The second pass of bit_table_scan alone (the first one, popc_blocksum_block, is then run
+// by a kernel of the caller that has other work to do beside it).
+int bit_table_scan_prefix(const BitTable &t, hipStream_t s, int32_t *mirror = nullptr);
+
+// Block-wide exclusive scan of one int per thread (kScanThreads threads).
+__device__ __forceinline__ int block_exclusive_scan(int v, int *lds /* [kScanThreads/64 + 1] */,
+                                                    int *block_total) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  int incl = v;
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    int o = __shfl_up(incl, d, 64);
+    if (lane >= d) incl += o;
+  }
+  if (lane == 63) lds[wave] = incl;
+  __syncthreads();
+  int wave_off = 0, tot = 0;
+#pragma unroll
+  for (int w = 0; w < kScanThreads / 64; ++w) {
+    int x = lds[w];
+    if (w < wave) wave_off += x;
+    tot += x;
+  }
+  __syncthreads();
+  *block_total = tot;
+  return wave_off + incl - v;
+}
+
+// First pass of the popcount scan for scan block `b` (kScanThreads threads):
+// blocksum[b] = popcount of the block's kScanBlockWords words.
+__device__ __forceinline__ void popc_blocksum_block(const uint32_t *__restrict__ bits,
+                                                    int64_t n_words, int64_t b,
+                                                    int32_t *__restrict__ blocksum, int *lds) {
+  int64_t base = b * kScanBlockWords + (int64_t)threadIdx.x * kScanItems;
+  int v = 0;
+#pragma unroll
+  for (int i = 0; i < kScanItems; ++i)
+    if (base + i < n_words) v += __popc(bits[base + i]);
+  int tot;
+  block_exclusive_scan(v, lds, &tot);
+  if (threadIdx.x == 0) blocksum[b] = tot;
+}
 
 __device__ __forceinline__ int bit_rank(const uint32_t *__restrict__ bits,
                                         const int32_t *__restrict__ prefix, uint32_t key) {
@@ -96,6 +140,11 @@ int read_back_view(const void **view, const void *src_dev, size_t bytes, hipStre
 // work queued on `s` after read_back_begin keeps the GPU busy while the host wakes up.
 int read_back_begin(const void *src_dev, size_t bytes, hipStream_t s);
 int read_back_end(const void **view);
+// The same without a copy: *mirror is the calling thread's pinned block as the device sees
+// it; a kernel queued on `s` writes its results there, read_back_mirror_queued records the
+// event behind that kernel, and read_back_end waits for it and returns the block.
+int read_back_mirror(int32_t **mirror);
+int read_back_mirror_queued(hipStream_t s);
 // The same, moved on to `dst_host`.
 int read_back(void *dst_host, const void *src_dev, size_t bytes, hipStream_t s);
 

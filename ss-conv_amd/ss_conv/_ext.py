@@ -42,7 +42,8 @@ _SIGNATURES = {
     "ssc_rulebook_count_ordered": (ctypes.c_int, [_vp, _i64, _gp, _vp, _sz, ctypes.POINTER(_i32),
                                                   ctypes.POINTER(_i32), _vp]),
     "ssc_rulebook_emit": (ctypes.c_int, [_vp, _i64, _gp, _vp, _sz, _vp, _vp, _vp, _vp]),
-    "ssc_rulebook_begin": (ctypes.c_int, [_vp, _i64, _gp, _vp, _sz, _vp, _vp, _vp]),
+    "ssc_rulebook_out_bound": (_sz, [_gp, _i64]),
+    "ssc_rulebook_begin": (ctypes.c_int, [_vp, _i64, _gp, _vp, _sz, _vp, _vp, _vp, _i64, _vp]),
     "ssc_rulebook_finish": (ctypes.c_int, [_gp, _i64, ctypes.POINTER(_i32), ctypes.POINTER(_i32)]),
     "ssc_rulebook_rows": (ctypes.c_int, [_gp, _i64, _vp, _sz, _vp, _vp]),
     "ssc_conv_workspace_bytes": (_sz, [_i64, _i32, _i32, _i32, _i64]),
@@ -179,6 +180,11 @@ def _geometry(batch_size, out_shape, ksize, stride, padding, dilation, subm, tra
     return g
 
 
+# Output rows are written before their number is known when a buffer for the largest
+# possible number of them is at most this large (the result then keeps that buffer alive).
+_ROWS_AHEAD_BYTES = 64 << 20
+
+
 class RulebookMeta(object):
     """What the library knows about a pairs tensor that it wrote itself: for which direction
     the pairs of every offset ascend in the rows that are accumulated into (`canonical`:
@@ -230,15 +236,26 @@ def get_indice_pairs_3d(indices, batch_size, out_spatial_shape, spatial_shape, k
     pairs = torch.empty((K, 2, n), dtype=torch.int32, device=dev)
     num = torch.empty((K,), dtype=torch.int32, device=dev)
     s = _stream(indices)
-    # marking, ranking and the pair lists are queued; the host then waits for the number of
-    # outputs only, while the pair lists are still being written
+    # Marking, ranking and the pair lists are queued; the host then waits for the number of
+    # outputs only, while the pair lists are still being written.  When room for any
+    # possible number of output rows is cheap (n * K rows at most), the rows are written in
+    # the same launch as the pairs and the result is a slice of that buffer; otherwise by a
+    # launch of their own once the number is known.
+    out_buf = None
+    if not subm and n > 0:
+        bound = _lib.ssc_rulebook_out_bound(gref, n)
+        if 0 < bound * 16 <= _ROWS_AHEAD_BYTES:
+            out_buf = torch.empty((bound, 4), dtype=torch.int32, device=dev)
     _check(_lib.ssc_rulebook_begin(_ptr(indices), n, gref, ws.data_ptr(), ws.numel(), _ptr(pairs),
-                                   num.data_ptr(), s))
+                                   num.data_ptr(), _ptr(out_buf),
+                                   0 if out_buf is None else out_buf.size(0), s))
     n_out = _i32(0)
     in_order = _i32(0)
     _check(_lib.ssc_rulebook_finish(gref, n, ctypes.byref(n_out), ctypes.byref(in_order)))
     if subm:
         outids = indices
+    elif out_buf is not None:
+        outids = out_buf[:n_out.value]
     else:
         # a geometry may leave no output at all (every candidate clipped): the library still
         # wants a valid pointer, so at least one row is allocated and the result is a slice
@@ -294,6 +311,21 @@ def _packed_filters(owner, filters, fs, K, c_in, c_out, stream):
                                          packed.data_ptr(), packed.numel(), stream))
         held[1][key] = packed
     return packed
+
+
+def prepack_filters(filters, c_in, c_out):
+    """Queue the packing of `filters` ([*kernel_size, Cin, Cout], float32 or half, on the GPU)
+    now and keep the result on the tensor, so that a convolution called with this tensor
+    later finds it: a layer that knows its filters before its rulebook packs them while the
+    rulebook is still being built."""
+    if not filters.is_cuda or filters.dtype not in _ENTRIES:
+        return
+    owner = filters
+    filters, fs_k, fs_ci, fs_co = _filter_strides(filters, c_in, c_out)
+    K = 1
+    for d in filters.shape[:-2]:
+        K *= d
+    _packed_filters(owner, filters, (fs_k, fs_ci, fs_co), K, c_in, c_out, _stream(filters))
 
 
 def _planned_conv(meta, features, owner, filters, fs, pairs, num, K, c_in, c_out, n_out, inverse):
