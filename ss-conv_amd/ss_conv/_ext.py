@@ -210,10 +210,14 @@ def rulebook_meta(indice_pairs):
     return meta
 
 
-def get_indice_pairs_3d(indices, batch_size, out_spatial_shape, spatial_shape, kernel_size, stride,
-                        padding, dilation, out_padding, subm, transpose):
-    """src/ss_conv_ops.cu:31 / src/conv/indice_conv.h:21-131.
-    Returns [outids[N_out,4], indicePairs[K,2,N], indiceNum[K]] (all int32)."""
+class _PendingRulebook(object):
+    """A rulebook between ssc_rulebook_begin and ssc_rulebook_finish: everything whose size
+    does not depend on the number of outputs is queued, the host has not waited yet."""
+    __slots__ = ("indices", "n", "geometry", "ws", "pairs", "num", "out_buf", "subm", "stream")
+
+
+def _rulebook_begin(indices, batch_size, out_spatial_shape, kernel_size, stride, padding, dilation,
+                    out_padding, subm, transpose):
     if indices.dim() != 2 or indices.size(1) != 4:
         raise RuntimeError("indices must be [N, 4] (batch, x, y, z)")
     for lst in (kernel_size, out_spatial_shape, stride, padding, out_padding, dilation):
@@ -232,42 +236,60 @@ def get_indice_pairs_3d(indices, batch_size, out_spatial_shape, spatial_shape, k
     nbytes = _lib.ssc_rulebook_workspace_bytes(gref, n)
     if nbytes == 0:  # geometry rejected: let the first call produce the message
         nbytes = 256
-    ws = _workspace(nbytes, dev)
-    pairs = torch.empty((K, 2, n), dtype=torch.int32, device=dev)
-    num = torch.empty((K,), dtype=torch.int32, device=dev)
-    s = _stream(indices)
+    r = _PendingRulebook()
+    r.indices, r.n, r.geometry, r.subm = indices, n, g, bool(subm)
+    r.ws = _workspace(nbytes, dev)
+    r.pairs = torch.empty((K, 2, n), dtype=torch.int32, device=dev)
+    r.num = torch.empty((K,), dtype=torch.int32, device=dev)
+    r.stream = _stream(indices)
     # Marking, ranking and the pair lists are queued; the host then waits for the number of
     # outputs only, while the pair lists are still being written.  When room for any
     # possible number of output rows is cheap (n * K rows at most), the rows are written in
     # the same launch as the pairs and the result is a slice of that buffer; otherwise by a
     # launch of their own once the number is known.
-    out_buf = None
+    r.out_buf = None
     if not subm and n > 0:
         bound = _lib.ssc_rulebook_out_bound(gref, n)
         if 0 < bound * 16 <= _ROWS_AHEAD_BYTES:
-            out_buf = torch.empty((bound, 4), dtype=torch.int32, device=dev)
-    _check(_lib.ssc_rulebook_begin(_ptr(indices), n, gref, ws.data_ptr(), ws.numel(), _ptr(pairs),
-                                   num.data_ptr(), _ptr(out_buf),
-                                   0 if out_buf is None else out_buf.size(0), s))
+            r.out_buf = torch.empty((bound, 4), dtype=torch.int32, device=dev)
+    _check(_lib.ssc_rulebook_begin(_ptr(indices), n, gref, r.ws.data_ptr(), r.ws.numel(),
+                                   _ptr(r.pairs), r.num.data_ptr(), _ptr(r.out_buf),
+                                   0 if r.out_buf is None else r.out_buf.size(0), r.stream))
+    return r
+
+
+def _rulebook_finish(r):
+    """Wait for the number of outputs; returns [outids, pairs, num]."""
+    gref = ctypes.byref(r.geometry)
     n_out = _i32(0)
     in_order = _i32(0)
-    _check(_lib.ssc_rulebook_finish(gref, n, ctypes.byref(n_out), ctypes.byref(in_order)))
-    if subm:
-        outids = indices
-    elif out_buf is not None:
-        outids = out_buf[:n_out.value]
+    _check(_lib.ssc_rulebook_finish(gref, r.n, ctypes.byref(n_out), ctypes.byref(in_order)))
+    if r.subm:
+        outids = r.indices
+    elif r.out_buf is not None:
+        outids = r.out_buf[:n_out.value]
     else:
         # a geometry may leave no output at all (every candidate clipped): the library still
         # wants a valid pointer, so at least one row is allocated and the result is a slice
-        out_buf = torch.empty((max(n_out.value, 1), 4), dtype=torch.int32, device=dev)
+        out_buf = torch.empty((max(n_out.value, 1), 4), dtype=torch.int32, device=r.pairs.device)
         outids = out_buf[:n_out.value]
-        _check(_lib.ssc_rulebook_rows(gref, n, ws.data_ptr(), ws.numel(), out_buf.data_ptr(), s))
+        _check(_lib.ssc_rulebook_rows(gref, r.n, r.ws.data_ptr(), r.ws.numel(), out_buf.data_ptr(),
+                                      r.stream))
     # Pairs of an offset always ascend in the input rows, and in the output rows too when
     # the input rows came in key order: the convolution may then skip its order check
     # (the first flag serves a call that accumulates into output rows, the second one
     # with `inverse`, which accumulates into input rows).
-    pairs._ssc_meta = RulebookMeta(pairs._version, (bool(in_order.value), True))
-    return [outids, pairs, num]
+    r.pairs._ssc_meta = RulebookMeta(r.pairs._version, (bool(in_order.value), True))
+    return [outids, r.pairs, r.num]
+
+
+def get_indice_pairs_3d(indices, batch_size, out_spatial_shape, spatial_shape, kernel_size, stride,
+                        padding, dilation, out_padding, subm, transpose):
+    """src/ss_conv_ops.cu:31 / src/conv/indice_conv.h:21-131.
+    Returns [outids[N_out,4], indicePairs[K,2,N], indiceNum[K]] (all int32)."""
+    return _rulebook_finish(_rulebook_begin(indices, batch_size, out_spatial_shape, kernel_size,
+                                            stride, padding, dilation, out_padding, subm,
+                                            transpose))
 
 
 def _filter_strides(filters, c_in, c_out):
@@ -328,6 +350,26 @@ def prepack_filters(filters, c_in, c_out):
     _packed_filters(owner, filters, (fs_k, fs_ci, fs_co), K, c_in, c_out, _stream(filters))
 
 
+def _plan_of(meta, pairs, num, K, c_in, c_out, elem_bytes, n_in, n_out, inverse, dev, stream):
+    """The plan of a (direction, channel counts, element type, row counts) combination over
+    a rulebook: built on first use, kept with the rulebook afterwards."""
+    stride = pairs.size(2)
+    key = (bool(inverse), c_in, c_out, elem_bytes, n_in, n_out)
+    plan = meta.plans.get(key)
+    if plan is None:
+        plan = _workspace(_lib.ssc_conv_plan_bytes(n_out, K, c_in, c_out, stride), dev)
+        scratch = _workspace(_lib.ssc_conv_plan_scratch_bytes(n_out, K, c_in, c_out, stride), dev)
+        flags = 2 if meta.canonical[1 if inverse else 0] else 0
+        _check(_lib.ssc_conv_plan_build(_ptr(pairs), stride, num.data_ptr(), K, int(bool(inverse)),
+                                        flags, n_in, n_out, c_in, c_out, elem_bytes,
+                                        plan.data_ptr(), plan.numel(), scratch.data_ptr(),
+                                        scratch.numel(), stream))
+        if len(meta.plans) >= RulebookMeta.MAX_PLANS:
+            meta.plans.clear()
+        meta.plans[key] = plan
+    return plan
+
+
 def _planned_conv(meta, features, owner, filters, fs, pairs, num, K, c_in, c_out, n_out, inverse):
     """out[n_out, c_out] through a cached plan: the schedule is built on the first call of a
     (direction, channel counts, element type, row counts) combination over this rulebook
@@ -336,26 +378,55 @@ def _planned_conv(meta, features, owner, filters, fs, pairs, num, K, c_in, c_out
     dev = features.device
     s = _stream(features)
     n_in = features.size(0)
-    stride = pairs.size(2)
-    eb = features.element_size()
-    key = (bool(inverse), c_in, c_out, eb, n_in, n_out)
-    plan = meta.plans.get(key)
-    if plan is None:
-        plan = _workspace(_lib.ssc_conv_plan_bytes(n_out, K, c_in, c_out, stride), dev)
-        scratch = _workspace(_lib.ssc_conv_plan_scratch_bytes(n_out, K, c_in, c_out, stride), dev)
-        flags = 2 if meta.canonical[1 if inverse else 0] else 0
-        _check(_lib.ssc_conv_plan_build(_ptr(pairs), stride, num.data_ptr(), K, int(bool(inverse)),
-                                        flags, n_in, n_out, c_in, c_out, eb, plan.data_ptr(),
-                                        plan.numel(), scratch.data_ptr(), scratch.numel(), s))
-        if len(meta.plans) >= RulebookMeta.MAX_PLANS:
-            meta.plans.clear()
-        meta.plans[key] = plan
     packed = _packed_filters(owner, filters, fs, K, c_in, c_out, s)
+    plan = _plan_of(meta, pairs, num, K, c_in, c_out, features.element_size(), n_in, n_out,
+                    inverse, dev, s)
     out = torch.empty((n_out, c_out), dtype=features.dtype, device=dev)
     _check(_ENTRIES[features.dtype][2](_ptr(features), n_in, c_in, packed.data_ptr(),
-                                       packed.numel(), plan.data_ptr(), plan.numel(), stride, K,
-                                       c_out, _ptr(out), n_out, s))
+                                       packed.numel(), plan.data_ptr(), plan.numel(), pairs.size(2),
+                                       K, c_out, _ptr(out), n_out, s))
     return out
+
+
+def rulebook_conv(features, filters, indices, batch_size, out_spatial_shape, kernel_size, stride,
+                  padding, dilation, out_padding, subm):
+    """get_indice_pairs_3d followed by indice_conv_fp32 / indice_conv_half over the new
+    rulebook, as a layer without a cached rulebook runs them (ss_conv/sp_ops/conv.py:131-150),
+    with the host's wait for the number of outputs placed behind everything that does not
+    need it: the rulebook is queued, the filters are packed and every argument is checked
+    first; after the wait only the plan and the kernel remain to be queued.
+    Returns (out_features, outids, pairs, num)."""
+    _need_gpu(features, filters, indices)
+    dtype = features.dtype
+    if dtype not in _ENTRIES or filters.dtype != dtype:
+        raise RuntimeError("rulebook_conv needs float32 or half features and filters of one type")
+    r = _rulebook_begin(indices, batch_size, out_spatial_shape, kernel_size, stride, padding,
+                        dilation, out_padding, subm, 0)
+    features = features.contiguous()
+    n_in, c_in = features.shape
+    c_out = filters.size(-1)
+    owner = filters
+    filters, fs_k, fs_ci, fs_co = _filter_strides(filters, c_in, c_out)
+    K = r.pairs.size(0)
+    kvol = 1
+    for d in filters.shape[:-2]:
+        kvol *= d
+    if kvol != K:
+        raise RuntimeError("filters have %d offsets but the rulebook has %d" % (kvol, K))
+    if n_in != r.n:
+        raise RuntimeError("features and indices must have the same number of rows")
+    dev = features.device
+    s = r.stream
+    packed = _packed_filters(owner, filters, (fs_k, fs_ci, fs_co), K, c_in, c_out, s)
+    run = _ENTRIES[dtype][2]
+    eb = features.element_size()
+    outids, pairs, num = _rulebook_finish(r)
+    n_out = outids.size(0)
+    plan = _plan_of(pairs._ssc_meta, pairs, num, K, c_in, c_out, eb, n_in, n_out, False, dev, s)
+    out = torch.empty((n_out, c_out), dtype=dtype, device=dev)
+    _check(run(_ptr(features), n_in, c_in, packed.data_ptr(), packed.numel(), plan.data_ptr(),
+               plan.numel(), n_in, K, c_out, _ptr(out), n_out, s))
+    return out, outids, pairs, num
 
 
 def _conv_any(features, owner, filters, fs, indice_pairs, pairs, num, K, c_in, c_out, n_out,

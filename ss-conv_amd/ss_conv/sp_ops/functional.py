@@ -71,6 +71,39 @@ class SubMConvFunction(_ConvBase):
         return SubMConvFunction._grad(ctx, grad_output)
 
 
+class SparseConvRulebookFunction(Function):
+    """Rulebook and convolution of a layer that has no cached rulebook, as one autograd node:
+    forward(features, filters, indices, batch_size, out_shape, ksize, stride, padding,
+    dilation, out_padding, subm) -> (out_features, outids or None when subm, pairs, num).
+    Same numbers as get_indice_pairs followed by indice_conv / indice_subm_conv; the host's
+    wait for the number of outputs sits behind the work that does not depend on it."""
+
+    @staticmethod
+    def forward(ctx, features, filters, indices, batch_size, out_shape, ksize, stride, padding,
+                dilation, out_padding, subm):
+        out, outids, pairs, num = _ext.rulebook_conv(features, filters, indices, batch_size,
+                                                     out_shape, ksize, stride, padding, dilation,
+                                                     out_padding, subm)
+        ctx.save_for_backward(pairs, num, features, filters)
+        ctx.ssc_meta = getattr(pairs, "_ssc_meta", None)
+        ctx.subm = bool(subm)
+        if subm:  # the outputs are the inputs: nothing new to return
+            ctx.mark_non_differentiable(pairs, num)
+            return out, None, pairs, num
+        ctx.mark_non_differentiable(outids, pairs, num)
+        return out, outids, pairs, num
+
+    @staticmethod
+    def backward(ctx, grad_output, *unused):
+        indice_pairs, indice_pair_num, features, filters = ctx.saved_tensors
+        if ctx.ssc_meta is not None and getattr(indice_pairs, "_ssc_meta", None) is None:
+            indice_pairs._ssc_meta = ctx.ssc_meta
+        input_bp, filters_bp = ops.indice_conv_backward(
+            features, filters, grad_output.contiguous(), indice_pairs, indice_pair_num, False,
+            ctx.subm)
+        return (input_bp, filters_bp) + (None,) * 9
+
+
 class SparseMaxPoolFunction(Function):
     @staticmethod
     def forward(ctx, features, indice_pairs, indice_pair_num, num_activate_out):
@@ -252,6 +285,7 @@ class ThreeInterpolate(Function):
 indice_conv = SparseConvFunction.apply
 indice_inverse_conv = SparseInverseConvFunction.apply
 indice_subm_conv = SubMConvFunction.apply
+rulebook_conv = SparseConvRulebookFunction.apply
 indice_maxpool = SparseMaxPoolFunction.apply
 indice_avgpool = SparseAvgPoolFunction.apply
 global_maxpool = GlobalMaxPool.apply

@@ -1426,3 +1426,41 @@ def test_layer_reuses_plan_under_an_indice_key(device):
         z = _ext.indice_conv_fp32(z, b.weight, pairs.clone(), st.indice_dict["s"][3],
                                   idx.shape[0], 0, 1)
         assert torch.equal(z, y.features)
+
+
+@pytest.mark.parametrize("subm,stride", [(False, 1), (False, 2), (True, 1)])
+def test_fused_rulebook_conv_equals_the_two_calls(subm, stride, device):
+    """A layer without a cached rulebook runs rulebook and convolution as one native
+    sequence (one autograd node); a layer that finds the rulebook under its indice_key runs
+    the convolution alone.  Same rulebook, same output bits, same gradients."""
+    from ss_conv.sp_ops.conv import SparseConvolution
+    from ss_conv.sp_ops.ops import get_indice_pairs
+    from ss_conv.sp_ops.functional import indice_conv, indice_subm_conv
+    from ss_conv.sp_ops.tensor import SparseTensor
+    rng = np.random.default_rng(77)
+    idx = random_voxels(rng, 3, 14, 900)
+    t = torch.from_numpy(idx).to(device)
+    torch.manual_seed(1)
+    layer = SparseConvolution(3, 24, 40, 3, stride=stride, padding=1, subm=subm, bias=True,
+                              indice_key="k").to(device)
+    x1 = torch.randn((idx.shape[0], 24), device=device, requires_grad=True)
+    st = SparseTensor(x1, t, [14] * 3, 3)
+    y1 = layer(st)                      # fused: builds the rulebook
+    outids, _, pairs, num, _ = st.indice_dict["k"]
+    g_idx, g_pairs, g_num = get_indice_pairs(t, 3, [14] * 3, 3, stride, 1, 1, 0, subm)
+    assert torch.equal(outids, g_idx) and torch.equal(pairs, g_pairs) and torch.equal(num, g_num)
+    go = torch.randn_like(y1.features)
+    y1.features.backward(go)
+    gx1, gw1, gb1 = x1.grad.clone(), layer.weight.grad.clone(), layer.bias.grad.clone()
+    layer.zero_grad()
+    x2 = x1.detach().clone().requires_grad_(True)
+    st2 = SparseTensor(x2, t, [14] * 3, 3)
+    st2.indice_dict = st.indice_dict    # cached rulebook: convolution alone
+    y2 = layer(st2)
+    assert torch.equal(y1.indices, y2.indices) and torch.equal(y1.features, y2.features)
+    y2.features.backward(go)
+    assert torch.equal(gx1, x2.grad) and torch.equal(gw1, layer.weight.grad)
+    assert torch.equal(gb1, layer.bias.grad)
+    fn = indice_subm_conv if subm else indice_conv
+    y3 = fn(x1.detach(), layer.weight.detach(), g_pairs.clone(), g_num, g_idx.shape[0])
+    assert torch.equal(y3 + layer.bias.detach(), y1.features.detach())
