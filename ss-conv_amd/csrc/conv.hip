@@ -39,6 +39,13 @@ constexpr int kMinTile = 64;
 // 16q .. 16q+15 of the chunk (lane group g has channels 16q + 4g .. +3), so a layer with
 // few input channels needs only its first loads.
 //
+// A chunk need not hold 64 channels: with ns < 16 MFMA steps per chunk it holds 4 ns, the
+// channels cc*4ns .. cc*4ns + 4ns - 1, and only the first ns of the 16 (q, j) slots carry
+// weights.  The quarters below ns / 4 are laid out as above.  In the quarter that is only
+// partly used (ns % 4 steps) step j must stand for four consecutive channels, one per lane
+// group, so there slot (q, lane group g, j) holds channel 16q + 4j + g of the chunk; the
+// rows staged in LDS follow the same rule (conv_fwd_kernel's producers).
+//
 // Half-precision filters are packed for v_mfma_f32_16x16x32_f16 instead, two steps of 32
 // channels per chunk (halves, 2 KiB per fragment):
 // packed[((k*NCB + ncb)*NCH + cc)*1024 + q*512 + lane*8 + j] =
@@ -51,6 +58,7 @@ struct PackArgs {
   int64_t fs_k, fs_ci, fs_co;
   int K, cin, cout, ncb, nch;
   void *packed_out;
+  int ns;  // MFMA steps per chunk (float filters; half filters always use whole chunks)
 };
 
 // Element idx of the packed filters.
@@ -73,7 +81,11 @@ __device__ __forceinline__ void pack_filter_element(const PackArgs &a, int64_t i
   } else {
     const int j = idx & 3, q = (idx >> 8) & 3;
     lane = (idx >> 2) & 63;
-    ci = cc * kKC + q * 16 + (lane >> 4) * 4 + j;
+    const int g = lane >> 4, full = a.ns >> 2, rem = a.ns & 3;
+    int cl = -1;  // channel inside the chunk, -1 for a slot without one
+    if (q < full) cl = q * 16 + g * 4 + j;
+    else if (q == full && j < rem) cl = q * 16 + j * 4 + g;
+    ci = cl < 0 ? cin : cc * (4 * a.ns) + cl;
   }
   int co = cb * 16 + (lane & 15);
   IO v = (IO)0.f;
@@ -698,10 +710,12 @@ struct StagePos {
 //
 // The waves-per-SIMD attribute states the occupancy the workgroup size gives anyway
 // (one workgroup per CU), so that the compiler uses the whole register budget.
-// NQ: 16-channel quarters of a chunk that hold input channels (4 unless the layer has
-// a single chunk with at most 48 channels): MFMA steps, fragment loads and staged-row
-// reads of the other quarters are left out.
-template <typename IO, int GATHER, int NCW, int NQ>
+// NS: MFMA steps (of 4 input channels) per chunk, 16 for chunks of 64 channels.  A layer
+// whose input channels do not fill whole chunks of 64 is cut into ceil(Cin / 64) chunks of
+// equal width 4 NS instead (200 channels: 4 chunks of 52, 13 steps each, where chunks of 64
+// would run 64 steps for 50 steps' worth of channels): MFMA steps, fragment loads, gathers
+// and staged-row reads beyond NS are left out.  Half precision always runs whole chunks.
+template <typename IO, int GATHER, int NCW, int NS>
 __global__ void __launch_bounds__((NCW + 4) * 64)
     __attribute__((amdgpu_waves_per_eu((NCW + 4) / 4, (NCW + 4) / 4)))
     conv_fwd_kernel(const IO *__restrict__ features, int cin, unsigned feat_bytes,
@@ -715,6 +729,10 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
   constexpr bool kHalf = kEB == 2;
   constexpr int kRowB = Io<IO>::kRowBytes;    // bytes of a staged row
   constexpr int kFragB = Io<IO>::kFragBytes;  // bytes of a packed filter fragment
+  static_assert(NS >= 1 && NS <= 16 && (!kHalf || NS == 16), "steps per chunk");
+  static_assert(GATHER != 1 || NS == 16, "the unchecked gather reads whole chunks of 64");
+  constexpr int kChunk = kHalf ? kKC : 4 * NS;  // input channels per chunk
+  constexpr int kQFull = NS / 4, kQRem = NS % 4;  // whole quarters, steps of the partial one
   typedef typename Io<IO>::Raw Raw;
   constexpr int kAS = kCN + 4;    // accumulator row stride in floats
   constexpr int NT = (NCW + 4) * 64;
@@ -815,9 +833,14 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
     const __amdgpu_buffer_rsrc_t rs_feat =
         __builtin_amdgcn_make_buffer_rsrc((void *)features, 0, (int)feat_bytes, kRsrcFlags);
     const int idx_voff = (pt >> 4) * 4;    // this thread's slot (plus 16 slots per element)
-    const int chunk_off = (pt & 15) * 4 * kEB;  // this thread's 4 channels of a 64-channel row chunk
-    // this thread's 4 channels of the last chunk lie beyond Cin
-    const bool beyond_cin = (nch - 1) * kKC + (pt & 15) * 4 >= cin;
+    const int piece = pt & 15;                  // this thread's 4 channels of a row chunk
+    const int chunk_off = piece * 4 * kEB;
+    // the chunk has no such piece (fewer than 16 steps), or, in the last chunk, the piece
+    // lies beyond Cin
+    const bool no_piece = !kHalf && piece >= NS;
+    const bool beyond_cin = (nch - 1) * kChunk + piece * 4 >= cin;
+    // a piece of the partly used quarter is staged one channel per lane group
+    const bool spread = !kHalf && kQRem != 0 && piece >= 4 * kQFull && piece < NS;
     typedef Raw Held;
     int idx[ID][NE];
     Held rows[RD][NE];
@@ -838,12 +861,13 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
 #pragma unroll
       for (int j = 0; j < NE; ++j) {
         if constexpr (GATHER == 1) {
-          r[j] = Io<IO>::gather(rs_feat, ix[j] + chunk_off, pos.cc * (kKC * kEB));
+          r[j] = Io<IO>::gather(rs_feat, ix[j] + chunk_off, pos.cc * (kChunk * kEB));
         } else if constexpr (GATHER == 2) {
-          const int off = (pos.cc == nch - 1 && beyond_cin) ? (int)kGatherPad : ix[j];
-          r[j] = Io<IO>::gather(rs_feat, off + chunk_off, pos.cc * (kKC * kEB));
+          const int off =
+              (no_piece || (pos.cc == nch - 1 && beyond_cin)) ? (int)kGatherPad : ix[j];
+          r[j] = Io<IO>::gather(rs_feat, off + chunk_off, pos.cc * (kChunk * kEB));
         } else {
-          const int ch = pos.cc * kKC + (pt & 15) * 4;
+          const int ch = pos.cc * kChunk + piece * 4;
           const int row = ix[j] < 0 ? 0 : ix[j];  // padding slots read row 0 and drop it
           const IO *fp = features + (int64_t)row * cin + ch;
           Held v = Io<IO>::zero();
@@ -852,16 +876,31 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
           } else {  // rows are not aligned: one element at a time
             v = Io<IO>::load_first(fp, cin - ch);
           }
-          if (ix[j] < 0) v = Io<IO>::zero();
+          if (ix[j] < 0 || no_piece) v = Io<IO>::zero();
           r[j] = v;
         }
       }
     };
-    char *const st_base = reinterpret_cast<char *>(abuf) + (pt >> 4) * kRowB + (pt & 15) * 4 * kEB;
+    // where this thread's piece goes in a staged row: its own 16 bytes, or, for a piece of
+    // the partly used quarter, element (piece - 4 kQFull) of each lane group's 16 bytes
+    char *const st_base = reinterpret_cast<char *>(abuf) + (pt >> 4) * kRowB +
+                          (spread ? (16 * kQFull + (piece - 4 * kQFull)) * kEB : piece * 4 * kEB);
     auto store_rows = [&](int parity, const Held (&r)[NE]) {
 #pragma unroll
-      for (int j = 0; j < NE; ++j)
-        *reinterpret_cast<Held *>(st_base + (parity * kStage + j * 16) * kRowB) = r[j];
+      for (int j = 0; j < NE; ++j) {
+        char *dst = st_base + (parity * kStage + j * 16) * kRowB;
+        if constexpr (!kHalf && kQRem != 0) {
+          if (spread) {
+            const float4v v = __builtin_bit_cast(float4v, r[j]);
+            reinterpret_cast<float *>(dst)[0] = v.x;
+            reinterpret_cast<float *>(dst)[4] = v.y;
+            reinterpret_cast<float *>(dst)[8] = v.z;
+            reinterpret_cast<float *>(dst)[12] = v.w;
+            continue;
+          }
+        }
+        if (!no_piece) *reinterpret_cast<Held *>(dst) = r[j];
+      }
     };
     // Prologue.  Loads are issued in the order the loop will wait for them (offsets,
     // then rows, oldest stage first): the wait counts of the loop are static, so
@@ -938,7 +977,7 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
     // 16-byte pieces of operands a lane handles per row block: weight fragment loads, and
     // as many reads of its staged row (float: 4 MFMA steps of 4 channels each, a quarter
     // of the chunk; half: one MFMA step of 32 channels, lane group g has 8 of them)
-    constexpr int NF = kHalf ? 2 : NQ;
+    constexpr int NF = kHalf ? 2 : (NS + 3) / 4;
     typedef std::conditional_t<kHalf, int4v, float4v> Frag;
     const int w_voff = lane * 16;  // this lane's 16 bytes of a KiB of fragments
     constexpr int kWStep = 1024;   // from one 16-byte piece to the next
@@ -1029,7 +1068,7 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
     // chain a handful of other instructions issue for free -- and no more than that:
     // everything else a block needs is therefore spread, one small piece per gap,
     // over the 16 gaps of the block, and scheduling barriers pin it there:
-    // (gap numbers for NQ = 4, i.e. 16 MFMAs a block)
+    // (gap numbers for NS = 16, i.e. 16 MFMAs a block)
     //   gap 2      fragment offset of block b+3 (from the schedule record); accumulator
     //              update of the previous block: add, write; once per stage, tile and
     //              last-of-tile of the next stage
@@ -1059,17 +1098,20 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
       // gaps of the pieces of a block (see above); with fewer than 16 MFMAs they move
       // closer together, in the same order
       // half: two MFMAs a block, so the pieces sit behind the first or the second
-      constexpr int kSteps = kHalf ? 2 : 4 * NQ;
-      constexpr bool kFull = !kHalf && NQ == 4;
-      constexpr int kGapAlu = kHalf ? 0 : kFull ? 2 : 1, kGapAcc = kHalf ? 0 : kGapAlu + 1;
-      constexpr int kGapW[4] = {kHalf ? 0 : kFull ? 4 : 2, kHalf ? 1 : kFull ? 7 : 3, kFull ? 9 : 4,
-                                12};
-      constexpr int kGapRow = kHalf ? 0 : kFull ? 5 : 2;  // after fragment load 0 in the same gap
-      constexpr int kGapA[4] = {kHalf ? 1 : kFull ? 6 : kSteps / 2,
-                                kHalf ? 1 : kFull ? 8 : kSteps / 2 + 1,
-                                kFull ? 10 : kSteps / 2 + 2, 11};
-      constexpr int kGapRec0 = kHalf ? 1 : kFull ? 13 : kSteps - 2;
-      constexpr int kGapRec1 = kHalf ? 1 : kFull ? 14 : kSteps - 1;
+      constexpr int kSteps = kHalf ? 2 : NS;
+      constexpr bool kFull = !kHalf && NS == 16;
+      // no piece may be placed behind the last MFMA
+      constexpr int kLast = kSteps - 1;
+      auto at = [](int gap) constexpr { return gap < (kHalf ? 1 : NS - 1) ? gap : (kHalf ? 1 : NS - 1); };
+      constexpr int kGapAlu = kHalf ? 0 : kFull ? 2 : at(1), kGapAcc = kHalf ? 0 : at(kGapAlu + 1);
+      constexpr int kGapW[4] = {kHalf ? 0 : kFull ? 4 : at(2), kHalf ? 1 : kFull ? 7 : at(3),
+                                kFull ? 9 : at(4), at(12)};
+      constexpr int kGapRow = kHalf ? 0 : kFull ? 5 : at(2);  // after fragment load 0 in the same gap
+      constexpr int kGapA[4] = {kHalf ? 1 : kFull ? 6 : at(kSteps / 2),
+                                kHalf ? 1 : kFull ? 8 : at(kSteps / 2 + 1),
+                                kFull ? 10 : at(kSteps / 2 + 2), at(11)};
+      constexpr int kGapRec0 = kHalf ? 1 : kFull ? 13 : (kSteps >= 2 ? kSteps - 2 : 0);
+      constexpr int kGapRec1 = kHalf ? 1 : kFull ? 14 : kLast;
 #pragma unroll
       for (int m = 0; m < 4; ++m) {
         const int slot = m;                 // == (4 * s + m) & 3
@@ -1186,6 +1228,7 @@ struct ConvPlan {
   int ncb, nch, T, ncw, n_wg, n_colblk;  // T: rows of the accumulator window
   int tile_rows;                         // largest tile height
   int gather;  // conv_fwd_kernel's GATHER
+  int ns;      // conv_fwd_kernel's NS: MFMA steps per chunk
   int64_t n_tiles, n_fine, words_per_k, grp_cap;  // n_tiles: upper bound
   size_t lds_bytes;
 };
@@ -1220,6 +1263,18 @@ static ConvPlan make_plan(int64_t n_in, int64_t n_out, int K, int c_in, int c_ou
   ConvPlan p;
   p.ncb = (int)ceil_div(c_out, 16);
   p.nch = (int)ceil_div(c_in, kKC);
+  // chunks of equal width: the fewest steps of 4 channels that cover Cin in nch chunks,
+  // rounded up to a width the kernel is built for
+  p.ns = 16;
+  if (elem_bytes == 4) {
+    const int want = (int)ceil_div(ceil_div(c_in, p.nch), 4);
+    constexpr int kBuilt[] = {1, 2, 3, 4, 6, 8, 10, 12, 13, 14, 15, 16};
+    for (int b : kBuilt)
+      if (b >= want) {
+        p.ns = b;
+        break;
+      }
+  }
   p.ncw = 4;
   p.T = pick_tile(p.ncw);
   p.tile_rows = p.T - kSpillRows;
@@ -1351,12 +1406,12 @@ static size_t conv_ws_bytes(int64_t n_out, int K, int c_in, int c_out, int64_t p
   return conv_ws_walk(nullptr, p, K, pair_stride, nullptr);
 }
 
-template <typename IO, int GATHER, int NCW, int NQ>
+template <typename IO, int GATHER, int NCW, int NS>
 static int launch_conv(const ConvPlan &p, const ConvWs &w, const IO *features, int64_t n_in,
                        int c_in, int K, IO *out, int c_out, hipStream_t s) {
   static bool attr_set = false;
   if (!attr_set) {
-    SSC_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(conv_fwd_kernel<IO, GATHER, NCW, NQ>),
+    SSC_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(conv_fwd_kernel<IO, GATHER, NCW, NS>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
     attr_set = true;
   }
@@ -1367,7 +1422,7 @@ static int launch_conv(const ConvPlan &p, const ConvWs &w, const IO *features, i
             (unsigned long long)packed_bytes, (unsigned long long)sched_bytes);
   const unsigned feat_bytes = GATHER != 0 ? (unsigned)((uint64_t)n_in * c_in * sizeof(IO)) : 0u;
   dim3 grid((unsigned)p.n_wg, (unsigned)p.n_colblk);
-  hipLaunchKernelGGL((conv_fwd_kernel<IO, GATHER, NCW, NQ>), grid, dim3((NCW + 4) * 64), p.lds_bytes, s, features, c_in,
+  hipLaunchKernelGGL((conv_fwd_kernel<IO, GATHER, NCW, NS>), grid, dim3((NCW + 4) * 64), p.lds_bytes, s, features, c_in,
                      feat_bytes, w.packed, (unsigned)packed_bytes, w.sched_in, w.sched_out,
                      w.grp_meta, (unsigned)sched_bytes, (unsigned)(p.grp_cap * 32), w.tile_grp,
                      w.wg_tile, p.nch, p.ncb, out, c_out, p.T);
@@ -1447,7 +1502,7 @@ static int conv_plan_build(const ConvPlan &p, const ConvWs &w, const int32_t *pa
   const int plane_g = inverse ? 1 : 0;
   const int plane_s = 1 - plane_g;
   const int64_t packed_n = pack ? (int64_t)K * p.ncb * p.nch * 1024 : 0;
-  PackArgs pk = {nullptr, 0, 0, 0, 0, 0, 0, 0, 0, nullptr};
+  PackArgs pk = {nullptr, 0, 0, 0, 0, 0, 0, 0, 0, nullptr, 16};
   if (pack) pk = *pack;
   if (!in_order) {  // otherwise the filters are packed beside the first kernel of the split
     if (pack) {
@@ -1525,24 +1580,26 @@ static int conv_run(const ConvPlan &p, const ConvWs &w, const IO *features, int6
   const bool prof = g_profile_on;
   const int slot = g_profile_count % kProfileRing;
   if (prof) SSC_HIP(hipEventRecord(g_profile_ev[slot][0], s));
-  // quarters of the (only) chunk that hold input channels; layers with several chunks
-  // run all four everywhere
-  const int nq = p.nch == 1 ? (int)ceil_div(c_in, 16) : 4;
-#define SSC_CONV_LAUNCH(G, Q) launch_conv<IO, G, 4, Q>(p, w, features, n_in, c_in, K, out, c_out, s)
+#define SSC_CONV_LAUNCH(G, S) launch_conv<IO, G, 4, S>(p, w, features, n_in, c_in, K, out, c_out, s)
+#define SSC_CONV_BY_STEPS(G)                                                            \
+  (p.ns == 1 ? SSC_CONV_LAUNCH(G, 1) : p.ns == 2 ? SSC_CONV_LAUNCH(G, 2)                 \
+   : p.ns == 3 ? SSC_CONV_LAUNCH(G, 3) : p.ns == 4 ? SSC_CONV_LAUNCH(G, 4)               \
+   : p.ns == 6 ? SSC_CONV_LAUNCH(G, 6) : p.ns == 8 ? SSC_CONV_LAUNCH(G, 8)               \
+   : p.ns == 10 ? SSC_CONV_LAUNCH(G, 10) : p.ns == 12 ? SSC_CONV_LAUNCH(G, 12)           \
+   : p.ns == 13 ? SSC_CONV_LAUNCH(G, 13) : p.ns == 14 ? SSC_CONV_LAUNCH(G, 14)           \
+   : p.ns == 15 ? SSC_CONV_LAUNCH(G, 15) : SSC_CONV_LAUNCH(G, 16))
   if constexpr (sizeof(IO) == 2) {
-    // half precision: one instance per gather mode (all four quarters)
-    rc = p.gather == 1 ? SSC_CONV_LAUNCH(1, 4)
-       : p.gather == 2 ? SSC_CONV_LAUNCH(2, 4) : SSC_CONV_LAUNCH(0, 4);
+    // half precision: one instance per gather mode (whole chunks)
+    rc = p.gather == 1 ? SSC_CONV_LAUNCH(1, 16)
+       : p.gather == 2 ? SSC_CONV_LAUNCH(2, 16) : SSC_CONV_LAUNCH(0, 16);
   } else if (p.gather == 1) {
-    rc = SSC_CONV_LAUNCH(1, 4);
+    rc = SSC_CONV_LAUNCH(1, 16);
   } else if (p.gather == 2) {
-    rc = nq == 1 ? SSC_CONV_LAUNCH(2, 1) : nq == 2 ? SSC_CONV_LAUNCH(2, 2)
-       : nq == 3 ? SSC_CONV_LAUNCH(2, 3) : SSC_CONV_LAUNCH(2, 4);
+    rc = SSC_CONV_BY_STEPS(2);
   } else {
-    rc = nq == 1 ? SSC_CONV_LAUNCH(0, 1) : nq == 2 ? SSC_CONV_LAUNCH(0, 2)
-       : nq == 3 ? SSC_CONV_LAUNCH(0, 3) : SSC_CONV_LAUNCH(0, 4);
+    rc = SSC_CONV_BY_STEPS(0);
   }
-  (void)nq;
+#undef SSC_CONV_BY_STEPS
 #undef SSC_CONV_LAUNCH
   if (rc != SSC_OK) return rc;
   if (prof) {
@@ -1585,7 +1642,7 @@ static int conv_fwd(const IO *features, int64_t n_in, int32_t c_in, const IO *fi
   ConvPlan p = make_plan(n_in, n_out, K, c_in, c_out, pair_stride, (int)sizeof(IO));
   ConvWs w;
   conv_ws_walk(workspace, p, K, pair_stride, &w);
-  const PackArgs pack = {filters, fs_k, fs_ci, fs_co, K, c_in, c_out, p.ncb, p.nch, w.packed};
+  const PackArgs pack = {filters, fs_k, fs_ci, fs_co, K, c_in, c_out, p.ncb, p.nch, w.packed, p.ns};
   const bool in_order = (subm & SSC_CONV_PAIRS_CANONICAL) != 0;
   rc = conv_plan_build<IO>(p, w, pairs, pair_stride, pair_num, K, inverse, in_order, c_in, n_out,
                            (int)sizeof(IO), &pack, s);
@@ -1603,7 +1660,7 @@ static int conv_pack(const IO *filters, int64_t fs_k, int64_t fs_ci, int64_t fs_
   SSC_CHECK(packed_bytes >= conv_packed_bytes(p, K), SSC_EWORKSPACE,
             "buffer of the packed filters too small: %zu < %zu", packed_bytes,
             conv_packed_bytes(p, K));
-  const PackArgs pack = {filters, fs_k, fs_ci, fs_co, K, c_in, c_out, p.ncb, p.nch, packed};
+  const PackArgs pack = {filters, fs_k, fs_ci, fs_co, K, c_in, c_out, p.ncb, p.nch, packed, p.ns};
   const int64_t packed_n = (int64_t)K * p.ncb * p.nch * 1024;
   hipLaunchKernelGGL(pack_filters_kernel<IO>, dim3((unsigned)ceil_div(packed_n, 256)), dim3(256), 0,
                      s, pack, (int32_t *)nullptr);
