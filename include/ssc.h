@@ -299,6 +299,22 @@ int ssc_pool_max_f32(const float *features, int32_t channels, const int32_t *pai
                      float *out, int64_t n_out, void *workspace, size_t workspace_bytes,
                      ssc_stream_t stream);
 
+/* ssc_pool_max_f32 for callers that cannot allocate device memory (code under HIP graph
+ * capture, serving loops with a fixed memory budget, harnesses that forbid hipMalloc).  No
+ * counterpart in the reference, whose every pooling call allocates its output and
+ * temporaries through torch (src/pool/indice_maxpool.h:24).  Same result, bit for bit; the
+ * pair table lives in an array inside the library (SSC_POOL_STATIC_ENTRIES int32 per GPU,
+ * held until the process ends) instead of a workspace, so the call -- the look-up of that
+ * array's address on the first call per device aside, which a caller under graph capture
+ * makes beforehand with n_out = 0 -- only enqueues kernels.  n_out * kernel_volume must
+ * not exceed SSC_POOL_STATIC_ENTRIES (SSC_EINVAL otherwise).  All calls on one GPU share the
+ * array: calls that overlap in time on one GPU (different streams, different host threads)
+ * race; calls on one stream do not. */
+#define SSC_POOL_STATIC_ENTRIES (4 << 20) /* 16 MiB */
+int ssc_pool_max_static_f32(const float *features, int32_t channels, const int32_t *pairs,
+                            int64_t pair_stride, const int32_t *pair_num, int32_t kernel_volume,
+                            float *out, int64_t n_out, ssc_stream_t stream);
+
 int ssc_pool_avg_f32(const float *features, int32_t channels, const int32_t *pairs,
                      int64_t pair_stride, const int32_t *pair_num, int32_t kernel_volume,
                      const int32_t *summaryrf /* [n_out] */, float *out, int64_t n_out,

@@ -13,6 +13,8 @@
 
 #include <math.h>
 
+#include <mutex>
+
 namespace ssc {
 
 typedef float float4v __attribute__((ext_vector_type(4)));
@@ -275,11 +277,57 @@ static int pool_common(const float *features, int channels, const int32_t *pairs
   return SSC_OK;
 }
 
+// ---- the pair table in library-owned memory ------------------------------------------------
+// ssc_pool_max_static_f32 keeps its [n_out, K] pair table in this array instead of a
+// caller-provided workspace, so the call allocates nothing.  Every GPU the library runs on
+// holds its own copy of the array (SSC_POOL_STATIC_ENTRIES * 4 bytes, until the process
+// ends) at its own address; host code never uses the symbol `scratch` itself, only the
+// address hipGetSymbolAddress reports for the current device.
+static __device__ __align__(256) int32_t scratch[SSC_POOL_STATIC_ENTRIES];
+
+constexpr int kMaxDevices = 64;
+static int32_t *g_scratch_of_device[kMaxDevices] = {};
+static std::mutex g_scratch_mutex;
+
+// The device address of `scratch` on the current device (looked up once per device).
+static int static_table(int32_t **table) {
+  int dev = -1;
+  SSC_HIP(hipGetDevice(&dev));
+  SSC_CHECK(dev >= 0 && dev < kMaxDevices, SSC_ERUNTIME, "device ordinal %d out of range", dev);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_of_device[dev] == nullptr) {
+    void *ptr = nullptr;
+    SSC_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+    SSC_CHECK(ptr != nullptr, SSC_EHIP, "hipGetSymbolAddress returned a null address");
+    g_scratch_of_device[dev] = static_cast<int32_t *>(ptr);
+  }
+  *table = g_scratch_of_device[dev];
+  return SSC_OK;
+}
+
 }  // namespace ssc
 
 using namespace ssc;
 
 extern "C" {
+
+int ssc_pool_max_static_f32(const float *features, int32_t channels, const int32_t *pairs,
+                            int64_t pair_stride, const int32_t *pair_num, int32_t kernel_volume,
+                            float *out, int64_t n_out, ssc_stream_t stream) {
+  const int K = kernel_volume;
+  SSC_CHECK(K >= 1 && K <= SSC_MAX_KERNEL_VOLUME, SSC_ERUNTIME, "kernel volume %d out of range", K);
+  SSC_CHECK(channels >= 1 && n_out >= 0 && pair_stride >= 0, SSC_EINVAL, "bad sizes");
+  SSC_CHECK(n_out * K <= (int64_t)SSC_POOL_STATIC_ENTRIES, SSC_EINVAL,
+            "n_out * kernel_volume = %lld exceeds the %lld entries of the library's pair table: "
+            "use ssc_pool_max_f32 with a workspace",
+            (long long)(n_out * K), (long long)SSC_POOL_STATIC_ENTRIES);
+  int32_t *table = nullptr;
+  int rc = static_table(&table);  // (also for n_out == 0: a first call sets the address up)
+  if (rc != SSC_OK) return rc;
+  // the table keeps the previous call's entries: pool_common clears what this call uses
+  return ssc_pool_max_f32(features, channels, pairs, pair_stride, pair_num, K, out, n_out, table,
+                          (size_t)SSC_POOL_STATIC_ENTRIES * sizeof(int32_t), stream);
+}
 
 size_t ssc_pool_workspace_bytes(int64_t n_out, int32_t kernel_volume) {
   if (n_out < 0 || kernel_volume < 1) return 0;

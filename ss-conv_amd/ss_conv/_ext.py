@@ -85,6 +85,7 @@ _SIGNATURES = {
     "ssc_pool_workspace_bytes": (_sz, [_i64, _i32]),
     "ssc_pool_max_f32": (ctypes.c_int, [_vp, _i32, _vp, _i64, _vp, _i32, _vp, _i64, _vp, _sz,
                                         _vp]),
+    "ssc_pool_max_static_f32": (ctypes.c_int, [_vp, _i32, _vp, _i64, _vp, _i32, _vp, _i64, _vp]),
     "ssc_pool_avg_f32": (ctypes.c_int, [_vp, _i32, _vp, _i64, _vp, _i32, _vp, _vp, _i64, _vp,
                                         _sz, _vp]),
     "ssc_summary_rf": (ctypes.c_int, [_vp, _i64, _vp, _i32, _vp, _i64, _vp, _sz, _vp]),
