@@ -386,7 +386,9 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    _ext.profile_conv(True)
+    # every fifth launch of the convolution kernel inside the timed region is timed with HIP
+    # events on its stream (timing every launch costs the step about 20 us of stream time)
+    _ext.profile_conv(True, every=5 if args.steps >= 20 else 1)
     # The interpreter's cyclic garbage collector stays out of the timed region, as in
     # timeit: a full collection of a process that has imported torch takes 30-40 ms, many
     # times the region itself, and when it falls due depends on allocation counts only.
@@ -401,6 +403,14 @@ def main():
     gc.enable()
     conv_ms = _ext.profile_conv_read()
     _ext.profile_conv(False)
+    # the same region with the collector left on, reported beside the headline figure: what
+    # a Python caller that does not manage the collector sees on average
+    torch.cuda.synchronize()
+    t2 = time.perf_counter()
+    for _ in range(args.steps):
+        out = step()
+    torch.cuda.synchronize()
+    ms_gc_on = (time.perf_counter() - t2) * 1e3 / args.steps
 
     n_out = out.features.shape[0]
     pair_num = out.indice_dict[None][3] if None in out.indice_dict else None
@@ -427,11 +437,14 @@ def main():
                                % (args.workload, cfg["batch"], cfg["points"], grid, c_in, c_out,
                                   cfg["kernel"], cfg["stride"], cfg["padding"]),
                    "n_in": int(n_in), "n_out": int(n_out), "pairs": P,
-                   "input_voxels_per_s": n_in / (ms_per_step * 1e-3)},
+                   "input_voxels_per_s": n_in / (ms_per_step * 1e-3),
+                   "timed_region": "cyclic garbage collector off (as timeit does)",
+                   "ms_per_step_gc_on": ms_gc_on},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": FP32_MFMA_PEAK_TFLOPS,
                      "unit": "TFLOP/s", "frac": achieved / FP32_MFMA_PEAK_TFLOPS,
                      "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
                      "kernel": "conv_fwd_kernel", "kernel_ms": conv_kernel_ms,
+                     "kernel_launches_timed": len(conv_ms),
                      "flops_per_launch": flops},
     }
 

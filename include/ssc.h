@@ -257,8 +257,9 @@ int ssc_conv_bwd_filter_f16(const void *features /* [n_in,c_in] half */, int64_t
 
 /* Timing of the convolution kernel alone (no counterpart in the reference, whose
  * timers are commented out, src/conv/indice_conv.h:295,319-341).  While enabled,
- * every ssc_conv_fwd_f32 call records a pair of HIP events on its stream right
- * around the launch of the MFMA kernel (ring of 512 calls).
+ * every enable-th convolution call (enable = 1: every call; the events themselves cost a
+ * few microseconds of stream time per timed call) records a pair of HIP events on its
+ * stream right around the launch of the MFMA kernel (ring of 512 timed calls).
  * ssc_profile_conv_read waits for the recorded calls and returns their
  * durations in milliseconds, oldest first; enabling again clears the ring. */
 int ssc_profile_conv(int32_t enable);

@@ -1434,7 +1434,9 @@ static int launch_conv(const ConvPlan &p, const ConvWs &w, const IO *features, i
 // on the caller's stream right around the launch of conv_fwd_kernel.
 constexpr int kProfileRing = 512;
 static bool g_profile_on = false;
-static int g_profile_count = 0;
+static int g_profile_count = 0;   // launches timed so far
+static int g_profile_calls = 0;   // launches seen since profiling was enabled
+static int g_profile_every = 1;   // every n-th launch is timed
 static hipEvent_t g_profile_ev[kProfileRing][2];
 static bool g_profile_init = false;
 
@@ -1453,7 +1455,9 @@ int ssc_profile_conv(int32_t enable) {
     g_profile_init = true;
   }
   g_profile_on = enable != 0;
+  g_profile_every = enable > 1 ? enable : 1;
   g_profile_count = 0;
+  g_profile_calls = 0;
   return SSC_OK;
 }
 
@@ -1577,7 +1581,7 @@ template <typename IO>
 static int conv_run(const ConvPlan &p, const ConvWs &w, const IO *features, int64_t n_in, int c_in,
                     int K, IO *out, int c_out, hipStream_t s) {
   int rc;
-  const bool prof = g_profile_on;
+  const bool prof = g_profile_on && (g_profile_calls++ % g_profile_every) == 0;
   const int slot = g_profile_count % kProfileRing;
   if (prof) SSC_HIP(hipEventRecord(g_profile_ev[slot][0], s));
 #define SSC_CONV_LAUNCH(G, S) launch_conv<IO, G, 4, S>(p, w, features, n_in, c_in, K, out, c_out, s)

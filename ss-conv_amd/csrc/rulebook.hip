@@ -167,6 +167,79 @@ __global__ void __launch_bounds__(256)
   }
 }
 
+// ---- marking by dilation -------------------------------------------------------------------
+// With stride 1 and dilation 1 the active outputs are the active inputs dilated by the
+// kernel's extent: output o is active when some input sits at o - p + k, 0 <= k < ks.  In
+// the shifted coordinate u = i + p that reads u - k = o, so an input table over
+// u in [0, os + ks - 1) per axis holds every input that can reach the grid.  Marking then
+// costs one atomic per input row (instead of one per row and (kx, ky)), and the output table
+// is computed word by word from the input table -- no atomics, every word written, so it
+// needs no clearing -- by the kernel that also sums the words' popcounts for the scan.
+// Rows of the output table must be whole words (os[2] a multiple of 32).
+struct DenseIn {
+  int U[3];  // extents of the input table per batch element
+  int Wz;    // words per z row
+};
+
+static inline bool dense_marking_applies(const Geom &g, int64_t n_in, DenseIn *d) {
+  if (g.subm || (g.os[2] & 31) != 0) return false;
+  for (int a = 0; a < 3; ++a)
+    if (g.st[a] != 1 || g.dl[a] != 1 || g.ks[a] > 32) return false;
+  for (int a = 0; a < 3; ++a) d->U[a] = g.os[a] + g.ks[a] - 1;
+  d->Wz = (d->U[2] + 31) / 32;
+  const int64_t in_words = (int64_t)g.batch * d->U[0] * d->U[1] * d->Wz;
+  // the dilation walks the whole table: not for a few voxels in a huge grid
+  return in_words < ((int64_t)1 << 26) && geom_cells(g) / 32 <= 64 * n_in;
+}
+
+static inline int64_t dense_in_words(const Geom &g, const DenseIn &d) {
+  return (int64_t)g.batch * d.U[0] * d.U[1] * d.Wz;
+}
+
+// As mark_count_kernel (same grid, same chunk counts, same flags), but the wave marks the
+// cells of its input rows in the input table instead of the output cells they reach.
+__global__ void __launch_bounds__(256)
+    mark_in_count_kernel(const int32_t *__restrict__ indices, int64_t n_in, Geom g, DenseIn d,
+                         uint32_t *__restrict__ in_bits, int32_t *__restrict__ chunk_count,
+                         int64_t n_chunks, int32_t *__restrict__ flags) {
+  int64_t chunk = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (chunk >= n_chunks) return;
+  const int lane = threadIdx.x & 63;
+  int64_t i = chunk * 64 + lane;
+  bool live = i < n_in;
+  int32_t row[4] = {0, 0, 0, 0};
+  if (live) *reinterpret_cast<int4 *>(row) = reinterpret_cast<const int4 *>(indices)[i];
+  if (blockIdx.y == 0 && i + 1 < n_in &&
+      !row_before(*reinterpret_cast<int4 *>(row), reinterpret_cast<const int4 *>(indices)[i + 1]))
+    atomicOr(flags, kFlagDisorder);
+  if (live && !batch_in_range(row, g)) {
+    if (blockIdx.y == 0) atomicOr(flags, kFlagBadRow);
+    live = false;
+  }
+  if (blockIdx.y == 0 && live) {
+    const int ux = row[1] + g.pd[0], uy = row[2] + g.pd[1], uz = row[3] + g.pd[2];
+    if ((unsigned)ux < (unsigned)d.U[0] && (unsigned)uy < (unsigned)d.U[1] &&
+        (unsigned)uz < (unsigned)d.U[2]) {
+      const int64_t w = (((int64_t)row[0] * d.U[0] + ux) * d.U[1] + uy) * d.Wz + (uz >> 5);
+      atomicOr(&in_bits[w], 1u << (uz & 31));
+    }
+  }
+  const int kx = blockIdx.y;
+  int k = kx * g.ks[1] * g.ks[2];
+  int ox = 0;
+  const bool okx = live && tap_to_out(row[1], kx, 1, g.pd[0], 1, g.os[0], &ox);
+  for (int ky = 0; ky < g.ks[1]; ++ky) {
+    int oy = 0;
+    const bool okxy = okx && tap_to_out(row[2], ky, 1, g.pd[1], 1, g.os[1], &oy);
+    for (int kz = 0; kz < g.ks[2]; ++kz, ++k) {
+      int oz = 0;
+      const bool ok = okxy && tap_to_out(row[3], kz, 1, g.pd[2], 1, g.os[2], &oz);
+      unsigned long long m = __ballot(ok);
+      if (lane == 0) chunk_count[(int64_t)k * n_chunks + chunk] = __popcll(m);
+    }
+  }
+}
+
 // Submanifold / unique: mark the cells of the rows themselves.
 __global__ void __launch_bounds__(256)
     mark_rows_kernel(const int32_t *__restrict__ coords, int64_t n, int d0, int d1, int d2, int d3,
@@ -308,6 +381,61 @@ __global__ void __launch_bounds__(kScanThreads)
     scan_chunks_of_tap(chunk_count, n_chunks, (int)(blockIdx.x - n_scan_blocks), pair_num, lds);
 }
 
+// Output table from the input table (see "marking by dilation"), the block sums of its
+// popcounts (added into blocksum[], which starts at zero), and, in the K blocks after the
+// table's, the scan of the chunk counts.  Word (b, x, y, zw) of the output is the OR over
+// (kx, ky) of the bits 32 zw + kz .. + 31, for every kz, of input row (b, x + kx, y + ky).
+// One word per thread.  KS > 0: the kernel's three extents equal KS (loops unrolled, all
+// loads of a thread in flight at once); KS = 0: any extents.
+template <int KS>
+__global__ void __launch_bounds__(kScanThreads)
+    dilate_blocksum_kernel(const uint32_t *__restrict__ in_bits, Geom g, DenseIn d,
+                           uint32_t *__restrict__ bits, int64_t n_words, int64_t n_word_blocks,
+                           int32_t *__restrict__ blocksum, int32_t *__restrict__ chunk_count,
+                           int64_t n_chunks, int32_t *__restrict__ pair_num) {
+  if ((int64_t)blockIdx.x >= n_word_blocks) {
+    __shared__ int lds[kScanThreads / 64 + 1];
+    scan_chunks_of_tap(chunk_count, n_chunks, (int)(blockIdx.x - n_word_blocks), pair_num, lds);
+    return;
+  }
+  const int ksx = KS > 0 ? KS : g.ks[0], ksy = KS > 0 ? KS : g.ks[1], ksz = KS > 0 ? KS : g.ks[2];
+  const int64_t w = (int64_t)blockIdx.x * kScanThreads + threadIdx.x;
+  int v = 0;
+  if (w < n_words) {
+    const uint32_t zw_n = (uint32_t)g.os[2] >> 5;  // words per output row
+    uint32_t t = (uint32_t)w;                       // (fewer than 2^26 words)
+    const int zw = (int)(t % zw_n);
+    t /= zw_n;
+    const int y = (int)(t % (uint32_t)g.os[1]);
+    t /= (uint32_t)g.os[1];
+    const int x = (int)(t % (uint32_t)g.os[0]);
+    const int b = (int)(t / (uint32_t)g.os[0]);
+    const uint32_t *rowp = in_bits + (((int64_t)b * d.U[0] + x) * d.U[1] + y) * d.Wz + zw;
+    const int64_t xstep = (int64_t)d.U[1] * d.Wz;
+    uint32_t out = 0u;
+#pragma unroll
+    for (int kx = 0; kx < ksx; ++kx) {
+#pragma unroll
+      for (int ky = 0; ky < ksy; ++ky) {
+        const uint32_t *p = rowp + kx * xstep + ky * d.Wz;
+        // (with ksz > 1, Wz > os[2] / 32: word zw + 1 exists)
+        const uint32_t lo = p[0], hi = ksz > 1 ? p[1] : 0u;
+        uint32_t acc = lo;
+#pragma unroll
+        for (int kz = 1; kz < ksz; ++kz) acc |= (lo >> kz) | (hi << (32 - kz));
+        out |= acc;
+      }
+    }
+    bits[w] = out;
+    v = __popc(out);
+  }
+#pragma unroll
+  for (int s = 32; s >= 1; s >>= 1) v += __shfl_xor(v, s, 64);
+  // (the kScanThreads words of a block lie in one scan block of kScanBlockWords words)
+  if ((threadIdx.x & 63) == 0 && v != 0)
+    atomicAdd(&blocksum[((int64_t)blockIdx.x * kScanThreads) / kScanBlockWords], v);
+}
+
 // Pair emission: same traversal as count_pairs_kernel; a row's slot inside tap k
 // is (pairs of earlier chunks) + (earlier lanes of this chunk), which makes the
 // pair list ascending in input row.  The wave also pads slots [num, n_in) of
@@ -317,6 +445,8 @@ __global__ void __launch_bounds__(kScanThreads)
 // do an unrelated job that needs nothing but the scanned table either: they decode the
 // table into out_indices[], strided over its words.  One launch, and the two jobs, each
 // short and bound by latency, run side by side.
+// KS > 0: the kernel's y and z extents equal KS (loops unrolled); KS = 0: any extents.
+template <int KS>
 __global__ void __launch_bounds__(256)
     write_pairs_kernel(const int32_t *__restrict__ indices, int64_t n_in, Geom g,
                        const uint32_t *__restrict__ bits, const int32_t *__restrict__ prefix,
@@ -344,41 +474,43 @@ __global__ void __launch_bounds__(256)
   // space, so the table word and its prefix are loaded once per word, not per tap.
   uint32_t word = 0xFFFFFFFFu, wbits = 0u;
   int wprefix = 0;
-  // blockIdx.y = kx: the taps of one x offset per wave, for more waves in flight
+  // blockIdx.y = kx: the taps of one x offset per wave, for more waves in flight (a wave
+  // per (kx, ky) was tried and is no faster: the kernel is bound by its stores)
   const int kx = blockIdx.y;
   int k = kx * g.ks[1] * g.ks[2];
-  {
-    int ox = 0;
-    const bool okx = usable && tap_to_out(row[1], kx, g.st[0], g.pd[0], g.dl[0], g.os[0], &ox);
-    for (int ky = 0; ky < g.ks[1]; ++ky) {
-      int oy = 0;
-      const bool okxy = okx && tap_to_out(row[2], ky, g.st[1], g.pd[1], g.dl[1], g.os[1], &oy);
-      const uint32_t base = (uint32_t)(((row[0] * g.os[0] + ox) * g.os[1] + oy) * g.os[2]);
-      for (int kz = 0; kz < g.ks[2]; ++kz, ++k) {
-        int oz = 0;
-        bool ok = okxy && tap_to_out(row[3], kz, g.st[2], g.pd[2], g.dl[2], g.os[2], &oz);
-        const uint32_t key = base + (uint32_t)oz;
-        if (ok && (key >> 5) != word) {
-          word = key >> 5;
-          wbits = bits[word];
-          wprefix = prefix[word];
-        }
-        if (ok && g.subm) ok = (wbits >> (key & 31u)) & 1u;
-        unsigned long long m = __ballot(ok);
-        int32_t *pin = pairs + ((int64_t)k * 2 + 0) * n_in;
-        int32_t *pout = pairs + ((int64_t)k * 2 + 1) * n_in;
-        if (ok) {
-          int slot = chunk_prefix[(int64_t)k * n_chunks + chunk] +
-                     __popcll(m & ((1ull << lane) - 1ull));
-          int r = wprefix + __popc(wbits & ((1u << (key & 31u)) - 1u));
-          if (g.subm) r = rank2row[r];
-          pin[slot] = (int32_t)i;
-          pout[slot] = r;
-        }
-        if (live && i >= pair_num[k]) {
-          pin[i] = -1;
-          pout[i] = -1;
-        }
+  int ox = 0;
+  const bool okx = usable && tap_to_out(row[1], kx, g.st[0], g.pd[0], g.dl[0], g.os[0], &ox);
+  const int ksy = KS > 0 ? KS : g.ks[1], ksz = KS > 0 ? KS : g.ks[2];
+#pragma unroll
+  for (int ky = 0; ky < ksy; ++ky) {
+    int oy = 0;
+    const bool okxy = okx && tap_to_out(row[2], ky, g.st[1], g.pd[1], g.dl[1], g.os[1], &oy);
+    const uint32_t base = (uint32_t)(((row[0] * g.os[0] + ox) * g.os[1] + oy) * g.os[2]);
+#pragma unroll
+    for (int kz = 0; kz < ksz; ++kz, ++k) {
+      int oz = 0;
+      bool ok = okxy && tap_to_out(row[3], kz, g.st[2], g.pd[2], g.dl[2], g.os[2], &oz);
+      const uint32_t key = base + (uint32_t)oz;
+      if (ok && (key >> 5) != word) {
+        word = key >> 5;
+        wbits = bits[word];
+        wprefix = prefix[word];
+      }
+      if (ok && g.subm) ok = (wbits >> (key & 31u)) & 1u;
+      unsigned long long m = __ballot(ok);
+      int32_t *pin = pairs + ((int64_t)k * 2 + 0) * n_in;
+      int32_t *pout = pairs + ((int64_t)k * 2 + 1) * n_in;
+      if (ok) {
+        int slot = chunk_prefix[(int64_t)k * n_chunks + chunk] +
+                   __popcll(m & ((1ull << lane) - 1ull));
+        int r = wprefix + __popc(wbits & ((1u << (key & 31u)) - 1u));
+        if (g.subm) r = rank2row[r];
+        pin[slot] = (int32_t)i;
+        pout[slot] = r;
+      }
+      if (live && i >= pair_num[k]) {
+        pin[i] = -1;
+        pout[i] = -1;
       }
     }
   }
@@ -422,12 +554,19 @@ struct RulebookWs {
   int32_t *chunk_count;  // [K, n_chunks]
   int32_t *rank2row;     // [n_in] (subm)
   int64_t n_chunks;
+  uint32_t *in_bits;     // input table of the dilation path (when it applies)
+  DenseIn dense;
+  bool use_dense;
 };
 
 static size_t rulebook_ws_bytes(const Geom &g, int64_t n_in) {
   int64_t n_chunks = ceil_div(n_in > 0 ? n_in : 1, 64);
+  DenseIn d;
+  const size_t dense = dense_marking_applies(g, n_in, &d)
+                           ? align_up((size_t)dense_in_words(g, d) * 4)
+                           : 0;
   return bit_table_bytes(geom_cells(g)) + align_up((size_t)g.K * n_chunks * 4) +
-         align_up((size_t)(n_in > 0 ? n_in : 1) * 4);
+         align_up((size_t)(n_in > 0 ? n_in : 1) * 4) + dense;
 }
 
 static RulebookWs rulebook_ws_carve(void *ws, const Geom &g, int64_t n_in) {
@@ -437,6 +576,8 @@ static RulebookWs rulebook_ws_carve(void *ws, const Geom &g, int64_t n_in) {
   w.n_chunks = ceil_div(n_in > 0 ? n_in : 1, 64);
   w.chunk_count = c.take<int32_t>((size_t)g.K * w.n_chunks);
   w.rank2row = c.take<int32_t>(n_in > 0 ? n_in : 1);
+  w.use_dense = dense_marking_applies(g, n_in, &w.dense);
+  w.in_bits = w.use_dense ? c.take<uint32_t>((size_t)dense_in_words(g, w.dense)) : nullptr;
   return w;
 }
 
@@ -468,6 +609,27 @@ static int rulebook_mark_and_scan(const int32_t *indices, int64_t n_in, const Ge
                                   const RulebookWs &w, int32_t *pair_num, int32_t *mirror,
                                   hipStream_t s) {
   int rc;
+  if (w.use_dense && pair_num != nullptr) {
+    // input table cleared (with the totals), inputs marked, outputs by dilation
+    BitTable in = w.table;
+    in.bits = w.in_bits;
+    in.n_words = dense_in_words(gg, w.dense);
+    if ((rc = bit_table_clear(in, s, true)) != SSC_OK) return rc;
+    hipLaunchKernelGGL(mark_in_count_kernel,
+                       dim3((unsigned)ceil_div(w.n_chunks, 4), (unsigned)gg.ks[0]), dim3(256), 0, s,
+                       indices, n_in, gg, w.dense, w.in_bits, w.chunk_count, w.n_chunks,
+                       w.table.total + 1);
+    SSC_LAUNCH_CHECK("mark_in_count");
+    const int64_t word_blocks = ceil_div(w.table.n_words, kScanThreads);
+    const int ks = (gg.ks[0] == gg.ks[1] && gg.ks[1] == gg.ks[2]) ? gg.ks[0] : 0;
+    auto kernel = ks == 3 ? dilate_blocksum_kernel<3> : ks == 5 ? dilate_blocksum_kernel<5>
+                                                                : dilate_blocksum_kernel<0>;
+    hipLaunchKernelGGL(kernel, dim3((unsigned)(word_blocks + gg.K)), dim3(kScanThreads), 0, s,
+                       w.in_bits, gg, w.dense, w.table.bits, w.table.n_words, word_blocks,
+                       w.table.blocksum, w.chunk_count, w.n_chunks, pair_num);
+    SSC_LAUNCH_CHECK("dilate_blocksum");
+    return bit_table_scan_prefix(w.table, s, mirror);
+  }
   if ((rc = bit_table_clear(w.table, s)) != SSC_OK) return rc;
   if (gg.subm) {
     hipLaunchKernelGGL(mark_rows_kernel, dim3((unsigned)ceil_div(n_in, 256)), dim3(256), 0, s,
@@ -512,9 +674,12 @@ static int rulebook_pairs(const int32_t *indices, int64_t n_in, const Geom &gg,
                            ? 0
                            : ceil_div(ceil_div(w.table.n_words, 256), chunk_blocks);
   if (row_blocks > 4096) row_blocks = 4096;
-  hipLaunchKernelGGL(write_pairs_kernel, dim3(chunk_blocks, (unsigned)(gg.ks[0] + row_blocks)),
-                     dim3(256), 0, s, indices, n_in, gg, w.table.bits, w.table.prefix, w.rank2row,
-                     w.chunk_count, w.n_chunks, pair_num, pairs, w.table.n_words, out_indices);
+  const int ks = gg.ks[1] == gg.ks[2] ? gg.ks[1] : 0;
+  auto kernel = ks == 3 ? write_pairs_kernel<3> : ks == 5 ? write_pairs_kernel<5>
+                : ks == 2 ? write_pairs_kernel<2> : write_pairs_kernel<0>;
+  hipLaunchKernelGGL(kernel, dim3(chunk_blocks, (unsigned)(gg.ks[0] + row_blocks)), dim3(256), 0,
+                     s, indices, n_in, gg, w.table.bits, w.table.prefix, w.rank2row, w.chunk_count,
+                     w.n_chunks, pair_num, pairs, w.table.n_words, out_indices);
   SSC_LAUNCH_CHECK("write_pairs");
   return SSC_OK;
 }

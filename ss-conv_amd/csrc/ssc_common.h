@@ -69,8 +69,9 @@ struct BitTable {
 static inline int64_t bit_words(int64_t n_bits) { return ceil_div(n_bits, 32); }
 size_t bit_table_bytes(int64_t n_bits);
 BitTable bit_table_carve(Carver &c, int64_t n_bits);
-// Enqueue: zero the table.
-int bit_table_clear(const BitTable &t, hipStream_t s);
+// Enqueue: zero the table and total[]; with blocksum_too also blocksum[] (for a first scan
+// pass that adds into it).
+int bit_table_clear(const BitTable &t, hipStream_t s, bool blocksum_too = false);
 // Enqueue: prefix[], total[0] from bits[].  With `mirror` (memory the device can write and
 // the host can read, see read_back_mirror), the kernel that writes total[0] also copies
 // total[0..3] there, which saves the copy a host that waits for them would otherwise queue.

@@ -182,8 +182,9 @@ def _geometry(batch_size, out_shape, ksize, stride, padding, dilation, subm, tra
 
 
 # Output rows are written before their number is known when a buffer for the largest
-# possible number of them is at most this large (the result then keeps that buffer alive).
-_ROWS_AHEAD_BYTES = 64 << 20
+# possible number of them is at most this large (a result that fills less than a quarter of
+# a buffer of more than 16 MiB is copied out of it).
+_ROWS_AHEAD_BYTES = 512 << 20
 
 
 class RulebookMeta(object):
@@ -269,6 +270,8 @@ def _rulebook_finish(r):
         outids = r.indices
     elif r.out_buf is not None:
         outids = r.out_buf[:n_out.value]
+        if r.out_buf.size(0) > 4 * max(n_out.value, 1) and r.out_buf.numel() * 4 > (16 << 20):
+            outids = outids.clone()  # do not keep a large, mostly unused buffer alive
     else:
         # a geometry may leave no output at all (every candidate clipped): the library still
         # wants a valid pointer, so at least one row is allocated and the result is a slice
@@ -985,9 +988,10 @@ def field_scale(x, scale, field_of):
     return y
 
 
-def profile_conv(enable):
-    """Start (clearing earlier samples) or stop timing of the convolution kernel."""
-    _check(_lib.ssc_profile_conv(int(bool(enable))))
+def profile_conv(enable, every=1):
+    """Start (clearing earlier samples) or stop timing of the convolution kernel; with
+    `every` = n only every n-th launch is timed."""
+    _check(_lib.ssc_profile_conv(max(1, int(every)) if enable else 0))
 
 
 def profile_conv_read():

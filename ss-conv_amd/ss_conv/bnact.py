@@ -190,9 +190,16 @@ def usable(x):
 
 
 def canonical(Rs):
-    """The layout the gate tables describe: scalars (if any) first, then non-scalar fields."""
+    """The layout the gate tables describe: a first entry of scalars (possibly with
+    multiplicity 0), then non-scalar fields.  A first entry of order > 0 has no gates in the
+    reference's count (n_non_scalar = sum(multiplicities[1:]), activation.py:44-52) although
+    its loop asks for one per field: such a layer keeps the torch code, which fails at
+    forward as the reference's does."""
     Rs = [(m, l) for m, l in Rs]
-    return len(Rs) > 0 and all(l > 0 for m, l in Rs[1:] if m > 0)
+    if len(Rs) == 0:
+        return False
+    first_ok = Rs[0][1] == 0 or Rs[0][0] == 0
+    return first_ok and all(l > 0 for m, l in Rs[1:] if m > 0)
 
 
 def to_device(tables, device):

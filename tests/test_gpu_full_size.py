@@ -1,5 +1,6 @@
-"""GPU parity at the full sizes of the benchmark configurations (32 clouds x 2048 points at
-64^3 with stride 1 and 2; 8 clouds x 16384 points at 128^3 with a 5^3 kernel).
+"""GPU parity at the full sizes of the benchmark configurations (2 clouds x 1024 points at
+32^3; 32 clouds x 2048 points at 64^3 with stride 1 and 2; the backbone on 32 clouds x 1024
+points at 64^3; 8 clouds x 16384 points at 128^3 with a 5^3 kernel).
 
 Rulebooks: bit-exact against the oracle, which runs these sizes in seconds.
 Convolution, forward and both gradients: against the oracle's gather-GEMM-scatter where
@@ -17,7 +18,7 @@ from test_gpu_parity import REL_L2, rel_l2
 
 pytestmark = pytest.mark.gpu
 
-FULL = ["cfg2", "cfg3", "cfg5"]
+FULL = ["cfg1", "cfg2", "cfg3", "cfg5"]
 
 
 def _channels(cfg, key):
@@ -126,3 +127,101 @@ def test_layer_chain_full_size(device):
     pooled = GlobalAvgPool()(mx.features.contiguous(), offs)
     assert pooled.shape == (cfg["batch"], 64)
     assert torch.allclose(pooled[:, 0], torch.full((cfg["batch"],), 3.0, device=device))
+
+
+def test_backbone_full_size(oracle, device):
+    """The fourth configuration at its real size: Point2Voxel (32 clouds x 1024 points, 64^3)
+    -> four stages of [Convolution k3 -> BatchNorm -> gated Activation], irreps (8,8,8,8) ->
+    (16,...) -> (32,...) -> (32,...), stride 2 at stages 2 and 3 -> GlobalAvgPool and
+    Voxel2Point.  Every stage is checked by itself on the tensors the GPU path hands it:
+    the rulebook bit-exact against the oracle, the convolution against a float64 statement
+    of the same sums (one GEMM and one index_add per offset) plus the column-sum property,
+    batch norm + gate, the segment mean and the interpolation against the oracle, and the
+    grid search for the three nearest voxel centres against the plain scan, bit for bit, on
+    the last stage's 16^3 grid."""
+    from ss_conv import _ext
+    from ss_conv.activation import Activation
+    from ss_conv.batchnorm import BatchNorm
+    from ss_conv.convolution import Convolution
+    from ss_conv.fused import BatchNormActivation
+    from ss_conv.pool import GlobalAvgPool
+    from ss_conv.sp_ops.voxelize import Point2Voxel, Voxel2Point
+    torch.manual_seed(4)
+    batch, grid = 32, 64
+    pts, feats, ids = synth.make_clouds(batch, 1024, seed=1, channels=3)
+    p2v = Point2Voxel([grid] * 3, [2.0 / grid] * 3)
+    vp, x, vi, _ = p2v(*[torch.from_numpy(a).to(device) for a in (pts, feats, ids)])
+    ref = oracle.point2voxel(pts, feats, ids, [grid] * 3, [2.0 / grid] * 3)
+    assert np.array_equal(x.indices.cpu().numpy(), ref["indices"])
+    assert np.array_equal(x.features.cpu().numpy(), ref["features"])
+    shape = [grid] * 3
+    rs_in = [(3, 0)]
+    as_np = lambda t: t.detach().cpu().numpy()  # noqa: E731
+    for si, (mult, stride) in enumerate(((8, 1), (16, 2), (32, 2), (32, 1))):
+        rs = synth.irreps(mult, 3)
+        n_gates = sum(m for m, _ in rs[1:])
+        rs_gated = rs + [(n_gates, 0)]
+        cin = sum(m * (2 * l + 1) for m, l in rs_in)
+        cout = sum(m * (2 * l + 1) for m, l in rs_gated)
+        conv = Convolution(rs_in, rs_gated, 3, stride=stride, padding=1).to(device).train()
+        block = BatchNormActivation(BatchNorm(rs_gated), Activation(rs, (torch.relu, torch.sigmoid)))
+        block = block.to(device).train()
+        print("stage", si + 1, "rows in", x.features.shape[0], cin, "->", cout, flush=True)
+        in_idx, f = x.indices, x.features
+        with torch.no_grad():
+            for p in block.parameters():
+                p.add_(torch.randn_like(p) * 0.3)
+            y = conv(x)
+            w = conv.kernel().detach().permute(2, 3, 4, 1, 0).reshape(27, cin, cout)
+        out_idx, _, pairs, num, _ = y.indice_dict[None]
+        want = oracle.canonicalize(*oracle.rulebook(as_np(in_idx), batch, shape, 3, stride, 1))
+        for g, r in zip((out_idx, pairs, num), want):
+            assert np.array_equal(as_np(g), r), si
+        n_out = out_idx.shape[0]
+        nums = as_np(num)
+        ref64 = torch.zeros((n_out, cout), dtype=torch.float64, device=device)
+        col_sums = torch.zeros(cout, dtype=torch.float64, device=device)
+        for kk in range(27):
+            m = int(nums[kk])
+            if m == 0:
+                continue
+            fi = f[pairs[kk, 0, :m].long()].double()
+            ref64.index_add_(0, pairs[kk, 1, :m].long(), fi @ w[kk].double())
+            col_sums += fi.sum(0) @ w[kk].double()
+        assert _rel(y.features, ref64) < REL_L2, si
+        assert _rel(y.features.double().sum(0), col_sums) < REL_L2, si
+        del ref64
+        y_np = as_np(y.features)
+        with torch.no_grad():
+            x = block(y)
+        params = dict(weight=as_np(block.bn.weight), bias=as_np(block.bn.bias),
+                      scalar_bias=as_np(block.act.scalar_act.bias),
+                      gate_bias=as_np(block.act.gate_act.bias))
+        o_feat = oracle.bn_gate_fwd(y_np, rs_gated, rs, params, training=True)
+        err = rel_l2(as_np(x.features), o_feat)
+        print("  rows out", n_out, "pairs", int(nums.sum()), "bn+gate rel-l2", err, flush=True)
+        assert err < REL_L2, (si, err)
+        shape = [int(v) for v in y.spatial_shape]
+        rs_in = rs
+    assert shape == [16, 16, 16]
+    # heads
+    offs = x.get_offsets().int().contiguous()
+    pooled = GlobalAvgPool()(x.features.contiguous(), offs)
+    want = oracle.segment_avg(as_np(x.features), as_np(offs))
+    assert rel_l2(as_np(pooled), want) < REL_L2
+    unit = [2.0 / s for s in shape]
+    v2p = Voxel2Point(unit_voxel_extent=unit)
+    at_points = v2p(x, vp, vi)
+    want = oracle.voxel2point(as_np(x.indices), as_np(x.features), shape, as_np(vp), as_np(vi),
+                              unit_voxel_extent=unit)[0]
+    assert rel_l2(as_np(at_points), want) < REL_L2
+    # the grid search against the plain scan on this stage's voxels
+    centres, _ = v2p._get_vertice_feats(x)
+    queries = torch.cat([vi.float().unsqueeze(1), vp], dim=1).contiguous()
+    u, origin = v2p._grid(x)
+    d_grid, i_grid = _ext.three_nn_grid(queries, centres, x.indices.contiguous(), batch,
+                                        [s + 1 for s in shape], origin, u)
+    d_scan = torch.empty_like(d_grid)
+    i_scan = torch.empty_like(i_grid)
+    _ext.three_nn(queries.shape[0], centres.shape[0], queries, centres, d_scan, i_scan)
+    assert torch.equal(i_grid, i_scan) and torch.equal(d_grid, d_scan)

@@ -363,3 +363,20 @@ def test_synthetic_generator_is_seeded():
     assert np.abs(a[0]).max() < 1.0 and a[1].shape == (200, 3) and a[2].tolist()[99:101] == [0, 1]
     idx = synth.voxel_indices(a[0], a[2], 16)
     assert idx.min() >= 0 and idx[:, 1:].max() < 16
+
+
+def test_layers_outside_the_native_layouts():
+    """A gated activation whose first entry is not a scalar field keeps the torch code (the
+    gate tables would ask for gates the reference never counts); a transposed convolution
+    is refused when it is constructed, not at its first forward."""
+    from ss_conv import bnact
+    from ss_conv.activation import Activation
+    from ss_conv.sp_ops.conv import SparseConvolution
+    assert bnact.canonical([(4, 0), (2, 1), (2, 2)])
+    assert bnact.canonical([(0, 0), (2, 1)])
+    assert not bnact.canonical([(4, 1), (2, 2)])
+    assert not bnact.canonical([(4, 0), (2, 0)])
+    act = Activation([(4, 1), (2, 2)], (torch.relu, torch.sigmoid))
+    assert not act._kernel_ok
+    with pytest.raises(NotImplementedError):
+        SparseConvolution(3, 4, 4, 3, transposed=True)
