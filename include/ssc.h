@@ -449,6 +449,41 @@ int ssc_p2v_compact(const float *points, const float *feats /* [n,channels] */,
                     int32_t *out_coords /* [m,4] */, int32_t *out_dest /* [n] or NULL */,
                     ssc_stream_t stream);
 
+/* Point2Voxel.forward (ss_conv/sp_ops/voxelize.py:29-99) as one call, for batch ids that are
+ * non-decreasing and lie in [0, n_ids): point filter and batch partition (as ssc_p2v_scan /
+ * ssc_p2v_compact), voxel index of every row, sorted unique voxels (torch.unique(dim=0),
+ * voxelize.py:88), the voxel of every row, and the per-voxel feature reduction (voxelize_fp,
+ * src/voxelize/voxelize_cuda_kernel.h:18-40: mode 1 first point, 2 last point, 3 sum,
+ * 4 mean; points of a voxel are added in ascending point order).  All kernels are queued
+ * with the data-dependent sizes kept on the device and every output sized for n rows
+ * (there are never more rows or voxels than points); the call SYNCHRONISES once, for
+ *   totals_host = {rows m, voxels v, flags, batch ids left without points}
+ * and the histograms hist_all_host[n_ids] / hist_valid_host[n_ids] (points and surviving
+ * points per id), while its last kernels still run.  The first m rows of out_points [n,3],
+ * out_ids [n], inverse [n] (voxel of each row) and the first v rows of out_indices [n,4],
+ * out_feats [n,channels], counts [n] (points per voxel), sel [n] (modes 1 and 2: the row a
+ * voxel took its features from; may be NULL otherwise) are valid; dest [n] is the output row
+ * of every input row (-1: dropped).  flags != 0 (bit 0: an id outside [0, n_ids), bit 1:
+ * ids decrease, bit 2: a voxel outside the grid): the outputs must be discarded and another
+ * path taken.  The unique-rows table spans n_ids * prod(limit + 1) cells (< 2^31).
+ * ssc_p2v_voxelize_bwd_f32: gradient of the features, feats_grad [n,channels] written
+ * completely (voxelize_bp, src/voxelize/voxelize_cuda_kernel.h:44-58, through dest /
+ * inverse instead of the point lists). */
+size_t ssc_p2v_voxelize_workspace_bytes(int64_t n, int32_t n_ids, const int32_t limit[3]);
+int ssc_p2v_voxelize_f32(const float *points /* [n,3] */, const float *feats /* [n,channels] */,
+                         const int64_t *batch_ids /* [n] */, int64_t n, int32_t channels,
+                         const float half_extent[3], const float unit[3], const int32_t limit[3],
+                         int32_t n_ids, int32_t mode, void *workspace, size_t workspace_bytes,
+                         float *out_points, int64_t *out_ids, int32_t *out_indices,
+                         float *out_feats, int32_t *inverse, int32_t *counts, int32_t *dest,
+                         int32_t *sel, int32_t *hist_all_host /* [n_ids] host */,
+                         int32_t *hist_valid_host /* [n_ids] host */,
+                         int32_t *totals_host /* [4] host */, ssc_stream_t stream);
+int ssc_p2v_voxelize_bwd_f32(const float *out_grad /* [v,channels] */, int32_t channels,
+                             const int32_t *dest /* [n] */, const int32_t *inverse,
+                             const int32_t *counts, const int32_t *sel, int32_t mode, int64_t n,
+                             float *feats_grad /* [n,channels] */, ssc_stream_t stream);
+
 int ssc_voxel_map(const int32_t *inverse /* [n] */, const int32_t *ids /* [n] */,
                   int32_t *out_maps /* [m,max_active+1] */, int32_t n_point, int32_t n_voxel,
                   int32_t max_active, int32_t mode, ssc_stream_t stream);

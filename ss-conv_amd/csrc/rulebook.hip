@@ -257,42 +257,6 @@ __global__ void __launch_bounds__(256)
   atomicOr(&bits[key >> 5], 1u << (key & 31u));
 }
 
-// Decode every set bit of word w into its (b,x,y,z) row, written at the bit's rank.
-__device__ __forceinline__ void emit_rows_of_word(const uint32_t *__restrict__ bits,
-                                                  const int32_t *__restrict__ prefix, int64_t w,
-                                                  int d1, int d2, int d3,
-                                                  int32_t *__restrict__ out) {
-  uint32_t b = bits[w];
-  if (b == 0) return;
-  int r = prefix[w];
-  // the word's first cell is decoded once; its other cells differ in z only, unless
-  // the word runs over the end of a z row (extents that are not multiples of 32)
-  uint32_t key0 = (uint32_t)(w * 32);
-  const int z0 = key0 % d3;
-  key0 /= d3;
-  const int y0 = key0 % d2;
-  key0 /= d2;
-  const int x0 = key0 % d1;
-  const int b0 = key0 / d1;
-  while (b) {
-    int bit = __ffs(b) - 1;
-    b &= b - 1;
-    int z = z0 + bit;
-    if (z < d3) {
-      reinterpret_cast<int4 *>(out)[r++] = make_int4(b0, x0, y0, z);
-    } else {
-      uint32_t key = (uint32_t)(w * 32 + bit);
-      z = key % d3;
-      key /= d3;
-      int y = key % d2;
-      key /= d2;
-      int x = key % d1;
-      int bb = key / d1;
-      reinterpret_cast<int4 *>(out)[r++] = make_int4(bb, x, y, z);
-    }
-  }
-}
-
 __global__ void __launch_bounds__(256)
     emit_rows_kernel(const uint32_t *__restrict__ bits, const int32_t *__restrict__ prefix,
                      int64_t n_words, int d1, int d2, int d3, int32_t *__restrict__ out) {

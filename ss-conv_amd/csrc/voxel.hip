@@ -661,10 +661,10 @@ namespace ssc {
 
 // Pass 1: one wave per 64 points.  inside bit per point (a ballot: no atomics),
 // histograms of all ids and of the surviving ids (one atomic per distinct id and
-// wave), flags[0] |= 1 for an id outside [0, SSC_P2V_MAX_IDS), flags[1] |= 1 when ids decrease.
+// wave), flags[0] |= 1 for an id outside [0, max_ids), flags[1] |= 1 when ids decrease.
 __global__ void __launch_bounds__(256)
     p2v_scan_kernel(const float *__restrict__ pts, const int64_t *__restrict__ ids, int64_t n,
-                    float hx, float hy, float hz, uint32_t *__restrict__ bits,
+                    float hx, float hy, float hz, int max_ids, uint32_t *__restrict__ bits,
                     int32_t *__restrict__ hist_all, int32_t *__restrict__ hist_valid,
                     int32_t *__restrict__ flags) {
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -676,12 +676,12 @@ __global__ void __launch_bounds__(256)
     const float x = pts[i * 3], y = pts[i * 3 + 1], z = pts[i * 3 + 2];
     inside = !(fabsf(x) > hx) && !(fabsf(y) > hy) && !(fabsf(z) > hz);
     id = ids[i];
-    if (id < 0 || id >= SSC_P2V_MAX_IDS) atomicOr(&flags[0], 1);
+    if (id < 0 || id >= max_ids) atomicOr(&flags[0], 1);
     if (i > 0 && ids[i - 1] > id) atomicOr(&flags[1], 1);
   }
   const unsigned long long in_mask = __ballot(inside);
   if (live && (lane & 31) == 0) bits[i >> 5] = (uint32_t)(in_mask >> (lane & 32));
-  const bool ok_id = live && id >= 0 && id < SSC_P2V_MAX_IDS;
+  const bool ok_id = live && id >= 0 && id < max_ids;
   unsigned long long todo = __ballot(ok_id);
   while (todo) {  // one trip per distinct id of the wave
     const int first = __ffsll((long long)todo) - 1;
@@ -696,13 +696,15 @@ __global__ void __launch_bounds__(256)
   }
 }
 
-// One block: start[e] = survivors with an id below e; shift[e] = ids below e that are
-// present but have no survivor (each of them receives one zero point).
-__global__ void __launch_bounds__(256)
-    p2v_prefix_kernel(const int32_t *__restrict__ hist_all, const int32_t *__restrict__ hist_valid,
-                      int32_t *__restrict__ start, int32_t *__restrict__ shift) {
+// One block of 256 threads: start[e] = survivors with an id below e; shift[e] = ids below e
+// that are present but have no survivor (each of them receives one zero point).  Returns
+// the number of such ids in *n_empty (thread 255 holds it).
+__device__ __forceinline__ void p2v_prefix_block(const int32_t *__restrict__ hist_all,
+                                                 const int32_t *__restrict__ hist_valid,
+                                                 int32_t *__restrict__ start,
+                                                 int32_t *__restrict__ shift, int *s_valid,
+                                                 int *s_empty, int *n_empty) {
   constexpr int PER = SSC_P2V_MAX_IDS / 256;
-  __shared__ int s_valid[256], s_empty[256];
   const int t = threadIdx.x;
   int sv = 0, se = 0;
   for (int j = 0; j < PER; ++j) {
@@ -725,6 +727,15 @@ __global__ void __launch_bounds__(256)
     bv += hist_valid[e];
     be += (hist_all[e] > 0 && hist_valid[e] == 0) ? 1 : 0;
   }
+  *n_empty = be;  // of thread 255: all of them
+}
+
+__global__ void __launch_bounds__(256)
+    p2v_prefix_kernel(const int32_t *__restrict__ hist_all, const int32_t *__restrict__ hist_valid,
+                      int32_t *__restrict__ start, int32_t *__restrict__ shift) {
+  __shared__ int s_valid[256], s_empty[256];
+  int n_empty;
+  p2v_prefix_block(hist_all, hist_valid, start, shift, s_valid, s_empty, &n_empty);
 }
 
 // Pass 2a: surviving point i goes to row rank(i) + shift[id]; threads n..n+MAX_IDS-1
@@ -738,14 +749,18 @@ __global__ void __launch_bounds__(256)
                        const int32_t *__restrict__ shift, float hx, float hy, float hz, float ux,
                        float uy, float uz, float *__restrict__ out_pts,
                        int64_t *__restrict__ out_ids, int32_t *__restrict__ coords,
-                       int32_t *__restrict__ dest) {
+                       int32_t *__restrict__ dest, int32_t *__restrict__ src, int max_ids,
+                       uint32_t *__restrict__ vox_bits, int d1, int d2, int d3,
+                       int32_t *__restrict__ flags) {
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   float x = 0.f, y = 0.f, z = 0.f;
   int64_t id;
   int pos;
   if (i < n) {
-    const bool inside = (bits[i >> 5] >> (i & 31)) & 1u;
     id = ids[i];
+    // (a caller that runs this kernel without looking at the scan's flags first may hold
+    // ids outside the tables: such a point is dropped, the flags tell)
+    const bool inside = ((bits[i >> 5] >> (i & 31)) & 1u) && id >= 0 && id < max_ids;
     pos = inside ? bit_rank(bits, prefix, (uint32_t)i) + shift[id] : -1;
     dest[i] = pos;
     if (!inside) return;
@@ -754,9 +769,10 @@ __global__ void __launch_bounds__(256)
     z = pts[i * 3 + 2];
   } else {
     id = i - n;
-    if (id >= SSC_P2V_MAX_IDS || hist_all[id] == 0 || hist_valid[id] != 0) return;
+    if (id >= max_ids || hist_all[id] == 0 || hist_valid[id] != 0) return;
     pos = start[id] + shift[id];
   }
+  if (src != nullptr) src[pos] = i < n ? (int32_t)i : -1;  // input row behind output row pos
   out_pts[(int64_t)pos * 3] = x;
   out_pts[(int64_t)pos * 3 + 1] = y;
   out_pts[(int64_t)pos * 3 + 2] = z;
@@ -765,6 +781,14 @@ __global__ void __launch_bounds__(256)
   const int vy = (int)((y + hy) / uy);
   const int vz = (int)((z + hz) / uz);
   reinterpret_cast<int4 *>(coords)[pos] = make_int4((int)id, vx, vy, vz);
+  if (vox_bits != nullptr) {  // mark the voxel in the table of the unique-rows step
+    if ((unsigned)vx < (unsigned)d1 && (unsigned)vy < (unsigned)d2 && (unsigned)vz < (unsigned)d3) {
+      const uint32_t key = (uint32_t)((((int)id * d1 + vx) * d2 + vy) * d3 + vz);
+      atomicOr(&vox_bits[key >> 5], 1u << (key & 31u));
+    } else {
+      atomicOr(&flags[0], 4);
+    }
+  }
 }
 
 // Pass 2b: feature rows follow their points (dest[i] from pass 2a, -1 = dropped);
@@ -836,8 +860,8 @@ int ssc_p2v_scan(const float *points, const int64_t *batch_ids, int64_t n,
   const int64_t clear_n = (w.flags + 2) - w.hist_all;
   if ((rc = fill_i32(w.hist_all, clear_n, 0, s)) != SSC_OK) return rc;
   hipLaunchKernelGGL(p2v_scan_kernel, dim3((unsigned)ceil_div(n, 256)), dim3(256), 0, s, points,
-                     batch_ids, n, half_extent[0], half_extent[1], half_extent[2], w.table.bits,
-                     w.hist_all, w.hist_valid, w.flags);
+                     batch_ids, n, half_extent[0], half_extent[1], half_extent[2],
+                     (int)SSC_P2V_MAX_IDS, w.table.bits, w.hist_all, w.hist_valid, w.flags);
   SSC_LAUNCH_CHECK("p2v_scan");
   if ((rc = bit_table_scan(w.table, s)) != SSC_OK) return rc;
   hipLaunchKernelGGL(p2v_prefix_kernel, dim3(1), dim3(256), 0, s, w.hist_all, w.hist_valid,
@@ -874,12 +898,371 @@ int ssc_p2v_compact(const float *points, const float *feats, const int64_t *batc
   hipLaunchKernelGGL(p2v_compact_kernel, dim3((unsigned)ceil_div(rows, 256)), dim3(256), 0, s,
                      points, batch_ids, n, w.table.bits, w.table.prefix, w.hist_all, w.hist_valid,
                      w.start, w.shift, half_extent[0], half_extent[1], half_extent[2], unit[0],
-                     unit[1], unit[2], out_points, out_ids, out_coords, dest);
+                     unit[1], unit[2], out_points, out_ids, out_coords, dest, (int32_t *)nullptr,
+                     (int)SSC_P2V_MAX_IDS, (uint32_t *)nullptr, 0, 0, 0, (int32_t *)nullptr);
   SSC_LAUNCH_CHECK("p2v_compact");
   hipLaunchKernelGGL(p2v_feats_kernel, dim3((unsigned)ceil_div(rows * channels, 256)), dim3(256), 0,
                      s, feats, n, (int)channels, dest, w.hist_all, w.hist_valid, w.start,
                      w.shift, out_feats);
   SSC_LAUNCH_CHECK("p2v_feats");
+  return SSC_OK;
+}
+}
+
+// ---- Point2Voxel in one call ---------------------------------------------------------------
+// Filter, batch partition, unique voxels and the per-voxel feature reduction of
+// Point2Voxel.forward (ss_conv/sp_ops/voxelize.py:40-99) queued as one chain of kernels that
+// keeps every data-dependent size on the device: outputs are written into buffers with room
+// for n rows (there are never more rows or voxels than points), the totals land in pinned
+// host memory, and the host waits once, for them, while the last two kernels still run.
+// The per-voxel point lists are linked chains (head[voxel], next[row]; built with an atomic
+// exchange, so in no particular order); the reduction brings each chain into ascending row
+// order through a bit map over row numbers held one word per lane, which makes the sums
+// independent of the race -- and leaves no [voxels, largest population] table to size.
+namespace ssc {
+
+// Everything the chain needs cleared, in one launch: a[0..n_a) = 0 (histograms and flags),
+// vox_bits[0..n_words) = 0, head[0..n_head) = -1, totals[0..8) = 0.
+__global__ void __launch_bounds__(256)
+    p2vx_clear_kernel(int32_t *__restrict__ a, int64_t n_a, uint32_t *__restrict__ vox_bits,
+                      int64_t n_words, int32_t *__restrict__ head, int64_t n_head,
+                      int32_t *__restrict__ totals) {
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t step = (int64_t)gridDim.x * blockDim.x;
+  if (i < 8) totals[i] = 0;
+  for (int64_t j = i; j < n_a; j += step) a[j] = 0;
+  for (int64_t j = i; j < n_head; j += step) head[j] = -1;
+  for (int64_t j = i; j < n_words; j += step) vox_bits[j] = 0u;
+}
+
+// Blocks below n_scan_blocks: first pass of the scan over the inside bits.  The block after
+// them: per-id start and shift, the number of ids left without points into extra[0], and
+// the two histograms (max_ids entries each) into the host-visible mirror.
+__global__ void __launch_bounds__(kScanThreads)
+    p2vx_blocksum_prefix_kernel(const uint32_t *__restrict__ bits, int64_t n_words,
+                                int32_t *__restrict__ blocksum, int64_t n_scan_blocks,
+                                const int32_t *__restrict__ hist_all,
+                                const int32_t *__restrict__ hist_valid,
+                                int32_t *__restrict__ start, int32_t *__restrict__ shift,
+                                int32_t *__restrict__ extra, int max_ids,
+                                int32_t *__restrict__ mirror_hist) {
+  __shared__ int s_a[256], s_b[256];
+  if ((int64_t)blockIdx.x < n_scan_blocks) {
+    popc_blocksum_block(bits, n_words, blockIdx.x, blocksum, s_a);
+    return;
+  }
+  int n_empty;
+  p2v_prefix_block(hist_all, hist_valid, start, shift, s_a, s_b, &n_empty);
+  if (threadIdx.x == 255) extra[0] = n_empty;
+  for (int e = threadIdx.x; e < max_ids; e += 256) {
+    mirror_hist[e] = hist_all[e];
+    mirror_hist[max_ids + e] = hist_valid[e];
+  }
+}
+
+// Blocks below link_blocks: row pos < rows: inverse[pos] = rank of its voxel, and the row is
+// pushed onto that voxel's chain.  The other blocks decode the voxel table into out_indices.
+__global__ void __launch_bounds__(256)
+    p2vx_link_kernel(const int32_t *__restrict__ coords, const int32_t *__restrict__ n_inside,
+                     const int32_t *__restrict__ extra, const uint32_t *__restrict__ vox_bits,
+                     const int32_t *__restrict__ vox_prefix, int64_t n_words, int d0, int d1,
+                     int d2, int d3, int64_t link_blocks, const int32_t *__restrict__ flags,
+                     int32_t *__restrict__ inverse, int32_t *__restrict__ head,
+                     int32_t *__restrict__ next, int32_t *__restrict__ out_indices) {
+  // With a flag set (ids outside the tables, ids out of order, a voxel outside the grid)
+  // the compaction has left rows unwritten and the caller will discard everything: the
+  // rows' tables must not be followed.
+  if ((flags[0] | flags[1]) != 0) return;
+  if ((int64_t)blockIdx.x >= link_blocks) {
+    const int64_t step = (int64_t)(gridDim.x - link_blocks) * blockDim.x;
+    int64_t w = ((int64_t)blockIdx.x - link_blocks) * blockDim.x + threadIdx.x;
+    for (; w < n_words; w += step) emit_rows_of_word(vox_bits, vox_prefix, w, d1, d2, d3, out_indices);
+    return;
+  }
+  const int64_t pos = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (pos >= (int64_t)n_inside[0] + extra[0]) return;
+  const int4 r = reinterpret_cast<const int4 *>(coords)[pos];
+  if (!((unsigned)r.x < (unsigned)d0 && (unsigned)r.y < (unsigned)d1 &&
+        (unsigned)r.z < (unsigned)d2 && (unsigned)r.w < (unsigned)d3)) {
+    inverse[pos] = -1;  // (flagged by the kernel that marked the table)
+    return;
+  }
+  const uint32_t key = (uint32_t)(((r.x * d1 + r.y) * d2 + r.z) * d3 + r.w);
+  const int rk = bit_rank(vox_bits, vox_prefix, key);
+  inverse[pos] = rk;
+  next[pos] = atomicExch(&head[rk], (int32_t)pos);
+}
+
+// One wave per voxel: walk the chain (count, smallest and largest row), then
+//   mode 1 / 2: the features of the first / last row,
+//   mode 3 / 4: sum over the rows in ascending order of mult * feats, mult = 1 / count in
+//               mode 4 (product rounded before the add, as in voxel_reduce_kernel).
+// Ascending order: rows of a window of 2048 row numbers are entered into a bit map, lane l
+// holding word l, and read back bit by bit; windows follow each other upwards.  Lanes run
+// along the channels.  src[row] is the input row behind a row (-1: a zero point).
+__global__ void __launch_bounds__(256)
+    p2vx_reduce_kernel(const float *__restrict__ feats, int C, const int32_t *__restrict__ src,
+                       const int32_t *__restrict__ head, const int32_t *__restrict__ next,
+                       const int32_t *__restrict__ n_voxel, const int32_t *__restrict__ flags,
+                       int mode, float *__restrict__ out, int32_t *__restrict__ counts,
+                       int32_t *__restrict__ sel) {
+  if ((flags[0] | flags[1]) != 0) return;  // (see p2vx_link_kernel)
+  const int lane = threadIdx.x & 63;
+  const int64_t v = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (v >= n_voxel[0]) return;  // (the same for the whole wave)
+  const int first = __builtin_amdgcn_readfirstlane(head[v]);
+  int n = 0, lo = 0x7FFFFFFF, hi = -1;
+  for (int p = first; p >= 0; p = __builtin_amdgcn_readfirstlane(next[p])) {
+    ++n;
+    lo = p < lo ? p : lo;
+    hi = p > hi ? p : hi;
+  }
+  if (lane == 0) counts[v] = n;
+  float *o = out + v * C;
+  if (mode == 1 || mode == 2) {
+    const int p = mode == 1 ? lo : hi;
+    if (lane == 0 && sel != nullptr) sel[v] = p;
+    const int sr = n > 0 ? __builtin_amdgcn_readfirstlane(src[p]) : -1;
+    for (int c = lane; c < C; c += 64) o[c] = sr >= 0 ? feats[(int64_t)sr * C + c] : 0.f;
+    return;
+  }
+  const float mult = (mode == 4 && n > 0) ? 1.f / (float)n : 1.f;
+  for (int c0 = 0; c0 < C; c0 += 256) {
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    auto add_row = [&](int p) {
+      const int sr = __builtin_amdgcn_readfirstlane(src[p]);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int c = c0 + lane + 64 * j;
+        if (c < C) {
+          const float f = sr >= 0 ? feats[(int64_t)sr * C + c] : 0.f;
+          const float t = mult * f;
+          acc[j] = acc[j] + t;
+        }
+      }
+    };
+    if (n == 1) {
+      add_row(lo);
+    } else if (n > 1) {
+      for (int base = lo & ~2047; base <= hi; base += 2048) {
+        uint32_t mine = 0u;
+        for (int p = first; p >= 0; p = __builtin_amdgcn_readfirstlane(next[p])) {
+          const int off = p - base;
+          if ((unsigned)off < 2048u && (off >> 5) == lane) mine |= 1u << (off & 31);
+        }
+        unsigned long long lanes = __ballot(mine != 0u);
+        while (lanes) {
+          const int l = __ffsll((long long)lanes) - 1;
+          lanes &= lanes - 1;
+          uint32_t w = (uint32_t)__shfl((int)mine, l, 64);
+          while (w) {
+            const int b = __ffs((int)w) - 1;
+            w &= w - 1;
+            add_row(base + l * 32 + b);
+          }
+        }
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int c = c0 + lane + 64 * j;
+      if (c < C) o[c] = acc[j];
+    }
+  }
+}
+
+// d_feats[i, c] of input row i: mult * d_out[voxel of its row] (modes 3 / 4), d_out for the
+// row its voxel took its features from (modes 1 / 2), 0 for a dropped row
+// (src/voxelize/voxelize_cuda_kernel.h:44-58 through the point lists).
+__global__ void __launch_bounds__(256)
+    p2vx_bwd_kernel(const float *__restrict__ d_out, int C, const int32_t *__restrict__ dest,
+                    const int32_t *__restrict__ inverse, const int32_t *__restrict__ counts,
+                    const int32_t *__restrict__ sel, int mode, int64_t n,
+                    float *__restrict__ d_feats) {
+  const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (e >= n * C) return;
+  const int64_t i = e / C;
+  const int c = (int)(e - i * C);
+  float g = 0.f;
+  const int pos = dest[i];
+  if (pos >= 0) {
+    const int v = inverse[pos];
+    if (v >= 0) {
+      if (mode == 1 || mode == 2) {
+        if (sel[v] == pos) g = d_out[(int64_t)v * C + c];
+      } else {
+        const float mult = mode == 4 ? 1.f / (float)counts[v] : 1.f;
+        g = mult * d_out[(int64_t)v * C + c];
+      }
+    }
+  }
+  d_feats[e] = g;
+}
+
+// mirror[0] = voxels, [1] = surviving points, [2] = ids left without points, [3] = flags
+// (bit 0: an id outside the table, bit 1: ids decrease, bit 2: a voxel outside the grid).
+__global__ void p2vx_totals_kernel(const int32_t *__restrict__ vox_total,
+                                   const int32_t *__restrict__ inside_total,
+                                   const int32_t *__restrict__ extra,
+                                   const int32_t *__restrict__ flags,
+                                   int32_t *__restrict__ mirror) {
+  if (threadIdx.x == 0) {
+    mirror[0] = vox_total[0];
+    mirror[1] = inside_total[0];
+    mirror[2] = extra[0];
+    mirror[3] = (flags[0] & 5) | ((flags[1] & 1) << 1);
+  }
+}
+
+struct P2vxWs {
+  BitTable inside;  // over the n points
+  BitTable vox;     // over the voxel grid
+  int32_t *hist_all, *hist_valid, *flags, *start, *shift;
+  int32_t *coords, *head, *next, *src, *totals;
+};
+
+static size_t p2vx_ws_walk(void *base, int64_t n, int64_t cells, P2vxWs *w) {
+  Carver c(base);
+  P2vxWs t;
+  const size_t rows = (size_t)(n > 0 ? n : 1);
+  t.inside = bit_table_carve(c, (int64_t)rows);
+  t.vox = bit_table_carve(c, cells);
+  t.hist_all = c.take<int32_t>(SSC_P2V_MAX_IDS);
+  t.hist_valid = c.take<int32_t>(SSC_P2V_MAX_IDS);  // directly behind hist_all
+  t.flags = c.take<int32_t>(2);                      // directly behind hist_valid
+  t.start = c.take<int32_t>(SSC_P2V_MAX_IDS);
+  t.shift = c.take<int32_t>(SSC_P2V_MAX_IDS);
+  t.coords = c.take<int32_t>(rows * 4);
+  t.head = c.take<int32_t>(rows);
+  t.next = c.take<int32_t>(rows);
+  t.src = c.take<int32_t>(rows);
+  t.totals = c.take<int32_t>(8);
+  if (w) *w = t;
+  return c.used;
+}
+
+static int64_t p2vx_cells(int32_t n_ids, const int32_t limit[3]) {
+  if (n_ids < 1 || n_ids > SSC_P2V_MAX_IDS) return 0;
+  int64_t cells = n_ids;
+  for (int a = 0; a < 3; ++a) {
+    if (limit[a] < 1) return 0;
+    cells *= (int64_t)limit[a] + 1;  // a point on the upper face has index == limit
+    if (cells >= ((int64_t)1 << 31)) return 0;
+  }
+  return cells;
+}
+
+}  // namespace ssc
+
+extern "C" {
+
+size_t ssc_p2v_voxelize_workspace_bytes(int64_t n, int32_t n_ids, const int32_t limit[3]) {
+  if (n < 0 || limit == nullptr) return 0;
+  const int64_t cells = ssc::p2vx_cells(n_ids, limit);
+  if (cells == 0) return 0;
+  return ssc::p2vx_ws_walk(nullptr, n, cells, nullptr);
+}
+
+int ssc_p2v_voxelize_f32(const float *points, const float *feats, const int64_t *batch_ids,
+                         int64_t n, int32_t channels, const float half_extent[3],
+                         const float unit[3], const int32_t limit[3], int32_t n_ids, int32_t mode,
+                         void *workspace, size_t workspace_bytes, float *out_points,
+                         int64_t *out_ids, int32_t *out_indices, float *out_feats,
+                         int32_t *inverse, int32_t *counts, int32_t *dest, int32_t *sel,
+                         int32_t *hist_all_host, int32_t *hist_valid_host, int32_t *totals_host,
+                         ssc_stream_t stream) {
+  SSC_CHECK(n > 0 && n < ((int64_t)1 << 31) && channels >= 1, SSC_EINVAL, "bad sizes");
+  SSC_CHECK(mode >= 1 && mode <= 4, SSC_EINVAL, "mode must be 1, 2, 3 or 4");
+  SSC_CHECK(points && feats && batch_ids && half_extent && unit && limit && workspace &&
+                out_points && out_ids && out_indices && out_feats && inverse && counts && dest &&
+                hist_all_host && hist_valid_host && totals_host,
+            SSC_EINVAL, "NULL pointer argument");
+  SSC_CHECK(mode >= 3 || sel != nullptr, SSC_EINVAL, "sel is NULL (modes 1 and 2 need it)");
+  const int64_t cells = p2vx_cells(n_ids, limit);
+  SSC_CHECK(cells > 0, SSC_EINVAL,
+            "n_ids must lie in [1, %d] and n_ids * prod(limit + 1) below 2^31",
+            (int)SSC_P2V_MAX_IDS);
+  SSC_CHECK(workspace_bytes >= p2vx_ws_walk(nullptr, n, cells, nullptr), SSC_EWORKSPACE,
+            "p2v workspace too small");
+  static_assert((16 + 2 * SSC_P2V_MAX_IDS) * sizeof(int32_t) <= kReadBackBytes, "pinned block");
+  hipStream_t s = (hipStream_t)stream;
+  P2vxWs w;
+  p2vx_ws_walk(workspace, n, cells, &w);
+  const int d1 = limit[0] + 1, d2 = limit[1] + 1, d3 = limit[2] + 1;
+  int rc;
+  int32_t *mirror = nullptr;
+  if ((rc = read_back_mirror(&mirror)) != SSC_OK) return rc;
+  // mirror: [0..3] sizes and flags (p2vx_totals_kernel), [16 ..) the two histograms
+  int32_t *extra = w.totals;  // [0]: ids left without points
+
+  const int64_t clear_a = (w.flags + 2) - w.hist_all;
+  const int64_t clear_most = w.vox.n_words > n ? w.vox.n_words : n;
+  const int64_t clear_blocks = ceil_div(clear_most > clear_a ? clear_most : clear_a, 256);
+  hipLaunchKernelGGL(p2vx_clear_kernel, dim3((unsigned)(clear_blocks < 4096 ? clear_blocks : 4096)),
+                     dim3(256), 0, s, w.hist_all, clear_a, w.vox.bits, w.vox.n_words, w.head, n,
+                     w.totals);
+  SSC_LAUNCH_CHECK("p2vx_clear");
+  hipLaunchKernelGGL(p2v_scan_kernel, dim3((unsigned)ceil_div(n, 256)), dim3(256), 0, s, points,
+                     batch_ids, n, half_extent[0], half_extent[1], half_extent[2], (int)n_ids,
+                     w.inside.bits, w.hist_all, w.hist_valid, w.flags);
+  SSC_LAUNCH_CHECK("p2v_scan");
+  hipLaunchKernelGGL(p2vx_blocksum_prefix_kernel, dim3((unsigned)(w.inside.n_scan_blocks + 1)),
+                     dim3(kScanThreads), 0, s, w.inside.bits, w.inside.n_words, w.inside.blocksum,
+                     w.inside.n_scan_blocks, w.hist_all, w.hist_valid, w.start, w.shift, extra,
+                     (int)n_ids, mirror + 16);
+  SSC_LAUNCH_CHECK("p2vx_blocksum_prefix");
+  if ((rc = bit_table_scan_prefix(w.inside, s, nullptr)) != SSC_OK) return rc;
+  const int64_t rows = n + n_ids;
+  hipLaunchKernelGGL(p2v_compact_kernel, dim3((unsigned)ceil_div(rows, 256)), dim3(256), 0, s,
+                     points, batch_ids, n, w.inside.bits, w.inside.prefix, w.hist_all, w.hist_valid,
+                     w.start, w.shift, half_extent[0], half_extent[1], half_extent[2], unit[0],
+                     unit[1], unit[2], out_points, out_ids, w.coords, dest, w.src, (int)n_ids,
+                     w.vox.bits, d1, d2, d3, w.flags);
+  SSC_LAUNCH_CHECK("p2v_compact");
+  // flags of the scan and of the marking travel with the voxel table's totals
+  if ((rc = bit_table_scan(w.vox, s, nullptr)) != SSC_OK) return rc;
+  // the host's copy of the sizes and flags: a small kernel behind the scans, then the event
+  // the host will wait for; the two kernels after it run while the host wakes up
+  hipLaunchKernelGGL(p2vx_totals_kernel, dim3(1), dim3(64), 0, s, w.vox.total, w.inside.total, extra,
+                     w.flags, mirror);
+  SSC_LAUNCH_CHECK("p2vx_totals");
+  if ((rc = read_back_mirror_queued(s)) != SSC_OK) return rc;
+  const int64_t link_blocks = ceil_div(n, 256);
+  int64_t row_blocks = ceil_div(w.vox.n_words, 256);
+  if (row_blocks > 2048) row_blocks = 2048;
+  hipLaunchKernelGGL(p2vx_link_kernel, dim3((unsigned)(link_blocks + row_blocks)), dim3(256), 0, s,
+                     w.coords, w.inside.total, extra, w.vox.bits, w.vox.prefix, w.vox.n_words,
+                     (int)n_ids, d1, d2, d3, link_blocks, w.flags, inverse, w.head, w.next,
+                     out_indices);
+  SSC_LAUNCH_CHECK("p2vx_link");
+  hipLaunchKernelGGL(p2vx_reduce_kernel, dim3((unsigned)ceil_div(n, 4)), dim3(256), 0, s, feats,
+                     (int)channels, w.src, w.head, w.next, w.vox.total, w.flags, (int)mode, out_feats,
+                     counts, sel);
+  SSC_LAUNCH_CHECK("p2vx_reduce");
+  const void *view;
+  if ((rc = read_back_end(&view)) != SSC_OK) return rc;
+  const int32_t *m = static_cast<const int32_t *>(view);
+  totals_host[0] = m[1] + m[2];  // rows: survivors + zero points
+  totals_host[1] = m[0];         // voxels
+  totals_host[2] = m[3];         // flags
+  totals_host[3] = m[2];         // ids left without points
+  memcpy(hist_all_host, m + 16, (size_t)n_ids * sizeof(int32_t));
+  memcpy(hist_valid_host, m + 16 + n_ids, (size_t)n_ids * sizeof(int32_t));
+  return SSC_OK;
+}
+
+int ssc_p2v_voxelize_bwd_f32(const float *out_grad, int32_t channels, const int32_t *dest,
+                             const int32_t *inverse, const int32_t *counts, const int32_t *sel,
+                             int32_t mode, int64_t n, float *feats_grad, ssc_stream_t stream) {
+  SSC_CHECK(n >= 0 && channels >= 1 && mode >= 1 && mode <= 4, SSC_EINVAL, "bad sizes");
+  if (n == 0) return SSC_OK;
+  SSC_CHECK(out_grad && dest && inverse && counts && feats_grad, SSC_EINVAL,
+            "NULL pointer argument");
+  SSC_CHECK(mode >= 3 || sel != nullptr, SSC_EINVAL, "sel is NULL (modes 1 and 2 need it)");
+  hipLaunchKernelGGL(p2vx_bwd_kernel, dim3((unsigned)ceil_div(n * channels, 256)), dim3(256), 0,
+                     (hipStream_t)stream, out_grad, (int)channels, dest, inverse, counts, sel,
+                     (int)mode, n, feats_grad);
+  SSC_LAUNCH_CHECK("p2vx_bwd");
   return SSC_OK;
 }
 }

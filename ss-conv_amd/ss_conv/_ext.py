@@ -99,6 +99,14 @@ _SIGNATURES = {
     "ssc_p2v_compact": (ctypes.c_int, [_vp, _vp, _vp, _i64, _i32, ctypes.POINTER(ctypes.c_float),
                                        ctypes.POINTER(ctypes.c_float), _vp, _sz, _vp, _vp, _vp,
                                        _vp, _vp, _vp]),
+    "ssc_p2v_voxelize_workspace_bytes": (_sz, [_i64, _i32, ctypes.POINTER(_i32)]),
+    "ssc_p2v_voxelize_f32": (ctypes.c_int, [_vp, _vp, _vp, _i64, _i32,
+                                            ctypes.POINTER(ctypes.c_float),
+                                            ctypes.POINTER(ctypes.c_float), ctypes.POINTER(_i32),
+                                            _i32, _i32, _vp, _sz, _vp, _vp, _vp, _vp, _vp, _vp, _vp,
+                                            _vp, _vp, _vp, _vp, _vp]),
+    "ssc_p2v_voxelize_bwd_f32": (ctypes.c_int, [_vp, _i32, _vp, _vp, _vp, _vp, _i32, _i64, _vp,
+                                                _vp]),
     "ssc_unique_workspace_bytes": (_sz, [ctypes.POINTER(_i32), _i64]),
     "ssc_unique_build": (ctypes.c_int, [_vp, _i64, ctypes.POINTER(_i32), _vp, _sz, _vp, _vp,
                                         ctypes.POINTER(_i32), _vp]),
@@ -859,6 +867,88 @@ def p2v_filter(points, feats, batch_ids, half_extent, unit):
     if needs_grad:  # keep the point features in the autograd graph
         out_f = _P2vFeatures.apply(feats, out_f, dest)
     return out_p, out_f, out_i, coords, origin_ids, alive[origin_ids].astype(np.float32)
+
+
+class _P2vVoxelFeatures(torch.autograd.Function):
+    """The voxel features of p2v_voxelize as a function of the point features: the forward
+    result is handed in (computed with everything else by the one native call); the
+    gradient of input row i is mult * grad[voxel of its row], or zero for a dropped row."""
+
+    @staticmethod
+    def forward(ctx, feats, voxel_feats, dest, inverse, counts, sel, mode):
+        ctx.save_for_backward(dest, inverse, counts)
+        ctx.sel, ctx.mode, ctx.shape = sel, mode, tuple(feats.shape)
+        return voxel_feats.clone()  # (an output must not be one of the inputs)
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        dest, inverse, counts = ctx.saved_tensors
+        n, c = ctx.shape
+        grad_out = grad_out.contiguous()
+        grad_in = torch.empty((n, c), dtype=torch.float32, device=grad_out.device)
+        _check(_lib.ssc_p2v_voxelize_bwd_f32(_ptr(grad_out), c, dest.data_ptr(),
+                                             inverse.data_ptr(), counts.data_ptr(),
+                                             _ptr(ctx.sel), ctx.mode, n, grad_in.data_ptr(),
+                                             _stream(grad_out)))
+        return grad_in, None, None, None, None, None, None
+
+
+def p2v_voxelize(points, feats, batch_ids, half_extent, unit, limit, mode, n_ids):
+    """Point2Voxel.forward (ss_conv/sp_ops/voxelize.py:29-99) in one native call with one
+    wait of the host, for float32 points / features and int64 batch ids that are
+    non-decreasing and lie in [0, n_ids).  Returns None when the inputs do not qualify (the
+    caller then takes another path; `n_ids` too small counts as not qualifying); otherwise
+    (valid_points [m,3], voxel_feats [v,C], voxel_indices [v,4], valid_ids [m], origin_ids,
+    alive) with origin_ids / alive as host arrays over the batch ids present."""
+    import numpy as np
+    if not (points.is_cuda and feats.is_cuda and batch_ids.is_cuda):
+        return None
+    if points.dtype != torch.float32 or feats.dtype != torch.float32 or \
+            batch_ids.dtype != torch.int64 or points.dim() != 2 or points.size(1) != 3:
+        return None
+    n = points.size(0)
+    if n == 0 or feats.dim() != 2 or feats.size(0) != n or batch_ids.numel() != n:
+        return None
+    n_ids = int(n_ids)
+    lim = (_i32 * 3)(*[int(v) for v in limit])
+    nbytes = _lib.ssc_p2v_voxelize_workspace_bytes(n, n_ids, lim) if 1 <= n_ids <= P2V_MAX_IDS \
+        else 0
+    if nbytes == 0:
+        return None
+    points, batch_ids = points.contiguous(), batch_ids.contiguous()
+    src_feats = feats.detach().contiguous()
+    dev = points.device
+    c = feats.size(1)
+    ws = _workspace(nbytes, dev)
+    h = (ctypes.c_float * 3)(*[float(v) for v in half_extent])
+    u = (ctypes.c_float * 3)(*[float(v) for v in unit])
+    out_p = torch.empty((n, 3), dtype=torch.float32, device=dev)
+    out_i = torch.empty((n,), dtype=torch.int64, device=dev)
+    vox_idx = torch.empty((n, 4), dtype=torch.int32, device=dev)
+    vox_f = torch.empty((n, c), dtype=torch.float32, device=dev)
+    # inverse, counts, dest and (modes 1 / 2) sel side by side
+    aux = torch.empty((4, n), dtype=torch.int32, device=dev)
+    sel = aux[3] if mode in (1, 2) else None
+    hist_all = np.empty(n_ids, dtype=np.int32)
+    hist_valid = np.empty(n_ids, dtype=np.int32)
+    totals = (_i32 * 4)()
+    _check(_lib.ssc_p2v_voxelize_f32(
+        _ptr(points), _ptr(src_feats), _ptr(batch_ids), n, c, h, u, lim, n_ids, int(mode),
+        ws.data_ptr(), ws.numel(), out_p.data_ptr(), out_i.data_ptr(), vox_idx.data_ptr(),
+        vox_f.data_ptr(), aux[0].data_ptr(), aux[1].data_ptr(), aux[2].data_ptr(), _ptr(sel),
+        hist_all.ctypes.data, hist_valid.ctypes.data, totals, _stream(points)))
+    m, v, flags = int(totals[0]), int(totals[1]), int(totals[2])
+    if flags or m == 0:
+        return None
+    present = hist_all > 0
+    origin_ids = np.nonzero(present)[0]
+    alive = (hist_valid > 0)[origin_ids]
+    if not alive.any():  # no point survived at all: the reference's special case
+        return None
+    vox_f = vox_f[:v]
+    if torch.is_grad_enabled() and feats.requires_grad:
+        vox_f = _P2vVoxelFeatures.apply(feats, vox_f, aux[2], aux[0], aux[1], sel, int(mode))
+    return out_p[:m], vox_f, vox_idx[:v], out_i[:m], origin_ids, alive.astype(np.float32)
 
 
 def unique_rows(coords, dims, return_counts=True):

@@ -30,6 +30,10 @@ class Point2Voxel(nn.Module):
                                               dtype=torch.float32)
         self.voxel_num_limit = np.array(voxel_num_limit)
         self.voxelization_mode = voxelization_mode
+        # 1 + the largest batch id of the last call: the next call sizes its tables for it
+        # before it has looked at its own ids (and falls back when they do not fit)
+        self._n_ids_hint = None
+        self.last_path = None  # which of the three ways the last forward took (diagnostics)
 
     def forward(self, point_cloud, feature, batch_ids):
         assert len(point_cloud.size()) == 2
@@ -45,11 +49,28 @@ class Point2Voxel(nn.Module):
         # reference's sequence of torch operations below.
         # (the native filter keeps the features in the autograd graph when they carry a
         # gradient, as the reference's boolean-mask indexing does)
+        # One native call with one wait of the host when this module has seen the range of
+        # batch ids before (the call checks that they still fit).
+        if self._n_ids_hint is not None and point_cloud.is_cuda:
+            one = _ext.p2v_voxelize(point_cloud, feature, batch_ids, half, unit,
+                                    self.voxel_num_limit, self.voxelization_mode,
+                                    self._n_ids_hint)
+            if one is not None:
+                valid_point_cloud, voxel_feats, voxel_index, valid_ids, origin_ids, alive = one
+                B1 = len(origin_ids)
+                valid_instance_flag = torch.ones(B1, dtype=torch.float32, device=device) \
+                    if bool(alive.all()) else torch.from_numpy(alive).to(device)
+                sparse_feat = SparseTensor(voxel_feats, voxel_index,
+                                           self.voxel_num_limit.astype(np.int64), B1)
+                self.last_path = "one call"
+                return valid_point_cloud, sparse_feat, valid_ids, valid_instance_flag
         fast = _ext.p2v_filter(point_cloud, feature, batch_ids, half, unit) \
             if point_cloud.is_cuda else None
         if fast is not None:
             valid_point_cloud, valid_feature, valid_ids, voxel_index, origin_ids, alive = fast
             B1 = len(origin_ids)
+            self._n_ids_hint = int(origin_ids[-1]) + 1
+            self.last_path = "native filter"
             # all clouds kept points (the usual case): a fill on the device instead of a
             # synchronous upload
             valid_instance_flag = torch.ones(B1, dtype=torch.float32, device=device) \
@@ -57,6 +78,7 @@ class Point2Voxel(nn.Module):
             return self._voxelize(valid_point_cloud, valid_feature, valid_ids, voxel_index,
                                   int(origin_ids[-1]), valid_instance_flag, B1)
 
+        self.last_path = "torch filter"
         half_t = torch.from_numpy(half).reshape(1, 3).to(device)
         unique_origin_ids = torch.unique(batch_ids)
         B1 = unique_origin_ids.size(0)

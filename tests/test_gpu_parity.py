@@ -1464,3 +1464,142 @@ def test_fused_rulebook_conv_equals_the_two_calls(subm, stride, device):
     fn = indice_subm_conv if subm else indice_conv
     y3 = fn(x1.detach(), layer.weight.detach(), g_pairs.clone(), g_num, g_idx.shape[0])
     assert torch.equal(y3 + layer.bias.detach(), y1.features.detach())
+
+
+def _p2v_same(a, b):
+    """Two Point2Voxel results, field by field, bit for bit."""
+    (vp1, st1, vi1, f1), (vp2, st2, vi2, f2) = a, b
+    assert torch.equal(vp1, vp2) and torch.equal(vi1, vi2) and torch.equal(f1, f2)
+    assert torch.equal(st1.indices, st2.indices) and st1.batch_size == st2.batch_size
+    assert torch.equal(st1.features, st2.features)
+    assert list(st1.spatial_shape) == list(st2.spatial_shape)
+
+
+@pytest.mark.parametrize("mode", [1, 2, 3, 4])
+def test_point2voxel_one_call_path(mode, oracle, device):
+    """A Point2Voxel module that has seen the range of batch ids once runs the whole forward
+    as one native call with one wait of the host.  Its result equals the oracle's and the
+    first call's, bit for bit: filtered points, ids, flags, voxel rows, voxel features."""
+    from ss_conv.sp_ops.voxelize import Point2Voxel
+    pts, feats, ids = synth.make_clouds(3, 700, seed=3, channels=6)
+    pts = pts * 1.2  # some points fall outside and are filtered
+    pts[ids == 1] = 50.0  # a cloud left without points: one zero point
+    grid = 16
+    ref = oracle.point2voxel(pts, feats, ids, [grid] * 3, [2.0 / grid] * 3, mode)
+    p2v = Point2Voxel([grid] * 3, [2.0 / grid] * 3, mode)
+    args = [torch.from_numpy(a).to(device) for a in (pts, feats, ids)]
+    first = p2v(*args)
+    assert p2v.last_path == "native filter"
+    second = p2v(*args)
+    assert p2v.last_path == "one call"
+    _p2v_same(first, second)
+    vp, st, vi, flag = second
+    assert np.array_equal(vp.cpu().numpy(), ref["valid_points"])
+    assert np.array_equal(vi.cpu().numpy(), ref["valid_ids"])
+    assert np.array_equal(flag.cpu().numpy(), ref["flag"])
+    assert np.array_equal(st.indices.cpu().numpy(), ref["indices"])
+    assert st.batch_size == ref["batch_size"]
+    assert np.array_equal(st.features.cpu().numpy(), ref["features"])
+    # ids beyond what the module has seen: the call notices and another path is taken
+    more = ids + 5
+    third = p2v(args[0], args[1], torch.from_numpy(more).to(device))
+    assert p2v.last_path == "native filter"
+    ref3 = oracle.point2voxel(pts, feats, more, [grid] * 3, [2.0 / grid] * 3, mode)
+    assert np.array_equal(third[1].indices.cpu().numpy(), ref3["indices"])
+    assert np.array_equal(third[1].features.cpu().numpy(), ref3["features"])
+    # unsorted ids: not for the native paths at all
+    perm = np.random.default_rng(0).permutation(len(ids))
+    fourth = p2v(*[torch.from_numpy(a[perm]).to(device) for a in (pts, feats, ids)])
+    assert p2v.last_path == "torch filter"
+    ref4 = oracle.point2voxel(pts[perm], feats[perm], ids[perm], [grid] * 3, [2.0 / grid] * 3, mode)
+    assert np.array_equal(fourth[1].features.cpu().numpy(), ref4["features"])
+
+
+@pytest.mark.parametrize("mode", [1, 2, 3, 4])
+def test_point2voxel_one_call_crowded_voxels_and_wide_rows(mode, oracle, device):
+    """Voxels with hundreds of points, spread over thousands of row numbers (the ordered
+    reduction walks several windows of its row bit map), and feature rows wider than one
+    pass of the wave over the channels."""
+    from ss_conv.sp_ops.voxelize import Point2Voxel
+    rng = np.random.default_rng(12)
+    n_per, B, C, grid = 6000, 2, 300, 4
+    pts = rng.uniform(-0.999, 0.999, size=(B * n_per, 3)).astype(np.float32)
+    feats = rng.normal(size=(B * n_per, C)).astype(np.float32)
+    ids = np.repeat(np.arange(B, dtype=np.int64), n_per)
+    ref = oracle.point2voxel(pts, feats, ids, [grid] * 3, [2.0 / grid] * 3, mode)
+    p2v = Point2Voxel([grid] * 3, [2.0 / grid] * 3, mode)
+    args = [torch.from_numpy(a).to(device) for a in (pts, feats, ids)]
+    first = p2v(*args)
+    second = p2v(*args)
+    assert p2v.last_path == "one call"
+    _p2v_same(first, second)
+    assert second[1].indices.shape[0] == B * grid ** 3
+    assert np.array_equal(second[1].features.cpu().numpy(), ref["features"])
+
+
+def test_point2voxel_one_call_random_configurations(oracle, device):
+    """The one-call path on seeded configurations: 1-5 clouds (some empty, some entirely
+    outside, ids with gaps), non-cubic limits, anisotropic extents, all modes, points on
+    cell faces, duplicated points."""
+    from ss_conv.sp_ops.voxelize import Point2Voxel
+    rng = np.random.default_rng(5)
+    taken = 0
+    for case in range(40):
+        B = int(rng.integers(1, 6))
+        limit = [int(rng.integers(2, 20)) for _ in range(3)]
+        unit = [float(rng.choice([0.05, 0.1, 0.125, 0.3, 0.07])) for _ in range(3)]
+        mode = int(rng.integers(1, 5))
+        C = int(rng.choice([1, 3, 6, 16, 33]))
+        counts = [int(rng.integers(0, 300)) for _ in range(B)]
+        if sum(counts) == 0:
+            counts[0] = 5
+        ids = np.concatenate([np.full(c, b, dtype=np.int64) for b, c in enumerate(counts)])
+        if rng.integers(0, 3) == 0:
+            ids = ids * 2 + 1
+        n = len(ids)
+        half = 0.5 * np.array(limit) * np.array(unit)
+        pts = (rng.uniform(-1.15, 1.15, size=(n, 3)) * half).astype(np.float32)
+        on_face = rng.integers(0, n, size=max(1, n // 10))
+        pts[on_face, rng.integers(0, 3)] = (np.round(pts[on_face, 0] / unit[0]) * unit[0]).astype(np.float32)
+        dup = rng.integers(0, n, size=max(1, n // 8))
+        pts[dup] = pts[rng.integers(0, n, size=len(dup))]
+        if B > 1 and rng.integers(0, 3) == 0:
+            pts[ids == ids[0]] = 1e3  # first cloud entirely outside
+        feats = rng.normal(size=(n, C)).astype(np.float32)
+        print("case", case, "B", B, "limit", limit, "mode", mode, "C", C, "n", n, flush=True)
+        ref = oracle.point2voxel(pts, feats, ids, limit, unit, mode)
+        p2v = Point2Voxel(limit, unit, mode)
+        args = [torch.from_numpy(a).to(device) for a in (pts, feats, ids)]
+        p2v(*args)
+        vp, st, vi, flag = p2v(*args)
+        if p2v.last_path == "one call":
+            taken += 1
+        assert np.array_equal(vp.cpu().numpy(), ref["valid_points"]), case
+        assert np.array_equal(vi.cpu().numpy(), ref["valid_ids"]), case
+        assert np.array_equal(flag.cpu().numpy(), ref["flag"]), case
+        assert np.array_equal(st.indices.cpu().numpy(), ref["indices"]), case
+        assert np.array_equal(st.features.cpu().numpy(), ref["features"]), case
+    assert taken >= 30
+
+
+@pytest.mark.parametrize("mode", [2, 3, 4])
+def test_point2voxel_one_call_gradients(mode, oracle, device):
+    """The gradient of the point features through the one-call path equals the one through
+    the per-voxel point lists (voxelize_bp) of the other path."""
+    from ss_conv.sp_ops.voxelize import Point2Voxel
+    pts, feats, ids = synth.make_clouds(3, 400, seed=8, channels=5)
+    pts = pts * 1.2
+    grid = 6
+    p2v = Point2Voxel([grid] * 3, [2.0 / grid] * 3, mode)
+    tp, ti = torch.from_numpy(pts).to(device), torch.from_numpy(ids).to(device)
+    grads = []
+    gv = None
+    for _ in range(2):
+        x = torch.from_numpy(feats).to(device).requires_grad_(True)
+        vp, st, vi, _ = p2v(tp, x, ti)
+        if gv is None:
+            gv = torch.randn_like(st.features)
+        st.features.backward(gv)
+        grads.append(x.grad.clone())
+    assert p2v.last_path == "one call"
+    assert torch.equal(grads[0], grads[1])
