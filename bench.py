@@ -24,10 +24,11 @@ for _p in (os.path.join(ROOT, "ss-conv_amd"), os.path.join(ROOT, "oracle")):
 
 FP32_MFMA_PEAK_TFLOPS = 157.3  # MI355X dense fp32 matrix peak
 
-# HBM bytes per launch of the convolution kernel, from rocprofv3 --pmc
-# FETCH_SIZE / WRITE_SIZE runs scaled by a copy kernel of known size
-# (summaries under profiles/); None until measured for a workload.
-MEASURED_TRAFFIC_BYTES = {"cfg2": int((18669.6 * 2.0 + 300076.5) * 1024)}
+# HBM bytes per launch of the convolution kernel for every workload this script offers, from
+# rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs scaled by a copy kernel of known size (the
+# summaries profiles/conv_fwd_<workload>_hbm_traffic.md give commands and counter values).
+MEASURED_TRAFFIC_BYTES = {"cfg1": 3029773, "cfg2": 345628507, "cfg3": 218923200,
+                          "cfg5": 96942593172}
 
 
 def parse_args():
@@ -46,6 +47,9 @@ def parse_args():
                     help="also time the other operators of the path (pools, global pools, "
                          "Point2Voxel, Voxel2Point) against their algorithmic HBM bytes; "
                          "table on stderr")
+    ap.add_argument("--p2v", action="store_true",
+                    help="also time Point2Voxel and Voxel2Point alone on the clouds of cfg2 and "
+                         "cfg5; table on stderr")
     ap.add_argument("--backbone", action="store_true",
                     help="also run the backbone of the fourth configuration (Point2Voxel -> four "
                          "[Convolution -> BatchNorm -> gated Activation] stages -> GlobalAvgPool + "
@@ -126,10 +130,19 @@ def ops_table(torch, _ext, synth, dev, seed):
     w = torch.randn(3, 3, 3, cin, cout, device=dev) / (K * cin) ** 0.5
     go = torch.randn(o_idx.shape[0], cout, device=dev)
     P = int(num.sum().item())
-    ms, _ = timed(lambda: _ext.indice_conv_backward_fp32(f, w, go, pairs, num, 0, 0), n=10)
+    _ext.indice_conv_backward_fp32(f, w, go, pairs, num, 0, 0)
+    torch.cuda.synchronize()
+    _ext.profile_conv(True)  # the input gradient is the forward kernel on the output gradient
+    ms, _ = timed(lambda: _ext.indice_conv_backward_fp32(f, w, go, pairs, num, 0, 0), n=10, warm=0)
+    in_ms = _ext.profile_conv_read()
+    _ext.profile_conv(False)
     rows.append("%-44s %8.3f ms %9.2f GFLOP %7.1f TFLOP/s %5.1f%% of fp32 MFMA peak"
                 % ("conv backward, cfg2 (input + filter gradient)", ms, 4.0 * P * cin * cout / 1e9,
                    4.0 * P * cin * cout / ms / 1e9, 4.0 * P * cin * cout / ms / 1e9 / 1.573))
+    t_in = sum(in_ms) / max(len(in_ms), 1)
+    rows.append("%-44s %8.3f ms %9.2f GFLOP %7.1f TFLOP/s %5.1f%% of fp32 MFMA peak"
+                % ("  of which the input-gradient kernel (128->64)", t_in, 2.0 * P * cin * cout / 1e9,
+                   2.0 * P * cin * cout / t_in / 1e9, 2.0 * P * cin * cout / t_in / 1e9 / 1.573))
     # the same layer on half-precision tensors (fp32 arithmetic, half the row bytes)
     fh, wh, goh = f.half(), w.half(), go.half()
     n_out_rows = o_idx.shape[0]
@@ -177,24 +190,9 @@ def ops_table(torch, _ext, synth, dev, seed):
     ms, _ = timed(lambda: gm(f, offs))
     report("GlobalMaxPool", ms, nbytes + 4 * C * B)
 
-    # Point2Voxel on the cfg2 clouds (65536 points, 64 channels) and Voxel2Point back
-    cfg = synth.CONFIGS["cfg2"]
-    pts, feats, ids = synth.config_clouds("cfg2", seed)
-    C = 64
-    tp = torch.from_numpy(pts).to(dev)
-    tf = torch.randn(tp.shape[0], C, device=dev)
-    ti = torch.from_numpy(ids).to(dev)
-    p2v = Point2Voxel([cfg["grid"]] * 3, [2.0 / cfg["grid"]] * 3)
-    ms, r = timed(lambda: p2v(tp, tf, ti), n=20)
-    N, M = tp.shape[0], r[1].features.shape[0]
-    report("Point2Voxel module (%d pts -> %d voxels, C=%d)" % (N, M, C), ms,
-           N * (12 + 8 + 4 * C) + M * (16 + 4 * C) + 4 * N, "2 host reads of data-dependent sizes")
-    v2p = Voxel2Point(unit_voxel_extent=[2.0 / cfg["grid"]] * 3)
-    vp, vs, vi = r[0], r[1], r[2]
-    ms, _ = timed(lambda: v2p(vs, vp, vi), n=20, warm=3)
-    n = vp.shape[0]
-    report("Voxel2Point module (%d pts, %d voxels, C=%d)" % (n, M, C), ms,
-           4 * C * 4 * n + 16 * (n + M) + 24 * n, "3-NN search: n*M/B distance tests")
+    # Point2Voxel on the cfg2 and cfg5 clouds (65536 / 131072 points, 64 channels) and
+    # Voxel2Point back
+    point_voxel_rows(torch, synth, dev, seed, timed, report)
 
     # BatchNorm + gated Activation after the cfg2 layer: irrep(8,8,8,8) fields = 128 columns
     # plus 24 gate scalars, on the layer's 600k output rows
@@ -259,6 +257,33 @@ def ops_table(torch, _ext, synth, dev, seed):
                 % ("backbone forward, 4th configuration (eval)", ms, 32, r[2].features.shape[0],
                    r[2].features.shape[1]))
     print("\n".join(rows), file=sys.stderr)
+
+
+def point_voxel_rows(torch, synth, dev, seed, timed, report):
+    """Point2Voxel (as a module that is called again and again, which is how a training loop
+    uses it) and Voxel2Point on the clouds of the second and fifth configuration."""
+    from ss_conv.sp_ops.voxelize import Point2Voxel, Voxel2Point
+    for name in ("cfg2", "cfg5"):
+        cfg = synth.CONFIGS[name]
+        pts, feats, ids = synth.config_clouds(name, seed)
+        C = 64
+        tp = torch.from_numpy(pts).to(dev)
+        tf = torch.randn(tp.shape[0], C, device=dev)
+        ti = torch.from_numpy(ids).to(dev)
+        p2v = Point2Voxel([cfg["grid"]] * 3, [2.0 / cfg["grid"]] * 3)
+        with torch.no_grad():
+            ms, r = timed(lambda: p2v(tp, tf, ti), n=20)
+        N, M = tp.shape[0], r[1].features.shape[0]
+        report("Point2Voxel module, %s (%d pts -> %d voxels, C=%d)" % (name, N, M, C), ms,
+               N * (12 + 8 + 4 * C) + M * (16 + 4 * C) + 4 * N,
+               "path: %s; one host wait" % p2v.last_path)
+        v2p = Voxel2Point(unit_voxel_extent=[2.0 / cfg["grid"]] * 3)
+        vp, vs, vi = r[0], r[1], r[2]
+        with torch.no_grad():
+            ms, _ = timed(lambda: v2p(vs, vp, vi), n=20, warm=3)
+        n = vp.shape[0]
+        report("Voxel2Point module, %s (%d pts, %d voxels, C=%d)" % (name, n, M, C), ms,
+               4 * C * 4 * n + 16 * (n + M) + 24 * n, "3-NN search around the query's cell")
 
 
 def build_backbone(torch, synth, dev, seed):
@@ -469,6 +494,25 @@ def main():
 
     if args.ops:
         ops_table(torch, _ext, synth, dev, args.seed)
+    if args.p2v:
+        rows = []
+
+        def timed_pv(fn, n=20, warm=3):
+            for _ in range(warm):
+                fn()
+            torch.cuda.synchronize()
+            a = time.perf_counter()
+            for _ in range(n):
+                r = fn()
+            torch.cuda.synchronize()
+            return (time.perf_counter() - a) * 1e3 / n, r
+
+        def report_pv(name, ms, nbytes, note=""):
+            gbs = nbytes / ms / 1e6
+            rows.append("%-58s %8.3f ms %9.2f MB %8.1f GB/s %5.1f%% of HBM  %s"
+                        % (name, ms, nbytes / 1e6, gbs, gbs / 80.0, note))
+        point_voxel_rows(torch, synth, dev, args.seed, timed_pv, report_pv)
+        print("\n".join(rows), file=sys.stderr)
     if args.backbone:
         backbone_table(torch, _ext, synth, dev, args.seed)
 
