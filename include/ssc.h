@@ -263,6 +263,10 @@ int ssc_conv_bwd_filter_f16(const void *features /* [n_in,c_in] half */, int64_t
  * ssc_profile_conv_read waits for the recorded calls and returns their
  * durations in milliseconds, oldest first; enabling again clears the ring. */
 int ssc_profile_conv(int32_t enable);
+/* Measurement knob, no counterpart in the reference: by_column = 0 keeps the convolution
+ * kernel from giving every XCD one column block of its own when the packed filters are
+ * larger than an L2 (the default, 1, lets it).  Results do not depend on it. */
+int ssc_conv_tuning(int32_t by_column);
 int ssc_profile_conv_read(float *ms /* host */, int32_t capacity, int32_t *count /* host */);
 
 /* ------------------------------------------------------------------------

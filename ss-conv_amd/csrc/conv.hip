@@ -723,7 +723,7 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
                     const int32_t *__restrict__ sched_in, const int32_t *__restrict__ sched_out,
                     const int32_t *__restrict__ grp_meta, unsigned sched_bytes, unsigned meta_bytes,
                     const int32_t *__restrict__ tile_grp, const int32_t *__restrict__ wg_tile,
-                    int nch, int ncb, IO *__restrict__ out, int cout, int T) {
+                    int nch, int ncb, IO *__restrict__ out, int cout, int T, int cols_per_xcd) {
   constexpr int kCN = 16 * NCW;   // output columns per workgroup
   constexpr int kEB = Io<IO>::kBytes;
   constexpr bool kHalf = kEB == 2;
@@ -748,16 +748,30 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
   const bool producer = wave >= NCW;
   // Consecutive workgroup ids land on different XCDs (8 of them, one L2 each): give
   // every XCD a contiguous run of tile ranges so neighbouring tiles, which gather
-  // the same input rows, share an L2.
-  int chunk = blockIdx.x;
+  // the same input rows, share an L2.  Which column blocks an XCD works on depends on the
+  // size of the packed filters.  Small ones (they stay in every L2): all column blocks of
+  // a run of ranges, so that the gathered rows are shared as well.  Large ones (an L2
+  // holds a fraction of them, and a workgroup walks all of its column block's fragments
+  // once per tile): one column block per XCD (cols_per_xcd: XCDs per column block), so that
+  // the 32 workgroups of an XCD ask for the same fragments at about the same time and
+  // one fetch serves them all.
+  int chunk = blockIdx.x, cblk = blockIdx.y;
   {
     const int nwg = gridDim.x;
-    if ((nwg & 7) == 0) chunk = (chunk & 7) * (nwg >> 3) + (chunk >> 3);
+    if (cols_per_xcd > 0) {
+      const int lin = blockIdx.y * nwg + blockIdx.x;  // dispatch order: XCD = lin % 8
+      const int xcd = lin & 7, slot = lin >> 3;
+      const int ncol = gridDim.y;  // divides 8
+      cblk = xcd % ncol;
+      chunk = (xcd / ncol) * ((nwg * ncol) >> 3) + slot;
+    } else if ((nwg & 7) == 0) {
+      chunk = (chunk & 7) * (nwg >> 3) + (chunk >> 3);
+    }
   }
   const int t_begin = wg_tile[chunk], t_end = wg_tile[chunk + 1];
   const int g_begin = tile_grp[t_begin], g_end = tile_grp[t_end];
   const int nstages = (g_end - g_begin) * nch;  // stages of this workgroup
-  const int col0 = blockIdx.y * kCN;
+  const int col0 = cblk * kCN;
 
   {
     float4v z = {0.f, 0.f, 0.f, 0.f};
@@ -969,7 +983,7 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
     const int l16 = lane & 15;
     // A column group beyond Cout multiplies with the last real one's fragments; its
     // accumulator columns are never written out.
-    const int cb = min((int)blockIdx.y * NCW + wave, ncb - 1);
+    const int cb = min(cblk * NCW + wave, ncb - 1);
     const __amdgpu_buffer_rsrc_t rs_w =
         __builtin_amdgcn_make_buffer_rsrc((void *)packed, 0, (int)packed_bytes, kRsrcFlags);
     const __amdgpu_buffer_rsrc_t rs_out =
@@ -1406,6 +1420,8 @@ static size_t conv_ws_bytes(int64_t n_out, int K, int c_in, int c_out, int64_t p
   return conv_ws_walk(nullptr, p, K, pair_stride, nullptr);
 }
 
+static bool g_conv_by_column = true;  // (switched by ssc_conv_tuning, for measurements)
+
 template <typename IO, int GATHER, int NCW, int NS>
 static int launch_conv(const ConvPlan &p, const ConvWs &w, const IO *features, int64_t n_in,
                        int c_in, int K, IO *out, int c_out, hipStream_t s) {
@@ -1422,10 +1438,18 @@ static int launch_conv(const ConvPlan &p, const ConvWs &w, const IO *features, i
             (unsigned long long)packed_bytes, (unsigned long long)sched_bytes);
   const unsigned feat_bytes = GATHER != 0 ? (unsigned)((uint64_t)n_in * c_in * sizeof(IO)) : 0u;
   dim3 grid((unsigned)p.n_wg, (unsigned)p.n_colblk);
+  // one column block per XCD when the packed filters are larger than an L2 can keep
+  // (4 MiB per XCD) and the grid divides that way (256 -> 256 channels, 7 MiB: 2.44 ->
+  // 2.24 ms on the 64^3 benchmark geometry; 128 -> 256 at stride 2, 3.5 MiB, is 5 % slower
+  // that way and stays with the row-major mapping)
+  const bool by_column = packed_bytes > ((uint64_t)4 << 20) && p.n_colblk > 1 &&
+                         8 % p.n_colblk == 0 && (p.n_wg * p.n_colblk) % 8 == 0 &&
+                         g_conv_by_column;
+  const int cols_per_xcd = by_column ? 8 / p.n_colblk : 0;
   hipLaunchKernelGGL((conv_fwd_kernel<IO, GATHER, NCW, NS>), grid, dim3((NCW + 4) * 64), p.lds_bytes, s, features, c_in,
                      feat_bytes, w.packed, (unsigned)packed_bytes, w.sched_in, w.sched_out,
                      w.grp_meta, (unsigned)sched_bytes, (unsigned)(p.grp_cap * 32), w.tile_grp,
-                     w.wg_tile, p.nch, p.ncb, out, c_out, p.T);
+                     w.wg_tile, p.nch, p.ncb, out, c_out, p.T, cols_per_xcd);
   SSC_LAUNCH_CHECK("conv_fwd");
   return SSC_OK;
 }
@@ -1458,6 +1482,11 @@ int ssc_profile_conv(int32_t enable) {
   g_profile_every = enable > 1 ? enable : 1;
   g_profile_count = 0;
   g_profile_calls = 0;
+  return SSC_OK;
+}
+
+int ssc_conv_tuning(int32_t by_column) {
+  g_conv_by_column = by_column != 0;
   return SSC_OK;
 }
 

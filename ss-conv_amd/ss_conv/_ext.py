@@ -78,6 +78,7 @@ _SIGNATURES = {
     "ssc_voxel_reduce_bwd_f32": (ctypes.c_int, [_vp, _vp, _vp, _i32, _i32, _i32, _i32, _i64, _vp]),
     "ssc_three_interp_bwd_f32": (ctypes.c_int, [_i32, _i32, _i32, _vp, _vp, _vp, _vp, _vp]),
     "ssc_profile_conv": (ctypes.c_int, [_i32]),
+    "ssc_conv_tuning": (ctypes.c_int, [_i32]),
     "ssc_profile_conv_read": (ctypes.c_int, [ctypes.POINTER(ctypes.c_float), _i32,
                                              ctypes.POINTER(_i32)]),
     "ssc_kernel_combine_f32": (ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32,
