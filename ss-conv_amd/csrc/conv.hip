@@ -43,8 +43,10 @@ constexpr int kMinTile = 64;
 // channels cc*4ns .. cc*4ns + 4ns - 1, and only the first ns of the 16 (q, j) slots carry
 // weights.  The quarters below ns / 4 are laid out as above.  In the quarter that is only
 // partly used (ns % 4 steps) step j must stand for four consecutive channels, one per lane
-// group, so there slot (q, lane group g, j) holds channel 16q + 4j + g of the chunk; the
-// rows staged in LDS follow the same rule (conv_fwd_kernel's producers).
+// group, so there slot (q, lane group g, j) holds channel 16q + 4j + g of the chunk (the
+// rows staged in LDS follow the same rule: conv_fwd_kernel's producers), and the quarter is
+// packed densely, ns % 4 floats per lane at float 256 (ns / 4) + lane (ns % 4) + j of the
+// fragment: a wave fetches 256 (ns % 4) bytes for it instead of a KiB.
 //
 // Half-precision filters are packed for v_mfma_f32_16x16x32_f16 instead, two steps of 32
 // channels per chunk (halves, 2 KiB per fragment):
@@ -79,12 +81,17 @@ __device__ __forceinline__ void pack_filter_element(const PackArgs &a, int64_t i
     lane = (idx >> 3) & 63;
     ci = cc * kKC + 32 * q + (lane >> 4) * 8 + j;
   } else {
-    const int j = idx & 3, q = (idx >> 8) & 3;
-    lane = (idx >> 2) & 63;
-    const int g = lane >> 4, full = a.ns >> 2, rem = a.ns & 3;
+    const int full = a.ns >> 2, rem = a.ns & 3;
+    const int f = (int)(idx & 1023);  // float inside the fragment
     int cl = -1;  // channel inside the chunk, -1 for a slot without one
-    if (q < full) cl = q * 16 + g * 4 + j;
-    else if (q == full && j < rem) cl = q * 16 + j * 4 + g;
+    lane = (f >> 2) & 63;
+    if (f < full * 256) {
+      cl = (f >> 8) * 16 + (lane >> 4) * 4 + (f & 3);
+    } else if (f - full * 256 < 64 * rem) {  // the partly used quarter, rem floats per lane
+      const int t = f - full * 256;
+      lane = t / rem;
+      cl = full * 16 + (t - lane * rem) * 4 + (lane >> 4);
+    }
     ci = cl < 0 ? cin : cc * (4 * a.ns) + cl;
   }
   int co = cb * 16 + (lane & 15);
@@ -632,6 +639,8 @@ __device__ __forceinline__ int buf_load1(__amdgpu_buffer_rsrc_t r, int voff, int
 // v_mfma_f32_16x16x4_f32.  _Float16: half rows in LDS, v_mfma_f32_16x16x32_f16; the
 // accumulators are fp32 either way and are rounded once, when a finished tile is written.
 typedef int int2v __attribute__((ext_vector_type(2)));
+typedef float float2v __attribute__((ext_vector_type(2)));
+typedef float float3v __attribute__((ext_vector_type(3)));
 typedef _Float16 half4v __attribute__((ext_vector_type(4)));
 typedef _Float16 half8v __attribute__((ext_vector_type(8)));
 template <typename IO> struct Io;
@@ -1058,6 +1067,28 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
       return b == 0 ? v.x : b == 1 ? v.y : b == 2 ? v.z : v.w;
     };
     auto fetch_w = [&](int soff, int slot, int q) {
+      if constexpr (!kHalf && kQRem != 0) {
+        if (q == kQFull) {  // the partly used quarter: kQRem floats per lane, densely packed
+          const int voff = kQFull * kWStep + lane * (4 * kQRem);
+          // The wider loads are cast to float vectors as a whole: with per-element casts
+          // of an integer vector this compiler shrinks the load to its first element.
+          if constexpr (kQRem == 1) {
+            w[slot][q].x = __builtin_bit_cast(float, buf_load1(rs_w, voff, soff));
+          } else if constexpr (kQRem == 2) {
+            const float2v t = __builtin_bit_cast(
+                float2v, __builtin_amdgcn_raw_buffer_load_b64(rs_w, voff, soff, 0));
+            w[slot][q].x = t.x;
+            w[slot][q].y = t.y;
+          } else {
+            const float3v t = __builtin_bit_cast(
+                float3v, __builtin_amdgcn_raw_buffer_load_b96(rs_w, voff, soff, 0));
+            w[slot][q].x = t.x;
+            w[slot][q].y = t.y;
+            w[slot][q].z = t.z;
+          }
+          return;
+        }
+      }
       w[slot][q] = __builtin_bit_cast(Frag, buf_load4(rs_w, w_voff + q * kWStep, soff));
     };
     auto fetch_orow = [&](const StagePos &pos, int m, int slot) {
