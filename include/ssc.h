@@ -329,6 +329,22 @@ int ssc_summary_rf(const int32_t *pairs, int64_t pair_stride, const int32_t *pai
                    int32_t kernel_volume, int32_t *rf /* [n_out] */, int64_t n_out,
                    void *workspace, size_t workspace_bytes, ssc_stream_t stream);
 
+/* Half-precision rulebook pooling -- replaces indice_maxpool_half / indice_avgpool_half
+ * (src/ss_conv_ops_api.cpp:29,34: indiceMaxPool<at::Half>, indiceAvgPool<at::Half>) and, further
+ * down, their backward passes (src/ss_conv_ops_api.cpp:30,35).  features, out (and the
+ * gradients) are IEEE half rows.  Arithmetic as at::Half's operators do it in the reference's
+ * kernels: every operation computes in float and rounds to half, so the average is
+ * out = half(out + half(in / half(rf))) over the offsets in ascending order; the maximum
+ * is exact in any type.  Workspace as for the float entries. */
+int ssc_pool_max_f16(const void *features, int32_t channels, const int32_t *pairs,
+                     int64_t pair_stride, const int32_t *pair_num, int32_t kernel_volume,
+                     void *out, int64_t n_out, void *workspace, size_t workspace_bytes,
+                     ssc_stream_t stream);
+int ssc_pool_avg_f16(const void *features, int32_t channels, const int32_t *pairs,
+                     int64_t pair_stride, const int32_t *pair_num, int32_t kernel_volume,
+                     const int32_t *summaryrf, void *out, int64_t n_out, void *workspace,
+                     size_t workspace_bytes, ssc_stream_t stream);
+
 /* Backward of rulebook pooling -- replaces indice_maxpool_backward_fp32 /
  * indice_avgpool_backward_fp32 (src/ss_conv_ops_api.cpp, src/pool/indice_maxpool.h:52-86,
  * src/pool/indice_avgpool.h:54-90).  in_grad [n_in, channels] is written completely:
@@ -345,6 +361,19 @@ int ssc_pool_avg_bwd_f32(const float *out_grad, int32_t channels, const int32_t 
                          int64_t pair_stride, const int32_t *pair_num, int32_t kernel_volume,
                          const int32_t *summaryrf, float *in_grad, int64_t n_in, void *workspace,
                          size_t workspace_bytes, ssc_stream_t stream);
+/* The same for half rows (indice_maxpool_backward_half / indice_avgpool_backward_half,
+ * src/ss_conv_ops_api.cpp:30,35): in_grad = half(in_grad + out_grad) where the input equals
+ * the pooled value, half(in_grad + half(out_grad / half(rf))) for the average. */
+int ssc_pool_max_bwd_f16(const void *features, const void *out_features, const void *out_grad,
+                         int32_t channels, const int32_t *pairs, int64_t pair_stride,
+                         const int32_t *pair_num, int32_t kernel_volume, void *in_grad,
+                         int64_t n_in, void *workspace, size_t workspace_bytes,
+                         ssc_stream_t stream);
+int ssc_pool_avg_bwd_f16(const void *out_grad, int32_t channels, const int32_t *pairs,
+                         int64_t pair_stride, const int32_t *pair_num, int32_t kernel_volume,
+                         const int32_t *summaryrf, void *in_grad, int64_t n_in, void *workspace,
+                         size_t workspace_bytes, ssc_stream_t stream);
+
 
 /* ------------------------------------------------------------------------
  * Segment ("global") pooling over row ranges offsets[s]..offsets[s+1].

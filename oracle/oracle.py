@@ -16,6 +16,9 @@ Pinning status (what each function is checked against, see tests/test_oracle_*.p
   conv_fwd                        torch.nn.functional.conv3d closed form; _ref gather/scatter
   maxpool_fwd                     F.max_pool3d(relu(dense)); _ref functor
   avgpool_fwd                     F.avg_pool3d(count_include_pad=True)
+  *pool_*_half                    maximum: the float routine on the widened rows (exact);
+                                  average: hand-rounded known answers (binary16 codec of
+                                  struct), exact cases equal to the float routine
   segment_avg / segment_max       numpy reductions
   point2voxel                     np.unique(axis=0) semantics, per-voxel means, invariants
   three_nn / three_interp         brute force with argsort on tiny inputs
@@ -401,6 +404,70 @@ def avgpool_fwd(features, pairs, num, n_out, rf=None):
             L.orc_avgpool_offset(_f(out), _f(features), _i(_i32(pairs[k, 0, :n])),
                                  _i(_i32(pairs[k, 1, :n])), n, c, _i(rf))
     return out
+
+
+def _f16(a):
+    return np.ascontiguousarray(a, dtype=np.float16)
+
+
+def maxpool_fwd_half(features, pairs, num, n_out):
+    """indiceMaxPool<at::Half> (src/pool/indice_maxpool.h:15-50, kernel statement
+    src/pool/indice_maxpool_cuda_functor.cu:39-43: if (in > out) out = in, output starts at 0).
+    Comparisons round nothing, so the order of the offsets does not matter."""
+    features = _f16(features)
+    out = np.zeros((n_out, features.shape[1]), dtype=np.float16)
+    for k in range(pairs.shape[0]):
+        n = int(num[k])
+        if n > 0:
+            ri, ro = pairs[k, 0, :n], pairs[k, 1, :n]
+            out[ro] = np.maximum(out[ro], features[ri])
+    return out
+
+
+def avgpool_fwd_half(features, pairs, num, n_out, rf=None):
+    """indiceAvgPool<at::Half> (src/pool/indice_avgpool.h:17-52), statement
+    src/pool/indice_avgpool_cuda_functor.cu:46: out = out + in / (T)rf with T = at::Half,
+    whose operators compute in float and round the result to half; offsets ascending (one
+    launch per offset).  numpy's float16 operators round the same way."""
+    features = _f16(features)
+    if rf is None:
+        rf = np.full(n_out, pairs.shape[0], dtype=np.int32)
+    rf16 = np.asarray(rf).astype(np.float32).astype(np.float16)
+    out = np.zeros((n_out, features.shape[1]), dtype=np.float16)
+    for k in range(pairs.shape[0]):
+        n = int(num[k])
+        if n > 0:
+            ri, ro = pairs[k, 0, :n], pairs[k, 1, :n]  # output rows are unique inside an offset
+            out[ro] = out[ro] + features[ri] / rf16[ro][:, None]
+    return out
+
+
+def maxpool_bwd_half(features, out_features, out_grad, pairs, num):
+    """src/pool/indice_maxpool_cuda_functor.cu:426-455 with T = at::Half:
+    if (in == out) din = half(din + dout), offsets ascending."""
+    features, out_features, out_grad = _f16(features), _f16(out_features), _f16(out_grad)
+    din = np.zeros_like(features)
+    for k in range(pairs.shape[0]):
+        n = int(num[k])
+        if n > 0:
+            ri, ro = pairs[k, 0, :n], pairs[k, 1, :n]  # input rows are unique inside an offset
+            hit = features[ri] == out_features[ro]
+            din[ri] = np.where(hit, din[ri] + out_grad[ro], din[ri])
+    return din
+
+
+def avgpool_bwd_half(out_grad, pairs, num, n_in, rf):
+    """src/pool/indice_avgpool_cuda_functor.cu:204 with T = at::Half:
+    din = half(din + half(dout / half(rf))), offsets ascending."""
+    out_grad = _f16(out_grad)
+    rf16 = np.asarray(rf).astype(np.float32).astype(np.float16)
+    din = np.zeros((n_in, out_grad.shape[1]), dtype=np.float16)
+    for k in range(pairs.shape[0]):
+        n = int(num[k])
+        if n > 0:
+            ri, ro = pairs[k, 0, :n], pairs[k, 1, :n]
+            din[ri] = din[ri] + out_grad[ro] / rf16[ro][:, None]
+    return din
 
 
 def segment_avg(feats, offsets):

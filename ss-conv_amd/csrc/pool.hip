@@ -18,6 +18,7 @@
 namespace ssc {
 
 typedef float float4v __attribute__((ext_vector_type(4)));
+typedef _Float16 half4v __attribute__((ext_vector_type(4)));
 
 // table[key row * K + k] = the other row of the pair; key_plane 1 keys by output rows
 // (forward), 0 by input rows (backward).
@@ -42,12 +43,43 @@ __global__ void __launch_bounds__(256)
   atomicAdd(&rf[pairs[((int64_t)k * 2 + 1) * pair_stride + j]], 1);  // integer: exact
 }
 
-// MODE 0: max with zero start (out = max(0, inputs));  MODE 1: sum of in / (float)rf.
-// VEC = 4 when C % 4 == 0 (16-byte accesses), else 1.
-template <int MODE, int VEC>
+// Element access for float and half rows.  Half arithmetic follows the reference's at::Half
+// operators (every statement of its kernels computes in float and rounds the result to
+// half): values travel as floats here and rnd<IO> rounds after every operation; for float it
+// is the identity.
+template <typename IO>
+__device__ __forceinline__ float rnd(float v) {
+  return (float)(IO)v;
+}
+template <typename IO, int VEC>
+__device__ __forceinline__ void load_row(const IO *p, float (&x)[VEC]) {
+  if constexpr (VEC == 4 && sizeof(IO) == 4) {
+    const float4v q = *reinterpret_cast<const float4v *>(p);
+    x[0] = q.x; x[1] = q.y; x[2] = q.z; x[3] = q.w;
+  } else if constexpr (VEC == 4) {
+    const half4v q = *reinterpret_cast<const half4v *>(p);
+    x[0] = (float)q.x; x[1] = (float)q.y; x[2] = (float)q.z; x[3] = (float)q.w;
+  } else {
+    x[0] = (float)p[0];
+  }
+}
+template <typename IO, int VEC>
+__device__ __forceinline__ void store_row(IO *p, const float (&x)[VEC]) {
+  if constexpr (VEC == 4 && sizeof(IO) == 4) {
+    *reinterpret_cast<float4v *>(p) = float4v{x[0], x[1], x[2], x[3]};
+  } else if constexpr (VEC == 4) {
+    *reinterpret_cast<half4v *>(p) = half4v{(_Float16)x[0], (_Float16)x[1], (_Float16)x[2], (_Float16)x[3]};
+  } else {
+    p[0] = (IO)x[0];
+  }
+}
+
+// MODE 0: max with zero start (out = max(0, inputs));  MODE 1: sum of in / (IO)rf.
+// VEC = 4 when C % 4 == 0 (16-byte accesses for float, 8-byte for half), else 1.
+template <typename IO, int MODE, int VEC>
 __global__ void __launch_bounds__(256)
-    pool_kernel(const float *__restrict__ in, int C, const int32_t *__restrict__ table, int K,
-                const int32_t *__restrict__ rf, float *__restrict__ out, int64_t n_out) {
+    pool_kernel(const IO *__restrict__ in, int C, const int32_t *__restrict__ table, int K,
+                const int32_t *__restrict__ rf, IO *__restrict__ out, int64_t n_out) {
   const int cv = C / VEC;
   int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (idx >= n_out * cv) return;
@@ -57,33 +89,23 @@ __global__ void __launch_bounds__(256)
 #pragma unroll
   for (int v = 0; v < VEC; ++v) acc[v] = 0.f;
   float div = 1.f;
-  if (MODE == 1) div = (float)rf[o];
+  if (MODE == 1) div = rnd<IO>((float)rf[o]);
   const int32_t *t = table + o * K;
   for (int k = 0; k < K; ++k) {
     int64_t i = t[k];
     if (i < 0) continue;
     float x[VEC];
-    if (VEC == 4) {
-      float4v q = *reinterpret_cast<const float4v *>(in + i * C + c);
-      x[0] = q.x; x[1 % VEC] = q.y; x[2 % VEC] = q.z; x[3 % VEC] = q.w;
-    } else {
-      x[0] = in[i * C + c];
-    }
+    load_row<IO, VEC>(in + i * C + c, x);
 #pragma unroll
     for (int v = 0; v < VEC; ++v) {
       if (MODE == 0) {
         if (acc[v] < x[v]) acc[v] = x[v];
       } else {
-        acc[v] = acc[v] + x[v] / div;
+        acc[v] = rnd<IO>(acc[v] + rnd<IO>(x[v] / div));
       }
     }
   }
-  if (VEC == 4) {
-    float4v q = {acc[0], acc[1 % VEC], acc[2 % VEC], acc[3 % VEC]};
-    *reinterpret_cast<float4v *>(out + o * C + c) = q;
-  } else {
-    out[o * C + c] = acc[0];
-  }
+  store_row<IO, VEC>(out + o * C + c, acc);
 }
 
 // Segment pooling: grid (segment, channel block of 64); 16 row lanes x 64
@@ -153,13 +175,13 @@ __global__ void __launch_bounds__(kSegRows * 64)
 // (src/pool/indice_maxpool_cuda_functor.cu:426-455: din[i] += dout[o] where in[i] == out[o];
 // src/pool/indice_avgpool_cuda_functor.cu: din[i] += dout[o] / (float)rf[o]).
 // table is [n_in, K] of output rows.  MODE 0 max, 1 average.
-template <int MODE, int VEC>
+template <typename IO, int MODE, int VEC>
 __global__ void __launch_bounds__(256)
-    pool_bwd_kernel(const float *__restrict__ in, const float *__restrict__ out,
-                    const float *__restrict__ dout, int C, const int32_t *__restrict__ table,
-                    int K, const int32_t *__restrict__ rf, float *__restrict__ din, int64_t n_in) {
-  // VEC = 4 when C % 4 == 0 (16-byte accesses), else 1; per column the arithmetic and its
-  // order are those of the one-column form
+    pool_bwd_kernel(const IO *__restrict__ in, const IO *__restrict__ out,
+                    const IO *__restrict__ dout, int C, const int32_t *__restrict__ table,
+                    int K, const int32_t *__restrict__ rf, IO *__restrict__ din, int64_t n_in) {
+  // VEC = 4 when C % 4 == 0, else 1; per column the arithmetic and its order are those of
+  // the one-column form
   const int cv = C / VEC;
   int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (idx >= n_in * cv) return;
@@ -172,45 +194,24 @@ __global__ void __launch_bounds__(256)
     acc[v] = 0.f;
     x[v] = 0.f;
   }
-  if (MODE == 0) {
-    if (VEC == 4) {
-      float4v q = *reinterpret_cast<const float4v *>(in + i * C + c);
-      x[0] = q.x; x[1 % VEC] = q.y; x[2 % VEC] = q.z; x[3 % VEC] = q.w;
-    } else {
-      x[0] = in[i * C + c];
-    }
-  }
+  if (MODE == 0) load_row<IO, VEC>(in + i * C + c, x);
   for (int k = 0; k < K; ++k) {
     int64_t o = t[k];
     if (o < 0) continue;
     float g[VEC], y[VEC];
-    if (VEC == 4) {
-      float4v q = *reinterpret_cast<const float4v *>(dout + o * C + c);
-      g[0] = q.x; g[1 % VEC] = q.y; g[2 % VEC] = q.z; g[3 % VEC] = q.w;
-      if (MODE == 0) {
-        float4v p = *reinterpret_cast<const float4v *>(out + o * C + c);
-        y[0] = p.x; y[1 % VEC] = p.y; y[2 % VEC] = p.z; y[3 % VEC] = p.w;
-      }
-    } else {
-      g[0] = dout[o * C + c];
-      if (MODE == 0) y[0] = out[o * C + c];
-    }
-    const float div = MODE == 1 ? (float)rf[o] : 1.f;
+    load_row<IO, VEC>(dout + o * C + c, g);
+    if (MODE == 0) load_row<IO, VEC>(out + o * C + c, y);
+    const float div = MODE == 1 ? rnd<IO>((float)rf[o]) : 1.f;
 #pragma unroll
     for (int v = 0; v < VEC; ++v) {
       if (MODE == 0) {
-        if (x[v] == y[v]) acc[v] = acc[v] + g[v];
+        if (x[v] == y[v]) acc[v] = rnd<IO>(acc[v] + g[v]);
       } else {
-        acc[v] = acc[v] + g[v] / div;
+        acc[v] = rnd<IO>(acc[v] + rnd<IO>(g[v] / div));
       }
     }
   }
-  if (VEC == 4) {
-    float4v q = {acc[0], acc[1 % VEC], acc[2 % VEC], acc[3 % VEC]};
-    *reinterpret_cast<float4v *>(din + i * C + c) = q;
-  } else {
-    din[i * C + c] = acc[0];
-  }
+  store_row<IO, VEC>(din + i * C + c, acc);
 }
 
 // Backward of the segment pools (src/pool/global_avgpool_cuda_kernel.cu:44-62,
@@ -255,8 +256,8 @@ __global__ void __launch_bounds__(256)
   if (a >= 0) din[(int64_t)a * C + (idx % C)] = dout[idx];
 }
 
-static int pool_common(const float *features, int channels, const int32_t *pairs,
-                       int64_t pair_stride, const int32_t *pair_num, int K, float *out,
+static int pool_common(const void *features, int channels, const int32_t *pairs,
+                       int64_t pair_stride, const int32_t *pair_num, int K, void *out,
                        int64_t n_out, void *ws, size_t ws_bytes, hipStream_t s,
                        int32_t **table_out) {
   SSC_CHECK(K >= 1 && K <= SSC_MAX_KERNEL_VOLUME, SSC_ERUNTIME, "kernel volume %d out of range", K);
@@ -334,51 +335,70 @@ size_t ssc_pool_workspace_bytes(int64_t n_out, int32_t kernel_volume) {
   return align_up((size_t)(n_out > 0 ? n_out : 1) * kernel_volume * 4);
 }
 
+}  // extern "C"
+
+// mode 0 max, 1 average
+template <typename IO>
+static int pool_fwd(int mode, const IO *features, int channels, const int32_t *pairs,
+                    int64_t pair_stride, const int32_t *pair_num, int K, const int32_t *summaryrf,
+                    IO *out, int64_t n_out, void *ws, size_t ws_bytes, hipStream_t s) {
+  SSC_CHECK(mode == 0 || n_out == 0 || summaryrf != nullptr, SSC_EINVAL, "summaryrf is NULL");
+  int32_t *table = nullptr;
+  int rc = pool_common(features, channels, pairs, pair_stride, pair_num, K, out, n_out, ws,
+                       ws_bytes, s, &table);
+  if (rc != SSC_OK || n_out == 0) return rc;
+  const int vec = (channels & 3) == 0 ? 4 : 1;
+  const int64_t n = n_out * (channels / vec);
+  const dim3 grid((unsigned)ceil_div(n, 256));
+#define SSC_POOL_FWD(M, V)                                                                     \
+  hipLaunchKernelGGL((pool_kernel<IO, M, V>), grid, dim3(256), 0, s, features, channels, table, \
+                     K, summaryrf, out, n_out)
+  if (mode == 0) {
+    if (vec == 4) SSC_POOL_FWD(0, 4); else SSC_POOL_FWD(0, 1);
+  } else {
+    if (vec == 4) SSC_POOL_FWD(1, 4); else SSC_POOL_FWD(1, 1);
+  }
+#undef SSC_POOL_FWD
+  SSC_LAUNCH_CHECK("pool");
+  return SSC_OK;
+}
+
+extern "C" {
+
 int ssc_pool_max_f32(const float *features, int32_t channels, const int32_t *pairs,
                      int64_t pair_stride, const int32_t *pair_num, int32_t kernel_volume,
                      float *out, int64_t n_out, void *workspace, size_t workspace_bytes,
                      ssc_stream_t stream) {
-  hipStream_t s = (hipStream_t)stream;
-  int32_t *table = nullptr;
-  int rc = pool_common(features, channels, pairs, pair_stride, pair_num, kernel_volume, out, n_out,
-                       workspace, workspace_bytes, s, &table);
-  if (rc != SSC_OK || n_out == 0) return rc;
-  if ((channels & 3) == 0) {
-    int64_t n = n_out * (channels / 4);
-    hipLaunchKernelGGL((pool_kernel<0, 4>), dim3((unsigned)ceil_div(n, 256)), dim3(256), 0, s,
-                       features, channels, table, kernel_volume, (const int32_t *)nullptr, out,
-                       n_out);
-  } else {
-    int64_t n = n_out * channels;
-    hipLaunchKernelGGL((pool_kernel<0, 1>), dim3((unsigned)ceil_div(n, 256)), dim3(256), 0, s,
-                       features, channels, table, kernel_volume, (const int32_t *)nullptr, out,
-                       n_out);
-  }
-  SSC_LAUNCH_CHECK("pool_max");
-  return SSC_OK;
+  return pool_fwd<float>(0, features, channels, pairs, pair_stride, pair_num, kernel_volume,
+                         nullptr, out, n_out, workspace, workspace_bytes, (hipStream_t)stream);
 }
 
 int ssc_pool_avg_f32(const float *features, int32_t channels, const int32_t *pairs,
                      int64_t pair_stride, const int32_t *pair_num, int32_t kernel_volume,
                      const int32_t *summaryrf, float *out, int64_t n_out, void *workspace,
                      size_t workspace_bytes, ssc_stream_t stream) {
-  hipStream_t s = (hipStream_t)stream;
-  SSC_CHECK(n_out == 0 || summaryrf != nullptr, SSC_EINVAL, "summaryrf is NULL");
-  int32_t *table = nullptr;
-  int rc = pool_common(features, channels, pairs, pair_stride, pair_num, kernel_volume, out, n_out,
-                       workspace, workspace_bytes, s, &table);
-  if (rc != SSC_OK || n_out == 0) return rc;
-  if ((channels & 3) == 0) {
-    int64_t n = n_out * (channels / 4);
-    hipLaunchKernelGGL((pool_kernel<1, 4>), dim3((unsigned)ceil_div(n, 256)), dim3(256), 0, s,
-                       features, channels, table, kernel_volume, summaryrf, out, n_out);
-  } else {
-    int64_t n = n_out * channels;
-    hipLaunchKernelGGL((pool_kernel<1, 1>), dim3((unsigned)ceil_div(n, 256)), dim3(256), 0, s,
-                       features, channels, table, kernel_volume, summaryrf, out, n_out);
-  }
-  SSC_LAUNCH_CHECK("pool_avg");
-  return SSC_OK;
+  return pool_fwd<float>(1, features, channels, pairs, pair_stride, pair_num, kernel_volume,
+                         summaryrf, out, n_out, workspace, workspace_bytes, (hipStream_t)stream);
+}
+
+int ssc_pool_max_f16(const void *features, int32_t channels, const int32_t *pairs,
+                     int64_t pair_stride, const int32_t *pair_num, int32_t kernel_volume,
+                     void *out, int64_t n_out, void *workspace, size_t workspace_bytes,
+                     ssc_stream_t stream) {
+  return pool_fwd<_Float16>(0, static_cast<const _Float16 *>(features), channels, pairs,
+                            pair_stride, pair_num, kernel_volume, nullptr,
+                            static_cast<_Float16 *>(out), n_out, workspace, workspace_bytes,
+                            (hipStream_t)stream);
+}
+
+int ssc_pool_avg_f16(const void *features, int32_t channels, const int32_t *pairs,
+                     int64_t pair_stride, const int32_t *pair_num, int32_t kernel_volume,
+                     const int32_t *summaryrf, void *out, int64_t n_out, void *workspace,
+                     size_t workspace_bytes, ssc_stream_t stream) {
+  return pool_fwd<_Float16>(1, static_cast<const _Float16 *>(features), channels, pairs,
+                            pair_stride, pair_num, kernel_volume, summaryrf,
+                            static_cast<_Float16 *>(out), n_out, workspace, workspace_bytes,
+                            (hipStream_t)stream);
 }
 
 int ssc_summary_rf(const int32_t *pairs, int64_t pair_stride, const int32_t *pair_num,
@@ -428,9 +448,12 @@ int ssc_segment_max_f32(const float *feats, const int32_t *offsets, float *out, 
   return SSC_OK;
 }
 
-static int pool_bwd(int mode, const float *features, const float *out_features,
-                    const float *out_grad, int channels, const int32_t *pairs, int64_t pair_stride,
-                    const int32_t *pair_num, int K, const int32_t *summaryrf, float *in_grad,
+}  // extern "C"
+
+template <typename IO>
+static int pool_bwd(int mode, const IO *features, const IO *out_features, const IO *out_grad,
+                    int channels, const int32_t *pairs, int64_t pair_stride,
+                    const int32_t *pair_num, int K, const int32_t *summaryrf, IO *in_grad,
                     int64_t n_in, void *ws, size_t ws_bytes, hipStream_t s) {
   SSC_CHECK(K >= 1 && K <= SSC_MAX_KERNEL_VOLUME, SSC_ERUNTIME, "kernel volume %d out of range", K);
   SSC_CHECK(channels >= 1 && n_in >= 0 && pair_stride >= 0, SSC_EINVAL, "bad sizes");
@@ -454,8 +477,8 @@ static int pool_bwd(int mode, const float *features, const float *out_features,
   const int vec = (channels & 3) == 0 ? 4 : 1;
   const int64_t n = n_in * (channels / vec);
   const dim3 grid((unsigned)ceil_div(n, 256));
-#define SSC_POOL_BWD(M, V)                                                                  \
-  hipLaunchKernelGGL((pool_bwd_kernel<M, V>), grid, dim3(256), 0, s, features, out_features, \
+#define SSC_POOL_BWD(M, V)                                                                      \
+  hipLaunchKernelGGL((pool_bwd_kernel<IO, M, V>), grid, dim3(256), 0, s, features, out_features, \
                      out_grad, channels, table, K, summaryrf, in_grad, n_in)
   if (mode == 0) {
     if (vec == 4) SSC_POOL_BWD(0, 4); else SSC_POOL_BWD(0, 1);
@@ -467,23 +490,47 @@ static int pool_bwd(int mode, const float *features, const float *out_features,
   return SSC_OK;
 }
 
+extern "C" {
+
 int ssc_pool_max_bwd_f32(const float *features, const float *out_features, const float *out_grad,
                          int32_t channels, const int32_t *pairs, int64_t pair_stride,
                          const int32_t *pair_num, int32_t kernel_volume, float *in_grad,
                          int64_t n_in, void *workspace, size_t workspace_bytes,
                          ssc_stream_t stream) {
-  return pool_bwd(0, features, out_features, out_grad, channels, pairs, pair_stride, pair_num,
-                  kernel_volume, nullptr, in_grad, n_in, workspace, workspace_bytes,
-                  (hipStream_t)stream);
+  return pool_bwd<float>(0, features, out_features, out_grad, channels, pairs, pair_stride,
+                         pair_num, kernel_volume, nullptr, in_grad, n_in, workspace,
+                         workspace_bytes, (hipStream_t)stream);
+}
+
+int ssc_pool_max_bwd_f16(const void *features, const void *out_features, const void *out_grad,
+                         int32_t channels, const int32_t *pairs, int64_t pair_stride,
+                         const int32_t *pair_num, int32_t kernel_volume, void *in_grad,
+                         int64_t n_in, void *workspace, size_t workspace_bytes,
+                         ssc_stream_t stream) {
+  typedef const _Float16 *H;
+  return pool_bwd<_Float16>(0, (H)features, (H)out_features, (H)out_grad, channels, pairs,
+                            pair_stride, pair_num, kernel_volume, nullptr,
+                            static_cast<_Float16 *>(in_grad), n_in, workspace, workspace_bytes,
+                            (hipStream_t)stream);
 }
 
 int ssc_pool_avg_bwd_f32(const float *out_grad, int32_t channels, const int32_t *pairs,
                          int64_t pair_stride, const int32_t *pair_num, int32_t kernel_volume,
                          const int32_t *summaryrf, float *in_grad, int64_t n_in, void *workspace,
                          size_t workspace_bytes, ssc_stream_t stream) {
-  return pool_bwd(1, nullptr, nullptr, out_grad, channels, pairs, pair_stride, pair_num,
-                  kernel_volume, summaryrf, in_grad, n_in, workspace, workspace_bytes,
-                  (hipStream_t)stream);
+  return pool_bwd<float>(1, nullptr, nullptr, out_grad, channels, pairs, pair_stride, pair_num,
+                         kernel_volume, summaryrf, in_grad, n_in, workspace, workspace_bytes,
+                         (hipStream_t)stream);
+}
+
+int ssc_pool_avg_bwd_f16(const void *out_grad, int32_t channels, const int32_t *pairs,
+                         int64_t pair_stride, const int32_t *pair_num, int32_t kernel_volume,
+                         const int32_t *summaryrf, void *in_grad, int64_t n_in, void *workspace,
+                         size_t workspace_bytes, ssc_stream_t stream) {
+  return pool_bwd<_Float16>(1, nullptr, nullptr, static_cast<const _Float16 *>(out_grad), channels,
+                            pairs, pair_stride, pair_num, kernel_volume, summaryrf,
+                            static_cast<_Float16 *>(in_grad), n_in, workspace, workspace_bytes,
+                            (hipStream_t)stream);
 }
 
 int ssc_segment_avg_bwd_f32(const float *out_grad, const int32_t *offsets, float *in_grad,

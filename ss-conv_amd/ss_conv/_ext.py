@@ -73,6 +73,10 @@ _SIGNATURES = {
                                             _vp, _sz, _vp]),
     "ssc_pool_avg_bwd_f32": (ctypes.c_int, [_vp, _i32, _vp, _i64, _vp, _i32, _vp, _vp, _i64, _vp,
                                             _sz, _vp]),
+    "ssc_pool_max_bwd_f16": (ctypes.c_int, [_vp, _vp, _vp, _i32, _vp, _i64, _vp, _i32, _vp, _i64,
+                                            _vp, _sz, _vp]),
+    "ssc_pool_avg_bwd_f16": (ctypes.c_int, [_vp, _i32, _vp, _i64, _vp, _i32, _vp, _vp, _i64, _vp,
+                                            _sz, _vp]),
     "ssc_segment_avg_bwd_f32": (ctypes.c_int, [_vp, _vp, _vp, _i64, _i32, _i32, _vp]),
     "ssc_segment_max_bwd_f32": (ctypes.c_int, [_vp, _vp, _vp, _i64, _i32, _i32, _vp]),
     "ssc_voxel_reduce_bwd_f32": (ctypes.c_int, [_vp, _vp, _vp, _i32, _i32, _i32, _i32, _i64, _vp]),
@@ -88,6 +92,11 @@ _SIGNATURES = {
                                         _vp]),
     "ssc_pool_max_static_f32": (ctypes.c_int, [_vp, _i32, _vp, _i64, _vp, _i32, _vp, _i64, _vp]),
     "ssc_pool_avg_f32": (ctypes.c_int, [_vp, _i32, _vp, _i64, _vp, _i32, _vp, _vp, _i64, _vp,
+                                        _sz, _vp]),
+    "ssc_pool_max_f16": (ctypes.c_int, [_vp, _i32, _vp, _i64, _vp, _i32, _vp, _i64, _vp, _sz,
+                                        _vp]),
+    "ssc_pool_max_static_f32": (ctypes.c_int, [_vp, _i32, _vp, _i64, _vp, _i32, _vp, _i64, _vp]),
+    "ssc_pool_avg_f16": (ctypes.c_int, [_vp, _i32, _vp, _i64, _vp, _i32, _vp, _vp, _i64, _vp,
                                         _sz, _vp]),
     "ssc_summary_rf": (ctypes.c_int, [_vp, _i64, _vp, _i32, _vp, _i64, _vp, _sz, _vp]),
     "ssc_segment_avg_f32": (ctypes.c_int, [_vp, _vp, _vp, _i32, _i32, _vp]),
@@ -540,10 +549,18 @@ def indice_conv_backward_half(features, filters, out_bp, indice_pairs, indice_nu
                                  out_bp, indice_pairs, indice_num, inverse, subm)
 
 
-def _pool_args(features, indice_pairs, indice_num):
+_POOL_ENTRIES = {
+    torch.float32: ("ssc_pool_max_f32", "ssc_pool_avg_f32", "ssc_pool_max_bwd_f32",
+                    "ssc_pool_avg_bwd_f32"),
+    torch.half: ("ssc_pool_max_f16", "ssc_pool_avg_f16", "ssc_pool_max_bwd_f16",
+                 "ssc_pool_avg_bwd_f16"),
+}
+
+
+def _pool_args(features, indice_pairs, indice_num, dtype):
     _need_gpu(features, indice_pairs)
-    if features.dtype != torch.float32:
-        raise RuntimeError("rulebook pooling needs float32 features")
+    if features.dtype != dtype:
+        raise RuntimeError("rulebook pooling: expected %s features, got %s" % (dtype, features.dtype))
     features = features.contiguous()
     pairs = indice_pairs.int().contiguous() if indice_pairs.dtype != torch.int32 \
         else indice_pairs.contiguous()
@@ -551,64 +568,113 @@ def _pool_args(features, indice_pairs, indice_num):
     return features, pairs, num
 
 
-def indice_maxpool_fp32(features, indice_pairs, indice_num, num_act):
-    """src/pool/indice_maxpool.h:15-50."""
-    features, pairs, num = _pool_args(features, indice_pairs, indice_num)
+def _same_type(features, *others):
+    for t in others:
+        if t.dtype != features.dtype:
+            raise RuntimeError("rulebook pooling: features and gradients must have one type")
+
+
+def _maxpool(dtype, features, indice_pairs, indice_num, num_act):
+    features, pairs, num = _pool_args(features, indice_pairs, indice_num, dtype)
     n_out, c, K = int(num_act), features.size(1), pairs.size(0)
-    out = torch.empty((n_out, c), dtype=torch.float32, device=features.device)
+    out = torch.empty((n_out, c), dtype=dtype, device=features.device)
     ws = _workspace(_lib.ssc_pool_workspace_bytes(n_out, K), features.device)
-    _check(_lib.ssc_pool_max_f32(_ptr(features), c, _ptr(pairs), pairs.size(2), num.data_ptr(), K,
-                                 _ptr(out), n_out, ws.data_ptr(), ws.numel(), _stream(features)))
+    _check(getattr(_lib, _POOL_ENTRIES[dtype][0])(
+        _ptr(features), c, _ptr(pairs), pairs.size(2), num.data_ptr(), K, _ptr(out), n_out,
+        ws.data_ptr(), ws.numel(), _stream(features)))
     return out
 
 
-def indice_avgpool_fp32(features, indice_pairs, indice_num, num_act, summaryrf):
-    """src/pool/indice_avgpool.h:17-52."""
-    features, pairs, num = _pool_args(features, indice_pairs, indice_num)
+def _avgpool(dtype, features, indice_pairs, indice_num, num_act, summaryrf):
+    features, pairs, num = _pool_args(features, indice_pairs, indice_num, dtype)
     n_out, c, K = int(num_act), features.size(1), pairs.size(0)
     rf = summaryrf.to(device=features.device, dtype=torch.int32).contiguous()
     if rf.numel() != n_out:
         raise RuntimeError("summaryrf must have one entry per output row")
-    out = torch.empty((n_out, c), dtype=torch.float32, device=features.device)
+    out = torch.empty((n_out, c), dtype=dtype, device=features.device)
     ws = _workspace(_lib.ssc_pool_workspace_bytes(n_out, K), features.device)
-    _check(_lib.ssc_pool_avg_f32(_ptr(features), c, _ptr(pairs), pairs.size(2), num.data_ptr(), K,
-                                 _ptr(rf), _ptr(out), n_out, ws.data_ptr(), ws.numel(),
-                                 _stream(features)))
+    _check(getattr(_lib, _POOL_ENTRIES[dtype][1])(
+        _ptr(features), c, _ptr(pairs), pairs.size(2), num.data_ptr(), K, _ptr(rf), _ptr(out),
+        n_out, ws.data_ptr(), ws.numel(), _stream(features)))
     return out
+
+
+def _maxpool_backward(dtype, features, out_features, out_bp, indice_pairs, indice_num):
+    features, pairs, num = _pool_args(features, indice_pairs, indice_num, dtype)
+    out_features = out_features.contiguous()
+    out_bp = out_bp.contiguous()
+    _need_gpu(out_features, out_bp)
+    _same_type(features, out_features, out_bp)
+    n_in, c = features.shape
+    K = pairs.size(0)
+    din = torch.empty((n_in, c), dtype=dtype, device=features.device)
+    ws = _workspace(_lib.ssc_pool_workspace_bytes(n_in, K), features.device)
+    _check(getattr(_lib, _POOL_ENTRIES[dtype][2])(
+        _ptr(features), _ptr(out_features), _ptr(out_bp), c, _ptr(pairs), pairs.size(2),
+        num.data_ptr(), K, _ptr(din), n_in, ws.data_ptr(), ws.numel(), _stream(features)))
+    return din
+
+
+def _avgpool_backward(dtype, features, out_bp, indice_pairs, indice_num, summaryrf):
+    features, pairs, num = _pool_args(features, indice_pairs, indice_num, dtype)
+    out_bp = out_bp.contiguous()
+    _need_gpu(out_bp, summaryrf)
+    _same_type(features, out_bp)
+    rf = summaryrf.int().contiguous()
+    n_in, c = features.shape
+    K = pairs.size(0)
+    din = torch.empty((n_in, c), dtype=dtype, device=features.device)
+    ws = _workspace(_lib.ssc_pool_workspace_bytes(n_in, K), features.device)
+    _check(getattr(_lib, _POOL_ENTRIES[dtype][3])(
+        _ptr(out_bp), c, _ptr(pairs), pairs.size(2), num.data_ptr(), K, _ptr(rf), _ptr(din), n_in,
+        ws.data_ptr(), ws.numel(), _stream(features)))
+    return din
+
+
+def indice_maxpool_fp32(features, indice_pairs, indice_num, num_act):
+    """src/pool/indice_maxpool.h:15-50."""
+    return _maxpool(torch.float32, features, indice_pairs, indice_num, num_act)
+
+
+def indice_maxpool_half(features, indice_pairs, indice_num, num_act):
+    """indice_maxpool_half (src/ss_conv_ops_api.cpp:34): src/pool/indice_maxpool.h:15-50 on
+    half rows."""
+    return _maxpool(torch.half, features, indice_pairs, indice_num, num_act)
+
+
+def indice_avgpool_fp32(features, indice_pairs, indice_num, num_act, summaryrf):
+    """src/pool/indice_avgpool.h:17-52."""
+    return _avgpool(torch.float32, features, indice_pairs, indice_num, num_act, summaryrf)
+
+
+def indice_avgpool_half(features, indice_pairs, indice_num, num_act, summaryrf):
+    """indice_avgpool_half (src/ss_conv_ops_api.cpp:29): every operation rounded to half, as
+    at::Half's operators do."""
+    return _avgpool(torch.half, features, indice_pairs, indice_num, num_act, summaryrf)
 
 
 def indice_maxpool_backward_fp32(features, out_features, out_bp, indice_pairs, indice_num):
     """src/pool/indice_maxpool.h:52-86: gradient of the pooled rows routed to the inputs
     that equal the maximum."""
-    features, pairs, num = _pool_args(features, indice_pairs, indice_num)
-    out_features = out_features.contiguous()
-    out_bp = out_bp.contiguous()
-    _need_gpu(out_features, out_bp)
-    n_in, c = features.shape
-    K = pairs.size(0)
-    din = torch.empty((n_in, c), dtype=torch.float32, device=features.device)
-    ws = _workspace(_lib.ssc_pool_workspace_bytes(n_in, K), features.device)
-    _check(_lib.ssc_pool_max_bwd_f32(_ptr(features), _ptr(out_features), _ptr(out_bp), c,
-                                     _ptr(pairs), pairs.size(2), num.data_ptr(), K, _ptr(din),
-                                     n_in, ws.data_ptr(), ws.numel(), _stream(features)))
-    return din
+    return _maxpool_backward(torch.float32, features, out_features, out_bp, indice_pairs,
+                             indice_num)
+
+
+def indice_maxpool_backward_half(features, out_features, out_bp, indice_pairs, indice_num):
+    """indice_maxpool_backward_half (src/ss_conv_ops_api.cpp:35)."""
+    return _maxpool_backward(torch.half, features, out_features, out_bp, indice_pairs, indice_num)
 
 
 def indice_avgpool_backward_fp32(features, out_features, out_bp, indice_pairs, indice_num,
                                  summaryrf):
     """src/pool/indice_avgpool.h:54-90."""
-    features, pairs, num = _pool_args(features, indice_pairs, indice_num)
-    out_bp = out_bp.contiguous()
-    _need_gpu(out_bp, summaryrf)
-    rf = summaryrf.int().contiguous()
-    n_in, c = features.shape
-    K = pairs.size(0)
-    din = torch.empty((n_in, c), dtype=torch.float32, device=features.device)
-    ws = _workspace(_lib.ssc_pool_workspace_bytes(n_in, K), features.device)
-    _check(_lib.ssc_pool_avg_bwd_f32(_ptr(out_bp), c, _ptr(pairs), pairs.size(2), num.data_ptr(),
-                                     K, _ptr(rf), _ptr(din), n_in, ws.data_ptr(), ws.numel(),
-                                     _stream(features)))
-    return din
+    return _avgpool_backward(torch.float32, features, out_bp, indice_pairs, indice_num, summaryrf)
+
+
+def indice_avgpool_backward_half(features, out_features, out_bp, indice_pairs, indice_num,
+                                 summaryrf):
+    """indice_avgpool_backward_half (src/ss_conv_ops_api.cpp:30)."""
+    return _avgpool_backward(torch.half, features, out_bp, indice_pairs, indice_num, summaryrf)
 
 
 def global_avgpool_bp(d_feats, offsets, out_maxidx, d_out, n_proposal, c):

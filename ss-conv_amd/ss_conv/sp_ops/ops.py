@@ -88,21 +88,29 @@ def indice_conv_backward(features, filters, out_bp, indice_pairs, indice_pair_nu
 def indice_maxpool_forward(features, indice_pairs, indice_pair_num, num_activate_out):
     if features.dtype == torch.float32:
         return _ext.indice_maxpool_fp32(features, indice_pairs, indice_pair_num, num_activate_out)
-    raise NotImplementedError("only float32 pooling is built")
+    if features.dtype == torch.half:
+        return _ext.indice_maxpool_half(features, indice_pairs, indice_pair_num, num_activate_out)
+    raise NotImplementedError("pooling is built for float32 and half features")
 
 
 def indice_maxpool_backward(features, out_features, out_bp, indice_pairs, indice_pair_num):
     if features.dtype == torch.float32:
         return _ext.indice_maxpool_backward_fp32(features, out_features, out_bp, indice_pairs,
                                                  indice_pair_num)
-    raise NotImplementedError("only float32 pooling is built")
+    if features.dtype == torch.half:
+        return _ext.indice_maxpool_backward_half(features, out_features, out_bp, indice_pairs,
+                                                 indice_pair_num)
+    raise NotImplementedError("pooling is built for float32 and half features")
 
 
 def indice_avgpool_forward(features, indice_pairs, indice_pair_num, num_activate_out, summaryrf):
     if features.dtype == torch.float32:
         return _ext.indice_avgpool_fp32(features, indice_pairs, indice_pair_num, num_activate_out,
                                         summaryrf)
-    raise NotImplementedError("only float32 pooling is built")
+    if features.dtype == torch.half:
+        return _ext.indice_avgpool_half(features, indice_pairs, indice_pair_num, num_activate_out,
+                                        summaryrf)
+    raise NotImplementedError("pooling is built for float32 and half features")
 
 
 def indice_avgpool_backward(features, out_features, out_bp, indice_pairs, indice_pair_num,
@@ -110,4 +118,7 @@ def indice_avgpool_backward(features, out_features, out_bp, indice_pairs, indice
     if features.dtype == torch.float32:
         return _ext.indice_avgpool_backward_fp32(features, out_features, out_bp, indice_pairs,
                                                  indice_pair_num, summaryrf)
-    raise NotImplementedError("only float32 pooling is built")
+    if features.dtype == torch.half:
+        return _ext.indice_avgpool_backward_half(features, out_features, out_bp, indice_pairs,
+                                                 indice_pair_num, summaryrf)
+    raise NotImplementedError("pooling is built for float32 and half features")

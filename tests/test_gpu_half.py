@@ -258,3 +258,44 @@ def test_convolution_layer_on_half_features(device):
     y32.backward(g.float())
     assert within_one_ulp(x_h.grad, x32.grad)
     assert conv.kernel.weight.grad is not None and torch.isfinite(conv.kernel.weight.grad).all()
+
+
+@pytest.mark.parametrize("k,s,p,c", [(2, 2, 0, 64), (3, 2, 1, 32), (3, 1, 1, 5), (3, 1, 1, 12)])
+def test_half_pools_match_oracle(k, s, p, c, oracle, device):
+    """ssc_pool_{max,avg}_f16 and their gradients (indice_maxpool_half, indice_avgpool_half,
+    indice_*pool_backward_half; src/ss_conv_ops_api.cpp:29-35) against the oracle's half
+    routines, bit for bit: every operation rounds to half, in the order of the offsets.
+    Forward through the raw entry points, backward through autograd as a layer runs it."""
+    from ss_conv import _ext
+    from ss_conv.sp_ops.functional import indice_avgpool, indice_maxpool
+    rng = np.random.default_rng(41)
+    n, grid = 400, 10
+    idx = random_voxels(rng, 2, grid, n)
+    feats = rng.normal(size=(n, c)).astype(np.float16)
+    o_idx, o_pairs, o_num = oracle.canonicalize(*oracle.rulebook(idx, 2, [grid] * 3, k, s, p))
+    n_out = o_idx.shape[0]
+    g_idx, g_pairs, g_num = [torch.from_numpy(x).to(device) for x in
+                             gpu_rulebook(idx, 2, grid, k, s, p)]
+    ft = torch.from_numpy(feats).to(device)
+    mx = _ext.indice_maxpool_half(ft, g_pairs, g_num, n_out)
+    assert mx.dtype == torch.half
+    want_mx = oracle.maxpool_fwd_half(feats, o_pairs, o_num, n_out)
+    assert np.array_equal(mx.cpu().numpy(), want_mx)
+    rf = _ext.indiceSummaryRF(g_pairs, g_num, n_out)
+    for r in (torch.full((n_out,), k ** 3, dtype=torch.int32, device=device), rf):
+        av = _ext.indice_avgpool_half(ft, g_pairs, g_num, n_out, r)
+        want = oracle.avgpool_fwd_half(feats, o_pairs, o_num, n_out, r.cpu().numpy())
+        assert np.array_equal(av.cpu().numpy(), want)
+    g_out = rng.normal(size=(n_out, c)).astype(np.float16)
+    gt = torch.from_numpy(g_out).to(device)
+    x = ft.clone().requires_grad_(True)
+    indice_maxpool(x, g_pairs, g_num, n_out).backward(gt)
+    assert np.array_equal(x.grad.cpu().numpy(),
+                          oracle.maxpool_bwd_half(feats, want_mx, g_out, o_pairs, o_num))
+    x = ft.clone().requires_grad_(True)
+    indice_avgpool(x, g_pairs, g_num, n_out).backward(gt)
+    want = oracle.avgpool_bwd_half(g_out, o_pairs, o_num, n,
+                                   np.full(n_out, k ** 3, dtype=np.int32))
+    assert np.array_equal(x.grad.cpu().numpy(), want)
+    with pytest.raises(RuntimeError):
+        _ext.indice_maxpool_half(ft.float(), g_pairs, g_num, n_out)

@@ -304,3 +304,68 @@ def test_combine_equals_einsum(oracle):
                 assert np.allclose(blk, want.reshape(blk.shape).numpy(), atol=1e-5)
             c0 += mi * d_in[j]
         r0 += mo * d_out[i]
+
+
+def _h(x):
+    """x rounded to binary16 by struct's codec (round to nearest even), as a float."""
+    import struct
+    return struct.unpack("<e", struct.pack("<e", float(x)))[0]
+
+
+def test_half_pools_known_answers(oracle):
+    """The half-precision pools round after every operation (at::Half's operators,
+    src/pool/indice_avgpool_cuda_functor.cu:46): known answers rounded by hand with struct's
+    binary16 codec, one window of three inputs; where every step is exact in half the result
+    equals the float routine's; the maximum equals the float routine on the widened rows."""
+    # one output row, three offsets with one pair each
+    pairs = np.zeros((3, 2, 1), dtype=np.int32)
+    pairs[:, 0, 0] = [0, 1, 2]
+    num = np.ones(3, dtype=np.int32)
+    vals = [0.7, 2.3, 5.1]
+    feats = np.array(vals, dtype=np.float16).reshape(3, 1)
+    rf = np.array([3], dtype=np.int32)
+    acc = 0.0
+    for v in vals:  # products of float(half) operands: exact in double, one rounding to float
+        q = _h(np.float32(np.float32(_h(v)) / np.float32(3.0)))
+        acc = _h(np.float32(np.float32(acc) + np.float32(q)))
+    got = oracle.avgpool_fwd_half(feats, pairs, num, 1, rf)
+    assert got.dtype == np.float16 and float(got[0, 0]) == acc
+    # rounding at every step shows: the float routine, rounded once at the end, differs
+    once = _h(oracle.avgpool_fwd(feats.astype(np.float32), pairs, num, 1, rf)[0, 0])
+    assert once != acc
+    # backward: din[i] = half(dout / half(rf)) for each of the three inputs
+    g = np.array([[0.3]], dtype=np.float16)
+    din = oracle.avgpool_bwd_half(g, pairs, num, 3, rf)
+    assert all(float(din[i, 0]) == _h(np.float32(np.float32(_h(0.3)) / np.float32(3.0))) for i in range(3))
+
+    # exact cases: small integers and a power-of-two window
+    rng = np.random.default_rng(5)
+    idx = random_voxels(rng, 2, 8, 120)
+    o_idx, pairs, num, _ = oracle.rulebook(idx, 2, [8] * 3, 2, 2, 0)
+    n_out = o_idx.shape[0]
+    ints = rng.integers(-8, 9, size=(120, 5)).astype(np.float32)
+    av = oracle.avgpool_fwd_half(ints, pairs, num, n_out)       # rf = 8: every quotient exact
+    assert np.array_equal(av.astype(np.float32), oracle.avgpool_fwd(ints, pairs, num, n_out))
+    x = rng.normal(size=(120, 5)).astype(np.float16)
+    mx = oracle.maxpool_fwd_half(x, pairs, num, n_out)
+    assert np.array_equal(mx.astype(np.float32),
+                          oracle.maxpool_fwd(x.astype(np.float32), pairs, num, n_out))
+    # max backward: integer gradients add exactly, so half and float routines agree
+    gi = rng.integers(-4, 5, size=(n_out, 5)).astype(np.float32)
+    a = oracle.maxpool_bwd_half(x, mx, gi, pairs, num)
+    b = oracle.maxpool_bwd(x.astype(np.float32), mx.astype(np.float32), gi, pairs, num)
+    assert np.array_equal(a.astype(np.float32), b)
+    # a window with overlap (3, stride 1): sums of halves that do round -- against a scalar
+    # loop with struct's codec
+    o_idx, pairs, num, _ = oracle.rulebook(idx, 2, [8] * 3, 3, 1, 1)
+    n_out = o_idx.shape[0]
+    rf = oracle.summary_rf(pairs, num, n_out)
+    x1 = rng.normal(size=(120, 1)).astype(np.float16)
+    got = oracle.avgpool_fwd_half(x1, pairs, num, n_out, rf)
+    want = np.zeros(n_out)
+    for k in range(pairs.shape[0]):
+        for j in range(int(num[k])):
+            i, o = int(pairs[k, 0, j]), int(pairs[k, 1, j])
+            q = _h(np.float32(np.float32(x1[i, 0]) / np.float32(_h(float(rf[o])))))
+            want[o] = _h(np.float32(np.float32(want[o]) + np.float32(q)))
+    assert np.array_equal(got[:, 0].astype(np.float64), want)
