@@ -289,11 +289,14 @@ def point_voxel_rows(torch, synth, dev, seed, timed, report):
 def build_backbone(torch, synth, dev, seed):
     """The backbone of the fourth configuration in evaluation mode: inputs, layers and a
     function that runs it and returns (pooled, point features, last SparseTensor, stages),
-    stages being the SparseTensor after every convolution."""
+    stages holding row counts, pair counts and channel counts of every convolution.
+    backbone(separate=True) runs convolution, batch norm and activation of a block one
+    after the other; by default a block is one fused.ConvBatchNormActivation, whose
+    convolution kernel applies the other two while it stores its rows."""
     from ss_conv.activation import Activation
     from ss_conv.batchnorm import BatchNorm
     from ss_conv.convolution import Convolution
-    from ss_conv.fused import BatchNormActivation
+    from ss_conv.fused import BatchNormActivation, ConvBatchNormActivation
     from ss_conv.pool import GlobalAvgPool
     from ss_conv.sp_ops.voxelize import Point2Voxel, Voxel2Point
     pts, feats, ids = synth.make_clouds(32, 1024, seed=seed, channels=3)
@@ -303,21 +306,21 @@ def build_backbone(torch, synth, dev, seed):
     for mult, stride in ((8, 1), (16, 2), (32, 2), (32, 1)):
         rs = synth.irreps(mult, 3)
         gated = rs + [(sum(m for m, l in rs[1:]), 0)]
-        conv = Convolution(rs_in, gated, 3, stride=stride, padding=1).to(dev).eval()
-        block = BatchNormActivation(BatchNorm(gated), Activation(rs, (torch.relu, torch.sigmoid)))
-        layers.append((conv, block.to(dev).eval()))
+        conv = Convolution(rs_in, gated, 3, stride=stride, padding=1)
+        bn, act = BatchNorm(gated), Activation(rs, (torch.relu, torch.sigmoid))
+        block = ConvBatchNormActivation(conv, bn, act).to(dev).eval()
+        layers.append((block, BatchNormActivation(bn, act).to(dev).eval()))
         rs_in = rs
     gap = GlobalAvgPool()
 
-    def backbone():
+    def backbone(separate=False):
         vp, x, vi, _ = p2v(tp, tf, ti)
         stages = []
-        for conv, block in layers:
+        for block, bn_act in layers:
             n_in = x.features.shape[0]
-            y = conv(x)
-            stages.append((n_in, y.features.shape[0], y.indice_dict[None][3], conv.in_channels,
-                           conv.out_channels))
-            x = block(y)
+            x = bn_act(block.conv(x)) if separate else block(x)
+            stages.append((n_in, x.features.shape[0], x.indice_dict[None][3],
+                           block.conv.in_channels, block.conv.out_channels))
         pooled = gap(x.features.contiguous(), x.get_offsets().int().contiguous())
         v2p = Voxel2Point(unit_voxel_extent=[2.0 / s for s in x.spatial_shape])
         return pooled, v2p(x, vp, vi), x, stages
@@ -329,16 +332,22 @@ def backbone_table(torch, _ext, synth, dev, seed, n=5, warm=2):
     stage: rows, pairs, flops, the MFMA kernel's time (HIP events around its launch) and
     its fraction of the fp32 MFMA peak; then the whole forward."""
     backbone = build_backbone(torch, synth, dev, seed)
-    with torch.no_grad():
-        for _ in range(warm):
-            r = backbone()
-        torch.cuda.synchronize()
-        _ext.profile_conv(True)
+
+    def run(**kw):
         a = time.perf_counter()
         for _ in range(n):
+            out = backbone(**kw)
+        torch.cuda.synchronize()
+        return (time.perf_counter() - a) * 1e3 / n, out
+
+    with torch.no_grad():
+        for _ in range(warm):
+            backbone(separate=True)
             r = backbone()
         torch.cuda.synchronize()
-        ms = (time.perf_counter() - a) * 1e3 / n
+        ms_sep, _ = run(separate=True)
+        _ext.profile_conv(True)
+        ms, r = run()
         conv_ms = _ext.profile_conv_read()
         _ext.profile_conv(False)
     stages = r[3]
@@ -351,8 +360,11 @@ def backbone_table(torch, _ext, synth, dev, seed, n=5, warm=2):
                     "%8.3f ms = %6.1f TFLOP/s = %5.1f%% of fp32 MFMA peak"
                     % (i + 1, n_in, n_out, cin, cout, P, fl / 1e9, t, fl / t / 1e9,
                        fl / t / 1e9 / (FP32_MFMA_PEAK_TFLOPS / 100.0)))
-    rows.append("  whole forward %.3f ms (%d voxels after stage 4, %d channels)"
-                % (ms, r[2].features.shape[0], r[2].features.shape[1]))
+    rows.append("  whole forward %.3f ms (%d voxels after stage 4, %d channels); %.3f ms with "
+                "convolution, batch norm and activation as separate kernels"
+                % (ms, r[2].features.shape[0], r[2].features.shape[1], ms_sep))
+    rows.append("  (kernel times: with batch norm and gate applied by the convolution kernel; "
+                "flops of the layer's own filter columns, gates included)")
     print("\n".join(rows), file=sys.stderr)
 
 

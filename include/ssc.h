@@ -217,6 +217,42 @@ int ssc_conv_run_f16(const void *features /* [n_in,c_in] half */, int64_t n_in, 
                      int64_t pair_stride, int32_t kernel_volume, int32_t c_out,
                      void *out /* [n_out,c_out] half */, int64_t n_out, ssc_stream_t stream);
 
+/* The convolution of ssc_conv_run_f32 with an evaluation-mode batch normalisation and the
+ * gated non-linearity applied to every output row before it is stored -- replaces the
+ * sequence conv -> bn -> activation of an evaluation-mode block
+ * (Common_utils/ss_conv_modules.py:105-117: Convolution.forward, then BatchNorm.forward with
+ * running statistics, ss_conv/batchnorm.py:49-136, then Activation._gate,
+ * ss_conv/activation.py:55-100) without writing the convolution's own output.
+ *
+ * The packed filters have c_cols columns (a multiple of 4) in an order of the caller's
+ * choice; the tables describe each of them (device memory, c_cols entries):
+ *   z = (x - shift[c]) * scale[c] + add[c]          (what ssc_bn_prepare_f32 returns)
+ *   mode[c] 0: y = z    1: y = act_scalar(z + pre_bias[c])
+ *           2: y = z * act_gate(z_g + pre_bias[g]), g = gate[c]
+ *           3: the column is not stored (gates, padding)
+ *   y is stored at out[row, dest[c]]; out has c_dest columns.
+ * The kernel works on blocks of 64 columns (c / 64).  The gates of a block are one run of at
+ * most 16 of its columns, gate_run[2b] the first and gate_run[2b+1] their number for block
+ * b (ceil(c_cols / 64) blocks): act_gate is evaluated once per gate and row, and a column of
+ * mode 2 must name a gate of its own block's run.  A column whose gate or dest breaks these
+ * rules is not stored.
+ * Plan and packed filters are those of ssc_conv_plan_build / ssc_conv_pack_filters_f32 for
+ * c_out = c_cols.  Refuses a rulebook without pairs (SSC_EINVAL). */
+typedef struct ssc_conv_epilogue {
+  const float *shift, *scale, *add, *pre_bias;
+  const int32_t *mode, *gate, *dest;
+  const int32_t *gate_run;
+  int32_t act_scalar, act_gate; /* SSC_ACT_* */
+  int32_t c_dest;
+} ssc_conv_epilogue;
+
+int ssc_conv_run_epilogue_f32(const float *features /* [n_in,c_in] */, int64_t n_in, int32_t c_in,
+                              const void *packed, size_t packed_bytes, const void *plan,
+                              size_t plan_bytes, int64_t pair_stride, int32_t kernel_volume,
+                              int32_t c_cols, const ssc_conv_epilogue *epilogue,
+                              float *out /* [n_out,c_dest] */, int64_t n_out,
+                              ssc_stream_t stream);
+
 /* ----------------------------------------------------------------------
  * Gradients of the sparse convolution -- replaces indice_conv_backward_fp32
  * (src/ss_conv_ops_api.cpp:22, src/conv/indice_conv.h:344-426).

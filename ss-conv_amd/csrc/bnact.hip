@@ -46,20 +46,12 @@ static BnShape bn_shape(int64_t n, int c, int max_tx = kBnThreads,
   return s;
 }
 
-__device__ __forceinline__ float act_fn(int kind, float u) {
-  switch (kind) {
-    case SSC_ACT_RELU: return u > 0.f ? u : 0.f;
-    case SSC_ACT_SIGMOID: return 1.f / (1.f + __expf(-u));
-    case SSC_ACT_TANH: return tanhf(u);
-    default: return u;
-  }
-}
 // derivative of act_fn at u
 __device__ __forceinline__ float act_grad(int kind, float u) {
   switch (kind) {
     case SSC_ACT_RELU: return u > 0.f ? 1.f : 0.f;
     case SSC_ACT_SIGMOID: {
-      float s = 1.f / (1.f + __expf(-u));
+      float s = __builtin_amdgcn_rcpf(1.f + __expf(-u));
       return s * (1.f - s);
     }
     case SSC_ACT_TANH: {

@@ -724,7 +724,22 @@ struct StagePos {
 // equal width 4 NS instead (200 channels: 4 chunks of 52, 13 steps each, where chunks of 64
 // would run 64 steps for 50 steps' worth of channels): MFMA steps, fragment loads, gathers
 // and staged-row reads beyond NS are left out.  Half precision always runs whole chunks.
-template <typename IO, int GATHER, int NCW, int NS>
+// What conv_fwd_kernel applies to a finished tile instead of storing its sums: per column c
+// of the accumulators z = (x - shift[c]) * scale[c] + add[c], then by mode[c]
+//   0  y = z                                          2  y = z * act_gate(z_g + pre[g]),
+//   1  y = act_scalar(z + pre[c])                        g = gate[c], a column of the same
+//   3  nothing is stored (gates, padding)                workgroup's column range
+// stored at column dest[c] of rows of c_dest columns.  The gates of a block of 64 columns
+// are one run of at most 16 columns (gate_run): act_gate is evaluated once per gate and
+// row, not once per gated column.  mode == nullptr: plain store.
+struct ConvEpilogue {
+  const float *shift, *scale, *add, *pre;  // [cout]
+  const int32_t *mode, *gate, *dest;       // [cout]
+  const int32_t *gate_run;                 // [2 * blocks of 64 columns]: first gate, gates
+  int act_s, act_g, c_dest;
+};
+
+template <typename IO, int GATHER, int NCW, int NS, bool EPI>
 __global__ void __launch_bounds__((NCW + 4) * 64)
     __attribute__((amdgpu_waves_per_eu((NCW + 4) / 4, (NCW + 4) / 4)))
     conv_fwd_kernel(const IO *__restrict__ features, int cin, unsigned feat_bytes,
@@ -732,7 +747,8 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
                     const int32_t *__restrict__ sched_in, const int32_t *__restrict__ sched_out,
                     const int32_t *__restrict__ grp_meta, unsigned sched_bytes, unsigned meta_bytes,
                     const int32_t *__restrict__ tile_grp, const int32_t *__restrict__ wg_tile,
-                    int nch, int ncb, IO *__restrict__ out, int cout, int T, int cols_per_xcd) {
+                    int nch, int ncb, IO *__restrict__ out, int cout, int T, int cols_per_xcd,
+                    ConvEpilogue epi) {
   constexpr int kCN = 16 * NCW;   // output columns per workgroup
   constexpr int kEB = Io<IO>::kBytes;
   constexpr bool kHalf = kEB == 2;
@@ -790,7 +806,140 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
 
   // Tile `tl` is complete: write its rows, clear the accumulators.
   // (slot0 = accumulator slot of the tile's first row; slots wrap around at T)
-  auto flush_tile = [&](int row0, int rows, int slot0) {
+  // Epilogue constants of this thread, loaded once: when a tile is written out a thread
+  // keeps its 4 columns (c_t) and walks down the rows; lane l of a row's 16 lanes also
+  // owns gate l of the workgroup's column block.
+  //   z = x * e_ca + e_cb (e_cb includes the bias in front of a scalar activation);
+  //   e_mg = mode | LDS column of the gate << 4;  e_dest = output column
+  //   gate l: activated value = act_gate(x * e_gca + e_gcb), LDS column e_gcl (-1: none)
+  float e_ca[4], e_cb[4], e_gca = 0.f, e_gcb = 0.f;
+  int e_mg[4], e_dest[4], e_gcl = -1;
+  bool e_any = false, e_vec = false;
+  if constexpr (EPI) {
+    const int c_t = (tid % (kCN / 4)) * 4, col = col0 + c_t;
+    const bool col_ok = col < cout;
+    static_assert(!EPI || kCN == 64, "the epilogue's gate runs are per block of 64 columns");
+    const int gfirst = epi.gate_run[2 * cblk], gcount = min(epi.gate_run[2 * cblk + 1], 16);
+    const bool run_ok = gfirst >= col0 && gfirst + gcount <= min(col0 + kCN, cout);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int c = col_ok ? col + i : 0;
+      int mode = col_ok ? epi.mode[c] : 3;
+      e_dest[i] = epi.dest[c];
+      const int g = epi.gate[c];
+      // tables that point outside the output row or outside the block's run of gates
+      // switch the column off
+      if (e_dest[i] < 0 || e_dest[i] >= epi.c_dest || mode < 0 || mode > 2 ||
+          (mode == 2 && (!run_ok || g < gfirst || g >= gfirst + gcount)))
+        mode = 3;
+      e_mg[i] = mode | ((mode == 2 ? g - col0 : c_t + i) << 4);
+      e_ca[i] = epi.scale[c];
+      e_cb[i] = epi.add[c] - epi.shift[c] * e_ca[i] + (mode == 1 ? epi.pre[c] : 0.f);
+    }
+    e_any = (e_mg[0] & 15) != 3 || (e_mg[1] & 15) != 3 || (e_mg[2] & 15) != 3 || (e_mg[3] & 15) != 3;
+    e_vec = (e_mg[0] & 15) != 3 && (e_mg[1] & 15) != 3 && (e_mg[2] & 15) != 3 &&
+            (e_mg[3] & 15) != 3 && e_dest[1] == e_dest[0] + 1 && e_dest[2] == e_dest[0] + 2 &&
+            e_dest[3] == e_dest[0] + 3 && ((e_dest[0] | epi.c_dest) & 3) == 0;
+    const int gi = (tid % (kCN / 4));
+    if (run_ok && gi < gcount) {
+      const int g = gfirst + gi;
+      e_gcl = g - col0;
+      e_gca = epi.scale[g];
+      e_gcb = epi.add[g] - epi.shift[g] * e_gca + epi.pre[g];
+    }
+  }
+  const int e_c_dest = epi.c_dest, e_act_s = epi.act_s, e_act_g = epi.act_g;
+  auto flush_tile = [&](int row0, int rows, int slot0) __attribute__((always_inline)) {
+    if constexpr (EPI) {
+      // Batch norm constants and gate applied on the way out (cout % 4 == 0).  Threads,
+      // columns and rows as in the plain store below.  The 16 lanes of a row sit in one wave
+      // and a wave's LDS operations execute in order: first the row's gates are replaced by
+      // their activated values (lane l: gate l), then every lane reads its sums and the
+      // gates of its columns, then the wave clears the row.
+      // FAST: scalar activation none or relu, gate activation none or sigmoid -- a few instructions
+      // per element and no branch (a taken branch costs a wave more than the arithmetic of
+      // a whole row); the other activations go through act_fn.
+      auto rows_out = [&](auto fast_tag) __attribute__((always_inline)) {
+        constexpr bool FAST = decltype(fast_tag)::value;
+        constexpr int U = 2;
+        constexpr int RS = NT / (kCN / 4);
+        const int r_t = tid / (kCN / 4), c_t = (tid % (kCN / 4)) * 4;
+        const float4v z = {0.f, 0.f, 0.f, 0.f};
+        // FAST: max(t, lo) is the scalar activation where there is one, t elsewhere
+        float lo[4];
+        bool gated[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          lo[i] = ((e_mg[i] & 15) == 1 && e_act_s == SSC_ACT_RELU) ? 0.f : -INFINITY;
+          gated[i] = (e_mg[i] & 15) == 2;
+        }
+        auto gate_act = [&](float x) -> float {
+          const float u = x * e_gca + e_gcb;
+          if constexpr (FAST)
+            return e_act_g == SSC_ACT_SIGMOID ? __builtin_amdgcn_rcpf(1.f + __expf(-u)) : u;
+          else
+            return act_fn(e_act_g, u);
+        };
+        float *gp = reinterpret_cast<float *>(out) + (int64_t)(row0 + r_t) * e_c_dest;
+        const int64_t gstep = (int64_t)RS * e_c_dest;
+        for (int r = r_t; r < rows; r += U * RS) {
+          const bool two = r + RS < rows;
+          int sl0 = slot0 + r, sl1 = slot0 + r + RS;
+          if (sl0 >= T) sl0 -= T;
+          if (sl1 >= T) sl1 -= T;
+          float *a0 = acc + sl0 * kAS, *a1 = acc + sl1 * kAS;
+          if (e_gcl >= 0) {
+            const float x0 = a0[e_gcl], x1 = two ? a1[e_gcl] : 0.f;
+            a0[e_gcl] = gate_act(x0);
+            if (two) a1[e_gcl] = gate_act(x1);
+          }
+          __builtin_amdgcn_sched_barrier(0);
+          float4v v0 = *reinterpret_cast<float4v *>(a0 + c_t), v1 = z, g1 = z;
+          float4v g0 = {a0[e_mg[0] >> 4], a0[e_mg[1] >> 4], a0[e_mg[2] >> 4], a0[e_mg[3] >> 4]};
+          if (two) {
+            v1 = *reinterpret_cast<float4v *>(a1 + c_t);
+            g1 = float4v{a1[e_mg[0] >> 4], a1[e_mg[1] >> 4], a1[e_mg[2] >> 4], a1[e_mg[3] >> 4]};
+          }
+          __builtin_amdgcn_sched_barrier(0);  // the clears stay behind every read above
+          *reinterpret_cast<float4v *>(a0 + c_t) = z;
+          if (two) *reinterpret_cast<float4v *>(a1 + c_t) = z;
+          if (e_any) {
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+              if (u == 1 && !two) break;
+              const float4v v = u == 0 ? v0 : v1, gv = u == 0 ? g0 : g1;
+              float4v y;
+#pragma unroll
+              for (int i = 0; i < 4; ++i) {
+                const float t = v[i] * e_ca[i] + e_cb[i];
+                if constexpr (FAST) {
+                  y[i] = fmaxf(t, lo[i]) * (gated[i] ? gv[i] : 1.f);
+                } else {  // every form, then select: no divergent branches
+                  const float ts = act_fn(e_act_s, t);
+                  const int m = e_mg[i] & 15;
+                  y[i] = m == 1 ? ts : m == 2 ? t * gv[i] : t;
+                }
+              }
+              float *p = gp + u * gstep;
+              if (e_vec) {
+                __builtin_nontemporal_store(y, reinterpret_cast<float4v *>(p + e_dest[0]));
+              } else {
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                  if ((e_mg[i] & 15) != 3) __builtin_nontemporal_store(y[i], p + e_dest[i]);
+              }
+            }
+          }
+          gp += U * gstep;
+        }
+      };
+      if ((e_act_s == SSC_ACT_NONE || e_act_s == SSC_ACT_RELU) &&
+          (e_act_g == SSC_ACT_NONE || e_act_g == SSC_ACT_SIGMOID))
+        rows_out(std::true_type());
+      else
+        rows_out(std::false_type());
+      return;
+    }
     if ((cout & 3) == 0) {
       // A thread keeps its 4 columns and walks down the rows, NT / (kCN / 4) rows per
       // step: addresses advance by constants, so a step is little more than its LDS
@@ -1453,12 +1602,13 @@ static size_t conv_ws_bytes(int64_t n_out, int K, int c_in, int c_out, int64_t p
 
 static bool g_conv_by_column = true;  // (switched by ssc_conv_tuning, for measurements)
 
-template <typename IO, int GATHER, int NCW, int NS>
+template <typename IO, int GATHER, int NCW, int NS, bool EPI>
 static int launch_conv(const ConvPlan &p, const ConvWs &w, const IO *features, int64_t n_in,
-                       int c_in, int K, IO *out, int c_out, hipStream_t s) {
+                       int c_in, int K, IO *out, int c_out, const ConvEpilogue &epi,
+                       hipStream_t s) {
   static bool attr_set = false;
   if (!attr_set) {
-    SSC_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(conv_fwd_kernel<IO, GATHER, NCW, NS>),
+    SSC_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(conv_fwd_kernel<IO, GATHER, NCW, NS, EPI>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
     attr_set = true;
   }
@@ -1477,10 +1627,10 @@ static int launch_conv(const ConvPlan &p, const ConvWs &w, const IO *features, i
                          8 % p.n_colblk == 0 && (p.n_wg * p.n_colblk) % 8 == 0 &&
                          g_conv_by_column;
   const int cols_per_xcd = by_column ? 8 / p.n_colblk : 0;
-  hipLaunchKernelGGL((conv_fwd_kernel<IO, GATHER, NCW, NS>), grid, dim3((NCW + 4) * 64), p.lds_bytes, s, features, c_in,
+  hipLaunchKernelGGL((conv_fwd_kernel<IO, GATHER, NCW, NS, EPI>), grid, dim3((NCW + 4) * 64), p.lds_bytes, s, features, c_in,
                      feat_bytes, w.packed, (unsigned)packed_bytes, w.sched_in, w.sched_out,
                      w.grp_meta, (unsigned)sched_bytes, (unsigned)(p.grp_cap * 32), w.tile_grp,
-                     w.wg_tile, p.nch, p.ncb, out, c_out, p.T, cols_per_xcd);
+                     w.wg_tile, p.nch, p.ncb, out, c_out, p.T, cols_per_xcd, epi);
   SSC_LAUNCH_CHECK("conv_fwd");
   return SSC_OK;
 }
@@ -1639,12 +1789,15 @@ static int conv_plan_build(const ConvPlan &p, const ConvWs &w, const int32_t *pa
 // Enqueue the convolution kernel over a built plan and packed filters.
 template <typename IO>
 static int conv_run(const ConvPlan &p, const ConvWs &w, const IO *features, int64_t n_in, int c_in,
-                    int K, IO *out, int c_out, hipStream_t s) {
+                    int K, IO *out, int c_out, hipStream_t s, const ConvEpilogue &epi = ConvEpilogue{}) {
   int rc;
   const bool prof = g_profile_on && (g_profile_calls++ % g_profile_every) == 0;
   const int slot = g_profile_count % kProfileRing;
   if (prof) SSC_HIP(hipEventRecord(g_profile_ev[slot][0], s));
-#define SSC_CONV_LAUNCH(G, S) launch_conv<IO, G, 4, S>(p, w, features, n_in, c_in, K, out, c_out, s)
+#define SSC_CONV_LAUNCH(G, S)                                                                   \
+  (sizeof(IO) == 4 && epi.mode != nullptr                                                       \
+       ? launch_conv<IO, G, 4, S, sizeof(IO) == 4>(p, w, features, n_in, c_in, K, out, c_out, epi, s) \
+       : launch_conv<IO, G, 4, S, false>(p, w, features, n_in, c_in, K, out, c_out, epi, s))
 #define SSC_CONV_BY_STEPS(G)                                                            \
   (p.ns == 1 ? SSC_CONV_LAUNCH(G, 1) : p.ns == 2 ? SSC_CONV_LAUNCH(G, 2)                 \
    : p.ns == 3 ? SSC_CONV_LAUNCH(G, 3) : p.ns == 4 ? SSC_CONV_LAUNCH(G, 4)               \
@@ -1753,7 +1906,51 @@ static int conv_planned(const IO *features, int64_t n_in, int32_t c_in, const vo
   return conv_run<IO>(p, w, features, n_in, c_in, K, out, c_out, s);
 }
 
+// conv_planned with the epilogue applied to every finished tile.
+static int conv_planned_epilogue(const float *features, int64_t n_in, int32_t c_in,
+                                 const void *packed, size_t packed_bytes, const void *plan,
+                                 size_t plan_bytes, int64_t pair_stride, int32_t K, int32_t c_cols,
+                                 const ssc_conv_epilogue *e, float *out, int64_t n_out,
+                                 hipStream_t s) {
+  int rc = conv_check_sizes(K, c_in, c_cols, n_in, n_out, pair_stride);
+  if (rc != SSC_OK) return rc;
+  SSC_CHECK(e != nullptr, SSC_EINVAL, "epilogue is NULL");
+  SSC_CHECK((c_cols & 3) == 0, SSC_EINVAL, "an epilogue needs a multiple of 4 filter columns");
+  SSC_CHECK(e->c_dest >= 1, SSC_EINVAL, "c_dest must be positive");
+  SSC_CHECK(e->act_scalar >= SSC_ACT_NONE && e->act_scalar <= SSC_ACT_TANH &&
+                e->act_gate >= SSC_ACT_NONE && e->act_gate <= SSC_ACT_TANH,
+            SSC_EINVAL, "unknown activation code");
+  if (n_out == 0) return SSC_OK;
+  SSC_CHECK(pair_stride > 0 && n_in > 0, SSC_EINVAL,
+            "no pairs: apply the normalisation to rows of zeros with ssc_bnact_fwd_f32");
+  SSC_CHECK(out && features && packed && plan, SSC_EINVAL, "NULL pointer argument");
+  SSC_CHECK(e->shift && e->scale && e->add && e->pre_bias && e->mode && e->gate && e->dest &&
+                e->gate_run,
+            SSC_EINVAL, "NULL table in the epilogue");
+  ConvPlan p = make_plan(n_in, n_out, K, c_in, c_cols, pair_stride, 4);
+  SSC_CHECK(packed_bytes >= conv_packed_bytes(p, K), SSC_EWORKSPACE,
+            "buffer of the packed filters too small");
+  SSC_CHECK(plan_bytes >= conv_plan_walk(nullptr, p, nullptr), SSC_EWORKSPACE,
+            "plan buffer too small");
+  ConvWs w = {};
+  w.packed = const_cast<void *>(packed);
+  conv_plan_walk(const_cast<void *>(plan), p, &w);
+  const ConvEpilogue epi = {e->shift, e->scale, e->add, e->pre_bias, e->mode, e->gate, e->dest,
+                            e->gate_run, e->act_scalar, e->act_gate, e->c_dest};
+  return conv_run<float>(p, w, features, n_in, c_in, K, out, c_cols, s, epi);
+}
+
 extern "C" {
+
+int ssc_conv_run_epilogue_f32(const float *features, int64_t n_in, int32_t c_in,
+                              const void *packed, size_t packed_bytes, const void *plan,
+                              size_t plan_bytes, int64_t pair_stride, int32_t kernel_volume,
+                              int32_t c_cols, const ssc_conv_epilogue *epilogue, float *out,
+                              int64_t n_out, ssc_stream_t stream) {
+  return conv_planned_epilogue(features, n_in, c_in, packed, packed_bytes, plan, plan_bytes,
+                               pair_stride, kernel_volume, c_cols, epilogue, out, n_out,
+                               (hipStream_t)stream);
+}
 
 int ssc_conv_fwd_f32(const float *features, int64_t n_in, int32_t c_in, const float *filters,
                      int64_t fs_k, int64_t fs_ci, int64_t fs_co, int32_t c_out,

@@ -185,6 +185,20 @@ int read_back_mirror_queued(hipStream_t s);
 // The same, moved on to `dst_host`.
 int read_back(void *dst_host, const void *src_dev, size_t bytes, hipStream_t s);
 
+// The activation functions of the gated non-linearity (SSC_ACT_* of ssc.h).
+#ifdef __HIPCC__
+__device__ __forceinline__ float act_fn(int kind, float u) {
+  switch (kind) {
+    case SSC_ACT_RELU: return u > 0.f ? u : 0.f;
+    // v_rcp_f32 (one unit in the last place) instead of a correctly rounded division: a
+    // fifth of the instructions, and the sigmoid is most of what a gated column costs
+    case SSC_ACT_SIGMOID: return __builtin_amdgcn_rcpf(1.f + __expf(-u));
+    case SSC_ACT_TANH: return tanhf(u);
+    default: return u;
+  }
+}
+#endif
+
 }  // namespace ssc
 
 #endif

@@ -60,6 +60,8 @@ _SIGNATURES = {
                                         _i64, _vp]),
     "ssc_conv_run_f16": (ctypes.c_int, [_vp, _i64, _i32, _vp, _sz, _vp, _sz, _i64, _i32, _i32, _vp,
                                         _i64, _vp]),
+    "ssc_conv_run_epilogue_f32": (ctypes.c_int, [_vp, _i64, _i32, _vp, _sz, _vp, _sz, _i64, _i32,
+                                                 _i32, _vp, _vp, _i64, _vp]),
     "ssc_conv_fwd_f32": (ctypes.c_int, [_vp, _i64, _i32, _vp, _i64, _i64, _i64, _i32, _vp, _i64,
                                         _vp, _i32, _i32, _i32, _vp, _i64, _vp, _sz, _vp]),
     "ssc_conv_fwd_f16": (ctypes.c_int, [_vp, _i64, _i32, _vp, _i64, _i64, _i64, _i32, _vp, _i64,
@@ -392,7 +394,58 @@ def _plan_of(meta, pairs, num, K, c_in, c_out, elem_bytes, n_in, n_out, inverse,
     return plan
 
 
-def _planned_conv(meta, features, owner, filters, fs, pairs, num, K, c_in, c_out, n_out, inverse):
+class _EpilogueStruct(ctypes.Structure):
+    """struct ssc_conv_epilogue of include/ssc.h."""
+    _fields_ = [("shift", _vp), ("scale", _vp), ("add", _vp), ("pre_bias", _vp), ("mode", _vp),
+                ("gate", _vp), ("dest", _vp), ("gate_run", _vp), ("act_scalar", _i32),
+                ("act_gate", _i32), ("c_dest", _i32)]
+
+
+class ConvEpilogue(object):
+    """Tables of ssc_conv_run_epilogue_f32, one entry per filter column (device tensors):
+    float32 shift, scale, add, pre_bias; int32 mode, gate, dest; gate_run with two int32 per
+    block of 64 columns; the activation codes and the number of columns of the rows that
+    are stored."""
+
+    def __init__(self, shift, scale, add, pre_bias, mode, gate, dest, gate_run, act_scalar,
+                 act_gate, c_dest):
+        self.tensors = (shift, scale, add, pre_bias, mode, gate, dest, gate_run)
+        n = shift.numel()
+        for t, dt in zip(self.tensors, (torch.float32,) * 4 + (torch.int32,) * 4):
+            size = 2 * ((n + 63) // 64) if t is gate_run else n
+            if not t.is_cuda or t.dtype != dt or t.numel() != size or not t.is_contiguous():
+                raise RuntimeError("epilogue tables: contiguous GPU vectors, float32 constants "
+                                   "and int32 tables with one entry per filter column, "
+                                   "gate_run with two per block of 64 columns")
+        self.c_cols = n
+        self.c_dest = int(c_dest)
+        self.struct = _EpilogueStruct(*[t.data_ptr() for t in self.tensors], int(act_scalar),
+                                      int(act_gate), int(c_dest))
+
+
+def _run_planned(features, n_in, c_in, packed, plan, pair_stride, K, c_out, n_out, s, epilogue):
+    """Queue the kernel over packed filters and a plan; with an epilogue the rows stored are
+    those of the normalised, gated result."""
+    dev = features.device
+    if epilogue is None:
+        out = torch.empty((n_out, c_out), dtype=features.dtype, device=dev)
+        _check(_ENTRIES[features.dtype][2](_ptr(features), n_in, c_in, packed.data_ptr(),
+                                           packed.numel(), plan.data_ptr(), plan.numel(),
+                                           pair_stride, K, c_out, _ptr(out), n_out, s))
+        return out
+    if features.dtype != torch.float32 or epilogue.c_cols != c_out:
+        raise RuntimeError("a convolution epilogue needs float32 rows and one table entry per "
+                           "filter column")
+    out = torch.empty((n_out, epilogue.c_dest), dtype=torch.float32, device=dev)
+    _check(_lib.ssc_conv_run_epilogue_f32(_ptr(features), n_in, c_in, packed.data_ptr(),
+                                          packed.numel(), plan.data_ptr(), plan.numel(),
+                                          pair_stride, K, c_out, ctypes.byref(epilogue.struct),
+                                          _ptr(out), n_out, s))
+    return out
+
+
+def _planned_conv(meta, features, owner, filters, fs, pairs, num, K, c_in, c_out, n_out, inverse,
+                  epilogue=None):
     """out[n_out, c_out] through a cached plan: the schedule is built on the first call of a
     (direction, channel counts, element type, row counts) combination over this rulebook
     and reused afterwards; later calls launch the filter packing (unless cached as well)
@@ -403,15 +456,12 @@ def _planned_conv(meta, features, owner, filters, fs, pairs, num, K, c_in, c_out
     packed = _packed_filters(owner, filters, fs, K, c_in, c_out, s)
     plan = _plan_of(meta, pairs, num, K, c_in, c_out, features.element_size(), n_in, n_out,
                     inverse, dev, s)
-    out = torch.empty((n_out, c_out), dtype=features.dtype, device=dev)
-    _check(_ENTRIES[features.dtype][2](_ptr(features), n_in, c_in, packed.data_ptr(),
-                                       packed.numel(), plan.data_ptr(), plan.numel(), pairs.size(2),
-                                       K, c_out, _ptr(out), n_out, s))
-    return out
+    return _run_planned(features, n_in, c_in, packed, plan, pairs.size(2), K, c_out, n_out, s,
+                        epilogue)
 
 
 def rulebook_conv(features, filters, indices, batch_size, out_spatial_shape, kernel_size, stride,
-                  padding, dilation, out_padding, subm):
+                  padding, dilation, out_padding, subm, epilogue=None):
     """get_indice_pairs_3d followed by indice_conv_fp32 / indice_conv_half over the new
     rulebook, as a layer without a cached rulebook runs them (ss_conv/sp_ops/conv.py:131-150),
     with the host's wait for the number of outputs placed behind everything that does not
@@ -440,14 +490,11 @@ def rulebook_conv(features, filters, indices, batch_size, out_spatial_shape, ker
     dev = features.device
     s = r.stream
     packed = _packed_filters(owner, filters, (fs_k, fs_ci, fs_co), K, c_in, c_out, s)
-    run = _ENTRIES[dtype][2]
     eb = features.element_size()
     outids, pairs, num = _rulebook_finish(r)
     n_out = outids.size(0)
     plan = _plan_of(pairs._ssc_meta, pairs, num, K, c_in, c_out, eb, n_in, n_out, False, dev, s)
-    out = torch.empty((n_out, c_out), dtype=dtype, device=dev)
-    _check(run(_ptr(features), n_in, c_in, packed.data_ptr(), packed.numel(), plan.data_ptr(),
-               plan.numel(), n_in, K, c_out, _ptr(out), n_out, s))
+    out = _run_planned(features, n_in, c_in, packed, plan, n_in, K, c_out, n_out, s, epilogue)
     return out, outids, pairs, num
 
 
@@ -491,6 +538,27 @@ def _indice_conv(dtype, name, features, filters, indice_pairs, indice_num, num_a
         raise RuntimeError("filters have %d offsets but the rulebook has %d" % (kvol, K))
     return _conv_any(features, owner, filters, (fs_k, fs_ci, fs_co), indice_pairs, pairs, num, K,
                      c_in, c_out, int(num_act_out), inverse, subm)
+
+
+def indice_conv_epilogue_fp32(features, filters, indice_pairs, indice_num, num_act_out, subm,
+                              epilogue):
+    """indice_conv_fp32 (forward direction) over a rulebook this library wrote, followed by
+    the evaluation-mode batch norm and gate of `epilogue` (ConvEpilogue) while the rows are
+    written: the block conv -> bn -> activation of Common_utils/ss_conv_modules.py:105-117
+    as one kernel.  `filters` carry one column per table entry."""
+    _need_gpu(features, filters, indice_pairs)
+    meta = rulebook_meta(indice_pairs)
+    if meta is None or indice_pairs.dtype != torch.int32 or not indice_pairs.is_contiguous():
+        raise RuntimeError("indice_conv_epilogue_fp32 needs a rulebook built by this library")
+    features = features.contiguous()
+    c_in = features.size(1)
+    c_out = filters.size(-1)
+    owner = filters
+    filters, fs_k, fs_ci, fs_co = _filter_strides(filters, c_in, c_out)
+    num = indice_num.to(device=features.device, dtype=torch.int32).contiguous()
+    K = indice_pairs.size(0)
+    return _planned_conv(meta, features, owner, filters, (fs_k, fs_ci, fs_co), indice_pairs, num, K,
+                         c_in, c_out, int(num_act_out), False, epilogue)
 
 
 def indice_conv_fp32(features, filters, indice_pairs, indice_num, num_act_out, inverse, subm):

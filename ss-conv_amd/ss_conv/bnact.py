@@ -92,6 +92,62 @@ def gate_layout(Rs, has_scalar_act, has_gate_act):
     return tables, c_out, n_gates
 
 
+def epilogue_layout(c_out, out_mode=None, gate_col=None, block=64):
+    """Column order in which a convolution computes its outputs when the evaluation-mode
+    batch norm and gate are applied as its rows are stored (ssc_conv_run_epilogue_f32): the
+    kernel works on blocks of `block` columns and a gate must sit in the block of the columns
+    it gates.  Each block holds a run of output columns in their own order (a multiple of 4,
+    so that a thread's four columns are four neighbours of the stored row), then the gates of
+    the fields that run touches (at most 16 in a block) -- a gate is computed once per block
+    that needs it, a gate no column reads not at all -- padded to the block size; the last
+    block to a multiple of 4.
+
+    out_mode / gate_col as in gate_layout() (None: no activation).  Returns CPU tensors
+    src[c] (column of the convolution's own output order, -1 for padding), mode[c] (0 copy,
+    1 scalar activation, 2 gated, 3 not stored), gate[c] (position of the gate of column c),
+    dest[c] (output column), all int32 with one entry per computed column, and
+    gate_run[2b], gate_run[2b+1]: first gate column and number of gates of block b."""
+    pad4 = lambda n: (n + 3) // 4 * 4  # noqa: E731
+    out_mode = [0] * c_out if out_mode is None else [int(v) for v in out_mode]
+    gate_col = [0] * c_out if gate_col is None else [int(v) for v in gate_col]
+    blocks, a = [], 0
+    while a < c_out:
+        b, gates = a, []
+        while b < c_out:
+            nb = min(b + 4, c_out)
+            g2 = list(gates)
+            for j in range(b, nb):
+                if out_mode[j] == 2 and gate_col[j] not in g2:
+                    g2.append(gate_col[j])
+            if pad4(nb - a) + pad4(len(g2)) > block or len(g2) > 16:
+                break
+            b, gates = nb, g2
+        if b == a:
+            raise ValueError("a block of %d columns cannot hold four outputs and their gates" % block)
+        blocks.append((a, b, gates))
+        a = b
+    src, mode, gate, dest, gate_run = [], [], [], [], []
+    for i, (a, b, gates) in enumerate(blocks):
+        base = len(src)
+        first_gate = base + pad4(b - a)
+        gate_run += [first_gate, len(gates)]
+        for j in range(a, b):
+            src.append(j)
+            mode.append(out_mode[j])
+            gate.append(first_gate + gates.index(gate_col[j]) if out_mode[j] == 2 else base + j - a)
+            dest.append(j)
+        end = base + (block if i + 1 < len(blocks) else pad4(b - a) + pad4(len(gates)))
+        for pos in range(base + b - a, end):
+            k = pos - first_gate
+            src.append(gates[k] if 0 <= k < len(gates) else -1)
+            mode.append(3)
+            gate.append(pos)
+            dest.append(0)
+    as_t = lambda v: torch.tensor(v, dtype=torch.int32)  # noqa: E731
+    return {"src": as_t(src), "mode": as_t(mode), "gate": as_t(gate), "dest": as_t(dest),
+            "gate_run": as_t(gate_run)}
+
+
 class BnActPlan:
     """What one call of the fused function needs besides tensors that carry gradients."""
 

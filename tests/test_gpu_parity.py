@@ -1603,3 +1603,93 @@ def test_point2voxel_one_call_gradients(mode, oracle, device):
         grads.append(x.grad.clone())
     assert p2v.last_path == "one call"
     assert torch.equal(grads[0], grads[1])
+
+
+EPILOGUE_CASES = [
+    # Rs of the activation, Cin, kernel, stride, pad, subm, indice_key
+    ([(10, 0), (6, 1), (4, 2), (2, 3)], 16, 3, 1, 1, False, None),    # 62 + 12 gates -> 80 columns
+    ([(10, 0), (6, 1), (4, 2), (2, 3)], 16, 3, 1, 1, True, "s0"),     # subm, cached rulebook
+    ([(32, 0), (32, 1), (32, 2)], 40, 3, 2, 1, False, None),          # 288 outputs, several blocks
+    ([(3, 0), (2, 1), (2, 2)], 5, 2, 2, 0, False, None),              # 19 outputs: scalar stores
+    ([(16, 0)], 8, 3, 1, 1, False, None),                             # scalars only, no gates
+]
+
+
+@pytest.mark.parametrize("case", EPILOGUE_CASES)
+def test_conv_epilogue_block_matches_oracle(case, oracle, device):
+    """fused.ConvBatchNormActivation in evaluation mode (ssc_conv_run_epilogue_f32: batch
+    norm constants and gate applied while the convolution stores its rows) against
+    oracle.bn_gate_fwd(oracle.conv_fwd(.)), and against the three layers run one after the
+    other on the GPU; in training mode the block is the three layers."""
+    from ss_conv import _ext
+    from ss_conv.fused import ConvBatchNormActivation
+    from ss_conv.sp_ops.conv import SparseConvolution
+    from ss_conv.sp_ops.tensor import SparseTensor
+    Rs, cin, k, s, p, subm, key = case
+    print("case", case, flush=True)
+    rng = np.random.default_rng(cin * 100 + k)
+    bn, act, Rs_bn = _bnact_modules(Rs, (torch.relu, torch.sigmoid), device, rng)
+    c_conv = sum(m * (2 * l + 1) for m, l in Rs_bn)
+    c_act = sum(m * (2 * l + 1) for m, l in Rs)
+    conv = SparseConvolution(3, cin, c_conv, k, s, p, bias=False, subm=subm, indice_key=key).to(device)
+    block = ConvBatchNormActivation(conv, bn, act).eval()
+    batch, grid, n = 2, 10, 500
+    idx = random_voxels(rng, batch, grid, n)
+    x_np = rng.normal(size=(n, cin)).astype(np.float32)
+    w_np = conv.weight.detach().cpu().numpy().reshape(-1, cin, c_conv)
+
+    def tensor():
+        return SparseTensor(torch.from_numpy(x_np).to(device), torch.from_numpy(idx).to(device),
+                            [grid] * 3, batch)
+
+    calls = {"epi": 0}
+    real = _ext._lib.ssc_conv_run_epilogue_f32
+
+    def counted(*a):
+        calls["epi"] += 1
+        return real(*a)
+
+    _ext._lib.ssc_conv_run_epilogue_f32 = counted
+    try:
+        with torch.no_grad():
+            st = tensor()
+            y1 = block(st)
+            if key is not None:   # second layer of the same key: the cached rulebook
+                st2 = tensor()
+                st2.indice_dict = y1.indice_dict
+                y2 = block(st2)
+                assert torch.equal(y1.features, y2.features)
+            torch.cuda.synchronize()
+    finally:
+        _ext._lib.ssc_conv_run_epilogue_f32 = real
+    assert calls["epi"] == (2 if key is not None else 1), calls
+    assert y1.features.shape[1] == c_act
+
+    r = oracle.rulebook(idx, batch, [grid] * 3, k, s, p, 1, subm)
+    o_idx, o_pairs, o_num = r[:3] if subm else oracle.canonicalize(*r)
+    z = oracle.conv_fwd(x_np, w_np, o_pairs, o_num, o_idx.shape[0])
+    sb, gb = act.biases()
+    as_np = lambda t: None if t is None else t.detach().cpu().numpy()  # noqa: E731
+    params = dict(weight=as_np(bn.weight), bias=as_np(bn.bias), scalar_bias=as_np(sb),
+                  gate_bias=as_np(gb))
+    running = (bn.running_mean.cpu().numpy().copy(), bn.running_var.cpu().numpy().copy())
+    want = oracle.bn_gate_fwd(z, Rs_bn, Rs, params, training=False, act_scalar="relu",
+                              act_gate="sigmoid" if gb is not None else None, running=running)
+    assert np.array_equal(y1.indices.cpu().numpy(), o_idx)
+    assert rel_l2(y1.features.cpu().numpy(), want) < REL_L2
+    # the three layers one after the other
+    with torch.no_grad():
+        sep = act(bn(conv(tensor())))
+    assert rel_l2(y1.features.cpu().numpy(), sep.features.cpu().numpy()) < 1e-6
+    # a change of the running statistics is seen by the next call
+    with torch.no_grad():
+        bn.running_var.mul_(1.5)
+        y3 = block(tensor())
+        sep = act(bn(conv(tensor())))
+    assert rel_l2(y3.features.cpu().numpy(), sep.features.cpu().numpy()) < 1e-6
+    # training mode: batch statistics, autograd -- the separate layers
+    block.train()
+    xt = torch.from_numpy(x_np).to(device).requires_grad_(True)
+    yt = block(SparseTensor(xt, torch.from_numpy(idx).to(device), [grid] * 3, batch))
+    yt.features.sum().backward()
+    assert xt.grad is not None and yt.features.shape[1] == c_act

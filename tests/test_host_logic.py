@@ -380,3 +380,38 @@ def test_layers_outside_the_native_layouts():
     assert not act._kernel_ok
     with pytest.raises(NotImplementedError):
         SparseConvolution(3, 4, 4, 3, transposed=True)
+
+
+def test_epilogue_layout_keeps_gates_with_their_columns():
+    """bnact.epilogue_layout: every output column appears once, in order inside its block;
+    a gated column's gate sits in the same block of 64; data runs start at multiples of 4;
+    gates that no column reads are not computed; sizes are multiples of 4."""
+    from ss_conv import bnact
+    cases = [[(10, 0), (6, 1), (4, 2), (2, 3)], [(32, 0), (32, 1), (32, 2), (32, 3)],
+             [(3, 0), (2, 1), (2, 2)], [(16, 0)], [(0, 0), (20, 3)], [(4, 0), (3, 0), (5, 1)]]
+    for Rs in cases:
+        tables, c_out, n_gates = bnact.gate_layout(Rs, True, True)
+        lay = bnact.epilogue_layout(c_out, tables["out_mode"].tolist(), tables["gate_col"].tolist())
+        src, mode, gate, dest = (lay[k].tolist() for k in ("src", "mode", "gate", "dest"))
+        n = len(src)
+        assert n % 4 == 0 and len(mode) == len(gate) == len(dest) == n
+        stored = [(dest[c], c) for c in range(n) if mode[c] != 3]
+        assert sorted(d for d, _ in stored) == list(range(c_out))
+        for d, c in stored:
+            assert src[c] == d and mode[c] == int(tables["out_mode"][d])
+            if c % 4 == 0:
+                assert d % 4 == 0
+            if mode[c] == 2:
+                g = gate[c]
+                first, count = lay["gate_run"].tolist()[2 * (c // 64):2 * (c // 64) + 2]
+                assert g // 64 == c // 64 and mode[g] == 3 and count <= 16
+                assert first <= g < first + count and (first + count - 1) // 64 == c // 64
+                assert src[g] == int(tables["gate_col"][d])
+        used = {int(tables["gate_col"][d]) for d in range(c_out) if int(tables["out_mode"][d]) == 2}
+        computed = {src[c] for c in range(n) if mode[c] == 3 and src[c] >= 0}
+        assert computed == used
+    # no activation: identity order, padded to a multiple of 4
+    lay = bnact.epilogue_layout(10)
+    assert lay["src"].tolist() == list(range(10)) + [-1, -1]
+    assert lay["mode"].tolist() == [0] * 10 + [3, 3]
+    assert lay["gate_run"].tolist() == [12, 0]
