@@ -205,6 +205,9 @@ def _geometry(batch_size, out_shape, ksize, stride, padding, dilation, subm, tra
 # possible number of them is at most this large (a result that fills less than a quarter of
 # a buffer of more than 16 MiB is copied out of it).
 _ROWS_AHEAD_BYTES = 512 << 20
+# largest plan / plan scratch allocated for the bound on the number of outputs, before the
+# real number has arrived
+_PLAN_AHEAD_BYTES = 256 << 20
 
 
 class RulebookMeta(object):
@@ -235,7 +238,8 @@ def rulebook_meta(indice_pairs):
 class _PendingRulebook(object):
     """A rulebook between ssc_rulebook_begin and ssc_rulebook_finish: everything whose size
     does not depend on the number of outputs is queued, the host has not waited yet."""
-    __slots__ = ("indices", "n", "geometry", "ws", "pairs", "num", "out_buf", "subm", "stream")
+    __slots__ = ("indices", "n", "geometry", "ws", "pairs", "num", "out_buf", "subm", "stream",
+                 "bound")
 
 
 def _rulebook_begin(indices, batch_size, out_spatial_shape, kernel_size, stride, padding, dilation,
@@ -270,8 +274,10 @@ def _rulebook_begin(indices, batch_size, out_spatial_shape, kernel_size, stride,
     # the same launch as the pairs and the result is a slice of that buffer; otherwise by a
     # launch of their own once the number is known.
     r.out_buf = None
+    r.bound = n if subm else 0  # most output rows there can be (0: not known)
     if not subm and n > 0:
         bound = _lib.ssc_rulebook_out_bound(gref, n)
+        r.bound = max(int(bound), 0)
         if 0 < bound * 16 <= _ROWS_AHEAD_BYTES:
             r.out_buf = torch.empty((bound, 4), dtype=torch.int32, device=dev)
     _check(_lib.ssc_rulebook_begin(_ptr(indices), n, gref, r.ws.data_ptr(), r.ws.numel(),
@@ -280,31 +286,42 @@ def _rulebook_begin(indices, batch_size, out_spatial_shape, kernel_size, stride,
     return r
 
 
-def _rulebook_finish(r):
-    """Wait for the number of outputs; returns [outids, pairs, num]."""
-    gref = ctypes.byref(r.geometry)
+def _rulebook_wait(r):
+    """Wait for the number of outputs: (n_out, whether the input rows came in key order)."""
     n_out = _i32(0)
     in_order = _i32(0)
-    _check(_lib.ssc_rulebook_finish(gref, r.n, ctypes.byref(n_out), ctypes.byref(in_order)))
+    _check(_lib.ssc_rulebook_finish(ctypes.byref(r.geometry), r.n, ctypes.byref(n_out),
+                                    ctypes.byref(in_order)))
+    return n_out.value, bool(in_order.value)
+
+
+def _rulebook_result(r, n_out, in_order):
+    """[outids, pairs, num] of a rulebook whose number of outputs has arrived."""
     if r.subm:
         outids = r.indices
     elif r.out_buf is not None:
-        outids = r.out_buf[:n_out.value]
-        if r.out_buf.size(0) > 4 * max(n_out.value, 1) and r.out_buf.numel() * 4 > (16 << 20):
+        outids = r.out_buf[:n_out]
+        if r.out_buf.size(0) > 4 * max(n_out, 1) and r.out_buf.numel() * 4 > (16 << 20):
             outids = outids.clone()  # do not keep a large, mostly unused buffer alive
     else:
         # a geometry may leave no output at all (every candidate clipped): the library still
         # wants a valid pointer, so at least one row is allocated and the result is a slice
-        out_buf = torch.empty((max(n_out.value, 1), 4), dtype=torch.int32, device=r.pairs.device)
-        outids = out_buf[:n_out.value]
-        _check(_lib.ssc_rulebook_rows(gref, r.n, r.ws.data_ptr(), r.ws.numel(), out_buf.data_ptr(),
-                                      r.stream))
+        out_buf = torch.empty((max(n_out, 1), 4), dtype=torch.int32, device=r.pairs.device)
+        outids = out_buf[:n_out]
+        _check(_lib.ssc_rulebook_rows(ctypes.byref(r.geometry), r.n, r.ws.data_ptr(), r.ws.numel(),
+                                      out_buf.data_ptr(), r.stream))
     # Pairs of an offset always ascend in the input rows, and in the output rows too when
     # the input rows came in key order: the convolution may then skip its order check
     # (the first flag serves a call that accumulates into output rows, the second one
     # with `inverse`, which accumulates into input rows).
-    r.pairs._ssc_meta = RulebookMeta(r.pairs._version, (bool(in_order.value), True))
+    r.pairs._ssc_meta = RulebookMeta(r.pairs._version, (in_order, True))
     return [outids, r.pairs, r.num]
+
+
+def _rulebook_finish(r):
+    """Wait for the number of outputs; returns [outids, pairs, num]."""
+    n_out, in_order = _rulebook_wait(r)
+    return _rulebook_result(r, n_out, in_order)
 
 
 def get_indice_pairs_3d(indices, batch_size, out_spatial_shape, spatial_shape, kernel_size, stride,
@@ -363,15 +380,15 @@ def prepack_filters(filters, c_in, c_out):
     """Queue the packing of `filters` ([*kernel_size, Cin, Cout], float32 or half, on the GPU)
     now and keep the result on the tensor, so that a convolution called with this tensor
     later finds it: a layer that knows its filters before its rulebook packs them while the
-    rulebook is still being built."""
+    rulebook is still being built.  Returns the packed buffer (None when nothing was done)."""
     if not filters.is_cuda or filters.dtype not in _ENTRIES:
-        return
+        return None
     owner = filters
     filters, fs_k, fs_ci, fs_co = _filter_strides(filters, c_in, c_out)
     K = 1
     for d in filters.shape[:-2]:
         K *= d
-    _packed_filters(owner, filters, (fs_k, fs_ci, fs_co), K, c_in, c_out, _stream(filters))
+    return _packed_filters(owner, filters, (fs_k, fs_ci, fs_co), K, c_in, c_out, _stream(filters))
 
 
 def _plan_of(meta, pairs, num, K, c_in, c_out, elem_bytes, n_in, n_out, inverse, dev, stream):
@@ -491,10 +508,31 @@ def rulebook_conv(features, filters, indices, batch_size, out_spatial_shape, ker
     s = r.stream
     packed = _packed_filters(owner, filters, (fs_k, fs_ci, fs_co), K, c_in, c_out, s)
     eb = features.element_size()
-    outids, pairs, num = _rulebook_finish(r)
-    n_out = outids.size(0)
-    plan = _plan_of(pairs._ssc_meta, pairs, num, K, c_in, c_out, eb, n_in, n_out, False, dev, s)
+    # Between the host's wake-up and the first launch of the plan the GPU has nothing to do:
+    # whatever can be prepared is prepared before the wait.  With a bound on the number of
+    # outputs at hand (and buffers of that size within reason) that includes the buffers of
+    # the plan, which is then queued straight after the wait; tensors and bookkeeping follow
+    # when the kernel is on its way.
+    plan = scratch = None
+    if 0 < r.bound <= 8 * max(n_in, 1) * K:
+        plan_bytes = _lib.ssc_conv_plan_bytes(r.bound, K, c_in, c_out, n_in)
+        scratch_bytes = _lib.ssc_conv_plan_scratch_bytes(r.bound, K, c_in, c_out, n_in)
+        if plan_bytes <= _PLAN_AHEAD_BYTES and scratch_bytes <= _PLAN_AHEAD_BYTES:
+            plan = _workspace(plan_bytes, dev)
+            scratch = _workspace(scratch_bytes, dev)
+    n_out, in_order = _rulebook_wait(r)
+    if plan is None or n_out == 0:
+        outids, pairs, num = _rulebook_result(r, n_out, in_order)
+        plan = _plan_of(pairs._ssc_meta, pairs, num, K, c_in, c_out, eb, n_in, n_out, False, dev, s)
+        out = _run_planned(features, n_in, c_in, packed, plan, n_in, K, c_out, n_out, s, epilogue)
+        return out, outids, pairs, num
+    _check(_lib.ssc_conv_plan_build(r.pairs.data_ptr(), n_in, r.num.data_ptr(), K, 0,
+                                    2 if in_order else 0, n_in, n_out, c_in, c_out, eb,
+                                    plan.data_ptr(), plan.numel(), scratch.data_ptr(),
+                                    scratch.numel(), s))
     out = _run_planned(features, n_in, c_in, packed, plan, n_in, K, c_out, n_out, s, epilogue)
+    outids, pairs, num = _rulebook_result(r, n_out, in_order)
+    pairs._ssc_meta.plans[(False, c_in, c_out, eb, n_in, n_out)] = plan
     return out, outids, pairs, num
 
 
