@@ -323,6 +323,17 @@ int ssc_kernel_combine_f32(const float *weight, const float *basis,
                            int32_t kernel_volume, int32_t c_in, int32_t c_out,
                            float *out /* [K,c_in,c_out] */, ssc_stream_t stream);
 
+/* The same synthesis with the filters also written in the convolution kernel's packed order
+ * (what ssc_conv_pack_filters_f32 makes of `out` read as [K, Cin, Cout]; `packed` of
+ * ssc_conv_packed_bytes(kernel_volume, c_in, c_out) bytes): a layer that synthesises its
+ * kernel on every training forward (ss_conv/convolution.py:56) saves the packing launch. */
+int ssc_kernel_combine_packed_f32(const float *weight, const float *basis,
+                                  const int32_t *chan_out, const int32_t *chan_in,
+                                  const int32_t *blocks, int32_t n_irreps_in,
+                                  int32_t kernel_volume, int32_t c_in, int32_t c_out,
+                                  float *out /* [K, c_in, c_out] */, void *packed,
+                                  size_t packed_bytes, ssc_stream_t stream);
+
 /* ------------------------------------------------------------------------
  * Rulebook pooling.  Replace indiceMaxPool<float> (src/pool/indice_maxpool.h:15-50,
  * kernels src/pool/indice_maxpool_cuda_functor.cu:22-156), indiceAvgPool<float>

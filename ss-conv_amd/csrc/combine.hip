@@ -3,6 +3,7 @@
 // One thread per output element; the per-channel descriptor tables replace the
 // reference's loop over irrep pairs, its einsum, both concatenations and the
 // permute.  The sum over beta runs in ascending order.
+#include "combine_element.h"
 #include "ssc_common.h"
 
 namespace ssc {
@@ -19,16 +20,7 @@ __global__ void __launch_bounds__(256)
   int64_t r = idx / cout;
   int ci = (int)(r % cin);
   int k = (int)(r / cin);
-  int i = chan_out[co * 3], u = chan_out[co * 3 + 1], a = chan_out[co * 3 + 2];
-  int j = chan_in[ci * 3], v = chan_in[ci * 3 + 1], b = chan_in[ci * 3 + 2];
-  const int32_t *blk = blocks + (i * n_j + j) * 6;
-  int w_off = blk[0], b_off = blk[1], n_beta = blk[2], m_in = blk[3], d_out = blk[4],
-      d_in = blk[5];
-  const float *w = weight + w_off + (u * m_in + v) * n_beta;
-  const float *bs = basis + b_off + ((int64_t)a * d_in + b) * K + k;
-  int64_t beta_stride = (int64_t)d_out * d_in * K;
-  float acc = 0.f;
-  for (int t = 0; t < n_beta; ++t) acc += w[t] * bs[t * beta_stride];
+  const float acc = combine_element(weight, basis, chan_out, chan_in, blocks, n_j, K, k, ci, co);
   out[idx] = acc;
 }
 

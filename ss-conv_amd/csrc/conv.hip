@@ -15,6 +15,7 @@
 // pairs are sorted (re-order them if not); split the output rows over the
 // workgroups by work and cut the ranges into tiles; build the row-block schedule;
 // launch the persistent kernel.
+#include "combine_element.h"
 #include "ssc_common.h"
 
 #include <type_traits>
@@ -63,19 +64,18 @@ struct PackArgs {
   int ns;  // MFMA steps per chunk (float filters; half filters always use whole chunks)
 };
 
-// Element idx of the packed filters.
+// Offset k, input channel ci and output channel co of element idx of the packed filters
+// (ci >= cin or co >= cout: a padding element).
 template <typename IO>
-__device__ __forceinline__ void pack_filter_element(const PackArgs &a, int64_t idx) {
-  const IO *__restrict__ w = static_cast<const IO *>(a.w);
-  const int64_t fs_k = a.fs_k, fs_ci = a.fs_ci, fs_co = a.fs_co;
-  const int cin = a.cin, cout = a.cout, ncb = a.ncb, nch = a.nch;
-  void *packed_out = a.packed_out;
+__device__ __forceinline__ void pack_decode(const PackArgs &a, int64_t idx, int &k, int &ci,
+                                            int &co) {
+  const int cin = a.cin, ncb = a.ncb, nch = a.nch;
   int64_t r = idx >> 10;
   int cc = r % nch;
   r /= nch;
   int cb = r % ncb;
-  int k = (int)(r / ncb);
-  int lane, ci;
+  k = (int)(r / ncb);
+  int lane;
   if constexpr (sizeof(IO) == 2) {
     const int j = idx & 7, q = (idx >> 9) & 1;
     lane = (idx >> 3) & 63;
@@ -94,10 +94,39 @@ __device__ __forceinline__ void pack_filter_element(const PackArgs &a, int64_t i
     }
     ci = cl < 0 ? cin : cc * (4 * a.ns) + cl;
   }
-  int co = cb * 16 + (lane & 15);
+  co = cb * 16 + (lane & 15);
+}
+
+// Element idx of the packed filters.
+template <typename IO>
+__device__ __forceinline__ void pack_filter_element(const PackArgs &a, int64_t idx) {
+  const IO *__restrict__ w = static_cast<const IO *>(a.w);
+  int k, ci, co;
+  pack_decode<IO>(a, idx, k, ci, co);
   IO v = (IO)0.f;
-  if (ci < cin && co < cout) v = w[k * fs_k + ci * fs_ci + co * fs_co];
-  static_cast<IO *>(packed_out)[idx] = v;
+  if (ci < a.cin && co < a.cout) v = w[k * a.fs_k + ci * a.fs_ci + co * a.fs_co];
+  static_cast<IO *>(a.packed_out)[idx] = v;
+}
+
+// Synthesis of the dense float kernel and its packing in one launch: one thread per packed
+// element computes the element (combine_element), stores it at its place in the packed
+// filters and in the dense [K, Cin, Cout] array (every dense element has exactly one packed
+// place; padding places get zero).
+__global__ void __launch_bounds__(256)
+    combine_pack_kernel(PackArgs a, const float *__restrict__ weight,
+                        const float *__restrict__ basis, const int32_t *__restrict__ chan_out,
+                        const int32_t *__restrict__ chan_in, const int32_t *__restrict__ blocks,
+                        int n_j, float *__restrict__ dense) {
+  int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= (int64_t)a.K * a.ncb * a.nch * 1024) return;
+  int k, ci, co;
+  pack_decode<float>(a, idx, k, ci, co);
+  float v = 0.f;
+  if (ci < a.cin && co < a.cout) {
+    v = combine_element(weight, basis, chan_out, chan_in, blocks, n_j, a.K, k, ci, co);
+    dense[((int64_t)k * a.cin + ci) * a.cout + co] = v;
+  }
+  static_cast<float *>(a.packed_out)[idx] = v;
 }
 
 template <typename IO>
@@ -2016,6 +2045,29 @@ int ssc_conv_plan_build(const int32_t *pairs, int64_t pair_stride, const int32_t
   return conv_plan_build<float>(p, w, pairs, pair_stride, pair_num, K, inverse,
                                 (flags & SSC_CONV_PAIRS_CANONICAL) != 0, c_in, n_out, elem_bytes,
                                 nullptr, (hipStream_t)stream);
+}
+
+int ssc_kernel_combine_packed_f32(const float *weight, const float *basis,
+                                  const int32_t *chan_out, const int32_t *chan_in,
+                                  const int32_t *blocks, int32_t n_irreps_in,
+                                  int32_t kernel_volume, int32_t c_in, int32_t c_out, float *out,
+                                  void *packed, size_t packed_bytes, ssc_stream_t stream) {
+  const int K = kernel_volume;
+  int rc = conv_check_sizes(K, c_in, c_out, 0, 0, 0);
+  if (rc != SSC_OK) return rc;
+  SSC_CHECK(weight && basis && chan_out && chan_in && blocks && out && packed, SSC_EINVAL,
+            "NULL pointer argument");
+  SSC_CHECK(n_irreps_in >= 1, SSC_EINVAL, "sizes must be positive");
+  const ConvPlan p = make_plan(0, 1, K, c_in, c_out, 0, 4);
+  SSC_CHECK(packed_bytes >= conv_packed_bytes(p, K), SSC_EWORKSPACE,
+            "buffer of the packed filters too small");
+  const PackArgs pk = {nullptr, 0, 0, 0, K, c_in, c_out, p.ncb, p.nch, packed, p.ns};
+  const int64_t n = (int64_t)K * p.ncb * p.nch * 1024;
+  hipLaunchKernelGGL(combine_pack_kernel, dim3((unsigned)ceil_div(n, 256)), dim3(256), 0,
+                     (hipStream_t)stream, pk, weight, basis, chan_out, chan_in, blocks,
+                     (int)n_irreps_in, out);
+  SSC_LAUNCH_CHECK("combine_pack");
+  return SSC_OK;
 }
 
 int ssc_conv_pack_filters_f32(const float *filters, int64_t fs_k, int64_t fs_ci, int64_t fs_co,

@@ -89,6 +89,8 @@ _SIGNATURES = {
                                              ctypes.POINTER(_i32)]),
     "ssc_kernel_combine_f32": (ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32,
                                               _vp, _vp]),
+    "ssc_kernel_combine_packed_f32": (ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32,
+                                                     _i32, _vp, _vp, _sz, _vp]),
     "ssc_pool_workspace_bytes": (_sz, [_i64, _i32]),
     "ssc_pool_max_f32": (ctypes.c_int, [_vp, _i32, _vp, _i64, _vp, _i32, _vp, _i64, _vp, _sz,
                                         _vp]),
@@ -944,15 +946,33 @@ def three_interpolate_fp(c, m, n, feats, idx, weight, out):
 
 # ---- entry points without a counterpart in the reference's binding ---------------------
 def kernel_combine(weight, basis, chan_out, chan_in, blocks, n_irreps_in, kernel_volume, c_in,
-                   c_out):
+                   c_out, packed=False):
     """Dense kernel [K, Cin, Cout] from the flat weight vector and the stacked
-    basis (ss_conv/utils/kernel.py:267-299 fused with convolution.py:56)."""
+    basis (ss_conv/utils/kernel.py:267-299 fused with convolution.py:56).  With `packed`
+    the same launch also writes the filters in the convolution kernel's packed order:
+    returns (dense, packed buffer)."""
     _need_gpu(weight, basis, chan_out, chan_in, blocks)
     out = torch.empty((kernel_volume, c_in, c_out), dtype=torch.float32, device=weight.device)
-    _check(_lib.ssc_kernel_combine_f32(_ptr(weight), _ptr(basis), _ptr(chan_out), _ptr(chan_in),
-                                       _ptr(blocks), int(n_irreps_in), int(kernel_volume),
-                                       int(c_in), int(c_out), _ptr(out), _stream(weight)))
-    return out
+    args = (_ptr(weight), _ptr(basis), _ptr(chan_out), _ptr(chan_in), _ptr(blocks),
+            int(n_irreps_in), int(kernel_volume), int(c_in), int(c_out), _ptr(out))
+    if not packed:
+        _check(_lib.ssc_kernel_combine_f32(*args, _stream(weight)))
+        return out
+    buf = _workspace(_lib.ssc_conv_packed_bytes(int(kernel_volume), int(c_in), int(c_out)),
+                     weight.device)
+    _check(_lib.ssc_kernel_combine_packed_f32(*args, buf.data_ptr(), buf.numel(), _stream(weight)))
+    return out, buf
+
+
+def attach_packed(filters, c_in, c_out, packed):
+    """Tell the convolution that `packed` holds `filters` ([*kernel_size, Cin, Cout], float32)
+    in its packed order, as prepack_filters would have left it."""
+    base, fs_k, fs_ci, fs_co = _filter_strides(filters, c_in, c_out)
+    K = 1
+    for d in base.shape[:-2]:
+        K *= d
+    filters._ssc_packed = (filters._version,
+                           {(base.data_ptr(), (fs_k, fs_ci, fs_co), K, c_in, c_out): packed})
 
 
 def voxel_coords(points, batch_ids, half_extent, unit):

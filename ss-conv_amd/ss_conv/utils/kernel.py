@@ -128,12 +128,15 @@ class _Combine(torch.autograd.Function):
     fixed basis, block by block (the blocks are small: torch einsum)."""
 
     @staticmethod
-    def forward(ctx, weight, module):
+    def forward(ctx, weight, module, pack):
         basis, chan_out, chan_in, blocks, _ = module._tables
         ctx.module = module
-        return _ext.kernel_combine(weight.detach().float().contiguous(), basis, chan_out, chan_in,
-                                   blocks, len(module.multiplicities_in), module.size ** 3,
-                                   module.n_in, module.n_out)
+        out = _ext.kernel_combine(weight.detach().float().contiguous(), basis, chan_out, chan_in,
+                                  blocks, len(module.multiplicities_in), module.size ** 3,
+                                  module.n_in, module.n_out, packed=pack)
+        if pack:
+            out, module.packed = out
+        return out
 
     @staticmethod
     def backward(ctx, grad):  # grad: [K, Cin, Cout]
@@ -153,7 +156,7 @@ class _Combine(torch.autograd.Function):
                     grads.append(torch.einsum("kvbua,nabk->uvn", g, basis).reshape(-1))
                 i_off += mj * dj
             o_off += mi * di
-        return torch.cat(grads), None
+        return torch.cat(grads), None, None
 
 
 class SE3Kernel(torch.nn.Module):
@@ -203,6 +206,7 @@ class SE3Kernel(torch.nn.Module):
                                      basis.type(torch.get_default_dtype()))
         self.weight = torch.nn.Parameter(torch.cat(weights))
         self._tables = None  # device tables for the native contraction, built on first use
+        self.packed = None   # packed filters left by the last combination(pack=True)
 
     def __repr__(self):
         return "{name} ({Rs_in} -> {Rs_out}, size={size})".format(
@@ -241,16 +245,19 @@ class SE3Kernel(torch.nn.Module):
         self._tables = (torch.cat(pieces).contiguous(), as_i32(chan_out), as_i32(chan_in),
                         as_i32(blocks), device)
 
-    def combination(self, weight):
+    def combination(self, weight, pack=False):
         """[Cout, Cin, k, k, k] view of the natively contracted [K, Cin, Cout] kernel
-        (reference: kernel.py:267-299).  Differentiable with respect to `weight`."""
+        (reference: kernel.py:267-299).  Differentiable with respect to `weight`.
+        With `pack` the same launch leaves the filters in the convolution kernel's packed
+        order in `self.packed` (for _ext.attach_packed)."""
         if not weight.is_cuda:
             raise RuntimeError("SE3Kernel runs on the GPU only: move the module to a cuda device")
         if self._tables is None or self._tables[4] != weight.device:
             self._build_tables(weight.device)
-        dense = _Combine.apply(weight, self)
+        self.packed = None
+        dense = _Combine.apply(weight, self, bool(pack))
         k = self.size
         return dense.permute(2, 1, 0).reshape(self.n_out, self.n_in, k, k, k)
 
-    def forward(self):  # pylint: disable=W
-        return self.combination(self.weight)
+    def forward(self, pack=False):  # pylint: disable=W
+        return self.combination(self.weight, pack)

@@ -657,6 +657,16 @@ def test_kernel_combine_matches_einsum(oracle, device):
                              ker.dims_out, ker.multiplicities_in, ker.dims_in, size)
         assert got.shape == ref.shape
         assert rel_l2(got, ref) < 1e-6
+        # synthesis and packing in one launch: the same dense kernel, and the packed filters
+        # that ssc_conv_pack_filters_f32 makes of it, bit for bit
+        from ss_conv import _ext
+        both = ker(pack=True).detach()
+        assert np.array_equal(both.cpu().numpy(), got)
+        fused = ker.packed
+        w = both.permute(2, 3, 4, 1, 0)
+        packed = _ext.prepack_filters(w, ker.n_in, ker.n_out)
+        assert fused is not None and fused.numel() == packed.numel()
+        assert torch.equal(fused, packed)
 
 
 def test_convolution_layer_end_to_end(oracle, device):
