@@ -177,6 +177,12 @@ def ops_table(torch, _ext, synth, dev, seed):
     mp = MaxPool(2, 2)
     ms, _ = timed(lambda: mp(st))
     report("MaxPool module (rulebook + kernel)", ms, nbytes + 16 * (n_in + n_out), "incl. rulebook")
+    xh = x.half()
+    hbytes = 2 * C * (n_in + n_out) + 8 * P
+    ms, _ = timed(lambda: _ext.indice_maxpool_half(xh, p_pairs, p_num, n_out))
+    report("max pool k2 s2, half rows (kernel)", ms, hbytes)
+    ms, _ = timed(lambda: _ext.indice_avgpool_half(xh, p_pairs, p_num, n_out, rf))
+    report("avg pool k2 s2, half rows (kernel)", ms, hbytes, "a rounding after every operation")
 
     # global pools: 32 segments over the pooled rows, 512 channels
     C = 512
@@ -230,6 +236,32 @@ def ops_table(torch, _ext, synth, dev, seed):
             bnact.usable = keep
         report("same layers as torch ops, training", ms, 4 * n_rows * fwd_cols,
                "same algorithmic bytes")
+    # the whole block conv -> bn -> activation on the cfg2 geometry in evaluation mode: one
+    # kernel (batch norm constants and gate applied while the rows are stored) against the
+    # convolution followed by the fused batch norm + activation pass
+    from ss_conv.fused import ConvBatchNormActivation
+    from ss_conv.sp_ops.conv import SparseConvolution
+    cfg = synth.CONFIGS["cfg2"]
+    pts2, _, ids2 = synth.config_clouds("cfg2", seed)
+    idx2 = torch.from_numpy(synth.voxel_indices(pts2, ids2, cfg["grid"])).to(dev)
+    conv = SparseConvolution(3, 64, c_in, 3, 1, 1, bias=False, indice_key="b").to(dev)
+    block = ConvBatchNormActivation(conv, bn, act).eval()
+    f2 = torch.randn(idx2.shape[0], 64, device=dev)
+    with torch.no_grad():
+        st2 = SparseTensor(f2, idx2, [cfg["grid"]] * 3, cfg["batch"])
+        y2 = block(st2)  # builds the rulebook, kept under the key
+
+        def again(fn):
+            t = SparseTensor(f2, idx2, [cfg["grid"]] * 3, cfg["batch"])
+            t.indice_dict = y2.indice_dict
+            return fn(t)
+        ms_one, _ = timed(lambda: again(block), n=10)
+        ms_sep, _ = timed(lambda: again(lambda t: fused.eval()(conv(t))), n=10)
+        fused.train()
+    rows.append("%-44s %8.3f ms   (cached rulebook and plan, %d rows, 64 -> %d -> %d ch)"
+                % ("conv+bn+act block, evaluation, one kernel", ms_one, y2.features.shape[0], c_in,
+                   c_out))
+    rows.append("%-44s %8.3f ms" % ("  the same as conv, then bn+act pass", ms_sep))
     xg = x.clone().requires_grad_(True)
     dy = torch.randn(n_rows, c_out, device=dev)
 
