@@ -1703,3 +1703,87 @@ def test_conv_epilogue_block_matches_oracle(case, oracle, device):
     yt = block(SparseTensor(xt, torch.from_numpy(idx).to(device), [grid] * 3, batch))
     yt.features.sum().backward()
     assert xt.grad is not None and yt.features.shape[1] == c_act
+
+
+def test_conv_epilogue_block_other_layers(oracle, device):
+    """The evaluation-mode block with tanh activations (the kernel's general form), with a
+    batch norm or an activation only, and the cases that stay with the separate layers (a
+    convolution with bias, half-precision rows, an empty input): always the result of the
+    three layers run one after the other."""
+    from ss_conv import _ext
+    from ss_conv.activation import Activation
+    from ss_conv.batchnorm import BatchNorm
+    from ss_conv.fused import ConvBatchNormActivation
+    from ss_conv.sp_ops.conv import SparseConvolution
+    from ss_conv.sp_ops.tensor import SparseTensor
+    rng = np.random.default_rng(5)
+    Rs = [(6, 0), (5, 1), (3, 2)]
+    batch, grid, n, cin = 2, 9, 400, 12
+    idx = torch.from_numpy(random_voxels(rng, batch, grid, n)).to(device)
+    x = torch.from_numpy(rng.normal(size=(n, cin)).astype(np.float32)).to(device)
+
+    def tensor(feats=x, rows=idx):
+        return SparseTensor(feats, rows, [grid] * 3, batch)
+
+    calls = {"epi": 0}
+    real = _ext._lib.ssc_conv_run_epilogue_f32
+
+    def counted(*a):
+        calls["epi"] += 1
+        return real(*a)
+
+    def check(block, expect_kernel, make=tensor, tol=1e-6):
+        before = calls["epi"]
+        with torch.no_grad():
+            got = block(make()).features
+            y = block.conv(make())
+            if block.bn is not None:
+                y = block.bn(y)
+            if block.activation is not None:
+                y = block.activation(y)
+        assert calls["epi"] - before == (1 if expect_kernel else 0)
+        assert got.shape == y.features.shape
+        if got.numel():
+            assert rel_l2(got.float().cpu().numpy(), y.features.float().cpu().numpy()) < tol
+
+    _ext._lib.ssc_conv_run_epilogue_f32 = counted
+    try:
+        bn, act, Rs_bn = _bnact_modules(Rs, (torch.tanh, torch.tanh), device, rng)
+        c_conv = bn.num_channels
+        conv = SparseConvolution(3, cin, c_conv, 3, 1, 1, bias=False).to(device)
+        check(ConvBatchNormActivation(conv, bn, act).eval(), True)
+        # oracle for the tanh block
+        block = ConvBatchNormActivation(conv, bn, act).eval()
+        with torch.no_grad():
+            out = block(tensor())
+        r = oracle.rulebook(idx.cpu().numpy(), batch, [grid] * 3, 3, 1, 1)
+        o_idx, o_pairs, o_num = oracle.canonicalize(*r)
+        z = oracle.conv_fwd(x.cpu().numpy(), conv.weight.detach().cpu().numpy().reshape(27, cin, c_conv),
+                            o_pairs, o_num, o_idx.shape[0])
+        sb, gb = act.biases()
+        as_np = lambda t: None if t is None else t.detach().cpu().numpy()  # noqa: E731
+        want = oracle.bn_gate_fwd(z, Rs_bn, Rs, dict(weight=as_np(bn.weight), bias=as_np(bn.bias),
+                                                     scalar_bias=as_np(sb), gate_bias=as_np(gb)),
+                                  training=False, act_scalar="tanh", act_gate="tanh",
+                                  running=(as_np(bn.running_mean), as_np(bn.running_var)))
+        assert rel_l2(out.features.cpu().numpy(), want) < REL_L2
+        # batch norm only, activation only (no biases), relu scalars without gate activation
+        check(ConvBatchNormActivation(conv, bn, None).eval(), True)
+        check(ConvBatchNormActivation(conv, None, Activation(Rs, (torch.relu, torch.sigmoid),
+                                                             bias=False).to(device)).eval(), True)
+        conv2 = SparseConvolution(3, cin, sum(m * (2 * l + 1) for m, l in Rs), 3, 1, 1,
+                                  bias=False).to(device)
+        check(ConvBatchNormActivation(conv2, BatchNorm(Rs).to(device),
+                                      Activation(Rs, (torch.relu, None)).to(device)).eval(), True)
+        # not for the kernel: bias, half rows, no rows, nothing to apply
+        biased = SparseConvolution(3, cin, c_conv, 3, 1, 1, bias=True).to(device)
+        check(ConvBatchNormActivation(biased, bn, act).eval(), False)
+        check(ConvBatchNormActivation(conv.half(), None, Activation(Rs, (torch.relu, torch.sigmoid),
+                                                                    bias=False).to(device)).eval(),
+              False, make=lambda: tensor(x.half()), tol=2e-3)
+        conv.float()
+        check(ConvBatchNormActivation(conv, bn, act).eval(), False,
+              make=lambda: tensor(x[:0], idx[:0]))
+        check(ConvBatchNormActivation(conv, None, None).eval(), False)
+    finally:
+        _ext._lib.ssc_conv_run_epilogue_f32 = real
