@@ -27,8 +27,7 @@ FP32_MFMA_PEAK_TFLOPS = 157.3  # MI355X dense fp32 matrix peak
 # HBM bytes per launch of the convolution kernel for every workload this script offers, from
 # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs scaled by a copy kernel of known size (the
 # summaries profiles/conv_fwd_<workload>_hbm_traffic.md give commands and counter values).
-MEASURED_TRAFFIC_BYTES = {"cfg1": 3029773, "cfg2": 345628507, "cfg3": 218923200,
-                          "cfg5": 96942593172}
+MEASURED_TRAFFIC_BYTES = {"cfg1": 3019427, "cfg2": 345657650, "cfg3": 218237827, "cfg5": 56163851226}
 
 
 def parse_args():
