@@ -602,6 +602,23 @@ int ssc_three_nn_grid(int32_t n, int32_t m, const float *unknown /* [n,4] */,
                       const float unit[3], float *dist2 /* [n,3] */, int32_t *idx /* [n,3] */,
                       void *workspace, size_t workspace_bytes, ssc_stream_t stream);
 
+/* Voxel2Point.forward with points (ss_conv/sp_ops/voxelize.py:131-160) as one call: the
+ * voxel centres ((index * unit - 0.5 extent) + 0.5 unit, as the reference rounds them), the
+ * three nearest centres of every point among the voxels of its batch element (the search of
+ * ssc_three_nn_grid: same indices and ties as ssc_three_nn), the inverse-distance weights
+ * 1 / (sqrt(d2) + 1e-8) normalised to sum 1, and the interpolation of ssc_three_interp_f32.
+ * points [n,3] with batch_ids [n] (int64); voxel_indices [m,4] (b, x, y, z), distinct, m >= 1;
+ * dims: cells per axis of the search grid (at least the largest index + 1).  Returns
+ * out [n,channels] and, for the backward pass (ssc_three_interp_bwd_f32), idx [n,3] and
+ * weight [n,3]. */
+size_t ssc_v2p_workspace_bytes(int32_t n, int32_t m, int32_t batch_size, const int32_t dims[3]);
+int ssc_v2p_interpolate_f32(const float *points, const int64_t *batch_ids, int32_t n,
+                            const int32_t *voxel_indices, const float *voxel_feats, int32_t m,
+                            int32_t channels, int32_t batch_size, const int32_t dims[3],
+                            const float unit[3], const float extent[3], float *out, int32_t *idx,
+                            float *weight, void *workspace, size_t workspace_bytes,
+                            ssc_stream_t stream);
+
 int ssc_three_interp_f32(int32_t c, int32_t m, int32_t n, const float *feats /* [m,c] */,
                          const int32_t *idx /* [n,3] */, const float *weight /* [n,3] */,
                          float *out /* [n,c] */, ssc_stream_t stream);

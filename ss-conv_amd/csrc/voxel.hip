@@ -637,6 +637,108 @@ int ssc_three_nn_grid(int32_t n, int32_t m, const float *unknown, const float *k
   return SSC_OK;
 }
 
+}  // extern "C"
+
+// ---- Voxel2Point as one call ----------------------------------------------------------------
+// What Voxel2Point.forward does with a dozen tensor operations around the search and the
+// interpolation (ss_conv/sp_ops/voxelize.py:131-160), as kernels of one call.
+namespace ssc {
+
+struct V2pGrid {
+  float unit[3], half_extent[3], half_unit[3];
+};
+
+// unknown[i] = (batch id, x, y, z) of point i; known[j] = (b, centre of voxel j) with
+// centre = (index * unit - 0.5 extent) + 0.5 unit, the three roundings of the reference's
+// expression (voxelize.py:139).
+__global__ void __launch_bounds__(256)
+    v2p_prepare_kernel(const float *__restrict__ pts, const int64_t *__restrict__ ids, int n,
+                       const int32_t *__restrict__ vox, int m, V2pGrid g,
+                       float *__restrict__ unknown, float *__restrict__ known) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) {
+    const float4v u = {(float)ids[i], pts[(int64_t)i * 3], pts[(int64_t)i * 3 + 1],
+                       pts[(int64_t)i * 3 + 2]};
+    reinterpret_cast<float4v *>(unknown)[i] = u;
+  }
+  if (i < m) {
+    const int4 r = reinterpret_cast<const int4 *>(vox)[i];
+    float4v k;
+    k.x = (float)r.x;
+    k.y = ((float)r.y * g.unit[0] - g.half_extent[0]) + g.half_unit[0];
+    k.z = ((float)r.z * g.unit[1] - g.half_extent[1]) + g.half_unit[1];
+    k.w = ((float)r.w * g.unit[2] - g.half_extent[2]) + g.half_unit[2];
+    reinterpret_cast<float4v *>(known)[i] = k;
+  }
+}
+
+// weight[q, j] = r_j / ((r_0 + r_1) + r_2) with r_j = 1 / (sqrt(dist2[q, j]) + 1e-8)
+// (voxelize.py:156-159).
+__global__ void __launch_bounds__(256)
+    v2p_weight_kernel(const float *__restrict__ dist2, int n, float *__restrict__ weight) {
+  const int q = blockIdx.x * blockDim.x + threadIdx.x;
+  if (q >= n) return;
+  const float r0 = 1.0f / (sqrtf(dist2[q * 3]) + 1e-8f);
+  const float r1 = 1.0f / (sqrtf(dist2[q * 3 + 1]) + 1e-8f);
+  const float r2 = 1.0f / (sqrtf(dist2[q * 3 + 2]) + 1e-8f);
+  const float norm = (r0 + r1) + r2;
+  weight[q * 3] = r0 / norm;
+  weight[q * 3 + 1] = r1 / norm;
+  weight[q * 3 + 2] = r2 / norm;
+}
+
+}  // namespace ssc
+
+extern "C" {
+
+size_t ssc_v2p_workspace_bytes(int32_t n, int32_t m, int32_t batch_size, const int32_t dims[3]) {
+  const size_t search = ssc_three_nn_grid_workspace_bytes(n, m, batch_size, dims);
+  if (search == 0) return 0;
+  return search + align_up((size_t)(n > 0 ? n : 1) * 16) + align_up((size_t)(m > 0 ? m : 1) * 16) +
+         align_up((size_t)(n > 0 ? n : 1) * 12);
+}
+
+int ssc_v2p_interpolate_f32(const float *points, const int64_t *batch_ids, int32_t n,
+                            const int32_t *voxel_indices, const float *voxel_feats, int32_t m,
+                            int32_t channels, int32_t batch_size, const int32_t dims[3],
+                            const float unit[3], const float extent[3], float *out, int32_t *idx,
+                            float *weight, void *workspace, size_t workspace_bytes,
+                            ssc_stream_t stream) {
+  SSC_CHECK(n >= 0 && m >= 1 && channels >= 1, SSC_EINVAL, "bad sizes");
+  SSC_CHECK(unit && extent && dims, SSC_EINVAL, "NULL pointer argument");
+  if (n == 0) return SSC_OK;
+  SSC_CHECK(points && batch_ids && voxel_indices && voxel_feats && out && idx && weight &&
+                workspace,
+            SSC_EINVAL, "NULL pointer argument");
+  const size_t search = ssc_three_nn_grid_workspace_bytes(n, m, batch_size, dims);
+  SSC_CHECK(search > 0 && workspace_bytes >= ssc_v2p_workspace_bytes(n, m, batch_size, dims),
+            SSC_EWORKSPACE, "v2p workspace too small");
+  hipStream_t s = (hipStream_t)stream;
+  Carver c(workspace);
+  char *search_ws = c.take<char>(search);
+  float *unknown = c.take<float>((size_t)n * 4);
+  float *known = c.take<float>((size_t)m * 4);
+  float *dist2 = c.take<float>((size_t)n * 3);
+  V2pGrid g;
+  float origin[3];
+  for (int a = 0; a < 3; ++a) {
+    g.unit[a] = unit[a];
+    g.half_extent[a] = 0.5f * extent[a];
+    g.half_unit[a] = 0.5f * unit[a];
+    origin[a] = -0.5f * extent[a];
+  }
+  hipLaunchKernelGGL(v2p_prepare_kernel, dim3((unsigned)ceil_div(n > m ? n : m, 256)), dim3(256),
+                     0, s, points, batch_ids, n, voxel_indices, m, g, unknown, known);
+  SSC_LAUNCH_CHECK("v2p_prepare");
+  int rc = ssc_three_nn_grid(n, m, unknown, known, voxel_indices, batch_size, dims, origin, unit,
+                             dist2, idx, search_ws, search, stream);
+  if (rc != SSC_OK) return rc;
+  hipLaunchKernelGGL(v2p_weight_kernel, dim3((unsigned)ceil_div(n, 256)), dim3(256), 0, s, dist2, n,
+                     weight);
+  SSC_LAUNCH_CHECK("v2p_weight");
+  return ssc_three_interp_f32(channels, m, n, voxel_feats, idx, weight, out, stream);
+}
+
 int ssc_three_interp_f32(int32_t c, int32_t m, int32_t n, const float *feats, const int32_t *idx,
                          const float *weight, float *out, ssc_stream_t stream) {
   (void)m;

@@ -139,6 +139,11 @@ _SIGNATURES = {
                                          ctypes.POINTER(ctypes.c_float),
                                          ctypes.POINTER(ctypes.c_float), _vp, _vp, _vp, _sz, _vp]),
     "ssc_three_interp_f32": (ctypes.c_int, [_i32, _i32, _i32, _vp, _vp, _vp, _vp, _vp]),
+    "ssc_v2p_workspace_bytes": (_sz, [_i32, _i32, _i32, ctypes.POINTER(_i32)]),
+    "ssc_v2p_interpolate_f32": (ctypes.c_int, [_vp, _vp, _i32, _vp, _vp, _i32, _i32, _i32,
+                                               ctypes.POINTER(_i32), ctypes.POINTER(ctypes.c_float),
+                                               ctypes.POINTER(ctypes.c_float), _vp, _vp, _vp, _vp,
+                                               _sz, _vp]),
     "ssc_bn_workspace_bytes": (_sz, [_i64, _i32]),
     "ssc_bn_prepare_f32": (ctypes.c_int, [_vp, _i64, _i32, _vp, _vp, _vp, _vp, _i32, _i32,
                                           ctypes.c_float, ctypes.c_float, _vp, _vp, _vp, _vp, _vp,
@@ -930,6 +935,57 @@ def three_nn_grid(unknown, known, voxel_indices, batch_size, dims, origin, unit)
                                   int(batch_size), d, o, u, _ptr(dist2), _ptr(idx), ws.data_ptr(),
                                   ws.numel(), _stream(unknown)))
     return dist2, idx
+
+
+class _V2pInterpolate(torch.autograd.Function):
+    """Voxel features read back at points, one native call; differentiable in the features
+    (the gradient is the interpolation's, through the saved indices and weights)."""
+
+    @staticmethod
+    def forward(ctx, feats, points, batch_ids, voxel_indices, batch_size, dims, unit, extent):
+        n, m, c = points.size(0), feats.size(0), feats.size(1)
+        dev = feats.device
+        d = (_i32 * 3)(*[int(v) for v in dims])
+        u = (ctypes.c_float * 3)(*[float(v) for v in unit])
+        e = (ctypes.c_float * 3)(*[float(v) for v in extent])
+        nbytes = _lib.ssc_v2p_workspace_bytes(n, m, int(batch_size), d)
+        if nbytes == 0:
+            raise RuntimeError("v2p_interpolate: batch_size * prod(dims) must be positive and "
+                               "below 2^31")
+        ws = _workspace(nbytes, dev)
+        out = torch.empty((n, c), dtype=torch.float32, device=dev)
+        idx = torch.empty((n, 3), dtype=torch.int32, device=dev)
+        weight = torch.empty((n, 3), dtype=torch.float32, device=dev)
+        _check(_lib.ssc_v2p_interpolate_f32(_ptr(points), _ptr(batch_ids), n, _ptr(voxel_indices),
+                                            _ptr(feats), m, c, int(batch_size), d, u, e, _ptr(out),
+                                            _ptr(idx), _ptr(weight), ws.data_ptr(), ws.numel(),
+                                            _stream(feats)))
+        ctx.saved = (idx, weight, m)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        idx, weight, m = ctx.saved
+        n, c = grad_out.size()
+        grad = torch.zeros((m, c), dtype=torch.float32, device=grad_out.device)
+        three_interpolate_bp(c, n, m, grad_out.contiguous(), idx, weight, grad)
+        return (grad,) + (None,) * 7
+
+
+def v2p_interpolate(feats, points, batch_ids, voxel_indices, batch_size, dims, unit, extent):
+    """Voxel2Point.forward with points (ss_conv/sp_ops/voxelize.py:131-160) as one call:
+    feats [m, C] float32 of the voxels voxel_indices [m, 4] int32 (distinct), read at
+    points [n, 3] float32 of the batch elements batch_ids [n] int64, on a grid of `dims`
+    cells of size `unit` that spans `extent` around the origin.  Returns [n, C]."""
+    _need_gpu(feats, points, batch_ids, voxel_indices)
+    if feats.dtype != torch.float32 or points.dtype != torch.float32 or \
+            batch_ids.dtype != torch.int64 or voxel_indices.dtype != torch.int32:
+        raise RuntimeError("v2p_interpolate: float32 features and points, int64 ids, int32 voxels")
+    if voxel_indices.size(0) != feats.size(0) or feats.size(0) < 1 or \
+            batch_ids.size(0) != points.size(0):
+        raise RuntimeError("v2p_interpolate: one feature row per voxel (at least one), one id per point")
+    return _V2pInterpolate.apply(feats.contiguous(), points.contiguous(), batch_ids.contiguous(),
+                                 voxel_indices.contiguous(), batch_size, dims, unit, extent)
 
 
 def three_interpolate_fp(c, m, n, feats, idx, weight, out):

@@ -154,12 +154,41 @@ class Voxel2Point(nn.Module):
         self._consts = {}  # (device, grid shape) -> (unit, extent) on the device
 
     def forward(self, sparse_feat, point_cloud=None, batch_ids=None):
+        if point_cloud is not None and self._one_call_ok(sparse_feat, point_cloud, batch_ids):
+            # centres, search, weights and interpolation as one native call
+            unit, extent = self._unit_extent(sparse_feat)
+            return _ext.v2p_interpolate(
+                sparse_feat.features, point_cloud, batch_ids, sparse_feat.indices,
+                sparse_feat.batch_size,
+                # (a point on the upper face of the grid has voxel index == shape,
+                # voxelize.py:85-86)
+                [int(v) + 1 for v in sparse_feat.spatial_shape], unit, extent)
         vx_points, vx_feats = self._get_vertice_feats(sparse_feat)
         if point_cloud is not None:
             assert batch_ids is not None
             points = torch.cat([batch_ids.float().unsqueeze(1), point_cloud], dim=1)
             return self._get_point_feats(points.contiguous(), vx_points, vx_feats, sparse_feat)
         return vx_points[:, 1:].contiguous(), vx_feats, vx_points[:, 0].contiguous()
+
+    @staticmethod
+    def _one_call_ok(sparse_tensor, point_cloud, batch_ids):
+        feat, idx = sparse_tensor.features, sparse_tensor.indices
+        return (batch_ids is not None and feat.is_cuda and point_cloud.is_cuda and idx.is_cuda
+                and batch_ids.is_cuda and feat.dtype == torch.float32 and feat.dim() == 2
+                and point_cloud.dtype == torch.float32 and idx.dtype == torch.int32
+                and batch_ids.dtype == torch.int64 and feat.size(0) >= 1
+                and point_cloud.dim() == 2 and point_cloud.size(1) == 3)
+
+    def _unit_extent(self, sparse_tensor):
+        """(unit, extent) of the voxel grid as float32 host arrays: the numbers that
+        _get_vertice_feats puts on the device."""
+        shape = np.asarray(sparse_tensor.spatial_shape, dtype=np.float64)
+        if self.voxel_extent is not None:
+            unit, extent = self.voxel_extent / shape, self.voxel_extent
+        else:
+            unit, extent = self.unit_voxel_extent, self.unit_voxel_extent * shape
+        return (np.asarray(unit, dtype=np.float64).astype(np.float32),
+                np.asarray(extent, dtype=np.float64).astype(np.float32))
 
     def _get_vertice_feats(self, sparse_tensor):
         feat = sparse_tensor.features

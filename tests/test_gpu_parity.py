@@ -1787,3 +1787,41 @@ def test_conv_epilogue_block_other_layers(oracle, device):
         check(ConvBatchNormActivation(conv, None, None).eval(), False)
     finally:
         _ext._lib.ssc_conv_run_epilogue_f32 = real
+
+
+def test_voxel2point_one_call_equals_the_separate_steps(oracle, device):
+    """ssc_v2p_interpolate_f32 (centres, search, weights and interpolation in one call, what
+    Voxel2Point.forward runs) against the module's step-by-step form and the oracle: output,
+    and the gradient with respect to the voxel features; clouds with a far-away point (the
+    list of unsettled queries), an empty batch element and points on the grid's upper face."""
+    from ss_conv.sp_ops.voxelize import Point2Voxel, Voxel2Point
+    for seed, grid, npts in ((6, 16, 500), (9, 8, 300), (12, 32, 2000)):
+        pts, feats, ids = synth.make_clouds(3, npts, seed=seed, channels=12)
+        pts = pts.copy()
+        pts[0] = [0.99, 0.99, 0.99]      # a corner of the grid
+        pts[1] = [1.0, -1.0, 1.0]        # on the upper face: voxel index == shape
+        ids = ids.copy()
+        ids[ids == 1] = 2                # batch element 1 has no points
+        dp, df, di = [torch.from_numpy(x).to(device) for x in (pts, feats, ids)]
+        vp, st, vi, _ = Point2Voxel([grid] * 3, [2.0 / grid] * 3)(dp, df, di)
+        for kw in (dict(unit_voxel_extent=[2.0 / grid] * 3), dict(voxel_extent=[2.0] * 3)):
+            v2p = Voxel2Point(**kw)
+            st.features = st.features.detach().requires_grad_(True)
+            out = v2p(st, vp, vi)
+            g = torch.randn_like(out)
+            out.backward(g)
+            grad_one = st.features.grad.clone()
+            keep = Voxel2Point.__dict__["_one_call_ok"]
+            Voxel2Point._one_call_ok = staticmethod(lambda *a: False)
+            try:
+                st.features = st.features.detach().requires_grad_(True)
+                ref = v2p(st, vp, vi)
+                ref.backward(g)
+            finally:
+                Voxel2Point._one_call_ok = keep
+            assert rel_l2(out.detach().cpu().numpy(), ref.detach().cpu().numpy()) < 1e-6
+            assert rel_l2(grad_one.cpu().numpy(), st.features.grad.cpu().numpy()) < 1e-6
+            want, _, _ = oracle.voxel2point(st.indices.cpu().numpy(),
+                                            st.features.detach().cpu().numpy(), [grid] * 3,
+                                            vp.cpu().numpy(), vi.cpu().numpy(), **kw)
+            assert rel_l2(out.detach().cpu().numpy(), want) < 1e-6
