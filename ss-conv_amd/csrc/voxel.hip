@@ -352,7 +352,7 @@ int ssc_three_nn_ws(int32_t n, int32_t m, const float *unknown, const float *kno
 // plain scan as well.
 namespace ssc {
 
-constexpr int kGridNnMaxShell = 3;
+constexpr int kGridNnMaxShell = 4;
 
 struct GridNn {
   int batch, dim[3];
