@@ -1622,6 +1622,8 @@ EPILOGUE_CASES = [
     ([(32, 0), (32, 1), (32, 2)], 40, 3, 2, 1, False, None),          # 288 outputs, several blocks
     ([(3, 0), (2, 1), (2, 2)], 5, 2, 2, 0, False, None),              # 19 outputs: scalar stores
     ([(16, 0)], 8, 3, 1, 1, False, None),                             # scalars only, no gates
+    # 6.9 MB of packed filters in four column blocks: one column block per XCD
+    ([(40, 0), (24, 1), (16, 2)], 256, 3, 1, 1, False, None),
 ]
 
 
