@@ -24,6 +24,10 @@ for _p in (os.path.join(ROOT, "ss-conv_amd"), os.path.join(ROOT, "oracle")):
 
 FP32_MFMA_PEAK_TFLOPS = 157.3  # MI355X dense fp32 matrix peak
 
+# the step is run for this long before the warm-up steps, to bring an idle GPU to its
+# sustained clock
+CLOCK_WARMUP_MS = 100
+
 # HBM bytes per launch of the convolution kernel for every workload this script offers, from
 # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs scaled by a copy kernel of known size (the
 # summaries profiles/conv_fwd_<workload>_hbm_traffic.md give commands and counter values).
@@ -38,6 +42,9 @@ def parse_args():
     ap.add_argument("--workload", default="cfg2", choices=["cfg1", "cfg2", "cfg3", "cfg5"])
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--time-every", type=int, default=0, metavar="N",
+                    help="time every N-th launch of the convolution kernel with HIP events "
+                         "(default: every other one, every launch below 20 steps)")
     ap.add_argument("--calibration-copy", type=int, default=0, metavar="MIB",
                     help="also run one plain device copy of MIB mebibytes before the timed "
                          "region (the known-size kernel that scales rocprofv3's FETCH_SIZE / "
@@ -443,6 +450,17 @@ def main():
         with torch.no_grad():
             return conv(x)
 
+    gc.collect()
+    # A GPU that has idled while the host prepared the inputs runs its first tens of
+    # milliseconds of work at a lower clock (the convolution kernel takes 0.33 ms in a step
+    # that follows 2 ms of work, 0.30 ms after 40 ms of it).  The step is therefore run for
+    # CLOCK_WARMUP_MS before the warm-up steps proper, so that the timed steps are those of a
+    # GPU at its sustained clock; the JSON line says so (config.clock_warmup_ms).
+    t_warm = time.perf_counter()
+    while (time.perf_counter() - t_warm) * 1e3 < CLOCK_WARMUP_MS:
+        for _ in range(10):
+            out = step()
+        torch.cuda.synchronize()
     for _ in range(args.warmup):
         out = step()
     torch.cuda.synchronize()
@@ -454,13 +472,15 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    # every fifth launch of the convolution kernel inside the timed region is timed with HIP
-    # events on its stream (timing every launch costs the step about 20 us of stream time)
-    _ext.profile_conv(True, every=5 if args.steps >= 20 else 1)
+    # every other launch of the convolution kernel inside the timed region is timed with HIP
+    # events on its stream (a pair of events costs the stream a few microseconds)
+    _ext.profile_conv(True, every=args.time_every or (2 if args.steps >= 20 else 1))
     # The interpreter's cyclic garbage collector stays out of the timed region, as in
     # timeit: a full collection of a process that has imported torch takes 30-40 ms, many
     # times the region itself, and when it falls due depends on allocation counts only.
-    gc.collect()
+    # (The one collection that empties the backlog runs before the warm-up steps: the
+    # hundred steps after a full collection are each about 15 us slower, collector on or
+    # off, than steps that follow other steps.)
     gc.disable()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
@@ -507,6 +527,7 @@ def main():
                    "n_in": int(n_in), "n_out": int(n_out), "pairs": P,
                    "input_voxels_per_s": n_in / (ms_per_step * 1e-3),
                    "timed_region": "cyclic garbage collector off (as timeit does)",
+                   "clock_warmup_ms": CLOCK_WARMUP_MS,
                    "ms_per_step_gc_on": ms_gc_on},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": FP32_MFMA_PEAK_TFLOPS,
                      "unit": "TFLOP/s", "frac": achieved / FP32_MFMA_PEAK_TFLOPS,
