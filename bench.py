@@ -126,6 +126,21 @@ def ops_table(torch, _ext, synth, dev, seed):
         rows.append("%-44s %8.3f ms %9.2f MB %8.1f GB/s %5.1f%% of HBM  %s"
                     % (name, ms, nbytes / 1e6, gbs, gbs / 80.0, note))
 
+    # what a dependent launch costs whatever it does: 200 one-element kernels in a row between
+    # two events (the floor under every operator below that is a chain of small kernels)
+    one = torch.zeros(1, device=dev)
+    for _ in range(20):
+        one.add_(1.0)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    e0.record()
+    for _ in range(200):
+        one.add_(1.0)
+    e1.record()
+    torch.cuda.synchronize()
+    rows.append("%-44s %8.2f us each (200 dependent one-element kernels on one stream)"
+                % ("dependent launch floor", e0.elapsed_time(e1) * 1e3 / 200))
+
     # convolution backward on the benchmark layer (cfg2: 64 -> 128 channels)
     cfg = synth.CONFIGS["cfg2"]
     pts, feats, ids = synth.config_clouds("cfg2", seed)
