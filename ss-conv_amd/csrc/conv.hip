@@ -323,9 +323,11 @@ constexpr int kSplitGranule = 64;
 // still there when that tile's turn comes.
 constexpr int kSpillRows = 160;
 
-// cost of a tile beyond its pairs, in pair slots: some padding per offset, and about
-// two stages' worth of time for writing it out
-__device__ __forceinline__ int64_t split_tile_cost(int K) { return (int64_t)K * 2 + 128; }
+// cost of a tile beyond its pairs, in pair slots: padding per offset, and about a stage's
+// worth of time for writing it out (measured: 2 K + 128 and 3 K + 64 are as good on the
+// 27-offset benchmark layers; with 125 offsets 4 K + 64 is 4 % faster than 2 K + 128, and
+// more than that slower again)
+__device__ __forceinline__ int64_t split_tile_cost(int K) { return (int64_t)K * 4 + 64; }
 
 // Work in rows below cell b of the fine grid (scaled by T to stay in integers).
 __device__ __forceinline__ int64_t split_work(int64_t pairs_below, int64_t b, int64_t n_out,
