@@ -201,6 +201,22 @@ def test_backbone_full_size(oracle, device):
         err = rel_l2(as_np(x.features), o_feat)
         print("  rows out", n_out, "pairs", int(nums.sum()), "bn+gate rel-l2", err, flush=True)
         assert err < REL_L2, (si, err)
+        # the same block in evaluation mode as one kernel (batch norm constants and gate
+        # applied while the convolution stores its rows) against the three layers one after
+        # the other and against the oracle on the float64 sums
+        from ss_conv.fused import ConvBatchNormActivation
+        from ss_conv.sp_ops.tensor import SparseTensor
+        one = ConvBatchNormActivation(conv, block.bn, block.act).eval()
+        with torch.no_grad():
+            got = one(SparseTensor(f, in_idx, shape, batch))
+            sep = block(conv(SparseTensor(f, in_idx, shape, batch)))
+        assert torch.equal(got.indices, sep.indices)
+        assert _rel(got.features, sep.features.double()) < 1e-6, si
+        running = (as_np(block.bn.running_mean), as_np(block.bn.running_var))
+        o_eval = oracle.bn_gate_fwd(y_np, rs_gated, rs, params, training=False, running=running)
+        assert rel_l2(as_np(got.features), o_eval) < REL_L2, si
+        conv.train()
+        block.train()
         shape = [int(v) for v in y.spatial_shape]
         rs_in = rs
     assert shape == [16, 16, 16]
