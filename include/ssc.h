@@ -299,10 +299,14 @@ int ssc_conv_bwd_filter_f16(const void *features /* [n_in,c_in] half */, int64_t
  * ssc_profile_conv_read waits for the recorded calls and returns their
  * durations in milliseconds, oldest first; enabling again clears the ring. */
 int ssc_profile_conv(int32_t enable);
-/* Measurement knob, no counterpart in the reference: by_column = 0 keeps the convolution
- * kernel from giving every XCD one column block of its own when the packed filters are
- * larger than an L2 (the default, 1, lets it).  Results do not depend on it. */
-int ssc_conv_tuning(int32_t by_column);
+/* Measurement knob, no counterpart in the reference; flags (default 1):
+ *   1  lets the convolution kernel give every XCD one column block of its own when the
+ *      packed filters are larger than an L2 (0: never);
+ *   2  no launch of its own for a last group of 16 output columns that would be alone in
+ *      its block of 64 (Cout = 72, 136).  This flag changes the sizes ssc_conv_plan_bytes
+ *      and its like return: set it before any plan is sized or built and do not mix plans
+ *      across a change.  Results agree up to the order of the float sums of that group. */
+int ssc_conv_tuning(int32_t flags);
 int ssc_profile_conv_read(float *ms /* host */, int32_t capacity, int32_t *count /* host */);
 
 /* ------------------------------------------------------------------------

@@ -770,7 +770,7 @@ struct ConvEpilogue {
   int act_s, act_g, c_dest;
 };
 
-template <typename IO, int GATHER, int NCW, int NS, bool EPI>
+template <typename IO, int GATHER, int NCW, int NS, bool EPI, bool TAIL>
 __global__ void __launch_bounds__((NCW + 4) * 64)
     __attribute__((amdgpu_waves_per_eu((NCW + 4) / 4, (NCW + 4) / 4)))
     conv_fwd_kernel(const IO *__restrict__ features, int cin, unsigned feat_bytes,
@@ -779,7 +779,7 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
                     const int32_t *__restrict__ grp_meta, unsigned sched_bytes, unsigned meta_bytes,
                     const int32_t *__restrict__ tile_grp, const int32_t *__restrict__ wg_tile,
                     int nch, int ncb, IO *__restrict__ out, int cout, int T, int cols_per_xcd,
-                    ConvEpilogue epi) {
+                    int col_base, ConvEpilogue epi) {
   constexpr int kCN = 16 * NCW;   // output columns per workgroup
   constexpr int kEB = Io<IO>::kBytes;
   constexpr bool kHalf = kEB == 2;
@@ -827,7 +827,8 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
   const int t_begin = wg_tile[chunk], t_end = wg_tile[chunk + 1];
   const int g_begin = tile_grp[t_begin], g_end = tile_grp[t_end];
   const int nstages = (g_end - g_begin) * nch;  // stages of this workgroup
-  const int col0 = cblk * kCN;
+  const int col0 = col_base + cblk * kCN;
+  static_assert(!TAIL || (NCW == 4 && !kHalf), "the one-column-group form is built for float");
 
   {
     float4v z = {0.f, 0.f, 0.f, 0.f};
@@ -850,7 +851,8 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
     const int c_t = (tid % (kCN / 4)) * 4, col = col0 + c_t;
     const bool col_ok = col < cout;
     static_assert(!EPI || kCN == 64, "the epilogue's gate runs are per block of 64 columns");
-    const int gfirst = epi.gate_run[2 * cblk], gcount = min(epi.gate_run[2 * cblk + 1], 16);
+    const int eblk = col0 / kCN;  // block of 64 columns the workgroup's columns start
+    const int gfirst = epi.gate_run[2 * eblk], gcount = min(epi.gate_run[2 * eblk + 1], 16);
     const bool run_ok = gfirst >= col0 && gfirst + gcount <= min(col0 + kCN, cout);
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -881,6 +883,23 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
   }
   const int e_c_dest = epi.c_dest, e_act_s = epi.act_s, e_act_g = epi.act_g;
   auto flush_tile = [&](int row0, int rows, int slot0) __attribute__((always_inline)) {
+    if constexpr (TAIL) {
+      // The four consumer waves each hold a partial sum of the one column group, in the
+      // 16 columns a wave owns: add them up in the first 16, clear the others, and write
+      // the tile out as any other.
+      const float4v z = {0.f, 0.f, 0.f, 0.f};
+      for (int r = tid >> 2; r < rows; r += NT / 4) {
+        int sl = slot0 + r;
+        if (sl >= T) sl -= T;
+        float4v *ap = reinterpret_cast<float4v *>(acc + sl * kAS + (tid & 3) * 4);
+        const float4v v = (ap[0] + ap[4]) + (ap[8] + ap[12]);
+        ap[0] = v;
+        ap[4] = z;
+        ap[8] = z;
+        ap[12] = z;
+      }
+      __syncthreads();
+    }
     if constexpr (EPI) {
       // Batch norm constants and gate applied on the way out (cout % 4 == 0).  Threads,
       // columns and rows as in the plain store below.  The 16 lanes of a row sit in one wave
@@ -1172,7 +1191,8 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
     const int l16 = lane & 15;
     // A column group beyond Cout multiplies with the last real one's fragments; its
     // accumulator columns are never written out.
-    const int cb = min(cblk * NCW + wave, ncb - 1);
+    // (The one-column-group form: every wave multiplies with the fragments of that group.)
+    const int cb = TAIL ? col_base / 16 : min(col0 / 16 + wave, ncb - 1);
     const __amdgpu_buffer_rsrc_t rs_w =
         __builtin_amdgcn_make_buffer_rsrc((void *)packed, 0, (int)packed_bytes, kRsrcFlags);
     const __amdgpu_buffer_rsrc_t rs_out =
@@ -1283,6 +1303,100 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
     // LDS address of this lane's 4 columns in accumulator row 0
     const int acc_lane = acc_base + (wave * 16 + g * 4) * 4;
     const int dummy_addr = T * kAS * 4 + acc_lane;
+    if constexpr (TAIL) {
+      // One column group for four consumer waves: wave m multiplies row block m of every
+      // group and keeps its products in the 16 accumulator columns it owns (a partial sum
+      // of the group's columns over the pairs of its blocks; flush_tile adds the four up).
+      // A stage is 1 row block of NS MFMAs per wave instead of 4; the products of a group's
+      // chunks stay in registers and reach the accumulators once per group.
+      // Rings indexed by stage number (the loop is unrolled over four stages):
+      //   w[s & 3]     fragments of stage s, fetched three stages ahead
+      //   kof[s & 3]   fragment offset of the block's kernel offset, loaded seven stages
+      //                ahead (four before the fetch that needs it)
+      //   orow[s & 3]  accumulator row of this lane's pair, tl[s & 3] the tile of the stage:
+      //                loaded four stages ahead, into the slot the stage before just used
+      int kof[4];
+      int4v tl[4];
+      const char *const ab_wave = a_base + wave * 16 * kRowB;
+      auto load_kof = [&](const StagePos &pos) -> int {
+        return buf_load1(rs_meta, wave * 4, pos.g * 32);
+      };
+      StagePos p_cur = {g_begin, 0};  // stage being multiplied
+      StagePos p_f = {g_begin, 0};    // stage whose fragments are fetched next
+      StagePos p_k = {g_begin, 0};    // stage whose fragment offset is loaded next
+      StagePos p_m = {g_begin, 0};    // stage whose accumulator rows and tile are loaded next
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        kof[j] = load_kof(p_k);
+        p_k.advance(nch);
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        fetch_orow(p_m, wave, j);
+        tl[j] = load_rec_tail(p_m);
+        p_m.advance(nch);
+      }
+#pragma unroll
+      for (int j = 0; j < 3; ++j) {
+        const int soff = frag_soff(kof[j], w_soff0 + p_f.cc * kFragB);
+#pragma unroll
+        for (int q = 0; q < NF; ++q) fetch_w(soff, j, q);
+        p_f.advance(nch);
+        kof[j] = load_kof(p_k);
+        p_k.advance(nch);
+      }
+      float4v d = float4v{0.f, 0.f, 0.f, 0.f};
+      __syncthreads();
+      auto stage = [&](auto phase) {
+        constexpr int ph = decltype(phase)::value;  // == stage number & 3
+        constexpr int nx = (ph + 3) & 3;
+        {
+          const int soff = frag_soff(kof[nx], w_soff0 + p_f.cc * kFragB);
+#pragma unroll
+          for (int q = 0; q < NF; ++q) fetch_w(soff, nx, q);
+          p_f.advance(nch);
+          kof[nx] = load_kof(p_k);
+          p_k.advance(nch);
+        }
+        const char *ab = ab_wave + (ph & 1) * kStage * kRowB;
+        Frag a[NF];
+#pragma unroll
+        for (int q = 0; q < NF; ++q) a[q] = *reinterpret_cast<const Frag *>(ab + q * 64);
+        const bool commit = p_cur.cc == nch - 1;  // the group's last chunk
+        const int addr = commit ? orow[ph] + acc_lane : dummy_addr;
+        const float4v accr = lds_load4(addr);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 0; i < NS; ++i)
+          d = __builtin_amdgcn_mfma_f32_16x16x4f32(w[ph][i >> 2][i & 3], a[i >> 2][i & 3], d, 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        const TileEnd e = tile_end_of(tl[ph], p_cur);
+        if (commit) {
+          lds_store4(addr, accr + d);
+          d = float4v{0.f, 0.f, 0.f, 0.f};
+        }
+        fetch_orow(p_m, wave, ph);
+        tl[ph] = load_rec_tail(p_m);
+        p_m.advance(nch);
+        p_cur.advance(nch);
+        __syncthreads();
+        if (e.last) {
+          flush_tile(e.row0, e.rows, e.slot0);
+          __syncthreads();
+        }
+      };
+      // whole groups of four stages first, the remainder after the loop (see the producers)
+      int s = 0;
+      for (; s + 4 <= nstages; s += 4) {
+        stage(std::integral_constant<int, 0>());
+        stage(std::integral_constant<int, 1>());
+        stage(std::integral_constant<int, 2>());
+        stage(std::integral_constant<int, 3>());
+      }
+      if (s < nstages) stage(std::integral_constant<int, 0>());
+      if (s + 1 < nstages) stage(std::integral_constant<int, 1>());
+      if (s + 2 < nstages) stage(std::integral_constant<int, 2>());
+    } else {
     Pending pend;  // nothing pending yet: the first write adds zero to the dummy row
     pend.addr = dummy_addr;
     pend.accr = float4v{0.f, 0.f, 0.f, 0.f};
@@ -1446,6 +1560,7 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
       step(std::integral_constant<int, 1>());
     }
     if (s < nstages) step(std::integral_constant<int, 0>());
+    }
   }
 }
 
@@ -1456,6 +1571,14 @@ struct ConvPlan {
   int ns;      // conv_fwd_kernel's NS: MFMA steps per chunk
   int64_t n_tiles, n_fine, words_per_k, grp_cap;  // n_tiles: upper bound
   size_t lds_bytes;
+  // Launches.  As a rule one, over all column blocks (n_colblk of them side by side, the
+  // CUs shared out among them).  A last column group that would be alone in its block of
+  // four (Cout = 72: 5 groups) behind at most two full blocks gets no column block, where
+  // three of four consumer waves would multiply for nothing: the full blocks take one launch
+  // each over all CUs (n_launch of them, n_colblk = 1) and the kernel's one-column-group
+  // form a last one (has_tail), all over the same plan.
+  int n_launch;
+  bool has_tail;
 };
 
 static size_t conv_lds_bytes(int T, int ncw) {
@@ -1483,6 +1606,24 @@ static int device_cu_count() {
   return cus;
 }
 
+// (switched by ssc_conv_tuning, for measurements)
+static bool g_conv_by_column = true;  // one column block per XCD for large filters
+static bool g_conv_tail = true;       // a launch of its own for a lone last column group
+
+// The sizes that follow from the number of workgroups per column block.
+static void plan_split(ConvPlan &p, int n_wg, int64_t n_out, int K, int64_t pair_stride) {
+  p.n_wg = n_wg;
+  // upper bound of the tile count: every workgroup's range ends with a partial tile
+  p.n_tiles = ceil_div(n_out > 0 ? n_out : 1, p.tile_rows) + n_wg;
+  p.n_fine = ceil_div(n_out > 0 ? n_out : 1, kSplitGranule);
+  p.words_per_k = ceil_div(n_out > 0 ? n_out : 1, 32);
+  // groups: pairs/64 plus, per (tile, offset), up to one partial block, plus one
+  // partial (or empty) group per tile, plus the groups the kernel's prefetches may
+  // touch beyond the end of the schedule
+  int64_t max_pairs_k = pair_stride < n_out ? pair_stride : n_out;
+  p.grp_cap = ((int64_t)K * (max_pairs_k / 16 + 1) + p.n_tiles * K) / 4 + 2 * p.n_tiles + 4 + 16;
+}
+
 static ConvPlan make_plan(int64_t n_in, int64_t n_out, int K, int c_in, int c_out,
                           int64_t pair_stride, int elem_bytes = 4) {
   ConvPlan p;
@@ -1508,21 +1649,18 @@ static ConvPlan make_plan(int64_t n_in, int64_t n_out, int K, int c_in, int c_ou
   p.gather = 0;
   if ((c_in & 3) == 0 && (uint64_t)n_in * c_in * elem_bytes <= (uint64_t)kGatherPad)
     p.gather = (c_in % kKC) == 0 ? 1 : 2;
-  p.n_colblk = (int)ceil_div(p.ncb, p.ncw);
+  // (wider layers: the launches of one column block each cost more than the lone group
+  // in a block of its own does -- 128 -> 256 channels at stride 2 takes 0.255 ms as four
+  // launches against 0.185 ms as one, 200 -> 200 with 125 offsets 17.6 against 16.8 ms)
+  p.has_tail = g_conv_tail && elem_bytes == 4 && p.ncb % p.ncw == 1 && p.ncb / p.ncw <= 2;
+  const int blocks = p.has_tail ? p.ncb / p.ncw : (int)ceil_div(p.ncb, p.ncw);
+  p.n_colblk = p.has_tail ? 1 : blocks;
+  p.n_launch = p.has_tail ? blocks : 1;
   int n_wg = device_cu_count() / p.n_colblk;
   if (n_wg < 1) n_wg = 1;
   if (n_wg > 256) n_wg = 256;  // the split kernel is one block of 256 threads
   if (n_wg >= 8) n_wg = n_wg / 8 * 8;
-  p.n_wg = n_wg;
-  // upper bound of the tile count: every workgroup's range ends with a partial tile
-  p.n_tiles = ceil_div(n_out > 0 ? n_out : 1, p.tile_rows) + n_wg;
-  p.n_fine = ceil_div(n_out > 0 ? n_out : 1, kSplitGranule);
-  p.words_per_k = ceil_div(n_out > 0 ? n_out : 1, 32);
-  // groups: pairs/64 plus, per (tile, offset), up to one partial block, plus one
-  // partial (or empty) group per tile, plus the groups the kernel's prefetches may
-  // touch beyond the end of the schedule
-  int64_t max_pairs_k = pair_stride < n_out ? pair_stride : n_out;
-  p.grp_cap = ((int64_t)K * (max_pairs_k / 16 + 1) + p.n_tiles * K) / 4 + 2 * p.n_tiles + 4 + 16;
+  plan_split(p, n_wg, n_out, K, pair_stride);
   p.lds_bytes = conv_lds_bytes(p.T, p.ncw);
   return p;
 }
@@ -1631,15 +1769,13 @@ static size_t conv_ws_bytes(int64_t n_out, int K, int c_in, int c_out, int64_t p
   return conv_ws_walk(nullptr, p, K, pair_stride, nullptr);
 }
 
-static bool g_conv_by_column = true;  // (switched by ssc_conv_tuning, for measurements)
-
-template <typename IO, int GATHER, int NCW, int NS, bool EPI>
+template <typename IO, int GATHER, int NCW, int NS, bool EPI, bool TAIL>
 static int launch_conv(const ConvPlan &p, const ConvWs &w, const IO *features, int64_t n_in,
-                       int c_in, int K, IO *out, int c_out, const ConvEpilogue &epi,
-                       hipStream_t s) {
+                       int c_in, int K, IO *out, int c_out, int col_base,
+                       const ConvEpilogue &epi, hipStream_t s) {
   static bool attr_set = false;
   if (!attr_set) {
-    SSC_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(conv_fwd_kernel<IO, GATHER, NCW, NS, EPI>),
+    SSC_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(conv_fwd_kernel<IO, GATHER, NCW, NS, EPI, TAIL>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
     attr_set = true;
   }
@@ -1649,6 +1785,9 @@ static int launch_conv(const ConvPlan &p, const ConvWs &w, const IO *features, i
             "convolution too large for 32-bit buffer offsets (filters %llu B, schedule %llu B)",
             (unsigned long long)packed_bytes, (unsigned long long)sched_bytes);
   const unsigned feat_bytes = GATHER != 0 ? (unsigned)((uint64_t)n_in * c_in * sizeof(IO)) : 0u;
+  SSC_CHECK(p.n_wg >= 1 && p.n_colblk >= 1 && col_base % 16 == 0 &&
+                col_base + (p.n_colblk - 1) * 16 * NCW < c_out,
+            SSC_ERUNTIME, "convolution launch outside the output columns");
   dim3 grid((unsigned)p.n_wg, (unsigned)p.n_colblk);
   // one column block per XCD when the packed filters are larger than an L2 can keep
   // (4 MiB per XCD) and the grid divides that way (256 -> 256 channels, 7 MiB: 2.44 ->
@@ -1658,11 +1797,37 @@ static int launch_conv(const ConvPlan &p, const ConvWs &w, const IO *features, i
                          8 % p.n_colblk == 0 && (p.n_wg * p.n_colblk) % 8 == 0 &&
                          g_conv_by_column;
   const int cols_per_xcd = by_column ? 8 / p.n_colblk : 0;
-  hipLaunchKernelGGL((conv_fwd_kernel<IO, GATHER, NCW, NS, EPI>), grid, dim3((NCW + 4) * 64), p.lds_bytes, s, features, c_in,
+  hipLaunchKernelGGL((conv_fwd_kernel<IO, GATHER, NCW, NS, EPI, TAIL>), grid, dim3((NCW + 4) * 64), p.lds_bytes, s, features, c_in,
                      feat_bytes, w.packed, (unsigned)packed_bytes, w.sched_in, w.sched_out,
                      w.grp_meta, (unsigned)sched_bytes, (unsigned)(p.grp_cap * 32), w.tile_grp,
-                     w.wg_tile, p.nch, p.ncb, out, c_out, p.T, cols_per_xcd, epi);
+                     w.wg_tile, p.nch, p.ncb, out, c_out, p.T, cols_per_xcd, col_base, epi);
   SSC_LAUNCH_CHECK("conv_fwd");
+  return SSC_OK;
+}
+
+// The launches of a plan (ConvPlan): the column blocks, all at once or one after the other,
+// then the one-column-group form for a lone last group.
+template <typename IO, int GATHER, int NS>
+static int launch_all(const ConvPlan &p, const ConvWs &w, const IO *features, int64_t n_in,
+                      int c_in, int K, IO *out, int c_out, const ConvEpilogue &epi,
+                      hipStream_t s) {
+  constexpr bool kFloat = sizeof(IO) == 4;
+  const bool with_epi = kFloat && epi.mode != nullptr;
+  for (int l = 0; l < p.n_launch; ++l) {
+    const int col_base = l * p.n_colblk * 16 * p.ncw;
+    const int rc = with_epi ? launch_conv<IO, GATHER, 4, NS, kFloat, false>(
+                                  p, w, features, n_in, c_in, K, out, c_out, col_base, epi, s)
+                            : launch_conv<IO, GATHER, 4, NS, false, false>(
+                                  p, w, features, n_in, c_in, K, out, c_out, col_base, epi, s);
+    if (rc != SSC_OK) return rc;
+  }
+  if (p.has_tail) {
+    const int col_base = (p.ncb - 1) * 16;
+    return with_epi ? launch_conv<IO, GATHER, 4, NS, kFloat, kFloat>(
+                          p, w, features, n_in, c_in, K, out, c_out, col_base, epi, s)
+                    : launch_conv<IO, GATHER, 4, NS, false, kFloat>(
+                          p, w, features, n_in, c_in, K, out, c_out, col_base, epi, s);
+  }
   return SSC_OK;
 }
 
@@ -1697,8 +1862,9 @@ int ssc_profile_conv(int32_t enable) {
   return SSC_OK;
 }
 
-int ssc_conv_tuning(int32_t by_column) {
-  g_conv_by_column = by_column != 0;
+int ssc_conv_tuning(int32_t flags) {
+  g_conv_by_column = (flags & 1) != 0;
+  g_conv_tail = (flags & 2) == 0;
   return SSC_OK;
 }
 
@@ -1825,10 +1991,8 @@ static int conv_run(const ConvPlan &p, const ConvWs &w, const IO *features, int6
   const bool prof = g_profile_on && (g_profile_calls++ % g_profile_every) == 0;
   const int slot = g_profile_count % kProfileRing;
   if (prof) SSC_HIP(hipEventRecord(g_profile_ev[slot][0], s));
-#define SSC_CONV_LAUNCH(G, S)                                                                   \
-  (sizeof(IO) == 4 && epi.mode != nullptr                                                       \
-       ? launch_conv<IO, G, 4, S, sizeof(IO) == 4>(p, w, features, n_in, c_in, K, out, c_out, epi, s) \
-       : launch_conv<IO, G, 4, S, false>(p, w, features, n_in, c_in, K, out, c_out, epi, s))
+#define SSC_CONV_LAUNCH(G, S) \
+  launch_all<IO, G, S>(p, w, features, n_in, c_in, K, out, c_out, epi, s)
 #define SSC_CONV_BY_STEPS(G)                                                            \
   (p.ns == 1 ? SSC_CONV_LAUNCH(G, 1) : p.ns == 2 ? SSC_CONV_LAUNCH(G, 2)                 \
    : p.ns == 3 ? SSC_CONV_LAUNCH(G, 3) : p.ns == 4 ? SSC_CONV_LAUNCH(G, 4)               \

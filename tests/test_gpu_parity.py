@@ -336,6 +336,29 @@ def test_conv_is_reproducible(oracle, device):
     assert torch.equal(a, b)
 
 
+@pytest.mark.parametrize("shape", [(64, 72), (128, 136), (40, 8), (37, 3)])
+def test_conv_lone_last_column_group(shape, oracle, device):
+    """Cout = 64 b + (1..16) with b <= 2: the full blocks of 64 columns take a launch each and
+    the last group of 16 the kernel's one-column-group form (four consumer waves sharing the
+    row blocks of the one group).  Against the oracle, bit-reproducible, and equal up to
+    the order of the float sums to the launch that gives the group a column block of its own
+    (ssc_conv_tuning flag 2)."""
+    from ss_conv import _ext
+    cin, cout = shape
+    print("shape", shape, flush=True)
+    a, ref = _conv_case(oracle, device, 2500, 16, 3, 1, 1, cin, cout, seed=31)
+    b, _ = _conv_case(oracle, device, 2500, 16, 3, 1, 1, cin, cout, seed=31)
+    assert torch.equal(a, b)
+    try:
+        assert _ext._lib.ssc_conv_tuning(1 | 2) == 0
+        c, _ = _conv_case(oracle, device, 2500, 16, 3, 1, 1, cin, cout, seed=31)
+    finally:
+        _ext._lib.ssc_conv_tuning(1)
+    assert rel_l2(a.cpu().numpy(), c.cpu().numpy()) < 1e-6
+    # the sizes the plan functions report follow the flag back
+    assert _ext._lib.ssc_conv_plan_bytes(1000, 27, cin, cout, 1000) > 0
+
+
 def test_conv_inverse(oracle, device):
     """inverse=1 swaps the pair planes: features live on the outputs of the forward rulebook."""
     from ss_conv import _ext
