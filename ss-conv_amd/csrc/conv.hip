@@ -450,106 +450,97 @@ __global__ void __launch_bounds__(256)
 // share_first/share_cnt[t*K + k]: the pairs of offset k that tile t works on.  They
 // begin where the previous tile of the same workgroup stopped and end with the last
 // pair of a row of tile t, rounded up to a whole row block with pairs of the next
-// tile's rows as far as spill[] allows.  One thread per (workgroup, offset) walks
-// the workgroup's tiles in order.
+// tile's rows as far as spill[] allows.
+//
+// range_sched_kernel: one block per workgroup range.  Threads over the offsets walk the range's tiles in order
+// (the shares), then a wave per tile scans its offsets -- kofs[t*K + k] = row blocks of
+// tile t before offset k, tile_nmb[t] = its row blocks, its groups (at least one) -- then
+// the first wave numbers the groups of the range's tiles: tile_loc[t] = groups of the range
+// before tile t, tile_rng[t] = the range, range_grp[w] = groups of range w.  What is left
+// of the prefix over all tiles, the sum over the ranges before a tile's own (at most 256
+// numbers), every block of sched_fill_kernel takes for itself: three dependent launches
+// (shares, counts, a one-block scan) became one.
 __global__ void __launch_bounds__(256)
-    share_kernel(const int32_t *__restrict__ segs, const int32_t *__restrict__ spill, int K,
-                 int n_wg, const int32_t *__restrict__ wg_tile,
-                 int32_t *__restrict__ share_first, int32_t *__restrict__ share_cnt) {
-  const int idx = blockIdx.x * blockDim.x + threadIdx.x;
-  if (idx >= n_wg * K) return;
-  const int w = idx / K, k = idx - w * K;
+    range_sched_kernel(const int32_t *__restrict__ segs, const int32_t *__restrict__ spill, int K,
+                       const int32_t *__restrict__ wg_tile, int32_t *__restrict__ share_first,
+                       int32_t *__restrict__ share_cnt, int32_t *__restrict__ kofs,
+                       int32_t *__restrict__ tile_nmb, int32_t *__restrict__ tile_loc,
+                       int32_t *__restrict__ tile_rng, int32_t *__restrict__ range_grp) {
+  const int w = blockIdx.x;
   const int t0 = wg_tile[w], t1 = wg_tile[w + 1];
-  if (t0 >= t1) return;
-  int s = segs[(int64_t)t0 * K + k];
-  // eight tiles at a time: their loads are issued together, the chain through s is
-  // arithmetic only
-  constexpr int U = 8;
-  for (int tb = t0; tb < t1; tb += U) {
-    int q[U], lim[U];
+  for (int k = threadIdx.x; k < K && t0 < t1; k += blockDim.x) {
+    int s = segs[(int64_t)t0 * K + k];
+    // eight tiles at a time: their loads are issued together, the chain through s is
+    // arithmetic only
+    constexpr int U = 8;
+    for (int tb = t0; tb < t1; tb += U) {
+      int q[U], lim[U];
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const int t = tb + u < t1 ? tb + u : t1 - 1;
-      q[u] = segs[(int64_t)(t + 1) * K + k];    // first pair of a later tile's row
-      lim[u] = spill[(int64_t)(t + 1) * K + k];  // >= q
-    }
+      for (int u = 0; u < U; ++u) {
+        const int t = tb + u < t1 ? tb + u : t1 - 1;
+        q[u] = segs[(int64_t)(t + 1) * K + k];    // first pair of a later tile's row
+        lim[u] = spill[(int64_t)(t + 1) * K + k];  // >= q
+      }
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const int t = tb + u;
-      if (t < t1) {
-        int e = s;
-        if (q[u] > s) {
-          e = s + ((q[u] - s + 15) & ~15);
-          if (e > lim[u]) e = lim[u];
+      for (int u = 0; u < U; ++u) {
+        const int t = tb + u;
+        if (t < t1) {
+          int e = s;
+          if (q[u] > s) {
+            e = s + ((q[u] - s + 15) & ~15);
+            if (e > lim[u]) e = lim[u];
+          }
+          share_first[(int64_t)t * K + k] = s;
+          share_cnt[(int64_t)t * K + k] = e - s;
+          s = e;
         }
-        share_first[(int64_t)t * K + k] = s;
-        share_cnt[(int64_t)t * K + k] = e - s;
-        s = e;
       }
     }
   }
-}
-
-// One wave per tile, lanes over the offsets: kofs[t*K + k] = row blocks of tile t
-// before offset k, tile_nmb[t] = its row blocks, tile_cnt[t] = its groups (at least one).
-__global__ void __launch_bounds__(256)
-    sched_count_kernel(const int32_t *__restrict__ share_cnt, int K,
-                       const int32_t *__restrict__ n_tiles_dev, int32_t *__restrict__ tile_cnt,
-                       int32_t *__restrict__ tile_nmb, int32_t *__restrict__ kofs) {
-  const int lane = threadIdx.x & 63;
-  const int64_t t = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
-  if (t >= n_tiles_dev[0]) return;  // the same for the whole wave
-  int run = 0;
-  for (int k0 = 0; k0 < K; k0 += 64) {
-    const int k = k0 + lane;
-    const int nb = k < K ? (share_cnt[t * K + k] + 15) >> 4 : 0;
-    int incl = nb;
-#pragma unroll
-    for (int d = 1; d < 64; d <<= 1) {
-      int o = __shfl_up(incl, d, 64);
-      if (lane >= d) incl += o;
-    }
-    if (k < K) kofs[t * K + k] = run + incl - nb;
-    run += __shfl(incl, 63, 64);
-  }
-  if (lane == 0) {
-    tile_nmb[t] = run;
-    int groups = (run + 3) >> 2;
-    tile_cnt[t] = groups > 0 ? groups : 1;
-  }
-}
-
-// tile_grp[0..n_tiles]: exclusive prefix of tile_cnt (one block).
-__global__ void __launch_bounds__(kScanThreads)
-    sched_scan_kernel(const int32_t *__restrict__ tile_cnt,
-                      const int32_t *__restrict__ n_tiles_dev, int32_t *__restrict__ tile_grp) {
-  __shared__ int lds[kScanThreads / 64 + 1];
-  const int64_t n_tiles = n_tiles_dev[0];
+  __threadfence_block();
+  __syncthreads();
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  int carry = 0;
-  for (int64_t base = 0; base < n_tiles; base += kScanThreads) {
-    int64_t i = base + threadIdx.x;
-    int v = i < n_tiles ? tile_cnt[i] : 0;
-    int incl = v;
+  for (int64_t t = t0 + wave; t < t1; t += blockDim.x >> 6) {
+    int run = 0;
+    for (int k0 = 0; k0 < K; k0 += 64) {
+      const int k = k0 + lane;
+      const int nb = k < K ? (share_cnt[t * K + k] + 15) >> 4 : 0;
+      int incl = nb;
 #pragma unroll
-    for (int d = 1; d < 64; d <<= 1) {
-      int o = __shfl_up(incl, d, 64);
-      if (lane >= d) incl += o;
+      for (int d = 1; d < 64; d <<= 1) {
+        int o = __shfl_up(incl, d, 64);
+        if (lane >= d) incl += o;
+      }
+      if (k < K) kofs[t * K + k] = run + incl - nb;
+      run += __shfl(incl, 63, 64);
     }
-    if (lane == 63) lds[wave] = incl;
-    __syncthreads();
-    int wave_off = 0, tot = 0;
-#pragma unroll
-    for (int w = 0; w < kScanThreads / 64; ++w) {
-      int x = lds[w];
-      if (w < wave) wave_off += x;
-      tot += x;
+    if (lane == 0) {
+      tile_nmb[t] = run;
+      const int groups = (run + 3) >> 2;
+      tile_loc[t] = groups > 0 ? groups : 1;  // a tile without pairs gets an empty group
     }
-    __syncthreads();
-    if (i < n_tiles) tile_grp[i] = carry + wave_off + incl - v;
-    carry += tot;
   }
-  if (threadIdx.x == 0) tile_grp[n_tiles] = carry;
+  __threadfence_block();
+  __syncthreads();
+  if (wave == 0) {
+    int carry = 0;
+    for (int base = t0; base < t1; base += 64) {
+      const int t = base + lane;
+      const int v = t < t1 ? tile_loc[t] : 0;
+      int incl = v;
+#pragma unroll
+      for (int d = 1; d < 64; d <<= 1) {
+        int o = __shfl_up(incl, d, 64);
+        if (lane >= d) incl += o;
+      }
+      if (t < t1) {
+        tile_loc[t] = carry + incl - v;
+        tile_rng[t] = w;
+      }
+      carry += __shfl(incl, 63, 64);
+    }
+    if (lane == 0) range_grp[w] = carry;
+  }
 }
 
 // 16 threads per (tile, offset): lane i fills slot i of each of its row blocks; the
@@ -559,20 +550,50 @@ __global__ void __launch_bounds__(256)
                       const int32_t *__restrict__ sorted, int64_t pair_stride, int plane_g,
                       const int32_t *__restrict__ share_first,
                       const int32_t *__restrict__ share_cnt, const int32_t *__restrict__ kofs,
-                      const int32_t *__restrict__ tile_nmb, const int32_t *__restrict__ tile_grp,
-                      int K, const int32_t *__restrict__ n_tiles_dev,
+                      const int32_t *__restrict__ tile_nmb, const int32_t *__restrict__ tile_loc,
+                      const int32_t *__restrict__ tile_rng, const int32_t *__restrict__ range_grp,
+                      int n_wg, int32_t *__restrict__ tile_grp, int K,
+                      const int32_t *__restrict__ n_tiles_dev,
                       const int32_t *__restrict__ tile_row0,
                       const int32_t *__restrict__ tile_slot0, int T, uint32_t in_scale,
                       uint32_t in_pad, int out_scale, int k_scale,
                       int32_t *__restrict__ sched_in, int32_t *__restrict__ sched_out,
                       int32_t *__restrict__ grp_meta) {
+  // groups before every range (n_wg <= 256 of them): exclusive prefix of range_grp
+  __shared__ int range_g0[257];
+  {
+    __shared__ int wave_sum[4];
+    const int w = threadIdx.x, wl = w & 63;
+    const int v = w < n_wg ? range_grp[w] : 0;
+    int incl = v;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      int o = __shfl_up(incl, d, 64);
+      if (wl >= d) incl += o;
+    }
+    if (wl == 63) wave_sum[w >> 6] = incl;
+    __syncthreads();
+    int before = 0;
+    for (int i = 0; i < (w >> 6); ++i) before += wave_sum[i];
+    range_g0[w] = before + incl - v;
+    if (w == 255) range_g0[256] = before + incl;
+    __syncthreads();
+  }
   int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   int64_t tk = gid >> 4;
   int lane = (int)(gid & 15);
-  if (tk >= (int64_t)n_tiles_dev[0] * K) return;
+  const int64_t n_tiles = n_tiles_dev[0];
+  if (tk >= n_tiles * K) return;
   int64_t t = tk / K;
   int k = (int)(tk - t * K);
-  const int64_t g0 = tile_grp[t], g1 = tile_grp[t + 1];
+  const int rng = tile_rng[t];
+  const int64_t g0 = range_g0[rng] + tile_loc[t];
+  const int64_t g1 = (t + 1 < n_tiles && tile_rng[t + 1] == rng) ? range_g0[rng] + tile_loc[t + 1]
+                                                                : range_g0[rng + 1];
+  if (k == 0 && lane == 0) {  // the tiles' first groups, for the convolution kernel
+    tile_grp[t] = (int32_t)g0;
+    if (t + 1 == n_tiles) tile_grp[n_tiles] = (int32_t)g1;
+  }
   if (k == 0) {
     for (int64_t g = g0 + lane; g < g1; g += 16) {
       const int rows = tile_row0[t + 1] - tile_row0[t];
@@ -1682,7 +1703,7 @@ struct ConvWs {
   int32_t *sorted;
   uint32_t *bits;
   int32_t *prefix;
-  int32_t *tile_cnt, *tile_nmb, *kofs;
+  int32_t *tile_loc, *tile_nmb, *kofs, *tile_rng, *range_grp;
   int32_t *fine_segs, *range_row0, *tile_row0, *n_tiles_dev;
   int32_t *spill_end, *tile_slot0, *spill, *share_first, *share_cnt;
 };
@@ -1718,7 +1739,7 @@ static size_t conv_scratch_walk(void *base, const ConvPlan &p, int K, int64_t pa
   t.sorted = c.take<int32_t>((size_t)K * 2 * pair_stride);
   t.bits = c.take<uint32_t>((size_t)K * p.words_per_k);
   t.prefix = c.take<int32_t>((size_t)K * p.words_per_k);
-  t.tile_cnt = c.take<int32_t>((size_t)p.n_tiles);
+  t.tile_loc = c.take<int32_t>((size_t)p.n_tiles);
   t.tile_nmb = c.take<int32_t>((size_t)p.n_tiles);
   t.kofs = c.take<int32_t>((size_t)p.n_tiles * K);
   t.fine_segs = c.take<int32_t>((size_t)(p.n_fine + 1) * K);
@@ -1730,13 +1751,15 @@ static size_t conv_scratch_walk(void *base, const ConvPlan &p, int K, int64_t pa
   t.share_first = c.take<int32_t>((size_t)p.n_tiles * K);
   t.share_cnt = c.take<int32_t>((size_t)p.n_tiles * K);
   t.n_tiles_dev = c.take<int32_t>(1);
+  t.tile_rng = c.take<int32_t>((size_t)p.n_tiles + 1);
+  t.range_grp = c.take<int32_t>((size_t)p.n_wg + 1);
   if (w) {
     w->flag = t.flag;
     w->segs = t.segs;
     w->sorted = t.sorted;
     w->bits = t.bits;
     w->prefix = t.prefix;
-    w->tile_cnt = t.tile_cnt;
+    w->tile_loc = t.tile_loc;
     w->tile_nmb = t.tile_nmb;
     w->kofs = t.kofs;
     w->fine_segs = t.fine_segs;
@@ -1748,6 +1771,8 @@ static size_t conv_scratch_walk(void *base, const ConvPlan &p, int K, int64_t pa
     w->share_first = t.share_first;
     w->share_cnt = t.share_cnt;
     w->n_tiles_dev = t.n_tiles_dev;
+    w->tile_rng = t.tile_rng;
+    w->range_grp = t.range_grp;
   }
   return c.used;
 }
@@ -1965,17 +1990,15 @@ static int conv_plan_build(const ConvPlan &p, const ConvWs &w, const int32_t *pa
                      w.flag, pairs, w.sorted, pair_stride, plane_s, pair_num, K, w.n_tiles_dev,
                      w.tile_row0, n_out, w.fine_segs, kSplitGranule, w.spill_end, w.segs, w.spill);
   SSC_LAUNCH_CHECK("tile_segments");
-  hipLaunchKernelGGL(share_kernel, dim3((unsigned)ceil_div((int64_t)p.n_wg * K, 256)), dim3(256),
-                     0, s, w.segs, w.spill, K, p.n_wg, w.wg_tile, w.share_first, w.share_cnt);
-  hipLaunchKernelGGL(sched_count_kernel, dim3((unsigned)ceil_div(p.n_tiles, 4)), dim3(256), 0, s,
-                     w.share_cnt, K, w.n_tiles_dev, w.tile_cnt, w.tile_nmb, w.kofs);
-  hipLaunchKernelGGL(sched_scan_kernel, dim3(1), dim3(kScanThreads), 0, s, w.tile_cnt,
-                     w.n_tiles_dev, w.tile_grp);
+  hipLaunchKernelGGL(range_sched_kernel, dim3((unsigned)p.n_wg), dim3(256), 0, s, w.segs, w.spill,
+                     K, w.wg_tile, w.share_first, w.share_cnt, w.kofs, w.tile_nmb, w.tile_loc,
+                     w.tile_rng, w.range_grp);
   const int frag_bytes = elem_bytes == 2 ? Io<_Float16>::kFragBytes : Io<float>::kFragBytes;
   hipLaunchKernelGGL(sched_fill_kernel, dim3((unsigned)ceil_div(p.n_tiles * K * 16, 256)),
                      dim3(256), 0, s, w.flag, pairs, w.sorted, pair_stride, plane_g,
-                     w.share_first, w.share_cnt, w.kofs, w.tile_nmb, w.tile_grp, K,
-                     w.n_tiles_dev, w.tile_row0, w.tile_slot0, p.T,
+                     w.share_first, w.share_cnt, w.kofs, w.tile_nmb, w.tile_loc, w.tile_rng,
+                     w.range_grp, p.n_wg, w.tile_grp, K, w.n_tiles_dev, w.tile_row0,
+                     w.tile_slot0, p.T,
                      p.gather ? (uint32_t)c_in * (uint32_t)elem_bytes : 1u,
                      p.gather ? kGatherPad : 0xFFFFFFFFu, (16 * p.ncw + 4) * 4,
                      p.ncb * p.nch * frag_bytes, w.sched_in, w.sched_out, w.grp_meta);
