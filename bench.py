@@ -4,7 +4,7 @@ One step = one forward of ss_conv.convolution.Convolution on the voxelised
 batch, with everything the reference runs per training forward: rulebook build
 (count + emit), steerable kernel synthesis, and the MFMA sparse convolution.
 Inputs (voxel indices and features) are resident in HBM before the timed
-region.  Workload: BASELINE config 2 by default (32 clouds x 2048 surface
+region.  Workload: the second benchmark configuration by default (32 clouds x 2048 surface
 points, 64^3 grid, irreps (4,4,4,4) -> (8,8,8,8), i.e. 64 -> 128 channels,
 kernel 3, stride 1, padding 1, fp32).
 
