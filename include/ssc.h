@@ -54,7 +54,9 @@ typedef struct ssc_geometry {
   int32_t padding[3];
   int32_t dilation[3];
   int32_t subm;      /* 1: submanifold (stride forced to 1, padding to ksize/2; indice_conv.h:70-74) */
-  int32_t transpose; /* must be 0: transposed rulebooks are not built */
+  int32_t transpose; /* 1: transposed convolution, out = in*stride - padding + k*dilation with
+                        out_shape from get_deconv_output_size (geometry.h:82-138, 190-237);
+                        ignored when subm is set, as in the reference (indice_conv.h:76-101) */
 } ssc_geometry;
 
 /* ------------------------------------------------------------------------

@@ -110,6 +110,12 @@ def conv_output_size(in_shape, ksize, stride, padding, dilation):
     return out
 
 
+def deconv_output_size(in_shape, ksize, stride, padding, dilation, output_padding):
+    """ss_conv/sp_ops/ops.py:26-36 (the dilation does not enter the reference's formula)."""
+    return [(in_shape[i] - 1) * stride[i] - 2 * padding[i] + ksize[i] + output_padding[i]
+            for i in range(len(in_shape))]
+
+
 def flat_key(idx, shape):
     """((b*X+x)*Y+y)*Z+z, utils/tensorview.h:457-468 plus the batch term of
     src/conv/indice_cuda_functor.cu:60-61."""
@@ -121,7 +127,7 @@ def flat_key(idx, shape):
 # rulebook
 # ---------------------------------------------------------------------------
 def _rulebook(fn_conv, fn_subm, indices, batch_size, in_shape, ksize, stride, padding, dilation,
-              subm, need_grid):
+              subm, need_grid, fn_deconv=None, transpose=False, out_padding=0):
     indices = _i32(indices)
     n = indices.shape[0]
     ks, st, pd, dl = _triple(ksize), _triple(stride), _triple(padding), _triple(dilation)
@@ -132,6 +138,9 @@ def _rulebook(fn_conv, fn_subm, indices, batch_size, in_shape, ksize, stride, pa
     if subm:  # src/conv/indice_conv.h:70-74
         st, pd = [1, 1, 1], [k // 2 for k in ks]
         out_shape = list(in_shape)
+    elif transpose:  # ss_conv/sp_ops/ops.py:65-68, src/conv/indice_conv.h:86-93
+        out_shape = deconv_output_size(list(in_shape), ks, st, pd, dl, _triple(out_padding))
+        fn_conv = fn_deconv
     else:
         out_shape = conv_output_size(list(in_shape), ks, st, pd, dl)
     K = ks[0] * ks[1] * ks[2]
@@ -158,22 +167,27 @@ def _rulebook(fn_conv, fn_subm, indices, batch_size, in_shape, ksize, stride, pa
     return out_idx, pairs, num, out_shape
 
 
-def rulebook(indices, batch_size, in_shape, ksize, stride=1, padding=0, dilation=1, subm=False):
+def rulebook(indices, batch_size, in_shape, ksize, stride=1, padding=0, dilation=1, subm=False,
+             transpose=False, out_padding=0):
     """CPU rulebook of the reference (first-touch output numbering):
-    src/conv/geometry.h:140-189 (regular), 241-288 (submanifold), driven as in
-    src/conv/indice_conv.h:21-131.  Returns (out_indices, pairs[K,2,N], num[K], out_shape)."""
+    src/conv/geometry.h:140-189 (regular), 190-237 (transposed), 241-288 (submanifold), driven
+    as in src/conv/indice_conv.h:21-131.  Returns (out_indices, pairs[K,2,N], num[K], out_shape)."""
     L = lib()
     return _rulebook(L.orc_rulebook_conv, L.orc_rulebook_subm, indices, batch_size, in_shape,
-                     ksize, stride, padding, dilation, subm, need_grid=False)
+                     ksize, stride, padding, dilation, subm, need_grid=False,
+                     fn_deconv=L.orc_rulebook_deconv, transpose=transpose,
+                     out_padding=out_padding)
 
 
 def ref_rulebook(indices, batch_size, in_shape, ksize, stride=1, padding=0, dilation=1,
-                 subm=False):
+                 subm=False, transpose=False, out_padding=0):
     """Same call into the compiled reference sources (oracle/_ref)."""
     R = ref_lib()
     assert R is not None, "oracle/_ref/libssc_ref.so not built"
     return _rulebook(R.ref_rulebook_conv, R.ref_rulebook_subm, indices, batch_size, in_shape,
-                     ksize, stride, padding, dilation, subm, need_grid=True)
+                     ksize, stride, padding, dilation, subm, need_grid=True,
+                     fn_deconv=R.ref_rulebook_deconv, transpose=transpose,
+                     out_padding=out_padding)
 
 
 def canonicalize(out_idx, pairs, num, out_shape):

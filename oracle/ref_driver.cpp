@@ -5,7 +5,8 @@
 // resulting oracle/_ref/libssc_ref.so is used by the tests to pin the C
 // restatement in ssc_oracle.c; nothing in the product loads it.
 //
-//   rulebook:   getIndicePairsConv / getIndicePairsSubM   (src/conv/geometry.h:140-189, 241-288)
+//   rulebook:   getIndicePairsConv / getIndicePairsDeConv / getIndicePairsSubM
+//                                                         (src/conv/geometry.h:140-189, 190-237, 241-288)
 //   max pool:   SparseMaxPoolForwardFunctor<tv::CPU>      (src/pool/indice_maxpool_cpp_functor.cpp:16-35)
 //   conv parts: SparseGatherFunctor / SparseScatterAddFunctor<tv::CPU>
 //                                                         (src/conv/reordering_cpp_functor.cpp:15-44)
@@ -27,6 +28,20 @@ int ref_rulebook_conv(const int *indices, int n_in, int batch, const int *ks, co
   tv::TensorView<int> t_num(pair_num, {K});
   return getIndicePairsConv<int, int, 3>(t_in, t_out, t_grid, t_pairs, t_num, ks, st, pd, dl,
                                          out_shape);
+}
+
+int ref_rulebook_deconv(const int *indices, int n_in, int batch, const int *ks, const int *st,
+                        const int *pd, const int *dl, const int *out_shape, int *out_indices,
+                        int *grid, int *pairs, int *pair_num) {
+  int K = ks[0] * ks[1] * ks[2];
+  int vol = out_shape[0] * out_shape[1] * out_shape[2];
+  tv::TensorView<const int> t_in(indices, {n_in, 4});
+  tv::TensorView<int> t_out(out_indices, {n_in * K, 4});
+  tv::TensorView<int> t_grid(grid, {batch * vol});
+  tv::TensorView<int> t_pairs(pairs, {K, 2, n_in});
+  tv::TensorView<int> t_num(pair_num, {K});
+  return getIndicePairsDeConv<int, int, 3>(t_in, t_out, t_grid, t_pairs, t_num, ks, st, pd, dl,
+                                           out_shape);
 }
 
 int ref_rulebook_subm(const int *indices, int n_in, int batch, const int *ks, const int *st,

@@ -55,6 +55,43 @@ static int orc_valid_out_pos(const int *in, const int *ks, const int *st, const 
   return n;
 }
 
+/* getValidOutPosTranspose, src/conv/geometry.h:82-138: the outputs a transposed
+ * convolution reaches from `in` are in*s - p + k*d per dimension, visited from the
+ * largest downwards, last dimension fastest; the offset of a candidate is its kernel
+ * index sum_dim m_dim * ((out - lo) / d), m = (k1*k2, k2, 1). */
+static int orc_valid_out_pos_transpose(const int *in, const int *ks, const int *st,
+                                       const int *pd, const int *dl, const int *out_shape,
+                                       int *out) {
+  int lo[ND], hi[ND], cnt[ND];
+  for (int a = 0; a < ND; ++a) {
+    lo[a] = in[a] * st[a] - pd[a];
+    hi[a] = lo[a] + (ks[a] - 1) * dl[a];
+    cnt[a] = (hi[a] - lo[a]) / dl[a] + 1;
+  }
+  int n = 0;
+  for (int cx = 0; cx < cnt[0]; ++cx)
+    for (int cy = 0; cy < cnt[1]; ++cy)
+      for (int cz = 0; cz < cnt[2]; ++cz) {
+        int c[ND] = {cx, cy, cz};
+        int ok = 1, off = 0, m = 1;
+        int pos[ND];
+        for (int a = ND - 1; a >= 0; --a) {
+          pos[a] = hi[a] - c[a] * dl[a];
+          if (pos[a] < 0 || pos[a] > out_shape[a] - 1) ok = 0;
+          off += m * (pos[a] - lo[a]) / dl[a];
+          m *= ks[a];
+        }
+        if (ok) {
+          out[n * 4 + 0] = pos[0];
+          out[n * 4 + 1] = pos[1];
+          out[n * 4 + 2] = pos[2];
+          out[n * 4 + 3] = off;
+          ++n;
+        }
+      }
+  return n;
+}
+
 static int64_t orc_flat(const int *pos, const int *shape) {
   /* utils/tensorview.h:457-468 (rowArrayIdx) */
   return ((int64_t)pos[0] * shape[1] + pos[1]) * shape[2] + pos[2];
@@ -66,9 +103,31 @@ static int64_t orc_flat(const int *pos, const int *shape) {
  *   indices[n_in,4] (b,x,y,z); out_indices[cap,4]; pairs[K,2,n_in] pre-filled
  *   with -1 by the caller (indice_conv.h:49); pair_num[K] pre-zeroed.
  * Returns the number of active outputs, or -1 when memory runs out. */
+typedef int (*orc_candidates)(const int *, const int *, const int *, const int *, const int *,
+                              const int *, int *);
+static int orc_rulebook_with(orc_candidates candidates, const int *indices, int n_in, int batch,
+                             const int *ks, const int *st, const int *pd, const int *dl,
+                             const int *out_shape, int *out_indices, int *pairs, int *pair_num);
+
 int orc_rulebook_conv(const int *indices, int n_in, int batch, const int *ks, const int *st,
                       const int *pd, const int *dl, const int *out_shape, int *out_indices,
                       int *pairs, int *pair_num) {
+  return orc_rulebook_with(orc_valid_out_pos, indices, n_in, batch, ks, st, pd, dl, out_shape,
+                           out_indices, pairs, pair_num);
+}
+
+/* Transposed convolution rulebook, src/conv/geometry.h:190-237: the loop of the regular
+ * rulebook over the candidates of getValidOutPosTranspose. */
+int orc_rulebook_deconv(const int *indices, int n_in, int batch, const int *ks, const int *st,
+                        const int *pd, const int *dl, const int *out_shape, int *out_indices,
+                        int *pairs, int *pair_num) {
+  return orc_rulebook_with(orc_valid_out_pos_transpose, indices, n_in, batch, ks, st, pd, dl,
+                           out_shape, out_indices, pairs, pair_num);
+}
+
+static int orc_rulebook_with(orc_candidates candidates, const int *indices, int n_in, int batch,
+                             const int *ks, const int *st, const int *pd, const int *dl,
+                             const int *out_shape, int *out_indices, int *pairs, int *pair_num) {
   int64_t vol = (int64_t)out_shape[0] * out_shape[1] * out_shape[2];
   int K = ks[0] * ks[1] * ks[2];
   int *grid = (int *)malloc(sizeof(int) * (size_t)(vol * batch));
@@ -78,7 +137,7 @@ int orc_rulebook_conv(const int *indices, int n_in, int batch, const int *ks, co
   int n_out = 0;
   for (int j = 0; j < n_in; ++j) {
     int b = indices[j * 4];
-    int nc = orc_valid_out_pos(indices + j * 4 + 1, ks, st, pd, dl, out_shape, cand);
+    int nc = candidates(indices + j * 4 + 1, ks, st, pd, dl, out_shape, cand);
     for (int c = 0; c < nc; ++c) {
       const int *p = cand + c * 4;
       int off = p[3];

@@ -15,13 +15,14 @@ struct Geom {
   int os[3], ks[3], st[3], pd[3], dl[3];
   int K;
   int subm;
+  int tr;  // transposed convolution: out = in * stride - padding + k * dilation
 };
 
 static int make_geom(const ssc_geometry *g, Geom *o) {
   SSC_CHECK(g != nullptr, SSC_EINVAL, "geometry is NULL");
-  SSC_CHECK(g->transpose == 0, SSC_EINVAL, "transposed rulebooks are not supported");
   o->batch = g->batch_size;
   o->subm = g->subm != 0;
+  o->tr = !o->subm && g->transpose != 0;  // src/conv/indice_conv.h:76-101: subm comes first
   o->K = 1;
   for (int a = 0; a < 3; ++a) {
     o->os[a] = g->out_shape[a];
@@ -57,8 +58,15 @@ static inline int64_t geom_cells(const Geom &g) {
 // one dimension: (in + p - k*d) / s when that is a non-negative multiple of s
 // and inside the output extent.  Equivalent to the candidate enumeration of
 // src/conv/geometry.h:18-80 (stride>1 with dilation>1 is rejected on the host).
+// Transposed (`tr`): in*s - p + k*d when inside the extent (src/conv/geometry.h:82-138).
 __device__ __forceinline__ bool tap_to_out(int in, int k, int s, int p, int d, int extent,
-                                           int *out) {
+                                           int *out, bool tr = false) {
+  if (tr) {
+    const int t = in * s - p + k * d;
+    if (t < 0 || t >= extent) return false;
+    *out = t;
+    return true;
+  }
   int t = in + p - k * d;
   if (t < 0) return false;
   int q = t / s;
@@ -73,9 +81,10 @@ __device__ __forceinline__ bool pair_key(const Geom &g, const int32_t *__restric
   int ky = (k / g.ks[2]) % g.ks[1];
   int kx = k / (g.ks[2] * g.ks[1]);
   int ox, oy, oz;
-  if (!tap_to_out(row[1], kx, g.st[0], g.pd[0], g.dl[0], g.os[0], &ox)) return false;
-  if (!tap_to_out(row[2], ky, g.st[1], g.pd[1], g.dl[1], g.os[1], &oy)) return false;
-  if (!tap_to_out(row[3], kz, g.st[2], g.pd[2], g.dl[2], g.os[2], &oz)) return false;
+  const bool tr = g.tr != 0;
+  if (!tap_to_out(row[1], kx, g.st[0], g.pd[0], g.dl[0], g.os[0], &ox, tr)) return false;
+  if (!tap_to_out(row[2], ky, g.st[1], g.pd[1], g.dl[1], g.os[1], &oy, tr)) return false;
+  if (!tap_to_out(row[3], kz, g.st[2], g.pd[2], g.dl[2], g.os[2], &oz, tr)) return false;
   *key = (uint32_t)(((row[0] * g.os[0] + ox) * g.os[1] + oy) * g.os[2] + oz);
   return true;
 }
@@ -141,15 +150,18 @@ __global__ void __launch_bounds__(256)
   int k = kx * g.ks[1] * g.ks[2];
   {
     int ox = 0;
-    const bool okx = live && tap_to_out(row[1], kx, g.st[0], g.pd[0], g.dl[0], g.os[0], &ox);
+    const bool tr = g.tr != 0;
+    const bool okx = live && tap_to_out(row[1], kx, g.st[0], g.pd[0], g.dl[0], g.os[0], &ox, tr);
     for (int ky = 0; ky < g.ks[1]; ++ky) {
       int oy = 0;
-      const bool okxy = okx && tap_to_out(row[2], ky, g.st[1], g.pd[1], g.dl[1], g.os[1], &oy);
+      const bool okxy =
+          okx && tap_to_out(row[2], ky, g.st[1], g.pd[1], g.dl[1], g.os[1], &oy, tr);
       const uint32_t base = (uint32_t)(((row[0] * g.os[0] + ox) * g.os[1] + oy) * g.os[2]);
       uint32_t word = 0xFFFFFFFFu, mask = 0u;
       for (int kz = 0; kz < g.ks[2]; ++kz, ++k) {
         int oz = 0;
-        const bool ok = okxy && tap_to_out(row[3], kz, g.st[2], g.pd[2], g.dl[2], g.os[2], &oz);
+        const bool ok =
+            okxy && tap_to_out(row[3], kz, g.st[2], g.pd[2], g.dl[2], g.os[2], &oz, tr);
         unsigned long long m = __ballot(ok);
         if (lane == 0) chunk_count[(int64_t)k * n_chunks + chunk] = __popcll(m);
         if (ok) {
@@ -182,7 +194,7 @@ struct DenseIn {
 };
 
 static inline bool dense_marking_applies(const Geom &g, int64_t n_in, DenseIn *d) {
-  if (g.subm || (g.os[2] & 31) != 0) return false;
+  if (g.subm || g.tr || (g.os[2] & 31) != 0) return false;
   for (int a = 0; a < 3; ++a)
     if (g.st[a] != 1 || g.dl[a] != 1 || g.ks[a] > 32) return false;
   for (int a = 0; a < 3; ++a) d->U[a] = g.os[a] + g.ks[a] - 1;
@@ -443,17 +455,18 @@ __global__ void __launch_bounds__(256)
   const int kx = blockIdx.y;
   int k = kx * g.ks[1] * g.ks[2];
   int ox = 0;
-  const bool okx = usable && tap_to_out(row[1], kx, g.st[0], g.pd[0], g.dl[0], g.os[0], &ox);
+  const bool tr = g.tr != 0;
+  const bool okx = usable && tap_to_out(row[1], kx, g.st[0], g.pd[0], g.dl[0], g.os[0], &ox, tr);
   const int ksy = KS > 0 ? KS : g.ks[1], ksz = KS > 0 ? KS : g.ks[2];
 #pragma unroll
   for (int ky = 0; ky < ksy; ++ky) {
     int oy = 0;
-    const bool okxy = okx && tap_to_out(row[2], ky, g.st[1], g.pd[1], g.dl[1], g.os[1], &oy);
+    const bool okxy = okx && tap_to_out(row[2], ky, g.st[1], g.pd[1], g.dl[1], g.os[1], &oy, tr);
     const uint32_t base = (uint32_t)(((row[0] * g.os[0] + ox) * g.os[1] + oy) * g.os[2]);
 #pragma unroll
     for (int kz = 0; kz < ksz; ++kz, ++k) {
       int oz = 0;
-      bool ok = okxy && tap_to_out(row[3], kz, g.st[2], g.pd[2], g.dl[2], g.os[2], &oz);
+      bool ok = okxy && tap_to_out(row[3], kz, g.st[2], g.pd[2], g.dl[2], g.os[2], &oz, tr);
       const uint32_t key = base + (uint32_t)oz;
       if (ok && (key >> 5) != word) {
         word = key >> 5;

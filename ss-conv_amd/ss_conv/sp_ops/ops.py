@@ -23,7 +23,8 @@ def get_conv_output_size(input_size, kernel_size, stride, padding, dilation):
 
 
 def get_deconv_output_size(input_size, kernel_size, stride, padding, dilation, output_padding):
-    """Reference: ops.py:26-36 (kept for API parity; transposed rulebooks are not built)."""
+    """(in - 1) s - 2p + k + output_padding per axis (reference: ops.py:26-36; the dilation
+    does not enter)."""
     out = []
     for a in range(len(input_size)):
         if kernel_size[a] == -1:
@@ -55,8 +56,6 @@ def get_indice_pairs(indices, batch_size, spatial_shape, ksize=3, stride=1, padd
         out_shape = get_conv_output_size(spatial_shape, ksize, stride, padding, dilation)
     if ndim != 3:
         raise NotImplementedError("only 3-d rulebooks are built")
-    if transpose:
-        raise NotImplementedError("transposed rulebooks are not built")
     return _ext.get_indice_pairs_3d(indices, batch_size, list(out_shape), list(spatial_shape),
                                     ksize, stride, padding, dilation, out_padding, int(subm),
                                     int(transpose))

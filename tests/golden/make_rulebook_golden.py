@@ -1,7 +1,7 @@
-"""Writes tests/golden/rulebook_cases.npz from the REFERENCE's own CPU rulebook
-(src/conv/geometry.h:140-189, 241-288), compiled where it lies by oracle/Makefile
-into oracle/_ref/libssc_ref.so.  Run once in a container that has
-/root/reference; the .npz (inputs and expected outputs only) is committed.
+"""Writes tests/golden/rulebook_cases.npz and rulebook_transposed_cases.npz from the
+REFERENCE's own CPU rulebook (src/conv/geometry.h:140-189, 190-237, 241-288), compiled where
+it lies by oracle/Makefile into oracle/_ref/libssc_ref.so.  Run once in a container that has
+/root/reference; the .npz files (inputs and expected outputs only) are committed.
 
     python tests/golden/make_rulebook_golden.py
 """
@@ -26,6 +26,18 @@ CASES = [
     ("subm_k3", 2, 8, 100, 3, 1, 1, 1, True, 8),
     ("subm_k5", 2, 10, 150, 5, 1, 2, 1, True, 9),
     ("unsorted_rows", 2, 8, 60, 3, 1, 1, 1, False, 10),
+]
+
+
+TRANSPOSED_CASES = [
+    # name, batch, grid, n_voxels, kernel, stride, padding, dilation, output_padding, seed
+    ("t_k3s2p1", 2, 5, 40, 3, 2, 1, 1, 0, 21),
+    ("t_k3s2p1o1", 2, 5, 40, 3, 2, 1, 1, 1, 22),
+    ("t_k2s2p0", 3, 4, 30, 2, 2, 0, 1, 0, 23),
+    ("t_k3s1p1", 2, 8, 60, 3, 1, 1, 1, 0, 24),
+    ("t_k3s1p0d2", 2, 7, 50, 3, 1, 0, 2, 0, 25),
+    ("t_k4s3p1", 1, 4, 20, 4, 3, 1, 1, 0, 26),
+    ("t_k5s1p2", 1, 6, 40, 5, 1, 2, 1, 0, 27),
 ]
 
 
@@ -60,6 +72,20 @@ def main():
     out["known/num"] = num
     np.savez_compressed(os.path.join(HERE, "rulebook_cases.npz"), **out)
     print("wrote", len(out) // 5, "cases")
+    out = {}
+    for name, batch, grid, n, k, s, p, d, op, seed in TRANSPOSED_CASES:
+        rng = np.random.default_rng(seed)
+        idx = voxels(rng, batch, grid, n, shuffle=False)
+        o_idx, pairs, num, o_shape = O.ref_rulebook(idx, batch, [grid] * 3, k, s, p, d,
+                                                    transpose=True, out_padding=op)
+        out[name + "/params"] = np.array([batch, grid, k, s, p, d, op] + list(o_shape),
+                                         dtype=np.int32)
+        out[name + "/indices"] = idx
+        out[name + "/out_indices"] = o_idx
+        out[name + "/pairs"] = pairs
+        out[name + "/num"] = num
+    np.savez_compressed(os.path.join(HERE, "rulebook_transposed_cases.npz"), **out)
+    print("wrote", len(out) // 5, "transposed cases")
 
 
 if __name__ == "__main__":

@@ -55,12 +55,25 @@ def test_rulebook_full_size_matches_oracle(name, oracle, device):
 
 @pytest.mark.parametrize("name", FULL)
 def test_conv_full_size(name, oracle, device):
+    cfg = synth.CONFIGS[name]
+    _conv_full_size(name, _channels(cfg, "mult_in"), _channels(cfg, "mult_out"), oracle, device,
+                    with_oracle=name != "cfg5")  # cfg5's CPU restatement takes minutes
+
+
+@pytest.mark.parametrize("channels", [(64, 72), (128, 136), (152, 8)])
+def test_conv_full_size_lone_last_group(channels, oracle, device):
+    """Channel counts whose last group of 16 output columns runs the kernel's
+    one-column-group form (both gradients included: the input gradient of 64 -> 72 is a
+    72 -> 64 convolution), on the clouds of the second configuration."""
+    _conv_full_size("cfg2", channels[0], channels[1], oracle, device, with_oracle=True)
+
+
+def _conv_full_size(name, cin, cout, oracle, device, with_oracle):
     from ss_conv import _ext
-    print("config", name, flush=True)
+    print("config", name, cin, cout, flush=True)
     cfg, idx = _voxels(name)
     k = cfg["kernel"]
     K = k ** 3
-    cin, cout = _channels(cfg, "mult_in"), _channels(cfg, "mult_out")
     out_idx, pairs, num = _gpu_rulebook(cfg, idx, device)
     n_in, n_out = idx.shape[0], out_idx.shape[0]
     nums = num.cpu().numpy()
@@ -101,7 +114,7 @@ def test_conv_full_size(name, oracle, device):
     # rows no pair lands on are zero (every active output has at least one pair here, so
     # this holds trivially unless the rulebook and the convolution disagree on n_out)
     assert out.shape == (n_out, cout) and bool(torch.isfinite(out).all())
-    if name != "cfg5":  # the CPU restatement of this size takes seconds; cfg5's takes minutes
+    if with_oracle:  # the CPU restatement of these sizes takes seconds
         o_ref = oracle.conv_fwd(f.cpu().numpy(), w.cpu().numpy(), pairs.cpu().numpy(), nums,
                                 n_out, matmul=np.matmul)
         assert rel_l2(out.cpu().numpy(), o_ref) < REL_L2

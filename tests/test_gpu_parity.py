@@ -69,6 +69,96 @@ def test_rulebook_matches_oracle(case, oracle, device):
     assert np.array_equal(g_pairs, o_pairs)
 
 
+TRANSPOSED_CASES = [
+    # batch, grid, n, k, stride, pad, dil, output_padding
+    (2, 5, 40, 3, 2, 1, 1, 0),
+    (2, 5, 40, 3, 2, 1, 1, 1),
+    (3, 4, 30, 2, 2, 0, 1, 0),
+    (2, 8, 60, 3, 1, 1, 1, 0),
+    (2, 7, 50, 3, 1, 0, 2, 0),
+    (1, 4, 20, 4, 3, 1, 1, 0),
+    (2, 16, 1200, 3, 2, 1, 1, 1),
+    (1, 6, 216, 3, 2, 0, 1, 0),   # full grid
+]
+
+
+@pytest.mark.parametrize("case", TRANSPOSED_CASES)
+def test_transposed_rulebook_matches_oracle(case, oracle, device):
+    """transpose=True (src/conv/geometry.h:82-138, 190-237): bit-exact against the oracle in
+    canonical order, and against the golden rulebooks of the reference's own code where the
+    case is one of them."""
+    from ss_conv.sp_ops.ops import get_indice_pairs
+    batch, grid, n, k, s, p, d, op = case
+    rng = np.random.default_rng(hash(case) % 2 ** 31)
+    idx = random_voxels(rng, batch, grid, n)
+    print("case", case, flush=True)
+    o_idx, o_pairs, o_num, o_shape = oracle.rulebook(idx, batch, [grid] * 3, k, s, p, d,
+                                                     transpose=True, out_padding=op)
+    o_idx, o_pairs, o_num = oracle.canonicalize(o_idx, o_pairs, o_num, o_shape)
+    g_idx, g_pairs, g_num = get_indice_pairs(torch.from_numpy(idx).to(device), batch, [grid] * 3,
+                                             k, s, p, d, op, False, True)
+    assert np.array_equal(g_num.cpu().numpy(), o_num)
+    assert np.array_equal(g_idx.cpu().numpy(), o_idx)
+    assert np.array_equal(g_pairs.cpu().numpy(), o_pairs)
+
+
+def test_transposed_rulebook_matches_reference_golden(oracle, device):
+    import os
+    from ss_conv.sp_ops.ops import get_indice_pairs
+    z = np.load(os.path.join(os.path.dirname(__file__), "golden", "rulebook_transposed_cases.npz"))
+    for name in sorted({k.split("/")[0] for k in z.files}):
+        batch, grid, k, s, p, d, op = [int(v) for v in z[name + "/params"][:7]]
+        shape = [int(v) for v in z[name + "/params"][7:]]
+        want = oracle.canonicalize(z[name + "/out_indices"], z[name + "/pairs"], z[name + "/num"],
+                                   shape)
+        got = get_indice_pairs(torch.from_numpy(z[name + "/indices"]).to(device), batch,
+                               [grid] * 3, k, s, p, d, op, False, True)
+        for g, w in zip(got, want):
+            assert np.array_equal(g.cpu().numpy(), w), name
+
+
+def test_transposed_convolution_layer(oracle, device):
+    """SparseConvolution(transposed=True), forward and both gradients, against the oracle's
+    convolution over the oracle's transposed rulebook, and against torch's dense
+    conv_transpose3d of the same layer (an independent statement: the reference's
+    transposed convolution reaches out = in*s - p + k, torch's the same cells)."""
+    from ss_conv.sp_ops.conv import SparseConvolution
+    from ss_conv.sp_ops.tensor import SparseTensor
+    rng = np.random.default_rng(77)
+    batch, grid, n, cin, cout, k, s, p, op = 2, 6, 70, 5, 7, 3, 2, 1, 1
+    idx = random_voxels(rng, batch, grid, n)
+    x = rng.normal(size=(n, cin)).astype(np.float32)
+    layer = SparseConvolution(3, cin, cout, k, stride=s, padding=p, output_padding=op, bias=False,
+                              transposed=True).to(device)
+    w = layer.weight.detach().cpu().numpy().reshape(k ** 3, cin, cout)
+    feats = torch.from_numpy(x).to(device).requires_grad_(True)
+    out = layer(SparseTensor(feats, torch.from_numpy(idx).to(device), [grid] * 3, batch))
+    o_idx, o_pairs, o_num, o_shape = oracle.rulebook(idx, batch, [grid] * 3, k, s, p, 1,
+                                                     transpose=True, out_padding=op)
+    o_idx, o_pairs, o_num = oracle.canonicalize(o_idx, o_pairs, o_num, o_shape)
+    assert list(out.spatial_shape) == o_shape == [(grid - 1) * s - 2 * p + k + op] * 3
+    assert np.array_equal(out.indices.cpu().numpy(), o_idx)
+    ref = oracle.conv_fwd(x, w, o_pairs, o_num, o_idx.shape[0])
+    assert rel_l2(out.features.detach().cpu().numpy(), ref) < REL_L2
+    # dense statement: torch's transposed convolution wants [Cin, Cout, kx, ky, kz]
+    dense_in = torch.zeros((batch, cin, grid, grid, grid), dtype=torch.float64)
+    dense_in[idx[:, 0], :, idx[:, 1], idx[:, 2], idx[:, 3]] = torch.from_numpy(x).double()
+    wd = torch.from_numpy(w).double().reshape(k, k, k, cin, cout).permute(3, 4, 0, 1, 2)
+    dense = torch.nn.functional.conv_transpose3d(dense_in, wd, stride=s, padding=p,
+                                                 output_padding=op)
+    got = dense[o_idx[:, 0], :, o_idx[:, 1], o_idx[:, 2], o_idx[:, 3]].numpy()
+    assert rel_l2(out.features.detach().cpu().numpy(), got) < REL_L2
+    mask = torch.ones(dense.shape[0], dense.shape[2], dense.shape[3], dense.shape[4], dtype=torch.bool)
+    mask[o_idx[:, 0], o_idx[:, 1], o_idx[:, 2], o_idx[:, 3]] = False
+    assert float(dense.permute(0, 2, 3, 4, 1)[mask].abs().max()) == 0.0  # nothing outside the active rows
+    # gradients through the same pairs
+    g_out = rng.normal(size=ref.shape).astype(np.float32)
+    out.features.backward(torch.from_numpy(g_out).to(device))
+    d_in, d_w = oracle.conv_bwd(x, w, g_out, o_pairs, o_num)
+    assert rel_l2(feats.grad.cpu().numpy(), d_in) < REL_L2
+    assert rel_l2(layer.weight.grad.cpu().numpy().reshape(k ** 3, cin, cout), d_w) < REL_L2
+
+
 @pytest.mark.parametrize("case", [RULEBOOK_CASES[1], RULEBOOK_CASES[4], RULEBOOK_CASES[8]])
 @pytest.mark.parametrize("shuffle", [False, True])
 def test_rulebook_count_then_emit_entry_points(case, shuffle, device):

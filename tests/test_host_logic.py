@@ -44,8 +44,7 @@ def test_host_argument_checks_need_no_gpu():
     rc = lib.ssc_rulebook_count(None, 10, ctypes.byref(g), None, 0, ctypes.byref(n_out), None)
     assert rc == _ext.SSC_EINVAL
     g = _ext._geometry(1, [8] * 3, [3] * 3, [1] * 3, [1] * 3, [1] * 3, 0, 1)
-    assert lib.ssc_rulebook_count(None, 10, ctypes.byref(g), None, 0, ctypes.byref(n_out),
-                                  None) == _ext.SSC_EINVAL  # transposed
+    assert lib.ssc_rulebook_workspace_bytes(ctypes.byref(g), 10) > 0  # transposed: a geometry
     g = _ext._geometry(64, [512] * 3, [3] * 3, [1] * 3, [1] * 3, [1] * 3, 0, 0)
     assert lib.ssc_rulebook_count(None, 10, ctypes.byref(g), None, 0, ctypes.byref(n_out),
                                   None) == _ext.SSC_ERUNTIME  # 64 * 512^3 >= 2^31
@@ -368,7 +367,7 @@ def test_synthetic_generator_is_seeded():
 def test_layers_outside_the_native_layouts():
     """A gated activation whose first entry is not a scalar field keeps the torch code (the
     gate tables would ask for gates the reference never counts); a transposed convolution
-    is refused when it is constructed, not at its first forward."""
+    is a layer like any other (its output size follows ops.py:26-36 of the reference)."""
     from ss_conv import bnact
     from ss_conv.activation import Activation
     from ss_conv.sp_ops.conv import SparseConvolution
@@ -378,8 +377,11 @@ def test_layers_outside_the_native_layouts():
     assert not bnact.canonical([(4, 0), (2, 0)])
     act = Activation([(4, 1), (2, 2)], (torch.relu, torch.sigmoid))
     assert not act._kernel_ok
-    with pytest.raises(NotImplementedError):
-        SparseConvolution(3, 4, 4, 3, transposed=True)
+    layer = SparseConvolution(3, 4, 4, 3, stride=2, padding=1, output_padding=1, transposed=True)
+    assert layer.transposed and layer.output_padding == [1, 1, 1]
+    from ss_conv.sp_ops.ops import get_deconv_output_size
+    assert get_deconv_output_size([5, 6, 7], [3] * 3, [2] * 3, [1] * 3, [1] * 3, [1] * 3) == \
+        [10, 12, 14]
 
 
 def test_epilogue_layout_keeps_gates_with_their_columns():

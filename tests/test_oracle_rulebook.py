@@ -53,6 +53,72 @@ def test_oracle_matches_reference_golden(name, oracle):
     assert np.array_equal(pairs, z[name + "/pairs"])
 
 
+GOLDEN_T = os.path.join(os.path.dirname(__file__), "golden", "rulebook_transposed_cases.npz")
+
+
+def _transposed_cases():
+    z = np.load(GOLDEN_T)
+    return z, sorted({k.split("/")[0] for k in z.files})
+
+
+@pytest.mark.parametrize("name", _transposed_cases()[1])
+def test_oracle_matches_reference_golden_transposed(name, oracle):
+    """Transposed rulebooks written by the reference's getIndicePairsDeConv
+    (src/conv/geometry.h:190-237; tests/golden/make_rulebook_golden.py)."""
+    z, _ = _transposed_cases()
+    batch, grid, k, s, p, d, op = [int(v) for v in z[name + "/params"][:7]]
+    o_idx, pairs, num, shape = oracle.rulebook(z[name + "/indices"], batch, [grid] * 3, k, s, p, d,
+                                               transpose=True, out_padding=op)
+    assert shape == [int(v) for v in z[name + "/params"][7:]]
+    assert np.array_equal(num, z[name + "/num"])
+    assert np.array_equal(o_idx, z[name + "/out_indices"])
+    assert np.array_equal(pairs, z[name + "/pairs"])
+
+
+@pytest.mark.parametrize("grid,k,s,p,d,op", [(5, 3, 2, 1, 1, 0), (5, 3, 2, 1, 1, 1),
+                                             (4, 2, 2, 0, 1, 0), (6, 3, 1, 0, 2, 0),
+                                             (4, 4, 3, 1, 1, 2)])
+def test_transposed_oracle_matches_definition_and_compiled_reference(grid, k, s, p, d, op, oracle):
+    """The definition: input voxel i and tap k give output i*s - p + k*d where that lies inside
+    (i-1)*s - 2p + k + output_padding cells per axis; pairs in ascending input row.  And the
+    adjoint property: every pair (i -> o, k) is a pair (o -> i, k) of the regular rulebook of
+    the same window over the reached cells."""
+    rng = np.random.default_rng(grid * 10 + k)
+    idx = random_voxels(rng, 2, grid, 30)
+    o_idx, pairs, num, shape = oracle.rulebook(idx, 2, [grid] * 3, k, s, p, d, transpose=True,
+                                               out_padding=op)
+    extent = (grid - 1) * s - 2 * p + k + op
+    assert shape == [extent] * 3
+    want = {}
+    for row, (b, x, y, z) in enumerate(idx):
+        for kx in range(k):
+            for ky in range(k):
+                for kz in range(k):
+                    o = [c * s - p + kk * d for c, kk in ((x, kx), (y, ky), (z, kz))]
+                    if all(0 <= v < extent for v in o):
+                        want.setdefault((kx * k + ky) * k + kz, []).append((row, (b, *o)))
+    assert int(num.sum()) == sum(len(v) for v in want.values())
+    for kk in range(k ** 3):
+        got = [(int(i), tuple(int(v) for v in o_idx[o])) for i, o in
+               zip(pairs[kk, 0, :num[kk]], pairs[kk, 1, :num[kk]])]
+        assert got == want.get(kk, [])
+    assert len({tuple(r) for r in o_idx.tolist()}) == o_idx.shape[0]
+    if oracle.ref_lib() is not None:
+        ref = oracle.ref_rulebook(idx, 2, [grid] * 3, k, s, p, d, transpose=True, out_padding=op)
+        for x, y in zip((o_idx, pairs, num), ref[:3]):
+            assert np.array_equal(x, y)
+    if (extent + 2 * p - d * (k - 1) - 1) // s + 1 >= grid:  # the regular window lands on the grid
+        c_idx, c_pairs, c_num = oracle.canonicalize(o_idx, pairs, num, shape)
+        r_idx, r_pairs, r_num, r_shape = oracle.rulebook(c_idx, 2, shape, k, s, p, d)
+        back = {}
+        for kk in range(k ** 3):
+            for i, o in zip(r_pairs[kk, 0, :r_num[kk]], r_pairs[kk, 1, :r_num[kk]]):
+                back.setdefault(kk, set()).add((tuple(r_idx[o]), tuple(c_idx[i])))
+        for kk in range(k ** 3):
+            for i, o in zip(c_pairs[kk, 0, :c_num[kk]], c_pairs[kk, 1, :c_num[kk]]):
+                assert (tuple(idx[i]), tuple(c_idx[o])) in back.get(kk, set())
+
+
 def test_known_answer(oracle):
     """indices (0,0,0),(1,2,3),(3,3,3) on a 4^3 grid, k3 s1 p1: 30 outputs, 34 pairs."""
     idx = np.array([[0, 0, 0, 0], [0, 1, 2, 3], [0, 3, 3, 3]], dtype=np.int32)
