@@ -449,6 +449,50 @@ def test_conv_lone_last_column_group(shape, oracle, device):
     assert _ext._lib.ssc_conv_plan_bytes(1000, 27, cin, cout, 1000) > 0
 
 
+def test_conv_random_layers(device):
+    """Forty seeded random layers -- channel counts on both sides of every block and chunk
+    boundary (1 ... 200 in, 1 ... 152 out), kernels 1-3, strides 1-2, regular, submanifold and
+    transposed rulebooks -- forward and both gradients against a float64 statement of the
+    same sums (one GEMM and one index_add per offset, src/conv/indice_conv.h:296-338,
+    385-421) evaluated with torch on the GPU."""
+    from ss_conv import _ext
+    from ss_conv.sp_ops.ops import get_indice_pairs
+    rng = np.random.default_rng(2024)
+    for it in range(40):
+        batch, grid, n = int(rng.integers(1, 4)), int(rng.integers(5, 18)), int(rng.integers(1, 3000))
+        k, s = int(rng.choice([1, 2, 3])), int(rng.choice([1, 2]))
+        p = int(rng.integers(0, k))
+        tr = bool(rng.integers(0, 4) == 0)
+        subm = (not tr) and k == 3 and bool(rng.integers(0, 5) == 0)
+        cin = int(rng.choice([1, 3, 5, 8, 16, 37, 40, 64, 72, 100, 128, 152, 200]))
+        cout = int(rng.choice([1, 3, 7, 8, 16, 17, 24, 64, 65, 72, 80, 96, 129, 136, 144, 152]))
+        print("layer", it, (batch, grid, n, k, s, p, tr, subm, cin, cout), flush=True)
+        idx = torch.from_numpy(random_voxels(rng, batch, grid, min(n, batch * grid ** 3))).to(device)
+        o_idx, pairs, num = get_indice_pairs(idx, batch, [grid] * 3, k, s, p, 1, 0, subm, tr)
+        n_in, n_out, K = idx.shape[0], o_idx.shape[0], k ** 3
+        gen = torch.Generator(device).manual_seed(it)
+        f = torch.randn((n_in, cin), device=device, generator=gen)
+        w = torch.randn((K, cin, cout), device=device, generator=gen) / (K * cin) ** 0.5
+        go = torch.randn((n_out, cout), device=device, generator=gen)
+        w5 = w.reshape(k, k, k, cin, cout)
+        out = _ext.indice_conv_fp32(f, w5, pairs, num, n_out, 0, int(subm))
+        d_in, d_w = _ext.indice_conv_backward_fp32(f, w5, go, pairs, num, 0, int(subm))
+        ref = torch.zeros((n_out, cout), dtype=torch.float64, device=device)
+        ref_in = torch.zeros((n_in, cin), dtype=torch.float64, device=device)
+        ref_w = torch.zeros((K, cin, cout), dtype=torch.float64, device=device)
+        for kk, m in enumerate(num.cpu().tolist()):
+            if m:
+                i_rows, o_rows = pairs[kk, 0, :m].long(), pairs[kk, 1, :m].long()
+                fi, gk, wk = f[i_rows].double(), go[o_rows].double(), w[kk].double()
+                ref.index_add_(0, o_rows, fi @ wk)
+                ref_in.index_add_(0, i_rows, gk @ wk.t())
+                ref_w[kk] = fi.t() @ gk
+        for got, want in ((out, ref), (d_in, ref_in), (d_w.reshape(K, cin, cout), ref_w)):
+            if want.numel():
+                err = float((got.double() - want).norm() / want.norm().clamp_min(1e-30))
+                assert err < REL_L2, (it, err)
+
+
 def test_conv_inverse(oracle, device):
     """inverse=1 swaps the pair planes: features live on the outputs of the forward rulebook."""
     from ss_conv import _ext
