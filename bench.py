@@ -62,6 +62,10 @@ def parse_args():
                          "Voxel2Point, evaluation mode) and print, stage by stage, pairs, flops "
                          "and the convolution kernel's time and fraction of the fp32 MFMA peak; "
                          "table on stderr")
+    ap.add_argument("--thin-layers", action="store_true",
+                    help="also time layers whose last group of 16 output columns would be alone "
+                         "in its block of 64 (64->72, 128->136, 152->8, 128->16), with the "
+                         "kernel's one-column-group form and without (table on stderr)")
     ap.add_argument("--breakdown", action="store_true",
                     help="also print per-phase timings to stderr")
     return ap.parse_args()
@@ -380,6 +384,48 @@ def build_backbone(torch, synth, dev, seed):
     return backbone
 
 
+def thin_layer_table(torch, _ext, synth, dev, seed):
+    """Layers with Cout = 64 b + (1 ... 16), b <= 2, on the clouds of the second and third
+    configuration: the convolution kernel's time (HIP events around its launches) with the
+    last column group shared by the four consumer waves (the default) and with the group
+    in a column block of its own (ssc_conv_tuning flag 2)."""
+    from ss_conv.sp_ops.ops import get_indice_pairs
+    rows = []
+    for name, cin, cout, k, stride, pad in (("cfg2", 64, 72, 3, 1, 1), ("cfg2", 128, 136, 3, 1, 1),
+                                            ("cfg2", 152, 8, 3, 1, 1), ("cfg3", 128, 16, 3, 2, 1)):
+        cfg = synth.CONFIGS[name]
+        pts, _, ids = synth.config_clouds(name, seed)
+        idx = torch.from_numpy(synth.voxel_indices(pts, ids, cfg["grid"])).to(dev)
+        o_idx, pairs, num = get_indice_pairs(idx, cfg["batch"], [cfg["grid"]] * 3, k, stride, pad)
+        P, K = int(num.sum().item()), k ** 3
+        f = torch.randn(idx.shape[0], cin, device=dev)
+        w = torch.randn(k, k, k, cin, cout, device=dev) / (K * cin) ** 0.5
+        times, outs = [], []
+        for flags in (1, 1 | 2):
+            _ext._lib.ssc_conv_tuning(flags)
+            pr = pairs.clone()  # a rulebook without a plan of the other form
+            try:
+                for _ in range(3):
+                    out = _ext.indice_conv_fp32(f, w, pr, num, o_idx.shape[0], 0, 0)
+                torch.cuda.synchronize()
+                _ext.profile_conv(True)
+                for _ in range(10):
+                    out = _ext.indice_conv_fp32(f, w, pr, num, o_idx.shape[0], 0, 0)
+                ms = _ext.profile_conv_read()
+            finally:
+                _ext.profile_conv(False)
+                _ext._lib.ssc_conv_tuning(1)
+            times.append(sum(ms) / len(ms))
+            outs.append(out)
+        err = float((outs[0] - outs[1]).norm() / outs[1].norm())
+        gf = 2.0 * P * cin * cout / 1e9
+        rows.append("%s clouds, %3d -> %3d ch, k%d s%d: %d pairs, %.3f GFLOP; kernel %.3f ms (%.1f%% "
+                    "of fp32 MFMA peak), %.3f ms with the group in a block of its own; rel-L2 "
+                    "between the two %.1e"
+                    % (name, cin, cout, k, stride, P, gf, times[0], gf / times[0] / 1.573, times[1], err))
+    print("\n".join(rows), file=sys.stderr)
+
+
 def backbone_table(torch, _ext, synth, dev, seed, n=5, warm=2):
     """Runs the backbone of the fourth configuration and prints one row per convolution
     stage: rows, pairs, flops, the MFMA kernel's time (HIP events around its launch) and
@@ -594,6 +640,8 @@ def main():
         print("\n".join(rows), file=sys.stderr)
     if args.backbone:
         backbone_table(torch, _ext, synth, dev, args.seed)
+    if args.thin_layers:
+        thin_layer_table(torch, _ext, synth, dev, args.seed)
 
     if not args.no_cpu_baseline:
         w = conv.kernel().detach().permute(2, 3, 4, 1, 0).reshape(K, c_in, c_out).cpu().numpy()
