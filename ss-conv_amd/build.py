@@ -13,7 +13,7 @@ ROOT = os.path.dirname(HERE)
 CSRC = os.path.join(HERE, "csrc")
 LIB_DIR = os.path.join(HERE, "lib")
 LIB = os.path.join(LIB_DIR, "libssc.so")
-SOURCES = ["common.hip", "rulebook.hip", "conv.hip", "conv_bwd.hip", "combine.hip", "pool.hip",
+SOURCES = ["common.hip", "rulebook.hip", "conv.hip", "conv_tail.hip", "conv_bwd.hip", "combine.hip", "pool.hip",
            "voxel.hip", "bnact.hip"]
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",
