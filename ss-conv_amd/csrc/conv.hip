@@ -803,19 +803,25 @@ static int launch_all(const ConvPlan &p, const ConvWs &w, const IO *features, in
   const bool with_epi = kFloat && epi.mode != nullptr;
   for (int l = 0; l < p.n_launch; ++l) {
     const int col_base = l * p.n_colblk * 16 * p.ncw;
-    const int rc = with_epi ? launch_conv<IO, GATHER, 4, NS, kFloat, false>(
-                                  p, w, features, n_in, c_in, K, out, c_out, col_base, epi, s)
-                            : launch_conv<IO, GATHER, 4, NS, false, false>(
-                                  p, w, features, n_in, c_in, K, out, c_out, col_base, epi, s);
+    int rc;
+    if constexpr (kFloat) {
+      rc = with_epi ? launch_conv_f32<GATHER, NS, true, false>(p, w, features, n_in, c_in, K, out,
+                                                               c_out, col_base, epi, s)
+                    : launch_conv<float, GATHER, 4, NS, false, false>(p, w, features, n_in, c_in, K,
+                                                                      out, c_out, col_base, epi, s);
+    } else {
+      rc = launch_conv<IO, GATHER, 4, NS, false, false>(p, w, features, n_in, c_in, K, out, c_out,
+                                                        col_base, epi, s);
+    }
     if (rc != SSC_OK) return rc;
   }
   if (p.has_tail) {
     const int col_base = (p.ncb - 1) * 16;
     if constexpr (kFloat) {
-      return with_epi ? launch_conv_tail<GATHER, NS, true>(p, w, features, n_in, c_in, K, out,
-                                                           c_out, col_base, epi, s)
-                      : launch_conv_tail<GATHER, NS, false>(p, w, features, n_in, c_in, K, out,
-                                                            c_out, col_base, epi, s);
+      return with_epi ? launch_conv_f32<GATHER, NS, true, true>(p, w, features, n_in, c_in, K, out,
+                                                                c_out, col_base, epi, s)
+                      : launch_conv_f32<GATHER, NS, false, true>(p, w, features, n_in, c_in, K, out,
+                                                                 c_out, col_base, epi, s);
     } else {
       SSC_CHECK(false, SSC_ERUNTIME, "the one-column-group form is built for float rows");
     }

@@ -1,7 +1,8 @@
 // The convolution kernel (conv_fwd_kernel), what a launch of it needs to know of a plan,
-// and the launch itself.  Two translation units instantiate it: conv.hip the form with
-// column blocks of four groups, conv_tail.hip the one-column-group form -- compiled side
-// by side, the two halves of the instances take half the time.
+// and the launch itself.  Four translation units instantiate it: conv.hip the plain form
+// (float and half rows), conv_epi.hip the one with the epilogue, conv_tail.hip and
+// conv_tail_epi.hip the one-column-group form without and with it -- compiled side by
+// side, the quarters of the instances take a third of the time.
 #pragma once
 #include "ssc_common.h"
 
@@ -1050,10 +1051,11 @@ inline int launch_conv(const ConvPlan &p, const ConvWs &w, const IO *features, i
   return SSC_OK;
 }
 
-// The one-column-group form on float rows (defined and instantiated in conv_tail.hip).
-template <int GATHER, int NS, bool EPI>
-int launch_conv_tail(const ConvPlan &p, const ConvWs &w, const float *features, int64_t n_in,
-                     int c_in, int K, float *out, int c_out, int col_base,
-                     const ConvEpilogue &epi, hipStream_t s);
+// The instances on float rows that conv.hip does not compile itself (conv_instances.h):
+// with the epilogue, and the one-column-group form with and without it.
+template <int GATHER, int NS, bool EPI, bool TAIL>
+int launch_conv_f32(const ConvPlan &p, const ConvWs &w, const float *features, int64_t n_in,
+                    int c_in, int K, float *out, int c_out, int col_base,
+                    const ConvEpilogue &epi, hipStream_t s);
 
 }  // namespace ssc
