@@ -452,7 +452,8 @@ __global__ void __launch_bounds__(256)
 // of the prefix over all tiles, the sum over the ranges before a tile's own (at most 256
 // numbers), every block of sched_fill_kernel takes for itself: three dependent launches
 // (shares, counts, a one-block scan) became one.
-__global__ void __launch_bounds__(256)
+constexpr int kRangeSchedThreads = 1024;  // sixteen tiles at a time in the second step
+__global__ void __launch_bounds__(kRangeSchedThreads)
     range_sched_kernel(const int32_t *__restrict__ segs, const int32_t *__restrict__ spill, int K,
                        const int32_t *__restrict__ wg_tile, int32_t *__restrict__ share_first,
                        int32_t *__restrict__ share_cnt, int32_t *__restrict__ kofs,
@@ -537,6 +538,8 @@ __global__ void __launch_bounds__(256)
 
 // 16 threads per (tile, offset): lane i fills slot i of each of its row blocks; the
 // threads of offset 0 also write the tile's padding blocks and its group -> tile map.
+// (Blocks that take several times 16 (tile, offset) combinations, to compute the prefix over
+// the ranges they start with less often, are slower: 19 against 14 us on the benchmark layer.)
 __global__ void __launch_bounds__(256)
     sched_fill_kernel(const int32_t *__restrict__ flag, const int32_t *__restrict__ pairs,
                       const int32_t *__restrict__ sorted, int64_t pair_stride, int plane_g,
@@ -571,10 +574,11 @@ __global__ void __launch_bounds__(256)
     if (w == 255) range_g0[256] = before + incl;
     __syncthreads();
   }
+  const int64_t n_tiles = n_tiles_dev[0];
+  const int32_t *src = flag[0] ? sorted : pairs;
   int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   int64_t tk = gid >> 4;
   int lane = (int)(gid & 15);
-  const int64_t n_tiles = n_tiles_dev[0];
   if (tk >= n_tiles * K) return;
   int64_t t = tk / K;
   int k = (int)(tk - t * K);
@@ -600,7 +604,6 @@ __global__ void __launch_bounds__(256)
       if (lane == 0) grp_meta[(mb >> 2) * 8 + (mb & 3)] = 0;
     }
   }
-  const int32_t *src = flag[0] ? sorted : pairs;
   int s0 = share_first[t * K + k];
   int n = share_cnt[t * K + k];
   if (n <= 0) return;
@@ -610,15 +613,31 @@ __global__ void __launch_bounds__(256)
   // accumulator slot of a row: rows map to slots modulo the window height T; the
   // rows a tile touches span less than T, so one conditional subtraction does it
   const int slot_off = tile_slot0[t] - tile_row0[t];
-  for (int p = lane; p < ((n + 15) & ~15); p += 16, ++mb) {
-    sched_in[mb * 16 + lane] = p < n ? (int32_t)((uint32_t)pg[p] * in_scale) : (int32_t)in_pad;
-    int slot = T;
-    if (p < n) {
-      slot = ps[p] + slot_off;
-      if (slot >= T) slot -= T;
+  // four row blocks at a time: their loads are issued together
+  const int n16 = (n + 15) & ~15;
+  for (int p0 = lane; p0 < n16; p0 += 64, mb += 4) {
+    int gi[4], so[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int p = p0 + 16 * u;
+      gi[u] = p < n ? pg[p] : 0;
+      so[u] = p < n ? ps[p] : 0;
     }
-    sched_out[mb * 16 + lane] = slot * out_scale;
-    if (lane == 0) grp_meta[(mb >> 2) * 8 + (mb & 3)] = k * k_scale;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int p = p0 + 16 * u;
+      if (p < n16) {
+        const int64_t b = mb + u;
+        sched_in[b * 16 + lane] = p < n ? (int32_t)((uint32_t)gi[u] * in_scale) : (int32_t)in_pad;
+        int slot = T;
+        if (p < n) {
+          slot = so[u] + slot_off;
+          if (slot >= T) slot -= T;
+        }
+        sched_out[b * 16 + lane] = slot * out_scale;
+        if (lane == 0) grp_meta[(b >> 2) * 8 + (b & 3)] = k * k_scale;
+      }
+    }
   }
 }
 
@@ -963,9 +982,9 @@ static int conv_plan_build(const ConvPlan &p, const ConvWs &w, const int32_t *pa
                      w.flag, pairs, w.sorted, pair_stride, plane_s, pair_num, K, w.n_tiles_dev,
                      w.tile_row0, n_out, w.fine_segs, kSplitGranule, w.spill_end, w.segs, w.spill);
   SSC_LAUNCH_CHECK("tile_segments");
-  hipLaunchKernelGGL(range_sched_kernel, dim3((unsigned)p.n_wg), dim3(256), 0, s, w.segs, w.spill,
-                     K, w.wg_tile, w.share_first, w.share_cnt, w.kofs, w.tile_nmb, w.tile_loc,
-                     w.tile_rng, w.range_grp);
+  hipLaunchKernelGGL(range_sched_kernel, dim3((unsigned)p.n_wg), dim3(kRangeSchedThreads), 0, s,
+                     w.segs, w.spill, K, w.wg_tile, w.share_first, w.share_cnt, w.kofs, w.tile_nmb,
+                     w.tile_loc, w.tile_rng, w.range_grp);
   const int frag_bytes = elem_bytes == 2 ? Io<_Float16>::kFragBytes : Io<float>::kFragBytes;
   hipLaunchKernelGGL(sched_fill_kernel, dim3((unsigned)ceil_div(p.n_tiles * K * 16, 256)),
                      dim3(256), 0, s, w.flag, pairs, w.sorted, pair_stride, plane_g,

@@ -358,10 +358,10 @@ __global__ void __launch_bounds__(kScanThreads)
 }
 
 // Output table from the input table (see "marking by dilation"), the block sums of its
-// popcounts (added into blocksum[], which starts at zero), and, in the K blocks after the
+// popcounts (blocksum[], one store per block), and, in the K blocks after the
 // table's, the scan of the chunk counts.  Word (b, x, y, zw) of the output is the OR over
 // (kx, ky) of the bits 32 zw + kz .. + 31, for every kz, of input row (b, x + kx, y + ky).
-// One word per thread.  KS > 0: the kernel's three extents equal KS (loops unrolled, all
+// KS > 0: the kernel's three extents equal KS (loops unrolled, all
 // loads of a thread in flight at once); KS = 0: any extents.
 template <int KS>
 __global__ void __launch_bounds__(kScanThreads)
@@ -374,12 +374,19 @@ __global__ void __launch_bounds__(kScanThreads)
     scan_chunks_of_tap(chunk_count, n_chunks, (int)(blockIdx.x - n_word_blocks), pair_num, lds);
     return;
   }
+  // One block per scan block of kScanBlockWords words, kScanItems words per thread: the
+  // block's popcount is one plain store.  (A block per kScanThreads words with an atomic
+  // add per wave put 32 atomics on every block sum; device-scope atomics on one address
+  // are served one after the other, and that chain, not the loads, was the kernel's time.)
   const int ksx = KS > 0 ? KS : g.ks[0], ksy = KS > 0 ? KS : g.ks[1], ksz = KS > 0 ? KS : g.ks[2];
-  const int64_t w = (int64_t)blockIdx.x * kScanThreads + threadIdx.x;
+  const uint32_t zw_n = (uint32_t)g.os[2] >> 5;  // words per output row
+  const int64_t xstep = (int64_t)d.U[1] * d.Wz;
   int v = 0;
-  if (w < n_words) {
-    const uint32_t zw_n = (uint32_t)g.os[2] >> 5;  // words per output row
-    uint32_t t = (uint32_t)w;                       // (fewer than 2^26 words)
+#pragma unroll 2
+  for (int it = 0; it < kScanItems; ++it) {
+    const int64_t w = (int64_t)blockIdx.x * kScanBlockWords + it * kScanThreads + threadIdx.x;
+    if (w >= n_words) break;
+    uint32_t t = (uint32_t)w;  // (fewer than 2^26 words)
     const int zw = (int)(t % zw_n);
     t /= zw_n;
     const int y = (int)(t % (uint32_t)g.os[1]);
@@ -387,7 +394,6 @@ __global__ void __launch_bounds__(kScanThreads)
     const int x = (int)(t % (uint32_t)g.os[0]);
     const int b = (int)(t / (uint32_t)g.os[0]);
     const uint32_t *rowp = in_bits + (((int64_t)b * d.U[0] + x) * d.U[1] + y) * d.Wz + zw;
-    const int64_t xstep = (int64_t)d.U[1] * d.Wz;
     uint32_t out = 0u;
 #pragma unroll
     for (int kx = 0; kx < ksx; ++kx) {
@@ -403,25 +409,20 @@ __global__ void __launch_bounds__(kScanThreads)
       }
     }
     bits[w] = out;
-    v = __popc(out);
+    v += __popc(out);
   }
 #pragma unroll
   for (int s = 32; s >= 1; s >>= 1) v += __shfl_xor(v, s, 64);
-  // (the kScanThreads words of a block lie in one scan block of kScanBlockWords words)
-  if ((threadIdx.x & 63) == 0 && v != 0)
-    atomicAdd(&blocksum[((int64_t)blockIdx.x * kScanThreads) / kScanBlockWords], v);
+  __shared__ int wave_sum[kScanThreads / 64];
+  if ((threadIdx.x & 63) == 0) wave_sum[threadIdx.x >> 6] = v;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int total = 0;
+#pragma unroll
+    for (int i = 0; i < kScanThreads / 64; ++i) total += wave_sum[i];
+    blocksum[blockIdx.x] = total;
+  }
 }
-
-// Pair emission: same traversal as count_pairs_kernel; a row's slot inside tap k
-// is (pairs of earlier chunks) + (earlier lanes of this chunk), which makes the
-// pair list ascending in input row.  The wave also pads slots [num, n_in) of
-// its own 64-slot window with -1.
-//
-// The grid's rows y >= ks[0] (a regular convolution has them, a submanifold one does not)
-// do an unrelated job that needs nothing but the scanned table either: they decode the
-// table into out_indices[], strided over its words.  One launch, and the two jobs, each
-// short and bound by latency, run side by side.
-// KS > 0: the kernel's y and z extents equal KS (loops unrolled); KS = 0: any extents.
 template <int KS>
 __global__ void __launch_bounds__(256)
     write_pairs_kernel(const int32_t *__restrict__ indices, int64_t n_in, Geom g,
@@ -597,7 +598,7 @@ static int rulebook_mark_and_scan(const int32_t *indices, int64_t n_in, const Ge
                        indices, n_in, gg, w.dense, w.in_bits, w.chunk_count, w.n_chunks,
                        w.table.total + 1);
     SSC_LAUNCH_CHECK("mark_in_count");
-    const int64_t word_blocks = ceil_div(w.table.n_words, kScanThreads);
+    const int64_t word_blocks = w.table.n_scan_blocks;
     const int ks = (gg.ks[0] == gg.ks[1] && gg.ks[1] == gg.ks[2]) ? gg.ks[0] : 0;
     auto kernel = ks == 3 ? dilate_blocksum_kernel<3> : ks == 5 ? dilate_blocksum_kernel<5>
                                                                 : dilate_blocksum_kernel<0>;
