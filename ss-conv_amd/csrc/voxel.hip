@@ -762,18 +762,29 @@ int ssc_three_interp_f32(int32_t c, int32_t m, int32_t n, const float *feats, co
 namespace ssc {
 
 // Pass 1: one wave per 64 points.  inside bit per point (a ballot: no atomics),
-// histograms of all ids and of the surviving ids (one atomic per distinct id and
-// wave), flags[0] |= 1 for an id outside [0, max_ids), flags[1] |= 1 when ids decrease.
-__global__ void __launch_bounds__(256)
+// histograms of all ids and of the surviving ids, flags[0] |= 1 for an id outside
+// [0, max_ids), flags[1] |= 1 when ids decrease.  The waves of a block add their counts up
+// in LDS first (bins for the ids first .. first + 63, `first` the id of the block's first
+// point; any other id goes straight to memory) and the block then issues one atomic per
+// id it saw: atomics on one address are served one after the other, and with a wave's
+// worth of points per atomic a cloud of 16384 points put 256 of them on its counter.
+constexpr int kP2vScanThreads = 1024;
+__global__ void __launch_bounds__(kP2vScanThreads)
     p2v_scan_kernel(const float *__restrict__ pts, const int64_t *__restrict__ ids, int64_t n,
                     float hx, float hy, float hz, int max_ids, uint32_t *__restrict__ bits,
                     int32_t *__restrict__ hist_all, int32_t *__restrict__ hist_valid,
                     int32_t *__restrict__ flags) {
+  __shared__ int s_all[64], s_valid[64];
+  __shared__ int s_first;
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   const int lane = threadIdx.x & 63;
   const bool live = i < n;
   bool inside = false;
   int64_t id = -1;
+  if (threadIdx.x < 64) {
+    s_all[threadIdx.x] = 0;
+    s_valid[threadIdx.x] = 0;
+  }
   if (live) {
     const float x = pts[i * 3], y = pts[i * 3 + 1], z = pts[i * 3 + 2];
     inside = !(fabsf(x) > hx) && !(fabsf(y) > hy) && !(fabsf(z) > hz);
@@ -781,6 +792,9 @@ __global__ void __launch_bounds__(256)
     if (id < 0 || id >= max_ids) atomicOr(&flags[0], 1);
     if (i > 0 && ids[i - 1] > id) atomicOr(&flags[1], 1);
   }
+  if (threadIdx.x == 0) s_first = (int)(id < 0 ? 0 : (id >= max_ids ? max_ids - 1 : id));
+  __syncthreads();
+  const int first_id = s_first;
   const unsigned long long in_mask = __ballot(inside);
   if (live && (lane & 31) == 0) bits[i >> 5] = (uint32_t)(in_mask >> (lane & 32));
   const bool ok_id = live && id >= 0 && id < max_ids;
@@ -790,11 +804,23 @@ __global__ void __launch_bounds__(256)
     const int v = __shfl((int)id, first, 64);
     const unsigned long long same = __ballot(ok_id && (int)id == v);
     if (lane == first) {
-      atomicAdd(&hist_all[v], __popcll(same));
       const int nv = __popcll(same & in_mask);
-      if (nv) atomicAdd(&hist_valid[v], nv);
+      const unsigned bin = (unsigned)(v - first_id);
+      if (bin < 64u) {
+        atomicAdd(&s_all[bin], __popcll(same));
+        if (nv) atomicAdd(&s_valid[bin], nv);
+      } else {
+        atomicAdd(&hist_all[v], __popcll(same));
+        if (nv) atomicAdd(&hist_valid[v], nv);
+      }
     }
     todo &= ~same;
+  }
+  __syncthreads();
+  if (threadIdx.x < 64) {
+    const int a = s_all[threadIdx.x], b = s_valid[threadIdx.x];
+    if (a) atomicAdd(&hist_all[first_id + threadIdx.x], a);
+    if (b) atomicAdd(&hist_valid[first_id + threadIdx.x], b);
   }
 }
 
@@ -961,7 +987,8 @@ int ssc_p2v_scan(const float *points, const int64_t *batch_ids, int64_t n,
   // alignment padding, which the fill covers as well)
   const int64_t clear_n = (w.flags + 2) - w.hist_all;
   if ((rc = fill_i32(w.hist_all, clear_n, 0, s)) != SSC_OK) return rc;
-  hipLaunchKernelGGL(p2v_scan_kernel, dim3((unsigned)ceil_div(n, 256)), dim3(256), 0, s, points,
+  hipLaunchKernelGGL(p2v_scan_kernel, dim3((unsigned)ceil_div(n, kP2vScanThreads)),
+                     dim3(kP2vScanThreads), 0, s, points,
                      batch_ids, n, half_extent[0], half_extent[1], half_extent[2],
                      (int)SSC_P2V_MAX_IDS, w.table.bits, w.hist_all, w.hist_valid, w.flags);
   SSC_LAUNCH_CHECK("p2v_scan");
@@ -1304,7 +1331,8 @@ int ssc_p2v_voxelize_f32(const float *points, const float *feats, const int64_t 
                      dim3(256), 0, s, w.hist_all, clear_a, w.vox.bits, w.vox.n_words, w.head, n,
                      w.totals);
   SSC_LAUNCH_CHECK("p2vx_clear");
-  hipLaunchKernelGGL(p2v_scan_kernel, dim3((unsigned)ceil_div(n, 256)), dim3(256), 0, s, points,
+  hipLaunchKernelGGL(p2v_scan_kernel, dim3((unsigned)ceil_div(n, kP2vScanThreads)),
+                     dim3(kP2vScanThreads), 0, s, points,
                      batch_ids, n, half_extent[0], half_extent[1], half_extent[2], (int)n_ids,
                      w.inside.bits, w.hist_all, w.hist_valid, w.flags);
   SSC_LAUNCH_CHECK("p2v_scan");
