@@ -31,7 +31,7 @@ CLOCK_WARMUP_MS = 100
 # HBM bytes per launch of the convolution kernel for every workload this script offers, from
 # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs scaled by a copy kernel of known size (the
 # summaries profiles/conv_fwd_<workload>_hbm_traffic.md give commands and counter values).
-MEASURED_TRAFFIC_BYTES = {"cfg1": 3035023, "cfg2": 345576980, "cfg3": 218961080, "cfg5": 56198008824}
+MEASURED_TRAFFIC_BYTES = {"cfg1": 3016591, "cfg2": 345582696, "cfg3": 219239659, "cfg5": 56045076175}
 
 
 def parse_args():
