@@ -307,7 +307,10 @@ int ssc_profile_conv(int32_t enable);
  *   2  no launch of its own for a last group of 16 output columns that would be alone in
  *      its block of 64 (Cout = 72, 136).  This flag changes the sizes ssc_conv_plan_bytes
  *      and its like return: set it before any plan is sized or built and do not mix plans
- *      across a change.  Results agree up to the order of the float sums of that group. */
+ *      across a change.  Results agree up to the order of the float sums of that group.
+ *   4  the ranges of output rows per column block rounded down to a multiple of 8 (leaves
+ *      CUs without a workgroup where the column blocks do not divide them that way; the
+ *      default gives every CU one).  Changes the same sizes; results do not depend on it. */
 int ssc_conv_tuning(int32_t flags);
 int ssc_profile_conv_read(float *ms /* host */, int32_t capacity, int32_t *count /* host */);
 

@@ -669,6 +669,7 @@ static int device_cu_count() {
 
 // (switched by ssc_conv_tuning, for measurements)
 static bool g_conv_tail = true;       // a launch of its own for a lone last column group
+static bool g_conv_round8 = false;    // ranges per column block: a multiple of 8 only
 
 // The sizes that follow from the number of workgroups per column block.
 static void plan_split(ConvPlan &p, int n_wg, int64_t n_out, int K, int64_t pair_stride) {
@@ -719,7 +720,9 @@ static ConvPlan make_plan(int64_t n_in, int64_t n_out, int K, int c_in, int c_ou
   int n_wg = device_cu_count() / p.n_colblk;
   if (n_wg < 1) n_wg = 1;
   if (n_wg > 256) n_wg = 256;  // the split kernel is one block of 256 threads
-  if (n_wg >= 8) n_wg = n_wg / 8 * 8;
+  // (every CU a workgroup, also where the column blocks do not divide the CUs by a
+  // multiple of 8: the kernel then deals its workgroups to the XCDs by its general rule)
+  if (n_wg >= 8 && g_conv_round8) n_wg = n_wg / 8 * 8;
   plan_split(p, n_wg, n_out, K, pair_stride);
   p.lds_bytes = conv_lds_bytes(p.T, p.ncw);
   return p;
@@ -882,6 +885,7 @@ int ssc_profile_conv(int32_t enable) {
 int ssc_conv_tuning(int32_t flags) {
   g_conv_by_column = (flags & 1) != 0;
   g_conv_tail = (flags & 2) == 0;
+  g_conv_round8 = (flags & 4) != 0;
   return SSC_OK;
 }
 

@@ -231,6 +231,15 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
       chunk = (xcd / ncol) * ((nwg * ncol) >> 3) + slot;
     } else if ((nwg & 7) == 0) {
       chunk = (chunk & 7) * (nwg >> 3) + (chunk >> 3);
+    } else if (cols_per_xcd < 0) {
+      // any other grid: the (range, column block) items, numbered range by range, are
+      // dealt to the XCDs in contiguous runs; XCD x has the workgroups x, x + 8, ...
+      const int ncol = gridDim.y, total = nwg * ncol;
+      const int lin = blockIdx.y * nwg + blockIdx.x;
+      const int xcd = lin & 7, slot = lin >> 3;
+      const int item = xcd * (total >> 3) + min(xcd, total & 7) + slot;
+      chunk = item / ncol;
+      cblk = item - chunk * ncol;
     }
   }
   const int t_begin = wg_tile[chunk], t_end = wg_tile[chunk + 1];
@@ -1042,7 +1051,9 @@ inline int launch_conv(const ConvPlan &p, const ConvWs &w, const IO *features, i
   const bool by_column = packed_bytes > ((uint64_t)4 << 20) && p.n_colblk > 1 &&
                          8 % p.n_colblk == 0 && (p.n_wg * p.n_colblk) % 8 == 0 &&
                          g_conv_by_column;
-  const int cols_per_xcd = by_column ? 8 / p.n_colblk : 0;
+  // (-1: a grid that is no multiple of 8 wide takes the kernel's mapping for any grid)
+  const int cols_per_xcd = by_column ? 8 / p.n_colblk
+                           : ((p.n_wg & 7) != 0 && p.n_wg * p.n_colblk >= 16) ? -1 : 0;
   hipLaunchKernelGGL((conv_fwd_kernel<IO, GATHER, NCW, NS, EPI, TAIL>), grid, dim3((NCW + 4) * 64), p.lds_bytes, s, features, c_in,
                      feat_bytes, w.packed, (unsigned)packed_bytes, w.sched_in, w.sched_out,
                      w.grp_meta, (unsigned)sched_bytes, (unsigned)(p.grp_cap * 32), w.tile_grp,
