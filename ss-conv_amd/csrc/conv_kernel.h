@@ -232,14 +232,20 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
     } else if ((nwg & 7) == 0) {
       chunk = (chunk & 7) * (nwg >> 3) + (chunk >> 3);
     } else if (cols_per_xcd < 0) {
-      // any other grid: the (range, column block) items, numbered range by range, are
-      // dealt to the XCDs in contiguous runs; XCD x has the workgroups x, x + 8, ...
+      // any other grid: the (range, column block) items, numbered range by range (-1) or
+      // column block by column block (-2), are dealt to the XCDs in contiguous runs; XCD x
+      // has the workgroups x, x + 8, ...
       const int ncol = gridDim.y, total = nwg * ncol;
       const int lin = blockIdx.y * nwg + blockIdx.x;
       const int xcd = lin & 7, slot = lin >> 3;
       const int item = xcd * (total >> 3) + min(xcd, total & 7) + slot;
-      chunk = item / ncol;
-      cblk = item - chunk * ncol;
+      if (cols_per_xcd == -1) {
+        chunk = item / ncol;
+        cblk = item - chunk * ncol;
+      } else {  // filters larger than an L2: column block by column block (an XCD sees few)
+        cblk = item / nwg;
+        chunk = item - cblk * nwg;
+      }
     }
   }
   const int t_begin = wg_tile[chunk], t_end = wg_tile[chunk + 1];
@@ -1052,8 +1058,9 @@ inline int launch_conv(const ConvPlan &p, const ConvWs &w, const IO *features, i
                          8 % p.n_colblk == 0 && (p.n_wg * p.n_colblk) % 8 == 0 &&
                          g_conv_by_column;
   // (-1: a grid that is no multiple of 8 wide takes the kernel's mapping for any grid)
+  const bool big = packed_bytes > ((uint64_t)4 << 20) && p.n_colblk > 1 && g_conv_by_column;
   const int cols_per_xcd = by_column ? 8 / p.n_colblk
-                           : ((p.n_wg & 7) != 0 && p.n_wg * p.n_colblk >= 16) ? -1 : 0;
+                           : ((p.n_wg & 7) != 0 && p.n_wg * p.n_colblk >= 16) ? (big ? -2 : -1) : 0;
   hipLaunchKernelGGL((conv_fwd_kernel<IO, GATHER, NCW, NS, EPI, TAIL>), grid, dim3((NCW + 4) * 64), p.lds_bytes, s, features, c_in,
                      feat_bytes, w.packed, (unsigned)packed_bytes, w.sched_in, w.sched_out,
                      w.grp_meta, (unsigned)sched_bytes, (unsigned)(p.grp_cap * 32), w.tile_grp,
