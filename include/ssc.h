@@ -310,7 +310,16 @@ int ssc_profile_conv(int32_t enable);
  *      across a change.  Results agree up to the order of the float sums of that group.
  *   4  the ranges of output rows per column block rounded down to a multiple of 8 (leaves
  *      CUs without a workgroup where the column blocks do not divide them that way; the
- *      default gives every CU one).  Changes the same sizes; results do not depend on it. */
+ *      default gives every CU one).  Changes the same sizes; results do not depend on it.
+ *   8  no five-group form: float layers of more than 192 input channels whose last group
+ *      of 16 output columns would be alone in its block of 64 (Cout = 200, 72 + 64 n)
+ *      otherwise run one launch per block of 64 columns, the last of which takes the lone
+ *      group along.  Changes the same sizes; results agree up to the order of the float
+ *      sums of that group.
+ *  16  no second work split: plans of long kernels (an estimated thousand stages or more
+ *      per workgroup) otherwise deal the output rows to the workgroups twice, the second
+ *      time by the row-block counts the first split came to.  Results do not depend on it.
+ *  32  the second work split for every plan, whatever its size (for tests). */
 int ssc_conv_tuning(int32_t flags);
 int ssc_profile_conv_read(float *ms /* host */, int32_t capacity, int32_t *count /* host */);
 

@@ -314,6 +314,9 @@ constexpr int kSplitGranule = 64;
 // modulo the window height, so what such a block adds to the next tile's rows is
 // still there when that tile's turn comes.
 constexpr int kSpillRows = 160;
+// (the five-group form, whose window is 376 rows: 200 -> 200 channels with 125 offsets takes
+// 14.3 ms with 160, 13.9 with 192 or 224, 14.7 with 128)
+constexpr int kSpillRowsFive = 192;
 
 // cost of a tile beyond its pairs, in pair slots: padding per offset, and about a stage's
 // worth of time for writing it out (measured: 2 K + 128 and 3 K + 64 are as good on the
@@ -356,6 +359,80 @@ __global__ void __launch_bounds__(256)
   if (r > n_out) r = n_out;
   for (int64_t w = w0; w < w1; ++w)
     range_row0[w] = (w == 0) ? 0 : (w == n_wg ? (int32_t)n_out : (int32_t)r);
+}
+
+// The split again, from what the first one turned out to cost.  The schedule of the first
+// split is counted by then: range_grp[w] row-block groups for range w, where the model
+// above had promised every range the same work -- what a tile pads depends on how many
+// offsets it meets with how many pairs each, which the model does not see, and the slowest
+// workgroup sets the kernel's time.  Here a row's modelled work counts with the factor its
+// range showed, groups per modelled work, and the boundaries are placed anew for equal
+// corrected work: boundary b of the fine grid has
+//   cum(b) = groups of the ranges before b's range + groups of that range * the part of
+//            its modelled work that lies below b,
+// and the ranges whose target (w / n_wg of all groups) lies in (cum(b-1), cum(b)] begin
+// there.  row_old: range_row0 of the first split; row_new: that of the second.
+__global__ void __launch_bounds__(256)
+    split_rebalance_kernel(const int32_t *__restrict__ fine_segs, int K, int64_t nb,
+                           int64_t n_out, int T, int n_wg, const int32_t *__restrict__ row_old,
+                           const int32_t *__restrict__ range_grp, int32_t *__restrict__ row_new) {
+  __shared__ int row_s[257];
+  __shared__ double work_s[257];  // modelled work below the first row of range w
+  __shared__ double grp_s[257];   // groups of the ranges before range w
+  auto cell_of = [&](int64_t row) -> int64_t { return (row + kSplitGranule - 1) / kSplitGranule; };
+  auto work_below = [&](int64_t cell) -> double {
+    int64_t below = 0;
+    for (int k = 0; k < K; ++k) below += fine_segs[cell * K + k];
+    return (double)split_work(below, cell, n_out, T, K);
+  };
+  for (int w = threadIdx.x; w <= n_wg; w += blockDim.x) {  // n_wg <= 256
+    int r = row_old[w];
+    if (w == 0) r = 0;
+    if (w == n_wg) r = (int)n_out;
+    row_s[w] = r;
+    work_s[w] = work_below(cell_of(r));  // range boundaries lie on the grid, or at the end
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    double run = 0.0;
+    for (int w = 0; w < n_wg; ++w) {
+      grp_s[w] = run;
+      run += (double)range_grp[w];
+    }
+    grp_s[n_wg] = run;
+  }
+  __syncthreads();
+  const int64_t b = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (b > nb) return;
+  const double total = grp_s[n_wg];
+  // corrected work below cell c
+  auto cum = [&](int64_t c) -> double {
+    if (c >= nb) return total;
+    int64_t r = c * kSplitGranule;
+    if (r > n_out) r = n_out;
+    // the last range that begins at or before row r and does not end there
+    int lo = 0, hi = n_wg - 1;
+    while (lo < hi) {
+      const int mid = (lo + hi + 1) >> 1;
+      if (row_s[mid] <= r) lo = mid;
+      else hi = mid - 1;
+    }
+    const double span = work_s[lo + 1] - work_s[lo];
+    const double part = span > 0.0 ? (work_below(c) - work_s[lo]) / span : 0.0;
+    const double g = grp_s[lo + 1] - grp_s[lo];
+    return grp_s[lo] + g * (part < 0.0 ? 0.0 : part > 1.0 ? 1.0 : part);
+  };
+  auto reached = [&](double c) -> int64_t {
+    if (total <= 0.0) return n_wg + 1;
+    const int64_t v = (int64_t)(c * (double)n_wg / total) + 1;
+    return v > n_wg + 1 ? n_wg + 1 : v;
+  };
+  const int64_t w0 = b > 0 ? reached(cum(b - 1)) : 0;
+  const int64_t w1 = reached(cum(b));
+  int64_t r = b * kSplitGranule;
+  if (r > n_out) r = n_out;
+  for (int64_t w = w0; w < w1; ++w)
+    row_new[w] = (w == 0) ? 0 : (w == n_wg ? (int32_t)n_out : (int32_t)r);
 }
 
 // One block.  wg_tile[0..n_wg]: first tile of every workgroup; tile_row0[0..n_tiles]:
@@ -642,14 +719,14 @@ __global__ void __launch_bounds__(256)
 }
 
 
-static size_t conv_lds_bytes(int T, int ncw) {
-  return ((size_t)(T + 1) * (16 * ncw + 4) + 2 * (size_t)kStage * kAStride) * 4;
+static size_t conv_lds_bytes(int T, int acc_cols) {
+  return ((size_t)(T + 1) * (acc_cols + 4) + 2 * (size_t)kStage * kAStride) * 4;
 }
 
-static int pick_tile(int ncw) {
+static int pick_tile(int acc_cols) {
   // One workgroup per CU: (almost) all of the 160 KB of LDS goes to the accumulators.
-  size_t budget = 160 * 1024 - conv_lds_bytes(0, ncw) - 512;
-  int t = (int)(budget / ((size_t)(16 * ncw + 4) * 4));
+  size_t budget = 160 * 1024 - conv_lds_bytes(0, acc_cols) - 512;
+  int t = (int)(budget / ((size_t)(acc_cols + 4) * 4));
   t = t / 8 * 8;
   if (t < kMinTile) t = kMinTile;
   return t;
@@ -669,6 +746,10 @@ static int device_cu_count() {
 
 // (switched by ssc_conv_tuning, for measurements)
 static bool g_conv_tail = true;       // a launch of its own for a lone last column group
+static bool g_conv_five = true;       // the lone last group as a fifth one of the last block
+constexpr int64_t kRebalanceStages = 1000;
+static int64_t g_conv_rebalance_stages = kRebalanceStages;
+static bool g_conv_rebalance = true;  // long kernels: a second work split from the first one's counts
 static bool g_conv_round8 = false;    // ranges per column block: a multiple of 8 only
 
 // The sizes that follow from the number of workgroups per column block.
@@ -703,8 +784,12 @@ static ConvPlan make_plan(int64_t n_in, int64_t n_out, int K, int c_in, int c_ou
       }
   }
   p.ncw = 4;
-  p.T = pick_tile(p.ncw);
-  p.tile_rows = p.T - kSpillRows;
+  // the five-group form: a lone last group goes along with the last full block (the
+  // kernel needs four chunks for it, one for each wave's turn at the fifth group's sums)
+  p.five = g_conv_five && elem_bytes == 4 && p.ncb % p.ncw == 1 && p.ncb > p.ncw && p.nch >= 4;
+  p.acc_cols = p.five ? 16 * p.ncw + 16 : 16 * p.ncw;
+  p.T = pick_tile(p.acc_cols);
+  p.tile_rows = p.T - (p.five ? kSpillRowsFive : kSpillRows);
   // the gather can be a range-checked buffer load when rows are multiples of four
   // channels and byte offsets into the features (plus the padding marker) fit 32 bits
   p.gather = 0;
@@ -713,10 +798,11 @@ static ConvPlan make_plan(int64_t n_in, int64_t n_out, int K, int c_in, int c_ou
   // (wider layers: the launches of one column block each cost more than the lone group
   // in a block of its own does -- 128 -> 256 channels at stride 2 takes 0.255 ms as four
   // launches against 0.185 ms as one, 200 -> 200 with 125 offsets 17.6 against 16.8 ms)
-  p.has_tail = g_conv_tail && elem_bytes == 4 && p.ncb % p.ncw == 1 && p.ncb / p.ncw <= 2;
-  const int blocks = p.has_tail ? p.ncb / p.ncw : (int)ceil_div(p.ncb, p.ncw);
-  p.n_colblk = p.has_tail ? 1 : blocks;
-  p.n_launch = p.has_tail ? blocks : 1;
+  p.has_tail = !p.five && g_conv_tail && elem_bytes == 4 && p.ncb % p.ncw == 1 && p.ncb / p.ncw <= 2;
+  const bool serial = p.has_tail || p.five;
+  const int blocks = serial ? p.ncb / p.ncw : (int)ceil_div(p.ncb, p.ncw);
+  p.n_colblk = serial ? 1 : blocks;
+  p.n_launch = serial ? blocks : 1;
   int n_wg = device_cu_count() / p.n_colblk;
   if (n_wg < 1) n_wg = 1;
   if (n_wg > 256) n_wg = 256;  // the split kernel is one block of 256 threads
@@ -724,7 +810,15 @@ static ConvPlan make_plan(int64_t n_in, int64_t n_out, int K, int c_in, int c_ou
   // multiple of 8: the kernel then deals its workgroups to the XCDs by its general rule)
   if (n_wg >= 8 && g_conv_round8) n_wg = n_wg / 8 * 8;
   plan_split(p, n_wg, n_out, K, pair_stride);
-  p.lds_bytes = conv_lds_bytes(p.T, p.ncw);
+  p.lds_bytes = conv_lds_bytes(p.T, p.acc_cols);
+  // A second work split (split_rebalance_kernel) where the kernel runs long enough for four
+  // more small launches: some thousand stages per workgroup, estimated from the most pairs
+  // the rows can have -- a regular layer has about min(N_in, N_out) K, a strided one fewer.
+  {
+    const int64_t rows = n_in > 0 && n_in < n_out ? n_in : n_out;
+    const int64_t stages = rows * K / 2 / kStage * p.nch / (p.n_wg > 0 ? p.n_wg : 1);
+    p.rebalance = g_conv_rebalance && stages >= g_conv_rebalance_stages;
+  }
   return p;
 }
 
@@ -774,6 +868,7 @@ static size_t conv_scratch_walk(void *base, const ConvPlan &p, int K, int64_t pa
   t.n_tiles_dev = c.take<int32_t>(1);
   t.tile_rng = c.take<int32_t>((size_t)p.n_tiles + 1);
   t.range_grp = c.take<int32_t>((size_t)p.n_wg + 1);
+  t.range_row1 = c.take<int32_t>((size_t)p.n_wg + 1);
   if (w) {
     w->flag = t.flag;
     w->segs = t.segs;
@@ -794,6 +889,7 @@ static size_t conv_scratch_walk(void *base, const ConvPlan &p, int K, int64_t pa
     w->n_tiles_dev = t.n_tiles_dev;
     w->tile_rng = t.tile_rng;
     w->range_grp = t.range_grp;
+    w->range_row1 = t.range_row1;
   }
   return c.used;
 }
@@ -823,27 +919,47 @@ static int launch_all(const ConvPlan &p, const ConvWs &w, const IO *features, in
                       hipStream_t s) {
   constexpr bool kFloat = sizeof(IO) == 4;
   const bool with_epi = kFloat && epi.mode != nullptr;
+  if (p.five) {
+    // the epilogue is not built for the fifth group: with it the lone group takes a launch
+    // of its own, as a block of which one consumer wave in four has columns
+    if constexpr (kFloat) {
+      const int n_launch = with_epi ? p.n_launch + 1 : p.n_launch;
+      for (int l = 0; l < n_launch; ++l) {
+        const int col_base = l * 16 * p.ncw;
+        const int xcol = !with_epi && l == p.n_launch - 1 ? (p.ncb - 1) * 16 : -1;
+        const int rc =
+            with_epi ? launch_conv_f32<GATHER, NS, true, 2>(p, w, features, n_in, c_in, K, out,
+                                                            c_out, col_base, xcol, epi, s)
+                     : launch_conv_f32<GATHER, NS, false, 2>(p, w, features, n_in, c_in, K, out,
+                                                             c_out, col_base, xcol, epi, s);
+        if (rc != SSC_OK) return rc;
+      }
+      return SSC_OK;
+    } else {
+      SSC_CHECK(false, SSC_ERUNTIME, "the five-group form is built for float rows");
+    }
+  }
   for (int l = 0; l < p.n_launch; ++l) {
     const int col_base = l * p.n_colblk * 16 * p.ncw;
     int rc;
     if constexpr (kFloat) {
-      rc = with_epi ? launch_conv_f32<GATHER, NS, true, false>(p, w, features, n_in, c_in, K, out,
-                                                               c_out, col_base, epi, s)
-                    : launch_conv<float, GATHER, 4, NS, false, false>(p, w, features, n_in, c_in, K,
-                                                                      out, c_out, col_base, epi, s);
+      rc = with_epi ? launch_conv_f32<GATHER, NS, true, 0>(p, w, features, n_in, c_in, K, out,
+                                                           c_out, col_base, -1, epi, s)
+                    : launch_conv<float, GATHER, 4, NS, false, 0>(p, w, features, n_in, c_in, K,
+                                                                  out, c_out, col_base, -1, epi, s);
     } else {
-      rc = launch_conv<IO, GATHER, 4, NS, false, false>(p, w, features, n_in, c_in, K, out, c_out,
-                                                        col_base, epi, s);
+      rc = launch_conv<IO, GATHER, 4, NS, false, 0>(p, w, features, n_in, c_in, K, out, c_out,
+                                                    col_base, -1, epi, s);
     }
     if (rc != SSC_OK) return rc;
   }
   if (p.has_tail) {
     const int col_base = (p.ncb - 1) * 16;
     if constexpr (kFloat) {
-      return with_epi ? launch_conv_f32<GATHER, NS, true, true>(p, w, features, n_in, c_in, K, out,
-                                                                c_out, col_base, epi, s)
-                      : launch_conv_f32<GATHER, NS, false, true>(p, w, features, n_in, c_in, K, out,
-                                                                 c_out, col_base, epi, s);
+      return with_epi ? launch_conv_f32<GATHER, NS, true, 1>(p, w, features, n_in, c_in, K, out,
+                                                             c_out, col_base, -1, epi, s)
+                      : launch_conv_f32<GATHER, NS, false, 1>(p, w, features, n_in, c_in, K, out,
+                                                              c_out, col_base, -1, epi, s);
     } else {
       SSC_CHECK(false, SSC_ERUNTIME, "the one-column-group form is built for float rows");
     }
@@ -886,6 +1002,9 @@ int ssc_conv_tuning(int32_t flags) {
   g_conv_by_column = (flags & 1) != 0;
   g_conv_tail = (flags & 2) == 0;
   g_conv_round8 = (flags & 4) != 0;
+  g_conv_five = (flags & 8) == 0;
+  g_conv_rebalance = (flags & 16) == 0;
+  g_conv_rebalance_stages = (flags & 32) != 0 ? 0 : kRebalanceStages;
   return SSC_OK;
 }
 
@@ -977,18 +1096,34 @@ static int conv_plan_build(const ConvPlan &p, const ConvWs &w, const int32_t *pa
                      kSplitGranule, w.fine_segs, pk);
   hipLaunchKernelGGL(split_bounds_kernel, dim3((unsigned)ceil_div(p.n_fine + 1, 256)), dim3(256), 0,
                      s, w.fine_segs, K, p.n_fine, n_out, p.tile_rows, p.n_wg, w.range_row0);
-  hipLaunchKernelGGL(split_rows_kernel, dim3(1), dim3(256), 0, s, w.range_row0, n_out, p.tile_rows,
-                     p.T, p.n_wg, w.wg_tile, w.tile_row0, w.n_tiles_dev, w.spill_end,
-                     w.tile_slot0);
-  SSC_LAUNCH_CHECK("split");
-  int64_t nseg = (p.n_tiles + 1) * K;
-  hipLaunchKernelGGL(tile_segments_kernel, dim3((unsigned)ceil_div(nseg, 256)), dim3(256), 0, s,
-                     w.flag, pairs, w.sorted, pair_stride, plane_s, pair_num, K, w.n_tiles_dev,
-                     w.tile_row0, n_out, w.fine_segs, kSplitGranule, w.spill_end, w.segs, w.spill);
-  SSC_LAUNCH_CHECK("tile_segments");
-  hipLaunchKernelGGL(range_sched_kernel, dim3((unsigned)p.n_wg), dim3(kRangeSchedThreads), 0, s,
-                     w.segs, w.spill, K, w.wg_tile, w.share_first, w.share_cnt, w.kofs, w.tile_nmb,
-                     w.tile_loc, w.tile_rng, w.range_grp);
+  // the ranges' tiles, their segments, shares and row-block counts
+  const int64_t nseg = (p.n_tiles + 1) * K;
+  auto tiles_of = [&](const int32_t *range_row0) -> int {
+    hipLaunchKernelGGL(split_rows_kernel, dim3(1), dim3(256), 0, s, range_row0, n_out, p.tile_rows,
+                       p.T, p.n_wg, w.wg_tile, w.tile_row0, w.n_tiles_dev, w.spill_end,
+                       w.tile_slot0);
+    SSC_LAUNCH_CHECK("split");
+    hipLaunchKernelGGL(tile_segments_kernel, dim3((unsigned)ceil_div(nseg, 256)), dim3(256), 0, s,
+                       w.flag, pairs, w.sorted, pair_stride, plane_s, pair_num, K, w.n_tiles_dev,
+                       w.tile_row0, n_out, w.fine_segs, kSplitGranule, w.spill_end, w.segs,
+                       w.spill);
+    SSC_LAUNCH_CHECK("tile_segments");
+    hipLaunchKernelGGL(range_sched_kernel, dim3((unsigned)p.n_wg), dim3(kRangeSchedThreads), 0, s,
+                       w.segs, w.spill, K, w.wg_tile, w.share_first, w.share_cnt, w.kofs,
+                       w.tile_nmb, w.tile_loc, w.tile_rng, w.range_grp);
+    SSC_LAUNCH_CHECK("range_sched");
+    return SSC_OK;
+  };
+  int rc = tiles_of(w.range_row0);
+  if (rc != SSC_OK) return rc;
+  if (p.rebalance) {  // long kernels: once more, from the groups the ranges came to
+    hipLaunchKernelGGL(split_rebalance_kernel, dim3((unsigned)ceil_div(p.n_fine + 1, 256)),
+                       dim3(256), 0, s, w.fine_segs, K, p.n_fine, n_out, p.tile_rows, p.n_wg,
+                       w.range_row0, w.range_grp, w.range_row1);
+    SSC_LAUNCH_CHECK("split_rebalance");
+    rc = tiles_of(w.range_row1);
+    if (rc != SSC_OK) return rc;
+  }
   const int frag_bytes = elem_bytes == 2 ? Io<_Float16>::kFragBytes : Io<float>::kFragBytes;
   hipLaunchKernelGGL(sched_fill_kernel, dim3((unsigned)ceil_div(p.n_tiles * K * 16, 256)),
                      dim3(256), 0, s, w.flag, pairs, w.sorted, pair_stride, plane_g,
@@ -996,7 +1131,7 @@ static int conv_plan_build(const ConvPlan &p, const ConvWs &w, const int32_t *pa
                      w.range_grp, p.n_wg, w.tile_grp, K, w.n_tiles_dev, w.tile_row0,
                      w.tile_slot0, p.T,
                      p.gather ? (uint32_t)c_in * (uint32_t)elem_bytes : 1u,
-                     p.gather ? kGatherPad : 0xFFFFFFFFu, (16 * p.ncw + 4) * 4,
+                     p.gather ? kGatherPad : 0xFFFFFFFFu, (p.acc_cols + 4) * 4,
                      p.ncb * p.nch * frag_bytes, w.sched_in, w.sched_out, w.grp_meta);
   SSC_LAUNCH_CHECK("schedule");
   return SSC_OK;

@@ -1,0 +1,4 @@
+// The convolution kernel on float rows in its five-group form with the epilogue (conv_instances.h).
+#include "conv_instances.h"
+
+SSC_CONV_INSTANCES(true, 2)

@@ -179,7 +179,9 @@ struct ConvEpilogue {
   int act_s, act_g, c_dest;
 };
 
-template <typename IO, int GATHER, int NCW, int NS, bool EPI, bool TAIL>
+// FORM: 0 the kernel as described above; 1 the one-column-group form; 2 the five-group form
+// (see the consumers).
+template <typename IO, int GATHER, int NCW, int NS, bool EPI, int FORM>
 __global__ void __launch_bounds__((NCW + 4) * 64)
     __attribute__((amdgpu_waves_per_eu((NCW + 4) / 4, (NCW + 4) / 4)))
     conv_fwd_kernel(const IO *__restrict__ features, int cin, unsigned feat_bytes,
@@ -188,7 +190,8 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
                     const int32_t *__restrict__ grp_meta, unsigned sched_bytes, unsigned meta_bytes,
                     const int32_t *__restrict__ tile_grp, const int32_t *__restrict__ wg_tile,
                     int nch, int ncb, IO *__restrict__ out, int cout, int T, int cols_per_xcd,
-                    int col_base, ConvEpilogue epi) {
+                    int col_base, int xcol, ConvEpilogue epi) {
+  constexpr bool TAIL = FORM == 1, FIVE = FORM == 2;
   constexpr int kCN = 16 * NCW;   // output columns per workgroup
   constexpr int kEB = Io<IO>::kBytes;
   constexpr bool kHalf = kEB == 2;
@@ -199,7 +202,8 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
   constexpr int kChunk = kHalf ? kKC : 4 * NS;  // input channels per chunk
   constexpr int kQFull = NS / 4, kQRem = NS % 4;  // whole quarters, steps of the partial one
   typedef typename Io<IO>::Raw Raw;
-  constexpr int kAS = kCN + 4;    // accumulator row stride in floats
+  // accumulator row stride in floats (the five-group form: 16 more columns)
+  constexpr int kAS = kCN + (FIVE ? 16 : 0) + 4;
   constexpr int NT = (NCW + 4) * 64;
   constexpr int NP = 256;  // producer threads
   constexpr int NE = kStage * 16 / NP;
@@ -252,7 +256,7 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
   const int g_begin = tile_grp[t_begin], g_end = tile_grp[t_end];
   const int nstages = (g_end - g_begin) * nch;  // stages of this workgroup
   const int col0 = col_base + cblk * kCN;
-  static_assert(!TAIL || (NCW == 4 && !kHalf), "the one-column-group form is built for float");
+  static_assert(FORM == 0 || (NCW == 4 && !kHalf), "the other forms are built for float");
 
   {
     float4v z = {0.f, 0.f, 0.f, 0.f};
@@ -307,6 +311,28 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
   }
   const int e_c_dest = epi.c_dest, e_act_s = epi.act_s, e_act_g = epi.act_g;
   auto flush_tile = [&](int row0, int rows, int slot0) __attribute__((always_inline)) {
+    if constexpr (FIVE) {
+      // the fifth column group (accumulator columns kCN .. kCN + 15): four threads a row
+      if (xcol >= 0) {
+        const float4v z = {0.f, 0.f, 0.f, 0.f};
+        const int c4 = (tid & 3) * 4;
+        for (int r = tid >> 2; r < rows; r += NT / 4) {
+          int sl = slot0 + r;
+          if (sl >= T) sl -= T;
+          float4v *ap = reinterpret_cast<float4v *>(acc + sl * kAS + kCN + c4);
+          const float4v v = *ap;
+          *ap = z;
+          IO *gp = out + (int64_t)(row0 + r) * cout + xcol + c4;
+          if ((cout & 3) == 0) {
+            if (xcol + c4 < cout) Io<IO>::store_stream(gp, v);
+          } else {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+              if (xcol + c4 + i < cout) __builtin_nontemporal_store((IO)v[i], gp + i);
+          }
+        }
+      }
+    }
     if constexpr (TAIL) {
       // The four consumer waves each hold a partial sum of the one column group, in the
       // 16 columns a wave owns: add them up in the first 16, clear the others, and write
@@ -591,6 +617,10 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
       p_idx.advance(nch);
       __syncthreads();
       if (last) {
+        if constexpr (FIVE) {  // the consumers add the last group's fifth-group products
+#pragma unroll
+          for (int i = 0; i < 4; ++i) __syncthreads();
+        }
         flush_tile(t_row0, t_rows, t_slot0);
         __syncthreads();
       }
@@ -690,31 +720,32 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
     auto rec_k = [](const int4v &v, int b) -> int {
       return b == 0 ? v.x : b == 1 ? v.y : b == 2 ? v.z : v.w;
     };
-    auto fetch_w = [&](int soff, int slot, int q) {
+    auto fetch_frag = [&](Frag &dst, int soff, int q) {
       if constexpr (!kHalf && kQRem != 0) {
         if (q == kQFull) {  // the partly used quarter: kQRem floats per lane, densely packed
           const int voff = kQFull * kWStep + lane * (4 * kQRem);
           // The wider loads are cast to float vectors as a whole: with per-element casts
           // of an integer vector this compiler shrinks the load to its first element.
           if constexpr (kQRem == 1) {
-            w[slot][q].x = __builtin_bit_cast(float, buf_load1(rs_w, voff, soff));
+            dst.x = __builtin_bit_cast(float, buf_load1(rs_w, voff, soff));
           } else if constexpr (kQRem == 2) {
             const float2v t = __builtin_bit_cast(
                 float2v, __builtin_amdgcn_raw_buffer_load_b64(rs_w, voff, soff, 0));
-            w[slot][q].x = t.x;
-            w[slot][q].y = t.y;
+            dst.x = t.x;
+            dst.y = t.y;
           } else {
             const float3v t = __builtin_bit_cast(
                 float3v, __builtin_amdgcn_raw_buffer_load_b96(rs_w, voff, soff, 0));
-            w[slot][q].x = t.x;
-            w[slot][q].y = t.y;
-            w[slot][q].z = t.z;
+            dst.x = t.x;
+            dst.y = t.y;
+            dst.z = t.z;
           }
           return;
         }
       }
-      w[slot][q] = __builtin_bit_cast(Frag, buf_load4(rs_w, w_voff + q * kWStep, soff));
+      dst = __builtin_bit_cast(Frag, buf_load4(rs_w, w_voff + q * kWStep, soff));
     };
+    auto fetch_w = [&](int soff, int slot, int q) { fetch_frag(w[slot][q], soff, q); };
     auto fetch_orow = [&](const StagePos &pos, int m, int slot) {
       orow[slot] = buf_load1(rs_out, l16 * 4 + m * 64, pos.g * 256);
     };
@@ -821,6 +852,36 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
       if (s + 1 < nstages) stage(std::integral_constant<int, 1>());
       if (s + 2 < nstages) stage(std::integral_constant<int, 2>());
     } else {
+    // The five-group form (a launch with xcol >= 0).  Besides its own column group, of
+    // which it multiplies the four row blocks of a stage, wave w multiplies row block w with
+    // the fragments of a fifth group (output columns xcol .., accumulator columns kCN ..):
+    // five blocks of MFMAs per stage and wave instead of four, and no SIMD that multiplies
+    // for a column block of one group.  The products of a row block stay in registers over
+    // the chunks of its group (dx).  Two row blocks of a group may hold the same output row,
+    // so the four waves must not add to the fifth group's accumulators between the same two
+    // barriers: wave w adds its products of a finished group (dprev, at aprev) during chunk
+    // w of the next group (nch >= 4, the host launches the form for such layers only), in
+    // the order of the row blocks, as the other column groups see their offsets; when a
+    // tile ends they are added at once, a barrier between each two waves.
+    //   wx[s & 1]  fragments of the fifth group for stage s, fetched one stage ahead
+    //   kofx       fragment offset of row block `wave` of the next stage
+    //   orowx      accumulator row of this lane's pair in row block `wave` of this stage
+    Frag wx[2][NF];
+    int kofx = 0, orowx = 0;
+    float4v dx = float4v{0.f, 0.f, 0.f, 0.f}, dprev = float4v{0.f, 0.f, 0.f, 0.f};
+    const int acc_lane_x = acc_base + (kCN + g * 4) * 4;
+    const int dummy_x = T * kAS * 4 + acc_lane_x;
+    int aprev = dummy_x;
+    bool x_pending = false;
+    const bool x_on = FIVE && xcol >= 0;
+    const char *const abx = a_base + wave * 16 * kRowB;
+    const int w_soffx = (x_on ? xcol / 16 : 0) * nch * kFragB;
+    auto load_kofx = [&](const StagePos &pos) -> int {
+      return buf_load1(rs_meta, wave * 4, pos.g * 32);
+    };
+    auto load_orowx = [&](const StagePos &pos) -> int {
+      return buf_load1(rs_out, l16 * 4 + wave * 64, pos.g * 256);
+    };
     Pending pend;  // nothing pending yet: the first write adds zero to the dummy row
     pend.addr = dummy_addr;
     pend.accr = float4v{0.f, 0.f, 0.f, 0.f};
@@ -916,6 +977,11 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
 #pragma unroll
             for (int qq = 0; qq < NF; ++qq)
               if (i == kGapA[qq]) load_a(m + 1, qq, a[(m + 1) & 1]);
+          } else if constexpr (FIVE) {  // row block `wave`, for the fifth group
+#pragma unroll
+            for (int qq = 0; qq < NF; ++qq)
+              if (i == kGapA[qq])
+                a[0][qq] = *reinterpret_cast<const Frag *>(abx + par * kStage * kRowB + qq * 64);
           }
           // this stage's record was last used by block 0: refill it for the stage
           // after the next
@@ -925,6 +991,42 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
         }
         __builtin_amdgcn_sched_barrier(0);
         pend.d = d;
+      }
+      if constexpr (FIVE) {
+        if (x_on) {
+          // gaps: 0 read of the accumulator row this wave adds to in this stage (the dummy
+          // row in other stages); 3 that update, fragment offset of the next stage;
+          // 4, 6, 8, 10 its fragments; 11, 12 the next offset and accumulator row
+          const bool mine = x_pending && cur.cc == wave;
+          const int caddr = mine ? aprev : dummy_x;
+          float4v accx = float4v{0.f, 0.f, 0.f, 0.f};
+          int soffx = 0;
+          constexpr int kGapXW[4] = {at(4), at(6), at(8), at(10)};
+#pragma unroll
+          for (int i = 0; i < kSteps; ++i) {
+            __builtin_amdgcn_sched_barrier(0);
+            dx = __builtin_amdgcn_mfma_f32_16x16x4f32(wx[par][i >> 2][i & 3], a[0][i >> 2][i & 3],
+                                                      dx, 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            if (i == at(0)) accx = lds_load4(caddr);
+            if (i == at(3)) {
+              soffx = frag_soff(kofx, w_soffx + next.cc * kFragB);
+              lds_store4(caddr, accx + dprev);
+            }
+#pragma unroll
+            for (int qq = 0; qq < NF; ++qq)
+              if (i == kGapXW[qq]) fetch_frag(wx[par ^ 1][qq], soffx, qq);
+            if (i == at(11)) kofx = load_kofx(after);
+          }
+          __builtin_amdgcn_sched_barrier(0);
+          if (cur.cc == nch - 1) {  // the group is complete
+            dprev = dx;
+            aprev = orowx + acc_lane_x;
+            dx = float4v{0.f, 0.f, 0.f, 0.f};
+            x_pending = true;
+          }
+          orowx = load_orowx(next);
+        }
       }
       __builtin_amdgcn_sched_barrier(0);
       if (last_cur) {  // the tile is written out after this stage: finish its last update
@@ -963,6 +1065,18 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
           __builtin_amdgcn_sched_barrier(0);
         }
       }
+      if constexpr (FIVE) {
+        if (x_on) {  // in the loop's order: fragments, next offset, accumulator row
+          kofx = load_kofx(p_cur);
+          const int soffx = frag_soff(kofx, w_soffx + p_cur.cc * kFragB);
+          __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+          for (int q = 0; q < NF; ++q) fetch_frag(wx[0][q], soffx, q);
+          __builtin_amdgcn_sched_barrier(0);
+          kofx = load_kofx(p_next);
+          orowx = load_orowx(p_cur);
+        }
+      }
     }
     __syncthreads();
     auto step = [&](auto parity) {
@@ -972,6 +1086,15 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
       p_after.advance(nch);
       __syncthreads();
       if (end.last) {
+        if constexpr (FIVE) {
+          // the last group's products of the fifth group, wave after wave
+#pragma unroll
+          for (int wv = 0; wv < 4; ++wv) {
+            if (x_on && wave == wv) lds_store4(aprev, lds_load4(aprev) + dprev);
+            __syncthreads();
+          }
+          x_pending = false;
+        }
         flush_tile(end.row0, end.rows, end.slot0);
         __syncthreads();
       }
@@ -1001,8 +1124,13 @@ struct ConvPlan {
   // three of four consumer waves would multiply for nothing: the full blocks take one launch
   // each over all CUs (n_launch of them, n_colblk = 1) and the kernel's one-column-group
   // form a last one (has_tail), all over the same plan.
+  // Or, for layers of four or more channel chunks, the last full block's launch takes the
+  // lone group along as a fifth one (five): every launch is then of the five-group form,
+  // whose accumulator rows are 16 columns wider (acc_cols), xcol >= 0 in the last only.
   int n_launch;
-  bool has_tail;
+  bool has_tail, five;
+  bool rebalance;  // the work split is made twice, the second time from the first one's counts
+  int acc_cols;  // accumulator columns of a workgroup: 64, or 80 in the five-group form
 };
 
 // Device buffers of a convolution call, in three groups with different lifetimes:
@@ -1022,7 +1150,7 @@ struct ConvWs {
   int32_t *sorted;
   uint32_t *bits;
   int32_t *prefix;
-  int32_t *tile_loc, *tile_nmb, *kofs, *tile_rng, *range_grp;
+  int32_t *tile_loc, *tile_nmb, *kofs, *tile_rng, *range_grp, *range_row1;
   int32_t *fine_segs, *range_row0, *tile_row0, *n_tiles_dev;
   int32_t *spill_end, *tile_slot0, *spill, *share_first, *share_cnt;
 };
@@ -1030,13 +1158,13 @@ struct ConvWs {
 // (switched by ssc_conv_tuning, for measurements)
 inline bool g_conv_by_column = true;  // one column block per XCD for large filters
 
-template <typename IO, int GATHER, int NCW, int NS, bool EPI, bool TAIL>
+template <typename IO, int GATHER, int NCW, int NS, bool EPI, int FORM>
 inline int launch_conv(const ConvPlan &p, const ConvWs &w, const IO *features, int64_t n_in,
-                       int c_in, int K, IO *out, int c_out, int col_base,
+                       int c_in, int K, IO *out, int c_out, int col_base, int xcol,
                        const ConvEpilogue &epi, hipStream_t s) {
   static bool attr_set = false;
   if (!attr_set) {
-    SSC_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(conv_fwd_kernel<IO, GATHER, NCW, NS, EPI, TAIL>),
+    SSC_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(conv_fwd_kernel<IO, GATHER, NCW, NS, EPI, FORM>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
     attr_set = true;
   }
@@ -1049,6 +1177,9 @@ inline int launch_conv(const ConvPlan &p, const ConvWs &w, const IO *features, i
   SSC_CHECK(p.n_wg >= 1 && p.n_colblk >= 1 && col_base % 16 == 0 &&
                 col_base + (p.n_colblk - 1) * 16 * NCW < c_out,
             SSC_ERUNTIME, "convolution launch outside the output columns");
+  SSC_CHECK(FORM == 2 ? (xcol < 0 || (xcol % 16 == 0 && xcol < c_out && p.nch >= 4 && p.n_colblk == 1))
+                      : xcol < 0,
+            SSC_ERUNTIME, "convolution launch with a fifth column group it is not built for");
   dim3 grid((unsigned)p.n_wg, (unsigned)p.n_colblk);
   // one column block per XCD when the packed filters are larger than an L2 can keep
   // (4 MiB per XCD) and the grid divides that way (256 -> 256 channels, 7 MiB: 2.44 ->
@@ -1061,19 +1192,19 @@ inline int launch_conv(const ConvPlan &p, const ConvWs &w, const IO *features, i
   const bool big = packed_bytes > ((uint64_t)4 << 20) && p.n_colblk > 1 && g_conv_by_column;
   const int cols_per_xcd = by_column ? 8 / p.n_colblk
                            : ((p.n_wg & 7) != 0 && p.n_wg * p.n_colblk >= 16) ? (big ? -2 : -1) : 0;
-  hipLaunchKernelGGL((conv_fwd_kernel<IO, GATHER, NCW, NS, EPI, TAIL>), grid, dim3((NCW + 4) * 64), p.lds_bytes, s, features, c_in,
+  hipLaunchKernelGGL((conv_fwd_kernel<IO, GATHER, NCW, NS, EPI, FORM>), grid, dim3((NCW + 4) * 64), p.lds_bytes, s, features, c_in,
                      feat_bytes, w.packed, (unsigned)packed_bytes, w.sched_in, w.sched_out,
                      w.grp_meta, (unsigned)sched_bytes, (unsigned)(p.grp_cap * 32), w.tile_grp,
-                     w.wg_tile, p.nch, p.ncb, out, c_out, p.T, cols_per_xcd, col_base, epi);
+                     w.wg_tile, p.nch, p.ncb, out, c_out, p.T, cols_per_xcd, col_base, xcol, epi);
   SSC_LAUNCH_CHECK("conv_fwd");
   return SSC_OK;
 }
 
 // The instances on float rows that conv.hip does not compile itself (conv_instances.h):
-// with the epilogue, and the one-column-group form with and without it.
-template <int GATHER, int NS, bool EPI, bool TAIL>
+// with the epilogue, and the one-column-group and five-group forms with and without it.
+template <int GATHER, int NS, bool EPI, int FORM>
 int launch_conv_f32(const ConvPlan &p, const ConvWs &w, const float *features, int64_t n_in,
-                    int c_in, int K, float *out, int c_out, int col_base,
+                    int c_in, int K, float *out, int c_out, int col_base, int xcol,
                     const ConvEpilogue &epi, hipStream_t s);
 
 }  // namespace ssc

@@ -1,4 +1,4 @@
 // The convolution kernel on float rows in its one-column-group form (conv_instances.h).
 #include "conv_instances.h"
 
-SSC_CONV_INSTANCES(false, true)
+SSC_CONV_INSTANCES(false, 1)

@@ -449,6 +449,48 @@ def test_conv_lone_last_column_group(shape, oracle, device):
     assert _ext._lib.ssc_conv_plan_bytes(1000, 27, cin, cout, 1000) > 0
 
 
+@pytest.mark.parametrize("shape", [(200, 72), (256, 200), (197, 70), (260, 136)])
+def test_conv_five_group_form(shape, oracle, device):
+    """More than 192 input channels (four chunks or more) and Cout = 64 b + (1..16), b >= 1:
+    one launch per block of 64 columns, the last of which takes the lone last group of 16
+    along as a fifth one (every wave multiplies one of its row blocks for it).  Against the
+    oracle, bit-reproducible, and equal up to the order of the float sums to the launch that
+    gives the group a column block of its own (ssc_conv_tuning flag 8)."""
+    from ss_conv import _ext
+    cin, cout = shape
+    print("shape", shape, flush=True)
+    a, ref = _conv_case(oracle, device, 2500, 16, 3, 1, 1, cin, cout, seed=37)
+    b, _ = _conv_case(oracle, device, 2500, 16, 3, 1, 1, cin, cout, seed=37)
+    assert torch.equal(a, b)
+    try:
+        assert _ext._lib.ssc_conv_tuning(1 | 8) == 0
+        c, _ = _conv_case(oracle, device, 2500, 16, 3, 1, 1, cin, cout, seed=37)
+    finally:
+        _ext._lib.ssc_conv_tuning(1)
+    assert rel_l2(a.cpu().numpy(), c.cpu().numpy()) < 1e-6
+    assert _ext._lib.ssc_conv_plan_bytes(1000, 27, cin, cout, 1000) > 0
+
+
+@pytest.mark.parametrize("case", [(2500, 16, 3, 1, 1, 64, 128), (900, 12, 3, 2, 1, 128, 256),
+                                  (400, 10, 5, 1, 2, 200, 200), (5, 8, 3, 1, 1, 5, 7),
+                                  (2500, 16, 3, 1, 1, 64, 72), (3000, 16, 3, 1, 1, 3, 152)])
+def test_conv_second_work_split(case, oracle, device):
+    """The work split made twice (plans of long kernels; forced here by ssc_conv_tuning flag
+    32): the second split moves the boundaries between the workgroups' ranges of output
+    rows, nothing else, so the sums and their order stay what they are -- bit-equal to the
+    plan of one split, and against the oracle."""
+    from ss_conv import _ext
+    print("case", case, flush=True)
+    n, grid, k, s, p, cin, cout = case
+    a, _ = _conv_case(oracle, device, n, grid, k, s, p, cin, cout, seed=41)
+    try:
+        assert _ext._lib.ssc_conv_tuning(1 | 32) == 0
+        b, _ = _conv_case(oracle, device, n, grid, k, s, p, cin, cout, seed=41)
+    finally:
+        _ext._lib.ssc_conv_tuning(1)
+    assert torch.equal(a, b)
+
+
 def test_conv_random_layers(device):
     """Forty seeded random layers -- channel counts on both sides of every block and chunk
     boundary (1 ... 200 in, 1 ... 152 out), kernels 1-3, strides 1-2, regular, submanifold and
@@ -1781,6 +1823,9 @@ EPILOGUE_CASES = [
     ([(16, 0)], 8, 3, 1, 1, False, None),                             # scalars only, no gates
     # 6.9 MB of packed filters in four column blocks: one column block per XCD
     ([(40, 0), (24, 1), (16, 2)], 256, 3, 1, 1, False, None),
+    # a plan of the five-group form (200 input channels, 74 columns in 5 groups): with the
+    # epilogue the lone group takes a launch of its own
+    ([(10, 0), (6, 1), (4, 2), (2, 3)], 200, 3, 1, 1, False, None),
 ]
 
 
