@@ -28,10 +28,11 @@ FP32_MFMA_PEAK_TFLOPS = 157.3  # MI355X dense fp32 matrix peak
 # sustained clock
 CLOCK_WARMUP_MS = 100
 
-# HBM bytes per launch of the convolution kernel for every workload this script offers, from
-# rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs scaled by a copy kernel of known size (the
-# summaries profiles/conv_fwd_<workload>_hbm_traffic.md give commands and counter values).
-MEASURED_TRAFFIC_BYTES = {"cfg1": 3016591, "cfg2": 345582696, "cfg3": 219239659, "cfg5": 56045076175}
+# HBM bytes per launch of the convolution kernel (per call for cfg5, whose call is three
+# launches) for every workload this script offers, from rocprofv3 --pmc FETCH_SIZE /
+# WRITE_SIZE runs scaled by a copy kernel of known size (the summaries
+# profiles/conv_fwd_<workload>_hbm_traffic.md give commands and counter values).
+MEASURED_TRAFFIC_BYTES = {"cfg1": 3042208, "cfg2": 345618323, "cfg3": 218785754, "cfg5": 70539916921}
 
 
 def parse_args():
@@ -385,14 +386,16 @@ def build_backbone(torch, synth, dev, seed):
 
 
 def thin_layer_table(torch, _ext, synth, dev, seed):
-    """Layers with Cout = 64 b + (1 ... 16), b <= 2, on the clouds of the second and third
+    """Layers with Cout = 64 b + (1 ... 16) on the clouds of the second and third
     configuration: the convolution kernel's time (HIP events around its launches) with the
-    last column group shared by the four consumer waves (the default) and with the group
-    in a column block of its own (ssc_conv_tuning flag 2)."""
+    last column group shared by the four consumer waves (the default: a launch of its own
+    for b <= 2, or, with more than 192 input channels, as a fifth group of the last block)
+    and with the group in a column block of its own (ssc_conv_tuning flags 2 and 8)."""
     from ss_conv.sp_ops.ops import get_indice_pairs
     rows = []
     for name, cin, cout, k, stride, pad in (("cfg2", 64, 72, 3, 1, 1), ("cfg2", 128, 136, 3, 1, 1),
-                                            ("cfg2", 152, 8, 3, 1, 1), ("cfg3", 128, 16, 3, 2, 1)):
+                                            ("cfg2", 152, 8, 3, 1, 1), ("cfg3", 128, 16, 3, 2, 1),
+                                            ("cfg3", 256, 72, 3, 2, 1), ("cfg2", 256, 136, 3, 1, 1)):
         cfg = synth.CONFIGS[name]
         pts, _, ids = synth.config_clouds(name, seed)
         idx = torch.from_numpy(synth.voxel_indices(pts, ids, cfg["grid"])).to(dev)
@@ -401,7 +404,7 @@ def thin_layer_table(torch, _ext, synth, dev, seed):
         f = torch.randn(idx.shape[0], cin, device=dev)
         w = torch.randn(k, k, k, cin, cout, device=dev) / (K * cin) ** 0.5
         times, outs = [], []
-        for flags in (1, 1 | 2):
+        for flags in (1, 1 | 2 | 8):
             _ext._lib.ssc_conv_tuning(flags)
             pr = pairs.clone()  # a rulebook without a plan of the other form
             try:

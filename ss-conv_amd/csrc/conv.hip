@@ -747,7 +747,7 @@ static int device_cu_count() {
 // (switched by ssc_conv_tuning, for measurements)
 static bool g_conv_tail = true;       // a launch of its own for a lone last column group
 static bool g_conv_five = true;       // the lone last group as a fifth one of the last block
-constexpr int64_t kRebalanceStages = 1000;
+constexpr int64_t kRebalanceStages = 1500;
 static int64_t g_conv_rebalance_stages = kRebalanceStages;
 static bool g_conv_rebalance = true;  // long kernels: a second work split from the first one's counts
 static bool g_conv_round8 = false;    // ranges per column block: a multiple of 8 only
@@ -812,11 +812,13 @@ static ConvPlan make_plan(int64_t n_in, int64_t n_out, int K, int c_in, int c_ou
   plan_split(p, n_wg, n_out, K, pair_stride);
   p.lds_bytes = conv_lds_bytes(p.T, p.acc_cols);
   // A second work split (split_rebalance_kernel) where the kernel runs long enough for four
-  // more small launches: some thousand stages per workgroup, estimated from the most pairs
-  // the rows can have -- a regular layer has about min(N_in, N_out) K, a strided one fewer.
+  // more small launches (30 us; the split evens out 3-15 % of the kernel's time, more with
+  // more ranges): 1500 stages per workgroup or more, estimated from the pairs the layer is
+  // likely to have -- N_in K where the outputs outnumber the inputs (stride 1), a quarter of
+  // N_out K for submanifold and strided layers.
   {
-    const int64_t rows = n_in > 0 && n_in < n_out ? n_in : n_out;
-    const int64_t stages = rows * K / 2 / kStage * p.nch / (p.n_wg > 0 ? p.n_wg : 1);
+    const int64_t pairs = n_in > 0 && n_in < n_out ? n_in * K : n_out * K / 4;
+    const int64_t stages = pairs / kStage * p.nch / (p.n_wg > 0 ? p.n_wg : 1);
     p.rebalance = g_conv_rebalance && stages >= g_conv_rebalance_stages;
   }
   return p;
