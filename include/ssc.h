@@ -318,7 +318,9 @@ int ssc_profile_conv(int32_t enable);
  *      sums of that group.
  *  16  no second work split: plans of long kernels (an estimated thousand stages or more
  *      per workgroup) otherwise deal the output rows to the workgroups twice, the second
- *      time by the row-block counts the first split came to.  Results do not depend on it.
+ *      time by the row-block counts the first split came to.  Results do not depend on it
+ *      (but for the last bits of a last group computed by a launch of its own, flag 2, whose
+ *      four partial sums follow the tiles).
  *  32  the second work split for every plan, whatever its size (for tests). */
 int ssc_conv_tuning(int32_t flags);
 int ssc_profile_conv_read(float *ms /* host */, int32_t capacity, int32_t *count /* host */);

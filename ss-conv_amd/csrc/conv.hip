@@ -306,7 +306,10 @@ __global__ void __launch_bounds__(256)
 // of each offset, writing the tile out).  Pairs per row come from a fine grid of
 // kSplitGranule rows; range boundaries lie on that grid.  Each range is then cut
 // into tiles of equal height <= T.
-constexpr int kSplitGranule = 64;
+// (16 rows where a range has fewer than 2048: with 3.5 cells of 64 rows to a range -- the
+// input gradient of the 64 -> 128 benchmark layer, 57 k rows for 256 workgroups -- the
+// ranges' work differed by 14 %)
+constexpr int kSplitGranule = 64, kSplitGranuleSmall = 16;
 // The accumulator window of a workgroup holds kSpillRows more rows than a tile is
 // high: the last row block that an offset contributes to a tile may then be filled
 // up with the offset's next pairs, whose rows lie in the following tile (at most
@@ -326,8 +329,8 @@ __device__ __forceinline__ int64_t split_tile_cost(int K) { return (int64_t)K * 
 
 // Work in rows below cell b of the fine grid (scaled by T to stay in integers).
 __device__ __forceinline__ int64_t split_work(int64_t pairs_below, int64_t b, int64_t n_out,
-                                              int T, int K) {
-  int64_t r = b * kSplitGranule;
+                                              int T, int K, int granule) {
+  int64_t r = b * granule;
   if (r > n_out) r = n_out;
   return pairs_below * T + r * split_tile_cost(K);
 }
@@ -337,7 +340,7 @@ __device__ __forceinline__ int64_t split_work(int64_t pairs_below, int64_t b, in
 // (work(b-1), work(b)].  range_row0[w], w = 0..n_wg.
 __global__ void __launch_bounds__(256)
     split_bounds_kernel(const int32_t *__restrict__ fine_segs, int K, int64_t nb, int64_t n_out,
-                        int T, int n_wg, int32_t *__restrict__ range_row0) {
+                        int T, int n_wg, int granule, int32_t *__restrict__ range_row0) {
   int64_t b = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (b > nb) return;
   int64_t below = 0, below_prev = 0, all = 0;
@@ -346,16 +349,16 @@ __global__ void __launch_bounds__(256)
     if (b > 0) below_prev += fine_segs[(b - 1) * K + k];
     all += fine_segs[nb * K + k];
   }
-  const int64_t total = split_work(all, nb, n_out, T, K);
+  const int64_t total = split_work(all, nb, n_out, T, K, granule);
   // ranges w with ceil(total * w / n_wg) <= work, i.e. w <= work * n_wg / total
   auto reached = [&](int64_t work) -> int64_t {
     if (total <= 0) return n_wg + 1;
     int64_t c = work * n_wg / total + 1;
     return c > n_wg + 1 ? n_wg + 1 : c;
   };
-  const int64_t w0 = b > 0 ? reached(split_work(below_prev, b - 1, n_out, T, K)) : 0;
-  const int64_t w1 = reached(split_work(below, b, n_out, T, K));
-  int64_t r = b * kSplitGranule;
+  const int64_t w0 = b > 0 ? reached(split_work(below_prev, b - 1, n_out, T, K, granule)) : 0;
+  const int64_t w1 = reached(split_work(below, b, n_out, T, K, granule));
+  int64_t r = b * granule;
   if (r > n_out) r = n_out;
   for (int64_t w = w0; w < w1; ++w)
     range_row0[w] = (w == 0) ? 0 : (w == n_wg ? (int32_t)n_out : (int32_t)r);
@@ -374,16 +377,17 @@ __global__ void __launch_bounds__(256)
 // there.  row_old: range_row0 of the first split; row_new: that of the second.
 __global__ void __launch_bounds__(256)
     split_rebalance_kernel(const int32_t *__restrict__ fine_segs, int K, int64_t nb,
-                           int64_t n_out, int T, int n_wg, const int32_t *__restrict__ row_old,
+                           int64_t n_out, int T, int n_wg, int granule,
+                           const int32_t *__restrict__ row_old,
                            const int32_t *__restrict__ range_grp, int32_t *__restrict__ row_new) {
   __shared__ int row_s[257];
   __shared__ double work_s[257];  // modelled work below the first row of range w
   __shared__ double grp_s[257];   // groups of the ranges before range w
-  auto cell_of = [&](int64_t row) -> int64_t { return (row + kSplitGranule - 1) / kSplitGranule; };
+  auto cell_of = [&](int64_t row) -> int64_t { return (row + granule - 1) / granule; };
   auto work_below = [&](int64_t cell) -> double {
     int64_t below = 0;
     for (int k = 0; k < K; ++k) below += fine_segs[cell * K + k];
-    return (double)split_work(below, cell, n_out, T, K);
+    return (double)split_work(below, cell, n_out, T, K, granule);
   };
   for (int w = threadIdx.x; w <= n_wg; w += blockDim.x) {  // n_wg <= 256
     int r = row_old[w];
@@ -408,7 +412,7 @@ __global__ void __launch_bounds__(256)
   // corrected work below cell c
   auto cum = [&](int64_t c) -> double {
     if (c >= nb) return total;
-    int64_t r = c * kSplitGranule;
+    int64_t r = c * granule;
     if (r > n_out) r = n_out;
     // the last range that begins at or before row r and does not end there
     int lo = 0, hi = n_wg - 1;
@@ -429,7 +433,7 @@ __global__ void __launch_bounds__(256)
   };
   const int64_t w0 = b > 0 ? reached(cum(b - 1)) : 0;
   const int64_t w1 = reached(cum(b));
-  int64_t r = b * kSplitGranule;
+  int64_t r = b * granule;
   if (r > n_out) r = n_out;
   for (int64_t w = w0; w < w1; ++w)
     row_new[w] = (w == 0) ? 0 : (w == n_wg ? (int32_t)n_out : (int32_t)r);
@@ -757,7 +761,8 @@ static void plan_split(ConvPlan &p, int n_wg, int64_t n_out, int K, int64_t pair
   p.n_wg = n_wg;
   // upper bound of the tile count: every workgroup's range ends with a partial tile
   p.n_tiles = ceil_div(n_out > 0 ? n_out : 1, p.tile_rows) + n_wg;
-  p.n_fine = ceil_div(n_out > 0 ? n_out : 1, kSplitGranule);
+  p.granule = n_out / n_wg < 2048 ? kSplitGranuleSmall : kSplitGranule;
+  p.n_fine = ceil_div(n_out > 0 ? n_out : 1, p.granule);
   p.words_per_k = ceil_div(n_out > 0 ? n_out : 1, 32);
   // groups: pairs/64 plus, per (tile, offset), up to one partial block, plus one
   // partial (or empty) group per tile, plus the groups the kernel's prefetches may
@@ -1095,9 +1100,9 @@ static int conv_plan_build(const ConvPlan &p, const ConvWs &w, const int32_t *pa
   }
   hipLaunchKernelGGL(grid_segments_kernel<PACK_IO>, seg_grid, dim3(256), 0, s, w.flag,
                      in_order ? 1 : 0, pairs, w.sorted, pair_stride, plane_s, pair_num, K, p.n_fine,
-                     kSplitGranule, w.fine_segs, pk);
+                     p.granule, w.fine_segs, pk);
   hipLaunchKernelGGL(split_bounds_kernel, dim3((unsigned)ceil_div(p.n_fine + 1, 256)), dim3(256), 0,
-                     s, w.fine_segs, K, p.n_fine, n_out, p.tile_rows, p.n_wg, w.range_row0);
+                     s, w.fine_segs, K, p.n_fine, n_out, p.tile_rows, p.n_wg, p.granule, w.range_row0);
   // the ranges' tiles, their segments, shares and row-block counts
   const int64_t nseg = (p.n_tiles + 1) * K;
   auto tiles_of = [&](const int32_t *range_row0) -> int {
@@ -1107,7 +1112,7 @@ static int conv_plan_build(const ConvPlan &p, const ConvWs &w, const int32_t *pa
     SSC_LAUNCH_CHECK("split");
     hipLaunchKernelGGL(tile_segments_kernel, dim3((unsigned)ceil_div(nseg, 256)), dim3(256), 0, s,
                        w.flag, pairs, w.sorted, pair_stride, plane_s, pair_num, K, w.n_tiles_dev,
-                       w.tile_row0, n_out, w.fine_segs, kSplitGranule, w.spill_end, w.segs,
+                       w.tile_row0, n_out, w.fine_segs, p.granule, w.spill_end, w.segs,
                        w.spill);
     SSC_LAUNCH_CHECK("tile_segments");
     hipLaunchKernelGGL(range_sched_kernel, dim3((unsigned)p.n_wg), dim3(kRangeSchedThreads), 0, s,
@@ -1121,7 +1126,7 @@ static int conv_plan_build(const ConvPlan &p, const ConvWs &w, const int32_t *pa
   if (p.rebalance) {  // long kernels: once more, from the groups the ranges came to
     hipLaunchKernelGGL(split_rebalance_kernel, dim3((unsigned)ceil_div(p.n_fine + 1, 256)),
                        dim3(256), 0, s, w.fine_segs, K, p.n_fine, n_out, p.tile_rows, p.n_wg,
-                       w.range_row0, w.range_grp, w.range_row1);
+                       p.granule, w.range_row0, w.range_grp, w.range_row1);
     SSC_LAUNCH_CHECK("split_rebalance");
     rc = tiles_of(w.range_row1);
     if (rc != SSC_OK) return rc;

@@ -1117,6 +1117,7 @@ struct ConvPlan {
   int gather;  // conv_fwd_kernel's GATHER
   int ns;      // conv_fwd_kernel's NS: MFMA steps per chunk
   int64_t n_tiles, n_fine, words_per_k, grp_cap;  // n_tiles: upper bound
+  int granule;  // rows per cell of the grid the work split places its boundaries on
   size_t lds_bytes;
   // Launches.  As a rule one, over all column blocks (n_colblk of them side by side, the
   // CUs shared out among them).  A last column group that would be alone in its block of
