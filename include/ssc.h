@@ -310,7 +310,8 @@ int ssc_profile_conv(int32_t enable);
  *      across a change.  Results agree up to the order of the float sums of that group.
  *   4  the ranges of output rows per column block rounded down to a multiple of 8 (leaves
  *      CUs without a workgroup where the column blocks do not divide them that way; the
- *      default gives every CU one).  Changes the same sizes; results do not depend on it.
+ *      default gives every CU one).  Changes the same sizes; results agree up to the order
+ *      of the float sums (see 16).
  *   8  no five-group form: float layers of more than 192 input channels whose last group
  *      of 16 output columns would be alone in its block of 64 (Cout = 200, 72 + 64 n)
  *      otherwise run one launch per block of 64 columns, the last of which takes the lone
@@ -318,9 +319,10 @@ int ssc_profile_conv(int32_t enable);
  *      sums of that group.
  *  16  no second work split: plans of long kernels (an estimated thousand stages or more
  *      per workgroup) otherwise deal the output rows to the workgroups twice, the second
- *      time by the row-block counts the first split came to.  Results do not depend on it
- *      (but for the last bits of a last group computed by a launch of its own, flag 2, whose
- *      four partial sums follow the tiles).
+ *      time by the row-block counts the first split came to.  Results agree up to the
+ *      order of the float sums (an output row's products are added offset by offset within
+ *      a row-block group and chunk by chunk over the groups; which offsets share a group
+ *      follows the tiles); every plan by itself is bit-reproducible.
  *  32  the second work split for every plan, whatever its size (for tests). */
 int ssc_conv_tuning(int32_t flags);
 int ssc_profile_conv_read(float *ms /* host */, int32_t capacity, int32_t *count /* host */);
