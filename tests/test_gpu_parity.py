@@ -501,7 +501,7 @@ def test_conv_second_work_split(case, oracle, device):
 
 def test_conv_random_layers(device):
     """Forty seeded random layers -- channel counts on both sides of every block and chunk
-    boundary (1 ... 200 in, 1 ... 152 out), kernels 1-3, strides 1-2, regular, submanifold and
+    boundary (1 ... 260 in, 1 ... 200 out), kernels 1-3, strides 1-2, regular, submanifold and
     transposed rulebooks -- forward and both gradients against a float64 statement of the
     same sums (one GEMM and one index_add per offset, src/conv/indice_conv.h:296-338,
     385-421) evaluated with torch on the GPU."""
@@ -514,8 +514,8 @@ def test_conv_random_layers(device):
         p = int(rng.integers(0, k))
         tr = bool(rng.integers(0, 4) == 0)
         subm = (not tr) and k == 3 and bool(rng.integers(0, 5) == 0)
-        cin = int(rng.choice([1, 3, 5, 8, 16, 37, 40, 64, 72, 100, 128, 152, 200]))
-        cout = int(rng.choice([1, 3, 7, 8, 16, 17, 24, 64, 65, 72, 80, 96, 129, 136, 144, 152]))
+        cin = int(rng.choice([1, 3, 5, 8, 16, 37, 40, 64, 72, 100, 128, 152, 200, 197, 260]))
+        cout = int(rng.choice([1, 3, 7, 8, 16, 17, 24, 64, 65, 72, 80, 96, 129, 136, 144, 152, 200]))
         print("layer", it, (batch, grid, n, k, s, p, tr, subm, cin, cout), flush=True)
         idx = torch.from_numpy(random_voxels(rng, batch, grid, min(n, batch * grid ** 3))).to(device)
         o_idx, pairs, num = get_indice_pairs(idx, batch, [grid] * 3, k, s, p, 1, 0, subm, tr)
