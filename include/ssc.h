@@ -323,7 +323,12 @@ int ssc_profile_conv(int32_t enable);
  *      order of the float sums (an output row's products are added offset by offset within
  *      a row-block group and chunk by chunk over the groups; which offsets share a group
  *      follows the tiles); every plan by itself is bit-reproducible.
- *  32  the second work split for every plan, whatever its size (for tests). */
+ *  32  the second work split for every plan, whatever its size (for tests).
+ *  64  one range of output rows to a workgroup for every plan: plans of middle size (an
+ *      estimated 80 row-block groups per workgroup or more, and no second split) otherwise
+ *      cut the rows into two ranges per workgroup and give a workgroup two of them by the
+ *      groups they came to, many with few.  Changes the sizes; results as for 16.
+ * 128  two ranges to a workgroup for every plan (for tests). */
 int ssc_conv_tuning(int32_t flags);
 int ssc_profile_conv_read(float *ms /* host */, int32_t capacity, int32_t *count /* host */);
 

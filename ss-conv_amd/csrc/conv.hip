@@ -310,6 +310,7 @@ __global__ void __launch_bounds__(256)
 // input gradient of the 64 -> 128 benchmark layer, 57 k rows for 256 workgroups -- the
 // ranges' work differed by 14 %)
 constexpr int kSplitGranule = 64, kSplitGranuleSmall = 16;
+constexpr int kMaxRanges = 512;  // two for each of at most 256 workgroups
 // The accumulator window of a workgroup holds kSpillRows more rows than a tile is
 // high: the last row block that an offset contributes to a tile may then be filled
 // up with the offset's next pairs, whose rows lie in the following tile (at most
@@ -380,16 +381,16 @@ __global__ void __launch_bounds__(256)
                            int64_t n_out, int T, int n_wg, int granule,
                            const int32_t *__restrict__ row_old,
                            const int32_t *__restrict__ range_grp, int32_t *__restrict__ row_new) {
-  __shared__ int row_s[257];
-  __shared__ double work_s[257];  // modelled work below the first row of range w
-  __shared__ double grp_s[257];   // groups of the ranges before range w
+  __shared__ int row_s[kMaxRanges + 1];
+  __shared__ double work_s[kMaxRanges + 1];  // modelled work below the first row of range w
+  __shared__ double grp_s[kMaxRanges + 1];   // groups of the ranges before range w
   auto cell_of = [&](int64_t row) -> int64_t { return (row + granule - 1) / granule; };
   auto work_below = [&](int64_t cell) -> double {
     int64_t below = 0;
     for (int k = 0; k < K; ++k) below += fine_segs[cell * K + k];
     return (double)split_work(below, cell, n_out, T, K, granule);
   };
-  for (int w = threadIdx.x; w <= n_wg; w += blockDim.x) {  // n_wg <= 256
+  for (int w = threadIdx.x; w <= n_wg; w += blockDim.x) {  // n_wg ranges, <= kMaxRanges
     int r = row_old[w];
     if (w == 0) r = 0;
     if (w == n_wg) r = (int)n_out;
@@ -445,14 +446,14 @@ __global__ void __launch_bounds__(256)
 // first row of tile t itself when t starts a workgroup's range: no spill across
 // ranges); tile_slot0[t]: accumulator slot of the first row of tile t.  T is the
 // largest tile height, window the height of the accumulator window.
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(kMaxRanges)
     split_rows_kernel(const int32_t *__restrict__ range_row0, int64_t n_out, int T, int window,
                       int n_wg, int32_t *__restrict__ wg_tile, int32_t *__restrict__ tile_row0,
                       int32_t *__restrict__ n_tiles_dev, int32_t *__restrict__ spill_end,
                       int32_t *__restrict__ tile_slot0) {
-  __shared__ int row_s[257];
-  __shared__ int tile_s[257];
-  for (int w = threadIdx.x; w <= n_wg; w += blockDim.x) {  // n_wg <= 256
+  __shared__ int row_s[kMaxRanges + 1];
+  __shared__ int tile_s[kMaxRanges + 1];
+  for (int w = threadIdx.x; w <= n_wg; w += blockDim.x) {  // n_wg ranges, <= kMaxRanges
     int r = range_row0[w];
     if (w == 0) r = 0;
     if (w == n_wg) r = (int)n_out;
@@ -460,8 +461,8 @@ __global__ void __launch_bounds__(256)
   }
   __syncthreads();
   {
-    // exclusive scan of the tile counts of the (at most 256) ranges, one per thread
-    __shared__ int wave_sum[4];
+    // exclusive scan of the tile counts of the ranges, one per thread
+    __shared__ int wave_sum[kMaxRanges / 64];
     const int w = threadIdx.x, lane = w & 63;
     const int nt = w < n_wg ? (row_s[w + 1] - row_s[w] + T - 1) / T : 0;
     int incl = nt;
@@ -475,7 +476,7 @@ __global__ void __launch_bounds__(256)
     int before = 0;
     for (int i = 0; i < (w >> 6); ++i) before += wave_sum[i];
     if (w < n_wg) tile_s[w] = before + incl - nt;
-    if (w == 255) {
+    if (w == kMaxRanges - 1) {
       const int run = before + incl;
       tile_s[n_wg] = run;
       n_tiles_dev[0] = run;
@@ -617,6 +618,63 @@ __global__ void __launch_bounds__(kRangeSchedThreads)
   }
 }
 
+// Two ranges to a workgroup (n_rng = 2 n_wg): which two, by the row-block groups the ranges
+// came to.  What a range costs is known only once its schedule is counted, and the ranges
+// of equal modelled work differ by 5-10 % there.  Inside every run of 32 consecutive ranges
+// (neighbours in the rows, whose gathers share an L2) the range with the most groups goes
+// with the one with the fewest, the second with the last but one, ...: 16 workgroups whose
+// sums differ far less than the ranges do.  One block.  range_g0[r]: first group of range r
+// in the schedule, where a workgroup's two ranges follow each other, the one of the lower
+// rows first; wg_grp[v], v = 0..n_wg: first group of workgroup v.
+__global__ void __launch_bounds__(kMaxRanges)
+    range_assign_kernel(const int32_t *__restrict__ range_grp, int n_rng, int n_wg,
+                        int32_t *__restrict__ range_g0, int32_t *__restrict__ wg_grp) {
+  __shared__ int cnt_s[kMaxRanges];
+  __shared__ int member_s[kMaxRanges];  // the two ranges of workgroup v: [2v], [2v + 1]
+  __shared__ int sum_s[kMaxRanges / 2 + 1];
+  const int r = threadIdx.x;
+  const int c = r < n_rng ? range_grp[r] : 0;
+  cnt_s[r] = c;
+  __syncthreads();
+  if (r < n_rng) {
+    const int base = r & ~31;
+    const int width = min(32, n_rng - base);  // even: n_rng is
+    int rank = 0;
+    for (int j = 0; j < width; ++j) {
+      const int cj = cnt_s[base + j];
+      rank += (cj > c || (cj == c && base + j < r)) ? 1 : 0;
+    }
+    const int q = rank < width / 2 ? rank : width - 1 - rank;
+    member_s[2 * (base / 2 + q) + (rank < width / 2 ? 0 : 1)] = r;
+  }
+  __syncthreads();
+  if (r < n_wg) {
+    const int a = member_s[2 * r], b = member_s[2 * r + 1];
+    if (a > b) {
+      member_s[2 * r] = b;
+      member_s[2 * r + 1] = a;
+    }
+    sum_s[r] = cnt_s[a] + cnt_s[b];
+  }
+  __syncthreads();
+  if (r == 0) {  // at most 256 sums
+    int run = 0;
+    for (int v = 0; v < n_wg; ++v) {
+      const int t = sum_s[v];
+      sum_s[v] = run;
+      run += t;
+    }
+    sum_s[n_wg] = run;
+  }
+  __syncthreads();
+  if (r <= n_wg) wg_grp[r] = sum_s[r];
+  if (r < n_wg) {
+    const int a = member_s[2 * r], b = member_s[2 * r + 1];
+    range_g0[a] = sum_s[r];
+    range_g0[b] = sum_s[r] + cnt_s[a];
+  }
+}
+
 // 16 threads per (tile, offset): lane i fills slot i of each of its row blocks; the
 // threads of offset 0 also write the tile's padding blocks and its group -> tile map.
 // (Blocks that take several times 16 (tile, offset) combinations, to compute the prefix over
@@ -628,16 +686,20 @@ __global__ void __launch_bounds__(256)
                       const int32_t *__restrict__ share_cnt, const int32_t *__restrict__ kofs,
                       const int32_t *__restrict__ tile_nmb, const int32_t *__restrict__ tile_loc,
                       const int32_t *__restrict__ tile_rng, const int32_t *__restrict__ range_grp,
-                      int n_wg, int32_t *__restrict__ tile_grp, int K,
+                      int n_wg, const int32_t *__restrict__ range_g0_paired,
+                      int32_t *__restrict__ wg_grp, int32_t *__restrict__ tile_grp, int K,
                       const int32_t *__restrict__ n_tiles_dev,
                       const int32_t *__restrict__ tile_row0,
                       const int32_t *__restrict__ tile_slot0, int T, uint32_t in_scale,
                       uint32_t in_pad, int out_scale, int k_scale,
                       int32_t *__restrict__ sched_in, int32_t *__restrict__ sched_out,
                       int32_t *__restrict__ grp_meta) {
-  // groups before every range (n_wg <= 256 of them): exclusive prefix of range_grp
+  // groups before every range (n_wg <= 256 of them): exclusive prefix of range_grp, which
+  // is also where the workgroups begin (block 0 writes that down for the convolution
+  // kernel) -- or, with two ranges to a workgroup, what range_assign_kernel found
+  // (range_g0_paired)
   __shared__ int range_g0[257];
-  {
+  if (range_g0_paired == nullptr) {
     __shared__ int wave_sum[4];
     const int w = threadIdx.x, wl = w & 63;
     const int v = w < n_wg ? range_grp[w] : 0;
@@ -654,6 +716,10 @@ __global__ void __launch_bounds__(256)
     range_g0[w] = before + incl - v;
     if (w == 255) range_g0[256] = before + incl;
     __syncthreads();
+    if (blockIdx.x == 0) {
+      for (int i = threadIdx.x; i <= n_wg; i += blockDim.x)
+        wg_grp[i] = range_g0[i];
+    }
   }
   const int64_t n_tiles = n_tiles_dev[0];
   const int32_t *src = flag[0] ? sorted : pairs;
@@ -664,9 +730,10 @@ __global__ void __launch_bounds__(256)
   int64_t t = tk / K;
   int k = (int)(tk - t * K);
   const int rng = tile_rng[t];
-  const int64_t g0 = range_g0[rng] + tile_loc[t];
-  const int64_t g1 = (t + 1 < n_tiles && tile_rng[t + 1] == rng) ? range_g0[rng] + tile_loc[t + 1]
-                                                                : range_g0[rng + 1];
+  const int64_t rg0 = range_g0_paired ? range_g0_paired[rng] : range_g0[rng];
+  const int64_t g0 = rg0 + tile_loc[t];
+  const int64_t g1 = (t + 1 < n_tiles && tile_rng[t + 1] == rng) ? rg0 + tile_loc[t + 1]
+                                                                : rg0 + range_grp[rng];
   if (k == 0 && lane == 0) {  // the tiles' first groups, for the convolution kernel
     tile_grp[t] = (int32_t)g0;
     if (t + 1 == n_tiles) tile_grp[n_tiles] = (int32_t)g1;
@@ -752,16 +819,20 @@ static int device_cu_count() {
 static bool g_conv_tail = true;       // a launch of its own for a lone last column group
 static bool g_conv_five = true;       // the lone last group as a fifth one of the last block
 constexpr int64_t kRebalanceStages = 1500;
+constexpr int64_t kPairGroups = 80;  // estimated groups per workgroup from which ranges are paired
+static bool g_conv_pair = true, g_conv_pair_always = false;
 static int64_t g_conv_rebalance_stages = kRebalanceStages;
 static bool g_conv_rebalance = true;  // long kernels: a second work split from the first one's counts
 static bool g_conv_round8 = false;    // ranges per column block: a multiple of 8 only
 
 // The sizes that follow from the number of workgroups per column block.
-static void plan_split(ConvPlan &p, int n_wg, int64_t n_out, int K, int64_t pair_stride) {
+static void plan_split(ConvPlan &p, int n_wg, int n_rng, int64_t n_out, int K,
+                       int64_t pair_stride) {
   p.n_wg = n_wg;
-  // upper bound of the tile count: every workgroup's range ends with a partial tile
-  p.n_tiles = ceil_div(n_out > 0 ? n_out : 1, p.tile_rows) + n_wg;
-  p.granule = n_out / n_wg < 2048 ? kSplitGranuleSmall : kSplitGranule;
+  p.n_rng = n_rng;
+  // upper bound of the tile count: every range ends with a partial tile
+  p.n_tiles = ceil_div(n_out > 0 ? n_out : 1, p.tile_rows) + n_rng;
+  p.granule = n_out / n_rng < 2048 ? kSplitGranuleSmall : kSplitGranule;
   p.n_fine = ceil_div(n_out > 0 ? n_out : 1, p.granule);
   p.words_per_k = ceil_div(n_out > 0 ? n_out : 1, 32);
   // groups: pairs/64 plus, per (tile, offset), up to one partial block, plus one
@@ -810,22 +881,29 @@ static ConvPlan make_plan(int64_t n_in, int64_t n_out, int K, int c_in, int c_ou
   p.n_launch = serial ? blocks : 1;
   int n_wg = device_cu_count() / p.n_colblk;
   if (n_wg < 1) n_wg = 1;
-  if (n_wg > 256) n_wg = 256;  // the split kernel is one block of 256 threads
+  if (n_wg > 256) n_wg = 256;  // the kernels of the split hold a number per workgroup in LDS
   // (every CU a workgroup, also where the column blocks do not divide the CUs by a
   // multiple of 8: the kernel then deals its workgroups to the XCDs by its general rule)
   if (n_wg >= 8 && g_conv_round8) n_wg = n_wg / 8 * 8;
-  plan_split(p, n_wg, n_out, K, pair_stride);
-  p.lds_bytes = conv_lds_bytes(p.T, p.acc_cols);
+  // estimates from the pairs the layer is likely to have -- N_in K where the outputs
+  // outnumber the inputs (stride 1), a quarter of N_out K for submanifold and strided
+  // layers: stages and row-block groups per workgroup
+  const int64_t est_pairs = n_in > 0 && n_in < n_out ? n_in * K : n_out * K / 4;
+  const int64_t est_groups = est_pairs / kStage / n_wg;
+  const int64_t est_stages = est_groups * p.nch;
   // A second work split (split_rebalance_kernel) where the kernel runs long enough for four
   // more small launches (30 us; the split evens out 3-15 % of the kernel's time, more with
-  // more ranges): 1500 stages per workgroup or more, estimated from the pairs the layer is
-  // likely to have -- N_in K where the outputs outnumber the inputs (stride 1), a quarter of
-  // N_out K for submanifold and strided layers.
-  {
-    const int64_t pairs = n_in > 0 && n_in < n_out ? n_in * K : n_out * K / 4;
-    const int64_t stages = pairs / kStage * p.nch / (p.n_wg > 0 ? p.n_wg : 1);
-    p.rebalance = g_conv_rebalance && stages >= g_conv_rebalance_stages;
-  }
+  // more ranges): 1500 stages per workgroup or more.
+  p.rebalance = g_conv_rebalance && est_stages >= g_conv_rebalance_stages;
+  // Two ranges to a workgroup, paired by what they came to (range_assign_kernel): one more
+  // small launch and one more range end per workgroup, whose last row blocks cannot be
+  // filled from a next tile (K / 8 groups), against the 5-10 % by which single ranges
+  // differ.  Not with the second split, which leaves less than that to even out.
+  const bool pair = g_conv_pair && n_wg >= 2 &&
+                    (g_conv_pair_always ||
+                     (!p.rebalance && est_groups >= kPairGroups && est_groups >= (int64_t)K / 2));
+  plan_split(p, n_wg, pair ? 2 * n_wg : n_wg, n_out, K, pair_stride);
+  p.lds_bytes = conv_lds_bytes(p.T, p.acc_cols);
   return p;
 }
 
@@ -838,13 +916,15 @@ static size_t conv_packed_bytes(const ConvPlan &p, int K) {
 static size_t conv_plan_walk(void *base, const ConvPlan &p, ConvWs *w) {
   Carver c(base);
   int32_t *tile_grp = c.take<int32_t>((size_t)p.n_tiles + 1);
-  int32_t *wg_tile = c.take<int32_t>((size_t)p.n_wg + 1);
+  int32_t *wg_tile = c.take<int32_t>((size_t)p.n_rng + 1);
+  int32_t *wg_grp = c.take<int32_t>((size_t)p.n_wg + 1);
   int32_t *sched_in = c.take<int32_t>((size_t)p.grp_cap * 64);
   int32_t *sched_out = c.take<int32_t>((size_t)p.grp_cap * 64);
   int32_t *grp_meta = c.take<int32_t>((size_t)p.grp_cap * 8);
   if (w) {
     w->tile_grp = tile_grp;
     w->wg_tile = wg_tile;
+    w->wg_grp = wg_grp;
     w->sched_in = sched_in;
     w->sched_out = sched_out;
     w->grp_meta = grp_meta;
@@ -865,7 +945,7 @@ static size_t conv_scratch_walk(void *base, const ConvPlan &p, int K, int64_t pa
   t.tile_nmb = c.take<int32_t>((size_t)p.n_tiles);
   t.kofs = c.take<int32_t>((size_t)p.n_tiles * K);
   t.fine_segs = c.take<int32_t>((size_t)(p.n_fine + 1) * K);
-  t.range_row0 = c.take<int32_t>((size_t)p.n_wg + 1);
+  t.range_row0 = c.take<int32_t>((size_t)p.n_rng + 1);
   t.tile_row0 = c.take<int32_t>((size_t)p.n_tiles + 1);
   t.spill_end = c.take<int32_t>((size_t)p.n_tiles + 1);
   t.tile_slot0 = c.take<int32_t>((size_t)p.n_tiles + 1);
@@ -874,8 +954,9 @@ static size_t conv_scratch_walk(void *base, const ConvPlan &p, int K, int64_t pa
   t.share_cnt = c.take<int32_t>((size_t)p.n_tiles * K);
   t.n_tiles_dev = c.take<int32_t>(1);
   t.tile_rng = c.take<int32_t>((size_t)p.n_tiles + 1);
-  t.range_grp = c.take<int32_t>((size_t)p.n_wg + 1);
-  t.range_row1 = c.take<int32_t>((size_t)p.n_wg + 1);
+  t.range_grp = c.take<int32_t>((size_t)p.n_rng + 1);
+  t.range_row1 = c.take<int32_t>((size_t)p.n_rng + 1);
+  t.range_g0 = c.take<int32_t>((size_t)p.n_rng + 1);
   if (w) {
     w->flag = t.flag;
     w->segs = t.segs;
@@ -897,6 +978,7 @@ static size_t conv_scratch_walk(void *base, const ConvPlan &p, int K, int64_t pa
     w->tile_rng = t.tile_rng;
     w->range_grp = t.range_grp;
     w->range_row1 = t.range_row1;
+    w->range_g0 = t.range_g0;
   }
   return c.used;
 }
@@ -1012,6 +1094,8 @@ int ssc_conv_tuning(int32_t flags) {
   g_conv_five = (flags & 8) == 0;
   g_conv_rebalance = (flags & 16) == 0;
   g_conv_rebalance_stages = (flags & 32) != 0 ? 0 : kRebalanceStages;
+  g_conv_pair = (flags & 64) == 0;
+  g_conv_pair_always = (flags & 128) != 0;
   return SSC_OK;
 }
 
@@ -1102,12 +1186,12 @@ static int conv_plan_build(const ConvPlan &p, const ConvWs &w, const int32_t *pa
                      in_order ? 1 : 0, pairs, w.sorted, pair_stride, plane_s, pair_num, K, p.n_fine,
                      p.granule, w.fine_segs, pk);
   hipLaunchKernelGGL(split_bounds_kernel, dim3((unsigned)ceil_div(p.n_fine + 1, 256)), dim3(256), 0,
-                     s, w.fine_segs, K, p.n_fine, n_out, p.tile_rows, p.n_wg, p.granule, w.range_row0);
+                     s, w.fine_segs, K, p.n_fine, n_out, p.tile_rows, p.n_rng, p.granule, w.range_row0);
   // the ranges' tiles, their segments, shares and row-block counts
   const int64_t nseg = (p.n_tiles + 1) * K;
   auto tiles_of = [&](const int32_t *range_row0) -> int {
-    hipLaunchKernelGGL(split_rows_kernel, dim3(1), dim3(256), 0, s, range_row0, n_out, p.tile_rows,
-                       p.T, p.n_wg, w.wg_tile, w.tile_row0, w.n_tiles_dev, w.spill_end,
+    hipLaunchKernelGGL(split_rows_kernel, dim3(1), dim3(kMaxRanges), 0, s, range_row0, n_out,
+                       p.tile_rows, p.T, p.n_rng, w.wg_tile, w.tile_row0, w.n_tiles_dev, w.spill_end,
                        w.tile_slot0);
     SSC_LAUNCH_CHECK("split");
     hipLaunchKernelGGL(tile_segments_kernel, dim3((unsigned)ceil_div(nseg, 256)), dim3(256), 0, s,
@@ -1115,7 +1199,7 @@ static int conv_plan_build(const ConvPlan &p, const ConvWs &w, const int32_t *pa
                        w.tile_row0, n_out, w.fine_segs, p.granule, w.spill_end, w.segs,
                        w.spill);
     SSC_LAUNCH_CHECK("tile_segments");
-    hipLaunchKernelGGL(range_sched_kernel, dim3((unsigned)p.n_wg), dim3(kRangeSchedThreads), 0, s,
+    hipLaunchKernelGGL(range_sched_kernel, dim3((unsigned)p.n_rng), dim3(kRangeSchedThreads), 0, s,
                        w.segs, w.spill, K, w.wg_tile, w.share_first, w.share_cnt, w.kofs,
                        w.tile_nmb, w.tile_loc, w.tile_rng, w.range_grp);
     SSC_LAUNCH_CHECK("range_sched");
@@ -1125,17 +1209,24 @@ static int conv_plan_build(const ConvPlan &p, const ConvWs &w, const int32_t *pa
   if (rc != SSC_OK) return rc;
   if (p.rebalance) {  // long kernels: once more, from the groups the ranges came to
     hipLaunchKernelGGL(split_rebalance_kernel, dim3((unsigned)ceil_div(p.n_fine + 1, 256)),
-                       dim3(256), 0, s, w.fine_segs, K, p.n_fine, n_out, p.tile_rows, p.n_wg,
+                       dim3(256), 0, s, w.fine_segs, K, p.n_fine, n_out, p.tile_rows, p.n_rng,
                        p.granule, w.range_row0, w.range_grp, w.range_row1);
     SSC_LAUNCH_CHECK("split_rebalance");
     rc = tiles_of(w.range_row1);
     if (rc != SSC_OK) return rc;
   }
+  const bool paired = p.n_rng != p.n_wg;
+  if (paired) {
+    hipLaunchKernelGGL(range_assign_kernel, dim3(1), dim3(kMaxRanges), 0, s, w.range_grp, p.n_rng,
+                       p.n_wg, w.range_g0, w.wg_grp);
+    SSC_LAUNCH_CHECK("range_assign");
+  }
   const int frag_bytes = elem_bytes == 2 ? Io<_Float16>::kFragBytes : Io<float>::kFragBytes;
   hipLaunchKernelGGL(sched_fill_kernel, dim3((unsigned)ceil_div(p.n_tiles * K * 16, 256)),
                      dim3(256), 0, s, w.flag, pairs, w.sorted, pair_stride, plane_g,
                      w.share_first, w.share_cnt, w.kofs, w.tile_nmb, w.tile_loc, w.tile_rng,
-                     w.range_grp, p.n_wg, w.tile_grp, K, w.n_tiles_dev, w.tile_row0,
+                     w.range_grp, p.n_wg, paired ? w.range_g0 : (const int32_t *)nullptr,
+                     w.wg_grp, w.tile_grp, K, w.n_tiles_dev, w.tile_row0,
                      w.tile_slot0, p.T,
                      p.gather ? (uint32_t)c_in * (uint32_t)elem_bytes : 1u,
                      p.gather ? kGatherPad : 0xFFFFFFFFu, (p.acc_cols + 4) * 4,

@@ -188,7 +188,7 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
                     const void *__restrict__ packed, unsigned packed_bytes,
                     const int32_t *__restrict__ sched_in, const int32_t *__restrict__ sched_out,
                     const int32_t *__restrict__ grp_meta, unsigned sched_bytes, unsigned meta_bytes,
-                    const int32_t *__restrict__ tile_grp, const int32_t *__restrict__ wg_tile,
+                    const int32_t *__restrict__ wg_grp,
                     int nch, int ncb, IO *__restrict__ out, int cout, int T, int cols_per_xcd,
                     int col_base, int xcol, ConvEpilogue epi) {
   constexpr bool TAIL = FORM == 1, FIVE = FORM == 2;
@@ -252,8 +252,7 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
       }
     }
   }
-  const int t_begin = wg_tile[chunk], t_end = wg_tile[chunk + 1];
-  const int g_begin = tile_grp[t_begin], g_end = tile_grp[t_end];
+  const int g_begin = wg_grp[chunk], g_end = wg_grp[chunk + 1];  // this workgroup's groups
   const int nstages = (g_end - g_begin) * nch;  // stages of this workgroup
   const int col0 = col_base + cblk * kCN;
   static_assert(FORM == 0 || (NCW == 4 && !kHalf), "the other forms are built for float");
@@ -1113,6 +1112,7 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
 
 struct ConvPlan {
   int ncb, nch, T, ncw, n_wg, n_colblk;  // T: rows of the accumulator window
+  int n_rng;  // ranges of output rows: one for every workgroup of a column block, or two
   int tile_rows;                         // largest tile height
   int gather;  // conv_fwd_kernel's GATHER
   int ns;      // conv_fwd_kernel's NS: MFMA steps per chunk
@@ -1143,7 +1143,7 @@ struct ConvPlan {
 struct ConvWs {
   void *packed;
   // plan
-  int32_t *tile_grp, *wg_tile;
+  int32_t *tile_grp, *wg_tile, *wg_grp;
   int32_t *sched_in, *sched_out, *grp_meta;
   // scratch
   int32_t *flag;
@@ -1151,7 +1151,7 @@ struct ConvWs {
   int32_t *sorted;
   uint32_t *bits;
   int32_t *prefix;
-  int32_t *tile_loc, *tile_nmb, *kofs, *tile_rng, *range_grp, *range_row1;
+  int32_t *tile_loc, *tile_nmb, *kofs, *tile_rng, *range_grp, *range_row1, *range_g0;
   int32_t *fine_segs, *range_row0, *tile_row0, *n_tiles_dev;
   int32_t *spill_end, *tile_slot0, *spill, *share_first, *share_cnt;
 };
@@ -1195,8 +1195,8 @@ inline int launch_conv(const ConvPlan &p, const ConvWs &w, const IO *features, i
                            : ((p.n_wg & 7) != 0 && p.n_wg * p.n_colblk >= 16) ? (big ? -2 : -1) : 0;
   hipLaunchKernelGGL((conv_fwd_kernel<IO, GATHER, NCW, NS, EPI, FORM>), grid, dim3((NCW + 4) * 64), p.lds_bytes, s, features, c_in,
                      feat_bytes, w.packed, (unsigned)packed_bytes, w.sched_in, w.sched_out,
-                     w.grp_meta, (unsigned)sched_bytes, (unsigned)(p.grp_cap * 32), w.tile_grp,
-                     w.wg_tile, p.nch, p.ncb, out, c_out, p.T, cols_per_xcd, col_base, xcol, epi);
+                     w.grp_meta, (unsigned)sched_bytes, (unsigned)(p.grp_cap * 32), w.wg_grp,
+                     p.nch, p.ncb, out, c_out, p.T, cols_per_xcd, col_base, xcol, epi);
   SSC_LAUNCH_CHECK("conv_fwd");
   return SSC_OK;
 }

@@ -474,20 +474,22 @@ def test_conv_five_group_form(shape, oracle, device):
 @pytest.mark.parametrize("case", [(2500, 16, 3, 1, 1, 64, 128), (900, 12, 3, 2, 1, 128, 256),
                                   (400, 10, 5, 1, 2, 200, 200), (5, 8, 3, 1, 1, 5, 7),
                                   (2500, 16, 3, 1, 1, 64, 72), (3000, 16, 3, 1, 1, 3, 152)])
-def test_conv_second_work_split(case, oracle, device):
+@pytest.mark.parametrize("flags", [32, 128, 32 | 128])
+def test_conv_second_work_split(case, flags, oracle, device):
     """The work split made twice (plans of long kernels; forced here by ssc_conv_tuning flag
-    32): the second split moves the boundaries between the workgroups' ranges of output
-    rows, nothing else.  Against the oracle, and equal to the plan of one split up to the
+    32) and two ranges of output rows to a workgroup, paired by the row-block groups they
+    came to (plans of middle size; forced by flag 128): either moves the boundaries between
+    the workgroups' ranges of output rows, nothing else.  Against the oracle, and equal to the plan of one split up to the
     order of the float sums: an output row's products are added offset by offset within a
     row-block group and chunk by chunk over the groups, and which offsets share a group
     moves with the tiles.  With one channel chunk and no lone last group that order is
     fixed: bit-equal."""
     from ss_conv import _ext
-    print("case", case, flush=True)
+    print("case", case, "flags", flags, flush=True)
     n, grid, k, s, p, cin, cout = case
     a, _ = _conv_case(oracle, device, n, grid, k, s, p, cin, cout, seed=41)
     try:
-        assert _ext._lib.ssc_conv_tuning(1 | 32) == 0
+        assert _ext._lib.ssc_conv_tuning(1 | flags) == 0
         b, _ = _conv_case(oracle, device, n, grid, k, s, p, cin, cout, seed=41)
         c, _ = _conv_case(oracle, device, n, grid, k, s, p, cin, cout, seed=41)
     finally:
