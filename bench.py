@@ -32,7 +32,7 @@ CLOCK_WARMUP_MS = 100
 # launches) for every workload this script offers, from rocprofv3 --pmc FETCH_SIZE /
 # WRITE_SIZE runs scaled by a copy kernel of known size (the summaries
 # profiles/conv_fwd_<workload>_hbm_traffic.md give commands and counter values).
-MEASURED_TRAFFIC_BYTES = {"cfg1": 3042208, "cfg2": 345618323, "cfg3": 218785754, "cfg5": 70539916921}
+MEASURED_TRAFFIC_BYTES = {"cfg1": 3416157, "cfg2": 344742917, "cfg3": 228204239, "cfg5": 70496920042}
 
 
 def parse_args():
