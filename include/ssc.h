@@ -325,7 +325,7 @@ int ssc_profile_conv(int32_t enable);
  *      follows the tiles); every plan by itself is bit-reproducible.
  *  32  the second work split for every plan, whatever its size (for tests).
  *  64  one range of output rows to a workgroup for every plan: plans of middle size (an
- *      estimated 80 row-block groups per workgroup or more, and no second split) otherwise
+ *      estimated 250 row-block groups per workgroup or more, and no second split) otherwise
  *      cut the rows into two ranges per workgroup and give a workgroup two of them by the
  *      groups they came to, many with few.  Changes the sizes; results as for 16.
  * 128  two ranges to a workgroup for every plan (for tests). */

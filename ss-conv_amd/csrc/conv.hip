@@ -819,7 +819,10 @@ static int device_cu_count() {
 static bool g_conv_tail = true;       // a launch of its own for a lone last column group
 static bool g_conv_five = true;       // the lone last group as a fifth one of the last block
 constexpr int64_t kRebalanceStages = 1500;
-constexpr int64_t kPairGroups = 80;  // estimated groups per workgroup from which ranges are paired
+// estimated groups per workgroup from which ranges are paired (the benchmark layer, 200 to
+// a workgroup: 216 -> 210 in the largest but no time gained for the launch it costs; the
+// third configuration, 55: one more range end each, 3499 -> 3691 groups, evens nothing out)
+constexpr int64_t kPairGroups = 250;
 static bool g_conv_pair = true, g_conv_pair_always = false;
 static int64_t g_conv_rebalance_stages = kRebalanceStages;
 static bool g_conv_rebalance = true;  // long kernels: a second work split from the first one's counts
@@ -886,9 +889,13 @@ static ConvPlan make_plan(int64_t n_in, int64_t n_out, int K, int c_in, int c_ou
   // multiple of 8: the kernel then deals its workgroups to the XCDs by its general rule)
   if (n_wg >= 8 && g_conv_round8) n_wg = n_wg / 8 * 8;
   // estimates from the pairs the layer is likely to have -- N_in K where the outputs
-  // outnumber the inputs (stride 1), a quarter of N_out K for submanifold and strided
-  // layers: stages and row-block groups per workgroup
-  const int64_t est_pairs = n_in > 0 && n_in < n_out ? n_in * K : n_out * K / 4;
+  // outnumber the inputs (stride 1), an eighth of that where the inputs outnumber the
+  // outputs (stride 2; also the input gradient of a stride-1 layer, which has N_out K), a
+  // quarter of N_out K for submanifold layers and where N_in is not known: stages and
+  // row-block groups per workgroup
+  const int64_t est_pairs = n_in <= 0 || n_in == n_out ? n_out * K / 4
+                            : n_in < n_out             ? n_in * K
+                                                       : n_in * K / 8;
   const int64_t est_groups = est_pairs / kStage / n_wg;
   const int64_t est_stages = est_groups * p.nch;
   // A second work split (split_rebalance_kernel) where the kernel runs long enough for four
@@ -899,8 +906,9 @@ static ConvPlan make_plan(int64_t n_in, int64_t n_out, int K, int c_in, int c_ou
   // small launch and one more range end per workgroup, whose last row blocks cannot be
   // filled from a next tile (K / 8 groups), against the 5-10 % by which single ranges
   // differ.  Not with the second split, which leaves less than that to even out.
+  // (N_in unknown: the plan is only being sized, for the larger of the two)
   const bool pair = g_conv_pair && n_wg >= 2 &&
-                    (g_conv_pair_always ||
+                    (g_conv_pair_always || n_in <= 0 ||
                      (!p.rebalance && est_groups >= kPairGroups && est_groups >= (int64_t)K / 2));
   plan_split(p, n_wg, pair ? 2 * n_wg : n_wg, n_out, K, pair_stride);
   p.lds_bytes = conv_lds_bytes(p.T, p.acc_cols);
