@@ -440,7 +440,7 @@ __global__ void __launch_bounds__(256)
     row_new[w] = (w == 0) ? 0 : (w == n_wg ? (int32_t)n_out : (int32_t)r);
 }
 
-// One block.  wg_tile[0..n_wg]: first tile of every workgroup; tile_row0[0..n_tiles]:
+// One block.  wg_tile[0..n_wg]: first tile of every range (n_wg of them); tile_row0[0..n_tiles]:
 // first row of every tile; n_tiles_dev[0]: number of tiles; spill_end[0..n_tiles]:
 // rows below spill_end[t] may be touched by the last row blocks of tile t-1 (the
 // first row of tile t itself when t starts a workgroup's range: no spill across
@@ -687,7 +687,7 @@ __global__ void __launch_bounds__(256)
                       const int32_t *__restrict__ tile_nmb, const int32_t *__restrict__ tile_loc,
                       const int32_t *__restrict__ tile_rng, const int32_t *__restrict__ range_grp,
                       int n_wg, const int32_t *__restrict__ range_g0_paired,
-                      int32_t *__restrict__ wg_grp, int32_t *__restrict__ tile_grp, int K,
+                      int32_t *__restrict__ wg_grp, int K,
                       const int32_t *__restrict__ n_tiles_dev,
                       const int32_t *__restrict__ tile_row0,
                       const int32_t *__restrict__ tile_slot0, int T, uint32_t in_scale,
@@ -734,10 +734,6 @@ __global__ void __launch_bounds__(256)
   const int64_t g0 = rg0 + tile_loc[t];
   const int64_t g1 = (t + 1 < n_tiles && tile_rng[t + 1] == rng) ? rg0 + tile_loc[t + 1]
                                                                 : rg0 + range_grp[rng];
-  if (k == 0 && lane == 0) {  // the tiles' first groups, for the convolution kernel
-    tile_grp[t] = (int32_t)g0;
-    if (t + 1 == n_tiles) tile_grp[n_tiles] = (int32_t)g1;
-  }
   if (k == 0) {
     for (int64_t g = g0 + lane; g < g1; g += 16) {
       const int rows = tile_row0[t + 1] - tile_row0[t];
@@ -923,14 +919,12 @@ static size_t conv_packed_bytes(const ConvPlan &p, int K) {
 
 static size_t conv_plan_walk(void *base, const ConvPlan &p, ConvWs *w) {
   Carver c(base);
-  int32_t *tile_grp = c.take<int32_t>((size_t)p.n_tiles + 1);
   int32_t *wg_tile = c.take<int32_t>((size_t)p.n_rng + 1);
   int32_t *wg_grp = c.take<int32_t>((size_t)p.n_wg + 1);
   int32_t *sched_in = c.take<int32_t>((size_t)p.grp_cap * 64);
   int32_t *sched_out = c.take<int32_t>((size_t)p.grp_cap * 64);
   int32_t *grp_meta = c.take<int32_t>((size_t)p.grp_cap * 8);
   if (w) {
-    w->tile_grp = tile_grp;
     w->wg_tile = wg_tile;
     w->wg_grp = wg_grp;
     w->sched_in = sched_in;
@@ -1234,7 +1228,7 @@ static int conv_plan_build(const ConvPlan &p, const ConvWs &w, const int32_t *pa
                      dim3(256), 0, s, w.flag, pairs, w.sorted, pair_stride, plane_g,
                      w.share_first, w.share_cnt, w.kofs, w.tile_nmb, w.tile_loc, w.tile_rng,
                      w.range_grp, p.n_wg, paired ? w.range_g0 : (const int32_t *)nullptr,
-                     w.wg_grp, w.tile_grp, K, w.n_tiles_dev, w.tile_row0,
+                     w.wg_grp, K, w.n_tiles_dev, w.tile_row0,
                      w.tile_slot0, p.T,
                      p.gather ? (uint32_t)c_in * (uint32_t)elem_bytes : 1u,
                      p.gather ? kGatherPad : 0xFFFFFFFFu, (p.acc_cols + 4) * 4,

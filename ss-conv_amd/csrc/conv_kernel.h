@@ -1143,7 +1143,7 @@ struct ConvPlan {
 struct ConvWs {
   void *packed;
   // plan
-  int32_t *tile_grp, *wg_tile, *wg_grp;
+  int32_t *wg_tile, *wg_grp;  // first tile of every range; first group of every workgroup
   int32_t *sched_in, *sched_out, *grp_meta;
   // scratch
   int32_t *flag;
