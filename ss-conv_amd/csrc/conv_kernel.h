@@ -1,8 +1,9 @@
 // The convolution kernel (conv_fwd_kernel), what a launch of it needs to know of a plan,
-// and the launch itself.  Four translation units instantiate it: conv.hip the plain form
+// and the launch itself.  Six translation units instantiate it: conv.hip the plain form
 // (float and half rows), conv_epi.hip the one with the epilogue, conv_tail.hip and
-// conv_tail_epi.hip the one-column-group form without and with it -- compiled side by
-// side, the quarters of the instances take a third of the time.
+// conv_tail_epi.hip the one-column-group form without and with it, conv_five.hip and
+// conv_five_epi.hip the five-group form -- compiled side by side, the parts of the
+// instances take a third of the time.
 #pragma once
 #include "ssc_common.h"
 
