@@ -1011,13 +1011,10 @@ static int launch_all(const ConvPlan &p, const ConvWs &w, const IO *features, in
   constexpr bool kFloat = sizeof(IO) == 4;
   const bool with_epi = kFloat && epi.mode != nullptr;
   if (p.five) {
-    // the epilogue is not built for the fifth group: with it the lone group takes a launch
-    // of its own, as a block of which one consumer wave in four has columns
     if constexpr (kFloat) {
-      const int n_launch = with_epi ? p.n_launch + 1 : p.n_launch;
-      for (int l = 0; l < n_launch; ++l) {
+      for (int l = 0; l < p.n_launch; ++l) {
         const int col_base = l * 16 * p.ncw;
-        const int xcol = !with_epi && l == p.n_launch - 1 ? (p.ncb - 1) * 16 : -1;
+        const int xcol = l == p.n_launch - 1 ? (p.ncb - 1) * 16 : -1;
         const int rc =
             with_epi ? launch_conv_f32<GATHER, NS, true, 2>(p, w, features, n_in, c_in, K, out,
                                                             c_out, col_base, xcol, epi, s)

@@ -269,49 +269,67 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
   // Epilogue constants of this thread, loaded once: when a tile is written out a thread
   // keeps its 4 columns (c_t) and walks down the rows; lane l of a row's 16 lanes also
   // owns gate l of the workgroup's column block.
-  //   z = x * e_ca + e_cb (e_cb includes the bias in front of a scalar activation);
-  //   e_mg = mode | LDS column of the gate << 4;  e_dest = output column
-  //   gate l: activated value = act_gate(x * e_gca + e_gcb), LDS column e_gcl (-1: none)
-  float e_ca[4], e_cb[4], e_gca = 0.f, e_gcb = 0.f;
-  int e_mg[4], e_dest[4], e_gcl = -1;
-  bool e_any = false, e_vec = false;
-  if constexpr (EPI) {
-    const int c_t = (tid % (kCN / 4)) * 4, col = col0 + c_t;
-    const bool col_ok = col < cout;
+  //   z = x * ca + cb (cb includes the bias in front of a scalar activation);
+  //   mg = mode | LDS column of the gate << 4;  dest = output column
+  //   gate l: activated value = act_gate(x * gca + gcb), LDS column gcl (-1: none)
+  // LDS columns count from the first column of the block (a fifth group's from its own).
+  // (EpiConsts: ca, cb, mg, dest per column of the thread; gca, gcb, gcl of its gate)
+  struct EpiConsts {
+    float ca[4], cb[4], gca, gcb;
+    int mg[4], dest[4], gcl;
+    bool any, vec;
+  };
+  // bcol0: first output column of the block of 64 the columns belong to; ncols: how many of
+  // the block's columns the workgroup has (64, or the 16 of a fifth group)
+  auto epi_consts = [&](int bcol0, int ncols) -> EpiConsts {
+    EpiConsts e;
+    e.gca = 0.f;
+    e.gcb = 0.f;
+    e.gcl = -1;
+    const int c_t = (tid % (kCN / 4)) * 4, col = bcol0 + c_t;
+    const bool col_ok = col < cout && c_t < ncols;
     static_assert(!EPI || kCN == 64, "the epilogue's gate runs are per block of 64 columns");
-    const int eblk = col0 / kCN;  // block of 64 columns the workgroup's columns start
+    const int eblk = bcol0 / kCN;  // block of 64 columns the workgroup's columns start
     const int gfirst = epi.gate_run[2 * eblk], gcount = min(epi.gate_run[2 * eblk + 1], 16);
-    const bool run_ok = gfirst >= col0 && gfirst + gcount <= min(col0 + kCN, cout);
+    const bool run_ok = gfirst >= bcol0 && gfirst + gcount <= min(bcol0 + ncols, cout);
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int c = col_ok ? col + i : 0;
       int mode = col_ok ? epi.mode[c] : 3;
-      e_dest[i] = epi.dest[c];
+      e.dest[i] = epi.dest[c];
       const int g = epi.gate[c];
       // tables that point outside the output row or outside the block's run of gates
       // switch the column off
-      if (e_dest[i] < 0 || e_dest[i] >= epi.c_dest || mode < 0 || mode > 2 ||
+      if (e.dest[i] < 0 || e.dest[i] >= epi.c_dest || mode < 0 || mode > 2 ||
           (mode == 2 && (!run_ok || g < gfirst || g >= gfirst + gcount)))
         mode = 3;
-      e_mg[i] = mode | ((mode == 2 ? g - col0 : c_t + i) << 4);
-      e_ca[i] = epi.scale[c];
-      e_cb[i] = epi.add[c] - epi.shift[c] * e_ca[i] + (mode == 1 ? epi.pre[c] : 0.f);
+      e.mg[i] = mode | ((mode == 2 ? g - bcol0 : col_ok ? c_t + i : 0) << 4);
+      e.ca[i] = epi.scale[c];
+      e.cb[i] = epi.add[c] - epi.shift[c] * e.ca[i] + (mode == 1 ? epi.pre[c] : 0.f);
     }
-    e_any = (e_mg[0] & 15) != 3 || (e_mg[1] & 15) != 3 || (e_mg[2] & 15) != 3 || (e_mg[3] & 15) != 3;
-    e_vec = (e_mg[0] & 15) != 3 && (e_mg[1] & 15) != 3 && (e_mg[2] & 15) != 3 &&
-            (e_mg[3] & 15) != 3 && e_dest[1] == e_dest[0] + 1 && e_dest[2] == e_dest[0] + 2 &&
-            e_dest[3] == e_dest[0] + 3 && ((e_dest[0] | epi.c_dest) & 3) == 0;
+    e.any = (e.mg[0] & 15) != 3 || (e.mg[1] & 15) != 3 || (e.mg[2] & 15) != 3 || (e.mg[3] & 15) != 3;
+    e.vec = (e.mg[0] & 15) != 3 && (e.mg[1] & 15) != 3 && (e.mg[2] & 15) != 3 &&
+            (e.mg[3] & 15) != 3 && e.dest[1] == e.dest[0] + 1 && e.dest[2] == e.dest[0] + 2 &&
+            e.dest[3] == e.dest[0] + 3 && ((e.dest[0] | epi.c_dest) & 3) == 0;
     const int gi = (tid % (kCN / 4));
     if (run_ok && gi < gcount) {
       const int g = gfirst + gi;
-      e_gcl = g - col0;
-      e_gca = epi.scale[g];
-      e_gcb = epi.add[g] - epi.shift[g] * e_gca + epi.pre[g];
+      e.gcl = g - bcol0;
+      e.gca = epi.scale[g];
+      e.gcb = epi.add[g] - epi.shift[g] * e.gca + epi.pre[g];
+    }
+    return e;
+  };
+  EpiConsts ec = {}, ecx = {};  // of the workgroup's block of 64 columns; of a fifth group
+  if constexpr (EPI) {
+    ec = epi_consts(col0, kCN);
+    if constexpr (FIVE) {
+      if (xcol >= 0) ecx = epi_consts(xcol, 16);
     }
   }
   const int e_c_dest = epi.c_dest, e_act_s = epi.act_s, e_act_g = epi.act_g;
   auto flush_tile = [&](int row0, int rows, int slot0) __attribute__((always_inline)) {
-    if constexpr (FIVE) {
+    if constexpr (FIVE && !EPI) {
       // the fifth column group (accumulator columns kCN .. kCN + 15): four threads a row
       if (xcol >= 0) {
         const float4v z = {0.f, 0.f, 0.f, 0.f};
@@ -359,22 +377,27 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
       // FAST: scalar activation none or relu, gate activation none or sigmoid -- a few instructions
       // per element and no branch (a taken branch costs a wave more than the arithmetic of
       // a whole row); the other activations go through act_fn.
-      auto rows_out = [&](auto fast_tag) __attribute__((always_inline)) {
+      // (e: the constants; XG: the pass over a fifth group, whose 16 columns begin at
+      // accumulator column kCN and belong to the first four of a row's 16 threads)
+      auto rows_out = [&](auto fast_tag, auto x_tag, const EpiConsts &e) __attribute__((always_inline)) {
         constexpr bool FAST = decltype(fast_tag)::value;
+        constexpr bool XG = decltype(x_tag)::value;
         constexpr int U = 2;
         constexpr int RS = NT / (kCN / 4);
         const int r_t = tid / (kCN / 4), c_t = (tid % (kCN / 4)) * 4;
+        const bool own = !XG || c_t < 16;  // the thread has columns
+        constexpr int kCol0 = XG ? kCN : 0;
         const float4v z = {0.f, 0.f, 0.f, 0.f};
         // FAST: max(t, lo) is the scalar activation where there is one, t elsewhere
         float lo[4];
         bool gated[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          lo[i] = ((e_mg[i] & 15) == 1 && e_act_s == SSC_ACT_RELU) ? 0.f : -INFINITY;
-          gated[i] = (e_mg[i] & 15) == 2;
+          lo[i] = ((e.mg[i] & 15) == 1 && e_act_s == SSC_ACT_RELU) ? 0.f : -INFINITY;
+          gated[i] = (e.mg[i] & 15) == 2;
         }
         auto gate_act = [&](float x) -> float {
-          const float u = x * e_gca + e_gcb;
+          const float u = x * e.gca + e.gcb;
           if constexpr (FAST)
             return e_act_g == SSC_ACT_SIGMOID ? __builtin_amdgcn_rcpf(1.f + __expf(-u)) : u;
           else
@@ -387,23 +410,23 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
           int sl0 = slot0 + r, sl1 = slot0 + r + RS;
           if (sl0 >= T) sl0 -= T;
           if (sl1 >= T) sl1 -= T;
-          float *a0 = acc + sl0 * kAS, *a1 = acc + sl1 * kAS;
-          if (e_gcl >= 0) {
-            const float x0 = a0[e_gcl], x1 = two ? a1[e_gcl] : 0.f;
-            a0[e_gcl] = gate_act(x0);
-            if (two) a1[e_gcl] = gate_act(x1);
+          float *a0 = acc + sl0 * kAS + kCol0, *a1 = acc + sl1 * kAS + kCol0;
+          if (e.gcl >= 0) {
+            const float x0 = a0[e.gcl], x1 = two ? a1[e.gcl] : 0.f;
+            a0[e.gcl] = gate_act(x0);
+            if (two) a1[e.gcl] = gate_act(x1);
           }
           __builtin_amdgcn_sched_barrier(0);
-          float4v v0 = *reinterpret_cast<float4v *>(a0 + c_t), v1 = z, g1 = z;
-          float4v g0 = {a0[e_mg[0] >> 4], a0[e_mg[1] >> 4], a0[e_mg[2] >> 4], a0[e_mg[3] >> 4]};
+          float4v v0 = own ? *reinterpret_cast<float4v *>(a0 + c_t) : z, v1 = z, g1 = z;
+          float4v g0 = {a0[e.mg[0] >> 4], a0[e.mg[1] >> 4], a0[e.mg[2] >> 4], a0[e.mg[3] >> 4]};
           if (two) {
-            v1 = *reinterpret_cast<float4v *>(a1 + c_t);
-            g1 = float4v{a1[e_mg[0] >> 4], a1[e_mg[1] >> 4], a1[e_mg[2] >> 4], a1[e_mg[3] >> 4]};
+            if (own) v1 = *reinterpret_cast<float4v *>(a1 + c_t);
+            g1 = float4v{a1[e.mg[0] >> 4], a1[e.mg[1] >> 4], a1[e.mg[2] >> 4], a1[e.mg[3] >> 4]};
           }
           __builtin_amdgcn_sched_barrier(0);  // the clears stay behind every read above
-          *reinterpret_cast<float4v *>(a0 + c_t) = z;
-          if (two) *reinterpret_cast<float4v *>(a1 + c_t) = z;
-          if (e_any) {
+          if (own) *reinterpret_cast<float4v *>(a0 + c_t) = z;
+          if (two && own) *reinterpret_cast<float4v *>(a1 + c_t) = z;
+          if (e.any) {
 #pragma unroll
             for (int u = 0; u < U; ++u) {
               if (u == 1 && !two) break;
@@ -411,33 +434,42 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
               float4v y;
 #pragma unroll
               for (int i = 0; i < 4; ++i) {
-                const float t = v[i] * e_ca[i] + e_cb[i];
+                const float t = v[i] * e.ca[i] + e.cb[i];
                 if constexpr (FAST) {
                   y[i] = fmaxf(t, lo[i]) * (gated[i] ? gv[i] : 1.f);
                 } else {  // every form, then select: no divergent branches
                   const float ts = act_fn(e_act_s, t);
-                  const int m = e_mg[i] & 15;
+                  const int m = e.mg[i] & 15;
                   y[i] = m == 1 ? ts : m == 2 ? t * gv[i] : t;
                 }
               }
               float *p = gp + u * gstep;
-              if (e_vec) {
-                __builtin_nontemporal_store(y, reinterpret_cast<float4v *>(p + e_dest[0]));
+              if (e.vec) {
+                __builtin_nontemporal_store(y, reinterpret_cast<float4v *>(p + e.dest[0]));
               } else {
 #pragma unroll
                 for (int i = 0; i < 4; ++i)
-                  if ((e_mg[i] & 15) != 3) __builtin_nontemporal_store(y[i], p + e_dest[i]);
+                  if ((e.mg[i] & 15) != 3) __builtin_nontemporal_store(y[i], p + e.dest[i]);
               }
             }
           }
           gp += U * gstep;
         }
       };
-      if ((e_act_s == SSC_ACT_NONE || e_act_s == SSC_ACT_RELU) &&
-          (e_act_g == SSC_ACT_NONE || e_act_g == SSC_ACT_SIGMOID))
-        rows_out(std::true_type());
+      const bool fast = (e_act_s == SSC_ACT_NONE || e_act_s == SSC_ACT_RELU) &&
+                        (e_act_g == SSC_ACT_NONE || e_act_g == SSC_ACT_SIGMOID);
+      if constexpr (FIVE) {
+        if (xcol >= 0) {
+          if (fast)
+            rows_out(std::true_type(), std::true_type(), ecx);
+          else
+            rows_out(std::false_type(), std::true_type(), ecx);
+        }
+      }
+      if (fast)
+        rows_out(std::true_type(), std::false_type(), ec);
       else
-        rows_out(std::false_type());
+        rows_out(std::false_type(), std::false_type(), ec);
       return;
     }
     if ((cout & 3) == 0) {

@@ -1833,9 +1833,10 @@ EPILOGUE_CASES = [
     ([(16, 0)], 8, 3, 1, 1, False, None),                             # scalars only, no gates
     # 6.9 MB of packed filters in four column blocks: one column block per XCD
     ([(40, 0), (24, 1), (16, 2)], 256, 3, 1, 1, False, None),
-    # a plan of the five-group form (200 input channels, 74 columns in 5 groups): with the
-    # epilogue the lone group takes a launch of its own
+    # plans of the five-group form (200 and 256 input channels, 80 computed columns in 5
+    # groups): the epilogue of the fifth group
     ([(10, 0), (6, 1), (4, 2), (2, 3)], 200, 3, 1, 1, False, None),
+    ([(20, 0), (8, 1), (4, 2)], 256, 3, 2, 1, False, None),
 ]
 
 
@@ -1919,11 +1920,13 @@ def test_conv_epilogue_block_matches_oracle(case, oracle, device):
     assert xt.grad is not None and yt.features.shape[1] == c_act
 
 
-def test_conv_epilogue_block_other_layers(oracle, device):
+@pytest.mark.parametrize("fields", [([(6, 0), (5, 1), (3, 2)], 12), ([(20, 0), (8, 1), (4, 2)], 200)])
+def test_conv_epilogue_block_other_layers(fields, oracle, device):
     """The evaluation-mode block with tanh activations (the kernel's general form), with a
     batch norm or an activation only, and the cases that stay with the separate layers (a
     convolution with bias, half-precision rows, an empty input): always the result of the
-    three layers run one after the other."""
+    three layers run one after the other.  (The second set of fields: 200 input channels and
+    80 computed columns, a plan of the five-group form.)"""
     from ss_conv import _ext
     from ss_conv.activation import Activation
     from ss_conv.batchnorm import BatchNorm
@@ -1931,8 +1934,8 @@ def test_conv_epilogue_block_other_layers(oracle, device):
     from ss_conv.sp_ops.conv import SparseConvolution
     from ss_conv.sp_ops.tensor import SparseTensor
     rng = np.random.default_rng(5)
-    Rs = [(6, 0), (5, 1), (3, 2)]
-    batch, grid, n, cin = 2, 9, 400, 12
+    Rs, cin = fields
+    batch, grid, n = 2, 9, 400
     idx = torch.from_numpy(random_voxels(rng, batch, grid, n)).to(device)
     x = torch.from_numpy(rng.normal(size=(n, cin)).astype(np.float32)).to(device)
 
