@@ -284,10 +284,23 @@ def ops_table(torch, _ext, synth, dev, seed):
         ms_one, _ = timed(lambda: again(block), n=10)
         ms_sep, _ = timed(lambda: again(lambda t: fused.eval()(conv(t))), n=10)
         fused.train()
+        # the same block on half-precision rows and filters (the tables stay float32)
+        conv.half()
+        f2h = f2.half()
+
+        def again_half(fn):
+            t = SparseTensor(f2h, idx2, [cfg["grid"]] * 3, cfg["batch"])
+            t.indice_dict = y2.indice_dict
+            return fn(t)
+        block_half = ConvBatchNormActivation(conv, bn, act).eval()
+        again_half(block_half)
+        ms_half, _ = timed(lambda: again_half(block_half), n=10)
+        conv.float()
     rows.append("%-44s %8.3f ms   (cached rulebook and plan, %d rows, 64 -> %d -> %d ch)"
                 % ("conv+bn+act block, evaluation, one kernel", ms_one, y2.features.shape[0], c_in,
                    c_out))
     rows.append("%-44s %8.3f ms" % ("  the same as conv, then bn+act pass", ms_sep))
+    rows.append("%-44s %8.3f ms" % ("  the one kernel on half rows and filters", ms_half))
     xg = x.clone().requires_grad_(True)
     dy = torch.randn(n_rows, c_out, device=dev)
 

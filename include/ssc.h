@@ -254,6 +254,16 @@ int ssc_conv_run_epilogue_f32(const float *features /* [n_in,c_in] */, int64_t n
                               int32_t c_cols, const ssc_conv_epilogue *epilogue,
                               float *out /* [n_out,c_dest] */, int64_t n_out,
                               ssc_stream_t stream);
+/* The same on half-precision rows (features, packed filters of ssc_conv_pack_filters_f16,
+ * plan built with elem_bytes 2, out: half): the sums and the epilogue's arithmetic in fp32,
+ * the tables float32 as above, one rounding per stored element. */
+int ssc_conv_run_epilogue_f16(const void *features /* [n_in,c_in] half */, int64_t n_in,
+                              int32_t c_in, const void *packed, size_t packed_bytes,
+                              const void *plan, size_t plan_bytes, int64_t pair_stride,
+                              int32_t kernel_volume, int32_t c_cols,
+                              const ssc_conv_epilogue *epilogue,
+                              void *out /* [n_out,c_dest] half */, int64_t n_out,
+                              ssc_stream_t stream);
 
 /* ----------------------------------------------------------------------
  * Gradients of the sparse convolution -- replaces indice_conv_backward_fp32

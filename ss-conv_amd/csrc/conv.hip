@@ -1009,7 +1009,7 @@ static int launch_all(const ConvPlan &p, const ConvWs &w, const IO *features, in
                       int c_in, int K, IO *out, int c_out, const ConvEpilogue &epi,
                       hipStream_t s) {
   constexpr bool kFloat = sizeof(IO) == 4;
-  const bool with_epi = kFloat && epi.mode != nullptr;
+  const bool with_epi = epi.mode != nullptr;
   if (p.five) {
     if constexpr (kFloat) {
       for (int l = 0; l < p.n_launch; ++l) {
@@ -1036,8 +1036,10 @@ static int launch_all(const ConvPlan &p, const ConvWs &w, const IO *features, in
                     : launch_conv<float, GATHER, 4, NS, false, 0>(p, w, features, n_in, c_in, K,
                                                                   out, c_out, col_base, -1, epi, s);
     } else {
-      rc = launch_conv<IO, GATHER, 4, NS, false, 0>(p, w, features, n_in, c_in, K, out, c_out,
-                                                    col_base, -1, epi, s);
+      rc = with_epi ? launch_conv<IO, GATHER, 4, NS, true, 0>(p, w, features, n_in, c_in, K, out,
+                                                              c_out, col_base, -1, epi, s)
+                    : launch_conv<IO, GATHER, 4, NS, false, 0>(p, w, features, n_in, c_in, K, out,
+                                                               c_out, col_base, -1, epi, s);
     }
     if (rc != SSC_OK) return rc;
   }
@@ -1353,10 +1355,11 @@ static int conv_planned(const IO *features, int64_t n_in, int32_t c_in, const vo
 }
 
 // conv_planned with the epilogue applied to every finished tile.
-static int conv_planned_epilogue(const float *features, int64_t n_in, int32_t c_in,
+template <typename IO>
+static int conv_planned_epilogue(const IO *features, int64_t n_in, int32_t c_in,
                                  const void *packed, size_t packed_bytes, const void *plan,
                                  size_t plan_bytes, int64_t pair_stride, int32_t K, int32_t c_cols,
-                                 const ssc_conv_epilogue *e, float *out, int64_t n_out,
+                                 const ssc_conv_epilogue *e, IO *out, int64_t n_out,
                                  hipStream_t s) {
   int rc = conv_check_sizes(K, c_in, c_cols, n_in, n_out, pair_stride);
   if (rc != SSC_OK) return rc;
@@ -1373,7 +1376,7 @@ static int conv_planned_epilogue(const float *features, int64_t n_in, int32_t c_
   SSC_CHECK(e->shift && e->scale && e->add && e->pre_bias && e->mode && e->gate && e->dest &&
                 e->gate_run,
             SSC_EINVAL, "NULL table in the epilogue");
-  ConvPlan p = make_plan(n_in, n_out, K, c_in, c_cols, pair_stride, 4);
+  ConvPlan p = make_plan(n_in, n_out, K, c_in, c_cols, pair_stride, (int)sizeof(IO));
   SSC_CHECK(packed_bytes >= conv_packed_bytes(p, K), SSC_EWORKSPACE,
             "buffer of the packed filters too small");
   SSC_CHECK(plan_bytes >= conv_plan_walk(nullptr, p, nullptr), SSC_EWORKSPACE,
@@ -1383,7 +1386,7 @@ static int conv_planned_epilogue(const float *features, int64_t n_in, int32_t c_
   conv_plan_walk(const_cast<void *>(plan), p, &w);
   const ConvEpilogue epi = {e->shift, e->scale, e->add, e->pre_bias, e->mode, e->gate, e->dest,
                             e->gate_run, e->act_scalar, e->act_gate, e->c_dest};
-  return conv_run<float>(p, w, features, n_in, c_in, K, out, c_cols, s, epi);
+  return conv_run<IO>(p, w, features, n_in, c_in, K, out, c_cols, s, epi);
 }
 
 extern "C" {
@@ -1393,9 +1396,20 @@ int ssc_conv_run_epilogue_f32(const float *features, int64_t n_in, int32_t c_in,
                               size_t plan_bytes, int64_t pair_stride, int32_t kernel_volume,
                               int32_t c_cols, const ssc_conv_epilogue *epilogue, float *out,
                               int64_t n_out, ssc_stream_t stream) {
-  return conv_planned_epilogue(features, n_in, c_in, packed, packed_bytes, plan, plan_bytes,
-                               pair_stride, kernel_volume, c_cols, epilogue, out, n_out,
-                               (hipStream_t)stream);
+  return conv_planned_epilogue<float>(features, n_in, c_in, packed, packed_bytes, plan,
+                                      plan_bytes, pair_stride, kernel_volume, c_cols, epilogue,
+                                      out, n_out, (hipStream_t)stream);
+}
+
+int ssc_conv_run_epilogue_f16(const void *features, int64_t n_in, int32_t c_in,
+                              const void *packed, size_t packed_bytes, const void *plan,
+                              size_t plan_bytes, int64_t pair_stride, int32_t kernel_volume,
+                              int32_t c_cols, const ssc_conv_epilogue *epilogue, void *out,
+                              int64_t n_out, ssc_stream_t stream) {
+  return conv_planned_epilogue<_Float16>(static_cast<const _Float16 *>(features), n_in, c_in,
+                                         packed, packed_bytes, plan, plan_bytes, pair_stride,
+                                         kernel_volume, c_cols, epilogue,
+                                         static_cast<_Float16 *>(out), n_out, (hipStream_t)stream);
 }
 
 int ssc_conv_fwd_f32(const float *features, int64_t n_in, int32_t c_in, const float *filters,

@@ -403,7 +403,7 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
           else
             return act_fn(e_act_g, u);
         };
-        float *gp = reinterpret_cast<float *>(out) + (int64_t)(row0 + r_t) * e_c_dest;
+        IO *gp = out + (int64_t)(row0 + r_t) * e_c_dest;
         const int64_t gstep = (int64_t)RS * e_c_dest;
         for (int r = r_t; r < rows; r += U * RS) {
           const bool two = r + RS < rows;
@@ -443,13 +443,13 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
                   y[i] = m == 1 ? ts : m == 2 ? t * gv[i] : t;
                 }
               }
-              float *p = gp + u * gstep;
+              IO *p = gp + u * gstep;
               if (e.vec) {
-                __builtin_nontemporal_store(y, reinterpret_cast<float4v *>(p + e.dest[0]));
+                Io<IO>::store_stream(p + e.dest[0], y);
               } else {
 #pragma unroll
                 for (int i = 0; i < 4; ++i)
-                  if ((e.mg[i] & 15) != 3) __builtin_nontemporal_store(y[i], p + e.dest[i]);
+                  if ((e.mg[i] & 15) != 3) __builtin_nontemporal_store((IO)y[i], p + e.dest[i]);
               }
             }
           }

@@ -62,6 +62,8 @@ _SIGNATURES = {
                                         _i64, _vp]),
     "ssc_conv_run_epilogue_f32": (ctypes.c_int, [_vp, _i64, _i32, _vp, _sz, _vp, _sz, _i64, _i32,
                                                  _i32, _vp, _vp, _i64, _vp]),
+    "ssc_conv_run_epilogue_f16": (ctypes.c_int, [_vp, _i64, _i32, _vp, _sz, _vp, _sz, _i64, _i32,
+                                                 _i32, _vp, _vp, _i64, _vp]),
     "ssc_conv_fwd_f32": (ctypes.c_int, [_vp, _i64, _i32, _vp, _i64, _i64, _i64, _i32, _vp, _i64,
                                         _vp, _i32, _i32, _i32, _vp, _i64, _vp, _sz, _vp]),
     "ssc_conv_fwd_f16": (ctypes.c_int, [_vp, _i64, _i32, _vp, _i64, _i64, _i64, _i32, _vp, _i64,
@@ -457,14 +459,16 @@ def _run_planned(features, n_in, c_in, packed, plan, pair_stride, K, c_out, n_ou
                                            packed.numel(), plan.data_ptr(), plan.numel(),
                                            pair_stride, K, c_out, _ptr(out), n_out, s))
         return out
-    if features.dtype != torch.float32 or epilogue.c_cols != c_out:
-        raise RuntimeError("a convolution epilogue needs float32 rows and one table entry per "
-                           "filter column")
-    out = torch.empty((n_out, epilogue.c_dest), dtype=torch.float32, device=dev)
-    _check(_lib.ssc_conv_run_epilogue_f32(_ptr(features), n_in, c_in, packed.data_ptr(),
-                                          packed.numel(), plan.data_ptr(), plan.numel(),
-                                          pair_stride, K, c_out, ctypes.byref(epilogue.struct),
-                                          _ptr(out), n_out, s))
+    if features.dtype not in (torch.float32, torch.float16) or epilogue.c_cols != c_out:
+        raise RuntimeError("a convolution epilogue needs float32 or float16 rows and one table "
+                           "entry per filter column")
+    out = torch.empty((n_out, epilogue.c_dest), dtype=features.dtype, device=dev)
+    # (looked up by name at every call: tests count the calls through these attributes)
+    entry = (_lib.ssc_conv_run_epilogue_f32 if features.dtype == torch.float32
+             else _lib.ssc_conv_run_epilogue_f16)
+    _check(entry(_ptr(features), n_in, c_in, packed.data_ptr(), packed.numel(), plan.data_ptr(),
+                 plan.numel(), pair_stride, K, c_out, ctypes.byref(epilogue.struct), _ptr(out),
+                 n_out, s))
     return out
 
 

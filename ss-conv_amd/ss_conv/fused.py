@@ -116,24 +116,25 @@ class ConvBatchNormActivation(nn.Module):
         with torch.no_grad():
             wp = weight.new_zeros(tuple(weight.shape[:-1]) + (src.numel(),))
             wp[..., valid] = weight.detach()[..., src[valid]]
+            # the tables are float32 whatever the rows are
+            f32 = lambda t: None if t is None else t.detach().float().contiguous()  # noqa: E731
+            zeros = lambda *shape: torch.zeros(shape, dtype=torch.float32, device=dev)  # noqa: E731
             if bn is not None:
                 shift, scale, add, _ = _ext.bn_prepare(
-                    weight.new_zeros((1, c_conv)), bn.layout(dev), False, bn.eps, bn.momentum,
-                    None if bn.weight is None else bn.weight.detach().contiguous(),
-                    None if bn.bias is None else bn.bias.detach().contiguous(),
-                    bn.running_mean, bn.running_var)
+                    zeros(1, c_conv), bn.layout(dev), False, bn.eps, bn.momentum,
+                    f32(bn.weight), f32(bn.bias), f32(bn.running_mean), f32(bn.running_var))
             else:
-                shift, add = weight.new_zeros(c_conv), weight.new_zeros(c_conv)
-                scale = weight.new_ones(c_conv)
-            pre = weight.new_zeros(c_conv)
+                shift, add = zeros(c_conv), zeros(c_conv)
+                scale = torch.ones(c_conv, dtype=torch.float32, device=dev)
+            pre = zeros(c_conv)
             codes = (_ext.ACT_NONE, _ext.ACT_NONE)
             c_dest = c_conv
             if self._has_act():
                 codes, c_dest = act._codes, act._c_out
                 if sb is not None:
-                    pre[:act.multiplicities[0]] = sb.detach()
+                    pre[:act.multiplicities[0]] = sb.detach().float()
                 if gb is not None:
-                    pre[act._c_out:act._c_out + act._n_gates] = gb.detach()
+                    pre[act._c_out:act._c_out + act._n_gates] = gb.detach().float()
             pick = src.clamp(min=0)
             epi = _ext.ConvEpilogue(shift[pick].contiguous(), scale[pick].contiguous(),
                                     add[pick].contiguous(), pre[pick].contiguous(),

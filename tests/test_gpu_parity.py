@@ -1923,8 +1923,8 @@ def test_conv_epilogue_block_matches_oracle(case, oracle, device):
 @pytest.mark.parametrize("fields", [([(6, 0), (5, 1), (3, 2)], 12), ([(20, 0), (8, 1), (4, 2)], 200)])
 def test_conv_epilogue_block_other_layers(fields, oracle, device):
     """The evaluation-mode block with tanh activations (the kernel's general form), with a
-    batch norm or an activation only, and the cases that stay with the separate layers (a
-    convolution with bias, half-precision rows, an empty input): always the result of the
+    batch norm or an activation only, on half-precision rows, and the cases that stay with
+    the separate layers (a convolution with bias, an empty input): always the result of the
     three layers run one after the other.  (The second set of fields: 200 input channels and
     80 computed columns, a plan of the five-group form.)"""
     from ss_conv import _ext
@@ -1944,10 +1944,15 @@ def test_conv_epilogue_block_other_layers(fields, oracle, device):
 
     calls = {"epi": 0}
     real = _ext._lib.ssc_conv_run_epilogue_f32
+    real_half = _ext._lib.ssc_conv_run_epilogue_f16
 
     def counted(*a):
         calls["epi"] += 1
         return real(*a)
+
+    def counted_half(*a):
+        calls["epi"] += 1
+        return real_half(*a)
 
     def check(block, expect_kernel, make=tensor, tol=1e-6):
         before = calls["epi"]
@@ -1964,6 +1969,7 @@ def test_conv_epilogue_block_other_layers(fields, oracle, device):
             assert rel_l2(got.float().cpu().numpy(), y.features.float().cpu().numpy()) < tol
 
     _ext._lib.ssc_conv_run_epilogue_f32 = counted
+    _ext._lib.ssc_conv_run_epilogue_f16 = counted_half
     try:
         bn, act, Rs_bn = _bnact_modules(Rs, (torch.tanh, torch.tanh), device, rng)
         c_conv = bn.num_channels
@@ -1992,18 +1998,29 @@ def test_conv_epilogue_block_other_layers(fields, oracle, device):
                                   bias=False).to(device)
         check(ConvBatchNormActivation(conv2, BatchNorm(Rs).to(device),
                                       Activation(Rs, (torch.relu, None)).to(device)).eval(), True)
-        # not for the kernel: bias, half rows, no rows, nothing to apply
-        biased = SparseConvolution(3, cin, c_conv, 3, 1, 1, bias=True).to(device)
-        check(ConvBatchNormActivation(biased, bn, act).eval(), False)
+        # half-precision rows and filters (ssc_conv_run_epilogue_f16; the tables stay float32)
         check(ConvBatchNormActivation(conv.half(), None, Activation(Rs, (torch.relu, torch.sigmoid),
                                                                     bias=False).to(device)).eval(),
-              False, make=lambda: tensor(x.half()), tol=2e-3)
+              True, make=lambda: tensor(x.half()), tol=2e-3)
+        # (with the batch norm, whose own forward does not take half rows: against the
+        # float32 block)
+        before = calls["epi"]
+        with torch.no_grad():
+            got = ConvBatchNormActivation(conv, bn, act).eval()(tensor(x.half())).features
         conv.float()
+        with torch.no_grad():
+            want = ConvBatchNormActivation(conv, bn, act).eval()(tensor()).features
+        assert calls["epi"] - before == 2 and got.dtype == torch.float16
+        assert rel_l2(got.float().cpu().numpy(), want.cpu().numpy()) < 4e-3
+        # not for the kernel: bias, no rows, nothing to apply
+        biased = SparseConvolution(3, cin, c_conv, 3, 1, 1, bias=True).to(device)
+        check(ConvBatchNormActivation(biased, bn, act).eval(), False)
         check(ConvBatchNormActivation(conv, bn, act).eval(), False,
               make=lambda: tensor(x[:0], idx[:0]))
         check(ConvBatchNormActivation(conv, None, None).eval(), False)
     finally:
         _ext._lib.ssc_conv_run_epilogue_f32 = real
+        _ext._lib.ssc_conv_run_epilogue_f16 = real_half
 
 
 def test_voxel2point_one_call_equals_the_separate_steps(oracle, device):
