@@ -1014,12 +1014,19 @@ static int launch_all(const ConvPlan &p, const ConvWs &w, const IO *features, in
     if constexpr (kFloat) {
       for (int l = 0; l < p.n_launch; ++l) {
         const int col_base = l * 16 * p.ncw;
-        const int xcol = l == p.n_launch - 1 ? (p.ncb - 1) * 16 : -1;
-        const int rc =
-            with_epi ? launch_conv_f32<GATHER, NS, true, 2>(p, w, features, n_in, c_in, K, out,
-                                                            c_out, col_base, xcol, epi, s)
-                     : launch_conv_f32<GATHER, NS, false, 2>(p, w, features, n_in, c_in, K, out,
-                                                             c_out, col_base, xcol, epi, s);
+        int rc;
+        if (l == p.n_launch - 1) {  // with the lone group as a fifth one
+          const int xcol = (p.ncb - 1) * 16;
+          rc = with_epi ? launch_conv_f32<GATHER, NS, true, 2>(p, w, features, n_in, c_in, K, out,
+                                                               c_out, col_base, xcol, epi, s)
+                        : launch_conv_f32<GATHER, NS, false, 2>(p, w, features, n_in, c_in, K, out,
+                                                                c_out, col_base, xcol, epi, s);
+        } else {  // the plain kernel on the plan's wider accumulator rows
+          rc = with_epi ? launch_conv_f32<GATHER, NS, true, 3>(p, w, features, n_in, c_in, K, out,
+                                                               c_out, col_base, -1, epi, s)
+                        : launch_conv_f32<GATHER, NS, false, 3>(p, w, features, n_in, c_in, K, out,
+                                                                c_out, col_base, -1, epi, s);
+        }
         if (rc != SSC_OK) return rc;
       }
       return SSC_OK;

@@ -1,8 +1,9 @@
 // The convolution kernel (conv_fwd_kernel), what a launch of it needs to know of a plan,
-// and the launch itself.  Six translation units instantiate it: conv.hip the plain form
+// and the launch itself.  Eight translation units instantiate it: conv.hip the plain form
 // (float and half rows), conv_epi.hip the one with the epilogue, conv_tail.hip and
 // conv_tail_epi.hip the one-column-group form without and with it, conv_five.hip and
-// conv_five_epi.hip the five-group form -- compiled side by side, the parts of the
+// conv_five_epi.hip the five-group form, conv_wide.hip and conv_wide_epi.hip the plain
+// kernel over plans of the five-group form -- compiled side by side, the parts of the
 // instances take a third of the time.
 #pragma once
 #include "ssc_common.h"
@@ -181,7 +182,8 @@ struct ConvEpilogue {
 };
 
 // FORM: 0 the kernel as described above; 1 the one-column-group form; 2 the five-group form
-// (see the consumers).
+// (see the consumers); 3 the plain kernel on a plan of the five-group form, whose accumulator
+// rows are 16 columns wider (the launches of such a plan that have no fifth group).
 template <typename IO, int GATHER, int NCW, int NS, bool EPI, int FORM>
 __global__ void __launch_bounds__((NCW + 4) * 64)
     __attribute__((amdgpu_waves_per_eu((NCW + 4) / 4, (NCW + 4) / 4)))
@@ -192,7 +194,7 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
                     const int32_t *__restrict__ wg_grp,
                     int nch, int ncb, IO *__restrict__ out, int cout, int T, int cols_per_xcd,
                     int col_base, int xcol, ConvEpilogue epi) {
-  constexpr bool TAIL = FORM == 1, FIVE = FORM == 2;
+  constexpr bool TAIL = FORM == 1, FIVE = FORM == 2, WIDE = FORM == 3;
   constexpr int kCN = 16 * NCW;   // output columns per workgroup
   constexpr int kEB = Io<IO>::kBytes;
   constexpr bool kHalf = kEB == 2;
@@ -204,7 +206,7 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
   constexpr int kQFull = NS / 4, kQRem = NS % 4;  // whole quarters, steps of the partial one
   typedef typename Io<IO>::Raw Raw;
   // accumulator row stride in floats (the five-group form: 16 more columns)
-  constexpr int kAS = kCN + (FIVE ? 16 : 0) + 4;
+  constexpr int kAS = kCN + (FIVE || WIDE ? 16 : 0) + 4;
   constexpr int NT = (NCW + 4) * 64;
   constexpr int NP = 256;  // producer threads
   constexpr int NE = kStage * 16 / NP;
@@ -323,9 +325,7 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
   EpiConsts ec = {}, ecx = {};  // of the workgroup's block of 64 columns; of a fifth group
   if constexpr (EPI) {
     ec = epi_consts(col0, kCN);
-    if constexpr (FIVE) {
-      if (xcol >= 0) ecx = epi_consts(xcol, 16);
-    }
+    if constexpr (FIVE) ecx = epi_consts(xcol, 16);
   }
   const int e_c_dest = epi.c_dest, e_act_s = epi.act_s, e_act_g = epi.act_g;
   auto flush_tile = [&](int row0, int rows, int slot0) __attribute__((always_inline)) {
@@ -884,7 +884,7 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
       if (s + 1 < nstages) stage(std::integral_constant<int, 1>());
       if (s + 2 < nstages) stage(std::integral_constant<int, 2>());
     } else {
-    // The five-group form (a launch with xcol >= 0).  Besides its own column group, of
+    // The five-group form.  Besides its own column group, of
     // which it multiplies the four row blocks of a stage, wave w multiplies row block w with
     // the fragments of a fifth group (output columns xcol .., accumulator columns kCN ..):
     // five blocks of MFMAs per stage and wave instead of four, and no SIMD that multiplies
@@ -905,7 +905,7 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
     const int dummy_x = T * kAS * 4 + acc_lane_x;
     int aprev = dummy_x;
     bool x_pending = false;
-    const bool x_on = FIVE && xcol >= 0;
+    constexpr bool x_on = FIVE;  // (a launch of the form has a fifth group: xcol >= 0)
     const char *const abx = a_base + wave * 16 * kRowB;
     const int w_soffx = (x_on ? xcol / 16 : 0) * nch * kFragB;
     auto load_kofx = [&](const StagePos &pos) -> int {
@@ -1211,8 +1211,9 @@ inline int launch_conv(const ConvPlan &p, const ConvWs &w, const IO *features, i
   SSC_CHECK(p.n_wg >= 1 && p.n_colblk >= 1 && col_base % 16 == 0 &&
                 col_base + (p.n_colblk - 1) * 16 * NCW < c_out,
             SSC_ERUNTIME, "convolution launch outside the output columns");
-  SSC_CHECK(FORM == 2 ? (xcol < 0 || (xcol % 16 == 0 && xcol < c_out && p.nch >= 4 && p.n_colblk == 1))
-                      : xcol < 0,
+  SSC_CHECK(FORM == 2 ? (xcol >= 0 && xcol % 16 == 0 && xcol < c_out && p.nch >= 4 &&
+                         p.n_colblk == 1 && p.five)
+                      : (xcol < 0 && p.five == (FORM == 3)),
             SSC_ERUNTIME, "convolution launch with a fifth column group it is not built for");
   dim3 grid((unsigned)p.n_wg, (unsigned)p.n_colblk);
   // one column block per XCD when the packed filters are larger than an L2 can keep
