@@ -310,6 +310,7 @@ __global__ void __launch_bounds__(256)
 // input gradient of the 64 -> 128 benchmark layer, 57 k rows for 256 workgroups -- the
 // ranges' work differed by 14 %)
 constexpr int kSplitGranule = 64, kSplitGranuleSmall = 16;
+constexpr int kTileSlack = 24;
 constexpr int kMaxRanges = 512;  // two for each of at most 256 workgroups
 // The accumulator window of a workgroup holds kSpillRows more rows than a tile is
 // high: the last row block that an offset contributes to a tile may then be filled
@@ -464,7 +465,12 @@ __global__ void __launch_bounds__(kMaxRanges)
     // exclusive scan of the tile counts of the ranges, one per thread
     __shared__ int wave_sum[kMaxRanges / 64];
     const int w = threadIdx.x, lane = w & 63;
-    const int nt = w < n_wg ? (row_s[w + 1] - row_s[w] + T - 1) / T : 0;
+    // (a range a little longer than a whole number of tiles does not get one more: its
+    // tiles grow by up to kTileSlack rows in all, at the cost of as many rows of spill --
+    // every tile more pads the last row block of every offset once more)
+    const int rows_w = w < n_wg ? row_s[w + 1] - row_s[w] : 0;
+    int nt = (rows_w + T - 1 - kTileSlack) / T;
+    if (nt < 1 && rows_w > 0) nt = 1;
     int incl = nt;
 #pragma unroll
     for (int d = 1; d < 64; d <<= 1) {
@@ -495,7 +501,8 @@ __global__ void __launch_bounds__(kMaxRanges)
       for (int j = 0; j < nt; ++j) {
         const int r = row_s[w] + j * h;
         tile_row0[tile_s[w] + j] = r;
-        spill_end[tile_s[w] + j] = j == 0 ? r : min(r + window - T, row_s[w + 1]);
+        // (tile and spill fill the window: a tile lower than the highest spills further)
+        spill_end[tile_s[w] + j] = j == 0 ? r : min(r + window - h, row_s[w + 1]);
         tile_slot0[tile_s[w] + j] = (j * h) % window;
       }
     }
