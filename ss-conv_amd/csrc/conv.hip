@@ -447,6 +447,28 @@ __global__ void __launch_bounds__(256)
 // first row of tile t itself when t starts a workgroup's range: no spill across
 // ranges); tile_slot0[t]: accumulator slot of the first row of tile t.  T is the
 // largest tile height, window the height of the accumulator window.
+// How a range of `rows` output rows is cut into tiles: nt tiles, all of height h but the last,
+// which has what is left.  T is the height a tile has when the window behind it keeps the
+// usual room for spilled row blocks (window - T rows).  The last tile of a range spills
+// nowhere -- the next rows are another workgroup's -- so it may fill the window: it is
+// given up to window - T - kTileSlack rows more than the others.  And a range a little
+// longer than a whole number of tiles does not get one more: its tiles grow by up to
+// kTileSlack rows in all, at the cost of as many rows of spill.  (Every tile more pads the
+// last row block of every offset once more.)
+__device__ __forceinline__ void range_tiles(int rows, int T, int window, int *nt, int *h) {
+  if (rows <= 0) {
+    *nt = 0;
+    *h = 0;
+    return;
+  }
+  const int bonus = window - T - kTileSlack;  // > 0: T <= window - 160
+  const int eff = rows - bonus;
+  int n = (eff - kTileSlack + T - 1) / T;
+  if (eff - kTileSlack <= 0 || n < 1) n = 1;
+  *nt = n;
+  *h = n > 1 ? (eff + n - 1) / n : rows;
+}
+
 __global__ void __launch_bounds__(kMaxRanges)
     split_rows_kernel(const int32_t *__restrict__ range_row0, int64_t n_out, int T, int window,
                       int n_wg, int32_t *__restrict__ wg_tile, int32_t *__restrict__ tile_row0,
@@ -465,12 +487,8 @@ __global__ void __launch_bounds__(kMaxRanges)
     // exclusive scan of the tile counts of the ranges, one per thread
     __shared__ int wave_sum[kMaxRanges / 64];
     const int w = threadIdx.x, lane = w & 63;
-    // (a range a little longer than a whole number of tiles does not get one more: its
-    // tiles grow by up to kTileSlack rows in all, at the cost of as many rows of spill --
-    // every tile more pads the last row block of every offset once more)
-    const int rows_w = w < n_wg ? row_s[w + 1] - row_s[w] : 0;
-    int nt = (rows_w + T - 1 - kTileSlack) / T;
-    if (nt < 1 && rows_w > 0) nt = 1;
+    int nt = 0, h_unused = 0;
+    if (w < n_wg) range_tiles(row_s[w + 1] - row_s[w], T, window, &nt, &h_unused);
     int incl = nt;
 #pragma unroll
     for (int d = 1; d < 64; d <<= 1) {
@@ -495,9 +513,9 @@ __global__ void __launch_bounds__(kMaxRanges)
     wg_tile[w] = tile_s[w];
     if (w == n_wg) break;
     const int rows = row_s[w + 1] - row_s[w];
-    const int nt = tile_s[w + 1] - tile_s[w];
+    int nt = 0, h = 0;
+    range_tiles(rows, T, window, &nt, &h);  // nt == tile_s[w + 1] - tile_s[w]
     if (nt > 0) {
-      const int h = (rows + nt - 1) / nt;
       for (int j = 0; j < nt; ++j) {
         const int r = row_s[w] + j * h;
         tile_row0[tile_s[w] + j] = r;
