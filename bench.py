@@ -32,7 +32,7 @@ CLOCK_WARMUP_MS = 100
 # launches) for every workload this script offers, from rocprofv3 --pmc FETCH_SIZE /
 # WRITE_SIZE runs scaled by a copy kernel of known size (the summaries
 # profiles/conv_fwd_<workload>_hbm_traffic.md give commands and counter values).
-MEASURED_TRAFFIC_BYTES = {"cfg1": 3423455, "cfg2": 345550170, "cfg3": 227896858, "cfg5": 70491494271}
+MEASURED_TRAFFIC_BYTES = {"cfg1": 3416327, "cfg2": 345545343, "cfg3": 229620287, "cfg5": 68985036509}
 
 
 def parse_args():
