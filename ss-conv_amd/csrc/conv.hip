@@ -305,7 +305,7 @@ __global__ void __launch_bounds__(256)
 // share of what every tile costs on top of its pairs (padding of the last row block
 // of each offset, writing the tile out).  Pairs per row come from a fine grid of
 // kSplitGranule rows; range boundaries lie on that grid.  Each range is then cut
-// into tiles of equal height <= T.
+// into tiles (range_tiles below: equal heights of about T at most, a higher last one).
 // (16 rows where a range has fewer than 2048: with 3.5 cells of 64 rows to a range -- the
 // input gradient of the 64 -> 128 benchmark layer, 57 k rows for 256 workgroups -- the
 // ranges' work differed by 14 %)
