@@ -194,6 +194,8 @@ int ssc_conv_fwd_f16(const void *features /* [n_in,c_in] half */, int64_t n_in, 
  *   ssc_conv_run_*: the MFMA kernel alone.  Results are bit-identical to ssc_conv_fwd_*.
  * Pairs with one scatter row twice inside an offset are not supported by either form (a
  * rulebook never has them). */
+/* Both sizes grow with n_out (and never shrink for a smaller one): buffers sized for an
+ * upper bound of n_out serve a plan over any number of rows up to that bound. */
 size_t ssc_conv_plan_bytes(int64_t n_out, int32_t kernel_volume, int32_t c_in, int32_t c_out,
                            int64_t pair_stride);
 size_t ssc_conv_plan_scratch_bytes(int64_t n_out, int32_t kernel_volume, int32_t c_in,
@@ -204,6 +206,12 @@ int ssc_conv_plan_build(const int32_t *pairs /* [K,2,pair_stride] */, int64_t pa
                         int32_t inverse, int32_t flags, int64_t n_in, int64_t n_out, int32_t c_in,
                         int32_t c_out, int32_t elem_bytes, void *plan, size_t plan_bytes,
                         void *scratch, size_t scratch_bytes, ssc_stream_t stream);
+/* How a workgroup's range of `rows` output rows is cut into tiles for a layer of these
+ * channel counts (host arithmetic only, no GPU needed; no counterpart in the reference): the
+ * range gets *n_tiles tiles, all of *height rows but the last, which has the rest -- more
+ * than none and at most *window rows, the height of the accumulator window. */
+int ssc_conv_tile_cut(int32_t rows, int32_t c_in, int32_t c_out, int32_t *n_tiles,
+                      int32_t *height, int32_t *window);
 int ssc_conv_pack_filters_f32(const float *filters, int64_t fs_k, int64_t fs_ci, int64_t fs_co,
                               int32_t kernel_volume, int32_t c_in, int32_t c_out, void *packed,
                               size_t packed_bytes, ssc_stream_t stream);

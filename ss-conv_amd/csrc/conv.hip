@@ -455,7 +455,7 @@ __global__ void __launch_bounds__(256)
 // longer than a whole number of tiles does not get one more: its tiles grow by up to
 // kTileSlack rows in all, at the cost of as many rows of spill.  (Every tile more pads the
 // last row block of every offset once more.)
-__device__ __forceinline__ void range_tiles(int rows, int T, int window, int *nt, int *h) {
+__host__ __device__ __forceinline__ void range_tiles(int rows, int T, int window, int *nt, int *h) {
   if (rows <= 0) {
     *nt = 0;
     *h = 0;
@@ -465,8 +465,18 @@ __device__ __forceinline__ void range_tiles(int rows, int T, int window, int *nt
   const int eff = rows - bonus;
   int n = (eff - kTileSlack + T - 1) / T;
   if (eff - kTileSlack <= 0 || n < 1) n = 1;
-  *nt = n;
-  *h = n > 1 ? (eff + n - 1) / n : rows;
+  if (n == 1) {
+    *nt = 1;
+    *h = rows;
+    return;
+  }
+  // h <= T + kTileSlack.  Tiles of that height until what is left fits the last one: with
+  // hundreds of tiles to a range the rounding of h adds up to whole tiles, and n tiles of
+  // height h would reach beyond the range's end.  The last tile has between bonus + 1 and
+  // bonus + h rows.
+  const int hh = (eff + n - 1) / n;
+  *h = hh;
+  *nt = (eff + hh - 1) / hh;
 }
 
 __global__ void __launch_bounds__(kMaxRanges)
@@ -850,13 +860,16 @@ static bool g_conv_rebalance = true;  // long kernels: a second work split from 
 static bool g_conv_round8 = false;    // ranges per column block: a multiple of 8 only
 
 // The sizes that follow from the number of workgroups per column block.
+// `sizing`: the plan is only being sized (the number of input rows, and with it the number
+// of ranges, is not known): the finer grid, so that a buffer sized for n_out rows is large
+// enough for a plan over any smaller number of rows as well.
 static void plan_split(ConvPlan &p, int n_wg, int n_rng, int64_t n_out, int K,
-                       int64_t pair_stride) {
+                       int64_t pair_stride, bool sizing) {
   p.n_wg = n_wg;
   p.n_rng = n_rng;
   // upper bound of the tile count: every range ends with a partial tile
   p.n_tiles = ceil_div(n_out > 0 ? n_out : 1, p.tile_rows) + n_rng;
-  p.granule = n_out / n_rng < 2048 ? kSplitGranuleSmall : kSplitGranule;
+  p.granule = sizing || n_out / n_rng < 2048 ? kSplitGranuleSmall : kSplitGranule;
   p.n_fine = ceil_div(n_out > 0 ? n_out : 1, p.granule);
   p.words_per_k = ceil_div(n_out > 0 ? n_out : 1, 32);
   // groups: pairs/64 plus, per (tile, offset), up to one partial block, plus one
@@ -931,7 +944,7 @@ static ConvPlan make_plan(int64_t n_in, int64_t n_out, int K, int c_in, int c_ou
   const bool pair = g_conv_pair && n_wg >= 2 &&
                     (g_conv_pair_always || n_in <= 0 ||
                      (!p.rebalance && est_groups >= kPairGroups && est_groups >= (int64_t)K / 2));
-  plan_split(p, n_wg, pair ? 2 * n_wg : n_wg, n_out, K, pair_stride);
+  plan_split(p, n_wg, pair ? 2 * n_wg : n_wg, n_out, K, pair_stride, n_in <= 0);
   p.lds_bytes = conv_lds_bytes(p.T, p.acc_cols);
   return p;
 }
@@ -1465,6 +1478,19 @@ int ssc_conv_fwd_f16(const void *features, int64_t n_in, int32_t c_in, const voi
                             static_cast<const _Float16 *>(filters), fs_k, fs_ci, fs_co, c_out,
                             pairs, pair_stride, pair_num, kernel_volume, inverse, subm,
                             static_cast<_Float16 *>(out), n_out, workspace, workspace_bytes, stream);
+}
+
+int ssc_conv_tile_cut(int32_t rows, int32_t c_in, int32_t c_out, int32_t *n_tiles, int32_t *height,
+                      int32_t *window) {
+  SSC_CHECK(rows >= 0 && c_in >= 1 && c_out >= 1 && n_tiles && height && window, SSC_EINVAL,
+            "bad argument");
+  const ConvPlan p = make_plan(0, 1, 1, c_in, c_out, 0);
+  int nt = 0, h = 0;
+  range_tiles(rows, p.tile_rows, p.T, &nt, &h);
+  *n_tiles = nt;
+  *height = h;
+  *window = p.T;
+  return SSC_OK;
 }
 
 size_t ssc_conv_packed_bytes(int32_t kernel_volume, int32_t c_in, int32_t c_out) {

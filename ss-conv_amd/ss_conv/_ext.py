@@ -50,6 +50,8 @@ _SIGNATURES = {
     "ssc_conv_plan_bytes": (_sz, [_i64, _i32, _i32, _i32, _i64]),
     "ssc_conv_plan_scratch_bytes": (_sz, [_i64, _i32, _i32, _i32, _i64]),
     "ssc_conv_packed_bytes": (_sz, [_i32, _i32, _i32]),
+    "ssc_conv_tile_cut": (ctypes.c_int, [_i32, _i32, _i32, ctypes.POINTER(_i32),
+                                         ctypes.POINTER(_i32), ctypes.POINTER(_i32)]),
     "ssc_conv_plan_build": (ctypes.c_int, [_vp, _i64, _vp, _i32, _i32, _i32, _i64, _i64, _i32, _i32,
                                            _i32, _vp, _sz, _vp, _sz, _vp]),
     "ssc_conv_pack_filters_f32": (ctypes.c_int, [_vp, _i64, _i64, _i64, _i32, _i32, _i32, _vp, _sz,

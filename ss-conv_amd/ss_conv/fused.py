@@ -143,9 +143,19 @@ class ConvBatchNormActivation(nn.Module):
         self._held = (key, wp, epi)
         return wp, epi
 
+    def _tail_wants_grad(self):
+        """Whether autograd is on and a parameter of the batch norm or the activation asks for
+        a gradient (fine-tuning affine or bias parameters on frozen statistics): the one-kernel
+        path builds no graph, so such a call takes the separate layers."""
+        if not torch.is_grad_enabled():
+            return False
+        return any(p.requires_grad for m in (self.bn, self.activation) if m is not None
+                   for p in m.parameters())
+
     def forward(self, input):  # pylint: disable=W
         conv = self.conv
-        if not self.training and input.features.is_cuda and self._block_layout():
+        if not self.training and input.features.is_cuda and self._block_layout() \
+                and not self._tail_wants_grad():
             feats = input.features
             weight = conv.eval_weight(feats) if hasattr(conv, "eval_weight") else conv.weight
             if weight is not None and conv.epilogue_ok(input, weight):

@@ -1685,6 +1685,38 @@ def test_fused_rulebook_conv_equals_the_two_calls(subm, stride, device):
     assert torch.equal(y3 + layer.bias.detach(), y1.features.detach())
 
 
+def test_fused_layer_on_a_dense_grid(device):
+    """A grid the outputs nearly fill: the layer sizes its plan for the bound on the number
+    of outputs (every cell: 4 x 64^3) before that number arrives, and the real number (about
+    0.9 M) falls where the work split uses a finer grid than it would for the bound.  The
+    buffers sized for the bound must do."""
+    from ss_conv.sp_ops.conv import SparseConvolution
+    from ss_conv.sp_ops.ops import get_indice_pairs
+    from ss_conv.sp_ops.functional import indice_conv
+    from ss_conv.sp_ops.tensor import SparseTensor
+    rng = np.random.default_rng(5)
+    idx = random_voxels(rng, 4, 64, 75000)
+    t = torch.from_numpy(idx).to(device)
+    torch.manual_seed(2)
+    layer = SparseConvolution(3, 64, 64, 3, stride=1, padding=1, bias=False).to(device)
+    x = torch.randn((idx.shape[0], 64), device=device)
+    with torch.no_grad():
+        y = layer(SparseTensor(x, t, [64] * 3, 4))
+        n_out = y.indices.shape[0]
+        assert 0.67 * 4 * 64 ** 3 < n_out < 4 * 64 ** 3, n_out
+        g_idx, g_pairs, g_num = get_indice_pairs(t, 4, [64] * 3, 3, 1, 1, 1, 0, False)
+        assert torch.equal(y.indices, g_idx)
+        y2 = indice_conv(x, layer.weight, g_pairs, g_num, n_out)
+        assert torch.equal(y.features, y2)
+        # a sample of rows against float64 sums over the pairs
+        w = layer.weight.double().reshape(27, 64, 64)
+        ref = torch.zeros((n_out, 64), dtype=torch.float64, device=device)
+        for k in range(27):
+            m = int(g_num[k])
+            ref.index_add_(0, g_pairs[k, 1, :m].long(), x[g_pairs[k, 0, :m].long()].double() @ w[k])
+        assert rel_l2(y.features.double().cpu().numpy(), ref.cpu().numpy()) < 1e-5
+
+
 def _p2v_same(a, b):
     """Two Point2Voxel results, field by field, bit for bit."""
     (vp1, st1, vi1, f1), (vp2, st2, vi2, f2) = a, b

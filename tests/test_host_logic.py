@@ -72,6 +72,59 @@ def test_cpu_tensors_are_rejected():
                               torch.zeros(27, dtype=torch.int32), 2, 0, 0)
 
 
+def test_plan_buffers_sized_for_a_bound_serve_every_smaller_row_count():
+    """A layer sizes plan and scratch for an upper bound of the number of output rows before
+    that number is known; the plan is then built for the real number.  The sizes must not
+    shrink when n_out grows, across the thresholds where the work split changes its grid
+    (fewer than 2048 rows to a range) and its number of ranges."""
+    from ss_conv import _ext
+    lib = _ext._lib
+    for K, c_in, c_out, stride in ((27, 64, 64, 200000), (27, 64, 128, 57304), (125, 200, 200, 106731),
+                                   (8, 256, 256, 85349), (27, 3, 152, 30000), (27, 512, 608, 4000)):
+        sizes = []
+        ns = sorted(set([1, 15, 16, 17, 63, 64, 65, 1000, 2047 * 128, 2048 * 128, 2048 * 256 - 1,
+                         2048 * 256, 2048 * 256 + 1, 2048 * 512 - 1, 2048 * 512, 2048 * 512 + 1,
+                         600000, 750000, 900000, 1048576, 3000000] +
+                        [int(1.17 ** e) for e in range(10, 100)]))
+        for n in ns:
+            sizes.append((lib.ssc_conv_plan_bytes(n, K, c_in, c_out, stride),
+                          lib.ssc_conv_plan_scratch_bytes(n, K, c_in, c_out, stride),
+                          lib.ssc_conv_workspace_bytes(n, K, c_in, c_out, stride)))
+        for a, b, n in zip(sizes, sizes[1:], ns[1:]):
+            assert b[0] >= a[0] and b[1] >= a[1] and b[2] >= a[2], (K, c_in, c_out, n, a, b)
+    # the case of the report: bound 1048576 rows, 900000 real ones
+    assert lib.ssc_conv_plan_scratch_bytes(1048576, 27, 64, 64, 200000) >= \
+        lib.ssc_conv_plan_scratch_bytes(900000, 27, 64, 64, 200000)
+
+
+def test_tile_cut_of_a_range():
+    """Every tile of a range has rows, the heights add up to the range, tiles but the last
+    keep room for spilled row blocks behind them and the last one fits the window -- also
+    for ranges of hundreds of tiles (tens of millions of output rows)."""
+    from ss_conv import _ext
+    lib = _ext._lib
+    nt, h, win = ctypes.c_int32(), ctypes.c_int32(), ctypes.c_int32()
+    for c_in, c_out in ((64, 128), (200, 200), (64, 72), (3, 16)):
+        rows_list = list(range(0, 1400)) + [304 * k + d for k in (5, 50, 300, 440, 441, 600, 2000, 7000)
+                                            for d in (-161, -1, 0, 1, 23, 24, 25, 135, 137, 303)]
+        for rows in rows_list:
+            assert lib.ssc_conv_tile_cut(rows, c_in, c_out, ctypes.byref(nt), ctypes.byref(h),
+                                         ctypes.byref(win)) == 0
+            if rows == 0:
+                assert nt.value == 0
+                continue
+            n, hh, w = nt.value, h.value, win.value
+            assert n >= 1 and hh >= 1
+            last = rows - (n - 1) * hh
+            assert 0 < last <= w, (rows, n, hh, w)
+            if n > 1:
+                # a tile and the 160 (192) rows of spill behind it fit the window, give or
+                # take the slack of 24 rows
+                assert hh + 136 <= w, (rows, n, hh, w)
+    assert lib.ssc_conv_tile_cut(-1, 64, 64, ctypes.byref(nt), ctypes.byref(h),
+                                 ctypes.byref(win)) == _ext.SSC_EINVAL
+
+
 # ---- shape arithmetic and the tensor type ---------------------------------------------------
 @pytest.mark.parametrize("size,k,s,p,d", [(64, 3, 1, 1, 1), (64, 3, 2, 1, 1), (32, 2, 2, 0, 1),
                                           (17, 5, 1, 2, 1), (20, 3, 1, 2, 2), (9, 3, 3, 0, 1)])
