@@ -33,6 +33,11 @@ CLOCK_WARMUP_MS = 100
 # WRITE_SIZE runs scaled by a copy kernel of known size (the summaries
 # profiles/conv_fwd_<workload>_hbm_traffic.md give commands and counter values).
 MEASURED_TRAFFIC_BYTES = {"cfg1": 3416327, "cfg2": 345545343, "cfg3": 229620287, "cfg5": 68985036509}
+# the same for all kernels of one rulebook call and of one Point2Voxel call
+# (profiles/rulebook_hbm_traffic.md, profiles/point_voxel_hbm_traffic.md)
+RULEBOOK_TRAFFIC_BYTES = {"cfg2": 37000000, "cfg5": 188500000}
+P2V_TRAFFIC_BYTES = {"cfg2": 62500000, "cfg5": 116400000}
+HBM_PEAK_GBS = 8000.0
 
 
 def parse_args():
@@ -40,7 +45,9 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="cfg2", choices=["cfg1", "cfg2", "cfg3", "cfg5"])
+    ap.add_argument("--workload", default="cfg2", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5"],
+                    help="cfg4: the backbone of the fourth configuration (evaluation mode), one "
+                         "step = one forward of the whole backbone")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--time-every", type=int, default=0, metavar="N",
@@ -101,6 +108,115 @@ def cpu_baseline(idx, feats, dense_w, cfg, n_out_expected):
             "sample": "full %s layer (rulebook + gather/GEMM/scatter conv), median of %d runs, "
                       "%.2f s each; rulebook and gather/scatter single-thread C, GEMM numpy BLAS"
                       % (cfg["name"], len(times), t)}, out
+
+
+def gpu_span_us(torch, dev, queue, reps=20):
+    """GPU time in microseconds of the kernels `queue()` enqueues on the current stream: a
+    pair of events around them, behind a fill kernel that keeps the GPU busy while the host
+    enqueues (so the span holds no host time), minus what an empty pair of events reads in
+    the same position.  queue() returns a function that finishes the call (waits, results),
+    run after the second event is recorded.  Medians over `reps` calls; returns
+    (span, empty span)."""
+    filler = torch.empty(192 << 20, dtype=torch.uint8, device=dev)
+    spans, empties = [], []
+    for rep in range(reps + 3):
+        for what in (0, 1):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            torch.cuda.synchronize()
+            filler.zero_()
+            e0.record()
+            done = queue() if what else None
+            e1.record()
+            if done is not None:
+                done()
+            torch.cuda.synchronize()
+            if rep >= 3:
+                (spans if what else empties).append(e0.elapsed_time(e1) * 1e3)
+    med = lambda v: sorted(v)[len(v) // 2]  # noqa: E731
+    return med(spans), med(empties)
+
+
+def rulebook_figure(torch, _ext, dev, indices, batch, shape, k, stride, pad, workload):
+    """The rulebook of the layer by itself: GPU time of its kernels (events on their stream)
+    against its algorithmic bytes 16 N_in + 16 N_out + 8 P + 4 K, and the call as the host
+    sees it (get_indice_pairs with its wait)."""
+    from ss_conv.sp_ops.ops import get_indice_pairs
+    K = k ** 3
+    out_idx, _, num = get_indice_pairs(indices, batch, shape, k, stride, pad)
+    n_in, n_out, P = indices.shape[0], out_idx.shape[0], int(num.sum().item())
+    nbytes = 16 * n_in + 16 * n_out + 8 * P + 4 * K
+
+    def queue():
+        r = _ext._rulebook_begin(indices, batch, shape, [k] * 3, [stride] * 3, [pad] * 3, [1] * 3,
+                                 [0] * 3, 0, 0)
+        return lambda: _ext._rulebook_finish(r)
+    span, empty = gpu_span_us(torch, dev, queue)
+    gpu_us = max(span - empty, 1e-3)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(20):
+        get_indice_pairs(indices, batch, shape, k, stride, pad)
+    torch.cuda.synchronize()
+    call_us = (time.perf_counter() - t0) * 1e6 / 20
+    gbs = nbytes / gpu_us / 1e3
+    return {"workload": workload, "bytes": nbytes, "gpu_us": gpu_us, "gbs": gbs,
+            "frac_hbm": gbs / HBM_PEAK_GBS, "traffic": RULEBOOK_TRAFFIC_BYTES.get(workload),
+            "call_us": call_us, "event_pair_us": empty,
+            "n_in": n_in, "n_out": n_out, "pairs": P,
+            "how": "HIP events around the kernels of one ssc_rulebook_begin on their stream, "
+                   "median of 20, an empty event pair subtracted; call_us: get_indice_pairs "
+                   "with its host wait, mean of 20"}
+
+
+def point2voxel_figure(torch, _ext, synth, dev, workload, seed, channels=64):
+    """Point2Voxel on the clouds of a configuration: the module call as the host sees it --
+    a first call (a fresh module) and repeated calls -- and the GPU time of its kernels,
+    against its algorithmic bytes N (12 + 8 + 4 C) + M (16 + 4 C) + 4 N."""
+    from ss_conv.sp_ops.voxelize import Point2Voxel
+    cfg = synth.CONFIGS[workload]
+    pts, _, ids = synth.config_clouds(workload, seed)
+    tp = torch.from_numpy(pts).to(dev)
+    tf = torch.randn(tp.shape[0], channels, device=dev)
+    ti = torch.from_numpy(ids).to(dev)
+    grid = cfg["grid"]
+    make = lambda: Point2Voxel([grid] * 3, [2.0 / grid] * 3)  # noqa: E731
+    with torch.no_grad():
+        p2v = make()
+        r = p2v(tp, tf, ti)
+        torch.cuda.synchronize()
+        firsts = []
+        for _ in range(10):
+            m = make()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            m(tp, tf, ti)
+            torch.cuda.synchronize()
+            firsts.append((time.perf_counter() - t0) * 1e6)
+        first_path = m.last_path
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(50):
+            p2v(tp, tf, ti)
+        torch.cuda.synchronize()
+        call_us = (time.perf_counter() - t0) * 1e6 / 50
+
+        def queue():
+            p2v(tp, tf, ti)
+            return None
+        span, empty = gpu_span_us(torch, dev, queue)
+    N, M = tp.shape[0], r[1].features.shape[0]
+    nbytes = N * (12 + 8 + 4 * channels) + M * (16 + 4 * channels) + 4 * N
+    gpu_us = max(span - empty, 1e-3)
+    gbs = nbytes / gpu_us / 1e3
+    return {"workload": workload, "points": N, "voxels": M, "channels": channels, "bytes": nbytes,
+            "gpu_us": gpu_us, "gbs": gbs, "frac_hbm": gbs / HBM_PEAK_GBS,
+            "traffic": P2V_TRAFFIC_BYTES.get(workload),
+            "call_us": call_us, "first_call_us": sorted(firsts)[len(firsts) // 2],
+            "path": p2v.last_path, "first_call_path": first_path, "event_pair_us": empty,
+            "how": "gpu_us: HIP events around one module call (its one host wait included), "
+                   "median of 20, an empty event pair subtracted; call_us: mean of 50 calls of "
+                   "one module, host-timed; first_call_us: median of 10 first calls of fresh "
+                   "modules"}
 
 
 def ops_table(torch, _ext, synth, dev, seed):
@@ -483,6 +599,83 @@ def backbone_table(torch, _ext, synth, dev, seed, n=5, warm=2):
     print("\n".join(rows), file=sys.stderr)
 
 
+def backbone_line(args, torch, _ext, synth, dev):
+    """--workload cfg4: one step = one forward of the backbone of the fourth configuration
+    in evaluation mode (Point2Voxel, four [Convolution -> BatchNorm -> gated Activation]
+    blocks, GlobalAvgPool, Voxel2Point).  The JSON line carries the whole forward as
+    ms_per_step, every stage's convolution kernel time (HIP events around its launches) and,
+    as roofline, the flops of the four convolutions over the sum of their kernel times."""
+    backbone = build_backbone(torch, synth, dev, args.seed)
+    with torch.no_grad():
+        t_warm = time.perf_counter()
+        while (time.perf_counter() - t_warm) * 1e3 < CLOCK_WARMUP_MS:
+            r = backbone()
+            torch.cuda.synchronize()
+        for _ in range(args.warmup):
+            r = backbone()
+        torch.cuda.synchronize()
+        gc.collect()
+        n_st = len(r[3])
+        steps = args.steps
+        _ext.profile_conv(True, every=1)
+        gc.disable()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            r = backbone()
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        gc.enable()
+        conv_ms = _ext.profile_conv_read()
+        _ext.profile_conv(False)
+        torch.cuda.synchronize()
+        t2 = time.perf_counter()
+        for _ in range(max(steps // 4, 1)):
+            backbone(separate=True)
+        torch.cuda.synchronize()
+        ms_sep = (time.perf_counter() - t2) * 1e3 / max(steps // 4, 1)
+    ms_per_step = (t1 - t0) * 1e3 / steps
+    stages, flops_sum, kernel_sum, rows_sum = [], 0.0, 0.0, 0
+    conv_ms = conv_ms[len(conv_ms) % n_st:]  # the ring holds whole forwards
+    for i, (n_in, n_out, num, cin, cout) in enumerate(r[3]):
+        P = int(num.sum().item())
+        mine = conv_ms[i::n_st]
+        t = sum(mine) / max(len(mine), 1)
+        fl = 2.0 * P * cin * cout
+        flops_sum += fl
+        kernel_sum += t
+        rows_sum += n_out
+        stages.append({"stage": i + 1, "n_in": int(n_in), "n_out": int(n_out), "c_in": int(cin),
+                       "c_out": int(cout), "pairs": P, "gflop": fl / 1e9, "kernel_ms": t,
+                       "tflops": fl / t / 1e9 if t > 0 else 0.0,
+                       "frac_mfma": fl / t / 1e9 / FP32_MFMA_PEAK_TFLOPS if t > 0 else 0.0})
+    achieved = flops_sum / (kernel_sum * 1e-3) / 1e12 if kernel_sum > 0 else 0.0
+    result = {
+        "metric": "SS-Conv backbone forward: active output voxels/s over its four convolution "
+                  "stages (Point2Voxel + 4 x [conv + bn + gate] + GlobalAvgPool + Voxel2Point)",
+        "value": rows_sum / (ms_per_step * 1e-3), "unit": "active output voxels/s",
+        "n_gpus": 1, "steps": steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "cfg4: backbone, 32 clouds x 1024 pts, 64^3 grid, 3 -> 152 -> 304 "
+                               "-> 608 -> 608 filter columns (gates included), strides 1, 2, 2, 1, "
+                               "evaluation mode",
+                   "stages": stages, "clock_warmup_ms": CLOCK_WARMUP_MS,
+                   "timed_region": "cyclic garbage collector off (as timeit does)",
+                   "ms_per_step_separate_layers": ms_sep,
+                   "voxels_after_stage_4": int(r[2].features.shape[0]),
+                   "channels_after_stage_4": int(r[2].features.shape[1])},
+        "roofline": {"bound": "mfma", "achieved": achieved, "peak": FP32_MFMA_PEAK_TFLOPS,
+                     "unit": "TFLOP/s", "frac": achieved / FP32_MFMA_PEAK_TFLOPS, "traffic": None,
+                     "kernel": "conv_fwd_kernel (the four stages' launches; batch norm and gate "
+                               "applied by the kernel)",
+                     "kernel_ms": kernel_sum, "kernel_launches_timed": len(conv_ms),
+                     "flops_per_launch": flops_sum},
+        "cpu_baseline": None,
+    }
+    print(json.dumps(result))
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -502,6 +695,11 @@ def main():
         print("bench.py needs a GPU", file=sys.stderr)
         sys.exit(2)
     dev = torch.device("cuda:0")
+    if args.workload == "cfg4":
+        if args.steps == 100 and args.warmup == 20:  # the defaults are sized for a 0.4 ms step
+            args.steps, args.warmup = 20, 5
+        backbone_line(args, torch, _ext, synth, dev)
+        return
     cfg = dict(synth.CONFIGS[args.workload], name=args.workload)
     grid = cfg["grid"]
     rs_in = synth.irreps(cfg["mult_in"], cfg["lmax"])
@@ -613,6 +811,15 @@ def main():
                      "kernel_launches_timed": len(conv_ms),
                      "flops_per_launch": flops},
     }
+
+    # the two bandwidth-bound callers of the layer that the metric names, measured in this
+    # process: the rulebook of this workload and Point2Voxel on its clouds
+    with torch.no_grad():
+        result["rulebook"] = rulebook_figure(torch, _ext, dev, indices, st.batch_size,
+                                             list(st.spatial_shape), cfg["kernel"], cfg["stride"],
+                                             cfg["padding"], args.workload)
+        result["point2voxel"] = point2voxel_figure(torch, _ext, synth, dev, args.workload,
+                                                   args.seed)
 
     if args.breakdown:
         def timed(fn, n=10):

@@ -120,6 +120,84 @@ def _conv_full_size(name, cin, cout, oracle, device, with_oracle):
         assert rel_l2(out.cpu().numpy(), o_ref) < REL_L2
 
 
+def test_conv_cfg5_against_the_oracle_fixture(device):
+    """The fifth configuration's convolution (200 -> 200 channels, 125 offsets: the five-group
+    form, three launches) against the CPU oracle at full size.  The oracle needs minutes
+    for this layer, so tests/golden/make_conv_cfg5_golden.py ran it once and kept 2048
+    sampled output rows, their voxel keys, the column sums and the sum of squares of the
+    whole output; the inputs are seeded numpy draws, regenerated here."""
+    import os
+    import sys
+    from ss_conv import _ext
+    here = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+    sys.path.insert(0, here)
+    try:
+        from make_conv_cfg5_golden import cfg5_inputs
+    finally:
+        sys.path.remove(here)
+    gold = np.load(os.path.join(here, "conv_cfg5_rows.npz"))
+    cfg, idx, f, w = cfg5_inputs()
+    k = cfg["kernel"]
+    c = f.shape[1]
+    out_idx, pairs, num = _gpu_rulebook(cfg, idx, device)
+    n_out = out_idx.shape[0]
+    assert idx.shape[0] == int(gold["n_in"]) and n_out == int(gold["n_out"])
+    assert int(num.sum().item()) == int(gold["pairs"])
+    rows = torch.from_numpy(gold["rows"]).long().to(device)
+    assert np.array_equal(out_idx[rows].cpu().numpy(), gold["out_row_keys"])
+    tf = torch.from_numpy(f).to(device)
+    tw = torch.from_numpy(w).to(device).reshape(k, k, k, c, c)
+    out = _ext.indice_conv_fp32(tf, tw, pairs, num, n_out, 0, 0)
+    got = out[rows].cpu().numpy()
+    assert rel_l2(got, gold["out_rows"]) < REL_L2
+    # every element of the sampled rows, not only their norm
+    scale = float(np.sqrt((gold["out_rows"].astype(np.float64) ** 2).mean()))
+    assert float(np.abs(got - gold["out_rows"]).max()) < 1e-4 * scale
+    assert rel_l2(out.double().sum(0).cpu().numpy(), gold["col_sums"]) < REL_L2
+    sq = float((out.double() ** 2).sum().item())
+    assert abs(sq - float(gold["sq_sum"])) < 1e-5 * float(gold["sq_sum"])
+
+
+def test_downsampling_block_full_size(oracle, device):
+    """The third configuration as stated: the stride-2 layer (128 -> 256 channels) on 32
+    clouds x 2048 points at 64^3, then MaxPool and AvgPool with kernel 2, stride 2 over its
+    85 k x 256 output -- rulebooks and pooled rows bit-exact against the oracle (the pools
+    keep the reference's operation order), the convolution against the oracle's
+    gather-GEMM-scatter."""
+    from ss_conv.pool import AvgPool, MaxPool
+    from ss_conv.sp_ops.conv import SparseConvolution
+    from ss_conv.sp_ops.tensor import SparseTensor
+    cfg, idx = _voxels("cfg3")
+    grid, batch = cfg["grid"], cfg["batch"]
+    cin, cout = _channels(cfg, "mult_in"), _channels(cfg, "mult_out")
+    rng = np.random.default_rng(12)
+    f = rng.standard_normal((idx.shape[0], cin), dtype=np.float32)
+    torch.manual_seed(3)
+    conv = SparseConvolution(3, cin, cout, 3, stride=2, padding=1, bias=False).to(device)
+    t = torch.from_numpy(idx).to(device)
+    with torch.no_grad():
+        y = conv(SparseTensor(torch.from_numpy(f).to(device), t, [grid] * 3, batch))
+        mx = MaxPool(2, 2)(y)
+        av = AvgPool(2, 2)(y)
+    o_idx, o_pairs, o_num = oracle.canonicalize(*oracle.rulebook(idx, batch, [grid] * 3, 3, 2, 1))
+    assert np.array_equal(y.indices.cpu().numpy(), o_idx)
+    assert y.features.shape == (o_idx.shape[0], cout) and cout == 256
+    w = conv.weight.detach().reshape(27, cin, cout).cpu().numpy()
+    ref = oracle.conv_fwd(f, w, o_pairs, o_num, o_idx.shape[0], matmul=np.matmul)
+    y_np = y.features.cpu().numpy()
+    assert rel_l2(y_np, ref) < REL_L2
+    half = [int(v) for v in y.spatial_shape]
+    assert half == [grid // 2] * 3
+    p_idx, p_pairs, p_num = oracle.canonicalize(*oracle.rulebook(o_idx, batch, half, 2, 2, 0))
+    assert np.array_equal(mx.indices.cpu().numpy(), p_idx)
+    assert np.array_equal(av.indices.cpu().numpy(), p_idx)
+    # the pools on the GPU's own convolution output: bit for bit
+    assert np.array_equal(mx.features.cpu().numpy(),
+                          oracle.maxpool_fwd(y_np, p_pairs, p_num, p_idx.shape[0]))
+    assert np.array_equal(av.features.cpu().numpy(),
+                          oracle.avgpool_fwd(y_np, p_pairs, p_num, p_idx.shape[0]))
+
+
 def test_layer_chain_full_size(device):
     """cfg3's stride-2 layer followed by average pooling and the global pools at full size:
     sizes and invariants (pooling a non-negative tensor's maximum dominates its average;
