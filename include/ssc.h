@@ -120,16 +120,52 @@ int ssc_rulebook_emit(const int32_t *indices, int64_t n_in, const ssc_geometry *
  * ssc_rulebook_count) returns SSC_EINVAL; the reference reads and writes outside its grid
  * buffer for such a row (src/conv/indice_cuda_functor.cu:60-61). */
 size_t ssc_rulebook_out_bound(const ssc_geometry *g, int64_t n_in);
+/* clean_table (may be NULL): device memory of at least ssc_rulebook_clean_table_bytes() bytes
+ * that is ALL ZERO when the call's kernels start and that they leave all zero again.  A
+ * caller that keeps such a buffer per stream (zeroed once, at least as large as the largest
+ * size asked for so far) saves every regular stride-1 rulebook the launch that clears its
+ * tables; the size is 0 for geometries that have no use for it.  Calls that share the buffer
+ * must not overlap in time, and after a call that failed it must be zeroed again. */
+size_t ssc_rulebook_clean_table_bytes(const ssc_geometry *g, int64_t n_in);
 int ssc_rulebook_begin(const int32_t *indices, int64_t n_in, const ssc_geometry *g,
                        void *workspace, size_t workspace_bytes,
                        int32_t *pairs /* [K,2,n_in] device */, int32_t *pair_num /* [K] device */,
                        int32_t *out_indices /* [out_capacity,4] device, or NULL */,
-                       int64_t out_capacity, ssc_stream_t stream);
+                       int64_t out_capacity, void *clean_table, size_t clean_table_bytes,
+                       ssc_stream_t stream);
 int ssc_rulebook_finish(const ssc_geometry *g, int64_t n_in, int32_t *n_out_host /* host */,
                         int32_t *in_order_host /* host */);
 int ssc_rulebook_rows(const ssc_geometry *g, int64_t n_in, void *workspace,
                       size_t workspace_bytes, int32_t *out_indices /* [n_out,4] device */,
                       ssc_stream_t stream);
+
+/* Rulebook and convolution plan of one layer that has no rulebook yet, in one pair of calls --
+ * what a layer's forward does between get_indice_pairs and indice_conv
+ * (ss_conv/sp_ops/conv.py:131-150, src/conv/indice_conv.h:21-131 then 247-343):
+ *   ssc_rulebook_conv_begin is ssc_rulebook_begin, and for a regular convolution with
+ *     stride 1 and dilation 1 (whose rulebook counts, on its way, the outputs and the pairs
+ *     of every cell of the grid) it also deals the output rows to the convolution kernel's
+ *     workgroups, in a launch the rulebook makes anyway, into the head of `scratch`
+ *     (ssc_conv_plan_scratch_bytes of ssc_rulebook_out_bound() rows; may be NULL);
+ *   ssc_rulebook_conv_finish is ssc_rulebook_finish followed by ssc_conv_plan_build for the
+ *     forward direction over the new pairs (pair_stride = n_in), into `plan` and `scratch`
+ *     sized for any number of rows from n_out up to the bound; where the rulebook dealt the
+ *     rows and the input rows came in key order, the plan needs three launches instead of six.
+ * Same host thread for both; one layer between them at a time.  The plan is the one
+ * ssc_conv_run_* expects; compared with ssc_conv_plan_build's the ranges begin at other
+ * rows, so results agree up to the order of the float sums. */
+int ssc_rulebook_conv_begin(const int32_t *indices, int64_t n_in, const ssc_geometry *g,
+                            void *workspace, size_t workspace_bytes,
+                            int32_t *pairs /* [K,2,n_in] */, int32_t *pair_num /* [K] */,
+                            int32_t *out_indices /* [out_capacity,4] or NULL */,
+                            int64_t out_capacity, void *clean_table, size_t clean_table_bytes,
+                            int32_t c_in, int32_t c_out, int32_t elem_bytes, void *scratch,
+                            size_t scratch_bytes, ssc_stream_t stream);
+int ssc_rulebook_conv_finish(const ssc_geometry *g, int64_t n_in, int32_t *n_out_host /* host */,
+                             int32_t *in_order_host /* host */, const int32_t *pairs,
+                             const int32_t *pair_num, int32_t c_in, int32_t c_out,
+                             int32_t elem_bytes, void *plan, size_t plan_bytes, void *scratch,
+                             size_t scratch_bytes, ssc_stream_t stream);
 
 /* ------------------------------------------------------------------------
  * Sparse convolution forward.  Replaces indiceConv<float>

@@ -81,42 +81,12 @@ __global__ void __launch_bounds__(kScanThreads)
   popc_blocksum_block(bits, n_words, blockIdx.x, blocksum, lds);
 }
 
-// Pass 2: exclusive prefix per word.  Every block first adds up the sums of the blocks
-// before it (at most 2^31 / 32 / kScanBlockWords = 32768 values), which saves the launch
-// of a scan over blocksum[]; the last block also writes the total.
+// Pass 2 (popc_prefix_block, ssc_common.h): exclusive prefix per word.
 __global__ void __launch_bounds__(kScanThreads)
     popc_prefix_kernel(const uint32_t *__restrict__ bits, int64_t n_words,
                        const int32_t *__restrict__ blocksum, int32_t *__restrict__ prefix,
                        int32_t *__restrict__ total, int32_t *__restrict__ mirror) {
-  __shared__ int lds[kScanThreads / 64 + 1];
-  int before = 0;
-  for (int64_t b = threadIdx.x; b < (int64_t)blockIdx.x; b += kScanThreads) before += blocksum[b];
-  int block_off;
-  block_exclusive_scan(before, lds, &block_off);
-  int64_t base = (int64_t)blockIdx.x * kScanBlockWords + (int64_t)threadIdx.x * kScanItems;
-  int c[kScanItems];
-  int v = 0;
-#pragma unroll
-  for (int i = 0; i < kScanItems; ++i) {
-    c[i] = base + i < n_words ? __popc(bits[base + i]) : 0;
-    v += c[i];
-  }
-  int tot;
-  int ex = block_exclusive_scan(v, lds, &tot) + block_off;
-#pragma unroll
-  for (int i = 0; i < kScanItems; ++i) {
-    if (base + i < n_words) prefix[base + i] = ex;
-    ex += c[i];
-  }
-  if (blockIdx.x == gridDim.x - 1 && threadIdx.x == 0) {
-    total[0] = block_off + tot;
-    if (mirror != nullptr) {  // total[1..3] were written by kernels before this one
-      mirror[0] = block_off + tot;
-      mirror[1] = total[1];
-      mirror[2] = total[2];
-      mirror[3] = total[3];
-    }
-  }
+  popc_prefix_block(bits, n_words, blocksum, prefix, total, mirror, blockIdx.x == gridDim.x - 1);
 }
 
 int bit_table_scan_prefix(const BitTable &t, hipStream_t s, int32_t *mirror) {

@@ -311,7 +311,6 @@ __global__ void __launch_bounds__(256)
 // ranges' work differed by 14 %)
 constexpr int kSplitGranule = 64, kSplitGranuleSmall = 16;
 constexpr int kTileSlack = 24;
-constexpr int kMaxRanges = 512;  // two for each of at most 256 workgroups
 // The accumulator window of a workgroup holds kSpillRows more rows than a tile is
 // high: the last row block that an offset contributes to a tile may then be filled
 // up with the offset's next pairs, whose rows lie in the following tile (at most
@@ -535,6 +534,184 @@ __global__ void __launch_bounds__(kMaxRanges)
       }
     }
   }
+}
+
+// The tiles and their segments in one launch, from range boundaries that are there already
+// (a rulebook placed them: SplitRequest) and from the pairs' side: a block takes a run of
+// kSegChunk consecutive pairs of one offset, whose scatter rows ascend.  Every block first
+// works out, in LDS, the rows and the first tile of every range (what split_rows_kernel
+// computes); a tile is then a function of its range and its number in it.  The run holds
+// the first pair at or beyond the first row of every tile whose first row lies in (row of
+// the pair before the run, row of the run's last pair]: for those tiles -- a handful -- a
+// thread each bisects the run's rows in LDS and writes segs[] and spill[] as
+// tile_segments_kernel does.  Block (0, 0) also writes the tables of the tiles for the
+// kernels that follow (wg_tile, tile_row0, spill_end, tile_slot0, n_tiles_dev) and clears
+// flag[0]: the pairs are in order.
+struct TileOf {
+  int t;       // tile
+  int row0;    // its first row
+  int spill;   // spill_end of the tile
+};
+__device__ __forceinline__ TileOf tile_of_row(int r, const int *row_s, const int *tile_s,
+                                              int n_rng, int T, int window) {
+  // the last range that begins at or before r (a range without rows is never the last such)
+  int lo = 0, hi = n_rng - 1;
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) >> 1;
+    if (row_s[mid] <= r) lo = mid;
+    else hi = mid - 1;
+  }
+  int nt, h;
+  range_tiles(row_s[lo + 1] - row_s[lo], T, window, &nt, &h);
+  int j = h > 0 ? (r - row_s[lo]) / h : 0;
+  if (j > nt - 1) j = nt - 1;
+  if (j < 0) j = 0;
+  TileOf o;
+  o.t = tile_s[lo] + j;
+  o.row0 = row_s[lo] + j * h;
+  o.spill = j == 0 ? o.row0 : min(o.row0 + window - h, row_s[lo + 1]);
+  return o;
+}
+
+// Tile t by its number: the range that holds it, then as above.
+__device__ __forceinline__ TileOf tile_by_index(int t, const int *row_s, const int *tile_s,
+                                                int n_rng, int T, int window) {
+  int lo = 0, hi = n_rng - 1;  // the last range whose first tile is at or before t
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) >> 1;
+    if (tile_s[mid] <= t) lo = mid;
+    else hi = mid - 1;
+  }
+  int nt, h;
+  range_tiles(row_s[lo + 1] - row_s[lo], T, window, &nt, &h);
+  const int j = t - tile_s[lo];
+  TileOf o;
+  o.t = t;
+  o.row0 = row_s[lo] + j * h;
+  o.spill = j == 0 ? o.row0 : min(o.row0 + window - h, row_s[lo + 1]);
+  return o;
+}
+
+constexpr int kSegChunk = 2048;  // pairs of one offset to a block
+__global__ void __launch_bounds__(256)
+    pair_tile_segments_kernel(int32_t *__restrict__ flag, const int32_t *__restrict__ pairs,
+                              int64_t pair_stride, int plane_s,
+                              const int32_t *__restrict__ pair_num, int K,
+                              const int32_t *__restrict__ range_row0, int n_rng, int T,
+                              int window, int n_out, int32_t *__restrict__ wg_tile, int32_t *__restrict__ tile_row0,
+                              int32_t *__restrict__ n_tiles_dev, int32_t *__restrict__ spill_end,
+                              int32_t *__restrict__ tile_slot0, int32_t *__restrict__ segs,
+                              int32_t *__restrict__ spill) {
+  __shared__ int row_s[kMaxRanges + 1];
+  __shared__ int tile_s[kMaxRanges + 1];
+  __shared__ int wave_sum[4];
+  // (the loads of the run's rows are issued first: they are not needed before the tables
+  // of the ranges stand)
+  const int k = blockIdx.y;
+  const int64_t j0 = (int64_t)blockIdx.x * kSegChunk;
+  const int32_t *s = pairs + ((int64_t)k * 2 + plane_s) * pair_stride;
+  constexpr int kPer = (kSegChunk + 15 + 255) / 256;
+  int held[kPer];
+#pragma unroll
+  for (int u = 0; u < kPer; ++u) {
+    const int64_t idx = j0 + threadIdx.x + 256 * u;
+    held[u] = idx < pair_stride ? s[idx] : 0x7FFFFFFF;
+  }
+  const int r_before = j0 > 0 && j0 <= pair_stride ? s[j0 - 1] : -1;
+  const int n = pair_num[k];
+  // rows and tile counts of the ranges: two ranges to a thread (n_rng <= 512)
+  for (int w = threadIdx.x; w <= n_rng; w += 256) {
+    int r = range_row0[w];
+    if (w == 0) r = 0;
+    if (w == n_rng) r = n_out;
+    row_s[w] = r;
+  }
+  __syncthreads();
+  {
+    const int w0 = 2 * threadIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    int nt0 = 0, nt1 = 0, h_unused = 0;
+    if (w0 < n_rng) range_tiles(row_s[w0 + 1] - row_s[w0], T, window, &nt0, &h_unused);
+    if (w0 + 1 < n_rng) range_tiles(row_s[w0 + 2] - row_s[w0 + 1], T, window, &nt1, &h_unused);
+    const int v = nt0 + nt1;
+    int incl = v;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      int o = __shfl_up(incl, d, 64);
+      if (lane >= d) incl += o;
+    }
+    if (lane == 63) wave_sum[wave] = incl;
+    __syncthreads();
+    int before = 0;
+    for (int i = 0; i < wave; ++i) before += wave_sum[i];
+    const int ex = before + incl - v;
+    if (w0 <= n_rng) tile_s[w0] = ex;
+    if (w0 + 1 <= n_rng) tile_s[w0 + 1] = ex + nt0;
+    if (w0 + 2 == n_rng) tile_s[n_rng] = ex + v;  // (512 ranges: no thread has w0 = n_rng)
+    __syncthreads();
+  }
+  const int n_tiles = tile_s[n_rng];
+  if (blockIdx.x == 0 && blockIdx.y == 0) {
+    if (threadIdx.x == 0) {
+      flag[0] = 0;
+      n_tiles_dev[0] = n_tiles;
+      tile_row0[n_tiles] = n_out;
+      spill_end[n_tiles] = n_out;
+    }
+    for (int w = threadIdx.x; w <= n_rng; w += 256) {
+      wg_tile[w] = tile_s[w];
+      if (w == n_rng) break;
+      int nt = 0, h = 0;
+      range_tiles(row_s[w + 1] - row_s[w], T, window, &nt, &h);
+      for (int j = 0; j < nt; ++j) {
+        const int r = row_s[w] + j * h;
+        tile_row0[tile_s[w] + j] = r;
+        spill_end[tile_s[w] + j] = j == 0 ? r : min(r + window - h, row_s[w + 1]);
+        tile_slot0[tile_s[w] + j] = (j * h) % window;
+      }
+    }
+  }
+  // the block's run of the offset's pairs: their rows (and those of the 15 pairs behind
+  // them, for the spill) in LDS
+  __shared__ int rows[kSegChunk + 16];
+  if (n == 0) {  // no pair: every tile's segment is empty
+    if (blockIdx.x == 0)
+      for (int t = threadIdx.x; t <= n_tiles; t += 256) {
+        segs[(int64_t)t * K + k] = 0;
+        spill[(int64_t)t * K + k] = 0;
+      }
+    return;
+  }
+  if (j0 >= n) return;
+  const int cnt = n - j0 < kSegChunk ? (int)(n - j0) : kSegChunk;
+#pragma unroll
+  for (int u = 0; u < kPer; ++u) {
+    const int i = threadIdx.x + 256 * u;
+    if (i < kSegChunk + 15) rows[i] = j0 + i < n ? held[u] : 0x7FFFFFFF;
+  }
+  const int r_prev = r_before;
+  __syncthreads();
+  // the tiles whose first row lies in (row of the pair before the run, row of its last pair]
+  const int t_lo = j0 > 0 ? tile_of_row(r_prev, row_s, tile_s, n_rng, T, window).t + 1 : 0;
+  const int t_hi = tile_of_row(rows[cnt - 1], row_s, tile_s, n_rng, T, window).t;
+  for (int t = t_lo + threadIdx.x; t <= t_hi; t += 256) {
+    const TileOf tl = tile_by_index(t, row_s, tile_s, n_rng, T, window);
+    int lo = 0, hi = cnt - 1;  // the first pair of the run at or beyond the tile's first row
+    while (lo < hi) {
+      const int mid = (lo + hi) >> 1;
+      if (rows[mid] < tl.row0) lo = mid + 1;
+      else hi = mid;
+    }
+    int beyond = 0;
+#pragma unroll
+    for (int q = 0; q < 15; ++q) beyond += rows[lo + q] < tl.spill ? 1 : 0;  // rows ascend
+    segs[(int64_t)t * K + k] = (int32_t)(j0 + lo);
+    spill[(int64_t)t * K + k] = (int32_t)(j0 + lo + beyond);
+  }
+  if (j0 + cnt == n)  // the offset's last run: tiles beyond its last pair
+    for (int t = t_hi + 1 + threadIdx.x; t <= n_tiles; t += 256) {
+      segs[(int64_t)t * K + k] = n;
+      spill[(int64_t)t * K + k] = n;
+    }
 }
 
 // ---- row-block schedule -----------------------------------------------------------------
@@ -972,11 +1149,22 @@ static size_t conv_plan_walk(void *base, const ConvPlan &p, ConvWs *w) {
   return c.used;
 }
 
+// The head of the scratch buffer, whose layout does not depend on the plan: flag and
+// range_row0 (a rulebook that places the range boundaries itself writes them before the
+// number of output rows, and with it the plan, is known).
+static size_t conv_scratch_head(void *base, ConvWs *w) {
+  Carver c(base);
+  w->flag = c.take<int32_t>(1);
+  w->range_row0 = c.take<int32_t>((size_t)kMaxRanges + 1);
+  return c.used;
+}
+
 static size_t conv_scratch_walk(void *base, const ConvPlan &p, int K, int64_t pair_stride,
                                 ConvWs *w) {
   Carver c(base);
   ConvWs t;
   t.flag = c.take<int32_t>(1);
+  t.range_row0 = c.take<int32_t>((size_t)kMaxRanges + 1);
   t.segs = c.take<int32_t>((size_t)(p.n_tiles + 1) * K);
   t.sorted = c.take<int32_t>((size_t)K * 2 * pair_stride);
   t.bits = c.take<uint32_t>((size_t)K * p.words_per_k);
@@ -985,7 +1173,6 @@ static size_t conv_scratch_walk(void *base, const ConvPlan &p, int K, int64_t pa
   t.tile_nmb = c.take<int32_t>((size_t)p.n_tiles);
   t.kofs = c.take<int32_t>((size_t)p.n_tiles * K);
   t.fine_segs = c.take<int32_t>((size_t)(p.n_fine + 1) * K);
-  t.range_row0 = c.take<int32_t>((size_t)p.n_rng + 1);
   t.tile_row0 = c.take<int32_t>((size_t)p.n_tiles + 1);
   t.spill_end = c.take<int32_t>((size_t)p.n_tiles + 1);
   t.tile_slot0 = c.take<int32_t>((size_t)p.n_tiles + 1);
@@ -1186,13 +1373,30 @@ template <typename PACK_IO>
 static int conv_plan_build(const ConvPlan &p, const ConvWs &w, const int32_t *pairs,
                            int64_t pair_stride, const int32_t *pair_num, int K, int inverse,
                            bool in_order, int c_in, int64_t n_out, int elem_bytes,
-                           const PackArgs *pack, hipStream_t s) {
+                           const PackArgs *pack, hipStream_t s, bool seeded = false) {
   const int plane_g = inverse ? 1 : 0;
   const int plane_s = 1 - plane_g;
+  if (seeded) {
+    // The range boundaries are in w.range_row0 already (a rulebook placed them, see
+    // SplitRequest): the tiles and their segments in one launch from the pairs' side, then
+    // the schedule.  For pairs in order, plans without a second split and nothing to pack.
+    SSC_CHECK(in_order && !p.rebalance && pack == nullptr, SSC_ERUNTIME,
+              "a seeded plan needs pairs in order and a single work split");
+    hipLaunchKernelGGL(pair_tile_segments_kernel,
+                       dim3((unsigned)ceil_div(pair_stride, kSegChunk), (unsigned)K), dim3(256), 0, s,
+                       w.flag, pairs, pair_stride, plane_s, pair_num, K, w.range_row0, p.n_rng,
+                       p.tile_rows, p.T, (int)n_out, w.wg_tile, w.tile_row0, w.n_tiles_dev,
+                       w.spill_end, w.tile_slot0, w.segs, w.spill);
+    SSC_LAUNCH_CHECK("pair_tile_segments");
+    hipLaunchKernelGGL(range_sched_kernel, dim3((unsigned)p.n_rng), dim3(kRangeSchedThreads), 0, s,
+                       w.segs, w.spill, K, w.wg_tile, w.share_first, w.share_cnt, w.kofs,
+                       w.tile_nmb, w.tile_loc, w.tile_rng, w.range_grp);
+    SSC_LAUNCH_CHECK("range_sched");
+  }
   const int64_t packed_n = pack ? (int64_t)K * p.ncb * p.nch * 1024 : 0;
   PackArgs pk = {nullptr, 0, 0, 0, 0, 0, 0, 0, 0, nullptr, 16};
   if (pack) pk = *pack;
-  if (!in_order) {  // otherwise the filters are packed beside the first kernel of the split
+  if (!in_order && !seeded) {  // otherwise the filters are packed beside the first kernel of the split
     if (pack) {
       hipLaunchKernelGGL(pack_filters_kernel<PACK_IO>, dim3((unsigned)ceil_div(packed_n, 256)),
                          dim3(256), 0, s, pk, w.flag);
@@ -1204,7 +1408,7 @@ static int conv_plan_build(const ConvPlan &p, const ConvWs &w, const int32_t *pa
   }
 
   dim3 pair_grid((unsigned)ceil_div(pair_stride, 256), (unsigned)K);
-  if (!in_order) {  // otherwise flag[0] is 0: pairs in order
+  if (!in_order && !seeded) {  // otherwise flag[0] is 0: pairs in order
     hipLaunchKernelGGL(check_sorted_kernel, pair_grid, dim3(256), 0, s, pairs, pair_stride, plane_s,
                        pair_num, w.flag);
     SSC_LAUNCH_CHECK("check_sorted");
@@ -1228,11 +1432,14 @@ static int conv_plan_build(const ConvPlan &p, const ConvWs &w, const int32_t *pa
     int64_t rows = ceil_div(ceil_div(packed_n > 0 ? packed_n : 1, 256), pair_grid.x);
     seg_grid.y += (unsigned)(rows < 4096 ? rows : 4096);
   }
-  hipLaunchKernelGGL(grid_segments_kernel<PACK_IO>, seg_grid, dim3(256), 0, s, w.flag,
-                     in_order ? 1 : 0, pairs, w.sorted, pair_stride, plane_s, pair_num, K, p.n_fine,
-                     p.granule, w.fine_segs, pk);
-  hipLaunchKernelGGL(split_bounds_kernel, dim3((unsigned)ceil_div(p.n_fine + 1, 256)), dim3(256), 0,
-                     s, w.fine_segs, K, p.n_fine, n_out, p.tile_rows, p.n_rng, p.granule, w.range_row0);
+  if (!seeded) {
+    hipLaunchKernelGGL(grid_segments_kernel<PACK_IO>, seg_grid, dim3(256), 0, s, w.flag,
+                       in_order ? 1 : 0, pairs, w.sorted, pair_stride, plane_s, pair_num, K,
+                       p.n_fine, p.granule, w.fine_segs, pk);
+    hipLaunchKernelGGL(split_bounds_kernel, dim3((unsigned)ceil_div(p.n_fine + 1, 256)), dim3(256),
+                       0, s, w.fine_segs, K, p.n_fine, n_out, p.tile_rows, p.n_rng, p.granule,
+                       w.range_row0);
+  }
   // the ranges' tiles, their segments, shares and row-block counts
   const int64_t nseg = (p.n_tiles + 1) * K;
   auto tiles_of = [&](const int32_t *range_row0) -> int {
@@ -1251,7 +1458,7 @@ static int conv_plan_build(const ConvPlan &p, const ConvWs &w, const int32_t *pa
     SSC_LAUNCH_CHECK("range_sched");
     return SSC_OK;
   };
-  int rc = tiles_of(w.range_row0);
+  int rc = seeded ? SSC_OK : tiles_of(w.range_row0);
   if (rc != SSC_OK) return rc;
   if (p.rebalance) {  // long kernels: once more, from the groups the ranges came to
     hipLaunchKernelGGL(split_rebalance_kernel, dim3((unsigned)ceil_div(p.n_fine + 1, 256)),
@@ -1534,6 +1741,83 @@ int ssc_conv_plan_build(const int32_t *pairs, int64_t pair_stride, const int32_t
   return conv_plan_build<float>(p, w, pairs, pair_stride, pair_num, K, inverse,
                                 (flags & SSC_CONV_PAIRS_CANONICAL) != 0, c_in, n_out, elem_bytes,
                                 nullptr, (hipStream_t)stream);
+}
+
+// A rulebook between ssc_rulebook_conv_begin and ssc_rulebook_conv_finish on this host thread:
+// whether the rulebook was asked to place the range boundaries, and for how many ranges.
+struct PendingLayer {
+  bool seeded = false;
+  int n_rng = 0;
+};
+static thread_local PendingLayer g_pending_layer;
+
+int ssc_rulebook_conv_begin(const int32_t *indices, int64_t n_in, const ssc_geometry *g,
+                            void *workspace, size_t workspace_bytes, int32_t *pairs,
+                            int32_t *pair_num, int32_t *out_indices, int64_t out_capacity,
+                            void *clean_table, size_t clean_table_bytes, int32_t c_in,
+                            int32_t c_out, int32_t elem_bytes, void *scratch,
+                            size_t scratch_bytes, ssc_stream_t stream) {
+  g_pending_layer = PendingLayer();
+  SSC_CHECK(g != nullptr, SSC_EINVAL, "geometry is NULL");
+  SSC_CHECK(c_in >= 1 && c_out >= 1, SSC_EINVAL, "channel counts must be positive");
+  SSC_CHECK(elem_bytes == 4 || elem_bytes == 2, SSC_EINVAL, "elem_bytes must be 4 or 2");
+  SplitRequest rq = {0, 0, 0, nullptr};
+  const SplitRequest *ask = nullptr;
+  int64_t K = 1;
+  for (int a = 0; a < 3; ++a) K *= g->ksize[a] > 0 ? g->ksize[a] : 1;
+  if (scratch != nullptr && n_in > 0 && K <= SSC_MAX_KERNEL_VOLUME && !g->subm && !g->transpose) {
+    // what the plan will look like when the outputs outnumber the inputs, as they do for
+    // the geometries whose rulebook can place the boundaries (stride 1, a padded kernel)
+    const ConvPlan p = make_plan(n_in, n_in + 1, (int)K, c_in, c_out, n_in, elem_bytes);
+    ConvWs w = {};
+    const size_t head = conv_scratch_head(scratch, &w);
+    if (!p.rebalance && scratch_bytes >= head) {
+      rq.n_rng = p.n_rng;
+      rq.tile_rows = p.tile_rows;
+      rq.tile_cost = (long long)K * 4 + 64;  // split_tile_cost
+      rq.range_row0 = w.range_row0;
+      ask = &rq;
+    }
+  }
+  bool seeded = false;
+  int rc = rulebook_begin_impl(indices, n_in, g, workspace, workspace_bytes, pairs, pair_num,
+                               out_indices, out_capacity, clean_table, clean_table_bytes, ask,
+                               &seeded, (hipStream_t)stream);
+  if (rc != SSC_OK) return rc;
+  g_pending_layer.seeded = seeded;
+  g_pending_layer.n_rng = rq.n_rng;
+  return SSC_OK;
+}
+
+int ssc_rulebook_conv_finish(const ssc_geometry *g, int64_t n_in, int32_t *n_out_host,
+                             int32_t *in_order_host, const int32_t *pairs,
+                             const int32_t *pair_num, int32_t c_in, int32_t c_out,
+                             int32_t elem_bytes, void *plan, size_t plan_bytes, void *scratch,
+                             size_t scratch_bytes, ssc_stream_t stream) {
+  const PendingLayer pending = g_pending_layer;
+  g_pending_layer = PendingLayer();
+  int rc = ssc_rulebook_finish(g, n_in, n_out_host, in_order_host);
+  if (rc != SSC_OK) return rc;
+  const int64_t n_out = *n_out_host;
+  int K = 1;
+  for (int a = 0; a < 3; ++a) K *= g->ksize[a];
+  rc = conv_check_sizes(K, c_in, c_out, n_in, n_out, n_in);
+  if (rc != SSC_OK) return rc;
+  SSC_CHECK(elem_bytes == 4 || elem_bytes == 2, SSC_EINVAL, "elem_bytes must be 4 or 2");
+  if (n_out == 0 || n_in == 0) return SSC_OK;  // nothing to schedule
+  SSC_CHECK(pairs && pair_num && plan && scratch, SSC_EINVAL, "NULL pointer argument");
+  const ConvPlan p = make_plan(n_in, n_out, K, c_in, c_out, n_in, elem_bytes);
+  SSC_CHECK(plan_bytes >= conv_plan_walk(nullptr, p, nullptr), SSC_EWORKSPACE,
+            "plan buffer too small");
+  SSC_CHECK(scratch_bytes >= conv_scratch_walk(nullptr, p, K, n_in, nullptr), SSC_EWORKSPACE,
+            "plan scratch too small");
+  ConvWs w = {};
+  conv_plan_walk(plan, p, &w);
+  conv_scratch_walk(scratch, p, K, n_in, &w);
+  const bool in_order = *in_order_host != 0;
+  const bool seeded = pending.seeded && in_order && !p.rebalance && pending.n_rng == p.n_rng;
+  return conv_plan_build<float>(p, w, pairs, n_in, pair_num, K, 0, in_order, c_in, n_out,
+                                elem_bytes, nullptr, (hipStream_t)stream, seeded);
 }
 
 int ssc_kernel_combine_packed_f32(const float *weight, const float *basis,

@@ -363,12 +363,19 @@ __global__ void __launch_bounds__(kScanThreads)
 // (kx, ky) of the bits 32 zw + kz .. + 31, for every kz, of input row (b, x + kx, y + ky).
 // KS > 0: the kernel's three extents equal KS (loops unrolled, all
 // loads of a thread in flight at once); KS = 0: any extents.
-template <int KS>
+// SEED: the kernel also leaves, for every word, the output rows and the pairs that lie in
+// the words of its scan block before it (seed_rows[], seed_pairs[]), and the block's pairs
+// (pairsum[]): the work measure of the convolution's plan (see SplitRequest).  The pairs
+// that land on the outputs of a word are the set input bits over all taps -- the popcounts of
+// the same shifted words the OR is taken of.
+template <int KS, bool SEED>
 __global__ void __launch_bounds__(kScanThreads)
     dilate_blocksum_kernel(const uint32_t *__restrict__ in_bits, Geom g, DenseIn d,
                            uint32_t *__restrict__ bits, int64_t n_words, int64_t n_word_blocks,
                            int32_t *__restrict__ blocksum, int32_t *__restrict__ chunk_count,
-                           int64_t n_chunks, int32_t *__restrict__ pair_num) {
+                           int64_t n_chunks, int32_t *__restrict__ pair_num,
+                           int32_t *__restrict__ seed_rows, int32_t *__restrict__ seed_pairs,
+                           int32_t *__restrict__ pairsum) {
   if ((int64_t)blockIdx.x >= n_word_blocks) {
     __shared__ int lds[kScanThreads / 64 + 1];
     scan_chunks_of_tap(chunk_count, n_chunks, (int)(blockIdx.x - n_word_blocks), pair_num, lds);
@@ -382,10 +389,19 @@ __global__ void __launch_bounds__(kScanThreads)
   const uint32_t zw_n = (uint32_t)g.os[2] >> 5;  // words per output row
   const int64_t xstep = (int64_t)d.U[1] * d.Wz;
   int v = 0;
+  __shared__ int word_rows[SEED ? kScanBlockWords : 1], word_pairs[SEED ? kScanBlockWords : 1];
 #pragma unroll 2
   for (int it = 0; it < kScanItems; ++it) {
     const int64_t w = (int64_t)blockIdx.x * kScanBlockWords + it * kScanThreads + threadIdx.x;
-    if (w >= n_words) break;
+    if (w >= n_words) {
+      if constexpr (SEED) {
+        word_rows[it * kScanThreads + threadIdx.x] = 0;
+        word_pairs[it * kScanThreads + threadIdx.x] = 0;
+        continue;
+      } else {
+        break;
+      }
+    }
     uint32_t t = (uint32_t)w;  // (fewer than 2^26 words)
     const int zw = (int)(t % zw_n);
     t /= zw_n;
@@ -395,6 +411,7 @@ __global__ void __launch_bounds__(kScanThreads)
     const int b = (int)(t / (uint32_t)g.os[0]);
     const uint32_t *rowp = in_bits + (((int64_t)b * d.U[0] + x) * d.U[1] + y) * d.Wz + zw;
     uint32_t out = 0u;
+    int landing = 0;
 #pragma unroll
     for (int kx = 0; kx < ksx; ++kx) {
 #pragma unroll
@@ -403,13 +420,55 @@ __global__ void __launch_bounds__(kScanThreads)
         // (with ksz > 1, Wz > os[2] / 32: word zw + 1 exists)
         const uint32_t lo = p[0], hi = ksz > 1 ? p[1] : 0u;
         uint32_t acc = lo;
+        if constexpr (SEED) landing += __popc(lo);
 #pragma unroll
-        for (int kz = 1; kz < ksz; ++kz) acc |= (lo >> kz) | (hi << (32 - kz));
+        for (int kz = 1; kz < ksz; ++kz) {
+          const uint32_t shifted = (lo >> kz) | (hi << (32 - kz));
+          acc |= shifted;
+          if constexpr (SEED) landing += __popc(shifted);
+        }
         out |= acc;
       }
     }
     bits[w] = out;
     v += __popc(out);
+    if constexpr (SEED) {
+      word_rows[it * kScanThreads + threadIdx.x] = __popc(out);
+      word_pairs[it * kScanThreads + threadIdx.x] = landing;
+    }
+  }
+  if constexpr (SEED) {
+    // prefixes over the block's words in their order: every thread takes kScanItems
+    // consecutive words
+    __shared__ int lds[kScanThreads / 64 + 1];
+    __syncthreads();
+    const int first = threadIdx.x * kScanItems;
+    int cr[kScanItems], cp[kScanItems], sr = 0, sp = 0;
+#pragma unroll
+    for (int i = 0; i < kScanItems; ++i) {
+      cr[i] = word_rows[first + i];
+      cp[i] = word_pairs[first + i];
+      sr += cr[i];
+      sp += cp[i];
+    }
+    int tot_r, tot_p;
+    int er = block_exclusive_scan(sr, lds, &tot_r);
+    int ep = block_exclusive_scan(sp, lds, &tot_p);
+    const int64_t w0 = (int64_t)blockIdx.x * kScanBlockWords + first;
+#pragma unroll
+    for (int i = 0; i < kScanItems; ++i) {
+      if (w0 + i < n_words) {
+        seed_rows[w0 + i] = er;
+        seed_pairs[w0 + i] = ep;
+      }
+      er += cr[i];
+      ep += cp[i];
+    }
+    if (threadIdx.x == 0) {
+      blocksum[blockIdx.x] = tot_r;
+      pairsum[blockIdx.x] = tot_p;
+    }
+    return;
   }
 #pragma unroll
   for (int s = 32; s >= 1; s >>= 1) v += __shfl_xor(v, s, 64);
@@ -423,6 +482,130 @@ __global__ void __launch_bounds__(kScanThreads)
     blocksum[blockIdx.x] = total;
   }
 }
+
+// The second pass of the table's scan (popc_prefix_block) and, in the blocks after the
+// table's, the placing of the range boundaries of a SplitRequest: 16 ranges to a block, 16
+// lanes to a range.  Range w begins at the first cell c (a word of the table) with
+//   work(c) = pairs below c * tile_rows + rows below c * tile_cost  >=  w / n_rng of the total,
+// its first row being the rows below c.  Every such block first adds up the block sums of
+// rows and pairs in LDS (at most kSeedMaxBlocks of each); a range's lanes then find the scan
+// block by bisection there and the cell inside it by three rounds of 16 probes.
+__global__ void __launch_bounds__(kScanThreads)
+    prefix_split_kernel(const uint32_t *__restrict__ bits, int64_t n_words, int64_t n_scan_blocks,
+                        const int32_t *__restrict__ blocksum, int32_t *__restrict__ prefix,
+                        int32_t *__restrict__ total, int32_t *__restrict__ mirror,
+                        const int32_t *__restrict__ pairsum,
+                        const int32_t *__restrict__ seed_rows,
+                        const int32_t *__restrict__ seed_pairs, SplitRequest rq) {
+  if ((int64_t)blockIdx.x < n_scan_blocks) {
+    popc_prefix_block(bits, n_words, blocksum, prefix, total, mirror,
+                      (int64_t)blockIdx.x == n_scan_blocks - 1);
+    return;
+  }
+  __shared__ int rows_base[kSeedMaxBlocks + 1];
+  __shared__ long long pairs_base[kSeedMaxBlocks + 1];
+  __shared__ int lds[kScanThreads / 64 + 1];
+  __shared__ long long wave_p[kScanThreads / 64];
+  const int nb = (int)n_scan_blocks;  // <= kSeedMaxBlocks
+  {
+    // exclusive prefixes of the block sums: every thread a run of consecutive blocks
+    constexpr int kPer = kSeedMaxBlocks / kScanThreads;
+    const int first = threadIdx.x * kPer;
+    int r[kPer], sr = 0;
+    long long pp[kPer], sp = 0;
+#pragma unroll
+    for (int i = 0; i < kPer; ++i) {
+      r[i] = first + i < nb ? blocksum[first + i] : 0;
+      pp[i] = first + i < nb ? (long long)pairsum[first + i] : 0;
+      sr += r[i];
+      sp += pp[i];
+    }
+    int tot_r;
+    int er = block_exclusive_scan(sr, lds, &tot_r);
+    // the pairs as 64-bit sums: scan inside the wave, then over the waves
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    long long incl = sp;
+#pragma unroll
+    for (int dd = 1; dd < 64; dd <<= 1) {
+      const long long o = __shfl_up(incl, dd, 64);
+      if (lane >= dd) incl += o;
+    }
+    if (lane == 63) wave_p[wave] = incl;
+    __syncthreads();
+    long long ep = incl - sp;
+    for (int i = 0; i < wave; ++i) ep += wave_p[i];
+#pragma unroll
+    for (int i = 0; i < kPer; ++i) {
+      if (first + i <= nb) {
+        rows_base[first + i] = er;
+        pairs_base[first + i] = ep;
+      }
+      er += r[i];
+      ep += pp[i];
+    }
+    if (threadIdx.x == kScanThreads - 1 && first + kPer <= nb) {  // nb == kSeedMaxBlocks
+      rows_base[nb] = er;
+      pairs_base[nb] = ep;
+    }
+    __syncthreads();
+  }
+  const long long n_out = rows_base[nb];
+  const long long T = rq.tile_rows, cost = rq.tile_cost;
+  const long long total_work = pairs_base[nb] * T + n_out * cost;
+  auto work_of_block = [&](int b) -> long long { return pairs_base[b] * T + rows_base[b] * cost; };
+  auto work_of_cell = [&](long long c) -> long long {
+    if (c >= n_words) return total_work;
+    const int b = (int)(c >> 11);  // kScanBlockWords = 2048 words to a scan block
+    return (pairs_base[b] + seed_pairs[c]) * T + ((long long)rows_base[b] + seed_rows[c]) * cost;
+  };
+  static_assert(kScanBlockWords == 2048, "the cell search assumes scan blocks of 2048 words");
+  const int sub = threadIdx.x & 15;
+  const int w = ((int)(blockIdx.x - n_scan_blocks) * (kScanThreads / 16)) + (threadIdx.x >> 4);
+  const bool mine = w >= 1 && w < rq.n_rng;
+  // ceil(total * w / n_rng); ranges without a target (w = 0, w >= n_rng) search for nothing
+  long long target = mine ? (total_work * w + rq.n_rng - 1) / rq.n_rng : 0;
+  // the scan block: the last one whose work before it is below the target
+  int lo_b = 0, hi_b = nb;  // work_of_block(lo_b) < target (or lo_b = 0) ; answer in block lo_b
+  while (hi_b - lo_b > 1) {
+    const int mid = (lo_b + hi_b) >> 1;
+    if (work_of_block(mid) < target) lo_b = mid;
+    else hi_b = mid;
+  }
+  long long lo = (long long)lo_b * kScanBlockWords;  // work(lo) < target <= work(lo + width),
+  int width = kScanBlockWords;                       // or the target is not positive
+  const int shift = (threadIdx.x & 63) & ~15;
+#pragma unroll
+  for (int round = 0; round < 3; ++round) {
+    const int stride = width >> 4;  // 128, 8, then single cells
+    const long long c = stride > 0 ? lo + (long long)stride * (sub + 1) : lo + sub + 1;
+    const bool reached = work_of_cell(c) >= target;
+    const unsigned hits = (unsigned)((__ballot(reached) >> shift) & 0xFFFFull);
+    // (the last probe of the first two rounds is lo + width, which reaches the target)
+    const int first = hits ? __ffs(hits) - 1 : 15;
+    if (stride > 0) {
+      lo += (long long)stride * first;
+      width = stride;
+    } else {
+      lo += first + 1;  // the cell itself
+      width = 0;
+    }
+  }
+  // after the rounds of 128 and 8 the third one probed the 8 cells lo + 1 .. lo + 8 (lanes
+  // 0..7; lanes 8..15 probe beyond and reach the target as well): lo is the first cell that
+  // reaches it
+  if (sub == 0) {
+    if (mine) {
+      long long c = target > 0 ? lo : 0;
+      if (c > n_words) c = n_words;
+      long long row = c >= n_words ? n_out
+                                   : (long long)rows_base[(int)(c >> 11)] + seed_rows[c];
+      rq.range_row0[w] = (int32_t)row;
+    } else if (w == 0) {
+      rq.range_row0[0] = 0;
+      rq.range_row0[rq.n_rng] = (int32_t)n_out;
+    }
+  }
+}
 template <int KS>
 __global__ void __launch_bounds__(256)
     write_pairs_kernel(const int32_t *__restrict__ indices, int64_t n_in, Geom g,
@@ -430,13 +613,18 @@ __global__ void __launch_bounds__(256)
                        const int32_t *__restrict__ rank2row,
                        const int32_t *__restrict__ chunk_prefix, int64_t n_chunks,
                        const int32_t *__restrict__ pair_num, int32_t *__restrict__ pairs,
-                       int64_t n_words, int32_t *__restrict__ out_indices) {
+                       int64_t n_words, int32_t *__restrict__ out_indices,
+                       uint32_t *__restrict__ clean, int64_t clean_words) {
   if ((int)blockIdx.y >= g.ks[0]) {
+    // the rows of the grid beyond the kernel's x extent: the output rows, and the words of
+    // a table that no kernel reads any more and the next call expects to find zero
     const int64_t step = (int64_t)(gridDim.y - g.ks[0]) * gridDim.x * blockDim.x;
-    int64_t w = ((int64_t)(blockIdx.y - g.ks[0]) * gridDim.x + blockIdx.x) * blockDim.x +
-                threadIdx.x;
-    for (; w < n_words; w += step)
-      emit_rows_of_word(bits, prefix, w, g.os[0], g.os[1], g.os[2], out_indices);
+    const int64_t w0 = ((int64_t)(blockIdx.y - g.ks[0]) * gridDim.x + blockIdx.x) * blockDim.x +
+                       threadIdx.x;
+    if (out_indices != nullptr)
+      for (int64_t w = w0; w < n_words; w += step)
+        emit_rows_of_word(bits, prefix, w, g.os[0], g.os[1], g.os[2], out_indices);
+    for (int64_t w = w0; w < clean_words; w += step) clean[w] = 0u;
     return;
   }
   int64_t chunk = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
@@ -535,7 +723,15 @@ struct RulebookWs {
   uint32_t *in_bits;     // input table of the dilation path (when it applies)
   DenseIn dense;
   bool use_dense;
+  // seed of a convolution's work split (dilation path, tables of at most kSeedMaxBlocks scan
+  // blocks): rows and pairs before every word inside its scan block, pairs of every block
+  bool can_seed;
+  int32_t *seed_rows, *seed_pairs, *pairsum;
 };
+
+static inline bool seed_applies(const Geom &g) {
+  return ceil_div(bit_words(geom_cells(g)), kScanBlockWords) <= kSeedMaxBlocks;
+}
 
 static size_t rulebook_ws_bytes(const Geom &g, int64_t n_in) {
   int64_t n_chunks = ceil_div(n_in > 0 ? n_in : 1, 64);
@@ -543,8 +739,22 @@ static size_t rulebook_ws_bytes(const Geom &g, int64_t n_in) {
   const size_t dense = dense_marking_applies(g, n_in, &d)
                            ? align_up((size_t)dense_in_words(g, d) * 4)
                            : 0;
+  const size_t seed = dense > 0 && seed_applies(g)
+                          ? 2 * align_up((size_t)bit_words(geom_cells(g)) * 4) +
+                                align_up((size_t)(kSeedMaxBlocks + 1) * 4)
+                          : 0;
   return bit_table_bytes(geom_cells(g)) + align_up((size_t)g.K * n_chunks * 4) +
-         align_up((size_t)(n_in > 0 ? n_in : 1) * 4) + dense;
+         align_up((size_t)(n_in > 0 ? n_in : 1) * 4) + dense + seed;
+}
+
+// Bytes of the table a caller may keep between calls (ssc_rulebook_clean_table_bytes): a
+// header of 256 bytes that holds the table's totals and flags, then the input table of the
+// dilation path.  0 when the geometry does not take that path.
+constexpr size_t kCleanHeader = 256;
+static size_t rulebook_clean_bytes(const Geom &g, int64_t n_in) {
+  DenseIn d;
+  if (n_in <= 0 || !dense_marking_applies(g, n_in, &d)) return 0;
+  return kCleanHeader + align_up((size_t)dense_in_words(g, d) * 4);
 }
 
 static RulebookWs rulebook_ws_carve(void *ws, const Geom &g, int64_t n_in) {
@@ -556,6 +766,13 @@ static RulebookWs rulebook_ws_carve(void *ws, const Geom &g, int64_t n_in) {
   w.rank2row = c.take<int32_t>(n_in > 0 ? n_in : 1);
   w.use_dense = dense_marking_applies(g, n_in, &w.dense);
   w.in_bits = w.use_dense ? c.take<uint32_t>((size_t)dense_in_words(g, w.dense)) : nullptr;
+  w.can_seed = w.use_dense && seed_applies(g);
+  w.seed_rows = w.seed_pairs = w.pairsum = nullptr;
+  if (w.can_seed) {
+    w.seed_rows = c.take<int32_t>((size_t)w.table.n_words);
+    w.seed_pairs = c.take<int32_t>((size_t)w.table.n_words);
+    w.pairsum = c.take<int32_t>((size_t)kSeedMaxBlocks + 1);
+  }
   return w;
 }
 
@@ -585,14 +802,16 @@ static int rulebook_check(const ssc_geometry *g, Geom *gg, const int32_t *indice
 // rulebook_pairs must be told so).
 static int rulebook_mark_and_scan(const int32_t *indices, int64_t n_in, const Geom &gg,
                                   const RulebookWs &w, int32_t *pair_num, int32_t *mirror,
-                                  hipStream_t s) {
+                                  hipStream_t s, const SplitRequest *split = nullptr,
+                                  bool table_is_clean = false) {
   int rc;
   if (w.use_dense && pair_num != nullptr) {
-    // input table cleared (with the totals), inputs marked, outputs by dilation
+    // input table cleared (with the totals) unless the caller keeps one that every call
+    // leaves clean, inputs marked, outputs by dilation
     BitTable in = w.table;
     in.bits = w.in_bits;
     in.n_words = dense_in_words(gg, w.dense);
-    if ((rc = bit_table_clear(in, s, true)) != SSC_OK) return rc;
+    if (!table_is_clean && (rc = bit_table_clear(in, s, true)) != SSC_OK) return rc;
     hipLaunchKernelGGL(mark_in_count_kernel,
                        dim3((unsigned)ceil_div(w.n_chunks, 4), (unsigned)gg.ks[0]), dim3(256), 0, s,
                        indices, n_in, gg, w.dense, w.in_bits, w.chunk_count, w.n_chunks,
@@ -600,13 +819,27 @@ static int rulebook_mark_and_scan(const int32_t *indices, int64_t n_in, const Ge
     SSC_LAUNCH_CHECK("mark_in_count");
     const int64_t word_blocks = w.table.n_scan_blocks;
     const int ks = (gg.ks[0] == gg.ks[1] && gg.ks[1] == gg.ks[2]) ? gg.ks[0] : 0;
-    auto kernel = ks == 3 ? dilate_blocksum_kernel<3> : ks == 5 ? dilate_blocksum_kernel<5>
-                                                                : dilate_blocksum_kernel<0>;
+    const bool seed = split != nullptr && w.can_seed;
+    auto kernel = seed ? (ks == 3   ? dilate_blocksum_kernel<3, true>
+                          : ks == 5 ? dilate_blocksum_kernel<5, true>
+                                    : dilate_blocksum_kernel<0, true>)
+                       : (ks == 3   ? dilate_blocksum_kernel<3, false>
+                          : ks == 5 ? dilate_blocksum_kernel<5, false>
+                                    : dilate_blocksum_kernel<0, false>);
     hipLaunchKernelGGL(kernel, dim3((unsigned)(word_blocks + gg.K)), dim3(kScanThreads), 0, s,
                        w.in_bits, gg, w.dense, w.table.bits, w.table.n_words, word_blocks,
-                       w.table.blocksum, w.chunk_count, w.n_chunks, pair_num);
+                       w.table.blocksum, w.chunk_count, w.n_chunks, pair_num, w.seed_rows,
+                       w.seed_pairs, w.pairsum);
     SSC_LAUNCH_CHECK("dilate_blocksum");
-    return bit_table_scan_prefix(w.table, s, mirror);
+    if (!seed) return bit_table_scan_prefix(w.table, s, mirror);
+    // the scan's second pass, and beside it the range boundaries of the convolution's plan
+    const int64_t split_blocks = ceil_div(split->n_rng, kScanThreads / 16);
+    hipLaunchKernelGGL(prefix_split_kernel, dim3((unsigned)(word_blocks + split_blocks)),
+                       dim3(kScanThreads), 0, s, w.table.bits, w.table.n_words, word_blocks,
+                       w.table.blocksum, w.table.prefix, w.table.total, mirror, w.pairsum,
+                       w.seed_rows, w.seed_pairs, *split);
+    SSC_LAUNCH_CHECK("prefix_split");
+    return SSC_OK;
   }
   if ((rc = bit_table_clear(w.table, s)) != SSC_OK) return rc;
   if (gg.subm) {
@@ -632,7 +865,8 @@ static int rulebook_mark_and_scan(const int32_t *indices, int64_t n_in, const Ge
 // chunks_scanned: rulebook_mark_and_scan has scanned the chunk counts already.
 static int rulebook_pairs(const int32_t *indices, int64_t n_in, const Geom &gg,
                           const RulebookWs &w, int32_t *out_indices, int32_t *pairs,
-                          int32_t *pair_num, bool chunks_scanned, hipStream_t s) {
+                          int32_t *pair_num, bool chunks_scanned, hipStream_t s,
+                          uint32_t *clean = nullptr, int64_t clean_words = 0) {
   unsigned chunk_blocks = (unsigned)ceil_div(w.n_chunks, 4);
   if (gg.subm) {  // a regular convolution's counts were taken while marking the table
     hipLaunchKernelGGL(rank_to_row_kernel, dim3((unsigned)ceil_div(n_in, 256)), dim3(256), 0, s,
@@ -651,13 +885,18 @@ static int rulebook_pairs(const int32_t *indices, int64_t n_in, const Geom &gg,
   int64_t row_blocks = (gg.subm || out_indices == nullptr)
                            ? 0
                            : ceil_div(ceil_div(w.table.n_words, 256), chunk_blocks);
+  if (clean != nullptr) {
+    const int64_t clean_blocks = ceil_div(ceil_div(clean_words, 256), chunk_blocks);
+    if (clean_blocks > row_blocks) row_blocks = clean_blocks;
+  }
   if (row_blocks > 4096) row_blocks = 4096;
   const int ks = gg.ks[1] == gg.ks[2] ? gg.ks[1] : 0;
   auto kernel = ks == 3 ? write_pairs_kernel<3> : ks == 5 ? write_pairs_kernel<5>
                 : ks == 2 ? write_pairs_kernel<2> : write_pairs_kernel<0>;
   hipLaunchKernelGGL(kernel, dim3(chunk_blocks, (unsigned)(gg.ks[0] + row_blocks)), dim3(256), 0,
                      s, indices, n_in, gg, w.table.bits, w.table.prefix, w.rank2row, w.chunk_count,
-                     w.n_chunks, pair_num, pairs, w.table.n_words, out_indices);
+                     w.n_chunks, pair_num, pairs, w.table.n_words,
+                     gg.subm ? (int32_t *)nullptr : out_indices, clean, clean_words);
   SSC_LAUNCH_CHECK("write_pairs");
   return SSC_OK;
 }
@@ -738,13 +977,32 @@ size_t ssc_rulebook_out_bound(const ssc_geometry *g, int64_t n_in) {
   return (size_t)rulebook_out_bound(gg, n_in);
 }
 
+size_t ssc_rulebook_clean_table_bytes(const ssc_geometry *g, int64_t n_in) {
+  Geom gg;
+  if (n_in < 0 || make_geom(g, &gg) != SSC_OK) return 0;
+  return rulebook_clean_bytes(gg, n_in);
+}
+
 int ssc_rulebook_begin(const int32_t *indices, int64_t n_in, const ssc_geometry *g,
                        void *workspace, size_t workspace_bytes, int32_t *pairs, int32_t *pair_num,
-                       int32_t *out_indices, int64_t out_capacity, ssc_stream_t stream) {
+                       int32_t *out_indices, int64_t out_capacity, void *clean_table,
+                       size_t clean_table_bytes, ssc_stream_t stream) {
+  bool seeded = false;
+  return ssc::rulebook_begin_impl(indices, n_in, g, workspace, workspace_bytes, pairs, pair_num,
+                                  out_indices, out_capacity, clean_table, clean_table_bytes,
+                                  nullptr, &seeded, (hipStream_t)stream);
+}
+}  // extern "C"
+
+int ssc::rulebook_begin_impl(const int32_t *indices, int64_t n_in, const ssc_geometry *g,
+                             void *workspace, size_t workspace_bytes, int32_t *pairs,
+                             int32_t *pair_num, int32_t *out_indices, int64_t out_capacity,
+                             void *clean_table, size_t clean_table_bytes,
+                             const SplitRequest *split, bool *seeded, hipStream_t s) {
   Geom gg;
+  *seeded = false;
   int rc = rulebook_check(g, &gg, indices, n_in, workspace, workspace_bytes);
   if (rc != SSC_OK) return rc;
-  hipStream_t s = (hipStream_t)stream;
   SSC_CHECK(pair_num != nullptr, SSC_EINVAL, "pair_num is NULL");
   if (n_in == 0) return fill_i32(pair_num, gg.K, 0, s);
   SSC_CHECK(pairs != nullptr, SSC_EINVAL, "pairs is NULL");
@@ -757,10 +1015,32 @@ int ssc_rulebook_begin(const int32_t *indices, int64_t n_in, const ssc_geometry 
   // sizes do not depend on the totals, are computed while the host wakes up
   int32_t *mirror = nullptr;
   if ((rc = read_back_mirror(&mirror)) != SSC_OK) return rc;
-  if ((rc = rulebook_mark_and_scan(indices, n_in, gg, w, pair_num, mirror, s)) != SSC_OK) return rc;
+  if (split != nullptr && !(w.can_seed && split->n_rng >= 1 && split->n_rng <= kMaxRanges &&
+                            split->range_row0 != nullptr))
+    split = nullptr;
+  *seeded = split != nullptr;
+  // A table the caller keeps between calls: all zero now, and all zero again when the
+  // kernels queued here are done (the launch of the pair lists clears it: by then nothing
+  // reads it any more).  It holds the input table of the dilation path behind a header with
+  // the totals and flags, and saves the launch that would clear them.
+  uint32_t *clean = nullptr;
+  int64_t clean_words = 0;
+  const size_t clean_need = rulebook_clean_bytes(gg, n_in);
+  if (clean_table != nullptr && w.use_dense && clean_need > 0 && clean_table_bytes >= clean_need) {
+    clean = static_cast<uint32_t *>(clean_table);
+    clean_words = (int64_t)(clean_need / 4);
+    w.table.total = static_cast<int32_t *>(clean_table);
+    w.in_bits = clean + kCleanHeader / 4;
+  }
+  if ((rc = rulebook_mark_and_scan(indices, n_in, gg, w, pair_num, mirror, s, split,
+                                   clean != nullptr)) != SSC_OK)
+    return rc;
   if ((rc = read_back_mirror_queued(s)) != SSC_OK) return rc;
-  return rulebook_pairs(indices, n_in, gg, w, out_indices, pairs, pair_num, true, s);
+  return rulebook_pairs(indices, n_in, gg, w, out_indices, pairs, pair_num, true, s, clean,
+                        clean_words);
 }
+
+extern "C" {
 
 int ssc_rulebook_finish(const ssc_geometry *g, int64_t n_in, int32_t *n_out_host,
                         int32_t *in_order_host) {

@@ -119,6 +119,48 @@ __device__ __forceinline__ void popc_blocksum_block(const uint32_t *__restrict__
   if (threadIdx.x == 0) blocksum[b] = tot;
 }
 
+// Second pass of the popcount scan for scan block blockIdx.x (kScanThreads threads):
+// exclusive prefix per word.  Every block first adds up the sums of the blocks before it
+// (at most 2^31 / 32 / kScanBlockWords = 32768 values), which saves the launch of a scan
+// over blocksum[]; the table's last block (`last`) also writes the total, and with `mirror`
+// copies total[0..3] there (total[1..3] were written by kernels before this one).
+__device__ __forceinline__ void popc_prefix_block(const uint32_t *__restrict__ bits,
+                                                  int64_t n_words,
+                                                  const int32_t *__restrict__ blocksum,
+                                                  int32_t *__restrict__ prefix,
+                                                  int32_t *__restrict__ total,
+                                                  int32_t *__restrict__ mirror, bool last) {
+  __shared__ int lds[kScanThreads / 64 + 1];
+  int before = 0;
+  for (int64_t b = threadIdx.x; b < (int64_t)blockIdx.x; b += kScanThreads) before += blocksum[b];
+  int block_off;
+  block_exclusive_scan(before, lds, &block_off);
+  int64_t base = (int64_t)blockIdx.x * kScanBlockWords + (int64_t)threadIdx.x * kScanItems;
+  int c[kScanItems];
+  int v = 0;
+#pragma unroll
+  for (int i = 0; i < kScanItems; ++i) {
+    c[i] = base + i < n_words ? __popc(bits[base + i]) : 0;
+    v += c[i];
+  }
+  int tot;
+  int ex = block_exclusive_scan(v, lds, &tot) + block_off;
+#pragma unroll
+  for (int i = 0; i < kScanItems; ++i) {
+    if (base + i < n_words) prefix[base + i] = ex;
+    ex += c[i];
+  }
+  if (last && threadIdx.x == 0) {
+    total[0] = block_off + tot;
+    if (mirror != nullptr) {
+      mirror[0] = block_off + tot;
+      mirror[1] = total[1];
+      mirror[2] = total[2];
+      mirror[3] = total[3];
+    }
+  }
+}
+
 __device__ __forceinline__ int bit_rank(const uint32_t *__restrict__ bits,
                                         const int32_t *__restrict__ prefix, uint32_t key) {
   uint32_t w = key >> 5;
@@ -161,6 +203,28 @@ __device__ __forceinline__ void emit_rows_of_word(const uint32_t *__restrict__ b
     }
   }
 }
+
+// ---- work split of a convolution, seeded by the rulebook ----------------------------------
+// A regular stride-1 rulebook knows, cell by cell of its output table, how many output rows
+// and how many pairs lie below the cell (the popcounts its dilation step takes anyway).  That
+// is the work measure the convolution's plan deals its output rows to the workgroups by, so
+// the rulebook can place the ranges' boundaries itself, in a launch it makes anyway: the
+// plan is then built without its own passes over the pairs for that purpose.
+constexpr int kMaxRanges = 512;       // two for each of at most 256 workgroups
+constexpr int kSeedMaxBlocks = 2048;  // scan blocks of a table whose block sums fit in LDS
+struct SplitRequest {
+  int n_rng;           // ranges to cut the output rows into (<= kMaxRanges)
+  int tile_rows;       // weight of a pair relative to tile_cost (see split_work in conv.hip)
+  long long tile_cost; // cost of a row's share of a tile, in the same unit
+  int32_t *range_row0; // [n_rng + 1] device: first output row of every range
+};
+// ssc_rulebook_begin with an optional split request.  *seeded = whether range_row0 will be
+// written (the geometry takes the dilation path and the table is small enough).
+int rulebook_begin_impl(const int32_t *indices, int64_t n_in, const ssc_geometry *g,
+                        void *workspace, size_t workspace_bytes, int32_t *pairs,
+                        int32_t *pair_num, int32_t *out_indices, int64_t out_capacity,
+                        void *clean_table, size_t clean_table_bytes, const SplitRequest *split,
+                        bool *seeded, hipStream_t s);
 
 // Enqueue: fill an int32 array (a kernel, so the call may be graph-captured).
 int fill_i32(int32_t *p, int64_t n, int32_t v, hipStream_t s);

@@ -43,9 +43,16 @@ _SIGNATURES = {
                                                   ctypes.POINTER(_i32), _vp]),
     "ssc_rulebook_emit": (ctypes.c_int, [_vp, _i64, _gp, _vp, _sz, _vp, _vp, _vp, _vp]),
     "ssc_rulebook_out_bound": (_sz, [_gp, _i64]),
-    "ssc_rulebook_begin": (ctypes.c_int, [_vp, _i64, _gp, _vp, _sz, _vp, _vp, _vp, _i64, _vp]),
+    "ssc_rulebook_clean_table_bytes": (_sz, [_gp, _i64]),
+    "ssc_rulebook_begin": (ctypes.c_int, [_vp, _i64, _gp, _vp, _sz, _vp, _vp, _vp, _i64, _vp, _sz,
+                                          _vp]),
     "ssc_rulebook_finish": (ctypes.c_int, [_gp, _i64, ctypes.POINTER(_i32), ctypes.POINTER(_i32)]),
     "ssc_rulebook_rows": (ctypes.c_int, [_gp, _i64, _vp, _sz, _vp, _vp]),
+    "ssc_rulebook_conv_begin": (ctypes.c_int, [_vp, _i64, _gp, _vp, _sz, _vp, _vp, _vp, _i64, _vp,
+                                               _sz, _i32, _i32, _i32, _vp, _sz, _vp]),
+    "ssc_rulebook_conv_finish": (ctypes.c_int, [_gp, _i64, ctypes.POINTER(_i32),
+                                                ctypes.POINTER(_i32), _vp, _vp, _i32, _i32, _i32,
+                                                _vp, _sz, _vp, _sz, _vp]),
     "ssc_conv_workspace_bytes": (_sz, [_i64, _i32, _i32, _i32, _i64]),
     "ssc_conv_plan_bytes": (_sz, [_i64, _i32, _i32, _i32, _i64]),
     "ssc_conv_plan_scratch_bytes": (_sz, [_i64, _i32, _i32, _i32, _i64]),
@@ -246,15 +253,35 @@ def rulebook_meta(indice_pairs):
     return meta
 
 
+# One buffer per (device, stream) that every rulebook call finds all zero and leaves all
+# zero (ssc_rulebook_begin's clean_table): zeroed when it is made, grown when a call asks for
+# more, dropped when a call fails.
+_clean_tables = {}
+
+
+def _clean_table(nbytes, dev, stream):
+    key = (dev.index, stream)
+    held = _clean_tables.get(key)
+    if held is None or held.numel() < nbytes:
+        held = torch.zeros(max(int(nbytes), 1 << 20), dtype=torch.uint8, device=dev)
+        _clean_tables[key] = held
+    return held
+
+
 class _PendingRulebook(object):
     """A rulebook between ssc_rulebook_begin and ssc_rulebook_finish: everything whose size
     does not depend on the number of outputs is queued, the host has not waited yet."""
     __slots__ = ("indices", "n", "geometry", "ws", "pairs", "num", "out_buf", "subm", "stream",
-                 "bound")
+                 "bound", "plan", "scratch", "conv")
 
 
 def _rulebook_begin(indices, batch_size, out_spatial_shape, kernel_size, stride, padding, dilation,
-                    out_padding, subm, transpose):
+                    out_padding, subm, transpose, conv=None):
+    """Queue a rulebook.  With `conv` = (c_in, c_out, element bytes) of the convolution that
+    will run over it, and buffers for its plan within reason, the plan's buffers are
+    allocated here (for the bound on the number of outputs) and the rulebook is asked to
+    deal the output rows to the convolution's workgroups on its way
+    (ssc_rulebook_conv_begin)."""
     if indices.dim() != 2 or indices.size(1) != 4:
         raise RuntimeError("indices must be [N, 4] (batch, x, y, z)")
     for lst in (kernel_size, out_spatial_shape, stride, padding, out_padding, dilation):
@@ -291,10 +318,47 @@ def _rulebook_begin(indices, batch_size, out_spatial_shape, kernel_size, stride,
         r.bound = max(int(bound), 0)
         if 0 < bound * 16 <= _ROWS_AHEAD_BYTES:
             r.out_buf = torch.empty((bound, 4), dtype=torch.int32, device=dev)
-    _check(_lib.ssc_rulebook_begin(_ptr(indices), n, gref, r.ws.data_ptr(), r.ws.numel(),
-                                   _ptr(r.pairs), r.num.data_ptr(), _ptr(r.out_buf),
-                                   0 if r.out_buf is None else r.out_buf.size(0), r.stream))
+    r.plan = r.scratch = r.conv = None
+    if conv is not None and n > 0 and 0 < r.bound <= 8 * n * K:
+        c_in, c_out, eb = conv
+        plan_bytes = _lib.ssc_conv_plan_bytes(r.bound, K, c_in, c_out, n)
+        scratch_bytes = _lib.ssc_conv_plan_scratch_bytes(r.bound, K, c_in, c_out, n)
+        if plan_bytes <= _PLAN_AHEAD_BYTES and scratch_bytes <= _PLAN_AHEAD_BYTES:
+            r.plan = _workspace(plan_bytes, dev)
+            r.scratch = _workspace(scratch_bytes, dev)
+            r.conv = (int(c_in), int(c_out), int(eb))
+    clean_bytes = _lib.ssc_rulebook_clean_table_bytes(gref, n)
+    clean = _clean_table(clean_bytes, dev, r.stream) if clean_bytes > 0 else None
+    try:
+        if r.conv is not None:
+            _check(_lib.ssc_rulebook_conv_begin(
+                _ptr(indices), n, gref, r.ws.data_ptr(), r.ws.numel(), _ptr(r.pairs),
+                r.num.data_ptr(), _ptr(r.out_buf), 0 if r.out_buf is None else r.out_buf.size(0),
+                _ptr(clean), 0 if clean is None else clean.numel(),
+                r.conv[0], r.conv[1], r.conv[2], r.scratch.data_ptr(), r.scratch.numel(),
+                r.stream))
+        else:
+            _check(_lib.ssc_rulebook_begin(_ptr(indices), n, gref, r.ws.data_ptr(), r.ws.numel(),
+                                           _ptr(r.pairs), r.num.data_ptr(), _ptr(r.out_buf),
+                                           0 if r.out_buf is None else r.out_buf.size(0),
+                                           _ptr(clean), 0 if clean is None else clean.numel(),
+                                           r.stream))
+    except Exception:
+        _clean_tables.pop((dev.index, r.stream), None)  # it may not be clean any more
+        raise
     return r
+
+
+def _rulebook_conv_wait(r):
+    """Wait for the number of outputs of a rulebook begun with `conv` and queue the plan of
+    the convolution (ssc_rulebook_conv_finish): (n_out, input rows in key order)."""
+    n_out = _i32(0)
+    in_order = _i32(0)
+    _check(_lib.ssc_rulebook_conv_finish(
+        ctypes.byref(r.geometry), r.n, ctypes.byref(n_out), ctypes.byref(in_order),
+        _ptr(r.pairs), r.num.data_ptr(), r.conv[0], r.conv[1], r.conv[2], r.plan.data_ptr(),
+        r.plan.numel(), r.scratch.data_ptr(), r.scratch.numel(), r.stream))
+    return n_out.value, bool(in_order.value)
 
 
 def _rulebook_wait(r):
@@ -502,50 +566,45 @@ def rulebook_conv(features, filters, indices, batch_size, out_spatial_shape, ker
     dtype = features.dtype
     if dtype not in _ENTRIES or filters.dtype != dtype:
         raise RuntimeError("rulebook_conv needs float32 or half features and filters of one type")
-    r = _rulebook_begin(indices, batch_size, out_spatial_shape, kernel_size, stride, padding,
-                        dilation, out_padding, subm, 0)
     features = features.contiguous()
     n_in, c_in = features.shape
     c_out = filters.size(-1)
+    eb = features.element_size()
+    # Between the host's wake-up and the first launch of the plan the GPU has nothing to do:
+    # whatever can be prepared is prepared before the wait.  With a bound on the number of
+    # outputs at hand (and buffers of that size within reason) that includes the buffers of
+    # the plan, which is then queued straight after the wait by the call that waits; tensors
+    # and bookkeeping follow when the kernel is on its way.
+    r = _rulebook_begin(indices, batch_size, out_spatial_shape, kernel_size, stride, padding,
+                        dilation, out_padding, subm, 0, conv=(c_in, c_out, eb))
     owner = filters
     filters, fs_k, fs_ci, fs_co = _filter_strides(filters, c_in, c_out)
     K = r.pairs.size(0)
     kvol = 1
     for d in filters.shape[:-2]:
         kvol *= d
-    if kvol != K:
-        raise RuntimeError("filters have %d offsets but the rulebook has %d" % (kvol, K))
-    if n_in != r.n:
-        raise RuntimeError("features and indices must have the same number of rows")
     dev = features.device
     s = r.stream
+    bad = None
+    if kvol != K:
+        bad = "filters have %d offsets but the rulebook has %d" % (kvol, K)
+    elif n_in != r.n:
+        bad = "features and indices must have the same number of rows"
+    if bad is not None:
+        _rulebook_wait(r)  # (the rulebook is queued: end it before raising)
+        raise RuntimeError(bad)
     packed = _packed_filters(owner, filters, (fs_k, fs_ci, fs_co), K, c_in, c_out, s)
-    eb = features.element_size()
-    # Between the host's wake-up and the first launch of the plan the GPU has nothing to do:
-    # whatever can be prepared is prepared before the wait.  With a bound on the number of
-    # outputs at hand (and buffers of that size within reason) that includes the buffers of
-    # the plan, which is then queued straight after the wait; tensors and bookkeeping follow
-    # when the kernel is on its way.
-    plan = scratch = None
-    if 0 < r.bound <= 8 * max(n_in, 1) * K:
-        plan_bytes = _lib.ssc_conv_plan_bytes(r.bound, K, c_in, c_out, n_in)
-        scratch_bytes = _lib.ssc_conv_plan_scratch_bytes(r.bound, K, c_in, c_out, n_in)
-        if plan_bytes <= _PLAN_AHEAD_BYTES and scratch_bytes <= _PLAN_AHEAD_BYTES:
-            plan = _workspace(plan_bytes, dev)
-            scratch = _workspace(scratch_bytes, dev)
-    n_out, in_order = _rulebook_wait(r)
-    if plan is None or n_out == 0:
+    if r.conv is None:
+        n_out, in_order = _rulebook_wait(r)
         outids, pairs, num = _rulebook_result(r, n_out, in_order)
         plan = _plan_of(pairs._ssc_meta, pairs, num, K, c_in, c_out, eb, n_in, n_out, False, dev, s)
         out = _run_planned(features, n_in, c_in, packed, plan, n_in, K, c_out, n_out, s, epilogue)
         return out, outids, pairs, num
-    _check(_lib.ssc_conv_plan_build(r.pairs.data_ptr(), n_in, r.num.data_ptr(), K, 0,
-                                    2 if in_order else 0, n_in, n_out, c_in, c_out, eb,
-                                    plan.data_ptr(), plan.numel(), scratch.data_ptr(),
-                                    scratch.numel(), s))
-    out = _run_planned(features, n_in, c_in, packed, plan, n_in, K, c_out, n_out, s, epilogue)
+    n_out, in_order = _rulebook_conv_wait(r)
+    out = _run_planned(features, n_in, c_in, packed, r.plan, n_in, K, c_out, n_out, s, epilogue)
     outids, pairs, num = _rulebook_result(r, n_out, in_order)
-    pairs._ssc_meta.plans[(False, c_in, c_out, eb, n_in, n_out)] = plan
+    if n_out > 0:
+        pairs._ssc_meta.plans[(False, c_in, c_out, eb, n_in, n_out)] = r.plan
     return out, outids, pairs, num
 
 

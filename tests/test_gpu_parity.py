@@ -201,6 +201,52 @@ def test_rulebook_count_then_emit_entry_points(case, shuffle, device):
     assert torch.equal(pairs, want[1]) and torch.equal(num, want[2])
 
 
+def test_rulebook_clean_table_contract(oracle, device):
+    """ssc_rulebook_begin with a table the caller keeps between calls: it must be all zero
+    again when the call's kernels are done, whatever geometries share it, and the rulebook
+    must be the one the call without it builds (and the oracle's)."""
+    import ctypes
+    from ss_conv import _ext
+    lib = _ext._lib
+    rng = np.random.default_rng(21)
+    table = None
+    for batch, grid, n, k, p in ((2, 32, 3000, 3, 1), (1, 64, 9000, 5, 2), (3, 32, 500, 3, 1),
+                                 (2, 32, 4000, 3, 0)):
+        idx = random_voxels(rng, batch, grid, n)
+        t = torch.from_numpy(idx).to(device)
+        os_ = grid + 2 * p - (k - 1)
+        g = _ext._geometry(batch, [os_] * 3, [k] * 3, [1] * 3, [p] * 3, [1] * 3, 0, 0)
+        gref = ctypes.byref(g)
+        need = lib.ssc_rulebook_clean_table_bytes(gref, n)
+        if os_ % 32 == 0:
+            assert need > 0
+        if table is None or table.numel() < need:
+            table = torch.zeros(max(need, 1), dtype=torch.uint8, device=device)
+        K = k ** 3
+        results = []
+        for with_table in (True, False, True):
+            nbytes = lib.ssc_rulebook_workspace_bytes(gref, n)
+            ws = torch.empty(nbytes, dtype=torch.uint8, device=device)
+            pairs = torch.full((K, 2, n), -7, dtype=torch.int32, device=device)
+            num = torch.full((K,), -7, dtype=torch.int32, device=device)
+            n_out, in_order = ctypes.c_int32(0), ctypes.c_int32(-1)
+            assert lib.ssc_rulebook_begin(t.data_ptr(), n, gref, ws.data_ptr(), nbytes,
+                                          pairs.data_ptr(), num.data_ptr(), None, 0,
+                                          table.data_ptr() if with_table and need else None,
+                                          table.numel() if with_table and need else 0, None) == 0
+            assert lib.ssc_rulebook_finish(gref, n, ctypes.byref(n_out), ctypes.byref(in_order)) == 0
+            out = torch.empty((max(n_out.value, 1), 4), dtype=torch.int32, device=device)
+            assert lib.ssc_rulebook_rows(gref, n, ws.data_ptr(), nbytes, out.data_ptr(), None) == 0
+            torch.cuda.synchronize()
+            assert int(table.count_nonzero().item()) == 0, (batch, grid, n, k, p)
+            assert in_order.value == 1
+            results.append((out[:n_out.value].cpu().numpy(), pairs.cpu().numpy(), num.cpu().numpy()))
+        want = oracle.canonicalize(*oracle.rulebook(idx, batch, [grid] * 3, k, 1, p))
+        for got in results:
+            for a, b in zip(got, want):
+                assert np.array_equal(a, b)
+
+
 def test_rulebook_few_voxels_in_a_large_grid(oracle, device):
     """300 voxels in 40 x 128^3 cells: the table has 2.6 M words, the input five chunks.
     (The blocks that decode the table into output rows ride on the grid of the kernel that
@@ -1707,8 +1753,10 @@ def test_fused_layer_on_a_dense_grid(device):
         g_idx, g_pairs, g_num = get_indice_pairs(t, 4, [64] * 3, 3, 1, 1, 1, 0, False)
         assert torch.equal(y.indices, g_idx)
         y2 = indice_conv(x, layer.weight, g_pairs, g_num, n_out)
-        assert torch.equal(y.features, y2)
-        # a sample of rows against float64 sums over the pairs
+        # (the layer's plan has its range boundaries from the rulebook, the call's from its
+        # own passes over the pairs: the same sums in another order)
+        assert rel_l2(y.features.cpu().numpy(), y2.cpu().numpy()) < 1e-6
+        # against float64 sums over the pairs
         w = layer.weight.double().reshape(27, 64, 64)
         ref = torch.zeros((n_out, 64), dtype=torch.float64, device=device)
         for k in range(27):
