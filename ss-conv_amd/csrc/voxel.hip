@@ -2,6 +2,8 @@
 // per-voxel feature reduction, 3-nearest-neighbour search and interpolation.
 #include "ssc_common.h"
 
+#include <type_traits>
+
 // Products and sums below are rounded separately, as the scalar statements of the
 // reference are: no fused multiply-add contraction in this file.  (Plain operators
 // only: the __fmul_rn / __fadd_rn wrappers are compiled before this pragma and
@@ -773,9 +775,10 @@ __global__ void __launch_bounds__(kP2vScanThreads)
     p2v_scan_kernel(const float *__restrict__ pts, const int64_t *__restrict__ ids, int64_t n,
                     float hx, float hy, float hz, int max_ids, uint32_t *__restrict__ bits,
                     int32_t *__restrict__ hist_all, int32_t *__restrict__ hist_valid,
-                    int32_t *__restrict__ flags) {
+                    int32_t *__restrict__ flags, int32_t *__restrict__ block_inside = nullptr) {
   __shared__ int s_all[64], s_valid[64];
-  __shared__ int s_first;
+  __shared__ int s_first, s_inside;
+  if (threadIdx.x == 0) s_inside = 0;
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   const int lane = threadIdx.x & 63;
   const bool live = i < n;
@@ -797,6 +800,9 @@ __global__ void __launch_bounds__(kP2vScanThreads)
   const int first_id = s_first;
   const unsigned long long in_mask = __ballot(inside);
   if (live && (lane & 31) == 0) bits[i >> 5] = (uint32_t)(in_mask >> (lane & 32));
+  // (with block_inside: the block's number of inside points, for a compaction that ranks
+  // its points without a scan of the bits)
+  if (block_inside != nullptr && lane == 0 && in_mask) atomicAdd(&s_inside, __popcll(in_mask));
   const bool ok_id = live && id >= 0 && id < max_ids;
   unsigned long long todo = __ballot(ok_id);
   while (todo) {  // one trip per distinct id of the wave
@@ -822,6 +828,7 @@ __global__ void __launch_bounds__(kP2vScanThreads)
     if (a) atomicAdd(&hist_all[first_id + threadIdx.x], a);
     if (b) atomicAdd(&hist_valid[first_id + threadIdx.x], b);
   }
+  if (block_inside != nullptr && threadIdx.x == 0) block_inside[blockIdx.x] = s_inside;
 }
 
 // One block of 256 threads: start[e] = survivors with an id below e; shift[e] = ids below e
@@ -1064,29 +1071,164 @@ __global__ void __launch_bounds__(256)
   for (int64_t j = i; j < n_words; j += step) vox_bits[j] = 0u;
 }
 
-// Blocks below n_scan_blocks: first pass of the scan over the inside bits.  The block after
-// them: per-id start and shift, the number of ids left without points into extra[0], and
-// the two histograms (max_ids entries each) into the host-visible mirror.
+// The compaction of the one-call chain: p2v_compact_kernel without the scans before it.  A
+// block takes the kP2vScanThreads points of one block of p2v_scan_kernel (the blocks after
+// the points' take the ids, for the zero points of ids left without survivors) and works
+// out for itself what the scans would have told it: the inside points before the block (a
+// sum over block_inside[], at most n / 1024 numbers), the rank of a point inside the block
+// (the popcounts of the block's 32 words of inside bits), and start / shift of every id (a
+// scan of the two histograms, n_ids numbers, in LDS).  The last block of points leaves the
+// number of inside points in inside_total[0]; block 0 the number of ids left without points
+// in extra[0] and the two histograms in mirror_hist (memory the host reads).
+constexpr int kP2vIdsPerThread = SSC_P2V_MAX_IDS / kP2vScanThreads;
+__global__ void __launch_bounds__(kP2vScanThreads)
+    p2vx_compact_kernel(const float *__restrict__ pts, const int64_t *__restrict__ ids, int64_t n,
+                        const uint32_t *__restrict__ bits,
+                        const int32_t *__restrict__ block_inside, int n_point_blocks,
+                        const int32_t *__restrict__ hist_all,
+                        const int32_t *__restrict__ hist_valid, float hx, float hy, float hz,
+                        float ux, float uy, float uz, float *__restrict__ out_pts,
+                        int64_t *__restrict__ out_ids, int32_t *__restrict__ coords,
+                        int32_t *__restrict__ dest, int32_t *__restrict__ src, int n_ids,
+                        uint32_t *__restrict__ vox_bits, int d1, int d2, int d3,
+                        int32_t *__restrict__ flags, int32_t *__restrict__ inside_total,
+                        int32_t *__restrict__ extra, int32_t *__restrict__ mirror_hist) {
+  static_assert(kP2vIdsPerThread >= 1 && kP2vIdsPerThread * kP2vScanThreads == SSC_P2V_MAX_IDS,
+                "ids per thread");
+  __shared__ int s_start[SSC_P2V_MAX_IDS], s_shift[SSC_P2V_MAX_IDS];
+  __shared__ int s_wave_a[kP2vScanThreads / 64], s_wave_b[kP2vScanThreads / 64];
+  __shared__ int s_word[32], s_wprefix[32];
+  __shared__ int s_before;
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+  // start[e] = survivors with an id below e; shift[e] = ids below e that are present but
+  // have no survivor: every thread a run of consecutive ids, then a scan over the threads
+  int hv[kP2vIdsPerThread], he[kP2vIdsPerThread], sv = 0, se = 0;
+#pragma unroll
+  for (int j = 0; j < kP2vIdsPerThread; ++j) {
+    const int e = t * kP2vIdsPerThread + j;
+    const int a = e < n_ids ? hist_all[e] : 0, v = e < n_ids ? hist_valid[e] : 0;
+    hv[j] = v;
+    he[j] = (a > 0 && v == 0) ? 1 : 0;
+    sv += hv[j];
+    se += he[j];
+    if (blockIdx.x == 0 && e < n_ids) {
+      mirror_hist[e] = a;
+      mirror_hist[n_ids + e] = v;
+    }
+  }
+  // the inside points of the blocks before this one (blocks of ids: of all blocks)
+  int before = 0;
+  const int upto = (int)blockIdx.x < n_point_blocks ? (int)blockIdx.x : n_point_blocks;
+  for (int b = t; b < upto; b += kP2vScanThreads) before += block_inside[b];
+  int iv = sv, ie = se, ib = before;
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    const int ov = __shfl_up(iv, d, 64), oe = __shfl_up(ie, d, 64);
+    if (lane >= d) {
+      iv += ov;
+      ie += oe;
+    }
+  }
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) ib += __shfl_xor(ib, d, 64);
+  if (lane == 63) {
+    s_wave_a[wave] = iv;
+    s_wave_b[wave] = ie;
+  }
+  if (t == 0) s_before = 0;
+  if (t < 32) {
+    const int64_t w = (int64_t)blockIdx.x * (kP2vScanThreads / 32) + t;
+    s_word[t] = ((int)blockIdx.x < n_point_blocks && w * 32 < n) ? (int)bits[w] : 0;
+  }
+  __syncthreads();
+  if (lane == 0 && ib) atomicAdd(&s_before, ib);
+  int bv = iv - sv, be = ie - se;
+  int all_e = 0;
+  for (int u = 0; u < kP2vScanThreads / 64; ++u) {
+    if (u < wave) {
+      bv += s_wave_a[u];
+      be += s_wave_b[u];
+    }
+    all_e += s_wave_b[u];
+  }
+#pragma unroll
+  for (int j = 0; j < kP2vIdsPerThread; ++j) {
+    const int e = t * kP2vIdsPerThread + j;
+    s_start[e] = bv;
+    s_shift[e] = be;
+    bv += hv[j];
+    be += he[j];
+  }
+  if (t < 32) {  // (one half of the first wave)
+    const int c = __popc((uint32_t)s_word[t]);
+    int incl = c;
+#pragma unroll
+    for (int d = 1; d < 32; d <<= 1) {
+      const int o = __shfl_up(incl, d, 64);
+      if (t >= d) incl += o;
+    }
+    s_wprefix[t] = incl - c;
+  }
+  __syncthreads();
+  if (blockIdx.x == 0 && t == 0) extra[0] = all_e;
+  if ((int)blockIdx.x == n_point_blocks - 1 && t == 0)
+    inside_total[0] = s_before + s_wprefix[31] + __popc((uint32_t)s_word[31]);
+  float x = 0.f, y = 0.f, z = 0.f;
+  int64_t id;
+  int pos;
+  const int64_t i = (int64_t)blockIdx.x * kP2vScanThreads + t;
+  if ((int)blockIdx.x < n_point_blocks) {
+    if (i >= n) return;
+    id = ids[i];
+    const uint32_t word = (uint32_t)s_word[t >> 5];
+    const bool inside = ((word >> (t & 31)) & 1u) && id >= 0 && id < n_ids;
+    pos = inside ? s_before + s_wprefix[t >> 5] + __popc(word & ((1u << (t & 31)) - 1u)) +
+                       s_shift[inside ? (int)id : 0]
+                 : -1;
+    dest[i] = pos;
+    if (!inside) return;
+    x = pts[i * 3];
+    y = pts[i * 3 + 1];
+    z = pts[i * 3 + 2];
+  } else {
+    id = (int64_t)((int)blockIdx.x - n_point_blocks) * kP2vScanThreads + t;
+    if (id >= n_ids || hist_all[id] == 0 || hist_valid[id] != 0) return;
+    pos = s_start[id] + s_shift[id];
+  }
+  src[pos] = (int)blockIdx.x < n_point_blocks ? (int32_t)i : -1;  // input row behind row pos
+  out_pts[(int64_t)pos * 3] = x;
+  out_pts[(int64_t)pos * 3 + 1] = y;
+  out_pts[(int64_t)pos * 3 + 2] = z;
+  out_ids[pos] = id;
+  const int vx = (int)((x + hx) / ux);
+  const int vy = (int)((y + hy) / uy);
+  const int vz = (int)((z + hz) / uz);
+  reinterpret_cast<int4 *>(coords)[pos] = make_int4((int)id, vx, vy, vz);
+  if ((unsigned)vx < (unsigned)d1 && (unsigned)vy < (unsigned)d2 && (unsigned)vz < (unsigned)d3) {
+    const uint32_t key = (uint32_t)((((int)id * d1 + vx) * d2 + vy) * d3 + vz);
+    atomicOr(&vox_bits[key >> 5], 1u << (key & 31u));
+  } else {
+    atomicOr(&flags[0], 4);
+  }
+}
+
+// First pass of the scan over the voxel table; block 0 also hands the chain's other totals
+// to the table's total[] -- [1] surviving points, [2] ids left without points, [3] flags
+// (bit 0: an id outside the table, bit 1: ids decrease, bit 2: a voxel outside the grid) --
+// from where the scan's second pass copies them, with the number of voxels, to the host.
 __global__ void __launch_bounds__(kScanThreads)
-    p2vx_blocksum_prefix_kernel(const uint32_t *__restrict__ bits, int64_t n_words,
-                                int32_t *__restrict__ blocksum, int64_t n_scan_blocks,
-                                const int32_t *__restrict__ hist_all,
-                                const int32_t *__restrict__ hist_valid,
-                                int32_t *__restrict__ start, int32_t *__restrict__ shift,
-                                int32_t *__restrict__ extra, int max_ids,
-                                int32_t *__restrict__ mirror_hist) {
-  __shared__ int s_a[256], s_b[256];
-  if ((int64_t)blockIdx.x < n_scan_blocks) {
-    popc_blocksum_block(bits, n_words, blockIdx.x, blocksum, s_a);
-    return;
+    p2vx_vox_blocksum_kernel(const uint32_t *__restrict__ bits, int64_t n_words,
+                             int32_t *__restrict__ blocksum,
+                             const int32_t *__restrict__ inside_total,
+                             const int32_t *__restrict__ extra,
+                             const int32_t *__restrict__ flags, int32_t *__restrict__ vox_total) {
+  __shared__ int lds[kScanThreads / 64 + 1];
+  if (blockIdx.x == 0 && threadIdx.x == 0) {
+    vox_total[1] = inside_total[0];
+    vox_total[2] = extra[0];
+    vox_total[3] = (flags[0] & 5) | ((flags[1] & 1) << 1);
   }
-  int n_empty;
-  p2v_prefix_block(hist_all, hist_valid, start, shift, s_a, s_b, &n_empty);
-  if (threadIdx.x == 255) extra[0] = n_empty;
-  for (int e = threadIdx.x; e < max_ids; e += 256) {
-    mirror_hist[e] = hist_all[e];
-    mirror_hist[max_ids + e] = hist_valid[e];
-  }
+  popc_blocksum_block(bits, n_words, blockIdx.x, blocksum, lds);
 }
 
 // Blocks below link_blocks: row pos < rows: inverse[pos] = rank of its voxel, and the row is
@@ -1122,40 +1264,22 @@ __global__ void __launch_bounds__(256)
   next[pos] = atomicExch(&head[rk], (int32_t)pos);
 }
 
-// One wave per voxel: walk the chain (count, smallest and largest row), then
+// The feature reduction of the one-call chain.  Sixteen lanes per voxel (four voxels to a
+// wave): the lanes walk the voxel's chain together (count, smallest and largest row, the
+// first four rows), then
 //   mode 1 / 2: the features of the first / last row,
 //   mode 3 / 4: sum over the rows in ascending order of mult * feats, mult = 1 / count in
 //               mode 4 (product rounded before the add, as in voxel_reduce_kernel).
-// Ascending order: rows of a window of 2048 row numbers are entered into a bit map, lane l
-// holding word l, and read back bit by bit; windows follow each other upwards.  Lanes run
-// along the channels.  src[row] is the input row behind a row (-1: a zero point).
-__global__ void __launch_bounds__(256)
-    p2vx_reduce_kernel(const float *__restrict__ feats, int C, const int32_t *__restrict__ src,
-                       const int32_t *__restrict__ head, const int32_t *__restrict__ next,
-                       const int32_t *__restrict__ n_voxel, const int32_t *__restrict__ flags,
-                       int mode, float *__restrict__ out, int32_t *__restrict__ counts,
-                       int32_t *__restrict__ sel) {
-  if ((flags[0] | flags[1]) != 0) return;  // (see p2vx_link_kernel)
-  const int lane = threadIdx.x & 63;
-  const int64_t v = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (v >= n_voxel[0]) return;  // (the same for the whole wave)
-  const int first = __builtin_amdgcn_readfirstlane(head[v]);
-  int n = 0, lo = 0x7FFFFFFF, hi = -1;
-  for (int p = first; p >= 0; p = __builtin_amdgcn_readfirstlane(next[p])) {
-    ++n;
-    lo = p < lo ? p : lo;
-    hi = p > hi ? p : hi;
-  }
-  if (lane == 0) counts[v] = n;
-  float *o = out + v * C;
-  if (mode == 1 || mode == 2) {
-    const int p = mode == 1 ? lo : hi;
-    if (lane == 0 && sel != nullptr) sel[v] = p;
-    const int sr = n > 0 ? __builtin_amdgcn_readfirstlane(src[p]) : -1;
-    for (int c = lane; c < C; c += 64) o[c] = sr >= 0 ? feats[(int64_t)sr * C + c] : 0.f;
-    return;
-  }
-  const float mult = (mode == 4 && n > 0) ? 1.f / (float)n : 1.f;
+// Nearly every voxel holds a point or two: up to four rows are ordered in registers.  A
+// voxel with more is left to the whole wave afterwards (p2vx_reduce_long): rows of a window
+// of 2048 row numbers are entered into a bit map, lane l holding word l, and read back bit
+// by bit; windows follow each other upwards.  Lanes run along the channels.  src[row] is
+// the input row behind a row (-1: a zero point).
+__device__ __forceinline__ void p2vx_reduce_long(const float *__restrict__ feats, int C,
+                                                 const int32_t *__restrict__ src,
+                                                 const int32_t *__restrict__ next, int first,
+                                                 int lo, int hi, float mult,
+                                                 float *__restrict__ o, int lane) {
   for (int c0 = 0; c0 < C; c0 += 256) {
     float acc[4] = {0.f, 0.f, 0.f, 0.f};
     auto add_row = [&](int p) {
@@ -1170,25 +1294,21 @@ __global__ void __launch_bounds__(256)
         }
       }
     };
-    if (n == 1) {
-      add_row(lo);
-    } else if (n > 1) {
-      for (int base = lo & ~2047; base <= hi; base += 2048) {
-        uint32_t mine = 0u;
-        for (int p = first; p >= 0; p = __builtin_amdgcn_readfirstlane(next[p])) {
-          const int off = p - base;
-          if ((unsigned)off < 2048u && (off >> 5) == lane) mine |= 1u << (off & 31);
-        }
-        unsigned long long lanes = __ballot(mine != 0u);
-        while (lanes) {
-          const int l = __ffsll((long long)lanes) - 1;
-          lanes &= lanes - 1;
-          uint32_t w = (uint32_t)__shfl((int)mine, l, 64);
-          while (w) {
-            const int b = __ffs((int)w) - 1;
-            w &= w - 1;
-            add_row(base + l * 32 + b);
-          }
+    for (int base = lo & ~2047; base <= hi; base += 2048) {
+      uint32_t mine = 0u;
+      for (int p = first; p >= 0; p = __builtin_amdgcn_readfirstlane(next[p])) {
+        const int off = p - base;
+        if ((unsigned)off < 2048u && (off >> 5) == lane) mine |= 1u << (off & 31);
+      }
+      unsigned long long lanes = __ballot(mine != 0u);
+      while (lanes) {
+        const int l = __ffsll((long long)lanes) - 1;
+        lanes &= lanes - 1;
+        uint32_t w = (uint32_t)__shfl((int)mine, l, 64);
+        while (w) {
+          const int b = __ffs((int)w) - 1;
+          w &= w - 1;
+          add_row(base + l * 32 + b);
         }
       }
     }
@@ -1197,6 +1317,103 @@ __global__ void __launch_bounds__(256)
       const int c = c0 + lane + 64 * j;
       if (c < C) o[c] = acc[j];
     }
+  }
+}
+
+constexpr int kP2vGroup = 8;    // lanes to a voxel
+constexpr int kP2vShort = 4;    // rows ordered in registers
+// VEC: 4 when the rows hold a multiple of four channels (16-byte loads and stores), else 1.
+template <int VEC>
+__global__ void __launch_bounds__(256)
+    p2vx_reduce_kernel(const float *__restrict__ feats, int C, const int32_t *__restrict__ src,
+                       const int32_t *__restrict__ head, const int32_t *__restrict__ next,
+                       const int32_t *__restrict__ n_voxel, const int32_t *__restrict__ flags,
+                       int mode, float *__restrict__ out, int32_t *__restrict__ counts,
+                       int32_t *__restrict__ sel) {
+  if ((flags[0] | flags[1]) != 0) return;  // (see p2vx_link_kernel)
+  const int lane = threadIdx.x & 63, gl = lane & (kP2vGroup - 1);
+  const int64_t v = ((int64_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * (64 / kP2vGroup) +
+                    (lane / kP2vGroup);
+  const bool live = v < n_voxel[0];
+  const int first = live ? head[v] : -1;
+  int n = 0, lo = 0x7FFFFFFF, hi = -1;
+  int r[kP2vShort];
+#pragma unroll
+  for (int q = 0; q < kP2vShort; ++q) r[q] = 0x7FFFFFFF;
+  for (int p = first; p >= 0; p = next[p]) {
+#pragma unroll
+    for (int q = 0; q < kP2vShort; ++q)
+      if (n == q) r[q] = p;
+    ++n;
+    lo = p < lo ? p : lo;
+    hi = p > hi ? p : hi;
+  }
+  if (live && gl == 0) counts[v] = n;
+  float *o = out + v * C;
+  const bool is_long = live && (mode == 3 || mode == 4) && n > kP2vShort;
+  using Vec = typename std::conditional<VEC == 4, float4, float>::type;
+  auto load = [&](int sr, int c) -> Vec {
+    if constexpr (VEC == 4) {
+      return sr >= 0 ? *reinterpret_cast<const float4 *>(feats + (int64_t)sr * C + c)
+                     : make_float4(0.f, 0.f, 0.f, 0.f);
+    } else {
+      return sr >= 0 ? feats[(int64_t)sr * C + c] : 0.f;
+    }
+  };
+  if (live && (mode == 1 || mode == 2)) {
+    const int p = mode == 1 ? lo : hi;
+    if (gl == 0 && sel != nullptr) sel[v] = p;
+    const int sr = n > 0 ? src[p] : -1;
+    for (int c = gl * VEC; c < C; c += kP2vGroup * VEC) *reinterpret_cast<Vec *>(o + c) = load(sr, c);
+  } else if (live && !is_long) {
+    // ascending rows: a sorting network over the (at most) four row numbers, unused places
+    // holding the largest integer
+    auto order = [](int &a, int &b) {
+      const int x = a < b ? a : b, y = a < b ? b : a;
+      a = x;
+      b = y;
+    };
+    order(r[0], r[1]);
+    order(r[2], r[3]);
+    order(r[0], r[2]);
+    order(r[1], r[3]);
+    order(r[1], r[2]);
+    const float mult = (mode == 4 && n > 0) ? 1.f / (float)n : 1.f;
+    int sr[kP2vShort];
+#pragma unroll
+    for (int q = 0; q < kP2vShort; ++q) sr[q] = q < n ? src[r[q]] : -1;
+    for (int c = gl * VEC; c < C; c += kP2vGroup * VEC) {
+      Vec f[kP2vShort];
+#pragma unroll
+      for (int q = 0; q < kP2vShort; ++q)
+        if (q < n) f[q] = load(sr[q], c);
+      float acc[VEC];
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) acc[e] = 0.f;
+#pragma unroll
+      for (int q = 0; q < kP2vShort; ++q) {
+        if (q < n) {
+          const float *fe = reinterpret_cast<const float *>(&f[q]);
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) {
+            const float t = mult * fe[e];
+            acc[e] = acc[e] + t;
+          }
+        }
+      }
+      *reinterpret_cast<Vec *>(o + c) = *reinterpret_cast<const Vec *>(acc);
+    }
+  }
+  // voxels with more rows, one after the other, by the whole wave
+  unsigned long long todo = __ballot(is_long && gl == 0);
+  while (todo) {
+    const int l = __ffsll((long long)todo) - 1;
+    todo &= todo - 1;
+    const int64_t vv = (int64_t)__shfl((int)v, l, 64);  // (fewer than 2^31 voxels)
+    const int f1 = __shfl(first, l, 64), n1 = __shfl(n, l, 64);
+    const int lo1 = __shfl(lo, l, 64), hi1 = __shfl(hi, l, 64);
+    const float mult = mode == 4 ? 1.f / (float)n1 : 1.f;
+    p2vx_reduce_long(feats, C, src, next, f1, lo1, hi1, mult, out + vv * C, lane);
   }
 }
 
@@ -1226,21 +1443,6 @@ __global__ void __launch_bounds__(256)
     }
   }
   d_feats[e] = g;
-}
-
-// mirror[0] = voxels, [1] = surviving points, [2] = ids left without points, [3] = flags
-// (bit 0: an id outside the table, bit 1: ids decrease, bit 2: a voxel outside the grid).
-__global__ void p2vx_totals_kernel(const int32_t *__restrict__ vox_total,
-                                   const int32_t *__restrict__ inside_total,
-                                   const int32_t *__restrict__ extra,
-                                   const int32_t *__restrict__ flags,
-                                   int32_t *__restrict__ mirror) {
-  if (threadIdx.x == 0) {
-    mirror[0] = vox_total[0];
-    mirror[1] = inside_total[0];
-    mirror[2] = extra[0];
-    mirror[3] = (flags[0] & 5) | ((flags[1] & 1) << 1);
-  }
 }
 
 struct P2vxWs {
@@ -1321,7 +1523,7 @@ int ssc_p2v_voxelize_f32(const float *points, const float *feats, const int64_t 
   int rc;
   int32_t *mirror = nullptr;
   if ((rc = read_back_mirror(&mirror)) != SSC_OK) return rc;
-  // mirror: [0..3] sizes and flags (p2vx_totals_kernel), [16 ..) the two histograms
+  // mirror: [0..3] sizes and flags (the voxel table's scan), [16 ..) the two histograms
   int32_t *extra = w.totals;  // [0]: ids left without points
 
   const int64_t clear_a = (w.flags + 2) - w.hist_all;
@@ -1331,31 +1533,31 @@ int ssc_p2v_voxelize_f32(const float *points, const float *feats, const int64_t 
                      dim3(256), 0, s, w.hist_all, clear_a, w.vox.bits, w.vox.n_words, w.head, n,
                      w.totals);
   SSC_LAUNCH_CHECK("p2vx_clear");
-  hipLaunchKernelGGL(p2v_scan_kernel, dim3((unsigned)ceil_div(n, kP2vScanThreads)),
-                     dim3(kP2vScanThreads), 0, s, points,
-                     batch_ids, n, half_extent[0], half_extent[1], half_extent[2], (int)n_ids,
-                     w.inside.bits, w.hist_all, w.hist_valid, w.flags);
+  const int64_t point_blocks = ceil_div(n, kP2vScanThreads);
+  hipLaunchKernelGGL(p2v_scan_kernel, dim3((unsigned)point_blocks), dim3(kP2vScanThreads), 0, s,
+                     points, batch_ids, n, half_extent[0], half_extent[1], half_extent[2],
+                     (int)n_ids, w.inside.bits, w.hist_all, w.hist_valid, w.flags,
+                     w.inside.prefix /* the blocks' inside counts */);
   SSC_LAUNCH_CHECK("p2v_scan");
-  hipLaunchKernelGGL(p2vx_blocksum_prefix_kernel, dim3((unsigned)(w.inside.n_scan_blocks + 1)),
-                     dim3(kScanThreads), 0, s, w.inside.bits, w.inside.n_words, w.inside.blocksum,
-                     w.inside.n_scan_blocks, w.hist_all, w.hist_valid, w.start, w.shift, extra,
-                     (int)n_ids, mirror + 16);
-  SSC_LAUNCH_CHECK("p2vx_blocksum_prefix");
-  if ((rc = bit_table_scan_prefix(w.inside, s, nullptr)) != SSC_OK) return rc;
-  const int64_t rows = n + n_ids;
-  hipLaunchKernelGGL(p2v_compact_kernel, dim3((unsigned)ceil_div(rows, 256)), dim3(256), 0, s,
-                     points, batch_ids, n, w.inside.bits, w.inside.prefix, w.hist_all, w.hist_valid,
-                     w.start, w.shift, half_extent[0], half_extent[1], half_extent[2], unit[0],
-                     unit[1], unit[2], out_points, out_ids, w.coords, dest, w.src, (int)n_ids,
-                     w.vox.bits, d1, d2, d3, w.flags);
-  SSC_LAUNCH_CHECK("p2v_compact");
-  // flags of the scan and of the marking travel with the voxel table's totals
-  if ((rc = bit_table_scan(w.vox, s, nullptr)) != SSC_OK) return rc;
-  // the host's copy of the sizes and flags: a small kernel behind the scans, then the event
-  // the host will wait for; the two kernels after it run while the host wakes up
-  hipLaunchKernelGGL(p2vx_totals_kernel, dim3(1), dim3(64), 0, s, w.vox.total, w.inside.total, extra,
-                     w.flags, mirror);
-  SSC_LAUNCH_CHECK("p2vx_totals");
+  // the compaction ranks its points from the blocks' counts and scans the histograms for
+  // itself: no scan of the inside bits, no launch for the per-id tables
+  hipLaunchKernelGGL(p2vx_compact_kernel,
+                     dim3((unsigned)(point_blocks + ceil_div(n_ids, kP2vScanThreads))),
+                     dim3(kP2vScanThreads), 0, s, points, batch_ids, n, w.inside.bits,
+                     w.inside.prefix, (int)point_blocks, w.hist_all, w.hist_valid, half_extent[0],
+                     half_extent[1], half_extent[2], unit[0], unit[1], unit[2], out_points,
+                     out_ids, w.coords, dest, w.src, (int)n_ids, w.vox.bits, d1, d2, d3, w.flags,
+                     w.inside.total, extra, mirror + 16);
+  SSC_LAUNCH_CHECK("p2vx_compact");
+  // the scan of the voxel table; its first pass hands the other totals and the flags to the
+  // table's total[], its second pass copies all of them to the host's mirror: [0] voxels,
+  // [1] surviving points, [2] ids left without points, [3] flags.  Then the event the host
+  // will wait for; the two kernels after it run while the host wakes up
+  hipLaunchKernelGGL(p2vx_vox_blocksum_kernel, dim3((unsigned)w.vox.n_scan_blocks),
+                     dim3(kScanThreads), 0, s, w.vox.bits, w.vox.n_words, w.vox.blocksum,
+                     w.inside.total, extra, w.flags, w.vox.total);
+  SSC_LAUNCH_CHECK("p2vx_vox_blocksum");
+  if ((rc = bit_table_scan_prefix(w.vox, s, mirror)) != SSC_OK) return rc;
   if ((rc = read_back_mirror_queued(s)) != SSC_OK) return rc;
   const int64_t link_blocks = ceil_div(n, 256);
   int64_t row_blocks = ceil_div(w.vox.n_words, 256);
@@ -1365,7 +1567,10 @@ int ssc_p2v_voxelize_f32(const float *points, const float *feats, const int64_t 
                      (int)n_ids, d1, d2, d3, link_blocks, w.flags, inverse, w.head, w.next,
                      out_indices);
   SSC_LAUNCH_CHECK("p2vx_link");
-  hipLaunchKernelGGL(p2vx_reduce_kernel, dim3((unsigned)ceil_div(n, 4)), dim3(256), 0, s, feats,
+  // (16-byte accesses need rows of a multiple of four channels from aligned bases)
+  const bool vec4 = (channels & 3) == 0 && (((uintptr_t)feats | (uintptr_t)out_feats) & 15) == 0;
+  hipLaunchKernelGGL(vec4 ? p2vx_reduce_kernel<4> : p2vx_reduce_kernel<1>,
+                     dim3((unsigned)ceil_div(n, 4 * (64 / kP2vGroup))), dim3(256), 0, s, feats,
                      (int)channels, w.src, w.head, w.next, w.vox.total, w.flags, (int)mode, out_feats,
                      counts, sel);
   SSC_LAUNCH_CHECK("p2vx_reduce");

@@ -30,9 +30,10 @@ class Point2Voxel(nn.Module):
                                               dtype=torch.float32)
         self.voxel_num_limit = np.array(voxel_num_limit)
         self.voxelization_mode = voxelization_mode
-        # 1 + the largest batch id of the last call: the next call sizes its tables for it
-        # before it has looked at its own ids (and falls back when they do not fit)
-        self._n_ids_hint = None
+        # The one-call path sizes its tables for batch ids below this number before it has
+        # looked at the ids (the call checks on the device that they fit, and falls back
+        # when they do not): 64 for a first call, 1 + the largest id of the last call after.
+        self._n_ids_hint = 64
         self.last_path = None  # which of the three ways the last forward took (diagnostics)
 
     def forward(self, point_cloud, feature, batch_ids):
@@ -63,6 +64,7 @@ class Point2Voxel(nn.Module):
                 sparse_feat = SparseTensor(voxel_feats, voxel_index,
                                            self.voxel_num_limit.astype(np.int64), B1)
                 self.last_path = "one call"
+                self._n_ids_hint = int(origin_ids[-1]) + 1
                 return valid_point_cloud, sparse_feat, valid_ids, valid_instance_flag
         fast = _ext.p2v_filter(point_cloud, feature, batch_ids, half, unit) \
             if point_cloud.is_cuda else None

@@ -1776,9 +1776,11 @@ def _p2v_same(a, b):
 
 @pytest.mark.parametrize("mode", [1, 2, 3, 4])
 def test_point2voxel_one_call_path(mode, oracle, device):
-    """A Point2Voxel module that has seen the range of batch ids once runs the whole forward
-    as one native call with one wait of the host.  Its result equals the oracle's and the
-    first call's, bit for bit: filtered points, ids, flags, voxel rows, voxel features."""
+    """Point2Voxel runs the whole forward as one native call with one wait of the host when
+    the batch ids fit the tables it sized beforehand (ids below 64 on a first call, below 1 +
+    the largest id of the last call afterwards).  Its result equals the oracle's and that of
+    the step-by-step path, bit for bit: filtered points, ids, flags, voxel rows, voxel
+    features."""
     from ss_conv.sp_ops.voxelize import Point2Voxel
     pts, feats, ids = synth.make_clouds(3, 700, seed=3, channels=6)
     pts = pts * 1.2  # some points fall outside and are filtered
@@ -1787,11 +1789,15 @@ def test_point2voxel_one_call_path(mode, oracle, device):
     ref = oracle.point2voxel(pts, feats, ids, [grid] * 3, [2.0 / grid] * 3, mode)
     p2v = Point2Voxel([grid] * 3, [2.0 / grid] * 3, mode)
     args = [torch.from_numpy(a).to(device) for a in (pts, feats, ids)]
+    p2v._n_ids_hint = None  # (no tables sized beforehand: the step-by-step path)
     first = p2v(*args)
     assert p2v.last_path == "native filter"
     second = p2v(*args)
     assert p2v.last_path == "one call"
     _p2v_same(first, second)
+    fresh = Point2Voxel([grid] * 3, [2.0 / grid] * 3, mode)
+    _p2v_same(fresh(*args), second)  # a module's first call
+    assert fresh.last_path == "one call"
     vp, st, vi, flag = second
     assert np.array_equal(vp.cpu().numpy(), ref["valid_points"])
     assert np.array_equal(vi.cpu().numpy(), ref["valid_ids"])
@@ -1828,7 +1834,9 @@ def test_point2voxel_one_call_crowded_voxels_and_wide_rows(mode, oracle, device)
     ref = oracle.point2voxel(pts, feats, ids, [grid] * 3, [2.0 / grid] * 3, mode)
     p2v = Point2Voxel([grid] * 3, [2.0 / grid] * 3, mode)
     args = [torch.from_numpy(a).to(device) for a in (pts, feats, ids)]
+    p2v._n_ids_hint = None  # (the step-by-step path first)
     first = p2v(*args)
+    assert p2v.last_path == "native filter"
     second = p2v(*args)
     assert p2v.last_path == "one call"
     _p2v_same(first, second)
@@ -1893,6 +1901,7 @@ def test_point2voxel_one_call_gradients(mode, oracle, device):
     tp, ti = torch.from_numpy(pts).to(device), torch.from_numpy(ids).to(device)
     grads = []
     gv = None
+    p2v._n_ids_hint = None  # (the first call by the other path)
     for _ in range(2):
         x = torch.from_numpy(feats).to(device).requires_grad_(True)
         vp, st, vi, _ = p2v(tp, x, ti)
