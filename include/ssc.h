@@ -382,7 +382,11 @@ int ssc_profile_conv(int32_t enable);
  *      estimated 250 row-block groups per workgroup or more, and no second split) otherwise
  *      cut the rows into two ranges per workgroup and give a workgroup two of them by the
  *      groups they came to, many with few.  Changes the sizes; results as for 16.
- * 128  two ranges to a workgroup for every plan (for tests). */
+ * 128  two ranges to a workgroup for every plan (for tests).
+ * 256  no kernel of its own for float layers of at most 8 input channels (the first layer of
+ *      a network on raw point features), which otherwise compute every output row in
+ *      registers from a table of its input rows instead of on the matrix pipeline.  Changes
+ *      the sizes; results agree up to the order of the float sums. */
 int ssc_conv_tuning(int32_t flags);
 int ssc_profile_conv_read(float *ms /* host */, int32_t capacity, int32_t *count /* host */);
 

@@ -14,7 +14,7 @@ CSRC = os.path.join(HERE, "csrc")
 LIB_DIR = os.path.join(HERE, "lib")
 LIB = os.path.join(LIB_DIR, "libssc.so")
 SOURCES = ["common.hip", "rulebook.hip", "conv.hip", "conv_epi.hip", "conv_tail.hip",
-           "conv_tail_epi.hip", "conv_five.hip", "conv_five_epi.hip", "conv_wide.hip", "conv_wide_epi.hip", "conv_bwd.hip", "combine.hip", "pool.hip", "voxel.hip", "bnact.hip"]
+           "conv_tail_epi.hip", "conv_five.hip", "conv_five_epi.hip", "conv_wide.hip", "conv_wide_epi.hip", "conv_small.hip", "conv_bwd.hip", "combine.hip", "pool.hip", "voxel.hip", "bnact.hip"]
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",
     # packed fp32 VALU ops are kept off for every device function of this library

@@ -1035,6 +1035,7 @@ static bool g_conv_pair = true, g_conv_pair_always = false;
 static int64_t g_conv_rebalance_stages = kRebalanceStages;
 static bool g_conv_rebalance = true;  // long kernels: a second work split from the first one's counts
 static bool g_conv_round8 = false;    // ranges per column block: a multiple of 8 only
+static bool g_conv_small = true;      // layers of at most 8 input channels: conv_small_kernel
 
 // The sizes that follow from the number of workgroups per column block.
 // `sizing`: the plan is only being sized (the number of input rows, and with it the number
@@ -1123,6 +1124,10 @@ static ConvPlan make_plan(int64_t n_in, int64_t n_out, int K, int c_in, int c_ou
                      (!p.rebalance && est_groups >= kPairGroups && est_groups >= (int64_t)K / 2));
   plan_split(p, n_wg, pair ? 2 * n_wg : n_wg, n_out, K, pair_stride, n_in <= 0);
   p.lds_bytes = conv_lds_bytes(p.T, p.acc_cols);
+  p.small = g_conv_small && conv_small_applies(K, c_in, c_out, elem_bytes);
+  if (p.small) p.rebalance = false;
+  p.kvol = K;
+  p.out_rows = n_out;
   return p;
 }
 
@@ -1134,6 +1139,12 @@ static size_t conv_packed_bytes(const ConvPlan &p, int K) {
 
 static size_t conv_plan_walk(void *base, const ConvPlan &p, ConvWs *w) {
   Carver c(base);
+  if (p.small) {  // the plan is the table of every output row's input rows, nothing else
+    int32_t *table =
+        c.take<int32_t>((size_t)p.kvol * (size_t)(p.out_rows > 0 ? p.out_rows : 1));
+    if (w) w->small_table = table;
+    return c.used;
+  }
   int32_t *wg_tile = c.take<int32_t>((size_t)p.n_rng + 1);
   int32_t *wg_grp = c.take<int32_t>((size_t)p.n_wg + 1);
   int32_t *sched_in = c.take<int32_t>((size_t)p.grp_cap * 64);
@@ -1222,9 +1233,16 @@ static size_t conv_ws_walk(void *base, const ConvPlan &p, int K, int64_t pair_st
 }
 
 static size_t conv_ws_bytes(int64_t n_out, int K, int c_in, int c_out, int64_t pair_stride) {
-  // the workspace does not depend on the number of input rows
+  // the workspace does not depend on the number of input rows (nor on the element type,
+  // which is not known here: room for the plan of either)
   ConvPlan p = make_plan(0, n_out, K, c_in, c_out, pair_stride);
-  return conv_ws_walk(nullptr, p, K, pair_stride, nullptr);
+  size_t bytes = conv_ws_walk(nullptr, p, K, pair_stride, nullptr);
+  if (p.small) {
+    p.small = false;
+    const size_t other = conv_ws_walk(nullptr, p, K, pair_stride, nullptr);
+    if (other > bytes) bytes = other;
+  }
+  return bytes;
 }
 
 // The launches of a plan (ConvPlan): the column blocks, all at once or one after the other,
@@ -1329,6 +1347,7 @@ int ssc_conv_tuning(int32_t flags) {
   g_conv_rebalance_stages = (flags & 32) != 0 ? 0 : kRebalanceStages;
   g_conv_pair = (flags & 64) == 0;
   g_conv_pair_always = (flags & 128) != 0;
+  g_conv_small = (flags & 256) == 0;
   return SSC_OK;
 }
 
@@ -1426,6 +1445,17 @@ static int conv_plan_build(const ConvPlan &p, const ConvWs &w, const int32_t *pa
     SSC_LAUNCH_CHECK("resort");
   }
 
+  if (p.small) {
+    // a layer of a handful of input channels: the plan is the table of every output row's
+    // input rows (conv_small.hip); the filters, if any, by a launch of their own
+    if (in_order && pack) {
+      hipLaunchKernelGGL(pack_filters_kernel<PACK_IO>, dim3((unsigned)ceil_div(packed_n, 256)),
+                         dim3(256), 0, s, pk, w.flag);
+      SSC_LAUNCH_CHECK("pack_filters");
+    }
+    return conv_small_build_table(w.flag, in_order, pairs, w.sorted, pair_stride, plane_s, pair_num,
+                                  K, n_out, w.small_table, s);
+  }
   // work split on the fine grid, then the tiles and their segments
   dim3 seg_grid = pair_grid;
   if (in_order) {  // extra rows: pack the filters (if any) and clear flag[0]
@@ -1496,6 +1526,20 @@ static int conv_run(const ConvPlan &p, const ConvWs &w, const IO *features, int6
   const bool prof = g_profile_on && (g_profile_calls++ % g_profile_every) == 0;
   const int slot = g_profile_count % kProfileRing;
   if (prof) SSC_HIP(hipEventRecord(g_profile_ev[slot][0], s));
+  if (p.small) {
+    if constexpr (sizeof(IO) == 4) {
+      rc = conv_small_run(features, c_in, w.packed, p.ncb, p.ns, w.small_table, K, out, c_out,
+                          p.out_rows, epi, s);
+      if (rc != SSC_OK) return rc;
+      if (prof) {
+        SSC_HIP(hipEventRecord(g_profile_ev[slot][1], s));
+        ++g_profile_count;
+      }
+      return SSC_OK;
+    } else {
+      SSC_CHECK(false, SSC_ERUNTIME, "the kernel for few input channels is built for float rows");
+    }
+  }
 #define SSC_CONV_LAUNCH(G, S) \
   launch_all<IO, G, S>(p, w, features, n_in, c_in, K, out, c_out, epi, s)
 #define SSC_CONV_BY_STEPS(G)                                                            \
@@ -1708,8 +1752,16 @@ size_t ssc_conv_packed_bytes(int32_t kernel_volume, int32_t c_in, int32_t c_out)
 size_t ssc_conv_plan_bytes(int64_t n_out, int32_t kernel_volume, int32_t c_in, int32_t c_out,
                            int64_t pair_stride) {
   if (n_out < 0 || kernel_volume < 1 || c_in < 1 || c_out < 1 || pair_stride < 0) return 0;
-  return conv_plan_walk(nullptr, make_plan(0, n_out, kernel_volume, c_in, c_out, pair_stride),
-                        nullptr);
+  // (the element type is not known here: room for the plan of either, which differ for
+  // layers of a handful of input channels)
+  ConvPlan p = make_plan(0, n_out, kernel_volume, c_in, c_out, pair_stride);
+  size_t bytes = conv_plan_walk(nullptr, p, nullptr);
+  if (p.small) {
+    p.small = false;
+    const size_t other = conv_plan_walk(nullptr, p, nullptr);
+    if (other > bytes) bytes = other;
+  }
+  return bytes;
 }
 
 size_t ssc_conv_plan_scratch_bytes(int64_t n_out, int32_t kernel_volume, int32_t c_in,
@@ -1771,7 +1823,7 @@ int ssc_rulebook_conv_begin(const int32_t *indices, int64_t n_in, const ssc_geom
     const ConvPlan p = make_plan(n_in, n_in + 1, (int)K, c_in, c_out, n_in, elem_bytes);
     ConvWs w = {};
     const size_t head = conv_scratch_head(scratch, &w);
-    if (!p.rebalance && scratch_bytes >= head) {
+    if (!p.rebalance && !p.small && scratch_bytes >= head) {
       rq.n_rng = p.n_rng;
       rq.tile_rows = p.tile_rows;
       rq.tile_cost = (long long)K * 4 + 64;  // split_tile_cost
@@ -1815,7 +1867,8 @@ int ssc_rulebook_conv_finish(const ssc_geometry *g, int64_t n_in, int32_t *n_out
   conv_plan_walk(plan, p, &w);
   conv_scratch_walk(scratch, p, K, n_in, &w);
   const bool in_order = *in_order_host != 0;
-  const bool seeded = pending.seeded && in_order && !p.rebalance && pending.n_rng == p.n_rng;
+  const bool seeded =
+      pending.seeded && in_order && !p.rebalance && !p.small && pending.n_rng == p.n_rng;
   return conv_plan_build<float>(p, w, pairs, n_in, pair_num, K, 0, in_order, c_in, n_out,
                                 elem_bytes, nullptr, (hipStream_t)stream, seeded);
 }

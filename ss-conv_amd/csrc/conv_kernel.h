@@ -1165,7 +1165,22 @@ struct ConvPlan {
   bool has_tail, five;
   bool rebalance;  // the work split is made twice, the second time from the first one's counts
   int acc_cols;  // accumulator columns of a workgroup: 64, or 80 in the five-group form
+  // a layer of a handful of input channels: no schedule, no matrix kernel -- the plan is a
+  // table of every output row's input rows and the rows are computed by conv_small_kernel
+  bool small;
+  int kvol;           // kernel volume and number of output rows the plan was made for
+  int64_t out_rows;
 };
+
+// conv_small.hip
+bool conv_small_applies(int K, int c_in, int c_out, int elem_bytes);
+int conv_small_build_table(const int32_t *flag, bool in_order, const int32_t *pairs,
+                           const int32_t *sorted, int64_t pair_stride, int plane_s,
+                           const int32_t *pair_num, int K, int64_t n_out, int32_t *table,
+                           hipStream_t s);
+int conv_small_run(const float *features, int c_in, const void *packed, int ncb, int ns,
+                   const int32_t *table, int K, float *out, int c_out, int64_t n_out,
+                   const ConvEpilogue &epi, hipStream_t s);
 
 // Device buffers of a convolution call, in three groups with different lifetimes:
 //   packed   the filters in MFMA fragment order: as long as the filters keep their values;
@@ -1178,6 +1193,7 @@ struct ConvWs {
   // plan
   int32_t *wg_tile, *wg_grp;  // first tile of every range; first group of every workgroup
   int32_t *sched_in, *sched_out, *grp_meta;
+  int32_t *small_table;  // [K, n_out] (plans of ConvPlan::small, which have nothing else)
   // scratch
   int32_t *flag;
   int32_t *segs;
