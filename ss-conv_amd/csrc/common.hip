@@ -109,6 +109,8 @@ struct ReadBack {
   char *pinned = nullptr;
   hipEvent_t done = nullptr;
   bool pending = false;
+  int ticket = 0;       // last ticket handed out (read_back_mirror_ticket)
+  int spin_ticket = 0;  // the wait in progress ends when this ticket shows up (0: on the event)
 };
 static thread_local ReadBack g_read_back;
 
@@ -117,7 +119,7 @@ static int read_back_init(ReadBack &r) {
   // address and coherent with the host at event boundaries)
   if (r.pinned == nullptr)
     SSC_HIP(hipHostMalloc((void **)&r.pinned, kReadBackBytes,
-                          hipHostMallocPortable | hipHostMallocMapped));
+                          hipHostMallocPortable | hipHostMallocMapped | hipHostMallocCoherent));
   if (r.done == nullptr) SSC_HIP(hipEventCreateWithFlags(&r.done, hipEventDisableTiming));
   return SSC_OK;
 }
@@ -132,12 +134,20 @@ int read_back_mirror(int32_t **mirror) {
   return SSC_OK;
 }
 
-int read_back_mirror_queued(hipStream_t s) {
+int read_back_mirror_queued(hipStream_t s, int ticket) {
   ReadBack &r = g_read_back;
   SSC_CHECK(r.done != nullptr, SSC_ERUNTIME, "read_back_mirror was not called on this thread");
   SSC_HIP(hipEventRecord(r.done, s));
   r.pending = true;
+  r.spin_ticket = ticket;
   return SSC_OK;
+}
+
+int read_back_mirror_ticket() {
+  ReadBack &r = g_read_back;
+  r.ticket = r.ticket >= 0x3FFFFFFF ? 1 : r.ticket + 1;  // never 0
+  if (r.pinned != nullptr) reinterpret_cast<volatile int32_t *>(r.pinned)[kMirrorTicket] = 0;
+  return r.ticket;
 }
 
 int read_back_begin(const void *src_dev, size_t bytes, hipStream_t s) {
@@ -156,6 +166,27 @@ int read_back_end(const void **view) {
   ReadBack &r = g_read_back;
   SSC_CHECK(r.pending, SSC_ERUNTIME, "no read-back was started on this thread");
   r.pending = false;
+  if (r.spin_ticket != 0) {
+    // The kernel that knows the results stores them in the pinned block and then, with a
+    // release at system scope, the ticket: the host sees both while the kernel -- which has
+    // other work to do -- still runs.  Should the store not show (it does on this
+    // hardware), the event behind the kernel ends the wait.
+    const volatile int32_t *m = reinterpret_cast<const volatile int32_t *>(r.pinned);
+    const int want = r.spin_ticket;
+    r.spin_ticket = 0;
+    for (unsigned spins = 1;; ++spins) {
+      if (m[kMirrorTicket] == want) break;
+      if ((spins & 1023u) == 0) {
+        const hipError_t e = hipEventQuery(r.done);
+        if (e == hipSuccess) break;
+        if (e != hipErrorNotReady)
+          return ::ssc::fail(SSC_EHIP, "hipEventQuery failed: %s", hipGetErrorString(e));
+      }
+    }
+    __atomic_thread_fence(__ATOMIC_ACQUIRE);
+    *view = r.pinned;
+    return SSC_OK;
+  }
   SSC_HIP(hipEventSynchronize(r.done));
   *view = r.pinned;
   return SSC_OK;

@@ -490,18 +490,15 @@ __global__ void __launch_bounds__(kScanThreads)
 // its first row being the rows below c.  Every such block first adds up the block sums of
 // rows and pairs in LDS (at most kSeedMaxBlocks of each); a range's lanes then find the scan
 // block by bisection there and the cell inside it by three rounds of 16 probes.
-__global__ void __launch_bounds__(kScanThreads)
-    prefix_split_kernel(const uint32_t *__restrict__ bits, int64_t n_words, int64_t n_scan_blocks,
-                        const int32_t *__restrict__ blocksum, int32_t *__restrict__ prefix,
-                        int32_t *__restrict__ total, int32_t *__restrict__ mirror,
-                        const int32_t *__restrict__ pairsum,
-                        const int32_t *__restrict__ seed_rows,
-                        const int32_t *__restrict__ seed_pairs, SplitRequest rq) {
-  if ((int64_t)blockIdx.x < n_scan_blocks) {
-    popc_prefix_block(bits, n_words, blocksum, prefix, total, mirror,
-                      (int64_t)blockIdx.x == n_scan_blocks - 1);
-    return;
-  }
+// The range boundaries of a SplitRequest (see prefix_split_kernel), for the group of 16
+// ranges `group` (kScanThreads threads).
+__device__ __forceinline__ void split_ranges_block(int group, int64_t n_words,
+                                                   int64_t n_scan_blocks,
+                                                   const int32_t *__restrict__ blocksum,
+                                                   const int32_t *__restrict__ pairsum,
+                                                   const int32_t *__restrict__ seed_rows,
+                                                   const int32_t *__restrict__ seed_pairs,
+                                                   const SplitRequest &rq) {
   __shared__ int rows_base[kSeedMaxBlocks + 1];
   __shared__ long long pairs_base[kSeedMaxBlocks + 1];
   __shared__ int lds[kScanThreads / 64 + 1];
@@ -560,7 +557,7 @@ __global__ void __launch_bounds__(kScanThreads)
   };
   static_assert(kScanBlockWords == 2048, "the cell search assumes scan blocks of 2048 words");
   const int sub = threadIdx.x & 15;
-  const int w = ((int)(blockIdx.x - n_scan_blocks) * (kScanThreads / 16)) + (threadIdx.x >> 4);
+  const int w = group * (kScanThreads / 16) + (threadIdx.x >> 4);
   const bool mine = w >= 1 && w < rq.n_rng;
   // ceil(total * w / n_rng); ranges without a target (w = 0, w >= n_rng) search for nothing
   long long target = mine ? (total_work * w + rq.n_rng - 1) / rq.n_rng : 0;
@@ -606,7 +603,37 @@ __global__ void __launch_bounds__(kScanThreads)
     }
   }
 }
-template <int KS>
+__global__ void __launch_bounds__(kScanThreads)
+    prefix_split_kernel(const uint32_t *__restrict__ bits, int64_t n_words, int64_t n_scan_blocks,
+                        const int32_t *__restrict__ blocksum, int32_t *__restrict__ prefix,
+                        int32_t *__restrict__ total, int32_t *__restrict__ mirror,
+                        const int32_t *__restrict__ pairsum,
+                        const int32_t *__restrict__ seed_rows,
+                        const int32_t *__restrict__ seed_pairs, SplitRequest rq) {
+  if ((int64_t)blockIdx.x < n_scan_blocks) {
+    popc_prefix_block(bits, n_words, blocksum, prefix, total, mirror,
+                      (int64_t)blockIdx.x == n_scan_blocks - 1);
+    return;
+  }
+  split_ranges_block((int)(blockIdx.x - n_scan_blocks), n_words, n_scan_blocks, blocksum, pairsum,
+                     seed_rows, seed_pairs, rq);
+}
+
+// What the two-level form of write_pairs_kernel needs besides the table: the scan blocks'
+// sums (the prefix of a word is then the sum of the blocks before its own plus its prefix
+// inside the block, seed_rows[]: no launch for the scan's second pass), a SplitRequest to
+// serve on the way (n_rng = 0: none), and where the totals go.
+struct TwoLevel {
+  const int32_t *blocksum, *pairsum, *seed_rows, *seed_pairs;
+  int64_t n_scan_blocks;
+  SplitRequest split;
+  int split_blocks;
+  int32_t *total, *mirror;
+  int ticket;
+  int clear_total;  // total[] lies in a table kept clean between calls: zero it once read
+};
+
+template <int KS, bool TWO>
 __global__ void __launch_bounds__(256)
     write_pairs_kernel(const int32_t *__restrict__ indices, int64_t n_in, Geom g,
                        const uint32_t *__restrict__ bits, const int32_t *__restrict__ prefix,
@@ -614,16 +641,81 @@ __global__ void __launch_bounds__(256)
                        const int32_t *__restrict__ chunk_prefix, int64_t n_chunks,
                        const int32_t *__restrict__ pair_num, int32_t *__restrict__ pairs,
                        int64_t n_words, int32_t *__restrict__ out_indices,
-                       uint32_t *__restrict__ clean, int64_t clean_words) {
-  if ((int)blockIdx.y >= g.ks[0]) {
+                       uint32_t *__restrict__ clean, int64_t clean_words, int row_blocks,
+                       TwoLevel two) {
+  __shared__ int base_s[TWO ? kSeedMaxBlocks + 1 : 1];
+  if constexpr (TWO) {
+    static_assert(kScanThreads == 256, "one block size for the table's scan and this kernel");
+    if (blockIdx.y == 0) {
+      // the first row of the grid (its blocks start first: the host is waiting for the
+      // totals): the range boundaries of the convolution's plan, and one block for the totals
+      if ((int)blockIdx.x < two.split_blocks) {
+        split_ranges_block((int)blockIdx.x, n_words, two.n_scan_blocks, two.blocksum, two.pairsum,
+                           two.seed_rows, two.seed_pairs, two.split);
+        return;
+      }
+      if ((int)blockIdx.x != two.split_blocks) return;
+    }
+    // sums of the scan blocks before every block (at most kSeedMaxBlocks of them)
+    __shared__ int lds[kScanThreads / 64 + 1];
+    constexpr int kPer = kSeedMaxBlocks / kScanThreads;
+    const int nb = (int)two.n_scan_blocks, first = threadIdx.x * kPer;
+    int r[kPer], sr = 0;
+#pragma unroll
+    for (int i = 0; i < kPer; ++i) {
+      r[i] = first + i < nb ? two.blocksum[first + i] : 0;
+      sr += r[i];
+    }
+    int tot;
+    int er = block_exclusive_scan(sr, lds, &tot);
+#pragma unroll
+    for (int i = 0; i < kPer; ++i) {
+      if (first + i <= nb) base_s[first + i] = er;
+      er += r[i];
+    }
+    if (threadIdx.x == kScanThreads - 1 && first + kPer <= nb) base_s[nb] = er;
+    __syncthreads();
+    if (blockIdx.y == 0) {
+      // the totals: the number of outputs and the flags, for later kernels and for the
+      // host, which is waiting for the ticket while this launch still runs
+      if (threadIdx.x == 0) {
+        two.total[0] = tot;
+        volatile int32_t *m = two.mirror;
+        m[0] = tot;
+        m[1] = two.total[1];
+        m[2] = two.total[2];
+        m[3] = two.total[3];
+        __hip_atomic_store(two.mirror + kMirrorTicket, two.ticket, __ATOMIC_RELEASE,
+                           __HIP_MEMORY_SCOPE_SYSTEM);
+        if (two.clear_total) {
+          two.total[0] = 0;
+          two.total[1] = 0;
+          two.total[2] = 0;
+          two.total[3] = 0;
+        }
+      }
+      return;
+    }
+  }
+  const int by = (int)blockIdx.y - (TWO ? 1 : 0);  // (the two-level form's first row is above)
+  if (by >= g.ks[0]) {
     // the rows of the grid beyond the kernel's x extent: the output rows, and the words of
     // a table that no kernel reads any more and the next call expects to find zero
-    const int64_t step = (int64_t)(gridDim.y - g.ks[0]) * gridDim.x * blockDim.x;
-    const int64_t w0 = ((int64_t)(blockIdx.y - g.ks[0]) * gridDim.x + blockIdx.x) * blockDim.x +
+    const int64_t step = (int64_t)row_blocks * gridDim.x * blockDim.x;
+    const int64_t w0 = ((int64_t)(by - g.ks[0]) * gridDim.x + blockIdx.x) * blockDim.x +
                        threadIdx.x;
-    if (out_indices != nullptr)
-      for (int64_t w = w0; w < n_words; w += step)
-        emit_rows_of_word(bits, prefix, w, g.os[0], g.os[1], g.os[2], out_indices);
+    if (out_indices != nullptr) {
+      for (int64_t w = w0; w < n_words; w += step) {
+        if constexpr (TWO) {
+          const uint32_t b = bits[w];
+          if (b != 0)
+            emit_rows_of_word_at(b, base_s[w >> 11] + two.seed_rows[w], w, g.os[0], g.os[1],
+                                 g.os[2], out_indices);
+        } else {
+          emit_rows_of_word(bits, prefix, w, g.os[0], g.os[1], g.os[2], out_indices);
+        }
+      }
+    }
     for (int64_t w = w0; w < clean_words; w += step) clean[w] = 0u;
     return;
   }
@@ -640,8 +732,10 @@ __global__ void __launch_bounds__(256)
   uint32_t word = 0xFFFFFFFFu, wbits = 0u;
   int wprefix = 0;
   // blockIdx.y = kx: the taps of one x offset per wave, for more waves in flight (a wave
-  // per (kx, ky) was tried and is no faster: the kernel is bound by its stores)
-  const int kx = blockIdx.y;
+  // per (kx, ky) was tried and is no faster, and fetching the table words of all (kx, ky)
+  // before any is used is slower, 15.5 against 13.7 us on the benchmark layer: the kernel is
+  // bound by its stores)
+  const int kx = by;
   int k = kx * g.ks[1] * g.ks[2];
   int ox = 0;
   const bool tr = g.tr != 0;
@@ -660,7 +754,8 @@ __global__ void __launch_bounds__(256)
       if (ok && (key >> 5) != word) {
         word = key >> 5;
         wbits = bits[word];
-        wprefix = prefix[word];
+        if constexpr (TWO) wprefix = base_s[word >> 11] + two.seed_rows[word];
+        else wprefix = prefix[word];
       }
       if (ok && g.subm) ok = (wbits >> (key & 31u)) & 1u;
       unsigned long long m = __ballot(ok);
@@ -803,7 +898,7 @@ static int rulebook_check(const ssc_geometry *g, Geom *gg, const int32_t *indice
 static int rulebook_mark_and_scan(const int32_t *indices, int64_t n_in, const Geom &gg,
                                   const RulebookWs &w, int32_t *pair_num, int32_t *mirror,
                                   hipStream_t s, const SplitRequest *split = nullptr,
-                                  bool table_is_clean = false) {
+                                  bool table_is_clean = false, bool two_level = false) {
   int rc;
   if (w.use_dense && pair_num != nullptr) {
     // input table cleared (with the totals) unless the caller keeps one that every call
@@ -819,7 +914,9 @@ static int rulebook_mark_and_scan(const int32_t *indices, int64_t n_in, const Ge
     SSC_LAUNCH_CHECK("mark_in_count");
     const int64_t word_blocks = w.table.n_scan_blocks;
     const int ks = (gg.ks[0] == gg.ks[1] && gg.ks[1] == gg.ks[2]) ? gg.ks[0] : 0;
-    const bool seed = split != nullptr && w.can_seed;
+    // (two_level: the launch of the pair lists works with the scan blocks' sums and the
+    // prefixes inside the blocks, which this kernel's seeded form leaves: no second pass)
+    const bool seed = (split != nullptr || two_level) && w.can_seed;
     auto kernel = seed ? (ks == 3   ? dilate_blocksum_kernel<3, true>
                           : ks == 5 ? dilate_blocksum_kernel<5, true>
                                     : dilate_blocksum_kernel<0, true>)
@@ -831,7 +928,8 @@ static int rulebook_mark_and_scan(const int32_t *indices, int64_t n_in, const Ge
                        w.table.blocksum, w.chunk_count, w.n_chunks, pair_num, w.seed_rows,
                        w.seed_pairs, w.pairsum);
     SSC_LAUNCH_CHECK("dilate_blocksum");
-    if (!seed) return bit_table_scan_prefix(w.table, s, mirror);
+    if (two_level) return SSC_OK;
+    if (!seed || split == nullptr) return bit_table_scan_prefix(w.table, s, mirror);
     // the scan's second pass, and beside it the range boundaries of the convolution's plan
     const int64_t split_blocks = ceil_div(split->n_rng, kScanThreads / 16);
     hipLaunchKernelGGL(prefix_split_kernel, dim3((unsigned)(word_blocks + split_blocks)),
@@ -866,7 +964,8 @@ static int rulebook_mark_and_scan(const int32_t *indices, int64_t n_in, const Ge
 static int rulebook_pairs(const int32_t *indices, int64_t n_in, const Geom &gg,
                           const RulebookWs &w, int32_t *out_indices, int32_t *pairs,
                           int32_t *pair_num, bool chunks_scanned, hipStream_t s,
-                          uint32_t *clean = nullptr, int64_t clean_words = 0) {
+                          uint32_t *clean = nullptr, int64_t clean_words = 0,
+                          const TwoLevel *two = nullptr) {
   unsigned chunk_blocks = (unsigned)ceil_div(w.n_chunks, 4);
   if (gg.subm) {  // a regular convolution's counts were taken while marking the table
     hipLaunchKernelGGL(rank_to_row_kernel, dim3((unsigned)ceil_div(n_in, 256)), dim3(256), 0, s,
@@ -891,12 +990,23 @@ static int rulebook_pairs(const int32_t *indices, int64_t n_in, const Geom &gg,
   }
   if (row_blocks > 4096) row_blocks = 4096;
   const int ks = gg.ks[1] == gg.ks[2] ? gg.ks[1] : 0;
-  auto kernel = ks == 3 ? write_pairs_kernel<3> : ks == 5 ? write_pairs_kernel<5>
-                : ks == 2 ? write_pairs_kernel<2> : write_pairs_kernel<0>;
+  if (two != nullptr) {  // one more row of the grid: range boundaries and totals
+    auto kernel = ks == 3 ? write_pairs_kernel<3, true> : ks == 5 ? write_pairs_kernel<5, true>
+                  : ks == 2 ? write_pairs_kernel<2, true> : write_pairs_kernel<0, true>;
+    hipLaunchKernelGGL(kernel, dim3(chunk_blocks, (unsigned)(gg.ks[0] + row_blocks + 1)),
+                       dim3(256), 0, s, indices, n_in, gg, w.table.bits, w.table.prefix, w.rank2row,
+                       w.chunk_count, w.n_chunks, pair_num, pairs, w.table.n_words, out_indices,
+                       clean, clean_words, (int)row_blocks, *two);
+    SSC_LAUNCH_CHECK("write_pairs");
+    return SSC_OK;
+  }
+  auto kernel = ks == 3 ? write_pairs_kernel<3, false> : ks == 5 ? write_pairs_kernel<5, false>
+                : ks == 2 ? write_pairs_kernel<2, false> : write_pairs_kernel<0, false>;
   hipLaunchKernelGGL(kernel, dim3(chunk_blocks, (unsigned)(gg.ks[0] + row_blocks)), dim3(256), 0,
                      s, indices, n_in, gg, w.table.bits, w.table.prefix, w.rank2row, w.chunk_count,
                      w.n_chunks, pair_num, pairs, w.table.n_words,
-                     gg.subm ? (int32_t *)nullptr : out_indices, clean, clean_words);
+                     gg.subm ? (int32_t *)nullptr : out_indices, clean, clean_words,
+                     (int)row_blocks, TwoLevel{});
   SSC_LAUNCH_CHECK("write_pairs");
   return SSC_OK;
 }
@@ -1032,12 +1142,31 @@ int ssc::rulebook_begin_impl(const int32_t *indices, int64_t n_in, const ssc_geo
     w.table.total = static_cast<int32_t *>(clean_table);
     w.in_bits = clean + kCleanHeader / 4;
   }
+  // With room for the output rows at hand the dilation path needs no launch for the scan's
+  // second pass: the launch of the pair lists takes the prefixes in two levels, places the
+  // range boundaries and hands the totals to the host, which sees them (read_back_end) while
+  // that launch still runs.
+  const int split_blocks = split ? (int)ceil_div(split->n_rng, kScanThreads / 16) : 0;
+  const bool two_level = w.use_dense && w.can_seed && out_indices != nullptr &&
+                         ceil_div(w.n_chunks, 4) > split_blocks;
   if ((rc = rulebook_mark_and_scan(indices, n_in, gg, w, pair_num, mirror, s, split,
-                                   clean != nullptr)) != SSC_OK)
+                                   clean != nullptr, two_level)) != SSC_OK)
     return rc;
-  if ((rc = read_back_mirror_queued(s)) != SSC_OK) return rc;
-  return rulebook_pairs(indices, n_in, gg, w, out_indices, pairs, pair_num, true, s, clean,
-                        clean_words);
+  if (!two_level) {
+    if ((rc = read_back_mirror_queued(s)) != SSC_OK) return rc;
+    return rulebook_pairs(indices, n_in, gg, w, out_indices, pairs, pair_num, true, s, clean,
+                          clean_words);
+  }
+  TwoLevel two = {w.table.blocksum, w.pairsum, w.seed_rows, w.seed_pairs, w.table.n_scan_blocks,
+                  split ? *split : SplitRequest{0, 0, 0, nullptr}, split_blocks, w.table.total,
+                  mirror, read_back_mirror_ticket(), clean != nullptr ? 1 : 0};
+  // (the header of a clean table holds the totals: the block that hands them to the host
+  // clears it, the other blocks the words behind it)
+  if ((rc = rulebook_pairs(indices, n_in, gg, w, out_indices, pairs, pair_num, true, s,
+                           clean ? clean + kCleanHeader / 4 : nullptr,
+                           clean ? clean_words - (int64_t)(kCleanHeader / 4) : 0, &two)) != SSC_OK)
+    return rc;
+  return read_back_mirror_queued(s, two.ticket);
 }
 
 extern "C" {

@@ -169,13 +169,21 @@ __device__ __forceinline__ int bit_rank(const uint32_t *__restrict__ bits,
 }
 
 // Decode every set bit of word w into its (b,x,y,z) row, written at the bit's rank.
+__device__ __forceinline__ void emit_rows_of_word_at(uint32_t b, int r, int64_t w, int d1,
+                                                     int d2, int d3,
+                                                     int32_t *__restrict__ out);
 __device__ __forceinline__ void emit_rows_of_word(const uint32_t *__restrict__ bits,
                                                   const int32_t *__restrict__ prefix, int64_t w,
                                                   int d1, int d2, int d3,
                                                   int32_t *__restrict__ out) {
-  uint32_t b = bits[w];
+  const uint32_t b = bits[w];
   if (b == 0) return;
-  int r = prefix[w];
+  emit_rows_of_word_at(b, prefix[w], w, d1, d2, d3, out);
+}
+// The same for a word b whose first set bit has rank r.
+__device__ __forceinline__ void emit_rows_of_word_at(uint32_t b, int r, int64_t w, int d1,
+                                                     int d2, int d3,
+                                                     int32_t *__restrict__ out) {
   // the word's first cell is decoded once; its other cells differ in z only, unless
   // the word runs over the end of a z row (extents that are not multiples of 32)
   uint32_t key0 = (uint32_t)(w * 32);
@@ -211,7 +219,8 @@ __device__ __forceinline__ void emit_rows_of_word(const uint32_t *__restrict__ b
 // the rulebook can place the ranges' boundaries itself, in a launch it makes anyway: the
 // plan is then built without its own passes over the pairs for that purpose.
 constexpr int kMaxRanges = 512;       // two for each of at most 256 workgroups
-constexpr int kSeedMaxBlocks = 2048;  // scan blocks of a table whose block sums fit in LDS
+constexpr int kSeedMaxBlocks = 512;   // scan blocks of a table whose block sums are scanned in LDS by
+                                      // every block that needs them (512: 33 M cells)
 struct SplitRequest {
   int n_rng;           // ranges to cut the output rows into (<= kMaxRanges)
   int tile_rows;       // weight of a pair relative to tile_cost (see split_work in conv.hip)
@@ -245,7 +254,14 @@ int read_back_end(const void **view);
 // it; a kernel queued on `s` writes its results there, read_back_mirror_queued records the
 // event behind that kernel, and read_back_end waits for it and returns the block.
 int read_back_mirror(int32_t **mirror);
-int read_back_mirror_queued(hipStream_t s);
+int read_back_mirror_queued(hipStream_t s, int ticket = 0);
+// For a kernel that stores its results into the mirror while it still has other work to
+// do: the kernel stores the results, then `ticket` (read_back_mirror_ticket(), never 0) into
+// mirror[kMirrorTicket] with a release at system scope; read_back_mirror_queued(s, ticket)
+// behind the launch; read_back_end then returns as soon as the ticket shows up in the host's
+// view of the block, not when the kernel ends.
+constexpr int kMirrorTicket = 8;
+int read_back_mirror_ticket();
 // The same, moved on to `dst_host`.
 int read_back(void *dst_host, const void *src_dev, size_t bytes, hipStream_t s);
 
