@@ -229,19 +229,40 @@ _PLAN_AHEAD_BYTES = 256 << 20
 
 
 class RulebookMeta(object):
-    """What the library knows about a pairs tensor that it wrote itself: for which direction
-    the pairs of every offset ascend in the rows that are accumulated into (`canonical`:
-    (forward, inverse)), and the convolution plans built over it so far.  It hangs on the
-    tensor object as ``_ssc_meta`` and counts only while the tensor's version counter stands
-    where it stood when the rulebook was written: an in-place edit of the pairs makes the
-    convolution treat them as pairs of unknown origin."""
-    __slots__ = ("version", "canonical", "plans")
+    """What the library knows about a rulebook it wrote itself: for which direction the pairs
+    of every offset ascend in the rows that are accumulated into (`canonical`: (forward,
+    inverse)), and the convolution plans built over it so far (`plans`, least recently used
+    first; at most MAX_PLANS are kept).
+
+    The owner is the SparseTensor: ``plan_dict[indice_key]`` holds it beside
+    ``indice_dict[indice_key]`` and travels with it to the layer's outputs.  For the native
+    calls, which get tensors and nothing else, a binding to the pairs tensor rides on the
+    tensor object (``_ssc_meta``), valid while that tensor's version counter stands where it
+    stood: an in-place edit of the pairs makes the convolution treat them as pairs of unknown
+    origin.  A pairs tensor of other identity (a clone, a tensor that came back from a
+    checkpoint) is bound to the same plans by adopt_meta once it has been compared with the
+    tensor the plans were built over."""
+    __slots__ = ("version", "canonical", "plans", "pairs_ref")
     MAX_PLANS = 8
 
-    def __init__(self, version, canonical):
+    def __init__(self, version, canonical, plans=None, pairs_ref=None):
+        import collections
         self.version = version
         self.canonical = canonical
-        self.plans = {}
+        self.plans = collections.OrderedDict() if plans is None else plans
+        self.pairs_ref = pairs_ref  # the tensor the plans were built over
+
+    def get_plan(self, key):
+        plan = self.plans.get(key)
+        if plan is not None:
+            self.plans.move_to_end(key)
+        return plan
+
+    def put_plan(self, key, plan):
+        self.plans[key] = plan
+        self.plans.move_to_end(key)
+        while len(self.plans) > RulebookMeta.MAX_PLANS:
+            self.plans.popitem(last=False)  # the least recently used one
 
 
 def rulebook_meta(indice_pairs):
@@ -251,6 +272,38 @@ def rulebook_meta(indice_pairs):
             indice_pairs.dtype != torch.int32 or not indice_pairs.is_contiguous():
         return None
     return meta
+
+
+def adopt_meta(indice_pairs, meta):
+    """Bind `indice_pairs` to the plans of `meta` (the record a SparseTensor keeps under the
+    rulebook's indice_key) when the tensor carries no valid binding of its own: at once when
+    it is the tensor the plans were built over, after one comparison of the contents when it
+    is another tensor of the same shape (a clone).  Returns the binding in force, or None."""
+    own = rulebook_meta(indice_pairs)
+    if own is not None or meta is None:
+        return own
+    ref = meta.pairs_ref
+    if ref is None or not indice_pairs.is_cuda or indice_pairs.dtype != torch.int32 or \
+            not indice_pairs.is_contiguous() or indice_pairs.shape != ref.shape or \
+            indice_pairs.device != ref.device:
+        return None
+    same = indice_pairs.data_ptr() == ref.data_ptr() and indice_pairs._version == meta.version
+    if not same:
+        if ref._version != meta.version or not bool(torch.equal(indice_pairs, ref)):
+            return None
+    bound = RulebookMeta(indice_pairs._version, meta.canonical, plans=meta.plans,
+                         pairs_ref=indice_pairs)
+    indice_pairs._ssc_meta = bound
+    return bound
+
+
+def forget_packed(filters):
+    """Drop the packed copy of `filters` that the convolution keeps with the tensor.  The
+    copy is reused while the tensor's version counter stands still, and an edit through
+    ``.data`` (``w.data.copy_(...)``, an EMA swap, ``w.data.normal_()``) does not move that
+    counter: call this after such an edit."""
+    if hasattr(filters, "_ssc_packed"):
+        del filters._ssc_packed
 
 
 # One buffer per (device, stream) that every rulebook call finds all zero and leaves all
@@ -389,7 +442,7 @@ def _rulebook_result(r, n_out, in_order):
     # the input rows came in key order: the convolution may then skip its order check
     # (the first flag serves a call that accumulates into output rows, the second one
     # with `inverse`, which accumulates into input rows).
-    r.pairs._ssc_meta = RulebookMeta(r.pairs._version, (in_order, True))
+    r.pairs._ssc_meta = RulebookMeta(r.pairs._version, (in_order, True), pairs_ref=r.pairs)
     return [outids, r.pairs, r.num]
 
 
@@ -471,7 +524,7 @@ def _plan_of(meta, pairs, num, K, c_in, c_out, elem_bytes, n_in, n_out, inverse,
     a rulebook: built on first use, kept with the rulebook afterwards."""
     stride = pairs.size(2)
     key = (bool(inverse), c_in, c_out, elem_bytes, n_in, n_out)
-    plan = meta.plans.get(key)
+    plan = meta.get_plan(key)
     if plan is None:
         plan = _workspace(_lib.ssc_conv_plan_bytes(n_out, K, c_in, c_out, stride), dev)
         scratch = _workspace(_lib.ssc_conv_plan_scratch_bytes(n_out, K, c_in, c_out, stride), dev)
@@ -480,9 +533,7 @@ def _plan_of(meta, pairs, num, K, c_in, c_out, elem_bytes, n_in, n_out, inverse,
                                         flags, n_in, n_out, c_in, c_out, elem_bytes,
                                         plan.data_ptr(), plan.numel(), scratch.data_ptr(),
                                         scratch.numel(), stream))
-        if len(meta.plans) >= RulebookMeta.MAX_PLANS:
-            meta.plans.clear()
-        meta.plans[key] = plan
+        meta.put_plan(key, plan)
     return plan
 
 
@@ -604,7 +655,7 @@ def rulebook_conv(features, filters, indices, batch_size, out_spatial_shape, ker
     out = _run_planned(features, n_in, c_in, packed, r.plan, n_in, K, c_out, n_out, s, epilogue)
     outids, pairs, num = _rulebook_result(r, n_out, in_order)
     if n_out > 0:
-        pairs._ssc_meta.plans[(False, c_in, c_out, eb, n_in, n_out)] = r.plan
+        pairs._ssc_meta.put_plan((False, c_in, c_out, eb, n_in, n_out), r.plan)
     return out, outids, pairs, num
 
 

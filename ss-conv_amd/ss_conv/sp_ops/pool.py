@@ -41,6 +41,7 @@ class _SparsePool(nn.Module):
                                       indice_pairs_num.to(device), outids.shape[0])
         out_tensor = SparseTensor(out_features, outids, out_spatial_shape, batch_size)
         out_tensor.indice_dict = input.indice_dict
+        out_tensor.plan_dict = getattr(input, "plan_dict", {})
         out_tensor.grid = input.grid
         return out_tensor
 

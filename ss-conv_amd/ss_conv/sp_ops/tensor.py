@@ -20,7 +20,10 @@ class SparseTensor(object):
     ``indice_dict`` caches rulebooks under their ``indice_key`` as
     (outids, indices, pairs, pair_num, spatial_shape) (reference: sp_ops/conv.py:136);
     ``grid`` is carried for signature parity only: the rulebook needs no dense
-    int32 grid here.
+    int32 grid here.  ``plan_dict`` holds, under the same keys, what the native
+    convolution keeps with a rulebook (order promises and the plans built over it,
+    ss_conv._ext.RulebookMeta); like ``indice_dict`` it is shared with the tensors a
+    layer returns.
     """
 
     def __init__(self, features, indices, spatial_shape, batch_size, grid=None):
@@ -29,6 +32,7 @@ class SparseTensor(object):
         self.spatial_shape = spatial_shape
         self.batch_size = batch_size
         self.indice_dict = {}
+        self.plan_dict = {}
         self.grid = grid
 
     @property

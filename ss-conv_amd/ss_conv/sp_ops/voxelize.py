@@ -61,8 +61,11 @@ class Point2Voxel(nn.Module):
                 B1 = len(origin_ids)
                 valid_instance_flag = torch.ones(B1, dtype=torch.float32, device=device) \
                     if bool(alive.all()) else torch.from_numpy(alive).to(device)
+                # (the rows carry the clouds' own ids: with gaps in the ids the tensor's batch
+                # size is 1 + the largest one, so that every row lies inside the grid)
                 sparse_feat = SparseTensor(voxel_feats, voxel_index,
-                                           self.voxel_num_limit.astype(np.int64), B1)
+                                           self.voxel_num_limit.astype(np.int64),
+                                           max(B1, int(origin_ids[-1]) + 1))
                 self.last_path = "one call"
                 self._n_ids_hint = int(origin_ids[-1]) + 1
                 return valid_point_cloud, sparse_feat, valid_ids, valid_instance_flag
@@ -136,7 +139,7 @@ class Point2Voxel(nn.Module):
         sparse_feat = voxelization(valid_feature.float().contiguous(), v2p_maps.detach(),
                                    self.voxelization_mode)
         sparse_feat = SparseTensor(sparse_feat, occupied_index.detach(),
-                                   self.voxel_num_limit.astype(np.int64), B1)
+                                   self.voxel_num_limit.astype(np.int64), max(B1, max_id + 1))
         return valid_point_cloud, sparse_feat, valid_ids, valid_instance_flag
 
 

@@ -681,7 +681,7 @@ def test_point2voxel_matches_oracle(mode, oracle, device):
     assert np.array_equal(vi.cpu().numpy(), ref["valid_ids"])
     assert np.array_equal(flag.cpu().numpy(), ref["flag"])
     assert np.array_equal(st.indices.cpu().numpy(), ref["indices"])
-    assert st.batch_size == ref["batch_size"]
+    assert st.batch_size == max(ref["batch_size"], int(ref["valid_ids"].max()) + 1)
     assert np.array_equal(st.features.cpu().numpy(), ref["features"])
 
 
@@ -727,6 +727,37 @@ def test_point2voxel_empty_batch_element(oracle, device):
         torch.from_numpy(ids).to(device))
     assert flag.cpu().tolist() == [0.0, 0.0, 0.0]
     assert np.array_equal(st.indices.cpu().numpy(), ref["indices"])
+
+
+def test_point2voxel_gapped_ids_feed_a_convolution(oracle, device):
+    """Clouds whose batch ids have gaps (1, 4, 6): the SparseTensor's batch size is 1 + the
+    largest id, so the layer that follows finds every row inside its grid, and its result is
+    that of the same clouds numbered 0, 1, 2."""
+    from ss_conv.sp_ops.conv import SparseConvolution
+    from ss_conv.sp_ops.voxelize import Point2Voxel
+    pts, feats, ids = synth.make_clouds(3, 300, seed=5, channels=4)
+    gapped = np.array([1, 4, 6], dtype=np.int64)[ids]
+    grid = 8
+    torch.manual_seed(0)
+    conv = SparseConvolution(3, 4, 6, 3, stride=1, padding=1, bias=False).to(device)
+    outs = []
+    for use in (ids, gapped):
+        p2v = Point2Voxel([grid] * 3, [2.0 / grid] * 3)
+        _, st, _, _ = p2v(*[torch.from_numpy(a).to(device) for a in (pts, feats, use)])
+        assert st.batch_size == int(use.max()) + 1
+        with torch.no_grad():
+            outs.append(conv(st))
+    a, b = outs
+    remap = torch.tensor([1, 4, 6], dtype=torch.int32, device=device)
+    assert torch.equal(remap[a.indices[:, 0].long()], b.indices[:, 0])
+    assert torch.equal(a.indices[:, 1:], b.indices[:, 1:])
+    assert torch.equal(a.features, b.features)
+    for mod in (1, 2):  # both paths of the module (one call; filter, unique, lists)
+        p2v = Point2Voxel([grid] * 3, [2.0 / grid] * 3)
+        if mod == 2:
+            p2v._n_ids_hint = None
+        _, st, _, _ = p2v(*[torch.from_numpy(x).to(device) for x in (pts, feats, gapped)])
+        assert st.batch_size == 7
 
 
 def test_point2voxel_unsorted_ids_and_outliers(oracle, device):
@@ -795,7 +826,7 @@ def test_point_voxel_random_configurations(seed, oracle, device):
         assert np.array_equal(vi.cpu().numpy(), ref["valid_ids"]), case
         assert np.array_equal(flag.cpu().numpy(), ref["flag"]), case
         assert np.array_equal(st.indices.cpu().numpy(), ref["indices"]), case
-        assert st.batch_size == ref["batch_size"], case
+        assert st.batch_size == max(ref["batch_size"], int(ref["valid_ids"].max()) + 1), case
         assert np.array_equal(st.features.cpu().numpy(), ref["features"]), case
         v2p = Voxel2Point(unit_voxel_extent=unit)
         out = v2p(st, vp, vi)
@@ -1693,6 +1724,81 @@ def test_layer_reuses_plan_under_an_indice_key(device):
         assert torch.equal(z, y.features)
 
 
+def test_cloned_pairs_keep_their_plan(device):
+    """The plans of a rulebook belong to the SparseTensor (plan_dict, keyed like indice_dict),
+    not to one tensor object: pairs that come back as a clone under the same key are bound
+    to the same plans after one comparison, pairs with other contents are not, and the plans
+    kept per rulebook are evicted least recently used first."""
+    from ss_conv import _ext
+    from ss_conv.sp_ops.conv import SparseConvolution
+    from ss_conv.sp_ops.tensor import SparseTensor
+    rng = np.random.default_rng(3)
+    idx = random_voxels(rng, 2, 12, 700)
+    t = torch.from_numpy(idx).to(device)
+    torch.manual_seed(5)
+    layer = SparseConvolution(3, 16, 24, 3, stride=1, padding=1, subm=True, bias=False,
+                              indice_key="s").to(device)
+    x = torch.randn((idx.shape[0], 16), device=device)
+    with torch.no_grad():
+        st = SparseTensor(x, t, [12] * 3, 2)
+        y = layer(st)
+        meta = st.plan_dict["s"]
+        assert y.plan_dict is st.plan_dict and len(meta.plans) == 1
+        plan = next(iter(meta.plans.values()))
+        # the same rulebook as other tensor objects
+        outids, ind, pairs, num, shape = st.indice_dict["s"]
+        st2 = SparseTensor(x, t, [12] * 3, 2)
+        st2.indice_dict = {"s": (outids, ind, pairs.clone(), num.clone(), shape)}
+        st2.plan_dict = st.plan_dict
+        calls = []
+        keep = _ext._lib.ssc_conv_plan_build
+        _ext._lib.ssc_conv_plan_build = lambda *a: calls.append(1) or keep(*a)
+        try:
+            y2 = layer(st2)
+        finally:
+            _ext._lib.ssc_conv_plan_build = keep
+        assert not calls and torch.equal(y2.features, y.features)
+        assert next(iter(st.plan_dict["s"].plans.values())) is plan
+        # other pairs under the key: no binding, the call builds its own schedule
+        other = pairs.clone()
+        other[0, :, :2] = pairs[0, :, :2].flip(1)  # the same pairs in another order
+        st3 = SparseTensor(x, t, [12] * 3, 2)
+        st3.indice_dict = {"s": (outids, ind, other, num, shape)}
+        st3.plan_dict = st.plan_dict
+        y3 = layer(st3)
+        assert _ext.rulebook_meta(other) is None
+        assert rel_l2(y3.features.cpu().numpy(), y.features.cpu().numpy()) < 1e-6
+        # least recently used first
+        for c in range(_ext.RulebookMeta.MAX_PLANS + 2):
+            meta.put_plan(("k", c), object())
+            assert meta.get_plan(("k", 0)) is not None  # kept alive by use
+        assert len(meta.plans) == _ext.RulebookMeta.MAX_PLANS
+        assert meta.get_plan(("k", 1)) is None and meta.get_plan(("k", 0)) is not None
+
+
+def test_packed_filters_follow_explicit_invalidation(device):
+    """The packed copy of a layer's filters is reused while the weight's version counter
+    stands still; an edit through .data does not move it, forget_packed does."""
+    from ss_conv import _ext
+    from ss_conv.sp_ops.conv import SparseConvolution
+    from ss_conv.sp_ops.tensor import SparseTensor
+    rng = np.random.default_rng(4)
+    idx = random_voxels(rng, 1, 10, 300)
+    t = torch.from_numpy(idx).to(device)
+    torch.manual_seed(6)
+    layer = SparseConvolution(3, 8, 8, 3, stride=1, padding=1, bias=False).to(device).eval()
+    x = torch.randn((idx.shape[0], 8), device=device)
+    with torch.no_grad():
+        y0 = layer(SparseTensor(x, t, [10] * 3, 1)).features
+        layer.weight.mul_(2.0)  # moves the version counter: repacked
+        y1 = layer(SparseTensor(x, t, [10] * 3, 1)).features
+        assert torch.allclose(y1, 2.0 * y0, rtol=1e-6, atol=1e-6)
+        layer.weight.data.mul_(0.5)  # does not: the stale copy is used until told
+        _ext.forget_packed(layer.weight)
+        y2 = layer(SparseTensor(x, t, [10] * 3, 1)).features
+        assert torch.allclose(y2, y0, rtol=1e-6, atol=1e-6)
+
+
 @pytest.mark.parametrize("subm,stride", [(False, 1), (False, 2), (True, 1)])
 def test_fused_rulebook_conv_equals_the_two_calls(subm, stride, device):
     """A layer without a cached rulebook runs rulebook and convolution as one native
@@ -1803,7 +1909,7 @@ def test_point2voxel_one_call_path(mode, oracle, device):
     assert np.array_equal(vi.cpu().numpy(), ref["valid_ids"])
     assert np.array_equal(flag.cpu().numpy(), ref["flag"])
     assert np.array_equal(st.indices.cpu().numpy(), ref["indices"])
-    assert st.batch_size == ref["batch_size"]
+    assert st.batch_size == max(ref["batch_size"], int(ref["valid_ids"].max()) + 1)
     assert np.array_equal(st.features.cpu().numpy(), ref["features"])
     # ids beyond what the module has seen: the call notices and another path is taken
     more = ids + 5
