@@ -153,14 +153,28 @@ int ssc_rulebook_rows(const ssc_geometry *g, int64_t n_in, void *workspace,
  *     rows and the input rows came in key order, the plan needs three launches instead of six.
  * Same host thread for both; one layer between them at a time.  The plan is the one
  * ssc_conv_run_* expects; compared with ssc_conv_plan_build's the ranges begin at other
- * rows, so results agree up to the order of the float sums. */
+ * rows, so results agree up to the order of the float sums.
+ * `filters` (may be NULL): the arguments of ssc_kernel_combine_packed_f32 for the layer's
+ * own filters (c_in and c_out are the call's).  The synthesis depends on nothing the
+ * rulebook computes, so it is enqueued inside the rulebook's first launch where that launch
+ * has a grid to share (stride 1, dilation 1) and as a launch of its own before it elsewhere:
+ * either way `out` and `packed` are ready for whatever the stream runs after this call. */
+typedef struct ssc_combine_job {
+  const float *weight, *basis;
+  const int32_t *chan_out, *chan_in, *blocks;
+  int32_t n_irreps_in, kernel_volume;
+  float *out;   /* [K,c_in,c_out] */
+  void *packed; /* ssc_conv_packed_bytes(kernel_volume, c_in, c_out) */
+  size_t packed_bytes;
+} ssc_combine_job;
 int ssc_rulebook_conv_begin(const int32_t *indices, int64_t n_in, const ssc_geometry *g,
                             void *workspace, size_t workspace_bytes,
                             int32_t *pairs /* [K,2,n_in] */, int32_t *pair_num /* [K] */,
                             int32_t *out_indices /* [out_capacity,4] or NULL */,
                             int64_t out_capacity, void *clean_table, size_t clean_table_bytes,
                             int32_t c_in, int32_t c_out, int32_t elem_bytes, void *scratch,
-                            size_t scratch_bytes, ssc_stream_t stream);
+                            size_t scratch_bytes, const ssc_combine_job *filters,
+                            ssc_stream_t stream);
 int ssc_rulebook_conv_finish(const ssc_geometry *g, int64_t n_in, int32_t *n_out_host /* host */,
                              int32_t *in_order_host /* host */, const int32_t *pairs,
                              const int32_t *pair_num, int32_t c_in, int32_t c_out,

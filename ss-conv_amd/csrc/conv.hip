@@ -17,9 +17,11 @@
 // launch the persistent kernel.
 #include "combine_element.h"
 #include "conv_kernel.h"
+#include "conv_pack.h"
 #include "ssc_common.h"
 
 namespace ssc {
+static_assert(kPackKC == kKC, "conv_pack.h packs half filters in chunks of kKC channels");
 
 
 // ---- weight packing ---------------------------------------------------------------------
@@ -48,58 +50,6 @@ namespace ssc {
 // i.e. one 16-byte load per lane and step.  Which of a step's 32 channels sits in which of
 // a lane's 8 slots does not matter for the sum as long as the staged rows use the same
 // assignment; they do (lane group g reads channels 32q + 8g .. +7 of its row).
-struct PackArgs {
-  const void *w;  // filters, addressed as w[k*fs_k + ci*fs_ci + co*fs_co]
-  int64_t fs_k, fs_ci, fs_co;
-  int K, cin, cout, ncb, nch;
-  void *packed_out;
-  int ns;  // MFMA steps per chunk (float filters; half filters always use whole chunks)
-};
-
-// Offset k, input channel ci and output channel co of element idx of the packed filters
-// (ci >= cin or co >= cout: a padding element).
-template <typename IO>
-__device__ __forceinline__ void pack_decode(const PackArgs &a, int64_t idx, int &k, int &ci,
-                                            int &co) {
-  const int cin = a.cin, ncb = a.ncb, nch = a.nch;
-  int64_t r = idx >> 10;
-  int cc = r % nch;
-  r /= nch;
-  int cb = r % ncb;
-  k = (int)(r / ncb);
-  int lane;
-  if constexpr (sizeof(IO) == 2) {
-    const int j = idx & 7, q = (idx >> 9) & 1;
-    lane = (idx >> 3) & 63;
-    ci = cc * kKC + 32 * q + (lane >> 4) * 8 + j;
-  } else {
-    const int full = a.ns >> 2, rem = a.ns & 3;
-    const int f = (int)(idx & 1023);  // float inside the fragment
-    int cl = -1;  // channel inside the chunk, -1 for a slot without one
-    lane = (f >> 2) & 63;
-    if (f < full * 256) {
-      cl = (f >> 8) * 16 + (lane >> 4) * 4 + (f & 3);
-    } else if (f - full * 256 < 64 * rem) {  // the partly used quarter, rem floats per lane
-      const int t = f - full * 256;
-      lane = t / rem;
-      cl = full * 16 + (t - lane * rem) * 4 + (lane >> 4);
-    }
-    ci = cl < 0 ? cin : cc * (4 * a.ns) + cl;
-  }
-  co = cb * 16 + (lane & 15);
-}
-
-// Element idx of the packed filters.
-template <typename IO>
-__device__ __forceinline__ void pack_filter_element(const PackArgs &a, int64_t idx) {
-  const IO *__restrict__ w = static_cast<const IO *>(a.w);
-  int k, ci, co;
-  pack_decode<IO>(a, idx, k, ci, co);
-  IO v = (IO)0.f;
-  if (ci < a.cin && co < a.cout) v = w[k * a.fs_k + ci * a.fs_ci + co * a.fs_co];
-  static_cast<IO *>(a.packed_out)[idx] = v;
-}
-
 // Synthesis of the dense float kernel and its packing in one launch: one thread per packed
 // element computes the element (combine_element), stores it at its place in the packed
 // filters and in the dense [K, Cin, Cout] array (every dense element has exactly one packed
@@ -111,14 +61,18 @@ __global__ void __launch_bounds__(256)
                         int n_j, float *__restrict__ dense) {
   int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (idx >= (int64_t)a.K * a.ncb * a.nch * 1024) return;
-  int k, ci, co;
-  pack_decode<float>(a, idx, k, ci, co);
-  float v = 0.f;
-  if (ci < a.cin && co < a.cout) {
-    v = combine_element(weight, basis, chan_out, chan_in, blocks, n_j, a.K, k, ci, co);
-    dense[((int64_t)k * a.cin + ci) * a.cout + co] = v;
-  }
-  static_cast<float *>(a.packed_out)[idx] = v;
+  const CombineJob job = {a, weight, basis, chan_out, chan_in, blocks, n_j, dense};
+  combine_pack_element(job, idx);
+}
+
+// (for a rulebook that was handed a CombineJob it cannot take along)
+int launch_combine_pack(const CombineJob &job, hipStream_t s) {
+  const int64_t n = combine_job_elements(job);
+  hipLaunchKernelGGL(combine_pack_kernel, dim3((unsigned)ceil_div(n, 256)), dim3(256), 0, s, job.pk,
+                     job.weight, job.basis, job.chan_out, job.chan_in, job.blocks, job.n_j,
+                     job.dense);
+  SSC_LAUNCH_CHECK("combine_pack");
+  return SSC_OK;
 }
 
 template <typename IO>
@@ -1795,6 +1749,30 @@ int ssc_conv_plan_build(const int32_t *pairs, int64_t pair_stride, const int32_t
                                 nullptr, (hipStream_t)stream);
 }
 
+// The checked form of "synthesise and pack these filters".
+static int combine_job_of(const float *weight, const float *basis, const int32_t *chan_out,
+                          const int32_t *chan_in, const int32_t *blocks, int32_t n_irreps_in,
+                          int32_t K, int32_t c_in, int32_t c_out, float *out, void *packed,
+                          size_t packed_bytes, CombineJob *job) {
+  int rc = conv_check_sizes(K, c_in, c_out, 0, 0, 0);
+  if (rc != SSC_OK) return rc;
+  SSC_CHECK(weight && basis && chan_out && chan_in && blocks && out && packed, SSC_EINVAL,
+            "NULL pointer argument");
+  SSC_CHECK(n_irreps_in >= 1, SSC_EINVAL, "sizes must be positive");
+  const ConvPlan p = make_plan(0, 1, K, c_in, c_out, 0, 4);
+  SSC_CHECK(packed_bytes >= conv_packed_bytes(p, K), SSC_EWORKSPACE,
+            "buffer of the packed filters too small");
+  job->pk = PackArgs{nullptr, 0, 0, 0, K, c_in, c_out, p.ncb, p.nch, packed, p.ns};
+  job->weight = weight;
+  job->basis = basis;
+  job->chan_out = chan_out;
+  job->chan_in = chan_in;
+  job->blocks = blocks;
+  job->n_j = (int)n_irreps_in;
+  job->dense = out;
+  return SSC_OK;
+}
+
 // A rulebook between ssc_rulebook_conv_begin and ssc_rulebook_conv_finish on this host thread:
 // whether the rulebook was asked to place the range boundaries, and for how many ranges.
 struct PendingLayer {
@@ -1808,11 +1786,19 @@ int ssc_rulebook_conv_begin(const int32_t *indices, int64_t n_in, const ssc_geom
                             int32_t *pair_num, int32_t *out_indices, int64_t out_capacity,
                             void *clean_table, size_t clean_table_bytes, int32_t c_in,
                             int32_t c_out, int32_t elem_bytes, void *scratch,
-                            size_t scratch_bytes, ssc_stream_t stream) {
+                            size_t scratch_bytes, const ssc_combine_job *filters,
+                            ssc_stream_t stream) {
   g_pending_layer = PendingLayer();
   SSC_CHECK(g != nullptr, SSC_EINVAL, "geometry is NULL");
   SSC_CHECK(c_in >= 1 && c_out >= 1, SSC_EINVAL, "channel counts must be positive");
   SSC_CHECK(elem_bytes == 4 || elem_bytes == 2, SSC_EINVAL, "elem_bytes must be 4 or 2");
+  CombineJob job = {};
+  if (filters != nullptr) {
+    int rc = combine_job_of(filters->weight, filters->basis, filters->chan_out, filters->chan_in,
+                            filters->blocks, filters->n_irreps_in, filters->kernel_volume, c_in,
+                            c_out, filters->out, filters->packed, filters->packed_bytes, &job);
+    if (rc != SSC_OK) return rc;
+  }
   SplitRequest rq = {0, 0, 0, nullptr};
   const SplitRequest *ask = nullptr;
   int64_t K = 1;
@@ -1834,7 +1820,7 @@ int ssc_rulebook_conv_begin(const int32_t *indices, int64_t n_in, const ssc_geom
   bool seeded = false;
   int rc = rulebook_begin_impl(indices, n_in, g, workspace, workspace_bytes, pairs, pair_num,
                                out_indices, out_capacity, clean_table, clean_table_bytes, ask,
-                               &seeded, (hipStream_t)stream);
+                               &seeded, (hipStream_t)stream, filters ? &job : nullptr);
   if (rc != SSC_OK) return rc;
   g_pending_layer.seeded = seeded;
   g_pending_layer.n_rng = rq.n_rng;
@@ -1878,22 +1864,11 @@ int ssc_kernel_combine_packed_f32(const float *weight, const float *basis,
                                   const int32_t *blocks, int32_t n_irreps_in,
                                   int32_t kernel_volume, int32_t c_in, int32_t c_out, float *out,
                                   void *packed, size_t packed_bytes, ssc_stream_t stream) {
-  const int K = kernel_volume;
-  int rc = conv_check_sizes(K, c_in, c_out, 0, 0, 0);
+  CombineJob job;
+  int rc = combine_job_of(weight, basis, chan_out, chan_in, blocks, n_irreps_in, kernel_volume,
+                          c_in, c_out, out, packed, packed_bytes, &job);
   if (rc != SSC_OK) return rc;
-  SSC_CHECK(weight && basis && chan_out && chan_in && blocks && out && packed, SSC_EINVAL,
-            "NULL pointer argument");
-  SSC_CHECK(n_irreps_in >= 1, SSC_EINVAL, "sizes must be positive");
-  const ConvPlan p = make_plan(0, 1, K, c_in, c_out, 0, 4);
-  SSC_CHECK(packed_bytes >= conv_packed_bytes(p, K), SSC_EWORKSPACE,
-            "buffer of the packed filters too small");
-  const PackArgs pk = {nullptr, 0, 0, 0, K, c_in, c_out, p.ncb, p.nch, packed, p.ns};
-  const int64_t n = (int64_t)K * p.ncb * p.nch * 1024;
-  hipLaunchKernelGGL(combine_pack_kernel, dim3((unsigned)ceil_div(n, 256)), dim3(256), 0,
-                     (hipStream_t)stream, pk, weight, basis, chan_out, chan_in, blocks,
-                     (int)n_irreps_in, out);
-  SSC_LAUNCH_CHECK("combine_pack");
-  return SSC_OK;
+  return launch_combine_pack(job, (hipStream_t)stream);
 }
 
 int ssc_conv_pack_filters_f32(const float *filters, int64_t fs_k, int64_t fs_ci, int64_t fs_co,

@@ -6,6 +6,7 @@
 // this path sees) and a popcount prefix turns membership into the rank of the
 // key, i.e. the output row.  No sort, no probing, no result-bearing atomics:
 // atomicOr on the bit table is order independent.
+#include "conv_pack.h"
 #include "ssc_common.h"
 
 namespace ssc {
@@ -210,10 +211,24 @@ static inline int64_t dense_in_words(const Geom &g, const DenseIn &d) {
 
 // As mark_count_kernel (same grid, same chunk counts, same flags), but the wave marks the
 // cells of its input rows in the input table instead of the output cells they reach.
+// JOB: the grid rows from ks[0] on synthesise and pack the layer's filters (work that
+// depends on nothing here and that the layer would otherwise launch by itself).
+template <bool JOB>
 __global__ void __launch_bounds__(256)
     mark_in_count_kernel(const int32_t *__restrict__ indices, int64_t n_in, Geom g, DenseIn d,
                          uint32_t *__restrict__ in_bits, int32_t *__restrict__ chunk_count,
-                         int64_t n_chunks, int32_t *__restrict__ flags) {
+                         int64_t n_chunks, int32_t *__restrict__ flags, CombineJob job,
+                         int64_t job_elements) {
+  if constexpr (JOB) {
+    if ((int)blockIdx.y >= g.ks[0]) {
+      const int64_t step = (int64_t)(gridDim.y - g.ks[0]) * gridDim.x * 256;
+      for (int64_t idx = ((int64_t)(blockIdx.y - g.ks[0]) * gridDim.x + blockIdx.x) * 256 +
+                         threadIdx.x;
+           idx < job_elements; idx += step)
+        combine_pack_element(job, idx);
+      return;
+    }
+  }
   int64_t chunk = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (chunk >= n_chunks) return;
   const int lane = threadIdx.x & 63;
@@ -898,7 +913,8 @@ static int rulebook_check(const ssc_geometry *g, Geom *gg, const int32_t *indice
 static int rulebook_mark_and_scan(const int32_t *indices, int64_t n_in, const Geom &gg,
                                   const RulebookWs &w, int32_t *pair_num, int32_t *mirror,
                                   hipStream_t s, const SplitRequest *split = nullptr,
-                                  bool table_is_clean = false, bool two_level = false) {
+                                  bool table_is_clean = false, bool two_level = false,
+                                  const CombineJob *job = nullptr) {
   int rc;
   if (w.use_dense && pair_num != nullptr) {
     // input table cleared (with the totals) unless the caller keeps one that every call
@@ -907,10 +923,20 @@ static int rulebook_mark_and_scan(const int32_t *indices, int64_t n_in, const Ge
     in.bits = w.in_bits;
     in.n_words = dense_in_words(gg, w.dense);
     if (!table_is_clean && (rc = bit_table_clear(in, s, true)) != SSC_OK) return rc;
-    hipLaunchKernelGGL(mark_in_count_kernel,
-                       dim3((unsigned)ceil_div(w.n_chunks, 4), (unsigned)gg.ks[0]), dim3(256), 0, s,
-                       indices, n_in, gg, w.dense, w.in_bits, w.chunk_count, w.n_chunks,
-                       w.table.total + 1);
+    const int64_t mark_blocks = ceil_div(w.n_chunks, 4);
+    if (job != nullptr) {
+      const int64_t n = combine_job_elements(*job);
+      const int64_t rows = std::min<int64_t>(ceil_div(ceil_div(n, 256), mark_blocks), 1024);
+      hipLaunchKernelGGL(mark_in_count_kernel<true>,
+                         dim3((unsigned)mark_blocks, (unsigned)(gg.ks[0] + rows)), dim3(256), 0, s,
+                         indices, n_in, gg, w.dense, w.in_bits, w.chunk_count, w.n_chunks,
+                         w.table.total + 1, *job, n);
+    } else {
+      hipLaunchKernelGGL(mark_in_count_kernel<false>,
+                         dim3((unsigned)mark_blocks, (unsigned)gg.ks[0]), dim3(256), 0, s, indices,
+                         n_in, gg, w.dense, w.in_bits, w.chunk_count, w.n_chunks,
+                         w.table.total + 1, CombineJob{}, (int64_t)0);
+    }
     SSC_LAUNCH_CHECK("mark_in_count");
     const int64_t word_blocks = w.table.n_scan_blocks;
     const int ks = (gg.ks[0] == gg.ks[1] && gg.ks[1] == gg.ks[2]) ? gg.ks[0] : 0;
@@ -1100,7 +1126,7 @@ int ssc_rulebook_begin(const int32_t *indices, int64_t n_in, const ssc_geometry 
   bool seeded = false;
   return ssc::rulebook_begin_impl(indices, n_in, g, workspace, workspace_bytes, pairs, pair_num,
                                   out_indices, out_capacity, clean_table, clean_table_bytes,
-                                  nullptr, &seeded, (hipStream_t)stream);
+                                  nullptr, &seeded, (hipStream_t)stream, nullptr);
 }
 }  // extern "C"
 
@@ -1108,14 +1134,20 @@ int ssc::rulebook_begin_impl(const int32_t *indices, int64_t n_in, const ssc_geo
                              void *workspace, size_t workspace_bytes, int32_t *pairs,
                              int32_t *pair_num, int32_t *out_indices, int64_t out_capacity,
                              void *clean_table, size_t clean_table_bytes,
-                             const SplitRequest *split, bool *seeded, hipStream_t s) {
+                             const SplitRequest *split, bool *seeded, hipStream_t s,
+                             const CombineJob *job) {
   Geom gg;
   *seeded = false;
   int rc = rulebook_check(g, &gg, indices, n_in, workspace, workspace_bytes);
   if (rc != SSC_OK) return rc;
   SSC_CHECK(pair_num != nullptr, SSC_EINVAL, "pair_num is NULL");
+  SSC_CHECK(n_in == 0 || pairs != nullptr, SSC_EINVAL, "pairs is NULL");
+  // the filters' job rides on the dilation path's first launch; any other path runs it first
+  DenseIn job_dense;
+  const bool job_rides = job != nullptr && n_in > 0 && dense_marking_applies(gg, n_in, &job_dense);
+  if (job != nullptr && !job_rides && (rc = launch_combine_pack(*job, s)) != SSC_OK) return rc;
+  if (!job_rides) job = nullptr;
   if (n_in == 0) return fill_i32(pair_num, gg.K, 0, s);
-  SSC_CHECK(pairs != nullptr, SSC_EINVAL, "pairs is NULL");
   SSC_CHECK(out_indices == nullptr || out_capacity >= rulebook_out_bound(gg, n_in), SSC_EINVAL,
             "out_indices holds %lld rows, fewer than the bound of %lld", (long long)out_capacity,
             (long long)rulebook_out_bound(gg, n_in));
@@ -1150,7 +1182,7 @@ int ssc::rulebook_begin_impl(const int32_t *indices, int64_t n_in, const ssc_geo
   const bool two_level = w.use_dense && w.can_seed && out_indices != nullptr &&
                          ceil_div(w.n_chunks, 4) > split_blocks;
   if ((rc = rulebook_mark_and_scan(indices, n_in, gg, w, pair_num, mirror, s, split,
-                                   clean != nullptr, two_level)) != SSC_OK)
+                                   clean != nullptr, two_level, job)) != SSC_OK)
     return rc;
   if (!two_level) {
     if ((rc = read_back_mirror_queued(s)) != SSC_OK) return rc;

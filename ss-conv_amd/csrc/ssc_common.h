@@ -228,12 +228,15 @@ struct SplitRequest {
   int32_t *range_row0; // [n_rng + 1] device: first output row of every range
 };
 // ssc_rulebook_begin with an optional split request.  *seeded = whether range_row0 will be
-// written (the geometry takes the dilation path and the table is small enough).
+// written (the geometry takes the dilation path and the table is small enough).  `job`
+// (optional, conv_pack.h): synthesis and packing of a layer's filters, enqueued with the
+// rulebook's first launch where that has room for it and before it otherwise.
+struct CombineJob;
 int rulebook_begin_impl(const int32_t *indices, int64_t n_in, const ssc_geometry *g,
                         void *workspace, size_t workspace_bytes, int32_t *pairs,
                         int32_t *pair_num, int32_t *out_indices, int64_t out_capacity,
                         void *clean_table, size_t clean_table_bytes, const SplitRequest *split,
-                        bool *seeded, hipStream_t s);
+                        bool *seeded, hipStream_t s, const CombineJob *job);
 
 // Enqueue: fill an int32 array (a kernel, so the call may be graph-captured).
 int fill_i32(int32_t *p, int64_t n, int32_t v, hipStream_t s);

@@ -49,7 +49,7 @@ _SIGNATURES = {
     "ssc_rulebook_finish": (ctypes.c_int, [_gp, _i64, ctypes.POINTER(_i32), ctypes.POINTER(_i32)]),
     "ssc_rulebook_rows": (ctypes.c_int, [_gp, _i64, _vp, _sz, _vp, _vp]),
     "ssc_rulebook_conv_begin": (ctypes.c_int, [_vp, _i64, _gp, _vp, _sz, _vp, _vp, _vp, _i64, _vp,
-                                               _sz, _i32, _i32, _i32, _vp, _sz, _vp]),
+                                               _sz, _i32, _i32, _i32, _vp, _sz, _vp, _vp]),
     "ssc_rulebook_conv_finish": (ctypes.c_int, [_gp, _i64, ctypes.POINTER(_i32),
                                                 ctypes.POINTER(_i32), _vp, _vp, _i32, _i32, _i32,
                                                 _vp, _sz, _vp, _sz, _vp]),
@@ -220,12 +220,14 @@ def _geometry(batch_size, out_shape, ksize, stride, padding, dilation, subm, tra
 
 
 # Output rows are written before their number is known when a buffer for the largest
-# possible number of them is at most this large (a result that fills less than a quarter of
-# a buffer of more than 16 MiB is copied out of it).
-_ROWS_AHEAD_BYTES = 512 << 20
+# possible number of them is at most this large (a result that fills less than half of a
+# buffer of more than 4 MiB is copied out of it, so that no rulebook keeps more than twice
+# its rows alive).
+_ROWS_AHEAD_BYTES = 256 << 20
 # largest plan / plan scratch allocated for the bound on the number of outputs, before the
-# real number has arrived
-_PLAN_AHEAD_BYTES = 256 << 20
+# real number has arrived (the scratch is dropped when the plan is built; the plan, kept
+# with the rulebook, is at most this much larger than one sized for the real number)
+_PLAN_AHEAD_BYTES = 128 << 20
 
 
 class RulebookMeta(object):
@@ -382,6 +384,7 @@ def _rulebook_begin(indices, batch_size, out_spatial_shape, kernel_size, stride,
             r.conv = (int(c_in), int(c_out), int(eb))
     clean_bytes = _lib.ssc_rulebook_clean_table_bytes(gref, n)
     clean = _clean_table(clean_bytes, dev, r.stream) if clean_bytes > 0 else None
+    job = _take_combine(K, r.conv[0], r.conv[1], dev, r.stream) if r.conv is not None else None
     try:
         if r.conv is not None:
             _check(_lib.ssc_rulebook_conv_begin(
@@ -389,7 +392,7 @@ def _rulebook_begin(indices, batch_size, out_spatial_shape, kernel_size, stride,
                 r.num.data_ptr(), _ptr(r.out_buf), 0 if r.out_buf is None else r.out_buf.size(0),
                 _ptr(clean), 0 if clean is None else clean.numel(),
                 r.conv[0], r.conv[1], r.conv[2], r.scratch.data_ptr(), r.scratch.numel(),
-                r.stream))
+                ctypes.byref(job) if job is not None else None, r.stream))
         else:
             _check(_lib.ssc_rulebook_begin(_ptr(indices), n, gref, r.ws.data_ptr(), r.ws.numel(),
                                            _ptr(r.pairs), r.num.data_ptr(), _ptr(r.out_buf),
@@ -429,7 +432,7 @@ def _rulebook_result(r, n_out, in_order):
         outids = r.indices
     elif r.out_buf is not None:
         outids = r.out_buf[:n_out]
-        if r.out_buf.size(0) > 4 * max(n_out, 1) and r.out_buf.numel() * 4 > (16 << 20):
+        if r.out_buf.size(0) > 2 * max(n_out, 1) and r.out_buf.numel() * 4 > (4 << 20):
             outids = outids.clone()  # do not keep a large, mostly unused buffer alive
     else:
         # a geometry may leave no output at all (every candidate clipped): the library still
@@ -490,6 +493,7 @@ def _packed_filters(owner, filters, fs, K, c_in, c_out, stream):
     caller passed (`owner`), one per way of reading it (forward, or transposed for the input
     gradient), and reused while that tensor's version counter stands still: evaluation-mode
     layers, whose kernel is synthesised once, pack once."""
+    flush_combine()
     key = (filters.data_ptr(), tuple(fs), K, c_in, c_out)
     held = getattr(owner, "_ssc_packed", None)
     if held is None or held[0] != owner._version:
@@ -1117,13 +1121,34 @@ def three_interpolate_fp(c, m, n, feats, idx, weight, out):
 
 
 # ---- entry points without a counterpart in the reference's binding ---------------------
+class _CombineJob(ctypes.Structure):
+    """ssc_combine_job of include/ssc.h."""
+    _fields_ = [("weight", _vp), ("basis", _vp), ("chan_out", _vp), ("chan_in", _vp),
+                ("blocks", _vp), ("n_irreps_in", _i32), ("kernel_volume", _i32), ("out", _vp),
+                ("packed", _vp), ("packed_bytes", _sz)]
+
+
+class _DeferredCombine(object):
+    """A synthesis-and-packing of filters that kernel_combine(defer=True) has not queued."""
+    __slots__ = ("args", "tensors", "packed", "stream", "sizes")
+
+
+_deferred = []  # at most one _DeferredCombine
+
+
 def kernel_combine(weight, basis, chan_out, chan_in, blocks, n_irreps_in, kernel_volume, c_in,
-                   c_out, packed=False):
+                   c_out, packed=False, defer=False):
     """Dense kernel [K, Cin, Cout] from the flat weight vector and the stacked
     basis (ss_conv/utils/kernel.py:267-299 fused with convolution.py:56).  With `packed`
     the same launch also writes the filters in the convolution kernel's packed order:
-    returns (dense, packed buffer)."""
+    returns (dense, packed buffer).
+    With `defer` (and `packed`) nothing is queued yet: the next rulebook_conv on this host
+    thread's way takes the work into the first launch of its rulebook, and anything else
+    that needs the filters (the packed-filter lookups here) or flush_combine() queues it as
+    a launch of its own.  The caller must end with flush_combine() before the tensors can
+    be read by anything outside this module."""
     _need_gpu(weight, basis, chan_out, chan_in, blocks)
+    flush_combine()
     out = torch.empty((kernel_volume, c_in, c_out), dtype=torch.float32, device=weight.device)
     args = (_ptr(weight), _ptr(basis), _ptr(chan_out), _ptr(chan_in), _ptr(blocks),
             int(n_irreps_in), int(kernel_volume), int(c_in), int(c_out), _ptr(out))
@@ -1132,8 +1157,40 @@ def kernel_combine(weight, basis, chan_out, chan_in, blocks, n_irreps_in, kernel
         return out
     buf = _workspace(_lib.ssc_conv_packed_bytes(int(kernel_volume), int(c_in), int(c_out)),
                      weight.device)
+    if defer:
+        job = _DeferredCombine()
+        job.args, job.packed, job.stream = args, buf, _stream(weight)
+        job.tensors = (weight, basis, chan_out, chan_in, blocks, out)
+        job.sizes = (int(kernel_volume), int(c_in), int(c_out), weight.device)
+        _deferred.append(job)
+        return out, buf
     _check(_lib.ssc_kernel_combine_packed_f32(*args, buf.data_ptr(), buf.numel(), _stream(weight)))
     return out, buf
+
+
+def flush_combine():
+    """Queue what kernel_combine(defer=True) left, if nobody has taken it."""
+    while _deferred:
+        job = _deferred.pop()
+        _check(_lib.ssc_kernel_combine_packed_f32(*job.args, job.packed.data_ptr(),
+                                                  job.packed.numel(), job.stream))
+
+
+def _take_combine(K, c_in, c_out, dev, stream):
+    """The deferred job as an ssc_combine_job for a rulebook of these sizes on this stream
+    (None, and the job queued by itself, when it does not fit)."""
+    if not _deferred:
+        return None
+    job = _deferred[-1]
+    if job.sizes != (K, c_in, c_out, dev) or job.stream != stream:
+        flush_combine()
+        return None
+    _deferred.pop()
+    a = job.args
+    st = _CombineJob(a[0], a[1], a[2], a[3], a[4], a[5], a[6], a[9], job.packed.data_ptr(),
+                     job.packed.numel())
+    st._keep = job  # the tensors outlive the call
+    return st
 
 
 def attach_packed(filters, c_in, c_out, packed):

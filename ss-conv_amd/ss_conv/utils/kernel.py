@@ -133,7 +133,8 @@ class _Combine(torch.autograd.Function):
         ctx.module = module
         out = _ext.kernel_combine(weight.detach().float().contiguous(), basis, chan_out, chan_in,
                                   blocks, len(module.multiplicities_in), module.size ** 3,
-                                  module.n_in, module.n_out, packed=pack)
+                                  module.n_in, module.n_out, packed=bool(pack),
+                                  defer=pack == "defer")
         if pack:
             out, module.packed = out
         return out
@@ -249,13 +250,15 @@ class SE3Kernel(torch.nn.Module):
         """[Cout, Cin, k, k, k] view of the natively contracted [K, Cin, Cout] kernel
         (reference: kernel.py:267-299).  Differentiable with respect to `weight`.
         With `pack` the same launch leaves the filters in the convolution kernel's packed
-        order in `self.packed` (for _ext.attach_packed)."""
+        order in `self.packed` (for _ext.attach_packed); with pack="defer" that launch is
+        left to the rulebook the caller queues next (_ext.kernel_combine), and the caller
+        ends with _ext.flush_combine()."""
         if not weight.is_cuda:
             raise RuntimeError("SE3Kernel runs on the GPU only: move the module to a cuda device")
         if self._tables is None or self._tables[4] != weight.device:
             self._build_tables(weight.device)
         self.packed = None
-        dense = _Combine.apply(weight, self, bool(pack))
+        dense = _Combine.apply(weight, self, pack if pack == "defer" else bool(pack))
         k = self.size
         return dense.permute(2, 1, 0).reshape(self.n_out, self.n_in, k, k, k)
 
