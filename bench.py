@@ -190,8 +190,8 @@ def point2voxel_figure(torch, _ext, synth, dev, workload, seed, channels=64):
             torch.cuda.synchronize()
             t0 = time.perf_counter()
             m(tp, tf, ti)
-            torch.cuda.synchronize()
             firsts.append((time.perf_counter() - t0) * 1e6)
+            torch.cuda.synchronize()
         first_path = m.last_path
         torch.cuda.synchronize()
         t0 = time.perf_counter()
@@ -216,7 +216,8 @@ def point2voxel_figure(torch, _ext, synth, dev, workload, seed, channels=64):
             "how": "gpu_us: HIP events around one module call (its one host wait included), "
                    "median of 20, an empty event pair subtracted; call_us: mean of 50 calls of "
                    "one module, host-timed; first_call_us: median of 10 first calls of fresh "
-                   "modules"}
+                   "modules on an idle GPU, host-timed like call_us (the call returns after "
+                   "its one host wait, its last two kernels still running)"}
 
 
 def ops_table(torch, _ext, synth, dev, seed):

@@ -636,7 +636,8 @@ int ssc_p2v_compact(const float *points, const float *feats /* [n,channels] */,
  * 4 mean; points of a voxel are added in ascending point order).  All kernels are queued
  * with the data-dependent sizes kept on the device and every output sized for n rows
  * (there are never more rows or voxels than points); the call SYNCHRONISES once, for
- *   totals_host = {rows m, voxels v, flags, batch ids left without points}
+ *   totals_host = {rows m, voxels v, flags, batch ids left without points,
+ *                  ids present, ids present that kept points, largest id present, 0}
  * and the histograms hist_all_host[n_ids] / hist_valid_host[n_ids] (points and surviving
  * points per id), while its last kernels still run.  The first m rows of out_points [n,3],
  * out_ids [n], inverse [n] (voxel of each row) and the first v rows of out_indices [n,4],
@@ -657,7 +658,7 @@ int ssc_p2v_voxelize_f32(const float *points /* [n,3] */, const float *feats /* 
                          float *out_feats, int32_t *inverse, int32_t *counts, int32_t *dest,
                          int32_t *sel, int32_t *hist_all_host /* [n_ids] host */,
                          int32_t *hist_valid_host /* [n_ids] host */,
-                         int32_t *totals_host /* [4] host */, ssc_stream_t stream);
+                         int32_t *totals_host /* [8] host */, ssc_stream_t stream);
 int ssc_p2v_voxelize_bwd_f32(const float *out_grad /* [v,channels] */, int32_t channels,
                              const int32_t *dest /* [n] */, const int32_t *inverse,
                              const int32_t *counts, const int32_t *sel, int32_t mode, int64_t n,

@@ -85,23 +85,24 @@ __global__ void __launch_bounds__(kScanThreads)
 __global__ void __launch_bounds__(kScanThreads)
     popc_prefix_kernel(const uint32_t *__restrict__ bits, int64_t n_words,
                        const int32_t *__restrict__ blocksum, int32_t *__restrict__ prefix,
-                       int32_t *__restrict__ total, int32_t *__restrict__ mirror) {
-  popc_prefix_block(bits, n_words, blocksum, prefix, total, mirror, blockIdx.x == gridDim.x - 1);
+                       int32_t *__restrict__ total, int32_t *__restrict__ mirror, int ticket) {
+  popc_prefix_block(bits, n_words, blocksum, prefix, total, mirror, blockIdx.x == gridDim.x - 1,
+                    ticket);
 }
 
-int bit_table_scan_prefix(const BitTable &t, hipStream_t s, int32_t *mirror) {
+int bit_table_scan_prefix(const BitTable &t, hipStream_t s, int32_t *mirror, int ticket) {
   hipLaunchKernelGGL(popc_prefix_kernel, dim3((unsigned)t.n_scan_blocks), dim3(kScanThreads), 0, s,
-                     t.bits, t.n_words, t.blocksum, t.prefix, t.total, mirror);
+                     t.bits, t.n_words, t.blocksum, t.prefix, t.total, mirror, ticket);
   SSC_LAUNCH_CHECK("popc_prefix");
   return SSC_OK;
 }
 
-int bit_table_scan(const BitTable &t, hipStream_t s, int32_t *mirror) {
+int bit_table_scan(const BitTable &t, hipStream_t s, int32_t *mirror, int ticket) {
   if (t.n_words <= 0) return fill_i32(t.total, 1, 0, s);
   hipLaunchKernelGGL(popc_blocksum_kernel, dim3((unsigned)t.n_scan_blocks), dim3(kScanThreads), 0,
                      s, t.bits, t.n_words, t.blocksum);
   SSC_LAUNCH_CHECK("popc_blocksum");
-  return bit_table_scan_prefix(t, s, mirror);
+  return bit_table_scan_prefix(t, s, mirror, ticket);
 }
 
 // The pinned block and the event of the calling host thread.

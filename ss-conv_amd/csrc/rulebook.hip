@@ -624,10 +624,10 @@ __global__ void __launch_bounds__(kScanThreads)
                         int32_t *__restrict__ total, int32_t *__restrict__ mirror,
                         const int32_t *__restrict__ pairsum,
                         const int32_t *__restrict__ seed_rows,
-                        const int32_t *__restrict__ seed_pairs, SplitRequest rq) {
+                        const int32_t *__restrict__ seed_pairs, SplitRequest rq, int ticket) {
   if ((int64_t)blockIdx.x < n_scan_blocks) {
     popc_prefix_block(bits, n_words, blocksum, prefix, total, mirror,
-                      (int64_t)blockIdx.x == n_scan_blocks - 1);
+                      (int64_t)blockIdx.x == n_scan_blocks - 1, ticket);
     return;
   }
   split_ranges_block((int)(blockIdx.x - n_scan_blocks), n_words, n_scan_blocks, blocksum, pairsum,
@@ -914,7 +914,7 @@ static int rulebook_mark_and_scan(const int32_t *indices, int64_t n_in, const Ge
                                   const RulebookWs &w, int32_t *pair_num, int32_t *mirror,
                                   hipStream_t s, const SplitRequest *split = nullptr,
                                   bool table_is_clean = false, bool two_level = false,
-                                  const CombineJob *job = nullptr) {
+                                  const CombineJob *job = nullptr, int ticket = 0) {
   int rc;
   if (w.use_dense && pair_num != nullptr) {
     // input table cleared (with the totals) unless the caller keeps one that every call
@@ -955,13 +955,13 @@ static int rulebook_mark_and_scan(const int32_t *indices, int64_t n_in, const Ge
                        w.seed_pairs, w.pairsum);
     SSC_LAUNCH_CHECK("dilate_blocksum");
     if (two_level) return SSC_OK;
-    if (!seed || split == nullptr) return bit_table_scan_prefix(w.table, s, mirror);
+    if (!seed || split == nullptr) return bit_table_scan_prefix(w.table, s, mirror, ticket);
     // the scan's second pass, and beside it the range boundaries of the convolution's plan
     const int64_t split_blocks = ceil_div(split->n_rng, kScanThreads / 16);
     hipLaunchKernelGGL(prefix_split_kernel, dim3((unsigned)(word_blocks + split_blocks)),
                        dim3(kScanThreads), 0, s, w.table.bits, w.table.n_words, word_blocks,
                        w.table.blocksum, w.table.prefix, w.table.total, mirror, w.pairsum,
-                       w.seed_rows, w.seed_pairs, *split);
+                       w.seed_rows, w.seed_pairs, *split, ticket);
     SSC_LAUNCH_CHECK("prefix_split");
     return SSC_OK;
   }
@@ -971,18 +971,18 @@ static int rulebook_mark_and_scan(const int32_t *indices, int64_t n_in, const Ge
                        indices, n_in, gg.batch, gg.os[0], gg.os[1], gg.os[2], w.table.bits,
                        w.table.total + 1, 1);
     SSC_LAUNCH_CHECK("mark_rows");
-    return bit_table_scan(w.table, s, mirror);
+    return bit_table_scan(w.table, s, mirror, ticket);
   }
   hipLaunchKernelGGL(mark_count_kernel, dim3((unsigned)ceil_div(w.n_chunks, 4), (unsigned)gg.ks[0]),
                      dim3(256), 0, s, indices, n_in, gg, w.table.bits, w.chunk_count, w.n_chunks,
                      w.table.total + 1);
   SSC_LAUNCH_CHECK("mark_count");
-  if (pair_num == nullptr) return bit_table_scan(w.table, s, mirror);
+  if (pair_num == nullptr) return bit_table_scan(w.table, s, mirror, ticket);
   hipLaunchKernelGGL(blocksum_scan_chunks_kernel, dim3((unsigned)(w.table.n_scan_blocks + gg.K)),
                      dim3(kScanThreads), 0, s, w.table.bits, w.table.n_words, w.table.blocksum,
                      w.table.n_scan_blocks, w.chunk_count, w.n_chunks, pair_num);
   SSC_LAUNCH_CHECK("blocksum_scan_chunks");
-  return bit_table_scan_prefix(w.table, s, mirror);
+  return bit_table_scan_prefix(w.table, s, mirror, ticket);
 }
 
 // Enqueue: the pair lists and, with out_indices, the output rows (one launch for both).
@@ -1181,17 +1181,20 @@ int ssc::rulebook_begin_impl(const int32_t *indices, int64_t n_in, const ssc_geo
   const int split_blocks = split ? (int)ceil_div(split->n_rng, kScanThreads / 16) : 0;
   const bool two_level = w.use_dense && w.can_seed && out_indices != nullptr &&
                          ceil_div(w.n_chunks, 4) > split_blocks;
+  // (the kernel that finishes the scan stores a ticket behind the totals, for the host to
+  // spin on: it then sees them a few microseconds before the event behind the kernel says so)
+  const int ticket = read_back_mirror_ticket();
   if ((rc = rulebook_mark_and_scan(indices, n_in, gg, w, pair_num, mirror, s, split,
-                                   clean != nullptr, two_level, job)) != SSC_OK)
+                                   clean != nullptr, two_level, job, ticket)) != SSC_OK)
     return rc;
   if (!two_level) {
-    if ((rc = read_back_mirror_queued(s)) != SSC_OK) return rc;
+    if ((rc = read_back_mirror_queued(s, ticket)) != SSC_OK) return rc;
     return rulebook_pairs(indices, n_in, gg, w, out_indices, pairs, pair_num, true, s, clean,
                           clean_words);
   }
   TwoLevel two = {w.table.blocksum, w.pairsum, w.seed_rows, w.seed_pairs, w.table.n_scan_blocks,
                   split ? *split : SplitRequest{0, 0, 0, nullptr}, split_blocks, w.table.total,
-                  mirror, read_back_mirror_ticket(), clean != nullptr ? 1 : 0};
+                  mirror, ticket, clean != nullptr ? 1 : 0};
   // (the header of a clean table holds the totals: the block that hands them to the host
   // clears it, the other blocks the words behind it)
   if ((rc = rulebook_pairs(indices, n_in, gg, w, out_indices, pairs, pair_num, true, s,

@@ -75,10 +75,11 @@ int bit_table_clear(const BitTable &t, hipStream_t s, bool blocksum_too = false)
 // Enqueue: prefix[], total[0] from bits[].  With `mirror` (memory the device can write and
 // the host can read, see read_back_mirror), the kernel that writes total[0] also copies
 // total[0..3] there, which saves the copy a host that waits for them would otherwise queue.
-int bit_table_scan(const BitTable &t, hipStream_t s, int32_t *mirror = nullptr);
+int bit_table_scan(const BitTable &t, hipStream_t s, int32_t *mirror = nullptr, int ticket = 0);
 // The second pass of bit_table_scan alone (the first one, popc_blocksum_block, is then run
 // by a kernel of the caller that has other work to do beside it).
-int bit_table_scan_prefix(const BitTable &t, hipStream_t s, int32_t *mirror = nullptr);
+int bit_table_scan_prefix(const BitTable &t, hipStream_t s, int32_t *mirror = nullptr,
+                          int ticket = 0);
 
 // Block-wide exclusive scan of one int per thread (kScanThreads threads).
 __device__ __forceinline__ int block_exclusive_scan(int v, int *lds /* [kScanThreads/64 + 1] */,
@@ -124,12 +125,14 @@ __device__ __forceinline__ void popc_blocksum_block(const uint32_t *__restrict__
 // (at most 2^31 / 32 / kScanBlockWords = 32768 values), which saves the launch of a scan
 // over blocksum[]; the table's last block (`last`) also writes the total, and with `mirror`
 // copies total[0..3] there (total[1..3] were written by kernels before this one).
+constexpr int kMirrorTicket = 8;  // where in the host mirror a ticket goes (see read_back_mirror_ticket)
 __device__ __forceinline__ void popc_prefix_block(const uint32_t *__restrict__ bits,
                                                   int64_t n_words,
                                                   const int32_t *__restrict__ blocksum,
                                                   int32_t *__restrict__ prefix,
                                                   int32_t *__restrict__ total,
-                                                  int32_t *__restrict__ mirror, bool last) {
+                                                  int32_t *__restrict__ mirror, bool last,
+                                                  int ticket = 0) {
   __shared__ int lds[kScanThreads / 64 + 1];
   int before = 0;
   for (int64_t b = threadIdx.x; b < (int64_t)blockIdx.x; b += kScanThreads) before += blocksum[b];
@@ -157,6 +160,10 @@ __device__ __forceinline__ void popc_prefix_block(const uint32_t *__restrict__ b
       mirror[1] = total[1];
       mirror[2] = total[2];
       mirror[3] = total[3];
+      // (a host that spins on the ticket sees the four values with it: read_back_end)
+      if (ticket != 0)
+        __hip_atomic_store(mirror + kMirrorTicket, ticket, __ATOMIC_RELEASE,
+                           __HIP_MEMORY_SCOPE_SYSTEM);
     }
   }
 }
@@ -263,7 +270,6 @@ int read_back_mirror_queued(hipStream_t s, int ticket = 0);
 // mirror[kMirrorTicket] with a release at system scope; read_back_mirror_queued(s, ticket)
 // behind the launch; read_back_end then returns as soon as the ticket shows up in the host's
 // view of the block, not when the kernel ends.
-constexpr int kMirrorTicket = 8;
 int read_back_mirror_ticket();
 // The same, moved on to `dst_host`.
 int read_back(void *dst_host, const void *src_dev, size_t bytes, hipStream_t s);

@@ -1557,8 +1557,9 @@ int ssc_p2v_voxelize_f32(const float *points, const float *feats, const int64_t 
                      dim3(kScanThreads), 0, s, w.vox.bits, w.vox.n_words, w.vox.blocksum,
                      w.inside.total, extra, w.flags, w.vox.total);
   SSC_LAUNCH_CHECK("p2vx_vox_blocksum");
-  if ((rc = bit_table_scan_prefix(w.vox, s, mirror)) != SSC_OK) return rc;
-  if ((rc = read_back_mirror_queued(s)) != SSC_OK) return rc;
+  const int ticket = read_back_mirror_ticket();
+  if ((rc = bit_table_scan_prefix(w.vox, s, mirror, ticket)) != SSC_OK) return rc;
+  if ((rc = read_back_mirror_queued(s, ticket)) != SSC_OK) return rc;
   const int64_t link_blocks = ceil_div(n, 256);
   int64_t row_blocks = ceil_div(w.vox.n_words, 256);
   if (row_blocks > 2048) row_blocks = 2048;
@@ -1583,6 +1584,20 @@ int ssc_p2v_voxelize_f32(const float *points, const float *feats, const int64_t 
   totals_host[3] = m[2];         // ids left without points
   memcpy(hist_all_host, m + 16, (size_t)n_ids * sizeof(int32_t));
   memcpy(hist_valid_host, m + 16 + n_ids, (size_t)n_ids * sizeof(int32_t));
+  // what callers ask the histograms first: how many ids there are, how many of them kept
+  // points, and the largest one
+  int present = 0, alive = 0, largest = -1;
+  for (int i = 0; i < n_ids; ++i) {
+    if (hist_all_host[i] > 0) {
+      ++present;
+      largest = i;
+      alive += hist_valid_host[i] > 0;
+    }
+  }
+  totals_host[4] = present;
+  totals_host[5] = alive;
+  totals_host[6] = largest;
+  totals_host[7] = 0;
   return SSC_OK;
 }
 

@@ -1315,14 +1315,40 @@ class _P2vVoxelFeatures(torch.autograd.Function):
         return grad_in, None, None, None, None, None, None
 
 
-def p2v_voxelize(points, feats, batch_ids, half_extent, unit, limit, mode, n_ids):
+class P2vConsts(object):
+    """What p2v_voxelize needs of a module's grid, converted once: half extent, unit and limit
+    as the arrays the native call takes."""
+    __slots__ = ("half", "unit", "limit", "ws_bytes")
+
+    def __init__(self, half_extent, unit, limit):
+        self.half = (ctypes.c_float * 3)(*[float(v) for v in half_extent])
+        self.unit = (ctypes.c_float * 3)(*[float(v) for v in unit])
+        self.limit = (_i32 * 3)(*[int(v) for v in limit])
+        self.ws_bytes = {}  # (points, ids) -> workspace size
+
+
+_p2v_scratch = {}  # (device index, stream) -> buffers that hold nothing between two calls
+
+
+def _p2v_scratch_of(dev, stream, key, nbytes):
+    """A buffer of the one-call Point2Voxel that nothing reads after the call's kernels: one
+    per device, stream and use, kept and reused (the kernels of two calls on a stream run in
+    order), regrown when a call needs more."""
+    held = _p2v_scratch.get((dev.index, stream, key))
+    if held is None or held.numel() < nbytes:
+        held = _workspace(nbytes, dev)
+        _p2v_scratch[(dev.index, stream, key)] = held
+    return held
+
+
+def p2v_voxelize(points, feats, batch_ids, consts, mode, n_ids):
     """Point2Voxel.forward (ss_conv/sp_ops/voxelize.py:29-99) in one native call with one
     wait of the host, for float32 points / features and int64 batch ids that are
-    non-decreasing and lie in [0, n_ids).  Returns None when the inputs do not qualify (the
-    caller then takes another path; `n_ids` too small counts as not qualifying); otherwise
-    (valid_points [m,3], voxel_feats [v,C], voxel_indices [v,4], valid_ids [m], origin_ids,
-    alive) with origin_ids / alive as host arrays over the batch ids present."""
-    import numpy as np
+    non-decreasing and lie in [0, n_ids); `consts` is the grid as a P2vConsts.  Returns None
+    when the inputs do not qualify (the caller then takes another path; `n_ids` too small
+    counts as not qualifying); otherwise (valid_points [m,3], voxel_feats [v,C],
+    voxel_indices [v,4], valid_ids [m], ids present, largest id, alive) with `alive` a host
+    array of 0/1 floats over the ids present, or None when every one of them kept points."""
     if not (points.is_cuda and feats.is_cuda and batch_ids.is_cuda):
         return None
     if points.dtype != torch.float32 or feats.dtype != torch.float32 or \
@@ -1332,45 +1358,55 @@ def p2v_voxelize(points, feats, batch_ids, half_extent, unit, limit, mode, n_ids
     if n == 0 or feats.dim() != 2 or feats.size(0) != n or batch_ids.numel() != n:
         return None
     n_ids = int(n_ids)
-    lim = (_i32 * 3)(*[int(v) for v in limit])
-    nbytes = _lib.ssc_p2v_voxelize_workspace_bytes(n, n_ids, lim) if 1 <= n_ids <= P2V_MAX_IDS \
-        else 0
+    nbytes = consts.ws_bytes.get((n, n_ids))
+    if nbytes is None:
+        nbytes = _lib.ssc_p2v_voxelize_workspace_bytes(n, n_ids, consts.limit) \
+            if 1 <= n_ids <= P2V_MAX_IDS else 0
+        if len(consts.ws_bytes) < 64:
+            consts.ws_bytes[(n, n_ids)] = nbytes
     if nbytes == 0:
         return None
     points, batch_ids = points.contiguous(), batch_ids.contiguous()
-    src_feats = feats.detach().contiguous()
+    wants_grad = torch.is_grad_enabled() and feats.requires_grad
+    src_feats = feats.detach().contiguous() if feats.requires_grad else feats.contiguous()
     dev = points.device
     c = feats.size(1)
-    ws = _workspace(nbytes, dev)
-    h = (ctypes.c_float * 3)(*[float(v) for v in half_extent])
-    u = (ctypes.c_float * 3)(*[float(v) for v in unit])
+    stream = _stream(points)
+    ws = _p2v_scratch_of(dev, stream, "ws", nbytes)
     out_p = torch.empty((n, 3), dtype=torch.float32, device=dev)
     out_i = torch.empty((n,), dtype=torch.int64, device=dev)
     vox_idx = torch.empty((n, 4), dtype=torch.int32, device=dev)
     vox_f = torch.empty((n, c), dtype=torch.float32, device=dev)
-    # inverse, counts, dest and (modes 1 / 2) sel side by side
-    aux = torch.empty((4, n), dtype=torch.int32, device=dev)
-    sel = aux[3] if mode in (1, 2) else None
-    hist_all = np.empty(n_ids, dtype=np.int32)
-    hist_valid = np.empty(n_ids, dtype=np.int32)
-    totals = (_i32 * 4)()
+    # inverse, counts, dest and (modes 1 / 2) sel side by side: the backward pass reads them,
+    # a call without one leaves them in a buffer the next call writes over
+    if wants_grad:
+        aux = torch.empty((4, n), dtype=torch.int32, device=dev)
+        a0 = aux.data_ptr()
+    else:
+        aux = None
+        a0 = _p2v_scratch_of(dev, stream, "aux", 16 * n).data_ptr()
+    sel = a0 + 12 * n if mode in (1, 2) else None
+    hist = (_i32 * (2 * n_ids))()
+    totals = (_i32 * 8)()
     _check(_lib.ssc_p2v_voxelize_f32(
-        _ptr(points), _ptr(src_feats), _ptr(batch_ids), n, c, h, u, lim, n_ids, int(mode),
-        ws.data_ptr(), ws.numel(), out_p.data_ptr(), out_i.data_ptr(), vox_idx.data_ptr(),
-        vox_f.data_ptr(), aux[0].data_ptr(), aux[1].data_ptr(), aux[2].data_ptr(), _ptr(sel),
-        hist_all.ctypes.data, hist_valid.ctypes.data, totals, _stream(points)))
-    m, v, flags = int(totals[0]), int(totals[1]), int(totals[2])
-    if flags or m == 0:
+        points.data_ptr(), src_feats.data_ptr(), batch_ids.data_ptr(), n, c, consts.half,
+        consts.unit, consts.limit, n_ids, int(mode), ws.data_ptr(), ws.numel(),
+        out_p.data_ptr(), out_i.data_ptr(), vox_idx.data_ptr(), vox_f.data_ptr(), a0, a0 + 4 * n,
+        a0 + 8 * n, sel, hist, ctypes.byref(hist, 4 * n_ids), totals, stream))
+    m, v, flags, present, kept, largest = totals[0], totals[1], totals[2], totals[4], \
+        totals[5], totals[6]
+    if flags or m == 0 or kept == 0:  # (no point survived at all: the reference's special case)
         return None
-    present = hist_all > 0
-    origin_ids = np.nonzero(present)[0]
-    alive = (hist_valid > 0)[origin_ids]
-    if not alive.any():  # no point survived at all: the reference's special case
-        return None
+    alive = None
+    if kept != present:
+        import numpy as np
+        h = np.frombuffer(hist, dtype=np.int32)
+        alive = (h[n_ids:][h[:n_ids] > 0] > 0).astype(np.float32)
     vox_f = vox_f[:v]
-    if torch.is_grad_enabled() and feats.requires_grad:
-        vox_f = _P2vVoxelFeatures.apply(feats, vox_f, aux[2], aux[0], aux[1], sel, int(mode))
-    return out_p[:m], vox_f, vox_idx[:v], out_i[:m], origin_ids, alive.astype(np.float32)
+    if wants_grad:
+        vox_f = _P2vVoxelFeatures.apply(feats, vox_f, aux[2], aux[0], aux[1],
+                                        aux[3] if mode in (1, 2) else None, int(mode))
+    return out_p[:m], vox_f, vox_idx[:v], out_i[:m], present, largest, alive
 
 
 def unique_rows(coords, dims, return_counts=True):

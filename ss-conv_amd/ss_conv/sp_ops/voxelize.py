@@ -23,6 +23,8 @@ class Point2Voxel(nn.Module):
     reduction are native kernels; row filtering and the batch sort are torch ops.
     """
 
+    _n_ids_seen = 64  # see _n_ids_hint
+
     def __init__(self, voxel_num_limit=[64, 64, 64], unit_voxel_extent=[0.05, 0.05, 0.05],
                  voxelization_mode=4):
         super().__init__()
@@ -32,43 +34,54 @@ class Point2Voxel(nn.Module):
         self.voxelization_mode = voxelization_mode
         # The one-call path sizes its tables for batch ids below this number before it has
         # looked at the ids (the call checks on the device that they fit, and falls back
-        # when they do not): 64 for a first call, 1 + the largest id of the last call after.
-        self._n_ids_hint = 64
+        # when they do not): 1 + the largest id of the last call, of this module or, for its
+        # first call, of any other (64 before any call).
+        self._n_ids_hint = Point2Voxel._n_ids_seen
+        self._consts = None
         self.last_path = None  # which of the three ways the last forward took (diagnostics)
+
+    def _grid_consts(self):
+        """(half extent, unit) as float32 arrays, the same for the one-call path
+        (_ext.P2vConsts) and the grid shape as int64: made again when the module's extent or
+        limit were changed."""
+        key = (self.unit_voxel_extent.numpy().tobytes(), self.voxel_num_limit.tobytes())
+        held = self._consts
+        if held is None or held[0] != key:
+            unit = self.unit_voxel_extent.numpy().astype(np.float32)
+            limit = self.voxel_num_limit.astype(np.float32)
+            half = np.float32(0.5) * (limit * unit)  # fp32 throughout, as on the device
+            held = (key, (half, unit, _ext.P2vConsts(half, unit, self.voxel_num_limit),
+                          self.voxel_num_limit.astype(np.int64)))
+            self._consts = held
+        return held[1]
 
     def forward(self, point_cloud, feature, batch_ids):
         assert len(point_cloud.size()) == 2
         C = feature.size(1)
         device = point_cloud.device
 
-        unit = self.unit_voxel_extent.numpy().astype(np.float32)
-        limit = self.voxel_num_limit.astype(np.float32)
-        half = np.float32(0.5) * (limit * unit)  # fp32 throughout, as on the device
-
         # Clouds concatenated in batch order with small non-negative ids: filter and
         # partition in native kernels (one host read); anything else takes the
         # reference's sequence of torch operations below.
         # (the native filter keeps the features in the autograd graph when they carry a
         # gradient, as the reference's boolean-mask indexing does)
-        # One native call with one wait of the host when this module has seen the range of
-        # batch ids before (the call checks that they still fit).
+        # One native call with one wait of the host when the batch ids lie below the number
+        # the tables were sized for (the call checks that on the device).
         if self._n_ids_hint is not None and point_cloud.is_cuda:
-            one = _ext.p2v_voxelize(point_cloud, feature, batch_ids, half, unit,
-                                    self.voxel_num_limit, self.voxelization_mode,
-                                    self._n_ids_hint)
+            one = _ext.p2v_voxelize(point_cloud, feature, batch_ids, self._grid_consts()[2],
+                                    self.voxelization_mode, self._n_ids_hint)
             if one is not None:
-                valid_point_cloud, voxel_feats, voxel_index, valid_ids, origin_ids, alive = one
-                B1 = len(origin_ids)
+                valid_point_cloud, voxel_feats, voxel_index, valid_ids, B1, max_id, alive = one
                 valid_instance_flag = torch.ones(B1, dtype=torch.float32, device=device) \
-                    if bool(alive.all()) else torch.from_numpy(alive).to(device)
+                    if alive is None else torch.from_numpy(alive).to(device)
                 # (the rows carry the clouds' own ids: with gaps in the ids the tensor's batch
                 # size is 1 + the largest one, so that every row lies inside the grid)
-                sparse_feat = SparseTensor(voxel_feats, voxel_index,
-                                           self.voxel_num_limit.astype(np.int64),
-                                           max(B1, int(origin_ids[-1]) + 1))
+                sparse_feat = SparseTensor(voxel_feats, voxel_index, self._grid_consts()[3].copy(),
+                                           max(B1, max_id + 1))
                 self.last_path = "one call"
-                self._n_ids_hint = int(origin_ids[-1]) + 1
+                self._n_ids_hint = Point2Voxel._n_ids_seen = max_id + 1
                 return valid_point_cloud, sparse_feat, valid_ids, valid_instance_flag
+        half, unit = self._grid_consts()[:2]
         fast = _ext.p2v_filter(point_cloud, feature, batch_ids, half, unit) \
             if point_cloud.is_cuda else None
         if fast is not None:
