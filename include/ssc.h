@@ -400,7 +400,11 @@ int ssc_profile_conv(int32_t enable);
  * 256  no kernel of its own for float layers of at most 8 input channels (the first layer of
  *      a network on raw point features), which otherwise compute every output row in
  *      registers from a table of its input rows instead of on the matrix pipeline.  Changes
- *      the sizes; results agree up to the order of the float sums. */
+ *      the sizes; results agree up to the order of the float sums.
+ * 512  the schedule filled by a launch of its own for every plan: plans with one range to a
+ *      workgroup and a single work split otherwise have it filled range by range by the
+ *      launch that counts the ranges' row blocks.  Results are bit-identical (only where in
+ *      its buffers a range's part of the schedule lies differs). */
 int ssc_conv_tuning(int32_t flags);
 int ssc_profile_conv_read(float *ms /* host */, int32_t capacity, int32_t *count /* host */);
 

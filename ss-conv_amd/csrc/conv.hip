@@ -467,6 +467,7 @@ __global__ void __launch_bounds__(kMaxRanges)
       const int run = before + incl;
       tile_s[n_wg] = run;
       n_tiles_dev[0] = run;
+      n_tiles_dev[1] = 0;  // (the cursor of range_sched_kernel<true>)
       tile_row0[run] = (int32_t)n_out;
       spill_end[run] = (int32_t)n_out;
     }
@@ -608,6 +609,7 @@ __global__ void __launch_bounds__(256)
     if (threadIdx.x == 0) {
       flag[0] = 0;
       n_tiles_dev[0] = n_tiles;
+      n_tiles_dev[1] = 0;  // (the cursor of range_sched_kernel<true>)
       tile_row0[n_tiles] = n_out;
       spill_end[n_tiles] = n_out;
     }
@@ -700,15 +702,116 @@ __global__ void __launch_bounds__(256)
 // of the prefix over all tiles, the sum over the ranges before a tile's own (at most 256
 // numbers), every block of sched_fill_kernel takes for itself: three dependent launches
 // (shares, counts, a one-block scan) became one.
+// FILL (plans with one range to a workgroup and a single work split): the block goes on to
+// fill its range's part of the schedule (what sched_fill_kernel does, sixteen threads to a
+// (tile, offset)), at the groups it takes from a cursor that all ranges share -- in whatever
+// order the blocks get there: a workgroup of the convolution finds its groups through
+// wg_grp, and nothing else depends on where in the buffers they lie.
+// What the schedule of one (tile, offset) is filled from and into (sched_fill_item).
+struct SchedFill {
+  const int32_t *pairs, *sorted, *flag;
+  int64_t pair_stride;
+  int plane_g;
+  const int32_t *tile_row0, *tile_slot0;
+  int T;
+  uint32_t in_scale, in_pad;
+  int out_scale, k_scale;
+  int32_t *sched_in, *sched_out, *grp_meta;
+};
+
+// Lane `lane` of the 16 threads of (tile t, offset k) fills slot `lane` of each of their row
+// blocks; the threads of offset 0 also write the tile's padding blocks and the tile fields of
+// its groups [g0, g1).
+// `first` (optional): what the loads of the first four row blocks return, issued by the
+// caller together with those of other combinations (first[0..3] gather rows, [4..7] scatter
+// rows, [8] tile_row0[t], [9] tile_slot0[t]).
+__device__ __forceinline__ void sched_fill_item(const SchedFill &f, int64_t t, int k, int lane,
+                                                int64_t g0, int64_t g1, int s0, int n, int kof,
+                                                int nmb, const int *first = nullptr) {
+  const int T = f.T, out_scale = f.out_scale, k_scale = f.k_scale, plane_g = f.plane_g;
+  const uint32_t in_scale = f.in_scale, in_pad = f.in_pad;
+  const int64_t pair_stride = f.pair_stride;
+  const int32_t *__restrict__ tile_row0 = f.tile_row0, *__restrict__ tile_slot0 = f.tile_slot0;
+  int32_t *__restrict__ sched_in = f.sched_in, *__restrict__ sched_out = f.sched_out,
+                       *__restrict__ grp_meta = f.grp_meta;
+  const int32_t *src = f.flag[0] ? f.sorted : f.pairs;
+  if (k == 0) {
+    for (int64_t g = g0 + lane; g < g1; g += 16) {
+      const int rows = tile_row0[t + 1] - tile_row0[t];
+      grp_meta[g * 8 + 4] = tile_row0[t];
+      grp_meta[g * 8 + 5] = g + 1 == g1 ? rows : -rows;
+      grp_meta[g * 8 + 6] = tile_slot0[t];
+      grp_meta[g * 8 + 7] = 0;
+    }
+    for (int64_t mb = g0 * 4 + nmb; mb < g1 * 4; ++mb) {
+      sched_in[mb * 16 + lane] = (int32_t)in_pad;
+      sched_out[mb * 16 + lane] = T * out_scale;
+      if (lane == 0) grp_meta[(mb >> 2) * 8 + (mb & 3)] = 0;
+    }
+  }
+  if (n <= 0) return;
+  const int32_t *pg = src + ((int64_t)k * 2 + plane_g) * pair_stride + s0;
+  const int32_t *ps = src + ((int64_t)k * 2 + (1 - plane_g)) * pair_stride + s0;
+  int64_t mb = g0 * 4 + kof;
+  // accumulator slot of a row: rows map to slots modulo the window height T; the
+  // rows a tile touches span less than T, so one conditional subtraction does it
+  const int slot_off = first ? first[9] - first[8] : tile_slot0[t] - tile_row0[t];
+  // four row blocks at a time: their loads are issued together
+  const int n16 = (n + 15) & ~15;
+  for (int p0 = lane; p0 < n16; p0 += 64, mb += 4) {
+    int gi[4], so[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int p = p0 + 16 * u;
+      if (first != nullptr && p0 == lane) {
+        gi[u] = first[u];
+        so[u] = first[4 + u];
+      } else {
+        gi[u] = p < n ? pg[p] : 0;
+        so[u] = p < n ? ps[p] : 0;
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int p = p0 + 16 * u;
+      if (p < n16) {
+        const int64_t b = mb + u;
+        sched_in[b * 16 + lane] = p < n ? (int32_t)((uint32_t)gi[u] * in_scale) : (int32_t)in_pad;
+        int slot = T;
+        if (p < n) {
+          slot = so[u] + slot_off;
+          if (slot >= T) slot -= T;
+        }
+        sched_out[b * 16 + lane] = slot * out_scale;
+        if (lane == 0) grp_meta[(b >> 2) * 8 + (b & 3)] = k * k_scale;
+      }
+    }
+  }
+}
+
 constexpr int kRangeSchedThreads = 1024;  // sixteen tiles at a time in the second step
-__global__ void __launch_bounds__(kRangeSchedThreads)
-    range_sched_kernel(const int32_t *__restrict__ segs, const int32_t *__restrict__ spill, int K,
-                       const int32_t *__restrict__ wg_tile, int32_t *__restrict__ share_first,
-                       int32_t *__restrict__ share_cnt, int32_t *__restrict__ kofs,
-                       int32_t *__restrict__ tile_nmb, int32_t *__restrict__ tile_loc,
-                       int32_t *__restrict__ tile_rng, int32_t *__restrict__ range_grp) {
-  const int w = blockIdx.x;
-  const int t0 = wg_tile[w], t1 = wg_tile[w + 1];
+constexpr int kFillItems = 2048;  // (tile, offset) combinations of a range whose shares stay in LDS
+constexpr int kFillTiles = 256;   // tiles of such a range
+
+// The steps of range_sched_kernel for one range.  LDS: shares, block offsets and the tiles'
+// counts live in LDS (the FILL form, a range of at most kFillItems (tile, offset)
+// combinations and kFillTiles tiles: what follows reads them without a trip to memory) --
+// otherwise in the global arrays, where sched_fill_kernel finds them.
+template <bool FILL, bool LDS>
+__device__ __forceinline__ void range_sched_steps(
+    const int32_t *__restrict__ segs, const int32_t *__restrict__ spill, int K, int w, int t0,
+    int t1, int32_t *share_first, int32_t *share_cnt, int32_t *kofs, int32_t *tile_nmb,
+    int32_t *tile_loc, int32_t *__restrict__ tile_rng, int32_t *__restrict__ range_grp,
+    const SchedFill &fill, int32_t *__restrict__ cursor, int32_t *__restrict__ wg_grp,
+    int *sf_s, int *sc_s, int *ko_s, int *tn_s, int *tl_s, int *range_base_s) {
+  auto item = [&](int64_t t, int k) -> int64_t { return LDS ? (t - t0) * K + k : t * K + k; };
+  int *const sf = LDS ? sf_s : share_first;
+  int *const sc = LDS ? sc_s : share_cnt;
+  int *const ko = LDS ? ko_s : kofs;
+  // (indices, not shifted pointers: an LDS pointer must stay inside its array)
+  auto tile = [&](int64_t t) -> int64_t { return LDS ? t - t0 : t; };
+  int *const tn = LDS ? tn_s : tile_nmb;
+  int *const tl = LDS ? tl_s : tile_loc;
   for (int k = threadIdx.x; k < K && t0 < t1; k += blockDim.x) {
     int s = segs[(int64_t)t0 * K + k];
     // eight tiles at a time: their loads are issued together, the chain through s is
@@ -731,8 +834,8 @@ __global__ void __launch_bounds__(kRangeSchedThreads)
             e = s + ((q[u] - s + 15) & ~15);
             if (e > lim[u]) e = lim[u];
           }
-          share_first[(int64_t)t * K + k] = s;
-          share_cnt[(int64_t)t * K + k] = e - s;
+          sf[item(t, k)] = s;
+          sc[item(t, k)] = e - s;
           s = e;
         }
       }
@@ -745,20 +848,20 @@ __global__ void __launch_bounds__(kRangeSchedThreads)
     int run = 0;
     for (int k0 = 0; k0 < K; k0 += 64) {
       const int k = k0 + lane;
-      const int nb = k < K ? (share_cnt[t * K + k] + 15) >> 4 : 0;
+      const int nb = k < K ? (sc[item(t, k)] + 15) >> 4 : 0;
       int incl = nb;
 #pragma unroll
       for (int d = 1; d < 64; d <<= 1) {
         int o = __shfl_up(incl, d, 64);
         if (lane >= d) incl += o;
       }
-      if (k < K) kofs[t * K + k] = run + incl - nb;
+      if (k < K) ko[item(t, k)] = run + incl - nb;
       run += __shfl(incl, 63, 64);
     }
     if (lane == 0) {
-      tile_nmb[t] = run;
+      tn[tile(t)] = run;
       const int groups = (run + 3) >> 2;
-      tile_loc[t] = groups > 0 ? groups : 1;  // a tile without pairs gets an empty group
+      tl[tile(t)] = groups > 0 ? groups : 1;  // a tile without pairs gets an empty group
     }
   }
   __threadfence_block();
@@ -767,7 +870,7 @@ __global__ void __launch_bounds__(kRangeSchedThreads)
     int carry = 0;
     for (int base = t0; base < t1; base += 64) {
       const int t = base + lane;
-      const int v = t < t1 ? tile_loc[t] : 0;
+      const int v = t < t1 ? tl[tile(t)] : 0;
       int incl = v;
 #pragma unroll
       for (int d = 1; d < 64; d <<= 1) {
@@ -775,13 +878,90 @@ __global__ void __launch_bounds__(kRangeSchedThreads)
         if (lane >= d) incl += o;
       }
       if (t < t1) {
-        tile_loc[t] = carry + incl - v;
-        tile_rng[t] = w;
+        tl[tile(t)] = carry + incl - v;
+        if (!FILL) tile_rng[t] = w;
       }
       carry += __shfl(incl, 63, 64);
     }
     if (lane == 0) range_grp[w] = carry;
+    if (FILL && lane == 0) {
+      const int base = atomicAdd(cursor, carry);
+      wg_grp[2 * w] = base;
+      wg_grp[2 * w + 1] = base + carry;
+      range_base_s[0] = base;
+      range_base_s[1] = base + carry;
+    }
   }
+  if (!FILL) return;
+  __threadfence_block();
+  __syncthreads();
+  const int64_t base = range_base_s[0], end = range_base_s[1];
+  // A team of sixteen threads takes three (tile, offset) combinations at a time and issues
+  // the loads of all three before it stores anything: a range has a few hundred combinations
+  // for its 64 teams, and one after the other each would wait for its own loads.
+  const int team = threadIdx.x >> 4, l16 = threadIdx.x & 15;
+  constexpr int U = 3, kTeams = kRangeSchedThreads / 16;
+  const int64_t tk_end = (int64_t)t1 * K;
+  const int32_t *src = fill.flag[0] ? fill.sorted : fill.pairs;
+  for (int64_t tk0 = (int64_t)t0 * K + team; tk0 < tk_end; tk0 += U * kTeams) {
+    int first[U][10], s0[U], n[U];
+    int64_t tt[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int64_t tk = tk0 + u * kTeams;
+      const bool live = tk < tk_end;
+      const int64_t t = live ? tk / K : t0;
+      const int k = live ? (int)(tk - t * K) : 0;
+      tt[u] = t;
+      s0[u] = sf[item(t, k)];
+      n[u] = live ? sc[item(t, k)] : 0;
+      const int32_t *pg = src + ((int64_t)k * 2 + fill.plane_g) * fill.pair_stride + s0[u];
+      const int32_t *ps = src + ((int64_t)k * 2 + (1 - fill.plane_g)) * fill.pair_stride + s0[u];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int p = l16 + 16 * j;
+        first[u][j] = p < n[u] ? pg[p] : 0;
+        first[u][4 + j] = p < n[u] ? ps[p] : 0;
+      }
+      first[u][8] = fill.tile_row0[t];
+      first[u][9] = fill.tile_slot0[t];
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int64_t tk = tk0 + u * kTeams;
+      if (tk < tk_end) {
+        const int64_t t = tt[u];
+        const int k = (int)(tk - t * K);
+        const int64_t g0 = base + tl[tile(t)];
+        const int64_t g1 = t + 1 < t1 ? base + tl[tile(t + 1)] : end;
+        sched_fill_item(fill, t, k, l16, g0, g1, s0[u], n[u], ko[item(t, k)], tn[tile(t)],
+                        first[u]);
+      }
+    }
+  }
+}
+
+template <bool FILL>
+__global__ void __launch_bounds__(kRangeSchedThreads)
+    range_sched_kernel(const int32_t *__restrict__ segs, const int32_t *__restrict__ spill, int K,
+                       const int32_t *__restrict__ wg_tile, int32_t *share_first,
+                       int32_t *share_cnt, int32_t *kofs, int32_t *tile_nmb, int32_t *tile_loc,
+                       int32_t *__restrict__ tile_rng, int32_t *__restrict__ range_grp,
+                       SchedFill fill, int32_t *__restrict__ cursor,
+                       int32_t *__restrict__ wg_grp) {
+  const int w = blockIdx.x;
+  __shared__ int range_base_s[2];
+  __shared__ int sf_s[FILL ? kFillItems : 1], sc_s[FILL ? kFillItems : 1],
+      ko_s[FILL ? kFillItems : 1], tn_s[FILL ? kFillTiles : 1], tl_s[FILL ? kFillTiles : 1];
+  const int t0 = wg_tile[w], t1 = wg_tile[w + 1];
+  if (FILL && (int64_t)(t1 - t0) * K <= kFillItems && t1 - t0 <= kFillTiles)
+    range_sched_steps<FILL, true>(segs, spill, K, w, t0, t1, share_first, share_cnt, kofs,
+                                  tile_nmb, tile_loc, tile_rng, range_grp, fill, cursor, wg_grp,
+                                  sf_s, sc_s, ko_s, tn_s, tl_s, range_base_s);
+  else
+    range_sched_steps<FILL, false>(segs, spill, K, w, t0, t1, share_first, share_cnt, kofs,
+                                   tile_nmb, tile_loc, tile_rng, range_grp, fill, cursor, wg_grp,
+                                   sf_s, sc_s, ko_s, tn_s, tl_s, range_base_s);
 }
 
 // Two ranges to a workgroup (n_rng = 2 n_wg): which two, by the row-block groups the ranges
@@ -791,7 +971,7 @@ __global__ void __launch_bounds__(kRangeSchedThreads)
 // with the one with the fewest, the second with the last but one, ...: 16 workgroups whose
 // sums differ far less than the ranges do.  One block.  range_g0[r]: first group of range r
 // in the schedule, where a workgroup's two ranges follow each other, the one of the lower
-// rows first; wg_grp[v], v = 0..n_wg: first group of workgroup v.
+// rows first; wg_grp[2 v], wg_grp[2 v + 1]: first group of workgroup v and the one behind its last.
 __global__ void __launch_bounds__(kMaxRanges)
     range_assign_kernel(const int32_t *__restrict__ range_grp, int n_rng, int n_wg,
                         int32_t *__restrict__ range_g0, int32_t *__restrict__ wg_grp) {
@@ -833,7 +1013,10 @@ __global__ void __launch_bounds__(kMaxRanges)
     sum_s[n_wg] = run;
   }
   __syncthreads();
-  if (r <= n_wg) wg_grp[r] = sum_s[r];
+  if (r < n_wg) {
+    wg_grp[2 * r] = sum_s[r];
+    wg_grp[2 * r + 1] = sum_s[r + 1];
+  }
   if (r < n_wg) {
     const int a = member_s[2 * r], b = member_s[2 * r + 1];
     range_g0[a] = sum_s[r];
@@ -883,8 +1066,10 @@ __global__ void __launch_bounds__(256)
     if (w == 255) range_g0[256] = before + incl;
     __syncthreads();
     if (blockIdx.x == 0) {
-      for (int i = threadIdx.x; i <= n_wg; i += blockDim.x)
-        wg_grp[i] = range_g0[i];
+      for (int i = threadIdx.x; i < n_wg; i += blockDim.x) {
+        wg_grp[2 * i] = range_g0[i];
+        wg_grp[2 * i + 1] = range_g0[i + 1];
+      }
     }
   }
   const int64_t n_tiles = n_tiles_dev[0];
@@ -900,55 +1085,10 @@ __global__ void __launch_bounds__(256)
   const int64_t g0 = rg0 + tile_loc[t];
   const int64_t g1 = (t + 1 < n_tiles && tile_rng[t + 1] == rng) ? rg0 + tile_loc[t + 1]
                                                                 : rg0 + range_grp[rng];
-  if (k == 0) {
-    for (int64_t g = g0 + lane; g < g1; g += 16) {
-      const int rows = tile_row0[t + 1] - tile_row0[t];
-      grp_meta[g * 8 + 4] = tile_row0[t];
-      grp_meta[g * 8 + 5] = g + 1 == g1 ? rows : -rows;
-      grp_meta[g * 8 + 6] = tile_slot0[t];
-      grp_meta[g * 8 + 7] = 0;
-    }
-    for (int64_t mb = g0 * 4 + tile_nmb[t]; mb < g1 * 4; ++mb) {
-      sched_in[mb * 16 + lane] = (int32_t)in_pad;
-      sched_out[mb * 16 + lane] = T * out_scale;
-      if (lane == 0) grp_meta[(mb >> 2) * 8 + (mb & 3)] = 0;
-    }
-  }
-  int s0 = share_first[t * K + k];
-  int n = share_cnt[t * K + k];
-  if (n <= 0) return;
-  const int32_t *pg = src + ((int64_t)k * 2 + plane_g) * pair_stride + s0;
-  const int32_t *ps = src + ((int64_t)k * 2 + (1 - plane_g)) * pair_stride + s0;
-  int64_t mb = g0 * 4 + kofs[t * K + k];
-  // accumulator slot of a row: rows map to slots modulo the window height T; the
-  // rows a tile touches span less than T, so one conditional subtraction does it
-  const int slot_off = tile_slot0[t] - tile_row0[t];
-  // four row blocks at a time: their loads are issued together
-  const int n16 = (n + 15) & ~15;
-  for (int p0 = lane; p0 < n16; p0 += 64, mb += 4) {
-    int gi[4], so[4];
-#pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      const int p = p0 + 16 * u;
-      gi[u] = p < n ? pg[p] : 0;
-      so[u] = p < n ? ps[p] : 0;
-    }
-#pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      const int p = p0 + 16 * u;
-      if (p < n16) {
-        const int64_t b = mb + u;
-        sched_in[b * 16 + lane] = p < n ? (int32_t)((uint32_t)gi[u] * in_scale) : (int32_t)in_pad;
-        int slot = T;
-        if (p < n) {
-          slot = so[u] + slot_off;
-          if (slot >= T) slot -= T;
-        }
-        sched_out[b * 16 + lane] = slot * out_scale;
-        if (lane == 0) grp_meta[(b >> 2) * 8 + (b & 3)] = k * k_scale;
-      }
-    }
-  }
+  SchedFill f = {pairs, sorted, flag, pair_stride, plane_g, tile_row0, tile_slot0, T, in_scale,
+                 in_pad, out_scale, k_scale, sched_in, sched_out, grp_meta};
+  sched_fill_item(f, t, k, lane, g0, g1, share_first[t * K + k], share_cnt[t * K + k],
+                  kofs[t * K + k], tile_nmb[t]);
 }
 
 
@@ -987,6 +1127,7 @@ constexpr int64_t kRebalanceStages = 1500;
 constexpr int64_t kPairGroups = 250;
 static bool g_conv_pair = true, g_conv_pair_always = false;
 static int64_t g_conv_rebalance_stages = kRebalanceStages;
+static bool g_conv_fuse_fill = true;  // range_sched_kernel<true> instead of sched_fill_kernel
 static bool g_conv_rebalance = true;  // long kernels: a second work split from the first one's counts
 static bool g_conv_round8 = false;    // ranges per column block: a multiple of 8 only
 static bool g_conv_small = true;      // layers of at most 8 input channels: conv_small_kernel
@@ -1100,7 +1241,7 @@ static size_t conv_plan_walk(void *base, const ConvPlan &p, ConvWs *w) {
     return c.used;
   }
   int32_t *wg_tile = c.take<int32_t>((size_t)p.n_rng + 1);
-  int32_t *wg_grp = c.take<int32_t>((size_t)p.n_wg + 1);
+  int32_t *wg_grp = c.take<int32_t>(2 * (size_t)p.n_wg);
   int32_t *sched_in = c.take<int32_t>((size_t)p.grp_cap * 64);
   int32_t *sched_out = c.take<int32_t>((size_t)p.grp_cap * 64);
   int32_t *grp_meta = c.take<int32_t>((size_t)p.grp_cap * 8);
@@ -1144,7 +1285,7 @@ static size_t conv_scratch_walk(void *base, const ConvPlan &p, int K, int64_t pa
   t.spill = c.take<int32_t>((size_t)(p.n_tiles + 1) * K);
   t.share_first = c.take<int32_t>((size_t)p.n_tiles * K);
   t.share_cnt = c.take<int32_t>((size_t)p.n_tiles * K);
-  t.n_tiles_dev = c.take<int32_t>(1);
+  t.n_tiles_dev = c.take<int32_t>(2);  // [1]: cursor over the schedule's groups
   t.tile_rng = c.take<int32_t>((size_t)p.n_tiles + 1);
   t.range_grp = c.take<int32_t>((size_t)p.n_rng + 1);
   t.range_row1 = c.take<int32_t>((size_t)p.n_rng + 1);
@@ -1302,6 +1443,7 @@ int ssc_conv_tuning(int32_t flags) {
   g_conv_pair = (flags & 64) == 0;
   g_conv_pair_always = (flags & 128) != 0;
   g_conv_small = (flags & 256) == 0;
+  g_conv_fuse_fill = (flags & 512) == 0;
   return SSC_OK;
 }
 
@@ -1349,6 +1491,24 @@ static int conv_plan_build(const ConvPlan &p, const ConvWs &w, const int32_t *pa
                            const PackArgs *pack, hipStream_t s, bool seeded = false) {
   const int plane_g = inverse ? 1 : 0;
   const int plane_s = 1 - plane_g;
+  int rc;
+  const int frag_bytes = elem_bytes == 2 ? Io<_Float16>::kFragBytes : Io<float>::kFragBytes;
+  const SchedFill fill = {pairs, w.sorted, w.flag, pair_stride, plane_g, w.tile_row0,
+                          w.tile_slot0, p.T,
+                          p.gather ? (uint32_t)c_in * (uint32_t)elem_bytes : 1u,
+                          p.gather ? kGatherPad : 0xFFFFFFFFu, (p.acc_cols + 4) * 4,
+                          p.ncb * p.nch * frag_bytes, w.sched_in, w.sched_out, w.grp_meta};
+  // One range to a workgroup and a single work split: the launch that counts a range's row
+  // blocks goes on to fill its schedule (no sched_fill_kernel).
+  const bool fuse_fill = g_conv_fuse_fill && !p.rebalance && p.n_rng == p.n_wg;
+  auto range_sched = [&]() -> int {
+    hipLaunchKernelGGL(fuse_fill ? range_sched_kernel<true> : range_sched_kernel<false>,
+                       dim3((unsigned)p.n_rng), dim3(kRangeSchedThreads), 0, s, w.segs, w.spill,
+                       K, w.wg_tile, w.share_first, w.share_cnt, w.kofs, w.tile_nmb, w.tile_loc,
+                       w.tile_rng, w.range_grp, fill, w.n_tiles_dev + 1, w.wg_grp);
+    SSC_LAUNCH_CHECK("range_sched");
+    return SSC_OK;
+  };
   if (seeded) {
     // The range boundaries are in w.range_row0 already (a rulebook placed them, see
     // SplitRequest): the tiles and their segments in one launch from the pairs' side, then
@@ -1361,10 +1521,8 @@ static int conv_plan_build(const ConvPlan &p, const ConvWs &w, const int32_t *pa
                        p.tile_rows, p.T, (int)n_out, w.wg_tile, w.tile_row0, w.n_tiles_dev,
                        w.spill_end, w.tile_slot0, w.segs, w.spill);
     SSC_LAUNCH_CHECK("pair_tile_segments");
-    hipLaunchKernelGGL(range_sched_kernel, dim3((unsigned)p.n_rng), dim3(kRangeSchedThreads), 0, s,
-                       w.segs, w.spill, K, w.wg_tile, w.share_first, w.share_cnt, w.kofs,
-                       w.tile_nmb, w.tile_loc, w.tile_rng, w.range_grp);
-    SSC_LAUNCH_CHECK("range_sched");
+    if ((rc = range_sched()) != SSC_OK) return rc;
+    if (fuse_fill) return SSC_OK;
   }
   const int64_t packed_n = pack ? (int64_t)K * p.ncb * p.nch * 1024 : 0;
   PackArgs pk = {nullptr, 0, 0, 0, 0, 0, 0, 0, 0, nullptr, 16};
@@ -1436,14 +1594,11 @@ static int conv_plan_build(const ConvPlan &p, const ConvWs &w, const int32_t *pa
                        w.tile_row0, n_out, w.fine_segs, p.granule, w.spill_end, w.segs,
                        w.spill);
     SSC_LAUNCH_CHECK("tile_segments");
-    hipLaunchKernelGGL(range_sched_kernel, dim3((unsigned)p.n_rng), dim3(kRangeSchedThreads), 0, s,
-                       w.segs, w.spill, K, w.wg_tile, w.share_first, w.share_cnt, w.kofs,
-                       w.tile_nmb, w.tile_loc, w.tile_rng, w.range_grp);
-    SSC_LAUNCH_CHECK("range_sched");
-    return SSC_OK;
+    return range_sched();
   };
-  int rc = seeded ? SSC_OK : tiles_of(w.range_row0);
+  rc = seeded ? SSC_OK : tiles_of(w.range_row0);
   if (rc != SSC_OK) return rc;
+  if (fuse_fill) return SSC_OK;
   if (p.rebalance) {  // long kernels: once more, from the groups the ranges came to
     hipLaunchKernelGGL(split_rebalance_kernel, dim3((unsigned)ceil_div(p.n_fine + 1, 256)),
                        dim3(256), 0, s, w.fine_segs, K, p.n_fine, n_out, p.tile_rows, p.n_rng,
@@ -1458,7 +1613,6 @@ static int conv_plan_build(const ConvPlan &p, const ConvWs &w, const int32_t *pa
                        p.n_wg, w.range_g0, w.wg_grp);
     SSC_LAUNCH_CHECK("range_assign");
   }
-  const int frag_bytes = elem_bytes == 2 ? Io<_Float16>::kFragBytes : Io<float>::kFragBytes;
   hipLaunchKernelGGL(sched_fill_kernel, dim3((unsigned)ceil_div(p.n_tiles * K * 16, 256)),
                      dim3(256), 0, s, w.flag, pairs, w.sorted, pair_stride, plane_g,
                      w.share_first, w.share_cnt, w.kofs, w.tile_nmb, w.tile_loc, w.tile_rng,

@@ -255,7 +255,7 @@ __global__ void __launch_bounds__((NCW + 4) * 64)
       }
     }
   }
-  const int g_begin = wg_grp[chunk], g_end = wg_grp[chunk + 1];  // this workgroup's groups
+  const int g_begin = wg_grp[2 * chunk], g_end = wg_grp[2 * chunk + 1];  // this workgroup's groups
   const int nstages = (g_end - g_begin) * nch;  // stages of this workgroup
   const int col0 = col_base + cblk * kCN;
   static_assert(FORM == 0 || (NCW == 4 && !kHalf), "the other forms are built for float");
@@ -1191,7 +1191,7 @@ int conv_small_run(const float *features, int c_in, const void *packed, int ncb,
 struct ConvWs {
   void *packed;
   // plan
-  int32_t *wg_tile, *wg_grp;  // first tile of every range; first group of every workgroup
+  int32_t *wg_tile, *wg_grp;  // first tile of every range; first and end group of every workgroup
   int32_t *sched_in, *sched_out, *grp_meta;
   int32_t *small_table;  // [K, n_out] (plans of ConvPlan::small, which have nothing else)
   // scratch

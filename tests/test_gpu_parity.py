@@ -519,6 +519,29 @@ def test_conv_five_group_form(shape, oracle, device):
 
 @pytest.mark.parametrize("case", [(2500, 16, 3, 1, 1, 64, 128), (900, 12, 3, 2, 1, 128, 256),
                                   (400, 10, 5, 1, 2, 200, 200), (5, 8, 3, 1, 1, 5, 7),
+                                  (2500, 16, 3, 1, 1, 64, 72), (1, 4, 3, 1, 1, 16, 16)])
+def test_conv_schedule_filled_range_by_range(case, oracle, device):
+    """Plans with one range to a workgroup have their schedule filled by the launch that counts
+    the ranges' row blocks, every range at the groups it takes from a shared cursor; with
+    ssc_conv_tuning flag 512 a launch of its own fills it with the ranges in order.  The
+    convolution's result does not depend on where a range's groups lie: bit-equal, run after
+    run."""
+    from ss_conv import _ext
+    print("case", case, flush=True)
+    n, grid, k, s, p, cin, cout = case
+    a, _ = _conv_case(oracle, device, n, grid, k, s, p, cin, cout, seed=43)
+    a2, _ = _conv_case(oracle, device, n, grid, k, s, p, cin, cout, seed=43)
+    try:
+        assert _ext._lib.ssc_conv_tuning(1 | 512) == 0
+        b, _ = _conv_case(oracle, device, n, grid, k, s, p, cin, cout, seed=43)
+    finally:
+        _ext._lib.ssc_conv_tuning(1)
+    assert torch.equal(a, a2)
+    assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("case", [(2500, 16, 3, 1, 1, 64, 128), (900, 12, 3, 2, 1, 128, 256),
+                                  (400, 10, 5, 1, 2, 200, 200), (5, 8, 3, 1, 1, 5, 7),
                                   (2500, 16, 3, 1, 1, 64, 72), (3000, 16, 3, 1, 1, 3, 152)])
 @pytest.mark.parametrize("flags", [32, 128, 32 | 128])
 def test_conv_second_work_split(case, flags, oracle, device):
