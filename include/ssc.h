@@ -156,9 +156,9 @@ int ssc_rulebook_rows(const ssc_geometry *g, int64_t n_in, void *workspace,
  * rows, so results agree up to the order of the float sums.
  * `filters` (may be NULL): the arguments of ssc_kernel_combine_packed_f32 for the layer's
  * own filters (c_in and c_out are the call's).  The synthesis depends on nothing the
- * rulebook computes, so it is enqueued inside the rulebook's first launch where that launch
- * has a grid to share (stride 1, dilation 1) and as a launch of its own before it elsewhere:
- * either way `out` and `packed` are ready for whatever the stream runs after this call. */
+ * rulebook computes, so it is enqueued inside the rulebook's first launch (more blocks of the
+ * kernel that marks the rows' cells; a launch of its own when there are no rows): `out` and
+ * `packed` are ready for whatever the stream runs after this call. */
 typedef struct ssc_combine_job {
   const float *weight, *basis;
   const int32_t *chan_out, *chan_in, *blocks;

@@ -119,6 +119,16 @@ __device__ __forceinline__ bool row_usable(const int32_t *row, const Geom &g) {
   return cell_in_range(*reinterpret_cast<const int4 *>(row), g.batch, g.os[0], g.os[1], g.os[2]);
 }
 
+// The share of grid row `row` of `rows` (of gridDim.x blocks of 256 threads each) in a
+// layer's filter job.
+__device__ __forceinline__ void combine_job_rows(const CombineJob &job, int64_t job_elements,
+                                                 int row, int rows) {
+  const int64_t step = (int64_t)rows * gridDim.x * 256;
+  for (int64_t idx = ((int64_t)row * gridDim.x + blockIdx.x) * 256 + threadIdx.x;
+       idx < job_elements; idx += step)
+    combine_pack_element(job, idx);
+}
+
 // Regular conv: mark every output cell reachable from an active input, and count
 // the pairs of every 64-row chunk (chunk_count is [K, n_chunks]; for a regular
 // convolution a pair exists wherever the geometry allows it, so the counts do not
@@ -128,10 +138,20 @@ __device__ __forceinline__ bool row_usable(const int32_t *row, const Geom &g) {
 // in the key space: their bits are gathered into one mask per 32-bit word, the word
 // is read first, and the atomic is issued only when it would change the word
 // (most cells are reached from several inputs).
+// JOB: the grid rows from ks[0] on synthesise and pack the layer's filters (work that
+// depends on nothing here and that the layer would otherwise launch by itself).
+template <bool JOB>
 __global__ void __launch_bounds__(256)
     mark_count_kernel(const int32_t *__restrict__ indices, int64_t n_in, Geom g,
                       uint32_t *__restrict__ bits, int32_t *__restrict__ chunk_count,
-                      int64_t n_chunks, int32_t *__restrict__ disorder) {
+                      int64_t n_chunks, int32_t *__restrict__ disorder, CombineJob job,
+                      int64_t job_elements) {
+  if constexpr (JOB) {
+    if ((int)blockIdx.y >= g.ks[0]) {
+      combine_job_rows(job, job_elements, (int)blockIdx.y - g.ks[0], (int)gridDim.y - g.ks[0]);
+      return;
+    }
+  }
   int64_t chunk = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (chunk >= n_chunks) return;
   const int lane = threadIdx.x & 63;
@@ -211,8 +231,7 @@ static inline int64_t dense_in_words(const Geom &g, const DenseIn &d) {
 
 // As mark_count_kernel (same grid, same chunk counts, same flags), but the wave marks the
 // cells of its input rows in the input table instead of the output cells they reach.
-// JOB: the grid rows from ks[0] on synthesise and pack the layer's filters (work that
-// depends on nothing here and that the layer would otherwise launch by itself).
+// JOB: as for mark_count_kernel.
 template <bool JOB>
 __global__ void __launch_bounds__(256)
     mark_in_count_kernel(const int32_t *__restrict__ indices, int64_t n_in, Geom g, DenseIn d,
@@ -221,11 +240,7 @@ __global__ void __launch_bounds__(256)
                          int64_t job_elements) {
   if constexpr (JOB) {
     if ((int)blockIdx.y >= g.ks[0]) {
-      const int64_t step = (int64_t)(gridDim.y - g.ks[0]) * gridDim.x * 256;
-      for (int64_t idx = ((int64_t)(blockIdx.y - g.ks[0]) * gridDim.x + blockIdx.x) * 256 +
-                         threadIdx.x;
-           idx < job_elements; idx += step)
-        combine_pack_element(job, idx);
+      combine_job_rows(job, job_elements, (int)blockIdx.y - g.ks[0], (int)gridDim.y - g.ks[0]);
       return;
     }
   }
@@ -268,9 +283,22 @@ __global__ void __launch_bounds__(256)
 }
 
 // Submanifold / unique: mark the cells of the rows themselves.
+// JOB: the blocks behind those of the rows work on a layer's filter job (see mark_count_kernel).
+template <bool JOB>
 __global__ void __launch_bounds__(256)
     mark_rows_kernel(const int32_t *__restrict__ coords, int64_t n, int d0, int d1, int d2, int d3,
-                     uint32_t *__restrict__ bits, int32_t *__restrict__ flags, int want_order) {
+                     uint32_t *__restrict__ bits, int32_t *__restrict__ flags, int want_order,
+                     CombineJob job, int64_t job_elements) {
+  if constexpr (JOB) {
+    const int64_t row_blocks = (n + 255) / 256;
+    if ((int64_t)blockIdx.x >= row_blocks) {
+      const int64_t step = ((int64_t)gridDim.x - row_blocks) * 256;
+      for (int64_t idx = ((int64_t)blockIdx.x - row_blocks) * 256 + threadIdx.x;
+           idx < job_elements; idx += step)
+        combine_pack_element(job, idx);
+      return;
+    }
+  }
   int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= n) return;
   int4 r = reinterpret_cast<const int4 *>(coords)[i];
@@ -967,15 +995,35 @@ static int rulebook_mark_and_scan(const int32_t *indices, int64_t n_in, const Ge
   }
   if ((rc = bit_table_clear(w.table, s)) != SSC_OK) return rc;
   if (gg.subm) {
-    hipLaunchKernelGGL(mark_rows_kernel, dim3((unsigned)ceil_div(n_in, 256)), dim3(256), 0, s,
-                       indices, n_in, gg.batch, gg.os[0], gg.os[1], gg.os[2], w.table.bits,
-                       w.table.total + 1, 1);
+    if (job != nullptr) {
+      const int64_t n = combine_job_elements(*job);
+      const int64_t more = std::min<int64_t>(ceil_div(n, 256), 4096);
+      hipLaunchKernelGGL(mark_rows_kernel<true>, dim3((unsigned)(ceil_div(n_in, 256) + more)),
+                         dim3(256), 0, s, indices, n_in, gg.batch, gg.os[0], gg.os[1], gg.os[2],
+                         w.table.bits, w.table.total + 1, 1, *job, n);
+    } else {
+      hipLaunchKernelGGL(mark_rows_kernel<false>, dim3((unsigned)ceil_div(n_in, 256)), dim3(256), 0,
+                         s, indices, n_in, gg.batch, gg.os[0], gg.os[1], gg.os[2], w.table.bits,
+                         w.table.total + 1, 1, CombineJob{}, (int64_t)0);
+    }
     SSC_LAUNCH_CHECK("mark_rows");
     return bit_table_scan(w.table, s, mirror, ticket);
   }
-  hipLaunchKernelGGL(mark_count_kernel, dim3((unsigned)ceil_div(w.n_chunks, 4), (unsigned)gg.ks[0]),
-                     dim3(256), 0, s, indices, n_in, gg, w.table.bits, w.chunk_count, w.n_chunks,
-                     w.table.total + 1);
+  {
+    const int64_t mark_blocks = ceil_div(w.n_chunks, 4);
+    if (job != nullptr) {
+      const int64_t n = combine_job_elements(*job);
+      const int64_t rows = std::min<int64_t>(ceil_div(ceil_div(n, 256), mark_blocks), 1024);
+      hipLaunchKernelGGL(mark_count_kernel<true>,
+                         dim3((unsigned)mark_blocks, (unsigned)(gg.ks[0] + rows)), dim3(256), 0, s,
+                         indices, n_in, gg, w.table.bits, w.chunk_count, w.n_chunks,
+                         w.table.total + 1, *job, n);
+    } else {
+      hipLaunchKernelGGL(mark_count_kernel<false>, dim3((unsigned)mark_blocks, (unsigned)gg.ks[0]),
+                         dim3(256), 0, s, indices, n_in, gg, w.table.bits, w.chunk_count,
+                         w.n_chunks, w.table.total + 1, CombineJob{}, (int64_t)0);
+    }
+  }
   SSC_LAUNCH_CHECK("mark_count");
   if (pair_num == nullptr) return bit_table_scan(w.table, s, mirror, ticket);
   hipLaunchKernelGGL(blocksum_scan_chunks_kernel, dim3((unsigned)(w.table.n_scan_blocks + gg.K)),
@@ -1142,11 +1190,11 @@ int ssc::rulebook_begin_impl(const int32_t *indices, int64_t n_in, const ssc_geo
   if (rc != SSC_OK) return rc;
   SSC_CHECK(pair_num != nullptr, SSC_EINVAL, "pair_num is NULL");
   SSC_CHECK(n_in == 0 || pairs != nullptr, SSC_EINVAL, "pairs is NULL");
-  // the filters' job rides on the dilation path's first launch; any other path runs it first
-  DenseIn job_dense;
-  const bool job_rides = job != nullptr && n_in > 0 && dense_marking_applies(gg, n_in, &job_dense);
-  if (job != nullptr && !job_rides && (rc = launch_combine_pack(*job, s)) != SSC_OK) return rc;
-  if (!job_rides) job = nullptr;
+  // the filters' job rides on the first launch that looks at the rows; without rows it runs alone
+  if (job != nullptr && n_in == 0) {
+    if ((rc = launch_combine_pack(*job, s)) != SSC_OK) return rc;
+    job = nullptr;
+  }
   if (n_in == 0) return fill_i32(pair_num, gg.K, 0, s);
   SSC_CHECK(out_indices == nullptr || out_capacity >= rulebook_out_bound(gg, n_in), SSC_EINVAL,
             "out_indices holds %lld rows, fewer than the bound of %lld", (long long)out_capacity,
@@ -1279,8 +1327,9 @@ int ssc_unique_count(const int32_t *coords, int64_t n, const int32_t dims[4], vo
   Carver c(workspace);
   BitTable t = bit_table_carve(c, cells);
   if ((rc = bit_table_clear(t, s)) != SSC_OK) return rc;
-  hipLaunchKernelGGL(mark_rows_kernel, dim3((unsigned)ceil_div(n, 256)), dim3(256), 0, s, coords,
-                     n, dims[0], dims[1], dims[2], dims[3], t.bits, t.total + 1, 0);
+  hipLaunchKernelGGL(mark_rows_kernel<false>, dim3((unsigned)ceil_div(n, 256)), dim3(256), 0, s,
+                     coords, n, dims[0], dims[1], dims[2], dims[3], t.bits, t.total + 1, 0,
+                     CombineJob{}, (int64_t)0);
   SSC_LAUNCH_CHECK("mark_rows");
   if ((rc = bit_table_scan(t, s)) != SSC_OK) return rc;
   int32_t host[2];
@@ -1330,8 +1379,9 @@ int ssc_unique_build(const int32_t *coords, int64_t n, const int32_t dims[4], vo
   // total[0]: the number of distinct rows (written by the scan); total[1]: flags;
   // total[2]: the largest count; all cleared with the table
   if ((rc = bit_table_clear(t, s)) != SSC_OK) return rc;
-  hipLaunchKernelGGL(mark_rows_kernel, dim3((unsigned)ceil_div(n, 256)), dim3(256), 0, s, coords,
-                     n, dims[0], dims[1], dims[2], dims[3], t.bits, t.total + 1, 0);
+  hipLaunchKernelGGL(mark_rows_kernel<false>, dim3((unsigned)ceil_div(n, 256)), dim3(256), 0, s,
+                     coords, n, dims[0], dims[1], dims[2], dims[3], t.bits, t.total + 1, 0,
+                     CombineJob{}, (int64_t)0);
   SSC_LAUNCH_CHECK("mark_rows");
   if ((rc = bit_table_scan(t, s)) != SSC_OK) return rc;
   if ((rc = fill_i32(counts, n, 0, s)) != SSC_OK) return rc;

@@ -1056,6 +1056,38 @@ def test_conv_backward_matches_oracle(case, oracle, device):
     assert rel_l2(e_w.cpu().numpy().reshape(K, cout, cin), oref_w) < REL_L2
 
 
+@pytest.mark.parametrize("geom", [dict(stride=1, padding=1), dict(stride=2, padding=1),
+                                  dict(stride=1, padding=1, subm=True),
+                                  dict(stride=1, padding=1, subm=True, indice_key="k")])
+def test_training_layer_filters_ride_on_the_rulebook(geom, device):
+    """A training-mode Convolution leaves the synthesis and packing of its filters to the first
+    launch of the rulebook it queues (to a launch of its own when the rulebook is already
+    there: the second call under an indice_key).  Same filters, same plan as the
+    evaluation-mode layer, which synthesises them by itself: bit-equal rows, and the dense
+    kernel the autograd graph holds equals the module's."""
+    from ss_conv.convolution import Convolution
+    from ss_conv.sp_ops.tensor import SparseTensor
+    torch.manual_seed(4)
+    rs_in, rs_out = [(3, 0), (2, 1), (1, 2)], [(4, 0), (3, 1), (1, 2)]
+    rng = np.random.default_rng(6)
+    grid, n = 11, 400
+    idx = torch.from_numpy(random_voxels(rng, 2, grid, n)).to(device)
+    conv = Convolution(rs_in, rs_out, 3, **geom).to(device)
+    feats = torch.from_numpy(rng.normal(size=(n, conv.in_channels)).astype(np.float32)).to(device)
+    make = lambda: SparseTensor(feats, idx, [grid] * 3, 2)  # noqa: E731
+    with torch.no_grad():
+        conv.eval()
+        want = conv(make())
+        conv.train()
+        x = make()
+        got = conv(x)
+        again = conv(x) if geom.get("indice_key") else None  # the rulebook is cached now
+    assert torch.equal(got.indices, want.indices)
+    assert torch.equal(got.features, want.features)
+    if again is not None:
+        assert torch.equal(again.features, want.features)
+
+
 def test_layer_gradients(oracle, device):
     """loss.backward() through Convolution: gradient of the input features against the
     restated backward, gradient of kernel.weight against torch autograd through an
