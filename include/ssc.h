@@ -406,6 +406,13 @@ int ssc_profile_conv(int32_t enable);
  *      launch that counts the ranges' row blocks.  Results are bit-identical (only where in
  *      its buffers a range's part of the schedule lies differs). */
 int ssc_conv_tuning(int32_t flags);
+/* Tell the library that the caller queues index work (ssc_rulebook_*, ssc_conv_plan_build) on
+ * a stream of its own, where it runs while a convolution on another stream holds every CU
+ * with nearly all of its LDS (the convolution kernel leaves about 4 KB of a CU's 160 KB):
+ * with on != 0 those calls pick kernels that fit into what is left (smaller blocks, two
+ * launches for the schedule instead of one) and so run beside the convolution instead of
+ * behind it.  Results are the same bit for bit.  Returns the previous setting (default 0). */
+int ssc_index_beside_conv(int32_t on);
 int ssc_profile_conv_read(float *ms /* host */, int32_t capacity, int32_t *count /* host */);
 
 /* ------------------------------------------------------------------------

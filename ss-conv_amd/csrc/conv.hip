@@ -547,7 +547,11 @@ __device__ __forceinline__ TileOf tile_by_index(int t, const int *row_s, const i
   return o;
 }
 
-constexpr int kSegChunk = 2048;  // pairs of one offset to a block
+// CHUNK: pairs of one offset to a block (kSegChunk; kSegChunkSmall for blocks that are to fit
+// beside a workgroup of the convolution, which leaves a few KB of a CU's LDS).  Dynamic LDS:
+// 2 (n_rng + 1) ints.
+constexpr int kSegChunk = 2048, kSegChunkSmall = 256;
+template <int CHUNK>
 __global__ void __launch_bounds__(256)
     pair_tile_segments_kernel(int32_t *__restrict__ flag, const int32_t *__restrict__ pairs,
                               int64_t pair_stride, int plane_s,
@@ -557,15 +561,15 @@ __global__ void __launch_bounds__(256)
                               int32_t *__restrict__ n_tiles_dev, int32_t *__restrict__ spill_end,
                               int32_t *__restrict__ tile_slot0, int32_t *__restrict__ segs,
                               int32_t *__restrict__ spill) {
-  __shared__ int row_s[kMaxRanges + 1];
-  __shared__ int tile_s[kMaxRanges + 1];
+  extern __shared__ int range_dyn[];
+  int *const row_s = range_dyn, *const tile_s = range_dyn + n_rng + 1;
   __shared__ int wave_sum[4];
   // (the loads of the run's rows are issued first: they are not needed before the tables
   // of the ranges stand)
   const int k = blockIdx.y;
-  const int64_t j0 = (int64_t)blockIdx.x * kSegChunk;
+  const int64_t j0 = (int64_t)blockIdx.x * CHUNK;
   const int32_t *s = pairs + ((int64_t)k * 2 + plane_s) * pair_stride;
-  constexpr int kPer = (kSegChunk + 15 + 255) / 256;
+  constexpr int kPer = (CHUNK + 15 + 255) / 256;
   int held[kPer];
 #pragma unroll
   for (int u = 0; u < kPer; ++u) {
@@ -628,7 +632,7 @@ __global__ void __launch_bounds__(256)
   }
   // the block's run of the offset's pairs: their rows (and those of the 15 pairs behind
   // them, for the spill) in LDS
-  __shared__ int rows[kSegChunk + 16];
+  __shared__ int rows[CHUNK + 16];
   if (n == 0) {  // no pair: every tile's segment is empty
     if (blockIdx.x == 0)
       for (int t = threadIdx.x; t <= n_tiles; t += 256) {
@@ -638,11 +642,11 @@ __global__ void __launch_bounds__(256)
     return;
   }
   if (j0 >= n) return;
-  const int cnt = n - j0 < kSegChunk ? (int)(n - j0) : kSegChunk;
+  const int cnt = n - j0 < CHUNK ? (int)(n - j0) : CHUNK;
 #pragma unroll
   for (int u = 0; u < kPer; ++u) {
     const int i = threadIdx.x + 256 * u;
-    if (i < kSegChunk + 15) rows[i] = j0 + i < n ? held[u] : 0x7FFFFFFF;
+    if (i < CHUNK + 15) rows[i] = j0 + i < n ? held[u] : 0x7FFFFFFF;
   }
   const int r_prev = r_before;
   __syncthreads();
@@ -1096,9 +1100,13 @@ static size_t conv_lds_bytes(int T, int acc_cols) {
   return ((size_t)(T + 1) * (acc_cols + 4) + 2 * (size_t)kStage * kAStride) * 4;
 }
 
+constexpr size_t kLdsLeft = 4096 + 256;
 static int pick_tile(int acc_cols) {
   // One workgroup per CU: (almost) all of the 160 KB of LDS goes to the accumulators.
-  size_t budget = 160 * 1024 - conv_lds_bytes(0, acc_cols) - 512;
+  // (kLdsLeft bytes stay free: the kernels of the index work -- rulebooks and plans of other
+  // layers, queued on a stream of their own -- are built to fit there, beside this kernel's
+  // workgroups)
+  size_t budget = 160 * 1024 - conv_lds_bytes(0, acc_cols) - kLdsLeft;
   int t = (int)(budget / ((size_t)(acc_cols + 4) * 4));
   t = t / 8 * 8;
   if (t < kMinTile) t = kMinTile;
@@ -1128,6 +1136,9 @@ constexpr int64_t kPairGroups = 250;
 static bool g_conv_pair = true, g_conv_pair_always = false;
 static int64_t g_conv_rebalance_stages = kRebalanceStages;
 static bool g_conv_fuse_fill = true;  // range_sched_kernel<true> instead of sched_fill_kernel
+// Index work (rulebooks, plans) is queued on a stream of its own and runs while a convolution
+// holds every CU with nearly all of its LDS: kernels are picked that need little LDS.
+static bool g_index_beside_conv = false;
 static bool g_conv_rebalance = true;  // long kernels: a second work split from the first one's counts
 static bool g_conv_round8 = false;    // ranges per column block: a multiple of 8 only
 static bool g_conv_small = true;      // layers of at most 8 input channels: conv_small_kernel
@@ -1447,6 +1458,12 @@ int ssc_conv_tuning(int32_t flags) {
   return SSC_OK;
 }
 
+int ssc_index_beside_conv(int32_t on) {
+  const int old = g_index_beside_conv ? 1 : 0;
+  g_index_beside_conv = on != 0;
+  return old;
+}
+
 int ssc_profile_conv_read(float *ms, int32_t capacity, int32_t *count) {
   SSC_CHECK(ms != nullptr && count != nullptr, SSC_EINVAL, "NULL pointer argument");
   int n = g_profile_count < kProfileRing ? g_profile_count : kProfileRing;
@@ -1500,7 +1517,10 @@ static int conv_plan_build(const ConvPlan &p, const ConvWs &w, const int32_t *pa
                           p.ncb * p.nch * frag_bytes, w.sched_in, w.sched_out, w.grp_meta};
   // One range to a workgroup and a single work split: the launch that counts a range's row
   // blocks goes on to fill its schedule (no sched_fill_kernel).
-  const bool fuse_fill = g_conv_fuse_fill && !p.rebalance && p.n_rng == p.n_wg;
+  // (not for index work queued beside a running convolution: there two small kernels that
+  // fit next to its workgroups beat one that has to wait for a CU of its own)
+  const bool fuse_fill =
+      g_conv_fuse_fill && !g_index_beside_conv && !p.rebalance && p.n_rng == p.n_wg;
   auto range_sched = [&]() -> int {
     hipLaunchKernelGGL(fuse_fill ? range_sched_kernel<true> : range_sched_kernel<false>,
                        dim3((unsigned)p.n_rng), dim3(kRangeSchedThreads), 0, s, w.segs, w.spill,
@@ -1515,8 +1535,11 @@ static int conv_plan_build(const ConvPlan &p, const ConvWs &w, const int32_t *pa
     // the schedule.  For pairs in order, plans without a second split and nothing to pack.
     SSC_CHECK(in_order && !p.rebalance && pack == nullptr, SSC_ERUNTIME,
               "a seeded plan needs pairs in order and a single work split");
-    hipLaunchKernelGGL(pair_tile_segments_kernel,
-                       dim3((unsigned)ceil_div(pair_stride, kSegChunk), (unsigned)K), dim3(256), 0, s,
+    const int chunk = g_index_beside_conv ? kSegChunkSmall : kSegChunk;
+    hipLaunchKernelGGL(g_index_beside_conv ? pair_tile_segments_kernel<kSegChunkSmall>
+                                           : pair_tile_segments_kernel<kSegChunk>,
+                       dim3((unsigned)ceil_div(pair_stride, chunk), (unsigned)K), dim3(256),
+                       2 * ((size_t)p.n_rng + 1) * sizeof(int), s,
                        w.flag, pairs, pair_stride, plane_s, pair_num, K, w.range_row0, p.n_rng,
                        p.tile_rows, p.T, (int)n_out, w.wg_tile, w.tile_row0, w.n_tiles_dev,
                        w.spill_end, w.tile_slot0, w.segs, w.spill);

@@ -432,19 +432,9 @@ __global__ void __launch_bounds__(kScanThreads)
   const uint32_t zw_n = (uint32_t)g.os[2] >> 5;  // words per output row
   const int64_t xstep = (int64_t)d.U[1] * d.Wz;
   int v = 0;
-  __shared__ int word_rows[SEED ? kScanBlockWords : 1], word_pairs[SEED ? kScanBlockWords : 1];
-#pragma unroll 2
-  for (int it = 0; it < kScanItems; ++it) {
-    const int64_t w = (int64_t)blockIdx.x * kScanBlockWords + it * kScanThreads + threadIdx.x;
-    if (w >= n_words) {
-      if constexpr (SEED) {
-        word_rows[it * kScanThreads + threadIdx.x] = 0;
-        word_pairs[it * kScanThreads + threadIdx.x] = 0;
-        continue;
-      } else {
-        break;
-      }
-    }
+  // One word of the output table: the OR of its taps' shifted input words; *landing = the
+  // pairs that land on its cells.
+  auto word_of = [&](int64_t w, int *landing) -> uint32_t {
     uint32_t t = (uint32_t)w;  // (fewer than 2^26 words)
     const int zw = (int)(t % zw_n);
     t /= zw_n;
@@ -454,7 +444,7 @@ __global__ void __launch_bounds__(kScanThreads)
     const int b = (int)(t / (uint32_t)g.os[0]);
     const uint32_t *rowp = in_bits + (((int64_t)b * d.U[0] + x) * d.U[1] + y) * d.Wz + zw;
     uint32_t out = 0u;
-    int landing = 0;
+    int land = 0;
 #pragma unroll
     for (int kx = 0; kx < ksx; ++kx) {
 #pragma unroll
@@ -463,44 +453,44 @@ __global__ void __launch_bounds__(kScanThreads)
         // (with ksz > 1, Wz > os[2] / 32: word zw + 1 exists)
         const uint32_t lo = p[0], hi = ksz > 1 ? p[1] : 0u;
         uint32_t acc = lo;
-        if constexpr (SEED) landing += __popc(lo);
+        if constexpr (SEED) land += __popc(lo);
 #pragma unroll
         for (int kz = 1; kz < ksz; ++kz) {
           const uint32_t shifted = (lo >> kz) | (hi << (32 - kz));
           acc |= shifted;
-          if constexpr (SEED) landing += __popc(shifted);
+          if constexpr (SEED) land += __popc(shifted);
         }
         out |= acc;
       }
     }
-    bits[w] = out;
-    v += __popc(out);
-    if constexpr (SEED) {
-      word_rows[it * kScanThreads + threadIdx.x] = __popc(out);
-      word_pairs[it * kScanThreads + threadIdx.x] = landing;
-    }
-  }
+    *landing = land;
+    return out;
+  };
   if constexpr (SEED) {
-    // prefixes over the block's words in their order: every thread takes kScanItems
-    // consecutive words
+    // Every thread takes kScanItems consecutive words, so that the prefixes over the block's
+    // words in their order need the threads' sums and nothing else: no table of the words'
+    // counts in LDS (a block then fits beside a workgroup that has taken nearly all of a
+    // CU's LDS, as the convolution's do).
     __shared__ int lds[kScanThreads / 64 + 1];
-    __syncthreads();
-    const int first = threadIdx.x * kScanItems;
+    const int64_t w0 = (int64_t)blockIdx.x * kScanBlockWords + (int64_t)threadIdx.x * kScanItems;
     int cr[kScanItems], cp[kScanItems], sr = 0, sp = 0;
+    uint32_t ob[kScanItems];
 #pragma unroll
     for (int i = 0; i < kScanItems; ++i) {
-      cr[i] = word_rows[first + i];
-      cp[i] = word_pairs[first + i];
+      ob[i] = 0u;
+      cp[i] = 0;
+      if (w0 + i < n_words) ob[i] = word_of(w0 + i, &cp[i]);
+      cr[i] = __popc(ob[i]);
       sr += cr[i];
       sp += cp[i];
     }
     int tot_r, tot_p;
     int er = block_exclusive_scan(sr, lds, &tot_r);
     int ep = block_exclusive_scan(sp, lds, &tot_p);
-    const int64_t w0 = (int64_t)blockIdx.x * kScanBlockWords + first;
 #pragma unroll
     for (int i = 0; i < kScanItems; ++i) {
       if (w0 + i < n_words) {
+        bits[w0 + i] = ob[i];
         seed_rows[w0 + i] = er;
         seed_pairs[w0 + i] = ep;
       }
@@ -512,6 +502,15 @@ __global__ void __launch_bounds__(kScanThreads)
       pairsum[blockIdx.x] = tot_p;
     }
     return;
+  }
+#pragma unroll 2
+  for (int it = 0; it < kScanItems; ++it) {
+    const int64_t w = (int64_t)blockIdx.x * kScanBlockWords + it * kScanThreads + threadIdx.x;
+    if (w >= n_words) break;
+    int unused;
+    const uint32_t out = word_of(w, &unused);
+    bits[w] = out;
+    v += __popc(out);
   }
 #pragma unroll
   for (int s = 32; s >= 1; s >>= 1) v += __shfl_xor(v, s, 64);
@@ -533,6 +532,16 @@ __global__ void __launch_bounds__(kScanThreads)
 // its first row being the rows below c.  Every such block first adds up the block sums of
 // rows and pairs in LDS (at most kSeedMaxBlocks of each); a range's lanes then find the scan
 // block by bisection there and the cell inside it by three rounds of 16 probes.
+// Dynamic LDS of the kernels that add up the scan blocks' sums: a long long and an int for
+// every scan block and one more (as much as the table needs, not room for kSeedMaxBlocks: a
+// block of theirs then fits beside a workgroup that has taken nearly all of a CU's LDS).
+static inline size_t seed_lds_bytes(int64_t n_scan_blocks) {
+  return (size_t)(n_scan_blocks + 1) * 12 + 8;
+}
+__device__ __forceinline__ int *seed_lds_rows(long long *dyn, int64_t n_scan_blocks) {
+  return reinterpret_cast<int *>(dyn + n_scan_blocks + 1);
+}
+
 // The range boundaries of a SplitRequest (see prefix_split_kernel), for the group of 16
 // ranges `group` (kScanThreads threads).
 __device__ __forceinline__ void split_ranges_block(int group, int64_t n_words,
@@ -541,9 +550,10 @@ __device__ __forceinline__ void split_ranges_block(int group, int64_t n_words,
                                                    const int32_t *__restrict__ pairsum,
                                                    const int32_t *__restrict__ seed_rows,
                                                    const int32_t *__restrict__ seed_pairs,
-                                                   const SplitRequest &rq) {
-  __shared__ int rows_base[kSeedMaxBlocks + 1];
-  __shared__ long long pairs_base[kSeedMaxBlocks + 1];
+                                                   const SplitRequest &rq, long long *pairs_base,
+                                                   int *rows_base) {
+  // (pairs_base, rows_base: n_scan_blocks + 1 entries each in the kernel's dynamic LDS, see
+  // seed_lds_bytes)
   __shared__ int lds[kScanThreads / 64 + 1];
   __shared__ long long wave_p[kScanThreads / 64];
   const int nb = (int)n_scan_blocks;  // <= kSeedMaxBlocks
@@ -658,8 +668,9 @@ __global__ void __launch_bounds__(kScanThreads)
                       (int64_t)blockIdx.x == n_scan_blocks - 1, ticket);
     return;
   }
+  extern __shared__ long long seed_dyn[];
   split_ranges_block((int)(blockIdx.x - n_scan_blocks), n_words, n_scan_blocks, blocksum, pairsum,
-                     seed_rows, seed_pairs, rq);
+                     seed_rows, seed_pairs, rq, seed_dyn, seed_lds_rows(seed_dyn, n_scan_blocks));
 }
 
 // What the two-level form of write_pairs_kernel needs besides the table: the scan blocks'
@@ -686,7 +697,8 @@ __global__ void __launch_bounds__(256)
                        int64_t n_words, int32_t *__restrict__ out_indices,
                        uint32_t *__restrict__ clean, int64_t clean_words, int row_blocks,
                        TwoLevel two) {
-  __shared__ int base_s[TWO ? kSeedMaxBlocks + 1 : 1];
+  extern __shared__ long long seed_dyn[];  // (TWO: seed_lds_bytes; otherwise none)
+  int *const base_s = TWO ? seed_lds_rows(seed_dyn, two.n_scan_blocks) : nullptr;
   if constexpr (TWO) {
     static_assert(kScanThreads == 256, "one block size for the table's scan and this kernel");
     if (blockIdx.y == 0) {
@@ -694,7 +706,7 @@ __global__ void __launch_bounds__(256)
       // totals): the range boundaries of the convolution's plan, and one block for the totals
       if ((int)blockIdx.x < two.split_blocks) {
         split_ranges_block((int)blockIdx.x, n_words, two.n_scan_blocks, two.blocksum, two.pairsum,
-                           two.seed_rows, two.seed_pairs, two.split);
+                           two.seed_rows, two.seed_pairs, two.split, seed_dyn, base_s);
         return;
       }
       if ((int)blockIdx.x != two.split_blocks) return;
@@ -987,7 +999,7 @@ static int rulebook_mark_and_scan(const int32_t *indices, int64_t n_in, const Ge
     // the scan's second pass, and beside it the range boundaries of the convolution's plan
     const int64_t split_blocks = ceil_div(split->n_rng, kScanThreads / 16);
     hipLaunchKernelGGL(prefix_split_kernel, dim3((unsigned)(word_blocks + split_blocks)),
-                       dim3(kScanThreads), 0, s, w.table.bits, w.table.n_words, word_blocks,
+                       dim3(kScanThreads), seed_lds_bytes(word_blocks), s, w.table.bits, w.table.n_words, word_blocks,
                        w.table.blocksum, w.table.prefix, w.table.total, mirror, w.pairsum,
                        w.seed_rows, w.seed_pairs, *split, ticket);
     SSC_LAUNCH_CHECK("prefix_split");
@@ -1068,7 +1080,7 @@ static int rulebook_pairs(const int32_t *indices, int64_t n_in, const Geom &gg,
     auto kernel = ks == 3 ? write_pairs_kernel<3, true> : ks == 5 ? write_pairs_kernel<5, true>
                   : ks == 2 ? write_pairs_kernel<2, true> : write_pairs_kernel<0, true>;
     hipLaunchKernelGGL(kernel, dim3(chunk_blocks, (unsigned)(gg.ks[0] + row_blocks + 1)),
-                       dim3(256), 0, s, indices, n_in, gg, w.table.bits, w.table.prefix, w.rank2row,
+                       dim3(256), seed_lds_bytes(two->n_scan_blocks), s, indices, n_in, gg, w.table.bits, w.table.prefix, w.rank2row,
                        w.chunk_count, w.n_chunks, pair_num, pairs, w.table.n_words, out_indices,
                        clean, clean_words, (int)row_blocks, *two);
     SSC_LAUNCH_CHECK("write_pairs");

@@ -95,6 +95,7 @@ _SIGNATURES = {
     "ssc_voxel_reduce_bwd_f32": (ctypes.c_int, [_vp, _vp, _vp, _i32, _i32, _i32, _i32, _i64, _vp]),
     "ssc_three_interp_bwd_f32": (ctypes.c_int, [_i32, _i32, _i32, _vp, _vp, _vp, _vp, _vp]),
     "ssc_profile_conv": (ctypes.c_int, [_i32]),
+    "ssc_index_beside_conv": (ctypes.c_int, [_i32]),
     "ssc_conv_tuning": (ctypes.c_int, [_i32]),
     "ssc_profile_conv_read": (ctypes.c_int, [ctypes.POINTER(ctypes.c_float), _i32,
                                              ctypes.POINTER(_i32)]),
@@ -224,6 +225,7 @@ def _geometry(batch_size, out_shape, ksize, stride, padding, dilation, subm, tra
 # buffer of more than 4 MiB is copied out of it, so that no rulebook keeps more than twice
 # its rows alive).
 _ROWS_AHEAD_BYTES = 256 << 20
+_ROWS_KEEP_BYTES = 64 << 20  # unused rows of such a buffer beyond which the result is copied out of it
 # largest plan / plan scratch allocated for the bound on the number of outputs, before the
 # real number has arrived (the scratch is dropped when the plan is built; the plan, kept
 # with the rulebook, is at most this much larger than one sized for the real number)
@@ -323,11 +325,107 @@ def _clean_table(nbytes, dev, stream):
     return held
 
 
+# ---- index work on a stream of its own -------------------------------------------------------
+# A rulebook and the plan of the convolution over it depend on the voxel indices only, not on
+# the features: they are queued on a second stream of the device (default priority), and the
+# kernel that needs them waits for that stream's event on the caller's stream.  A layer's
+# rulebook reads the output indices of the rulebook before it -- written on the same second
+# stream -- so in a stack of layers the index work of layer i + 1 runs while the convolution
+# of layer i still does, and the host, which waits for that stream only, is not held up by
+# the convolutions either.  Tensors written there are allocated there (the caching allocator
+# reuses a block in the order of the stream it was allocated on) and recorded on the caller's
+# stream before they are handed out.
+_index_streams = {}  # device index -> _IndexStream
+_index_overlap = os.environ.get("SSC_INDEX_STREAM", "1") != "0"
+_lib.ssc_index_beside_conv(1 if _index_overlap else 0)
+_INDEX_STREAM_MIN_WORK = 1 << 18  # rows * offsets below which the second stream is not worth its events
+_INDEX_AHEAD_EVERY = 8  # the host runs at most about three times this many rulebooks ahead
+
+
+class _IndexStream(object):
+    __slots__ = ("stream", "handle", "calls", "events")
+
+    def __init__(self, dev):
+        self.stream = torch.cuda.Stream(device=dev)
+        self.handle = self.stream.cuda_stream
+        self.calls = 0
+        self.events = []
+
+
+def index_stream(enable):
+    """Switch the second stream for index work on or off (on by default; the environment
+    variable SSC_INDEX_STREAM=0 switches it off from the start).  Returns the old setting."""
+    global _index_overlap
+    old = _index_overlap
+    _index_overlap = bool(enable)
+    _lib.ssc_index_beside_conv(1 if _index_overlap else 0)
+    return old
+
+
+def _index_stream_for(dev, main, work):
+    """The device's stream for index work, or None when this call's stays on `main`."""
+    if not _index_overlap or work < _INDEX_STREAM_MIN_WORK or torch.cuda.is_current_stream_capturing():
+        return None
+    st = _index_streams.get(dev.index)
+    if st is None:
+        st = _index_streams[dev.index] = _IndexStream(dev)
+    if st.handle == main.cuda_stream:
+        return None
+    # The host waits for the second stream only, so nothing else stops it from queueing
+    # convolutions faster than they run: every few rulebooks an event goes behind the
+    # caller's stream, and the host waits for the one before the one before last.
+    st.calls += 1
+    if st.calls % _INDEX_AHEAD_EVERY == 0:
+        ev = torch.cuda.Event()
+        ev.record(main)
+        st.events.append(ev)
+        if len(st.events) > 2:
+            st.events.pop(0).synchronize()
+    return st
+
+
+def _side_ready(t):
+    """Whether the second stream may read `t` without waiting for the caller's stream: it
+    wrote the tensor itself, or has waited for it once and the tensor has not changed since."""
+    return getattr(t, "_ssc_side_ready", None) == t._version
+
+
+def _mark_side_ready(t):
+    t._ssc_side_ready = t._version
+
+
+class _NoStream(object):
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *a):
+        return False
+
+
+_no_stream = _NoStream()
+
+
+def _index_ctx(r):
+    """Allocate and queue torch work on the rulebook's stream."""
+    return torch.cuda.stream(r.side.stream) if r.side is not None else _no_stream
+
+
+def _index_done(r, *tensors):
+    """The caller's stream goes on behind what the second stream has queued so far, and the
+    tensors it will use there are recorded on it."""
+    if r.side is None:
+        return
+    r.main.wait_stream(r.side.stream)
+    for t in tensors:
+        if t is not None:
+            t.record_stream(r.main)
+
+
 class _PendingRulebook(object):
     """A rulebook between ssc_rulebook_begin and ssc_rulebook_finish: everything whose size
     does not depend on the number of outputs is queued, the host has not waited yet."""
     __slots__ = ("indices", "n", "geometry", "ws", "pairs", "num", "out_buf", "subm", "stream",
-                 "bound", "plan", "scratch", "conv")
+                 "bound", "plan", "scratch", "conv", "main", "side")
 
 
 def _rulebook_begin(indices, batch_size, out_spatial_shape, kernel_size, stride, padding, dilation,
@@ -357,10 +455,28 @@ def _rulebook_begin(indices, batch_size, out_spatial_shape, kernel_size, stride,
         nbytes = 256
     r = _PendingRulebook()
     r.indices, r.n, r.geometry, r.subm = indices, n, g, bool(subm)
+    r.main = torch.cuda.current_stream(dev)
+    r.side = _index_stream_for(dev, r.main, n * K)
+    if r.side is not None:
+        if not _side_ready(indices):
+            r.side.stream.wait_stream(r.main)
+            _mark_side_ready(indices)
+        indices.record_stream(r.side.stream)
+        r.stream = r.side.handle
+    else:
+        r.stream = r.main.cuda_stream
+    with _index_ctx(r):
+        _rulebook_queue(r, gref, K, nbytes, conv)
+    return r
+
+
+def _rulebook_queue(r, gref, K, nbytes, conv):
+    """Allocate a rulebook's buffers and queue it (on the current torch stream = r.stream)."""
+    indices, n, subm = r.indices, r.n, r.subm
+    dev = indices.device
     r.ws = _workspace(nbytes, dev)
     r.pairs = torch.empty((K, 2, n), dtype=torch.int32, device=dev)
     r.num = torch.empty((K,), dtype=torch.int32, device=dev)
-    r.stream = _stream(indices)
     # Marking, ranking and the pair lists are queued; the host then waits for the number of
     # outputs only, while the pair lists are still being written.  When room for any
     # possible number of output rows is cheap (n * K rows at most), the rows are written in
@@ -384,7 +500,10 @@ def _rulebook_begin(indices, batch_size, out_spatial_shape, kernel_size, stride,
             r.conv = (int(c_in), int(c_out), int(eb))
     clean_bytes = _lib.ssc_rulebook_clean_table_bytes(gref, n)
     clean = _clean_table(clean_bytes, dev, r.stream) if clean_bytes > 0 else None
-    job = _take_combine(K, r.conv[0], r.conv[1], dev, r.stream) if r.conv is not None else None
+    # (a layer's filter job rides on the rulebook's first launch when that runs on the
+    # caller's stream; on the second stream it would have to wait for the weights there)
+    job = _take_combine(K, r.conv[0], r.conv[1], dev, r.stream) \
+        if r.conv is not None and r.side is None else None
     try:
         if r.conv is not None:
             _check(_lib.ssc_rulebook_conv_begin(
@@ -402,7 +521,6 @@ def _rulebook_begin(indices, batch_size, out_spatial_shape, kernel_size, stride,
     except Exception:
         _clean_tables.pop((dev.index, r.stream), None)  # it may not be clean any more
         raise
-    return r
 
 
 def _rulebook_conv_wait(r):
@@ -427,32 +545,39 @@ def _rulebook_wait(r):
 
 
 def _rulebook_result(r, n_out, in_order):
-    """[outids, pairs, num] of a rulebook whose number of outputs has arrived."""
-    if r.subm:
-        outids = r.indices
-    elif r.out_buf is not None:
-        outids = r.out_buf[:n_out]
-        if r.out_buf.size(0) > 2 * max(n_out, 1) and r.out_buf.numel() * 4 > (4 << 20):
-            outids = outids.clone()  # do not keep a large, mostly unused buffer alive
-    else:
-        # a geometry may leave no output at all (every candidate clipped): the library still
-        # wants a valid pointer, so at least one row is allocated and the result is a slice
-        out_buf = torch.empty((max(n_out, 1), 4), dtype=torch.int32, device=r.pairs.device)
-        outids = out_buf[:n_out]
-        _check(_lib.ssc_rulebook_rows(ctypes.byref(r.geometry), r.n, r.ws.data_ptr(), r.ws.numel(),
-                                      out_buf.data_ptr(), r.stream))
+    """[outids, pairs, num] of a rulebook whose number of outputs has arrived.  What is left
+    to queue goes on the rulebook's stream: callers follow with _index_done."""
+    with _index_ctx(r):
+        if r.subm:
+            outids = r.indices
+        elif r.out_buf is not None:
+            outids = r.out_buf[:n_out]
+            if (r.out_buf.size(0) - n_out) * 16 > _ROWS_KEEP_BYTES:
+                outids = outids.clone()  # do not keep a large, mostly unused buffer alive
+        else:
+            # a geometry may leave no output at all (every candidate clipped): the library
+            # still wants a valid pointer, so at least one row is allocated and the result is
+            # a slice
+            out_buf = torch.empty((max(n_out, 1), 4), dtype=torch.int32, device=r.pairs.device)
+            outids = out_buf[:n_out]
+            _check(_lib.ssc_rulebook_rows(ctypes.byref(r.geometry), r.n, r.ws.data_ptr(),
+                                          r.ws.numel(), out_buf.data_ptr(), r.stream))
     # Pairs of an offset always ascend in the input rows, and in the output rows too when
     # the input rows came in key order: the convolution may then skip its order check
     # (the first flag serves a call that accumulates into output rows, the second one
     # with `inverse`, which accumulates into input rows).
     r.pairs._ssc_meta = RulebookMeta(r.pairs._version, (in_order, True), pairs_ref=r.pairs)
+    if r.side is not None:
+        _mark_side_ready(outids)
     return [outids, r.pairs, r.num]
 
 
 def _rulebook_finish(r):
     """Wait for the number of outputs; returns [outids, pairs, num]."""
     n_out, in_order = _rulebook_wait(r)
-    return _rulebook_result(r, n_out, in_order)
+    res = _rulebook_result(r, n_out, in_order)
+    _index_done(r, *res)
+    return res
 
 
 def get_indice_pairs_3d(indices, batch_size, out_spatial_shape, spatial_shape, kernel_size, stride,
@@ -639,7 +764,7 @@ def rulebook_conv(features, filters, indices, batch_size, out_spatial_shape, ker
     for d in filters.shape[:-2]:
         kvol *= d
     dev = features.device
-    s = r.stream
+    s = r.main.cuda_stream  # the convolution's stream (the rulebook may be on another)
     bad = None
     if kvol != K:
         bad = "filters have %d offsets but the rulebook has %d" % (kvol, K)
@@ -647,17 +772,30 @@ def rulebook_conv(features, filters, indices, batch_size, out_spatial_shape, ker
         bad = "features and indices must have the same number of rows"
     if bad is not None:
         _rulebook_wait(r)  # (the rulebook is queued: end it before raising)
+        _index_done(r)
         raise RuntimeError(bad)
     packed = _packed_filters(owner, filters, (fs_k, fs_ci, fs_co), K, c_in, c_out, s)
     if r.conv is None:
         n_out, in_order = _rulebook_wait(r)
         outids, pairs, num = _rulebook_result(r, n_out, in_order)
-        plan = _plan_of(pairs._ssc_meta, pairs, num, K, c_in, c_out, eb, n_in, n_out, False, dev, s)
+        with _index_ctx(r):
+            plan = _plan_of(pairs._ssc_meta, pairs, num, K, c_in, c_out, eb, n_in, n_out, False,
+                            dev, r.stream)
+        _index_done(r, outids, pairs, num, plan)
         out = _run_planned(features, n_in, c_in, packed, plan, n_in, K, c_out, n_out, s, epilogue)
         return out, outids, pairs, num
     n_out, in_order = _rulebook_conv_wait(r)
-    out = _run_planned(features, n_in, c_in, packed, r.plan, n_in, K, c_out, n_out, s, epilogue)
-    outids, pairs, num = _rulebook_result(r, n_out, in_order)
+    if r.side is not None:
+        # (the convolution's stream waits for the other one once, behind everything that was
+        # queued there)
+        outids, pairs, num = _rulebook_result(r, n_out, in_order)
+        _index_done(r, outids, pairs, num, r.plan)
+        out = _run_planned(features, n_in, c_in, packed, r.plan, n_in, K, c_out, n_out, s,
+                           epilogue)
+    else:
+        out = _run_planned(features, n_in, c_in, packed, r.plan, n_in, K, c_out, n_out, s,
+                           epilogue)
+        outids, pairs, num = _rulebook_result(r, n_out, in_order)
     if n_out > 0:
         pairs._ssc_meta.put_plan((False, c_in, c_out, eb, n_in, n_out), r.plan)
     return out, outids, pairs, num

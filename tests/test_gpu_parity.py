@@ -1088,6 +1088,65 @@ def test_training_layer_filters_ride_on_the_rulebook(geom, device):
         assert torch.equal(again.features, want.features)
 
 
+def test_index_work_on_a_second_stream(device):
+    """Rulebooks and plans are queued on a second stream of the device, the convolutions and
+    pools on the caller's: a stack of layers over changing inputs, calls following each other
+    without a wait, gives bit for bit what it gives with everything on one stream.  Inputs are
+    made by torch kernels on the caller's stream right before each pass (the second stream
+    has to wait for them), the rulebooks under an indice_key are reused by later layers, and
+    tensors are dropped while kernels that read them may still be queued (the allocator must
+    not hand their memory out early)."""
+    from ss_conv import _ext
+    from ss_conv.convolution import Convolution
+    from ss_conv.pool import MaxPool
+    from ss_conv.sp_ops.tensor import SparseTensor
+    torch.manual_seed(12)
+    rs0, rs1, rs2 = [(4, 0), (2, 1)], [(6, 0), (3, 1), (1, 2)], [(8, 0), (4, 1)]
+    layers = [Convolution(rs0, rs1, 3, stride=1, padding=1).to(device),
+              Convolution(rs1, rs1, 3, stride=1, padding=1, subm=True, indice_key="a").to(device),
+              Convolution(rs1, rs2, 3, stride=2, padding=1).to(device),
+              Convolution(rs2, rs2, 3, stride=1, padding=1, subm=True, indice_key="b").to(device),
+              Convolution(rs2, rs2, 3, stride=1, padding=1, subm=True, indice_key="b").to(device)]
+    pool = MaxPool(2, 2)
+    for m in layers:
+        m.train()
+    grid, n = 20, 3000
+    rng = np.random.default_rng(21)
+    clouds = [torch.from_numpy(random_voxels(rng, 2, grid, n)).to(device) for _ in range(4)]
+
+    def run_all():
+        outs = []
+        for it in range(8):
+            idx = clouds[it % 4].clone()  # a new tensor, written on the caller's stream
+            feats = torch.randn(n, layers[0].in_channels, device=device,
+                                generator=torch.Generator(device).manual_seed(it))
+            x = SparseTensor(feats * 1.5, idx, [grid] * 3, 2)
+            for m in layers:
+                x = m(x)
+            y = pool(x)
+            outs.append((x.features, x.indices, y.features, y.indices))
+            del x, y, idx, feats
+        torch.cuda.synchronize()
+        return outs
+
+    keep = _ext._INDEX_STREAM_MIN_WORK
+    was = _ext.index_stream(True)
+    try:
+        _ext._INDEX_STREAM_MIN_WORK = 0  # (these layers are far below the size it is meant for)
+        with torch.no_grad():
+            two = run_all()
+            again = run_all()
+            _ext.index_stream(False)
+            one = run_all()
+    finally:
+        _ext._INDEX_STREAM_MIN_WORK = keep
+        _ext.index_stream(was)
+    for a, b, c in zip(two, again, one):
+        for ta, tb, tc in zip(a, b, c):
+            assert torch.equal(ta, tc)
+            assert torch.equal(tb, tc)
+
+
 def test_layer_gradients(oracle, device):
     """loss.backward() through Convolution: gradient of the input features against the
     restated backward, gradient of kernel.weight against torch autograd through an
