@@ -338,7 +338,7 @@ def _clean_table(nbytes, dev, stream):
 _index_streams = {}  # device index -> _IndexStream
 _index_overlap = os.environ.get("SSC_INDEX_STREAM", "1") != "0"
 _lib.ssc_index_beside_conv(1 if _index_overlap else 0)
-_INDEX_STREAM_MIN_WORK = 1 << 18  # rows * offsets below which the second stream is not worth its events
+_INDEX_STREAM_MIN_WORK = 1 << 20  # rows * offsets below which the second stream is not worth its events
 _INDEX_AHEAD_EVERY = 8  # the host runs at most about three times this many rulebooks ahead
 
 
