@@ -32,11 +32,11 @@ CLOCK_WARMUP_MS = 100
 # launches) for every workload this script offers, from rocprofv3 --pmc FETCH_SIZE /
 # WRITE_SIZE runs scaled by a copy kernel of known size (the summaries
 # profiles/conv_fwd_<workload>_hbm_traffic.md give commands and counter values).
-MEASURED_TRAFFIC_BYTES = {"cfg1": 3416327, "cfg2": 345545343, "cfg3": 229620287, "cfg5": 68985036509}
+MEASURED_TRAFFIC_BYTES = {"cfg1": 4065508, "cfg2": 346615562, "cfg3": 227771580, "cfg5": 69608189217}
 # the same for all kernels of one rulebook call and of one Point2Voxel call
 # (profiles/rulebook_hbm_traffic.md, profiles/point_voxel_hbm_traffic.md)
-RULEBOOK_TRAFFIC_BYTES = {"cfg2": 37000000, "cfg5": 188500000}
-P2V_TRAFFIC_BYTES = {"cfg2": 62500000, "cfg5": 116400000}
+RULEBOOK_TRAFFIC_BYTES = {"cfg2": 37500000, "cfg3": 28600000, "cfg5": 188400000}
+P2V_TRAFFIC_BYTES = {"cfg2": 60500000, "cfg5": 119300000}
 HBM_PEAK_GBS = 8000.0
 
 
@@ -74,6 +74,10 @@ def parse_args():
                     help="also time layers whose last group of 16 output columns would be alone "
                          "in its block of 64 (64->72, 128->136, 152->8, 128->16), with the "
                          "kernel's one-column-group form and without (table on stderr)")
+    ap.add_argument("--one-stream", action="store_true",
+                    help="queue the index work (rulebooks, plans) on the convolutions' stream "
+                         "instead of a second one: a step's kernels one after the other (for "
+                         "kernel traces and counters)")
     ap.add_argument("--breakdown", action="store_true",
                     help="also print per-phase timings to stderr")
     return ap.parse_args()
@@ -156,20 +160,30 @@ def rulebook_figure(torch, _ext, dev, indices, batch, shape, k, stride, pad, wor
     finally:
         _ext.index_stream(was)
     gpu_us = max(span - empty, 1e-3)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(20):
-        get_indice_pairs(indices, batch, shape, k, stride, pad)
-    torch.cuda.synchronize()
-    call_us = (time.perf_counter() - t0) * 1e6 / 20
+    def calls():
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(20):
+            get_indice_pairs(indices, batch, shape, k, stride, pad)
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) * 1e6 / 20
+    call_us_default = calls()
+    was = _ext.index_stream(False)
+    try:
+        call_us = calls()
+    finally:
+        _ext.index_stream(was)
     gbs = nbytes / gpu_us / 1e3
     return {"workload": workload, "bytes": nbytes, "gpu_us": gpu_us, "gbs": gbs,
             "frac_hbm": gbs / HBM_PEAK_GBS, "traffic": RULEBOOK_TRAFFIC_BYTES.get(workload),
-            "call_us": call_us, "event_pair_us": empty,
+            "call_us": call_us, "call_us_second_stream": call_us_default, "event_pair_us": empty,
             "n_in": n_in, "n_out": n_out, "pairs": P,
             "how": "HIP events around the kernels of one ssc_rulebook_begin on their stream, "
                    "median of 20, an empty event pair subtracted; call_us: get_indice_pairs "
-                   "with its host wait, mean of 20"}
+                   "with its host wait, mean of 20, the kernels on the caller's stream; "
+                   "call_us_second_stream: the same call as the library queues it by default, "
+                   "on a second stream (built to run beside a convolution, not to return "
+                   "sooner)"}
 
 
 def point2voxel_figure(torch, _ext, synth, dev, workload, seed, channels=64):
@@ -700,6 +714,8 @@ def main():
         print("bench.py needs a GPU", file=sys.stderr)
         sys.exit(2)
     dev = torch.device("cuda:0")
+    if args.one_stream:
+        _ext.index_stream(False)
     if args.workload == "cfg4":
         if args.steps == 100 and args.warmup == 20:  # the defaults are sized for a 0.4 ms step
             args.steps, args.warmup = 20, 5
