@@ -1101,12 +1101,14 @@ static size_t conv_lds_bytes(int T, int acc_cols) {
 }
 
 constexpr size_t kLdsLeft = 4096 + 256;
-static int pick_tile(int acc_cols) {
+static int pick_tile(int acc_cols, bool leave_room) {
   // One workgroup per CU: (almost) all of the 160 KB of LDS goes to the accumulators.
   // (kLdsLeft bytes stay free: the kernels of the index work -- rulebooks and plans of other
   // layers, queued on a stream of their own -- are built to fit there, beside this kernel's
   // workgroups)
-  size_t budget = 160 * 1024 - conv_lds_bytes(0, acc_cols) - kLdsLeft;
+  // (... unless the kernel will run for long: the index work of a neighbouring layer is
+  // small change next to it, and the rows of the window are worth more)
+  size_t budget = 160 * 1024 - conv_lds_bytes(0, acc_cols) - (leave_room ? kLdsLeft : 512);
   int t = (int)(budget / ((size_t)(acc_cols + 4) * 4));
   t = t / 8 * 8;
   if (t < kMinTile) t = kMinTile;
@@ -1185,8 +1187,6 @@ static ConvPlan make_plan(int64_t n_in, int64_t n_out, int K, int c_in, int c_ou
   // kernel needs four chunks for it, one for each wave's turn at the fifth group's sums)
   p.five = g_conv_five && elem_bytes == 4 && p.ncb % p.ncw == 1 && p.ncb > p.ncw && p.nch >= 4;
   p.acc_cols = p.five ? 16 * p.ncw + 16 : 16 * p.ncw;
-  p.T = pick_tile(p.acc_cols);
-  p.tile_rows = p.T - (p.five ? kSpillRowsFive : kSpillRows);
   // the gather can be a range-checked buffer load when rows are multiples of four
   // channels and byte offsets into the features (plus the padding marker) fit 32 bits
   p.gather = 0;
@@ -1220,6 +1220,13 @@ static ConvPlan make_plan(int64_t n_in, int64_t n_out, int K, int c_in, int c_ou
   // more small launches (30 us; the split evens out 3-15 % of the kernel's time, more with
   // more ranges): 1500 stages per workgroup or more.
   p.rebalance = g_conv_rebalance && est_stages >= g_conv_rebalance_stages;
+  // The accumulator window: all of the LDS for kernels that run long (a second split, or
+  // ranges worth pairing), a few KB less for the others (see pick_tile); sizing calls
+  // (N_in unknown) count with the smaller window, which has more tiles.
+  const bool long_kernel =
+      n_in > 0 && (est_stages >= kRebalanceStages || est_groups >= kPairGroups);
+  p.T = pick_tile(p.acc_cols, !long_kernel);
+  p.tile_rows = p.T - (p.five ? kSpillRowsFive : kSpillRows);
   // Two ranges to a workgroup, paired by what they came to (range_assign_kernel): one more
   // small launch and one more range end per workgroup, whose last row blocks cannot be
   // filled from a next tile (K / 8 groups), against the 5-10 % by which single ranges

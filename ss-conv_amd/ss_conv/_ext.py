@@ -337,7 +337,17 @@ def _clean_table(nbytes, dev, stream):
 # stream before they are handed out.
 _index_streams = {}  # device index -> _IndexStream
 _index_overlap = os.environ.get("SSC_INDEX_STREAM", "1") != "0"
-_lib.ssc_index_beside_conv(1 if _index_overlap else 0)
+_beside_now = [False]  # what the library was last told (ssc_index_beside_conv)
+
+
+def _beside(on):
+    """Tell the library whether the index work queued next runs on the second stream (it
+    then picks kernels that fit beside a convolution)."""
+    if _beside_now[0] != on:
+        _lib.ssc_index_beside_conv(1 if on else 0)
+        _beside_now[0] = on
+
+
 _INDEX_STREAM_MIN_WORK = 1 << 20  # rows * offsets below which the second stream is not worth its events
 _INDEX_AHEAD_EVERY = 8  # the host runs at most about three times this many rulebooks ahead
 
@@ -358,7 +368,6 @@ def index_stream(enable):
     global _index_overlap
     old = _index_overlap
     _index_overlap = bool(enable)
-    _lib.ssc_index_beside_conv(1 if _index_overlap else 0)
     return old
 
 
@@ -457,6 +466,7 @@ def _rulebook_begin(indices, batch_size, out_spatial_shape, kernel_size, stride,
     r.indices, r.n, r.geometry, r.subm = indices, n, g, bool(subm)
     r.main = torch.cuda.current_stream(dev)
     r.side = _index_stream_for(dev, r.main, n * K)
+    _beside(r.side is not None)
     if r.side is not None:
         if not _side_ready(indices):
             r.side.stream.wait_stream(r.main)
@@ -648,13 +658,15 @@ def prepack_filters(filters, c_in, c_out):
     return _packed_filters(owner, filters, (fs_k, fs_ci, fs_co), K, c_in, c_out, _stream(filters))
 
 
-def _plan_of(meta, pairs, num, K, c_in, c_out, elem_bytes, n_in, n_out, inverse, dev, stream):
+def _plan_of(meta, pairs, num, K, c_in, c_out, elem_bytes, n_in, n_out, inverse, dev, stream,
+             beside=False):
     """The plan of a (direction, channel counts, element type, row counts) combination over
     a rulebook: built on first use, kept with the rulebook afterwards."""
     stride = pairs.size(2)
     key = (bool(inverse), c_in, c_out, elem_bytes, n_in, n_out)
     plan = meta.get_plan(key)
     if plan is None:
+        _beside(beside)
         plan = _workspace(_lib.ssc_conv_plan_bytes(n_out, K, c_in, c_out, stride), dev)
         scratch = _workspace(_lib.ssc_conv_plan_scratch_bytes(n_out, K, c_in, c_out, stride), dev)
         flags = 2 if meta.canonical[1 if inverse else 0] else 0
@@ -780,7 +792,7 @@ def rulebook_conv(features, filters, indices, batch_size, out_spatial_shape, ker
         outids, pairs, num = _rulebook_result(r, n_out, in_order)
         with _index_ctx(r):
             plan = _plan_of(pairs._ssc_meta, pairs, num, K, c_in, c_out, eb, n_in, n_out, False,
-                            dev, r.stream)
+                            dev, r.stream, beside=r.side is not None)
         _index_done(r, outids, pairs, num, plan)
         out = _run_planned(features, n_in, c_in, packed, plan, n_in, K, c_out, n_out, s, epilogue)
         return out, outids, pairs, num
@@ -813,6 +825,7 @@ def _conv_any(features, owner, filters, fs, indice_pairs, pairs, num, K, c_in, c
     out = torch.empty((n_out, c_out), dtype=features.dtype, device=features.device)
     ws = _workspace(_lib.ssc_conv_workspace_bytes(n_out, K, c_in, c_out, pairs.size(2)),
                     features.device)
+    _beside(False)
     _check(_ENTRIES[features.dtype][0](
         _ptr(features), features.size(0), c_in, _ptr(filters), fs[0], fs[1], fs[2], c_out,
         _ptr(pairs), pairs.size(2), num.data_ptr(), K, int(bool(inverse)), int(bool(subm)),
