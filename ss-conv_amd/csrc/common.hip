@@ -209,6 +209,6 @@ int read_back(void *dst_host, const void *src_dev, size_t bytes, hipStream_t s) 
 }  // namespace ssc
 
 extern "C" {
-int ssc_version(void) { return 100; }
+int ssc_version(void) { return 103; }
 const char *ssc_last_error(void) { return ssc::g_error; }
 }

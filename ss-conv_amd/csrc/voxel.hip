@@ -1264,7 +1264,7 @@ __global__ void __launch_bounds__(256)
   next[pos] = atomicExch(&head[rk], (int32_t)pos);
 }
 
-// The feature reduction of the one-call chain.  Sixteen lanes per voxel (four voxels to a
+// The feature reduction of the one-call chain.  Eight lanes per voxel (eight voxels to a
 // wave): the lanes walk the voxel's chain together (count, smallest and largest row, the
 // first four rows), then
 //   mode 1 / 2: the features of the first / last row,
