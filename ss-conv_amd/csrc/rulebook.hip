@@ -525,13 +525,6 @@ __global__ void __launch_bounds__(kScanThreads)
   }
 }
 
-// The second pass of the table's scan (popc_prefix_block) and, in the blocks after the
-// table's, the placing of the range boundaries of a SplitRequest: 16 ranges to a block, 16
-// lanes to a range.  Range w begins at the first cell c (a word of the table) with
-//   work(c) = pairs below c * tile_rows + rows below c * tile_cost  >=  w / n_rng of the total,
-// its first row being the rows below c.  Every such block first adds up the block sums of
-// rows and pairs in LDS (at most kSeedMaxBlocks of each); a range's lanes then find the scan
-// block by bisection there and the cell inside it by three rounds of 16 probes.
 // Dynamic LDS of the kernels that add up the scan blocks' sums: a long long and an int for
 // every scan block and one more (as much as the table needs, not room for kSeedMaxBlocks: a
 // block of theirs then fits beside a workgroup that has taken nearly all of a CU's LDS).
@@ -542,8 +535,13 @@ __device__ __forceinline__ int *seed_lds_rows(long long *dyn, int64_t n_scan_blo
   return reinterpret_cast<int *>(dyn + n_scan_blocks + 1);
 }
 
-// The range boundaries of a SplitRequest (see prefix_split_kernel), for the group of 16
-// ranges `group` (kScanThreads threads).
+// The placing of the range boundaries of a SplitRequest, for the group of 16 ranges `group`
+// (kScanThreads threads: 16 lanes to a range).  Range w begins at the first cell c (a word
+// of the table) with
+//   work(c) = pairs below c * tile_rows + rows below c * tile_cost  >=  w / n_rng of the total,
+// its first row being the rows below c.  The block first adds up the block sums of rows and
+// pairs in LDS (at most kSeedMaxBlocks of each); a range's lanes then find the scan block by
+// bisection there and the cell inside it by three rounds of 16 probes.
 __device__ __forceinline__ void split_ranges_block(int group, int64_t n_words,
                                                    int64_t n_scan_blocks,
                                                    const int32_t *__restrict__ blocksum,
@@ -656,6 +654,11 @@ __device__ __forceinline__ void split_ranges_block(int group, int64_t n_words,
     }
   }
 }
+
+// The second pass of the table's scan (popc_prefix_block) and, in the blocks after the
+// table's, the range boundaries of a SplitRequest (split_ranges_block): for rulebooks whose
+// pair launch does not take the prefixes in two levels (no room for the output rows at
+// hand).  Dynamic LDS: seed_lds_bytes.
 __global__ void __launch_bounds__(kScanThreads)
     prefix_split_kernel(const uint32_t *__restrict__ bits, int64_t n_words, int64_t n_scan_blocks,
                         const int32_t *__restrict__ blocksum, int32_t *__restrict__ prefix,
