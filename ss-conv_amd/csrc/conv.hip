@@ -547,11 +547,13 @@ __device__ __forceinline__ TileOf tile_by_index(int t, const int *row_s, const i
   return o;
 }
 
-// CHUNK: pairs of one offset to a block (kSegChunk; kSegChunkSmall for blocks that are to fit
-// beside a workgroup of the convolution, which leaves a few KB of a CU's LDS).  Dynamic LDS:
-// 2 (n_rng + 1) ints.
-constexpr int kSegChunk = 2048, kSegChunkSmall = 256;
-template <int CHUNK>
+// CHUNK: pairs of one offset to a block.  LDSROWS: the run's rows are staged in LDS and a
+// thread bisects them for its tile; otherwise they stay in memory and sixteen lanes find a
+// tile's first pair in three rounds of sixteen probes (next to nothing in LDS: such a block
+// fits beside a workgroup of the convolution, which leaves a few KB of a CU's LDS).
+// Dynamic LDS: 2 (n_rng + 1) ints.
+constexpr int kSegChunk = 2048;
+template <int CHUNK, bool LDSROWS>
 __global__ void __launch_bounds__(256)
     pair_tile_segments_kernel(int32_t *__restrict__ flag, const int32_t *__restrict__ pairs,
                               int64_t pair_stride, int plane_s,
@@ -569,12 +571,14 @@ __global__ void __launch_bounds__(256)
   const int k = blockIdx.y;
   const int64_t j0 = (int64_t)blockIdx.x * CHUNK;
   const int32_t *s = pairs + ((int64_t)k * 2 + plane_s) * pair_stride;
-  constexpr int kPer = (CHUNK + 15 + 255) / 256;
+  constexpr int kPer = LDSROWS ? (CHUNK + 15 + 255) / 256 : 1;
   int held[kPer];
+  if constexpr (LDSROWS) {
 #pragma unroll
-  for (int u = 0; u < kPer; ++u) {
-    const int64_t idx = j0 + threadIdx.x + 256 * u;
-    held[u] = idx < pair_stride ? s[idx] : 0x7FFFFFFF;
+    for (int u = 0; u < kPer; ++u) {
+      const int64_t idx = j0 + threadIdx.x + 256 * u;
+      held[u] = idx < pair_stride ? s[idx] : 0x7FFFFFFF;
+    }
   }
   const int r_before = j0 > 0 && j0 <= pair_stride ? s[j0 - 1] : -1;
   const int n = pair_num[k];
@@ -632,7 +636,7 @@ __global__ void __launch_bounds__(256)
   }
   // the block's run of the offset's pairs: their rows (and those of the 15 pairs behind
   // them, for the spill) in LDS
-  __shared__ int rows[CHUNK + 16];
+  __shared__ int rows[LDSROWS ? CHUNK + 16 : 1];
   if (n == 0) {  // no pair: every tile's segment is empty
     if (blockIdx.x == 0)
       for (int t = threadIdx.x; t <= n_tiles; t += 256) {
@@ -643,29 +647,59 @@ __global__ void __launch_bounds__(256)
   }
   if (j0 >= n) return;
   const int cnt = n - j0 < CHUNK ? (int)(n - j0) : CHUNK;
-#pragma unroll
-  for (int u = 0; u < kPer; ++u) {
-    const int i = threadIdx.x + 256 * u;
-    if (i < CHUNK + 15) rows[i] = j0 + i < n ? held[u] : 0x7FFFFFFF;
-  }
   const int r_prev = r_before;
-  __syncthreads();
-  // the tiles whose first row lies in (row of the pair before the run, row of its last pair]
-  const int t_lo = j0 > 0 ? tile_of_row(r_prev, row_s, tile_s, n_rng, T, window).t + 1 : 0;
-  const int t_hi = tile_of_row(rows[cnt - 1], row_s, tile_s, n_rng, T, window).t;
-  for (int t = t_lo + threadIdx.x; t <= t_hi; t += 256) {
-    const TileOf tl = tile_by_index(t, row_s, tile_s, n_rng, T, window);
-    int lo = 0, hi = cnt - 1;  // the first pair of the run at or beyond the tile's first row
-    while (lo < hi) {
-      const int mid = (lo + hi) >> 1;
-      if (rows[mid] < tl.row0) lo = mid + 1;
-      else hi = mid;
-    }
-    int beyond = 0;
+  int t_hi;
+  if constexpr (LDSROWS) {
 #pragma unroll
-    for (int q = 0; q < 15; ++q) beyond += rows[lo + q] < tl.spill ? 1 : 0;  // rows ascend
-    segs[(int64_t)t * K + k] = (int32_t)(j0 + lo);
-    spill[(int64_t)t * K + k] = (int32_t)(j0 + lo + beyond);
+    for (int u = 0; u < kPer; ++u) {
+      const int i = threadIdx.x + 256 * u;
+      if (i < CHUNK + 15) rows[i] = j0 + i < n ? held[u] : 0x7FFFFFFF;
+    }
+    __syncthreads();
+    // the tiles whose first row lies in (row of the pair before the run, row of its last pair]
+    const int t_lo = j0 > 0 ? tile_of_row(r_prev, row_s, tile_s, n_rng, T, window).t + 1 : 0;
+    t_hi = tile_of_row(rows[cnt - 1], row_s, tile_s, n_rng, T, window).t;
+    for (int t = t_lo + threadIdx.x; t <= t_hi; t += 256) {
+      const TileOf tl = tile_by_index(t, row_s, tile_s, n_rng, T, window);
+      int lo = 0, hi = cnt - 1;  // the first pair of the run at or beyond the tile's first row
+      while (lo < hi) {
+        const int mid = (lo + hi) >> 1;
+        if (rows[mid] < tl.row0) lo = mid + 1;
+        else hi = mid;
+      }
+      int beyond = 0;
+#pragma unroll
+      for (int q = 0; q < 15; ++q) beyond += rows[lo + q] < tl.spill ? 1 : 0;  // rows ascend
+      segs[(int64_t)t * K + k] = (int32_t)(j0 + lo);
+      spill[(int64_t)t * K + k] = (int32_t)(j0 + lo + beyond);
+    }
+  } else {
+    auto row_at = [&](int i) -> int { return j0 + i < n ? s[j0 + i] : 0x7FFFFFFF; };
+    const int t_lo = j0 > 0 ? tile_of_row(r_prev, row_s, tile_s, n_rng, T, window).t + 1 : 0;
+    t_hi = tile_of_row(row_at(cnt - 1), row_s, tile_s, n_rng, T, window).t;
+    const int sub = threadIdx.x & 15, shift = threadIdx.x & 48;
+    for (int t = t_lo + (threadIdx.x >> 4); t <= t_hi; t += 16) {
+      const TileOf tl = tile_by_index(t, row_s, tile_s, n_rng, T, window);
+      // the first pair of the run at or beyond the tile's first row lies in [lo, lo + len),
+      // and the last pair of that stretch is at or beyond it (rows ascend; the run's last
+      // pair is, t being at most the tile of its row)
+      int lo = 0, len = cnt;
+      while (len > 1) {
+        const int step = (len + 15) >> 4;
+        const int upto = (sub + 1) * step < len ? (sub + 1) * step : len;
+        const bool at = row_at(lo + upto - 1) >= tl.row0;
+        const unsigned m = (unsigned)(__ballot(at) >> shift) & 0xFFFFu;
+        const int f = __ffs(m) - 1;  // (the stretch's last probe is set)
+        lo += f * step;
+        len = (f + 1) * step < len ? step : len - f * step;
+      }
+      const bool in_spill = sub < 15 && row_at(lo + sub) < tl.spill;
+      const int beyond = __popc((unsigned)(__ballot(in_spill) >> shift) & 0xFFFFu);
+      if (sub == 0) {
+        segs[(int64_t)t * K + k] = (int32_t)(j0 + lo);
+        spill[(int64_t)t * K + k] = (int32_t)(j0 + lo + beyond);
+      }
+    }
   }
   if (j0 + cnt == n)  // the offset's last run: tiles beyond its last pair
     for (int t = t_hi + 1 + threadIdx.x; t <= n_tiles; t += 256) {
@@ -1542,10 +1576,9 @@ static int conv_plan_build(const ConvPlan &p, const ConvWs &w, const int32_t *pa
     // the schedule.  For pairs in order, plans without a second split and nothing to pack.
     SSC_CHECK(in_order && !p.rebalance && pack == nullptr, SSC_ERUNTIME,
               "a seeded plan needs pairs in order and a single work split");
-    const int chunk = g_index_beside_conv ? kSegChunkSmall : kSegChunk;
-    hipLaunchKernelGGL(g_index_beside_conv ? pair_tile_segments_kernel<kSegChunkSmall>
-                                           : pair_tile_segments_kernel<kSegChunk>,
-                       dim3((unsigned)ceil_div(pair_stride, chunk), (unsigned)K), dim3(256),
+    auto segments_kernel = g_index_beside_conv ? pair_tile_segments_kernel<kSegChunk, false>
+                                               : pair_tile_segments_kernel<kSegChunk, true>;
+    hipLaunchKernelGGL(segments_kernel, dim3((unsigned)ceil_div(pair_stride, kSegChunk), (unsigned)K), dim3(256),
                        2 * ((size_t)p.n_rng + 1) * sizeof(int), s,
                        w.flag, pairs, pair_stride, plane_s, pair_num, K, w.range_row0, p.n_rng,
                        p.tile_rows, p.T, (int)n_out, w.wg_tile, w.tile_row0, w.n_tiles_dev,
