@@ -148,11 +148,25 @@ struct Best3 {
   }
 };
 
+// weight[j] = r_j / ((r_0 + r_1) + r_2) with r_j = 1 / (sqrt(d_j) + 1e-8)
+// (ss_conv/sp_ops/voxelize.py:156-159), for kernels that know a query's three distances.
+__device__ __forceinline__ void nn_weights(float d1, float d2, float d3, float *__restrict__ w) {
+  const float r0 = 1.0f / (sqrtf(d1) + 1e-8f);
+  const float r1 = 1.0f / (sqrtf(d2) + 1e-8f);
+  const float r2 = 1.0f / (sqrtf(d3) + 1e-8f);
+  const float norm = (r0 + r1) + r2;
+  w[0] = r0 / norm;
+  w[1] = r1 / norm;
+  w[2] = r2 / norm;
+}
+
+// weight (optional): the interpolation weights of the queries written, beside dist2 / idx.
 __global__ void __launch_bounds__(kNnTile)
     three_nn_kernel(int n, int m, const float *__restrict__ unknown,
                     const float *__restrict__ known, const float *__restrict__ tile_range,
                     float *__restrict__ dist2, int32_t *__restrict__ idx,
-                    const int32_t *__restrict__ only_if, int only_above) {
+                    const int32_t *__restrict__ only_if, int only_above,
+                    float *__restrict__ weight = nullptr) {
   // (a condition on a device-side counter, the same for every thread of the grid)
   if (only_if && only_if[0] <= only_above) return;
   __shared__ float4v tile[kNnTile];
@@ -226,6 +240,7 @@ __global__ void __launch_bounds__(kNnTile)
   if (q < n && sub == 0) {
     dist2[q * 3] = best.b1; dist2[q * 3 + 1] = best.b2; dist2[q * 3 + 2] = best.b3;
     idx[q * 3] = best.i1; idx[q * 3 + 1] = best.i2; idx[q * 3 + 2] = best.i3;
+    if (weight != nullptr) nn_weights(best.b1, best.b2, best.b3, weight + q * 3);
   }
 }
 
@@ -361,14 +376,26 @@ struct GridNn {
   float origin[3], unit[3];
 };
 
+// The grid as Voxel2Point states it: centre of a voxel = (index * unit - half_extent) +
+// half_unit, the three roundings of the reference's expression (voxelize.py:139).
+struct V2pGrid {
+  float unit[3], half_extent[3], half_unit[3];
+};
+__device__ __forceinline__ float v2p_centre(int index, const V2pGrid &g, int a) {
+  return ((float)index * g.unit[a] - g.half_extent[a]) + g.half_unit[a];
+}
+
 __device__ __forceinline__ bool nng_inside(const int4 &r, const GridNn &g) {
   return r.x >= 0 && r.x < g.batch && r.y >= 0 && r.y < g.dim[0] && r.z >= 0 && r.z < g.dim[1] &&
          r.w >= 0 && r.w < g.dim[2];
 }
 
+// disorder[0] is set when the rows do not come in strictly ascending key order (for rows in
+// that order the rank of a cell is its row).
 __global__ void __launch_bounds__(256)
     nng_mark_kernel(const int32_t *__restrict__ coords, int m, GridNn g,
-                    uint32_t *__restrict__ bits, int32_t *__restrict__ unsettled) {
+                    uint32_t *__restrict__ bits, int32_t *__restrict__ unsettled,
+                    int32_t *__restrict__ disorder) {
   const int j = blockIdx.x * blockDim.x + threadIdx.x;
   if (j >= m) return;
   const int4 r = reinterpret_cast<const int4 *>(coords)[j];
@@ -377,13 +404,21 @@ __global__ void __launch_bounds__(256)
     return;
   }
   const uint32_t key = (uint32_t)(((r.x * g.dim[0] + r.y) * g.dim[1] + r.z) * g.dim[2] + r.w);
+  if (j + 1 < m) {
+    const int4 q = reinterpret_cast<const int4 *>(coords)[j + 1];
+    const uint32_t next =
+        (uint32_t)(((q.x * g.dim[0] + q.y) * g.dim[1] + q.z) * g.dim[2] + q.w);
+    if (!nng_inside(q, g) || next <= key) atomicOr(disorder, 1);
+  }
   atomicOr(&bits[key >> 5], 1u << (key & 31u));
 }
 
 __global__ void __launch_bounds__(256)
     nng_rank2row_kernel(const int32_t *__restrict__ coords, int m, GridNn g,
                         const uint32_t *__restrict__ bits, const int32_t *__restrict__ prefix,
-                        int32_t *__restrict__ rank2row) {
+                        int32_t *__restrict__ rank2row, const int32_t *__restrict__ skip_if_ordered) {
+  // (rows in key order, and a search that ranks its candidates by cell: nobody reads the map)
+  if (skip_if_ordered != nullptr && skip_if_ordered[0] == 0) return;
   const int j = blockIdx.x * blockDim.x + threadIdx.x;
   if (j >= m) return;
   const int4 r = reinterpret_cast<const int4 *>(coords)[j];
@@ -413,13 +448,23 @@ __device__ __forceinline__ void nng_merge_lanes(Best3 &b) {
   }
 }
 
+// CENTRES (Voxel2Point's own call): the known points are the centres of the voxels as vg
+// states them, so a candidate's distance comes from its cell -- the same three roundings that
+// wrote known[] -- and nothing is loaded for it but the table word that holds its bit; with
+// the voxel rows in key order (disorder[0] == 0) a cell's rank is its row, so candidates are
+// ranked by (distance, cell) and only a query's three winners are looked up; otherwise a
+// candidate's row comes from rank2row as in the other form.  weight (optional) as for
+// three_nn_kernel.
+template <bool CENTRES>
 __global__ void __launch_bounds__(256)
     three_nn_grid_kernel(int n, int m, const float *__restrict__ unknown,
                          const float *__restrict__ known, GridNn g,
                          const uint32_t *__restrict__ bits, const int32_t *__restrict__ prefix,
                          const int32_t *__restrict__ rank2row, float *__restrict__ dist2,
                          int32_t *__restrict__ idx, int32_t *__restrict__ counter,
-                         int32_t *__restrict__ list) {
+                         int32_t *__restrict__ list, V2pGrid vg,
+                         const int32_t *__restrict__ disorder, float *__restrict__ weight) {
+  const bool by_cell = CENTRES && disorder[0] == 0;
   const int q = blockIdx.x * (256 / kGridNnLanes) + threadIdx.x / kGridNnLanes;
   const int sub = threadIdx.x % kGridNnLanes;
   const bool live = q < n;  // dead groups run along (the shuffles want every lane)
@@ -442,6 +487,7 @@ __global__ void __launch_bounds__(256)
     c[a] = v < 0 ? 0 : (v >= g.dim[a] ? g.dim[a] - 1 : v);
   }
   for (int r = 0; r <= kGridNnMaxShell; ++r) {
+    if (__all(settled)) break;  // (every query of the wave: the same decision in all lanes)
     Best3 cur = none;
     if (!settled) {
       const int x0 = max(c[0] - r, 0), x1 = min(c[0] + r, g.dim[0] - 1);
@@ -453,23 +499,52 @@ __global__ void __launch_bounds__(256)
         // cells of the shell only: in the interior of the box just the two end cells in z
         const bool face = abs(x - c[0]) == r || abs(y - c[1]) == r;
         const uint32_t base = (uint32_t)(((b * g.dim[0] + x) * g.dim[1] + y) * g.dim[2]);
-        uint32_t wi = 0xFFFFFFFFu, w = 0u;
-        int wp = 0;
-        for (int z = z0; z <= z1; ++z) {
-          if (!face && abs(z - c[2]) != r) continue;
-          const uint32_t key = base + (uint32_t)z;
-          if ((key >> 5) != wi) {
-            wi = key >> 5;
-            w = bits[wi];
-            wp = w ? prefix[wi] : 0;
+        float xx = 0.f, yy = 0.f;  // (CENTRES) the column's share of the distance
+        if constexpr (CENTRES) {
+          const float dx = u.y - v2p_centre(x, vg, 0), dy = u.z - v2p_centre(y, vg, 1);
+          xx = dx * dx;
+          yy = dy * dy;
+        }
+        // The column's cells of the shell are neighbours along z: one or two words of the
+        // table (2 r + 1 <= 9 cells).  Their set bits are taken from a mask, so the empty
+        // cells -- nearly all of them -- cost nothing.  (Loading the words of four of a
+        // lane's columns before looking at any: 43 against 46 us on clouds of 65 k points,
+        // 63 against 57 on 131 k.)
+        const uint32_t k0 = base + (uint32_t)z0, k1 = base + (uint32_t)z1;
+        for (uint32_t wi = k0 >> 5; wi <= (k1 >> 5); ++wi) {
+          const uint32_t w = bits[wi];
+          if (w == 0u) continue;
+          const uint32_t lo_bit = wi == (k0 >> 5) ? (k0 & 31u) : 0u;
+          const uint32_t hi_bit = wi == (k1 >> 5) ? (k1 & 31u) : 31u;
+          uint32_t cand = w & (0xFFFFFFFFu << lo_bit) & (0xFFFFFFFFu >> (31u - hi_bit));
+          if (!face) {  // only the column's two end cells belong to the shell
+            uint32_t ends = 0u;
+            const int za = c[2] - r, zb = c[2] + r;
+            if (za >= z0 && ((base + (uint32_t)za) >> 5) == wi)
+              ends |= 1u << ((base + (uint32_t)za) & 31u);
+            if (zb <= z1 && ((base + (uint32_t)zb) >> 5) == wi)
+              ends |= 1u << ((base + (uint32_t)zb) & 31u);
+            cand &= ends;
           }
-          if ((w >> (key & 31u)) & 1u) {
-            const int row = rank2row[wp + __popc(w & ((1u << (key & 31u)) - 1u))];
-            const float4v p = reinterpret_cast<const float4v *>(known)[row];
-            if (p.x == u.x) {
-              const float dx = u.y - p.y, dy = u.z - p.z, dz = u.w - p.w;
-              const float xx = dx * dx, yy = dy * dy, zz = dz * dz;
-              cur.insert((xx + yy) + zz, row);
+          if (cand == 0u) continue;
+          const int wp = by_cell ? 0 : prefix[wi];
+          while (cand != 0u) {
+            const uint32_t bit = (uint32_t)__ffs((int)cand) - 1u;
+            cand &= cand - 1u;
+            const uint32_t key = (wi << 5) + bit;
+            if constexpr (CENTRES) {
+              const float dz = u.w - v2p_centre((int)(key - base), vg, 2);
+              const float zz = dz * dz;
+              const int id = by_cell ? (int)key : rank2row[wp + __popc(w & ((1u << bit) - 1u))];
+              cur.insert((xx + yy) + zz, id);
+            } else {
+              const int row = rank2row[wp + __popc(w & ((1u << bit) - 1u))];
+              const float4v p = reinterpret_cast<const float4v *>(known)[row];
+              if (p.x == u.x) {
+                const float dx = u.y - p.y, dy = u.z - p.z, dz = u.w - p.w;
+                const float x2 = dx * dx, y2 = dy * dy, z2 = dz * dz;
+                cur.insert((x2 + y2) + z2, row);
+              }
             }
           }
         }
@@ -500,8 +575,14 @@ __global__ void __launch_bounds__(256)
     }
   }
   if (live && sub == 0) {
+    if (by_cell) {  // the winners' rows: the ranks of their cells
+      if (acc.b1 < INFINITY) acc.i1 = bit_rank(bits, prefix, (uint32_t)acc.i1);
+      if (acc.b2 < INFINITY) acc.i2 = bit_rank(bits, prefix, (uint32_t)acc.i2);
+      if (acc.b3 < INFINITY) acc.i3 = bit_rank(bits, prefix, (uint32_t)acc.i3);
+    }
     dist2[q * 3] = acc.b1; dist2[q * 3 + 1] = acc.b2; dist2[q * 3 + 2] = acc.b3;
     idx[q * 3] = acc.i1; idx[q * 3 + 1] = acc.i2; idx[q * 3 + 2] = acc.i3;
+    if (weight != nullptr) nn_weights(acc.b1, acc.b2, acc.b3, weight + q * 3);
   }
 }
 
@@ -512,7 +593,8 @@ __global__ void __launch_bounds__(256)
     three_nn_list_kernel(int n, int m, const float *__restrict__ unknown,
                          const float *__restrict__ known, const int32_t *__restrict__ counter,
                          const int32_t *__restrict__ list, int redo_above,
-                         float *__restrict__ dist2, int32_t *__restrict__ idx) {
+                         float *__restrict__ dist2, int32_t *__restrict__ idx,
+                         float *__restrict__ weight) {
   __shared__ float sd[4][3];
   __shared__ int si[4][3];
   const int count = counter[0];
@@ -558,6 +640,7 @@ __global__ void __launch_bounds__(256)
           if (sd[w][k] < INFINITY) best.insert(sd[w][k], si[w][k]);
       dist2[q * 3] = best.b1; dist2[q * 3 + 1] = best.b2; dist2[q * 3 + 2] = best.b3;
       idx[q * 3] = best.i1; idx[q * 3 + 1] = best.i2; idx[q * 3 + 2] = best.i3;
+      if (weight != nullptr) nn_weights(best.b1, best.b2, best.b3, weight + q * 3);
     }
     __syncthreads();
   }
@@ -581,6 +664,65 @@ size_t ssc_three_nn_grid_workspace_bytes(int32_t n, int32_t m, int32_t batch_siz
          align_up((size_t)(n > 0 ? n : 1) * sizeof(int32_t));
 }
 
+// The grid search, queued.  vg (optional): the known points are the voxels' centres as vg
+// states them (three_nn_grid_kernel<true>); weight (optional): the interpolation weights are
+// written with the result; table_cleared: the caller has zeroed the table and its totals.
+static int nn_grid_enqueue(int32_t n, int32_t m, const float *unknown, const float *known,
+                           const int32_t *voxel_indices, int32_t batch_size,
+                           const int32_t dims[3], const float origin[3], const float unit[3],
+                           float *dist2, int32_t *idx, void *workspace, hipStream_t s,
+                           const V2pGrid *vg, float *weight, bool table_cleared) {
+  const int64_t cells = nng_cells(batch_size, dims);
+  GridNn g;
+  g.batch = batch_size;
+  for (int a = 0; a < 3; ++a) {
+    g.dim[a] = dims[a];
+    g.origin[a] = origin[a];
+    g.unit[a] = unit[a];
+  }
+  Carver c(workspace);
+  BitTable t = bit_table_carve(c, cells);
+  int32_t *rank2row = c.take<int32_t>((size_t)(m > 0 ? m : 1));
+  int32_t *list = c.take<int32_t>((size_t)n);
+  // t.total[1] and [2] are cleared with the table and not used by the scan: the counter of
+  // the queries left open, and the flag "voxel rows not in key order"
+  int32_t *counter = t.total + 1, *disorder = t.total + 2;
+  int rc;
+  if (!table_cleared && (rc = bit_table_clear(t, s)) != SSC_OK) return rc;
+  if (m > 0) {
+    hipLaunchKernelGGL(nng_mark_kernel, dim3((unsigned)ceil_div(m, 256)), dim3(256), 0, s,
+                       voxel_indices, m, g, t.bits, counter, disorder);
+    SSC_LAUNCH_CHECK("nng_mark");
+  }
+  if ((rc = bit_table_scan(t, s)) != SSC_OK) return rc;
+  if (m > 0) {
+    hipLaunchKernelGGL(nng_rank2row_kernel, dim3((unsigned)ceil_div(m, 256)), dim3(256), 0, s,
+                       voxel_indices, m, g, t.bits, t.prefix, rank2row,
+                       vg != nullptr ? disorder : (const int32_t *)nullptr);
+    SSC_LAUNCH_CHECK("nng_rank2row");
+  }
+  const dim3 grid((unsigned)ceil_div(n, 256 / kGridNnLanes));
+  if (vg != nullptr) {
+    hipLaunchKernelGGL(three_nn_grid_kernel<true>, grid, dim3(256), 0, s, n, m, unknown, known, g,
+                       t.bits, t.prefix, rank2row, dist2, idx, counter, list, *vg, disorder,
+                       weight);
+  } else {
+    hipLaunchKernelGGL(three_nn_grid_kernel<false>, grid, dim3(256), 0, s, n, m, unknown, known,
+                       g, t.bits, t.prefix, rank2row, dist2, idx, counter, list, V2pGrid{},
+                       disorder, weight);
+  }
+  SSC_LAUNCH_CHECK("three_nn_grid");
+  const int redo_above = n / 8;
+  hipLaunchKernelGGL(three_nn_list_kernel, dim3(512), dim3(256), 0, s, n, m, unknown, known,
+                     counter, list, redo_above, dist2, idx, weight);
+  SSC_LAUNCH_CHECK("three_nn_list");
+  hipLaunchKernelGGL(three_nn_kernel, dim3((unsigned)ceil_div(n, kNnTile / kNnLanes)), dim3(kNnTile),
+                     0, s, n, m, unknown, known, (const float *)nullptr, dist2, idx,
+                     (const int32_t *)counter, redo_above, weight);
+  SSC_LAUNCH_CHECK("three_nn");
+  return SSC_OK;
+}
+
 int ssc_three_nn_grid(int32_t n, int32_t m, const float *unknown, const float *known,
                       const int32_t *voxel_indices, int32_t batch_size, const int32_t dims[3],
                       const float origin[3], const float unit[3], float *dist2, int32_t *idx,
@@ -596,47 +738,8 @@ int ssc_three_nn_grid(int32_t n, int32_t m, const float *unknown, const float *k
   SSC_CHECK(workspace != nullptr &&
                 workspace_bytes >= ssc_three_nn_grid_workspace_bytes(n, m, batch_size, dims),
             SSC_EWORKSPACE, "three_nn_grid workspace too small");
-  hipStream_t s = (hipStream_t)stream;
-  GridNn g;
-  g.batch = batch_size;
-  for (int a = 0; a < 3; ++a) {
-    g.dim[a] = dims[a];
-    g.origin[a] = origin[a];
-    g.unit[a] = unit[a];
-  }
-  Carver c(workspace);
-  BitTable t = bit_table_carve(c, cells);
-  int32_t *rank2row = c.take<int32_t>((size_t)(m > 0 ? m : 1));
-  int32_t *list = c.take<int32_t>((size_t)n);
-  // t.total[1] is cleared with the table and not used by the scan: the counter of the
-  // queries left open
-  int32_t *counter = t.total + 1;
-  int rc;
-  if ((rc = bit_table_clear(t, s)) != SSC_OK) return rc;
-  if (m > 0) {
-    hipLaunchKernelGGL(nng_mark_kernel, dim3((unsigned)ceil_div(m, 256)), dim3(256), 0, s,
-                       voxel_indices, m, g, t.bits, counter);
-    SSC_LAUNCH_CHECK("nng_mark");
-  }
-  if ((rc = bit_table_scan(t, s)) != SSC_OK) return rc;
-  if (m > 0) {
-    hipLaunchKernelGGL(nng_rank2row_kernel, dim3((unsigned)ceil_div(m, 256)), dim3(256), 0, s,
-                       voxel_indices, m, g, t.bits, t.prefix, rank2row);
-    SSC_LAUNCH_CHECK("nng_rank2row");
-  }
-  hipLaunchKernelGGL(three_nn_grid_kernel, dim3((unsigned)ceil_div(n, 256 / kGridNnLanes)),
-                     dim3(256), 0, s, n, m, unknown, known, g, t.bits, t.prefix, rank2row, dist2,
-                     idx, counter, list);
-  SSC_LAUNCH_CHECK("three_nn_grid");
-  const int redo_above = n / 8;
-  hipLaunchKernelGGL(three_nn_list_kernel, dim3(512), dim3(256), 0, s, n, m, unknown, known,
-                     counter, list, redo_above, dist2, idx);
-  SSC_LAUNCH_CHECK("three_nn_list");
-  hipLaunchKernelGGL(three_nn_kernel, dim3((unsigned)ceil_div(n, kNnTile / kNnLanes)), dim3(kNnTile),
-                     0, s, n, m, unknown, known, (const float *)nullptr, dist2, idx,
-                     (const int32_t *)counter, redo_above);
-  SSC_LAUNCH_CHECK("three_nn");
-  return SSC_OK;
+  return nn_grid_enqueue(n, m, unknown, known, voxel_indices, batch_size, dims, origin, unit,
+                         dist2, idx, workspace, (hipStream_t)stream, nullptr, nullptr, false);
 }
 
 }  // extern "C"
@@ -646,17 +749,21 @@ int ssc_three_nn_grid(int32_t n, int32_t m, const float *unknown, const float *k
 // interpolation (ss_conv/sp_ops/voxelize.py:131-160), as kernels of one call.
 namespace ssc {
 
-struct V2pGrid {
-  float unit[3], half_extent[3], half_unit[3];
-};
-
-// unknown[i] = (batch id, x, y, z) of point i; known[j] = (b, centre of voxel j) with
-// centre = (index * unit - 0.5 extent) + 0.5 unit, the three roundings of the reference's
-// expression (voxelize.py:139).
+// unknown[i] = (batch id, x, y, z) of point i; known[j] = (b, centre of voxel j) (v2p_centre).
+// The blocks behind those of the points and voxels zero the search's table and its totals
+// (what bit_table_clear would do in a launch of its own).
 __global__ void __launch_bounds__(256)
     v2p_prepare_kernel(const float *__restrict__ pts, const int64_t *__restrict__ ids, int n,
                        const int32_t *__restrict__ vox, int m, V2pGrid g,
-                       float *__restrict__ unknown, float *__restrict__ known) {
+                       float *__restrict__ unknown, float *__restrict__ known, int row_blocks,
+                       uint32_t *__restrict__ bits, int64_t n_words, int32_t *__restrict__ total) {
+  if ((int)blockIdx.x >= row_blocks) {
+    const int64_t step = (int64_t)(gridDim.x - row_blocks) * blockDim.x;
+    int64_t w = (int64_t)(blockIdx.x - row_blocks) * blockDim.x + threadIdx.x;
+    if (w < 4) total[w] = 0;
+    for (; w < n_words; w += step) bits[w] = 0u;
+    return;
+  }
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i < n) {
     const float4v u = {(float)ids[i], pts[(int64_t)i * 3], pts[(int64_t)i * 3 + 1],
@@ -667,26 +774,11 @@ __global__ void __launch_bounds__(256)
     const int4 r = reinterpret_cast<const int4 *>(vox)[i];
     float4v k;
     k.x = (float)r.x;
-    k.y = ((float)r.y * g.unit[0] - g.half_extent[0]) + g.half_unit[0];
-    k.z = ((float)r.z * g.unit[1] - g.half_extent[1]) + g.half_unit[1];
-    k.w = ((float)r.w * g.unit[2] - g.half_extent[2]) + g.half_unit[2];
+    k.y = v2p_centre(r.y, g, 0);
+    k.z = v2p_centre(r.z, g, 1);
+    k.w = v2p_centre(r.w, g, 2);
     reinterpret_cast<float4v *>(known)[i] = k;
   }
-}
-
-// weight[q, j] = r_j / ((r_0 + r_1) + r_2) with r_j = 1 / (sqrt(dist2[q, j]) + 1e-8)
-// (voxelize.py:156-159).
-__global__ void __launch_bounds__(256)
-    v2p_weight_kernel(const float *__restrict__ dist2, int n, float *__restrict__ weight) {
-  const int q = blockIdx.x * blockDim.x + threadIdx.x;
-  if (q >= n) return;
-  const float r0 = 1.0f / (sqrtf(dist2[q * 3]) + 1e-8f);
-  const float r1 = 1.0f / (sqrtf(dist2[q * 3 + 1]) + 1e-8f);
-  const float r2 = 1.0f / (sqrtf(dist2[q * 3 + 2]) + 1e-8f);
-  const float norm = (r0 + r1) + r2;
-  weight[q * 3] = r0 / norm;
-  weight[q * 3 + 1] = r1 / norm;
-  weight[q * 3 + 2] = r2 / norm;
 }
 
 }  // namespace ssc
@@ -729,15 +821,21 @@ int ssc_v2p_interpolate_f32(const float *points, const int64_t *batch_ids, int32
     g.half_unit[a] = 0.5f * unit[a];
     origin[a] = -0.5f * extent[a];
   }
-  hipLaunchKernelGGL(v2p_prepare_kernel, dim3((unsigned)ceil_div(n > m ? n : m, 256)), dim3(256),
-                     0, s, points, batch_ids, n, voxel_indices, m, g, unknown, known);
+  // (the table of the search, as nn_grid_enqueue will carve it from the same bytes)
+  Carver cs(search_ws);
+  const BitTable t = bit_table_carve(cs, nng_cells(batch_size, dims));
+  const int row_blocks = (int)ceil_div(n > m ? n : m, 256);
+  int64_t clear_blocks = ceil_div(t.n_words, 256 * 4);
+  if (clear_blocks > 2048) clear_blocks = 2048;
+  if (clear_blocks < 1) clear_blocks = 1;
+  hipLaunchKernelGGL(v2p_prepare_kernel, dim3((unsigned)(row_blocks + clear_blocks)), dim3(256), 0,
+                     s, points, batch_ids, n, voxel_indices, m, g, unknown, known, row_blocks,
+                     t.bits, t.n_words, t.total);
   SSC_LAUNCH_CHECK("v2p_prepare");
-  int rc = ssc_three_nn_grid(n, m, unknown, known, voxel_indices, batch_size, dims, origin, unit,
-                             dist2, idx, search_ws, search, stream);
+  // the search ranks its candidates by the centres of their cells and writes the weights
+  int rc = nn_grid_enqueue(n, m, unknown, known, voxel_indices, batch_size, dims, origin, unit,
+                           dist2, idx, search_ws, s, &g, weight, true);
   if (rc != SSC_OK) return rc;
-  hipLaunchKernelGGL(v2p_weight_kernel, dim3((unsigned)ceil_div(n, 256)), dim3(256), 0, s, dist2, n,
-                     weight);
-  SSC_LAUNCH_CHECK("v2p_weight");
   return ssc_three_interp_f32(channels, m, n, voxel_feats, idx, weight, out, stream);
 }
 
