@@ -801,6 +801,7 @@ def main():
     try:
         for _ in range(3):
             out = step()
+        _ext.profile_conv(True, every=args.time_every or (2 if args.steps >= 20 else 1))
         gc.disable()
         torch.cuda.synchronize()
         t3 = time.perf_counter()
@@ -809,6 +810,8 @@ def main():
         torch.cuda.synchronize()
         ms_one_stream = (time.perf_counter() - t3) * 1e3 / args.steps
         gc.enable()
+        conv_ms_alone = _ext.profile_conv_read()
+        _ext.profile_conv(False)
     finally:
         _ext.index_stream(was)
 
@@ -850,7 +853,13 @@ def main():
                      "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
                      "kernel": "conv_fwd_kernel", "kernel_ms": conv_kernel_ms,
                      "kernel_launches_timed": len(conv_ms),
-                     "flops_per_launch": flops},
+                     "flops_per_launch": flops,
+                     # the same kernel with nothing beside it (the one-stream region: in the
+                     # timed region the next step's index work shares the CUs with it)
+                     "kernel_ms_one_stream": sum(conv_ms_alone) / max(len(conv_ms_alone), 1),
+                     "frac_one_stream": (flops / (sum(conv_ms_alone) / max(len(conv_ms_alone), 1)
+                                                  * 1e-3) / 1e12 / FP32_MFMA_PEAK_TFLOPS)
+                     if conv_ms_alone else None},
     }
 
     # the two bandwidth-bound callers of the layer that the metric names, measured in this
