@@ -7,6 +7,7 @@ library the import fails, and without a GPU every call raises.
 """
 import ctypes
 import os
+import threading
 
 import torch
 
@@ -221,9 +222,7 @@ def _geometry(batch_size, out_shape, ksize, stride, padding, dilation, subm, tra
 
 
 # Output rows are written before their number is known when a buffer for the largest
-# possible number of them is at most this large (a result that fills less than half of a
-# buffer of more than 4 MiB is copied out of it, so that no rulebook keeps more than twice
-# its rows alive).
+# possible number of them is at most this large; the result is a slice of that buffer.
 _ROWS_AHEAD_BYTES = 256 << 20
 _ROWS_KEEP_BYTES = 64 << 20  # unused rows of such a buffer beyond which the result is copied out of it
 # largest plan / plan scratch allocated for the bound on the number of outputs, before the
@@ -430,6 +429,22 @@ def _index_done(r, *tensors):
             t.record_stream(r.main)
 
 
+_scratch_held = {}  # (thread, device index, stream, use) -> buffer
+
+
+def _stream_scratch(dev, stream, key, nbytes):
+    """A buffer that only the kernels of one call at a time use, all on `stream`: one per
+    host thread, device, stream and use, kept and reused (the kernels of two calls on a
+    stream run in order), regrown when a call needs more.  Allocated under whatever torch
+    stream is current, which callers make the one the kernels run on."""
+    k = (threading.get_ident(), dev.index, stream, key)
+    held = _scratch_held.get(k)
+    if held is None or held.numel() < nbytes:
+        held = _workspace(nbytes, dev)
+        _scratch_held[k] = held
+    return held
+
+
 class _PendingRulebook(object):
     """A rulebook between ssc_rulebook_begin and ssc_rulebook_finish: everything whose size
     does not depend on the number of outputs is queued, the host has not waited yet."""
@@ -484,7 +499,8 @@ def _rulebook_queue(r, gref, K, nbytes, conv):
     """Allocate a rulebook's buffers and queue it (on the current torch stream = r.stream)."""
     indices, n, subm = r.indices, r.n, r.subm
     dev = indices.device
-    r.ws = _workspace(nbytes, dev)
+    # (workspace and plan scratch hold nothing between two calls: kept per stream)
+    r.ws = _stream_scratch(dev, r.stream, "rulebook", nbytes)
     r.pairs = torch.empty((K, 2, n), dtype=torch.int32, device=dev)
     r.num = torch.empty((K,), dtype=torch.int32, device=dev)
     # Marking, ranking and the pair lists are queued; the host then waits for the number of
@@ -506,7 +522,7 @@ def _rulebook_queue(r, gref, K, nbytes, conv):
         scratch_bytes = _lib.ssc_conv_plan_scratch_bytes(r.bound, K, c_in, c_out, n)
         if plan_bytes <= _PLAN_AHEAD_BYTES and scratch_bytes <= _PLAN_AHEAD_BYTES:
             r.plan = _workspace(plan_bytes, dev)
-            r.scratch = _workspace(scratch_bytes, dev)
+            r.scratch = _stream_scratch(dev, r.stream, "plan", scratch_bytes)
             r.conv = (int(c_in), int(c_out), int(eb))
     clean_bytes = _lib.ssc_rulebook_clean_table_bytes(gref, n)
     clean = _clean_table(clean_bytes, dev, r.stream) if clean_bytes > 0 else None
@@ -1478,18 +1494,9 @@ class P2vConsts(object):
         self.ws_bytes = {}  # (points, ids) -> workspace size
 
 
-_p2v_scratch = {}  # (device index, stream) -> buffers that hold nothing between two calls
-
-
 def _p2v_scratch_of(dev, stream, key, nbytes):
-    """A buffer of the one-call Point2Voxel that nothing reads after the call's kernels: one
-    per device, stream and use, kept and reused (the kernels of two calls on a stream run in
-    order), regrown when a call needs more."""
-    held = _p2v_scratch.get((dev.index, stream, key))
-    if held is None or held.numel() < nbytes:
-        held = _workspace(nbytes, dev)
-        _p2v_scratch[(dev.index, stream, key)] = held
-    return held
+    """A buffer of the one-call Point2Voxel that nothing reads after the call's kernels."""
+    return _stream_scratch(dev, stream, "p2v " + key, nbytes)
 
 
 def p2v_voxelize(points, feats, batch_ids, consts, mode, n_ids):
