@@ -1147,6 +1147,57 @@ def test_index_work_on_a_second_stream(device):
             assert torch.equal(tb, tc)
 
 
+def test_index_work_on_a_second_stream_training_step(device):
+    """A training step -- forward, loss, backward through three layers, the first two sharing
+    a rulebook under an indice_key -- with rulebooks and plans on the second stream: the
+    gradients of the features and of every layer's weights equal those of the same step on
+    one stream, bit for bit, over several steps that follow each other without a wait."""
+    from ss_conv import _ext
+    from ss_conv.convolution import Convolution
+    from ss_conv.sp_ops.tensor import SparseTensor
+    torch.manual_seed(13)
+    rs0, rs1 = [(4, 0), (2, 1)], [(6, 0), (3, 1), (1, 2)]
+    layers = [Convolution(rs0, rs1, 3, stride=1, padding=1, subm=True, indice_key="s").to(device),
+              Convolution(rs1, rs1, 3, stride=1, padding=1, subm=True, indice_key="s").to(device),
+              Convolution(rs1, rs0, 3, stride=2, padding=1).to(device)]
+    for m in layers:
+        m.train()
+    grid, n = 18, 2500
+    rng = np.random.default_rng(22)
+    clouds = [torch.from_numpy(random_voxels(rng, 2, grid, n)).to(device) for _ in range(3)]
+
+    def run_all():
+        outs = []
+        for it in range(5):
+            idx = clouds[it % 3].clone()
+            feats = torch.randn(n, layers[0].in_channels, device=device,
+                                generator=torch.Generator(device).manual_seed(100 + it))
+            feats.requires_grad_(True)
+            for m in layers:
+                m.zero_grad(set_to_none=True)
+            x = SparseTensor(feats, idx, [grid] * 3, 2)
+            for m in layers:
+                x = m(x)
+            (x.features * x.features).sum().backward()
+            outs.append([feats.grad.clone()] + [m.kernel.weight.grad.clone() for m in layers])
+        torch.cuda.synchronize()
+        return outs
+
+    keep = _ext._INDEX_STREAM_MIN_WORK
+    was = _ext.index_stream(True)
+    try:
+        _ext._INDEX_STREAM_MIN_WORK = 0
+        two = run_all()
+        _ext.index_stream(False)
+        one = run_all()
+    finally:
+        _ext._INDEX_STREAM_MIN_WORK = keep
+        _ext.index_stream(was)
+    for a, b in zip(two, one):
+        for ta, tb in zip(a, b):
+            assert torch.equal(ta, tb)
+
+
 def test_layer_gradients(oracle, device):
     """loss.backward() through Convolution: gradient of the input features against the
     restated backward, gradient of kernel.weight against torch autograd through an
