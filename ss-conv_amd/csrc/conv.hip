@@ -1254,11 +1254,13 @@ static ConvPlan make_plan(int64_t n_in, int64_t n_out, int K, int c_in, int c_ou
   // more small launches (30 us; the split evens out 3-15 % of the kernel's time, more with
   // more ranges): 1500 stages per workgroup or more.
   p.rebalance = g_conv_rebalance && est_stages >= g_conv_rebalance_stages;
-  // The accumulator window: all of the LDS for kernels that run long (a second split, or
-  // ranges worth pairing), a few KB less for the others (see pick_tile); sizing calls
-  // (N_in unknown) count with the smaller window, which has more tiles.
-  const bool long_kernel =
-      n_in > 0 && (est_stages >= kRebalanceStages || est_groups >= kPairGroups);
+  // The accumulator window: all of the LDS for kernels that run long (those that get a second
+  // split: about 2 ms and up), a few KB less for the others (see pick_tile); sizing calls
+  // (N_in unknown) count with the smaller window, which has more tiles.  (Kernels of middle
+  // size lose and gain about the same, 10.49 against 10.48 ms for the backbone whose stages
+  // they are; layers whose pairs the estimate overstates -- a strided layer with more
+  // outputs than inputs -- are short kernels and gain.)
+  const bool long_kernel = n_in > 0 && est_stages >= kRebalanceStages;
   p.T = pick_tile(p.acc_cols, !long_kernel);
   p.tile_rows = p.T - (p.five ? kSpillRowsFive : kSpillRows);
   // Two ranges to a workgroup, paired by what they came to (range_assign_kernel): one more

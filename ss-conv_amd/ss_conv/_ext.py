@@ -347,7 +347,14 @@ def _beside(on):
         _beside_now[0] = on
 
 
-_INDEX_STREAM_MIN_WORK = 1 << 20  # rows * offsets below which the second stream is not worth its events
+# The second stream pays where the kernel that waits for the index work -- the convolution of
+# this layer, and with it, in a stack of like layers, the one the index work runs beside --
+# is several times as long as the index work itself: from an estimated 20 GFLOP of convolution
+# on (0.25 ms; the benchmark layer has 25, and gains 10 %; a strided layer of 13 GFLOP behind
+# thirteen small launches gains nothing), and for rulebooks without a convolution from a
+# million row-offset combinations on.
+_INDEX_STREAM_MIN_FLOPS = 2e10
+_INDEX_STREAM_MIN_WORK = 1 << 20
 _INDEX_AHEAD_EVERY = 8  # the host runs at most about three times this many rulebooks ahead
 
 
@@ -370,9 +377,9 @@ def index_stream(enable):
     return old
 
 
-def _index_stream_for(dev, main, work):
+def _index_stream_for(dev, main):
     """The device's stream for index work, or None when this call's stays on `main`."""
-    if not _index_overlap or work < _INDEX_STREAM_MIN_WORK or torch.cuda.is_current_stream_capturing():
+    if not _index_overlap or torch.cuda.is_current_stream_capturing():
         return None
     st = _index_streams.get(dev.index)
     if st is None:
@@ -480,7 +487,12 @@ def _rulebook_begin(indices, batch_size, out_spatial_shape, kernel_size, stride,
     r = _PendingRulebook()
     r.indices, r.n, r.geometry, r.subm = indices, n, g, bool(subm)
     r.main = torch.cuda.current_stream(dev)
-    r.side = _index_stream_for(dev, r.main, n * K)
+    if conv is None:
+        worth = n * K >= _INDEX_STREAM_MIN_WORK
+    else:  # pairs ~ rows * offsets / prod(stride), two flops per pair, input and output channel
+        pairs = n * K / max(int(stride[0]) * int(stride[1]) * int(stride[2]), 1)
+        worth = 2.0 * pairs * conv[0] * conv[1] >= _INDEX_STREAM_MIN_FLOPS
+    r.side = _index_stream_for(dev, r.main) if worth else None
     _beside(r.side is not None)
     if r.side is not None:
         if not _side_ready(indices):

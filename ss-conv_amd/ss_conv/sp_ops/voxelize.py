@@ -38,6 +38,7 @@ class Point2Voxel(nn.Module):
         # first call, of any other (64 before any call).
         self._n_ids_hint = Point2Voxel._n_ids_seen
         self._consts = None
+        self._grid_consts()  # (converted here, not by the first call)
         self.last_path = None  # which of the three ways the last forward took (diagnostics)
 
     def _grid_consts(self):

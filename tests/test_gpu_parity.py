@@ -1129,17 +1129,18 @@ def test_index_work_on_a_second_stream(device):
         torch.cuda.synchronize()
         return outs
 
-    keep = _ext._INDEX_STREAM_MIN_WORK
+    keep = _ext._INDEX_STREAM_MIN_WORK, _ext._INDEX_STREAM_MIN_FLOPS
     was = _ext.index_stream(True)
     try:
-        _ext._INDEX_STREAM_MIN_WORK = 0  # (these layers are far below the size it is meant for)
+        # (these layers are far below the size it is meant for)
+        _ext._INDEX_STREAM_MIN_WORK = _ext._INDEX_STREAM_MIN_FLOPS = 0
         with torch.no_grad():
             two = run_all()
             again = run_all()
             _ext.index_stream(False)
             one = run_all()
     finally:
-        _ext._INDEX_STREAM_MIN_WORK = keep
+        _ext._INDEX_STREAM_MIN_WORK, _ext._INDEX_STREAM_MIN_FLOPS = keep
         _ext.index_stream(was)
     for a, b, c in zip(two, again, one):
         for ta, tb, tc in zip(a, b, c):
@@ -1183,15 +1184,15 @@ def test_index_work_on_a_second_stream_training_step(device):
         torch.cuda.synchronize()
         return outs
 
-    keep = _ext._INDEX_STREAM_MIN_WORK
+    keep = _ext._INDEX_STREAM_MIN_WORK, _ext._INDEX_STREAM_MIN_FLOPS
     was = _ext.index_stream(True)
     try:
-        _ext._INDEX_STREAM_MIN_WORK = 0
+        _ext._INDEX_STREAM_MIN_WORK = _ext._INDEX_STREAM_MIN_FLOPS = 0
         two = run_all()
         _ext.index_stream(False)
         one = run_all()
     finally:
-        _ext._INDEX_STREAM_MIN_WORK = keep
+        _ext._INDEX_STREAM_MIN_WORK, _ext._INDEX_STREAM_MIN_FLOPS = keep
         _ext.index_stream(was)
     for a, b in zip(two, one):
         for ta, tb in zip(a, b):
