@@ -52,7 +52,7 @@ def parse_args():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--time-every", type=int, default=0, metavar="N",
                     help="time every N-th launch of the convolution kernel with HIP events "
-                         "(default: every other one, every launch below 20 steps)")
+                         "(default: every fourth one, every launch below 20 steps)")
     ap.add_argument("--calibration-copy", type=int, default=0, metavar="MIB",
                     help="also run one plain device copy of MIB mebibytes before the timed "
                          "region (the known-size kernel that scales rocprofv3's FETCH_SIZE / "
@@ -768,9 +768,10 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    # every other launch of the convolution kernel inside the timed region is timed with HIP
-    # events on its stream (a pair of events costs the stream a few microseconds)
-    _ext.profile_conv(True, every=args.time_every or (2 if args.steps >= 20 else 1))
+    # every fourth launch of the convolution kernel inside the timed region is timed with HIP
+    # events on its stream (a pair of events costs the stream 7-10 us: the kernel behind it
+    # cannot be set up while the one before it still runs)
+    _ext.profile_conv(True, every=args.time_every or (4 if args.steps >= 20 else 1))
     # The interpreter's cyclic garbage collector stays out of the timed region, as in
     # timeit: a full collection of a process that has imported torch takes 30-40 ms, many
     # times the region itself, and when it falls due depends on allocation counts only.
@@ -801,7 +802,7 @@ def main():
     try:
         for _ in range(3):
             out = step()
-        _ext.profile_conv(True, every=args.time_every or (2 if args.steps >= 20 else 1))
+        _ext.profile_conv(True, every=args.time_every or (4 if args.steps >= 20 else 1))
         gc.disable()
         torch.cuda.synchronize()
         t3 = time.perf_counter()

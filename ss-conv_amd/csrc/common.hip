@@ -53,22 +53,26 @@ BitTable bit_table_carve(Carver &c, int64_t n_bits) {
   return t;
 }
 
-// bits[] = 0, total[0..3] = 0 and (when asked for) blocksum[] = 0 in one launch.
+// bits[] = 0, total[0..3] = 0 and (when asked for) blocksum[] = 0 and a counter for every
+// word, per_word[] = 0, in one launch.
 __global__ void __launch_bounds__(256)
     bit_clear_kernel(uint32_t *__restrict__ bits, int64_t n_words, int32_t *__restrict__ total,
-                     int32_t *__restrict__ blocksum, int64_t n_blocksum) {
+                     int32_t *__restrict__ blocksum, int64_t n_blocksum,
+                     int32_t *__restrict__ per_word) {
   int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i < 4) total[i] = 0;
   const int64_t step = (int64_t)gridDim.x * blockDim.x;
   for (int64_t j = i; j < n_blocksum; j += step) blocksum[j] = 0;
+  if (per_word != nullptr)
+    for (int64_t j = i; j < n_words; j += step) per_word[j] = 0;
   for (; i < n_words; i += step) bits[i] = 0u;
 }
 
-int bit_table_clear(const BitTable &t, hipStream_t s, bool blocksum_too) {
+int bit_table_clear(const BitTable &t, hipStream_t s, bool blocksum_too, int32_t *per_word) {
   const int64_t want = ceil_div(t.n_words > 0 ? t.n_words : 1, 256);
   const int blocks = (int)(want < 8192 ? want : 8192);
   hipLaunchKernelGGL(bit_clear_kernel, dim3(blocks), dim3(256), 0, s, t.bits, t.n_words, t.total,
-                     t.blocksum, blocksum_too ? t.n_scan_blocks : (int64_t)0);
+                     t.blocksum, blocksum_too ? t.n_scan_blocks : (int64_t)0, per_word);
   SSC_LAUNCH_CHECK("bit_clear");
   return SSC_OK;
 }

@@ -1316,6 +1316,7 @@ static size_t conv_scratch_head(void *base, ConvWs *w) {
   Carver c(base);
   w->flag = c.take<int32_t>(1);
   w->range_row0 = c.take<int32_t>((size_t)kMaxRanges + 1);
+  w->range_row0_alt = c.take<int32_t>((size_t)kMaxRanges + 1);
   return c.used;
 }
 
@@ -1325,6 +1326,7 @@ static size_t conv_scratch_walk(void *base, const ConvPlan &p, int K, int64_t pa
   ConvWs t;
   t.flag = c.take<int32_t>(1);
   t.range_row0 = c.take<int32_t>((size_t)kMaxRanges + 1);
+  t.range_row0_alt = c.take<int32_t>((size_t)kMaxRanges + 1);
   t.segs = c.take<int32_t>((size_t)(p.n_tiles + 1) * K);
   t.sorted = c.take<int32_t>((size_t)K * 2 * pair_stride);
   t.bits = c.take<uint32_t>((size_t)K * p.words_per_k);
@@ -1355,6 +1357,7 @@ static size_t conv_scratch_walk(void *base, const ConvPlan &p, int K, int64_t pa
     w->kofs = t.kofs;
     w->fine_segs = t.fine_segs;
     w->range_row0 = t.range_row0;
+    w->range_row0_alt = t.range_row0_alt;
     w->tile_row0 = t.tile_row0;
     w->spill_end = t.spill_end;
     w->tile_slot0 = t.tile_slot0;
@@ -1474,9 +1477,11 @@ extern "C" {
 
 int ssc_profile_conv(int32_t enable) {
   if (enable && !g_profile_init) {
+    // (events that only measure time: without the system-scope fence, whose cache
+    // write-back and invalidation would be charged to the kernels around them)
     for (int i = 0; i < kProfileRing; ++i) {
-      SSC_HIP(hipEventCreate(&g_profile_ev[i][0]));
-      SSC_HIP(hipEventCreate(&g_profile_ev[i][1]));
+      SSC_HIP(hipEventCreateWithFlags(&g_profile_ev[i][0], hipEventDisableSystemFence));
+      SSC_HIP(hipEventCreateWithFlags(&g_profile_ev[i][1], hipEventDisableSystemFence));
     }
     g_profile_init = true;
   }
@@ -1993,10 +1998,12 @@ static int combine_job_of(const float *weight, const float *basis, const int32_t
 }
 
 // A rulebook between ssc_rulebook_conv_begin and ssc_rulebook_conv_finish on this host thread:
-// whether the rulebook was asked to place the range boundaries, and for how many ranges.
+// whether the rulebook was asked to place the range boundaries, and for which cuts (number
+// of ranges and tile height of the request and of its alternative; 0 ranges: none).
 struct PendingLayer {
   bool seeded = false;
-  int n_rng = 0;
+  int n_rng[2] = {0, 0};
+  int tile_rows[2] = {0, 0};
 };
 static thread_local PendingLayer g_pending_layer;
 
@@ -2018,21 +2025,37 @@ int ssc_rulebook_conv_begin(const int32_t *indices, int64_t n_in, const ssc_geom
                             c_out, filters->out, filters->packed, filters->packed_bytes, &job);
     if (rc != SSC_OK) return rc;
   }
-  SplitRequest rq = {0, 0, 0, nullptr};
+  SplitRequest rq = {0, 0, 0, nullptr, 0, 0, nullptr};
   const SplitRequest *ask = nullptr;
   int64_t K = 1;
   for (int a = 0; a < 3; ++a) K *= g->ksize[a] > 0 ? g->ksize[a] : 1;
   if (scratch != nullptr && n_in > 0 && K <= SSC_MAX_KERNEL_VOLUME && !g->subm && !g->transpose) {
-    // what the plan will look like when the outputs outnumber the inputs, as they do for
-    // the geometries whose rulebook can place the boundaries (stride 1, a padded kernel)
-    const ConvPlan p = make_plan(n_in, n_in + 1, (int)K, c_in, c_out, n_in, elem_bytes);
+    // What the plan will look like depends on whether the outputs outnumber the inputs
+    // (make_plan's estimate of the pairs).  At stride 1 with a padded kernel they do; a
+    // strided layer can go either way (a sparse cloud loses few rows to a stride of 2), so
+    // its rulebook is asked for the cut of either plan where the two differ.
+    bool strided = false;
+    for (int a = 0; a < 3; ++a) strided = strided || g->stride[a] != 1 || g->dilation[a] != 1;
     ConvWs w = {};
     const size_t head = conv_scratch_head(scratch, &w);
-    if (!p.rebalance && !p.small && scratch_bytes >= head) {
-      rq.n_rng = p.n_rng;
-      rq.tile_rows = p.tile_rows;
+    const ConvPlan more = make_plan(n_in, n_in + 1, (int)K, c_in, c_out, n_in, elem_bytes);
+    const ConvPlan fewer =
+        make_plan(n_in, n_in > 1 ? n_in - 1 : 1, (int)K, c_in, c_out, n_in, elem_bytes);
+    const bool more_ok = !more.rebalance && !more.small;
+    const bool fewer_ok = strided && n_in > 1 && !fewer.rebalance && !fewer.small &&
+                          !(more_ok && fewer.n_rng == more.n_rng &&
+                            fewer.tile_rows == more.tile_rows);
+    if (scratch_bytes >= head && (more_ok || fewer_ok)) {
+      const ConvPlan &first = more_ok ? more : fewer;
+      rq.n_rng = first.n_rng;
+      rq.tile_rows = first.tile_rows;
       rq.tile_cost = (long long)K * 4 + 64;  // split_tile_cost
       rq.range_row0 = w.range_row0;
+      if (more_ok && fewer_ok) {
+        rq.n_rng_alt = fewer.n_rng;
+        rq.tile_rows_alt = fewer.tile_rows;
+        rq.range_row0_alt = w.range_row0_alt;
+      }
       ask = &rq;
     }
   }
@@ -2042,7 +2065,10 @@ int ssc_rulebook_conv_begin(const int32_t *indices, int64_t n_in, const ssc_geom
                                &seeded, (hipStream_t)stream, filters ? &job : nullptr);
   if (rc != SSC_OK) return rc;
   g_pending_layer.seeded = seeded;
-  g_pending_layer.n_rng = rq.n_rng;
+  g_pending_layer.n_rng[0] = rq.n_rng;
+  g_pending_layer.tile_rows[0] = rq.tile_rows;
+  g_pending_layer.n_rng[1] = rq.n_rng_alt;
+  g_pending_layer.tile_rows[1] = rq.tile_rows_alt;
   return SSC_OK;
 }
 
@@ -2072,8 +2098,18 @@ int ssc_rulebook_conv_finish(const ssc_geometry *g, int64_t n_in, int32_t *n_out
   conv_plan_walk(plan, p, &w);
   conv_scratch_walk(scratch, p, K, n_in, &w);
   const bool in_order = *in_order_host != 0;
-  const bool seeded =
-      pending.seeded && in_order && !p.rebalance && !p.small && pending.n_rng == p.n_rng;
+  // the cut the rulebook placed for this plan, if any: the one of the same tile height
+  // before one that only has the plan's number of ranges (the height is a weight in the
+  // work measure, not a condition)
+  int cut = -1;
+  if (pending.seeded && in_order && !p.rebalance && !p.small) {
+    for (int c = 1; c >= 0; --c)
+      if (pending.n_rng[c] == p.n_rng) cut = c;
+    for (int c = 1; c >= 0; --c)
+      if (pending.n_rng[c] == p.n_rng && pending.tile_rows[c] == p.tile_rows) cut = c;
+  }
+  const bool seeded = cut >= 0;
+  if (cut == 1) w.range_row0 = w.range_row0_alt;
   return conv_plan_build<float>(p, w, pairs, n_in, pair_num, K, 0, in_order, c_in, n_out,
                                 elem_bytes, nullptr, (hipStream_t)stream, seeded);
 }

@@ -1201,7 +1201,7 @@ struct ConvWs {
   uint32_t *bits;
   int32_t *prefix;
   int32_t *tile_loc, *tile_nmb, *kofs, *tile_rng, *range_grp, *range_row1, *range_g0;
-  int32_t *fine_segs, *range_row0, *tile_row0, *n_tiles_dev;
+  int32_t *fine_segs, *range_row0, *range_row0_alt, *tile_row0, *n_tiles_dev;
   int32_t *spill_end, *tile_slot0, *spill, *share_first, *share_cnt;
 };
 

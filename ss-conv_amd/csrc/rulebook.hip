@@ -140,12 +140,15 @@ __device__ __forceinline__ void combine_job_rows(const CombineJob &job, int64_t 
 // (most cells are reached from several inputs).
 // JOB: the grid rows from ks[0] on synthesise and pack the layer's filters (work that
 // depends on nothing here and that the layer would otherwise launch by itself).
+// word_pairs (optional, zero on entry): word_pairs[w] += the pairs that land on the cells of
+// table word w (integer adds: the sums do not depend on their order), the work measure of a
+// convolution's plan (see SplitRequest).
 template <bool JOB>
 __global__ void __launch_bounds__(256)
     mark_count_kernel(const int32_t *__restrict__ indices, int64_t n_in, Geom g,
                       uint32_t *__restrict__ bits, int32_t *__restrict__ chunk_count,
                       int64_t n_chunks, int32_t *__restrict__ disorder, CombineJob job,
-                      int64_t job_elements) {
+                      int64_t job_elements, int32_t *__restrict__ word_pairs) {
   if constexpr (JOB) {
     if ((int)blockIdx.y >= g.ks[0]) {
       combine_job_rows(job, job_elements, (int)blockIdx.y - g.ks[0], (int)gridDim.y - g.ks[0]);
@@ -173,6 +176,13 @@ __global__ void __launch_bounds__(256)
     int ox = 0;
     const bool tr = g.tr != 0;
     const bool okx = live && tap_to_out(row[1], kx, g.st[0], g.pd[0], g.dl[0], g.os[0], &ox, tr);
+    // the cells a row reaches through the taps of one (kx, ky) are distinct: every bit of
+    // `mask` is one pair
+    auto flush = [&](uint32_t word, uint32_t mask) {
+      if (mask == 0u) return;
+      if ((bits[word] & mask) != mask) atomicOr(&bits[word], mask);
+      if (word_pairs != nullptr) atomicAdd(&word_pairs[word], __popc(mask));
+    };
     for (int ky = 0; ky < g.ks[1]; ++ky) {
       int oy = 0;
       const bool okxy =
@@ -188,14 +198,37 @@ __global__ void __launch_bounds__(256)
         if (ok) {
           const uint32_t key = base + (uint32_t)oz;
           if ((key >> 5) != word) {
-            if (mask != 0u && (bits[word] & mask) != mask) atomicOr(&bits[word], mask);
+            flush(word, mask);
             word = key >> 5;
             mask = 0u;
           }
           mask |= 1u << (key & 31u);
         }
       }
+      if (word_pairs == nullptr) {
+        flush(word, mask);
+        continue;
+      }
+      // The rows of a wave are neighbours in key order, so the words their taps end in come
+      // in runs of equal lanes: the first lane of a run adds the run's pairs with one atomic
+      // (a wave's 64 adds to one address would be served one after the other).
       if (mask != 0u && (bits[word] & mask) != mask) atomicOr(&bits[word], mask);
+      const int cnt = __popc(mask);
+      if (mask == 0u) word = 0xFFFFFFFFu;
+      const uint32_t before = __shfl_up(word, 1, 64);
+      const bool head = lane == 0 || word != before;
+      const unsigned long long heads = __ballot(head);
+      int incl = cnt;
+#pragma unroll
+      for (int dd = 1; dd < 64; dd <<= 1) {
+        const int o = __shfl_up(incl, dd, 64);
+        if (lane >= dd) incl += o;
+      }
+      // the run of a first lane ends before the next first lane
+      const unsigned long long later = lane < 63 ? heads >> (lane + 1) : 0ull;
+      const int last = later != 0ull ? lane + __ffsll((long long)later) - 1 : 63;
+      const int run = __shfl(incl, last, 64) - (incl - cnt);
+      if (head && run > 0) atomicAdd(&word_pairs[word], run);
     }
   }
 }
@@ -388,16 +421,52 @@ __global__ void __launch_bounds__(kScanThreads)
 // below n_scan_blocks run the first pass of the table's popcount scan, the K blocks after
 // them scan the chunk counts of one tap each (regular convolutions only: a submanifold
 // rulebook counts its pairs after the table is ranked).
+// SEED: the blocks of the table also leave, for every word, the output rows and the pairs
+// that lie in the words of its scan block before it (seed_rows[]; seed_pairs[], which holds
+// the words' own pairs on entry, as mark_count_kernel counted them), and the block's pairs
+// (pairsum[]), as the seeded form of dilate_blocksum_kernel does for the dilation path.
+template <bool SEED>
 __global__ void __launch_bounds__(kScanThreads)
     blocksum_scan_chunks_kernel(const uint32_t *__restrict__ bits, int64_t n_words,
                                 int32_t *__restrict__ blocksum, int64_t n_scan_blocks,
                                 int32_t *__restrict__ chunk_count, int64_t n_chunks,
-                                int32_t *__restrict__ pair_num) {
+                                int32_t *__restrict__ pair_num, int32_t *__restrict__ seed_rows,
+                                int32_t *__restrict__ seed_pairs, int32_t *__restrict__ pairsum) {
   __shared__ int lds[kScanThreads / 64 + 1];
-  if ((int64_t)blockIdx.x < n_scan_blocks)
-    popc_blocksum_block(bits, n_words, blockIdx.x, blocksum, lds);
-  else
+  if ((int64_t)blockIdx.x >= n_scan_blocks) {
     scan_chunks_of_tap(chunk_count, n_chunks, (int)(blockIdx.x - n_scan_blocks), pair_num, lds);
+    return;
+  }
+  if constexpr (SEED) {
+    // every thread kScanItems consecutive words, as the second pass of the table's scan
+    const int64_t w0 = (int64_t)blockIdx.x * kScanBlockWords + (int64_t)threadIdx.x * kScanItems;
+    int cr[kScanItems], cp[kScanItems], sr = 0, sp = 0;
+#pragma unroll
+    for (int i = 0; i < kScanItems; ++i) {
+      cr[i] = w0 + i < n_words ? __popc(bits[w0 + i]) : 0;
+      cp[i] = w0 + i < n_words ? seed_pairs[w0 + i] : 0;
+      sr += cr[i];
+      sp += cp[i];
+    }
+    int tot_r, tot_p;
+    int er = block_exclusive_scan(sr, lds, &tot_r);
+    int ep = block_exclusive_scan(sp, lds, &tot_p);
+#pragma unroll
+    for (int i = 0; i < kScanItems; ++i) {
+      if (w0 + i < n_words) {
+        seed_rows[w0 + i] = er;
+        seed_pairs[w0 + i] = ep;
+      }
+      er += cr[i];
+      ep += cp[i];
+    }
+    if (threadIdx.x == 0) {
+      blocksum[blockIdx.x] = tot_r;
+      pairsum[blockIdx.x] = tot_p;
+    }
+  } else {
+    popc_blocksum_block(bits, n_words, blockIdx.x, blocksum, lds);
+  }
 }
 
 // Output table from the input table (see "marking by dilation"), the block sums of its
@@ -655,6 +724,28 @@ __device__ __forceinline__ void split_ranges_block(int group, int64_t n_words,
   }
 }
 
+// Block `block` of the blocks that serve a SplitRequest (split_request_blocks): the first
+// ones place the boundaries of the request itself, the others those of its alternative.
+__device__ __forceinline__ void split_request_block(int block, int64_t n_words,
+                                                    int64_t n_scan_blocks,
+                                                    const int32_t *__restrict__ blocksum,
+                                                    const int32_t *__restrict__ pairsum,
+                                                    const int32_t *__restrict__ seed_rows,
+                                                    const int32_t *__restrict__ seed_pairs,
+                                                    const SplitRequest &rq, long long *pairs_base,
+                                                    int *rows_base) {
+  const int main_blocks = (rq.n_rng + kScanThreads / 16 - 1) / (kScanThreads / 16);
+  if (block < main_blocks) {
+    split_ranges_block(block, n_words, n_scan_blocks, blocksum, pairsum, seed_rows, seed_pairs, rq,
+                       pairs_base, rows_base);
+  } else {
+    const SplitRequest alt = {rq.n_rng_alt, rq.tile_rows_alt, rq.tile_cost, rq.range_row0_alt,
+                              0, 0, nullptr};
+    split_ranges_block(block - main_blocks, n_words, n_scan_blocks, blocksum, pairsum, seed_rows,
+                       seed_pairs, alt, pairs_base, rows_base);
+  }
+}
+
 // The second pass of the table's scan (popc_prefix_block) and, in the blocks after the
 // table's, the range boundaries of a SplitRequest (split_ranges_block): for rulebooks whose
 // pair launch does not take the prefixes in two levels (no room for the output rows at
@@ -672,8 +763,8 @@ __global__ void __launch_bounds__(kScanThreads)
     return;
   }
   extern __shared__ long long seed_dyn[];
-  split_ranges_block((int)(blockIdx.x - n_scan_blocks), n_words, n_scan_blocks, blocksum, pairsum,
-                     seed_rows, seed_pairs, rq, seed_dyn, seed_lds_rows(seed_dyn, n_scan_blocks));
+  split_request_block((int)(blockIdx.x - n_scan_blocks), n_words, n_scan_blocks, blocksum, pairsum,
+                      seed_rows, seed_pairs, rq, seed_dyn, seed_lds_rows(seed_dyn, n_scan_blocks));
 }
 
 // What the two-level form of write_pairs_kernel needs besides the table: the scan blocks'
@@ -708,8 +799,8 @@ __global__ void __launch_bounds__(256)
       // the first row of the grid (its blocks start first: the host is waiting for the
       // totals): the range boundaries of the convolution's plan, and one block for the totals
       if ((int)blockIdx.x < two.split_blocks) {
-        split_ranges_block((int)blockIdx.x, n_words, two.n_scan_blocks, two.blocksum, two.pairsum,
-                           two.seed_rows, two.seed_pairs, two.split, seed_dyn, base_s);
+        split_request_block((int)blockIdx.x, n_words, two.n_scan_blocks, two.blocksum, two.pairsum,
+                            two.seed_rows, two.seed_pairs, two.split, seed_dyn, base_s);
         return;
       }
       if ((int)blockIdx.x != two.split_blocks) return;
@@ -876,8 +967,9 @@ struct RulebookWs {
   uint32_t *in_bits;     // input table of the dilation path (when it applies)
   DenseIn dense;
   bool use_dense;
-  // seed of a convolution's work split (dilation path, tables of at most kSeedMaxBlocks scan
-  // blocks): rows and pairs before every word inside its scan block, pairs of every block
+  // seed of a convolution's work split (regular convolutions, tables of at most
+  // kSeedMaxBlocks scan blocks): rows and pairs before every word inside its scan block,
+  // pairs of every block
   bool can_seed;
   int32_t *seed_rows, *seed_pairs, *pairsum;
 };
@@ -892,7 +984,7 @@ static size_t rulebook_ws_bytes(const Geom &g, int64_t n_in) {
   const size_t dense = dense_marking_applies(g, n_in, &d)
                            ? align_up((size_t)dense_in_words(g, d) * 4)
                            : 0;
-  const size_t seed = dense > 0 && seed_applies(g)
+  const size_t seed = !g.subm && seed_applies(g)
                           ? 2 * align_up((size_t)bit_words(geom_cells(g)) * 4) +
                                 align_up((size_t)(kSeedMaxBlocks + 1) * 4)
                           : 0;
@@ -919,7 +1011,7 @@ static RulebookWs rulebook_ws_carve(void *ws, const Geom &g, int64_t n_in) {
   w.rank2row = c.take<int32_t>(n_in > 0 ? n_in : 1);
   w.use_dense = dense_marking_applies(g, n_in, &w.dense);
   w.in_bits = w.use_dense ? c.take<uint32_t>((size_t)dense_in_words(g, w.dense)) : nullptr;
-  w.can_seed = w.use_dense && seed_applies(g);
+  w.can_seed = !g.subm && seed_applies(g);
   w.seed_rows = w.seed_pairs = w.pairsum = nullptr;
   if (w.can_seed) {
     w.seed_rows = c.take<int32_t>((size_t)w.table.n_words);
@@ -945,6 +1037,19 @@ static int rulebook_check(const ssc_geometry *g, Geom *gg, const int32_t *indice
   SSC_CHECK(workspace_bytes >= rulebook_ws_bytes(*gg, n_in), SSC_EWORKSPACE,
             "rulebook workspace too small: %zu < %zu", workspace_bytes,
             rulebook_ws_bytes(*gg, n_in));
+  return SSC_OK;
+}
+
+// Enqueue: the scan's second pass, and beside it the range boundaries of a convolution's plan.
+static int launch_prefix_split(const RulebookWs &w, const SplitRequest &split, int32_t *mirror,
+                               int ticket, hipStream_t s) {
+  const int64_t word_blocks = w.table.n_scan_blocks;
+  hipLaunchKernelGGL(prefix_split_kernel,
+                     dim3((unsigned)(word_blocks + split_request_blocks(split))),
+                     dim3(kScanThreads), seed_lds_bytes(word_blocks), s, w.table.bits,
+                     w.table.n_words, word_blocks, w.table.blocksum, w.table.prefix, w.table.total,
+                     mirror, w.pairsum, w.seed_rows, w.seed_pairs, split, ticket);
+  SSC_LAUNCH_CHECK("prefix_split");
   return SSC_OK;
 }
 
@@ -999,16 +1104,13 @@ static int rulebook_mark_and_scan(const int32_t *indices, int64_t n_in, const Ge
     SSC_LAUNCH_CHECK("dilate_blocksum");
     if (two_level) return SSC_OK;
     if (!seed || split == nullptr) return bit_table_scan_prefix(w.table, s, mirror, ticket);
-    // the scan's second pass, and beside it the range boundaries of the convolution's plan
-    const int64_t split_blocks = ceil_div(split->n_rng, kScanThreads / 16);
-    hipLaunchKernelGGL(prefix_split_kernel, dim3((unsigned)(word_blocks + split_blocks)),
-                       dim3(kScanThreads), seed_lds_bytes(word_blocks), s, w.table.bits, w.table.n_words, word_blocks,
-                       w.table.blocksum, w.table.prefix, w.table.total, mirror, w.pairsum,
-                       w.seed_rows, w.seed_pairs, *split, ticket);
-    SSC_LAUNCH_CHECK("prefix_split");
-    return SSC_OK;
+    return launch_prefix_split(w, *split, mirror, ticket, s);
   }
-  if ((rc = bit_table_clear(w.table, s)) != SSC_OK) return rc;
+  // (a regular convolution off the dilation path -- strided, dilated -- whose plan is to be
+  // seeded or whose pair launch takes the prefixes in two levels: the marking kernel counts
+  // the pairs of every table word on its way, in seed_pairs[], zeroed with the table)
+  const bool seed = !gg.subm && pair_num != nullptr && (split != nullptr || two_level) && w.can_seed;
+  if ((rc = bit_table_clear(w.table, s, false, seed ? w.seed_pairs : nullptr)) != SSC_OK) return rc;
   if (gg.subm) {
     if (job != nullptr) {
       const int64_t n = combine_job_elements(*job);
@@ -1026,26 +1128,31 @@ static int rulebook_mark_and_scan(const int32_t *indices, int64_t n_in, const Ge
   }
   {
     const int64_t mark_blocks = ceil_div(w.n_chunks, 4);
+    int32_t *word_pairs = seed ? w.seed_pairs : nullptr;
     if (job != nullptr) {
       const int64_t n = combine_job_elements(*job);
       const int64_t rows = std::min<int64_t>(ceil_div(ceil_div(n, 256), mark_blocks), 1024);
       hipLaunchKernelGGL(mark_count_kernel<true>,
                          dim3((unsigned)mark_blocks, (unsigned)(gg.ks[0] + rows)), dim3(256), 0, s,
                          indices, n_in, gg, w.table.bits, w.chunk_count, w.n_chunks,
-                         w.table.total + 1, *job, n);
+                         w.table.total + 1, *job, n, word_pairs);
     } else {
       hipLaunchKernelGGL(mark_count_kernel<false>, dim3((unsigned)mark_blocks, (unsigned)gg.ks[0]),
                          dim3(256), 0, s, indices, n_in, gg, w.table.bits, w.chunk_count,
-                         w.n_chunks, w.table.total + 1, CombineJob{}, (int64_t)0);
+                         w.n_chunks, w.table.total + 1, CombineJob{}, (int64_t)0, word_pairs);
     }
   }
   SSC_LAUNCH_CHECK("mark_count");
   if (pair_num == nullptr) return bit_table_scan(w.table, s, mirror, ticket);
-  hipLaunchKernelGGL(blocksum_scan_chunks_kernel, dim3((unsigned)(w.table.n_scan_blocks + gg.K)),
+  auto sums_kernel = seed ? blocksum_scan_chunks_kernel<true> : blocksum_scan_chunks_kernel<false>;
+  hipLaunchKernelGGL(sums_kernel, dim3((unsigned)(w.table.n_scan_blocks + gg.K)),
                      dim3(kScanThreads), 0, s, w.table.bits, w.table.n_words, w.table.blocksum,
-                     w.table.n_scan_blocks, w.chunk_count, w.n_chunks, pair_num);
+                     w.table.n_scan_blocks, w.chunk_count, w.n_chunks, pair_num, w.seed_rows,
+                     w.seed_pairs, w.pairsum);
   SSC_LAUNCH_CHECK("blocksum_scan_chunks");
-  return bit_table_scan_prefix(w.table, s, mirror, ticket);
+  if (two_level) return SSC_OK;
+  if (!seed || split == nullptr) return bit_table_scan_prefix(w.table, s, mirror, ticket);
+  return launch_prefix_split(w, *split, mirror, ticket, s);
 }
 
 // Enqueue: the pair lists and, with out_indices, the output rows (one launch for both).
@@ -1220,8 +1327,10 @@ int ssc::rulebook_begin_impl(const int32_t *indices, int64_t n_in, const ssc_geo
   // sizes do not depend on the totals, are computed while the host wakes up
   int32_t *mirror = nullptr;
   if ((rc = read_back_mirror(&mirror)) != SSC_OK) return rc;
-  if (split != nullptr && !(w.can_seed && split->n_rng >= 1 && split->n_rng <= kMaxRanges &&
-                            split->range_row0 != nullptr))
+  if (split != nullptr &&
+      !(w.can_seed && split->n_rng >= 1 && split->n_rng <= kMaxRanges &&
+        split->range_row0 != nullptr && split->n_rng_alt >= 0 && split->n_rng_alt <= kMaxRanges &&
+        (split->n_rng_alt == 0 || split->range_row0_alt != nullptr)))
     split = nullptr;
   *seeded = split != nullptr;
   // A table the caller keeps between calls: all zero now, and all zero again when the
@@ -1241,8 +1350,8 @@ int ssc::rulebook_begin_impl(const int32_t *indices, int64_t n_in, const ssc_geo
   // second pass: the launch of the pair lists takes the prefixes in two levels, places the
   // range boundaries and hands the totals to the host, which sees them (read_back_end) while
   // that launch still runs.
-  const int split_blocks = split ? (int)ceil_div(split->n_rng, kScanThreads / 16) : 0;
-  const bool two_level = w.use_dense && w.can_seed && out_indices != nullptr &&
+  const int split_blocks = split ? split_request_blocks(*split) : 0;
+  const bool two_level = w.can_seed && out_indices != nullptr &&
                          ceil_div(w.n_chunks, 4) > split_blocks;
   // (the kernel that finishes the scan stores a ticket behind the totals, for the host to
   // spin on: it then sees them a few microseconds before the event behind the kernel says so)
@@ -1256,7 +1365,8 @@ int ssc::rulebook_begin_impl(const int32_t *indices, int64_t n_in, const ssc_geo
                           clean_words);
   }
   TwoLevel two = {w.table.blocksum, w.pairsum, w.seed_rows, w.seed_pairs, w.table.n_scan_blocks,
-                  split ? *split : SplitRequest{0, 0, 0, nullptr}, split_blocks, w.table.total,
+                  split ? *split : SplitRequest{0, 0, 0, nullptr, 0, 0, nullptr}, split_blocks,
+                  w.table.total,
                   mirror, ticket, clean != nullptr ? 1 : 0};
   // (the header of a clean table holds the totals: the block that hands them to the host
   // clears it, the other blocks the words behind it)

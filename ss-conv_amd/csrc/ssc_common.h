@@ -70,8 +70,9 @@ static inline int64_t bit_words(int64_t n_bits) { return ceil_div(n_bits, 32); }
 size_t bit_table_bytes(int64_t n_bits);
 BitTable bit_table_carve(Carver &c, int64_t n_bits);
 // Enqueue: zero the table and total[]; with blocksum_too also blocksum[] (for a first scan
-// pass that adds into it).
-int bit_table_clear(const BitTable &t, hipStream_t s, bool blocksum_too = false);
+// pass that adds into it); with per_word also that array of one counter for every word.
+int bit_table_clear(const BitTable &t, hipStream_t s, bool blocksum_too = false,
+                    int32_t *per_word = nullptr);
 // Enqueue: prefix[], total[0] from bits[].  With `mirror` (memory the device can write and
 // the host can read, see read_back_mirror), the kernel that writes total[0] also copies
 // total[0..3] there, which saves the copy a host that waits for them would otherwise queue.
@@ -233,7 +234,16 @@ struct SplitRequest {
   int tile_rows;       // weight of a pair relative to tile_cost (see split_work in conv.hip)
   long long tile_cost; // cost of a row's share of a tile, in the same unit
   int32_t *range_row0; // [n_rng + 1] device: first output row of every range
+  // A second cut of the same rows (n_rng_alt = 0: none), for a caller whose plan depends on
+  // the number of output rows, which only the rulebook's totals will tell: it asks for the
+  // cut of either plan and uses the one that applies.
+  int n_rng_alt, tile_rows_alt;
+  int32_t *range_row0_alt;
 };
+// Blocks of kScanThreads threads that place the boundaries of a request (16 lanes to a range).
+static inline int split_request_blocks(const SplitRequest &rq) {
+  return (int)(ceil_div(rq.n_rng, kScanThreads / 16) + ceil_div(rq.n_rng_alt, kScanThreads / 16));
+}
 // ssc_rulebook_begin with an optional split request.  *seeded = whether range_row0 will be
 // written (the geometry takes the dilation path and the table is small enough).  `job`
 // (optional, conv_pack.h): synthesis and packing of a layer's filters, enqueued with the

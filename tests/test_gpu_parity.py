@@ -2003,6 +2003,55 @@ def test_fused_rulebook_conv_equals_the_two_calls(subm, stride, device):
     assert torch.equal(y3 + layer.bias.detach(), y1.features.detach())
 
 
+@pytest.mark.parametrize("batch,grid,n_vox", [(4, 64, 45000), (2, 32, 45000)])
+def test_strided_layer_with_its_plan_cut_by_the_rulebook(batch, grid, n_vox, device):
+    """A strided layer's rulebook counts the pairs of every table word while it marks the
+    outputs and places the range boundaries of the convolution's plan itself.  Whether the
+    outputs outnumber the inputs (a sparse cloud, first case) or not (a dense one, second
+    case) decides what the plan looks like -- two ranges to a workgroup or one, at these
+    sizes -- and is known only when the rulebook's totals arrive: the rulebook places the
+    cut of either plan.  Same rulebook as get_indice_pairs, same output as the convolution
+    over those pairs, whose plan comes from its own passes over the pairs (the same sums in
+    another order)."""
+    from ss_conv.sp_ops.conv import SparseConvolution
+    from ss_conv.sp_ops.ops import get_indice_pairs
+    from ss_conv.sp_ops.functional import indice_conv
+    from ss_conv.sp_ops.tensor import SparseTensor
+    rng = np.random.default_rng(31)
+    idx = random_voxels(rng, batch, grid, n_vox)
+    t = torch.from_numpy(idx).to(device)
+    torch.manual_seed(3)
+    layer = SparseConvolution(3, 16, 256, 3, stride=2, padding=1, bias=False,
+                              indice_key="s").to(device)
+    x = torch.randn((idx.shape[0], 16), device=device)
+    with torch.no_grad():
+        st = SparseTensor(x, t, [grid] * 3, batch)
+        y = layer(st)
+        outids, _, pairs, num, _ = st.indice_dict["s"]
+        g_idx, g_pairs, g_num = get_indice_pairs(t, batch, [grid] * 3, 3, 2, 1, 1, 0, False)
+        assert torch.equal(outids, g_idx) and torch.equal(pairs, g_pairs)
+        assert torch.equal(num, g_num)
+        n_out = g_idx.shape[0]
+        assert (n_out > n_vox) == (grid == 64), (n_out, n_vox)
+        y2 = indice_conv(x, layer.weight, g_pairs, g_num, n_out)
+        assert torch.allclose(y.features, y2, rtol=1e-5, atol=1e-5)
+        # against the oracle on a sample of rows: float64 sums over the pairs
+        gp = g_pairs.cpu().numpy()
+        gn = g_num.cpu().numpy()
+        w = layer.weight.detach().cpu().numpy().reshape(27, 16, 256).astype(np.float64)
+        xf = x.cpu().numpy().astype(np.float64)
+        rows = rng.choice(n_out, size=64, replace=False)
+        want = np.zeros((64, 256))
+        pos = {int(r): j for j, r in enumerate(rows)}
+        for k in range(27):
+            o = gp[k, 1, :gn[k]]
+            hit = np.nonzero(np.isin(o, rows))[0]
+            for h in hit:
+                want[pos[int(o[h])]] += xf[gp[k, 0, h]] @ w[k]
+        got = y.features[torch.from_numpy(rows).to(device)].cpu().numpy()
+        assert np.abs(got - want).max() <= 1e-4 * max(np.abs(want).max(), 1.0)
+
+
 def test_fused_layer_on_a_dense_grid(device):
     """A grid the outputs nearly fill: the layer sizes its plan for the bound on the number
     of outputs (every cell: 4 x 64^3) before that number arrives, and the real number (about
