@@ -249,10 +249,17 @@ def ops_table(torch, _ext, synth, dev, seed):
     from ss_conv.sp_ops.tensor import SparseTensor
     from ss_conv.sp_ops.voxelize import Point2Voxel, Voxel2Point
 
-    def timed(fn, n=20, warm=3):
+    def timed(fn, n=20, warm=3, busy_ms=40.0):
+        # (a GPU that has idled runs its first tens of milliseconds at a lower clock: every
+        # row is measured behind busy_ms of the same work, as the layer step is)
         for _ in range(warm):
             fn()
         torch.cuda.synchronize()
+        t_busy = time.perf_counter()
+        while (time.perf_counter() - t_busy) * 1e3 < busy_ms:
+            for _ in range(5):
+                fn()
+            torch.cuda.synchronize()
         a = time.perf_counter()
         for _ in range(n):
             r = fn()
@@ -291,10 +298,10 @@ def ops_table(torch, _ext, synth, dev, seed):
     w = torch.randn(3, 3, 3, cin, cout, device=dev) / (K * cin) ** 0.5
     go = torch.randn(o_idx.shape[0], cout, device=dev)
     P = int(num.sum().item())
-    _ext.indice_conv_backward_fp32(f, w, go, pairs, num, 0, 0)
-    torch.cuda.synchronize()
+    ms, _ = timed(lambda: _ext.indice_conv_backward_fp32(f, w, go, pairs, num, 0, 0), n=10)
     _ext.profile_conv(True)  # the input gradient is the forward kernel on the output gradient
-    ms, _ = timed(lambda: _ext.indice_conv_backward_fp32(f, w, go, pairs, num, 0, 0), n=10, warm=0)
+    for _ in range(10):
+        _ext.indice_conv_backward_fp32(f, w, go, pairs, num, 0, 0)
     in_ms = _ext.profile_conv_read()
     _ext.profile_conv(False)
     rows.append("%-44s %8.3f ms %9.2f GFLOP %7.1f TFLOP/s %5.1f%% of fp32 MFMA peak"
