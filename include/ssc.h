@@ -142,15 +142,18 @@ int ssc_rulebook_rows(const ssc_geometry *g, int64_t n_in, void *workspace,
 /* Rulebook and convolution plan of one layer that has no rulebook yet, in one pair of calls --
  * what a layer's forward does between get_indice_pairs and indice_conv
  * (ss_conv/sp_ops/conv.py:131-150, src/conv/indice_conv.h:21-131 then 247-343):
- *   ssc_rulebook_conv_begin is ssc_rulebook_begin, and for a regular convolution with
- *     stride 1 and dilation 1 (whose rulebook counts, on its way, the outputs and the pairs
- *     of every cell of the grid) it also deals the output rows to the convolution kernel's
- *     workgroups, in a launch the rulebook makes anyway, into the head of `scratch`
- *     (ssc_conv_plan_scratch_bytes of ssc_rulebook_out_bound() rows; may be NULL);
+ *   ssc_rulebook_conv_begin is ssc_rulebook_begin, and for a regular convolution (any
+ *     stride and dilation; its rulebook counts, on its way, the outputs and the pairs of
+ *     every word of its table of cells, for tables of up to 2^25 cells) it also deals the
+ *     output rows to the convolution kernel's workgroups, in a launch the rulebook makes
+ *     anyway, into the head of `scratch` (ssc_conv_plan_scratch_bytes of
+ *     ssc_rulebook_out_bound() rows; may be NULL) -- for a strided layer, whose plan depends
+ *     on whether the outputs will outnumber the inputs, once for either case;
  *   ssc_rulebook_conv_finish is ssc_rulebook_finish followed by ssc_conv_plan_build for the
  *     forward direction over the new pairs (pair_stride = n_in), into `plan` and `scratch`
  *     sized for any number of rows from n_out up to the bound; where the rulebook dealt the
- *     rows and the input rows came in key order, the plan needs three launches instead of six.
+ *     rows and the input rows came in key order, the plan needs two to four launches
+ *     instead of six or seven.
  * Same host thread for both; one layer between them at a time.  The plan is the one
  * ssc_conv_run_* expects; compared with ssc_conv_plan_build's the ranges begin at other
  * rows, so results agree up to the order of the float sums.
