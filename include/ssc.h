@@ -414,7 +414,8 @@ int ssc_conv_tuning(int32_t flags);
  * with nearly all of its LDS (the convolution kernel leaves about 4 KB of a CU's 160 KB):
  * with on != 0 those calls pick kernels that fit into what is left (smaller blocks, two
  * launches for the schedule instead of one) and so run beside the convolution instead of
- * behind it.  Results are the same bit for bit.  Returns the previous setting (default 0). */
+ * behind it.  Results are the same bit for bit.  A setting of the calling host thread;
+ * returns its previous value (default 0). */
 int ssc_index_beside_conv(int32_t on);
 int ssc_profile_conv_read(float *ms /* host */, int32_t capacity, int32_t *count /* host */);
 

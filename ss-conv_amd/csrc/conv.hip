@@ -1174,7 +1174,7 @@ static int64_t g_conv_rebalance_stages = kRebalanceStages;
 static bool g_conv_fuse_fill = true;  // range_sched_kernel<true> instead of sched_fill_kernel
 // Index work (rulebooks, plans) is queued on a stream of its own and runs while a convolution
 // holds every CU with nearly all of its LDS: kernels are picked that need little LDS.
-static bool g_index_beside_conv = false;
+static thread_local bool g_index_beside_conv = false;  // (a setting of the calling host thread)
 static bool g_conv_rebalance = true;  // long kernels: a second work split from the first one's counts
 static bool g_conv_round8 = false;    // ranges per column block: a multiple of 8 only
 static bool g_conv_small = true;      // layers of at most 8 input channels: conv_small_kernel

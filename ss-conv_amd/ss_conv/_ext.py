@@ -336,15 +336,15 @@ def _clean_table(nbytes, dev, stream):
 # stream before they are handed out.
 _index_streams = {}  # device index -> _IndexStream
 _index_overlap = os.environ.get("SSC_INDEX_STREAM", "1") != "0"
-_beside_now = [False]  # what the library was last told (ssc_index_beside_conv)
+_beside_now = threading.local()  # .on: what the library was last told on this host thread
 
 
 def _beside(on):
     """Tell the library whether the index work queued next runs on the second stream (it
     then picks kernels that fit beside a convolution)."""
-    if _beside_now[0] != on:
+    if getattr(_beside_now, "on", False) != on:
         _lib.ssc_index_beside_conv(1 if on else 0)
-        _beside_now[0] = on
+        _beside_now.on = on
 
 
 # The second stream pays where the kernel that waits for the index work -- the convolution of
@@ -1312,7 +1312,15 @@ class _DeferredCombine(object):
     __slots__ = ("args", "tensors", "packed", "stream", "sizes")
 
 
-_deferred = []  # at most one _DeferredCombine
+_deferred_tls = threading.local()
+
+
+def _deferred_jobs():
+    """This host thread's deferred jobs (at most one _DeferredCombine)."""
+    jobs = getattr(_deferred_tls, "jobs", None)
+    if jobs is None:
+        jobs = _deferred_tls.jobs = []
+    return jobs
 
 
 def kernel_combine(weight, basis, chan_out, chan_in, blocks, n_irreps_in, kernel_volume, c_in,
@@ -1341,7 +1349,7 @@ def kernel_combine(weight, basis, chan_out, chan_in, blocks, n_irreps_in, kernel
         job.args, job.packed, job.stream = args, buf, _stream(weight)
         job.tensors = (weight, basis, chan_out, chan_in, blocks, out)
         job.sizes = (int(kernel_volume), int(c_in), int(c_out), weight.device)
-        _deferred.append(job)
+        _deferred_jobs().append(job)
         return out, buf
     _check(_lib.ssc_kernel_combine_packed_f32(*args, buf.data_ptr(), buf.numel(), _stream(weight)))
     return out, buf
@@ -1349,8 +1357,9 @@ def kernel_combine(weight, basis, chan_out, chan_in, blocks, n_irreps_in, kernel
 
 def flush_combine():
     """Queue what kernel_combine(defer=True) left, if nobody has taken it."""
-    while _deferred:
-        job = _deferred.pop()
+    jobs = _deferred_jobs()
+    while jobs:
+        job = jobs.pop()
         _check(_lib.ssc_kernel_combine_packed_f32(*job.args, job.packed.data_ptr(),
                                                   job.packed.numel(), job.stream))
 
@@ -1358,13 +1367,14 @@ def flush_combine():
 def _take_combine(K, c_in, c_out, dev, stream):
     """The deferred job as an ssc_combine_job for a rulebook of these sizes on this stream
     (None, and the job queued by itself, when it does not fit)."""
-    if not _deferred:
+    jobs = _deferred_jobs()
+    if not jobs:
         return None
-    job = _deferred[-1]
+    job = jobs[-1]
     if job.sizes != (K, c_in, c_out, dev) or job.stream != stream:
         flush_combine()
         return None
-    _deferred.pop()
+    jobs.pop()
     a = job.args
     st = _CombineJob(a[0], a[1], a[2], a[3], a[4], a[5], a[6], a[9], job.packed.data_ptr(),
                      job.packed.numel())
