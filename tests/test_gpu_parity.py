@@ -2052,6 +2052,66 @@ def test_strided_layer_with_its_plan_cut_by_the_rulebook(batch, grid, n_vox, dev
         assert np.abs(got - want).max() <= 1e-4 * max(np.abs(want).max(), 1.0)
 
 
+@pytest.mark.parametrize("seed", [0, 1])
+def test_fused_layer_random_geometries(seed, oracle, device):
+    """The layer's own sequence -- rulebook, the plan's range boundaries placed by the
+    rulebook, convolution -- on geometries of every kind: kernel size, stride, padding and
+    dilation differing per axis, grids that are no cubes and whose rows are no whole table
+    words, a few thousand voxels, so that a plan has many ranges; sparse and dense clouds
+    (outputs more or fewer than inputs).  Rulebook bit-exact against the oracle's, features
+    against the oracle's convolution over those pairs."""
+    from ss_conv.sp_ops.conv import SparseConvolution
+    from ss_conv.sp_ops.tensor import SparseTensor
+    rng = np.random.default_rng(1000 + seed)
+    done = 0
+    while done < 14:
+        batch = int(rng.integers(1, 4))
+        shape = [int(rng.integers(8, 40)) for _ in range(3)]
+        if rng.integers(0, 2):
+            shape[2] = int(rng.choice([32, 64]))  # whole table words: the dilation path at stride 1
+        ks = [int(rng.integers(1, 4)) for _ in range(3)]
+        st = [int(rng.integers(1, 4)) for _ in range(3)]
+        if rng.integers(0, 3) == 0:
+            st = [1, 1, 1]
+        dl = [int(rng.integers(1, 3)) if t == 1 else 1 for t in st]
+        pd = [int(rng.integers(0, 3)) for _ in range(3)]
+        out_shape = [(n + 2 * p - d * (k - 1) - 1) // t + 1
+                     for n, p, d, k, t in zip(shape, pd, dl, ks, st)]
+        if min(out_shape) < 1 or ks == [1, 1, 1]:
+            continue
+        done += 1
+        cells = batch * shape[0] * shape[1] * shape[2]
+        n = int(rng.integers(1500, 9000))
+        n = min(n, int(cells * float(rng.choice([0.05, 0.3, 0.9]))) + 1)
+        flat = np.sort(rng.choice(cells, size=n, replace=False))
+        vol = shape[0] * shape[1] * shape[2]
+        b, r = flat // vol, flat % vol
+        idx = np.stack([b, r // (shape[1] * shape[2]), (r // shape[2]) % shape[1],
+                        r % shape[2]], 1).astype(np.int32)
+        cin, cout = int(rng.choice([4, 12, 16, 24])), int(rng.choice([16, 40, 64, 72, 256]))
+        case = (batch, shape, ks, st, pd, dl, n, cin, cout)
+        print("case", case, flush=True)
+        o_idx, o_pairs, o_num = oracle.canonicalize(*oracle.rulebook(idx, batch, shape, ks, st, pd,
+                                                                     dl, False))
+        torch.manual_seed(seed * 100 + done)
+        layer = SparseConvolution(3, cin, cout, ks, stride=st, padding=pd, dilation=dl,
+                                  bias=False, indice_key="r").to(device)
+        f = rng.normal(size=(n, cin)).astype(np.float32)
+        with torch.no_grad():
+            x = SparseTensor(torch.from_numpy(f).to(device), torch.from_numpy(idx).to(device),
+                             shape, batch)
+            y = layer(x)
+        outids, _, pairs, num, _ = x.indice_dict["r"]
+        assert np.array_equal(outids.cpu().numpy(), o_idx), case
+        assert np.array_equal(pairs.cpu().numpy(), o_pairs), case
+        assert np.array_equal(num.cpu().numpy(), o_num), case
+        assert list(y.spatial_shape) == out_shape, case
+        K = ks[0] * ks[1] * ks[2]
+        w = layer.weight.detach().cpu().numpy().reshape(K, cin, cout)
+        want = oracle.conv_fwd(f, w, o_pairs, o_num, o_idx.shape[0], matmul=np.matmul)
+        assert rel_l2(y.features.cpu().numpy(), want) < REL_L2, case
+
+
 def test_fused_layer_on_a_dense_grid(device):
     """A grid the outputs nearly fill: the layer sizes its plan for the bound on the number
     of outputs (every cell: 4 x 64^3) before that number arrives, and the real number (about
