@@ -177,6 +177,22 @@ for _name, (_res, _args) in _SIGNATURES.items():
 
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)
 
+# ssc_conv_tuning changes what plans look like (ranges, column blocks, launches), and a plan
+# built under one setting must not be run under another: the kernel would walk a schedule
+# that is laid out otherwise.  Every call through this module's handle of the library is
+# noted here, and the plans kept with a rulebook are keyed by the setting they were built
+# under (_plan_of), so a change leaves the old plans unused instead of misread.
+_tuning_now = [1]
+_raw_conv_tuning = _lib.ssc_conv_tuning
+
+
+def _conv_tuning(flags):
+    _tuning_now[0] = int(flags)
+    return _raw_conv_tuning(int(flags))
+
+
+_lib.ssc_conv_tuning = _conv_tuning
+
 SSC_EINVAL, SSC_ERUNTIME, SSC_EWORKSPACE, SSC_EHIP = -1, -2, -3, -4
 
 
@@ -691,7 +707,7 @@ def _plan_of(meta, pairs, num, K, c_in, c_out, elem_bytes, n_in, n_out, inverse,
     """The plan of a (direction, channel counts, element type, row counts) combination over
     a rulebook: built on first use, kept with the rulebook afterwards."""
     stride = pairs.size(2)
-    key = (bool(inverse), c_in, c_out, elem_bytes, n_in, n_out)
+    key = (bool(inverse), c_in, c_out, elem_bytes, n_in, n_out, _tuning_now[0])
     plan = meta.get_plan(key)
     if plan is None:
         _beside(beside)
@@ -837,7 +853,7 @@ def rulebook_conv(features, filters, indices, batch_size, out_spatial_shape, ker
                            epilogue)
         outids, pairs, num = _rulebook_result(r, n_out, in_order)
     if n_out > 0:
-        pairs._ssc_meta.put_plan((False, c_in, c_out, eb, n_in, n_out), r.plan)
+        pairs._ssc_meta.put_plan((False, c_in, c_out, eb, n_in, n_out, _tuning_now[0]), r.plan)
     return out, outids, pairs, num
 
 

@@ -495,6 +495,33 @@ def test_conv_lone_last_column_group(shape, oracle, device):
     assert _ext._lib.ssc_conv_plan_bytes(1000, 27, cin, cout, 1000) > 0
 
 
+def test_plans_are_kept_apart_by_tuning_setting(device):
+    """ssc_conv_tuning changes what a plan looks like (here: a launch of its own for the lone
+    last column group, or a column block of its own): the binding keys the plans it keeps
+    with a rulebook by the setting they were built under, so a call under another setting
+    over the same pairs tensor builds its own plan instead of walking the old one."""
+    from ss_conv import _ext
+    from ss_conv.sp_ops.ops import get_indice_pairs
+    rng = np.random.default_rng(8)
+    idx = torch.from_numpy(random_voxels(rng, 2, 16, 2500)).to(device)
+    o_idx, pairs, num = get_indice_pairs(idx, 2, [16] * 3, 3, 1, 1)
+    f = torch.randn(idx.shape[0], 64, device=device)
+    w = torch.randn(3, 3, 3, 64, 72, device=device) / 40.0
+    n_out = o_idx.shape[0]
+    a = _ext.indice_conv_fp32(f, w, pairs, num, n_out, 0, 0)
+    meta = _ext.rulebook_meta(pairs)
+    assert len(meta.plans) == 1
+    try:
+        assert _ext._lib.ssc_conv_tuning(1 | 2) == 0
+        b = _ext.indice_conv_fp32(f, w, pairs, num, n_out, 0, 0)
+        assert len(meta.plans) == 2
+    finally:
+        _ext._lib.ssc_conv_tuning(1)
+    c = _ext.indice_conv_fp32(f, w, pairs, num, n_out, 0, 0)
+    assert len(meta.plans) == 2 and torch.equal(a, c)
+    assert rel_l2(b.cpu().numpy(), a.cpu().numpy()) < 1e-6
+
+
 @pytest.mark.parametrize("shape", [(200, 72), (256, 200), (197, 70), (260, 136)])
 def test_conv_five_group_form(shape, oracle, device):
     """More than 192 input channels (four chunks or more) and Cout = 64 b + (1..16), b >= 1:
