@@ -32,7 +32,7 @@ CLOCK_WARMUP_MS = 100
 # launches) for every workload this script offers, from rocprofv3 --pmc FETCH_SIZE /
 # WRITE_SIZE runs scaled by a copy kernel of known size (the summaries
 # profiles/conv_fwd_<workload>_hbm_traffic.md give commands and counter values).
-MEASURED_TRAFFIC_BYTES = {"cfg1": 4163988, "cfg2": 346630319, "cfg3": 229352772, "cfg5": 68946166884}
+MEASURED_TRAFFIC_BYTES = {"cfg1": 4173070, "cfg2": 346645302, "cfg3": 227819460, "cfg5": 69089450913}
 # the same for all kernels of one rulebook call and of one Point2Voxel call
 # (profiles/rulebook_hbm_traffic.md, profiles/point_voxel_hbm_traffic.md)
 RULEBOOK_TRAFFIC_BYTES = {"cfg2": 37500000, "cfg3": 28600000, "cfg5": 188400000}
