@@ -1346,7 +1346,7 @@ int ssc::rulebook_begin_impl(const int32_t *indices, int64_t n_in, const ssc_geo
     w.table.total = static_cast<int32_t *>(clean_table);
     w.in_bits = clean + kCleanHeader / 4;
   }
-  // With room for the output rows at hand the dilation path needs no launch for the scan's
+  // With room for the output rows at hand a regular rulebook needs no launch for the scan's
   // second pass: the launch of the pair lists takes the prefixes in two levels, places the
   // range boundaries and hands the totals to the host, which sees them (read_back_end) while
   // that launch still runs.

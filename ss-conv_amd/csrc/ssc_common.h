@@ -221,11 +221,12 @@ __device__ __forceinline__ void emit_rows_of_word_at(uint32_t b, int r, int64_t 
 }
 
 // ---- work split of a convolution, seeded by the rulebook ----------------------------------
-// A regular stride-1 rulebook knows, cell by cell of its output table, how many output rows
-// and how many pairs lie below the cell (the popcounts its dilation step takes anyway).  That
-// is the work measure the convolution's plan deals its output rows to the workgroups by, so
-// the rulebook can place the ranges' boundaries itself, in a launch it makes anyway: the
-// plan is then built without its own passes over the pairs for that purpose.
+// A regular rulebook knows, word by word of its output table, how many output rows and how
+// many pairs lie below the word (at stride 1 the popcounts its dilation step takes anyway;
+// otherwise the marking kernel counts the pairs of every word on its way).  That is the work
+// measure the convolution's plan deals its output rows to the workgroups by, so the rulebook
+// can place the ranges' boundaries itself, in a launch it makes anyway: the plan is then
+// built without its own passes over the pairs for that purpose.
 constexpr int kMaxRanges = 512;       // two for each of at most 256 workgroups
 constexpr int kSeedMaxBlocks = 512;   // scan blocks of a table whose block sums are scanned in LDS by
                                       // every block that needs them (512: 33 M cells)
@@ -245,7 +246,7 @@ static inline int split_request_blocks(const SplitRequest &rq) {
   return (int)(ceil_div(rq.n_rng, kScanThreads / 16) + ceil_div(rq.n_rng_alt, kScanThreads / 16));
 }
 // ssc_rulebook_begin with an optional split request.  *seeded = whether range_row0 will be
-// written (the geometry takes the dilation path and the table is small enough).  `job`
+// written (a regular convolution whose table has at most kSeedMaxBlocks scan blocks).  `job`
 // (optional, conv_pack.h): synthesis and packing of a layer's filters, enqueued with the
 // rulebook's first launch where that has room for it and before it otherwise.
 struct CombineJob;
